@@ -1,0 +1,327 @@
+"""Pins the C oracle (oracle/ncnn_int8_oracle.c) without running ncnn.
+
+ncnn's own tests for this path are differential (naive vs optimised, no literal vectors), so the
+oracle is pinned by what the mathematics fixes: hand-listed rounding cases, an independent numpy
+int64/float32 statement (tests/npref.py), brute force on tiny inputs, and structural identities.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+import npref
+from oracle import oracle
+
+F = np.float32
+
+
+# ----------------------------------------------------------------------------- float2int8
+def test_float2int8_special_cases():
+    below_half = np.nextafter(F(0.5), F(0))  # 0.49999997: trunc(v+0.5) implementations give 1 here
+    cases = [
+        (0.0, 0), (-0.0, 0), (0.5, 1), (-0.5, -1), (1.5, 2), (-1.5, -2), (2.5, 3), (-2.5, -3),
+        (float(below_half), 0), (-float(below_half), 0), (0.4999, 0), (126.5, 127), (-126.5, -127),
+        (126.49999, 126), (127.49, 127), (127.5, 127), (-127.5, -127), (128.0, 127), (-128.0, -127),
+        (200.0, 127), (-200.0, -127), (1e9, 127), (-1e9, -127), (3e9, -127), (-3e9, -127),
+        (float("inf"), -127), (float("-inf"), -127), (float("nan"), -127),
+    ]
+    for v, want in cases:
+        assert int(oracle.float2int8(F(v))) == want, v
+
+
+def test_float2int8_matches_float64_rounding_on_grid():
+    rng = np.random.default_rng(1)
+    v = np.concatenate([rng.uniform(-140, 140, 4000), np.arange(-130, 130) + 0.5, np.arange(-130, 130) - 0.5]).astype(F)
+    v = np.concatenate([v, np.nextafter(v, F(np.inf)), np.nextafter(v, F(-np.inf))])
+    got = oracle.quantize(v[None, :], [1.0])[0]
+    assert np.array_equal(got, npref.float2int8(v))
+    assert got.min() >= -127 and got.max() <= 127
+
+
+def test_activation_closed_forms():
+    assert oracle.activation(-1.0, 1) == 0.0 and oracle.activation(2.0, 1) == 2.0
+    assert oracle.activation(-2.0, 2, (0.25,)) == -0.5
+    assert oracle.activation(7.0, 3, (0.0, 6.0)) == 6.0 and oracle.activation(-1.0, 3, (0.0, 6.0)) == 0.0
+    a, b = 1.0 / 6.0, 0.5  # hardswish
+    assert oracle.activation(-4.0, 6, (a, b)) == 0.0
+    assert oracle.activation(5.0, 6, (a, b)) == 5.0
+    x = F(1.25)
+    assert oracle.activation(float(x), 6, (a, b)) == float(x * (x * F(a) + F(b)))
+    rng = np.random.default_rng(0)
+    v = rng.uniform(-8, 8, 200).astype(F)
+    for t, p in ((0, (0, 0)), (1, (0, 0)), (2, (0.1, 0)), (3, (0.0, 6.0)), (6, (a, b))):
+        want = npref.activation(v, t, p)
+        got = np.array([oracle.activation(float(z), t, p) for z in v], F)
+        assert np.array_equal(got, want), t
+
+
+# ----------------------------------------------------------------------------- quantize
+def test_quantize_per_row_and_single_scale():
+    rng = np.random.default_rng(2)
+    x = rng.uniform(-3, 3, (5, 37)).astype(F)
+    s = rng.uniform(10, 60, 5).astype(F)
+    assert np.array_equal(oracle.quantize(x, s), npref.float2int8(x * s[:, None]))
+    assert np.array_equal(oracle.quantize(x, s[:1]), npref.float2int8(x * s[0]))
+
+
+# ----------------------------------------------------------------------------- convolution
+def _conv_case(rng, c, h, w, outc, kernel, dilation, stride, pads, group, term, act, act_params, bias, int8_in,
+               by_group, pad_value=0.0):
+    cg = c // group
+    kw, kh = kernel
+    x = rng.uniform(-1, 1, (c, h, w)).astype(F)
+    wt = rng.integers(-127, 128, (outc, cg, kh, kw)).astype(np.int8)
+    nws = group if by_group else outc
+    w_scales = rng.uniform(20, 200, nws).astype(F)
+    nas = group if by_group else 1
+    in_scales = np.full(nas, F(127) / np.abs(x).max(), F)
+    top_scales = np.full(nas, F(rng.uniform(5, 40)), F)
+    b = rng.uniform(-0.1, 0.1, outc).astype(F) if bias else None
+    if int8_in:
+        x = npref.float2int8(x * in_scales[0])
+    d = oracle.make_desc((c, h, w), outc, kernel, dilation, stride, pads, pad_value, int(bias), group, term, act, act_params)
+    return d, x, wt, b, w_scales, in_scales, top_scales
+
+
+CONV_SHAPES = [
+    # c, h, w, outc, kernel(w,h), dilation, stride, pads(l,r,t,b)
+    (3, 9, 11, 4, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (5, 8, 7, 6, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (4, 12, 10, 8, (3, 2), (2, 1), (2, 1), (2, 1, 0, 1)),
+    (2, 13, 13, 3, (5, 5), (1, 1), (2, 2), (-233, -233, -233, -233)),
+    (2, 10, 9, 3, (4, 3), (1, 2), (3, 2), (-234, -234, -234, -234)),
+    (7, 6, 6, 5, (3, 3), (1, 1), (1, 1), (0, 0, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES)
+@pytest.mark.parametrize("term,act,act_params,bias,int8_in", [
+    (1, 0, (0, 0), False, False), (2, 1, (0, 0), True, False), (101, 3, (0.0, 6.0), True, True),
+    (102, 2, (0.1, 0), True, False), (1, 6, (1 / 6.0, 0.5), True, True)])
+def test_convolution_matches_numpy(shape, term, act, act_params, bias, int8_in):
+    rng = np.random.default_rng(hash((shape, term, act)) % (2 ** 32))
+    c, h, w, outc, kernel, dilation, stride, pads = shape
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, c, h, w, outc, kernel, dilation, stride, pads, 1, term, act, act_params,
+                                           bias, int8_in, False)
+    got, gacc = oracle.convolution_int8(d, x, wt, b, ws, ins[0], tops[0], want_acc=True)
+    want, wacc = npref.conv_family(x, wt, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act,
+                                   act_params, False)
+    assert np.array_equal(gacc, wacc)
+    assert got.dtype == want.dtype and np.array_equal(got, want)
+
+
+def test_convolution_brute_force_tiny():
+    # literal definition, python loops, no shared code with either implementation
+    rng = np.random.default_rng(5)
+    c, h, w, outc = 2, 4, 5, 3
+    xq = rng.integers(-127, 128, (c, h, w)).astype(np.int8)
+    wt = rng.integers(-127, 128, (outc, c, 3, 3)).astype(np.int8)
+    d = oracle.make_desc((c, h, w), outc, (3, 3), pads=(1, 1, 1, 1), int8_scale_term=1)
+    _, acc = oracle.convolution_int8(d, xq, wt, None, np.ones(outc, F), 1.0, want_acc=True)
+    for p, i, j in itertools.product(range(outc), range(h), range(w)):
+        s = 0
+        for q, ky, kx in itertools.product(range(c), range(3), range(3)):
+            y, x_ = i + ky - 1, j + kx - 1
+            if 0 <= y < h and 0 <= x_ < w:
+                s += int(xq[q, y, x_]) * int(wt[p, q, ky, kx])
+        assert acc[p, i, j] == s
+
+
+def test_convolution_nonzero_pad_value_is_cast_to_int8_after_quantisation():
+    rng = np.random.default_rng(6)
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, 3, 6, 6, 4, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 1, 1, 0, (0, 0), False,
+                                           False, False, pad_value=3.7)
+    got, acc = oracle.convolution_int8(d, x, wt, b, ws, ins[0], want_acc=True)
+    want, wacc = npref.conv_family(x, wt, b, ws, ins, tops, 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7)
+    assert np.array_equal(acc, wacc) and np.array_equal(got, want)
+    # border byte is 3 (C cast), not quantize(3.7*scale)
+    assert acc[0, 0, 0] != npref.conv_family(x, wt, b, ws, ins, tops, 4, (3, 3), pads=(1, 1, 1, 1), pad_value=0.0)[1][0, 0, 0]
+
+
+def test_zero_weight_scale_gives_activation_of_bias():
+    rng = np.random.default_rng(7)
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, 3, 5, 5, 4, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 1, 1, 1, (0, 0), True,
+                                           False, False)
+    ws[2] = 0
+    got = oracle.convolution_int8(d, x, wt, b, ws, ins[0])
+    assert np.all(got[2] == max(b[2], 0))
+
+
+def test_1x1_convolution_equals_gemm_rows():
+    rng = np.random.default_rng(8)
+    c, h, w, outc = 16, 5, 7, 6
+    xq = rng.integers(-127, 128, (c, h, w)).astype(np.int8)
+    wt = rng.integers(-127, 128, (outc, c, 1, 1)).astype(np.int8)
+    d = oracle.make_desc((c, h, w), outc, (1, 1))
+    _, acc = oracle.convolution_int8(d, xq, wt, None, np.ones(outc, F), 1.0, want_acc=True)
+    _, gacc = oracle.gemm_int8(wt.reshape(outc, c), xq.reshape(c, h * w).T.copy(), np.ones(outc, F), [1.0], want_acc=True)
+    assert np.array_equal(acc.reshape(outc, h * w), gacc)
+
+
+# ----------------------------------------------------------------------------- depthwise / group
+@pytest.mark.parametrize("c,outc,group", [(6, 6, 6), (8, 8, 8), (6, 12, 3), (8, 4, 2), (4, 4, 1)])
+@pytest.mark.parametrize("term,act,act_params,stride,int8_in", [
+    (1, 0, (0, 0), (1, 1), False), (101, 3, (0.0, 6.0), (2, 2), True), (102, 1, (0, 0), (1, 1), False),
+    (2, 3, (0.0, 6.0), (2, 2), False)])
+def test_depthwise_and_group_match_numpy(c, outc, group, term, act, act_params, stride, int8_in):
+    rng = np.random.default_rng(hash((c, outc, group, term)) % (2 ** 32))
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, c, 9, 10, outc, (3, 3), (1, 1), stride, (1, 1, 1, 1), group, term, act,
+                                           act_params, True, int8_in, True)
+    if term in (2, 102):
+        ws[:] = ws[0]  # the layer broadcasts a single weight scale to every group
+    got, gacc = oracle.convolutiondepthwise_int8(d, x, wt, b, ws, ins, tops, want_acc=True)
+    want, wacc = npref.conv_family(x, wt, b, ws, ins, tops, outc, (3, 3), (1, 1), stride, (1, 1, 1, 1), 0.0, group, term,
+                                   act, act_params, True)
+    assert np.array_equal(gacc, wacc)
+    assert got.dtype == want.dtype and np.array_equal(got, want)
+
+
+def test_depthwise_equals_group_conv_with_group_equal_channels_and_group1_equals_conv():
+    rng = np.random.default_rng(9)
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, 4, 7, 7, 8, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 1, 1, 1, (0, 0), True,
+                                           True, True)
+    # group == 1: depthwise layer arithmetic with one scale per group must equal Convolution with that scale everywhere
+    got_dw = oracle.convolutiondepthwise_int8(d, x, wt, b, ws[:1], ins[:1], None)
+    got_cv = oracle.convolution_int8(d, x, wt, b, np.full(8, ws[0], F), ins[0])
+    assert np.array_equal(got_dw, got_cv)
+
+
+def test_invalid_group_is_rejected_with_minus_100():
+    rng = np.random.default_rng(10)
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, 6, 5, 5, 6, (3, 3), (1, 1), (1, 1), (0, 0, 0, 0), 1, 1, 0, (0, 0), False,
+                                           True, True)
+    d.group = 4
+    with pytest.raises(RuntimeError, match="-100"):
+        oracle.convolutiondepthwise_int8(d, x, wt, b, np.ones(4, F), np.ones(4, F), None)
+
+
+# ----------------------------------------------------------------------------- inner product
+@pytest.mark.parametrize("rows,num_input,num_output,act,bias,int8_in", [
+    (1, 64, 10, 0, False, False), (1, 2048, 100, 1, True, False), (5, 33, 7, 3, True, False), (3, 16, 4, 0, True, True)])
+def test_innerproduct_matches_numpy(rows, num_input, num_output, act, bias, int8_in):
+    rng = np.random.default_rng(rows * 1000 + num_input)
+    x = rng.uniform(-1, 1, (rows, num_input)).astype(F)
+    in_scale = F(127) / np.abs(x).max()
+    wt = rng.integers(-127, 128, (num_output, num_input)).astype(np.int8)
+    ws = rng.uniform(10, 20, num_output).astype(F)
+    ws[0] = 0 if num_output > 4 else ws[0]
+    b = rng.uniform(-1, 1, num_output).astype(F) if bias else None
+    if int8_in:
+        x = npref.float2int8(x * in_scale)
+    got, gacc = oracle.innerproduct_int8(x, wt, b, ws, in_scale, act, (0.0, 6.0), want_acc=True)
+    want, wacc = npref.innerproduct(x, wt, b, ws, in_scale, act, (0.0, 6.0))
+    assert np.array_equal(gacc, wacc) and np.array_equal(got, want)
+
+
+# ----------------------------------------------------------------------------- gemm int8
+def test_gemm_quantize_rows_matches_numpy_and_zero_row_scale_is_one():
+    rng = np.random.default_rng(11)
+    a = rng.normal(0, 1, (9, 77)).astype(F)
+    a[4] = 0
+    aq, s = oracle.gemm_quantize_rows(a)
+    wq, wsc = npref.gemm_quantize_rows(a)
+    assert np.array_equal(s, wsc) and np.array_equal(aq, wq)
+    assert s[4] == 1.0 and not aq[4].any()
+    assert np.abs(aq).max(axis=1)[np.arange(9) != 4].min() == 127  # absmax element maps to +-127
+
+
+def test_gemm_quantize_tensor():
+    rng = np.random.default_rng(12)
+    b = rng.normal(0, 0.02, (6, 40)).astype(F)
+    bq, s = oracle.gemm_quantize_tensor(b)
+    assert s == F(127) / np.abs(b).max()
+    assert np.array_equal(bq, npref.float2int8(b * s))
+
+
+@pytest.mark.parametrize("bt", [-1, 0, 1, 2, 3, 4])
+@pytest.mark.parametrize("alpha,beta,transpose,per_col", [(1.0, 1.0, False, False), (0.5, 2.0, True, False),
+                                                          (1.0, 1.0, False, True), (1.7, 0.3, False, True)])
+def test_gemm_int8_matches_numpy(bt, alpha, beta, transpose, per_col):
+    rng = np.random.default_rng(100 + bt)
+    m, n, k = 13, 17, 96
+    a = rng.normal(0, 1, (m, k)).astype(F)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sb = rng.uniform(50, 500, n if per_col else 1).astype(F)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    got, gacc = oracle.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose, want_acc=True)
+    want, wacc = npref.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose)
+    assert np.array_equal(gacc, wacc) and np.array_equal(got, want)
+
+
+def test_gemm_operands_are_not_transposed():
+    # asymmetric one-hot probes: acc[i][j] must be sum_k A[i][k]*B[j][k]
+    aq = np.zeros((2, 4), np.int8)
+    bq = np.zeros((3, 4), np.int8)
+    aq[1, 2] = 5
+    bq[2, 2] = -7
+    _, acc = oracle.gemm_int8(aq, bq, np.ones(2, F), [1.0], want_acc=True)
+    want = np.zeros((2, 3), np.int32)
+    want[1, 2] = -35
+    assert np.array_equal(acc, want)
+
+
+# ----------------------------------------------------------------------------- block quant
+@pytest.mark.parametrize("bits", [4, 6, 8])
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_blockquant_pack_unpack_inverse(bits, block):
+    rng = np.random.default_rng(bits * 10 + block)
+    n, k = 5, 200  # k not a multiple of any block size
+    w = rng.normal(0, 0.02, (n, k)).astype(F)
+    w[1, 64:128] = 0  # an all-zero block -> scale 1
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    q_np = npref.blockquant_unpack_all(packed, k, bits)
+    q_c = np.array([[oracle.blockquant_unpack(packed[j], kk, bits) for kk in range(k)] for j in range(n)])
+    assert np.array_equal(q_np, q_c)
+    qmax = (1 << (bits - 1)) - 1
+    assert q_c.max() <= qmax and q_c.min() >= -qmax
+    # re-deriving q from the definition (scale = qmax/absmax per block, round half away)
+    for j in range(n):
+        for bi in range((k + block - 1) // block):
+            blk = w[j, bi * block: (bi + 1) * block]
+            am = np.abs(blk).max()
+            s = F(1) if am == 0 else F(qmax) / am
+            assert scales[j, bi] == s
+            want = np.clip(npref.float2int8(blk * s).astype(int), -qmax, qmax)
+            assert np.array_equal(q_c[j, bi * block: (bi + 1) * block], want)
+
+
+def test_blockquant_unpack_known_bit_patterns():
+    # 4-bit: byte 0xF1 -> low nibble 1, high nibble -1 ; 6-bit stream 0b11_111110, 0b0000_0001 -> -2, 7
+    assert [oracle.blockquant_unpack(np.array([0xF1], np.uint8), k, 4) for k in range(2)] == [1, -1]
+    row = np.array([0b11111110, 0b00000001, 0x00], np.uint8)
+    assert [oracle.blockquant_unpack(row, k, 6) for k in range(2)] == [-2, 7]
+    assert oracle.blockquant_unpack(np.array([0x80, 0x7F], np.uint8), 0, 8) == -128
+    assert oracle.blockquant_unpack(np.array([0x80, 0x7F], np.uint8), 1, 8) == 127
+
+
+@pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
+    (8, 64, 1, 24, 256, -1, False), (8, 64, 4, 16, 200, 4, False), (4, 32, 3, 9, 100, 3, True),
+    (6, 128, 2, 7, 300, 1, True), (8, 32, 16, 8, 64, 0, False), (4, 64, 1, 5, 65, 2, False)])
+def test_blockquant_gemm_matches_float64_within_sequential_sum_error(bits, block, m, n, k, bt, in_sc):
+    rng = np.random.default_rng(bits + block + m + n + k)
+    a = rng.normal(0, 1, (m, k)).astype(F)
+    w = rng.normal(0, 0.02, (n, k)).astype(F)
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    ins = (0.75 + (np.arange(k) % 5) * 0.15).astype(F) if in_sc else None
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    got = oracle.gemm_blockquant(a, packed, scales, bits, block, ins, c, bt, 1.25, 0.5)
+    val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins, c, bt, 1.25, 0.5)
+    # sequential binary32 summation of k terms: |err| <= k * 2^-24 * sum|terms| (first-order bound)
+    assert np.all(np.abs(got - val) <= (k + 4) * 2.0 ** -24 * floor + 1e-30)
+
+
+def test_blockquant_gemm_exact_on_power_of_two_data():
+    # every product and partial sum exactly representable -> the sequential fp32 sum has no rounding
+    k, n, m = 128, 6, 2
+    rng = np.random.default_rng(3)
+    q = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    scales = np.full((n, k // 64), F(4.0), F)  # descale 0.25 exact
+    a = rng.integers(-8, 9, (m, k)).astype(F)
+    got = oracle.gemm_blockquant(a, q.view(np.uint8), scales, 8, 64)
+    want = (a.astype(np.int64) @ q.astype(np.int64).T) * 0.25
+    assert np.array_equal(got, want.astype(F))
