@@ -1,0 +1,166 @@
+/*
+ * ncnnhip -- C ABI of the MI355X (gfx950) implementation of ncnn's int8 / block-quant hot path.
+ *
+ * Plain pointers and sizes only.  Every `*_dev` / device pointer is memory obtained from
+ * ncnnhip_malloc (or any hipMalloc'd buffer); `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  All launch functions are asynchronous on `stream`, allocate
+ * nothing and never synchronise; temporaries are passed in by the caller.
+ *
+ * Return values follow ncnn's layer convention (src/layer/convolution.cpp:402-403,
+ * src/layer.cpp:69): 0 success, -100 out of memory, -1 any other failure;
+ * ncnnhip_last_error() gives the text of the last failure on the calling thread.
+ *
+ * Layouts are ncnn::Mat layouts (src/mat.h:341-381): a 3-D blob is [c][h][w] with `cstep`
+ * elements between channels, a batch adds `nstep` elements between samples, a 2-D blob is
+ * [h][w] rows.  Strides are in ELEMENTS of the pointed-to type.
+ */
+#ifndef NCNNHIP_H
+#define NCNNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* every declaration below is exported from libncnnhip.so (the library is built with hidden default visibility) */
+#pragma GCC visibility push(default)
+
+#define NCNNHIP_OK 0
+#define NCNNHIP_ERROR (-1)
+#define NCNNHIP_OOM (-100)
+
+/* ------------------------------------------------------------------ runtime plumbing
+ * Replaces what ncnn's only device back-end does through VkAllocator / VkCompute
+ * (src/net.cpp:2906-2930): buffers, one stream per Extractor, uploads and downloads. */
+int ncnnhip_init(int device);
+const char* ncnnhip_last_error(void);
+int ncnnhip_device_info(char* name, size_t name_len, int* compute_units, size_t* total_mem);
+int ncnnhip_stream_create(void** stream);
+int ncnnhip_stream_destroy(void* stream);
+int ncnnhip_stream_synchronize(void* stream);
+int ncnnhip_device_synchronize(void);
+int ncnnhip_malloc(void** dev, size_t bytes);
+int ncnnhip_free(void* dev);
+int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream);
+int ncnnhip_memcpy_d2h(void* host, const void* dev, size_t bytes, void* stream);
+int ncnnhip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+int ncnnhip_memset(void* dev, int byte, size_t bytes, void* stream);
+int ncnnhip_event_create(void** event);
+int ncnnhip_event_destroy(void* event);
+int ncnnhip_event_record(void* event, void* stream);
+int ncnnhip_event_synchronize(void* event);
+int ncnnhip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ------------------------------------------------------------------ fused activation
+ * ncnn activation_type / activation_params (src/layer/fused_activation.h:10-64):
+ * 0 none, 1 relu, 2 leaky(p0), 3 clip[p0,p1], 4 sigmoid, 5 mish, 6 hardswish(p0,p1). */
+typedef struct ncnnhip_activation
+{
+    int type;
+    float p0;
+    float p1;
+} ncnnhip_activation;
+
+/* ------------------------------------------------------------------ Quantize
+ * Quantize::forward, src/layer/quantize.cpp:48-111 (reached through quantize_to_int8,
+ * src/mat.cpp:2406-2427): y = float2int8(x * scale), one scale or one per row.
+ * rows = h of a 2-D blob or c of a 3-D blob (cols = w*h of a channel); `batch` samples. */
+int ncnnhip_quantize(const float* x_dev, size_t x_stride, size_t x_nstep, int8_t* y_dev, size_t y_stride, size_t y_nstep,
+                     int rows, int cols, int batch, const float* scales_dev, int nscales, void* stream);
+
+/* ------------------------------------------------------------------ Convolution / ConvolutionDepthWise
+ * Geometry of Convolution::load_param ids 0,1,11,2,12,3,13,4,15,14,16,18 (src/layer/convolution.cpp:18-38)
+ * plus ConvolutionDepthWise id 7 (src/layer/convolutiondepthwise.cpp:34). */
+typedef struct ncnnhip_conv_desc
+{
+    int w, h, c;    /* input blob */
+    int batch;      /* Mat.n; folded into the pixel dimension */
+    int num_output;
+    int kernel_w, kernel_h;
+    int dilation_w, dilation_h;
+    int stride_w, stride_h;
+    int pad_left, pad_right, pad_top, pad_bottom; /* raw param values incl. -233 / -234 */
+    float pad_value;                              /* border byte = (signed char)pad_value */
+    int group;                                    /* 1 for Convolution */
+} ncnnhip_conv_desc;
+
+/* Output extent after make_padding (src/layer/convolution.cpp:328-372, 412-413). */
+int ncnnhip_conv_out_shape(const ncnnhip_conv_desc* desc, int* outw, int* outh);
+
+/* Host helper used at create_pipeline: expands ncnn's scale tables to one value per output
+ * channel with the reference's own expression
+ *   scale_in[p] = w_scale == 0 ? 0 : 1.f / (in_scale * w_scale)
+ * (src/layer/convolution.cpp:476-480; per-group indexing src/layer/convolutiondepthwise.cpp:529-533).
+ * n_w_scales is num_output (Convolution, InnerProduct) or group (depthwise); n_in_scales 1 or group. */
+int ncnnhip_fold_input_scales(const float* w_scales, int n_w_scales, const float* in_scales, int n_in_scales,
+                              int num_output, float* scale_in_out);
+
+/* Convolution::forward_int8 (src/layer/convolution.cpp:383-508) and
+ * ConvolutionDepthWise::forward_int8 (src/layer/convolutiondepthwise.cpp:418-636) after input
+ * quantisation.  x is int8 [batch][c][h][w]; weight int8 [num_output][c/group][kh][kw];
+ * scale_in / bias / scale_out hold one float per OUTPUT CHANNEL (bias, scale_out may be NULL).
+ * scale_out != NULL selects the requantising epilogue (int8 output), otherwise fp32 output.
+ * acc_out (optional, may be NULL) receives the raw int32 accumulators [batch][num_output][outh*outw]. */
+int ncnnhip_conv_int8(const ncnnhip_conv_desc* desc, const int8_t* x_dev, size_t x_cstep, size_t x_nstep,
+                      const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
+                      const float* scale_out_dev, ncnnhip_activation act, void* out_dev, size_t out_cstep,
+                      size_t out_nstep, int32_t* acc_out_dev, void* stream);
+
+/* ------------------------------------------------------------------ InnerProduct
+ * InnerProduct::forward_int8 (src/layer/innerproduct.cpp:168-273) after input quantisation:
+ * x int8 [rows][num_input] -> fp32 [rows][num_output];  scale_in / bias per output channel. */
+int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output,
+                              const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
+                              ncnnhip_activation act, float* out_dev, size_t out_stride, int32_t* acc_out_dev,
+                              void* stream);
+
+/* ------------------------------------------------------------------ Gemm int8
+ * Dynamic per-row quantisation of A (src/layer/gemm.cpp:791-823): scales[i] = 127/absmax_i (1 for a
+ * zero row), aq = float2int8(a*scale). */
+int ncnnhip_gemm_quantize_rows(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_dev, size_t aq_stride,
+                               float* scales_dev, void* stream);
+/* Dynamic whole-tensor quantisation of a non-constant B (src/layer/gemm.cpp:826-860). scale_dev[0]
+ * receives 127/absmax. */
+int ncnnhip_gemm_quantize_tensor(const float* b_dev, size_t b_stride, int rows, int cols, int8_t* bq_dev,
+                                 size_t bq_stride, float* scale_dev, void* stream);
+/* Transposes used for transA=1 / transB=0 / output_transpose (src/layer/gemm.cpp:751-788, 862-882). */
+int ncnnhip_transpose_f32(const float* src_dev, size_t src_stride, int rows, int cols, float* dst_dev, size_t dst_stride,
+                          void* stream);
+int ncnnhip_transpose_s8(const int8_t* src_dev, size_t src_stride, int rows, int cols, int8_t* dst_dev, size_t dst_stride,
+                         void* stream);
+
+/* gemm_transB_int8 (src/layer/gemm.cpp:495-567): out = alpha*((float)acc / (sA_i*sB) + beta*C).
+ * aq [M][K], bq [N][K] (K contiguous).  n_b_scales == 1 is ncnn's per-tensor B scale;
+ * n_b_scales == N applies the same expression with a per-column scale (not expressible in ncnn).
+ * broadcast_type_c: -1 no C, 0 scalar, 1/2 per row, 3 [M][N] (row stride N), 4 per column. */
+int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_dev, size_t bq_stride, int M, int N, int K,
+                      const float* a_scales_dev, const float* b_scales_dev, int n_b_scales, const float* c_dev,
+                      int broadcast_type_c, float alpha, float beta, int output_transpose, float* out_dev,
+                      size_t out_stride, int32_t* acc_out_dev, void* stream);
+
+/* ------------------------------------------------------------------ block-quantised Gemm
+ * Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483): a fp32 [M][K];
+ * b packed [N][ceil(K*bits/8)] LSB-first `bits`-wide signed fields (bits 4/6/8);
+ * scales fp32 [N][ceil(K/block)] exactly as stored in the .bin (value = qmax/absmax, the kernel
+ * multiplies by 1.f/scale); in_scales optional fp32 [K]; out fp32 [M][N]. */
+int ncnnhip_gemm_blockquant(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* b_dev, int bits,
+                            int block, const float* scales_dev, const float* in_scales_dev, const float* c_dev,
+                            int broadcast_type_c, float alpha, float beta, float* out_dev, size_t out_stride,
+                            void* stream);
+
+/* Benchmark-only variant of the same contraction taking IEEE half activations (the block-quant
+ * LLM-decode configuration feeds fp16 activations; ncnn's layer itself rejects non-fp32 input,
+ * src/layer/gemm.cpp:341-345).  a is fp16 [M][K]. */
+int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* b_dev,
+                                 int bits, int block, const float* scales_dev, float* out_dev, size_t out_stride,
+                                 void* stream);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NCNNHIP_H */

@@ -1,0 +1,56 @@
+"""Build recipe for the in-tree native libraries (hipcc cross-compiles gfx950 without a GPU)."""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+LIBNCNNHIP = os.path.join(LIBDIR, "libncnnhip.so")
+
+HIP_SOURCES = ["runtime.hip", "quantize.hip", "gemm_int8.hip", "gemm_int8_pipelined.hip", "conv_int8.hip", "blockquant.hip"]
+
+# -ffp-contract=off: the reference arithmetic is separate mul and add, never FMA.
+# packed-fp32 ops are switched off for this pool's gfx950 parts.
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fvisibility=hidden",
+               "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option"]
+
+
+def _run(cmd):
+    print("+ " + " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_kernels(jobs=8):
+    os.makedirs(LIBDIR, exist_ok=True)
+    objdir = os.path.join(ROOT, "build", "obj")
+    os.makedirs(objdir, exist_ok=True)
+    procs = []
+    objs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = ["hipcc"] + HIPCC_FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
+        print("+ " + " ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd)))
+        if len(procs) >= jobs:
+            s, p = procs.pop(0)
+            if p.wait() != 0:
+                raise RuntimeError("hipcc failed on " + s)
+    for s, p in procs:
+        if p.wait() != 0:
+            raise RuntimeError("hipcc failed on " + s)
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBNCNNHIP] + objs)
+    return LIBNCNNHIP
+
+
+def build_all():
+    build_kernels()
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built", LIBNCNNHIP)
+    sys.exit(0)

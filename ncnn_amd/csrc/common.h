@@ -1,0 +1,121 @@
+// Shared host/device helpers for the gfx950 kernels.
+#ifndef NCNNHIP_COMMON_H
+#define NCNNHIP_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "ncnnhip.h"
+
+namespace ncnnhip {
+
+// ---- error plumbing (host) --------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int map_hip_error(hipError_t e, const char* what);
+
+#define NCNNHIP_CHECK(expr)                                          \
+    do                                                               \
+    {                                                                \
+        hipError_t _e = (expr);                                      \
+        if (_e != hipSuccess) return ::ncnnhip::map_hip_error(_e, #expr); \
+    } while (0)
+
+#define NCNNHIP_REQUIRE(cond, ...)                \
+    do                                            \
+    {                                             \
+        if (!(cond))                              \
+        {                                         \
+            ::ncnnhip::set_error(__VA_ARGS__);    \
+            return NCNNHIP_ERROR;                 \
+        }                                         \
+    } while (0)
+
+static inline hipStream_t as_stream(void* s)
+{
+    return reinterpret_cast<hipStream_t>(s);
+}
+
+static inline int launch_status(const char* what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return map_hip_error(e, what);
+    return NCNNHIP_OK;
+}
+
+// ---- device arithmetic: every float op is a single rounded IEEE binary32 op -------------
+// (the intrinsics keep the compiler from contracting mul+add into an FMA)
+
+__device__ __forceinline__ float mul_rn(float a, float b)
+{
+    return __fmul_rn(a, b);
+}
+__device__ __forceinline__ float add_rn(float a, float b)
+{
+    return __fadd_rn(a, b);
+}
+__device__ __forceinline__ float div_rn(float a, float b)
+{
+    return __fdiv_rn(a, b);
+}
+
+// round half away from zero, saturate to [-127,127]; NaN and |v| >= 2^31 give -127 like the
+// x86 float->int conversion the reference runs on (INT_MIN, then clamped).
+__device__ __forceinline__ int float2int8(float v)
+{
+    float r = roundf(v);
+    if (!(fabsf(r) < 2147483648.f)) return -127;
+    int q = (int)r;
+    q = q > 127 ? 127 : q;
+    q = q < -127 ? -127 : q;
+    return q;
+}
+
+__device__ __forceinline__ float apply_activation(float v, const ncnnhip_activation& a)
+{
+    switch (a.type)
+    {
+    case 1:
+        v = fmaxf(v, 0.f);
+        break;
+    case 2:
+        v = v > 0.f ? v : mul_rn(v, a.p0);
+        break;
+    case 3:
+        if (v < a.p0) v = a.p0;
+        if (v > a.p1) v = a.p1;
+        break;
+    case 4:
+        v = fminf(v, 88.3762626647949f);
+        v = fmaxf(v, -88.3762626647949f);
+        v = div_rn(1.f, add_rn(1.f, expf(-v)));
+        break;
+    case 5:
+        v = mul_rn(v, tanhf(logf(add_rn(expf(v), 1.f))));
+        break;
+    case 6:
+    {
+        float lower = div_rn(-a.p1, a.p0);
+        float upper = add_rn(div_rn(1.f, a.p0), lower);
+        if (v < lower)
+            v = 0.f;
+        else if (v > upper)
+            ;
+        else
+            v = mul_rn(v, add_rn(mul_rn(v, a.p0), a.p1));
+        break;
+    }
+    default:
+        break;
+    }
+    return v;
+}
+
+static inline int ceil_div(long long a, long long b)
+{
+    return (int)((a + b - 1) / b);
+}
+
+} // namespace ncnnhip
+
+#endif // NCNNHIP_COMMON_H

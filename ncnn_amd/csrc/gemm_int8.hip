@@ -1,0 +1,144 @@
+// int8 Gemm and InnerProduct launchers on top of the MFMA tile contraction.
+#include "epilogues.h"
+#include "mfma_tile.h"
+
+namespace ncnnhip {
+
+template<int BM, int BN, typename Epilogue>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(DenseOperand a, DenseOperand b, Epilogue epi, int M, int N, int K)
+{
+    mfma_tile_body<BM, BN, DenseOperand, Epilogue>(a, b, epi, M, N, K, blockIdx.y * BM, blockIdx.x * BN);
+}
+
+// skinny case (one or a few activation rows): one wavefront per output channel streams the
+// weight row with 16-byte loads and reduces with cross-lane adds; no matrix cores involved.
+__global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__ x, size_t xs, int rows, int K,
+                                                       const int8_t* __restrict__ wgt, int num_output, FcEpilogue epi, int vec)
+{
+    const int lane = threadIdx.x & 63;
+    const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (p >= num_output) return;
+    const int8_t* wr = wgt + (size_t)p * K;
+    for (int r = 0; r < rows; r++)
+    {
+        const int8_t* xr = x + (size_t)r * xs;
+        int acc = 0;
+        if (vec)
+        {
+            for (int k = lane * 16; k + 16 <= K; k += 64 * 16)
+            {
+                const v4i wv = *reinterpret_cast<const v4i*>(wr + k);
+                const v4i xv = *reinterpret_cast<const v4i*>(xr + k);
+#pragma unroll
+                for (int d = 0; d < 4; d++) acc = __builtin_amdgcn_sdot4(wv[d], xv[d], acc, false);
+            }
+            for (int k = (K & ~15) + lane; k < K; k += 64) acc += (int)wr[k] * (int)xr[k];
+        }
+        else
+        {
+            for (int k = lane; k < K; k += 64) acc += (int)wr[k] * (int)xr[k];
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        if (lane == 0) epi(p, r, acc);
+    }
+}
+
+static inline bool aligned16(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+static DenseOperand make_dense(const int8_t* base, size_t stride, int rows, int K)
+{
+    DenseOperand d;
+    d.base = base;
+    d.stride = stride;
+    d.rows = rows;
+    d.K = K;
+    d.vec = aligned16(base) && stride % 16 == 0;
+    return d;
+}
+
+int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K,
+                               const GemmEpilogue& epi, hipStream_t stream, bool* handled);
+
+} // namespace ncnnhip
+
+using namespace ncnnhip;
+
+extern "C" {
+
+int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_dev, size_t bq_stride, int M, int N, int K,
+                      const float* a_scales_dev, const float* b_scales_dev, int n_b_scales, const float* c_dev,
+                      int broadcast_type_c, float alpha, float beta, int output_transpose, float* out_dev,
+                      size_t out_stride, int32_t* acc_out_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(aq_dev && bq_dev && a_scales_dev && b_scales_dev && out_dev, "ncnnhip_gemm_int8: null pointer");
+    NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1, "ncnnhip_gemm_int8: bad shape %d %d %d", M, N, K);
+    NCNNHIP_REQUIRE(aq_stride >= (size_t)K && bq_stride >= (size_t)K, "ncnnhip_gemm_int8: operand stride below K");
+    NCNNHIP_REQUIRE(n_b_scales == 1 || n_b_scales == N, "ncnnhip_gemm_int8: %d B scales for N=%d", n_b_scales, N);
+    NCNNHIP_REQUIRE(broadcast_type_c >= -1 && broadcast_type_c <= 4, "ncnnhip_gemm_int8: broadcast_type_c %d", broadcast_type_c);
+    NCNNHIP_REQUIRE(broadcast_type_c < 0 || c_dev, "ncnnhip_gemm_int8: C pointer missing");
+    NCNNHIP_REQUIRE(out_stride >= (size_t)(output_transpose ? M : N), "ncnnhip_gemm_int8: output stride too small");
+
+    GemmEpilogue epi;
+    epi.a_scales = a_scales_dev;
+    epi.b_scales = b_scales_dev;
+    epi.per_col = n_b_scales != 1;
+    epi.c = c_dev;
+    epi.bt = c_dev ? broadcast_type_c : -1;
+    epi.alpha = alpha;
+    epi.beta = beta;
+    epi.transpose = output_transpose;
+    epi.out = out_dev;
+    epi.out_stride = out_stride;
+    epi.N = N;
+    epi.acc_out = acc_out_dev;
+
+    bool handled = false;
+    int ret = launch_gemm_int8_pipelined(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, epi, as_stream(stream), &handled);
+    if (handled) return ret;
+
+    DenseOperand a = make_dense(aq_dev, aq_stride, M, K);
+    DenseOperand b = make_dense(bq_dev, bq_stride, N, K);
+    dim3 grid(ceil_div(N, 128), ceil_div(M, 128));
+    NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_gemm_int8: M too large");
+    hipLaunchKernelGGL((gemm_tile_kernel<128, 128, GemmEpilogue>), grid, dim3(256), 0, as_stream(stream), a, b, epi, M, N, K);
+    return launch_status("gemm_tile_kernel");
+}
+
+int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output,
+                              const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
+                              ncnnhip_activation act, float* out_dev, size_t out_stride, int32_t* acc_out_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(x_dev && weight_dev && scale_in_dev && out_dev, "ncnnhip_innerproduct_int8: null pointer");
+    NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1, "ncnnhip_innerproduct_int8: bad shape");
+    NCNNHIP_REQUIRE(x_stride >= (size_t)num_input && out_stride >= (size_t)num_output, "ncnnhip_innerproduct_int8: stride too small");
+
+    FcEpilogue epi;
+    epi.scale_in = scale_in_dev;
+    epi.bias = bias_dev;
+    epi.act = act;
+    epi.out = out_dev;
+    epi.out_stride = out_stride;
+    epi.num_output = num_output;
+    epi.acc_out = acc_out_dev;
+
+    if (rows <= 8)
+    {
+        const int vec = aligned16(x_dev) && aligned16(weight_dev) && x_stride % 16 == 0 && num_input % 16 == 0;
+        hipLaunchKernelGGL(fc_gemv_kernel, dim3(ceil_div(num_output, 4)), dim3(256), 0, as_stream(stream), x_dev, x_stride, rows,
+                           num_input, weight_dev, num_output, epi, vec);
+        return launch_status("fc_gemv_kernel");
+    }
+
+    DenseOperand a = make_dense(weight_dev, (size_t)num_input, num_output, num_input);
+    DenseOperand b = make_dense(x_dev, x_stride, rows, num_input);
+    dim3 grid(ceil_div(rows, 64), ceil_div(num_output, 128));
+    NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_innerproduct_int8: num_output too large");
+    hipLaunchKernelGGL((gemm_tile_kernel<128, 64, FcEpilogue>), grid, dim3(256), 0, as_stream(stream), a, b, epi, num_output, rows, num_input);
+    return launch_status("gemm_tile_kernel<fc>");
+}
+
+} // extern "C"

@@ -1,0 +1,174 @@
+// Device plumbing behind the C ABI: buffers, streams, events, error text.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace ncnnhip {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int map_hip_error(hipError_t e, const char* what)
+{
+    set_error("%s: %s", what, hipGetErrorString(e));
+    (void)hipGetLastError(); // clear the sticky per-thread error
+    return e == hipErrorOutOfMemory ? NCNNHIP_OOM : NCNNHIP_ERROR;
+}
+
+} // namespace ncnnhip
+
+using namespace ncnnhip;
+
+extern "C" {
+
+int ncnnhip_init(int device)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+    {
+        set_error("no HIP device available (%s)", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        (void)hipGetLastError();
+        return NCNNHIP_ERROR;
+    }
+    NCNNHIP_REQUIRE(device >= 0 && device < count, "device %d out of range (count %d)", device, count);
+    NCNNHIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    NCNNHIP_CHECK(hipGetDeviceProperties(&prop, device));
+    NCNNHIP_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, "kernels are built for gfx950 only, device is %s",
+                    prop.gcnArchName);
+    return NCNNHIP_OK;
+}
+
+const char* ncnnhip_last_error(void)
+{
+    return g_error;
+}
+
+int ncnnhip_device_info(char* name, size_t name_len, int* compute_units, size_t* total_mem)
+{
+    int dev = 0;
+    NCNNHIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    NCNNHIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (name && name_len)
+    {
+        snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (total_mem) *total_mem = prop.totalGlobalMem;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_stream_create(void** stream)
+{
+    NCNNHIP_REQUIRE(stream, "null stream out pointer");
+    hipStream_t s;
+    NCNNHIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_stream_destroy(void* stream)
+{
+    if (stream) NCNNHIP_CHECK(hipStreamDestroy(as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_stream_synchronize(void* stream)
+{
+    NCNNHIP_CHECK(hipStreamSynchronize(as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_device_synchronize(void)
+{
+    NCNNHIP_CHECK(hipDeviceSynchronize());
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_malloc(void** dev, size_t bytes)
+{
+    NCNNHIP_REQUIRE(dev, "null out pointer");
+    *dev = 0;
+    if (bytes == 0) bytes = 4;
+    NCNNHIP_CHECK(hipMalloc(dev, bytes));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_free(void* dev)
+{
+    if (dev) NCNNHIP_CHECK(hipFree(dev));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream)
+{
+    if (bytes == 0) return NCNNHIP_OK;
+    NCNNHIP_CHECK(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_memcpy_d2h(void* host, const void* dev, size_t bytes, void* stream)
+{
+    if (bytes == 0) return NCNNHIP_OK;
+    NCNNHIP_CHECK(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream)
+{
+    if (bytes == 0) return NCNNHIP_OK;
+    NCNNHIP_CHECK(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_memset(void* dev, int byte, size_t bytes, void* stream)
+{
+    if (bytes == 0) return NCNNHIP_OK;
+    NCNNHIP_CHECK(hipMemsetAsync(dev, byte, bytes, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_event_create(void** event)
+{
+    NCNNHIP_REQUIRE(event, "null out pointer");
+    hipEvent_t e;
+    NCNNHIP_CHECK(hipEventCreate(&e));
+    *event = e;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_event_destroy(void* event)
+{
+    if (event) NCNNHIP_CHECK(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_event_record(void* event, void* stream)
+{
+    NCNNHIP_CHECK(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_event_synchronize(void* event)
+{
+    NCNNHIP_CHECK(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    NCNNHIP_CHECK(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+    return NCNNHIP_OK;
+}
+
+} // extern "C"

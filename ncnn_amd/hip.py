@@ -1,0 +1,312 @@
+"""ctypes signatures for include/ncnnhip.h plus a thin numpy <-> device-buffer convenience layer."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_PKG, "lib", "libncnnhip.so")
+
+c_void_pp = C.POINTER(C.c_void_p)
+
+
+class NcnnHipError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("ncnnhip error %d: %s" % (code, text))
+        self.code = code
+
+
+class Activation(C.Structure):
+    _fields_ = [("type", C.c_int), ("p0", C.c_float), ("p1", C.c_float)]
+
+    @classmethod
+    def make(cls, act_type=0, params=(0.0, 0.0)):
+        p = list(params) + [0.0, 0.0]
+        return cls(int(act_type), float(p[0]), float(p[1]))
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("w", "h", "c", "batch", "num_output", "kernel_w", "kernel_h", "dilation_w", "dilation_h",
+                                       "stride_w", "stride_h", "pad_left", "pad_right", "pad_top", "pad_bottom")] + \
+               [("pad_value", C.c_float), ("group", C.c_int)]
+
+
+def library_path():
+    return _LIB
+
+
+_SIGNATURES = {
+    "ncnnhip_init": [C.c_int],
+    "ncnnhip_device_info": [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_size_t)],
+    "ncnnhip_stream_create": [c_void_pp],
+    "ncnnhip_stream_destroy": [C.c_void_p],
+    "ncnnhip_stream_synchronize": [C.c_void_p],
+    "ncnnhip_device_synchronize": [],
+    "ncnnhip_malloc": [c_void_pp, C.c_size_t],
+    "ncnnhip_free": [C.c_void_p],
+    "ncnnhip_memcpy_h2d": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_memcpy_d2h": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_memcpy_d2d": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_memset": [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p],
+    "ncnnhip_event_create": [c_void_pp],
+    "ncnnhip_event_destroy": [C.c_void_p],
+    "ncnnhip_event_record": [C.c_void_p, C.c_void_p],
+    "ncnnhip_event_synchronize": [C.c_void_p],
+    "ncnnhip_event_elapsed_ms": [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)],
+    "ncnnhip_quantize": [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int,
+                         C.c_void_p, C.c_int, C.c_void_p],
+    "ncnnhip_conv_out_shape": [C.POINTER(ConvDesc), C.POINTER(C.c_int), C.POINTER(C.c_int)],
+    "ncnnhip_fold_input_scales": [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
+    "ncnnhip_conv_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                          Activation, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
+                                  C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_quantize_tensor": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_transpose_f32": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_transpose_s8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_int8": [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
+                          C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_blockquant": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_blockquant_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                     C.c_void_p, C.c_size_t, C.c_void_p],
+}
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["ncnnhip_last_error"])
+
+_lib = None
+
+
+def lib():
+    """Loads libncnnhip.so.  Raises if it has not been built -- there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise NcnnHipError(-1, "%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                                   "(or python ncnn_amd/build.py) first" % _LIB)
+        _lib = C.CDLL(_LIB)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(_lib, name)
+            fn.argtypes = argtypes
+            fn.restype = C.c_int
+        _lib.ncnnhip_last_error.restype = C.c_char_p
+        _lib.ncnnhip_last_error.argtypes = []
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise NcnnHipError(code, lib().ncnnhip_last_error().decode("utf-8", "replace"))
+
+
+class DeviceBuffer:
+    """A hipMalloc'd buffer with the numpy shape/dtype it mirrors."""
+
+    def __init__(self, nbytes, shape=None, dtype=np.uint8):
+        self.ptr = C.c_void_p()
+        self.nbytes = int(nbytes)
+        self.shape = shape
+        self.dtype = np.dtype(dtype)
+        check(lib().ncnnhip_malloc(C.byref(self.ptr), self.nbytes))
+
+    @classmethod
+    def from_numpy(cls, arr, stream=None):
+        arr = np.ascontiguousarray(arr)
+        buf = cls(arr.nbytes, arr.shape, arr.dtype)
+        check(lib().ncnnhip_memcpy_h2d(buf.ptr, arr.ctypes.data_as(C.c_void_p), arr.nbytes, stream))
+        check(lib().ncnnhip_stream_synchronize(stream))
+        return buf
+
+    @classmethod
+    def empty(cls, shape, dtype):
+        shape = tuple(int(s) for s in np.atleast_1d(shape))
+        return cls(int(np.prod(shape)) * np.dtype(dtype).itemsize, shape, dtype)
+
+    def to_numpy(self, stream=None):
+        out = np.empty(self.shape, self.dtype)
+        check(lib().ncnnhip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), self.ptr, out.nbytes, stream))
+        check(lib().ncnnhip_stream_synchronize(stream))
+        return out
+
+    def fill_bytes(self, byte, stream=None):
+        check(lib().ncnnhip_memset(self.ptr, int(byte), self.nbytes, stream))
+
+    def free(self):
+        if self.ptr:
+            lib().ncnnhip_free(self.ptr)
+            self.ptr = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _ptr(buf):
+    if buf is None:
+        return None
+    return buf.ptr if isinstance(buf, DeviceBuffer) else buf
+
+
+class Runtime:
+    """Numpy-in / numpy-out convenience calls; each uploads its operands, launches on one stream and
+    downloads the result.  Used by the tests and the smoke check; the benchmark drives the C ABI directly."""
+
+    def __init__(self, device=0):
+        check(lib().ncnnhip_init(device))
+        self.stream = C.c_void_p()
+        check(lib().ncnnhip_stream_create(C.byref(self.stream)))
+
+    def sync(self):
+        check(lib().ncnnhip_stream_synchronize(self.stream))
+
+    def device_info(self):
+        name = C.create_string_buffer(128)
+        cu, mem = C.c_int(), C.c_size_t()
+        check(lib().ncnnhip_device_info(name, 128, C.byref(cu), C.byref(mem)))
+        return name.value.decode(), cu.value, mem.value
+
+    def up(self, arr):
+        return None if arr is None else DeviceBuffer.from_numpy(arr, self.stream)
+
+    # -- Quantize -------------------------------------------------------------------------
+    def quantize(self, x, scales):
+        x = np.ascontiguousarray(x, np.float32)
+        scales = np.ascontiguousarray(np.atleast_1d(scales), np.float32)
+        rows, cols = x.shape
+        dx, ds = self.up(x), self.up(scales)
+        dy = DeviceBuffer.empty((rows, cols), np.int8)
+        check(lib().ncnnhip_quantize(dx.ptr, cols, 0, dy.ptr, cols, 0, rows, cols, 1, ds.ptr, scales.size, self.stream))
+        return dy.to_numpy(self.stream)
+
+    # -- Convolution / ConvolutionDepthWise -------------------------------------------------
+    def fold_input_scales(self, w_scales, in_scales, num_output):
+        w_scales = np.ascontiguousarray(np.atleast_1d(w_scales), np.float32)
+        in_scales = np.ascontiguousarray(np.atleast_1d(in_scales), np.float32)
+        out = np.empty(num_output, np.float32)
+        check(lib().ncnnhip_fold_input_scales(w_scales.ctypes.data, w_scales.size, in_scales.ctypes.data, in_scales.size,
+                                              num_output, out.ctypes.data))
+        return out
+
+    def conv_layer(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
+                   pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), want_acc=False):
+        """Whole forward_int8 of Convolution (group == 1, per-output-channel weight scales) or
+        ConvolutionDepthWise (scale tables with `group` entries): x is [c][h][w] or [n][c][h][w], fp32 or int8."""
+        x = np.ascontiguousarray(x)
+        if x.ndim == 3:
+            x = x[None]
+        n, c, h, w = x.shape
+        d = ConvDesc(w, h, c, n, num_output, kernel[0], kernel[1], dilation[0], dilation[1], stride[0], stride[1],
+                     pads[0], pads[1], pads[2], pads[3], float(pad_value), group)
+        ow, oh = C.c_int(), C.c_int()
+        check(lib().ncnnhip_conv_out_shape(C.byref(d), C.byref(ow), C.byref(oh)))
+        ow, oh = ow.value, oh.value
+        w_scales = np.atleast_1d(np.asarray(w_scales, np.float32))
+        in_scales = np.atleast_1d(np.asarray(in_scales, np.float32))
+        scale_in = self.fold_input_scales(w_scales, in_scales, num_output)
+        cstep, nstep = h * w, c * h * w
+        if x.dtype == np.int8:
+            dxq = self.up(x)
+        else:
+            per_channel = np.repeat(in_scales, c // in_scales.size).astype(np.float32) if in_scales.size > 1 else in_scales
+            dx, dsc = self.up(x.astype(np.float32)), self.up(per_channel)
+            dxq = DeviceBuffer.empty(x.shape, np.int8)
+            check(lib().ncnnhip_quantize(dx.ptr, cstep, nstep, dxq.ptr, cstep, nstep, c, cstep, n, dsc.ptr, per_channel.size, self.stream))
+        requant = term > 100
+        scale_out = None
+        if requant:
+            ts = np.atleast_1d(np.asarray(top_scales, np.float32))
+            scale_out = np.repeat(ts, num_output // ts.size).astype(np.float32)
+        dw_, dsi, db, dso = self.up(np.asarray(weight, np.int8)), self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32)), self.up(scale_out)
+        dout = DeviceBuffer.empty((n, num_output, oh, ow), np.int8 if requant else np.float32)
+        dacc = DeviceBuffer.empty((n, num_output, oh, ow), np.int32) if want_acc else None
+        check(lib().ncnnhip_conv_int8(C.byref(d), dxq.ptr, cstep, nstep, dw_.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params),
+                                      dout.ptr, oh * ow, num_output * oh * ow, _ptr(dacc), self.stream))
+        out = dout.to_numpy(self.stream)
+        if want_acc:
+            return out, dacc.to_numpy(self.stream)
+        return out
+
+    # -- InnerProduct -------------------------------------------------------------------------
+    def innerproduct_layer(self, x, weight, bias, w_scales, in_scale, act=0, act_params=(0.0, 0.0), want_acc=False):
+        x = np.ascontiguousarray(x)
+        rows, k = x.shape
+        weight = np.ascontiguousarray(weight, np.int8)
+        num_output = weight.shape[0]
+        scale_in = self.fold_input_scales(w_scales, [in_scale], num_output)
+        if x.dtype == np.int8:
+            dxq = self.up(x)
+        else:
+            dx, dsc = self.up(x.astype(np.float32)), self.up(np.asarray([in_scale], np.float32))
+            dxq = DeviceBuffer.empty((rows, k), np.int8)
+            check(lib().ncnnhip_quantize(dx.ptr, k, 0, dxq.ptr, k, 0, rows, k, 1, dsc.ptr, 1, self.stream))
+        dw_, dsi, db = self.up(weight), self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32))
+        dout = DeviceBuffer.empty((rows, num_output), np.float32)
+        dacc = DeviceBuffer.empty((rows, num_output), np.int32) if want_acc else None
+        check(lib().ncnnhip_innerproduct_int8(dxq.ptr, k, rows, k, num_output, dw_.ptr, dsi.ptr, _ptr(db), Activation.make(act, act_params),
+                                              dout.ptr, num_output, _ptr(dacc), self.stream))
+        out = dout.to_numpy(self.stream)
+        return (out, dacc.to_numpy(self.stream)) if want_acc else out
+
+    # -- Gemm int8 ----------------------------------------------------------------------------
+    def gemm_quantize_rows(self, a):
+        a = np.ascontiguousarray(a, np.float32)
+        m, k = a.shape
+        da = self.up(a)
+        daq, ds = DeviceBuffer.empty((m, k), np.int8), DeviceBuffer.empty((m,), np.float32)
+        check(lib().ncnnhip_gemm_quantize_rows(da.ptr, k, m, k, daq.ptr, k, ds.ptr, self.stream))
+        return daq.to_numpy(self.stream), ds.to_numpy(self.stream)
+
+    def gemm_quantize_tensor(self, b):
+        b = np.ascontiguousarray(b, np.float32)
+        n, k = b.shape
+        db = self.up(b)
+        dbq, ds = DeviceBuffer.empty((n, k), np.int8), DeviceBuffer.empty((1,), np.float32)
+        check(lib().ncnnhip_gemm_quantize_tensor(db.ptr, k, n, k, dbq.ptr, k, ds.ptr, self.stream))
+        return dbq.to_numpy(self.stream), ds.to_numpy(self.stream)[0]
+
+    def gemm_int8(self, aq, bq, a_scales, b_scales, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, output_transpose=False,
+                  want_acc=False):
+        aq, bq = np.ascontiguousarray(aq, np.int8), np.ascontiguousarray(bq, np.int8)
+        m, k = aq.shape
+        n = bq.shape[0]
+        b_scales = np.ascontiguousarray(np.atleast_1d(b_scales), np.float32)
+        daq, dbq, dsa, dsb = self.up(aq), self.up(bq), self.up(np.asarray(a_scales, np.float32)), self.up(b_scales)
+        dc = self.up(None if c is None else np.asarray(c, np.float32))
+        oshape = (n, m) if output_transpose else (m, n)
+        dout = DeviceBuffer.empty(oshape, np.float32)
+        dacc = DeviceBuffer.empty((m, n), np.int32) if want_acc else None
+        check(lib().ncnnhip_gemm_int8(daq.ptr, k, dbq.ptr, k, m, n, k, dsa.ptr, dsb.ptr, b_scales.size, _ptr(dc),
+                                      broadcast_type_c if c is not None else -1, alpha, beta, int(output_transpose), dout.ptr,
+                                      oshape[1], _ptr(dacc), self.stream))
+        out = dout.to_numpy(self.stream)
+        return (out, dacc.to_numpy(self.stream)) if want_acc else out
+
+    def transpose(self, a):
+        a = np.ascontiguousarray(a)
+        r, c_ = a.shape
+        da = self.up(a)
+        dt = DeviceBuffer.empty((c_, r), a.dtype)
+        fn = lib().ncnnhip_transpose_f32 if a.dtype == np.float32 else lib().ncnnhip_transpose_s8
+        check(fn(da.ptr, c_, r, c_, dt.ptr, r, self.stream))
+        return dt.to_numpy(self.stream)
+
+    # -- block-quantised Gemm -----------------------------------------------------------------
+    def gemm_blockquant(self, a, b_packed, scales, bits, block, in_scales=None, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0):
+        m, k = a.shape
+        b_packed = np.ascontiguousarray(b_packed, np.uint8)
+        n = b_packed.shape[0]
+        half = a.dtype == np.float16
+        da = self.up(np.ascontiguousarray(a, np.float16 if half else np.float32))
+        db, ds = self.up(b_packed), self.up(np.asarray(scales, np.float32))
+        dout = DeviceBuffer.empty((m, n), np.float32)
+        if half:
+            check(lib().ncnnhip_gemm_blockquant_f16a(da.ptr, k, m, n, k, db.ptr, bits, block, ds.ptr, dout.ptr, n, self.stream))
+        else:
+            dis = self.up(None if in_scales is None else np.asarray(in_scales, np.float32))
+            dc = self.up(None if c is None else np.asarray(c, np.float32))
+            check(lib().ncnnhip_gemm_blockquant(da.ptr, k, m, n, k, db.ptr, bits, block, ds.ptr, _ptr(dis), _ptr(dc),
+                                                broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
+        return dout.to_numpy(self.stream)

@@ -1,0 +1,275 @@
+"""GPU parity: every C-ABI launch against the CPU oracle on identical seeded inputs.
+
+int32 accumulators and requantised int8 outputs must be bit-exact.  fp32 outputs of the integer
+layers are produced by the same sequence of single fp32 operations as the reference, so they are
+required to be bit-exact too (stricter than the 1e-5 relative the task allows).  The block-quant
+Gemm accumulates in a different order than the reference's sequential sum and is held to
+|gpu - ref| <= 1e-5 * sum_k |a_k * w_k|.
+"""
+import numpy as np
+import pytest
+
+import cases
+import npref
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def rt():
+    import ncnn_amd
+    return ncnn_amd.Runtime(0)
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ----------------------------------------------------------------------------- quantize
+def test_quantize_matches_oracle(rt):
+    rng = np.random.default_rng(0)
+    for rows, cols in ((1, 5), (3, 1024), (7, 1031), (64, 3136)):
+        _say("quantize", rows, cols)
+        x = rng.uniform(-3, 3, (rows, cols)).astype(F)
+        x.flat[:8] = [0.5, -0.5, 1.5, -1.5, 0.49999997, 126.5, 1e9, -1e9][: min(8, x.size)]
+        for scales in (rng.uniform(5, 60, rows).astype(F), np.array([F(42.3)])):
+            assert np.array_equal(rt.quantize(x, scales), oracle.quantize(x, scales))
+    special = np.array([[np.nan, np.inf, -np.inf, 3e9, -3e9, 127.5, -127.5, 0.0]], F)
+    assert np.array_equal(rt.quantize(special, [1.0]), oracle.quantize(special, [1.0]))
+
+
+# ----------------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("m,k", [(5, 77), (9, 4096), (16, 4100), (33, 513)])
+def test_gemm_quantize_rows(rt, m, k):
+    _say("gemm_quantize_rows", m, k)
+    a = np.random.default_rng(m * k).standard_normal((m, k), dtype=F)
+    a[m // 2] = 0
+    gq, gs = rt.gemm_quantize_rows(a)
+    oq, os_ = oracle.gemm_quantize_rows(a)
+    assert np.array_equal(gs, os_) and np.array_equal(gq, oq)
+
+
+def test_gemm_quantize_tensor(rt):
+    b = (np.random.default_rng(3).standard_normal((37, 129), dtype=F) * F(0.02)).astype(F)
+    gq, gs = rt.gemm_quantize_tensor(b)
+    oq, os_ = oracle.gemm_quantize_tensor(b)
+    assert gs == os_ and np.array_equal(gq, oq)
+
+
+def test_transposes(rt):
+    rng = np.random.default_rng(4)
+    a = rng.standard_normal((45, 70), dtype=F)
+    assert np.array_equal(rt.transpose(a), a.T)
+    q = rng.integers(-127, 128, (33, 129)).astype(np.int8)
+    assert np.array_equal(rt.transpose(q), q.T)
+
+
+GEMM_SHAPES = [(13, 17, 96), (1, 1, 1), (128, 128, 64), (130, 257, 100), (64, 300, 77), (256, 512, 1024), (300, 200, 4100)]
+
+
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+@pytest.mark.parametrize("bt,alpha,beta,transpose,per_col", [(-1, 1.0, 1.0, False, False), (4, 1.0, 1.0, False, False),
+                                                             (3, 0.5, 2.0, True, False), (1, 1.7, 0.3, False, True),
+                                                             (0, 1.0, 1.0, False, True), (2, 1.0, -1.0, True, True)])
+def test_gemm_int8_bit_exact(rt, shape, bt, alpha, beta, transpose, per_col):
+    m, n, k = shape
+    _say("gemm_int8", shape, bt, alpha, beta, transpose, per_col)
+    a, bq, sb, _ = cases.gemm_case(m * 31 + n * 7 + k, m, n, k, per_col)
+    rng = np.random.default_rng(bt + 10)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    want, wacc = oracle.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose, want_acc=True)
+    got, gacc = rt.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose, want_acc=True)
+    assert np.array_equal(gacc, wacc)
+    assert np.array_equal(got, want)
+
+
+def test_gemm_int8_1024_cube_against_numpy_int_matmul(rt):
+    # one of the benchmark's own sizes; the accumulators are checked against an exact integer matmul
+    m = n = k = 1024
+    _say("gemm_int8 1024^3")
+    a, bq, sb, bias = cases.gemm_case(1024, m, n, k)
+    aq, sa = rt.gemm_quantize_rows(a)
+    oq, os_ = oracle.gemm_quantize_rows(a)
+    assert np.array_equal(aq, oq) and np.array_equal(sa, os_)
+    got, gacc = rt.gemm_int8(aq, bq, sa, sb, bias, 4, want_acc=True)
+    want, wacc = npref.gemm_int8(aq, bq, sa, sb, bias, 4)
+    assert np.array_equal(gacc, wacc)
+    assert np.array_equal(got, want)
+
+
+# ----------------------------------------------------------------------------- convolution
+CONV_CASES = [
+    # c, h, w, outc, kernel, dilation, stride, pads
+    (3, 9, 11, 4, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (5, 8, 7, 6, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (4, 12, 10, 8, (3, 2), (2, 1), (2, 1), (2, 1, 0, 1)),
+    (2, 13, 13, 3, (5, 5), (1, 1), (2, 2), (-233, -233, -233, -233)),
+    (2, 10, 9, 3, (4, 3), (1, 2), (3, 2), (-234, -234, -234, -234)),
+    (16, 20, 20, 130, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (64, 14, 14, 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (96, 7, 7, 200, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("shape", CONV_CASES)
+@pytest.mark.parametrize("term,act,act_params,bias,int8_in", [
+    (1, 1, (0, 0), True, False), (2, 0, (0, 0), False, False), (101, 3, (0.0, 6.0), True, True), (102, 2, (0.1, 0), True, False),
+    (1, 6, (1 / 6.0, 0.5), True, True)])
+def test_convolution_bit_exact(rt, shape, term, act, act_params, bias, int8_in):
+    c, h, w, outc, kernel, dilation, stride, pads = shape
+    _say("conv", shape, term, act, bias, int8_in)
+    x, wq, b, ws, ins, tops = cases.conv_case(c * 100 + outc + term, c, h, w, outc, kernel, 1, term, bias, int8_in)
+    d = oracle.make_desc((c, h, w), outc, kernel, dilation, stride, pads, 0.0, int(bias), 1, term, act, act_params)
+    want, wacc = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0], None if tops is None else tops[0], want_acc=True)
+    got, gacc = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act, act_params, want_acc=True)
+    assert np.array_equal(gacc[0], wacc)
+    assert got.dtype == want.dtype and np.array_equal(got[0], want)
+
+
+def test_convolution_nonzero_pad_value(rt):
+    x, wq, b, ws, ins, tops = cases.conv_case(5, 3, 6, 6, 4, (3, 3))
+    d = oracle.make_desc((3, 6, 6), 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7, bias_term=1)
+    want = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0])
+    got = rt.conv_layer(x[0], wq, b, ws, ins, None, 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7)
+    assert np.array_equal(got[0], want)
+
+
+def test_convolution_zero_weight_scale(rt):
+    x, wq, b, ws, ins, tops = cases.conv_case(6, 8, 6, 6, 5, (3, 3))
+    ws[3] = 0
+    got = rt.conv_layer(x[0], wq, b, ws, ins, None, 5, (3, 3), pads=(1, 1, 1, 1), act=1)
+    assert np.all(got[0, 3] == max(b[3], 0))
+
+
+@pytest.mark.parametrize("name,c,h,w,outc,kernel,stride,pads,term,act", [
+    ("single-layer config 3x3 64->64 @56", 64, 56, 56, 64, (3, 3), (1, 1), (1, 1, 1, 1), 1, 1),
+    ("resnet stem 7x7/2 3->64 @112 (reduced from 224)", 3, 112, 112, 64, (7, 7), (2, 2), (3, 3, 3, 3), 2, 0),
+    ("resnet 1x1 256->64 @28 requant", 256, 28, 28, 64, (1, 1), (1, 1), (0, 0, 0, 0), 102, 1),
+    ("resnet 1x1/2 256->512 @28 fp32 out", 256, 28, 28, 512, (1, 1), (2, 2), (0, 0, 0, 0), 2, 0),
+    ("resnet 3x3 512->512 @7 requant", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 102, 1),
+    ("mobilenetv2 pointwise 96->24 @56 relu6", 96, 56, 56, 24, (1, 1), (1, 1), (0, 0, 0, 0), 101, 3),
+])
+def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pads, term, act):
+    _say("conv net-shape", name)
+    int8_in = term > 100
+    x, wq, b, ws, ins, tops = cases.conv_case(len(name), c, h, w, outc, kernel, 1, term, True, int8_in)
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, 1), stride, pads, 0.0, 1, 1, term, act, (0.0, 6.0))
+    want, wacc = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0], None if tops is None else tops[0], want_acc=True)
+    got, gacc = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, (1, 1), stride, pads, 0.0, 1, term, act, (0.0, 6.0), want_acc=True)
+    assert np.array_equal(gacc[0], wacc)
+    assert np.array_equal(got[0], want)
+    if act in (1, 3):
+        assert got.min() >= 0
+
+
+def test_convolution_batch_equals_per_sample_loop(rt):
+    # ncnn runs a batch as a per-sample loop (src/net.cpp:654-700); the folded launch must match it
+    x, wq, b, ws, ins, tops = cases.conv_case(77, 16, 14, 14, 40, (3, 3), 1, 101, True, False, batch=3)
+    d = oracle.make_desc((16, 14, 14), 40, (3, 3), pads=(1, 1, 1, 1), bias_term=1, int8_scale_term=101, activation_type=1)
+    got = rt.conv_layer(x, wq, b, ws, ins, tops, 40, (3, 3), pads=(1, 1, 1, 1), term=101, act=1)
+    for i in range(3):
+        assert np.array_equal(got[i], oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], tops[0]))
+
+
+# ----------------------------------------------------------------------------- depthwise / group
+@pytest.mark.parametrize("c,outc,group,h,w,stride", [(6, 6, 6, 9, 10, (1, 1)), (32, 32, 32, 56, 56, (1, 1)), (96, 96, 96, 28, 28, (2, 2)),
+                                                      (6, 12, 3, 9, 10, (1, 1)), (8, 4, 2, 12, 12, (2, 2)), (64, 64, 4, 14, 14, (1, 1))])
+@pytest.mark.parametrize("term,act,int8_in", [(1, 0, False), (101, 3, True), (102, 1, False), (2, 3, False)])
+def test_depthwise_and_group_bit_exact(rt, c, outc, group, h, w, stride, term, act, int8_in):
+    _say("dw/group", c, outc, group, h, w, stride, term, act, int8_in)
+    x, wq, b, ws, ins, tops = cases.conv_case(c + outc + group + term, c, h, w, outc, (3, 3), group, term, True, int8_in, by_group=True)
+    if term in (2, 102):
+        ws[:] = ws[0]
+    d = oracle.make_desc((c, h, w), outc, (3, 3), (1, 1), stride, (1, 1, 1, 1), 0.0, 1, group, term, act, (0.0, 6.0))
+    want, wacc = oracle.convolutiondepthwise_int8(d, x[0], wq, b, ws, ins, tops, want_acc=True)
+    got, gacc = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, (3, 3), (1, 1), stride, (1, 1, 1, 1), 0.0, group, term, act, (0.0, 6.0), want_acc=True)
+    assert np.array_equal(gacc[0], wacc)
+    assert got.dtype == want.dtype and np.array_equal(got[0], want)
+
+
+def test_depthwise_5x5_dilated_generic_kernel(rt):
+    x, wq, b, ws, ins, tops = cases.conv_case(91, 8, 15, 13, 8, (5, 3), 8, 101, True, True, by_group=True)
+    d = oracle.make_desc((8, 15, 13), 8, (5, 3), (2, 1), (1, 2), (-233,) * 4, 0.0, 1, 8, 101, 1)
+    want = oracle.convolutiondepthwise_int8(d, x[0], wq, b, ws, ins, tops)
+    got = rt.conv_layer(x[0], wq, b, ws, ins, tops, 8, (5, 3), (2, 1), (1, 2), (-233,) * 4, 0.0, 8, 101, 1)
+    assert np.array_equal(got[0], want)
+
+
+def test_invalid_group_returns_minus_100(rt):
+    import ncnn_amd
+    x, wq, b, ws, ins, tops = cases.conv_case(1, 6, 5, 5, 6, (3, 3), 6, 1, False, True, by_group=True)
+    with pytest.raises(ncnn_amd.NcnnHipError) as e:
+        rt.conv_layer(x[0], wq, b, np.ones(4, F), np.ones(4, F), None, 6, (3, 3), group=4)
+    assert e.value.code in (-1, -100)
+
+
+# ----------------------------------------------------------------------------- inner product
+@pytest.mark.parametrize("rows,k,n,act,bias,int8_in", [(1, 2048, 1000, 0, True, False), (1, 1280, 1000, 0, True, True), (1, 33, 7, 1, False, False),
+                                                        (5, 64, 10, 3, True, False), (16, 512, 300, 0, True, False), (70, 100, 130, 1, True, True)])
+def test_innerproduct_bit_exact(rt, rows, k, n, act, bias, int8_in):
+    _say("innerproduct", rows, k, n, act, bias, int8_in)
+    rng = np.random.default_rng(rows + k + n)
+    x = rng.uniform(-1, 1, (rows, k)).astype(F)
+    in_scale = F(127) / np.abs(x).max()
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    ws = rng.uniform(10, 20, n).astype(F)
+    ws[1 % n] = 0
+    b = rng.uniform(-1, 1, n).astype(F) if bias else None
+    if int8_in:
+        x = oracle.quantize(x, [in_scale])
+    want, wacc = oracle.innerproduct_int8(x, wq, b, ws, in_scale, act, (0.0, 6.0), want_acc=True)
+    got, gacc = rt.innerproduct_layer(x, wq, b, ws, in_scale, act, (0.0, 6.0), want_acc=True)
+    assert np.array_equal(gacc, wacc) and np.array_equal(got, want)
+
+
+# ----------------------------------------------------------------------------- block quant
+def _bq_check(got, a, packed, scales, bits, block, ins=None, c=None, bt=-1, alpha=1.0, beta=1.0):
+    val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins, c, bt, alpha, beta)
+    ref = oracle.gemm_blockquant(a, packed, scales, bits, block, ins, c, bt, alpha, beta)
+    tol = 1e-5 * floor + 1e-30
+    assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) / tol))
+    assert np.all(np.abs(got - val) <= tol), float(np.max(np.abs(got - val) / tol))
+
+
+@pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
+    (8, 64, 1, 24, 256, -1, False), (8, 64, 4, 16, 200, 4, False), (4, 32, 3, 9, 100, 3, True), (6, 128, 2, 7, 300, 1, True),
+    (8, 32, 16, 8, 64, 0, False), (4, 64, 1, 5, 65, 2, False), (8, 128, 5, 33, 1024, 4, True), (8, 64, 3, 10, 4096 + 16, -1, False)])
+def test_blockquant_small(rt, bits, block, m, n, k, bt, in_sc):
+    _say("blockquant", bits, block, m, n, k, bt, in_sc)
+    rng = np.random.default_rng(bits + block + m + n + k)
+    a = rng.standard_normal((m, k), dtype=F)
+    w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    ins = (0.75 + (np.arange(k) % 5) * 0.15).astype(F) if in_sc else None
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    got = rt.gemm_blockquant(a, packed, scales, bits, block, ins, c, bt, 1.25, 0.5)
+    _bq_check(got, a, packed, scales, bits, block, ins, c, bt, 1.25, 0.5)
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+@pytest.mark.parametrize("n,k", [(512, 4096), (256, 11008)])
+def test_blockquant_decode_shapes_fp32_and_fp16_activations(rt, m, n, k):
+    # the decode configuration's K with a reduced N (rows are independent, so N only scales the work)
+    _say("blockquant decode", m, n, k)
+    a, packed, scales = cases.blockquant_case(m * 7 + n + k, m, n, k)
+    got32 = rt.gemm_blockquant(a, packed, scales, 8, 64)
+    _bq_check(got32, a, packed, scales, 8, 64)
+    got16 = rt.gemm_blockquant(a.astype(np.float16), packed, scales, 8, 64)
+    assert np.array_equal(got16, got32)  # fp16-representable activations: both entry points see the same numbers
+
+
+def test_blockquant_exact_on_power_of_two_data(rt):
+    k, n, m = 128, 6, 2
+    rng = np.random.default_rng(3)
+    q = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    scales = np.full((n, k // 64), F(4.0), F)
+    a = rng.integers(-8, 9, (m, k)).astype(F)
+    got = rt.gemm_blockquant(a, q.view(np.uint8), scales, 8, 64)
+    assert np.array_equal(got, ((a.astype(np.int64) @ q.astype(np.int64).T) * 0.25).astype(F))
