@@ -133,7 +133,8 @@ int ncnnhip_transpose_s8(const int8_t* src_dev, size_t src_stride, int rows, int
 
 /* gemm_transB_int8 (src/layer/gemm.cpp:495-567): out = alpha*((float)acc / (sA_i*sB) + beta*C).
  * aq [M][K], bq [N][K] (K contiguous).  n_b_scales == 1 is ncnn's per-tensor B scale;
- * n_b_scales == N applies the same expression with a per-column scale (not expressible in ncnn).
+ * n_b_scales == N is a per-column generalisation that ncnn cannot express:
+ * out = alpha*(((float)acc * (1/sA_i)) * (1/sB_j) + beta*C).
  * broadcast_type_c: -1 no C, 0 scalar, 1/2 per row, 3 [M][N] (row stride N), 4 per column. */
 int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_dev, size_t bq_stride, int M, int N, int K,
                       const float* a_scales_dev, const float* b_scales_dev, int n_b_scales, const float* c_dev,

@@ -7,7 +7,8 @@
 
 namespace ncnnhip {
 
-// out = alpha * ((float)acc * (1/(sA_i*sB)) + beta*C)   -- every step one rounded fp32 op
+// out = alpha * ((float)acc * (1/(sA_i*sB)) + beta*C)   -- every step one rounded fp32 op.
+// With one B scale per column the dequantisation is ((float)acc * (1/sA_i)) * (1/sB_j).
 struct GemmEpilogue
 {
     const float* a_scales;
@@ -25,9 +26,11 @@ struct GemmEpilogue
     __device__ __forceinline__ void operator()(int i, int j, int acc) const
     {
         if (acc_out) acc_out[(size_t)i * N + j] = acc;
-        const float sb = per_col ? b_scales[j] : b_scales[0];
-        const float descale = div_rn(1.f, mul_rn(a_scales[i], sb));
-        float f = mul_rn((float)acc, descale);
+        float f;
+        if (per_col)
+            f = mul_rn(mul_rn((float)acc, div_rn(1.f, a_scales[i])), div_rn(1.f, b_scales[j]));
+        else
+            f = mul_rn((float)acc, div_rn(1.f, mul_rn(a_scales[i], b_scales[0])));
         if (bt >= 0)
         {
             float cv;

@@ -1,13 +1,202 @@
-// Large aligned int8 Gemm: software-pipelined MFMA kernel (placeholder dispatcher for now).
+// Large aligned int8 Gemm on the gfx950 matrix cores.
+//
+// One workgroup (4 wavefronts, one per SIMD) owns a 256x256 output tile; each wavefront owns a
+// 128x128 quadrant = 4x4 v_mfma_i32_32x32x32_i8 blocks = 256 int32 accumulators per lane.
+// K is walked in 64-byte steps through a 4-deep ring of LDS stages (32 KB each: 256 A rows and
+// 256 B rows of 64 bytes).  Stages are filled with direct global->LDS 128-bit loads (no register
+// staging), three steps ahead of the step being multiplied, so HBM/L2 latency is covered by
+// about three steps of matrix work.
+//
+// LDS layout of one operand stage: row r occupies bytes [64 r, 64 r + 64); its four 16-byte
+// chunks are stored at chunk position c ^ ((r >> 2) & 3).  A direct-to-LDS load writes the 64
+// lanes' 16-byte items back to back, so the swizzle is applied by choosing which global chunk
+// each lane fetches.  With it, any 16 consecutive rows read at one K offset hit 16 different
+// 16-byte bank groups.
+//
+// Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to XCDs)
+// works on a compact block of output tiles and re-uses its A/B panels out of its own L2.
 #include "epilogues.h"
 #include "mfma_tile.h"
 
+#define AS1 __attribute__((address_space(1)))
+#define AS3 __attribute__((address_space(3)))
+
 namespace ncnnhip {
 
-int launch_gemm_int8_pipelined(const int8_t*, size_t, const int8_t*, size_t, int, int, int, const GemmEpilogue&, hipStream_t, bool* handled)
+constexpr int PT = 256;            // tile edge
+constexpr int PK = 64;             // K bytes per stage
+constexpr int STAGES = 4;
+constexpr int OPERAND_BYTES = PT * PK;        // 16 KB
+constexpr int STAGE_BYTES = 2 * OPERAND_BYTES; // 32 KB
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
+#define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
+
+template<bool PER_COL, int BT>
+__global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __restrict__ A, size_t lda, const int8_t* __restrict__ B,
+                                                                 size_t ldb, int nk, int tiles_m, int tiles_n,
+                                                                 const float* __restrict__ a_scales, const float* __restrict__ b_scales,
+                                                                 const float* __restrict__ cvec, float alpha, float beta,
+                                                                 float* __restrict__ out, size_t ldo)
+{
+    __shared__ __attribute__((aligned(1024))) int8_t smem[STAGES * STAGE_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    // ---- XCD-aware tile choice: 8 XCDs take contiguous ranges of a 4-row-grouped tile order
+    int b = blockIdx.x;
+    const int T = tiles_m * tiles_n;
+    if ((T & 7) == 0) b = (b & 7) * (T >> 3) + (b >> 3);
+    constexpr int GM = 4;
+    const int per_group = GM * tiles_n;
+    const int group = b / per_group;
+    const int first_m = group * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int in_group = b - group * per_group;
+    const int tile_m = first_m + in_group % gsz;
+    const int tile_n = in_group / gsz;
+
+    // ---- per-lane global sources of the direct-to-LDS loads
+    // load i of wave w fills LDS rows (i*4 + w)*16 .. +16 of the operand stage
+    const int ld_row = wave * 16 + (lane >> 2);                 // + i*64
+    const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);        // swizzled source chunk
+    const int8_t* ga = A + ((size_t)tile_m * PT + ld_row) * lda + ld_chunk * 16;
+    const int8_t* gb = B + ((size_t)tile_n * PT + ld_row) * ldb + ld_chunk * 16;
+    const size_t a_step = 64 * lda, b_step = 64 * ldb;
+
+    auto issue_stage = [&](int t) {
+        int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024;
+        int8_t* sb = sa + OPERAND_BYTES;
+        const int8_t* pa = ga + (size_t)t * PK;
+        const int8_t* pb = gb + (size_t)t * PK;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+        {
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(pa + i * a_step), (AS3 void*)(sa + i * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(pb + i * b_step), (AS3 void*)(sb + i * 4096), 16, 0, 0);
+        }
+    };
+
+    v16i acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // ---- per-lane LDS read offsets: fragment row l32 (+32 per block), K chunk ks*2 + lhi, swizzled
+    const int sw = (l32 >> 2) & 3;
+    const int rd_a0 = (wm * 128 + l32) * PK + ((0 + lhi) ^ sw) * 16;
+    const int rd_a1 = (wm * 128 + l32) * PK + ((2 + lhi) ^ sw) * 16;
+    const int rd_b0 = OPERAND_BYTES + (wn * 128 + l32) * PK + ((0 + lhi) ^ sw) * 16;
+    const int rd_b1 = OPERAND_BYTES + (wn * 128 + l32) * PK + ((2 + lhi) ^ sw) * 16;
+
+    // ---- prologue: three steps in flight
+    if (0 < nk) issue_stage(0);
+    if (1 < nk) issue_stage(1);
+    if (2 < nk) issue_stage(2);
+
+    for (int t = 0; t < nk; t++)
+    {
+        // wait for step t (8 loads per step; newer steps may stay in flight)
+        if (t + 2 < nk)
+            WAIT_VMCNT(16);
+        else if (t + 1 < nk)
+            WAIT_VMCNT(8);
+        else
+            WAIT_VMCNT(0);
+        __builtin_amdgcn_s_barrier(); // step t visible to all waves; everyone is done with step t-1
+        if (t + 3 < nk) issue_stage(t + 3); // overwrites the stage of step t-1
+
+        const int8_t* st = smem + (t & (STAGES - 1)) * STAGE_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+        {
+            v4i fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const v4i*>(st + (ks ? rd_a1 : rd_a0) + i * 32 * PK);
+#pragma unroll
+            for (int j = 0; j < 4; j++) fb[j] = *reinterpret_cast<const v4i*>(st + (ks ? rd_b1 : rd_b0) + j * 32 * PK);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // ---- fused epilogue: dequantise, bias, scale, store fp32
+    const int row_base = tile_m * PT + wm * 128 + 4 * lhi;
+    const int col_base = tile_n * PT + wn * 128 + l32;
+    float colscale[4], colc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+    {
+        const int col = col_base + j * 32;
+        colscale[j] = PER_COL ? div_rn(1.f, b_scales[col]) : 0.f;
+        colc[j] = BT == 4 ? mul_rn(cvec[col], beta) : 0.f;
+    }
+    const float sb0 = b_scales[0];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+    {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int row = row_base + i * 32 + 8 * (r >> 2) + (r & 3);
+            const float sa = a_scales[row];
+            const float rowscale = PER_COL ? div_rn(1.f, sa) : div_rn(1.f, mul_rn(sa, sb0));
+            float* orow = out + (size_t)row * ldo + col_base;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                float f = mul_rn((float)acc[i][j][r], rowscale);
+                if (PER_COL) f = mul_rn(f, colscale[j]);
+                if (BT == 4) f = add_rn(f, colc[j]);
+                f = mul_rn(f, alpha);
+                orow[j * 32] = f;
+            }
+        }
+    }
+}
+
+static inline bool al16(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K,
+                               const GemmEpilogue& epi, hipStream_t stream, bool* handled)
 {
     *handled = false;
-    return NCNNHIP_OK;
+    if (M % PT || N % PT || K % PK || aq_stride % 16 || bq_stride % 16 || !al16(aq) || !al16(bq)) return NCNNHIP_OK;
+    if (epi.transpose || epi.acc_out || !(epi.bt == -1 || epi.bt == 4)) return NCNNHIP_OK;
+    const int tm = M / PT, tn = N / PT, nk = K / PK;
+    if ((long long)tm * tn > 0x7fffffff) return NCNNHIP_OK;
+    *handled = true;
+    dim3 grid(tm * tn), block(256);
+#define LAUNCH(PC, BTV)                                                                                                                    \
+    hipLaunchKernelGGL((gemm_int8_256x256_kernel<PC, BTV>), grid, block, 0, stream, aq, aq_stride, bq, bq_stride, nk, tm, tn, epi.a_scales, \
+                       epi.b_scales, epi.c, epi.alpha, epi.beta, epi.out, epi.out_stride)
+    if (epi.per_col)
+    {
+        if (epi.bt == 4)
+            LAUNCH(true, 4);
+        else
+            LAUNCH(true, -1);
+    }
+    else
+    {
+        if (epi.bt == 4)
+            LAUNCH(false, 4);
+        else
+            LAUNCH(false, -1);
+    }
+#undef LAUNCH
+    return launch_status("gemm_int8_256x256_kernel");
 }
 
 } // namespace ncnnhip

@@ -418,7 +418,7 @@ ORACLE_API float oracle_gemm_quantize_tensor(const float* b, size_t b_stride, in
  * gemm_transB_int8 (gemm.cpp:495-567): aq [M][K], bq [N][K] (B already transposed to
  * K-contiguous rows).
  *   b_scales: one value (ncnn's per-tensor B scale) when n_b_scales == 1.  n_b_scales == N is
- *   this repository's per-column generalisation of the same formula (descale = 1/(sA_i*sB_j));
+ *   this repository's per-column generalisation, f = ((float)acc * (1/sA_i)) * (1/sB_j);
  *   ncnn itself cannot express it, so that branch is pinned only by the numpy restatement.
  *   broadcast_type_c: -1 none, 0 scalar, 1/2 per row, 3 full [M][N], 4 per column.
  *   out: [M][N] (or [N][M] when output_transpose) with row stride out_stride.
@@ -439,8 +439,19 @@ ORACLE_API void oracle_gemm_int8(const int8_t* aq, size_t aq_stride, const int8_
             for (int k = 0; k < K; k++) acc += (int32_t)ar[k] * (int32_t)br[k];
             if (acc_out) acc_out[(size_t)i * N + j] = acc;
 
-            const float descale = 1.f / (a_scales[i] * (n_b_scales == 1 ? b_scales[0] : b_scales[j]));
-            float f = (float)acc * descale;
+            float f;
+            if (n_b_scales == 1)
+            {
+                const float descale = 1.f / (a_scales[i] * b_scales[0]);
+                f = (float)acc * descale;
+            }
+            else
+            {
+                const float da = 1.f / a_scales[i];
+                const float db = 1.f / b_scales[j];
+                f = (float)acc * da;
+                f = f * db;
+            }
             if (c && broadcast_type_c >= 0)
             {
                 float cv = 0.f;

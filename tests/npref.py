@@ -124,9 +124,11 @@ def gemm_int8(aq, bq, a_scales, b_scales, c=None, bt=-1, alpha=1.0, beta=1.0, tr
     m, n = acc.shape
     a_scales = np.asarray(a_scales, np.float32)
     b_scales = np.asarray(b_scales, np.float32).reshape(-1)
-    bs = b_scales[None, :] if b_scales.size == n and n != 1 else b_scales[:1][None, :]
-    descale = (F(1) / (a_scales[:, None] * bs)).astype(np.float32)
-    f = acc.astype(np.float32) * descale
+    if b_scales.size == 1:
+        descale = (F(1) / (a_scales[:, None] * b_scales[:1][None, :])).astype(np.float32)
+        f = acc.astype(np.float32) * descale
+    else:  # per-column generalisation: (acc * 1/sA_i) * 1/sB_j
+        f = (acc.astype(np.float32) * (F(1) / a_scales)[:, None]).astype(np.float32) * (F(1) / b_scales)[None, :]
     if c is not None and bt >= 0:
         c = np.asarray(c, np.float32)
         cv = {0: lambda: c.reshape(-1)[0], 1: lambda: c.reshape(m, 1), 2: lambda: c.reshape(m, 1),
