@@ -15,6 +15,8 @@
 //
 // Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to XCDs)
 // works on a compact block of output tiles and re-uses its A/B panels out of its own L2.
+#include <type_traits>
+
 #include "epilogues.h"
 #include "mfma_tile.h"
 
@@ -32,6 +34,7 @@ constexpr int STAGE_BYTES = 2 * OPERAND_BYTES; // 32 KB
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
 #define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
 
+
 template<bool PER_COL, int BT>
 __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __restrict__ A, size_t lda, const int8_t* __restrict__ B,
                                                                  size_t ldb, int nk, int tiles_m, int tiles_n,
@@ -42,7 +45,7 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     __shared__ __attribute__((aligned(1024))) int8_t smem[STAGES * STAGE_BYTES];
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform, lives in an SGPR
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -67,17 +70,15 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     const int8_t* gb = B + ((size_t)tile_n * PT + ld_row) * ldb + ld_chunk * 16;
     const size_t a_step = 64 * lda, b_step = 64 * ldb;
 
+    // quarter i of the loads of step t: 16 A rows and 16 B rows per wave
+    auto issue_quarter = [&](int t, int i) {
+        int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024 + i * 4096;
+        __builtin_amdgcn_global_load_lds((const AS1 void*)(ga + (size_t)t * PK + i * a_step), (AS3 void*)sa, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const AS1 void*)(gb + (size_t)t * PK + i * b_step), (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
+    };
     auto issue_stage = [&](int t) {
-        int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024;
-        int8_t* sb = sa + OPERAND_BYTES;
-        const int8_t* pa = ga + (size_t)t * PK;
-        const int8_t* pb = gb + (size_t)t * PK;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-        {
-            __builtin_amdgcn_global_load_lds((const AS1 void*)(pa + i * a_step), (AS3 void*)(sa + i * 4096), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const AS1 void*)(pb + i * b_step), (AS3 void*)(sb + i * 4096), 16, 0, 0);
-        }
+        for (int i = 0; i < 4; i++) issue_quarter(t, i);
     };
 
     v16i acc[4][4];
@@ -100,33 +101,107 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     if (1 < nk) issue_stage(1);
     if (2 < nk) issue_stage(2);
 
-    for (int t = 0; t < nk; t++)
-    {
-        // wait for step t (8 loads per step; newer steps may stay in flight)
+    // Fragment registers are double-buffered: while the 16 MFMAs of one K half-step run, the
+    // 8 LDS reads of the next half-step are already in flight.  The workgroup barrier sits
+    // between the two half-steps of a stage.
+    // The LDS reads and their waits are written as asm so that the wait before a group of MFMAs
+    // only covers the fragment set that group uses (lgkmcnt(8)) and leaves the 8 reads of the next
+    // set in flight.
+    v4i fa0[4], fb0[4], fa1[4], fb1[4];
+    const unsigned lds_base = (unsigned)(uintptr_t)(AS3 int8_t*)smem;
+    auto frag_addr_a = [&](int t, int ks) { return lds_base + (unsigned)((t & (STAGES - 1)) * STAGE_BYTES) + (ks ? rd_a1 : rd_a0); };
+    auto frag_addr_b = [&](int t, int ks) { return lds_base + (unsigned)((t & (STAGES - 1)) * STAGE_BYTES) + (ks ? rd_b1 : rd_b0); };
+#define LDS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
+    auto read_frags = [&](int t, int ks, v4i (&fa)[4], v4i (&fb)[4]) {
+        const unsigned pa = frag_addr_a(t, ks), pb = frag_addr_b(t, ks);
+        LDS_READ(fa[0], pa, 0);
+        LDS_READ(fb[0], pb, 0);
+        LDS_READ(fb[1], pb, 2048);
+        LDS_READ(fb[2], pb, 4096);
+        LDS_READ(fb[3], pb, 6144);
+        LDS_READ(fa[1], pa, 2048);
+        LDS_READ(fa[2], pa, 4096);
+        LDS_READ(fa[3], pa, 6144);
+    };
+    // waits until at most `pending` LDS reads are outstanding and ties the fragment registers to
+    // the wait so the MFMAs that use them cannot be moved above it
+#define WAIT_FRAGS(pending, fa, fb)                                                                                   \
+    asm volatile("s_waitcnt lgkmcnt(" #pending ")"                                                                    \
+                 : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
+#define PIN __builtin_amdgcn_sched_barrier(0)
+    auto mma_row = [&](int i, const v4i (&fa)[4], const v4i (&fb)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    auto wait_step = [&](int t) {
+        // wait for the loads of step t (8 per step; newer steps may stay in flight)
         if (t + 2 < nk)
             WAIT_VMCNT(16);
         else if (t + 1 < nk)
             WAIT_VMCNT(8);
         else
             WAIT_VMCNT(0);
-        __builtin_amdgcn_s_barrier(); // step t visible to all waves; everyone is done with step t-1
-        if (t + 3 < nk) issue_stage(t + 3); // overwrites the stage of step t-1
+    };
 
-        const int8_t* st = smem + (t & (STAGES - 1)) * STAGE_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
+    wait_step(0);
+    __builtin_amdgcn_s_barrier();
+    if (3 < nk) issue_stage(3);
+    read_frags(0, 0, fa0, fb0);
+
+    // One K step.  Schedule (F0/F1 = the two fragment register sets):
+    //   reads(t, second half) -> F1 | wait F0 | 16 MFMA(F0) | wait loads of step t+1, barrier |
+    //   4 x { 4 MFMA(F1), one quarter of the global->LDS loads of step t+4, 2 reads of (t+1, first half) -> F0 }
+    // so the matrix pipe always has a full MFMA group queued behind the barrier, and every LDS or
+    // global access is issued at least 16 MFMAs before its data is needed.
+    // STEADY means steps t+1 .. t+4 all exist (branch-free body).
+    auto k_step = [&](int t, auto steady) {
+        constexpr bool STEADY = decltype(steady)::value;
+        read_frags(t, 1, fa1, fb1);
+        WAIT_FRAGS(8, fa0, fb0);
+        PIN;
+        mma_row(0, fa0, fb0);
+        mma_row(1, fa0, fb0);
+        mma_row(2, fa0, fb0);
+        mma_row(3, fa0, fb0);
+        PIN;
+        const bool more = STEADY || t + 1 < nk;
+        const bool refill = STEADY || t + 4 < nk;
+        if (more)
         {
-            v4i fa[4], fb[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const v4i*>(st + (ks ? rd_a1 : rd_a0) + i * 32 * PK);
-#pragma unroll
-            for (int j = 0; j < 4; j++) fb[j] = *reinterpret_cast<const v4i*>(st + (ks ? rd_b1 : rd_b0) + j * 32 * PK);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            if (STEADY)
+                WAIT_VMCNT(16);
+            else
+                wait_step(t + 1);
         }
-    }
+        WAIT_FRAGS(0, fa1, fb1);      // this wave's reads of step t have landed
+        if (more) __builtin_amdgcn_s_barrier(); // step t+1 visible to all waves; nobody reads step t any more
+        PIN;
+        const unsigned pa = frag_addr_a(t + 1, 0), pb = frag_addr_b(t + 1, 0);
+        mma_row(0, fa1, fb1);
+        PIN;
+        if (refill) issue_quarter(t + 4, 0);
+        if (more) { LDS_READ(fa0[0], pa, 0); LDS_READ(fb0[0], pb, 0); }
+        PIN;
+        mma_row(1, fa1, fb1);
+        PIN;
+        if (refill) issue_quarter(t + 4, 1);
+        if (more) { LDS_READ(fb0[1], pb, 2048); LDS_READ(fb0[2], pb, 4096); }
+        PIN;
+        mma_row(2, fa1, fb1);
+        PIN;
+        if (refill) issue_quarter(t + 4, 2);
+        if (more) { LDS_READ(fb0[3], pb, 6144); LDS_READ(fa0[1], pa, 2048); }
+        PIN;
+        mma_row(3, fa1, fb1);
+        PIN;
+        if (refill) issue_quarter(t + 4, 3);
+        if (more) { LDS_READ(fa0[2], pa, 4096); LDS_READ(fa0[3], pa, 6144); }
+        PIN;
+    };
+
+    int t = 0;
+    for (; t + 4 < nk; t++) k_step(t, std::true_type{});
+    for (; t < nk; t++) k_step(t, std::false_type{});
 
     // ---- fused epilogue: dequantise, bias, scale, store fp32
     const int row_base = tile_m * PT + wm * 128 + 4 * lhi;
