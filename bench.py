@@ -138,9 +138,15 @@ def bench_blockquant(args, n, k, m):
     a, packed, scales = synth.blockquant8_operands(n + k + m, m, n, k)
     wbytes = packed.nbytes + scales.nbytes
     copies = int(np.ceil(512e6 / wbytes)) + 1
-    d_w = [rt.up(packed) for _ in range(copies)]
-    d_s = [rt.up(scales) for _ in range(copies)]
     half = args.act == "fp16"
+    if half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
+        pw, pd = rt.blockquant_pack(packed, scales, 64)
+        wbytes = n * k + scales.nbytes  # algorithmic bytes: the int8 weights and one fp32 scale per block
+        d_w = [rt.up(pw) for _ in range(copies)]
+        d_s = [rt.up(pd) for _ in range(copies)]
+    else:
+        d_w = [rt.up(packed) for _ in range(copies)]
+        d_s = [rt.up(scales) for _ in range(copies)]
     d_a = rt.up(a.astype(np.float16) if half else a)
     d_out = ncnn_amd.DeviceBuffer.empty((m, n), np.float32)
     st = rt.stream
@@ -148,7 +154,7 @@ def bench_blockquant(args, n, k, m):
     def launch(i):
         j = i % copies
         if half:
-            check(lib.ncnnhip_gemm_blockquant_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, 8, 64, d_s[j].ptr, d_out.ptr, n, st))
+            check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, None, -1, 1.0, 1.0, d_out.ptr, n, st))
         else:
             check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, 8, 64, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
 
@@ -175,7 +181,7 @@ def bench_blockquant(args, n, k, m):
         "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, int8 weights in blocks of 64, fp32 block scales, %s activations" % (m, n, k, args.act),
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "blockquant8_kernel", "bytes_per_launch": algo},
+                     "kernel": "blockquant8_mfma_kernel" if half else "blockquant8_stream_kernel", "bytes_per_launch": algo},
     }
 
 

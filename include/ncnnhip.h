@@ -158,6 +158,23 @@ int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, 
                                  int bits, int block, const float* scales_dev, float* out_dev, size_t out_stride,
                                  void* stream);
 
+/* Packed form of the 8-bit block-quantised weights, made once at create_pipeline (the repacking
+ * of constant weights into matrix-core tiles).  ncnn keeps B_data [N][K] and B_data_quantize_scales
+ * [N][ceil(K/block)] as loaded (src/layer/gemm.cpp:182-221); here they become
+ *   weights  [ceil(N/16)][ceil(K/64)][64][16] bytes, byte = q + 128, lane l = row l%16, K (l/16)*16..+15
+ *   descales [ceil(N/16)][ceil(K/64)][16] fp32 = 1.f/scale (the reference's per-block division).
+ * block must be 64 or 128.  Both functions run on the host. */
+int ncnnhip_blockquant_packed_size(int N, int K, int block, size_t* weight_bytes, size_t* descale_bytes);
+int ncnnhip_blockquant_pack(const uint8_t* b_host, const float* scales_host, int N, int K, int bits, int block,
+                            uint8_t* packed_w_host, float* packed_descale_host);
+/* Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483) on the packed weights with fp16
+ * activations a [M][K] (K % 16 == 0), any M; out fp32 [M][N].  Same C / alpha / beta meaning as
+ * ncnnhip_gemm_blockquant. */
+int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K,
+                                        const uint8_t* packed_w_dev, const float* packed_descale_dev, const float* c_dev,
+                                        int broadcast_type_c, float alpha, float beta, float* out_dev, size_t out_stride,
+                                        void* stream);
+
 #pragma GCC visibility pop
 
 #ifdef __cplusplus

@@ -37,60 +37,254 @@ __device__ __forceinline__ float to_f32(__half v)
 }
 
 // ---- 8-bit weights, K % 16 == 0, 16-byte aligned rows ------------------------------------
-template<typename AT, int MB>
-__global__ __launch_bounds__(256) void blockquant8_kernel(const AT* __restrict__ a, size_t a_stride, int M, int N, int K,
-                                                           const int8_t* __restrict__ b, int block_shift, int nblk,
-                                                           const float* __restrict__ scales, const float* __restrict__ in_scales,
-                                                           const float* __restrict__ c, int bt, float alpha, float beta,
-                                                           float* __restrict__ out, size_t out_stride)
+// Streaming kernel for up to MT activation rows at a time.
+//   * the activations (times the optional input scales) are staged once per workgroup in LDS as
+//     fp32, in K tiles of KT = 16384 / MT values;
+//   * every wavefront owns R consecutive weight rows; per row each lane fetches 16-byte chunks
+//     lane, lane+64, ... of the K tile, U chunks per batch, and all R*U 16-byte loads of a batch
+//     are issued before the first one is consumed, which is what keeps enough bytes in flight to
+//     cover HBM latency;
+//   * a chunk never straddles a quantisation block (block >= 32), so the 16 products of a chunk
+//     are summed first and the block's 1/scale is applied once per chunk.
+template<typename AT, int MT, int R, int U>
+__global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __restrict__ a, size_t a_stride, int m0, int M, int N, int K,
+                                                                  const int8_t* __restrict__ b, int block_shift, int nblk,
+                                                                  const float* __restrict__ scales, const float* __restrict__ in_scales,
+                                                                  const float* __restrict__ c, int bt, float alpha, float beta,
+                                                                  float* __restrict__ out, size_t out_stride)
 {
+    constexpr int KT = 16384 / MT;
+    __shared__ __attribute__((aligned(16))) float lds_a[MT * KT];
+
     const int lane = threadIdx.x & 63;
-    const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (j >= N) return;
-    const int8_t* br = b + (size_t)j * K;
-    const float* sr = scales + (size_t)j * nblk;
+    const int wave = threadIdx.x >> 6;
+    const int j0 = (blockIdx.x * 4 + wave) * R;
+    const int mcount = M - m0 < MT ? M - m0 : MT;
 
-    for (int i0 = 0; i0 < M; i0 += MB)
-    {
-        float sum[MB];
+    float acc[R][MT];
 #pragma unroll
-        for (int m = 0; m < MB; m++) sum[m] = 0.f;
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MT; m++) acc[r][m] = 0.f;
 
-        for (int k = lane * 16; k < K; k += 64 * 16)
-        {
-            const v4i_bq wv = *reinterpret_cast<const v4i_bq*>(br + k);
-            const float descale = div_rn(1.f, sr[k >> block_shift]);
-            float wf[16];
+    // A "batch" is R*U chunks per lane: rows j0..j0+R-1, chunks c0 + u*64 + lane of K tile kt0.
+    // Weight batches do not depend on LDS, so batch n+1 is always requested before batch n is
+    // multiplied, and the very first batch is requested before the activations are staged.
+    auto load_batch = [&](int kt0, int c0, v4i_bq (&w)[R][U], float (&d)[R][U]) {
+        const int kt = K - kt0 < KT ? K - kt0 : KT;
+        const int nch = kt >> 4;
 #pragma unroll
-            for (int t = 0; t < 16; t++) wf[t] = mul_rn((float)(int)(int8_t)(wv[t >> 2] >> ((t & 3) * 8)), descale);
+        for (int r = 0; r < R; r++)
 #pragma unroll
-            for (int m = 0; m < MB; m++)
+            for (int u = 0; u < U; u++)
             {
-                if (i0 + m < M)
+                const int ch = c0 + u * 64 + lane;
+                const int j = j0 + r;
+                const bool ok = ch < nch && j < N;
+                const size_t koff = (size_t)kt0 + ((size_t)ch << 4);
+                w[r][u] = ok ? *reinterpret_cast<const v4i_bq*>(b + (size_t)j * K + koff) : v4i_bq{0, 0, 0, 0};
+                d[r][u] = ok ? scales[(size_t)j * nblk + (koff >> block_shift)] : 1.f;
+            }
+    };
+    auto compute_batch = [&](int kt0, int c0, const v4i_bq (&w)[R][U], const float (&d)[R][U]) {
+        const int kt = K - kt0 < KT ? K - kt0 : KT;
+        const int nch = kt >> 4;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int ch = c0 + u * 64 + lane;
+            if (ch < nch)
+            {
+                float av[MT][16];
+#pragma unroll
+                for (int m = 0; m < MT; m++)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++)
+                    {
+                        const float4 t4 = *reinterpret_cast<const float4*>(&lds_a[m * KT + (ch << 4) + q4 * 4]);
+                        av[m][q4 * 4 + 0] = t4.x;
+                        av[m][q4 * 4 + 1] = t4.y;
+                        av[m][q4 * 4 + 2] = t4.z;
+                        av[m][q4 * 4 + 3] = t4.w;
+                    }
+#pragma unroll
+                for (int r = 0; r < R; r++)
                 {
-                    const AT* ar = a + (size_t)(i0 + m) * a_stride + k;
+                    float part[MT];
+#pragma unroll
+                    for (int m = 0; m < MT; m++) part[m] = 0.f;
 #pragma unroll
                     for (int t = 0; t < 16; t++)
                     {
-                        float v = to_f32(ar[t]);
-                        if (in_scales) v = mul_rn(v, in_scales[k + t]);
-                        sum[m] = add_rn(sum[m], mul_rn(v, wf[t]));
+                        const float q = (float)(int)(int8_t)(w[r][u][t >> 2] >> ((t & 3) * 8));
+#pragma unroll
+                        for (int m = 0; m < MT; m++) part[m] = fmaf(av[m][t], q, part[m]);
                     }
+                    const float descale = div_rn(1.f, d[r][u]);
+#pragma unroll
+                    for (int m = 0; m < MT; m++) acc[r][m] = fmaf(part[m], descale, acc[r][m]);
                 }
             }
         }
-#pragma unroll
-        for (int m = 0; m < MB; m++)
+    };
+    auto stage_tile = [&](int kt0) {
+        const int kt = K - kt0 < KT ? K - kt0 : KT;
+        for (int m = 0; m < MT; m++)
         {
-            const float total = wave_sum(sum[m]);
-            if (lane == 0 && i0 + m < M)
+            const bool live = m < mcount;
+            const AT* arow = a + (size_t)(m0 + (live ? m : 0)) * a_stride + kt0;
+            constexpr int VEC = 16 / (int)sizeof(AT);
+            const bool vec_ok = (reinterpret_cast<uintptr_t>(arow) & 15) == 0;
+            if (vec_ok)
             {
-                float f = total;
-                if (bt >= 0) f = add_rn(mul_rn(load_c(c, bt, i0 + m, j, N), beta), f);
-                out[(size_t)(i0 + m) * out_stride + j] = mul_rn(f, alpha);
+                const int nvec = kt / VEC; // kt % 16 == 0
+#pragma unroll 4
+                for (int v = threadIdx.x; v < nvec; v += 256)
+                {
+                    float tmp[VEC];
+                    if (live)
+                    {
+                        const v4i_bq raw = *reinterpret_cast<const v4i_bq*>(arow + v * VEC);
+                        if (sizeof(AT) == 4)
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) tmp[e] = __int_as_float(raw[e]);
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                            {
+                                tmp[(2 * e) % VEC] = __half2float(__ushort_as_half((unsigned short)(raw[e] & 0xffff)));
+                                tmp[(2 * e + 1) % VEC] = __half2float(__ushort_as_half((unsigned short)((unsigned)raw[e] >> 16)));
+                            }
+                        }
+                        if (in_scales)
+                        {
+#pragma unroll
+                            for (int e = 0; e < VEC; e++) tmp[e] = mul_rn(tmp[e], in_scales[kt0 + v * VEC + e]);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) tmp[e] = 0.f;
+                    }
+#pragma unroll
+                    for (int e = 0; e < VEC; e += 4)
+                        *reinterpret_cast<float4*>(&lds_a[m * KT + v * VEC + e]) = make_float4(tmp[e], tmp[e + 1], tmp[e + 2], tmp[e + 3]);
+                }
+            }
+            else
+            {
+                for (int k = threadIdx.x; k < kt; k += 256)
+                {
+                    float v = 0.f;
+                    if (live)
+                    {
+                        v = to_f32(arow[k]);
+                        if (in_scales) v = mul_rn(v, in_scales[kt0 + k]);
+                    }
+                    lds_a[m * KT + k] = v;
+                }
+            }
+        }
+    };
+
+    v4i_bq w0[R][U], w1[R][U];
+    float d0[R][U], d1[R][U];
+    load_batch(0, 0, w0, d0);
+    for (int kt0 = 0; kt0 < K; kt0 += KT)
+    {
+        const int kt = K - kt0 < KT ? K - kt0 : KT;
+        const int nch = kt >> 4;
+        if (kt0) __syncthreads(); // everyone is done with the previous activation tile
+        stage_tile(kt0);
+        __syncthreads();
+        // batches of this tile, two per trip so the two register sets alternate statically
+        for (int c0 = 0; c0 < nch; c0 += 2 * 64 * U)
+        {
+            const int c1 = c0 + 64 * U;
+            const int c2 = c1 + 64 * U;
+            if (c1 < nch)
+                load_batch(kt0, c1, w1, d1);
+            else if (kt0 + KT < K)
+                load_batch(kt0 + KT, 0, w1, d1);
+            compute_batch(kt0, c0, w0, d0);
+            if (c1 < nch)
+            {
+                if (c2 < nch)
+                    load_batch(kt0, c2, w0, d0);
+                else if (kt0 + KT < K)
+                    load_batch(kt0 + KT, 0, w0, d0);
+                compute_batch(kt0, c1, w1, d1);
+            }
+            else if (kt0 + KT < K)
+            {
+                // the prefetched first batch of the next tile sits in set 1: move it to set 0
+#pragma unroll
+                for (int r = 0; r < R; r++)
+#pragma unroll
+                    for (int u = 0; u < U; u++)
+                    {
+                        w0[r][u] = w1[r][u];
+                        d0[r][u] = d1[r][u];
+                    }
             }
         }
     }
+
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+        {
+            const float total = wave_sum(acc[r][m]);
+            const int j = j0 + r;
+            if (lane == 0 && j < N && m < mcount)
+            {
+                float f = total;
+                if (bt >= 0) f = add_rn(mul_rn(load_c(c, bt, m0 + m, j, N), beta), f);
+                out[(size_t)(m0 + m) * out_stride + j] = mul_rn(f, alpha);
+            }
+        }
+}
+
+template<typename AT>
+static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K, const int8_t* b8, int block, const float* scales,
+                              const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride,
+                              hipStream_t stream)
+{
+    const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
+    const int nblk = (K + block - 1) / block;
+#ifndef BQ_R
+#define BQ_R 2
+#endif
+    constexpr int R = BQ_R, U = 4;
+    dim3 grid(ceil_div(N, 4 * R));
+    for (int m0 = 0; m0 < M;)
+    {
+        const int left = M - m0;
+        if (left >= 4)
+        {
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 4, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+                               in_scales, c, bt, alpha, beta, out, out_stride);
+            m0 += 4;
+        }
+        else if (left >= 2)
+        {
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 2, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+                               in_scales, c, bt, alpha, beta, out, out_stride);
+            m0 += 2;
+        }
+        else
+        {
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 1, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+                               in_scales, c, bt, alpha, beta, out, out_stride);
+            m0 += 1;
+        }
+    }
+    return launch_status("blockquant8_stream_kernel");
 }
 
 // ---- any bits / block / alignment --------------------------------------------------------
@@ -138,6 +332,169 @@ __global__ __launch_bounds__(256) void blockquant_generic_kernel(const float* __
     }
 }
 
+// ---- matrix-core streaming kernel for packed 8-bit weights, up to 16 activation rows -------
+// Packed layout (made once when the weights are uploaded):
+//   weights   [ceil(N/16)][ceil(K/64)][64 lanes][16 bytes]: lane l of a tile holds row l%16,
+//             K offsets (l/16)*16 .. +15 of the 64-wide K block, each byte stored as q+128;
+//   descales  [ceil(N/16)][ceil(K/64)][16] fp32 = 1/scale of that row for that K block.
+// A workgroup owns 16 weight rows; its 4 wavefronts split K.  Per K block a lane issues one
+// 16-byte weight load, one 16-byte descale load and two 16-byte activation loads (fp16, straight
+// from L2), turns the 16 bytes into 16 halves with byte permutes (0x6400|u is the half 1024+u,
+// minus 1152 gives q exactly), and runs two v_mfma_f32_16x16x32_f16: rows = weight rows,
+// columns = activation rows.  Integer-valued q times an fp16 activation is exact in fp32, so the
+// only roundings are the fp32 accumulation and the one multiply by 1/scale per K block.
+#ifndef BQ_MFMA_U
+#define BQ_MFMA_U 2
+#endif
+#ifndef BQ_MFMA_NS
+#define BQ_MFMA_NS 4
+#endif
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ v8h bytes_to_halves(int lo, int hi)
+{
+    // lo, hi: 8 bytes u0..u7 (u = q + 128).  Build halves 0x6400|u = 1024+u, then subtract 1152.
+    union
+    {
+        int i[4];
+        v2h h2[4];
+        v8h h8;
+    } t;
+    t.i[0] = __builtin_amdgcn_perm(0x64646464, lo, 0x04010400);
+    t.i[1] = __builtin_amdgcn_perm(0x64646464, lo, 0x04030402);
+    t.i[2] = __builtin_amdgcn_perm(0x64646464, hi, 0x04010400);
+    t.i[3] = __builtin_amdgcn_perm(0x64646464, hi, 0x04030402);
+    const v2h off = {(_Float16)1152.f, (_Float16)1152.f};
+#pragma unroll
+    for (int e = 0; e < 4; e++) t.h2[e] = t.h2[e] - off;
+    return t.h8;
+}
+
+template<int NS, int U>
+__global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
+                                                                const v4i_bq* __restrict__ wpk, const float4* __restrict__ dpk,
+                                                                const float* __restrict__ c, int bt, float alpha, float beta,
+                                                                float* __restrict__ out, size_t out_stride)
+{
+    extern __shared__ __attribute__((aligned(16))) float4 lds_d[]; // descales of this tile: [kblocks][4] float4
+    __shared__ float red[4][64][4];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tile = blockIdx.x;
+    const int m = lane & 15;
+    const int kg = lane >> 4; // K group of this lane inside a 64-wide block
+
+    // K blocks of this wave
+    const int per_wave = (kblocks + 3) >> 2;
+    const int kb_begin = wave * per_wave;
+    const int kb_end = kb_begin + per_wave < kblocks ? kb_begin + per_wave : kblocks;
+    const int nkb = kb_end > kb_begin ? kb_end - kb_begin : 0;
+    auto block_of = [&](int i) { return kb_begin + i; }; // i-th block this wave processes
+
+    const v4i_bq* wt = wpk + ((size_t)tile * kblocks) * 64 + lane;
+    const __half* arow = a + (size_t)(m < M ? m : 0) * a_stride + kg * 16;
+    const bool a_live = m < M;
+
+    // Requests are issued in the order their data is consumed (loads return in order): the tile's
+    // descales, then per batch the activations (L2) followed by the weights (the HBM stream).  NS
+    // batches of U blocks are in flight in a ring of register sets, so the arithmetic of one small
+    // batch runs while the following ones are still arriving and little work is left once the last
+    // bytes land.
+    struct Batch
+    {
+        v4i_bq w[U], a0[U], a1[U];
+    };
+    auto load_batch = [&](int kb0, Batch& bt_) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const bool live = kb0 + u < nkb;
+            const int kb = block_of(live ? kb0 + u : 0);
+            const bool aok = live && a_live && kb * 64 + kg * 16 < K; // K % 16 == 0: a 16-half chunk is all in or all out
+            bt_.a0[u] = aok ? *reinterpret_cast<const v4i_bq*>(arow + (size_t)kb * 64) : v4i_bq{0, 0, 0, 0};
+            bt_.a1[u] = aok ? *reinterpret_cast<const v4i_bq*>(arow + (size_t)kb * 64 + 8) : v4i_bq{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const bool live = kb0 + u < nkb;
+            const int kb = block_of(live ? kb0 + u : 0);
+            bt_.w[u] = live ? wt[(size_t)kb * 64] : v4i_bq{(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+        }
+    };
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](int kb0, const Batch& bt_) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const bool live = kb0 + u < nkb;
+            const int kb = block_of(live ? kb0 + u : 0);
+            const v8h wa = bytes_to_halves(bt_.w[u][0], bt_.w[u][1]);
+            const v8h wb = bytes_to_halves(bt_.w[u][2], bt_.w[u][3]);
+            union
+            {
+                v4i_bq i;
+                v8h h;
+            } xa, xb;
+            xa.i = bt_.a0[u];
+            xb.i = bt_.a1[u];
+            v4f t = {0.f, 0.f, 0.f, 0.f};
+            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, t, 0, 0, 0);
+            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
+            const float4 d = live ? lds_d[kb * 4 + kg] : make_float4(0.f, 0.f, 0.f, 0.f);
+            acc[0] = fmaf(t[0], d.x, acc[0]);
+            acc[1] = fmaf(t[1], d.y, acc[1]);
+            acc[2] = fmaf(t[2], d.z, acc[2]);
+            acc[3] = fmaf(t[3], d.w, acc[3]);
+        }
+    };
+
+    // descales of the whole tile: requested first, written to LDS once they are here
+    const float4* dt = dpk + (size_t)tile * kblocks * 4;
+    const int nd = kblocks * 4;
+    float4 dreg[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) dreg[i] = threadIdx.x + i * 256 < nd ? dt[threadIdx.x + i * 256] : make_float4(0.f, 0.f, 0.f, 0.f);
+    Batch sets[NS];
+#pragma unroll
+    for (int q = 0; q < NS; q++) load_batch(q * U, sets[q]);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (threadIdx.x + i * 256 < nd) lds_d[threadIdx.x + i * 256] = dreg[i];
+    for (int i = threadIdx.x + 1024; i < nd; i += 256) lds_d[i] = dt[i]; // K beyond 16384
+    __syncthreads();
+    for (int kb0 = 0; kb0 < nkb; kb0 += NS * U)
+    {
+#pragma unroll
+        for (int q = 0; q < NS; q++)
+        {
+            compute(kb0 + q * U, sets[q]);                 // batch indices count from 0 inside this wave's range
+            load_batch(kb0 + (q + NS) * U, sets[q]);       // requests beyond the range are masked off
+        }
+    }
+
+    // combine the four K splits; accumulator r of lane l is (weight row (l/16)*4 + r, activation row l%16)
+#pragma unroll
+    for (int r = 0; r < 4; r++) red[wave][lane][r] = acc[r];
+    __syncthreads();
+    if (wave == 0 && m < M)
+    {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int j = tile * 16 + kg * 4 + r;
+            if (j < N)
+            {
+                float f = add_rn(add_rn(red[0][lane][r], red[1][lane][r]), add_rn(red[2][lane][r], red[3][lane][r]));
+                if (bt >= 0) f = add_rn(mul_rn(load_c(c, bt, m, j, N), beta), f);
+                out[(size_t)m * out_stride + j] = mul_rn(f, alpha);
+            }
+        }
+    }
+}
+
 static int check_blockquant(const void* a, const void* b, const void* scales, const void* out, int M, int N, int K, int bits, int block,
                             const void* c, int bt)
 {
@@ -172,20 +529,79 @@ int ncnnhip_gemm_blockquant(const float* a_dev, size_t a_stride, int M, int N, i
     dim3 grid(ceil_div(N, 4));
     if (bits == 8 && K % 16 == 0 && al16(b_dev))
     {
-        const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
-        const int8_t* b8 = reinterpret_cast<const int8_t*>(b_dev);
-        if (M == 1)
-            hipLaunchKernelGGL((blockquant8_kernel<float, 1>), grid, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, b8, shift, nblk,
-                               scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride);
-        else
-            hipLaunchKernelGGL((blockquant8_kernel<float, 4>), grid, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, b8, shift, nblk,
-                               scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride);
-        return launch_status("blockquant8_kernel");
+        return launch_blockquant8<float>(a_dev, a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev), block, scales_dev, in_scales_dev,
+                                         c_dev, bt, alpha, beta, out_dev, out_stride, as_stream(stream));
     }
     const int packed = (int)(((size_t)K * bits + 7) / 8);
     hipLaunchKernelGGL(blockquant_generic_kernel, grid, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, b_dev, bits, block, packed,
                        nblk, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride);
     return launch_status("blockquant_generic_kernel");
+}
+
+int ncnnhip_blockquant_packed_size(int N, int K, int block, size_t* weight_bytes, size_t* descale_bytes)
+{
+    NCNNHIP_REQUIRE(N >= 1 && K >= 1, "ncnnhip_blockquant_packed_size: bad shape");
+    NCNNHIP_REQUIRE(block == 64 || block == 128, "ncnnhip_blockquant_packed_size: packed layout needs block 64 or 128, got %d", block);
+    const size_t tiles = (size_t)(N + 15) / 16, kblocks = (size_t)(K + 63) / 64;
+    if (weight_bytes) *weight_bytes = tiles * kblocks * 1024;
+    if (descale_bytes) *descale_bytes = tiles * kblocks * 16 * sizeof(float);
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_blockquant_pack(const uint8_t* b_host, const float* scales_host, int N, int K, int bits, int block, uint8_t* packed_w_host,
+                            float* packed_descale_host)
+{
+    NCNNHIP_REQUIRE(b_host && scales_host && packed_w_host && packed_descale_host, "ncnnhip_blockquant_pack: null pointer");
+    NCNNHIP_REQUIRE(bits == 8, "ncnnhip_blockquant_pack: only 8-bit weights have a packed layout");
+    NCNNHIP_REQUIRE(block == 64 || block == 128, "ncnnhip_blockquant_pack: block %d", block);
+    const int tiles = (N + 15) / 16, kblocks = (K + 63) / 64, nblk = (K + block - 1) / block;
+    for (int t = 0; t < tiles; t++)
+        for (int kb = 0; kb < kblocks; kb++)
+        {
+            uint8_t* wt = packed_w_host + ((size_t)t * kblocks + kb) * 1024;
+            float* dt = packed_descale_host + ((size_t)t * kblocks + kb) * 16;
+            for (int l = 0; l < 64; l++)
+                for (int e = 0; e < 16; e++)
+                {
+                    const int j = t * 16 + (l & 15), k = kb * 64 + (l >> 4) * 16 + e;
+                    const int q = (j < N && k < K) ? (int)(int8_t)b_host[(size_t)j * K + k] : 0;
+                    wt[l * 16 + e] = (uint8_t)(q + 128);
+                }
+            for (int r = 0; r < 16; r++)
+            {
+                const int j = t * 16 + r;
+                // same single rounded division the reference performs per block (gemm.cpp:465)
+                volatile float sc = j < N ? scales_host[(size_t)j * nblk + (size_t)kb * 64 / block] : 1.f;
+                dt[r] = j < N ? 1.f / sc : 0.f;
+            }
+        }
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
+                                        const float* packed_descale_dev, const float* c_dev, int broadcast_type_c, float alpha, float beta,
+                                        float* out_dev, size_t out_stride, void* stream)
+{
+    NCNNHIP_REQUIRE(a_dev && packed_w_dev && packed_descale_dev && out_dev, "ncnnhip_gemm_blockquant_packed_f16a: null pointer");
+    NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1 && K % 16 == 0, "ncnnhip_gemm_blockquant_packed_f16a: bad shape %d %d %d (K must be a multiple of 16)", M, N, K);
+    NCNNHIP_REQUIRE(a_stride >= (size_t)K && a_stride % 8 == 0 && al16(a_dev), "ncnnhip_gemm_blockquant_packed_f16a: activation rows must be 16-byte aligned");
+    NCNNHIP_REQUIRE(out_stride >= (size_t)N, "ncnnhip_gemm_blockquant_packed_f16a: output stride too small");
+    const int bt = c_dev ? broadcast_type_c : -1;
+    NCNNHIP_REQUIRE(bt >= -1 && bt <= 4, "ncnnhip_gemm_blockquant_packed_f16a: C broadcast %d", bt);
+    NCNNHIP_REQUIRE((size_t)(K + 63) / 64 * 64 <= 60 * 1024, "ncnnhip_gemm_blockquant_packed_f16a: K %d too large for the descale stage", K);
+    const int tiles = (N + 15) / 16, kblocks = (K + 63) / 64;
+    const __half* ah = reinterpret_cast<const __half*>(a_dev);
+    for (int m0 = 0; m0 < M; m0 += 16)
+    {
+        const int mc = M - m0 < 16 ? M - m0 : 16;
+        const float* cc = c_dev;
+        if (cc && (bt == 1 || bt == 2)) cc += m0;
+        if (cc && bt == 3) cc += (size_t)m0 * N;
+        hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS, BQ_MFMA_U>), dim3(tiles), dim3(256), (size_t)kblocks * 64, as_stream(stream), ah + (size_t)m0 * a_stride, a_stride, mc, N, K,
+                           kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev), reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha,
+                           beta, out_dev + (size_t)m0 * out_stride, out_stride);
+    }
+    return launch_status("blockquant8_mfma_kernel");
 }
 
 int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* b_dev, int bits,
@@ -195,18 +611,8 @@ int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, 
     if (ret) return ret;
     NCNNHIP_REQUIRE(bits == 8 && K % 16 == 0 && al16(b_dev), "ncnnhip_gemm_blockquant_f16a: needs 8-bit weights, K %% 16 == 0, aligned rows");
     NCNNHIP_REQUIRE(a_stride >= (size_t)K && out_stride >= (size_t)N, "ncnnhip_gemm_blockquant_f16a: stride too small");
-    const int nblk = (K + block - 1) / block;
-    const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
-    dim3 grid(ceil_div(N, 4));
-    const __half* ah = reinterpret_cast<const __half*>(a_dev);
-    const int8_t* b8 = reinterpret_cast<const int8_t*>(b_dev);
-    if (M == 1)
-        hipLaunchKernelGGL((blockquant8_kernel<__half, 1>), grid, dim3(256), 0, as_stream(stream), ah, a_stride, M, N, K, b8, shift, nblk, scales_dev,
-                           (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride);
-    else
-        hipLaunchKernelGGL((blockquant8_kernel<__half, 4>), grid, dim3(256), 0, as_stream(stream), ah, a_stride, M, N, K, b8, shift, nblk, scales_dev,
-                           (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride);
-    return launch_status("blockquant8_kernel<half>");
+    return launch_blockquant8<__half>(reinterpret_cast<const __half*>(a_dev), a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev), block,
+                                      scales_dev, (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride, as_stream(stream));
 }
 
 } // extern "C"

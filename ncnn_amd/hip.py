@@ -69,6 +69,10 @@ _SIGNATURES = {
                           C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_blockquant": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_blockquant_packed_size": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "ncnnhip_blockquant_pack": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_blockquant_packed_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                            C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_blockquant_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                      C.c_void_p, C.c_size_t, C.c_void_p],
 }
@@ -309,4 +313,26 @@ class Runtime:
             dc = self.up(None if c is None else np.asarray(c, np.float32))
             check(lib().ncnnhip_gemm_blockquant(da.ptr, k, m, n, k, db.ptr, bits, block, ds.ptr, _ptr(dis), _ptr(dc),
                                                 broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
+        return dout.to_numpy(self.stream)
+
+    def blockquant_pack(self, b_packed, scales, block):
+        """Host-side repack of 8-bit block-quantised weights into the matrix-core tile layout."""
+        b_packed = np.ascontiguousarray(b_packed, np.uint8)
+        scales = np.ascontiguousarray(scales, np.float32)
+        n, k = b_packed.shape
+        wb, db = C.c_size_t(), C.c_size_t()
+        check(lib().ncnnhip_blockquant_packed_size(n, k, block, C.byref(wb), C.byref(db)))
+        pw = np.empty(wb.value, np.uint8)
+        pd = np.empty(db.value // 4, np.float32)
+        check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, 8, block, pw.ctypes.data, pd.ctypes.data))
+        return pw, pd
+
+    def gemm_blockquant_packed(self, a_half, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0):
+        a_half = np.ascontiguousarray(a_half, np.float16)
+        m, k = a_half.shape
+        da, dw_, dd = self.up(a_half), self.up(pw), self.up(pd)
+        dc = self.up(None if c is None else np.asarray(c, np.float32))
+        dout = DeviceBuffer.empty((m, n), np.float32)
+        check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, _ptr(dc), broadcast_type_c if c is not None else -1,
+                                                        alpha, beta, dout.ptr, n, self.stream))
         return dout.to_numpy(self.stream)

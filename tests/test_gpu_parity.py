@@ -265,6 +265,20 @@ def test_blockquant_decode_shapes_fp32_and_fp16_activations(rt, m, n, k):
     assert np.array_equal(got16, got32)  # fp16-representable activations: both entry points see the same numbers
 
 
+@pytest.mark.parametrize("m,n,k,block,bt", [(1, 512, 4096, 64, -1), (4, 256, 4096, 64, 4), (16, 256, 4096, 64, 3), (16, 250, 11008, 64, -1),
+                                            (3, 37, 208, 64, 1), (1, 16, 64, 64, 0), (20, 64, 1024, 128, 2), (7, 100, 4096 + 48, 128, -1)])
+def test_blockquant_packed_matrix_core_path(rt, m, n, k, block, bt):
+    _say("blockquant packed", m, n, k, block, bt)
+    a, packed, scales = cases.blockquant_case(m + n + k + block, m, n, k, 8, block)
+    rng = np.random.default_rng(bt + 50)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    pw, pd = rt.blockquant_pack(packed, scales, block)
+    got = rt.gemm_blockquant_packed(a.astype(np.float16), pw, pd, n, c, bt, 0.75, 1.5)
+    _bq_check(got, a, packed, scales, 8, block, None, c, bt, 0.75, 1.5)
+
+
 def test_blockquant_exact_on_power_of_two_data(rt):
     k, n, m = 128, 6, 2
     rng = np.random.default_rng(3)
