@@ -1,0 +1,114 @@
+/*
+ * C ABI of the host runtime (libncnn_amd.so): the subset of ncnn's own C API (src/c_api.h) that
+ * drives the int8 path end to end -- load_param, load_model, create_extractor, input, extract --
+ * plus the one call that installs the MI355X layers.  Names, argument meaning and return values
+ * are those of src/c_api.h at the cited lines, so a program written against ncnn's C API links
+ * against this library unchanged for these calls.
+ */
+#ifndef NCNN_AMD_C_API_H
+#define NCNN_AMD_C_API_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#pragma GCC visibility push(default)
+
+typedef struct __ncnn_allocator_t* ncnn_allocator_t; /* always NULL here: the library's own host allocator */
+typedef struct __ncnn_option_t* ncnn_option_t;
+typedef struct __ncnn_mat_t* ncnn_mat_t;
+typedef struct __ncnn_net_t* ncnn_net_t;
+typedef struct __ncnn_extractor_t* ncnn_extractor_t;
+
+/* src/c_api.h:58-95 */
+ncnn_option_t ncnn_option_create(void);
+void ncnn_option_destroy(ncnn_option_t opt);
+void ncnn_option_set_num_threads(ncnn_option_t opt, int num_threads);
+void ncnn_option_set_lightmode(ncnn_option_t opt, int enable); /* Option::lightmode */
+void ncnn_option_set_use_int8_inference(ncnn_option_t opt, int enable); /* Option::use_int8_inference */
+int ncnn_option_get_use_int8_inference(const ncnn_option_t opt);
+
+/* src/c_api.h:134-165; data is caller-owned memory laid out as ncnn::Mat lays it out */
+ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_2d_elem(int w, int h, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
+/* owning, batched 3-D blob (Mat::create(w,h,c,elemsize,elempack,n)); fill it through ncnn_mat_get_batch_data */
+ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, size_t elemsize, int n);
+void ncnn_mat_destroy(ncnn_mat_t mat);
+int ncnn_mat_get_dims(const ncnn_mat_t mat);
+int ncnn_mat_get_w(const ncnn_mat_t mat);
+int ncnn_mat_get_h(const ncnn_mat_t mat);
+int ncnn_mat_get_d(const ncnn_mat_t mat);
+int ncnn_mat_get_c(const ncnn_mat_t mat);
+int ncnn_mat_get_n(const ncnn_mat_t mat);
+size_t ncnn_mat_get_elemsize(const ncnn_mat_t mat);
+int ncnn_mat_get_elempack(const ncnn_mat_t mat);
+size_t ncnn_mat_get_cstep(const ncnn_mat_t mat);
+size_t ncnn_mat_get_nstep(const ncnn_mat_t mat);
+void* ncnn_mat_get_data(const ncnn_mat_t mat);
+void* ncnn_mat_get_batch_data(const ncnn_mat_t mat, int b);
+
+/* src/c_api.h:338-388 */
+ncnn_net_t ncnn_net_create(void);
+void ncnn_net_destroy(ncnn_net_t net);
+ncnn_option_t ncnn_net_get_option(ncnn_net_t net); /* borrowed: the net's own Option */
+void ncnn_net_set_option(ncnn_net_t net, ncnn_option_t opt);
+int ncnn_net_load_param(ncnn_net_t net, const char* path);
+int ncnn_net_load_model(ncnn_net_t net, const char* path);
+int ncnn_net_load_param_memory(ncnn_net_t net, const char* mem);
+size_t ncnn_net_load_model_memory(ncnn_net_t net, const unsigned char* mem);
+int ncnn_net_get_input_count(const ncnn_net_t net);
+int ncnn_net_get_output_count(const ncnn_net_t net);
+const char* ncnn_net_get_input_name(const ncnn_net_t net, int i);
+const char* ncnn_net_get_output_name(const ncnn_net_t net, int i);
+
+/* src/c_api.h:396-403 */
+ncnn_extractor_t ncnn_extractor_create(ncnn_net_t net);
+void ncnn_extractor_destroy(ncnn_extractor_t ex);
+void ncnn_extractor_set_option(ncnn_extractor_t ex, const ncnn_option_t opt);
+int ncnn_extractor_input(ncnn_extractor_t ex, const char* name, const ncnn_mat_t mat);
+int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* mat);
+
+/*
+ * Installs the MI355X implementations of Convolution, ConvolutionDepthWise, InnerProduct and
+ * Gemm on a net: four Net::register_custom_layer calls under the built-in type names
+ * (src/net.cpp:1214-1237, the route tests/test_squeezenet.cpp:320-404 exercises).  Call it
+ * before load_param.  Returns 0, or -1 if a registration was refused.
+ */
+int ncnnhip_register_int8_layers(ncnn_net_t net);
+
+/* Gives the extractor its own device stream and buffer pool (one hipStream per Extractor) by
+ * installing a host blob allocator that carries them; the allocator lives until
+ * ncnnhip_extractor_detach_stream or process end.  Optional: without it a per-thread stream is used. */
+void* ncnnhip_extractor_attach_stream(ncnn_extractor_t ex);
+void ncnnhip_extractor_detach_stream(void* handle);
+
+/* Introspection used by the host-logic tests: fields a layer holds after load_param / load_model. */
+int ncnn_net_get_layer_count(const ncnn_net_t net);
+const char* ncnn_net_get_layer_type(const ncnn_net_t net, int i);
+const char* ncnn_net_get_layer_name(const ncnn_net_t net, int i);
+int ncnn_net_get_layer_flags(const ncnn_net_t net, int i); /* bit0 one_blob_only, bit1 support_inplace, bit2 support_int8_storage, bit3 support_batch, bit4 support_packing */
+int ncnn_net_get_blob_count(const ncnn_net_t net);
+const char* ncnn_net_get_blob_name(const ncnn_net_t net, int i);
+int ncnn_net_get_blob_producer(const ncnn_net_t net, int i);
+int ncnn_net_get_blob_consumer(const ncnn_net_t net, int i);
+
+/* Parses one .param key=value tail ("0=64 1=3 10=0.0,6.0") and reports slot `id`: returns the slot
+ * type (0 unset, 2 int, 3 float, 5 int array, 6 float array, 7 string, -1 parse error); the raw
+ * 32-bit payload (or the array length) goes to *value_bits, array elements to array_bits[0..cap). */
+int ncnn_paramdict_probe(const char* text, int id, unsigned int* value_bits, unsigned int* array_bits, int cap);
+
+/* Reads one blob of `w` elements of load-type `type` (0 tagged / 1 raw fp32) from a .bin image and
+ * copies it as fp32 or int8 to out; returns the element size (4 or 1), 0 on failure. *consumed =
+ * bytes of the image used. */
+int ncnn_modelbin_probe(const unsigned char* mem, int w, int type, void* out, size_t* consumed);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NCNN_AMD_C_API_H */

@@ -46,8 +46,30 @@ def build_kernels(jobs=8):
     return LIBNCNNHIP
 
 
+HOST_SOURCES = ["ncnn/allocator.cpp", "ncnn/mat.cpp", "ncnn/option.cpp", "ncnn/datareader.cpp", "ncnn/paramdict.cpp", "ncnn/modelbin.cpp",
+                "ncnn/layer.cpp", "ncnn/net.cpp", "layers/glue_layers.cpp", "layers/hip_support.cpp", "layers/convolution_hip.cpp",
+                "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "c_api.cpp"]
+LIBNCNN_AMD = os.path.join(LIBDIR, "libncnn_amd.so")
+
+# strict IEEE on the host too: the load-time weight quantiser and the scale folding must round
+# exactly like the reference's scalar code
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fopenmp", "-fno-fast-math", "-ffp-contract=off", "-fvisibility=hidden", "-Wall", "-Wextra",
+              "-Wno-unused-parameter"]
+
+
+def build_host():
+    """libncnn_amd.so: the ncnn-API mirror (Mat, ParamDict, ModelBin, Net, Extractor), the four HIP layers and the C API.
+    It links against libncnnhip.so, which carries the kernels."""
+    hostdir = os.path.join(PKG, "host")
+    srcs = [os.path.join(hostdir, s) for s in HOST_SOURCES]
+    _run(["g++"] + HOST_FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", hostdir, "-shared", "-o", LIBNCNN_AMD] + srcs
+         + ["-L", LIBDIR, "-lncnnhip", "-Wl,-rpath,$ORIGIN"])
+    return LIBNCNN_AMD
+
+
 def build_all():
     build_kernels()
+    build_host()
 
 
 if __name__ == "__main__":

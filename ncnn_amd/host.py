@@ -1,0 +1,257 @@
+"""ctypes binding of libncnn_amd.so (include/ncnn_amd_c_api.h): the ncnn-API mirror with the HIP layers.
+
+The calls mirror ncnn's C API one to one: create a net, register the int8 layers, load_param, load_model,
+create an extractor, input, extract."""
+import ctypes as C
+import os
+import struct
+import tempfile
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_PKG, "lib", "libncnn_amd.so")
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise RuntimeError("%s is missing: build it with python ncnn_amd/build.py" % _LIB)
+        from . import hip
+        hip.lib()  # libncnnhip.so first (same directory, found through rpath as well)
+        L = C.CDLL(_LIB)
+        vp, ci, cs = C.c_void_p, C.c_int, C.c_size_t
+        sig = {
+            "ncnn_option_create": (vp, []), "ncnn_option_destroy": (None, [vp]), "ncnn_option_set_num_threads": (None, [vp, ci]),
+            "ncnn_option_set_lightmode": (None, [vp, ci]), "ncnn_option_set_use_int8_inference": (None, [vp, ci]),
+            "ncnn_option_get_use_int8_inference": (ci, [vp]),
+            "ncnn_mat_create_external_1d_elem": (vp, [ci, vp, cs, ci, vp]), "ncnn_mat_create_external_2d_elem": (vp, [ci, ci, vp, cs, ci, vp]),
+            "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, cs, ci]),
+            "ncnn_mat_destroy": (None, [vp]), "ncnn_mat_get_dims": (ci, [vp]), "ncnn_mat_get_w": (ci, [vp]), "ncnn_mat_get_h": (ci, [vp]),
+            "ncnn_mat_get_d": (ci, [vp]), "ncnn_mat_get_c": (ci, [vp]), "ncnn_mat_get_n": (ci, [vp]), "ncnn_mat_get_elemsize": (cs, [vp]),
+            "ncnn_mat_get_elempack": (ci, [vp]), "ncnn_mat_get_cstep": (cs, [vp]), "ncnn_mat_get_nstep": (cs, [vp]),
+            "ncnn_mat_get_data": (vp, [vp]), "ncnn_mat_get_batch_data": (vp, [vp, ci]),
+            "ncnn_net_create": (vp, []), "ncnn_net_destroy": (None, [vp]), "ncnn_net_get_option": (vp, [vp]), "ncnn_net_set_option": (None, [vp, vp]),
+            "ncnn_net_load_param": (ci, [vp, C.c_char_p]), "ncnn_net_load_model": (ci, [vp, C.c_char_p]),
+            "ncnn_net_load_param_memory": (ci, [vp, C.c_char_p]), "ncnn_net_load_model_memory": (cs, [vp, C.c_char_p]),
+            "ncnn_net_get_input_count": (ci, [vp]), "ncnn_net_get_output_count": (ci, [vp]),
+            "ncnn_net_get_input_name": (C.c_char_p, [vp, ci]), "ncnn_net_get_output_name": (C.c_char_p, [vp, ci]),
+            "ncnn_extractor_create": (vp, [vp]), "ncnn_extractor_destroy": (None, [vp]), "ncnn_extractor_set_option": (None, [vp, vp]),
+            "ncnn_extractor_input": (ci, [vp, C.c_char_p, vp]), "ncnn_extractor_extract": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
+            "ncnnhip_register_int8_layers": (ci, [vp]), "ncnnhip_extractor_attach_stream": (vp, [vp]), "ncnnhip_extractor_detach_stream": (None, [vp]),
+            "ncnn_net_get_layer_count": (ci, [vp]), "ncnn_net_get_layer_type": (C.c_char_p, [vp, ci]), "ncnn_net_get_layer_name": (C.c_char_p, [vp, ci]),
+            "ncnn_net_get_layer_flags": (ci, [vp, ci]), "ncnn_net_get_blob_count": (ci, [vp]), "ncnn_net_get_blob_name": (C.c_char_p, [vp, ci]),
+            "ncnn_net_get_blob_producer": (ci, [vp, ci]), "ncnn_net_get_blob_consumer": (ci, [vp, ci]),
+            "ncnn_paramdict_probe": (ci, [C.c_char_p, ci, C.POINTER(C.c_uint), C.POINTER(C.c_uint), ci]),
+            "ncnn_modelbin_probe": (ci, [C.c_char_p, ci, ci, vp, C.POINTER(cs)]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+# ---- probes (host logic tests) ---------------------------------------------------------------
+def paramdict_probe(text, pid):
+    v = C.c_uint(0)
+    arr = (C.c_uint * 64)()
+    t = lib().ncnn_paramdict_probe(text.encode(), pid, C.byref(v), arr, 64)
+    return t, v.value, list(arr)
+
+
+def modelbin_probe(blob, w, load_type):
+    out = np.zeros(w * 4 + 8, np.uint8)
+    used = C.c_size_t(0)
+    es = lib().ncnn_modelbin_probe(bytes(blob) + b"\0" * 16, w, load_type, out.ctypes.data, C.byref(used))
+    if es == 0:
+        return None, used.value
+    dt = np.int8 if es == 1 else np.float32
+    return out[: w * es].view(dt).copy(), used.value
+
+
+def _pad4(b):
+    return b + b"\0" * (-len(b) % 4)
+
+
+def tagged_fp32(a):
+    return struct.pack("<I", 0) + np.ascontiguousarray(a, np.float32).tobytes()
+
+
+def tagged_fp16(a):
+    return struct.pack("<I", 0x01306B47) + _pad4(np.ascontiguousarray(a, np.float16).tobytes())
+
+
+def tagged_int8(a):
+    return struct.pack("<I", 0x000D4B38) + _pad4(np.ascontiguousarray(a, np.int8).tobytes())
+
+
+# ---- Mat -------------------------------------------------------------------------------------------
+class Mat:
+    """Owns an ncnn_mat_t; numpy <-> ncnn::Mat layout conversion (plane padding to 16 bytes, batch stride)."""
+
+    def __init__(self, handle, keep=None):
+        self.h_ = handle
+        self._keep = keep
+
+    def __del__(self):
+        try:
+            if self.h_:
+                lib().ncnn_mat_destroy(self.h_)
+        except Exception:
+            pass
+
+    dims = property(lambda s: lib().ncnn_mat_get_dims(s.h_))
+    w = property(lambda s: lib().ncnn_mat_get_w(s.h_))
+    h = property(lambda s: lib().ncnn_mat_get_h(s.h_))
+    c = property(lambda s: lib().ncnn_mat_get_c(s.h_))
+    n = property(lambda s: lib().ncnn_mat_get_n(s.h_))
+    elemsize = property(lambda s: lib().ncnn_mat_get_elemsize(s.h_))
+    cstep = property(lambda s: lib().ncnn_mat_get_cstep(s.h_))
+    nstep = property(lambda s: lib().ncnn_mat_get_nstep(s.h_))
+
+    @classmethod
+    def batch3d(cls, w, h, c, elemsize, n):
+        return cls(lib().ncnn_mat_create_3d_batch(w, h, c, elemsize, n))
+
+    @classmethod
+    def from_numpy(cls, a):
+        """1-D [w], 2-D [h][w], 3-D [c][h][w] or 4-D [n][c][h][w] (a batch of 3-D blobs); fp32 or int8."""
+        a = np.ascontiguousarray(a)
+        assert a.dtype in (np.float32, np.int8)
+        es = a.dtype.itemsize
+        if a.ndim == 1:
+            return cls(lib().ncnn_mat_create_external_1d_elem(a.shape[0], a.ctypes.data, es, 1, None), keep=a)
+        if a.ndim == 2:
+            return cls(lib().ncnn_mat_create_external_2d_elem(a.shape[1], a.shape[0], a.ctypes.data, es, 1, None), keep=a)
+        if a.ndim == 3:
+            a = a[None]
+        n, c, h, w = a.shape
+        m = cls.batch3d(w, h, c, es, n)
+        for b in range(n):
+            base = lib().ncnn_mat_get_batch_data(m.h_, b)
+            buf = np.ctypeslib.as_array(C.cast(base, C.POINTER(C.c_uint8)), shape=(m.cstep * c * es,)).view(a.dtype).reshape(c, m.cstep)
+            buf[:, : h * w] = a[b].reshape(c, h * w)
+        return m
+
+    def to_numpy(self):
+        """1-D -> [w], 2-D -> [h][w], 3-D -> [c][h][w]; a batch adds a leading [n]."""
+        es = self.elemsize
+        dt = np.int8 if es == 1 else np.float32
+        d, w, h, c, n = self.dims, self.w, self.h, self.c, self.n
+        samples = []
+        for b in range(n):
+            base = lib().ncnn_mat_get_batch_data(self.h_, b)
+            if d == 1:
+                a = np.ctypeslib.as_array(C.cast(base, C.POINTER(C.c_uint8)), shape=(w * es,)).view(dt).copy()
+            elif d == 2:
+                a = np.ctypeslib.as_array(C.cast(base, C.POINTER(C.c_uint8)), shape=(w * h * es,)).view(dt).reshape(h, w).copy()
+            else:
+                buf = np.ctypeslib.as_array(C.cast(base, C.POINTER(C.c_uint8)), shape=(self.cstep * c * es,)).view(dt).reshape(c, self.cstep)
+                a = buf[:, : h * w].reshape(c, h, w).copy()
+            samples.append(a)
+        return np.stack(samples) if n > 1 else samples[0]
+
+
+# ---- Net / Extractor -------------------------------------------------------------------------------
+class Net:
+    def __init__(self):
+        self.h_ = lib().ncnn_net_create()
+
+    def __del__(self):
+        try:
+            if self.h_:
+                lib().ncnn_net_destroy(self.h_)
+                self.h_ = None
+        except Exception:
+            pass
+
+    def register_int8_layers(self):
+        return lib().ncnnhip_register_int8_layers(self.h_)
+
+    def set_use_int8_inference(self, enable):
+        lib().ncnn_option_set_use_int8_inference(lib().ncnn_net_get_option(self.h_), int(enable))
+
+    def set_lightmode(self, enable):
+        lib().ncnn_option_set_lightmode(lib().ncnn_net_get_option(self.h_), int(enable))
+
+    def load_param(self, path):
+        return lib().ncnn_net_load_param(self.h_, path.encode())
+
+    def load_param_mem(self, text):
+        return lib().ncnn_net_load_param_memory(self.h_, text.encode())
+
+    def load_model(self, path):
+        return lib().ncnn_net_load_model(self.h_, path.encode())
+
+    def load_model_mem(self, blob):
+        # through a file so that the int status is visible (the memory variant returns bytes consumed, like ncnn's)
+        with tempfile.NamedTemporaryFile(suffix=".bin") as f:
+            f.write(blob)
+            f.flush()
+            return self.load_model(f.name)
+
+    def layer_types(self):
+        return [lib().ncnn_net_get_layer_type(self.h_, i).decode() for i in range(lib().ncnn_net_get_layer_count(self.h_))]
+
+    def layer_names(self):
+        return [lib().ncnn_net_get_layer_name(self.h_, i).decode() for i in range(lib().ncnn_net_get_layer_count(self.h_))]
+
+    def layer_flags(self):
+        return [lib().ncnn_net_get_layer_flags(self.h_, i) for i in range(lib().ncnn_net_get_layer_count(self.h_))]
+
+    def input_names(self):
+        return [lib().ncnn_net_get_input_name(self.h_, i).decode() for i in range(lib().ncnn_net_get_input_count(self.h_))]
+
+    def output_names(self):
+        return [lib().ncnn_net_get_output_name(self.h_, i).decode() for i in range(lib().ncnn_net_get_output_count(self.h_))]
+
+    def blobs(self):
+        out = {}
+        for i in range(lib().ncnn_net_get_blob_count(self.h_)):
+            out[lib().ncnn_net_get_blob_name(self.h_, i).decode()] = (lib().ncnn_net_get_blob_producer(self.h_, i), lib().ncnn_net_get_blob_consumer(self.h_, i))
+        return out
+
+    def create_extractor(self, own_stream=True):
+        return Extractor(self, own_stream)
+
+
+class Extractor:
+    def __init__(self, net, own_stream=True):
+        self.net = net
+        self.h_ = lib().ncnn_extractor_create(net.h_)
+        self.stream_handle = lib().ncnnhip_extractor_attach_stream(self.h_) if own_stream else None
+        self._inputs = []
+
+    def __del__(self):
+        try:
+            if self.h_:
+                lib().ncnn_extractor_destroy(self.h_)
+                self.h_ = None
+            if self.stream_handle:
+                lib().ncnnhip_extractor_detach_stream(self.stream_handle)
+                self.stream_handle = None
+        except Exception:
+            pass
+
+    def set_lightmode(self, enable):
+        opt = lib().ncnn_option_create()
+        lib().ncnn_option_set_lightmode(opt, int(enable))
+        lib().ncnn_extractor_set_option(self.h_, opt)
+        lib().ncnn_option_destroy(opt)
+
+    def input(self, name, array):
+        m = array if isinstance(array, Mat) else Mat.from_numpy(array)
+        self._inputs.append(m)
+        return lib().ncnn_extractor_input(self.h_, name.encode(), m.h_)
+
+    def extract(self, name):
+        out = C.c_void_p()
+        ret = lib().ncnn_extractor_extract(self.h_, name.encode(), C.byref(out))
+        m = Mat(out.value)
+        if ret != 0:
+            raise RuntimeError("extract(%s) returned %d" % (name, ret))
+        return m.to_numpy()

@@ -1,0 +1,304 @@
+#include "ncnn_amd_c_api.h"
+
+#include <string.h>
+
+#include "layers/hip_layers.h"
+#include "layers/hip_support.h"
+#include "ncnn/datareader.h"
+#include "ncnn/modelbin.h"
+#include "ncnn/net.h"
+#include "ncnn/paramdict.h"
+
+using namespace ncnn;
+
+static Option* O(ncnn_option_t p)
+{
+    return (Option*)p;
+}
+static Mat* M(ncnn_mat_t p)
+{
+    return (Mat*)p;
+}
+static Net* N(ncnn_net_t p)
+{
+    return (Net*)p;
+}
+static Extractor* E(ncnn_extractor_t p)
+{
+    return (Extractor*)p;
+}
+
+extern "C" {
+
+ncnn_option_t ncnn_option_create(void)
+{
+    return (ncnn_option_t) new Option;
+}
+void ncnn_option_destroy(ncnn_option_t opt)
+{
+    delete O(opt);
+}
+void ncnn_option_set_num_threads(ncnn_option_t opt, int num_threads)
+{
+    O(opt)->num_threads = num_threads;
+}
+void ncnn_option_set_lightmode(ncnn_option_t opt, int enable)
+{
+    O(opt)->lightmode = enable != 0;
+}
+void ncnn_option_set_use_int8_inference(ncnn_option_t opt, int enable)
+{
+    O(opt)->use_int8_inference = enable != 0;
+}
+int ncnn_option_get_use_int8_inference(const ncnn_option_t opt)
+{
+    return O(opt)->use_int8_inference;
+}
+
+ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t)
+{
+    Mat* m = new Mat(w, data, elemsize);
+    m->elempack = elempack;
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_external_2d_elem(int w, int h, void* data, size_t elemsize, int elempack, ncnn_allocator_t)
+{
+    Mat* m = new Mat(w, h, data, elemsize);
+    m->elempack = elempack;
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, size_t elemsize, int elempack, ncnn_allocator_t)
+{
+    Mat* m = new Mat(w, h, c, data, elemsize);
+    m->elempack = elempack;
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, size_t elemsize, int n)
+{
+    Mat* m = new Mat;
+    m->create(w, h, c, elemsize, 1, n, (Allocator*)0);
+    return (ncnn_mat_t)m;
+}
+void ncnn_mat_destroy(ncnn_mat_t mat)
+{
+    delete M(mat);
+}
+int ncnn_mat_get_dims(const ncnn_mat_t mat)
+{
+    return M(mat)->dims;
+}
+int ncnn_mat_get_w(const ncnn_mat_t mat)
+{
+    return M(mat)->w;
+}
+int ncnn_mat_get_h(const ncnn_mat_t mat)
+{
+    return M(mat)->h;
+}
+int ncnn_mat_get_d(const ncnn_mat_t mat)
+{
+    return M(mat)->d;
+}
+int ncnn_mat_get_c(const ncnn_mat_t mat)
+{
+    return M(mat)->c;
+}
+int ncnn_mat_get_n(const ncnn_mat_t mat)
+{
+    return M(mat)->n;
+}
+size_t ncnn_mat_get_elemsize(const ncnn_mat_t mat)
+{
+    return M(mat)->elemsize;
+}
+int ncnn_mat_get_elempack(const ncnn_mat_t mat)
+{
+    return M(mat)->elempack;
+}
+size_t ncnn_mat_get_cstep(const ncnn_mat_t mat)
+{
+    return M(mat)->cstep;
+}
+size_t ncnn_mat_get_nstep(const ncnn_mat_t mat)
+{
+    return M(mat)->nstep;
+}
+void* ncnn_mat_get_data(const ncnn_mat_t mat)
+{
+    return M(mat)->data;
+}
+void* ncnn_mat_get_batch_data(const ncnn_mat_t mat, int b)
+{
+    return (unsigned char*)M(mat)->data + M(mat)->nstep * b * M(mat)->elemsize;
+}
+
+ncnn_net_t ncnn_net_create(void)
+{
+    return (ncnn_net_t) new Net;
+}
+void ncnn_net_destroy(ncnn_net_t net)
+{
+    delete N(net);
+}
+ncnn_option_t ncnn_net_get_option(ncnn_net_t net)
+{
+    return (ncnn_option_t)&N(net)->opt;
+}
+void ncnn_net_set_option(ncnn_net_t net, ncnn_option_t opt)
+{
+    N(net)->opt = *O(opt);
+}
+int ncnn_net_load_param(ncnn_net_t net, const char* path)
+{
+    return N(net)->load_param(path);
+}
+int ncnn_net_load_model(ncnn_net_t net, const char* path)
+{
+    return N(net)->load_model(path);
+}
+int ncnn_net_load_param_memory(ncnn_net_t net, const char* mem)
+{
+    return N(net)->load_param_mem(mem);
+}
+size_t ncnn_net_load_model_memory(ncnn_net_t net, const unsigned char* mem)
+{
+    return N(net)->load_model(mem);
+}
+int ncnn_net_get_input_count(const ncnn_net_t net)
+{
+    return (int)N(net)->input_names().size();
+}
+int ncnn_net_get_output_count(const ncnn_net_t net)
+{
+    return (int)N(net)->output_names().size();
+}
+const char* ncnn_net_get_input_name(const ncnn_net_t net, int i)
+{
+    return N(net)->input_names()[(size_t)i];
+}
+const char* ncnn_net_get_output_name(const ncnn_net_t net, int i)
+{
+    return N(net)->output_names()[(size_t)i];
+}
+
+ncnn_extractor_t ncnn_extractor_create(ncnn_net_t net)
+{
+    return (ncnn_extractor_t) new Extractor(N(net)->create_extractor());
+}
+void ncnn_extractor_destroy(ncnn_extractor_t ex)
+{
+    delete E(ex);
+}
+void ncnn_extractor_set_option(ncnn_extractor_t ex, const ncnn_option_t opt)
+{
+    E(ex)->set_light_mode(O(opt)->lightmode);
+    E(ex)->set_num_threads(O(opt)->num_threads);
+}
+int ncnn_extractor_input(ncnn_extractor_t ex, const char* name, const ncnn_mat_t mat)
+{
+    return E(ex)->input(name, *M(mat));
+}
+int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* mat)
+{
+    Mat out;
+    int ret = E(ex)->extract(name, out);
+    *mat = (ncnn_mat_t) new Mat(out);
+    return ret;
+}
+
+int ncnnhip_register_int8_layers(ncnn_net_t net)
+{
+    using namespace ncnn_amd;
+    int ret = 0;
+    ret |= N(net)->register_custom_layer("Convolution", Convolution_hip_creator, hip_layer_destroyer, net);
+    ret |= N(net)->register_custom_layer("ConvolutionDepthWise", ConvolutionDepthWise_hip_creator, hip_layer_destroyer, net);
+    ret |= N(net)->register_custom_layer("InnerProduct", InnerProduct_hip_creator, hip_layer_destroyer, net);
+    ret |= N(net)->register_custom_layer("Gemm", Gemm_hip_creator, hip_layer_destroyer, net);
+    return ret ? -1 : 0;
+}
+
+void* ncnnhip_extractor_attach_stream(ncnn_extractor_t ex)
+{
+    ncnn_amd::HipBlobAllocator* a = new ncnn_amd::HipBlobAllocator;
+    E(ex)->set_blob_allocator(a);
+    return a;
+}
+void ncnnhip_extractor_detach_stream(void* handle)
+{
+    delete (ncnn_amd::HipBlobAllocator*)handle;
+}
+
+int ncnn_net_get_layer_count(const ncnn_net_t net)
+{
+    return (int)N(net)->layers().size();
+}
+const char* ncnn_net_get_layer_type(const ncnn_net_t net, int i)
+{
+    return N(net)->layers()[(size_t)i]->type.c_str();
+}
+const char* ncnn_net_get_layer_name(const ncnn_net_t net, int i)
+{
+    return N(net)->layers()[(size_t)i]->name.c_str();
+}
+int ncnn_net_get_layer_flags(const ncnn_net_t net, int i)
+{
+    const Layer* l = N(net)->layers()[(size_t)i];
+    return (l->one_blob_only ? 1 : 0) | (l->support_inplace ? 2 : 0) | (l->support_int8_storage ? 4 : 0) | (l->support_batch ? 8 : 0) | (l->support_packing ? 16 : 0);
+}
+int ncnn_net_get_blob_count(const ncnn_net_t net)
+{
+    return (int)N(net)->blobs().size();
+}
+const char* ncnn_net_get_blob_name(const ncnn_net_t net, int i)
+{
+    return N(net)->blobs()[(size_t)i].name.c_str();
+}
+int ncnn_net_get_blob_producer(const ncnn_net_t net, int i)
+{
+    return N(net)->blobs()[(size_t)i].producer;
+}
+int ncnn_net_get_blob_consumer(const ncnn_net_t net, int i)
+{
+    return N(net)->blobs()[(size_t)i].consumer;
+}
+
+int ncnn_paramdict_probe(const char* text, int id, unsigned int* value_bits, unsigned int* array_bits, int cap)
+{
+    const unsigned char* cursor = (const unsigned char*)text;
+    DataReaderFromMemory dr(cursor);
+    ParamDict pd;
+    if (pd.load_param(dr) != 0) return -1;
+    const int t = pd.type(id);
+    if (t == 2 || t == 3)
+    {
+        const int raw = pd.get(id, 0); // the slot's 32 bits, whichever way it was written
+        memcpy(value_bits, &raw, 4);
+    }
+    else if (t == 5 || t == 6)
+    {
+        Mat v = pd.get(id, Mat());
+        *value_bits = (unsigned)v.w;
+        for (int i = 0; i < v.w && i < cap; i++) memcpy(array_bits + i, (const int*)v.data + i, 4);
+    }
+    else if (t == 7)
+    {
+        std::string s = pd.get(id, std::string());
+        *value_bits = (unsigned)s.size();
+        for (int i = 0; i < (int)s.size() && i < cap; i++) array_bits[i] = (unsigned char)s[(size_t)i];
+    }
+    return t;
+}
+
+int ncnn_modelbin_probe(const unsigned char* mem, int w, int type, void* out, size_t* consumed)
+{
+    const unsigned char* cursor = mem;
+    DataReaderFromMemory dr(cursor);
+    ModelBinFromDataReader mb(dr);
+    Mat m = mb.load(w, type);
+    if (consumed) *consumed = (size_t)(cursor - mem);
+    if (m.empty()) return 0;
+    memcpy(out, m.data, (size_t)w * m.elemsize);
+    return (int)m.elemsize;
+}
+
+} // extern "C"

@@ -1,0 +1,282 @@
+#include <string.h>
+
+#include <vector>
+
+#include "hip_layers.h"
+#include "hip_support.h"
+
+using namespace ncnn;
+
+namespace ncnn_amd {
+
+Convolution_hip::Convolution_hip(bool depthwise_type) : is_depthwise_type(depthwise_type)
+{
+    one_blob_only = true;
+    support_inplace = false;
+    support_batch = true; // Mat.n is folded into the pixel dimension of the implicit GEMM
+    d_weight = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
+    input_scale_count = 0;
+    group = 1;
+}
+
+Convolution_hip::~Convolution_hip()
+{
+    Option opt;
+    destroy_pipeline(opt);
+}
+
+int Convolution_hip::load_param(const ParamDict& pd)
+{
+    num_output = pd.get(0, 0);
+    kernel_w = pd.get(1, 0);
+    kernel_h = pd.get(11, kernel_w);
+    dilation_w = pd.get(2, 1);
+    dilation_h = pd.get(12, dilation_w);
+    stride_w = pd.get(3, 1);
+    stride_h = pd.get(13, stride_w);
+    pad_left = pd.get(4, 0);
+    pad_right = pd.get(15, pad_left);
+    pad_top = pd.get(14, pad_left);
+    pad_bottom = pd.get(16, pad_top);
+    pad_value = pd.get(18, 0.f);
+    bias_term = pd.get(5, 0);
+    weight_data_size = pd.get(6, 0);
+    group = is_depthwise_type ? pd.get(7, 1) : 1;
+    int8_scale_term = pd.get(8, 0);
+    activation_type = pd.get(9, 0);
+    activation_params = pd.get(10, Mat());
+    dynamic_weight = pd.get(19, 0);
+
+    if (dynamic_weight)
+    {
+        NCNN_LOGE("%s: dynamic weights are not part of the int8 path", type.c_str());
+        return -1;
+    }
+    if (group < 1 || num_output % group != 0) return -100; // the reference rejects an invalid group this way
+    if (!int8_scale_term)
+    {
+        NCNN_LOGE("%s %s: no int8_scale_term; only the quantised path runs on this device runtime", type.c_str(), name.c_str());
+        return -1;
+    }
+    support_int8_storage = true;
+    return 0;
+}
+
+int Convolution_hip::load_model(const ModelBin& mb)
+{
+    weight_data = mb.load(weight_data_size, 0);
+    if (weight_data.empty()) return -100;
+    if (bias_term)
+    {
+        bias_data = mb.load(num_output, 1);
+        if (bias_data.empty()) return -100;
+    }
+
+    if (!is_depthwise_type)
+    {
+        // Convolution: one weight scale per output channel, one input scale (+ one top scale)
+        weight_data_int8_scales = mb.load(num_output, 1);
+        bottom_blob_int8_scales = mb.load(1, 1);
+        if (int8_scale_term > 100) top_blob_int8_scales = mb.load(1, 1);
+    }
+    else
+    {
+        // ConvolutionDepthWise: term 1/101 stores one weight scale per group, term 2/102 a single
+        // one; every table is then held broadcast to `group` entries
+        const bool per_group = int8_scale_term == 1 || int8_scale_term == 101;
+        Mat ws = mb.load(per_group ? group : 1, 1);
+        Mat is = mb.load(1, 1);
+        if (ws.empty() || is.empty()) return -100;
+        weight_data_int8_scales.create(group);
+        bottom_blob_int8_scales.create(group);
+        for (int g = 0; g < group; g++)
+        {
+            weight_data_int8_scales[g] = per_group ? ws[g] : ws[0];
+            bottom_blob_int8_scales[g] = is[0];
+        }
+        if (int8_scale_term > 100)
+        {
+            Mat ts = mb.load(1, 1);
+            if (ts.empty()) return -100;
+            top_blob_int8_scales.create(group);
+            top_blob_int8_scales.fill(ts[0]);
+        }
+    }
+    if (weight_data_int8_scales.empty() || bottom_blob_int8_scales.empty()) return -100;
+    if (int8_scale_term > 100 && top_blob_int8_scales.empty()) return -100;
+
+    // fp32 weights in the file are quantised here, once: per output channel for Convolution,
+    // per group for ConvolutionDepthWise
+    if (weight_data.elemsize == 4u)
+    {
+        Option opt_q;
+        opt_q.num_threads = 1;
+        const int rows = is_depthwise_type ? group : num_output;
+        Mat as_rows = weight_data.reshape(weight_data_size / rows, rows);
+        Mat q;
+        quantize_to_int8(as_rows, q, weight_data_int8_scales, opt_q);
+        if (q.empty()) return -100;
+        weight_data = q.reshape(weight_data_size);
+    }
+    return 0;
+}
+
+int Convolution_hip::create_pipeline(const Option& /*opt*/)
+{
+    if (weight_data.elemsize != 1u)
+    {
+        NCNN_LOGE("%s %s: weights are not int8 after load_model", type.c_str(), name.c_str());
+        return -1;
+    }
+    std::vector<float> scale_in((size_t)num_output);
+    int rc = ncnnhip_fold_input_scales(weight_data_int8_scales, weight_data_int8_scales.w, bottom_blob_int8_scales, bottom_blob_int8_scales.w,
+                                       num_output, scale_in.data());
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_fold_input_scales");
+
+    int ret = upload_constant(weight_data.data, (size_t)weight_data_size, &d_weight);
+    if (ret == 0) ret = upload_constant(scale_in.data(), scale_in.size() * 4, &d_scale_in);
+    if (ret == 0 && bias_term) ret = upload_constant(bias_data.data, (size_t)num_output * 4, &d_bias);
+    if (ret == 0 && int8_scale_term > 100)
+    {
+        std::vector<float> so((size_t)num_output);
+        const int per = num_output / top_blob_int8_scales.w;
+        for (int p = 0; p < num_output; p++) so[(size_t)p] = top_blob_int8_scales[p / per];
+        ret = upload_constant(so.data(), so.size() * 4, &d_scale_out);
+    }
+    // input quantisation scales: the single value for Convolution; depthwise expands its per-group
+    // table to channels once the channel count is known, which is at forward time for the first
+    // blob -- the group table itself is what gets uploaded and indexed by channel/(channels/group)
+    if (ret == 0) ret = upload_constant(bottom_blob_int8_scales.data, (size_t)bottom_blob_int8_scales.w * 4, &d_input_scales);
+    input_scale_count = bottom_blob_int8_scales.w;
+    if (ret != 0) destroy_pipeline(Option());
+    return ret;
+}
+
+int Convolution_hip::destroy_pipeline(const Option& /*opt*/)
+{
+    void** all[] = {&d_weight, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
+    for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
+    {
+        if (*all[i]) ncnnhip_free(*all[i]);
+        *all[i] = 0;
+    }
+    return 0;
+}
+
+int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option& opt) const
+{
+    if (!opt.use_int8_inference)
+    {
+        NCNN_LOGE("%s %s: use_int8_inference is off and there is no fp32 path in this runtime", type.c_str(), name.c_str());
+        return -1;
+    }
+    if (!d_weight)
+    {
+        NCNN_LOGE("%s %s: forward before create_pipeline", type.c_str(), name.c_str());
+        return -1;
+    }
+    if (bottom_blob.dims != 3 || bottom_blob.elempack != 1 || (bottom_blob.elemsize != 4u && bottom_blob.elemsize != 1u))
+    {
+        NCNN_LOGE("%s %s: needs a pack-1 fp32 or int8 3-D blob", type.c_str(), name.c_str());
+        return -1;
+    }
+    const int channels = bottom_blob.c, batch = bottom_blob.n;
+    if (channels % group != 0 || num_output % group != 0) return -100;
+    if (weight_data_size != (num_output / group) * (channels / group) * kernel_w * kernel_h * group)
+    {
+        NCNN_LOGE("%s %s: weight_data_size %d does not match %d input channels", type.c_str(), name.c_str(), weight_data_size, channels);
+        return -1;
+    }
+
+    ncnnhip_conv_desc desc;
+    desc.w = bottom_blob.w;
+    desc.h = bottom_blob.h;
+    desc.c = channels;
+    desc.batch = batch;
+    desc.num_output = num_output;
+    desc.kernel_w = kernel_w;
+    desc.kernel_h = kernel_h;
+    desc.dilation_w = dilation_w;
+    desc.dilation_h = dilation_h;
+    desc.stride_w = stride_w;
+    desc.stride_h = stride_h;
+    desc.pad_left = pad_left;
+    desc.pad_right = pad_right;
+    desc.pad_top = pad_top;
+    desc.pad_bottom = pad_bottom;
+    desc.pad_value = pad_value;
+    desc.group = group;
+    int outw = 0, outh = 0;
+    int rc = ncnnhip_conv_out_shape(&desc, &outw, &outh);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_out_shape");
+
+    const bool requant = int8_scale_term > 100;
+    top_blob.create(outw, outh, num_output, requant ? (size_t)1u : (size_t)4u, 1, batch, opt.blob_allocator);
+    if (top_blob.empty()) return -100;
+
+    HipContext* ctx = context_for(opt);
+    int ret = ctx->ensure_ready();
+    if (ret != 0) return ret;
+    ScopedLeases leases(ctx);
+    void* st = ctx->stream;
+
+    void* d_in = leases.get(mat_bytes(bottom_blob));
+    void* d_out = leases.get(mat_bytes(top_blob));
+    if (!d_in || !d_out) return -100;
+    rc = ncnnhip_memcpy_h2d(d_in, bottom_blob.data, mat_bytes(bottom_blob), st);
+    if (rc != 0) return to_ncnn_status(rc, "upload bottom blob");
+
+    const int8_t* d_xq = (const int8_t*)d_in;
+    size_t q_cstep = bottom_blob.cstep, q_nstep = bottom_blob.nstep;
+    if (bottom_blob.elemsize == 4u)
+    {
+        // Quantize: one scale for Convolution, the group's scale for every channel of a group
+        q_cstep = alignSize((size_t)bottom_blob.w * bottom_blob.h, 16);
+        q_nstep = q_cstep * channels;
+        void* d_q = leases.get(q_nstep * batch);
+        if (!d_q) return -100;
+        const float* scales = (const float*)d_input_scales;
+        void* d_expanded = 0;
+        int nscales = 1;
+        if (input_scale_count > 1)
+        {
+            std::vector<float> per_channel((size_t)channels);
+            const int cg = channels / group;
+            for (int q = 0; q < channels; q++) per_channel[(size_t)q] = bottom_blob_int8_scales[q / cg];
+            d_expanded = leases.get((size_t)channels * 4);
+            if (!d_expanded) return -100;
+            rc = ncnnhip_memcpy_h2d(d_expanded, per_channel.data(), (size_t)channels * 4, st);
+            if (rc == 0) rc = ncnnhip_stream_synchronize(st); // per_channel dies with this scope
+            if (rc != 0) return to_ncnn_status(rc, "upload channel scales");
+            scales = (const float*)d_expanded;
+            nscales = channels;
+        }
+        rc = ncnnhip_quantize((const float*)d_in, bottom_blob.cstep, bottom_blob.nstep, (int8_t*)d_q, q_cstep, q_nstep, channels,
+                              bottom_blob.w * bottom_blob.h, batch, scales, nscales, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_quantize");
+        d_xq = (const int8_t*)d_q;
+    }
+
+    rc = ncnnhip_conv_int8(&desc, d_xq, q_cstep, q_nstep, (const int8_t*)d_weight, (const float*)d_scale_in, (const float*)d_bias,
+                           (const float*)d_scale_out, make_activation(activation_type, activation_params), d_out, top_blob.cstep,
+                           top_blob.nstep, 0, st);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_int8");
+    rc = ncnnhip_memcpy_d2h(top_blob.data, d_out, mat_bytes(top_blob), st);
+    if (rc == 0) rc = ncnnhip_stream_synchronize(st);
+    return to_ncnn_status(rc, "download top blob");
+}
+
+Layer* Convolution_hip_creator(void*)
+{
+    return new Convolution_hip(false);
+}
+Layer* ConvolutionDepthWise_hip_creator(void*)
+{
+    return new Convolution_hip(true);
+}
+void hip_layer_destroyer(Layer* layer, void*)
+{
+    delete layer;
+}
+
+} // namespace ncnn_amd

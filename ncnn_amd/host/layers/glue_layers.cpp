@@ -1,0 +1,421 @@
+// Host fp32 implementations of the few non-quantised layers that sit between the int8 layers
+// in the two benchmark nets (pack-1 semantics of the reference's naive layers):
+//   Input    src/layer/input.cpp:19-22          Split    src/layer/split.cpp
+//   ReLU     src/layer/relu.cpp                 Pooling  src/layer/pooling.cpp:18-415
+//   Eltwise  src/layer/eltwise.cpp:14-178       Flatten  src/layer/flatten.cpp
+//   Softmax  src/layer/softmax.cpp              Dropout  src/layer/dropout.cpp
+// They keep the same summation order as the reference loops, so fp32 results match it.
+#include <float.h>
+#include <math.h>
+
+#include <algorithm>
+
+#include "../ncnn/layer.h"
+
+namespace ncnn {
+
+// ---------------------------------------------------------------------------------- Input
+class Input : public Layer
+{
+public:
+    Input()
+    {
+        one_blob_only = true;
+        support_inplace = true;
+        support_batch = true;
+    }
+    virtual int load_param(const ParamDict& pd)
+    {
+        w = pd.get(0, 0);
+        h = pd.get(1, 0);
+        d = pd.get(11, 0);
+        c = pd.get(2, 0);
+        return 0;
+    }
+    virtual int forward_inplace(Mat&, const Option&) const
+    {
+        return 0;
+    }
+    int w, h, d, c;
+};
+
+// ---------------------------------------------------------------------------------- Split
+class Split : public Layer
+{
+public:
+    Split()
+    {
+        support_batch = true;
+        support_int8_storage = true; // int8 blobs pass through untouched
+    }
+    virtual int forward(const std::vector<Mat>& bottom_blobs, std::vector<Mat>& top_blobs, const Option&) const
+    {
+        for (size_t i = 0; i < top_blobs.size(); i++) top_blobs[i] = bottom_blobs[0]; // shared, refcounted
+        return 0;
+    }
+};
+
+// ---------------------------------------------------------------------------------- ReLU
+class ReLU : public Layer
+{
+public:
+    ReLU()
+    {
+        one_blob_only = true;
+        support_inplace = true;
+        support_int8_storage = true;
+    }
+    virtual int load_param(const ParamDict& pd)
+    {
+        slope = pd.get(0, 0.f);
+        return 0;
+    }
+    virtual int forward_inplace(Mat& m, const Option& opt) const
+    {
+        const size_t plane = (size_t)m.w * m.h * m.d;
+        if (m.elemsize == 1)
+        {
+            #pragma omp parallel for num_threads(opt.num_threads)
+            for (int q = 0; q < m.c; q++)
+            {
+                signed char* p = (signed char*)m.data + m.cstep * q;
+                for (size_t i = 0; i < plane; i++)
+                    if (p[i] < 0) p[i] = 0;
+            }
+            return 0;
+        }
+        #pragma omp parallel for num_threads(opt.num_threads)
+        for (int q = 0; q < m.c; q++)
+        {
+            float* p = (float*)m.data + m.cstep * q;
+            if (slope == 0.f)
+            {
+                for (size_t i = 0; i < plane; i++)
+                    if (p[i] < 0.f) p[i] = 0.f;
+            }
+            else
+            {
+                for (size_t i = 0; i < plane; i++)
+                    if (p[i] < 0.f) p[i] *= slope;
+            }
+        }
+        return 0;
+    }
+    float slope;
+};
+
+// ---------------------------------------------------------------------------------- Pooling
+class Pooling : public Layer
+{
+public:
+    Pooling()
+    {
+        one_blob_only = true;
+    }
+    virtual int load_param(const ParamDict& pd)
+    {
+        pooling_type = pd.get(0, 0);
+        kernel_w = pd.get(1, 0);
+        kernel_h = pd.get(11, kernel_w);
+        stride_w = pd.get(2, 1);
+        stride_h = pd.get(12, stride_w);
+        pad_left = pd.get(3, 0);
+        pad_right = pd.get(14, pad_left);
+        pad_top = pd.get(13, pad_left);
+        pad_bottom = pd.get(15, pad_top);
+        global_pooling = pd.get(4, 0);
+        pad_mode = pd.get(5, 0);
+        avgpool_count_include_pad = pd.get(6, 0);
+        adaptive_pooling = pd.get(7, 0);
+        if (adaptive_pooling)
+        {
+            NCNN_LOGE("Pooling: adaptive pooling is not part of this runtime");
+            return -1;
+        }
+        return 0;
+    }
+
+    virtual int forward(const Mat& bottom, Mat& top, const Option& opt) const
+    {
+        if (bottom.elemsize != 4u)
+        {
+            NCNN_LOGE("Pooling: only fp32 blobs are handled by this runtime");
+            return -1;
+        }
+        const int w = bottom.w, h = bottom.h, channels = bottom.c;
+        if (global_pooling)
+        {
+            top.create(channels, 4u, opt.blob_allocator);
+            if (top.empty()) return -100;
+            const int size = w * h;
+            #pragma omp parallel for num_threads(opt.num_threads)
+            for (int q = 0; q < channels; q++)
+            {
+                const float* p = (const float*)bottom.data + bottom.cstep * q;
+                if (pooling_type == 0)
+                {
+                    float m = p[0];
+                    for (int i = 0; i < size; i++) m = std::max(m, p[i]);
+                    top[q] = m;
+                }
+                else
+                {
+                    float s = 0.f;
+                    for (int i = 0; i < size; i++) s += p[i];
+                    top[q] = s / size;
+                }
+            }
+            return 0;
+        }
+
+        // resolve the border the reference would materialise: head pads, tail pads (+ the extra
+        // tail of "full" mode that keeps the last partial window)
+        int pt = pad_top, pb = pad_bottom, pl = pad_left, pr = pad_right;
+        if (pad_mode == 0)
+        {
+            const int wtail = (w + pad_left + pad_right - kernel_w) % stride_w;
+            const int htail = (h + pad_top + pad_bottom - kernel_h) % stride_h;
+            if (wtail != 0) pr += stride_w - wtail;
+            if (htail != 0) pb += stride_h - htail;
+        }
+        else if (pad_mode == 2 || pad_mode == 3)
+        {
+            const int wpad = kernel_w + (w - 1) / stride_w * stride_w - w;
+            const int hpad = kernel_h + (h - 1) / stride_h * stride_h - h;
+            pt = pb = pl = pr = 0;
+            if (wpad > 0 || hpad > 0)
+            {
+                const int hs = hpad / 2, hl = hpad - hpad / 2, ws = wpad / 2, wl = wpad - wpad / 2;
+                pt = pad_mode == 2 ? hs : hl;
+                pb = pad_mode == 2 ? hl : hs;
+                pl = pad_mode == 2 ? ws : wl;
+                pr = pad_mode == 2 ? wl : ws;
+            }
+        }
+        const int W = w + pl + pr, H = h + pt + pb;
+        const int outw = (W - kernel_w) / stride_w + 1;
+        const int outh = (H - kernel_h) / stride_h + 1;
+        top.create(outw, outh, channels, 4u, opt.blob_allocator);
+        if (top.empty()) return -100;
+
+        // average with count_include_pad=0 counts only taps inside the image plus, in modes 2/3,
+        // nothing else; the reference additionally counts the literal pads of modes 0/1 as
+        // outside.  Either way "inside" is the original image rectangle.
+        #pragma omp parallel for num_threads(opt.num_threads)
+        for (int q = 0; q < channels; q++)
+        {
+            const float* in = (const float*)bottom.data + bottom.cstep * q;
+            float* out = (float*)top.data + top.cstep * q;
+            for (int i = 0; i < outh; i++)
+            {
+                for (int j = 0; j < outw; j++)
+                {
+                    const int y0 = i * stride_h - pt, x0 = j * stride_w - pl;
+                    if (pooling_type == 0)
+                    {
+                        float m = -FLT_MAX;
+                        bool first = true;
+                        for (int ky = 0; ky < kernel_h; ky++)
+                            for (int kx = 0; kx < kernel_w; kx++)
+                            {
+                                const int y = y0 + ky, x = x0 + kx;
+                                const float v = (y >= 0 && y < h && x >= 0 && x < w) ? in[y * w + x] : -FLT_MAX;
+                                m = first ? v : std::max(m, v);
+                                first = false;
+                            }
+                        out[i * outw + j] = m;
+                    }
+                    else if (avgpool_count_include_pad == 0)
+                    {
+                        float s = 0.f;
+                        int area = 0;
+                        for (int ky = 0; ky < kernel_h; ky++)
+                        {
+                            const int y = y0 + ky;
+                            if (y < 0) continue;
+                            if (y >= h) break;
+                            for (int kx = 0; kx < kernel_w; kx++)
+                            {
+                                const int x = x0 + kx;
+                                if (x < 0) continue;
+                                if (x >= w) break;
+                                s += in[y * w + x];
+                                area++;
+                            }
+                        }
+                        out[i * outw + j] = s / area;
+                    }
+                    else
+                    {
+                        float s = 0.f;
+                        for (int ky = 0; ky < kernel_h; ky++)
+                            for (int kx = 0; kx < kernel_w; kx++)
+                            {
+                                const int y = y0 + ky, x = x0 + kx;
+                                s += (y >= 0 && y < h && x >= 0 && x < w) ? in[y * w + x] : 0.f;
+                            }
+                        out[i * outw + j] = s / (kernel_w * kernel_h);
+                    }
+                }
+            }
+        }
+        return 0;
+    }
+
+    int pooling_type, kernel_w, kernel_h, stride_w, stride_h, pad_left, pad_right, pad_top, pad_bottom;
+    int global_pooling, pad_mode, avgpool_count_include_pad, adaptive_pooling;
+};
+
+// ---------------------------------------------------------------------------------- Eltwise
+class Eltwise : public Layer
+{
+public:
+    virtual int load_param(const ParamDict& pd)
+    {
+        op_type = pd.get(0, 0);
+        coeffs = pd.get(1, Mat());
+        return 0;
+    }
+    virtual int forward(const std::vector<Mat>& bottoms, std::vector<Mat>& tops, const Option& opt) const
+    {
+        const Mat& a = bottoms[0];
+        if (bottoms.size() < 2 || a.elemsize != 4u) return -1;
+        Mat& top = tops[0];
+        top.create_like(a, opt.blob_allocator);
+        if (top.empty()) return -100;
+        const size_t plane = (size_t)a.w * a.h * a.d;
+        const bool weighted = op_type == 1 && coeffs.w != 0;
+        #pragma omp parallel for num_threads(opt.num_threads)
+        for (int q = 0; q < a.c; q++)
+        {
+            float* out = (float*)top.data + top.cstep * q;
+            const float* p0 = (const float*)a.data + a.cstep * q;
+            const float* p1 = (const float*)bottoms[1].data + bottoms[1].cstep * q;
+            if (op_type == 0)
+                for (size_t i = 0; i < plane; i++) out[i] = p0[i] * p1[i];
+            else if (op_type == 2)
+                for (size_t i = 0; i < plane; i++) out[i] = std::max(p0[i], p1[i]);
+            else if (weighted)
+                for (size_t i = 0; i < plane; i++) out[i] = p0[i] * coeffs[0] + p1[i] * coeffs[1];
+            else
+                for (size_t i = 0; i < plane; i++) out[i] = p0[i] + p1[i];
+            for (size_t b = 2; b < bottoms.size(); b++)
+            {
+                const float* pb = (const float*)bottoms[b].data + bottoms[b].cstep * q;
+                if (op_type == 0)
+                    for (size_t i = 0; i < plane; i++) out[i] *= pb[i];
+                else if (op_type == 2)
+                    for (size_t i = 0; i < plane; i++) out[i] = std::max(out[i], pb[i]);
+                else if (weighted)
+                    for (size_t i = 0; i < plane; i++) out[i] += pb[i] * coeffs[b];
+                else
+                    for (size_t i = 0; i < plane; i++) out[i] += pb[i];
+            }
+        }
+        return 0;
+    }
+    int op_type;
+    Mat coeffs;
+};
+
+// ---------------------------------------------------------------------------------- Flatten
+class Flatten : public Layer
+{
+public:
+    Flatten()
+    {
+        one_blob_only = true;
+    }
+    virtual int forward(const Mat& bottom, Mat& top, const Option& opt) const
+    {
+        const size_t plane = (size_t)bottom.w * bottom.h * bottom.d;
+        top.create((int)(plane * bottom.c), bottom.elemsize, opt.blob_allocator);
+        if (top.empty()) return -100;
+        for (int q = 0; q < bottom.c; q++)
+            memcpy((unsigned char*)top.data + plane * q * bottom.elemsize, (const unsigned char*)bottom.data + bottom.cstep * q * bottom.elemsize, plane * bottom.elemsize);
+        return 0;
+    }
+};
+
+// ---------------------------------------------------------------------------------- Softmax
+class Softmax : public Layer
+{
+public:
+    Softmax()
+    {
+        one_blob_only = true;
+        support_inplace = true;
+    }
+    virtual int load_param(const ParamDict& pd)
+    {
+        axis = pd.get(0, 0);
+        return 0;
+    }
+    virtual int forward_inplace(Mat& m, const Option&) const
+    {
+        // softmax over the outermost axis (axis 0), which is what classification heads use
+        if (axis != 0 || m.elemsize != 4u)
+        {
+            NCNN_LOGE("Softmax: only axis 0 on fp32 blobs is handled by this runtime");
+            return -1;
+        }
+        const int count = m.dims == 1 ? m.w : m.dims == 2 ? m.h : m.c;
+        const size_t inner = m.dims == 1 ? 1 : m.dims == 2 ? (size_t)m.w : (size_t)m.w * m.h * m.d;
+        const size_t step = m.dims == 1 ? 1 : m.dims == 2 ? (size_t)m.w : m.cstep;
+        float* base = m;
+        for (size_t i = 0; i < inner; i++)
+        {
+            float mx = -FLT_MAX;
+            for (int q = 0; q < count; q++) mx = std::max(mx, base[q * step + i]);
+            float sum = 0.f;
+            for (int q = 0; q < count; q++)
+            {
+                float& v = base[q * step + i];
+                v = expf(v - mx);
+                sum += v;
+            }
+            for (int q = 0; q < count; q++) base[q * step + i] /= sum;
+        }
+        return 0;
+    }
+    int axis;
+};
+
+// ---------------------------------------------------------------------------------- Dropout
+class Dropout : public Layer
+{
+public:
+    Dropout()
+    {
+        one_blob_only = true;
+        support_inplace = true;
+    }
+    virtual int load_param(const ParamDict& pd)
+    {
+        scale = pd.get(0, 1.f);
+        return 0;
+    }
+    virtual int forward_inplace(Mat& m, const Option&) const
+    {
+        if (scale == 1.f) return 0;
+        const size_t plane = (size_t)m.w * m.h * m.d;
+        for (int q = 0; q < m.c; q++)
+        {
+            float* p = (float*)m.data + m.cstep * q;
+            for (size_t i = 0; i < plane; i++) p[i] *= scale;
+        }
+        return 0;
+    }
+    float scale;
+};
+
+DEFINE_LAYER_CREATOR(Input)
+DEFINE_LAYER_CREATOR(Split)
+DEFINE_LAYER_CREATOR(ReLU)
+DEFINE_LAYER_CREATOR(Pooling)
+DEFINE_LAYER_CREATOR(Eltwise)
+DEFINE_LAYER_CREATOR(Flatten)
+DEFINE_LAYER_CREATOR(Softmax)
+DEFINE_LAYER_CREATOR(Dropout)
+
+} // namespace ncnn

@@ -1,0 +1,113 @@
+// The four ncnn::Layer implementations whose forward() runs on the MI355X.  They read the same
+// param ids and the same .bin order as the reference layers they replace and are installed with
+// Net::register_custom_layer under the built-in type names (see ncnnhip_register_int8_layers).
+#ifndef NCNN_AMD_HIP_LAYERS_H
+#define NCNN_AMD_HIP_LAYERS_H
+
+#include "../ncnn/layer.h"
+
+namespace ncnn_amd {
+
+// Convolution (src/layer/convolution.{h,cpp}) and ConvolutionDepthWise
+// (src/layer/convolutiondepthwise.{h,cpp}) share everything except the group count and how
+// the scale tables are indexed, so one class serves both type names.
+class Convolution_hip : public ncnn::Layer
+{
+public:
+    explicit Convolution_hip(bool depthwise_type);
+    virtual ~Convolution_hip();
+    virtual int load_param(const ncnn::ParamDict& pd);
+    virtual int load_model(const ncnn::ModelBin& mb);
+    virtual int create_pipeline(const ncnn::Option& opt);
+    virtual int destroy_pipeline(const ncnn::Option& opt);
+    virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+
+public:
+    // same member names as the reference layers
+    int num_output, kernel_w, kernel_h, dilation_w, dilation_h, stride_w, stride_h;
+    int pad_left, pad_right, pad_top, pad_bottom;
+    float pad_value;
+    int bias_term, weight_data_size, group, int8_scale_term, activation_type, dynamic_weight;
+    ncnn::Mat activation_params;
+    ncnn::Mat weight_data, bias_data;
+    ncnn::Mat weight_data_int8_scales, bottom_blob_int8_scales, top_blob_int8_scales;
+
+private:
+    const bool is_depthwise_type;
+    // device copies made at create_pipeline
+    void* d_weight;
+    void* d_bias;
+    void* d_scale_in;      // one per output channel: 1/(in_scale*w_scale), 0 when w_scale is 0
+    void* d_scale_out;     // one per output channel, only when requantising
+    void* d_input_scales;  // one per input channel, for quantising an fp32 bottom blob
+    int input_scale_count; // 1 or channels
+};
+
+// InnerProduct (src/layer/innerproduct.{h,cpp})
+class InnerProduct_hip : public ncnn::Layer
+{
+public:
+    InnerProduct_hip();
+    virtual ~InnerProduct_hip();
+    virtual int load_param(const ncnn::ParamDict& pd);
+    virtual int load_model(const ncnn::ModelBin& mb);
+    virtual int create_pipeline(const ncnn::Option& opt);
+    virtual int destroy_pipeline(const ncnn::Option& opt);
+    virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+
+public:
+    int num_output, bias_term, weight_data_size, int8_scale_term, activation_type;
+    ncnn::Mat activation_params;
+    ncnn::Mat weight_data, bias_data, weight_data_int8_scales, bottom_blob_int8_scales;
+
+private:
+    void* d_weight;
+    void* d_bias;
+    void* d_scale_in;
+    void* d_input_scale;
+};
+
+// Gemm with quantize_term (src/layer/gemm.{h,cpp}): int8 (per-row A, per-tensor B) and the
+// weight-only block-quantised form
+class Gemm_hip : public ncnn::Layer
+{
+public:
+    Gemm_hip();
+    virtual ~Gemm_hip();
+    virtual int load_param(const ncnn::ParamDict& pd);
+    virtual int load_model(const ncnn::ModelBin& mb);
+    virtual int create_pipeline(const ncnn::Option& opt);
+    virtual int destroy_pipeline(const ncnn::Option& opt);
+    virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+    virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+
+public:
+    float alpha, beta;
+    int transA, transB, constantA, constantB, constantC, constantM, constantN, constantK;
+    int constant_broadcast_type_C, output_N1M, output_elempack, output_elemtype, output_transpose;
+    int quantize_term, weight_block_quantize;
+    ncnn::Mat A_data, B_data, C_data, A_data_int8_scales, B_data_quantize_scales, B_data_input_scales;
+    float B_data_int8_scale;
+
+private:
+    int forward_int8(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+    int forward_block_quantize(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+    void* d_A;        // constant A as loaded (fp32 or int8), row-major as stored
+    void* d_B;        // constant B: int8 [N][K] for the int8 path (already K-contiguous), packed bytes for block quant
+    void* d_C;
+    void* d_A_scales; // [M] when A is constant int8
+    void* d_B_scale;  // [1]
+    void* d_B_block_scales;
+    void* d_B_input_scales;
+    int b_ready_int8; // constant B sits on the device quantised and transposed
+};
+
+ncnn::Layer* Convolution_hip_creator(void* userdata);
+ncnn::Layer* ConvolutionDepthWise_hip_creator(void* userdata);
+ncnn::Layer* InnerProduct_hip_creator(void* userdata);
+ncnn::Layer* Gemm_hip_creator(void* userdata);
+void hip_layer_destroyer(ncnn::Layer* layer, void* userdata);
+
+} // namespace ncnn_amd
+
+#endif // NCNN_AMD_HIP_LAYERS_H

@@ -1,0 +1,105 @@
+// Glue between the ncnn::Layer implementations and the C ABI in include/ncnnhip.h:
+// per-Extractor device context (one stream + a pool of device buffers), uploads of constant
+// tables at create_pipeline, and the mapping of C-ABI return codes to ncnn's 0 / -100 / -1.
+#ifndef NCNN_AMD_HIP_SUPPORT_H
+#define NCNN_AMD_HIP_SUPPORT_H
+
+#include <stddef.h>
+
+#include <vector>
+
+#include "../ncnn/allocator.h"
+#include "../ncnn/mat.h"
+#include "../ncnn/option.h"
+#include "ncnnhip.h"
+
+namespace ncnn_amd {
+
+// One stream and a grow-only set of device buffers.  forward() of a HIP layer borrows buffers for
+// the duration of the call; everything it launched has completed (stream synchronised) before
+// the buffers go back, so the pool needs no cross-call tracking.
+class HipContext
+{
+public:
+    HipContext();
+    ~HipContext();
+    int ensure_ready(); // lazily selects the device and creates the stream
+    void* stream;
+
+    struct Lease
+    {
+        void* ptr;
+        size_t bytes;
+        bool busy;
+    };
+    void* borrow(size_t bytes);
+    void give_back_all();
+
+private:
+    HipContext(const HipContext&);
+    HipContext& operator=(const HipContext&);
+    bool ready;
+    std::vector<Lease> pool;
+};
+
+// Host allocator to install with Extractor::set_blob_allocator(): it hands out ordinary host
+// memory (ncnn keeps a Mat's refcount inside the allocation and touches results on the host) and
+// carries the Extractor's device context -- "one hipStream per Extractor".  Layers find it through
+// opt.blob_allocator; without it a per-thread context is used.
+class HipBlobAllocator : public ncnn::Allocator
+{
+public:
+    HipBlobAllocator();
+    virtual ~HipBlobAllocator();
+    virtual void* fastMalloc(size_t size);
+    virtual void fastFree(void* ptr);
+    HipContext context;
+
+private:
+    ncnn::UnlockedPoolAllocator pool;
+};
+
+HipContext* context_for(const ncnn::Option& opt);
+
+// RAII: buffers borrowed during one forward() return to the pool when it goes out of scope
+class ScopedLeases
+{
+public:
+    explicit ScopedLeases(HipContext* c) : ctx(c) {}
+    ~ScopedLeases()
+    {
+        ctx->give_back_all();
+    }
+    void* get(size_t bytes)
+    {
+        return ctx->borrow(bytes);
+    }
+
+private:
+    HipContext* ctx;
+};
+
+// 0 stays 0, -100 stays -100 (out of memory), anything else becomes -1 and is logged
+int to_ncnn_status(int rc, const char* where);
+
+// constant table -> device (create_pipeline); *dev is freed with ncnnhip_free at destroy_pipeline
+int upload_constant(const void* host, size_t bytes, void** dev);
+
+// payload bytes of a Mat as it lies in memory (whole batch, including plane padding)
+static inline size_t mat_bytes(const ncnn::Mat& m)
+{
+    return (m.n > 1 ? m.nstep * m.n : m.total()) * m.elemsize;
+}
+
+static inline ncnnhip_activation make_activation(int type, const ncnn::Mat& params)
+{
+    ncnnhip_activation a;
+    a.type = type;
+    a.p0 = params.w > 0 ? params[0] : 0.f;
+    a.p1 = params.w > 1 ? params[1] : 0.f;
+    return a;
+}
+
+} // namespace ncnn_amd
+
+#endif // NCNN_AMD_HIP_SUPPORT_H

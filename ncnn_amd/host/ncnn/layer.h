@@ -1,0 +1,89 @@
+// ncnn::Layer, the operator plug-in interface (src/layer.h:20-142), and the layer factories.
+#ifndef NCNN_LAYER_H
+#define NCNN_LAYER_H
+
+#include <string>
+#include <vector>
+
+#include "mat.h"
+#include "modelbin.h"
+#include "option.h"
+#include "paramdict.h"
+#include "platform.h"
+
+namespace ncnn {
+
+class NCNN_EXPORT Layer
+{
+public:
+    Layer();
+    virtual ~Layer();
+
+    // all return 0 on success, -100 on allocation failure, -1 otherwise
+    virtual int load_param(const ParamDict& pd);
+    virtual int load_model(const ModelBin& mb);
+    virtual int create_pipeline(const Option& opt);
+    virtual int destroy_pipeline(const Option& opt);
+
+    bool one_blob_only;
+    bool support_inplace;
+    bool support_vulkan;
+    bool support_packing;
+    bool support_bf16_storage;
+    bool support_fp16_storage;
+    bool support_int8_storage;
+    bool support_tensor_storage;
+    bool support_vulkan_packing;
+    bool support_any_packing;
+    bool support_vulkan_any_packing;
+    bool support_batch; // takes a Mat with n > 1 whole; otherwise the net loops over samples
+    int featmask;
+
+    virtual int forward(const std::vector<Mat>& bottom_blobs, std::vector<Mat>& top_blobs, const Option& opt) const;
+    virtual int forward(const Mat& bottom_blob, Mat& top_blob, const Option& opt) const;
+    virtual int forward_inplace(std::vector<Mat>& bottom_top_blobs, const Option& opt) const;
+    virtual int forward_inplace(Mat& bottom_top_blob, const Option& opt) const;
+
+    void* userdata;
+    int typeindex;
+    std::string type;
+    std::string name;
+    std::vector<int> bottoms;
+    std::vector<int> tops;
+    std::vector<Mat> bottom_shapes;
+    std::vector<Mat> top_shapes;
+};
+
+typedef Layer* (*layer_creator_func)(void*);
+typedef void (*layer_destroyer_func)(Layer*, void*);
+
+struct layer_registry_entry
+{
+    const char* name;
+    layer_creator_func creator; // NULL: the type is known but has no host implementation
+};
+
+// built-in type table.  The four int8 hot-path types are listed (so that registering them
+// through Net::register_custom_layer takes the overwrite-builtin route) but deliberately have
+// no host implementation: without the HIP layers registered, loading a net that uses them fails.
+NCNN_EXPORT int layer_to_index(const char* type);
+NCNN_EXPORT Layer* create_layer(const char* type);
+NCNN_EXPORT Layer* create_layer(int index);
+NCNN_EXPORT Layer* create_layer_cpu(const char* type);
+NCNN_EXPORT Layer* create_layer_cpu(int index);
+
+#define DEFINE_LAYER_CREATOR(name)                          \
+    ::ncnn::Layer* name##_layer_creator(void* /*userdata*/) \
+    {                                                       \
+        return new name;                                    \
+    }
+
+#define DEFINE_LAYER_DESTROYER(name)                                      \
+    void name##_layer_destroyer(::ncnn::Layer* layer, void* /*userdata*/) \
+    {                                                                     \
+        delete layer;                                                     \
+    }
+
+} // namespace ncnn
+
+#endif // NCNN_LAYER_H

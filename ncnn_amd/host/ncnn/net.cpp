@@ -1,0 +1,749 @@
+#include "net.h"
+
+#include <stdint.h>
+#include <string.h>
+
+#include <map>
+#include <string>
+
+#include "datareader.h"
+#include "modelbin.h"
+#include "paramdict.h"
+
+namespace ncnn {
+
+struct CustomEntry
+{
+    std::string name; // empty for an overwritten built-in
+    int typeindex;    // built-in index for an overwrite, -1 otherwise
+    layer_creator_func creator;
+    layer_destroyer_func destroyer;
+    void* userdata;
+};
+
+static const int CUSTOM_BIT = 1 << 8; // type indexes of non-built-in custom layers carry this bit
+
+class NetPrivate
+{
+public:
+    explicit NetPrivate(Option& _opt) : opt(_opt) {}
+
+    Option& opt;
+    std::vector<Blob> blobs;
+    std::vector<Layer*> layers;
+    std::vector<int> input_idx, output_idx;
+    std::vector<const char*> input_nm, output_nm;
+    std::vector<CustomEntry> custom;    // new type names
+    std::vector<CustomEntry> overwrite; // replaced built-ins
+
+    const CustomEntry* find_overwrite(int typeindex) const
+    {
+        for (size_t i = 0; i < overwrite.size(); i++)
+            if (overwrite[i].typeindex == typeindex) return &overwrite[i];
+        return 0;
+    }
+
+    Layer* make_layer(const char* type)
+    {
+        const int builtin = layer_to_index(type);
+        Layer* layer = 0;
+        if (builtin >= 0)
+        {
+            if (const CustomEntry* e = find_overwrite(builtin))
+            {
+                layer = e->creator(e->userdata);
+                if (layer) layer->typeindex = builtin;
+            }
+            else
+                layer = create_layer(builtin);
+        }
+        else
+        {
+            for (size_t i = 0; i < custom.size() && !layer; i++)
+            {
+                if (custom[i].name == type && custom[i].creator)
+                {
+                    layer = custom[i].creator(custom[i].userdata);
+                    if (layer) layer->typeindex = CUSTOM_BIT | (int)i;
+                }
+            }
+        }
+        return layer;
+    }
+
+    void destroy_layer(Layer* layer)
+    {
+        const int ti = layer->typeindex;
+        const CustomEntry* e = 0;
+        if (ti >= 0 && (ti & CUSTOM_BIT))
+        {
+            const size_t i = (size_t)(ti & ~CUSTOM_BIT);
+            if (i < custom.size()) e = &custom[i];
+        }
+        else if (ti >= 0)
+            e = find_overwrite(ti);
+        if (e && e->destroyer)
+            e->destroyer(layer, e->userdata);
+        else
+            delete layer;
+    }
+
+    int forward_layer(int layer_index, std::vector<Mat>& blob_mats, const Option& opt) const;
+    int run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const Option& opt) const;
+};
+
+// int8 blob -> fp32 blob of the same shape (plain value conversion), batch aware
+static int expand_int8(const Mat& src, Mat& dst, Allocator* allocator)
+{
+    if (src.dims == 1)
+        dst.create(src.w, 4u, 1, src.n, allocator);
+    else if (src.dims == 2)
+        dst.create(src.w, src.h, 4u, 1, src.n, allocator);
+    else if (src.dims == 3)
+        dst.create(src.w, src.h, src.c, 4u, 1, src.n, allocator);
+    else
+        dst.create(src.w, src.h, src.d, src.c, 4u, 1, src.n, allocator);
+    if (dst.empty()) return -100;
+    const size_t plane = (size_t)src.w * src.h * src.d;
+    for (int b = 0; b < src.n; b++)
+        for (int q = 0; q < src.c; q++)
+        {
+            const signed char* p = (const signed char*)src.data + src.nstep * b + src.cstep * q;
+            float* o = (float*)dst.data + dst.nstep * b + dst.cstep * q;
+            for (size_t i = 0; i < plane; i++) o[i] = (float)p[i];
+        }
+    return 0;
+}
+
+// ---- executor -----------------------------------------------------------------------------
+
+int NetPrivate::forward_layer(int layer_index, std::vector<Mat>& blob_mats, const Option& opt) const
+{
+    const Layer* layer = layers[layer_index];
+    if (layer->bottoms.empty() && layer->type == "Input") return 0; // inputs are fed, not computed
+
+    // make sure every input exists, computing producers depth-first
+    for (size_t i = 0; i < layer->bottoms.size(); i++)
+    {
+        const int bi = layer->bottoms[i];
+        if (blob_mats[bi].dims == 0)
+        {
+            const int producer = blobs[bi].producer;
+            if (producer < 0)
+            {
+                NCNN_LOGE("blob %s has no producer and was not fed", blobs[bi].name.c_str());
+                return -1;
+            }
+            int ret = forward_layer(producer, blob_mats, opt);
+            if (ret != 0) return ret;
+            if (blob_mats[bi].dims == 0)
+            {
+                NCNN_LOGE("blob %s was not produced (missing input?)", blobs[bi].name.c_str());
+                return -1;
+            }
+        }
+    }
+    return run_layer(layer, blob_mats, opt);
+}
+
+int NetPrivate::run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const Option& opt) const
+{
+    // gather inputs; in light mode a blob is handed over (and dropped from the table) because
+    // every blob has exactly one consumer
+    std::vector<Mat> ins(layer->bottoms.size());
+    for (size_t i = 0; i < ins.size(); i++)
+    {
+        Mat& slot = blob_mats[layer->bottoms[i]];
+        ins[i] = slot;
+        if (opt.lightmode) slot.release();
+        if (ins[i].elemsize == 1u && !layer->support_int8_storage)
+        {
+            Mat wide;
+            int ret = expand_int8(ins[i], wide, opt.blob_allocator);
+            if (ret != 0) return ret;
+            ins[i] = wide;
+        }
+    }
+
+    if (layer->one_blob_only)
+    {
+        Mat bottom = ins[0];
+        ins.clear();
+        Mat top;
+        const bool loop_samples = bottom.n > 1 && !layer->support_batch;
+        if (layer->support_inplace)
+        {
+            // work on a private copy unless this is the only handle (light mode gave it to us)
+            if (!(opt.lightmode && bottom.refcount && *bottom.refcount == 1))
+            {
+                Mat own = bottom.clone(opt.blob_allocator);
+                if (own.empty()) return -100;
+                bottom = own;
+            }
+            if (loop_samples)
+            {
+                for (int b = 0; b < bottom.n; b++)
+                {
+                    Mat one = bottom.batch(b);
+                    int ret = layer->forward_inplace(one, opt);
+                    if (ret != 0) return ret;
+                }
+            }
+            else
+            {
+                int ret = layer->forward_inplace(bottom, opt);
+                if (ret != 0) return ret;
+            }
+            top = bottom;
+        }
+        else if (loop_samples)
+        {
+            // a layer that does not understand batches sees one sample at a time
+            for (int b = 0; b < bottom.n; b++)
+            {
+                Mat one_top;
+                int ret = layer->forward(bottom.batch(b), one_top, opt);
+                if (ret != 0) return ret;
+                if (b == 0)
+                {
+                    top.create_like(one_top, bottom.n, opt.blob_allocator);
+                    if (top.empty()) return -100;
+                }
+                memcpy((unsigned char*)top.data + top.nstep * b * top.elemsize, one_top.data, one_top.total() * one_top.elemsize);
+            }
+        }
+        else
+        {
+            int ret = layer->forward(bottom, top, opt);
+            if (ret != 0) return ret;
+        }
+        blob_mats[layer->tops[0]] = top;
+        return 0;
+    }
+
+    std::vector<Mat> outs(layer->tops.size());
+    bool any_batch = false;
+    for (size_t i = 0; i < ins.size(); i++) any_batch = any_batch || ins[i].n > 1;
+    if (any_batch && !layer->support_batch)
+    {
+        const int B = ins[0].n;
+        for (int b = 0; b < B; b++)
+        {
+            std::vector<Mat> one_in(ins.size()), one_out(outs.size());
+            for (size_t i = 0; i < ins.size(); i++) one_in[i] = ins[i].n > 1 ? ins[i].batch(b) : ins[i];
+            int ret = layer->forward(one_in, one_out, opt);
+            if (ret != 0) return ret;
+            for (size_t i = 0; i < outs.size(); i++)
+            {
+                if (b == 0)
+                {
+                    outs[i].create_like(one_out[i], B, opt.blob_allocator);
+                    if (outs[i].empty()) return -100;
+                }
+                memcpy((unsigned char*)outs[i].data + outs[i].nstep * b * outs[i].elemsize, one_out[i].data, one_out[i].total() * one_out[i].elemsize);
+            }
+        }
+    }
+    else
+    {
+        int ret = layer->forward(ins, outs, opt);
+        if (ret != 0) return ret;
+    }
+    for (size_t i = 0; i < outs.size(); i++) blob_mats[layer->tops[i]] = outs[i];
+    return 0;
+}
+
+// ---- Net ----------------------------------------------------------------------------------
+
+Net::Net() : d(new NetPrivate(opt)) {}
+
+Net::~Net()
+{
+    clear();
+    delete d;
+}
+
+int Net::register_custom_layer(const char* type, layer_creator_func creator, layer_destroyer_func destroyer, void* userdata)
+{
+    const int builtin = layer_to_index(type);
+    if (builtin >= 0)
+    {
+        for (size_t i = 0; i < d->overwrite.size(); i++)
+        {
+            if (d->overwrite[i].typeindex == builtin)
+            {
+                NCNN_LOGE("overwrite existing overwritten built-in layer type %s", type);
+                d->overwrite[i].creator = creator;
+                d->overwrite[i].destroyer = destroyer;
+                d->overwrite[i].userdata = userdata;
+                return 0;
+            }
+        }
+        CustomEntry e = {std::string(), builtin, creator, destroyer, userdata};
+        d->overwrite.push_back(e);
+        return 0;
+    }
+    for (size_t i = 0; i < d->custom.size(); i++)
+    {
+        if (d->custom[i].name == type)
+        {
+            NCNN_LOGE("overwrite existing custom layer type %s", type);
+            d->custom[i].creator = creator;
+            d->custom[i].destroyer = destroyer;
+            d->custom[i].userdata = userdata;
+            return 0;
+        }
+    }
+    CustomEntry e = {std::string(type), -1, creator, destroyer, userdata};
+    d->custom.push_back(e);
+    return 0;
+}
+
+int Net::register_custom_layer(int index, layer_creator_func creator, layer_destroyer_func destroyer, void* userdata)
+{
+    if (index < 0) return -1;
+    if (!(index & CUSTOM_BIT))
+    {
+        for (size_t i = 0; i < d->overwrite.size(); i++)
+        {
+            if (d->overwrite[i].typeindex == index)
+            {
+                d->overwrite[i].creator = creator;
+                d->overwrite[i].destroyer = destroyer;
+                d->overwrite[i].userdata = userdata;
+                return 0;
+            }
+        }
+        CustomEntry e = {std::string(), index, creator, destroyer, userdata};
+        d->overwrite.push_back(e);
+        return 0;
+    }
+    const size_t slot = (size_t)(index & ~CUSTOM_BIT);
+    if (d->custom.size() <= slot)
+    {
+        CustomEntry empty = {std::string(), -1, 0, 0, 0};
+        d->custom.resize(slot + 1, empty);
+    }
+    d->custom[slot].creator = creator;
+    d->custom[slot].destroyer = destroyer;
+    d->custom[slot].userdata = userdata;
+    return 0;
+}
+
+int Net::custom_layer_to_index(const char* type)
+{
+    for (size_t i = 0; i < d->custom.size(); i++)
+        if (d->custom[i].name == type) return (int)i;
+    return -1;
+}
+
+int Net::load_param(const DataReader& dr)
+{
+    int magic = 0;
+    if (dr.scan("%d", &magic) != 1)
+    {
+        NCNN_LOGE("parse magic failed");
+        return -1;
+    }
+    if (magic != 7767517)
+    {
+        NCNN_LOGE("param is too old, please regenerate");
+        return -1;
+    }
+    int layer_count = 0, blob_count = 0;
+    if (dr.scan("%d", &layer_count) != 1 || dr.scan("%d", &blob_count) != 1 || layer_count <= 0 || blob_count <= 0)
+    {
+        NCNN_LOGE("invalid layer_count or blob_count");
+        return -1;
+    }
+
+    d->layers.assign((size_t)layer_count, (Layer*)0);
+    d->blobs.assign((size_t)blob_count, Blob());
+    std::map<std::string, int> blob_of;
+    ParamDict pd;
+
+    for (int li = 0; li < layer_count; li++)
+    {
+        char type[256], name[256];
+        int nbottom = 0, ntop = 0;
+        if (dr.scan("%255s", type) != 1 || dr.scan("%255s", name) != 1 || dr.scan("%d", &nbottom) != 1 || dr.scan("%d", &ntop) != 1)
+        {
+            NCNN_LOGE("parse layer header failed at layer %d", li);
+            clear();
+            return -1;
+        }
+        Layer* layer = d->make_layer(type);
+        if (!layer)
+        {
+            NCNN_LOGE("layer %s not exists or registered", type);
+            clear();
+            return -1;
+        }
+        layer->type = type;
+        layer->name = name;
+        d->layers[li] = layer;
+
+        layer->bottoms.resize((size_t)nbottom);
+        for (int j = 0; j < nbottom; j++)
+        {
+            char bname[256];
+            if (dr.scan("%255s", bname) != 1)
+            {
+                NCNN_LOGE("parse bottom_name failed");
+                clear();
+                return -1;
+            }
+            std::map<std::string, int>::iterator it = blob_of.find(bname);
+            int bi;
+            if (it == blob_of.end())
+            {
+                bi = (int)blob_of.size();
+                if (bi >= blob_count)
+                {
+                    NCNN_LOGE("more blobs than declared (%d)", blob_count);
+                    clear();
+                    return -1;
+                }
+                blob_of[bname] = bi;
+                d->blobs[bi].name = bname;
+            }
+            else
+                bi = it->second;
+            d->blobs[bi].consumer = li;
+            layer->bottoms[j] = bi;
+        }
+        layer->tops.resize((size_t)ntop);
+        for (int j = 0; j < ntop; j++)
+        {
+            char bname[256];
+            if (dr.scan("%255s", bname) != 1)
+            {
+                NCNN_LOGE("parse blob_name failed");
+                clear();
+                return -1;
+            }
+            int bi;
+            std::map<std::string, int>::iterator it = blob_of.find(bname);
+            if (it == blob_of.end())
+            {
+                bi = (int)blob_of.size();
+                if (bi >= blob_count)
+                {
+                    NCNN_LOGE("more blobs than declared (%d)", blob_count);
+                    clear();
+                    return -1;
+                }
+                blob_of[bname] = bi;
+                d->blobs[bi].name = bname;
+            }
+            else
+                bi = it->second;
+            d->blobs[bi].producer = li;
+            layer->tops[j] = bi;
+        }
+
+        if (pd.load_param(dr) != 0)
+        {
+            NCNN_LOGE("ParamDict load_param %d %s failed", li, name);
+            continue;
+        }
+
+        // id 30: shape hints, [dims, w, h, c] per top blob;  id 31: feature mask
+        const Mat hints = pd.get(30, Mat());
+        if (!hints.empty())
+        {
+            const int* p = hints;
+            int pos = 0;
+            for (int j = 0; j < ntop && pos < hints.w; j++)
+            {
+                const int dims = p[pos];
+                if (pos + 4 > hints.w) break;
+                Blob& b = d->blobs[layer->tops[j]];
+                Mat s;
+                s.dims = dims;
+                s.w = p[pos + 1];
+                s.h = dims >= 2 ? p[pos + 2] : 1;
+                s.c = dims >= 3 ? p[pos + 3] : 1;
+                s.d = 1;
+                b.shape = s;
+                pos += 4;
+            }
+        }
+        layer->bottom_shapes.resize((size_t)nbottom);
+        for (int j = 0; j < nbottom; j++) layer->bottom_shapes[j] = d->blobs[layer->bottoms[j]].shape;
+        layer->top_shapes.resize((size_t)ntop);
+        for (int j = 0; j < ntop; j++) layer->top_shapes[j] = d->blobs[layer->tops[j]].shape;
+        layer->featmask = pd.get(31, 0);
+
+        int ret = layer->load_param(pd);
+        if (ret != 0)
+        {
+            NCNN_LOGE("layer load_param %d %s failed", li, name);
+            clear();
+            return -1;
+        }
+    }
+
+    // graph inputs are the tops of Input layers, outputs are blobs nobody consumes
+    for (int li = 0; li < layer_count; li++)
+        if (d->layers[li]->type == "Input")
+            for (size_t j = 0; j < d->layers[li]->tops.size(); j++) d->input_idx.push_back(d->layers[li]->tops[j]);
+    for (size_t bi = 0; bi < d->blobs.size(); bi++)
+        if (d->blobs[bi].producer >= 0 && d->blobs[bi].consumer < 0) d->output_idx.push_back((int)bi);
+    for (size_t i = 0; i < d->input_idx.size(); i++) d->input_nm.push_back(d->blobs[d->input_idx[i]].name.c_str());
+    for (size_t i = 0; i < d->output_idx.size(); i++) d->output_nm.push_back(d->blobs[d->output_idx[i]].name.c_str());
+    return 0;
+}
+
+int Net::load_param(FILE* fp)
+{
+    DataReaderFromStdio dr(fp);
+    return load_param(dr);
+}
+
+int Net::load_param(const char* protopath)
+{
+    FILE* fp = fopen(protopath, "rb");
+    if (!fp)
+    {
+        NCNN_LOGE("fopen %s failed", protopath);
+        return -1;
+    }
+    int ret = load_param(fp);
+    fclose(fp);
+    return ret;
+}
+
+int Net::load_param_mem(const char* mem)
+{
+    const unsigned char* cursor = (const unsigned char*)mem;
+    DataReaderFromMemory dr(cursor);
+    return load_param(dr);
+}
+
+int Net::load_model(const DataReader& dr)
+{
+    if (d->layers.empty())
+    {
+        NCNN_LOGE("network graph not ready");
+        return -1;
+    }
+    ModelBinFromDataReader mb(dr);
+    int status = 0;
+    for (size_t i = 0; i < d->layers.size(); i++)
+    {
+        Layer* layer = d->layers[i];
+        if (!layer)
+        {
+            NCNN_LOGE("load_model error at layer %d, parameter file has inconsistent content.", (int)i);
+            status = -1;
+            break;
+        }
+        int ret = layer->load_model(mb);
+        if (ret != 0)
+        {
+            NCNN_LOGE("layer load_model %d %s failed", (int)i, layer->name.c_str());
+            status = -1;
+            break;
+        }
+        Option layer_opt = opt;
+        if (layer->featmask & (1 << 3)) layer_opt.use_int8_inference = false;
+        if (layer->featmask & (1 << 7)) layer_opt.num_threads = 1;
+        ret = layer->create_pipeline(layer_opt);
+        if (ret != 0)
+        {
+            NCNN_LOGE("layer create_pipeline %d %s failed", (int)i, layer->name.c_str());
+            status = -1;
+            break;
+        }
+    }
+    return status;
+}
+
+int Net::load_model(FILE* fp)
+{
+    DataReaderFromStdio dr(fp);
+    return load_model(dr);
+}
+
+int Net::load_model(const char* modelpath)
+{
+    FILE* fp = fopen(modelpath, "rb");
+    if (!fp)
+    {
+        NCNN_LOGE("fopen %s failed", modelpath);
+        return -1;
+    }
+    int ret = load_model(fp);
+    fclose(fp);
+    return ret;
+}
+
+size_t Net::load_model(const unsigned char* mem)
+{
+    const unsigned char* cursor = mem;
+    DataReaderFromMemory dr(cursor);
+    load_model(dr);
+    return (size_t)(cursor - mem);
+}
+
+void Net::clear()
+{
+    for (size_t i = 0; i < d->layers.size(); i++)
+    {
+        Layer* layer = d->layers[i];
+        if (!layer) continue;
+        if (layer->destroy_pipeline(opt) != 0) NCNN_LOGE("layer destroy_pipeline failed");
+        d->destroy_layer(layer);
+    }
+    d->layers.clear();
+    d->blobs.clear();
+    d->input_idx.clear();
+    d->output_idx.clear();
+    d->input_nm.clear();
+    d->output_nm.clear();
+}
+
+Extractor Net::create_extractor() const
+{
+    return Extractor(this, d->blobs.size());
+}
+
+const std::vector<int>& Net::input_indexes() const
+{
+    return d->input_idx;
+}
+const std::vector<int>& Net::output_indexes() const
+{
+    return d->output_idx;
+}
+const std::vector<const char*>& Net::input_names() const
+{
+    return d->input_nm;
+}
+const std::vector<const char*>& Net::output_names() const
+{
+    return d->output_nm;
+}
+const std::vector<Blob>& Net::blobs() const
+{
+    return d->blobs;
+}
+const std::vector<Layer*>& Net::layers() const
+{
+    return d->layers;
+}
+
+int Net::find_blob_index_by_name(const char* name) const
+{
+    for (size_t i = 0; i < d->blobs.size(); i++)
+        if (d->blobs[i].name == name) return (int)i;
+    NCNN_LOGE("find_blob_index_by_name %s failed", name);
+    return -1;
+}
+
+int Net::find_layer_index_by_name(const char* name) const
+{
+    for (size_t i = 0; i < d->layers.size(); i++)
+        if (d->layers[i]->name == name) return (int)i;
+    NCNN_LOGE("find_layer_index_by_name %s failed", name);
+    return -1;
+}
+
+// ---- Extractor ----------------------------------------------------------------------------
+
+class ExtractorPrivate
+{
+public:
+    const Net* net;
+    std::vector<Mat> blob_mats;
+    Option opt;
+};
+
+Extractor::Extractor(const Net* net, size_t blob_count) : d(new ExtractorPrivate)
+{
+    d->net = net;
+    d->blob_mats.resize(blob_count);
+    d->opt = net->opt;
+}
+
+Extractor::~Extractor()
+{
+    clear();
+    delete d;
+}
+
+Extractor::Extractor(const Extractor& rhs) : d(new ExtractorPrivate)
+{
+    *d = *rhs.d;
+}
+
+Extractor& Extractor::operator=(const Extractor& rhs)
+{
+    if (this != &rhs) *d = *rhs.d;
+    return *this;
+}
+
+void Extractor::clear()
+{
+    d->blob_mats.clear();
+}
+void Extractor::set_light_mode(bool enable)
+{
+    d->opt.lightmode = enable;
+}
+void Extractor::set_num_threads(int num_threads)
+{
+    d->opt.num_threads = num_threads;
+}
+void Extractor::set_blob_allocator(Allocator* allocator)
+{
+    d->opt.blob_allocator = allocator;
+}
+void Extractor::set_workspace_allocator(Allocator* allocator)
+{
+    d->opt.workspace_allocator = allocator;
+}
+
+int Extractor::input(const char* blob_name, const Mat& in)
+{
+    const int bi = d->net->find_blob_index_by_name(blob_name);
+    if (bi < 0) return -1;
+    return input(bi, in);
+}
+
+int Extractor::input(int blob_index, const Mat& in)
+{
+    if (blob_index < 0 || blob_index >= (int)d->blob_mats.size()) return -1;
+    d->blob_mats[blob_index] = in;
+    return 0;
+}
+
+int Extractor::extract(const char* blob_name, Mat& feat, int type)
+{
+    const int bi = d->net->find_blob_index_by_name(blob_name);
+    if (bi < 0) return -1;
+    return extract(bi, feat, type);
+}
+
+int Extractor::extract(int blob_index, Mat& feat, int type)
+{
+    if (blob_index < 0 || blob_index >= (int)d->blob_mats.size()) return -1;
+    int ret = 0;
+    if (d->blob_mats[blob_index].dims == 0)
+    {
+        const int producer = d->net->d->blobs[blob_index].producer;
+        if (producer < 0) return -1;
+        ret = d->net->d->forward_layer(producer, d->blob_mats, d->opt);
+    }
+    feat = d->blob_mats[blob_index];
+    if (ret == 0 && type == 0 && feat.elemsize == 1u && !feat.empty())
+    {
+        Mat wide;
+        ret = expand_int8(feat, wide, d->opt.blob_allocator);
+        if (ret == 0) feat = wide;
+    }
+    return ret;
+}
+
+} // namespace ncnn

@@ -1,0 +1,97 @@
+// Net and Extractor: the caller-facing API that stays unchanged around the int8 layers
+// (public surface of src/net.h that the path uses; Vulkan and platform loaders left out).
+#ifndef NCNN_NET_H
+#define NCNN_NET_H
+
+#include <stdio.h>
+
+#include <vector>
+
+#include "blob.h"
+#include "layer.h"
+#include "mat.h"
+#include "option.h"
+#include "platform.h"
+
+namespace ncnn {
+
+class DataReader;
+class Extractor;
+class NetPrivate;
+class NCNN_EXPORT Net
+{
+public:
+    Net();
+    virtual ~Net();
+
+    Option opt;
+
+    // A built-in type name replaces that built-in (the route the HIP layers take); any other name
+    // adds a new type.  Must be called before load_param.
+    int register_custom_layer(const char* type, layer_creator_func creator, layer_destroyer_func destroyer = 0, void* userdata = 0);
+    int register_custom_layer(int index, layer_creator_func creator, layer_destroyer_func destroyer = 0, void* userdata = 0);
+    virtual int custom_layer_to_index(const char* type);
+
+    int load_param(const DataReader& dr);
+    int load_param(FILE* fp);
+    int load_param(const char* protopath);
+    int load_param_mem(const char* mem);
+
+    int load_model(const DataReader& dr);
+    int load_model(FILE* fp);
+    int load_model(const char* modelpath);
+    size_t load_model(const unsigned char* mem); // bytes consumed
+
+    void clear();
+
+    Extractor create_extractor() const;
+
+    const std::vector<int>& input_indexes() const;
+    const std::vector<int>& output_indexes() const;
+    const std::vector<const char*>& input_names() const;
+    const std::vector<const char*>& output_names() const;
+    const std::vector<Blob>& blobs() const;
+    const std::vector<Layer*>& layers() const;
+
+protected:
+    friend class Extractor;
+    int find_blob_index_by_name(const char* name) const;
+    int find_layer_index_by_name(const char* name) const;
+
+private:
+    Net(const Net&);
+    Net& operator=(const Net&);
+    NetPrivate* const d;
+};
+
+class ExtractorPrivate;
+class NCNN_EXPORT Extractor
+{
+public:
+    virtual ~Extractor();
+    Extractor(const Extractor&);
+    Extractor& operator=(const Extractor&);
+
+    void clear();
+    void set_light_mode(bool enable);
+    void set_num_threads(int num_threads);
+    void set_blob_allocator(Allocator* allocator);
+    void set_workspace_allocator(Allocator* allocator);
+
+    int input(const char* blob_name, const Mat& in);
+    int input(int blob_index, const Mat& in);
+    // type 0: int8 results are expanded to fp32; type 1: returned as stored
+    int extract(const char* blob_name, Mat& feat, int type = 0);
+    int extract(int blob_index, Mat& feat, int type = 0);
+
+protected:
+    friend Extractor Net::create_extractor() const;
+    Extractor(const Net* net, size_t blob_count);
+
+private:
+    ExtractorPrivate* const d;
+};
+
+} // namespace ncnn
+
+#endif // NCNN_NET_H

@@ -1,0 +1,167 @@
+"""End-to-end parity through the drop-in boundary: register the HIP layers, load_param, load_model,
+create_extractor, input, extract -- against the oracle-based executor on the same .param/.bin bytes."""
+import numpy as np
+import pytest
+
+import refnet
+from ncnn_amd import host, modelwriter as mw, zoo
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _load(param, blob):
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    assert net.load_param_mem(param) == 0
+    assert net.load_model_mem(blob) == 0
+    return net
+
+
+def test_tiny_net_every_blob_matches():
+    g, param, blob, info = zoo.build("tiny")
+    x = np.random.default_rng(0).uniform(0, 1, g.input_shape).astype(F)
+    ref = refnet.run(param, blob, x)
+    net = _load(param, blob)
+    for name in ("c1", "dw", "pw", "c2", "sum", "relu", "c3", "gap", "fc"):
+        ex = net.create_extractor()
+        ex.input("data", x)
+        got = ex.extract(name)
+        want = ref[name]
+        want = want.astype(F) if want.dtype == np.int8 else want  # extract() expands int8 blobs to fp32
+        assert got.shape == want.shape, name
+        assert np.array_equal(got, want), name
+    ex = net.create_extractor()
+    ex.input("data", x)
+    assert np.allclose(ex.extract("prob"), ref["prob"], rtol=1e-6, atol=1e-7)
+
+
+def test_tiny_net_lightmode_off_and_shared_thread_stream():
+    g, param, blob, info = zoo.build("tiny", seed=3)
+    x = np.random.default_rng(1).uniform(0, 1, g.input_shape).astype(F)
+    ref = refnet.run(param, blob, x)
+    net = _load(param, blob)
+    net.set_lightmode(False)
+    ex = net.create_extractor(own_stream=False)
+    ex.input("data", x)
+    assert np.array_equal(ex.extract("fc"), ref["fc"])
+    assert np.array_equal(ex.extract("c3"), ref["c3"].astype(F))  # still held with light mode off
+
+
+def test_batch_equals_per_sample():
+    g, param, blob, info = zoo.build("tiny", seed=5)
+    xs = np.random.default_rng(2).uniform(0, 1, (3,) + g.input_shape).astype(F)
+    net = _load(param, blob)
+    ex = net.create_extractor()
+    ex.input("data", xs)
+    got = ex.extract("fc")
+    assert got.shape[0] == 3
+    for i in range(3):
+        assert np.array_equal(got[i].reshape(-1), refnet.run(param, blob, xs[i])["fc"])
+
+
+def test_int8_inference_switched_off_is_an_error_not_a_fallback():
+    g, param, blob, info = zoo.build("tiny")
+    net = _load(param, blob)
+    net.set_use_int8_inference(False)
+    ex = net.create_extractor()
+    ex.input("data", np.zeros(g.input_shape, F))
+    with pytest.raises(RuntimeError):
+        ex.extract("fc")
+
+
+# ----------------------------------------------------------------------------- single layers through the boundary
+def _single(param_lines, blob, feeds, out):
+    net = _load(mw.assemble_param(param_lines), blob)
+    ex = net.create_extractor()
+    for k, v in feeds.items():
+        ex.input(k, v)
+    return ex.extract(out)
+
+
+def test_gemm_layer_int8_constant_b_with_bias():
+    rng = np.random.default_rng(4)
+    m, n, k = 37, 50, 96
+    a = rng.standard_normal((m, k), dtype=F)
+    bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sb = F(63.5)
+    c = rng.standard_normal((1, n), dtype=F)
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m),
+             mw.gemm_param("g", ["a"], "out", M=0, N=n, K=k, constantB=1, constantC=1, broadcast_type_C=4, quantize_term=2)]
+    blob = mw.weight_blob(bq) + mw.weight_blob(c) + mw.raw_f32(sb)
+    got = _single(lines, blob, {"a": a}, "out")
+    aq, sa = oracle.gemm_quantize_rows(a)
+    assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, [sb], c, 4))
+
+
+def test_gemm_layer_int8_two_dynamic_operands_transposed_output():
+    rng = np.random.default_rng(5)
+    m, n, k = 20, 33, 64
+    a = rng.standard_normal((m, k), dtype=F)
+    b = (rng.standard_normal((k, n), dtype=F) * F(0.02)).astype(F)  # transB = 0: stored [K][N]
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m), "Input in1 0 1 b 0=%d 1=%d" % (n, k),
+             mw.gemm_param("g", ["a", "b"], "out", transB=0, constantB=0, quantize_term=2, output_transpose=1, alpha=0.5)]
+    got = _single(lines, b"", {"a": a, "b": b}, "out")
+    aq, sa = oracle.gemm_quantize_rows(a)
+    bq, sb = oracle.gemm_quantize_tensor(b)
+    want = oracle.gemm_int8(aq, bq.T.copy(), sa, [sb], None, -1, 0.5, 1.0, True)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("bits,block,insc", [(8, 64, 0), (4, 32, 1), (6, 128, 0)])
+def test_gemm_layer_block_quant(bits, block, insc):
+    import npref
+    rng = np.random.default_rng(bits)
+    m, n, k = 4, 24, 200
+    a = rng.standard_normal((m, k), dtype=F)
+    w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    ins = (0.75 + (np.arange(k) % 5) * 0.15).astype(F) if insc else None
+    term = bits * 100 + insc * 10 + {32: 0, 64: 1, 128: 2}[block]
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m), mw.gemm_param("g", ["a"], "out", N=n, K=k, constantB=1, quantize_term=term)]
+    blob = mw.weight_blob(packed.view(np.int8)) + mw.raw_f32(scales) + (mw.raw_f32(ins) if insc else b"")
+    got = _single(lines, blob, {"a": a}, "out")
+    val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins)
+    assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
+
+
+def test_innerproduct_layer_2d_rows_and_fp32_weights_quantised_at_load():
+    rng = np.random.default_rng(6)
+    rows, k, n = 5, 48, 12
+    x = rng.uniform(-1, 1, (rows, k)).astype(F)
+    wf = rng.normal(0, 0.1, (n, k)).astype(F)
+    ws = (F(127) / np.abs(wf).max(axis=1)).astype(F)
+    in_scale = F(127) / np.abs(x).max()
+    b = rng.normal(size=n).astype(F)
+    lines = ["Input in0 0 1 x 0=%d 1=%d" % (k, rows), mw.innerproduct_param("fc", "x", "out", n, n * k, 1, 2, 1)]
+    blob = mw.conv_weights(wf.reshape(-1), b, ws, in_scale, None)  # fp32 weights in the file
+    got = _single(lines, blob, {"x": x}, "out")
+    wq = oracle.quantize_weights(wf, ws)
+    assert np.array_equal(got, oracle.innerproduct_int8(x, wq, b, ws, in_scale, 1))
+
+
+# ----------------------------------------------------------------------------- the two benchmark networks
+@pytest.mark.parametrize("which,hw", [("resnet50", 224), ("mobilenetv2", 224)])
+def test_benchmark_network_batch1_matches_oracle_executor(which, hw):
+    _say("building", which)
+    g, param, blob, info = zoo.build(which, input_hw=hw, n_calib=2)
+    x = np.random.default_rng(9).uniform(0, 1, g.input_shape).astype(F)
+    last_fc = "fc1000" if which == "resnet50" else "fc"
+    _say("oracle forward", which)
+    ref = refnet.run(param, blob, x, want=last_fc)
+    _say("device forward", which)
+    net = _load(param, blob)
+    ex = net.create_extractor()
+    ex.input("data", x)
+    got = ex.extract(last_fc)
+    assert np.array_equal(got, ref[last_fc])
+    # a requantised (int8) blob deep in the net, bit for bit
+    probe = "res4c_branch2b" if which == "resnet50" else "block10_dw"
+    ex = net.create_extractor()
+    ex.input("data", x)
+    assert np.array_equal(ex.extract(probe), ref[probe].astype(F))

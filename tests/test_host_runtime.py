@@ -1,0 +1,180 @@
+"""Host-side logic of the ncnn-API mirror (no GPU needed): .param parsing, .bin reading, Mat layout,
+graph loading with the HIP layers registered, and the C-ABI symbol tables of both libraries."""
+import ctypes as C
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import ncnn_amd
+from ncnn_amd import hip, host
+
+F = np.float32
+
+
+def bits(f):
+    return struct.unpack("<I", struct.pack("<f", f))[0]
+
+
+# ----------------------------------------------------------------------------- symbols
+def test_libncnnhip_exports_every_declared_symbol():
+    lib = hip.lib()
+    import re
+    hdr = open(os.path.join(os.path.dirname(ncnn_amd.__file__), "..", "include", "ncnnhip.h")).read()
+    declared = set(re.findall(r"\b(ncnnhip_[a-z0-9_]+)\s*\(", hdr))
+    assert declared == set(hip.EXPORTED_SYMBOLS), declared ^ set(hip.EXPORTED_SYMBOLS)
+    for name in declared:
+        getattr(lib, name)
+
+
+def test_libncnn_amd_exports_every_declared_symbol():
+    lib = host.lib()
+    import re
+    hdr = open(os.path.join(os.path.dirname(ncnn_amd.__file__), "..", "include", "ncnn_amd_c_api.h")).read()
+    declared = set(re.findall(r"\b(ncnn(?:hip)?_[a-z0-9_]+)\s*\(", hdr))
+    assert len(declared) > 40
+    for name in declared:
+        getattr(lib, name)
+
+
+# ----------------------------------------------------------------------------- ParamDict
+def test_paramdict_ints_floats_arrays():
+    t, v, arr = host.paramdict_probe("0=64 1=3 11=5 9=1 18=2.5 10=0.0,6.0 6=36864 -23303=3,1,2,3\n", 0)
+    assert (t, v) == (2, 64)
+    assert host.paramdict_probe("0=64 18=2.5\n", 18)[:2] == (3, bits(2.5))
+    t, n, arr = host.paramdict_probe("10=0.0,6.0 0=1\n", 10)
+    assert t == 6 and n == 2 and arr[:2] == [bits(0.0), bits(6.0)]
+    t, n, arr = host.paramdict_probe("-23303=3,1,2,3 0=1\n", 3)
+    assert t == 5 and n == 3 and arr[:3] == [1, 2, 3]
+    t, n, arr = host.paramdict_probe("-23310=2,0.000000e+00,6.000000e+00\n", 10)
+    assert t == 6 and arr[:2] == [bits(0.0), bits(6.0)]
+    assert host.paramdict_probe("0=1\n", 5)[0] == 0  # unset
+
+
+def test_paramdict_int_literal_read_as_float_is_the_bit_pattern():
+    # "0=1" for a float parameter yields the int's bits (1.4e-45), as in the reference's union storage
+    t, v, _ = host.paramdict_probe("0=1\n", 0)
+    assert t == 2 and v == 1
+
+
+@pytest.mark.parametrize("text,want", [("1.25", 1.25), ("-0.5", -0.5), ("6.000000e+00", 6.0), ("1.234567e-01", None), ("3.e2", 300.0),
+                                         ("1e-3", None), ("+2.5E1", 25.0), ("0.1", None), ("123456.789", None), ("7.0e-10", None)])
+def test_paramdict_float_parser_follows_the_reference_recipe(text, want):
+    # recipe: uint digits -> double (whole + frac/10^n), scaled by repeated *1e8 / *10, then rounded to float
+    def recipe(s):
+        neg = s.startswith("-")
+        s = s.lstrip("+-")
+        mant, _, ex = s.lower().partition("e")
+        whole, _, frac = mant.partition(".")
+        v = float(int(whole or "0") & 0xffffffff)
+        if frac:
+            v += (int(frac) & 0xffffffff) / float((10 ** len(frac)) & 0xffffffff)
+        if ex:
+            eneg = ex.startswith("-")
+            e = int(ex.lstrip("+-"))
+            scale = 1.0
+            while e >= 8:
+                scale *= 1e8
+                e -= 8
+            while e > 0:
+                scale *= 10.0
+                e -= 1
+            v = v / scale if eneg else v * scale
+        return np.float32(-v if neg else v)
+    t, v, _ = host.paramdict_probe("3=%s\n" % text, 3)
+    assert t == 3 and v == bits(float(recipe(text)))
+    if want is not None:
+        assert v == bits(want)
+
+
+def test_paramdict_rejects_id_out_of_range():
+    assert host.paramdict_probe("40=1\n", 0)[0] == -1
+
+
+# ----------------------------------------------------------------------------- ModelBin
+def test_modelbin_tags():
+    w = np.array([1.5, -2.0, 3.25], F)
+    q = np.array([1, -2, 3, -127, 127], np.int8)
+    assert np.array_equal(host.modelbin_probe(host.tagged_fp32(w), 3, 0)[0], w)
+    got, used = host.modelbin_probe(host.tagged_int8(q), 5, 0)
+    assert got.dtype == np.int8 and np.array_equal(got, q) and used == 4 + 8  # payload padded to 4 bytes
+    h = np.array([0.5, -1.0, 65504.0], np.float16)
+    got, used = host.modelbin_probe(host.tagged_fp16(h), 3, 0)
+    assert np.array_equal(got, h.astype(F)) and used == 4 + 8
+    got, used = host.modelbin_probe(w.tobytes(), 3, 1)
+    assert np.array_equal(got, w) and used == 12
+    raw = struct.pack("<I", 0x0002C056) + w.tobytes()
+    assert np.array_equal(host.modelbin_probe(raw, 3, 0)[0], w)
+    # table-coded weights: 256-entry fp32 table + one index byte per weight
+    table = np.arange(256, dtype=F) * F(0.5)
+    idx = np.array([3, 200, 7], np.uint8)
+    blob = struct.pack("<I", 0x01020304) + table.tobytes() + idx.tobytes() + b"\0"
+    assert np.array_equal(host.modelbin_probe(blob, 3, 0)[0], table[idx])
+
+
+# ----------------------------------------------------------------------------- Mat layout
+@pytest.mark.parametrize("w,h,c,es,n", [(56, 56, 64, 4, 1), (58, 58, 3, 1, 1), (7, 7, 5, 4, 3), (224, 224, 3, 4, 16), (3, 3, 2, 1, 2)])
+def test_mat_cstep_and_nstep_rules(w, h, c, es, n):
+    m = host.Mat.batch3d(w, h, c, es, n)
+    cstep = ((w * h * es + 15) // 16) * 16 // es
+    assert m.cstep == cstep
+    if n > 1:
+        assert m.nstep == ((cstep * c * es + 4095) // 4096) * 4096 // es
+    else:
+        assert m.nstep == cstep * c
+    assert (m.dims, m.w, m.h, m.c, m.n, m.elemsize) == (3, w, h, c, n, es)
+
+
+# ----------------------------------------------------------------------------- graph loading
+PARAM = """7767517
+7 8
+Input            data    0 1 data 0=8 1=8 2=4
+Convolution      c1      1 1 data c1 0=6 1=3 4=1 5=1 6=216 8=102 9=1
+Split            sp      1 2 c1 c1a c1b
+ConvolutionDepthWise dw  1 1 c1a dw 0=6 1=3 4=1 5=1 6=54 7=6 8=1 9=3 -23310=2,0.0,6.0
+Convolution      c2      1 1 c1b c2 0=6 1=1 5=0 6=36 8=2
+Eltwise          add     2 1 dw c2 sum 0=1
+ReLU             relu    1 1 sum out
+"""
+
+
+def test_load_param_with_hip_layers_registered():
+    net = host.Net()
+    net.register_int8_layers()
+    assert net.load_param_mem(PARAM) == 0
+    assert net.layer_types() == ["Input", "Convolution", "Split", "ConvolutionDepthWise", "Convolution", "Eltwise", "ReLU"]
+    flags = net.layer_flags()
+    # Convolution: one_blob_only, not inplace, int8 storage, batch folding, no packing
+    assert flags[1] == 1 | 4 | 8 and flags[3] == 1 | 4 | 8
+    assert net.input_names() == ["data"] and net.output_names() == ["out"]
+    blobs = net.blobs()
+    assert blobs["c1"] == (1, 2) and blobs["c1a"] == (2, 3) and blobs["sum"] == (5, 6) and blobs["out"] == (6, -1)
+
+
+def test_hot_layers_have_no_host_fallback():
+    # without the HIP layers a net using Convolution cannot even be built
+    net = host.Net()
+    assert net.load_param_mem(PARAM) != 0
+
+
+def test_non_quantised_convolution_is_refused():
+    net = host.Net()
+    net.register_int8_layers()
+    bad = PARAM.replace("8=102 9=1", "9=1")
+    assert net.load_param_mem(bad) != 0
+
+
+@pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="checks the failure mode on a machine without a GPU")
+def test_load_model_fails_loudly_without_a_gpu():
+    from ncnn_amd import modelwriter
+    rng = np.random.default_rng(0)
+    net = host.Net()
+    net.register_int8_layers()
+    assert net.load_param_mem(PARAM) == 0
+    binimg = b"".join([
+        modelwriter.conv_weights(rng.integers(-127, 128, 216).astype(np.int8), rng.normal(size=6).astype(F), np.full(6, 50, F), 20.0, 10.0),
+        modelwriter.conv_weights(rng.integers(-127, 128, 54).astype(np.int8), rng.normal(size=6).astype(F), np.full(6, 50, F), 10.0, None),
+        modelwriter.conv_weights(rng.integers(-127, 128, 36).astype(np.int8), None, np.full(6, 50, F), 10.0, None),
+    ])
+    assert net.load_model_mem(binimg) != 0  # create_pipeline needs the device
