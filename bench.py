@@ -62,6 +62,16 @@ def cpu_baseline_gemm(n, k, budget_s=12.0):
             "sample": "%d of %d rows of the same Gemm (N=%d, K=%d), scalar OpenMP oracle, %.1f s" % (rows, n, n, k, dt)}
 
 
+def measured_traffic(key):
+    """bytes per launch past L2 (read + write) from the committed counter summary, or None"""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            e = json.load(f).get(key)
+        return None if e is None else e["read_bytes"] + e["write_bytes"]
+    except (OSError, ValueError, KeyError):
+        return None
+
+
 def bench_gemm(args, size):
     import ncnn_amd
     from ncnn_amd.hip import check, lib as load
@@ -87,6 +97,9 @@ def bench_gemm(args, size):
         if ev:
             check(lib.ncnnhip_event_record(ev[2], st))
 
+    if args.calib_copy:
+        # one device-to-device copy of known size: gives counter runs (FETCH_SIZE / WRITE_SIZE) a dispatch to calibrate against
+        check(lib.ncnnhip_memcpy_d2d(d_out.ptr, d_a.ptr, m * k * 4, st))
     for _ in range(args.warmup):
         step()
     rt.sync()
@@ -120,7 +133,7 @@ def bench_gemm(args, size):
         "config": {"workload": "standalone int8 Gemm M=N=K=%d: per-row quantise A (fp32->int8) + int8 MFMA Gemm + fused dequantise/bias to fp32" % size,
                    "b_scale": args.b_scale, "kernel_ms": {"gemm_int8": gemm_ms, "quantize_rows": quant_ms}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": None, "kernel": "gemm_int8", "ops_per_launch": ops},
+                     "traffic": measured_traffic("gemm%d" % size), "kernel": "gemm_int8", "ops_per_launch": ops},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm(n, k)
@@ -196,6 +209,7 @@ def main():
                     help="per_column is the benchmark configuration; per_tensor is what ncnn's Gemm layer can express")
     ap.add_argument("--act", default="fp16", choices=["fp16", "fp32"], help="activation type of the block-quant workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true", help="issue one D2D copy of M*K*4 bytes first (calibrates HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU only (--gpus 1); multi-GPU figures are not produced")
