@@ -198,17 +198,138 @@ def bench_blockquant(args, n, k, m):
     }
 
 
+def bench_net(args, which, batch):
+    """The quantised layers of a ResNet-50 / MobileNetV2-shaped int8 net, each on device-resident synthetic blobs of
+    its real shape: fp32 inputs are quantised on the device first, int8 inputs feed the kernel directly, outputs are
+    requantised int8 or fp32 exactly as the generated model asks.  One step = one pass over all quantised layers."""
+    import ncnn_amd
+    from ncnn_amd.hip import Activation, ConvDesc, check, lib as load
+    from ncnn_amd import zoo
+    lib = load()
+    rt = ncnn_amd.Runtime(0)
+    st = rt.stream
+    g = getattr(zoo, which)()
+    rows = zoo.quantised_layer_table(g)
+    rng = np.random.default_rng(0)
+    plans = []
+    for r in rows:
+        if r["type"] == "InnerProduct":
+            k, n = int(np.prod(r["in_shape"])), r["out_shape"][0]
+            x = rng.uniform(-1, 1, (batch, k)).astype(np.float32)
+            plan = dict(row=r, kind="fc", k=k, n=n, d_x=rt.up(x), d_xq=ncnn_amd.DeviceBuffer.empty((batch, k), np.int8),
+                        d_w=rt.up(rng.integers(-127, 128, (n, k)).astype(np.int8)), d_si=rt.up(rng.uniform(1e-4, 1e-3, n).astype(np.float32)),
+                        d_b=rt.up(rng.uniform(-0.1, 0.1, n).astype(np.float32)), d_s=rt.up(np.array([50.0], np.float32)),
+                        d_out=ncnn_amd.DeviceBuffer.empty((batch, n), np.float32))
+        else:
+            c, h, w = r["in_shape"]
+            cout, oh, ow = r["out_shape"]
+            cstep = (h * w + 15) // 16 * 16
+            ocs = (oh * ow + (15 if r["int8_out"] else 3)) // (16 if r["int8_out"] else 4) * (16 if r["int8_out"] else 4)
+            desc = ConvDesc(w, h, c, batch, cout, r["k"], r["k"], 1, 1, r["stride"], r["stride"], r["pad"], r["pad"], r["pad"], r["pad"], 0.0, r["group"])
+            plan = dict(row=r, kind="conv", desc=desc, cstep=cstep, ocs=ocs,
+                        d_xq=rt.up(rng.integers(-127, 128, (batch, c, cstep)).astype(np.int8)),
+                        d_w=rt.up(rng.integers(-127, 128, cout * (c // r["group"]) * r["k"] * r["k"]).astype(np.int8)),
+                        d_si=rt.up(rng.uniform(1e-4, 1e-3, cout).astype(np.float32)), d_b=rt.up(rng.uniform(-0.1, 0.1, cout).astype(np.float32)),
+                        d_so=rt.up(np.full(cout, 20.0, np.float32)) if r["int8_out"] else None,
+                        d_out=ncnn_amd.DeviceBuffer.empty((batch, cout, ocs), np.int8 if r["int8_out"] else np.float32),
+                        act=Activation.make(r["act"], r["act_params"]))
+            if not r["int8_in"]:
+                plan["d_x"] = rt.up(rng.uniform(-1, 1, (batch, c, h * w)).astype(np.float32))
+                plan["d_s"] = rt.up(np.array([100.0], np.float32))
+            if r["group"] == 1:
+                # channels-last path: weights packed once (as create_pipeline does), activations transposed per step
+                nb, wb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
+                check(lib.ncnnhip_conv_nhwc_sizes(C.byref(desc), C.byref(nb), C.byref(wb), C.byref(sb)))
+                wq = rng.integers(-127, 128, cout * c * r["k"] * r["k"]).astype(np.int8)
+                pk = np.empty(wb.value, np.int8)
+                check(lib.ncnnhip_conv_pack_weights(C.byref(desc), wq.ctypes.data, pk.ctypes.data))
+                plan.update(d_pk=rt.up(pk), d_nhwc=ncnn_amd.DeviceBuffer(nb.value), d_ws=ncnn_amd.DeviceBuffer(max(sb.value, 4)), ws_bytes=sb.value)
+        plans.append(plan)
+
+    def run_layer(p):
+        r = p["row"]
+        if p["kind"] == "fc":
+            check(lib.ncnnhip_quantize(p["d_x"].ptr, p["k"], 0, p["d_xq"].ptr, p["k"], 0, batch, p["k"], 1, p["d_s"].ptr, 1, st))
+            check(lib.ncnnhip_innerproduct_int8(p["d_xq"].ptr, p["k"], batch, p["k"], p["n"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
+                                                Activation.make(0), p["d_out"].ptr, p["n"], None, st))
+            return
+        c, h, w = r["in_shape"]
+        if r["group"] == 1:
+            if r["int8_in"]:
+                check(lib.ncnnhip_to_nhwc_int8(C.byref(p["desc"]), p["d_xq"].ptr, 1, p["cstep"], c * p["cstep"], None, 1, p["d_nhwc"].ptr, st))
+            else:
+                check(lib.ncnnhip_to_nhwc_int8(C.byref(p["desc"]), p["d_x"].ptr, 4, h * w, c * h * w, p["d_s"].ptr, 1, p["d_nhwc"].ptr, st))
+            check(lib.ncnnhip_conv_int8_nhwc(C.byref(p["desc"]), p["d_nhwc"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr,
+                                             p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, p["ocs"], r["out_shape"][0] * p["ocs"],
+                                             p["d_ws"].ptr, p["ws_bytes"], st))
+            return
+        if not r["int8_in"]:
+            check(lib.ncnnhip_quantize(p["d_x"].ptr, h * w, c * h * w, p["d_xq"].ptr, p["cstep"], c * p["cstep"], c, h * w, batch, p["d_s"].ptr, 1, st))
+        check(lib.ncnnhip_conv_int8(C.byref(p["desc"]), p["d_xq"].ptr, p["cstep"], c * p["cstep"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
+                                    p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, p["ocs"], r["out_shape"][0] * p["ocs"], None, st))
+
+    def step():
+        for p in plans:
+            run_layer(p)
+
+    for _ in range(args.warmup):
+        step()
+    rt.sync()
+    # per-layer times (back-to-back launches of one layer)
+    table = []
+    for p in plans:
+        ev = _events(lib, check, 2)
+        reps = 10
+        check(lib.ncnnhip_event_record(ev[0], st))
+        for _ in range(reps):
+            run_layer(p)
+        check(lib.ncnnhip_event_record(ev[1], st))
+        check(lib.ncnnhip_event_synchronize(ev[1]))
+        us = _elapsed(lib, check, ev[0], ev[1]) * 1e3 / reps
+        r = p["row"]
+        table.append((r["name"], r["type"], r["in_shape"], r["out_shape"], r["k"], r["stride"], r["group"], 2.0 * r["macs"] * batch, us))
+    evs = _events(lib, check, 2)
+    check(lib.ncnnhip_device_synchronize())
+    t0 = time.perf_counter()
+    check(lib.ncnnhip_event_record(evs[0], st))
+    for _ in range(args.steps):
+        step()
+    check(lib.ncnnhip_event_record(evs[1], st))
+    check(lib.ncnnhip_device_synchronize())
+    wall = time.perf_counter() - t0
+    dev_ms = _elapsed(lib, check, evs[0], evs[1]) / args.steps
+    ops = sum(t[7] for t in table)
+    ms_per_step = wall * 1e3 / args.steps
+    if args.layer_table:
+        with open(args.layer_table, "w") as f:
+            f.write("%-22s %-22s %-18s %-18s k s group %12s %10s %10s\n" % ("layer", "type", "in", "out", "ops", "us", "TOPS"))
+            for t in sorted(table, key=lambda t: -t[8]):
+                f.write("%-22s %-22s %-18s %-18s %d %d %5d %12.0f %10.2f %10.2f\n" % (t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[7] / t[8] / 1e6))
+            f.write("sum of per-layer times %.1f us; whole pass %.1f us (device events)\n" % (sum(t[8] for t in table), dev_ms * 1e3))
+    worst = max(table, key=lambda t: t[8])
+    achieved = ops / (dev_ms * 1e-3) / 1e12
+    return {
+        "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "%s-shaped int8 net, the %d quantised layers (conv/depthwise/fc) on resident blobs, batch %d" % (which, len(plans), batch),
+                   "images_per_s": batch / (ms_per_step * 1e-3), "slowest_layer": [worst[0], worst[8]]},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
+                     "traffic": None, "kernel": "conv_tile_kernel (all layers of the pass)", "ops_per_launch": ops},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
-                    help="gemm<size> | blockquant:<N>x<K>x<M>")
+                    help="gemm<size> | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch>")
     ap.add_argument("--b-scale", dest="b_scale", default="per_column", choices=["per_column", "per_tensor"],
                     help="per_column is the benchmark configuration; per_tensor is what ncnn's Gemm layer can express")
     ap.add_argument("--act", default="fp16", choices=["fp16", "fp32"], help="activation type of the block-quant workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layer-table", default=None, help="net workloads: write the per-layer timing table to this file")
     ap.add_argument("--calib-copy", action="store_true", help="issue one D2D copy of M*K*4 bytes first (calibrates HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -218,6 +339,9 @@ def main():
     elif args.workload.startswith("blockquant:"):
         n, k, m = (int(v) for v in args.workload.split(":")[1].split("x"))
         line = bench_blockquant(args, n, k, m)
+    elif args.workload.startswith("net:"):
+        _, which, batch = args.workload.split(":")
+        line = bench_net(args, which, int(batch))
     else:
         raise SystemExit("unknown workload " + args.workload)
     print(json.dumps(line), flush=True)

@@ -108,6 +108,21 @@ int ncnnhip_conv_int8(const ncnnhip_conv_desc* desc, const int8_t* x_dev, size_t
                       const float* scale_out_dev, ncnnhip_activation act, void* out_dev, size_t out_cstep,
                       size_t out_nstep, int32_t* acc_out_dev, void* stream);
 
+/* Channels-last fast path of Convolution::forward_int8 (group 1).  The activations are first copied to
+ * [batch][h][w][Cp] int8, Cp = 16*ceil(c/16) -- from fp32 with the Quantize arithmetic (one scale or one per
+ * channel) or from int8 as is -- and the weights are repacked once (host side, at create_pipeline) to
+ * [num_output][kh*kw][Cp] with K padded to a multiple of 64.  Results are identical to ncnnhip_conv_int8.
+ * workspace: int32 scratch for layers whose K loop is split across workgroups (size from ncnnhip_conv_nhwc_sizes,
+ * may be 0); it is cleared by the call itself. */
+int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes);
+int ncnnhip_conv_pack_weights(const ncnnhip_conv_desc* desc, const int8_t* weight_host, int8_t* packed_host);
+int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x_elemsize, size_t x_cstep, size_t x_nstep,
+                         const float* scales_dev, int nscales, int8_t* nhwc_dev, void* stream);
+int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev,
+                           const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
+                           void* out_dev, size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes,
+                           void* stream);
+
 /* ------------------------------------------------------------------ InnerProduct
  * InnerProduct::forward_int8 (src/layer/innerproduct.cpp:168-273) after input quantisation:
  * x int8 [rows][num_input] -> fp32 [rows][num_output];  scale_in / bias per output channel. */

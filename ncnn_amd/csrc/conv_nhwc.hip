@@ -1,0 +1,465 @@
+// int8 Convolution (group 1) as an implicit GEMM over a channels-last int8 copy of the activations.
+//
+// ncnn hands over [c][h][w] planes; a K-contiguous MFMA operand needs, for one output pixel, runs of
+// consecutive input channels.  So the quantise pre-pass writes the blob as [n][h][w][Cp] int8 with the
+// channel count padded to Cp = 16*ceil(c/16) (pad channels are zero), and the weights are repacked once at
+// create_pipeline to [num_output][kh*kw][Cp] (K order tap-major, zero in the pad channels, K padded to a
+// multiple of 64).  One 16-byte chunk of the im2col row is then one aligned 16-byte global load: channels
+// q0..q0+15 of tap (ky,kx) at that pixel, or 16 border bytes when the tap falls outside the image.
+//
+// Kernel: BM output channels x BN output pixels per workgroup (4 wavefronts 2x2, v_mfma_i32_32x32x32_i8),
+// K walked in 64-byte steps; the global loads of step t+1 are issued into registers before the MFMAs of step t
+// and written to the other LDS buffer afterwards (one barrier per step).  Layers with few output pixels
+// (ResNet tail at batch 1) split K over blockIdx.z: partial int32 sums are added atomically into a zeroed
+// workspace -- integer addition, so the result is still exact -- and a second small kernel applies the epilogue.
+#include "epilogues.h"
+#include "mfma_tile.h"
+
+namespace ncnnhip {
+
+struct NhwcGeom
+{
+    int H, W, Cp;
+    int kw, kh, dw, dh, sw, sh;
+    int pad_top, pad_left;
+    int outw, outh;
+    int npix;   // batch * outh * outw
+    int ntaps;  // kh * kw
+    int K;      // ntaps * Cp rounded up to 64
+    int cout;
+    int pad_word; // border byte replicated 4x
+};
+
+__device__ __forceinline__ uint32_t pack4b(int a, int b, int c, int d)
+{
+    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+// [n][c][h][w] fp32 or int8  ->  [n][h][w][Cp] int8.  One thread: one pixel, 16 consecutive channels.
+template<typename T>
+__global__ __launch_bounds__(256) void to_nhwc_int8_kernel(const T* __restrict__ x, size_t cstep, size_t nstep, int c, int hw, int Cp,
+                                                            const float* __restrict__ scales, int nscales, int8_t* __restrict__ out)
+{
+    const int pix = blockIdx.x * 256 + threadIdx.x;
+    const int q0 = blockIdx.y * 16;
+    const int img = blockIdx.z;
+    if (pix >= hw) return;
+    const T* xp = x + (size_t)img * nstep + pix;
+    int v[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++)
+    {
+        const int q = q0 + e;
+        int val = 0;
+        if (q < c)
+        {
+            if (sizeof(T) == 4)
+            {
+                const float s = nscales == 1 ? scales[0] : scales[q];
+                val = float2int8(mul_rn((float)xp[(size_t)q * cstep], s));
+            }
+            else
+                val = (int)xp[(size_t)q * cstep];
+        }
+        v[e] = val;
+    }
+    v4i pk;
+    pk[0] = (int)pack4b(v[0], v[1], v[2], v[3]);
+    pk[1] = (int)pack4b(v[4], v[5], v[6], v[7]);
+    pk[2] = (int)pack4b(v[8], v[9], v[10], v[11]);
+    pk[3] = (int)pack4b(v[12], v[13], v[14], v[15]);
+    *reinterpret_cast<v4i*>(out + ((size_t)img * hw + pix) * Cp + q0) = pk;
+}
+
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* p, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+template<int BM, int BN, bool SPLITK>
+__global__ __launch_bounds__(256) void conv_nhwc_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
+                                                         int steps_per_split, int32_t* __restrict__ partial)
+{
+    constexpr int TM = BM / 64, TN = BN / 64;
+    constexpr int ACH = BM * 4 / 256 > 0 ? BM * 4 / 256 : 1; // 16-byte chunks of the weight tile per thread
+    constexpr int BCH = BN * 4 / 256 > 0 ? BN * 4 / 256 : 1;
+    __shared__ __attribute__((aligned(16))) int8_t lds[2][(BM + BN) * LDS_PITCH];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
+
+    const int total_steps = g.K / 64;
+    const int step_begin = SPLITK ? blockIdx.z * steps_per_split : 0;
+    int step_end = SPLITK ? step_begin + steps_per_split : total_steps;
+    if (step_end > total_steps) step_end = total_steps;
+    if (step_begin >= step_end) return;
+
+    // ---- per-thread chunk assignment: chunk id = tid + 256*i -> tile row id>>2, K chunk j = tid&3 (same j for all i)
+    const int j = threadIdx.x & 3;
+    const bool a_thread = BM * 4 >= 256 || threadIdx.x < BM * 4;
+    const bool b_thread = BN * 4 >= 256 || threadIdx.x < BN * 4;
+
+    // weight rows
+    const int8_t* a_ptr[ACH];
+    bool a_ok[ACH];
+#pragma unroll
+    for (int i = 0; i < ACH; i++)
+    {
+        const int r = row0 + ((threadIdx.x + 256 * i) >> 2);
+        a_ok[i] = a_thread && r < g.cout;
+        a_ptr[i] = wpk + (size_t)(a_ok[i] ? r : 0) * g.K + j * 16;
+    }
+    // output pixels
+    const int8_t* b_base[BCH];
+    int b_iy0[BCH], b_ix0[BCH];
+    bool b_ok[BCH];
+#pragma unroll
+    for (int i = 0; i < BCH; i++)
+    {
+        const int n = col0 + ((threadIdx.x + 256 * i) >> 2);
+        b_ok[i] = b_thread && n < g.npix;
+        const int nn = b_ok[i] ? n : 0;
+        const int plane = g.outw * g.outh;
+        const int img = nn / plane;
+        const int rem = nn - img * plane;
+        const int oy = rem / g.outw;
+        const int ox = rem - oy * g.outw;
+        b_iy0[i] = oy * g.sh - g.pad_top;
+        b_ix0[i] = ox * g.sw - g.pad_left;
+        b_base[i] = x + (size_t)img * g.H * g.W * g.Cp;
+    }
+    // this thread's position in K: tap (ky,kx) and first channel q0 of its 16-byte chunk, advanced by 64 per step
+    int q0, ky, kx, tap;
+    {
+        const int k = step_begin * 64 + j * 16;
+        tap = k / g.Cp;
+        q0 = k - tap * g.Cp;
+        ky = tap / g.kw;
+        kx = tap - ky * g.kw;
+    }
+
+    v4i ra[ACH], rb[BCH];
+    auto fetch = [&](int step) {
+#pragma unroll
+        for (int i = 0; i < ACH; i++) ra[i] = a_ok[i] ? *reinterpret_cast<const v4i*>(a_ptr[i] + (size_t)step * 64) : v4i{0, 0, 0, 0};
+        const int dy = ky * g.dh, dx = kx * g.dw;
+        const bool tap_ok = tap < g.ntaps;
+#pragma unroll
+        for (int i = 0; i < BCH; i++)
+        {
+            v4i v = {0, 0, 0, 0};
+            if (b_ok[i] && tap_ok)
+            {
+                const int iy = b_iy0[i] + dy, ix = b_ix0[i] + dx;
+                if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
+                    v = *reinterpret_cast<const v4i*>(b_base[i] + ((size_t)iy * g.W + ix) * g.Cp + q0);
+                else
+                    v = v4i{g.pad_word, g.pad_word, g.pad_word, g.pad_word};
+            }
+            rb[i] = v;
+        }
+        // advance to the next step
+        q0 += 64;
+        while (q0 >= g.Cp)
+        {
+            q0 -= g.Cp;
+            tap++;
+            if (++kx == g.kw)
+            {
+                kx = 0;
+                ky++;
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+        int8_t* As = lds[buf];
+        int8_t* Bs = lds[buf] + BM * LDS_PITCH;
+#pragma unroll
+        for (int i = 0; i < ACH; i++)
+            if (a_thread) *reinterpret_cast<v4i*>(As + ((threadIdx.x + 256 * i) >> 2) * LDS_PITCH + j * 16) = ra[i];
+#pragma unroll
+        for (int i = 0; i < BCH; i++)
+            if (b_thread) *reinterpret_cast<v4i*>(Bs + ((threadIdx.x + 256 * i) >> 2) * LDS_PITCH + j * 16) = rb[i];
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+
+    fetch(step_begin);
+    stash(0);
+    __syncthreads();
+    for (int t = step_begin; t < step_end; t++)
+    {
+        const int buf = (t - step_begin) & 1;
+        if (t + 1 < step_end) fetch(t + 1);
+        const int8_t* As = lds[buf];
+        const int8_t* Bs = lds[buf] + BM * LDS_PITCH;
+#pragma unroll
+        for (int ks = 0; ks < 64; ks += 32)
+        {
+            v4i fa[TM], fb[TN];
+#pragma unroll
+            for (int a = 0; a < TM; a++) fa[a] = *reinterpret_cast<const v4i*>(As + (wm * (BM / 2) + a * 32 + l32) * LDS_PITCH + ks + lhi * 16);
+#pragma unroll
+            for (int b = 0; b < TN; b++) fb[b] = *reinterpret_cast<const v4i*>(Bs + (wn * (BN / 2) + b * 32 + l32) * LDS_PITCH + ks + lhi * 16);
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int b = 0; b < TN; b++) acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a], fb[b], acc[a][b], 0, 0, 0);
+        }
+        if (t + 1 < step_end) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+            {
+                const int gi = row0 + wm * (BM / 2) + a * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                const int gj = col0 + wn * (BN / 2) + b * 32 + l32;
+                if (gi < g.cout && gj < g.npix)
+                {
+                    if (SPLITK)
+                        atomicAdd(partial + (size_t)gi * g.npix + gj, acc[a][b][r]);
+                    else
+                        epi(gi, gj, acc[a][b][r]);
+                }
+            }
+}
+
+__global__ __launch_bounds__(256) void conv_splitk_finish_kernel(const int32_t* __restrict__ partial, int cout, int npix, ConvEpilogue epi)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)cout * npix) return;
+    const int p = (int)(i / npix);
+    const int n = (int)(i - (size_t)p * npix);
+    epi(p, n, partial[i]);
+}
+
+struct Pads4
+{
+    int top, bottom, left, right;
+};
+
+static Pads4 resolve_pads_nhwc(const ncnnhip_conv_desc& d)
+{
+    Pads4 p = {0, 0, 0, 0};
+    const int kext_w = d.dilation_w * (d.kernel_w - 1) + 1, kext_h = d.dilation_h * (d.kernel_h - 1) + 1;
+    if (d.pad_left > 0 || d.pad_right > 0 || d.pad_top > 0 || d.pad_bottom > 0)
+    {
+        p.top = d.pad_top;
+        p.bottom = d.pad_bottom;
+        p.left = d.pad_left;
+        p.right = d.pad_right;
+        return p;
+    }
+    const bool upper = d.pad_left == -233 && d.pad_right == -233 && d.pad_top == -233 && d.pad_bottom == -233;
+    const bool lower = d.pad_left == -234 && d.pad_right == -234 && d.pad_top == -234 && d.pad_bottom == -234;
+    if (upper || lower)
+    {
+        const int wpad = kext_w + (d.w - 1) / d.stride_w * d.stride_w - d.w;
+        const int hpad = kext_h + (d.h - 1) / d.stride_h * d.stride_h - d.h;
+        if (wpad > 0 || hpad > 0)
+        {
+            p.top = upper ? hpad / 2 : hpad - hpad / 2;
+            p.left = upper ? wpad / 2 : wpad - wpad / 2;
+        }
+    }
+    return p;
+}
+
+static inline int padded_channels(int c)
+{
+    return (c + 15) / 16 * 16;
+}
+static inline int packed_k(const ncnnhip_conv_desc& d)
+{
+    return (d.kernel_w * d.kernel_h * padded_channels(d.c) + 63) / 64 * 64;
+}
+
+struct SplitPlan
+{
+    int bm, bn, splits, steps_per_split;
+};
+
+// enough workgroups to occupy the chip: shrink the tile first, then split K
+static SplitPlan plan_launch(int cout, long long npix, int steps)
+{
+    SplitPlan p;
+    p.bm = cout <= 64 ? 64 : 128;
+    p.bn = 128;
+    long long tiles = (long long)ceil_div(cout, p.bm) * ceil_div(npix, p.bn);
+    if (tiles < 256 && npix <= 64 * 1024)
+    {
+        p.bn = 64;
+        tiles = (long long)ceil_div(cout, p.bm) * ceil_div(npix, p.bn);
+    }
+    if (tiles < 128 && p.bm == 128)
+    {
+        p.bm = 64;
+        tiles = (long long)ceil_div(cout, p.bm) * ceil_div(npix, p.bn);
+    }
+    p.splits = 1;
+    if (tiles < 192 && steps >= 8)
+    {
+        int want = (int)((384 + tiles - 1) / tiles);
+        int max_splits = steps / 4; // at least 4 K steps per split
+        p.splits = want < max_splits ? want : max_splits;
+        if (p.splits < 1) p.splits = 1;
+    }
+    p.steps_per_split = ceil_div(steps, p.splits);
+    p.splits = ceil_div(steps, p.steps_per_split);
+    return p;
+}
+
+} // namespace ncnnhip
+
+using namespace ncnnhip;
+
+extern "C" {
+
+int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes)
+{
+    NCNNHIP_REQUIRE(desc && desc->group == 1, "ncnnhip_conv_nhwc_sizes: channels-last path handles group 1 only");
+    int outw, outh;
+    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
+    if (ret) return ret;
+    const int Cp = padded_channels(desc->c);
+    if (nhwc_bytes) *nhwc_bytes = (size_t)desc->batch * desc->h * desc->w * Cp;
+    if (packed_weight_bytes) *packed_weight_bytes = (size_t)desc->num_output * packed_k(*desc);
+    if (workspace_bytes)
+    {
+        const long long npix = (long long)desc->batch * outw * outh;
+        const SplitPlan p = plan_launch(desc->num_output, npix, packed_k(*desc) / 64);
+        *workspace_bytes = p.splits > 1 ? (size_t)desc->num_output * npix * sizeof(int32_t) : 0;
+    }
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_conv_pack_weights(const ncnnhip_conv_desc* desc, const int8_t* weight_host, int8_t* packed_host)
+{
+    NCNNHIP_REQUIRE(desc && weight_host && packed_host && desc->group == 1, "ncnnhip_conv_pack_weights: bad argument");
+    const int c = desc->c, Cp = padded_channels(c), taps = desc->kernel_w * desc->kernel_h, K = packed_k(*desc);
+    for (int p = 0; p < desc->num_output; p++)
+    {
+        int8_t* row = packed_host + (size_t)p * K;
+        for (int k = 0; k < K; k++) row[k] = 0;
+        for (int q = 0; q < c; q++)
+            for (int t = 0; t < taps; t++) row[t * Cp + q] = weight_host[((size_t)p * c + q) * taps + t];
+    }
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x_elemsize, size_t x_cstep, size_t x_nstep,
+                         const float* scales_dev, int nscales, int8_t* nhwc_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && x_dev && nhwc_dev, "ncnnhip_to_nhwc_int8: null pointer");
+    NCNNHIP_REQUIRE(x_elemsize == 1 || (x_elemsize == 4 && scales_dev && (nscales == 1 || nscales == desc->c)), "ncnnhip_to_nhwc_int8: bad element size / scales");
+    NCNNHIP_REQUIRE(desc->batch <= 65535, "ncnnhip_to_nhwc_int8: batch above 65535");
+    const int hw = desc->w * desc->h, Cp = padded_channels(desc->c);
+    NCNNHIP_REQUIRE(x_cstep >= (size_t)hw, "ncnnhip_to_nhwc_int8: channel stride below plane size");
+    dim3 grid(ceil_div(hw, 256), Cp / 16, desc->batch);
+    if (x_elemsize == 4)
+        hipLaunchKernelGGL(to_nhwc_int8_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)x_dev, x_cstep, x_nstep, desc->c, hw, Cp, scales_dev, nscales, nhwc_dev);
+    else
+        hipLaunchKernelGGL(to_nhwc_int8_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)x_dev, x_cstep, x_nstep, desc->c, hw, Cp, (const float*)0, 1, nhwc_dev);
+    return launch_status("to_nhwc_int8_kernel");
+}
+
+int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, size_t out_cstep,
+                           size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_nhwc: null pointer");
+    NCNNHIP_REQUIRE(desc->group == 1, "ncnnhip_conv_int8_nhwc: group must be 1");
+    int outw, outh;
+    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
+    if (ret) return ret;
+    const ncnnhip_conv_desc& d = *desc;
+    const long long plane = (long long)outw * outh, npix = plane * d.batch;
+    NCNNHIP_REQUIRE(npix < (1ll << 31) && out_cstep >= (size_t)plane, "ncnnhip_conv_int8_nhwc: bad output extent");
+    NCNNHIP_REQUIRE((long long)d.h * d.w * padded_channels(d.c) < (1ll << 31), "ncnnhip_conv_int8_nhwc: one input sample exceeds 2 GiB");
+    const Pads4 pads = resolve_pads_nhwc(d);
+
+    NhwcGeom g;
+    g.H = d.h;
+    g.W = d.w;
+    g.Cp = padded_channels(d.c);
+    g.kw = d.kernel_w;
+    g.kh = d.kernel_h;
+    g.dw = d.dilation_w;
+    g.dh = d.dilation_h;
+    g.sw = d.stride_w;
+    g.sh = d.stride_h;
+    g.pad_top = pads.top;
+    g.pad_left = pads.left;
+    g.outw = outw;
+    g.outh = outh;
+    g.npix = (int)npix;
+    g.ntaps = d.kernel_w * d.kernel_h;
+    g.K = packed_k(d);
+    g.cout = d.num_output;
+    const int pb = (int)(signed char)d.pad_value & 0xff;
+    g.pad_word = (int)((uint32_t)pb * 0x01010101u);
+
+    ConvEpilogue epi;
+    epi.scale_in = scale_in_dev;
+    epi.bias = bias_dev;
+    epi.scale_out = scale_out_dev;
+    epi.act = act;
+    epi.out = out_dev;
+    epi.out_cstep = out_cstep;
+    epi.out_nstep = out_nstep;
+    epi.pix_per_img = (int)plane;
+    epi.batch = d.batch;
+    epi.out_channel0 = 0;
+    epi.num_output = d.num_output;
+    epi.acc_out = 0;
+
+    const SplitPlan p = plan_launch(d.num_output, npix, g.K / 64);
+    hipStream_t st = as_stream(stream);
+    dim3 grid(ceil_div(npix, p.bn), ceil_div(d.num_output, p.bm), p.splits);
+    NCNNHIP_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ncnnhip_conv_int8_nhwc: grid too large");
+    int32_t* partial = 0;
+    if (p.splits > 1)
+    {
+        const size_t need = (size_t)d.num_output * npix * sizeof(int32_t);
+        NCNNHIP_REQUIRE(workspace_dev && workspace_bytes >= need, "ncnnhip_conv_int8_nhwc: workspace of %zu bytes required", need);
+        partial = (int32_t*)workspace_dev;
+        hipLaunchKernelGGL(zero_i32_kernel, dim3(ceil_div((long long)d.num_output * npix, 256)), dim3(256), 0, st, partial, (size_t)d.num_output * npix);
+    }
+#define LAUNCH_NHWC(BM_, BN_)                                                                                                                       \
+    do                                                                                                                                               \
+    {                                                                                                                                                \
+        if (p.splits > 1)                                                                                                                            \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial); \
+        else                                                                                                                                         \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial); \
+    } while (0)
+    if (p.bm == 128 && p.bn == 128)
+        LAUNCH_NHWC(128, 128);
+    else if (p.bm == 128)
+        LAUNCH_NHWC(128, 64);
+    else if (p.bn == 128)
+        LAUNCH_NHWC(64, 128);
+    else
+        LAUNCH_NHWC(64, 64);
+#undef LAUNCH_NHWC
+    if (p.splits > 1)
+        hipLaunchKernelGGL(conv_splitk_finish_kernel, dim3(ceil_div((long long)d.num_output * npix, 256)), dim3(256), 0, st, partial, d.num_output, (int)npix, epi);
+    return launch_status("conv_nhwc_kernel");
+}
+
+} // extern "C"

@@ -59,6 +59,11 @@ _SIGNATURES = {
     "ncnnhip_fold_input_scales": [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "ncnnhip_conv_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                           Activation, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_conv_nhwc_sizes": [C.POINTER(ConvDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "ncnnhip_conv_pack_weights": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p],
+    "ncnnhip_to_nhwc_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_conv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_size_t,
+                               C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
                                   C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -195,7 +200,7 @@ class Runtime:
         return out
 
     def conv_layer(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
-                   pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), want_acc=False):
+                   pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), want_acc=False, path="auto"):
         """Whole forward_int8 of Convolution (group == 1, per-output-channel weight scales) or
         ConvolutionDepthWise (scale tables with `group` entries): x is [c][h][w] or [n][c][h][w], fp32 or int8."""
         x = np.ascontiguousarray(x)
@@ -211,6 +216,30 @@ class Runtime:
         in_scales = np.atleast_1d(np.asarray(in_scales, np.float32))
         scale_in = self.fold_input_scales(w_scales, in_scales, num_output)
         cstep, nstep = h * w, c * h * w
+        requant = term > 100
+        if path == "auto":
+            path = "nhwc" if (group == 1 and not want_acc) else "chw"
+        if path == "nhwc":
+            # channels-last fast path: quantise+transpose, packed weights, same epilogue
+            nb, wb, sb_ = C.c_size_t(), C.c_size_t(), C.c_size_t()
+            check(lib().ncnnhip_conv_nhwc_sizes(C.byref(d), C.byref(nb), C.byref(wb), C.byref(sb_)))
+            wq = np.ascontiguousarray(weight, np.int8)
+            pk = np.empty(wb.value, np.int8)
+            check(lib().ncnnhip_conv_pack_weights(C.byref(d), wq.ctypes.data, pk.ctypes.data))
+            dx = self.up(x if x.dtype == np.int8 else x.astype(np.float32))
+            dsc = self.up(in_scales)
+            dn = DeviceBuffer(nb.value)
+            check(lib().ncnnhip_to_nhwc_int8(C.byref(d), dx.ptr, x.dtype.itemsize, cstep, nstep, dsc.ptr, in_scales.size, dn.ptr, self.stream))
+            scale_out = None
+            if requant:
+                ts = np.atleast_1d(np.asarray(top_scales, np.float32))
+                scale_out = np.repeat(ts, num_output // ts.size).astype(np.float32)
+            dpk, dsi, db, dso = self.up(pk), self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32)), self.up(scale_out)
+            dws = DeviceBuffer(max(sb_.value, 4))
+            dout = DeviceBuffer.empty((n, num_output, oh, ow), np.int8 if requant else np.float32)
+            check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), dn.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
+                                               oh * ow, num_output * oh * ow, dws.ptr, sb_.value, self.stream))
+            return dout.to_numpy(self.stream)
         if x.dtype == np.int8:
             dxq = self.up(x)
         else:
@@ -218,7 +247,6 @@ class Runtime:
             dx, dsc = self.up(x.astype(np.float32)), self.up(per_channel)
             dxq = DeviceBuffer.empty(x.shape, np.int8)
             check(lib().ncnnhip_quantize(dx.ptr, cstep, nstep, dxq.ptr, cstep, nstep, c, cstep, n, dsc.ptr, per_channel.size, self.stream))
-        requant = term > 100
         scale_out = None
         if requant:
             ts = np.atleast_1d(np.asarray(top_scales, np.float32))

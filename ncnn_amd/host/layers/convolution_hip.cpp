@@ -14,7 +14,7 @@ Convolution_hip::Convolution_hip(bool depthwise_type) : is_depthwise_type(depthw
     one_blob_only = true;
     support_inplace = false;
     support_batch = true; // Mat.n is folded into the pixel dimension of the implicit GEMM
-    d_weight = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
+    d_weight = d_weight_packed = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
     input_scale_count = 0;
     group = 1;
 }
@@ -133,7 +133,33 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
                                        num_output, scale_in.data());
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_fold_input_scales");
 
-    int ret = upload_constant(weight_data.data, (size_t)weight_data_size, &d_weight);
+    int ret = 0;
+    if (group == 1)
+    {
+        // the channels-last kernel reads weights as [num_output][tap][padded channels]; repack once here
+        const int taps = kernel_w * kernel_h;
+        if (num_output <= 0 || taps <= 0 || weight_data_size % (num_output * taps) != 0) return -1;
+        ncnnhip_conv_desc desc;
+        memset(&desc, 0, sizeof(desc));
+        desc.c = weight_data_size / (num_output * taps);
+        desc.w = kernel_w; // any extent the kernel fits in: only c, num_output and the kernel size matter for packing
+        desc.h = kernel_h;
+        desc.batch = 1;
+        desc.num_output = num_output;
+        desc.kernel_w = kernel_w;
+        desc.kernel_h = kernel_h;
+        desc.dilation_w = desc.dilation_h = desc.stride_w = desc.stride_h = 1;
+        desc.group = 1;
+        size_t packed_bytes = 0;
+        rc = ncnnhip_conv_nhwc_sizes(&desc, 0, &packed_bytes, 0);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
+        std::vector<int8_t> packed(packed_bytes);
+        rc = ncnnhip_conv_pack_weights(&desc, (const int8_t*)weight_data.data, packed.data());
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_pack_weights");
+        ret = upload_constant(packed.data(), packed_bytes, &d_weight_packed);
+    }
+    else
+        ret = upload_constant(weight_data.data, (size_t)weight_data_size, &d_weight);
     if (ret == 0) ret = upload_constant(scale_in.data(), scale_in.size() * 4, &d_scale_in);
     if (ret == 0 && bias_term) ret = upload_constant(bias_data.data, (size_t)num_output * 4, &d_bias);
     if (ret == 0 && int8_scale_term > 100)
@@ -154,7 +180,7 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
 
 int Convolution_hip::destroy_pipeline(const Option& /*opt*/)
 {
-    void** all[] = {&d_weight, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
+    void** all[] = {&d_weight, &d_weight_packed, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
@@ -170,7 +196,7 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
         NCNN_LOGE("%s %s: use_int8_inference is off and there is no fp32 path in this runtime", type.c_str(), name.c_str());
         return -1;
     }
-    if (!d_weight)
+    if (!d_weight && !d_weight_packed)
     {
         NCNN_LOGE("%s %s: forward before create_pipeline", type.c_str(), name.c_str());
         return -1;
@@ -225,6 +251,27 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
     if (!d_in || !d_out) return -100;
     rc = ncnnhip_memcpy_h2d(d_in, bottom_blob.data, mat_bytes(bottom_blob), st);
     if (rc != 0) return to_ncnn_status(rc, "upload bottom blob");
+
+    if (group == 1)
+    {
+        // channels-last path: quantise (or copy) into [n][h][w][Cp] int8, then the implicit GEMM
+        size_t nhwc_bytes = 0, packed_bytes = 0, workspace_bytes = 0;
+        rc = ncnnhip_conv_nhwc_sizes(&desc, &nhwc_bytes, &packed_bytes, &workspace_bytes);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
+        void* d_nhwc = leases.get(nhwc_bytes);
+        void* d_ws = workspace_bytes ? leases.get(workspace_bytes) : 0;
+        if (!d_nhwc || (workspace_bytes && !d_ws)) return -100;
+        rc = ncnnhip_to_nhwc_int8(&desc, d_in, (int)bottom_blob.elemsize, bottom_blob.cstep, bottom_blob.nstep, (const float*)d_input_scales, 1,
+                                  (int8_t*)d_nhwc, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_to_nhwc_int8");
+        rc = ncnnhip_conv_int8_nhwc(&desc, (const int8_t*)d_nhwc, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias,
+                                    (const float*)d_scale_out, make_activation(activation_type, activation_params), d_out, top_blob.cstep,
+                                    top_blob.nstep, d_ws, workspace_bytes, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");
+        rc = ncnnhip_memcpy_d2h(top_blob.data, d_out, mat_bytes(top_blob), st);
+        if (rc == 0) rc = ncnnhip_stream_synchronize(st);
+        return to_ncnn_status(rc, "download top blob");
+    }
 
     const int8_t* d_xq = (const int8_t*)d_in;
     size_t q_cstep = bottom_blob.cstep, q_nstep = bottom_blob.nstep;

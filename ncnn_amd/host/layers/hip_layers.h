@@ -35,7 +35,8 @@ public:
 private:
     const bool is_depthwise_type;
     // device copies made at create_pipeline
-    void* d_weight;
+    void* d_weight;        // group > 1: [num_output][c/group][kh][kw] as stored in the model
+    void* d_weight_packed; // group == 1: [num_output][kh*kw][16*ceil(c/16)] for the channels-last kernel
     void* d_bias;
     void* d_scale_in;      // one per output channel: 1/(in_scale*w_scale), 0 when w_scale is 0
     void* d_scale_out;     // one per output channel, only when requantising

@@ -309,6 +309,64 @@ def to_int8_model(g, absmax):
     return mw.assemble_param(lines), blob, info
 
 
+def infer_shapes(g):
+    """blob name -> (c, h, w) or (n,) for vectors, by walking the graph"""
+    shp = {"data": tuple(g.input_shape)}
+    for L in g.layers:
+        t = L["type"]
+        if t == "Input":
+            continue
+        i0 = shp[L["bottoms"][0]]
+        if t in ("Convolution", "ConvolutionDepthWise"):
+            c, h, w = i0
+            k, s, p = L["k"], L["stride"], L["pad"]
+            shp[L["tops"][0]] = (L["cout"], (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1)
+        elif t == "InnerProduct":
+            shp[L["tops"][0]] = (L["cout"],)
+        elif t == "Pooling":
+            c, h, w = i0
+            if L["global_pool"]:
+                shp[L["tops"][0]] = (c,)
+            else:
+                k, s = L["k"], L["stride"]
+                ph, pw = (s - (h - k) % s) % s, (s - (w - k) % s) % s
+                shp[L["tops"][0]] = (c, (h + ph - k) // s + 1, (w + pw - k) // s + 1)
+        elif t == "Split":
+            for top in L["tops"]:
+                shp[top] = i0
+        else:
+            shp[L["tops"][0]] = i0
+    return shp
+
+
+def quantised_layer_table(g):
+    """One row per quantised layer: what the hot path has to compute (shapes, MACs, whether input / output are int8)."""
+    shp = infer_shapes(g)
+    cons = _consumers(g)
+    producer = {}
+    for L in g.layers:
+        for top in L["tops"]:
+            producer[top] = L
+    rows = []
+    for L in g.layers:
+        if L["type"] not in QUANTISED:
+            continue
+        bottom, top = L["bottoms"][0], L["tops"][0]
+        src = producer[bottom]
+        while src["type"] == "Split":
+            src = producer[src["bottoms"][0]]
+        int8_in = src["type"] in QUANTISED and _all_quantised_consumers(src["tops"][0], cons)
+        row = dict(name=L["name"], type=L["type"], in_shape=shp[bottom], out_shape=shp[top], int8_in=int8_in)
+        if L["type"] == "InnerProduct":
+            row.update(macs=int(np.prod(L["w"].shape)), int8_out=False, k=1, stride=1, pad=0, group=1, act=0, act_params=())
+        else:
+            cout, oh, ow = shp[top]
+            row.update(macs=int(cout * oh * ow * L["w"].shape[1] * L["k"] * L["k"]), int8_out=_all_quantised_consumers(top, cons), k=L["k"],
+                       stride=L["stride"], pad=L["pad"], group=L["group"], act=L["act"], act_params=L["act_params"])
+        rows.append(row)
+    return rows
+
+
 def build(which, seed=None, input_hw=None, n_calib=8):
     make = {"resnet50": resnet50, "mobilenetv2": mobilenetv2, "tiny": tiny_net}[which]
     kw = {}

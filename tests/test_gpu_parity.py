@@ -129,14 +129,17 @@ def test_convolution_bit_exact(rt, shape, term, act, act_params, bias, int8_in):
     got, gacc = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act, act_params, want_acc=True)
     assert np.array_equal(gacc[0], wacc)
     assert got.dtype == want.dtype and np.array_equal(got[0], want)
+    fast = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act, act_params, path="nhwc")
+    assert fast.dtype == want.dtype and np.array_equal(fast[0], want)
 
 
 def test_convolution_nonzero_pad_value(rt):
     x, wq, b, ws, ins, tops = cases.conv_case(5, 3, 6, 6, 4, (3, 3))
     d = oracle.make_desc((3, 6, 6), 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7, bias_term=1)
     want = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0])
-    got = rt.conv_layer(x[0], wq, b, ws, ins, None, 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7)
-    assert np.array_equal(got[0], want)
+    for path in ("chw", "nhwc"):
+        got = rt.conv_layer(x[0], wq, b, ws, ins, None, 4, (3, 3), pads=(1, 1, 1, 1), pad_value=3.7, path=path)
+        assert np.array_equal(got[0], want), path
 
 
 def test_convolution_zero_weight_scale(rt):
@@ -153,6 +156,9 @@ def test_convolution_zero_weight_scale(rt):
     ("resnet 1x1/2 256->512 @28 fp32 out", 256, 28, 28, 512, (1, 1), (2, 2), (0, 0, 0, 0), 2, 0),
     ("resnet 3x3 512->512 @7 requant", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 102, 1),
     ("mobilenetv2 pointwise 96->24 @56 relu6", 96, 56, 56, 24, (1, 1), (1, 1), (0, 0, 0, 0), 101, 3),
+    ("wide plane 3x3 20->130 @180 (channel count off the 16 grid, 128x128 tiles)", 20, 180, 180, 130, (3, 3), (1, 1), (1, 1, 1, 1), 101, 1),
+    ("wide plane 1x1 40->48 @190 (64x128 tiles)", 40, 190, 190, 48, (1, 1), (1, 1), (0, 0, 0, 0), 1, 0),
+    ("resnet 3x3 512->512 @7 fp32 out (K split over workgroups)", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 1, 0),
 ])
 def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pads, term, act):
     _say("conv net-shape", name)
@@ -163,6 +169,8 @@ def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pad
     got, gacc = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, (1, 1), stride, pads, 0.0, 1, term, act, (0.0, 6.0), want_acc=True)
     assert np.array_equal(gacc[0], wacc)
     assert np.array_equal(got[0], want)
+    fast = rt.conv_layer(x[0], wq, b, ws, ins, tops, outc, kernel, (1, 1), stride, pads, 0.0, 1, term, act, (0.0, 6.0), path="nhwc")
+    assert np.array_equal(fast[0], want)
     if act in (1, 3):
         assert got.min() >= 0
 
