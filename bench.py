@@ -260,7 +260,7 @@ def bench_net(args, which, batch):
             else:
                 check(lib.ncnnhip_to_nhwc_int8(C.byref(p["desc"]), p["d_x"].ptr, 4, h * w, c * h * w, p["d_s"].ptr, 1, p["d_nhwc"].ptr, st))
             check(lib.ncnnhip_conv_int8_nhwc(C.byref(p["desc"]), p["d_nhwc"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr,
-                                             p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, p["ocs"], r["out_shape"][0] * p["ocs"],
+                                             p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, 0, p["ocs"], r["out_shape"][0] * p["ocs"],
                                              p["d_ws"].ptr, p["ws_bytes"], st))
             return
         if not r["int8_in"]:

@@ -88,6 +88,8 @@ typedef struct ncnnhip_conv_desc
 
 /* Output extent after make_padding (src/layer/convolution.cpp:328-372, 412-413). */
 int ncnnhip_conv_out_shape(const ncnnhip_conv_desc* desc, int* outw, int* outh);
+/* Head pads make_padding resolves to (literal values, or the SAME_UPPER / SAME_LOWER split, :348-371). */
+int ncnnhip_conv_resolved_pads(const ncnnhip_conv_desc* desc, int* pad_top, int* pad_left);
 
 /* Host helper used at create_pipeline: expands ncnn's scale tables to one value per output
  * channel with the reference's own expression
@@ -113,15 +115,65 @@ int ncnnhip_conv_int8(const ncnnhip_conv_desc* desc, const int8_t* x_dev, size_t
  * channel) or from int8 as is -- and the weights are repacked once (host side, at create_pipeline) to
  * [num_output][kh*kw][Cp] with K padded to a multiple of 64.  Results are identical to ncnnhip_conv_int8.
  * workspace: int32 scratch for layers whose K loop is split across workgroups (size from ncnnhip_conv_nhwc_sizes,
- * may be 0); it is cleared by the call itself. */
+ * may be 0); it is cleared by the call itself.
+ * out_layout NCNNHIP_PLANAR: out is ncnn's [batch][num_output][out_cstep] (out_nstep between samples);
+ * NCNNHIP_CHANNELS_LAST: out is [batch][outh*outw][16*ceil(num_output/16)], pad channels written as zero
+ * (out_cstep / out_nstep ignored) -- the form the next layer's kernel consumes without a conversion pass. */
+#define NCNNHIP_PLANAR 0
+#define NCNNHIP_CHANNELS_LAST 1
 int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes);
 int ncnnhip_conv_pack_weights(const ncnnhip_conv_desc* desc, const int8_t* weight_host, int8_t* packed_host);
 int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x_elemsize, size_t x_cstep, size_t x_nstep,
                          const float* scales_dev, int nscales, int8_t* nhwc_dev, void* stream);
 int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev,
                            const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
-                           void* out_dev, size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes,
-                           void* stream);
+                           void* out_dev, int out_layout, size_t out_cstep, size_t out_nstep, void* workspace_dev,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ device-resident blobs (channels-last)
+ * Between layers a 3-D blob stays in HBM as [batch][h*w][Cp] (Cp = ncnnhip_padded_channels(c), fp32 or int8, pad
+ * channels zero); 1-D / 2-D blobs are dense.  ncnn's planar Mat layout (src/mat.h:341-381) exists only at the host
+ * boundary.  This plays the part of the reference's VkMat upload / download and packing conversion
+ * (src/net.cpp:2107-2230, src/layer/vulkan/packing_vulkan.cpp) for this device. */
+int ncnnhip_padded_channels(int c);
+int ncnnhip_chw_to_nhwc(const void* src_dev, int elemsize, int c, int hw, int batch, size_t cstep, size_t nstep, void* dst_dev, void* stream);
+int ncnnhip_nhwc_to_chw(const void* src_dev, int elemsize, int c, int hw, int batch, void* dst_dev, size_t cstep, size_t nstep, void* stream);
+/* Quantize::forward (src/layer/quantize.cpp:48-111) on a channels-last fp32 blob of npix pixels: one scale or one per channel. */
+int ncnnhip_quantize_nhwc(const float* src_dev, int8_t* dst_dev, size_t npix, int c, const float* scales_dev, int nscales, void* stream);
+/* The executor's int8 -> fp32 value cast for layers without int8 storage support (src/net.cpp:3007-3012 does the same at extract). */
+int ncnnhip_int8_to_f32(const int8_t* src_dev, float* dst_dev, size_t count, void* stream);
+
+/* ConvolutionDepthWise::forward_int8, depthwise branch (channels == group == num_output,
+ * src/layer/convolutiondepthwise.cpp:505-559), channels-last int8 in, channels-last int8 (scale_out != NULL) or fp32 out.
+ * Weights repacked once to [kh*kw][Cp]; scale_in / bias / scale_out one float per channel. */
+int ncnnhip_dwconv_pack_weights(int channels, int taps, const int8_t* weight_host, int8_t* packed_host);
+int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev,
+                             const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
+                             void* out_nhwc_dev, void* stream);
+
+/* ------------------------------------------------------------------ fp32 layers between the int8 layers
+ * ReLU::forward_inplace (src/layer/relu.cpp): x < 0 ? x*slope : x; int8 blobs clamp at zero.  Flat over `count` elements. */
+int ncnnhip_relu(const void* src_dev, void* dst_dev, int elemsize, size_t count, float slope, void* stream);
+/* Dropout::forward_inplace (src/layer/dropout.cpp): x * scale. */
+int ncnnhip_scale(const float* src_dev, float* dst_dev, size_t count, float scale, void* stream);
+/* Eltwise::forward (src/layer/eltwise.cpp:14-178): op_type 0 product, 1 sum (with coefficients when ncoeffs != 0), 2 max,
+ * folded left to right over nsrc inputs.  srcs_dev is a HOST array of device pointers, coeffs_host a host array. */
+int ncnnhip_eltwise(const float* const* srcs_dev, int nsrc, int op_type, const float* coeffs_host, int ncoeffs, float* dst_dev, size_t count, void* stream);
+/* Pooling::forward (src/layer/pooling.cpp:18-415) on a channels-last fp32 blob.  pad_top / pad_left are the resolved head pads,
+ * outw / outh the resolved output extent (pad_mode is the caller's business); global_pooling writes dense [batch][c]. */
+typedef struct ncnnhip_pool_desc
+{
+    int w, h, c, batch;
+    int pooling_type; /* 0 max, 1 average */
+    int kernel_w, kernel_h, stride_w, stride_h;
+    int pad_top, pad_left;
+    int outw, outh;
+    int global_pooling;
+    int avgpool_count_include_pad;
+} ncnnhip_pool_desc;
+int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, float* dst_dev, void* stream);
+/* Softmax::forward_inplace (src/layer/softmax.cpp) over a dense vector of `count` values per sample. */
+int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream);
 
 /* ------------------------------------------------------------------ InnerProduct
  * InnerProduct::forward_int8 (src/layer/innerproduct.cpp:168-273) after input quantisation:

@@ -152,6 +152,16 @@ int ncnnhip_conv_out_shape(const ncnnhip_conv_desc* desc, int* outw, int* outh)
     return NCNNHIP_OK;
 }
 
+int ncnnhip_conv_resolved_pads(const ncnnhip_conv_desc* desc, int* pad_top, int* pad_left)
+{
+    int ret = check_desc(desc, "ncnnhip_conv_resolved_pads");
+    if (ret) return ret;
+    const ResolvedPads p = resolve_pads(*desc);
+    if (pad_top) *pad_top = p.top;
+    if (pad_left) *pad_left = p.left;
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_fold_input_scales(const float* w_scales, int n_w_scales, const float* in_scales, int n_in_scales, int num_output,
                               float* scale_in_out)
 {

@@ -77,9 +77,37 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* p, size_t n)
     if (i < n) p[i] = 0;
 }
 
-template<int BM, int BN, bool SPLITK>
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// channels-last store of output channels p0..p0+3 (p0 % 4 == 0) of output pixel n: one 4-byte (int8) or 16-byte
+// (fp32) word; channels at or beyond num_output are the blob's zero padding
+__device__ __forceinline__ void store4_channels_last(const ConvEpilogue& e, int out_cp, int p0, int n, const int* acc)
+{
+    float f[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+    {
+        const int p = p0 + k;
+        float r = 0.f;
+        if (p < e.num_output)
+        {
+            r = mul_rn((float)acc[k], e.scale_in[p]);
+            if (e.bias) r = add_rn(r, e.bias[p]);
+            r = apply_activation(r, e.act);
+            if (e.scale_out) r = (float)float2int8(mul_rn(r, e.scale_out[p]));
+        }
+        f[k] = r;
+    }
+    const size_t o = (size_t)n * out_cp + p0;
+    if (e.scale_out)
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(e.out) + o) = pack4b((int)f[0], (int)f[1], (int)f[2], (int)f[3]);
+    else
+        *reinterpret_cast<v4f*>(static_cast<float*>(e.out) + o) = v4f{f[0], f[1], f[2], f[3]};
+}
+
+template<int BM, int BN, bool SPLITK, bool CLAST>
 __global__ __launch_bounds__(256) void conv_nhwc_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                         int steps_per_split, int32_t* __restrict__ partial)
+                                                         int steps_per_split, int32_t* __restrict__ partial, int out_cp)
 {
     constexpr int TM = BM / 64, TN = BN / 64;
     constexpr int ACH = BM * 4 / 256 > 0 ? BM * 4 / 256 : 1; // 16-byte chunks of the weight tile per thread
@@ -220,6 +248,33 @@ __global__ __launch_bounds__(256) void conv_nhwc_kernel(const int8_t* __restrict
         __syncthreads();
     }
 
+    if (CLAST)
+    {
+        // accumulator registers 4*rg..4*rg+3 of a lane are four consecutive output channels of one pixel
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+            for (int b = 0; b < TN; b++)
+#pragma unroll
+                for (int rg = 0; rg < 4; rg++)
+                {
+                    const int p0 = row0 + wm * (BM / 2) + a * 32 + 8 * rg + 4 * lhi;
+                    const int gj = col0 + wn * (BN / 2) + b * 32 + l32;
+                    if (p0 < out_cp && gj < g.npix)
+                    {
+                        const int v[4] = {acc[a][b][rg * 4], acc[a][b][rg * 4 + 1], acc[a][b][rg * 4 + 2], acc[a][b][rg * 4 + 3]};
+                        if (SPLITK)
+                        {
+#pragma unroll
+                            for (int k = 0; k < 4; k++)
+                                if (p0 + k < g.cout) atomicAdd(partial + (size_t)gj * out_cp + p0 + k, v[k]);
+                        }
+                        else
+                            store4_channels_last(epi, out_cp, p0, gj, v);
+                    }
+                }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -237,6 +292,19 @@ __global__ __launch_bounds__(256) void conv_nhwc_kernel(const int8_t* __restrict
                         epi(gi, gj, acc[a][b][r]);
                 }
             }
+}
+
+// partial sums laid out [npix][out_cp]: one thread finishes four channels of one pixel
+__global__ __launch_bounds__(256) void conv_splitk_finish_clast_kernel(const int32_t* __restrict__ partial, int npix, int out_cp, ConvEpilogue epi)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int groups = out_cp / 4;
+    if (i >= (size_t)npix * groups) return;
+    const int n = (int)(i / groups);
+    const int p0 = (int)(i - (size_t)n * groups) * 4;
+    const v4i v = *reinterpret_cast<const v4i*>(partial + (size_t)n * out_cp + p0);
+    const int a[4] = {v[0], v[1], v[2], v[3]};
+    store4_channels_last(epi, out_cp, p0, n, a);
 }
 
 __global__ __launch_bounds__(256) void conv_splitk_finish_kernel(const int32_t* __restrict__ partial, int cout, int npix, ConvEpilogue epi)
@@ -343,7 +411,7 @@ int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, s
     {
         const long long npix = (long long)desc->batch * outw * outh;
         const SplitPlan p = plan_launch(desc->num_output, npix, packed_k(*desc) / 64);
-        *workspace_bytes = p.splits > 1 ? (size_t)desc->num_output * npix * sizeof(int32_t) : 0;
+        *workspace_bytes = p.splits > 1 ? (size_t)padded_channels(desc->num_output) * npix * sizeof(int32_t) : 0;
     }
     return NCNNHIP_OK;
 }
@@ -379,8 +447,8 @@ int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x
 }
 
 int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
-                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, size_t out_cstep,
-                           size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
+                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
+                           size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
 {
     NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_nhwc: null pointer");
     NCNNHIP_REQUIRE(desc->group == 1, "ncnnhip_conv_int8_nhwc: group must be 1");
@@ -389,7 +457,10 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
     if (ret) return ret;
     const ncnnhip_conv_desc& d = *desc;
     const long long plane = (long long)outw * outh, npix = plane * d.batch;
-    NCNNHIP_REQUIRE(npix < (1ll << 31) && out_cstep >= (size_t)plane, "ncnnhip_conv_int8_nhwc: bad output extent");
+    NCNNHIP_REQUIRE(out_layout == NCNNHIP_PLANAR || out_layout == NCNNHIP_CHANNELS_LAST, "ncnnhip_conv_int8_nhwc: unknown output layout %d", out_layout);
+    const bool clast = out_layout == NCNNHIP_CHANNELS_LAST;
+    const int out_cp = padded_channels(desc->num_output);
+    NCNNHIP_REQUIRE(npix < (1ll << 31) && (clast || out_cstep >= (size_t)plane), "ncnnhip_conv_int8_nhwc: bad output extent");
     NCNNHIP_REQUIRE((long long)d.h * d.w * padded_channels(d.c) < (1ll << 31), "ncnnhip_conv_int8_nhwc: one input sample exceeds 2 GiB");
     const Pads4 pads = resolve_pads_nhwc(d);
 
@@ -435,18 +506,22 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
     int32_t* partial = 0;
     if (p.splits > 1)
     {
-        const size_t need = (size_t)d.num_output * npix * sizeof(int32_t);
-        NCNNHIP_REQUIRE(workspace_dev && workspace_bytes >= need, "ncnnhip_conv_int8_nhwc: workspace of %zu bytes required", need);
+        const size_t words = (size_t)out_cp * npix;
+        NCNNHIP_REQUIRE(workspace_dev && workspace_bytes >= words * sizeof(int32_t), "ncnnhip_conv_int8_nhwc: workspace of %zu bytes required", words * sizeof(int32_t));
         partial = (int32_t*)workspace_dev;
-        hipLaunchKernelGGL(zero_i32_kernel, dim3(ceil_div((long long)d.num_output * npix, 256)), dim3(256), 0, st, partial, (size_t)d.num_output * npix);
+        hipLaunchKernelGGL(zero_i32_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, st, partial, words);
     }
 #define LAUNCH_NHWC(BM_, BN_)                                                                                                                       \
     do                                                                                                                                               \
     {                                                                                                                                                \
-        if (p.splits > 1)                                                                                                                            \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial); \
+        if (p.splits > 1 && clast)                                                                                                                   \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+        else if (p.splits > 1)                                                                                                                       \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+        else if (clast)                                                                                                                              \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
         else                                                                                                                                         \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial); \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
     } while (0)
     if (p.bm == 128 && p.bn == 128)
         LAUNCH_NHWC(128, 128);
@@ -457,7 +532,9 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
     else
         LAUNCH_NHWC(64, 64);
 #undef LAUNCH_NHWC
-    if (p.splits > 1)
+    if (p.splits > 1 && clast)
+        hipLaunchKernelGGL(conv_splitk_finish_clast_kernel, dim3(ceil_div((long long)(out_cp / 4) * npix, 256)), dim3(256), 0, st, partial, (int)npix, out_cp, epi);
+    else if (p.splits > 1)
         hipLaunchKernelGGL(conv_splitk_finish_kernel, dim3(ceil_div((long long)d.num_output * npix, 256)), dim3(256), 0, st, partial, d.num_output, (int)npix, epi);
     return launch_status("conv_nhwc_kernel");
 }

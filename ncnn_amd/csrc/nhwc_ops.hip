@@ -1,0 +1,531 @@
+// Device-resident blobs and the small fp32 layers that sit between the int8 layers.
+//
+// While a net runs, a 3-D blob lives in HBM channels-last: [n][h*w][cp] with cp = 16*ceil(c/16), fp32 or int8,
+// pad channels zero.  That is the K-contiguous operand the convolution kernels want, every elementwise or
+// window kernel is coalesced along channels, and one pixel's channels of an int8 blob are whole 16-byte words.
+// 1-D and 2-D blobs are dense [n][h][w].  ncnn's planar layout ([c][cstep] planes) exists only at the host
+// boundary: chw_to_nhwc after the upload, nhwc_to_chw before the download (and for Flatten, whose output order
+// is the planar one).
+//
+// Each kernel follows the reference's scalar statement order for its element (window sums run ky-major, kx-minor;
+// the global average sums pixels in index order), so fp32 results equal the host loops' bit for bit; Softmax
+// alone reduces in parallel and uses the device expf.
+#include <float.h>
+
+#include "common.h"
+
+namespace ncnnhip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// ---- planar <-> channels-last.  One workgroup: 64 pixels x 64 channels; a wavefront reads 64 consecutive
+// pixels of one plane and each lane writes 16 consecutive channels of its pixel.
+template<typename T>
+__global__ __launch_bounds__(256) void chw_to_nhwc_kernel(const T* __restrict__ src, size_t cstep, size_t nstep, int c, int hw, int cp, T* __restrict__ dst)
+{
+    const int pix = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int q0 = blockIdx.y * 64 + (threadIdx.x >> 6) * 16;
+    const int img = blockIdx.z;
+    if (pix >= hw || q0 >= cp) return;
+    const T* sp = src + (size_t)img * nstep + pix;
+    __attribute__((aligned(16))) T v[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) v[e] = (q0 + e < c) ? sp[(size_t)(q0 + e) * cstep] : (T)0;
+    T* dp = dst + ((size_t)img * hw + pix) * cp + q0;
+#pragma unroll
+    for (int e = 0; e < 16; e += 16 / sizeof(T))
+        *reinterpret_cast<v4i*>(dp + e) = *reinterpret_cast<const v4i*>(v + e);
+}
+
+template<typename T>
+__global__ __launch_bounds__(256) void nhwc_to_chw_kernel(const T* __restrict__ src, int c, int hw, int cp, T* __restrict__ dst, size_t cstep, size_t nstep)
+{
+    const int pix = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int q0 = blockIdx.y * 64 + (threadIdx.x >> 6) * 16;
+    const int img = blockIdx.z;
+    if (pix >= hw || q0 >= cp) return;
+    const T* sp = src + ((size_t)img * hw + pix) * cp + q0;
+    __attribute__((aligned(16))) T v[16];
+#pragma unroll
+    for (int e = 0; e < 16; e += 16 / sizeof(T))
+        *reinterpret_cast<v4i*>(v + e) = *reinterpret_cast<const v4i*>(sp + e);
+    T* dp = dst + (size_t)img * nstep + pix;
+#pragma unroll
+    for (int e = 0; e < 16; e++)
+        if (q0 + e < c) dp[(size_t)(q0 + e) * cstep] = v[e];
+}
+
+// ---- Quantize on a channels-last blob: 16 channels of one pixel per thread (64 bytes in, 16 out)
+__global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float* __restrict__ src, int8_t* __restrict__ dst, size_t chunks, int c, int cp,
+                                                             const float* __restrict__ scales, int nscales)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= chunks) return;
+    const int q0 = (int)(i % (size_t)(cp / 16)) * 16;
+    const float* sp = src + i * 16;
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; w++)
+    {
+        const v4f x = *reinterpret_cast<const v4f*>(sp + w * 4);
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            const int q = q0 + w * 4 + e;
+            int v = 0;
+            if (q < c) v = float2int8(mul_rn(x[e], nscales == 1 ? scales[0] : scales[q]));
+            word |= (uint32_t)(v & 0xff) << (8 * e);
+        }
+        out[w] = (int)word;
+    }
+    *reinterpret_cast<v4i*>(dst + i * 16) = out;
+}
+
+// ---- flat elementwise kernels (they run over pad channels too: zeros stay zeros)
+__global__ __launch_bounds__(256) void int8_to_f32_kernel(const int8_t* __restrict__ src, float* __restrict__ dst, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = (float)src[i];
+}
+
+__global__ __launch_bounds__(256) void relu_f32_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n4, float slope)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    v4f v = reinterpret_cast<const v4f*>(src)[i];
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        if (v[e] < 0.f) v[e] = slope == 0.f ? 0.f : mul_rn(v[e], slope);
+    reinterpret_cast<v4f*>(dst)[i] = v;
+}
+
+__global__ __launch_bounds__(256) void relu_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i] < 0 ? (int8_t)0 : src[i];
+}
+
+__global__ __launch_bounds__(256) void scale_f32_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n, float scale)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = mul_rn(src[i], scale);
+}
+
+// Eltwise (src/layer/eltwise.cpp:14-178): op 0 product, 1 sum (optionally with coefficients), 2 max.
+// first = 1: dst = a (op) b with the coefficients of the first two inputs; first = 0: dst = dst (op) b.
+__global__ __launch_bounds__(256) void eltwise_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ dst, size_t n4, int op,
+                                                       int weighted, float ca, float cb, int first)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const v4f x = reinterpret_cast<const v4f*>(a)[i];
+    const v4f y = reinterpret_cast<const v4f*>(b)[i];
+    v4f o;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+    {
+        if (op == 0)
+            o[e] = mul_rn(x[e], y[e]);
+        else if (op == 2)
+            o[e] = fmaxf(x[e], y[e]);
+        else if (weighted)
+            o[e] = add_rn(first ? mul_rn(x[e], ca) : x[e], mul_rn(y[e], cb));
+        else
+            o[e] = add_rn(x[e], y[e]);
+    }
+    reinterpret_cast<v4f*>(dst)[i] = o;
+}
+
+// ---- Pooling (src/layer/pooling.cpp:18-415) on a channels-last fp32 blob: 4 channels of one output pixel per thread
+struct PoolGeom
+{
+    int w, h, cp, outw, outh;
+    int kw, kh, sw, sh, pad_top, pad_left;
+    int type;              // 0 max, 1 average
+    int count_include_pad; // average only
+};
+
+__global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, PoolGeom g, size_t total)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int groups = g.cp / 4;
+    const int q4 = (int)(i % (size_t)groups);
+    size_t rest = i / (size_t)groups;
+    const int ox = (int)(rest % (size_t)g.outw);
+    rest /= (size_t)g.outw;
+    const int oy = (int)(rest % (size_t)g.outh);
+    const int img = (int)(rest / (size_t)g.outh);
+    const float* base = src + (size_t)img * g.h * g.w * g.cp + q4 * 4;
+    const int y0 = oy * g.sh - g.pad_top, x0 = ox * g.sw - g.pad_left;
+    v4f r;
+    if (g.type == 0)
+    {
+        r = v4f{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+        for (int ky = 0; ky < g.kh; ky++)
+            for (int kx = 0; kx < g.kw; kx++)
+            {
+                const int y = y0 + ky, x = x0 + kx;
+                if ((unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w)
+                {
+                    const v4f v = *reinterpret_cast<const v4f*>(base + ((size_t)y * g.w + x) * g.cp);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = fmaxf(r[e], v[e]);
+                }
+            }
+    }
+    else
+    {
+        r = v4f{0.f, 0.f, 0.f, 0.f};
+        int area = 0;
+        for (int ky = 0; ky < g.kh; ky++)
+            for (int kx = 0; kx < g.kw; kx++)
+            {
+                const int y = y0 + ky, x = x0 + kx;
+                if ((unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w)
+                {
+                    const v4f v = *reinterpret_cast<const v4f*>(base + ((size_t)y * g.w + x) * g.cp);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = add_rn(r[e], v[e]);
+                    area++;
+                }
+                else if (g.count_include_pad)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = add_rn(r[e], 0.f);
+                }
+            }
+        const float div = g.count_include_pad ? (float)(g.kw * g.kh) : (float)area;
+#pragma unroll
+        for (int e = 0; e < 4; e++) r[e] = div_rn(r[e], div);
+    }
+    *reinterpret_cast<v4f*>(dst + (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q4 * 4) = r;
+}
+
+// global pooling: [n][hw][cp] -> dense [n][c]; one thread per (sample, channel) walks the pixels in index order
+__global__ __launch_bounds__(256) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    const int img = blockIdx.y;
+    if (q >= c) return;
+    const float* p = src + (size_t)img * hw * cp + q;
+    float r;
+    if (type == 0)
+    {
+        r = p[0];
+        for (int i = 0; i < hw; i++) r = fmaxf(r, p[(size_t)i * cp]);
+    }
+    else
+    {
+        r = 0.f;
+        for (int i = 0; i < hw; i++) r = add_rn(r, p[(size_t)i * cp]);
+        r = div_rn(r, (float)hw);
+    }
+    dst[(size_t)img * c + q] = r;
+}
+
+// ---- Softmax over a dense vector (src/layer/softmax.cpp), one workgroup per sample
+__global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ src, float* __restrict__ dst, int count)
+{
+    __shared__ float red[256];
+    const float* p = src + (size_t)blockIdx.x * count;
+    float* o = dst + (size_t)blockIdx.x * count;
+    float m = -FLT_MAX;
+    for (int i = threadIdx.x; i < count; i += 256) m = fmaxf(m, p[i]);
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1)
+    {
+        if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    m = red[0];
+    __syncthreads();
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < count; i += 256)
+    {
+        const float e = expf(p[i] - m);
+        o[i] = e;
+        sum += e;
+    }
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1)
+    {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    sum = red[0];
+    for (int i = threadIdx.x; i < count; i += 256) o[i] = div_rn(o[i], sum);
+}
+
+// ---- depthwise int8 convolution on channels-last blobs (ConvolutionDepthWise::forward_int8, channels == group
+// == num_output, src/layer/convolutiondepthwise.cpp:505-559).  One thread: 16 channels of one output pixel;
+// weights repacked to [tap][cp].  Memory bound: one 16-byte load per tap, neighbours served by the caches.
+struct DwNhwcGeom
+{
+    int w, h, cp, c, outw, outh;
+    int kw, kh, dw, dh, sw, sh, pad_top, pad_left;
+    int pad_byte;
+    int out_f32;
+};
+
+__global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk, DwNhwcGeom g,
+                                                           const float* __restrict__ scale_in, const float* __restrict__ bias,
+                                                           const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out, size_t total)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int chunks = g.cp / 16;
+    const int q0 = (int)(i % (size_t)chunks) * 16;
+    size_t rest = i / (size_t)chunks;
+    const int ox = (int)(rest % (size_t)g.outw);
+    rest /= (size_t)g.outw;
+    const int oy = (int)(rest % (size_t)g.outh);
+    const int img = (int)(rest / (size_t)g.outh);
+    const int8_t* base = x + (size_t)img * g.h * g.w * g.cp + q0;
+    const int y0 = oy * g.sh - g.pad_top, x0 = ox * g.sw - g.pad_left;
+    const int padw = (int)((uint32_t)(g.pad_byte & 0xff) * 0x01010101u);
+
+    int acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0;
+    for (int ky = 0; ky < g.kh; ky++)
+        for (int kx = 0; kx < g.kw; kx++)
+        {
+            const int y = y0 + ky * g.dh, xx = x0 + kx * g.dw;
+            v4i v = {padw, padw, padw, padw};
+            if ((unsigned)y < (unsigned)g.h && (unsigned)xx < (unsigned)g.w) v = *reinterpret_cast<const v4i*>(base + ((size_t)y * g.w + xx) * g.cp);
+            const v4i wv = *reinterpret_cast<const v4i*>(wpk + (size_t)(ky * g.kw + kx) * g.cp + q0);
+#pragma unroll
+            for (int wd = 0; wd < 4; wd++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[wd * 4 + e] += (int)(int8_t)(v[wd] >> (8 * e)) * (int)(int8_t)(wv[wd] >> (8 * e));
+        }
+
+    const size_t o = (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q0;
+    float f[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++)
+    {
+        const int q = q0 + e;
+        float r = 0.f;
+        if (q < g.c)
+        {
+            r = mul_rn((float)acc[e], scale_in[q]);
+            if (bias) r = add_rn(r, bias[q]);
+            r = apply_activation(r, act);
+            if (!g.out_f32) r = (float)float2int8(mul_rn(r, scale_out[q]));
+        }
+        f[e] = r;
+    }
+    if (g.out_f32)
+    {
+#pragma unroll
+        for (int wd = 0; wd < 4; wd++) *reinterpret_cast<v4f*>(static_cast<float*>(out) + o + wd * 4) = v4f{f[wd * 4], f[wd * 4 + 1], f[wd * 4 + 2], f[wd * 4 + 3]};
+    }
+    else
+    {
+        v4i pk;
+#pragma unroll
+        for (int wd = 0; wd < 4; wd++)
+        {
+            uint32_t word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) word |= (uint32_t)((int)f[wd * 4 + e] & 0xff) << (8 * e);
+            pk[wd] = (int)word;
+        }
+        *reinterpret_cast<v4i*>(static_cast<int8_t*>(out) + o) = pk;
+    }
+}
+
+static inline int padded16(int c)
+{
+    return (c + 15) / 16 * 16;
+}
+
+} // namespace ncnnhip
+
+using namespace ncnnhip;
+
+extern "C" {
+
+int ncnnhip_padded_channels(int c)
+{
+    return padded16(c);
+}
+
+int ncnnhip_chw_to_nhwc(const void* src_dev, int elemsize, int c, int hw, int batch, size_t cstep, size_t nstep, void* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && (elemsize == 1 || elemsize == 4), "ncnnhip_chw_to_nhwc: bad argument");
+    NCNNHIP_REQUIRE(c > 0 && hw > 0 && batch > 0 && batch <= 65535 && cstep >= (size_t)hw, "ncnnhip_chw_to_nhwc: bad shape");
+    const int cp = padded16(c);
+    dim3 grid(ceil_div(hw, 64), ceil_div(cp, 64), batch);
+    NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_chw_to_nhwc: too many channels");
+    if (elemsize == 4)
+        hipLaunchKernelGGL(chw_to_nhwc_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)src_dev, cstep, nstep, c, hw, cp, (float*)dst_dev);
+    else
+        hipLaunchKernelGGL(chw_to_nhwc_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)src_dev, cstep, nstep, c, hw, cp, (int8_t*)dst_dev);
+    return launch_status("chw_to_nhwc_kernel");
+}
+
+int ncnnhip_nhwc_to_chw(const void* src_dev, int elemsize, int c, int hw, int batch, void* dst_dev, size_t cstep, size_t nstep, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && (elemsize == 1 || elemsize == 4), "ncnnhip_nhwc_to_chw: bad argument");
+    NCNNHIP_REQUIRE(c > 0 && hw > 0 && batch > 0 && batch <= 65535 && cstep >= (size_t)hw, "ncnnhip_nhwc_to_chw: bad shape");
+    const int cp = padded16(c);
+    dim3 grid(ceil_div(hw, 64), ceil_div(cp, 64), batch);
+    NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_nhwc_to_chw: too many channels");
+    if (elemsize == 4)
+        hipLaunchKernelGGL(nhwc_to_chw_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)src_dev, c, hw, cp, (float*)dst_dev, cstep, nstep);
+    else
+        hipLaunchKernelGGL(nhwc_to_chw_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)src_dev, c, hw, cp, (int8_t*)dst_dev, cstep, nstep);
+    return launch_status("nhwc_to_chw_kernel");
+}
+
+int ncnnhip_quantize_nhwc(const float* src_dev, int8_t* dst_dev, size_t npix, int c, const float* scales_dev, int nscales, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && scales_dev && c > 0 && (nscales == 1 || nscales == c), "ncnnhip_quantize_nhwc: bad argument");
+    if (npix == 0) return NCNNHIP_OK;
+    const int cp = padded16(c);
+    const size_t chunks = npix * (size_t)(cp / 16);
+    hipLaunchKernelGGL(quantize_nhwc_kernel, dim3(ceil_div((long long)chunks, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, chunks, c, cp, scales_dev, nscales);
+    return launch_status("quantize_nhwc_kernel");
+}
+
+int ncnnhip_int8_to_f32(const int8_t* src_dev, float* dst_dev, size_t count, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev, "ncnnhip_int8_to_f32: null pointer");
+    if (count == 0) return NCNNHIP_OK;
+    hipLaunchKernelGGL(int8_to_f32_kernel, dim3(ceil_div((long long)count, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, count);
+    return launch_status("int8_to_f32_kernel");
+}
+
+int ncnnhip_relu(const void* src_dev, void* dst_dev, int elemsize, size_t count, float slope, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && (elemsize == 1 || elemsize == 4), "ncnnhip_relu: bad argument");
+    if (count == 0) return NCNNHIP_OK;
+    if (elemsize == 1)
+    {
+        hipLaunchKernelGGL(relu_s8_kernel, dim3(ceil_div((long long)count, 256)), dim3(256), 0, as_stream(stream), (const int8_t*)src_dev, (int8_t*)dst_dev, count);
+        return launch_status("relu_s8_kernel");
+    }
+    NCNNHIP_REQUIRE(count % 4 == 0, "ncnnhip_relu: fp32 element count must be a multiple of 4 (device blobs are padded to it)");
+    hipLaunchKernelGGL(relu_f32_kernel, dim3(ceil_div((long long)(count / 4), 256)), dim3(256), 0, as_stream(stream), (const float*)src_dev, (float*)dst_dev, count / 4, slope);
+    return launch_status("relu_f32_kernel");
+}
+
+int ncnnhip_scale(const float* src_dev, float* dst_dev, size_t count, float scale, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev, "ncnnhip_scale: null pointer");
+    if (count == 0) return NCNNHIP_OK;
+    hipLaunchKernelGGL(scale_f32_kernel, dim3(ceil_div((long long)count, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, count, scale);
+    return launch_status("scale_f32_kernel");
+}
+
+int ncnnhip_eltwise(const float* const* srcs_dev, int nsrc, int op_type, const float* coeffs_host, int ncoeffs, float* dst_dev, size_t count, void* stream)
+{
+    NCNNHIP_REQUIRE(srcs_dev && dst_dev && nsrc >= 2 && op_type >= 0 && op_type <= 2, "ncnnhip_eltwise: bad argument");
+    NCNNHIP_REQUIRE(count % 4 == 0, "ncnnhip_eltwise: element count must be a multiple of 4 (device blobs are padded to it)");
+    const int weighted = op_type == 1 && ncoeffs != 0;
+    NCNNHIP_REQUIRE(!weighted || (coeffs_host && ncoeffs >= nsrc), "ncnnhip_eltwise: one coefficient per input required");
+    if (count == 0) return NCNNHIP_OK;
+    const size_t n4 = count / 4;
+    dim3 grid(ceil_div((long long)n4, 256));
+    hipLaunchKernelGGL(eltwise_kernel, grid, dim3(256), 0, as_stream(stream), srcs_dev[0], srcs_dev[1], dst_dev, n4, op_type, weighted,
+                       weighted ? coeffs_host[0] : 1.f, weighted ? coeffs_host[1] : 1.f, 1);
+    for (int b = 2; b < nsrc; b++)
+        hipLaunchKernelGGL(eltwise_kernel, grid, dim3(256), 0, as_stream(stream), (const float*)dst_dev, srcs_dev[b], dst_dev, n4, op_type, weighted, 1.f,
+                           weighted ? coeffs_host[b] : 1.f, 0);
+    return launch_status("eltwise_kernel");
+}
+
+int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, float* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && src_dev && dst_dev, "ncnnhip_pooling_nhwc: null pointer");
+    const ncnnhip_pool_desc& d = *desc;
+    NCNNHIP_REQUIRE(d.w > 0 && d.h > 0 && d.c > 0 && d.batch > 0 && (d.pooling_type == 0 || d.pooling_type == 1), "ncnnhip_pooling_nhwc: bad shape or type");
+    const int cp = padded16(d.c);
+    if (d.global_pooling)
+    {
+        NCNNHIP_REQUIRE(d.batch <= 65535, "ncnnhip_pooling_nhwc: batch above 65535");
+        hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 256), d.batch), dim3(256), 0, as_stream(stream), src_dev, dst_dev, d.c, d.w * d.h, cp, d.pooling_type);
+        return launch_status("global_pooling_nhwc_kernel");
+    }
+    NCNNHIP_REQUIRE(d.kernel_w > 0 && d.kernel_h > 0 && d.stride_w > 0 && d.stride_h > 0 && d.outw > 0 && d.outh > 0, "ncnnhip_pooling_nhwc: bad window");
+    // every window must start inside the padded image the reference would build
+    NCNNHIP_REQUIRE(d.pad_top >= 0 && d.pad_left >= 0, "ncnnhip_pooling_nhwc: negative pads");
+    PoolGeom g;
+    g.w = d.w;
+    g.h = d.h;
+    g.cp = cp;
+    g.outw = d.outw;
+    g.outh = d.outh;
+    g.kw = d.kernel_w;
+    g.kh = d.kernel_h;
+    g.sw = d.stride_w;
+    g.sh = d.stride_h;
+    g.pad_top = d.pad_top;
+    g.pad_left = d.pad_left;
+    g.type = d.pooling_type;
+    g.count_include_pad = d.avgpool_count_include_pad;
+    const size_t total = (size_t)d.batch * d.outh * d.outw * (cp / 4);
+    hipLaunchKernelGGL(pooling_nhwc_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
+    return launch_status("pooling_nhwc_kernel");
+}
+
+int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && count > 0 && batch > 0, "ncnnhip_softmax: bad argument");
+    hipLaunchKernelGGL(softmax_kernel, dim3(batch), dim3(256), 0, as_stream(stream), src_dev, dst_dev, count);
+    return launch_status("softmax_kernel");
+}
+
+int ncnnhip_dwconv_pack_weights(int channels, int taps, const int8_t* weight_host, int8_t* packed_host)
+{
+    NCNNHIP_REQUIRE(channels > 0 && taps > 0 && weight_host && packed_host, "ncnnhip_dwconv_pack_weights: bad argument");
+    const int cp = padded16(channels);
+    for (int t = 0; t < taps; t++)
+        for (int q = 0; q < cp; q++) packed_host[(size_t)t * cp + q] = q < channels ? weight_host[(size_t)q * taps + t] : (int8_t)0;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                             const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_nhwc_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_nhwc_dev, "ncnnhip_dwconv_int8_nhwc: null pointer");
+    const ncnnhip_conv_desc& d = *desc;
+    NCNNHIP_REQUIRE(d.group == d.c && d.num_output == d.c, "ncnnhip_dwconv_int8_nhwc: needs channels == group == num_output");
+    int outw, outh;
+    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
+    if (ret) return ret;
+    int pad_top, pad_left;
+    ret = ncnnhip_conv_resolved_pads(desc, &pad_top, &pad_left);
+    if (ret) return ret;
+    DwNhwcGeom g;
+    g.w = d.w;
+    g.h = d.h;
+    g.c = d.c;
+    g.cp = padded16(d.c);
+    g.outw = outw;
+    g.outh = outh;
+    g.kw = d.kernel_w;
+    g.kh = d.kernel_h;
+    g.dw = d.dilation_w;
+    g.dh = d.dilation_h;
+    g.sw = d.stride_w;
+    g.sh = d.stride_h;
+    g.pad_top = pad_top;
+    g.pad_left = pad_left;
+    g.pad_byte = (int)(signed char)d.pad_value;
+    g.out_f32 = scale_out_dev ? 0 : 1;
+    const size_t total = (size_t)d.batch * outh * outw * (g.cp / 16);
+    hipLaunchKernelGGL(dwconv_nhwc_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), nhwc_dev, packed_weight_dev, g, scale_in_dev,
+                       bias_dev, scale_out_dev, act, out_nhwc_dev, total);
+    return launch_status("dwconv_nhwc_kernel");
+}
+
+} // extern "C"

@@ -31,6 +31,11 @@ class ConvDesc(C.Structure):
                [("pad_value", C.c_float), ("group", C.c_int)]
 
 
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("w", "h", "c", "batch", "pooling_type", "kernel_w", "kernel_h", "stride_w", "stride_h", "pad_top", "pad_left",
+                                       "outw", "outh", "global_pooling", "avgpool_count_include_pad")]
+
+
 def library_path():
     return _LIB
 
@@ -62,8 +67,21 @@ _SIGNATURES = {
     "ncnnhip_conv_nhwc_sizes": [C.POINTER(ConvDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "ncnnhip_conv_pack_weights": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p],
     "ncnnhip_to_nhwc_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p],
-    "ncnnhip_conv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_size_t,
-                               C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_conv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_int,
+                               C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_conv_resolved_pads": [C.POINTER(ConvDesc), C.POINTER(C.c_int), C.POINTER(C.c_int)],
+    "ncnnhip_padded_channels": [C.c_int],
+    "ncnnhip_chw_to_nhwc": [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_nhwc_to_chw": [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p],
+    "ncnnhip_quantize_nhwc": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_void_p],
+    "ncnnhip_int8_to_f32": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_dwconv_pack_weights": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_dwconv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_void_p],
+    "ncnnhip_relu": [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p],
+    "ncnnhip_scale": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_void_p],
+    "ncnnhip_eltwise": [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.POINTER(C.c_float), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_pooling_nhwc": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_softmax": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
                                   C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -238,7 +256,7 @@ class Runtime:
             dws = DeviceBuffer(max(sb_.value, 4))
             dout = DeviceBuffer.empty((n, num_output, oh, ow), np.int8 if requant else np.float32)
             check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), dn.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
-                                               oh * ow, num_output * oh * ow, dws.ptr, sb_.value, self.stream))
+                                               0, oh * ow, num_output * oh * ow, dws.ptr, sb_.value, self.stream))
             return dout.to_numpy(self.stream)
         if x.dtype == np.int8:
             dxq = self.up(x)
@@ -260,6 +278,118 @@ class Runtime:
         if want_acc:
             return out, dacc.to_numpy(self.stream)
         return out
+
+    # -- device-resident (channels-last) blobs and the fp32 layers between the int8 layers -----
+    def to_channels_last(self, x):
+        """[n][c][h][w] (or [c][h][w]) fp32 / int8 numpy -> device [n][h*w][Cp] buffer."""
+        x = np.ascontiguousarray(x)
+        if x.ndim == 3:
+            x = x[None]
+        n, c, h, w = x.shape
+        cp = lib().ncnnhip_padded_channels(c)
+        dx = self.up(x)
+        out = DeviceBuffer.empty((n, h * w, cp), x.dtype)
+        check(lib().ncnnhip_chw_to_nhwc(dx.ptr, x.dtype.itemsize, c, h * w, n, h * w, c * h * w, out.ptr, self.stream))
+        return out
+
+    def from_channels_last(self, buf, n, c, h, w):
+        out = DeviceBuffer.empty((n, c, h, w), buf.dtype)
+        check(lib().ncnnhip_nhwc_to_chw(buf.ptr, buf.dtype.itemsize, c, h * w, n, out.ptr, h * w, c * h * w, self.stream))
+        return out.to_numpy(self.stream)
+
+    def quantize_channels_last(self, buf, c, scales):
+        n, hw, cp = buf.shape
+        ds = self.up(np.atleast_1d(np.asarray(scales, np.float32)))
+        out = DeviceBuffer.empty((n, hw, cp), np.int8)
+        check(lib().ncnnhip_quantize_nhwc(buf.ptr, out.ptr, n * hw, c, ds.ptr, ds.shape[0], self.stream))
+        return out
+
+    def relu(self, x, slope=0.0):
+        x = np.ascontiguousarray(x)
+        dx = self.up(x)
+        out = DeviceBuffer.empty(x.shape, x.dtype)
+        check(lib().ncnnhip_relu(dx.ptr, out.ptr, x.dtype.itemsize, x.size, float(slope), self.stream))
+        return out.to_numpy(self.stream)
+
+    def eltwise(self, xs, op_type=1, coeffs=None):
+        xs = [np.ascontiguousarray(x, np.float32) for x in xs]
+        bufs = [self.up(x) for x in xs]
+        ptrs = (C.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+        co = None if coeffs is None else (C.c_float * len(coeffs))(*[float(v) for v in coeffs])
+        out = DeviceBuffer.empty(xs[0].shape, np.float32)
+        check(lib().ncnnhip_eltwise(ptrs, len(bufs), int(op_type), co, 0 if coeffs is None else len(coeffs), out.ptr, xs[0].size, self.stream))
+        return out.to_numpy(self.stream)
+
+    def pooling(self, x, pooling_type, kernel, stride, pad_top_left, out_hw, global_pooling=False, count_include_pad=0):
+        """x [n][c][h][w] fp32; the border is given resolved (head pads and output extent)."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, c, h, w = x.shape
+        src = self.to_channels_last(x)
+        if global_pooling:
+            d = PoolDesc(w, h, c, n, pooling_type, 0, 0, 1, 1, 0, 0, 1, 1, 1, 0)
+            out = DeviceBuffer.empty((n, c), np.float32)
+            check(lib().ncnnhip_pooling_nhwc(C.byref(d), src.ptr, out.ptr, self.stream))
+            return out.to_numpy(self.stream)
+        oh, ow = out_hw
+        d = PoolDesc(w, h, c, n, pooling_type, kernel[0], kernel[1], stride[0], stride[1], pad_top_left[0], pad_top_left[1], ow, oh, 0, int(count_include_pad))
+        out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.float32)
+        check(lib().ncnnhip_pooling_nhwc(C.byref(d), src.ptr, out.ptr, self.stream))
+        return self.from_channels_last(out, n, c, oh, ow)
+
+    def softmax(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        n, count = x.shape
+        dx = self.up(x)
+        out = DeviceBuffer.empty(x.shape, np.float32)
+        check(lib().ncnnhip_softmax(dx.ptr, out.ptr, count, n, self.stream))
+        return out.to_numpy(self.stream)
+
+    def conv_channels_last(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
+                           pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0)):
+        """Convolution (group 1) or depthwise (group == c == num_output) entirely on channels-last device blobs:
+        upload+convert, quantise if fp32, kernel writing channels-last, convert back.  x is [n][c][h][w]."""
+        x = np.ascontiguousarray(x)
+        if x.ndim == 3:
+            x = x[None]
+        n, c, h, w = x.shape
+        d = ConvDesc(w, h, c, n, num_output, kernel[0], kernel[1], dilation[0], dilation[1], stride[0], stride[1],
+                     pads[0], pads[1], pads[2], pads[3], float(pad_value), group)
+        ow, oh = C.c_int(), C.c_int()
+        check(lib().ncnnhip_conv_out_shape(C.byref(d), C.byref(ow), C.byref(oh)))
+        ow, oh = ow.value, oh.value
+        w_scales = np.atleast_1d(np.asarray(w_scales, np.float32))
+        in_scales = np.atleast_1d(np.asarray(in_scales, np.float32))
+        scale_in = self.fold_input_scales(w_scales, in_scales, num_output)
+        requant = term > 100
+        src = self.to_channels_last(x)
+        if x.dtype != np.int8:
+            per_channel = np.repeat(in_scales, c // in_scales.size).astype(np.float32) if in_scales.size > 1 else in_scales
+            src = self.quantize_channels_last(src, c, per_channel)
+        scale_out = None
+        if requant:
+            ts = np.atleast_1d(np.asarray(top_scales, np.float32))
+            scale_out = np.repeat(ts, num_output // ts.size).astype(np.float32)
+        dsi, db, dso = self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32)), self.up(scale_out)
+        ocp = lib().ncnnhip_padded_channels(num_output)
+        dout = DeviceBuffer.empty((n, oh * ow, ocp), np.int8 if requant else np.float32)
+        wq = np.ascontiguousarray(weight, np.int8)
+        if group == 1:
+            nb, wb, sb_ = C.c_size_t(), C.c_size_t(), C.c_size_t()
+            check(lib().ncnnhip_conv_nhwc_sizes(C.byref(d), C.byref(nb), C.byref(wb), C.byref(sb_)))
+            pk = np.empty(wb.value, np.int8)
+            check(lib().ncnnhip_conv_pack_weights(C.byref(d), wq.ctypes.data, pk.ctypes.data))
+            dpk, dws = self.up(pk), DeviceBuffer(max(sb_.value, 4))
+            check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
+                                               1, 0, 0, dws.ptr, sb_.value, self.stream))
+        else:
+            taps = kernel[0] * kernel[1]
+            pk = np.empty(taps * src.shape[2], np.int8)
+            check(lib().ncnnhip_dwconv_pack_weights(c, taps, wq.ctypes.data, pk.ctypes.data))
+            dpk = self.up(pk)
+            check(lib().ncnnhip_dwconv_int8_nhwc(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr, self.stream))
+        raw = dout.to_numpy(self.stream)
+        assert not raw[:, :, num_output:].any(), "pad channels of a channels-last blob must be zero"
+        return self.from_channels_last(dout, n, num_output, oh, ow)
 
     # -- InnerProduct -------------------------------------------------------------------------
     def innerproduct_layer(self, x, weight, bias, w_scales, in_scale, act=0, act_params=(0.0, 0.0), want_acc=False):

@@ -265,8 +265,8 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
                                   (int8_t*)d_nhwc, st);
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_to_nhwc_int8");
         rc = ncnnhip_conv_int8_nhwc(&desc, (const int8_t*)d_nhwc, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias,
-                                    (const float*)d_scale_out, make_activation(activation_type, activation_params), d_out, top_blob.cstep,
-                                    top_blob.nstep, d_ws, workspace_bytes, st);
+                                    (const float*)d_scale_out, make_activation(activation_type, activation_params), d_out, NCNNHIP_PLANAR,
+                                    top_blob.cstep, top_blob.nstep, d_ws, workspace_bytes, st);
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");
         rc = ncnnhip_memcpy_d2h(top_blob.data, d_out, mat_bytes(top_blob), st);
         if (rc == 0) rc = ncnnhip_stream_synchronize(st);

@@ -1,0 +1,182 @@
+"""Device-resident (channels-last) blobs: layout round trips, the quantise pass, both convolution kernels writing
+channels-last, and the fp32 layers between them -- each against the oracle or a scalar restatement of the
+reference loop (pooling.cpp, eltwise.cpp, relu.cpp, softmax.cpp) on the same seeded inputs."""
+import numpy as np
+import pytest
+
+from tests import cases
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def rt():
+    import ncnn_amd
+    return ncnn_amd.Runtime(0)
+
+
+def _say(*a):
+    print("[case]", *a, flush=True)
+
+
+@pytest.mark.parametrize("n,c,h,w", [(1, 3, 5, 7), (2, 16, 9, 9), (3, 70, 13, 11), (1, 130, 1, 1)])
+@pytest.mark.parametrize("dtype", [np.float32, np.int8])
+def test_layout_round_trip_and_zero_padding(rt, n, c, h, w, dtype):
+    _say("layout", n, c, h, w, dtype)
+    rng = np.random.default_rng(c * h)
+    x = rng.integers(-127, 128, (n, c, h, w)).astype(dtype)
+    buf = rt.to_channels_last(x)
+    raw = buf.to_numpy(rt.stream)
+    assert raw.shape == (n, h * w, (c + 15) // 16 * 16)
+    assert np.array_equal(raw[:, :, :c], x.reshape(n, c, h * w).transpose(0, 2, 1))
+    assert not raw[:, :, c:].any()
+    assert np.array_equal(rt.from_channels_last(buf, n, c, h, w), x)
+
+
+@pytest.mark.parametrize("c,per_channel", [(3, False), (24, True), (64, False), (100, True)])
+def test_quantize_channels_last_matches_oracle(rt, c, per_channel):
+    rng = np.random.default_rng(c)
+    x = rng.uniform(-3, 3, (2, c, 6, 5)).astype(F)
+    x.flat[::97] = np.array([0.5, -0.5, 126.5, -126.5, 127.49, 200, -200, 1.5], F)[np.arange(x.flat[::97].size) % 8]
+    scales = rng.uniform(20, 60, c if per_channel else 1).astype(F)
+    want = oracle.quantize(x.transpose(1, 0, 2, 3).reshape(c, -1), scales).reshape(c, 2, 6, 5).transpose(1, 0, 2, 3)
+    q = rt.quantize_channels_last(rt.to_channels_last(x), c, scales)
+    raw = q.to_numpy(rt.stream)
+    assert not raw[:, :, c:].any()
+    assert np.array_equal(rt.from_channels_last(q, 2, c, 6, 5), want)
+
+
+CONV_CASES = [
+    # c, h, w, outc, kernel, dilation, stride, pads
+    (3, 9, 11, 4, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (5, 8, 7, 6, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (4, 12, 10, 8, (3, 2), (2, 1), (2, 1), (2, 1, 0, 1)),
+    (2, 13, 13, 3, (5, 5), (1, 1), (2, 2), (-233, -233, -233, -233)),
+    (16, 20, 20, 130, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (64, 14, 14, 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (96, 7, 7, 200, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (512, 7, 7, 72, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),   # K split over workgroups
+    (32, 150, 150, 136, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),  # 128-row tiles with a ragged last tile
+]
+
+
+@pytest.mark.parametrize("shape", CONV_CASES)
+@pytest.mark.parametrize("term,act,act_params,int8_in", [(2, 1, (0, 0), False), (102, 3, (0.0, 6.0), True), (101, 0, (0, 0), False)])
+def test_convolution_channels_last_bit_exact(rt, shape, term, act, act_params, int8_in):
+    c, h, w, outc, kernel, dilation, stride, pads = shape
+    _say("conv channels-last", shape, term, act, int8_in)
+    x, wq, b, ws, ins, tops = cases.conv_case(c * 10 + outc + term, c, h, w, outc, kernel, 1, term, True, int8_in)
+    d = oracle.make_desc((c, h, w), outc, kernel, dilation, stride, pads, 0.0, 1, 1, term, act, act_params)
+    want = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0], None if tops is None else tops[0])
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act, act_params)
+    assert got.dtype == want.dtype and np.array_equal(got[0], want)
+
+
+def test_convolution_channels_last_batch_and_pad_value(rt):
+    x, wq, b, ws, ins, tops = cases.conv_case(21, 20, 10, 9, 24, (3, 3), 1, 101, True, False, batch=3)
+    d = oracle.make_desc((20, 10, 9), 24, (3, 3), pads=(1, 1, 1, 1), pad_value=-2.2, bias_term=1, int8_scale_term=101, activation_type=1)
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, 24, (3, 3), pads=(1, 1, 1, 1), pad_value=-2.2, term=101, act=1)
+    for i in range(3):
+        assert np.array_equal(got[i], oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], tops[0]))
+
+
+@pytest.mark.parametrize("c,h,w,kernel,stride,dilation,pads", [
+    (6, 9, 10, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)), (32, 56, 56, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (96, 28, 28, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1)), (40, 15, 17, (5, 5), (1, 1), (2, 2), (-233, -233, -233, -233)),
+    (144, 14, 14, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1))])
+@pytest.mark.parametrize("term,act,int8_in", [(1, 0, False), (101, 3, True), (102, 1, False), (2, 3, False)])
+def test_depthwise_channels_last_bit_exact(rt, c, h, w, kernel, stride, dilation, pads, term, act, int8_in):
+    _say("depthwise channels-last", c, h, w, kernel, stride, term, act, int8_in)
+    by_group = term in (1, 101)
+    x, wq, b, ws, ins, tops = cases.conv_case(c + term, c, h, w, c, kernel, c, term, True, int8_in, by_group=True, batch=2)
+    if not by_group:
+        ws = np.full(c, ws[0], F)
+    d = oracle.make_desc((c, h, w), c, kernel, dilation, stride, pads, 0.0, 1, c, term, act, (0.0, 6.0))
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, c, kernel, dilation, stride, pads, 0.0, c, term, act, (0.0, 6.0))
+    for i in range(2):
+        want = oracle.convolutiondepthwise_int8(d, x[i], wq, b, ws, ins, tops)
+        assert got.dtype == want.dtype and np.array_equal(got[i], want)
+
+
+# ---- fp32 layers between the int8 layers --------------------------------------------------------------------
+def _pool_ref(x, kind, k, s, pt, pl, oh, ow, include_pad):
+    """Scalar restatement of Pooling::forward on one [c][h][w] sample with the border already resolved
+    (src/layer/pooling.cpp:150-330): windows anchored at (i*s - pad), taps outside the image are -FLT_MAX for max,
+    skipped (count_include_pad=0) or zero (=1) for average; sums run ky-major in float32."""
+    c, h, w = x.shape
+    out = np.zeros((c, oh, ow), F)
+    for q in range(c):
+        for i in range(oh):
+            for j in range(ow):
+                vals = []
+                for ky in range(k[1]):
+                    for kx in range(k[0]):
+                        y, xx = i * s[1] - pt + ky, j * s[0] - pl + kx
+                        vals.append(x[q, y, xx] if 0 <= y < h and 0 <= xx < w else None)
+                inside = [v for v in vals if v is not None]
+                if kind == 0:
+                    out[q, i, j] = max(inside) if inside else -np.finfo(F).max
+                else:
+                    acc = F(0)
+                    for v in inside:
+                        acc = F(acc + v)
+                    out[q, i, j] = F(acc / F(len(vals) if include_pad else len(inside)))
+    return out
+
+
+@pytest.mark.parametrize("kind,k,s,pt,pl,include_pad", [(0, (3, 3), (2, 2), 0, 0, 0), (0, (3, 3), (2, 2), 1, 1, 0), (0, (2, 3), (1, 2), 0, 1, 0),
+                                                         (1, (3, 3), (2, 2), 1, 1, 0), (1, (3, 3), (1, 1), 1, 1, 1), (1, (2, 2), (2, 2), 0, 0, 0)])
+def test_pooling_matches_scalar_restatement(rt, kind, k, s, pt, pl, include_pad):
+    rng = np.random.default_rng(kind * 10 + k[0])
+    n, c, h, w = 2, 20, 11, 12
+    x = rng.normal(0, 1, (n, c, h, w)).astype(F)
+    # tail pads of "full" mode: the last partial window is kept
+    oh = -(-(h + pt - k[1]) // s[1]) + 1
+    ow = -(-(w + pl - k[0]) // s[0]) + 1
+    got = rt.pooling(x, kind, k, s, (pt, pl), (oh, ow), count_include_pad=include_pad)
+    for i in range(n):
+        assert np.array_equal(got[i], _pool_ref(x[i], kind, k, s, pt, pl, oh, ow, include_pad))
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_global_pooling(rt, kind):
+    rng = np.random.default_rng(kind)
+    x = rng.normal(0, 1, (3, 70, 7, 7)).astype(F)
+    got = rt.pooling(x, kind, None, None, None, None, global_pooling=True)
+    flat = x.reshape(3, 70, 49)
+    want = flat.max(axis=2) if kind == 0 else (np.cumsum(flat, axis=2, dtype=F)[..., -1] / F(49)).astype(F)
+    assert np.array_equal(got, want)
+
+
+def test_relu_and_leaky_relu(rt):
+    rng = np.random.default_rng(3)
+    x = rng.normal(0, 1, 4096).astype(F)
+    assert np.array_equal(rt.relu(x), np.maximum(x, 0))
+    assert np.array_equal(rt.relu(x, 0.1), np.where(x < 0, (x * F(0.1)).astype(F), x))
+    q = rng.integers(-127, 128, 1000).astype(np.int8)
+    assert np.array_equal(rt.relu(q), np.maximum(q, 0))
+
+
+def test_eltwise_all_modes(rt):
+    rng = np.random.default_rng(4)
+    a, b, c = [rng.normal(0, 1, 2048).astype(F) for _ in range(3)]
+    assert np.array_equal(rt.eltwise([a, b], 1), a + b)
+    assert np.array_equal(rt.eltwise([a, b, c], 1), (a + b) + c)
+    assert np.array_equal(rt.eltwise([a, b, c], 0), (a * b) * c)
+    assert np.array_equal(rt.eltwise([a, b, c], 2), np.maximum(np.maximum(a, b), c))
+    co = [F(0.5), F(-1.25), F(3.0)]
+    want = ((a * co[0]).astype(F) + (b * co[1]).astype(F)).astype(F) + (c * co[2]).astype(F)
+    assert np.array_equal(rt.eltwise([a, b, c], 1, co), want.astype(F))
+
+
+def test_softmax_within_1e_6(rt):
+    # the device expf and a tree reduction replace libm expf and the sequential sum: tolerance, not bit parity
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 3, (4, 1000)).astype(F)
+    got = rt.softmax(x)
+    e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    want = e / e.sum(axis=1, keepdims=True)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-9)
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
