@@ -29,6 +29,11 @@ void ncnn_option_set_num_threads(ncnn_option_t opt, int num_threads);
 void ncnn_option_set_lightmode(ncnn_option_t opt, int enable); /* Option::lightmode */
 void ncnn_option_set_use_int8_inference(ncnn_option_t opt, int enable); /* Option::use_int8_inference */
 int ncnn_option_get_use_int8_inference(const ncnn_option_t opt);
+/* Option::use_hip_compute: layers with a device-resident overload keep their blobs in HBM between each other (the switch
+ * ncnn_option_set_use_vulkan_compute, src/c_api.h:85, is for the reference's GPU path).  Set on the net's option before
+ * ncnn_extractor_create. */
+void ncnn_option_set_use_hip_compute(ncnn_option_t opt, int enable);
+int ncnn_option_get_use_hip_compute(const ncnn_option_t opt);
 
 /* src/c_api.h:134-165; data is caller-owned memory laid out as ncnn::Mat lays it out */
 ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);

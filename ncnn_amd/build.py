@@ -46,7 +46,7 @@ def build_kernels(jobs=8):
     return LIBNCNNHIP
 
 
-HOST_SOURCES = ["ncnn/allocator.cpp", "ncnn/mat.cpp", "ncnn/option.cpp", "ncnn/datareader.cpp", "ncnn/paramdict.cpp", "ncnn/modelbin.cpp",
+HOST_SOURCES = ["ncnn/allocator.cpp", "ncnn/mat.cpp", "ncnn/option.cpp", "ncnn/datareader.cpp", "ncnn/paramdict.cpp", "ncnn/modelbin.cpp", "ncnn/hipmat.cpp",
                 "ncnn/layer.cpp", "ncnn/net.cpp", "layers/glue_layers.cpp", "layers/hip_support.cpp", "layers/convolution_hip.cpp",
                 "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "c_api.cpp"]
 LIBNCNN_AMD = os.path.join(LIBDIR, "libncnn_amd.so")

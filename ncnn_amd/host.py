@@ -27,6 +27,7 @@ def lib():
             "ncnn_option_create": (vp, []), "ncnn_option_destroy": (None, [vp]), "ncnn_option_set_num_threads": (None, [vp, ci]),
             "ncnn_option_set_lightmode": (None, [vp, ci]), "ncnn_option_set_use_int8_inference": (None, [vp, ci]),
             "ncnn_option_get_use_int8_inference": (ci, [vp]),
+            "ncnn_option_set_use_hip_compute": (None, [vp, ci]), "ncnn_option_get_use_hip_compute": (ci, [vp]),
             "ncnn_mat_create_external_1d_elem": (vp, [ci, vp, cs, ci, vp]), "ncnn_mat_create_external_2d_elem": (vp, [ci, ci, vp, cs, ci, vp]),
             "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, cs, ci]),
             "ncnn_mat_destroy": (None, [vp]), "ncnn_mat_get_dims": (ci, [vp]), "ncnn_mat_get_w": (ci, [vp]), "ncnn_mat_get_h": (ci, [vp]),
@@ -177,6 +178,10 @@ class Net:
 
     def set_lightmode(self, enable):
         lib().ncnn_option_set_lightmode(lib().ncnn_net_get_option(self.h_), int(enable))
+
+    def set_use_hip_compute(self, enable):
+        """Blobs stay in HBM between layers that have a device-resident overload; set before create_extractor."""
+        lib().ncnn_option_set_use_hip_compute(lib().ncnn_net_get_option(self.h_), int(enable))
 
     def load_param(self, path):
         return lib().ncnn_net_load_param(self.h_, path.encode())

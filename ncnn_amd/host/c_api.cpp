@@ -54,6 +54,14 @@ int ncnn_option_get_use_int8_inference(const ncnn_option_t opt)
 {
     return O(opt)->use_int8_inference;
 }
+void ncnn_option_set_use_hip_compute(ncnn_option_t opt, int enable)
+{
+    O(opt)->use_hip_compute = enable != 0;
+}
+int ncnn_option_get_use_hip_compute(const ncnn_option_t opt)
+{
+    return O(opt)->use_hip_compute;
+}
 
 ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t)
 {

@@ -14,7 +14,7 @@ Convolution_hip::Convolution_hip(bool depthwise_type) : is_depthwise_type(depthw
     one_blob_only = true;
     support_inplace = false;
     support_batch = true; // Mat.n is folded into the pixel dimension of the implicit GEMM
-    d_weight = d_weight_packed = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
+    d_weight = d_weight_packed = d_weight_dw = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
     input_scale_count = 0;
     group = 1;
 }
@@ -59,7 +59,40 @@ int Convolution_hip::load_param(const ParamDict& pd)
         return -1;
     }
     support_int8_storage = true;
+    // device-resident kernels exist for plain convolutions and for true depthwise ones; a grouped convolution in
+    // between takes host Mats (and still runs on the device, through the planar kernel)
+    const int taps = kernel_w * kernel_h;
+    const bool depthwise = group > 1 && group == num_output && taps > 0 && weight_data_size == num_output * taps;
+    support_hip = group == 1 || depthwise;
     return 0;
+}
+
+bool Convolution_hip::is_depthwise() const
+{
+    return group > 1 && group == num_output && weight_data_size == num_output * kernel_w * kernel_h;
+}
+
+ncnnhip_conv_desc Convolution_hip::describe(int w, int h, int channels, int batch) const
+{
+    ncnnhip_conv_desc desc;
+    desc.w = w;
+    desc.h = h;
+    desc.c = channels;
+    desc.batch = batch;
+    desc.num_output = num_output;
+    desc.kernel_w = kernel_w;
+    desc.kernel_h = kernel_h;
+    desc.dilation_w = dilation_w;
+    desc.dilation_h = dilation_h;
+    desc.stride_w = stride_w;
+    desc.stride_h = stride_h;
+    desc.pad_left = pad_left;
+    desc.pad_right = pad_right;
+    desc.pad_top = pad_top;
+    desc.pad_bottom = pad_bottom;
+    desc.pad_value = pad_value;
+    desc.group = group;
+    return desc;
 }
 
 int Convolution_hip::load_model(const ModelBin& mb)
@@ -160,6 +193,15 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
     }
     else
         ret = upload_constant(weight_data.data, (size_t)weight_data_size, &d_weight);
+    if (ret == 0 && is_depthwise())
+    {
+        // device-resident form of the depthwise kernel: weights as [tap][padded channels]
+        const int taps = kernel_w * kernel_h;
+        std::vector<int8_t> packed((size_t)taps * ncnnhip_padded_channels(num_output));
+        rc = ncnnhip_dwconv_pack_weights(num_output, taps, (const int8_t*)weight_data.data, packed.data());
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_dwconv_pack_weights");
+        ret = upload_constant(packed.data(), packed.size(), &d_weight_dw);
+    }
     if (ret == 0) ret = upload_constant(scale_in.data(), scale_in.size() * 4, &d_scale_in);
     if (ret == 0 && bias_term) ret = upload_constant(bias_data.data, (size_t)num_output * 4, &d_bias);
     if (ret == 0 && int8_scale_term > 100)
@@ -180,7 +222,7 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
 
 int Convolution_hip::destroy_pipeline(const Option& /*opt*/)
 {
-    void** all[] = {&d_weight, &d_weight_packed, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
+    void** all[] = {&d_weight, &d_weight_packed, &d_weight_dw, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
@@ -214,24 +256,7 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
         return -1;
     }
 
-    ncnnhip_conv_desc desc;
-    desc.w = bottom_blob.w;
-    desc.h = bottom_blob.h;
-    desc.c = channels;
-    desc.batch = batch;
-    desc.num_output = num_output;
-    desc.kernel_w = kernel_w;
-    desc.kernel_h = kernel_h;
-    desc.dilation_w = dilation_w;
-    desc.dilation_h = dilation_h;
-    desc.stride_w = stride_w;
-    desc.stride_h = stride_h;
-    desc.pad_left = pad_left;
-    desc.pad_right = pad_right;
-    desc.pad_top = pad_top;
-    desc.pad_bottom = pad_bottom;
-    desc.pad_value = pad_value;
-    desc.group = group;
+    ncnnhip_conv_desc desc = describe(bottom_blob.w, bottom_blob.h, channels, batch);
     int outw = 0, outh = 0;
     int rc = ncnnhip_conv_out_shape(&desc, &outw, &outh);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_out_shape");
@@ -311,6 +336,72 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
     rc = ncnnhip_memcpy_d2h(top_blob.data, d_out, mat_bytes(top_blob), st);
     if (rc == 0) rc = ncnnhip_stream_synchronize(st);
     return to_ncnn_status(rc, "download top blob");
+}
+
+// Device-resident form: bottom and top are channels-last blobs in HBM.  An fp32 bottom is quantised into scratch
+// (one coalesced pass), an int8 bottom -- written by the previous layer's requantising epilogue -- feeds the kernel
+// as it is.  Nothing is copied to or from the host and nothing waits.
+int Convolution_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option& opt) const
+{
+    if (!opt.use_int8_inference)
+    {
+        NCNN_LOGE("%s %s: use_int8_inference is off and there is no fp32 path in this runtime", type.c_str(), name.c_str());
+        return -1;
+    }
+    if (!d_scale_in || (group == 1 ? !d_weight_packed : !d_weight_dw))
+    {
+        NCNN_LOGE("%s %s: forward before create_pipeline", type.c_str(), name.c_str());
+        return -1;
+    }
+    if (bottom.dims != 3 || (bottom.elemsize != 4u && bottom.elemsize != 1u))
+    {
+        NCNN_LOGE("%s %s: needs a 3-D fp32 or int8 blob", type.c_str(), name.c_str());
+        return -1;
+    }
+    const int channels = bottom.c;
+    if (channels % group != 0) return -100;
+    if (weight_data_size != (num_output / group) * (channels / group) * kernel_w * kernel_h * group)
+    {
+        NCNN_LOGE("%s %s: weight_data_size %d does not match %d input channels", type.c_str(), name.c_str(), weight_data_size, channels);
+        return -1;
+    }
+    ncnnhip_conv_desc desc = describe(bottom.w, bottom.h, channels, bottom.n);
+    int outw = 0, outh = 0;
+    int rc = ncnnhip_conv_out_shape(&desc, &outw, &outh);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_out_shape");
+
+    const bool requant = int8_scale_term > 100;
+    top.create(outw, outh, num_output, requant ? (size_t)1u : (size_t)4u, bottom.n, &cmd);
+    if (top.empty()) return -100;
+    ScopedScratch scratch(&cmd);
+    void* st = cmd.stream;
+
+    const int8_t* xq = (const int8_t*)bottom.data;
+    if (bottom.elemsize == 4u)
+    {
+        void* q = scratch.get(bottom.count());
+        if (!q) return -100;
+        // every entry of a depthwise layer's input scale table holds the same value (load_model broadcasts the
+        // single stored scale), so one scale serves all channels
+        rc = ncnnhip_quantize_nhwc((const float*)bottom.data, (int8_t*)q, (size_t)bottom.n * bottom.h * bottom.w, channels, (const float*)d_input_scales, 1, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_quantize_nhwc");
+        xq = (const int8_t*)q;
+    }
+
+    const ncnnhip_activation act = make_activation(activation_type, activation_params);
+    if (group == 1)
+    {
+        size_t workspace_bytes = 0;
+        rc = ncnnhip_conv_nhwc_sizes(&desc, 0, 0, &workspace_bytes);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
+        void* ws = workspace_bytes ? scratch.get(workspace_bytes) : 0;
+        if (workspace_bytes && !ws) return -100;
+        rc = ncnnhip_conv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, (const float*)d_scale_out, act,
+                                    top.data, NCNNHIP_CHANNELS_LAST, 0, 0, ws, workspace_bytes, st);
+        return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");
+    }
+    rc = ncnnhip_dwconv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_dw, (const float*)d_scale_in, (const float*)d_bias, (const float*)d_scale_out, act, top.data, st);
+    return to_ncnn_status(rc, "ncnnhip_dwconv_int8_nhwc");
 }
 
 Layer* Convolution_hip_creator(void*)

@@ -11,8 +11,17 @@
 #include <algorithm>
 
 #include "../ncnn/layer.h"
+#include "ncnnhip.h"
 
 namespace ncnn {
+
+// C-ABI status -> ncnn's 0 / -100 / -1
+static int dev_status(int rc, const char* where)
+{
+    if (rc == 0) return 0;
+    NCNN_LOGE("%s failed: %s", where, ncnnhip_last_error());
+    return rc == NCNNHIP_OOM ? -100 : -1;
+}
 
 // ---------------------------------------------------------------------------------- Input
 class Input : public Layer
@@ -23,6 +32,11 @@ public:
         one_blob_only = true;
         support_inplace = true;
         support_batch = true;
+        support_hip = true;
+    }
+    virtual int forward_inplace_hip(HipMat&, HipCommand&, const Option&) const
+    {
+        return 0;
     }
     virtual int load_param(const ParamDict& pd)
     {
@@ -47,6 +61,12 @@ public:
     {
         support_batch = true;
         support_int8_storage = true; // int8 blobs pass through untouched
+        support_hip = true;
+    }
+    virtual int forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand&, const Option&) const
+    {
+        for (size_t i = 0; i < top_blobs.size(); i++) top_blobs[i] = bottom_blobs[0]; // shared, refcounted
+        return 0;
     }
     virtual int forward(const std::vector<Mat>& bottom_blobs, std::vector<Mat>& top_blobs, const Option&) const
     {
@@ -64,11 +84,22 @@ public:
         one_blob_only = true;
         support_inplace = true;
         support_int8_storage = true;
+        support_hip = true;
     }
     virtual int load_param(const ParamDict& pd)
     {
         slope = pd.get(0, 0.f);
         return 0;
+    }
+    virtual int forward_inplace_hip(HipMat& m, HipCommand& cmd, const Option&) const
+    {
+        // flat over the blob, pad channels included (zero stays zero)
+        if (m.elemsize == 4u && m.count() % 4 != 0)
+        {
+            // dense 1-D / 2-D blobs of odd size: the pool rounds allocations up to 64 KiB, so the tail is ours
+            return dev_status(ncnnhip_relu(m.data, m.data, 4, (m.count() + 3) / 4 * 4, slope, cmd.stream), "ncnnhip_relu");
+        }
+        return dev_status(ncnnhip_relu(m.data, m.data, (int)m.elemsize, m.count(), slope, cmd.stream), "ncnnhip_relu");
     }
     virtual int forward_inplace(Mat& m, const Option& opt) const
     {
@@ -132,7 +163,72 @@ public:
             NCNN_LOGE("Pooling: adaptive pooling is not part of this runtime");
             return -1;
         }
+        support_hip = true;
         return 0;
+    }
+
+    // head pads and output extent of the border the reference would materialise (pad_mode 0 keeps the last
+    // partial window, 1 drops it, 2/3 are the SAME splits)
+    void resolve(int w, int h, int& pt, int& pl, int& outw, int& outh) const
+    {
+        int pb = pad_bottom, pr = pad_right;
+        pt = pad_top;
+        pl = pad_left;
+        if (pad_mode == 0)
+        {
+            const int wtail = (w + pad_left + pad_right - kernel_w) % stride_w;
+            const int htail = (h + pad_top + pad_bottom - kernel_h) % stride_h;
+            if (wtail != 0) pr += stride_w - wtail;
+            if (htail != 0) pb += stride_h - htail;
+        }
+        else if (pad_mode == 2 || pad_mode == 3)
+        {
+            const int wpad = kernel_w + (w - 1) / stride_w * stride_w - w;
+            const int hpad = kernel_h + (h - 1) / stride_h * stride_h - h;
+            pt = pb = pl = pr = 0;
+            if (wpad > 0 || hpad > 0)
+            {
+                const int hs = hpad / 2, hl = hpad - hpad / 2, ws = wpad / 2, wl = wpad - wpad / 2;
+                pt = pad_mode == 2 ? hs : hl;
+                pb = pad_mode == 2 ? hl : hs;
+                pl = pad_mode == 2 ? ws : wl;
+                pr = pad_mode == 2 ? wl : ws;
+            }
+        }
+        outw = (w + pl + pr - kernel_w) / stride_w + 1;
+        outh = (h + pt + pb - kernel_h) / stride_h + 1;
+    }
+
+    virtual int forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option&) const
+    {
+        if (bottom.dims != 3 || bottom.elemsize != 4u)
+        {
+            NCNN_LOGE("Pooling: needs a 3-D fp32 blob");
+            return -1;
+        }
+        ncnnhip_pool_desc d;
+        memset(&d, 0, sizeof(d));
+        d.w = bottom.w;
+        d.h = bottom.h;
+        d.c = bottom.c;
+        d.batch = bottom.n;
+        d.pooling_type = pooling_type;
+        d.global_pooling = global_pooling;
+        d.avgpool_count_include_pad = avgpool_count_include_pad;
+        if (global_pooling)
+        {
+            top.create(bottom.c, 4u, bottom.n, &cmd);
+            if (top.empty()) return -100;
+            return dev_status(ncnnhip_pooling_nhwc(&d, (const float*)bottom.data, (float*)top.data, cmd.stream), "ncnnhip_pooling_nhwc");
+        }
+        d.kernel_w = kernel_w;
+        d.kernel_h = kernel_h;
+        d.stride_w = stride_w;
+        d.stride_h = stride_h;
+        resolve(bottom.w, bottom.h, d.pad_top, d.pad_left, d.outw, d.outh);
+        top.create(d.outw, d.outh, bottom.c, 4u, bottom.n, &cmd);
+        if (top.empty()) return -100;
+        return dev_status(ncnnhip_pooling_nhwc(&d, (const float*)bottom.data, (float*)top.data, cmd.stream), "ncnnhip_pooling_nhwc");
     }
 
     virtual int forward(const Mat& bottom, Mat& top, const Option& opt) const
@@ -168,33 +264,8 @@ public:
             return 0;
         }
 
-        // resolve the border the reference would materialise: head pads, tail pads (+ the extra
-        // tail of "full" mode that keeps the last partial window)
-        int pt = pad_top, pb = pad_bottom, pl = pad_left, pr = pad_right;
-        if (pad_mode == 0)
-        {
-            const int wtail = (w + pad_left + pad_right - kernel_w) % stride_w;
-            const int htail = (h + pad_top + pad_bottom - kernel_h) % stride_h;
-            if (wtail != 0) pr += stride_w - wtail;
-            if (htail != 0) pb += stride_h - htail;
-        }
-        else if (pad_mode == 2 || pad_mode == 3)
-        {
-            const int wpad = kernel_w + (w - 1) / stride_w * stride_w - w;
-            const int hpad = kernel_h + (h - 1) / stride_h * stride_h - h;
-            pt = pb = pl = pr = 0;
-            if (wpad > 0 || hpad > 0)
-            {
-                const int hs = hpad / 2, hl = hpad - hpad / 2, ws = wpad / 2, wl = wpad - wpad / 2;
-                pt = pad_mode == 2 ? hs : hl;
-                pb = pad_mode == 2 ? hl : hs;
-                pl = pad_mode == 2 ? ws : wl;
-                pr = pad_mode == 2 ? wl : ws;
-            }
-        }
-        const int W = w + pl + pr, H = h + pt + pb;
-        const int outw = (W - kernel_w) / stride_w + 1;
-        const int outh = (H - kernel_h) / stride_h + 1;
+        int pt, pl, outw, outh;
+        resolve(w, h, pt, pl, outw, outh);
         top.create(outw, outh, channels, 4u, opt.blob_allocator);
         if (top.empty()) return -100;
 
@@ -274,7 +345,27 @@ public:
     {
         op_type = pd.get(0, 0);
         coeffs = pd.get(1, Mat());
+        support_hip = true;
         return 0;
+    }
+    virtual int forward_hip(const std::vector<HipMat>& bottoms, std::vector<HipMat>& tops, HipCommand& cmd, const Option&) const
+    {
+        if (bottoms.size() < 2) return -1;
+        std::vector<const float*> srcs(bottoms.size());
+        for (size_t i = 0; i < bottoms.size(); i++)
+        {
+            if (bottoms[i].elemsize != 4u || bottoms[i].count() != bottoms[0].count())
+            {
+                NCNN_LOGE("Eltwise: inputs must be fp32 blobs of one shape");
+                return -1;
+            }
+            srcs[i] = (const float*)bottoms[i].data;
+        }
+        tops[0].create_like(bottoms[0], &cmd);
+        if (tops[0].empty()) return -100;
+        const size_t count = (bottoms[0].count() + 3) / 4 * 4; // allocations are rounded up, the tail is ours
+        return dev_status(ncnnhip_eltwise(srcs.data(), (int)srcs.size(), op_type, coeffs.w ? (const float*)coeffs.data : 0, coeffs.w, (float*)tops[0].data, count, cmd.stream),
+                          "ncnnhip_eltwise");
     }
     virtual int forward(const std::vector<Mat>& bottoms, std::vector<Mat>& tops, const Option& opt) const
     {
@@ -325,6 +416,26 @@ public:
     Flatten()
     {
         one_blob_only = true;
+        support_hip = true;
+        support_int8_storage = true;
+    }
+    virtual int forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option&) const
+    {
+        if (bottom.dims != 3)
+        {
+            // dense blobs are already flat: same memory, new shape
+            top = bottom;
+            top.dims = 1;
+            top.w = bottom.w * bottom.h;
+            top.h = 1;
+            return 0;
+        }
+        // the flattened order is the planar one: channel-major
+        const int hw = bottom.w * bottom.h;
+        top.create(hw * bottom.c, bottom.elemsize, bottom.n, &cmd);
+        if (top.empty()) return -100;
+        return dev_status(ncnnhip_nhwc_to_chw(bottom.data, (int)bottom.elemsize, bottom.c, hw, bottom.n, top.data, (size_t)hw, (size_t)hw * bottom.c, cmd.stream),
+                          "ncnnhip_nhwc_to_chw");
     }
     virtual int forward(const Mat& bottom, Mat& top, const Option& opt) const
     {
@@ -349,7 +460,17 @@ public:
     virtual int load_param(const ParamDict& pd)
     {
         axis = pd.get(0, 0);
+        support_hip = axis == 0;
         return 0;
+    }
+    virtual int forward_inplace_hip(HipMat& m, HipCommand& cmd, const Option&) const
+    {
+        if (m.dims != 1 || m.elemsize != 4u)
+        {
+            NCNN_LOGE("Softmax: the device overload handles 1-D fp32 blobs");
+            return -1;
+        }
+        return dev_status(ncnnhip_softmax((const float*)m.data, (float*)m.data, m.w, m.n, cmd.stream), "ncnnhip_softmax");
     }
     virtual int forward_inplace(Mat& m, const Option&) const
     {
@@ -393,7 +514,14 @@ public:
     virtual int load_param(const ParamDict& pd)
     {
         scale = pd.get(0, 1.f);
+        support_hip = true;
         return 0;
+    }
+    virtual int forward_inplace_hip(HipMat& m, HipCommand& cmd, const Option&) const
+    {
+        if (scale == 1.f) return 0;
+        if (m.elemsize != 4u) return -1;
+        return dev_status(ncnnhip_scale((const float*)m.data, (float*)m.data, m.count(), scale, cmd.stream), "ncnnhip_scale");
     }
     virtual int forward_inplace(Mat& m, const Option&) const
     {

@@ -5,6 +5,7 @@
 #define NCNN_AMD_HIP_LAYERS_H
 
 #include "../ncnn/layer.h"
+#include "ncnnhip.h"
 
 namespace ncnn_amd {
 
@@ -21,6 +22,7 @@ public:
     virtual int create_pipeline(const ncnn::Option& opt);
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+    virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
 
 public:
     // same member names as the reference layers
@@ -40,8 +42,11 @@ private:
     void* d_bias;
     void* d_scale_in;      // one per output channel: 1/(in_scale*w_scale), 0 when w_scale is 0
     void* d_scale_out;     // one per output channel, only when requantising
-    void* d_input_scales;  // one per input channel, for quantising an fp32 bottom blob
-    int input_scale_count; // 1 or channels
+    void* d_input_scales;  // the layer's input scale table (1 entry, or `group` entries for depthwise types)
+    int input_scale_count; // 1 or group
+    void* d_weight_dw;     // depthwise (channels == group == num_output): [kh*kw][16*ceil(c/16)]
+    bool is_depthwise() const;
+    ncnnhip_conv_desc describe(int w, int h, int channels, int batch) const;
 };
 
 // InnerProduct (src/layer/innerproduct.{h,cpp})
@@ -55,6 +60,7 @@ public:
     virtual int create_pipeline(const ncnn::Option& opt);
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+    virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
 
 public:
     int num_output, bias_term, weight_data_size, int8_scale_term, activation_type;

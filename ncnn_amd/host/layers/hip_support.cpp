@@ -4,51 +4,6 @@
 
 namespace ncnn_amd {
 
-HipContext::HipContext() : stream(0), ready(false) {}
-
-HipContext::~HipContext()
-{
-    for (size_t i = 0; i < pool.size(); i++) ncnnhip_free(pool[i].ptr);
-    if (stream) ncnnhip_stream_destroy(stream);
-}
-
-int HipContext::ensure_ready()
-{
-    if (ready) return 0;
-    int rc = ncnnhip_init(0);
-    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_init");
-    rc = ncnnhip_stream_create(&stream);
-    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_stream_create");
-    ready = true;
-    return 0;
-}
-
-void* HipContext::borrow(size_t bytes)
-{
-    if (bytes == 0) bytes = 4;
-    // smallest idle buffer that fits
-    int best = -1;
-    for (size_t i = 0; i < pool.size(); i++)
-        if (!pool[i].busy && pool[i].bytes >= bytes && (best < 0 || pool[i].bytes < pool[(size_t)best].bytes)) best = (int)i;
-    if (best >= 0)
-    {
-        pool[(size_t)best].busy = true;
-        return pool[(size_t)best].ptr;
-    }
-    Lease l;
-    l.bytes = (bytes + 0xffff) & ~(size_t)0xffff;
-    l.busy = true;
-    l.ptr = 0;
-    if (ncnnhip_malloc(&l.ptr, l.bytes) != 0 || !l.ptr) return 0;
-    pool.push_back(l);
-    return l.ptr;
-}
-
-void HipContext::give_back_all()
-{
-    for (size_t i = 0; i < pool.size(); i++) pool[i].busy = false;
-}
-
 HipBlobAllocator::HipBlobAllocator()
 {
     pool.set_size_compare_ratio(0.f);

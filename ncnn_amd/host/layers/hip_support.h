@@ -9,38 +9,17 @@
 #include <vector>
 
 #include "../ncnn/allocator.h"
+#include "../ncnn/hipmat.h"
 #include "../ncnn/mat.h"
 #include "../ncnn/option.h"
 #include "ncnnhip.h"
 
 namespace ncnn_amd {
 
-// One stream and a grow-only set of device buffers.  forward() of a HIP layer borrows buffers for
-// the duration of the call; everything it launched has completed (stream synchronised) before
-// the buffers go back, so the pool needs no cross-call tracking.
-class HipContext
-{
-public:
-    HipContext();
-    ~HipContext();
-    int ensure_ready(); // lazily selects the device and creates the stream
-    void* stream;
-
-    struct Lease
-    {
-        void* ptr;
-        size_t bytes;
-        bool busy;
-    };
-    void* borrow(size_t bytes);
-    void give_back_all();
-
-private:
-    HipContext(const HipContext&);
-    HipContext& operator=(const HipContext&);
-    bool ready;
-    std::vector<Lease> pool;
-};
+// One stream and a pool of device buffers: the same object that carries device-resident blobs.  forward() of a
+// HIP layer on host Mats borrows scratch for the duration of the call; everything it launched has completed
+// (stream synchronised) before the scratch goes back.
+typedef ncnn::HipCommand HipContext;
 
 // Host allocator to install with Extractor::set_blob_allocator(): it hands out ordinary host
 // memory (ncnn keeps a Mat's refcount inside the allocation and touches results on the host) and

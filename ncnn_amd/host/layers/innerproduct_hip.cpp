@@ -33,6 +33,7 @@ int InnerProduct_hip::load_param(const ParamDict& pd)
         return -1;
     }
     support_int8_storage = true;
+    support_hip = true;
     return 0;
 }
 
@@ -152,6 +153,69 @@ int InnerProduct_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Optio
     rc = ncnnhip_memcpy_d2h(top_blob.data, d_out, (size_t)rows * num_output * 4, st);
     if (rc == 0) rc = ncnnhip_stream_synchronize(st);
     return to_ncnn_status(rc, "download top blob");
+}
+
+// Device-resident form: the blob is already in HBM.  A 1-D blob (or a 3-D one with a single pixel, whose
+// channels-last rows are its channels) is one vector per sample; a 2-D blob with rows of num_input is a row-wise
+// GEMM; any other 3-D blob is flattened to the planar order first.  The batch folds into the row count.
+int InnerProduct_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option& opt) const
+{
+    if (!opt.use_int8_inference)
+    {
+        NCNN_LOGE("InnerProduct %s: use_int8_inference is off and there is no fp32 path in this runtime", name.c_str());
+        return -1;
+    }
+    if (!d_weight) return -1;
+    if (bottom.elemsize != 4u && bottom.elemsize != 1u) return -1;
+    const int num_input = weight_data_size / num_output;
+    ScopedScratch scratch(&cmd);
+    void* st = cmd.stream;
+
+    const void* x = bottom.data;
+    size_t x_stride = (size_t)num_input;
+    int rows = bottom.n;
+    if (bottom.dims == 2 && bottom.w == num_input)
+    {
+        rows = bottom.n * bottom.h;
+        top.create(num_output, bottom.h, 4u, bottom.n, &cmd);
+    }
+    else
+    {
+        const size_t count = bottom.dims == 3 ? (size_t)bottom.w * bottom.h * bottom.c : (size_t)bottom.w * bottom.h;
+        if (count != (size_t)num_input)
+        {
+            NCNN_LOGE("InnerProduct %s: blob has %zu values, weights expect %d", name.c_str(), count, num_input);
+            return -1;
+        }
+        if (bottom.dims == 3 && bottom.w * bottom.h == 1)
+            x_stride = (size_t)bottom.cp;
+        else if (bottom.dims == 3)
+        {
+            const int hw = bottom.w * bottom.h;
+            void* flat = scratch.get((size_t)bottom.n * num_input * bottom.elemsize);
+            if (!flat) return -100;
+            int rc = ncnnhip_nhwc_to_chw(bottom.data, (int)bottom.elemsize, bottom.c, hw, bottom.n, flat, (size_t)hw, (size_t)num_input, st);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_nhwc_to_chw");
+            x = flat;
+        }
+        top.create(num_output, 4u, bottom.n, &cmd);
+    }
+    if (top.empty()) return -100;
+
+    const int8_t* xq = (const int8_t*)x;
+    size_t q_stride = x_stride;
+    if (bottom.elemsize == 4u)
+    {
+        void* q = scratch.get((size_t)rows * num_input);
+        if (!q) return -100;
+        int rc = ncnnhip_quantize((const float*)x, x_stride, 0, (int8_t*)q, (size_t)num_input, 0, rows, num_input, 1, (const float*)d_input_scale, 1, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_quantize");
+        xq = (const int8_t*)q;
+        q_stride = (size_t)num_input;
+    }
+    int rc = ncnnhip_innerproduct_int8(xq, q_stride, rows, num_input, num_output, (const int8_t*)d_weight, (const float*)d_scale_in, (const float*)d_bias,
+                                       make_activation(activation_type, activation_params), (float*)top.data, (size_t)num_output, 0, st);
+    return to_ncnn_status(rc, "ncnnhip_innerproduct_int8");
 }
 
 Layer* InnerProduct_hip_creator(void*)

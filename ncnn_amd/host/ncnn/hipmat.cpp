@@ -1,0 +1,275 @@
+#include "hipmat.h"
+
+#include "ncnnhip.h"
+
+namespace ncnn {
+
+static int hip_status(int rc, const char* where)
+{
+    if (rc == 0) return 0;
+    NCNN_LOGE("%s failed: %s", where, ncnnhip_last_error());
+    return rc == NCNNHIP_OOM ? -100 : -1;
+}
+
+// ---- HipMat -----------------------------------------------------------------------------------
+
+HipMat::HipMat() : data(0), refcount(0), cmd(0), dims(0), w(0), h(0), c(0), n(0), cp(0), elemsize(0) {}
+
+HipMat::HipMat(const HipMat& m) : data(m.data), refcount(m.refcount), cmd(m.cmd), dims(m.dims), w(m.w), h(m.h), c(m.c), n(m.n), cp(m.cp), elemsize(m.elemsize)
+{
+    if (refcount) __sync_fetch_and_add(refcount, 1);
+}
+
+HipMat::~HipMat()
+{
+    release();
+}
+
+HipMat& HipMat::operator=(const HipMat& m)
+{
+    if (this == &m) return *this;
+    if (m.refcount) __sync_fetch_and_add(m.refcount, 1);
+    release();
+    data = m.data;
+    refcount = m.refcount;
+    cmd = m.cmd;
+    dims = m.dims;
+    w = m.w;
+    h = m.h;
+    c = m.c;
+    n = m.n;
+    cp = m.cp;
+    elemsize = m.elemsize;
+    return *this;
+}
+
+void HipMat::release()
+{
+    if (refcount && __sync_fetch_and_add(refcount, -1) == 1)
+    {
+        if (cmd && data) cmd->free(data);
+        delete refcount;
+    }
+    data = 0;
+    refcount = 0;
+    cmd = 0;
+    dims = w = h = c = n = cp = 0;
+    elemsize = 0;
+}
+
+void HipMat::allocate(HipCommand* command)
+{
+    size_t need = bytes();
+    if (need == 0) need = 4;
+    void* p = command->alloc(need);
+    if (!p)
+    {
+        dims = w = h = c = n = cp = 0;
+        elemsize = 0;
+        return;
+    }
+    data = p;
+    cmd = command;
+    refcount = new int(1);
+}
+
+void HipMat::create(int _w, size_t _elemsize, int _n, HipCommand* command)
+{
+    release();
+    dims = 1;
+    w = _w;
+    h = 1;
+    c = 1;
+    n = _n < 1 ? 1 : _n;
+    cp = 0;
+    elemsize = _elemsize;
+    allocate(command);
+}
+
+void HipMat::create(int _w, int _h, size_t _elemsize, int _n, HipCommand* command)
+{
+    release();
+    dims = 2;
+    w = _w;
+    h = _h;
+    c = 1;
+    n = _n < 1 ? 1 : _n;
+    cp = 0;
+    elemsize = _elemsize;
+    allocate(command);
+}
+
+void HipMat::create(int _w, int _h, int _c, size_t _elemsize, int _n, HipCommand* command)
+{
+    release();
+    dims = 3;
+    w = _w;
+    h = _h;
+    c = _c;
+    n = _n < 1 ? 1 : _n;
+    cp = ncnnhip_padded_channels(_c);
+    elemsize = _elemsize;
+    allocate(command);
+}
+
+void HipMat::create_like(const HipMat& m, HipCommand* command)
+{
+    if (m.dims == 1)
+        create(m.w, m.elemsize, m.n, command);
+    else if (m.dims == 2)
+        create(m.w, m.h, m.elemsize, m.n, command);
+    else
+        create(m.w, m.h, m.c, m.elemsize, m.n, command);
+}
+
+// ---- HipCommand ---------------------------------------------------------------------------------
+
+HipCommand::HipCommand() : stream(0), ready(false) {}
+
+HipCommand::~HipCommand()
+{
+    if (ready) ncnnhip_stream_synchronize(stream);
+    for (size_t i = 0; i < pool.size(); i++) ncnnhip_free(pool[i].ptr);
+    if (stream) ncnnhip_stream_destroy(stream);
+}
+
+int HipCommand::ensure_ready()
+{
+    if (ready) return 0;
+    int rc = ncnnhip_init(0);
+    if (rc != 0) return hip_status(rc, "ncnnhip_init");
+    rc = ncnnhip_stream_create(&stream);
+    if (rc != 0) return hip_status(rc, "ncnnhip_stream_create");
+    ready = true;
+    return 0;
+}
+
+void* HipCommand::take(size_t bytes, int state)
+{
+    if (bytes == 0) bytes = 4;
+    // smallest idle buffer that fits without wasting more than half of it
+    int best = -1;
+    for (size_t i = 0; i < pool.size(); i++)
+        if (pool[i].state == 0 && pool[i].bytes >= bytes && pool[i].bytes <= 2 * bytes + 0x10000 && (best < 0 || pool[i].bytes < pool[(size_t)best].bytes)) best = (int)i;
+    if (best >= 0)
+    {
+        pool[(size_t)best].state = state;
+        return pool[(size_t)best].ptr;
+    }
+    Slot s;
+    s.bytes = (bytes + 0xffff) & ~(size_t)0xffff;
+    s.state = state;
+    s.ptr = 0;
+    if (ncnnhip_malloc(&s.ptr, s.bytes) != 0 || !s.ptr) return 0;
+    pool.push_back(s);
+    return s.ptr;
+}
+
+void* HipCommand::alloc(size_t bytes)
+{
+    return take(bytes, 1);
+}
+
+void HipCommand::free(void* ptr)
+{
+    for (size_t i = 0; i < pool.size(); i++)
+        if (pool[i].ptr == ptr)
+        {
+            pool[i].state = 0;
+            return;
+        }
+}
+
+void* HipCommand::borrow(size_t bytes)
+{
+    return take(bytes, 2);
+}
+
+void HipCommand::give_back_all()
+{
+    for (size_t i = 0; i < pool.size(); i++)
+        if (pool[i].state == 2) pool[i].state = 0;
+}
+
+size_t HipCommand::pooled_bytes() const
+{
+    size_t s = 0;
+    for (size_t i = 0; i < pool.size(); i++) s += pool[i].bytes;
+    return s;
+}
+
+int HipCommand::synchronize()
+{
+    return hip_status(ncnnhip_stream_synchronize(stream), "ncnnhip_stream_synchronize");
+}
+
+static size_t host_bytes(const Mat& m)
+{
+    return (m.n > 1 ? m.nstep * m.n : m.total()) * m.elemsize;
+}
+
+int HipCommand::upload(const Mat& src, HipMat& dst)
+{
+    int ret = ensure_ready();
+    if (ret != 0) return ret;
+    if (src.empty() || src.elempack != 1 || (src.elemsize != 4u && src.elemsize != 1u) || src.dims < 1 || src.dims > 3)
+    {
+        NCNN_LOGE("HipCommand::upload: needs a pack-1 fp32 or int8 blob of 1 to 3 dimensions");
+        return -1;
+    }
+    if (src.dims == 3)
+    {
+        dst.create(src.w, src.h, src.c, src.elemsize, src.n, this);
+        if (dst.empty()) return -100;
+        // planar bytes as they lie on the host, then one layout kernel
+        ScopedScratch scratch(this);
+        void* staging = scratch.get(host_bytes(src));
+        if (!staging) return -100;
+        int rc = ncnnhip_memcpy_h2d(staging, src.data, host_bytes(src), stream);
+        if (rc == 0) rc = ncnnhip_chw_to_nhwc(staging, (int)src.elemsize, src.c, src.w * src.h, src.n, src.cstep, src.nstep, dst.data, stream);
+        // the copy out of pageable host memory must have left the caller's buffer before we return
+        if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
+        return hip_status(rc, "upload");
+    }
+    if (src.dims == 1)
+        dst.create(src.w, src.elemsize, src.n, this);
+    else
+        dst.create(src.w, src.h, src.elemsize, src.n, this);
+    if (dst.empty()) return -100;
+    const size_t sample = (size_t)src.w * src.h * src.elemsize;
+    int rc = 0;
+    for (int b = 0; b < src.n && rc == 0; b++)
+        rc = ncnnhip_memcpy_h2d((unsigned char*)dst.data + sample * b, (const unsigned char*)src.data + src.nstep * b * src.elemsize, sample, stream);
+    if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
+    return hip_status(rc, "upload");
+}
+
+int HipCommand::download(const HipMat& src, Mat& dst, Allocator* allocator)
+{
+    if (src.empty()) return -1;
+    if (src.dims == 3)
+    {
+        dst.create(src.w, src.h, src.c, src.elemsize, 1, src.n, allocator);
+        if (dst.empty()) return -100;
+        ScopedScratch scratch(this);
+        void* staging = scratch.get(host_bytes(dst));
+        if (!staging) return -100;
+        int rc = ncnnhip_nhwc_to_chw(src.data, (int)src.elemsize, src.c, src.w * src.h, src.n, staging, dst.cstep, dst.nstep, stream);
+        if (rc == 0) rc = ncnnhip_memcpy_d2h(dst.data, staging, host_bytes(dst), stream);
+        if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
+        return hip_status(rc, "download");
+    }
+    if (src.dims == 1)
+        dst.create(src.w, src.elemsize, 1, src.n, allocator);
+    else
+        dst.create(src.w, src.h, src.elemsize, 1, src.n, allocator);
+    if (dst.empty()) return -100;
+    const size_t sample = (size_t)src.w * src.h * src.elemsize;
+    int rc = 0;
+    for (int b = 0; b < src.n && rc == 0; b++)
+        rc = ncnnhip_memcpy_d2h((unsigned char*)dst.data + dst.nstep * b * dst.elemsize, (const unsigned char*)src.data + sample * b, sample, stream);
+    if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
+    return hip_status(rc, "download");
+}
+
+} // namespace ncnn

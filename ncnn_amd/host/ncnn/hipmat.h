@@ -1,0 +1,125 @@
+// Device-side counterparts of Mat and of the per-inference command object: the roles VkMat (src/mat.h:383-560)
+// and VkCompute (src/command.h:20-120) play for the reference's GPU path, shaped for one HIP stream.
+//
+// HipMat is a refcounted handle to a blob in HBM:
+//   dims 3: channels-last [n][h*w][cp], cp = 16*ceil(c/16), pad channels zero  (fp32 or int8)
+//   dims 1: dense [n][w]            dims 2: dense [n][h][w]
+// HipCommand owns the stream every kernel of one Extractor runs on and a pool of device buffers.  All work of an
+// Extractor is stream-ordered, so a buffer that goes back to the pool can be handed out again at once: whatever
+// still reads it was enqueued earlier on the same stream.
+#ifndef NCNN_HIPMAT_H
+#define NCNN_HIPMAT_H
+
+#include <stddef.h>
+
+#include <vector>
+
+#include "mat.h"
+#include "platform.h"
+
+namespace ncnn {
+
+class HipCommand;
+
+class NCNN_EXPORT HipMat
+{
+public:
+    HipMat();
+    HipMat(const HipMat& m);
+    ~HipMat();
+    HipMat& operator=(const HipMat& m);
+
+    // all return with empty() true when the pool cannot serve the request
+    void create(int w, size_t elemsize, int n, HipCommand* cmd);
+    void create(int w, int h, size_t elemsize, int n, HipCommand* cmd);
+    void create(int w, int h, int c, size_t elemsize, int n, HipCommand* cmd);
+    void create_like(const HipMat& m, HipCommand* cmd);
+    void release();
+
+    bool empty() const
+    {
+        return data == 0;
+    }
+    // elements as they lie in memory, padding included
+    size_t count() const
+    {
+        return dims == 3 ? (size_t)n * h * w * cp : (size_t)n * h * w;
+    }
+    size_t bytes() const
+    {
+        return count() * elemsize;
+    }
+    // true when this handle is the only one (an in-place kernel may overwrite the blob)
+    bool exclusive() const
+    {
+        return refcount && *refcount == 1;
+    }
+
+    void* data;
+    int* refcount; // host side
+    HipCommand* cmd;
+    int dims, w, h, c, n;
+    int cp; // channels as padded in memory (dims 3), else 0
+    size_t elemsize;
+
+private:
+    void allocate(HipCommand* cmd);
+};
+
+class NCNN_EXPORT HipCommand
+{
+public:
+    HipCommand();
+    ~HipCommand();
+    int ensure_ready(); // selects the device and creates the stream on first use
+    void* stream;
+
+    // blob memory (returned when the last HipMat handle goes)
+    void* alloc(size_t bytes);
+    void free(void* ptr);
+    // scratch for one forward call: everything borrowed goes back with give_back_all()
+    void* borrow(size_t bytes);
+    void give_back_all();
+
+    // host Mat (planar, any batch) -> device blob and back; download synchronises the stream
+    int upload(const Mat& src, HipMat& dst);
+    int download(const HipMat& src, Mat& dst, Allocator* allocator);
+    int synchronize();
+
+    size_t pooled_bytes() const;
+
+private:
+    HipCommand(const HipCommand&);
+    HipCommand& operator=(const HipCommand&);
+    struct Slot
+    {
+        void* ptr;
+        size_t bytes;
+        int state; // 0 idle, 1 blob, 2 borrowed scratch
+    };
+    void* take(size_t bytes, int state);
+    bool ready;
+    std::vector<Slot> pool;
+};
+
+// scratch borrowed during one forward() returns to the pool when this goes out of scope
+class ScopedScratch
+{
+public:
+    explicit ScopedScratch(HipCommand* c) : cmd(c) {}
+    ~ScopedScratch()
+    {
+        cmd->give_back_all();
+    }
+    void* get(size_t bytes)
+    {
+        return cmd->borrow(bytes);
+    }
+
+private:
+    HipCommand* cmd;
+};
+
+} // namespace ncnn
+
+#endif // NCNN_HIPMAT_H

@@ -18,6 +18,7 @@ Layer::Layer()
     support_any_packing = false;
     support_vulkan_any_packing = false;
     support_batch = false;
+    support_hip = false;
     featmask = 0;
     userdata = 0;
     typeindex = -1;
@@ -68,6 +69,22 @@ int Layer::forward_inplace(std::vector<Mat>&, const Option&) const
     return -1;
 }
 int Layer::forward_inplace(Mat&, const Option&) const
+{
+    return -1;
+}
+
+int Layer::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& opt) const
+{
+    // one-blob layers reached through the list form
+    if (!one_blob_only || bottom_blobs.size() != 1) return -1;
+    top_blobs.resize(1);
+    return forward_hip(bottom_blobs[0], top_blobs[0], cmd, opt);
+}
+int Layer::forward_hip(const HipMat&, HipMat&, HipCommand&, const Option&) const
+{
+    return -1;
+}
+int Layer::forward_inplace_hip(HipMat&, HipCommand&, const Option&) const
 {
     return -1;
 }

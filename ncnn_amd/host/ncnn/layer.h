@@ -5,6 +5,7 @@
 #include <string>
 #include <vector>
 
+#include "hipmat.h"
 #include "mat.h"
 #include "modelbin.h"
 #include "option.h"
@@ -37,12 +38,21 @@ public:
     bool support_any_packing;
     bool support_vulkan_any_packing;
     bool support_batch; // takes a Mat with n > 1 whole; otherwise the net loops over samples
+    // forward_hip is implemented: blobs stay in HBM between such layers (the part support_vulkan, src/layer.h:51-52,
+    // plays for the reference's GPU path).  A layer that sets it handles batches (HipMat::n) itself.
+    bool support_hip;
     int featmask;
 
     virtual int forward(const std::vector<Mat>& bottom_blobs, std::vector<Mat>& top_blobs, const Option& opt) const;
     virtual int forward(const Mat& bottom_blob, Mat& top_blob, const Option& opt) const;
     virtual int forward_inplace(std::vector<Mat>& bottom_top_blobs, const Option& opt) const;
     virtual int forward_inplace(Mat& bottom_top_blob, const Option& opt) const;
+
+    // device-resident overloads, same contract as the VkMat overloads of src/layer.h:111-117: inputs and outputs
+    // are blobs in HBM, all work is enqueued on cmd.stream, nothing is synchronised
+    virtual int forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& opt) const;
+    virtual int forward_hip(const HipMat& bottom_blob, HipMat& top_blob, HipCommand& cmd, const Option& opt) const;
+    virtual int forward_inplace_hip(HipMat& bottom_top_blob, HipCommand& cmd, const Option& opt) const;
 
     void* userdata;
     int typeindex;

@@ -4,10 +4,12 @@
 #include <string.h>
 
 #include <map>
+#include <memory>
 #include <string>
 
 #include "datareader.h"
 #include "modelbin.h"
+#include "ncnnhip.h"
 #include "paramdict.h"
 
 namespace ncnn {
@@ -22,6 +24,19 @@ struct CustomEntry
 };
 
 static const int CUSTOM_BIT = 1 << 8; // type indexes of non-built-in custom layers carry this bit
+
+// what one Extractor holds while it runs: every blob as a host Mat, a device HipMat, or both
+struct ExecState
+{
+    std::vector<Mat> host;
+    std::vector<HipMat> dev;
+    std::shared_ptr<HipCommand> cmd; // created on the first layer that runs device-resident
+
+    bool has(int blob) const
+    {
+        return host[(size_t)blob].dims != 0 || !dev[(size_t)blob].empty();
+    }
+};
 
 class NetPrivate
 {
@@ -88,8 +103,9 @@ public:
             delete layer;
     }
 
-    int forward_layer(int layer_index, std::vector<Mat>& blob_mats, const Option& opt) const;
-    int run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const Option& opt) const;
+    int forward_layer(int layer_index, ExecState& st, const Option& opt) const;
+    int run_layer(const Layer* layer, ExecState& st, const Option& opt) const;
+    int run_layer_hip(const Layer* layer, ExecState& st, const Option& opt) const;
 };
 
 // int8 blob -> fp32 blob of the same shape (plain value conversion), batch aware
@@ -117,7 +133,7 @@ static int expand_int8(const Mat& src, Mat& dst, Allocator* allocator)
 
 // ---- executor -----------------------------------------------------------------------------
 
-int NetPrivate::forward_layer(int layer_index, std::vector<Mat>& blob_mats, const Option& opt) const
+int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt) const
 {
     const Layer* layer = layers[layer_index];
     if (layer->bottoms.empty() && layer->type == "Input") return 0; // inputs are fed, not computed
@@ -126,7 +142,7 @@ int NetPrivate::forward_layer(int layer_index, std::vector<Mat>& blob_mats, cons
     for (size_t i = 0; i < layer->bottoms.size(); i++)
     {
         const int bi = layer->bottoms[i];
-        if (blob_mats[bi].dims == 0)
+        if (!st.has(bi))
         {
             const int producer = blobs[bi].producer;
             if (producer < 0)
@@ -134,20 +150,113 @@ int NetPrivate::forward_layer(int layer_index, std::vector<Mat>& blob_mats, cons
                 NCNN_LOGE("blob %s has no producer and was not fed", blobs[bi].name.c_str());
                 return -1;
             }
-            int ret = forward_layer(producer, blob_mats, opt);
+            int ret = forward_layer(producer, st, opt);
             if (ret != 0) return ret;
-            if (blob_mats[bi].dims == 0)
+            if (!st.has(bi))
             {
                 NCNN_LOGE("blob %s was not produced (missing input?)", blobs[bi].name.c_str());
                 return -1;
             }
         }
     }
-    return run_layer(layer, blob_mats, opt);
+    if (opt.use_hip_compute && layer->support_hip) return run_layer_hip(layer, st, opt);
+    return run_layer(layer, st, opt);
 }
 
-int NetPrivate::run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const Option& opt) const
+// A layer with forward_hip: inputs are made device-resident (uploaded once if they only exist on the host), the
+// outputs stay in HBM.  Nothing here waits for the GPU; only an upload out of pageable memory does.
+int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& opt) const
 {
+    if (!st.cmd) st.cmd.reset(new HipCommand);
+    HipCommand& cmd = *st.cmd;
+    int ret = cmd.ensure_ready();
+    if (ret != 0) return ret;
+
+    std::vector<HipMat> ins(layer->bottoms.size());
+    for (size_t i = 0; i < ins.size(); i++)
+    {
+        const size_t bi = (size_t)layer->bottoms[i];
+        if (st.dev[bi].empty())
+        {
+            ret = cmd.upload(st.host[bi], st.dev[bi]);
+            if (ret != 0) return ret;
+        }
+        ins[i] = st.dev[bi];
+        if (opt.lightmode)
+        {
+            st.dev[bi].release();
+            st.host[bi].release();
+        }
+        if (ins[i].elemsize == 1u && !layer->support_int8_storage)
+        {
+            HipMat wide;
+            if (ins[i].dims == 3)
+                wide.create(ins[i].w, ins[i].h, ins[i].c, 4u, ins[i].n, &cmd);
+            else if (ins[i].dims == 2)
+                wide.create(ins[i].w, ins[i].h, 4u, ins[i].n, &cmd);
+            else
+                wide.create(ins[i].w, 4u, ins[i].n, &cmd);
+            if (wide.empty()) return -100;
+            if (ncnnhip_int8_to_f32((const int8_t*)ins[i].data, (float*)wide.data, ins[i].count(), cmd.stream) != 0)
+            {
+                NCNN_LOGE("int8 -> fp32 cast failed: %s", ncnnhip_last_error());
+                return -1;
+            }
+            ins[i] = wide;
+        }
+    }
+
+    if (layer->one_blob_only)
+    {
+        HipMat top;
+        if (layer->support_inplace)
+        {
+            top = ins[0];
+            ins.clear();
+            if (!top.exclusive())
+            {
+                // someone else still reads this blob (a Split sibling, or the table outside light mode)
+                HipMat own;
+                own.create_like(top, &cmd);
+                if (own.empty()) return -100;
+                if (ncnnhip_memcpy_d2d(own.data, top.data, top.bytes(), cmd.stream) != 0) return -1;
+                top = own;
+            }
+            ret = layer->forward_inplace_hip(top, cmd, opt);
+        }
+        else
+            ret = layer->forward_hip(ins[0], top, cmd, opt);
+        if (ret != 0) return ret;
+        st.dev[(size_t)layer->tops[0]] = top;
+        st.host[(size_t)layer->tops[0]].release();
+        return 0;
+    }
+
+    std::vector<HipMat> outs(layer->tops.size());
+    ret = layer->forward_hip(ins, outs, cmd, opt);
+    if (ret != 0) return ret;
+    for (size_t i = 0; i < outs.size(); i++)
+    {
+        st.dev[(size_t)layer->tops[i]] = outs[i];
+        st.host[(size_t)layer->tops[i]].release();
+    }
+    return 0;
+}
+
+int NetPrivate::run_layer(const Layer* layer, ExecState& st, const Option& opt) const
+{
+    std::vector<Mat>& blob_mats = st.host;
+    // a blob that only exists in HBM comes back to the host for a layer without a device overload
+    for (size_t i = 0; i < layer->bottoms.size(); i++)
+    {
+        const size_t bi = (size_t)layer->bottoms[i];
+        if (blob_mats[bi].dims == 0 && !st.dev[bi].empty())
+        {
+            int ret = st.cmd->download(st.dev[bi], blob_mats[bi], opt.blob_allocator);
+            if (ret != 0) return ret;
+        }
+        if (opt.lightmode) st.dev[bi].release();
+    }
     // gather inputs; in light mode a blob is handed over (and dropped from the table) because
     // every blob has exactly one consumer
     std::vector<Mat> ins(layer->bottoms.size());
@@ -218,6 +327,7 @@ int NetPrivate::run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const
             if (ret != 0) return ret;
         }
         blob_mats[layer->tops[0]] = top;
+        st.dev[(size_t)layer->tops[0]].release();
         return 0;
     }
 
@@ -249,7 +359,11 @@ int NetPrivate::run_layer(const Layer* layer, std::vector<Mat>& blob_mats, const
         int ret = layer->forward(ins, outs, opt);
         if (ret != 0) return ret;
     }
-    for (size_t i = 0; i < outs.size(); i++) blob_mats[layer->tops[i]] = outs[i];
+    for (size_t i = 0; i < outs.size(); i++)
+    {
+        blob_mats[layer->tops[i]] = outs[i];
+        st.dev[(size_t)layer->tops[i]].release();
+    }
     return 0;
 }
 
@@ -656,14 +770,15 @@ class ExtractorPrivate
 {
 public:
     const Net* net;
-    std::vector<Mat> blob_mats;
+    ExecState st;
     Option opt;
 };
 
 Extractor::Extractor(const Net* net, size_t blob_count) : d(new ExtractorPrivate)
 {
     d->net = net;
-    d->blob_mats.resize(blob_count);
+    d->st.host.resize(blob_count);
+    d->st.dev.resize(blob_count);
     d->opt = net->opt;
 }
 
@@ -686,7 +801,9 @@ Extractor& Extractor::operator=(const Extractor& rhs)
 
 void Extractor::clear()
 {
-    d->blob_mats.clear();
+    d->st.host.clear();
+    d->st.dev.clear(); // device blobs return to the command's pool before the command itself goes
+    d->st.cmd.reset();
 }
 void Extractor::set_light_mode(bool enable)
 {
@@ -714,8 +831,9 @@ int Extractor::input(const char* blob_name, const Mat& in)
 
 int Extractor::input(int blob_index, const Mat& in)
 {
-    if (blob_index < 0 || blob_index >= (int)d->blob_mats.size()) return -1;
-    d->blob_mats[blob_index] = in;
+    if (blob_index < 0 || blob_index >= (int)d->st.host.size()) return -1;
+    d->st.host[(size_t)blob_index] = in;
+    d->st.dev[(size_t)blob_index].release();
     return 0;
 }
 
@@ -728,15 +846,18 @@ int Extractor::extract(const char* blob_name, Mat& feat, int type)
 
 int Extractor::extract(int blob_index, Mat& feat, int type)
 {
-    if (blob_index < 0 || blob_index >= (int)d->blob_mats.size()) return -1;
+    if (blob_index < 0 || blob_index >= (int)d->st.host.size()) return -1;
+    const size_t bi = (size_t)blob_index;
     int ret = 0;
-    if (d->blob_mats[blob_index].dims == 0)
+    if (!d->st.has(blob_index))
     {
-        const int producer = d->net->d->blobs[blob_index].producer;
+        const int producer = d->net->d->blobs[bi].producer;
         if (producer < 0) return -1;
-        ret = d->net->d->forward_layer(producer, d->blob_mats, d->opt);
+        ret = d->net->d->forward_layer(producer, d->st, d->opt);
     }
-    feat = d->blob_mats[blob_index];
+    if (ret == 0 && d->st.host[bi].dims == 0 && !d->st.dev[bi].empty())
+        ret = d->st.cmd->download(d->st.dev[bi], d->st.host[bi], d->opt.blob_allocator); // waits for the stream
+    feat = d->st.host[bi];
     if (ret == 0 && type == 0 && feat.elemsize == 1u && !feat.empty())
     {
         Mat wide;

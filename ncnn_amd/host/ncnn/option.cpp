@@ -16,6 +16,7 @@ Option::Option()
     use_sgemm_convolution = true;
     use_int8_inference = true;
     use_vulkan_compute = false;
+    use_hip_compute = false;
     use_bf16_storage = false;
     use_fp16_packed = true;
     use_fp16_storage = true;

@@ -23,6 +23,9 @@ public:
     bool use_sgemm_convolution;
     bool use_int8_inference; // gate of the int8 path in Convolution / ConvolutionDepthWise / InnerProduct
     bool use_vulkan_compute;
+    // run layers that implement forward_hip with device-resident blobs (what use_vulkan_compute, src/option.h:84,
+    // switches for the reference's GPU path); off: every layer sees host Mats
+    bool use_hip_compute;
     bool use_bf16_storage;
     bool use_fp16_packed;
     bool use_fp16_storage;

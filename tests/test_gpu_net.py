@@ -15,19 +15,24 @@ def _say(*a):
     print(*a, flush=True)
 
 
-def _load(param, blob):
+RESIDENT = pytest.mark.parametrize("resident", [False, True], ids=["host-blobs", "device-resident"])
+
+
+def _load(param, blob, resident=False):
     net = host.Net()
     assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(resident)  # blobs stay in HBM (channels-last) between layers, or cross the host per layer
     assert net.load_param_mem(param) == 0
     assert net.load_model_mem(blob) == 0
     return net
 
 
-def test_tiny_net_every_blob_matches():
+@RESIDENT
+def test_tiny_net_every_blob_matches(resident):
     g, param, blob, info = zoo.build("tiny")
     x = np.random.default_rng(0).uniform(0, 1, g.input_shape).astype(F)
     ref = refnet.run(param, blob, x)
-    net = _load(param, blob)
+    net = _load(param, blob, resident)
     for name in ("c1", "dw", "pw", "c2", "sum", "relu", "c3", "gap", "fc"):
         ex = net.create_extractor()
         ex.input("data", x)
@@ -41,11 +46,12 @@ def test_tiny_net_every_blob_matches():
     assert np.allclose(ex.extract("prob"), ref["prob"], rtol=1e-6, atol=1e-7)
 
 
-def test_tiny_net_lightmode_off_and_shared_thread_stream():
+@RESIDENT
+def test_tiny_net_lightmode_off_and_shared_thread_stream(resident):
     g, param, blob, info = zoo.build("tiny", seed=3)
     x = np.random.default_rng(1).uniform(0, 1, g.input_shape).astype(F)
     ref = refnet.run(param, blob, x)
-    net = _load(param, blob)
+    net = _load(param, blob, resident)
     net.set_lightmode(False)
     ex = net.create_extractor(own_stream=False)
     ex.input("data", x)
@@ -53,10 +59,11 @@ def test_tiny_net_lightmode_off_and_shared_thread_stream():
     assert np.array_equal(ex.extract("c3"), ref["c3"].astype(F))  # still held with light mode off
 
 
-def test_batch_equals_per_sample():
+@RESIDENT
+def test_batch_equals_per_sample(resident):
     g, param, blob, info = zoo.build("tiny", seed=5)
     xs = np.random.default_rng(2).uniform(0, 1, (3,) + g.input_shape).astype(F)
-    net = _load(param, blob)
+    net = _load(param, blob, resident)
     ex = net.create_extractor()
     ex.input("data", xs)
     got = ex.extract("fc")
@@ -154,14 +161,24 @@ def test_benchmark_network_batch1_matches_oracle_executor(which, hw):
     last_fc = "fc1000" if which == "resnet50" else "fc"
     _say("oracle forward", which)
     ref = refnet.run(param, blob, x, want=last_fc)
-    _say("device forward", which)
-    net = _load(param, blob)
+    for resident in (False, True):
+        _say("device forward", which, "device-resident" if resident else "host blobs")
+        net = _load(param, blob, resident)
+        ex = net.create_extractor()
+        ex.input("data", x)
+        got = ex.extract(last_fc)
+        assert np.array_equal(got, ref[last_fc])
+        # a requantised (int8) blob deep in the net, bit for bit
+        probe = "res4c_branch2b" if which == "resnet50" else "block10_dw"
+        ex = net.create_extractor()
+        ex.input("data", x)
+        assert np.array_equal(ex.extract(probe), ref[probe].astype(F))
+    # batch 2, device-resident: the folded batch equals the per-sample result
+    xs = np.stack([x, x[:, ::-1].copy()])
     ex = net.create_extractor()
-    ex.input("data", x)
+    ex.input("data", xs)
     got = ex.extract(last_fc)
-    assert np.array_equal(got, ref[last_fc])
-    # a requantised (int8) blob deep in the net, bit for bit
-    probe = "res4c_branch2b" if which == "resnet50" else "block10_dw"
-    ex = net.create_extractor()
-    ex.input("data", x)
-    assert np.array_equal(ex.extract(probe), ref[probe].astype(F))
+    assert np.array_equal(got[0].reshape(-1), ref[last_fc])
+    ex1 = net.create_extractor()
+    ex1.input("data", xs[1])
+    assert np.array_equal(got[1].reshape(-1), ex1.extract(last_fc).reshape(-1))
