@@ -198,7 +198,7 @@ def bench_blockquant(args, n, k, m):
     }
 
 
-def bench_net(args, which, batch):
+def bench_layers(args, which, batch):
     """The quantised layers of a ResNet-50 / MobileNetV2-shaped int8 net, each on device-resident synthetic blobs of
     its real shape: fp32 inputs are quantised on the device first, int8 inputs feed the kernel directly, outputs are
     requantised int8 or fp32 exactly as the generated model asks.  One step = one pass over all quantised layers."""
@@ -318,18 +318,69 @@ def bench_net(args, which, batch):
     }
 
 
+def bench_net(args, which, batch):
+    """A whole ResNet-50 / MobileNetV2-shaped int8 model through the product path: generated .param/.bin, Net with the
+    HIP layers registered and use_hip_compute on, one Extractor per inference.  The input batch is uploaded once
+    (resident in HBM, channels-last) before the timed region; a step enqueues every layer of one forward pass and
+    leaves the logits in HBM; the region ends with a stream synchronise."""
+    from ncnn_amd import host, zoo
+    g, param, blob, info = zoo.build(which, n_calib=1)
+    rows = zoo.quantised_layer_table(g)
+    ops = 2.0 * sum(r["macs"] for r in rows) * batch
+    net = host.Net()
+    if net.register_int8_layers() != 0 or net.load_param_mem(param) != 0:
+        raise SystemExit("bench.py: could not load the generated model")
+    net.set_use_hip_compute(True)
+    if net.load_model_mem(blob) != 0:
+        raise SystemExit("bench.py: load_model failed (no GPU?)")
+    out_name = "fc1000" if which == "resnet50" else "fc"
+    x = np.random.default_rng(0).uniform(0, 1, (batch,) + tuple(g.input_shape)).astype(np.float32)
+    xin = net.upload(x)
+
+    def step():
+        ex = net.create_extractor(own_stream=False)
+        ex.input_resident("data", xin)
+        return ex, ex.extract_resident(out_name)
+
+    ex = None
+    for _ in range(args.warmup):
+        ex, out = step()
+    if ex is not None:
+        ex.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ex, out = step()
+    ex.synchronize()
+    wall = time.perf_counter() - t0
+    logits = out.to_numpy()
+    if not np.isfinite(logits).all():
+        raise SystemExit("bench.py: non-finite logits")
+    ms_per_step = wall * 1e3 / args.steps
+    achieved = ops / (ms_per_step * 1e-3) / 1e12
+    return {
+        "metric": "int8 TOPS", "value": achieved, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "%s-shaped int8 model (%d layers, %d quantised), whole forward pass through Net/Extractor with device-resident blobs, batch %d"
+                               % (which, len(g.layers), len(rows), batch),
+                   "images_per_s": batch / (ms_per_step * 1e-3)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
+                     "traffic": None, "kernel": "whole pass (conv_nhwc_kernel dominates)", "ops_per_launch": ops},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
-                    help="gemm<size> | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch>")
+                    help="gemm<size> | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
+                         "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
     ap.add_argument("--b-scale", dest="b_scale", default="per_column", choices=["per_column", "per_tensor"],
                     help="per_column is the benchmark configuration; per_tensor is what ncnn's Gemm layer can express")
     ap.add_argument("--act", default="fp16", choices=["fp16", "fp32"], help="activation type of the block-quant workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--layer-table", default=None, help="net workloads: write the per-layer timing table to this file")
+    ap.add_argument("--layer-table", default=None, help="layers workloads: write the per-layer timing table to this file")
     ap.add_argument("--calib-copy", action="store_true", help="issue one D2D copy of M*K*4 bytes first (calibrates HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -342,6 +393,9 @@ def main():
     elif args.workload.startswith("net:"):
         _, which, batch = args.workload.split(":")
         line = bench_net(args, which, int(batch))
+    elif args.workload.startswith("layers:"):
+        _, which, batch = args.workload.split(":")
+        line = bench_layers(args, which, int(batch))
     else:
         raise SystemExit("unknown workload " + args.workload)
     print(json.dumps(line), flush=True)

@@ -84,6 +84,19 @@ int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* ma
  */
 int ncnnhip_register_int8_layers(ncnn_net_t net);
 
+/* Device-resident ends of an inference (Option::use_hip_compute on): a blob uploaded once with ncnnhip_net_upload feeds any
+ * number of extractors without another copy; ncnnhip_extractor_extract_hipmat enqueues the layers and returns the result
+ * where it lies in HBM without waiting; ncnnhip_extractor_synchronize waits for what the extractor enqueued;
+ * ncnnhip_hipmat_download waits and copies to a host Mat (caller destroys it).  The counterparts in the reference are the
+ * VkMat overloads of Extractor::input / extract (src/net.h:226-239).  Destroy every hipmat before its net. */
+typedef struct __ncnn_hipmat_t* ncnn_hipmat_t;
+int ncnnhip_net_upload(ncnn_net_t net, const ncnn_mat_t mat, ncnn_hipmat_t* out);
+void ncnnhip_hipmat_destroy(ncnn_hipmat_t m);
+int ncnnhip_hipmat_download(const ncnn_hipmat_t m, ncnn_mat_t* out);
+int ncnnhip_extractor_input_hipmat(ncnn_extractor_t ex, const char* name, const ncnn_hipmat_t m);
+int ncnnhip_extractor_extract_hipmat(ncnn_extractor_t ex, const char* name, ncnn_hipmat_t* out);
+int ncnnhip_extractor_synchronize(ncnn_extractor_t ex);
+
 /* Gives the extractor its own device stream and buffer pool (one hipStream per Extractor) by
  * installing a host blob allocator that carries them; the allocator lives until
  * ncnnhip_extractor_detach_stream or process end.  Optional: without it a per-thread stream is used. */

@@ -42,6 +42,9 @@ def lib():
             "ncnn_extractor_create": (vp, [vp]), "ncnn_extractor_destroy": (None, [vp]), "ncnn_extractor_set_option": (None, [vp, vp]),
             "ncnn_extractor_input": (ci, [vp, C.c_char_p, vp]), "ncnn_extractor_extract": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
             "ncnnhip_register_int8_layers": (ci, [vp]), "ncnnhip_extractor_attach_stream": (vp, [vp]), "ncnnhip_extractor_detach_stream": (None, [vp]),
+            "ncnnhip_net_upload": (ci, [vp, vp, C.POINTER(vp)]), "ncnnhip_hipmat_destroy": (None, [vp]), "ncnnhip_hipmat_download": (ci, [vp, C.POINTER(vp)]),
+            "ncnnhip_extractor_input_hipmat": (ci, [vp, C.c_char_p, vp]), "ncnnhip_extractor_extract_hipmat": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
+            "ncnnhip_extractor_synchronize": (ci, [vp]),
             "ncnn_net_get_layer_count": (ci, [vp]), "ncnn_net_get_layer_type": (C.c_char_p, [vp, ci]), "ncnn_net_get_layer_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_layer_flags": (ci, [vp, ci]), "ncnn_net_get_blob_count": (ci, [vp]), "ncnn_net_get_blob_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_blob_producer": (ci, [vp, ci]), "ncnn_net_get_blob_consumer": (ci, [vp, ci]),
@@ -158,9 +161,42 @@ class Mat:
 
 
 # ---- Net / Extractor -------------------------------------------------------------------------------
+class HipMat:
+    """Handle to a device-resident blob (keep the Net alive for as long as this exists)."""
+
+    def __init__(self, handle, net):
+        self.h_ = handle
+        self.net = net
+
+    def __del__(self):
+        try:
+            if self.h_:
+                lib().ncnnhip_hipmat_destroy(self.h_)
+                self.h_ = None
+        except Exception:
+            pass
+
+    def to_numpy(self):
+        out = C.c_void_p()
+        ret = lib().ncnnhip_hipmat_download(self.h_, C.byref(out))
+        m = Mat(out.value)
+        if ret != 0:
+            raise RuntimeError("download returned %d" % ret)
+        return m.to_numpy()
+
+
 class Net:
     def __init__(self):
         self.h_ = lib().ncnn_net_create()
+
+    def upload(self, array):
+        """numpy [c][h][w] / [n][c][h][w] -> device-resident blob usable as input of any extractor of this net."""
+        m = array if isinstance(array, Mat) else Mat.from_numpy(array)
+        out = C.c_void_p()
+        ret = lib().ncnnhip_net_upload(self.h_, m.h_, C.byref(out))
+        if ret != 0:
+            raise RuntimeError("upload returned %d" % ret)
+        return HipMat(out.value, self)
 
     def __del__(self):
         try:
@@ -252,6 +288,21 @@ class Extractor:
         m = array if isinstance(array, Mat) else Mat.from_numpy(array)
         self._inputs.append(m)
         return lib().ncnn_extractor_input(self.h_, name.encode(), m.h_)
+
+    def input_resident(self, name, hipmat):
+        return lib().ncnnhip_extractor_input_hipmat(self.h_, name.encode(), hipmat.h_)
+
+    def extract_resident(self, name):
+        """Enqueue the layers up to `name` and return the result where it lies in HBM, without waiting."""
+        out = C.c_void_p()
+        ret = lib().ncnnhip_extractor_extract_hipmat(self.h_, name.encode(), C.byref(out))
+        m = HipMat(out.value, self.net)
+        if ret != 0:
+            raise RuntimeError("extract_resident(%s) returned %d" % (name, ret))
+        return m
+
+    def synchronize(self):
+        return lib().ncnnhip_extractor_synchronize(self.h_)
 
     def extract(self, name):
         out = C.c_void_p()

@@ -214,6 +214,46 @@ int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* ma
     return ret;
 }
 
+int ncnnhip_net_upload(ncnn_net_t net, const ncnn_mat_t mat, ncnn_hipmat_t* out)
+{
+    HipMat* m = new HipMat;
+    int ret = N(net)->upload(*M(mat), *m);
+    if (ret != 0)
+    {
+        delete m;
+        m = 0;
+    }
+    *out = (ncnn_hipmat_t)m;
+    return ret;
+}
+void ncnnhip_hipmat_destroy(ncnn_hipmat_t m)
+{
+    delete (HipMat*)m;
+}
+int ncnnhip_hipmat_download(const ncnn_hipmat_t m, ncnn_mat_t* out)
+{
+    const HipMat* hm = (const HipMat*)m;
+    Mat host;
+    int ret = (hm && hm->cmd) ? hm->cmd->download(*hm, host, 0) : -1;
+    *out = (ncnn_mat_t) new Mat(host);
+    return ret;
+}
+int ncnnhip_extractor_input_hipmat(ncnn_extractor_t ex, const char* name, const ncnn_hipmat_t m)
+{
+    return E(ex)->input(name, *(const HipMat*)m);
+}
+int ncnnhip_extractor_extract_hipmat(ncnn_extractor_t ex, const char* name, ncnn_hipmat_t* out)
+{
+    HipMat* m = new HipMat;
+    int ret = E(ex)->extract(name, *m);
+    *out = (ncnn_hipmat_t)m;
+    return ret;
+}
+int ncnnhip_extractor_synchronize(ncnn_extractor_t ex)
+{
+    return E(ex)->synchronize();
+}
+
 int ncnnhip_register_int8_layers(ncnn_net_t net)
 {
     using namespace ncnn_amd;

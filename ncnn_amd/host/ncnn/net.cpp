@@ -5,6 +5,7 @@
 
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 
 #include "datareader.h"
@@ -103,6 +104,31 @@ public:
             delete layer;
     }
 
+    // Streams and buffer pools outlive the Extractors that use them: an Extractor takes an idle HipCommand (or a
+    // new one) when its first device-resident layer runs and hands it back when it is cleared, so steady-state
+    // inference allocates nothing.  Work left in flight by the previous user is ordered before the next user's
+    // on the same stream.
+    mutable std::mutex cmd_lock;
+    mutable std::vector<std::shared_ptr<HipCommand> > idle_cmds;
+    mutable std::shared_ptr<HipCommand> io_cmd; // carries blobs uploaded through Net::upload
+
+    std::shared_ptr<HipCommand> acquire_command() const
+    {
+        std::lock_guard<std::mutex> g(cmd_lock);
+        if (!idle_cmds.empty())
+        {
+            std::shared_ptr<HipCommand> c = idle_cmds.back();
+            idle_cmds.pop_back();
+            return c;
+        }
+        return std::shared_ptr<HipCommand>(new HipCommand);
+    }
+    void recycle_command(const std::shared_ptr<HipCommand>& c) const
+    {
+        std::lock_guard<std::mutex> g(cmd_lock);
+        idle_cmds.push_back(c);
+    }
+
     int forward_layer(int layer_index, ExecState& st, const Option& opt) const;
     int run_layer(const Layer* layer, ExecState& st, const Option& opt) const;
     int run_layer_hip(const Layer* layer, ExecState& st, const Option& opt) const;
@@ -167,7 +193,7 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
 // outputs stay in HBM.  Nothing here waits for the GPU; only an upload out of pageable memory does.
 int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& opt) const
 {
-    if (!st.cmd) st.cmd.reset(new HipCommand);
+    if (!st.cmd) st.cmd = acquire_command();
     HipCommand& cmd = *st.cmd;
     int ret = cmd.ensure_ready();
     if (ret != 0) return ret;
@@ -716,11 +742,23 @@ void Net::clear()
     d->output_idx.clear();
     d->input_nm.clear();
     d->output_nm.clear();
+    std::lock_guard<std::mutex> g(d->cmd_lock);
+    d->idle_cmds.clear();
+    d->io_cmd.reset();
 }
 
 Extractor Net::create_extractor() const
 {
     return Extractor(this, d->blobs.size());
+}
+
+int Net::upload(const Mat& src, HipMat& dst) const
+{
+    {
+        std::lock_guard<std::mutex> g(d->cmd_lock);
+        if (!d->io_cmd) d->io_cmd.reset(new HipCommand);
+    }
+    return d->io_cmd->upload(src, dst);
 }
 
 const std::vector<int>& Net::input_indexes() const
@@ -802,7 +840,8 @@ Extractor& Extractor::operator=(const Extractor& rhs)
 void Extractor::clear()
 {
     d->st.host.clear();
-    d->st.dev.clear(); // device blobs return to the command's pool before the command itself goes
+    d->st.dev.clear(); // device blobs return to the command's pool before the command itself moves on
+    if (d->st.cmd && d->st.cmd.use_count() == 1) d->net->d->recycle_command(d->st.cmd);
     d->st.cmd.reset();
 }
 void Extractor::set_light_mode(bool enable)
@@ -835,6 +874,54 @@ int Extractor::input(int blob_index, const Mat& in)
     d->st.host[(size_t)blob_index] = in;
     d->st.dev[(size_t)blob_index].release();
     return 0;
+}
+
+int Extractor::input(const char* blob_name, const HipMat& in)
+{
+    const int bi = d->net->find_blob_index_by_name(blob_name);
+    if (bi < 0) return -1;
+    return input(bi, in);
+}
+
+int Extractor::input(int blob_index, const HipMat& in)
+{
+    if (blob_index < 0 || blob_index >= (int)d->st.dev.size()) return -1;
+    d->st.dev[(size_t)blob_index] = in;
+    d->st.host[(size_t)blob_index].release();
+    return 0;
+}
+
+int Extractor::extract(const char* blob_name, HipMat& feat)
+{
+    const int bi = d->net->find_blob_index_by_name(blob_name);
+    if (bi < 0) return -1;
+    return extract(bi, feat);
+}
+
+int Extractor::extract(int blob_index, HipMat& feat)
+{
+    if (blob_index < 0 || blob_index >= (int)d->st.dev.size()) return -1;
+    const size_t bi = (size_t)blob_index;
+    int ret = 0;
+    if (!d->st.has(blob_index))
+    {
+        const int producer = d->net->d->blobs[bi].producer;
+        if (producer < 0) return -1;
+        ret = d->net->d->forward_layer(producer, d->st, d->opt);
+    }
+    if (ret == 0 && d->st.dev[bi].empty())
+    {
+        // produced by a layer without a device overload
+        if (!d->st.cmd) d->st.cmd = d->net->d->acquire_command();
+        ret = d->st.cmd->upload(d->st.host[bi], d->st.dev[bi]);
+    }
+    feat = d->st.dev[bi];
+    return ret;
+}
+
+int Extractor::synchronize()
+{
+    return d->st.cmd ? d->st.cmd->synchronize() : 0;
 }
 
 int Extractor::extract(const char* blob_name, Mat& feat, int type)

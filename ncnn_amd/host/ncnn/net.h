@@ -46,6 +46,10 @@ public:
 
     Extractor create_extractor() const;
 
+    // host Mat -> device-resident blob that any Extractor of this net accepts as an input (the copy has completed
+    // on return).  The blob's memory belongs to the net: release it before the net is cleared or destroyed.
+    int upload(const Mat& src, HipMat& dst) const;
+
     const std::vector<int>& input_indexes() const;
     const std::vector<int>& output_indexes() const;
     const std::vector<const char*>& input_names() const;
@@ -83,6 +87,15 @@ public:
     // type 0: int8 results are expanded to fp32; type 1: returned as stored
     int extract(const char* blob_name, Mat& feat, int type = 0);
     int extract(int blob_index, Mat& feat, int type = 0);
+
+    // device-resident ends of the pipeline (the VkMat overloads of src/net.h:226-239): a blob that is already in
+    // HBM goes in without a copy; extract enqueues the work and hands back the blob where it lies, without waiting.
+    // synchronize() waits for everything this Extractor has enqueued.
+    int input(const char* blob_name, const HipMat& in);
+    int input(int blob_index, const HipMat& in);
+    int extract(const char* blob_name, HipMat& feat);
+    int extract(int blob_index, HipMat& feat);
+    int synchronize();
 
 protected:
     friend Extractor Net::create_extractor() const;
