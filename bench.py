@@ -199,9 +199,10 @@ def bench_blockquant(args, n, k, m):
 
 
 def bench_layers(args, which, batch):
-    """The quantised layers of a ResNet-50 / MobileNetV2-shaped int8 net, each on device-resident synthetic blobs of
-    its real shape: fp32 inputs are quantised on the device first, int8 inputs feed the kernel directly, outputs are
-    requantised int8 or fp32 exactly as the generated model asks.  One step = one pass over all quantised layers."""
+    """The quantised layers of a ResNet-50 / MobileNetV2-shaped int8 net, each alone through the C ABI on device-resident
+    channels-last blobs of its real shape (the form the layers see inside a running net): fp32 inputs are quantised
+    first, int8 inputs feed the kernel directly, outputs are requantised int8 or fp32 as the generated model asks.
+    One step = one pass over all quantised layers; the table lists each layer's time with and without its quantise pass."""
     import ncnn_amd
     from ncnn_amd.hip import Activation, ConvDesc, check, lib as load
     from ncnn_amd import zoo
@@ -211,6 +212,7 @@ def bench_layers(args, which, batch):
     g = getattr(zoo, which)()
     rows = zoo.quantised_layer_table(g)
     rng = np.random.default_rng(0)
+    cp = lib.ncnnhip_padded_channels
     plans = []
     for r in rows:
         if r["type"] == "InnerProduct":
@@ -223,50 +225,48 @@ def bench_layers(args, which, batch):
         else:
             c, h, w = r["in_shape"]
             cout, oh, ow = r["out_shape"]
-            cstep = (h * w + 15) // 16 * 16
-            ocs = (oh * ow + (15 if r["int8_out"] else 3)) // (16 if r["int8_out"] else 4) * (16 if r["int8_out"] else 4)
             desc = ConvDesc(w, h, c, batch, cout, r["k"], r["k"], 1, 1, r["stride"], r["stride"], r["pad"], r["pad"], r["pad"], r["pad"], 0.0, r["group"])
-            plan = dict(row=r, kind="conv", desc=desc, cstep=cstep, ocs=ocs,
-                        d_xq=rt.up(rng.integers(-127, 128, (batch, c, cstep)).astype(np.int8)),
-                        d_w=rt.up(rng.integers(-127, 128, cout * (c // r["group"]) * r["k"] * r["k"]).astype(np.int8)),
+            plan = dict(row=r, kind="conv", desc=desc, npix=batch * h * w,
+                        d_xq=rt.up(rng.integers(-127, 128, (batch, h * w, cp(c))).astype(np.int8)),
                         d_si=rt.up(rng.uniform(1e-4, 1e-3, cout).astype(np.float32)), d_b=rt.up(rng.uniform(-0.1, 0.1, cout).astype(np.float32)),
                         d_so=rt.up(np.full(cout, 20.0, np.float32)) if r["int8_out"] else None,
-                        d_out=ncnn_amd.DeviceBuffer.empty((batch, cout, ocs), np.int8 if r["int8_out"] else np.float32),
+                        d_out=ncnn_amd.DeviceBuffer.empty((batch, oh * ow, cp(cout)), np.int8 if r["int8_out"] else np.float32),
                         act=Activation.make(r["act"], r["act_params"]))
             if not r["int8_in"]:
-                plan["d_x"] = rt.up(rng.uniform(-1, 1, (batch, c, h * w)).astype(np.float32))
+                plan["d_x"] = rt.up(rng.uniform(-1, 1, (batch, h * w, cp(c))).astype(np.float32))
                 plan["d_s"] = rt.up(np.array([100.0], np.float32))
+            taps = r["k"] * r["k"]
             if r["group"] == 1:
-                # channels-last path: weights packed once (as create_pipeline does), activations transposed per step
                 nb, wb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
                 check(lib.ncnnhip_conv_nhwc_sizes(C.byref(desc), C.byref(nb), C.byref(wb), C.byref(sb)))
-                wq = rng.integers(-127, 128, cout * c * r["k"] * r["k"]).astype(np.int8)
+                wq = rng.integers(-127, 128, cout * c * taps).astype(np.int8)
                 pk = np.empty(wb.value, np.int8)
                 check(lib.ncnnhip_conv_pack_weights(C.byref(desc), wq.ctypes.data, pk.ctypes.data))
-                plan.update(d_pk=rt.up(pk), d_nhwc=ncnn_amd.DeviceBuffer(nb.value), d_ws=ncnn_amd.DeviceBuffer(max(sb.value, 4)), ws_bytes=sb.value)
+                plan.update(d_pk=rt.up(pk), d_ws=ncnn_amd.DeviceBuffer(max(sb.value, 4)), ws_bytes=sb.value)
+            else:
+                assert r["group"] == c == cout, "the benchmark nets only hold plain and depthwise convolutions"
+                wq = rng.integers(-127, 128, c * taps).astype(np.int8)
+                pk = np.empty(taps * cp(c), np.int8)
+                check(lib.ncnnhip_dwconv_pack_weights(c, taps, wq.ctypes.data, pk.ctypes.data))
+                plan.update(d_pk=rt.up(pk))
         plans.append(plan)
 
-    def run_layer(p):
+    def run_layer(p, prepass=True):
         r = p["row"]
         if p["kind"] == "fc":
-            check(lib.ncnnhip_quantize(p["d_x"].ptr, p["k"], 0, p["d_xq"].ptr, p["k"], 0, batch, p["k"], 1, p["d_s"].ptr, 1, st))
+            if prepass:
+                check(lib.ncnnhip_quantize(p["d_x"].ptr, p["k"], 0, p["d_xq"].ptr, p["k"], 0, batch, p["k"], 1, p["d_s"].ptr, 1, st))
             check(lib.ncnnhip_innerproduct_int8(p["d_xq"].ptr, p["k"], batch, p["k"], p["n"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
                                                 Activation.make(0), p["d_out"].ptr, p["n"], None, st))
             return
-        c, h, w = r["in_shape"]
+        if prepass and not r["int8_in"]:
+            check(lib.ncnnhip_quantize_nhwc(p["d_x"].ptr, p["d_xq"].ptr, p["npix"], r["in_shape"][0], p["d_s"].ptr, 1, st))
+        so = p["d_so"].ptr if p["d_so"] else None
         if r["group"] == 1:
-            if r["int8_in"]:
-                check(lib.ncnnhip_to_nhwc_int8(C.byref(p["desc"]), p["d_xq"].ptr, 1, p["cstep"], c * p["cstep"], None, 1, p["d_nhwc"].ptr, st))
-            else:
-                check(lib.ncnnhip_to_nhwc_int8(C.byref(p["desc"]), p["d_x"].ptr, 4, h * w, c * h * w, p["d_s"].ptr, 1, p["d_nhwc"].ptr, st))
-            check(lib.ncnnhip_conv_int8_nhwc(C.byref(p["desc"]), p["d_nhwc"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr,
-                                             p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, 0, p["ocs"], r["out_shape"][0] * p["ocs"],
-                                             p["d_ws"].ptr, p["ws_bytes"], st))
-            return
-        if not r["int8_in"]:
-            check(lib.ncnnhip_quantize(p["d_x"].ptr, h * w, c * h * w, p["d_xq"].ptr, p["cstep"], c * p["cstep"], c, h * w, batch, p["d_s"].ptr, 1, st))
-        check(lib.ncnnhip_conv_int8(C.byref(p["desc"]), p["d_xq"].ptr, p["cstep"], c * p["cstep"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
-                                    p["d_so"].ptr if p["d_so"] else None, p["act"], p["d_out"].ptr, p["ocs"], r["out_shape"][0] * p["ocs"], None, st))
+            check(lib.ncnnhip_conv_int8_nhwc(C.byref(p["desc"]), p["d_xq"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr, so, p["act"], p["d_out"].ptr,
+                                             1, 0, 0, p["d_ws"].ptr, p["ws_bytes"], st))
+        else:
+            check(lib.ncnnhip_dwconv_int8_nhwc(C.byref(p["desc"]), p["d_xq"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr, so, p["act"], p["d_out"].ptr, st))
 
     def step():
         for p in plans:
@@ -275,19 +275,26 @@ def bench_layers(args, which, batch):
     for _ in range(args.warmup):
         step()
     rt.sync()
-    # per-layer times (back-to-back launches of one layer)
-    table = []
-    for p in plans:
+
+    def timed(p, prepass, reps=10):
         ev = _events(lib, check, 2)
-        reps = 10
         check(lib.ncnnhip_event_record(ev[0], st))
         for _ in range(reps):
-            run_layer(p)
+            run_layer(p, prepass)
         check(lib.ncnnhip_event_record(ev[1], st))
         check(lib.ncnnhip_event_synchronize(ev[1]))
-        us = _elapsed(lib, check, ev[0], ev[1]) * 1e3 / reps
+        return _elapsed(lib, check, ev[0], ev[1]) * 1e3 / reps
+
+    table = []
+    for p in plans:
         r = p["row"]
-        table.append((r["name"], r["type"], r["in_shape"], r["out_shape"], r["k"], r["stride"], r["group"], 2.0 * r["macs"] * batch, us))
+        us, us_kernel = timed(p, True), timed(p, False)
+        cin, cout = r["in_shape"][0], r["out_shape"][0]
+        in_px = batch * r["in_shape"][1] * r["in_shape"][2] if len(r["in_shape"]) == 3 else batch
+        out_px = batch * r["out_shape"][1] * r["out_shape"][2] if len(r["out_shape"]) == 3 else batch
+        # bytes the layer has to move at least once: int8 input, weights, output as stored
+        nbytes = in_px * cin + r["macs"] // max(out_px // batch, 1) + out_px * cout * (1 if r.get("int8_out") else 4)
+        table.append((r["name"], r["type"], r["in_shape"], r["out_shape"], r["k"], r["stride"], r["group"], 2.0 * r["macs"] * batch, us, us_kernel, nbytes))
     evs = _events(lib, check, 2)
     check(lib.ncnnhip_device_synchronize())
     t0 = time.perf_counter()
@@ -302,19 +309,22 @@ def bench_layers(args, which, batch):
     ms_per_step = wall * 1e3 / args.steps
     if args.layer_table:
         with open(args.layer_table, "w") as f:
-            f.write("%-22s %-22s %-18s %-18s k s group %12s %10s %10s\n" % ("layer", "type", "in", "out", "ops", "us", "TOPS"))
+            f.write("%-22s %-22s %-18s %-18s k s group %12s %9s %9s %8s %8s\n" % ("layer", "type", "in", "out", "ops", "us", "us_kernel", "TOPS", "GB/s"))
             for t in sorted(table, key=lambda t: -t[8]):
-                f.write("%-22s %-22s %-18s %-18s %d %d %5d %12.0f %10.2f %10.2f\n" % (t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[7] / t[8] / 1e6))
-            f.write("sum of per-layer times %.1f us; whole pass %.1f us (device events)\n" % (sum(t[8] for t in table), dev_ms * 1e3))
+                f.write("%-22s %-22s %-18s %-18s %d %d %5d %12.0f %9.2f %9.2f %8.2f %8.0f\n"
+                        % (t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9], t[7] / t[9] / 1e6, t[10] / t[9] / 1e3))
+            f.write("sum of per-layer times %.1f us (kernels alone %.1f us); whole pass %.1f us (device events)\n"
+                    % (sum(t[8] for t in table), sum(t[9] for t in table), dev_ms * 1e3))
     worst = max(table, key=lambda t: t[8])
     achieved = ops / (dev_ms * 1e-3) / 1e12
     return {
         "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "%s-shaped int8 net, the %d quantised layers (conv/depthwise/fc) on resident blobs, batch %d" % (which, len(plans), batch),
+        "config": {"workload": "%s-shaped int8 net, the %d quantised layers (conv/depthwise/fc) one by one on channels-last resident blobs, batch %d"
+                               % (which, len(plans), batch),
                    "images_per_s": batch / (ms_per_step * 1e-3), "slowest_layer": [worst[0], worst[8]]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": None, "kernel": "conv_tile_kernel (all layers of the pass)", "ops_per_launch": ops},
+                     "traffic": None, "kernel": "conv_nhwc_kernel (all layers of the pass)", "ops_per_launch": ops},
     }
 
 

@@ -1,0 +1,32 @@
+// Shared between the two channels-last convolution kernels (conv_nhwc.hip: any border value, planar or
+// channels-last output; conv_nhwc_pipelined.hip: zero border, channels-last output, direct-to-LDS pipeline).
+#ifndef NCNNHIP_CONV_NHWC_H
+#define NCNNHIP_CONV_NHWC_H
+
+#include "epilogues.h"
+
+namespace ncnnhip {
+
+struct NhwcGeom
+{
+    int H, W, Cp;
+    int kw, kh, dw, dh, sw, sh;
+    int pad_top, pad_left;
+    int outw, outh;
+    int npix;   // batch * outh * outw
+    int ntaps;  // kh * kw
+    int K;      // ntaps * Cp rounded up to 64
+    int cout;
+    int pad_word; // border byte replicated 4x
+};
+
+// int32 words of split-K scratch the pipelined kernel wants for this problem (0: it does not split)
+size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps);
+
+// Launches the pipelined kernel; the caller has checked: zero border byte, channels-last output.
+int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, void* workspace,
+                               size_t workspace_bytes, hipStream_t stream);
+
+} // namespace ncnnhip
+
+#endif // NCNNHIP_CONV_NHWC_H

@@ -12,23 +12,10 @@
 // and written to the other LDS buffer afterwards (one barrier per step).  Layers with few output pixels
 // (ResNet tail at batch 1) split K over blockIdx.z: partial int32 sums are added atomically into a zeroed
 // workspace -- integer addition, so the result is still exact -- and a second small kernel applies the epilogue.
-#include "epilogues.h"
+#include "conv_nhwc.h"
 #include "mfma_tile.h"
 
 namespace ncnnhip {
-
-struct NhwcGeom
-{
-    int H, W, Cp;
-    int kw, kh, dw, dh, sw, sh;
-    int pad_top, pad_left;
-    int outw, outh;
-    int npix;   // batch * outh * outw
-    int ntaps;  // kh * kw
-    int K;      // ntaps * Cp rounded up to 64
-    int cout;
-    int pad_word; // border byte replicated 4x
-};
 
 __device__ __forceinline__ uint32_t pack4b(int a, int b, int c, int d)
 {
@@ -411,7 +398,10 @@ int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, s
     {
         const long long npix = (long long)desc->batch * outw * outh;
         const SplitPlan p = plan_launch(desc->num_output, npix, packed_k(*desc) / 64);
-        *workspace_bytes = p.splits > 1 ? (size_t)padded_channels(desc->num_output) * npix * sizeof(int32_t) : 0;
+        size_t words = p.splits > 1 ? (size_t)padded_channels(desc->num_output) * npix : 0;
+        const size_t words_pipelined = conv_nhwc_pipelined_workspace_words(desc->num_output, npix, packed_k(*desc) / 64);
+        if (words_pipelined > words) words = words_pipelined;
+        *workspace_bytes = words * sizeof(int32_t);
     }
     return NCNNHIP_OK;
 }
@@ -499,8 +489,10 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
     epi.num_output = d.num_output;
     epi.acc_out = 0;
 
-    const SplitPlan p = plan_launch(d.num_output, npix, g.K / 64);
     hipStream_t st = as_stream(stream);
+    // zero border and channels-last output: the pipelined kernel
+    if (clast && pb == 0) return launch_conv_nhwc_pipelined(g, packed_weight_dev, nhwc_dev, epi, out_cp, workspace_dev, workspace_bytes, st);
+    const SplitPlan p = plan_launch(d.num_output, npix, g.K / 64);
     dim3 grid(ceil_div(npix, p.bn), ceil_div(d.num_output, p.bm), p.splits);
     NCNNHIP_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ncnnhip_conv_int8_nhwc: grid too large");
     int32_t* partial = 0;

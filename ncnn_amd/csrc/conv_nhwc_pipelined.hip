@@ -1,0 +1,374 @@
+// int8 Convolution (group 1, zero border) on channels-last blobs, pipelined for the gfx950 matrix cores.
+//
+// GEMM view: D[pixel][channel] = sum_k X[pixel][k] * W[channel][k], k = (tap, input channel), both operands
+// K-contiguous.  Pixels are the A operand and output channels the B operand of v_mfma_i32_32x32x32_i8, so a lane's
+// accumulators are 16 pixels of ONE output channel: its scale, bias and requantisation factor are loaded once, and a
+// wavefront store covers 32 consecutive channels of a pixel (128 contiguous bytes of an fp32 channels-last blob).
+//
+// One workgroup (4 wavefronts, 2x2) owns BM pixels x BN channels.  K is walked in 64-byte steps through a ring of
+// LDS stages filled by direct global->LDS 16-byte loads, STAGES-1 steps ahead of the step being multiplied.  A
+// stage holds [BM + BN rows][64 bytes]; the four 16-byte chunks of row r sit at position c ^ ((r >> 2) & 3) so
+// that the 128-bit fragment reads of 16 consecutive rows spread over all banks; the swizzle is applied by choosing
+// which source chunk a lane fetches.  The im2col gather is that choice of source address: (pixel, tap, 16
+// channels) is one aligned 16-byte word of the blob, or -- outside the image, beyond the last tap, beyond the last
+// pixel -- a line of zeros.
+//
+// Workgroup ids are dealt round-robin to the 8 XCDs; they are remapped so that an XCD works on consecutive tiles
+// (channel tiles of one pixel tile are neighbours and share the activations in that XCD's L2).
+// Small problems split K over workgroups: partial int32 sums are added into a zeroed [pixel][channel] scratch with
+// coalesced atomics (integer addition: exact in any order) and a second kernel applies the epilogue.
+#include <type_traits>
+
+#include "conv_nhwc.h"
+#include "mfma_tile.h"
+
+#define AS1 __attribute__((address_space(1)))
+#define AS3 __attribute__((address_space(3)))
+#define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
+
+namespace ncnnhip {
+
+__device__ __attribute__((aligned(64))) int8_t g_zero_line[64];
+
+template<int BM, int BN, int STAGES, bool SPLITK>
+__global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
+                                                                   int out_cp, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
+{
+    constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
+    constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
+    constexpr int STAGE_BYTES = (BM + BN) * 64;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[STAGES * STAGE_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    // ---- which tile: XCD x gets the x-th contiguous share of the tile list
+    int b = blockIdx.x;
+    {
+        const int T = gridDim.x, xcd = b & 7, idx = b >> 3, rem = T & 7;
+        b = xcd * (T >> 3) + (xcd < rem ? xcd : rem) + idx;
+    }
+    const int tn = b % tiles_n;
+    const int rest = b / tiles_n;
+    const int tm = rest % tiles_m;
+    const int split = rest / tiles_m;
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int total_steps = g.K / 64;
+    const int step_begin = SPLITK ? split * steps_per_split : 0;
+    int step_end = SPLITK ? step_begin + steps_per_split : total_steps;
+    if (step_end > total_steps) step_end = total_steps;
+    const int nk = step_end - step_begin;
+    if (nk <= 0) return;
+
+    // ---- sources of this lane's loads.  Load i of a wavefront fills LDS rows i*64 + wave*16 .. +16 of the operand;
+    // the lane's row is +lane/4 and it fetches source chunk (lane&3) ^ ((lane>>4)&3) into position lane&3.
+    const int ld_row = wave * 16 + (lane >> 2);
+    const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int8_t* zero = g_zero_line;
+
+    const int8_t* a_base[LA];
+    int a_iy0[LA], a_ix0[LA];
+#pragma unroll
+    for (int i = 0; i < LA; i++)
+    {
+        const int n = row0 + i * 64 + ld_row;
+        const bool ok = n < g.npix;
+        const int nn = ok ? n : 0;
+        const int plane = g.outw * g.outh;
+        const int img = nn / plane;
+        const int rem = nn - img * plane;
+        const int oy = rem / g.outw;
+        const int ox = rem - oy * g.outw;
+        // a pixel beyond the end gets coordinates that fail every bounds test
+        a_iy0[i] = ok ? oy * g.sh - g.pad_top : -0x40000000;
+        a_ix0[i] = ox * g.sw - g.pad_left;
+        a_base[i] = x + (size_t)img * g.H * g.W * g.Cp;
+    }
+    const int8_t* b_ptr[LB];
+#pragma unroll
+    for (int i = 0; i < LB; i++)
+    {
+        int ch = col0 + i * 64 + ld_row;
+        if (ch >= g.cout) ch = g.cout - 1; // a valid row; its products land in columns nobody stores
+        b_ptr[i] = wpk + (size_t)ch * g.K + (size_t)step_begin * 64 + ld_chunk * 16;
+    }
+    // this lane's position in K: tap (ky,kx) and first channel q0 of its 16-byte chunk; +64 bytes per stage issued
+    int q0, ky, kx, tap;
+    {
+        const int k = step_begin * 64 + ld_chunk * 16;
+        tap = k / g.Cp;
+        q0 = k - tap * g.Cp;
+        ky = tap / g.kw;
+        kx = tap - ky * g.kw;
+    }
+
+    // issues the loads of the next stage in sequence (s = 0, 1, 2, ... relative to step_begin)
+    auto issue = [&](int s) {
+        int8_t* stage = smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
+        const int dy = ky * g.dh, dx = kx * g.dw;
+        const bool tap_ok = tap < g.ntaps;
+#pragma unroll
+        for (int i = 0; i < LA; i++)
+        {
+            const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+            const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+            const int8_t* src = in ? a_base[i] + ((size_t)iy * g.W + ix) * g.Cp + q0 : zero;
+            __builtin_amdgcn_global_load_lds((const AS1 void*)src, (AS3 void*)(stage + i * 4096), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; i++)
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(b_ptr[i] + (size_t)s * 64), (AS3 void*)(stage + BM * 64 + i * 4096), 16, 0, 0);
+        q0 += 64;
+        while (q0 >= g.Cp)
+        {
+            q0 -= g.Cp;
+            tap++;
+            if (++kx == g.kw)
+            {
+                kx = 0;
+                ky++;
+            }
+        }
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][c][r] = 0;
+
+    // fragment read offsets inside a stage: row l32 of each 32-row block, K chunk ks*2 + lhi, swizzled
+    const int sw = (l32 >> 2) & 3;
+    const unsigned lds_base = (unsigned)(uintptr_t)(AS3 int8_t*)smem;
+    const unsigned rd_a = (unsigned)((wm * (BM / 2) + l32) * 64);
+    const unsigned rd_b = (unsigned)(BM * 64 + (wn * (BN / 2) + l32) * 64);
+    const unsigned ch0 = (unsigned)(((0 + lhi) ^ sw) * 16), ch1 = (unsigned)(((2 + lhi) ^ sw) * 16);
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; s++)
+        if (s < nk) issue(s);
+
+    for (int t = 0; t < nk; t++)
+    {
+        // this wavefront's loads of step t have landed (later stages may stay in flight) ...
+        const int ahead = nk - 1 - t < STAGES - 2 ? nk - 1 - t : STAGES - 2;
+        if (STAGES >= 4 && ahead == 2)
+            WAIT_VMCNT(2 * (LA + LB));
+        else if (ahead == 1)
+            WAIT_VMCNT(LA + LB);
+        else
+            WAIT_VMCNT(0);
+        // ... and everybody's: the barrier also says nobody still reads the stage refilled next
+        __builtin_amdgcn_s_barrier();
+        if (t + STAGES - 1 < nk) issue(t + STAGES - 1);
+
+        const unsigned st = lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+        {
+            v4i fa[TM], fb[TN];
+            const unsigned chunk = ks ? ch1 : ch0;
+#pragma unroll
+            for (int a = 0; a < TM; a++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[a]) : "v"(st + rd_a + chunk + (unsigned)(a * 32 * 64)));
+#pragma unroll
+            for (int c = 0; c < TN; c++) asm volatile("ds_read_b128 %0, %1" : "=v"(fb[c]) : "v"(st + rd_b + chunk + (unsigned)(c * 32 * 64)));
+            // the reads are asm, so the wait is too; passing each fragment through an (empty) volatile asm after it
+            // keeps the MFMAs, which consume those values, below the wait
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int a = 0; a < TM; a++) asm volatile("" : "+v"(fa[a]));
+#pragma unroll
+            for (int c = 0; c < TN; c++) asm volatile("" : "+v"(fb[c]));
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int c = 0; c < TN; c++) acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a], fb[c], acc[a][c], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: lane = one output channel per 32-column block, registers = pixels
+    if (SPLITK)
+    {
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+        {
+            const int ch = col0 + wn * (BN / 2) + c * 32 + l32;
+            if (ch >= g.cout) continue;
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                {
+                    const int pix = row0 + wm * (BM / 2) + a * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    if (pix < g.npix) atomicAdd(partial + (size_t)pix * out_cp + ch, acc[a][c][r]);
+                }
+        }
+        return;
+    }
+    // the activation type is uniform: branch on it once, outside the unrolled stores
+    auto finish = [&](auto act_tag) {
+        constexpr int ACT = decltype(act_tag)::value;
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+        {
+            const int ch = col0 + wn * (BN / 2) + c * 32 + l32;
+            if (ch >= out_cp) continue;
+            const bool real = ch < g.cout; // channels from cout up to out_cp are the blob's zero padding
+            const float s_in = real ? epi.scale_in[ch] : 0.f;
+            const float bias = (real && epi.bias) ? epi.bias[ch] : 0.f;
+            const float s_out = (real && epi.scale_out) ? epi.scale_out[ch] : 0.f;
+#pragma unroll
+            for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                {
+                    const int pix = row0 + wm * (BM / 2) + a * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    if (pix >= g.npix) continue;
+                    float f = mul_rn((float)acc[a][c][r], s_in);
+                    if (epi.bias) f = add_rn(f, bias);
+                    if (ACT == 1)
+                        f = fmaxf(f, 0.f);
+                    else if (ACT == 3)
+                    {
+                        if (f < epi.act.p0) f = epi.act.p0;
+                        if (f > epi.act.p1) f = epi.act.p1;
+                    }
+                    else if (ACT != 0)
+                        f = apply_activation(f, epi.act);
+                    if (!real) f = 0.f;
+                    const size_t o = (size_t)pix * out_cp + ch;
+                    if (epi.scale_out)
+                        static_cast<int8_t*>(epi.out)[o] = (int8_t)float2int8(mul_rn(f, s_out));
+                    else
+                        static_cast<float*>(epi.out)[o] = f;
+                }
+        }
+    };
+    if (epi.act.type == 0)
+        finish(std::integral_constant<int, 0>{});
+    else if (epi.act.type == 1)
+        finish(std::integral_constant<int, 1>{});
+    else if (epi.act.type == 3)
+        finish(std::integral_constant<int, 3>{});
+    else
+        finish(std::integral_constant<int, -1>{});
+}
+
+// partial sums [npix][out_cp] -> epilogue; one thread per (pixel, channel), channels fastest
+__global__ __launch_bounds__(256) void conv_pipelined_finish_kernel(const int32_t* __restrict__ partial, int npix, int out_cp, int cout, ConvEpilogue epi)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)npix * out_cp) return;
+    const int ch = (int)(i % (size_t)out_cp);
+    const bool real = ch < cout;
+    float f = 0.f;
+    if (real)
+    {
+        f = mul_rn((float)partial[i], epi.scale_in[ch]);
+        if (epi.bias) f = add_rn(f, epi.bias[ch]);
+        f = apply_activation(f, epi.act);
+    }
+    if (epi.scale_out)
+        static_cast<int8_t*>(epi.out)[i] = real ? (int8_t)float2int8(mul_rn(f, epi.scale_out[ch])) : (int8_t)0;
+    else
+        static_cast<float*>(epi.out)[i] = f;
+}
+
+__global__ __launch_bounds__(256) void zero_words_kernel(int32_t* p, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+struct PipePlan
+{
+    int bm, bn, tiles_m, tiles_n, splits, steps_per_split;
+};
+
+static PipePlan plan_pipelined(int cout, long long npix, int steps)
+{
+    PipePlan p;
+    // channel tile: the whole channel count in one tile when it fits (activations are then read once), else the
+    // width that pads least
+    if (cout <= 64)
+        p.bn = 64;
+    else if (cout <= 128)
+        p.bn = 128;
+    else
+        p.bn = (ceil_div(cout, 256) * 256 <= ceil_div(cout, 128) * 128) ? 256 : 128;
+    p.bm = 128;
+    auto tiles = [&]() { return (long long)ceil_div(npix, p.bm) * ceil_div(cout, p.bn); };
+    if (tiles() < 512) p.bm = 64;
+    if (tiles() < 256 && p.bn == 256) p.bn = 128;
+    if (tiles() < 256 && p.bn == 128 && cout > 64) p.bn = 64;
+    p.tiles_m = ceil_div(npix, p.bm);
+    p.tiles_n = ceil_div(cout, p.bn);
+    p.splits = 1;
+    const long long t = tiles();
+    if (t < 192 && steps >= 8)
+    {
+        const int want = (int)((384 + t - 1) / t);
+        const int max_splits = steps / 4; // at least 4 K steps per split
+        p.splits = want < max_splits ? want : max_splits;
+        if (p.splits < 1) p.splits = 1;
+    }
+    p.steps_per_split = ceil_div(steps, p.splits);
+    p.splits = ceil_div(steps, p.steps_per_split);
+    return p;
+}
+
+size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps)
+{
+    const PipePlan p = plan_pipelined(cout, npix, steps);
+    return p.splits > 1 ? (size_t)npix * ((cout + 15) / 16 * 16) : 0;
+}
+
+int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, void* workspace,
+                               size_t workspace_bytes, hipStream_t stream)
+{
+    const PipePlan p = plan_pipelined(g.cout, g.npix, g.K / 64);
+    const long long blocks = (long long)p.tiles_m * p.tiles_n * p.splits;
+    NCNNHIP_REQUIRE(blocks < (1ll << 31), "convolution: too many tiles");
+    int32_t* partial = 0;
+    const size_t words = (size_t)g.npix * out_cp;
+    if (p.splits > 1)
+    {
+        NCNNHIP_REQUIRE(workspace && workspace_bytes >= words * sizeof(int32_t), "convolution: workspace of %zu bytes required", words * sizeof(int32_t));
+        partial = (int32_t*)workspace;
+        hipLaunchKernelGGL(zero_words_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, words);
+    }
+    dim3 grid((unsigned)blocks), block(256);
+#define LAUNCH_PIPE(BM_, BN_, ST_)                                                                                                              \
+    do                                                                                                                                          \
+    {                                                                                                                                           \
+        if (p.splits > 1)                                                                                                                       \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true>), grid, block, 0, stream, wpk, x, g, epi, out_cp, p.tiles_m, p.tiles_n, \
+                               p.steps_per_split, partial);                                                                                     \
+        else                                                                                                                                    \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false>), grid, block, 0, stream, wpk, x, g, epi, out_cp, p.tiles_m, p.tiles_n, \
+                               p.steps_per_split, partial);                                                                                     \
+    } while (0)
+    if (p.bm == 128 && p.bn == 256)
+        LAUNCH_PIPE(128, 256, 3);
+    else if (p.bm == 128 && p.bn == 128)
+        LAUNCH_PIPE(128, 128, 3);
+    else if (p.bm == 128)
+        LAUNCH_PIPE(128, 64, 3);
+    else if (p.bn == 256)
+        LAUNCH_PIPE(64, 256, 3);
+    else if (p.bn == 128)
+        LAUNCH_PIPE(64, 128, 3);
+    else
+        LAUNCH_PIPE(64, 64, 3);
+#undef LAUNCH_PIPE
+    if (p.splits > 1)
+        hipLaunchKernelGGL(conv_pipelined_finish_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, g.npix, out_cp, g.cout, epi);
+    return launch_status("conv_nhwc_pipelined_kernel");
+}
+
+} // namespace ncnnhip
