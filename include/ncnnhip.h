@@ -130,6 +130,25 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
                            void* out_dev, int out_layout, size_t out_cstep, size_t out_nstep, void* workspace_dev,
                            size_t workspace_bytes, void* stream);
 
+/* The same convolution (fp32 channels-last output, zero border value) with the layers that follow it folded into its
+ * epilogue, element by element in the reference's order:
+ *   f = act(acc*scale_in + bias)                      Convolution::forward_int8, src/layer/convolution.cpp:476-502
+ *   f = f + residual                                  Eltwise sum of two inputs, src/layer/eltwise.cpp:95-118
+ *   f = max(f, 0)                  (relu_after)       ReLU slope 0, src/layer/relu.cpp:30-45
+ *   out = f;  quantised_out = float2int8(f * scale)   Quantize of the next convolution's input, src/layer/quantize.cpp:48-111
+ * Every step is optional (NULL / 0).  ncnnhip_conv_fusion_supported says whether a geometry can take this path. */
+typedef struct ncnnhip_conv_fusion
+{
+    const float* residual_dev;  /* channels-last fp32 blob of the output's shape */
+    int relu_after;
+    int8_t* quantised_out_dev;  /* channels-last int8 blob of the output's shape */
+    float quantise_scale;
+} ncnnhip_conv_fusion;
+int ncnnhip_conv_fusion_supported(const ncnnhip_conv_desc* desc);
+int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev,
+                                 const float* scale_in_dev, const float* bias_dev, ncnnhip_activation act, float* out_dev,
+                                 const ncnnhip_conv_fusion* fusion, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ device-resident blobs (channels-last)
  * Between layers a 3-D blob stays in HBM as [batch][h*w][Cp] (Cp = ncnnhip_padded_channels(c), fp32 or int8, pad
  * channels zero); 1-D / 2-D blobs are dense.  ncnn's planar Mat layout (src/mat.h:341-381) exists only at the host

@@ -20,12 +20,22 @@ struct NhwcGeom
     int pad_word; // border byte replicated 4x
 };
 
+// Optional tail of the pipelined kernel's fp32 epilogue: out = [relu](act(acc*scale_in + bias) + residual), and a
+// second, quantised copy of the result for the convolution that consumes it.
+struct ConvFusion
+{
+    const float* residual; // channels-last fp32, the output's shape; 0: none
+    int relu_after;
+    int8_t* q8_out;        // channels-last int8 copy: float2int8(result * q8_scale); 0: none
+    float q8_scale;
+};
+
 // int32 words of split-K scratch the pipelined kernel wants for this problem (0: it does not split)
 size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps);
 
 // Launches the pipelined kernel; the caller has checked: zero border byte, channels-last output.
-int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, void* workspace,
-                               size_t workspace_bytes, hipStream_t stream);
+int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
+                               void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 } // namespace ncnnhip
 

@@ -436,9 +436,9 @@ int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x
     return launch_status("to_nhwc_int8_kernel");
 }
 
-int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
-                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
-                           size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
+static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                               const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
+                               size_t out_cstep, size_t out_nstep, const ConvFusion& fusion, void* workspace_dev, size_t workspace_bytes, void* stream)
 {
     NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_nhwc: null pointer");
     NCNNHIP_REQUIRE(desc->group == 1, "ncnnhip_conv_int8_nhwc: group must be 1");
@@ -491,7 +491,8 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
 
     hipStream_t st = as_stream(stream);
     // zero border and channels-last output: the pipelined kernel
-    if (clast && pb == 0) return launch_conv_nhwc_pipelined(g, packed_weight_dev, nhwc_dev, epi, out_cp, workspace_dev, workspace_bytes, st);
+    if (clast && pb == 0) return launch_conv_nhwc_pipelined(g, packed_weight_dev, nhwc_dev, epi, fusion, out_cp, workspace_dev, workspace_bytes, st);
+    NCNNHIP_REQUIRE(!fusion.residual && !fusion.relu_after && !fusion.q8_out, "ncnnhip_conv_int8_nhwc_fused: needs channels-last output and a zero border value");
     const SplitPlan p = plan_launch(d.num_output, npix, g.K / 64);
     dim3 grid(ceil_div(npix, p.bn), ceil_div(d.num_output, p.bm), p.splits);
     NCNNHIP_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ncnnhip_conv_int8_nhwc: grid too large");
@@ -529,6 +530,36 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
     else if (p.splits > 1)
         hipLaunchKernelGGL(conv_splitk_finish_kernel, dim3(ceil_div((long long)d.num_output * npix, 256)), dim3(256), 0, st, partial, d.num_output, (int)npix, epi);
     return launch_status("conv_nhwc_kernel");
+}
+
+int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
+                           size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    const ConvFusion none = {0, 0, 0, 0.f};
+    return conv_int8_nhwc_impl(desc, nhwc_dev, packed_weight_dev, scale_in_dev, bias_dev, scale_out_dev, act, out_dev, out_layout, out_cstep, out_nstep, none,
+                               workspace_dev, workspace_bytes, stream);
+}
+
+int ncnnhip_conv_fusion_supported(const ncnnhip_conv_desc* desc)
+{
+    return desc && desc->group == 1 && (int)(signed char)desc->pad_value == 0;
+}
+
+int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                                 const float* bias_dev, ncnnhip_activation act, float* out_dev, const ncnnhip_conv_fusion* fusion, void* workspace_dev,
+                                 size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(fusion, "ncnnhip_conv_int8_nhwc_fused: null fusion");
+    NCNNHIP_REQUIRE(ncnnhip_conv_fusion_supported(desc), "ncnnhip_conv_int8_nhwc_fused: needs group 1 and a zero border value");
+    NCNNHIP_REQUIRE(!fusion->quantised_out_dev || fusion->quantise_scale != 0.f, "ncnnhip_conv_int8_nhwc_fused: quantised copy without a scale");
+    ConvFusion f;
+    f.residual = fusion->residual_dev;
+    f.relu_after = fusion->relu_after;
+    f.q8_out = fusion->quantised_out_dev;
+    f.q8_scale = fusion->quantise_scale;
+    return conv_int8_nhwc_impl(desc, nhwc_dev, packed_weight_dev, scale_in_dev, bias_dev, 0, act, out_dev, NCNNHIP_CHANNELS_LAST, 0, 0, f, workspace_dev,
+                               workspace_bytes, stream);
 }
 
 } // extern "C"

@@ -30,14 +30,24 @@ namespace ncnnhip {
 
 __device__ __attribute__((aligned(64))) int8_t g_zero_line[64];
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// four already-quantised values (integers in [-127,127] held as floats) -> four bytes
+__device__ __forceinline__ uint32_t pack4(const v4f& v)
+{
+    return (uint32_t)((int)v[0] & 0xff) | ((uint32_t)((int)v[1] & 0xff) << 8) | ((uint32_t)((int)v[2] & 0xff) << 16) | ((uint32_t)((int)v[3] & 0xff) << 24);
+}
+
 template<int BM, int BN, int STAGES, bool SPLITK>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   int out_cp, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
+                                                                   ConvFusion fusion, int out_cp, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
     constexpr int STAGE_BYTES = (BM + BN) * 64;
-    __shared__ __attribute__((aligned(1024))) int8_t smem[STAGES * STAGE_BYTES];
+    constexpr int EPILOGUE_BYTES = 4 * 32 * (BN / 2 + 4) * 4; // per wavefront 32 pixels x (BN/2 + 4) floats
+    constexpr int SMEM_BYTES = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[SMEM_BYTES];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -210,27 +220,42 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
         return;
     }
-    // the activation type is uniform: branch on it once, outside the unrolled stores
+    // Through LDS, so that global memory sees whole runs of channels: each wavefront stages 32 pixels x CW channels of
+    // results as [pixel][channel] floats (the pipeline stages are free by now), then every lane takes 4 consecutive
+    // channels of one pixel: a 16-byte residual load, a 16-byte fp32 store and a 4-byte int8 store, the wavefront
+    // covering 64/(CW/4) pixel rows of CW contiguous channels per instruction.
+    constexpr int CW = BN / 2;      // channels per wavefront
+    constexpr int LD = CW + 4;      // row pitch in floats
+    constexpr int G = CW / 4;       // 4-channel groups per row
+    __syncthreads();                // nobody reads the operand stages any more
+    float* tile = reinterpret_cast<float*>(smem) + wave * (32 * LD);
+    const bool to_int8 = epi.scale_out != 0;
+
+    float s_in[TN], bias[TN], s_out[TN];
+    bool real[TN];
+#pragma unroll
+    for (int c = 0; c < TN; c++)
+    {
+        const int ch = col0 + wn * CW + c * 32 + l32;
+        real[c] = ch < g.cout; // channels from cout up to out_cp are the blob's zero padding
+        s_in[c] = real[c] ? epi.scale_in[ch] : 0.f;
+        bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : 0.f;
+        s_out[c] = (real[c] && to_int8) ? epi.scale_out[ch] : 0.f;
+    }
+
+    // the activation type is uniform: branch on it once, outside the unrolled loops
     auto finish = [&](auto act_tag) {
         constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-        for (int c = 0; c < TN; c++)
+        for (int a = 0; a < TM; a++)
         {
-            const int ch = col0 + wn * (BN / 2) + c * 32 + l32;
-            if (ch >= out_cp) continue;
-            const bool real = ch < g.cout; // channels from cout up to out_cp are the blob's zero padding
-            const float s_in = real ? epi.scale_in[ch] : 0.f;
-            const float bias = (real && epi.bias) ? epi.bias[ch] : 0.f;
-            const float s_out = (real && epi.scale_out) ? epi.scale_out[ch] : 0.f;
 #pragma unroll
-            for (int a = 0; a < TM; a++)
+            for (int c = 0; c < TN; c++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                 {
-                    const int pix = row0 + wm * (BM / 2) + a * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                    if (pix >= g.npix) continue;
-                    float f = mul_rn((float)acc[a][c][r], s_in);
-                    if (epi.bias) f = add_rn(f, bias);
+                    float f = mul_rn((float)acc[a][c][r], s_in[c]);
+                    if (epi.bias) f = add_rn(f, bias[c]);
                     if (ACT == 1)
                         f = fmaxf(f, 0.f);
                     else if (ACT == 3)
@@ -240,13 +265,49 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                     }
                     else if (ACT != 0)
                         f = apply_activation(f, epi.act);
-                    if (!real) f = 0.f;
-                    const size_t o = (size_t)pix * out_cp + ch;
-                    if (epi.scale_out)
-                        static_cast<int8_t*>(epi.out)[o] = (int8_t)float2int8(mul_rn(f, s_out));
-                    else
-                        static_cast<float*>(epi.out)[o] = f;
+                    if (to_int8) f = (float)float2int8(mul_rn(f, s_out[c]));
+                    if (!real[c]) f = 0.f;
+                    tile[(8 * (r >> 2) + 4 * lhi + (r & 3)) * LD + c * 32 + l32] = f;
                 }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < G / 2; it++)
+            {
+                const int idx = it * 64 + lane;
+                const int p = idx / G, j = idx - p * G;
+                v4f v = *reinterpret_cast<const v4f*>(tile + p * LD + 4 * j);
+                const int pix = row0 + wm * (BM / 2) + a * 32 + p;
+                const int ch4 = col0 + wn * CW + 4 * j;
+                if (pix < g.npix && ch4 < out_cp)
+                {
+                    const size_t o = (size_t)pix * out_cp + ch4;
+                    if (to_int8)
+                        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(epi.out) + o) = pack4(v);
+                    else
+                    {
+                        if (fusion.residual)
+                        {
+                            const v4f res = *reinterpret_cast<const v4f*>(fusion.residual + o);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[e] = add_rn(v[e], res[e]);
+                        }
+                        if (fusion.relu_after)
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[e] = fmaxf(v[e], 0.f);
+                        }
+                        *reinterpret_cast<v4f*>(static_cast<float*>(epi.out) + o) = v;
+                        if (fusion.q8_out)
+                        {
+                            v4f q;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) q[e] = (float)float2int8(mul_rn(v[e], fusion.q8_scale));
+                            *reinterpret_cast<uint32_t*>(fusion.q8_out + o) = pack4(q);
+                        }
+                    }
+                }
+            }
+            if (a + 1 < TM) __syncthreads();
         }
     };
     if (epi.act.type == 0)
@@ -260,7 +321,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 }
 
 // partial sums [npix][out_cp] -> epilogue; one thread per (pixel, channel), channels fastest
-__global__ __launch_bounds__(256) void conv_pipelined_finish_kernel(const int32_t* __restrict__ partial, int npix, int out_cp, int cout, ConvEpilogue epi)
+__global__ __launch_bounds__(256) void conv_pipelined_finish_kernel(const int32_t* __restrict__ partial, int npix, int out_cp, int cout, ConvEpilogue epi,
+                                                                     ConvFusion fusion)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)npix * out_cp) return;
@@ -276,7 +338,12 @@ __global__ __launch_bounds__(256) void conv_pipelined_finish_kernel(const int32_
     if (epi.scale_out)
         static_cast<int8_t*>(epi.out)[i] = real ? (int8_t)float2int8(mul_rn(f, epi.scale_out[ch])) : (int8_t)0;
     else
+    {
+        if (fusion.residual) f = add_rn(f, fusion.residual[i]);
+        if (fusion.relu_after) f = fmaxf(f, 0.f);
         static_cast<float*>(epi.out)[i] = f;
+        if (fusion.q8_out) fusion.q8_out[i] = (int8_t)float2int8(mul_rn(f, fusion.q8_scale));
+    }
 }
 
 __global__ __launch_bounds__(256) void zero_words_kernel(int32_t* p, size_t n)
@@ -328,8 +395,8 @@ size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps)
     return p.splits > 1 ? (size_t)npix * ((cout + 15) / 16 * 16) : 0;
 }
 
-int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, void* workspace,
-                               size_t workspace_bytes, hipStream_t stream)
+int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
+                               void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
     const PipePlan p = plan_pipelined(g.cout, g.npix, g.K / 64);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * p.splits;
@@ -347,10 +414,10 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     do                                                                                                                                          \
     {                                                                                                                                           \
         if (p.splits > 1)                                                                                                                       \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true>), grid, block, 0, stream, wpk, x, g, epi, out_cp, p.tiles_m, p.tiles_n, \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true>), grid, block, 0, stream, wpk, x, g, epi, fusion, out_cp, p.tiles_m, p.tiles_n, \
                                p.steps_per_split, partial);                                                                                     \
         else                                                                                                                                    \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false>), grid, block, 0, stream, wpk, x, g, epi, out_cp, p.tiles_m, p.tiles_n, \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, out_cp, p.tiles_m, p.tiles_n, \
                                p.steps_per_split, partial);                                                                                     \
     } while (0)
     if (p.bm == 128 && p.bn == 256)
@@ -367,7 +434,7 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
         LAUNCH_PIPE(64, 64, 3);
 #undef LAUNCH_PIPE
     if (p.splits > 1)
-        hipLaunchKernelGGL(conv_pipelined_finish_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, g.npix, out_cp, g.cout, epi);
+        hipLaunchKernelGGL(conv_pipelined_finish_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, g.npix, out_cp, g.cout, epi, fusion);
     return launch_status("conv_nhwc_pipelined_kernel");
 }
 

@@ -31,6 +31,10 @@ class ConvDesc(C.Structure):
                [("pad_value", C.c_float), ("group", C.c_int)]
 
 
+class ConvFusion(C.Structure):
+    _fields_ = [("residual_dev", C.c_void_p), ("relu_after", C.c_int), ("quantised_out_dev", C.c_void_p), ("quantise_scale", C.c_float)]
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("w", "h", "c", "batch", "pooling_type", "kernel_w", "kernel_h", "stride_w", "stride_h", "pad_top", "pad_left",
                                        "outw", "outh", "global_pooling", "avgpool_count_include_pad")]
@@ -69,6 +73,9 @@ _SIGNATURES = {
     "ncnnhip_to_nhwc_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_conv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_int,
                                C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_conv_fusion_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_int8_nhwc_fused": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.POINTER(ConvFusion), C.c_void_p,
+                                     C.c_size_t, C.c_void_p],
     "ncnnhip_conv_resolved_pads": [C.POINTER(ConvDesc), C.POINTER(C.c_int), C.POINTER(C.c_int)],
     "ncnnhip_padded_channels": [C.c_int],
     "ncnnhip_chw_to_nhwc": [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -345,7 +352,8 @@ class Runtime:
         return out.to_numpy(self.stream)
 
     def conv_channels_last(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
-                           pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0)):
+                           pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), residual=None, relu_after=False,
+                           quantise_scale=None):
         """Convolution (group 1) or depthwise (group == c == num_output) entirely on channels-last device blobs:
         upload+convert, quantise if fp32, kernel writing channels-last, convert back.  x is [n][c][h][w]."""
         x = np.ascontiguousarray(x)
@@ -379,6 +387,15 @@ class Runtime:
             pk = np.empty(wb.value, np.int8)
             check(lib().ncnnhip_conv_pack_weights(C.byref(d), wq.ctypes.data, pk.ctypes.data))
             dpk, dws = self.up(pk), DeviceBuffer(max(sb_.value, 4))
+            if residual is not None or relu_after or quantise_scale is not None:
+                # the layers after the convolution folded into its epilogue; returns (fp32 result, its quantised copy or None)
+                dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))
+                dq8 = None if quantise_scale is None else DeviceBuffer.empty((n, oh * ow, ocp), np.int8)
+                fu = ConvFusion(_ptr(dres), int(relu_after), _ptr(dq8), float(quantise_scale or 0.0))
+                check(lib().ncnnhip_conv_int8_nhwc_fused(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), Activation.make(act, act_params), dout.ptr, C.byref(fu),
+                                                         dws.ptr, sb_.value, self.stream))
+                q8 = None if dq8 is None else self.from_channels_last(dq8, n, num_output, oh, ow)
+                return self.from_channels_last(dout, n, num_output, oh, ow), q8
             check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
                                                1, 0, 0, dws.ptr, sb_.value, self.stream))
         else:

@@ -343,6 +343,25 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
 // as it is.  Nothing is copied to or from the host and nothing waits.
 int Convolution_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option& opt) const
 {
+    return forward_hip_fused(bottom, 0, false, 0.f, top, cmd, opt);
+}
+
+float Convolution_hip::hip_input_quantise_scale() const
+{
+    return (support_hip && bottom_blob_int8_scales.w > 0) ? bottom_blob_int8_scales[0] : 0.f;
+}
+
+bool Convolution_hip::hip_can_fuse_tail() const
+{
+    // the folded tail lives in the fp32 epilogue of the pipelined kernel: plain convolution, zero border value
+    return support_hip && group == 1 && int8_scale_term <= 100 && (int)(signed char)pad_value == 0;
+}
+
+int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* residual, bool relu, float q8_scale, HipMat& top, HipCommand& cmd,
+                                       const Option& opt) const
+{
+    const bool fused = residual || relu || q8_scale != 0.f;
+    if (fused && !hip_can_fuse_tail()) return -1;
     if (!opt.use_int8_inference)
     {
         NCNN_LOGE("%s %s: use_int8_inference is off and there is no fp32 path in this runtime", type.c_str(), name.c_str());
@@ -376,8 +395,15 @@ int Convolution_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand& 
     ScopedScratch scratch(&cmd);
     void* st = cmd.stream;
 
+    if (residual && (residual->elemsize != 4u || residual->dims != 3 || residual->count() != top.count()))
+    {
+        NCNN_LOGE("%s %s: the residual blob does not have the output's shape", type.c_str(), name.c_str());
+        return -1;
+    }
     const int8_t* xq = (const int8_t*)bottom.data;
-    if (bottom.elemsize == 4u)
+    if (bottom.elemsize == 4u && bottom.q8 && !bottom.q8->empty() && bottom.q8_scale == bottom_blob_int8_scales[0] && bottom.q8->count() == bottom.count())
+        xq = (const int8_t*)bottom.q8->data; // the producer's epilogue already quantised this blob with our scale
+    else if (bottom.elemsize == 4u)
     {
         void* q = scratch.get(bottom.count());
         if (!q) return -100;
@@ -396,6 +422,25 @@ int Convolution_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand& 
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
         void* ws = workspace_bytes ? scratch.get(workspace_bytes) : 0;
         if (workspace_bytes && !ws) return -100;
+        if (fused)
+        {
+            ncnnhip_conv_fusion fu;
+            fu.residual_dev = residual ? (const float*)residual->data : 0;
+            fu.relu_after = relu ? 1 : 0;
+            fu.quantised_out_dev = 0;
+            fu.quantise_scale = q8_scale;
+            if (q8_scale != 0.f)
+            {
+                top.q8.reset(new HipMat);
+                top.q8->create(outw, outh, num_output, 1u, bottom.n, &cmd);
+                if (top.q8->empty()) return -100;
+                top.q8_scale = q8_scale;
+                fu.quantised_out_dev = (int8_t*)top.q8->data;
+            }
+            rc = ncnnhip_conv_int8_nhwc_fused(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, act, (float*)top.data,
+                                              &fu, ws, workspace_bytes, st);
+            return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc_fused");
+        }
         rc = ncnnhip_conv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, (const float*)d_scale_out, act,
                                     top.data, NCNNHIP_CHANNELS_LAST, 0, 0, ws, workspace_bytes, st);
         return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");

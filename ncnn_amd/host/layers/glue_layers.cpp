@@ -91,8 +91,13 @@ public:
         slope = pd.get(0, 0.f);
         return 0;
     }
+    virtual bool hip_plain_relu() const
+    {
+        return slope == 0.f;
+    }
     virtual int forward_inplace_hip(HipMat& m, HipCommand& cmd, const Option&) const
     {
+        m.q8.reset(); // a quantised copy travelling with the blob describes the values before this layer
         // flat over the blob, pad channels included (zero stays zero)
         if (m.elemsize == 4u && m.count() % 4 != 0)
         {
@@ -348,6 +353,10 @@ public:
         support_hip = true;
         return 0;
     }
+    virtual bool hip_plain_sum() const
+    {
+        return op_type == 1 && coeffs.w == 0;
+    }
     virtual int forward_hip(const std::vector<HipMat>& bottoms, std::vector<HipMat>& tops, HipCommand& cmd, const Option&) const
     {
         if (bottoms.size() < 2) return -1;
@@ -470,6 +479,7 @@ public:
             NCNN_LOGE("Softmax: the device overload handles 1-D fp32 blobs");
             return -1;
         }
+        m.q8.reset();
         return dev_status(ncnnhip_softmax((const float*)m.data, (float*)m.data, m.w, m.n, cmd.stream), "ncnnhip_softmax");
     }
     virtual int forward_inplace(Mat& m, const Option&) const
@@ -521,6 +531,7 @@ public:
     {
         if (scale == 1.f) return 0;
         if (m.elemsize != 4u) return -1;
+        m.q8.reset();
         return dev_status(ncnnhip_scale((const float*)m.data, (float*)m.data, m.count(), scale, cmd.stream), "ncnnhip_scale");
     }
     virtual int forward_inplace(Mat& m, const Option&) const

@@ -23,6 +23,10 @@ public:
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
     virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
+    virtual float hip_input_quantise_scale() const;
+    virtual bool hip_can_fuse_tail() const;
+    virtual int forward_hip_fused(const ncnn::HipMat& bottom_blob, const ncnn::HipMat* residual, bool relu, float q8_scale, ncnn::HipMat& top_blob,
+                                  ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
 
 public:
     // same member names as the reference layers

@@ -13,9 +13,9 @@ static int hip_status(int rc, const char* where)
 
 // ---- HipMat -----------------------------------------------------------------------------------
 
-HipMat::HipMat() : data(0), refcount(0), cmd(0), dims(0), w(0), h(0), c(0), n(0), cp(0), elemsize(0) {}
+HipMat::HipMat() : data(0), refcount(0), cmd(0), dims(0), w(0), h(0), c(0), n(0), cp(0), elemsize(0), q8_scale(0.f) {}
 
-HipMat::HipMat(const HipMat& m) : data(m.data), refcount(m.refcount), cmd(m.cmd), dims(m.dims), w(m.w), h(m.h), c(m.c), n(m.n), cp(m.cp), elemsize(m.elemsize)
+HipMat::HipMat(const HipMat& m) : data(m.data), refcount(m.refcount), cmd(m.cmd), dims(m.dims), w(m.w), h(m.h), c(m.c), n(m.n), cp(m.cp), elemsize(m.elemsize), q8(m.q8), q8_scale(m.q8_scale)
 {
     if (refcount) __sync_fetch_and_add(refcount, 1);
 }
@@ -40,6 +40,8 @@ HipMat& HipMat::operator=(const HipMat& m)
     n = m.n;
     cp = m.cp;
     elemsize = m.elemsize;
+    q8 = m.q8;
+    q8_scale = m.q8_scale;
     return *this;
 }
 
@@ -55,6 +57,8 @@ void HipMat::release()
     cmd = 0;
     dims = w = h = c = n = cp = 0;
     elemsize = 0;
+    q8.reset();
+    q8_scale = 0.f;
 }
 
 void HipMat::allocate(HipCommand* command)

@@ -12,6 +12,7 @@
 
 #include <stddef.h>
 
+#include <memory>
 #include <vector>
 
 #include "mat.h"
@@ -61,6 +62,10 @@ public:
     int dims, w, h, c, n;
     int cp; // channels as padded in memory (dims 3), else 0
     size_t elemsize;
+    // An fp32 blob may travel with an int8 copy of itself, float2int8(value * q8_scale), written by the kernel
+    // that produced it: the convolution that consumes the blob with that input scale then skips its Quantize pass.
+    std::shared_ptr<HipMat> q8;
+    float q8_scale;
 
 private:
     void allocate(HipCommand* cmd);

@@ -88,6 +88,26 @@ int Layer::forward_inplace_hip(HipMat&, HipCommand&, const Option&) const
 {
     return -1;
 }
+bool Layer::hip_plain_sum() const
+{
+    return false;
+}
+bool Layer::hip_plain_relu() const
+{
+    return false;
+}
+float Layer::hip_input_quantise_scale() const
+{
+    return 0.f;
+}
+bool Layer::hip_can_fuse_tail() const
+{
+    return false;
+}
+int Layer::forward_hip_fused(const HipMat&, const HipMat*, bool, float, HipMat&, HipCommand&, const Option&) const
+{
+    return -1;
+}
 
 // ---- built-in type table ------------------------------------------------------------------
 

@@ -54,6 +54,17 @@ public:
     virtual int forward_hip(const HipMat& bottom_blob, HipMat& top_blob, HipCommand& cmd, const Option& opt) const;
     virtual int forward_inplace_hip(HipMat& bottom_top_blob, HipCommand& cmd, const Option& opt) const;
 
+    // Hooks with which the device-resident executor folds elementwise neighbours into a producer's epilogue
+    // (conv -> Eltwise sum -> ReLU -> the next convolution's Quantize becomes one kernel).  Every statement of the
+    // folded layers is applied per element in the original order, so results do not change.
+    virtual bool hip_plain_sum() const;             // Eltwise: sum of exactly two inputs, no coefficients
+    virtual bool hip_plain_relu() const;            // ReLU with slope 0
+    virtual float hip_input_quantise_scale() const; // scale of this layer's own Quantize of an fp32 3-D bottom; 0: none
+    virtual bool hip_can_fuse_tail() const;         // forward_hip_fused works for this layer as configured
+    // top = [relu](forward(bottom) + *residual);  q8_scale != 0: top.q8 = Quantize(top, q8_scale) as well
+    virtual int forward_hip_fused(const HipMat& bottom_blob, const HipMat* residual, bool relu, float q8_scale, HipMat& top_blob, HipCommand& cmd,
+                                  const Option& opt) const;
+
     void* userdata;
     int typeindex;
     std::string type;

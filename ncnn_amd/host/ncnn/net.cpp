@@ -129,6 +129,23 @@ public:
         idle_cmds.push_back(c);
     }
 
+    // ---- epilogue fusion of the device-resident path (built once the model is loaded) --------------------
+    // tail_plan[L] for a layer L that is a plain ReLU or a plain two-input sum: the convolution whose epilogue can
+    // produce L's output directly.  quantise_scale[b]: the one input scale with which every quantising consumer
+    // of blob b (through Split layers) would quantise it, 0 if there is none or they differ.
+    struct TailPlan
+    {
+        int conv;     // layer index, -1: none
+        int eltwise;  // the sum layer
+        int residual; // blob index of the sum's other input
+        bool relu;
+    };
+    std::vector<TailPlan> tail_plan;
+    std::vector<float> quantise_scale;
+    void build_fusion_plan();
+    bool collect_quantise_scales(int blob, float& scale, bool& any) const;
+    int try_fused_tail(int layer_index, ExecState& st, const Option& opt, bool& done) const;
+
     int forward_layer(int layer_index, ExecState& st, const Option& opt) const;
     int run_layer(const Layer* layer, ExecState& st, const Option& opt) const;
     int run_layer_hip(const Layer* layer, ExecState& st, const Option& opt) const;
@@ -157,12 +174,136 @@ static int expand_int8(const Mat& src, Mat& dst, Allocator* allocator)
     return 0;
 }
 
+// ---- fusion plan ----------------------------------------------------------------------------
+
+// walks the consumers of a blob through Split layers; false when two quantising consumers disagree
+bool NetPrivate::collect_quantise_scales(int blob, float& scale, bool& any) const
+{
+    const int ci = blobs[(size_t)blob].consumer;
+    if (ci < 0) return true;
+    const Layer* consumer = layers[(size_t)ci];
+    if (consumer->type == "Split")
+    {
+        for (size_t i = 0; i < consumer->tops.size(); i++)
+            if (!collect_quantise_scales(consumer->tops[i], scale, any)) return false;
+        return true;
+    }
+    const float s = consumer->hip_input_quantise_scale();
+    if (s == 0.f) return true; // reads the fp32 values
+    if (any && s != scale) return false;
+    scale = s;
+    any = true;
+    return true;
+}
+
+void NetPrivate::build_fusion_plan()
+{
+    const TailPlan none = {-1, -1, -1, false};
+    tail_plan.assign(layers.size(), none);
+    quantise_scale.assign(blobs.size(), 0.f);
+    for (size_t b = 0; b < blobs.size(); b++)
+    {
+        float s = 0.f;
+        bool any = false;
+        if (collect_quantise_scales((int)b, s, any) && any) quantise_scale[b] = s;
+    }
+    // a sum whose (later) input is a convolution that can take the other input as a residual
+    for (size_t li = 0; li < layers.size(); li++)
+    {
+        const Layer* e = layers[li];
+        if (!e->support_hip || !e->hip_plain_sum() || e->bottoms.size() != 2 || e->tops.size() != 1) continue;
+        int best = -1, best_slot = -1;
+        for (int k = 0; k < 2; k++)
+        {
+            const int p = blobs[(size_t)e->bottoms[(size_t)k]].producer;
+            if (p < 0) continue;
+            const Layer* c = layers[(size_t)p];
+            if (c->support_hip && c->one_blob_only && c->bottoms.size() == 1 && c->tops.size() == 1 && c->hip_can_fuse_tail() && p > best)
+            {
+                best = p;
+                best_slot = k;
+            }
+        }
+        if (best < 0) continue;
+        TailPlan tp = {best, (int)li, e->bottoms[(size_t)(1 - best_slot)], false};
+        tail_plan[li] = tp;
+        // ... followed by a plain ReLU: that layer's output comes out of the same epilogue
+        const int ri = blobs[(size_t)e->tops[0]].consumer;
+        if (ri >= 0 && layers[(size_t)ri]->support_hip && layers[(size_t)ri]->hip_plain_relu() && layers[(size_t)ri]->bottoms.size() == 1)
+        {
+            tp.relu = true;
+            tail_plan[(size_t)ri] = tp;
+        }
+    }
+}
+
+// Runs layer_index (a sum, or the ReLU after it) as the epilogue of the convolution in its plan, if nothing on the
+// way has been computed yet and the intermediate blobs may be skipped (light mode).  done = false: not applicable,
+// the caller runs the layers one by one.
+int NetPrivate::try_fused_tail(int layer_index, ExecState& st, const Option& opt, bool& done) const
+{
+    done = false;
+    if (!opt.use_hip_compute || !opt.lightmode || tail_plan.size() != layers.size()) return 0;
+    const TailPlan& tp = tail_plan[(size_t)layer_index];
+    if (tp.conv < 0) return 0;
+    const Layer* conv = layers[(size_t)tp.conv];
+    const Layer* sum = layers[(size_t)tp.eltwise];
+    const Layer* last = layers[(size_t)layer_index];
+    if (st.has(conv->tops[0]) || st.has(sum->tops[0])) return 0; // an intermediate exists already (fed or extracted)
+
+    const int needed[2] = {conv->bottoms[0], tp.residual};
+    for (int k = 0; k < 2; k++)
+    {
+        const int bi = needed[k];
+        if (st.has(bi)) continue;
+        const int producer = blobs[(size_t)bi].producer;
+        if (producer < 0) return 0;
+        int ret = forward_layer(producer, st, opt);
+        if (ret != 0) return ret;
+        if (!st.has(bi)) return 0;
+    }
+    if (!st.cmd) st.cmd = acquire_command();
+    HipCommand& cmd = *st.cmd;
+    int ret = cmd.ensure_ready();
+    if (ret != 0) return ret;
+    HipMat ins[2];
+    for (int k = 0; k < 2; k++)
+    {
+        const size_t bi = (size_t)needed[k];
+        if (st.dev[bi].empty())
+        {
+            ret = cmd.upload(st.host[bi], st.dev[bi]);
+            if (ret != 0) return ret;
+        }
+        ins[k] = st.dev[bi];
+    }
+    if (ins[1].elemsize != 4u || ins[1].dims != 3) return 0; // the residual must be an fp32 blob: take the plain route
+    for (int k = 0; k < 2; k++)
+    {
+        st.dev[(size_t)needed[k]].release();
+        st.host[(size_t)needed[k]].release();
+    }
+    HipMat top;
+    ret = conv->forward_hip_fused(ins[0], &ins[1], tp.relu, quantise_scale[(size_t)last->tops[0]], top, cmd, opt);
+    if (ret != 0) return ret;
+    st.dev[(size_t)last->tops[0]] = top;
+    st.host[(size_t)last->tops[0]].release();
+    done = true;
+    return 0;
+}
+
 // ---- executor -----------------------------------------------------------------------------
 
 int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt) const
 {
     const Layer* layer = layers[layer_index];
     if (layer->bottoms.empty() && layer->type == "Input") return 0; // inputs are fed, not computed
+
+    {
+        bool done = false;
+        int ret = try_fused_tail(layer_index, st, opt, done);
+        if (ret != 0 || done) return ret;
+    }
 
     // make sure every input exists, computing producers depth-first
     for (size_t i = 0; i < layer->bottoms.size(); i++)
@@ -251,7 +392,13 @@ int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& o
             ret = layer->forward_inplace_hip(top, cmd, opt);
         }
         else
-            ret = layer->forward_hip(ins[0], top, cmd, opt);
+        {
+            const float qs = quantise_scale.size() == blobs.size() ? quantise_scale[(size_t)layer->tops[0]] : 0.f;
+            if (qs != 0.f && layer->hip_can_fuse_tail())
+                ret = layer->forward_hip_fused(ins[0], 0, false, qs, top, cmd, opt); // the consumers' Quantize rides along
+            else
+                ret = layer->forward_hip(ins[0], top, cmd, opt);
+        }
         if (ret != 0) return ret;
         st.dev[(size_t)layer->tops[0]] = top;
         st.host[(size_t)layer->tops[0]].release();
@@ -697,6 +844,7 @@ int Net::load_model(const DataReader& dr)
             break;
         }
     }
+    if (status == 0) d->build_fusion_plan();
     return status;
 }
 
@@ -742,6 +890,8 @@ void Net::clear()
     d->output_idx.clear();
     d->input_nm.clear();
     d->output_nm.clear();
+    d->tail_plan.clear();
+    d->quantise_scale.clear();
     std::lock_guard<std::mutex> g(d->cmd_lock);
     d->idle_cmds.clear();
     d->io_cmd.reset();

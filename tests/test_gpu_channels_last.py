@@ -180,3 +180,25 @@ def test_softmax_within_1e_6(rt):
     want = e / e.sum(axis=1, keepdims=True)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-9)
     assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("c,h,w,outc,kernel,pads", [(64, 14, 14, 256, (1, 1), (0, 0, 0, 0)), (24, 20, 18, 40, (3, 3), (1, 1, 1, 1)),
+                                                     (512, 7, 7, 200, (1, 1), (0, 0, 0, 0)), (2048, 7, 7, 48, (1, 1), (0, 0, 0, 0))])
+@pytest.mark.parametrize("relu", [False, True])
+def test_convolution_with_residual_relu_and_quantised_copy_in_the_epilogue(rt, c, h, w, outc, kernel, pads, relu):
+    """conv -> Eltwise sum -> ReLU -> Quantize folded into one kernel equals the four layers run one by one."""
+    _say("fused epilogue", c, h, w, outc, kernel, relu)
+    rng = np.random.default_rng(c + outc)
+    x, wq, b, ws, ins, tops = cases.conv_case(c + outc, c, h, w, outc, kernel, 1, 2, True, False, batch=2)
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, 1), (1, 1), pads, 0.0, 1, 1, 2, 0, (0.0, 0.0))
+    conv = np.stack([oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None) for i in range(2)])
+    res = rng.normal(0, 1, conv.shape).astype(F)
+    want = (conv + res).astype(F)
+    if relu:
+        want = np.maximum(want, 0)
+    next_scale = F(127) / np.abs(want).max()
+    want_q = oracle.quantize(want.reshape(-1, want.shape[-1]), [next_scale]).reshape(want.shape)
+    got, got_q = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, (1, 1), (1, 1), pads, 0.0, 1, 2, 0, (0.0, 0.0),
+                                       residual=res, relu_after=relu, quantise_scale=next_scale)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got_q, want_q)
