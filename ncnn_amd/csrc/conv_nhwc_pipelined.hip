@@ -44,6 +44,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
+    static_assert(STAGES >= 2 && STAGES <= 7 && (STAGES - 2) * (LA + LB) < 64, "the vmcnt field counts to 63");
     constexpr int STAGE_BYTES = (BM + BN) * 64;
     constexpr int EPILOGUE_BYTES = 4 * 32 * (BN / 2 + 4) * 4; // per wavefront 32 pixels x (BN/2 + 4) floats
     constexpr int SMEM_BYTES = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
@@ -167,12 +168,15 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     {
         // this wavefront's loads of step t have landed (later stages may stay in flight) ...
         const int ahead = nk - 1 - t < STAGES - 2 ? nk - 1 - t : STAGES - 2;
-        if (STAGES >= 4 && ahead == 2)
-            WAIT_VMCNT(2 * (LA + LB));
-        else if (ahead == 1)
-            WAIT_VMCNT(LA + LB);
-        else
-            WAIT_VMCNT(0);
+        switch (ahead)
+        {
+        case 0: WAIT_VMCNT(0); break;
+        case 1: WAIT_VMCNT(1 * (LA + LB)); break;
+        case 2: WAIT_VMCNT(2 * (LA + LB)); break;
+        case 3: WAIT_VMCNT(3 * (LA + LB)); break;
+        case 4: WAIT_VMCNT(4 * (LA + LB)); break;
+        default: WAIT_VMCNT(5 * (LA + LB)); break; // STAGES <= 7
+        }
         // ... and everybody's: the barrier also says nobody still reads the stage refilled next
         __builtin_amdgcn_s_barrier();
         if (t + STAGES - 1 < nk) issue(t + STAGES - 1);
@@ -420,6 +424,7 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, out_cp, p.tiles_m, p.tiles_n, \
                                p.steps_per_split, partial);                                                                                     \
     } while (0)
+    // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
     if (p.bm == 128 && p.bn == 256)
         LAUNCH_PIPE(128, 256, 3);
     else if (p.bm == 128 && p.bn == 128)

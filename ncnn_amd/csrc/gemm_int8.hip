@@ -10,8 +10,9 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(DenseOperand a, DenseOpe
     mfma_tile_body<BM, BN, DenseOperand, Epilogue>(a, b, epi, M, N, K, blockIdx.y * BM, blockIdx.x * BN);
 }
 
-// skinny case (one or a few activation rows): one wavefront per output channel streams the
-// weight row with 16-byte loads and reduces with cross-lane adds; no matrix cores involved.
+// skinny case (up to a few dozen activation rows): one wavefront per output channel streams the weight row with
+// 16-byte loads, multiplies it against up to 8 activation rows at a time held in registers (v_dot4_i32_i8) and
+// reduces with cross-lane adds; no matrix cores involved.  The layer is bound by reading the weights once.
 __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__ x, size_t xs, int rows, int K,
                                                        const int8_t* __restrict__ wgt, int num_output, FcEpilogue epi, int vec)
 {
@@ -19,28 +20,46 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__
     const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (p >= num_output) return;
     const int8_t* wr = wgt + (size_t)p * K;
-    for (int r = 0; r < rows; r++)
+    for (int r0 = 0; r0 < rows; r0 += 8)
     {
-        const int8_t* xr = x + (size_t)r * xs;
-        int acc = 0;
+        const int nr = rows - r0 < 8 ? rows - r0 : 8;
+        int acc[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) acc[r] = 0;
         if (vec)
         {
             for (int k = lane * 16; k + 16 <= K; k += 64 * 16)
             {
                 const v4i wv = *reinterpret_cast<const v4i*>(wr + k);
-                const v4i xv = *reinterpret_cast<const v4i*>(xr + k);
 #pragma unroll
-                for (int d = 0; d < 4; d++) acc = __builtin_amdgcn_sdot4(wv[d], xv[d], acc, false);
+                for (int r = 0; r < 8; r++)
+                    if (r < nr)
+                    {
+                        const v4i xv = *reinterpret_cast<const v4i*>(x + (size_t)(r0 + r) * xs + k);
+#pragma unroll
+                        for (int d = 0; d < 4; d++) acc[r] = __builtin_amdgcn_sdot4(wv[d], xv[d], acc[r], false);
+                    }
             }
-            for (int k = (K & ~15) + lane; k < K; k += 64) acc += (int)wr[k] * (int)xr[k];
+            for (int k = (K & ~15) + lane; k < K; k += 64)
+#pragma unroll
+                for (int r = 0; r < 8; r++)
+                    if (r < nr) acc[r] += (int)wr[k] * (int)x[(size_t)(r0 + r) * xs + k];
         }
         else
         {
-            for (int k = lane; k < K; k += 64) acc += (int)wr[k] * (int)xr[k];
+            for (int k = lane; k < K; k += 64)
+#pragma unroll
+                for (int r = 0; r < 8; r++)
+                    if (r < nr) acc[r] += (int)wr[k] * (int)x[(size_t)(r0 + r) * xs + k];
         }
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-        if (lane == 0) epi(p, r, acc);
+        for (int r = 0; r < 8; r++)
+        {
+            int v = acc[r];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0 && r < nr) epi(p, r0 + r, v);
+        }
     }
 }
 
@@ -125,7 +144,7 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
     epi.num_output = num_output;
     epi.acc_out = acc_out_dev;
 
-    if (rows <= 8)
+    if (rows <= 64)
     {
         const int vec = aligned16(x_dev) && aligned16(weight_dev) && x_stride % 16 == 0 && num_input % 16 == 0;
         hipLaunchKernelGGL(fc_gemv_kernel, dim3(ceil_div(num_output, 4)), dim3(256), 0, as_stream(stream), x_dev, x_stride, rows,

@@ -218,7 +218,7 @@ def test_invalid_group_returns_minus_100(rt):
 
 # ----------------------------------------------------------------------------- inner product
 @pytest.mark.parametrize("rows,k,n,act,bias,int8_in", [(1, 2048, 1000, 0, True, False), (1, 1280, 1000, 0, True, True), (1, 33, 7, 1, False, False),
-                                                        (5, 64, 10, 3, True, False), (16, 512, 300, 0, True, False), (70, 100, 130, 1, True, True)])
+                                                        (5, 64, 10, 3, True, False), (16, 512, 300, 0, True, False), (32, 2048, 1000, 0, True, False), (13, 520, 37, 1, True, True), (70, 100, 130, 1, True, True)])
 def test_innerproduct_bit_exact(rt, rows, k, n, act, bias, int8_in):
     _say("innerproduct", rows, k, n, act, bias, int8_in)
     rng = np.random.default_rng(rows + k + n)
