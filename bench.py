@@ -40,9 +40,31 @@ def _elapsed(lib, check, a, b):
     return ms.value
 
 
-def cpu_baseline_gemm(n, k, budget_s=12.0):
-    """Scalar oracle (ncnn's naive loop restated, OpenMP over rows) on a row sample of the same Gemm."""
-    from oracle import oracle
+def cpu_baseline_gemm(n, k, per_col, budget_s=12.0):
+    """The same Gemm on this host's cores, on a row sample: the x86 VNNI restatement of how the reference's CPU path
+    computes it (oracle/cpu_vnni_gemm.c, checked bit for bit against the scalar oracle); the scalar OpenMP oracle when
+    the host has no AVX512-VNNI."""
+    from oracle import cpubaseline, oracle
+    if cpubaseline.available():
+        threads = min(os.cpu_count() or 1, 16)
+        os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+        rng = np.random.default_rng(0)
+        bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+        sb = rng.uniform(40, 60, n if per_col else 1).astype(np.float32)
+        bias = np.zeros(n, np.float32)
+        packed = cpubaseline.pack_b(bq)  # constant weights: packed once, outside the timed region, as at create_pipeline
+        rows = min(n, 1024)
+        a = rng.standard_normal((rows, k), dtype=np.float32)
+        cpubaseline.gemm(a, packed, n, sb, bias)  # warm-up (threads, page faults)
+        times, t_start = [], time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 1000):
+            t0 = time.perf_counter()
+            cpubaseline.gemm(a, packed, n, sb, bias)
+            times.append(time.perf_counter() - t0)
+        dt = float(np.mean(times))
+        return {"value": 2.0 * rows * n * k / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+                "sample": "%d of %d rows of the same Gemm (N=%d, K=%d): per-row quantise + AVX512-VNNI int8 GEMM + dequantise/bias, OpenMP, mean of %d runs "
+                          "(%.1f s in all)" % (rows, n, n, k, len(times), sum(times))}
     threads = min(oracle.num_threads(), 16)
     oracle.set_num_threads(threads)
     rng = np.random.default_rng(0)
@@ -136,7 +158,7 @@ def bench_gemm(args, size):
                      "traffic": measured_traffic("gemm%d" % size), "kernel": "gemm_int8", "ops_per_launch": ops},
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_gemm(n, k)
+        line["cpu_baseline"] = cpu_baseline_gemm(n, k, args.b_scale == "per_column")
     return line
 
 
@@ -196,6 +218,98 @@ def bench_blockquant(args, n, k, m):
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "blockquant8_mfma_kernel" if half else "blockquant8_stream_kernel", "bytes_per_launch": algo},
     }
+
+
+def cpu_baseline_conv(c, h, w, cout, k, pad, budget_s=10.0):
+    """Scalar oracle (ncnn's naive Convolution::forward_int8 restated, OpenMP over output channels) on whole layers."""
+    from oracle import oracle
+    threads = min(oracle.num_threads(), 16)
+    oracle.set_num_threads(threads)
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, (c, h, w)).astype(np.float32)
+    wq = rng.integers(-127, 128, (cout, c, k, k)).astype(np.int8)
+    ws = rng.uniform(50, 100, cout).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, cout).astype(np.float32)
+    d = oracle.make_desc((c, h, w), cout, (k, k), (1, 1), (1, 1), (pad,) * 4, 0.0, 1, 1, 1, 1, (0.0, 0.0))
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t0 < budget_s and reps < 200):
+        oracle.convolution_int8(d, x, wq, b, ws, np.float32(127.0), None)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    oh, ow = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    return {"value": 2.0 * cout * oh * ow * c * k * k / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+            "sample": "%d whole forward passes of the same layer (quantise + convolution + epilogue), scalar OpenMP oracle, %.2f ms each" % (reps, dt * 1e3)}
+
+
+def bench_conv(args, spec):
+    """One Convolution layer, fp32 in -> fp32 out with ReLU (int8_scale_term 1), batch 1 unless stated: the single-layer
+    configuration.  spec = <cin>x<h>x<w>:<cout>:k<k>[:b<batch>].  A step is the layer as it runs inside a device-resident
+    net: Quantize of the fp32 blob + the implicit-GEMM kernel with its fused dequantise/bias/ReLU epilogue, back to back
+    on one stream (the layer is launch/latency bound: about 0.1 us of matrix work)."""
+    import ncnn_amd
+    from ncnn_amd.hip import Activation, ConvDesc, check, lib as load
+    lib = load()
+    rt = ncnn_amd.Runtime(0)
+    st = rt.stream
+    parts = spec.split(":")
+    c, h, w = (int(v) for v in parts[0].split("x"))
+    cout, k = int(parts[1]), int(parts[2][1:])
+    batch = int(parts[3][1:]) if len(parts) > 3 else 1
+    pad = k // 2
+    cp = lib.ncnnhip_padded_channels
+    rng = np.random.default_rng(0)
+    desc = ConvDesc(w, h, c, batch, cout, k, k, 1, 1, 1, 1, pad, pad, pad, pad, 0.0, 1)
+    nb, wb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    check(lib.ncnnhip_conv_nhwc_sizes(C.byref(desc), C.byref(nb), C.byref(wb), C.byref(sb)))
+    wq = rng.integers(-127, 128, cout * c * k * k).astype(np.int8)
+    pk = np.empty(wb.value, np.int8)
+    check(lib.ncnnhip_conv_pack_weights(C.byref(desc), wq.ctypes.data, pk.ctypes.data))
+    xf = np.zeros((batch, h * w, cp(c)), np.float32)
+    xf[:, :, :c] = rng.uniform(-1, 1, (batch, h * w, c))
+    d_x, d_xq = rt.up(xf), ncnn_amd.DeviceBuffer.empty((batch, h * w, cp(c)), np.int8)
+    d_s = rt.up(np.array([127.0], np.float32))
+    d_pk, d_si, d_b = rt.up(pk), rt.up(rng.uniform(1e-4, 1e-3, cout).astype(np.float32)), rt.up(rng.uniform(-0.1, 0.1, cout).astype(np.float32))
+    d_out = ncnn_amd.DeviceBuffer.empty((batch, h * w, cp(cout)), np.float32)
+    d_ws = ncnn_amd.DeviceBuffer(max(sb.value, 4))
+    act = Activation.make(1)
+
+    def quantise():
+        check(lib.ncnnhip_quantize_nhwc(d_x.ptr, d_xq.ptr, batch * h * w, c, d_s.ptr, 1, st))
+
+    def conv():
+        check(lib.ncnnhip_conv_int8_nhwc(C.byref(desc), d_xq.ptr, d_pk.ptr, d_si.ptr, d_b.ptr, None, act, d_out.ptr, 1, 0, 0, d_ws.ptr, sb.value, st))
+
+    for _ in range(args.warmup):
+        quantise()
+        conv()
+    rt.sync()
+    ev = _events(lib, check, 2)
+    check(lib.ncnnhip_event_record(ev[0], st))
+    for _ in range(args.steps):
+        conv()
+    check(lib.ncnnhip_event_record(ev[1], st))
+    check(lib.ncnnhip_event_synchronize(ev[1]))
+    kernel_ms = _elapsed(lib, check, ev[0], ev[1]) / args.steps
+    check(lib.ncnnhip_device_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        quantise()
+        conv()
+    check(lib.ncnnhip_device_synchronize())
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ops = 2.0 * batch * cout * h * w * c * k * k
+    achieved = ops / (kernel_ms * 1e-3) / 1e12
+    line = {
+        "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "Convolution %dx%d %d->%d on %dx%d, batch %d, fp32 in -> quantise -> int8 implicit GEMM -> fp32 out with ReLU; "
+                               "back-to-back launches, channels-last resident blobs" % (k, k, c, cout, h, w, batch), "kernel_us": kernel_ms * 1e3},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
+                     "traffic": None, "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
+    }
+    if not args.no_cpu and batch == 1:
+        line["cpu_baseline"] = cpu_baseline_conv(c, h, w, cout, k, pad)
+    return line
 
 
 def bench_layers(args, which, batch):
@@ -384,7 +498,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
-                    help="gemm<size> | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
+                    help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
     ap.add_argument("--b-scale", dest="b_scale", default="per_column", choices=["per_column", "per_tensor"],
                     help="per_column is the benchmark configuration; per_tensor is what ncnn's Gemm layer can express")
@@ -400,6 +514,8 @@ def main():
     elif args.workload.startswith("blockquant:"):
         n, k, m = (int(v) for v in args.workload.split(":")[1].split("x"))
         line = bench_blockquant(args, n, k, m)
+    elif args.workload.startswith("conv:"):
+        line = bench_conv(args, args.workload[5:])
     elif args.workload.startswith("net:"):
         _, which, batch = args.workload.split(":")
         line = bench_net(args, which, int(batch))

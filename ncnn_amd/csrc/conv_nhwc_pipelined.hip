@@ -381,10 +381,11 @@ static PipePlan plan_pipelined(int cout, long long npix, int steps)
     p.tiles_n = ceil_div(cout, p.bn);
     p.splits = 1;
     const long long t = tiles();
-    if (t < 192 && steps >= 8)
+    if (t < 192 && steps >= 16)
     {
+        // a split costs two more launches (clear + finish): only worth it for long K loops
         const int want = (int)((384 + t - 1) / t);
-        const int max_splits = steps / 4; // at least 4 K steps per split
+        const int max_splits = steps / 8; // at least 8 K steps per split
         p.splits = want < max_splits ? want : max_splits;
         if (p.splits < 1) p.splits = 1;
     }

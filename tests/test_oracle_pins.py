@@ -325,3 +325,26 @@ def test_blockquant_gemm_exact_on_power_of_two_data():
     got = oracle.gemm_blockquant(a, q.view(np.uint8), scales, 8, 64)
     want = (a.astype(np.int64) @ q.astype(np.int64).T) * 0.25
     assert np.array_equal(got, want.astype(F))
+
+
+# ----------------------------------------------------------------------------- the benchmark's x86 baseline
+@pytest.mark.parametrize("m,n,k,per_col", [(7, 50, 96, False), (33, 130, 1000, True), (4, 64, 64, False), (9, 17, 5, True)])
+def test_vnni_cpu_baseline_equals_the_scalar_oracle(m, n, k, per_col):
+    """The VNNI Gemm timed beside the GPU computes the same function as the scalar restatement: same int32 sums,
+    same fp32 results, including rows that quantise through the +-0.5 edge cases."""
+    from oracle import cpubaseline
+    if not cpubaseline.available():
+        pytest.skip("host CPU has no AVX512-VNNI")
+    rng = np.random.default_rng(m * n + k)
+    a = rng.standard_normal((m, k)).astype(F)
+    a[0, :] = 0                                   # zero row: scale 1
+    a[1, : min(k, 4)] = np.array([0.49999997, -0.49999997, 0.5, -0.5], F)[: min(k, 4)]
+    a[1, -1] = F(127.0) if k > 4 else a[1, -1]    # absmax 127 -> scale exactly 1: the values above meet float2int8 raw
+    bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sb = rng.uniform(20, 90, n if per_col else 1).astype(F)
+    bias = rng.standard_normal(n).astype(F)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    want, wacc = oracle.gemm_int8(aq, bq, sa, sb, bias, 4, want_acc=True)
+    got, gacc = cpubaseline.gemm(a, cpubaseline.pack_b(bq), n, sb, bias, want_acc=True)
+    assert np.array_equal(gacc, wacc)
+    assert np.array_equal(got, want)
