@@ -30,12 +30,30 @@ struct ConvFusion
     float q8_scale;
 };
 
+// The same kernel as a plain Gemm (a 1x1 convolution whose "pixels" are the rows of A): Gemm's dequantising epilogue
+//   out = alpha * ((float)acc * (1/(sA_i*sB)) + beta*C)     or, one B scale per column,  ((float)acc * (1/sA_i)) * (1/sB_j)
+// (Gemm::forward_int8, src/layer/gemm.cpp:509-555) replaces the convolution's.
+struct GemmTail
+{
+    const float* a_scales; // [M]
+    const float* b_scales; // [1] or [N]
+    int per_col;
+    const float* c;
+    int bt; // -1 none, 0 scalar, 1/2 per row, 4 per column
+    float alpha, beta;
+};
+
 // int32 words of split-K scratch the pipelined kernel wants for this problem (0: it does not split)
 size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps);
 
 // Launches the pipelined kernel; the caller has checked: zero border byte, channels-last output.
 int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
                                void* workspace, size_t workspace_bytes, hipStream_t stream);
+
+// D[M][N] = A[M][K] * B[N][K]^T through the pipelined kernel; handled = false when the shape does not fit it
+// (K % 64, N % 4, strides, alignment) and the caller should take another kernel.
+int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmTail& tail,
+                                   float* out, size_t out_stride, hipStream_t stream, bool* handled);
 
 } // namespace ncnnhip
 

@@ -38,9 +38,9 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
     return (uint32_t)((int)v[0] & 0xff) | ((uint32_t)((int)v[1] & 0xff) << 8) | ((uint32_t)((int)v[2] & 0xff) << 16) | ((uint32_t)((int)v[3] & 0xff) << 24);
 }
 
-template<int BM, int BN, int STAGES, bool SPLITK>
+template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   ConvFusion fusion, int out_cp, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
+                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
@@ -242,9 +242,65 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     {
         const int ch = col0 + wn * CW + c * 32 + l32;
         real[c] = ch < g.cout; // channels from cout up to out_cp are the blob's zero padding
-        s_in[c] = real[c] ? epi.scale_in[ch] : 0.f;
-        bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : 0.f;
-        s_out[c] = (real[c] && to_int8) ? epi.scale_out[ch] : 0.f;
+        if (GEMM)
+        {
+            // s_in: 1/sB_j (one scale per column) ; bias: beta*C_j (C broadcast per column)
+            s_in[c] = (real[c] && gemm.per_col) ? div_rn(1.f, gemm.b_scales[ch]) : 0.f;
+            bias[c] = (real[c] && gemm.bt == 4) ? mul_rn(gemm.c[ch], gemm.beta) : 0.f;
+            s_out[c] = 0.f;
+        }
+        else
+        {
+            s_in[c] = real[c] ? epi.scale_in[ch] : 0.f;
+            bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : 0.f;
+            s_out[c] = (real[c] && to_int8) ? epi.scale_out[ch] : 0.f;
+        }
+    }
+    if (GEMM)
+    {
+        const float sb0 = gemm.b_scales[0];
+        const float c0 = gemm.bt == 0 ? mul_rn(gemm.c[0], gemm.beta) : 0.f;
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+        {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+            {
+                const int pl = 8 * (r >> 2) + 4 * lhi + (r & 3);
+                int row = row0 + wm * (BM / 2) + a * 32 + pl;
+                if (row >= g.npix) row = g.npix - 1; // rows beyond M are staged but never stored
+                const float sa = gemm.a_scales[row];
+                const float rowscale = gemm.per_col ? div_rn(1.f, sa) : div_rn(1.f, mul_rn(sa, sb0));
+                const float crow = (gemm.bt == 1 || gemm.bt == 2) ? mul_rn(gemm.c[row], gemm.beta) : 0.f;
+#pragma unroll
+                for (int c = 0; c < TN; c++)
+                {
+                    float f = mul_rn((float)acc[a][c][r], rowscale);
+                    if (gemm.per_col) f = mul_rn(f, s_in[c]);
+                    if (gemm.bt == 4)
+                        f = add_rn(f, bias[c]);
+                    else if (gemm.bt == 0)
+                        f = add_rn(f, c0);
+                    else if (gemm.bt >= 0)
+                        f = add_rn(f, crow);
+                    f = mul_rn(f, gemm.alpha);
+                    tile[pl * LD + c * 32 + l32] = f;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < G / 2; it++)
+            {
+                const int idx = it * 64 + lane;
+                const int p = idx / G, j = idx - p * G;
+                const v4f v = *reinterpret_cast<const v4f*>(tile + p * LD + 4 * j);
+                const int pix = row0 + wm * (BM / 2) + a * 32 + p;
+                const int ch4 = col0 + wn * CW + 4 * j;
+                if (pix < g.npix && ch4 < col_limit) *reinterpret_cast<v4f*>(static_cast<float*>(epi.out) + (size_t)pix * out_cp + ch4) = v;
+            }
+            if (a + 1 < TM) __syncthreads();
+        }
+        return;
     }
 
     // the activation type is uniform: branch on it once, outside the unrolled loops
@@ -282,7 +338,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 v4f v = *reinterpret_cast<const v4f*>(tile + p * LD + 4 * j);
                 const int pix = row0 + wm * (BM / 2) + a * 32 + p;
                 const int ch4 = col0 + wn * CW + 4 * j;
-                if (pix < g.npix && ch4 < out_cp)
+                if (pix < g.npix && ch4 < col_limit)
                 {
                     const size_t o = (size_t)pix * out_cp + ch4;
                     if (to_int8)
@@ -415,14 +471,15 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
         hipLaunchKernelGGL(zero_words_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, words);
     }
     dim3 grid((unsigned)blocks), block(256);
+    const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
 #define LAUNCH_PIPE(BM_, BN_, ST_)                                                                                                              \
     do                                                                                                                                          \
     {                                                                                                                                           \
         if (p.splits > 1)                                                                                                                       \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true>), grid, block, 0, stream, wpk, x, g, epi, fusion, out_cp, p.tiles_m, p.tiles_n, \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
                                p.steps_per_split, partial);                                                                                     \
         else                                                                                                                                    \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, out_cp, p.tiles_m, p.tiles_n, \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
                                p.steps_per_split, partial);                                                                                     \
     } while (0)
     // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
@@ -442,6 +499,67 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     if (p.splits > 1)
         hipLaunchKernelGGL(conv_pipelined_finish_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, g.npix, out_cp, g.cout, epi, fusion);
     return launch_status("conv_nhwc_pipelined_kernel");
+}
+
+int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmTail& tail,
+                                   float* out, size_t out_stride, hipStream_t stream, bool* handled)
+{
+    *handled = false;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(aq) | reinterpret_cast<uintptr_t>(bq) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if (K % 64 || N % 4 || aq_stride % 16 || bq_stride != (size_t)K || out_stride % 4 || !aligned || tail.bt == 3) return NCNNHIP_OK;
+    if ((long long)M * (long long)aq_stride >= (1ll << 31)) return NCNNHIP_OK;
+    *handled = true;
+
+    NhwcGeom g;
+    g.H = 1;
+    g.W = M;
+    g.Cp = (int)aq_stride; // one "pixel" per row of A, its channels the K bytes of that row
+    g.kw = g.kh = g.dw = g.dh = g.sw = g.sh = 1;
+    g.pad_top = g.pad_left = 0;
+    g.outw = M;
+    g.outh = 1;
+    g.npix = M;
+    g.ntaps = 1;
+    g.K = K;
+    g.cout = N;
+    g.pad_word = 0;
+    ConvEpilogue epi;
+    epi.scale_in = epi.bias = epi.scale_out = 0;
+    epi.act.type = 0;
+    epi.act.p0 = epi.act.p1 = 0.f;
+    epi.out = out;
+    epi.out_cstep = epi.out_nstep = 0;
+    epi.pix_per_img = M;
+    epi.batch = 1;
+    epi.out_channel0 = 0;
+    epi.num_output = N;
+    epi.acc_out = 0;
+    const ConvFusion no_fusion = {0, 0, 0, 0.f};
+
+    // tiles as for a convolution, never split (Gemm's K loops are long enough to pipeline)
+    PipePlan p = plan_pipelined(N, M, K / 64);
+    p.splits = 1;
+    p.steps_per_split = K / 64;
+    const long long blocks = (long long)p.tiles_m * p.tiles_n;
+    NCNNHIP_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    dim3 grid((unsigned)blocks), block(256);
+#define LAUNCH_GEMM(BM_, BN_)                                                                                                                        \
+    hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
+                       p.tiles_m, p.tiles_n, p.steps_per_split, (int32_t*)0)
+    if (p.bm == 128 && p.bn == 256)
+        LAUNCH_GEMM(128, 256);
+    else if (p.bm == 128 && p.bn == 128)
+        LAUNCH_GEMM(128, 128);
+    else if (p.bm == 128)
+        LAUNCH_GEMM(128, 64);
+    else if (p.bn == 256)
+        LAUNCH_GEMM(64, 256);
+    else if (p.bn == 128)
+        LAUNCH_GEMM(64, 128);
+    else
+        LAUNCH_GEMM(64, 64);
+#undef LAUNCH_GEMM
+    return launch_status("conv_nhwc_pipelined_kernel<gemm>");
 }
 
 } // namespace ncnnhip

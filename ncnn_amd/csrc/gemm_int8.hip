@@ -1,4 +1,5 @@
 // int8 Gemm and InnerProduct launchers on top of the MFMA tile contraction.
+#include "conv_nhwc.h"
 #include "epilogues.h"
 #include "mfma_tile.h"
 
@@ -115,9 +116,28 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
     epi.N = N;
     epi.acc_out = acc_out_dev;
 
+    // big aligned problems: the 256x256 kernel (it needs a few hundred tiles to fill the chip)
     bool handled = false;
-    int ret = launch_gemm_int8_pipelined(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, epi, as_stream(stream), &handled);
-    if (handled) return ret;
+    int ret = NCNNHIP_OK;
+    if ((long long)M * N >= 256ll * 256 * 128)
+    {
+        ret = launch_gemm_int8_pipelined(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, epi, as_stream(stream), &handled);
+        if (handled) return ret;
+    }
+    // anything else with K % 64 == 0: the convolution's pipelined kernel run as a 1x1 convolution over the rows of A
+    if (!output_transpose && !acc_out_dev)
+    {
+        GemmTail tail;
+        tail.a_scales = a_scales_dev;
+        tail.b_scales = b_scales_dev;
+        tail.per_col = epi.per_col;
+        tail.c = c_dev;
+        tail.bt = epi.bt;
+        tail.alpha = alpha;
+        tail.beta = beta;
+        ret = launch_gemm_via_conv_pipelined(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, tail, out_dev, out_stride, as_stream(stream), &handled);
+        if (handled) return ret;
+    }
 
     DenseOperand a = make_dense(aq_dev, aq_stride, M, K);
     DenseOperand b = make_dense(bq_dev, bq_stride, N, K);

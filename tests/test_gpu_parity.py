@@ -86,6 +86,22 @@ def test_gemm_int8_bit_exact(rt, shape, bt, alpha, beta, transpose, per_col):
     got, gacc = rt.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose, want_acc=True)
     assert np.array_equal(gacc, wacc)
     assert np.array_equal(got, want)
+    # without the accumulator dump the launcher may pick a pipelined kernel: same answer
+    assert np.array_equal(rt.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, transpose), want)
+
+
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (100, 64, 64), (333, 260, 192), (64, 1000, 2048), (2048, 2048, 512)])
+@pytest.mark.parametrize("bt,alpha,beta,per_col", [(4, 1.0, 1.0, True), (-1, 1.0, 1.0, False), (1, 0.5, 2.0, False), (0, 1.0, 1.5, True)])
+def test_gemm_int8_mid_sizes_through_the_pipelined_kernels(rt, m, n, k, bt, alpha, beta, per_col):
+    """K % 64 == 0 shapes below the 256x256 kernel's range run as a 1x1 convolution over the rows of A."""
+    _say("gemm_int8 mid", m, n, k, bt, per_col)
+    a, bq, sb, _ = cases.gemm_case(m + n + k + bt, m, n, k, per_col)
+    rng = np.random.default_rng(bt + 20)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    want, _ = npref.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta)
+    assert np.array_equal(rt.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta), want)
 
 
 def test_gemm_int8_1024_cube_against_numpy_int_matmul(rt):
