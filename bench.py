@@ -360,8 +360,10 @@ def bench_layers(args, which, batch):
             else:
                 assert r["group"] == c == cout, "the benchmark nets only hold plain and depthwise convolutions"
                 wq = rng.integers(-127, 128, c * taps).astype(np.int8)
-                pk = np.empty(taps * cp(c), np.int8)
-                check(lib.ncnnhip_dwconv_pack_weights(c, taps, wq.ctypes.data, pk.ctypes.data))
+                nbytes = C.c_size_t()
+                check(lib.ncnnhip_dwconv_packed_bytes(c, r["k"], r["k"], C.byref(nbytes)))
+                pk = np.empty(nbytes.value, np.int8)
+                check(lib.ncnnhip_dwconv_pack_weights(c, r["k"], r["k"], wq.ctypes.data, pk.ctypes.data))
                 plan.update(d_pk=rt.up(pk))
         plans.append(plan)
 

@@ -164,8 +164,11 @@ int ncnnhip_int8_to_f32(const int8_t* src_dev, float* dst_dev, size_t count, voi
 
 /* ConvolutionDepthWise::forward_int8, depthwise branch (channels == group == num_output,
  * src/layer/convolutiondepthwise.cpp:505-559), channels-last int8 in, channels-last int8 (scale_out != NULL) or fp32 out.
- * Weights repacked once to [kh*kw][Cp]; scale_in / bias / scale_out one float per channel. */
-int ncnnhip_dwconv_pack_weights(int channels, int taps, const int8_t* weight_host, int8_t* packed_host);
+ * Weights repacked once (ncnnhip_dwconv_packed_bytes of host memory): [kh*kw][Cp] bytes, for 3x3 kernels followed by each
+ * kernel row as (w0, w1, w2, 0) per channel, the form the v_dot4 kernel multiplies.  scale_in / bias / scale_out: one float
+ * per channel. */
+int ncnnhip_dwconv_packed_bytes(int channels, int kernel_w, int kernel_h, size_t* bytes);
+int ncnnhip_dwconv_pack_weights(int channels, int kernel_w, int kernel_h, const int8_t* weight_host, int8_t* packed_host);
 int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev,
                              const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
                              void* out_nhwc_dev, void* stream);

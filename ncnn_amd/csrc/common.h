@@ -71,6 +71,18 @@ __device__ __forceinline__ int float2int8(float v)
     return q;
 }
 
+// the same value as (float)float2int8(v), computed without leaving the float pipe: round half away from zero as
+// trunc + exact remainder test, clamp with max/min (a NaN comes out as -127 either way), and the x86 conversion quirk
+// of the reference (|v| >= 2^31 converts to INT_MIN, hence -127) as one compare-select
+__device__ __forceinline__ float float2int8_as_float(float v)
+{
+    const float t = truncf(v);
+    const float d = v - t; // exact
+    float r = t + (fabsf(d) >= 0.5f ? copysignf(1.f, v) : 0.f);
+    r = fminf(fmaxf(r, -127.f), 127.f);
+    return fabsf(v) < 2147483648.f ? r : -127.f;
+}
+
 __device__ __forceinline__ float apply_activation(float v, const ncnnhip_activation& a)
 {
     switch (a.type)

@@ -179,30 +179,37 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
         // ... and everybody's: the barrier also says nobody still reads the stage refilled next
         __builtin_amdgcn_s_barrier();
-        if (t + STAGES - 1 < nk) issue(t + STAGES - 1);
-
         const unsigned st = lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
+        // fragment reads of both K halves go out first; the address arithmetic and the global loads of the stage
+        // refilled next are issued while they are in flight
+        v4i fa[2][TM], fb[2][TN];
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
         {
-            v4i fa[TM], fb[TN];
             const unsigned chunk = ks ? ch1 : ch0;
 #pragma unroll
-            for (int a = 0; a < TM; a++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[a]) : "v"(st + rd_a + chunk + (unsigned)(a * 32 * 64)));
+            for (int a = 0; a < TM; a++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[ks][a]) : "v"(st + rd_a + chunk + (unsigned)(a * 32 * 64)));
 #pragma unroll
-            for (int c = 0; c < TN; c++) asm volatile("ds_read_b128 %0, %1" : "=v"(fb[c]) : "v"(st + rd_b + chunk + (unsigned)(c * 32 * 64)));
-            // the reads are asm, so the wait is too; passing each fragment through an (empty) volatile asm after it
-            // keeps the MFMAs, which consume those values, below the wait
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            for (int c = 0; c < TN; c++) asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks][c]) : "v"(st + rd_b + chunk + (unsigned)(c * 32 * 64)));
+        }
+        if (t + STAGES - 1 < nk) issue(t + STAGES - 1);
+        // the reads are asm, so the wait is too; passing each fragment through an (empty) volatile asm after it
+        // keeps the MFMAs, which consume those values, below the wait
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int a = 0; a < TM; a++) asm volatile("" : "+v"(fa[a]));
+        for (int ks = 0; ks < 2; ks++)
+        {
 #pragma unroll
-            for (int c = 0; c < TN; c++) asm volatile("" : "+v"(fb[c]));
+            for (int a = 0; a < TM; a++) asm volatile("" : "+v"(fa[ks][a]));
+#pragma unroll
+            for (int c = 0; c < TN; c++) asm volatile("" : "+v"(fb[ks][c]));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
 #pragma unroll
             for (int a = 0; a < TM; a++)
 #pragma unroll
-                for (int c = 0; c < TN; c++) acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a], fb[c], acc[a][c], 0, 0, 0);
-        }
+                for (int c = 0; c < TN; c++) acc[a][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks][a], fb[ks][c], acc[a][c], 0, 0, 0);
     }
 
     // ---- epilogue: lane = one output channel per 32-column block, registers = pixels
@@ -311,6 +318,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         {
 #pragma unroll
             for (int c = 0; c < TN; c++)
+            {
+                if (col0 + wn * CW + c * 32 >= col_limit) continue; // a whole 32-channel block of tile padding (uniform per wavefront)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                 {
@@ -325,11 +334,36 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                     }
                     else if (ACT != 0)
                         f = apply_activation(f, epi.act);
-                    if (to_int8) f = (float)float2int8(mul_rn(f, s_out[c]));
-                    if (!real[c]) f = 0.f;
+                    if (to_int8) f = float2int8_as_float(mul_rn(f, s_out[c]));
+                    // pad channels carry zero scales and bias: with no activation or ReLU they are zero already
+                    if (ACT != 0 && ACT != 1 && !real[c]) f = 0.f;
                     tile[(8 * (r >> 2) + 4 * lhi + (r & 3)) * LD + c * 32 + l32] = f;
                 }
+            }
             __syncthreads();
+            if (to_int8)
+            {
+                // 16 channels of one pixel per lane: four LDS reads, one 16-byte store
+                constexpr int G16 = CW / 16;
+                constexpr int ITS = G16 / 2 > 0 ? G16 / 2 : 1;
+#pragma unroll
+                for (int it = 0; it < ITS; it++)
+                {
+                    const int idx = it * 64 + lane;
+                    const int p = idx / G16, j = idx - p * G16;
+                    const int pix = row0 + wm * (BM / 2) + a * 32 + p;
+                    const int ch16 = col0 + wn * CW + 16 * j;
+                    if (p < 32 && pix < g.npix && ch16 < col_limit)
+                    {
+                        v4i pk;
+#pragma unroll
+                        for (int w4 = 0; w4 < 4; w4++) pk[w4] = (int)pack4(*reinterpret_cast<const v4f*>(tile + p * LD + 16 * j + 4 * w4));
+                        *reinterpret_cast<v4i*>(static_cast<int8_t*>(epi.out) + (size_t)pix * out_cp + ch16) = pk;
+                    }
+                }
+            }
+            else
+            {
 #pragma unroll
             for (int it = 0; it < G / 2; it++)
             {
@@ -341,9 +375,6 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 if (pix < g.npix && ch4 < col_limit)
                 {
                     const size_t o = (size_t)pix * out_cp + ch4;
-                    if (to_int8)
-                        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(epi.out) + o) = pack4(v);
-                    else
                     {
                         if (fusion.residual)
                         {
@@ -361,11 +392,12 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                         {
                             v4f q;
 #pragma unroll
-                            for (int e = 0; e < 4; e++) q[e] = (float)float2int8(mul_rn(v[e], fusion.q8_scale));
+                            for (int e = 0; e < 4; e++) q[e] = float2int8_as_float(mul_rn(v[e], fusion.q8_scale));
                             *reinterpret_cast<uint32_t*>(fusion.q8_out + o) = pack4(q);
                         }
                     }
                 }
+            }
             }
             if (a + 1 < TM) __syncthreads();
         }
@@ -430,14 +462,16 @@ static PipePlan plan_pipelined(int cout, long long npix, int steps)
         p.bn = (ceil_div(cout, 256) * 256 <= ceil_div(cout, 128) * 128) ? 256 : 128;
     p.bm = 128;
     auto tiles = [&]() { return (long long)ceil_div(npix, p.bm) * ceil_div(cout, p.bn); };
-    if (tiles() < 512) p.bm = 64;
-    if (tiles() < 256 && p.bn == 256) p.bn = 128;
-    if (tiles() < 256 && p.bn == 128 && cout > 64) p.bn = 64;
+    // measured over the ResNet-50 / MobileNetV2 layers: more, smaller workgroups win until there are a few
+    // thousand of them (these layers are latency bound, not matrix-core bound)
+    if (tiles() < 100000) p.bm = 64;
+    if (tiles() < 1024 && p.bn == 256) p.bn = 128;
+    if (tiles() < 512 && p.bn == 128 && cout > 64) p.bn = 64;
     p.tiles_m = ceil_div(npix, p.bm);
     p.tiles_n = ceil_div(cout, p.bn);
     p.splits = 1;
     const long long t = tiles();
-    if (t < 192 && steps >= 16)
+    if (t < 128 && steps >= 32)
     {
         // a split costs two more launches (clear + finish): only worth it for long K loops
         const int want = (int)((384 + t - 1) / t);

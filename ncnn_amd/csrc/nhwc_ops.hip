@@ -168,12 +168,10 @@ __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restri
             for (int kx = 0; kx < g.kw; kx++)
             {
                 const int y = y0 + ky, x = x0 + kx;
-                if ((unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w)
-                {
-                    const v4f v = *reinterpret_cast<const v4f*>(base + ((size_t)y * g.w + x) * g.cp);
+                const bool in = (unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w;
+                const v4f v = *reinterpret_cast<const v4f*>(base + (in ? ((size_t)y * g.w + x) * g.cp : (size_t)0)); // unconditional: loads overlap
 #pragma unroll
-                    for (int e = 0; e < 4; e++) r[e] = fmaxf(r[e], v[e]);
-                }
+                for (int e = 0; e < 4; e++) r[e] = in ? fmaxf(r[e], v[e]) : r[e];
             }
     }
     else
@@ -296,8 +294,9 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
         for (int kx = 0; kx < g.kw; kx++)
         {
             const int y = y0 + ky * g.dh, xx = x0 + kx * g.dw;
-            v4i v = {padw, padw, padw, padw};
-            if ((unsigned)y < (unsigned)g.h && (unsigned)xx < (unsigned)g.w) v = *reinterpret_cast<const v4i*>(base + ((size_t)y * g.w + xx) * g.cp);
+            const bool in = (unsigned)y < (unsigned)g.h && (unsigned)xx < (unsigned)g.w;
+            v4i v = *reinterpret_cast<const v4i*>(base + (in ? ((size_t)y * g.w + xx) * g.cp : (size_t)0)); // unconditional: loads can overlap
+            if (!in) v = v4i{padw, padw, padw, padw};
             const v4i wv = *reinterpret_cast<const v4i*>(wpk + (size_t)(ky * g.kw + kx) * g.cp + q0);
 #pragma unroll
             for (int wd = 0; wd < 4; wd++)
@@ -318,7 +317,7 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
             r = mul_rn((float)acc[e], scale_in[q]);
             if (bias) r = add_rn(r, bias[q]);
             r = apply_activation(r, act);
-            if (!g.out_f32) r = (float)float2int8(mul_rn(r, scale_out[q]));
+            if (!g.out_f32) r = float2int8_as_float(mul_rn(r, scale_out[q]));
         }
         f[e] = r;
     }
@@ -339,6 +338,125 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
             pk[wd] = (int)word;
         }
         *reinterpret_cast<v4i*>(static_cast<int8_t*>(out) + o) = pk;
+    }
+}
+
+// 3x3, dilation 1: the matrix-free fast path.  v_dot4_i32_i8 sums four byte products of one dword pair, so the four
+// bytes must be four TAPS of one channel: the kernel transposes 4 neighbouring input pixels x 4 channels (bytes) with
+// 8 v_perm_b32 into 4 dwords "one channel, pixels x0..x0+3" and multiplies them against weights packed per channel and
+// kernel row as (w0, w1, w2, 0).  With stride 1 the same transposed dwords serve the next output too, against the
+// weights shifted one byte up (0, w0, w1, w2): a thread computes two adjacent outputs of 16 channels from 12 loads.
+template<int STRIDE>
+__global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __restrict__ x, const uint32_t* __restrict__ wrow /* [3][cp] */, DwNhwcGeom g,
+                                                              const float* __restrict__ scale_in, const float* __restrict__ bias,
+                                                              const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out, size_t total,
+                                                              int xgroups)
+{
+    constexpr int OUTS = STRIDE == 1 ? 2 : 1;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int chunks = g.cp / 16;
+    const int q0 = (int)(i % (size_t)chunks) * 16;
+    size_t rest = i / (size_t)chunks;
+    const int xg = (int)(rest % (size_t)xgroups);
+    rest /= (size_t)xgroups;
+    const int oy = (int)(rest % (size_t)g.outh);
+    const int img = (int)(rest / (size_t)g.outh);
+    const int ox0 = xg * OUTS;
+    const int8_t* base = x + (size_t)img * g.h * g.w * g.cp + q0;
+    const int y0 = oy * STRIDE - g.pad_top, x0 = ox0 * STRIDE - g.pad_left;
+    const int padw = (int)((uint32_t)(g.pad_byte & 0xff) * 0x01010101u);
+
+    int acc[OUTS][16];
+#pragma unroll
+    for (int o = 0; o < OUTS; o++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[o][e] = 0;
+
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++)
+    {
+        const int y = y0 + ky;
+        const bool yok = (unsigned)y < (unsigned)g.h;
+        v4i d[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+        {
+            // the load is unconditional (from the sample's first pixel when the tap is outside) so that all twelve can be
+            // in flight together; a guarded load would be waited for on the spot
+            const int xx = x0 + p;
+            const bool in = yok && (unsigned)xx < (unsigned)g.w && (p < 3 || OUTS == 2);
+            const v4i v = *reinterpret_cast<const v4i*>(base + (in ? ((size_t)y * g.w + xx) * g.cp : (size_t)0));
+            d[p] = in ? v : v4i{padw, padw, padw, padw};
+        }
+        const uint32_t* wr = wrow + (size_t)ky * g.cp + q0;
+#pragma unroll
+        for (int quad = 0; quad < 4; quad++)
+        {
+            const v4i wv = *reinterpret_cast<const v4i*>(wr + quad * 4); // 4 channels x (w0,w1,w2,0)
+            const uint32_t a0 = (uint32_t)d[0][quad], a1 = (uint32_t)d[1][quad], a2 = (uint32_t)d[2][quad], a3 = (uint32_t)d[3][quad];
+            // 4x4 byte transpose: t[c] = (pixel0.c, pixel1.c, pixel2.c, pixel3.c)
+            const uint32_t p01l = __builtin_amdgcn_perm(a1, a0, 0x05010400u), p01h = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
+            const uint32_t p23l = __builtin_amdgcn_perm(a3, a2, 0x05010400u), p23h = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
+            const uint32_t t[4] = {__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), __builtin_amdgcn_perm(p23l, p01l, 0x07060302u),
+                                   __builtin_amdgcn_perm(p23h, p01h, 0x05040100u), __builtin_amdgcn_perm(p23h, p01h, 0x07060302u)};
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+            {
+                acc[0][quad * 4 + c] = __builtin_amdgcn_sdot4((int)t[c], wv[c], acc[0][quad * 4 + c], false);
+                if (OUTS == 2) acc[1][quad * 4 + c] = __builtin_amdgcn_sdot4((int)t[c], (int)((uint32_t)wv[c] << 8), acc[1][quad * 4 + c], false);
+            }
+        }
+    }
+
+    float s_in[16], s_b[16], s_out[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++)
+    {
+        const int q = q0 + e < g.c ? q0 + e : g.c - 1; // clamped: the loads stay unconditional
+        s_in[e] = scale_in[q];
+        s_b[e] = bias ? bias[q] : 0.f;
+        s_out[e] = g.out_f32 ? 0.f : scale_out[q];
+    }
+#pragma unroll
+    for (int o = 0; o < OUTS; o++)
+    {
+        const int ox = ox0 + o;
+        if (ox >= g.outw) continue;
+        const size_t off = (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q0;
+        float f[16];
+#pragma unroll
+        for (int e = 0; e < 16; e++)
+        {
+            const int q = q0 + e;
+            float r = 0.f;
+            if (q < g.c)
+            {
+                r = mul_rn((float)acc[o][e], s_in[e]);
+                if (bias) r = add_rn(r, s_b[e]);
+                r = apply_activation(r, act);
+                if (!g.out_f32) r = float2int8_as_float(mul_rn(r, s_out[e]));
+            }
+            f[e] = r;
+        }
+        if (g.out_f32)
+        {
+#pragma unroll
+            for (int wd = 0; wd < 4; wd++) *reinterpret_cast<v4f*>(static_cast<float*>(out) + off + wd * 4) = v4f{f[wd * 4], f[wd * 4 + 1], f[wd * 4 + 2], f[wd * 4 + 3]};
+        }
+        else
+        {
+            v4i pk;
+#pragma unroll
+            for (int wd = 0; wd < 4; wd++)
+            {
+                uint32_t word = 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) word |= (uint32_t)((int)f[wd * 4 + e] & 0xff) << (8 * e);
+                pk[wd] = (int)word;
+            }
+            *reinterpret_cast<v4i*>(static_cast<int8_t*>(out) + off) = pk;
+        }
     }
 }
 
@@ -484,12 +602,33 @@ int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, 
     return launch_status("softmax_kernel");
 }
 
-int ncnnhip_dwconv_pack_weights(int channels, int taps, const int8_t* weight_host, int8_t* packed_host)
+static size_t dwconv_packed_bytes(int channels, int kernel_w, int kernel_h)
 {
-    NCNNHIP_REQUIRE(channels > 0 && taps > 0 && weight_host && packed_host, "ncnnhip_dwconv_pack_weights: bad argument");
-    const int cp = padded16(channels);
+    const size_t cp = (size_t)padded16(channels);
+    // [taps][cp] bytes, then for a 3x3 kernel [3][cp] dwords holding each kernel row as (w0, w1, w2, 0)
+    return (size_t)kernel_w * kernel_h * cp + ((kernel_w == 3 && kernel_h == 3) ? 3 * cp * 4 : 0);
+}
+
+int ncnnhip_dwconv_packed_bytes(int channels, int kernel_w, int kernel_h, size_t* bytes)
+{
+    NCNNHIP_REQUIRE(channels > 0 && kernel_w > 0 && kernel_h > 0 && bytes, "ncnnhip_dwconv_packed_bytes: bad argument");
+    *bytes = dwconv_packed_bytes(channels, kernel_w, kernel_h);
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_dwconv_pack_weights(int channels, int kernel_w, int kernel_h, const int8_t* weight_host, int8_t* packed_host)
+{
+    NCNNHIP_REQUIRE(channels > 0 && kernel_w > 0 && kernel_h > 0 && weight_host && packed_host, "ncnnhip_dwconv_pack_weights: bad argument");
+    const int cp = padded16(channels), taps = kernel_w * kernel_h;
     for (int t = 0; t < taps; t++)
         for (int q = 0; q < cp; q++) packed_host[(size_t)t * cp + q] = q < channels ? weight_host[(size_t)q * taps + t] : (int8_t)0;
+    if (kernel_w == 3 && kernel_h == 3)
+    {
+        int8_t* rows = packed_host + (size_t)taps * cp;
+        for (int ky = 0; ky < 3; ky++)
+            for (int q = 0; q < cp; q++)
+                for (int kx = 0; kx < 4; kx++) rows[((size_t)ky * cp + q) * 4 + kx] = (q < channels && kx < 3) ? weight_host[(size_t)q * 9 + ky * 3 + kx] : (int8_t)0;
+    }
     return NCNNHIP_OK;
 }
 
@@ -522,6 +661,21 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
     g.pad_left = pad_left;
     g.pad_byte = (int)(signed char)d.pad_value;
     g.out_f32 = scale_out_dev ? 0 : 1;
+    if (d.kernel_w == 3 && d.kernel_h == 3 && d.dilation_w == 1 && d.dilation_h == 1 && d.stride_w == d.stride_h && (d.stride_w == 1 || d.stride_w == 2))
+    {
+        const uint32_t* wrow = reinterpret_cast<const uint32_t*>(packed_weight_dev + (size_t)9 * g.cp);
+        const int outs = d.stride_w == 1 ? 2 : 1;
+        const int xgroups = ceil_div(outw, outs);
+        const size_t threads = (size_t)d.batch * outh * xgroups * (g.cp / 16);
+        dim3 grid3(ceil_div((long long)threads, 256));
+        if (d.stride_w == 1)
+            hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<1>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
+                               out_nhwc_dev, threads, xgroups);
+        else
+            hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<2>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
+                               out_nhwc_dev, threads, xgroups);
+        return launch_status("dwconv3x3_nhwc_kernel");
+    }
     const size_t total = (size_t)d.batch * outh * outw * (g.cp / 16);
     hipLaunchKernelGGL(dwconv_nhwc_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), nhwc_dev, packed_weight_dev, g, scale_in_dev,
                        bias_dev, scale_out_dev, act, out_nhwc_dev, total);

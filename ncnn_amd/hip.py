@@ -82,7 +82,8 @@ _SIGNATURES = {
     "ncnnhip_nhwc_to_chw": [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p],
     "ncnnhip_quantize_nhwc": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_void_p],
     "ncnnhip_int8_to_f32": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
-    "ncnnhip_dwconv_pack_weights": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_dwconv_packed_bytes": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
+    "ncnnhip_dwconv_pack_weights": [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_dwconv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_void_p],
     "ncnnhip_relu": [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p],
     "ncnnhip_scale": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_void_p],
@@ -399,9 +400,10 @@ class Runtime:
             check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
                                                1, 0, 0, dws.ptr, sb_.value, self.stream))
         else:
-            taps = kernel[0] * kernel[1]
-            pk = np.empty(taps * src.shape[2], np.int8)
-            check(lib().ncnnhip_dwconv_pack_weights(c, taps, wq.ctypes.data, pk.ctypes.data))
+            nbytes = C.c_size_t()
+            check(lib().ncnnhip_dwconv_packed_bytes(c, kernel[0], kernel[1], C.byref(nbytes)))
+            pk = np.empty(nbytes.value, np.int8)
+            check(lib().ncnnhip_dwconv_pack_weights(c, kernel[0], kernel[1], wq.ctypes.data, pk.ctypes.data))
             dpk = self.up(pk)
             check(lib().ncnnhip_dwconv_int8_nhwc(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr, self.stream))
         raw = dout.to_numpy(self.stream)

@@ -196,9 +196,11 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
     if (ret == 0 && is_depthwise())
     {
         // device-resident form of the depthwise kernel: weights as [tap][padded channels]
-        const int taps = kernel_w * kernel_h;
-        std::vector<int8_t> packed((size_t)taps * ncnnhip_padded_channels(num_output));
-        rc = ncnnhip_dwconv_pack_weights(num_output, taps, (const int8_t*)weight_data.data, packed.data());
+        size_t packed_bytes = 0;
+        rc = ncnnhip_dwconv_packed_bytes(num_output, kernel_w, kernel_h, &packed_bytes);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_dwconv_packed_bytes");
+        std::vector<int8_t> packed(packed_bytes);
+        rc = ncnnhip_dwconv_pack_weights(num_output, kernel_w, kernel_h, (const int8_t*)weight_data.data, packed.data());
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_dwconv_pack_weights");
         ret = upload_constant(packed.data(), packed.size(), &d_weight_dw);
     }
