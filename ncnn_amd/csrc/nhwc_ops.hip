@@ -341,123 +341,73 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
     }
 }
 
-// 3x3, dilation 1: the matrix-free fast path.  v_dot4_i32_i8 sums four byte products of one dword pair, so the four
-// bytes must be four TAPS of one channel: the kernel transposes 4 neighbouring input pixels x 4 channels (bytes) with
-// 8 v_perm_b32 into 4 dwords "one channel, pixels x0..x0+3" and multiplies them against weights packed per channel and
-// kernel row as (w0, w1, w2, 0).  With stride 1 the same transposed dwords serve the next output too, against the
-// weights shifted one byte up (0, w0, w1, w2): a thread computes two adjacent outputs of 16 channels from 12 loads.
+// 3x3, dilation 1: the fast path.  v_dot4_i32_i8 sums four byte products of one dword pair, so the four bytes must be
+// four TAPS of one channel: a thread owns 4 channels of one output pixel, loads the 3x3 input pixels as dwords (4
+// channels each), transposes each kernel row (3 pixels + a zero) with 8 v_perm_b32 into "one channel, pixels x0..x0+3"
+// and multiplies against weights packed per channel and kernel row as (w0, w1, w2, 0).  Consecutive lanes are
+// consecutive channel quads of a pixel, so every load and store of a wavefront is one contiguous run; ~40 VGPRs.
 template<int STRIDE>
 __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __restrict__ x, const uint32_t* __restrict__ wrow /* [3][cp] */, DwNhwcGeom g,
                                                               const float* __restrict__ scale_in, const float* __restrict__ bias,
-                                                              const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out, size_t total,
-                                                              int xgroups)
+                                                              const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out, size_t total)
 {
-    constexpr int OUTS = STRIDE == 1 ? 2 : 1;
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
-    const int chunks = g.cp / 16;
-    const int q0 = (int)(i % (size_t)chunks) * 16;
-    size_t rest = i / (size_t)chunks;
-    const int xg = (int)(rest % (size_t)xgroups);
-    rest /= (size_t)xgroups;
-    const int oy = (int)(rest % (size_t)g.outh);
-    const int img = (int)(rest / (size_t)g.outh);
-    const int ox0 = xg * OUTS;
+    const unsigned quads = (unsigned)g.cp / 4;
+    const unsigned q0 = (unsigned)(i % quads) * 4;
+    const unsigned pix = (unsigned)(i / quads); // < 2^32: checked by the launcher
+    const unsigned ox = pix % (unsigned)g.outw;
+    const unsigned rowi = pix / (unsigned)g.outw;
+    const unsigned oy = rowi % (unsigned)g.outh;
+    const unsigned img = rowi / (unsigned)g.outh;
     const int8_t* base = x + (size_t)img * g.h * g.w * g.cp + q0;
-    const int y0 = oy * STRIDE - g.pad_top, x0 = ox0 * STRIDE - g.pad_left;
-    const int padw = (int)((uint32_t)(g.pad_byte & 0xff) * 0x01010101u);
+    const int y0 = (int)oy * STRIDE - g.pad_top, x0 = (int)ox * STRIDE - g.pad_left;
+    const uint32_t padw = (uint32_t)(g.pad_byte & 0xff) * 0x01010101u;
 
-    int acc[OUTS][16];
-#pragma unroll
-    for (int o = 0; o < OUTS; o++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[o][e] = 0;
-
+    int acc[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int ky = 0; ky < 3; ky++)
     {
         const int y = y0 + ky;
         const bool yok = (unsigned)y < (unsigned)g.h;
-        v4i d[4];
+        uint32_t d[3];
 #pragma unroll
-        for (int p = 0; p < 4; p++)
+        for (int p = 0; p < 3; p++)
         {
-            // the load is unconditional (from the sample's first pixel when the tap is outside) so that all twelve can be
-            // in flight together; a guarded load would be waited for on the spot
+            // unconditional load (from the sample's first pixel when the tap is outside): all nine can be in flight
             const int xx = x0 + p;
-            const bool in = yok && (unsigned)xx < (unsigned)g.w && (p < 3 || OUTS == 2);
-            const v4i v = *reinterpret_cast<const v4i*>(base + (in ? ((size_t)y * g.w + xx) * g.cp : (size_t)0));
-            d[p] = in ? v : v4i{padw, padw, padw, padw};
+            const bool in = yok && (unsigned)xx < (unsigned)g.w;
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(base + (in ? ((size_t)y * g.w + xx) * g.cp : (size_t)0));
+            d[p] = in ? v : padw;
         }
-        const uint32_t* wr = wrow + (size_t)ky * g.cp + q0;
-#pragma unroll
-        for (int quad = 0; quad < 4; quad++)
-        {
-            const v4i wv = *reinterpret_cast<const v4i*>(wr + quad * 4); // 4 channels x (w0,w1,w2,0)
-            const uint32_t a0 = (uint32_t)d[0][quad], a1 = (uint32_t)d[1][quad], a2 = (uint32_t)d[2][quad], a3 = (uint32_t)d[3][quad];
-            // 4x4 byte transpose: t[c] = (pixel0.c, pixel1.c, pixel2.c, pixel3.c)
-            const uint32_t p01l = __builtin_amdgcn_perm(a1, a0, 0x05010400u), p01h = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
-            const uint32_t p23l = __builtin_amdgcn_perm(a3, a2, 0x05010400u), p23h = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
-            const uint32_t t[4] = {__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), __builtin_amdgcn_perm(p23l, p01l, 0x07060302u),
-                                   __builtin_amdgcn_perm(p23h, p01h, 0x05040100u), __builtin_amdgcn_perm(p23h, p01h, 0x07060302u)};
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-            {
-                acc[0][quad * 4 + c] = __builtin_amdgcn_sdot4((int)t[c], wv[c], acc[0][quad * 4 + c], false);
-                if (OUTS == 2) acc[1][quad * 4 + c] = __builtin_amdgcn_sdot4((int)t[c], (int)((uint32_t)wv[c] << 8), acc[1][quad * 4 + c], false);
-            }
-        }
+        const v4i wv = *reinterpret_cast<const v4i*>(wrow + (size_t)ky * g.cp + q0); // 4 channels x (w0,w1,w2,0)
+        // 4x4 byte transpose of (d0,d1,d2,0): t[c] = (pixel0.c, pixel1.c, pixel2.c, 0)
+        const uint32_t p01l = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), p01h = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+        const uint32_t p23l = __builtin_amdgcn_perm(0u, d[2], 0x05010400u), p23h = __builtin_amdgcn_perm(0u, d[2], 0x07030602u);
+        acc[0] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), wv[0], acc[0], false);
+        acc[1] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23l, p01l, 0x07060302u), wv[1], acc[1], false);
+        acc[2] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23h, p01h, 0x05040100u), wv[2], acc[2], false);
+        acc[3] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23h, p01h, 0x07060302u), wv[3], acc[3], false);
     }
 
-    float s_in[16], s_b[16], s_out[16];
+    const size_t off = (size_t)pix * g.cp + q0;
+    float f[4];
 #pragma unroll
-    for (int e = 0; e < 16; e++)
+    for (int e = 0; e < 4; e++)
     {
-        const int q = q0 + e < g.c ? q0 + e : g.c - 1; // clamped: the loads stay unconditional
-        s_in[e] = scale_in[q];
-        s_b[e] = bias ? bias[q] : 0.f;
-        s_out[e] = g.out_f32 ? 0.f : scale_out[q];
+        const int q = (int)q0 + e;
+        const int qc = q < g.c ? q : g.c - 1; // clamped: the table loads stay unconditional
+        float r = mul_rn((float)acc[e], scale_in[qc]);
+        if (bias) r = add_rn(r, bias[qc]);
+        r = apply_activation(r, act);
+        if (!g.out_f32) r = float2int8_as_float(mul_rn(r, scale_out[qc]));
+        f[e] = q < g.c ? r : 0.f;
     }
-#pragma unroll
-    for (int o = 0; o < OUTS; o++)
-    {
-        const int ox = ox0 + o;
-        if (ox >= g.outw) continue;
-        const size_t off = (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q0;
-        float f[16];
-#pragma unroll
-        for (int e = 0; e < 16; e++)
-        {
-            const int q = q0 + e;
-            float r = 0.f;
-            if (q < g.c)
-            {
-                r = mul_rn((float)acc[o][e], s_in[e]);
-                if (bias) r = add_rn(r, s_b[e]);
-                r = apply_activation(r, act);
-                if (!g.out_f32) r = float2int8_as_float(mul_rn(r, s_out[e]));
-            }
-            f[e] = r;
-        }
-        if (g.out_f32)
-        {
-#pragma unroll
-            for (int wd = 0; wd < 4; wd++) *reinterpret_cast<v4f*>(static_cast<float*>(out) + off + wd * 4) = v4f{f[wd * 4], f[wd * 4 + 1], f[wd * 4 + 2], f[wd * 4 + 3]};
-        }
-        else
-        {
-            v4i pk;
-#pragma unroll
-            for (int wd = 0; wd < 4; wd++)
-            {
-                uint32_t word = 0;
-#pragma unroll
-                for (int e = 0; e < 4; e++) word |= (uint32_t)((int)f[wd * 4 + e] & 0xff) << (8 * e);
-                pk[wd] = (int)word;
-            }
-            *reinterpret_cast<v4i*>(static_cast<int8_t*>(out) + off) = pk;
-        }
-    }
+    if (g.out_f32)
+        *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
+    else
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
+            (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
 }
 
 static inline int padded16(int c)
@@ -664,16 +614,16 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
     if (d.kernel_w == 3 && d.kernel_h == 3 && d.dilation_w == 1 && d.dilation_h == 1 && d.stride_w == d.stride_h && (d.stride_w == 1 || d.stride_w == 2))
     {
         const uint32_t* wrow = reinterpret_cast<const uint32_t*>(packed_weight_dev + (size_t)9 * g.cp);
-        const int outs = d.stride_w == 1 ? 2 : 1;
-        const int xgroups = ceil_div(outw, outs);
-        const size_t threads = (size_t)d.batch * outh * xgroups * (g.cp / 16);
+        const size_t pixels = (size_t)d.batch * outh * outw;
+        NCNNHIP_REQUIRE(pixels < (1ull << 32), "ncnnhip_dwconv_int8_nhwc: more than 2^32 output pixels");
+        const size_t threads = pixels * (g.cp / 4);
         dim3 grid3(ceil_div((long long)threads, 256));
         if (d.stride_w == 1)
             hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<1>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, threads, xgroups);
+                               out_nhwc_dev, threads);
         else
             hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<2>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, threads, xgroups);
+                               out_nhwc_dev, threads);
         return launch_status("dwconv3x3_nhwc_kernel");
     }
     const size_t total = (size_t)d.batch * outh * outw * (g.cp / 16);
