@@ -342,72 +342,128 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
 }
 
 // 3x3, dilation 1: the fast path.  v_dot4_i32_i8 sums four byte products of one dword pair, so the four bytes must be
-// four TAPS of one channel: a thread owns 4 channels of one output pixel, loads the 3x3 input pixels as dwords (4
-// channels each), transposes each kernel row (3 pixels + a zero) with 8 v_perm_b32 into "one channel, pixels x0..x0+3"
-// and multiplies against weights packed per channel and kernel row as (w0, w1, w2, 0).  Consecutive lanes are
-// consecutive channel quads of a pixel, so every load and store of a wavefront is one contiguous run; ~40 VGPRs.
+// four TAPS of one channel: a thread owns 4 channels of OUTS adjacent output pixels, loads each kernel row's input
+// pixels as dwords (4 channels each), transposes them with 8 v_perm_b32 into "one channel, pixels x0..x0+3" and
+// multiplies against weights packed per channel and kernel row as (w0, w1, w2, 0).  At stride 1 the same transposed
+// dwords serve the next output pixel against the weights shifted one byte up, (0, w0, w1, w2), so OUTS = 2.
+// Consecutive lanes are consecutive channel quads of a pixel: every load and store of a wavefront is a contiguous
+// run.  The kernel is bound by VALU issue (index arithmetic + ~20 single-rounded fp32 instructions of requantising
+// epilogue per output), so everything per-thread is amortised over as many outputs as the registers allow.
 template<int STRIDE>
 __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __restrict__ x, const uint32_t* __restrict__ wrow /* [3][cp] */, DwNhwcGeom g,
                                                               const float* __restrict__ scale_in, const float* __restrict__ bias,
-                                                              const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out, size_t total)
+                                                              const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out,
+                                                              unsigned quads, unsigned quads_magic, unsigned xgroups)
 {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const unsigned quads = (unsigned)g.cp / 4;
-    const unsigned q0 = (unsigned)(i % quads) * 4;
-    const unsigned pix = (unsigned)(i / quads); // < 2^32: checked by the launcher
-    const unsigned ox = pix % (unsigned)g.outw;
-    const unsigned rowi = pix / (unsigned)g.outw;
-    const unsigned oy = rowi % (unsigned)g.outh;
-    const unsigned img = rowi / (unsigned)g.outh;
+    constexpr int OUTS = STRIDE == 1 ? 2 : 1;
+    constexpr int PIX = STRIDE == 1 ? 4 : 3; // input pixels per kernel row
+    // blockIdx.y = output row (sample * outh + oy); within the row a thread is (x group, channel quad), quads fastest.
+    // xg = r / quads by multiplication with ceil(2^32 / quads), exact here because r * quads < 2^32
+    const unsigned r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= xgroups * quads) return;
+    unsigned xg = __umulhi(r, quads_magic);
+    if (xg * quads > r) xg--;
+    const unsigned q0 = (r - xg * quads) * 4;
+    const unsigned ox0 = xg * OUTS;
+    const unsigned oy = blockIdx.y % (unsigned)g.outh;
+    const unsigned img = blockIdx.y / (unsigned)g.outh;
     const int8_t* base = x + (size_t)img * g.h * g.w * g.cp + q0;
-    const int y0 = (int)oy * STRIDE - g.pad_top, x0 = (int)ox * STRIDE - g.pad_left;
+    const int y0 = (int)oy * STRIDE - g.pad_top, x0 = (int)ox0 * STRIDE - g.pad_left;
     const uint32_t padw = (uint32_t)(g.pad_byte & 0xff) * 0x01010101u;
 
-    int acc[4] = {0, 0, 0, 0};
+    // column offsets (clamped into the image so that every load is unconditional) and their validity
+    unsigned xoff[PIX];
+    bool xin[PIX];
+#pragma unroll
+    for (int p = 0; p < PIX; p++)
+    {
+        const int xx = x0 + p;
+        xin[p] = (unsigned)xx < (unsigned)g.w;
+        xoff[p] = (unsigned)(xin[p] ? xx : 0) * (unsigned)g.cp;
+    }
+
+    int acc[OUTS][4];
+#pragma unroll
+    for (int o = 0; o < OUTS; o++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[o][e] = 0;
 #pragma unroll
     for (int ky = 0; ky < 3; ky++)
     {
         const int y = y0 + ky;
-        const bool yok = (unsigned)y < (unsigned)g.h;
-        uint32_t d[3];
+        const bool yin = (unsigned)y < (unsigned)g.h;
+        const unsigned rowoff = (unsigned)(yin ? y : 0) * (unsigned)g.w * (unsigned)g.cp; // one sample < 2^31 bytes
+        uint32_t d[4];
 #pragma unroll
-        for (int p = 0; p < 3; p++)
+        for (int p = 0; p < PIX; p++)
         {
-            // unconditional load (from the sample's first pixel when the tap is outside): all nine can be in flight
-            const int xx = x0 + p;
-            const bool in = yok && (unsigned)xx < (unsigned)g.w;
-            const uint32_t v = *reinterpret_cast<const uint32_t*>(base + (in ? ((size_t)y * g.w + xx) * g.cp : (size_t)0));
-            d[p] = in ? v : padw;
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(base + rowoff + xoff[p]);
+            d[p] = (yin && xin[p]) ? v : padw;
         }
+        if (PIX == 3) d[3] = 0;
         const v4i wv = *reinterpret_cast<const v4i*>(wrow + (size_t)ky * g.cp + q0); // 4 channels x (w0,w1,w2,0)
-        // 4x4 byte transpose of (d0,d1,d2,0): t[c] = (pixel0.c, pixel1.c, pixel2.c, 0)
+        // 4x4 byte transpose: t[c] = (pixel0.c, pixel1.c, pixel2.c, pixel3.c)
         const uint32_t p01l = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), p01h = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
-        const uint32_t p23l = __builtin_amdgcn_perm(0u, d[2], 0x05010400u), p23h = __builtin_amdgcn_perm(0u, d[2], 0x07030602u);
-        acc[0] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), wv[0], acc[0], false);
-        acc[1] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23l, p01l, 0x07060302u), wv[1], acc[1], false);
-        acc[2] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23h, p01h, 0x05040100u), wv[2], acc[2], false);
-        acc[3] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_perm(p23h, p01h, 0x07060302u), wv[3], acc[3], false);
+        const uint32_t p23l = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), p23h = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+        const uint32_t t[4] = {__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), __builtin_amdgcn_perm(p23l, p01l, 0x07060302u),
+                               __builtin_amdgcn_perm(p23h, p01h, 0x05040100u), __builtin_amdgcn_perm(p23h, p01h, 0x07060302u)};
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+        {
+            acc[0][c] = __builtin_amdgcn_sdot4((int)t[c], wv[c], acc[0][c], false);
+            if (OUTS == 2) acc[1][c] = __builtin_amdgcn_sdot4((int)t[c], (int)((uint32_t)wv[c] << 8), acc[1][c], false);
+        }
     }
 
-    const size_t off = (size_t)pix * g.cp + q0;
-    float f[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++)
+    // per-channel tables: one vector load each when the channel count is a multiple of 4 (uniform), else clamped scalars
+    float s_in[4], s_b[4], s_out[4];
+    if ((g.c & 3) == 0)
     {
-        const int q = (int)q0 + e;
-        const int qc = q < g.c ? q : g.c - 1; // clamped: the table loads stay unconditional
-        float r = mul_rn((float)acc[e], scale_in[qc]);
-        if (bias) r = add_rn(r, bias[qc]);
-        r = apply_activation(r, act);
-        if (!g.out_f32) r = float2int8_as_float(mul_rn(r, scale_out[qc]));
-        f[e] = q < g.c ? r : 0.f;
+        const unsigned qc = q0 < (unsigned)g.c ? q0 : (unsigned)g.c - 4;
+        const v4f a = *reinterpret_cast<const v4f*>(scale_in + qc);
+        const v4f b = bias ? *reinterpret_cast<const v4f*>(bias + qc) : v4f{0.f, 0.f, 0.f, 0.f};
+        const v4f c = g.out_f32 ? v4f{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const v4f*>(scale_out + qc);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            s_in[e] = a[e];
+            s_b[e] = b[e];
+            s_out[e] = c[e];
+        }
     }
-    if (g.out_f32)
-        *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
     else
-        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
-            (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
+    {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            const int qc = (int)q0 + e < g.c ? (int)q0 + e : g.c - 1;
+            s_in[e] = scale_in[qc];
+            s_b[e] = bias ? bias[qc] : 0.f;
+            s_out[e] = g.out_f32 ? 0.f : scale_out[qc];
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < OUTS; o++)
+    {
+        const unsigned ox = ox0 + o;
+        if (ox >= (unsigned)g.outw) continue;
+        const size_t off = ((size_t)blockIdx.y * g.outw + ox) * g.cp + q0;
+        float f[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            float v = mul_rn((float)acc[o][e], s_in[e]);
+            if (bias) v = add_rn(v, s_b[e]);
+            v = apply_activation(v, act);
+            if (!g.out_f32) v = float2int8_as_float(mul_rn(v, s_out[e]));
+            f[e] = (int)q0 + e < g.c ? v : 0.f;
+        }
+        if (g.out_f32)
+            *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
+        else
+            *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
+                (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
+    }
 }
 
 static inline int padded16(int c)
@@ -611,19 +667,23 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
     g.pad_left = pad_left;
     g.pad_byte = (int)(signed char)d.pad_value;
     g.out_f32 = scale_out_dev ? 0 : 1;
-    if (d.kernel_w == 3 && d.kernel_h == 3 && d.dilation_w == 1 && d.dilation_h == 1 && d.stride_w == d.stride_h && (d.stride_w == 1 || d.stride_w == 2))
+    // the fast path indexes output rows with blockIdx.y and one sample with 31 bits; anything larger takes the generic kernel
+    const bool fits_fast = (size_t)d.batch * outh <= 65535 && (size_t)d.batch * outh * outw < (1ull << 32) && (size_t)outw * (g.cp / 4) * (g.cp / 4) < (1ull << 32) &&
+                           (size_t)d.h * d.w * g.cp < (1ull << 31);
+    if (fits_fast && d.kernel_w == 3 && d.kernel_h == 3 && d.dilation_w == 1 && d.dilation_h == 1 && d.stride_w == d.stride_h && (d.stride_w == 1 || d.stride_w == 2))
     {
         const uint32_t* wrow = reinterpret_cast<const uint32_t*>(packed_weight_dev + (size_t)9 * g.cp);
-        const size_t pixels = (size_t)d.batch * outh * outw;
-        NCNNHIP_REQUIRE(pixels < (1ull << 32), "ncnnhip_dwconv_int8_nhwc: more than 2^32 output pixels");
-        const size_t threads = pixels * (g.cp / 4);
-        dim3 grid3(ceil_div((long long)threads, 256));
+        const unsigned quads = (unsigned)g.cp / 4;
+        const unsigned xgroups = (unsigned)ceil_div(outw, d.stride_w == 1 ? 2 : 1);
+        const size_t rows = (size_t)d.batch * outh, row_threads = (size_t)xgroups * quads;
+        const unsigned quads_magic = (unsigned)(((1ull << 32) + quads - 1) / quads);
+        dim3 grid3(ceil_div((long long)row_threads, 256), (unsigned)rows);
         if (d.stride_w == 1)
             hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<1>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, threads);
+                               out_nhwc_dev, quads, quads_magic, xgroups);
         else
             hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<2>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, threads);
+                               out_nhwc_dev, quads, quads_magic, xgroups);
         return launch_status("dwconv3x3_nhwc_kernel");
     }
     const size_t total = (size_t)d.batch * outh * outw * (g.cp / 16);
