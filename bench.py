@@ -215,7 +215,8 @@ def bench_blockquant(args, n, k, m):
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, int8 weights in blocks of 64, fp32 block scales, %s activations" % (m, n, k, args.act),
                    "weight_copies_rotated": copies},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if half else None,
                      "kernel": "blockquant8_mfma_kernel" if half else "blockquant8_stream_kernel", "bytes_per_launch": algo},
     }
 
@@ -305,7 +306,7 @@ def bench_conv(args, spec):
         "config": {"workload": "Convolution %dx%d %d->%d on %dx%d, batch %d, fp32 in -> quantise -> int8 implicit GEMM -> fp32 out with ReLU; "
                                "back-to-back launches, channels-last resident blobs" % (k, k, c, cout, h, w, batch), "kernel_us": kernel_ms * 1e3},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": None, "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
+                     "traffic": measured_traffic("conv:" + spec), "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
     }
     if not args.no_cpu and batch == 1:
         line["cpu_baseline"] = cpu_baseline_conv(c, h, w, cout, k, pad)
