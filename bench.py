@@ -271,7 +271,7 @@ def bench_conv(args, spec):
     d_s = rt.up(np.array([127.0], np.float32))
     d_pk, d_si, d_b = rt.up(pk), rt.up(rng.uniform(1e-4, 1e-3, cout).astype(np.float32)), rt.up(rng.uniform(-0.1, 0.1, cout).astype(np.float32))
     d_out = ncnn_amd.DeviceBuffer.empty((batch, h * w, cp(cout)), np.float32)
-    d_ws = ncnn_amd.DeviceBuffer(max(sb.value, 4))
+    d_ws = ncnn_amd.DeviceBuffer.zeros(sb.value, st)
     act = Activation.make(1)
 
     def quantise():
@@ -357,7 +357,7 @@ def bench_layers(args, which, batch):
                 wq = rng.integers(-127, 128, cout * c * taps).astype(np.int8)
                 pk = np.empty(wb.value, np.int8)
                 check(lib.ncnnhip_conv_pack_weights(C.byref(desc), wq.ctypes.data, pk.ctypes.data))
-                plan.update(d_pk=rt.up(pk), d_ws=ncnn_amd.DeviceBuffer(max(sb.value, 4)), ws_bytes=sb.value)
+                plan.update(d_pk=rt.up(pk), d_ws=ncnn_amd.DeviceBuffer.zeros(sb.value, st), ws_bytes=sb.value)
             else:
                 assert r["group"] == c == cout, "the benchmark nets only hold plain and depthwise convolutions"
                 wq = rng.integers(-127, 128, c * taps).astype(np.int8)

@@ -114,8 +114,9 @@ int ncnnhip_conv_int8(const ncnnhip_conv_desc* desc, const int8_t* x_dev, size_t
  * [batch][h][w][Cp] int8, Cp = 16*ceil(c/16) -- from fp32 with the Quantize arithmetic (one scale or one per
  * channel) or from int8 as is -- and the weights are repacked once (host side, at create_pipeline) to
  * [num_output][kh*kw][Cp] with K padded to a multiple of 64.  Results are identical to ncnnhip_conv_int8.
- * workspace: int32 scratch for layers whose K loop is split across workgroups (size from ncnnhip_conv_nhwc_sizes,
- * may be 0); it is cleared by the call itself.
+ * workspace: scratch for layers whose K loop is split across workgroups (size from ncnnhip_conv_nhwc_sizes, may be 0).
+ * Zero-fill it ONCE after allocating it (ncnnhip_memset); every call leaves it fit for the next call, so one workspace of
+ * the largest size serves all layers of a net, one call at a time (calls that overlap on one workspace race).
  * out_layout NCNNHIP_PLANAR: out is ncnn's [batch][num_output][out_cstep] (out_nstep between samples);
  * NCNNHIP_CHANNELS_LAST: out is [batch][outh*outw][16*ceil(num_output/16)], pad channels written as zero
  * (out_cstep / out_nstep ignored) -- the form the next layer's kernel consumes without a conversion pass. */

@@ -43,7 +43,13 @@ struct GemmTail
     float alpha, beta;
 };
 
-// int32 words of split-K scratch the pipelined kernel wants for this problem (0: it does not split)
+// Workspace contract of the channels-last convolutions: the first SPLIT_COUNTER_BYTES hold one arrival counter per
+// output tile of a K-split launch.  They must be zero when a call starts (the caller clears the workspace once, after
+// allocating it) and are zero again when it has finished; the rest is scratch without a contract.
+constexpr int SPLIT_MAX_TILES = 1024;
+constexpr size_t SPLIT_COUNTER_BYTES = SPLIT_MAX_TILES * sizeof(unsigned);
+
+// int32 words of workspace (counters included) the pipelined kernel wants for this problem (0: it does not split)
 size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps);
 
 // Launches the pipelined kernel; the caller has checked: zero border byte, channels-last output.

@@ -398,7 +398,7 @@ int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, s
     {
         const long long npix = (long long)desc->batch * outw * outh;
         const SplitPlan p = plan_launch(desc->num_output, npix, packed_k(*desc) / 64);
-        size_t words = p.splits > 1 ? (size_t)padded_channels(desc->num_output) * npix : 0;
+        size_t words = p.splits > 1 ? SPLIT_COUNTER_BYTES / sizeof(int32_t) + (size_t)padded_channels(desc->num_output) * npix : 0;
         const size_t words_pipelined = conv_nhwc_pipelined_workspace_words(desc->num_output, npix, packed_k(*desc) / 64);
         if (words_pipelined > words) words = words_pipelined;
         *workspace_bytes = words * sizeof(int32_t);
@@ -500,8 +500,9 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc
     if (p.splits > 1)
     {
         const size_t words = (size_t)out_cp * npix;
-        NCNNHIP_REQUIRE(workspace_dev && workspace_bytes >= words * sizeof(int32_t), "ncnnhip_conv_int8_nhwc: workspace of %zu bytes required", words * sizeof(int32_t));
-        partial = (int32_t*)workspace_dev;
+        NCNNHIP_REQUIRE(workspace_dev && workspace_bytes >= SPLIT_COUNTER_BYTES + words * sizeof(int32_t), "ncnnhip_conv_int8_nhwc: workspace of %zu bytes required",
+                        SPLIT_COUNTER_BYTES + words * sizeof(int32_t));
+        partial = (int32_t*)((char*)workspace_dev + SPLIT_COUNTER_BYTES); // the counter region belongs to the pipelined kernel: left untouched (zero)
         hipLaunchKernelGGL(zero_i32_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, st, partial, words);
     }
 #define LAUNCH_NHWC(BM_, BN_)                                                                                                                       \

@@ -15,8 +15,10 @@
 //
 // Workgroup ids are dealt round-robin to the 8 XCDs; they are remapped so that an XCD works on consecutive tiles
 // (channel tiles of one pixel tile are neighbours and share the activations in that XCD's L2).
-// Small problems split K over workgroups: partial int32 sums are added into a zeroed [pixel][channel] scratch with
-// coalesced atomics (integer addition: exact in any order) and a second kernel applies the epilogue.
+// Small problems split K over workgroups inside the one launch: every workgroup of a tile but the last to finish
+// dumps its accumulator registers to scratch (register-major, fully coalesced) and bumps the tile's counter; the
+// last one adds the others' dumps to its own registers (integer addition: exact in any order), resets the counter
+// and runs the normal epilogue.  Nobody waits for anybody, so the grid may be larger than the chip.
 #include <type_traits>
 
 #include "conv_nhwc.h"
@@ -40,7 +42,7 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
 
 template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int steps_per_split, int32_t* __restrict__ partial)
+                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     int step_end = SPLITK ? step_begin + steps_per_split : total_steps;
     if (step_end > total_steps) step_end = total_steps;
     const int nk = step_end - step_begin;
-    if (nk <= 0) return;
+    if (!SPLITK && nk <= 0) return; // (a split workgroup always has steps, and must reach the tile counter in any case)
 
     // ---- sources of this lane's loads.  Load i of a wavefront fills LDS rows i*64 + wave*16 .. +16 of the operand;
     // the lane's row is +lane/4 and it fetches source chunk (lane&3) ^ ((lane>>4)&3) into position lane&3.
@@ -215,21 +217,40 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     // ---- epilogue: lane = one output channel per 32-column block, registers = pixels
     if (SPLITK)
     {
+        // Slice of this workgroup: [register][thread] int32.  The dump and its read-back are agent-scope atomic
+        // stores / loads: they go to the coherence point of the whole device (the XCDs' L2s are not coherent with each
+        // other inside a kernel) without the full L2 write-back and invalidate a fence would cost every workgroup.
+        constexpr int NREG = TM * TN * 16;
+        const int tile_id = tm * tiles_n + tn;
+        __shared__ unsigned arrived;
+        int* mine = partial + ((size_t)split * tiles_m * tiles_n + tile_id) * (size_t)(NREG * 256);
+        // optimistic dump: the last workgroup would not need it, but it does not know yet that it is the last
 #pragma unroll
-        for (int c = 0; c < TN; c++)
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+            for (int c = 0; c < TN; c++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    __hip_atomic_store(mine + ((a * TN + c) * 16 + r) * 256 + threadIdx.x, acc[a][c][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        WAIT_VMCNT(0); // this wavefront's stores have reached the coherence point ...
+        asm volatile("" ::: "memory");
+        __syncthreads(); // ... and everybody else's in the workgroup, before the counter moves
+        if (threadIdx.x == 0) arrived = atomicAdd(counters + tile_id, 1u);
+        __syncthreads();
+        if (arrived != (unsigned)(splits - 1)) return; // somebody else finishes this tile
+        for (int s2 = 0; s2 < splits; s2++)
         {
-            const int ch = col0 + wn * (BN / 2) + c * 32 + l32;
-            if (ch >= g.cout) continue;
+            if (s2 == split) continue;
+            const int* theirs = partial + ((size_t)s2 * tiles_m * tiles_n + tile_id) * (size_t)(NREG * 256);
 #pragma unroll
             for (int a = 0; a < TM; a++)
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                {
-                    const int pix = row0 + wm * (BM / 2) + a * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                    if (pix < g.npix) atomicAdd(partial + (size_t)pix * out_cp + ch, acc[a][c][r]);
-                }
+                for (int c = 0; c < TN; c++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        acc[a][c][r] += __hip_atomic_load(theirs + ((a * TN + c) * 16 + r) * 256 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        return;
+        if (threadIdx.x == 0) counters[tile_id] = 0u; // ready for the next launch
     }
     // Through LDS, so that global memory sees whole runs of channels: each wavefront stages 32 pixels x CW channels of
     // results as [pixel][channel] floats (the pipeline stages are free by now), then every lane takes 4 consecutive
@@ -412,38 +433,6 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         finish(std::integral_constant<int, -1>{});
 }
 
-// partial sums [npix][out_cp] -> epilogue; one thread per (pixel, channel), channels fastest
-__global__ __launch_bounds__(256) void conv_pipelined_finish_kernel(const int32_t* __restrict__ partial, int npix, int out_cp, int cout, ConvEpilogue epi,
-                                                                     ConvFusion fusion)
-{
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (size_t)npix * out_cp) return;
-    const int ch = (int)(i % (size_t)out_cp);
-    const bool real = ch < cout;
-    float f = 0.f;
-    if (real)
-    {
-        f = mul_rn((float)partial[i], epi.scale_in[ch]);
-        if (epi.bias) f = add_rn(f, epi.bias[ch]);
-        f = apply_activation(f, epi.act);
-    }
-    if (epi.scale_out)
-        static_cast<int8_t*>(epi.out)[i] = real ? (int8_t)float2int8(mul_rn(f, epi.scale_out[ch])) : (int8_t)0;
-    else
-    {
-        if (fusion.residual) f = add_rn(f, fusion.residual[i]);
-        if (fusion.relu_after) f = fmaxf(f, 0.f);
-        static_cast<float*>(epi.out)[i] = f;
-        if (fusion.q8_out) fusion.q8_out[i] = (int8_t)float2int8(mul_rn(f, fusion.q8_scale));
-    }
-}
-
-__global__ __launch_bounds__(256) void zero_words_kernel(int32_t* p, size_t n)
-{
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-
 struct PipePlan
 {
     int bm, bn, tiles_m, tiles_n, splits, steps_per_split;
@@ -471,11 +460,12 @@ static PipePlan plan_pipelined(int cout, long long npix, int steps)
     p.tiles_n = ceil_div(cout, p.bn);
     p.splits = 1;
     const long long t = tiles();
-    if (t < 128 && steps >= 32)
+    if (t < 128 && t <= SPLIT_MAX_TILES && steps >= 16)
     {
-        // a split costs two more launches (clear + finish): only worth it for long K loops
-        const int want = (int)((384 + t - 1) / t);
-        const int max_splits = steps / 8; // at least 8 K steps per split
+        // too few tiles to occupy the chip: split K until there is about one workgroup per CU, at least 8 steps each
+        // (measured best over the ResNet-50 / MobileNetV2 layers at batch 1 and 16)
+        const int want = (int)((256 + t - 1) / t);
+        const int max_splits = steps / 8;
         p.splits = want < max_splits ? want : max_splits;
         if (p.splits < 1) p.splits = 1;
     }
@@ -487,7 +477,8 @@ static PipePlan plan_pipelined(int cout, long long npix, int steps)
 size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps)
 {
     const PipePlan p = plan_pipelined(cout, npix, steps);
-    return p.splits > 1 ? (size_t)npix * ((cout + 15) / 16 * 16) : 0;
+    if (p.splits <= 1) return 0;
+    return SPLIT_COUNTER_BYTES / sizeof(int32_t) + (size_t)p.splits * p.tiles_m * p.tiles_n * p.bm * p.bn;
 }
 
 int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
@@ -497,12 +488,13 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     const long long blocks = (long long)p.tiles_m * p.tiles_n * p.splits;
     NCNNHIP_REQUIRE(blocks < (1ll << 31), "convolution: too many tiles");
     int32_t* partial = 0;
-    const size_t words = (size_t)g.npix * out_cp;
+    unsigned* counters = 0;
     if (p.splits > 1)
     {
-        NCNNHIP_REQUIRE(workspace && workspace_bytes >= words * sizeof(int32_t), "convolution: workspace of %zu bytes required", words * sizeof(int32_t));
-        partial = (int32_t*)workspace;
-        hipLaunchKernelGGL(zero_words_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, words);
+        const size_t need = SPLIT_COUNTER_BYTES + (size_t)p.splits * p.tiles_m * p.tiles_n * p.bm * p.bn * sizeof(int32_t);
+        NCNNHIP_REQUIRE(workspace && workspace_bytes >= need, "convolution: workspace of %zu bytes required", need);
+        counters = (unsigned*)workspace; // zero on entry (the caller cleared the workspace once), zero again on exit
+        partial = (int32_t*)((char*)workspace + SPLIT_COUNTER_BYTES);
     }
     dim3 grid((unsigned)blocks), block(256);
     const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
@@ -511,10 +503,10 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     {                                                                                                                                           \
         if (p.splits > 1)                                                                                                                       \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.steps_per_split, partial);                                                                                     \
+                               p.splits, p.steps_per_split, partial, counters);                                                                                     \
         else                                                                                                                                    \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.steps_per_split, partial);                                                                                     \
+                               p.splits, p.steps_per_split, partial, counters);                                                                                     \
     } while (0)
     // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
     if (p.bm == 128 && p.bn == 256)
@@ -530,8 +522,6 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     else
         LAUNCH_PIPE(64, 64, 3);
 #undef LAUNCH_PIPE
-    if (p.splits > 1)
-        hipLaunchKernelGGL(conv_pipelined_finish_kernel, dim3(ceil_div((long long)words, 256)), dim3(256), 0, stream, partial, g.npix, out_cp, g.cout, epi, fusion);
     return launch_status("conv_nhwc_pipelined_kernel");
 }
 
@@ -579,7 +569,7 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     dim3 grid((unsigned)blocks), block(256);
 #define LAUNCH_GEMM(BM_, BN_)                                                                                                                        \
     hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
-                       p.tiles_m, p.tiles_n, p.steps_per_split, (int32_t*)0)
+                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, (int32_t*)0, (unsigned*)0)
     if (p.bm == 128 && p.bn == 256)
         LAUNCH_GEMM(128, 256);
     else if (p.bm == 128 && p.bn == 128)

@@ -154,6 +154,14 @@ class DeviceBuffer:
         return buf
 
     @classmethod
+    def zeros(cls, nbytes, stream=None):
+        """A zero-filled byte buffer (the convolution workspace must be cleared once after allocation)."""
+        buf = cls(max(int(nbytes), 4))
+        check(lib().ncnnhip_memset(buf.ptr, 0, buf.nbytes, stream))
+        check(lib().ncnnhip_stream_synchronize(stream))
+        return buf
+
+    @classmethod
     def empty(cls, shape, dtype):
         shape = tuple(int(s) for s in np.atleast_1d(shape))
         return cls(int(np.prod(shape)) * np.dtype(dtype).itemsize, shape, dtype)
@@ -261,7 +269,7 @@ class Runtime:
                 ts = np.atleast_1d(np.asarray(top_scales, np.float32))
                 scale_out = np.repeat(ts, num_output // ts.size).astype(np.float32)
             dpk, dsi, db, dso = self.up(pk), self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32)), self.up(scale_out)
-            dws = DeviceBuffer(max(sb_.value, 4))
+            dws = DeviceBuffer.zeros(sb_.value, self.stream)
             dout = DeviceBuffer.empty((n, num_output, oh, ow), np.int8 if requant else np.float32)
             check(lib().ncnnhip_conv_int8_nhwc(C.byref(d), dn.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
                                                0, oh * ow, num_output * oh * ow, dws.ptr, sb_.value, self.stream))
@@ -387,7 +395,7 @@ class Runtime:
             check(lib().ncnnhip_conv_nhwc_sizes(C.byref(d), C.byref(nb), C.byref(wb), C.byref(sb_)))
             pk = np.empty(wb.value, np.int8)
             check(lib().ncnnhip_conv_pack_weights(C.byref(d), wq.ctypes.data, pk.ctypes.data))
-            dpk, dws = self.up(pk), DeviceBuffer(max(sb_.value, 4))
+            dpk, dws = self.up(pk), DeviceBuffer.zeros(sb_.value, self.stream)
             if residual is not None or relu_after or quantise_scale is not None:
                 # the layers after the convolution folded into its epilogue; returns (fp32 result, its quantised copy or None)
                 dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))

@@ -286,7 +286,7 @@ int Convolution_hip::forward(const Mat& bottom_blob, Mat& top_blob, const Option
         rc = ncnnhip_conv_nhwc_sizes(&desc, &nhwc_bytes, &packed_bytes, &workspace_bytes);
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
         void* d_nhwc = leases.get(nhwc_bytes);
-        void* d_ws = workspace_bytes ? leases.get(workspace_bytes) : 0;
+        void* d_ws = workspace_bytes ? ctx->zeroed_workspace(workspace_bytes) : 0;
         if (!d_nhwc || (workspace_bytes && !d_ws)) return -100;
         rc = ncnnhip_to_nhwc_int8(&desc, d_in, (int)bottom_blob.elemsize, bottom_blob.cstep, bottom_blob.nstep, (const float*)d_input_scales, 1,
                                   (int8_t*)d_nhwc, st);
@@ -422,7 +422,7 @@ int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* resid
         size_t workspace_bytes = 0;
         rc = ncnnhip_conv_nhwc_sizes(&desc, 0, 0, &workspace_bytes);
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_nhwc_sizes");
-        void* ws = workspace_bytes ? scratch.get(workspace_bytes) : 0;
+        void* ws = workspace_bytes ? cmd.zeroed_workspace(workspace_bytes) : 0;
         if (workspace_bytes && !ws) return -100;
         if (fused)
         {

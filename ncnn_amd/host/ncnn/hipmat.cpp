@@ -128,13 +128,35 @@ void HipMat::create_like(const HipMat& m, HipCommand* command)
 
 // ---- HipCommand ---------------------------------------------------------------------------------
 
-HipCommand::HipCommand() : stream(0), ready(false) {}
+HipCommand::HipCommand() : stream(0), ready(false), zero_ws(0), zero_ws_bytes(0) {}
 
 HipCommand::~HipCommand()
 {
     if (ready) ncnnhip_stream_synchronize(stream);
     for (size_t i = 0; i < pool.size(); i++) ncnnhip_free(pool[i].ptr);
+    if (zero_ws) ncnnhip_free(zero_ws);
     if (stream) ncnnhip_stream_destroy(stream);
+}
+
+void* HipCommand::zeroed_workspace(size_t bytes)
+{
+    if (bytes <= zero_ws_bytes) return zero_ws;
+    // grow: whatever still uses the old buffer was enqueued on this stream, so wait before freeing it
+    if (ncnnhip_stream_synchronize(stream) != 0) return 0;
+    if (zero_ws) ncnnhip_free(zero_ws);
+    zero_ws = 0;
+    zero_ws_bytes = 0;
+    const size_t rounded = (bytes + 0xfffff) & ~(size_t)0xfffff;
+    void* p = 0;
+    if (ncnnhip_malloc(&p, rounded) != 0 || !p) return 0;
+    if (ncnnhip_memset(p, 0, rounded, stream) != 0 || ncnnhip_stream_synchronize(stream) != 0)
+    {
+        ncnnhip_free(p);
+        return 0;
+    }
+    zero_ws = p;
+    zero_ws_bytes = rounded;
+    return zero_ws;
 }
 
 int HipCommand::ensure_ready()

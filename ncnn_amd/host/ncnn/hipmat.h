@@ -85,6 +85,9 @@ public:
     // scratch for one forward call: everything borrowed goes back with give_back_all()
     void* borrow(size_t bytes);
     void give_back_all();
+    // one persistent buffer, zero-filled when it is (re)allocated, for kernels that keep their scratch "zero at rest"
+    // (the arrival counters of the K-split convolution); used by one kernel at a time, like everything on this stream
+    void* zeroed_workspace(size_t bytes);
 
     // host Mat (planar, any batch) -> device blob and back; download synchronises the stream
     int upload(const Mat& src, HipMat& dst);
@@ -105,6 +108,8 @@ private:
     void* take(size_t bytes, int state);
     bool ready;
     std::vector<Slot> pool;
+    void* zero_ws;
+    size_t zero_ws_bytes;
 };
 
 // scratch borrowed during one forward() returns to the pool when this goes out of scope
