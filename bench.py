@@ -337,6 +337,9 @@ def bench_layers(args, which, batch):
                         d_w=rt.up(rng.integers(-127, 128, (n, k)).astype(np.int8)), d_si=rt.up(rng.uniform(1e-4, 1e-3, n).astype(np.float32)),
                         d_b=rt.up(rng.uniform(-0.1, 0.1, n).astype(np.float32)), d_s=rt.up(np.array([50.0], np.float32)),
                         d_out=ncnn_amd.DeviceBuffer.empty((batch, n), np.float32))
+            wsb = C.c_size_t()
+            check(lib.ncnnhip_innerproduct_workspace_bytes(batch, k, n, C.byref(wsb)))
+            plan.update(d_ws=ncnn_amd.DeviceBuffer.zeros(wsb.value, st), ws_bytes=wsb.value)
         else:
             c, h, w = r["in_shape"]
             cout, oh, ow = r["out_shape"]
@@ -373,8 +376,8 @@ def bench_layers(args, which, batch):
         if p["kind"] == "fc":
             if prepass:
                 check(lib.ncnnhip_quantize(p["d_x"].ptr, p["k"], 0, p["d_xq"].ptr, p["k"], 0, batch, p["k"], 1, p["d_s"].ptr, 1, st))
-            check(lib.ncnnhip_innerproduct_int8(p["d_xq"].ptr, p["k"], batch, p["k"], p["n"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
-                                                Activation.make(0), p["d_out"].ptr, p["n"], None, st))
+            check(lib.ncnnhip_innerproduct_int8_ws(p["d_xq"].ptr, p["k"], batch, p["k"], p["n"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
+                                                   Activation.make(0), p["d_out"].ptr, p["n"], p["d_ws"].ptr, p["ws_bytes"], st))
             return
         if prepass and not r["int8_in"]:
             check(lib.ncnnhip_quantize_nhwc(p["d_x"].ptr, p["d_xq"].ptr, p["npix"], r["in_shape"][0], p["d_s"].ptr, 1, st))

@@ -205,6 +205,13 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
                               const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
                               ncnnhip_activation act, float* out_dev, size_t out_stride, int32_t* acc_out_dev,
                               void* stream);
+/* The same with a workspace (zero-filled once after allocation, like the convolution's): from 8 activation rows up the layer
+ * then runs on the matrix cores as a 1x1 convolution over the rows, its K loop split across workgroups. */
+int ncnnhip_innerproduct_workspace_bytes(int rows, int num_input, int num_output, size_t* workspace_bytes);
+int ncnnhip_innerproduct_int8_ws(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output,
+                                 const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
+                                 ncnnhip_activation act, float* out_dev, size_t out_stride, void* workspace_dev,
+                                 size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ Gemm int8
  * Dynamic per-row quantisation of A (src/layer/gemm.cpp:791-823): scales[i] = 127/absmax_i (1 for a

@@ -61,6 +61,12 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
 int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmTail& tail,
                                    float* out, size_t out_stride, hipStream_t stream, bool* handled);
 
+// InnerProduct as a 1x1 convolution over the activation rows (rows = pixels, K = channels): same epilogue as the
+// convolution (scale_in, bias, activation), dense fp32 output with row stride out_stride.  handled = false when the
+// shape does not fit (K % 64, num_output % 4, strides, alignment, workspace) and the caller should take another kernel.
+int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int K, int num_output, const int8_t* weight, const ConvEpilogue& epi,
+                                 size_t out_stride, void* workspace, size_t workspace_bytes, hipStream_t stream, bool* handled);
+
 } // namespace ncnnhip
 
 #endif // NCNNHIP_CONV_NHWC_H

@@ -586,4 +586,65 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     return launch_status("conv_nhwc_pipelined_kernel<gemm>");
 }
 
+int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int K, int num_output, const int8_t* weight, const ConvEpilogue& epi,
+                                 size_t out_stride, void* workspace, size_t workspace_bytes, hipStream_t stream, bool* handled)
+{
+    *handled = false;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(epi.out)) & 15) == 0;
+    if (K % 64 || num_output % 4 || x_stride % 16 || out_stride % 4 || !aligned || epi.scale_out || epi.acc_out) return NCNNHIP_OK;
+    if ((long long)rows * (long long)x_stride >= (1ll << 31)) return NCNNHIP_OK;
+    const size_t need = conv_nhwc_pipelined_workspace_words(num_output, rows, K / 64) * sizeof(int32_t);
+    if (need > workspace_bytes || (need && !workspace)) return NCNNHIP_OK;
+    *handled = true;
+
+    NhwcGeom g;
+    g.H = 1;
+    g.W = rows;
+    g.Cp = (int)x_stride;
+    g.kw = g.kh = g.dw = g.dh = g.sw = g.sh = 1;
+    g.pad_top = g.pad_left = 0;
+    g.outw = rows;
+    g.outh = 1;
+    g.npix = rows;
+    g.ntaps = 1;
+    g.K = K;
+    g.cout = num_output;
+    g.pad_word = 0;
+    const ConvFusion no_fusion = {0, 0, 0, 0.f};
+    const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
+    const PipePlan p = plan_pipelined(num_output, rows, K / 64);
+    int32_t* partial = 0;
+    unsigned* counters = 0;
+    if (p.splits > 1)
+    {
+        counters = (unsigned*)workspace;
+        partial = (int32_t*)((char*)workspace + SPLIT_COUNTER_BYTES);
+    }
+    dim3 grid((unsigned)((long long)p.tiles_m * p.tiles_n * p.splits)), block(256);
+    // rows are few: only the 64-pixel tiles occur
+#define LAUNCH_FC(BN_)                                                                                                                                   \
+    do                                                                                                                                                   \
+    {                                                                                                                                                    \
+        if (p.splits > 1)                                                                                                                                \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, true, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,     \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, partial, counters);                       \
+        else                                                                                                                                             \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, false, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,    \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, partial, counters);                       \
+    } while (0)
+    if (p.bm != 64)
+    {
+        *handled = false;
+        return NCNNHIP_OK;
+    }
+    if (p.bn == 256)
+        LAUNCH_FC(256);
+    else if (p.bn == 128)
+        LAUNCH_FC(128);
+    else
+        LAUNCH_FC(64);
+#undef LAUNCH_FC
+    return launch_status("conv_nhwc_pipelined_kernel<fc>");
+}
+
 } // namespace ncnnhip

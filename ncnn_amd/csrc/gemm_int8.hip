@@ -180,4 +180,40 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
     return launch_status("gemm_tile_kernel<fc>");
 }
 
+int ncnnhip_innerproduct_workspace_bytes(int rows, int num_input, int num_output, size_t* workspace_bytes)
+{
+    NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1 && workspace_bytes, "ncnnhip_innerproduct_workspace_bytes: bad argument");
+    *workspace_bytes = (rows >= 8 && num_input % 64 == 0) ? conv_nhwc_pipelined_workspace_words(num_output, rows, num_input / 64) * sizeof(int32_t) : 0;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_innerproduct_int8_ws(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output, const int8_t* weight_dev,
+                                 const float* scale_in_dev, const float* bias_dev, ncnnhip_activation act, float* out_dev, size_t out_stride,
+                                 void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(x_dev && weight_dev && scale_in_dev && out_dev, "ncnnhip_innerproduct_int8_ws: null pointer");
+    NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1, "ncnnhip_innerproduct_int8_ws: bad shape");
+    NCNNHIP_REQUIRE(x_stride >= (size_t)num_input && out_stride >= (size_t)num_output, "ncnnhip_innerproduct_int8_ws: stride too small");
+    if (rows >= 8)
+    {
+        ConvEpilogue epi;
+        epi.scale_in = scale_in_dev;
+        epi.bias = bias_dev;
+        epi.scale_out = 0;
+        epi.act = act;
+        epi.out = out_dev;
+        epi.out_cstep = epi.out_nstep = 0;
+        epi.pix_per_img = rows;
+        epi.batch = 1;
+        epi.out_channel0 = 0;
+        epi.num_output = num_output;
+        epi.acc_out = 0;
+        bool handled = false;
+        int ret = launch_fc_via_conv_pipelined(x_dev, x_stride, rows, num_input, num_output, weight_dev, epi, out_stride, workspace_dev, workspace_bytes,
+                                               as_stream(stream), &handled);
+        if (handled) return ret;
+    }
+    return ncnnhip_innerproduct_int8(x_dev, x_stride, rows, num_input, num_output, weight_dev, scale_in_dev, bias_dev, act, out_dev, out_stride, 0, stream);
+}
+
 } // extern "C"

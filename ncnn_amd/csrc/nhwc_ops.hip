@@ -203,9 +203,9 @@ __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restri
 }
 
 // global pooling: [n][hw][cp] -> dense [n][c]; one thread per (sample, channel) walks the pixels in index order
-__global__ __launch_bounds__(256) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type)
+__global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type)
 {
-    const int q = blockIdx.x * 256 + threadIdx.x;
+    const int q = blockIdx.x * 64 + threadIdx.x; // one wavefront per workgroup: the few channels spread over as many CUs as possible
     const int img = blockIdx.y;
     if (q >= c) return;
     const float* p = src + (size_t)img * hw * cp + q;
@@ -576,7 +576,7 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
     if (d.global_pooling)
     {
         NCNNHIP_REQUIRE(d.batch <= 65535, "ncnnhip_pooling_nhwc: batch above 65535");
-        hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 256), d.batch), dim3(256), 0, as_stream(stream), src_dev, dst_dev, d.c, d.w * d.h, cp, d.pooling_type);
+        hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 64), d.batch), dim3(64), 0, as_stream(stream), src_dev, dst_dev, d.c, d.w * d.h, cp, d.pooling_type);
         return launch_status("global_pooling_nhwc_kernel");
     }
     NCNNHIP_REQUIRE(d.kernel_w > 0 && d.kernel_h > 0 && d.stride_w > 0 && d.stride_h > 0 && d.outw > 0 && d.outh > 0, "ncnnhip_pooling_nhwc: bad window");

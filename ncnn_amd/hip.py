@@ -92,6 +92,9 @@ _SIGNATURES = {
     "ncnnhip_softmax": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
                                   C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_innerproduct_workspace_bytes": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
+    "ncnnhip_innerproduct_int8_ws": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_size_t,
+                                     C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_quantize_tensor": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_transpose_f32": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
@@ -437,6 +440,15 @@ class Runtime:
         check(lib().ncnnhip_innerproduct_int8(dxq.ptr, k, rows, k, num_output, dw_.ptr, dsi.ptr, _ptr(db), Activation.make(act, act_params),
                                               dout.ptr, num_output, _ptr(dacc), self.stream))
         out = dout.to_numpy(self.stream)
+        # the workspace form (matrix cores, split K) must give the same values
+        wsb = C.c_size_t()
+        check(lib().ncnnhip_innerproduct_workspace_bytes(rows, k, num_output, C.byref(wsb)))
+        dws = DeviceBuffer.zeros(wsb.value, self.stream)
+        dout2 = DeviceBuffer.empty((rows, num_output), np.float32)
+        check(lib().ncnnhip_innerproduct_int8_ws(dxq.ptr, k, rows, k, num_output, dw_.ptr, dsi.ptr, _ptr(db), Activation.make(act, act_params),
+                                                 dout2.ptr, num_output, dws.ptr, wsb.value, self.stream))
+        if not np.array_equal(dout2.to_numpy(self.stream), out):
+            raise AssertionError("ncnnhip_innerproduct_int8_ws differs from ncnnhip_innerproduct_int8")
         return (out, dacc.to_numpy(self.stream)) if want_acc else out
 
     # -- Gemm int8 ----------------------------------------------------------------------------

@@ -213,9 +213,14 @@ int InnerProduct_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand&
         xq = (const int8_t*)q;
         q_stride = (size_t)num_input;
     }
-    int rc = ncnnhip_innerproduct_int8(xq, q_stride, rows, num_input, num_output, (const int8_t*)d_weight, (const float*)d_scale_in, (const float*)d_bias,
-                                       make_activation(activation_type, activation_params), (float*)top.data, (size_t)num_output, 0, st);
-    return to_ncnn_status(rc, "ncnnhip_innerproduct_int8");
+    size_t workspace_bytes = 0;
+    int rc = ncnnhip_innerproduct_workspace_bytes(rows, num_input, num_output, &workspace_bytes);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_innerproduct_workspace_bytes");
+    void* ws = workspace_bytes ? cmd.zeroed_workspace(workspace_bytes) : 0;
+    if (workspace_bytes && !ws) return -100;
+    rc = ncnnhip_innerproduct_int8_ws(xq, q_stride, rows, num_input, num_output, (const int8_t*)d_weight, (const float*)d_scale_in, (const float*)d_bias,
+                                      make_activation(activation_type, activation_params), (float*)top.data, (size_t)num_output, ws, workspace_bytes, st);
+    return to_ncnn_status(rc, "ncnnhip_innerproduct_int8_ws");
 }
 
 Layer* InnerProduct_hip_creator(void*)
