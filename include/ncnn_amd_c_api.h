@@ -97,6 +97,19 @@ int ncnnhip_extractor_input_hipmat(ncnn_extractor_t ex, const char* name, const 
 int ncnnhip_extractor_extract_hipmat(ncnn_extractor_t ex, const char* name, ncnn_hipmat_t* out);
 int ncnnhip_extractor_synchronize(ncnn_extractor_t ex);
 
+/* A forward pass recorded once and replayed with one launch (the reference's GPU path records a VkCompute command buffer
+ * and submits it, src/command.h:22-67).  record runs the pass from blob `input_name` (= input, resident) to `output_name`
+ * once and then records it; update_input copies new values into that same input blob; launch enqueues one replay;
+ * output hands out the result blob, which every launch rewrites (destroy the handle with ncnnhip_hipmat_destroy).
+ * One launch at a time per graph; destroy the graph before the net. */
+typedef struct __ncnn_hipgraph_t* ncnn_hipgraph_t;
+int ncnnhip_graph_record(ncnn_net_t net, const char* input_name, const ncnn_hipmat_t input, const char* output_name, ncnn_hipgraph_t* out);
+int ncnnhip_graph_update_input(ncnn_hipgraph_t g, const ncnn_mat_t mat);
+int ncnnhip_graph_replay(ncnn_hipgraph_t g);
+int ncnnhip_graph_synchronize(ncnn_hipgraph_t g);
+int ncnnhip_graph_output(ncnn_hipgraph_t g, ncnn_hipmat_t* out);
+void ncnnhip_graph_release(ncnn_hipgraph_t g);
+
 /* Gives the extractor its own device stream and buffer pool (one hipStream per Extractor) by
  * installing a host blob allocator that carries them; the allocator lives until
  * ncnnhip_extractor_detach_stream or process end.  Optional: without it a per-thread stream is used. */

@@ -41,6 +41,14 @@ int ncnnhip_stream_create(void** stream);
 int ncnnhip_stream_destroy(void* stream);
 int ncnnhip_stream_synchronize(void* stream);
 int ncnnhip_device_synchronize(void);
+/* Record once, replay with one call: what the reference's GPU path does with a recorded VkCompute command buffer
+ * (src/command.h:22-67, record_* then submit_and_wait).  Between begin and end every launch on `stream` is recorded
+ * instead of run; nothing may allocate, copy from pageable memory or synchronise on the capturing thread.  The
+ * executable graph replays the same kernels on the same buffers. */
+int ncnnhip_stream_begin_capture(void* stream);
+int ncnnhip_stream_end_capture(void* stream, void** graph_exec);
+int ncnnhip_graph_launch(void* graph_exec, void* stream);
+int ncnnhip_graph_destroy(void* graph_exec);
 int ncnnhip_malloc(void** dev, size_t bytes);
 int ncnnhip_free(void* dev);
 int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream);
@@ -195,6 +203,10 @@ typedef struct ncnnhip_pool_desc
     int avgpool_count_include_pad;
 } ncnnhip_pool_desc;
 int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, float* dst_dev, void* stream);
+/* Windowed max pooling (src/layer/pooling.cpp:105-222) of an int8 blob that holds Quantize(x, s), s > 0: the result is
+ * Quantize(maxpool(x), s), because rounding and clamping are monotonic (for |x*s| < 2^31; the caller knows a bound).  Lets a requantising convolution feed the
+ * quantising consumers of its pooled output without an fp32 blob in between. */
+int ncnnhip_maxpool_nhwc_int8(const ncnnhip_pool_desc* desc, const int8_t* src_dev, int8_t* dst_dev, void* stream);
 /* Softmax::forward_inplace (src/layer/softmax.cpp) over a dense vector of `count` values per sample. */
 int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream);
 

@@ -202,6 +202,45 @@ __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restri
     *reinterpret_cast<v4f*>(dst + (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q4 * 4) = r;
 }
 
+// Max pooling of an int8 blob, 16 channels of one output pixel per thread.  Quantize (round, clamp to [-127,127]) is
+// monotonic for a positive scale, so the maximum of the quantised values is the quantised maximum; a window without
+// any pixel gives -127, which is what -FLT_MAX quantises to.
+__global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, PoolGeom g, size_t total)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int groups = g.cp / 16;
+    const int q16 = (int)(i % (size_t)groups);
+    size_t rest = i / (size_t)groups;
+    const int ox = (int)(rest % (size_t)g.outw);
+    rest /= (size_t)g.outw;
+    const int oy = (int)(rest % (size_t)g.outh);
+    const int img = (int)(rest / (size_t)g.outh);
+    const int8_t* base = src + (size_t)img * g.h * g.w * g.cp + q16 * 16;
+    const int y0 = oy * g.sh - g.pad_top, x0 = ox * g.sw - g.pad_left;
+    int r[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) r[e] = -127;
+    for (int ky = 0; ky < g.kh; ky++)
+        for (int kx = 0; kx < g.kw; kx++)
+        {
+            const int y = y0 + ky, x = x0 + kx;
+            const bool in = (unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w;
+            const v4i v = *reinterpret_cast<const v4i*>(base + (in ? ((size_t)y * g.w + x) * g.cp : (size_t)0)); // unconditional: loads overlap
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+            {
+                const int b = (int)(int8_t)((unsigned)v[e >> 2] >> (8 * (e & 3)));
+                r[e] = in ? (b > r[e] ? b : r[e]) : r[e];
+            }
+        }
+    v4i o;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+        o[d] = (int)((unsigned)(r[4 * d] & 255) | ((unsigned)(r[4 * d + 1] & 255) << 8) | ((unsigned)(r[4 * d + 2] & 255) << 16) | ((unsigned)r[4 * d + 3] << 24));
+    *reinterpret_cast<v4i*>(dst + (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q16 * 16) = o;
+}
+
 // global pooling: [n][hw][cp] -> dense [n][c]; one thread per (sample, channel) walks the pixels in index order
 __global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type)
 {
@@ -209,18 +248,19 @@ __global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __
     const int img = blockIdx.y;
     if (q >= c) return;
     const float* p = src + (size_t)img * hw * cp + q;
-    float r;
-    if (type == 0)
+    // eight loads in flight, then folded in pixel order (the order of the reference's loop)
+    float r = type == 0 ? p[0] : 0.f;
+    int i = 0;
+    for (; i + 8 <= hw; i += 8)
     {
-        r = p[0];
-        for (int i = 0; i < hw; i++) r = fmaxf(r, p[(size_t)i * cp]);
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = p[(size_t)(i + e) * cp];
+#pragma unroll
+        for (int e = 0; e < 8; e++) r = type == 0 ? fmaxf(r, v[e]) : add_rn(r, v[e]);
     }
-    else
-    {
-        r = 0.f;
-        for (int i = 0; i < hw; i++) r = add_rn(r, p[(size_t)i * cp]);
-        r = div_rn(r, (float)hw);
-    }
+    for (; i < hw; i++) r = type == 0 ? fmaxf(r, p[(size_t)i * cp]) : add_rn(r, p[(size_t)i * cp]);
+    if (type != 0) r = div_rn(r, (float)hw);
     dst[(size_t)img * c + q] = r;
 }
 
@@ -599,6 +639,33 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
     const size_t total = (size_t)d.batch * d.outh * d.outw * (cp / 4);
     hipLaunchKernelGGL(pooling_nhwc_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
     return launch_status("pooling_nhwc_kernel");
+}
+
+int ncnnhip_maxpool_nhwc_int8(const ncnnhip_pool_desc* desc, const int8_t* src_dev, int8_t* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && src_dev && dst_dev, "ncnnhip_maxpool_nhwc_int8: null pointer");
+    const ncnnhip_pool_desc& d = *desc;
+    NCNNHIP_REQUIRE(d.w > 0 && d.h > 0 && d.c > 0 && d.batch > 0 && d.pooling_type == 0 && !d.global_pooling, "ncnnhip_maxpool_nhwc_int8: windowed max pooling only");
+    NCNNHIP_REQUIRE(d.kernel_w > 0 && d.kernel_h > 0 && d.stride_w > 0 && d.stride_h > 0 && d.outw > 0 && d.outh > 0, "ncnnhip_maxpool_nhwc_int8: bad window");
+    NCNNHIP_REQUIRE(d.pad_top >= 0 && d.pad_left >= 0, "ncnnhip_maxpool_nhwc_int8: negative pads");
+    NCNNHIP_REQUIRE(((reinterpret_cast<uintptr_t>(src_dev) | reinterpret_cast<uintptr_t>(dst_dev)) & 15) == 0, "ncnnhip_maxpool_nhwc_int8: blobs must be 16-byte aligned");
+    PoolGeom g;
+    g.w = d.w;
+    g.h = d.h;
+    g.cp = padded16(d.c);
+    g.outw = d.outw;
+    g.outh = d.outh;
+    g.kw = d.kernel_w;
+    g.kh = d.kernel_h;
+    g.sw = d.stride_w;
+    g.sh = d.stride_h;
+    g.pad_top = d.pad_top;
+    g.pad_left = d.pad_left;
+    g.type = 0;
+    g.count_include_pad = 0;
+    const size_t total = (size_t)d.batch * d.outh * d.outw * (g.cp / 16);
+    hipLaunchKernelGGL(maxpool_nhwc_s8_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
+    return launch_status("maxpool_nhwc_s8_kernel");
 }
 
 int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream)

@@ -89,6 +89,42 @@ int ncnnhip_stream_synchronize(void* stream)
     return NCNNHIP_OK;
 }
 
+int ncnnhip_stream_begin_capture(void* stream)
+{
+    NCNNHIP_REQUIRE(stream, "ncnnhip_stream_begin_capture: the default stream cannot be captured");
+    // thread-local: other threads keep allocating and synchronising; on this thread anything but stream work is an error
+    NCNNHIP_CHECK(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_stream_end_capture(void* stream, void** graph_exec)
+{
+    NCNNHIP_REQUIRE(stream && graph_exec, "ncnnhip_stream_end_capture: null pointer");
+    *graph_exec = 0;
+    hipGraph_t graph = 0;
+    NCNNHIP_CHECK(hipStreamEndCapture(as_stream(stream), &graph));
+    NCNNHIP_REQUIRE(graph, "ncnnhip_stream_end_capture: the capture was invalidated");
+    hipGraphExec_t exec = 0;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, 0, 0, 0);
+    (void)hipGraphDestroy(graph);
+    NCNNHIP_CHECK(e);
+    *graph_exec = exec;
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_graph_launch(void* graph_exec, void* stream)
+{
+    NCNNHIP_REQUIRE(graph_exec, "ncnnhip_graph_launch: null graph");
+    NCNNHIP_CHECK(hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_graph_destroy(void* graph_exec)
+{
+    if (graph_exec) NCNNHIP_CHECK(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_device_synchronize(void)
 {
     NCNNHIP_CHECK(hipDeviceSynchronize());

@@ -51,6 +51,10 @@ _SIGNATURES = {
     "ncnnhip_stream_destroy": [C.c_void_p],
     "ncnnhip_stream_synchronize": [C.c_void_p],
     "ncnnhip_device_synchronize": [],
+    "ncnnhip_stream_begin_capture": [C.c_void_p],
+    "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
+    "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
+    "ncnnhip_graph_destroy": [C.c_void_p],
     "ncnnhip_malloc": [c_void_pp, C.c_size_t],
     "ncnnhip_free": [C.c_void_p],
     "ncnnhip_memcpy_h2d": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
@@ -89,6 +93,7 @@ _SIGNATURES = {
     "ncnnhip_scale": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_void_p],
     "ncnnhip_eltwise": [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.POINTER(C.c_float), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_pooling_nhwc": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_maxpool_nhwc_int8": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
     "ncnnhip_softmax": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
                                   C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -353,6 +358,17 @@ class Runtime:
         d = PoolDesc(w, h, c, n, pooling_type, kernel[0], kernel[1], stride[0], stride[1], pad_top_left[0], pad_top_left[1], ow, oh, 0, int(count_include_pad))
         out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.float32)
         check(lib().ncnnhip_pooling_nhwc(C.byref(d), src.ptr, out.ptr, self.stream))
+        return self.from_channels_last(out, n, c, oh, ow)
+
+    def maxpool_int8(self, xq, kernel, stride, pad_top_left, out_hw):
+        """xq [n][c][h][w] int8 (quantised values); windowed max pooling on the int8 blob."""
+        xq = np.ascontiguousarray(xq, np.int8)
+        n, c, h, w = xq.shape
+        src = self.to_channels_last(xq)
+        oh, ow = out_hw
+        d = PoolDesc(w, h, c, n, 0, kernel[0], kernel[1], stride[0], stride[1], pad_top_left[0], pad_top_left[1], ow, oh, 0, 0)
+        out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.int8)
+        check(lib().ncnnhip_maxpool_nhwc_int8(C.byref(d), src.ptr, out.ptr, self.stream))
         return self.from_channels_last(out, n, c, oh, ow)
 
     def softmax(self, x):

@@ -45,6 +45,9 @@ def lib():
             "ncnnhip_net_upload": (ci, [vp, vp, C.POINTER(vp)]), "ncnnhip_hipmat_destroy": (None, [vp]), "ncnnhip_hipmat_download": (ci, [vp, C.POINTER(vp)]),
             "ncnnhip_extractor_input_hipmat": (ci, [vp, C.c_char_p, vp]), "ncnnhip_extractor_extract_hipmat": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
             "ncnnhip_extractor_synchronize": (ci, [vp]),
+            "ncnnhip_graph_record": (ci, [vp, C.c_char_p, vp, C.c_char_p, C.POINTER(vp)]), "ncnnhip_graph_update_input": (ci, [vp, vp]),
+            "ncnnhip_graph_replay": (ci, [vp]), "ncnnhip_graph_synchronize": (ci, [vp]), "ncnnhip_graph_output": (ci, [vp, C.POINTER(vp)]),
+            "ncnnhip_graph_release": (None, [vp]),
             "ncnn_net_get_layer_count": (ci, [vp]), "ncnn_net_get_layer_type": (C.c_char_p, [vp, ci]), "ncnn_net_get_layer_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_layer_flags": (ci, [vp, ci]), "ncnn_net_get_blob_count": (ci, [vp]), "ncnn_net_get_blob_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_blob_producer": (ci, [vp, ci]), "ncnn_net_get_blob_consumer": (ci, [vp, ci]),
@@ -185,9 +188,53 @@ class HipMat:
         return m.to_numpy()
 
 
+class HipGraph:
+    """A forward pass recorded once (Net.record) and replayed with one launch; output() is rewritten by every replay."""
+
+    def __init__(self, handle, net, keep):
+        self.h_ = handle
+        self.net = net
+        self.keep = keep  # the input blob must outlive the recording
+
+    def __del__(self):
+        try:
+            if self.h_:
+                lib().ncnnhip_graph_release(self.h_)
+                self.h_ = None
+        except Exception:
+            pass
+
+    def update_input(self, array):
+        m = array if isinstance(array, Mat) else Mat.from_numpy(array)
+        ret = lib().ncnnhip_graph_update_input(self.h_, m.h_)
+        if ret != 0:
+            raise RuntimeError("update_input returned %d" % ret)
+
+    def launch(self):
+        ret = lib().ncnnhip_graph_replay(self.h_)
+        if ret != 0:
+            raise RuntimeError("graph launch returned %d" % ret)
+
+    def synchronize(self):
+        return lib().ncnnhip_graph_synchronize(self.h_)
+
+    def output(self):
+        out = C.c_void_p()
+        lib().ncnnhip_graph_output(self.h_, C.byref(out))
+        return HipMat(out.value, self.net)
+
+
 class Net:
     def __init__(self):
         self.h_ = lib().ncnn_net_create()
+
+    def record(self, input_name, input_blob, output_name):
+        """Runs the pass from the resident input blob to output_name once, then records it for replay."""
+        out = C.c_void_p()
+        ret = lib().ncnnhip_graph_record(self.h_, input_name.encode(), input_blob.h_, output_name.encode(), C.byref(out))
+        if ret != 0:
+            raise RuntimeError("graph record returned %d" % ret)
+        return HipGraph(out.value, self, input_blob)
 
     def upload(self, array):
         """numpy [c][h][w] / [n][c][h][w] -> device-resident blob usable as input of any extractor of this net."""

@@ -254,6 +254,42 @@ int ncnnhip_extractor_synchronize(ncnn_extractor_t ex)
     return E(ex)->synchronize();
 }
 
+int ncnnhip_graph_record(ncnn_net_t net, const char* input_name, const ncnn_hipmat_t input, const char* output_name, ncnn_hipgraph_t* out)
+{
+    *out = 0;
+    if (!input) return -1;
+    HipGraph* g = new HipGraph;
+    int ret = g->record(*N(net), input_name, *(const HipMat*)input, output_name);
+    if (ret != 0)
+    {
+        delete g;
+        return ret;
+    }
+    *out = (ncnn_hipgraph_t)g;
+    return 0;
+}
+int ncnnhip_graph_update_input(ncnn_hipgraph_t g, const ncnn_mat_t mat)
+{
+    return ((HipGraph*)g)->update_input(*M(mat));
+}
+int ncnnhip_graph_replay(ncnn_hipgraph_t g)
+{
+    return ((HipGraph*)g)->launch();
+}
+int ncnnhip_graph_synchronize(ncnn_hipgraph_t g)
+{
+    return ((HipGraph*)g)->synchronize();
+}
+int ncnnhip_graph_output(ncnn_hipgraph_t g, ncnn_hipmat_t* out)
+{
+    *out = (ncnn_hipmat_t) new HipMat(((HipGraph*)g)->output());
+    return 0;
+}
+void ncnnhip_graph_release(ncnn_hipgraph_t g)
+{
+    delete (HipGraph*)g;
+}
+
 int ncnnhip_register_int8_layers(ncnn_net_t net)
 {
     using namespace ncnn_amd;

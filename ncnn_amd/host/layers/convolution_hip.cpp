@@ -1,4 +1,8 @@
+#include <math.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <algorithm>
 
 #include <vector>
 
@@ -14,7 +18,9 @@ Convolution_hip::Convolution_hip(bool depthwise_type) : is_depthwise_type(depthw
     one_blob_only = true;
     support_inplace = false;
     support_batch = true; // Mat.n is folded into the pixel dimension of the implicit GEMM
-    d_weight = d_weight_packed = d_weight_dw = d_bias = d_scale_in = d_scale_out = d_input_scales = 0;
+    d_weight = d_weight_packed = d_weight_dw = d_bias = d_scale_in = d_scale_out = d_scale_out_uniform = d_input_scales = 0;
+    uniform_scale_out = 0.f;
+    output_abs_bound = 0.0;
     input_scale_count = 0;
     group = 1;
 }
@@ -165,6 +171,20 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
     int rc = ncnnhip_fold_input_scales(weight_data_int8_scales, weight_data_int8_scales.w, bottom_blob_int8_scales, bottom_blob_int8_scales.w,
                                        num_output, scale_in.data());
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_fold_input_scales");
+    {
+        // |output| <= 127 * sum|w| * |scale_in| + |bias| for any input: what hip_prepare_requantise checks
+        const size_t per_out = (size_t)weight_data_size / (size_t)num_output;
+        const signed char* wq = (const signed char*)weight_data.data;
+        double bound = 0.0;
+        for (int p = 0; p < num_output; p++)
+        {
+            double sum = 0.0;
+            for (size_t k = 0; k < per_out; k++) sum += abs((int)wq[(size_t)p * per_out + k]);
+            double b = 127.0 * sum * fabs((double)scale_in[(size_t)p]) + (bias_term ? fabs((double)bias_data[p]) : 0.0);
+            if (!(b <= bound)) bound = b; // a NaN sticks
+        }
+        output_abs_bound = bound;
+    }
 
     int ret = 0;
     if (group == 1)
@@ -224,12 +244,13 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
 
 int Convolution_hip::destroy_pipeline(const Option& /*opt*/)
 {
-    void** all[] = {&d_weight, &d_weight_packed, &d_weight_dw, &d_bias, &d_scale_in, &d_scale_out, &d_input_scales};
+    void** all[] = {&d_weight, &d_weight_packed, &d_weight_dw, &d_bias, &d_scale_in, &d_scale_out, &d_scale_out_uniform, &d_input_scales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
         *all[i] = 0;
     }
+    uniform_scale_out = 0.f;
     return 0;
 }
 
@@ -362,6 +383,42 @@ bool Convolution_hip::hip_can_fuse_tail() const
 int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* residual, bool relu, float q8_scale, HipMat& top, HipCommand& cmd,
                                        const Option& opt) const
 {
+    return forward_device(bottom, residual, relu, q8_scale, 0.f, top, cmd, opt);
+}
+
+int Convolution_hip::hip_prepare_requantise(float scale)
+{
+    // fp32-output layers only: the reference's own requantising epilogue (convolution.cpp:489-496) then runs with
+    // the consumers' input scale in every channel, which is what their Quantize passes would compute
+    if (!support_hip || int8_scale_term > 100 || !(scale > 0.f) || !d_scale_in) return -1;
+    // Quantize is monotonic (so that it commutes with max pooling) only while value * scale stays inside the int32
+    // range: beyond it the reference's float2int8 wraps to -127.  The weights bound the output, so this is known now.
+    double gain = 1.0;
+    if (activation_type == 2 && activation_params.w >= 1) gain = std::max(1.0, fabs((double)activation_params[0]));
+    if (activation_type < 0 || activation_type > 3) return -1;
+    if (!(output_abs_bound * gain * (double)scale < 1073741824.0)) return -1;
+    if (uniform_scale_out == scale) return 0;
+    if (d_scale_out_uniform)
+    {
+        ncnnhip_free(d_scale_out_uniform);
+        d_scale_out_uniform = 0;
+        uniform_scale_out = 0.f;
+    }
+    std::vector<float> so((size_t)num_output, scale);
+    if (upload_constant(so.data(), so.size() * 4, &d_scale_out_uniform) != 0) return -1;
+    uniform_scale_out = scale;
+    return 0;
+}
+
+int Convolution_hip::forward_hip_requantised(const HipMat& bottom, float scale, HipMat& top, HipCommand& cmd, const Option& opt) const
+{
+    if (uniform_scale_out == 0.f || scale != uniform_scale_out) return -1;
+    return forward_device(bottom, 0, false, 0.f, scale, top, cmd, opt);
+}
+
+int Convolution_hip::forward_device(const HipMat& bottom, const HipMat* residual, bool relu, float q8_scale, float only_scale, HipMat& top, HipCommand& cmd,
+                                    const Option& opt) const
+{
     const bool fused = residual || relu || q8_scale != 0.f;
     if (fused && !hip_can_fuse_tail()) return -1;
     if (!opt.use_int8_inference)
@@ -391,9 +448,16 @@ int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* resid
     int rc = ncnnhip_conv_out_shape(&desc, &outw, &outh);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_out_shape");
 
-    const bool requant = int8_scale_term > 100;
+    if (bottom.elemsize == 1u && bottom.q8_scale != 0.f && bottom.q8_scale != bottom_blob_int8_scales[0])
+    {
+        NCNN_LOGE("%s %s: the int8 blob was quantised with scale %g, this layer expects %g", type.c_str(), name.c_str(), bottom.q8_scale, bottom_blob_int8_scales[0]);
+        return -1;
+    }
+    const bool requant = int8_scale_term > 100 || only_scale != 0.f;
+    const float* scale_out_table = (const float*)(only_scale != 0.f ? d_scale_out_uniform : d_scale_out);
     top.create(outw, outh, num_output, requant ? (size_t)1u : (size_t)4u, bottom.n, &cmd);
     if (top.empty()) return -100;
+    if (only_scale != 0.f) top.q8_scale = only_scale;
     ScopedScratch scratch(&cmd);
     void* st = cmd.stream;
 
@@ -443,11 +507,11 @@ int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* resid
                                               &fu, ws, workspace_bytes, st);
             return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc_fused");
         }
-        rc = ncnnhip_conv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, (const float*)d_scale_out, act,
+        rc = ncnnhip_conv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, scale_out_table, act,
                                     top.data, NCNNHIP_CHANNELS_LAST, 0, 0, ws, workspace_bytes, st);
         return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");
     }
-    rc = ncnnhip_dwconv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_dw, (const float*)d_scale_in, (const float*)d_bias, (const float*)d_scale_out, act, top.data, st);
+    rc = ncnnhip_dwconv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_dw, (const float*)d_scale_in, (const float*)d_bias, scale_out_table, act, top.data, st);
     return to_ncnn_status(rc, "ncnnhip_dwconv_int8_nhwc");
 }
 

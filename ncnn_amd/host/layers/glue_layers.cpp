@@ -204,9 +204,16 @@ public:
         outh = (h + pt + pb - kernel_h) / stride_h + 1;
     }
 
+    virtual bool hip_quantise_transparent() const
+    {
+        return support_hip && pooling_type == 0 && !global_pooling;
+    }
+
     virtual int forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option&) const
     {
-        if (bottom.dims != 3 || bottom.elemsize != 4u)
+        // an int8 blob only arrives here when the executor routed quantised values through this layer
+        const bool quantised = bottom.elemsize == 1u && bottom.q8_scale > 0.f && hip_quantise_transparent();
+        if (bottom.dims != 3 || (bottom.elemsize != 4u && !quantised))
         {
             NCNN_LOGE("Pooling: needs a 3-D fp32 blob");
             return -1;
@@ -231,8 +238,13 @@ public:
         d.stride_w = stride_w;
         d.stride_h = stride_h;
         resolve(bottom.w, bottom.h, d.pad_top, d.pad_left, d.outw, d.outh);
-        top.create(d.outw, d.outh, bottom.c, 4u, bottom.n, &cmd);
+        top.create(d.outw, d.outh, bottom.c, quantised ? (size_t)1u : (size_t)4u, bottom.n, &cmd);
         if (top.empty()) return -100;
+        if (quantised)
+        {
+            top.q8_scale = bottom.q8_scale;
+            return dev_status(ncnnhip_maxpool_nhwc_int8(&d, (const int8_t*)bottom.data, (int8_t*)top.data, cmd.stream), "ncnnhip_maxpool_nhwc_int8");
+        }
         return dev_status(ncnnhip_pooling_nhwc(&d, (const float*)bottom.data, (float*)top.data, cmd.stream), "ncnnhip_pooling_nhwc");
     }
 

@@ -27,6 +27,9 @@ public:
     virtual bool hip_can_fuse_tail() const;
     virtual int forward_hip_fused(const ncnn::HipMat& bottom_blob, const ncnn::HipMat* residual, bool relu, float q8_scale, ncnn::HipMat& top_blob,
                                   ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
+    virtual int hip_prepare_requantise(float scale);
+    virtual int forward_hip_requantised(const ncnn::HipMat& bottom_blob, float scale, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd,
+                                        const ncnn::Option& opt) const;
 
 public:
     // same member names as the reference layers
@@ -46,6 +49,11 @@ private:
     void* d_bias;
     void* d_scale_in;      // one per output channel: 1/(in_scale*w_scale), 0 when w_scale is 0
     void* d_scale_out;     // one per output channel, only when requantising
+    void* d_scale_out_uniform; // num_output copies of uniform_scale_out: the consumers' common input scale
+    float uniform_scale_out;   // 0: hip_prepare_requantise was not called
+    double output_abs_bound;   // no input makes an output (before the activation) larger in magnitude
+    int forward_device(const ncnn::HipMat& bottom_blob, const ncnn::HipMat* residual, bool relu, float q8_scale, float only_scale, ncnn::HipMat& top_blob,
+                       ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
     void* d_input_scales;  // the layer's input scale table (1 entry, or `group` entries for depthwise types)
     int input_scale_count; // 1 or group
     void* d_weight_dw;     // depthwise (channels == group == num_output): [kh*kw][16*ceil(c/16)]

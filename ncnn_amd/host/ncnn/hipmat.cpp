@@ -244,9 +244,27 @@ int HipCommand::upload(const Mat& src, HipMat& dst)
         return -1;
     }
     if (src.dims == 3)
-    {
         dst.create(src.w, src.h, src.c, src.elemsize, src.n, this);
-        if (dst.empty()) return -100;
+    else if (src.dims == 1)
+        dst.create(src.w, src.elemsize, src.n, this);
+    else
+        dst.create(src.w, src.h, src.elemsize, src.n, this);
+    if (dst.empty()) return -100;
+    return upload_into(src, dst);
+}
+
+int HipCommand::upload_into(const Mat& src, HipMat& dst)
+{
+    int ret = ensure_ready();
+    if (ret != 0) return ret;
+    if (src.empty() || dst.empty() || src.elempack != 1 || src.dims != dst.dims || src.elemsize != dst.elemsize || src.w != dst.w || src.n != dst.n
+        || (src.dims >= 2 && src.h != dst.h) || (src.dims == 3 && src.c != dst.c) || src.dims < 1 || src.dims > 3)
+    {
+        NCNN_LOGE("HipCommand::upload_into: the host blob does not have the device blob's shape and type");
+        return -1;
+    }
+    if (src.dims == 3)
+    {
         // planar bytes as they lie on the host, then one layout kernel
         ScopedScratch scratch(this);
         void* staging = scratch.get(host_bytes(src));
@@ -257,11 +275,6 @@ int HipCommand::upload(const Mat& src, HipMat& dst)
         if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
         return hip_status(rc, "upload");
     }
-    if (src.dims == 1)
-        dst.create(src.w, src.elemsize, src.n, this);
-    else
-        dst.create(src.w, src.h, src.elemsize, src.n, this);
-    if (dst.empty()) return -100;
     const size_t sample = (size_t)src.w * src.h * src.elemsize;
     int rc = 0;
     for (int b = 0; b < src.n && rc == 0; b++)

@@ -64,6 +64,8 @@ public:
     size_t elemsize;
     // An fp32 blob may travel with an int8 copy of itself, float2int8(value * q8_scale), written by the kernel
     // that produced it: the convolution that consumes the blob with that input scale then skips its Quantize pass.
+    // An int8 blob (elemsize 1, no twin) with q8_scale != 0 stands in for an fp32 blob of the model: the executor
+    // had its producer emit float2int8(value * q8_scale) directly because every consumer would quantise it so.
     std::shared_ptr<HipMat> q8;
     float q8_scale;
 
@@ -91,6 +93,7 @@ public:
 
     // host Mat (planar, any batch) -> device blob and back; download synchronises the stream
     int upload(const Mat& src, HipMat& dst);
+    int upload_into(const Mat& src, HipMat& dst); // dst exists and has src's shape: new values for the same buffer
     int download(const HipMat& src, Mat& dst, Allocator* allocator);
     int synchronize();
 

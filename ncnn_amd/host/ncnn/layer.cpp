@@ -108,6 +108,18 @@ int Layer::forward_hip_fused(const HipMat&, const HipMat*, bool, float, HipMat&,
 {
     return -1;
 }
+int Layer::hip_prepare_requantise(float)
+{
+    return -1;
+}
+int Layer::forward_hip_requantised(const HipMat&, float, HipMat&, HipCommand&, const Option&) const
+{
+    return -1;
+}
+bool Layer::hip_quantise_transparent() const
+{
+    return false;
+}
 
 // ---- built-in type table ------------------------------------------------------------------
 

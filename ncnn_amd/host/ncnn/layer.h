@@ -64,6 +64,13 @@ public:
     // top = [relu](forward(bottom) + *residual);  q8_scale != 0: top.q8 = Quantize(top, q8_scale) as well
     virtual int forward_hip_fused(const HipMat& bottom_blob, const HipMat* residual, bool relu, float q8_scale, HipMat& top_blob, HipCommand& cmd,
                                   const Option& opt) const;
+    // When every consumer of a layer's fp32 output quantises it with one positive scale, the executor asks the layer
+    // (once, after load_model) whether it can emit the quantised values alone; 0 = yes, and from then on
+    // forward_hip_requantised(bottom, scale) gives the int8 blob float2int8(forward(bottom) * scale).
+    virtual int hip_prepare_requantise(float scale);
+    virtual int forward_hip_requantised(const HipMat& bottom_blob, float scale, HipMat& top_blob, HipCommand& cmd, const Option& opt) const;
+    // forward_hip of an int8 blob holding Quantize(x, s), s > 0, gives Quantize(forward_hip(x), s) (windowed max pooling)
+    virtual bool hip_quantise_transparent() const;
 
     void* userdata;
     int typeindex;

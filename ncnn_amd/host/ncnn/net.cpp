@@ -32,6 +32,8 @@ struct ExecState
     std::vector<Mat> host;
     std::vector<HipMat> dev;
     std::shared_ptr<HipCommand> cmd; // created on the first layer that runs device-resident
+    int wanted;                      // the blob an extract call asked for (-1: none): it is produced as the model defines it
+    ExecState() : wanted(-1) {}
 
     bool has(int blob) const
     {
@@ -142,8 +144,15 @@ public:
     };
     std::vector<TailPlan> tail_plan;
     std::vector<float> quantise_scale;
+    // requant_scale[b] != 0: blob b is produced as int8, float2int8(value * scale), by its layer (a convolution
+    // that agreed in hip_prepare_requantise): every consumer, through Split and windowed max pooling, quantises with
+    // that one scale.  quantised_zone[b]: b holds such values when the plan is followed (b itself or downstream).
+    std::vector<float> requant_scale;
+    std::vector<char> quantised_zone;
     void build_fusion_plan();
     bool collect_quantise_scales(int blob, float& scale, bool& any) const;
+    bool all_consumers_quantise(int blob, float& scale, bool& any, std::vector<int>& zone) const;
+    bool follows_requant_plan(int blob, const ExecState& st, const Option& opt) const;
     int try_fused_tail(int layer_index, ExecState& st, const Option& opt, bool& done) const;
 
     int forward_layer(int layer_index, ExecState& st, const Option& opt) const;
@@ -196,11 +205,53 @@ bool NetPrivate::collect_quantise_scales(int blob, float& scale, bool& any) cons
     return true;
 }
 
+// true when every path from the blob ends, through Split and quantise-transparent layers, in a consumer that
+// quantises with the same scale; zone collects the blobs on the way
+bool NetPrivate::all_consumers_quantise(int blob, float& scale, bool& any, std::vector<int>& zone) const
+{
+    zone.push_back(blob);
+    const int ci = blobs[(size_t)blob].consumer;
+    if (ci < 0) return false; // a network output keeps the model's type
+    const Layer* consumer = layers[(size_t)ci];
+    if (consumer->type == "Split" || (consumer->support_hip && consumer->one_blob_only && consumer->hip_quantise_transparent()))
+    {
+        for (size_t i = 0; i < consumer->tops.size(); i++)
+            if (!all_consumers_quantise(consumer->tops[i], scale, any, zone)) return false;
+        return !consumer->tops.empty();
+    }
+    const float s = consumer->support_hip ? consumer->hip_input_quantise_scale() : 0.f;
+    if (!(s > 0.f) || (any && s != scale)) return false;
+    scale = s;
+    any = true;
+    return true;
+}
+
+bool NetPrivate::follows_requant_plan(int blob, const ExecState& st, const Option& opt) const
+{
+    if (!opt.use_hip_compute || !opt.lightmode || requant_scale.size() != blobs.size() || requant_scale[(size_t)blob] == 0.f) return false;
+    // an extract call that asks for a blob of this zone gets the model's own fp32 values
+    return st.wanted < 0 || !quantised_zone[(size_t)st.wanted];
+}
+
 void NetPrivate::build_fusion_plan()
 {
     const TailPlan none = {-1, -1, -1, false};
     tail_plan.assign(layers.size(), none);
     quantise_scale.assign(blobs.size(), 0.f);
+    requant_scale.assign(blobs.size(), 0.f);
+    quantised_zone.assign(blobs.size(), 0);
+    for (size_t b = 0; b < blobs.size(); b++)
+    {
+        const int p = blobs[b].producer;
+        if (p < 0 || !layers[(size_t)p]->support_hip || !layers[(size_t)p]->one_blob_only || layers[(size_t)p]->tops.size() != 1) continue;
+        float s = 0.f;
+        bool any = false;
+        std::vector<int> zone;
+        if (!all_consumers_quantise((int)b, s, any, zone) || !any) continue;
+        if (layers[(size_t)p]->hip_prepare_requantise(s) != 0) continue;
+        requant_scale[b] = s;
+        for (size_t i = 0; i < zone.size(); i++) quantised_zone[(size_t)zone[i]] = 1;
+    }
     for (size_t b = 0; b < blobs.size(); b++)
     {
         float s = 0.f;
@@ -354,7 +405,8 @@ int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& o
             st.dev[bi].release();
             st.host[bi].release();
         }
-        if (ins[i].elemsize == 1u && !layer->support_int8_storage)
+        const bool passes_quantised = ins[i].elemsize == 1u && ins[i].q8_scale > 0.f && layer->one_blob_only && layer->hip_quantise_transparent();
+        if (ins[i].elemsize == 1u && !layer->support_int8_storage && !passes_quantised)
         {
             HipMat wide;
             if (ins[i].dims == 3)
@@ -394,7 +446,9 @@ int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& o
         else
         {
             const float qs = quantise_scale.size() == blobs.size() ? quantise_scale[(size_t)layer->tops[0]] : 0.f;
-            if (qs != 0.f && layer->hip_can_fuse_tail())
+            if (follows_requant_plan(layer->tops[0], st, opt))
+                ret = layer->forward_hip_requantised(ins[0], requant_scale[(size_t)layer->tops[0]], top, cmd, opt); // only quantised values are wanted
+            else if (qs != 0.f && layer->hip_can_fuse_tail())
                 ret = layer->forward_hip_fused(ins[0], 0, false, qs, top, cmd, opt); // the consumers' Quantize rides along
             else
                 ret = layer->forward_hip(ins[0], top, cmd, opt);
@@ -892,6 +946,8 @@ void Net::clear()
     d->output_nm.clear();
     d->tail_plan.clear();
     d->quantise_scale.clear();
+    d->requant_scale.clear();
+    d->quantised_zone.clear();
     std::lock_guard<std::mutex> g(d->cmd_lock);
     d->idle_cmds.clear();
     d->io_cmd.reset();
@@ -1053,11 +1109,19 @@ int Extractor::extract(int blob_index, HipMat& feat)
     if (blob_index < 0 || blob_index >= (int)d->st.dev.size()) return -1;
     const size_t bi = (size_t)blob_index;
     int ret = 0;
+    // quantised stand-in values (see requant_scale) are not what the model defines for this blob: compute it again
+    if (!d->st.dev[bi].empty() && d->st.dev[bi].elemsize == 1u && d->st.dev[bi].q8_scale != 0.f)
+    {
+        d->st.dev[bi].release();
+        d->st.host[bi].release();
+    }
     if (!d->st.has(blob_index))
     {
         const int producer = d->net->d->blobs[bi].producer;
         if (producer < 0) return -1;
+        d->st.wanted = blob_index;
         ret = d->net->d->forward_layer(producer, d->st, d->opt);
+        d->st.wanted = -1;
     }
     if (ret == 0 && d->st.dev[bi].empty())
     {
@@ -1086,11 +1150,19 @@ int Extractor::extract(int blob_index, Mat& feat, int type)
     if (blob_index < 0 || blob_index >= (int)d->st.host.size()) return -1;
     const size_t bi = (size_t)blob_index;
     int ret = 0;
+    // quantised stand-in values (see requant_scale) are not what the model defines for this blob: compute it again
+    if (!d->st.dev[bi].empty() && d->st.dev[bi].elemsize == 1u && d->st.dev[bi].q8_scale != 0.f)
+    {
+        d->st.dev[bi].release();
+        d->st.host[bi].release();
+    }
     if (!d->st.has(blob_index))
     {
         const int producer = d->net->d->blobs[bi].producer;
         if (producer < 0) return -1;
+        d->st.wanted = blob_index;
         ret = d->net->d->forward_layer(producer, d->st, d->opt);
+        d->st.wanted = -1;
     }
     if (ret == 0 && d->st.host[bi].dims == 0 && !d->st.dev[bi].empty())
         ret = d->st.cmd->download(d->st.dev[bi], d->st.host[bi], d->opt.blob_allocator); // waits for the stream
@@ -1102,6 +1174,116 @@ int Extractor::extract(int blob_index, Mat& feat, int type)
         if (ret == 0) feat = wide;
     }
     return ret;
+}
+
+// ---- HipGraph --------------------------------------------------------------------------------
+
+class HipGraphPrivate
+{
+public:
+    HipGraphPrivate() : exec(0) {}
+    std::shared_ptr<HipCommand> cmd; // this graph's alone while it lives: its pool holds the recorded buffers
+    void* exec;
+    HipMat input, output;
+};
+
+HipGraph::HipGraph() : d(new HipGraphPrivate) {}
+
+HipGraph::~HipGraph()
+{
+    clear();
+    delete d;
+}
+
+void HipGraph::clear()
+{
+    if (d->cmd) d->cmd->synchronize();
+    if (d->exec) ncnnhip_graph_destroy(d->exec);
+    d->exec = 0;
+    d->output.release();
+    d->input.release();
+    d->cmd.reset(); // not handed back to the net: the net may be gone
+}
+
+int HipGraph::record(const Net& net, const char* input_name, const HipMat& input, const char* output_name)
+{
+    clear();
+    if (!net.opt.use_hip_compute || !net.opt.lightmode)
+    {
+        NCNN_LOGE("HipGraph::record: needs a net with use_hip_compute and lightmode");
+        return -1;
+    }
+    if (input.empty() || net.find_blob_index_by_name(input_name) < 0 || net.find_blob_index_by_name(output_name) < 0) return -1;
+    std::shared_ptr<HipCommand> cmd = net.d->acquire_command();
+    int ret = cmd->ensure_ready();
+    if (ret != 0) return ret;
+    // a plain pass first: every pool buffer, workspace and lazily created table exists afterwards, so the recorded
+    // pass allocates nothing
+    {
+        Extractor ex = net.create_extractor();
+        ex.d->st.cmd = cmd;
+        HipMat warm;
+        ret = ex.input(input_name, input);
+        if (ret == 0) ret = ex.extract(output_name, warm);
+        if (ret == 0) ret = cmd->synchronize();
+    }
+    if (ret != 0) return ret;
+    if (ncnnhip_stream_begin_capture(cmd->stream) != 0)
+    {
+        NCNN_LOGE("HipGraph::record: %s", ncnnhip_last_error());
+        return -1;
+    }
+    HipMat out;
+    {
+        Extractor ex = net.create_extractor();
+        ex.d->st.cmd = cmd;
+        ret = ex.input(input_name, input);
+        if (ret == 0) ret = ex.extract(output_name, out);
+    }
+    void* exec = 0;
+    const int rc = ncnnhip_stream_end_capture(cmd->stream, &exec); // also when the pass failed: the stream must leave capture mode
+    if (ret == 0 && rc != 0)
+    {
+        NCNN_LOGE("HipGraph::record: %s (a layer without a device overload on the way?)", ncnnhip_last_error());
+        ret = -1;
+    }
+    if (ret != 0)
+    {
+        if (exec) ncnnhip_graph_destroy(exec);
+        return ret;
+    }
+    d->cmd = cmd;
+    d->exec = exec;
+    d->input = input;
+    d->output = out;
+    return 0;
+}
+
+int HipGraph::update_input(const Mat& src)
+{
+    if (!d->exec) return -1;
+    return d->cmd->upload_into(src, d->input);
+}
+
+int HipGraph::launch()
+{
+    if (!d->exec) return -1;
+    if (ncnnhip_graph_launch(d->exec, d->cmd->stream) != 0)
+    {
+        NCNN_LOGE("HipGraph::launch: %s", ncnnhip_last_error());
+        return -1;
+    }
+    return 0;
+}
+
+int HipGraph::synchronize()
+{
+    return d->cmd ? d->cmd->synchronize() : 0;
+}
+
+const HipMat& HipGraph::output() const
+{
+    return d->output;
 }
 
 } // namespace ncnn

@@ -59,6 +59,7 @@ public:
 
 protected:
     friend class Extractor;
+    friend class HipGraph;
     int find_blob_index_by_name(const char* name) const;
     int find_layer_index_by_name(const char* name) const;
 
@@ -99,10 +100,39 @@ public:
 
 protected:
     friend Extractor Net::create_extractor() const;
+    friend class HipGraph;
     Extractor(const Net* net, size_t blob_count);
 
 private:
     ExtractorPrivate* const d;
+};
+
+// One forward pass of a device-resident net, recorded once and replayed with a single launch: at batch 1 a pass is
+// dozens of kernels of a few microseconds each and the host cannot describe them as fast as the GPU runs them.  The
+// reference's GPU path has the same split between recording and submitting (VkCompute, src/command.h:22-67).
+//   HipGraph g;  g.record(net, "data", in_dev, "prob");        // runs the pass once, then records it
+//   g.update_input(host_mat);  g.launch();  g.synchronize();   // any number of times
+//   g.output()                                                  // the result blob, rewritten by every launch
+// The recording reads the input blob's buffer and owns every buffer in between, so: one launch at a time per graph,
+// take what you need from output() before the next launch, and keep the net loaded while the graph lives.  Needs
+// use_hip_compute and light mode, and a path from input to output on which every layer has a device overload.
+class HipGraphPrivate;
+class NCNN_EXPORT HipGraph
+{
+public:
+    HipGraph();
+    ~HipGraph();
+    int record(const Net& net, const char* input_name, const HipMat& input, const char* output_name);
+    int update_input(const Mat& src); // same shape as the recorded input; the copy has completed on return
+    int launch();
+    int synchronize();
+    const HipMat& output() const;
+    void clear();
+
+private:
+    HipGraph(const HipGraph&);
+    HipGraph& operator=(const HipGraph&);
+    HipGraphPrivate* const d;
 };
 
 } // namespace ncnn

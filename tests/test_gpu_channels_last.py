@@ -140,6 +140,25 @@ def test_pooling_matches_scalar_restatement(rt, kind, k, s, pt, pl, include_pad)
         assert np.array_equal(got[i], _pool_ref(x[i], kind, k, s, pt, pl, oh, ow, include_pad))
 
 
+@pytest.mark.parametrize("k,s,pt,pl", [((3, 3), (2, 2), 0, 0), ((3, 3), (2, 2), 1, 1), ((2, 3), (1, 2), 0, 1), ((3, 3), (2, 2), 2, 2)])
+def test_int8_max_pooling_is_the_quantised_fp32_max_pooling(rt, k, s, pt, pl):
+    """Quantize is monotonic while value * scale stays inside the int32 range (beyond it the reference's float2int8
+    wraps to -127): pooling the quantised blob == quantising the pooled blob (the oracle's float2int8)."""
+    rng = np.random.default_rng(k[0] * 7 + pt)
+    n, c, h, w = 2, 37, 11, 12
+    x = rng.normal(0, 1, (n, c, h, w)).astype(F)
+    x[0, 0, 0, 0] = 1e6   # clamps to 127
+    x[0, 1, 0, 0] = -1e6  # clamps to -127
+    scale = F(50.0)
+    oh = -(-(h + pt - k[1]) // s[1]) + 1
+    ow = -(-(w + pl - k[0]) // s[0]) + 1
+    xq = oracle.quantize(x.reshape(1, -1), scale).reshape(x.shape)
+    got = rt.maxpool_int8(xq, k, s, (pt, pl), (oh, ow))
+    for i in range(n):
+        pooled = _pool_ref(x[i], 0, k, s, pt, pl, oh, ow, 0)
+        assert np.array_equal(got[i], oracle.quantize(pooled.reshape(1, -1), scale).reshape(pooled.shape))
+
+
 @pytest.mark.parametrize("kind", [0, 1])
 def test_global_pooling(rt, kind):
     rng = np.random.default_rng(kind)

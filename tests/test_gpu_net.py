@@ -173,6 +173,14 @@ def test_benchmark_network_batch1_matches_oracle_executor(which, hw):
         ex = net.create_extractor()
         ex.input("data", x)
         assert np.array_equal(ex.extract(probe), ref[probe].astype(F))
+        if which == "resnet50":
+            # the stem's convolution -> max pooling -> two quantising convolutions runs on quantised values when the
+            # whole net is asked for; asked for by name, its blobs still come out as the model defines them (fp32)
+            for name in ("conv1", "pool1"):
+                ex = net.create_extractor()
+                ex.input("data", x)
+                got = ex.extract(name)
+                assert got.dtype == F and np.array_equal(got, ref[name]), name
     # batch 2, device-resident: the folded batch equals the per-sample result
     xs = np.stack([x, x[:, ::-1].copy()])
     ex = net.create_extractor()
@@ -182,3 +190,38 @@ def test_benchmark_network_batch1_matches_oracle_executor(which, hw):
     ex1 = net.create_extractor()
     ex1.input("data", xs[1])
     assert np.array_equal(got[1].reshape(-1), ex1.extract(last_fc).reshape(-1))
+
+
+@pytest.mark.parametrize("which,batch", [("tiny", 1), ("tiny", 3), ("mobilenetv2", 1), ("resnet50", 2)])
+def test_recorded_pass_replays_like_the_eager_pass(which, batch):
+    """A pass recorded into a graph and replayed: every replay, with new input values and with eager work and
+    synchronisations in between, gives the eager Extractor's result bit for bit."""
+    _say("building", which)
+    kw = {} if which == "tiny" else {"input_hw": 96, "n_calib": 1}
+    g, param, blob, info = zoo.build(which, **kw)
+    out_name = {"tiny": "fc", "mobilenetv2": "fc", "resnet50": "fc1000"}[which]
+    net = _load(param, blob, True)
+    rng = np.random.default_rng(11)
+    shape = (batch,) + tuple(g.input_shape)
+    x0 = rng.uniform(0, 1, shape).astype(F)
+
+    def eager(x):
+        ex = net.create_extractor()
+        ex.input("data", x if batch > 1 else x[0])
+        return np.asarray(ex.extract(out_name)).reshape(batch, -1)
+
+    xin = net.upload(x0 if batch > 1 else x0[0])
+    graph = net.record("data", xin, out_name)
+    graph.launch()
+    graph.synchronize()
+    assert np.array_equal(graph.output().to_numpy().reshape(batch, -1), eager(x0))
+    for i in range(4):
+        x = rng.uniform(0, 1, shape).astype(F)
+        want = eager(x)  # eager work on another stream of the same net between the replays
+        graph.update_input(x if batch > 1 else x[0])
+        graph.launch()
+        if i % 2:
+            graph.launch()  # back-to-back replays of the same values
+        graph.synchronize()
+        got = graph.output().to_numpy().reshape(batch, -1)
+        assert np.array_equal(got, want), i
