@@ -83,6 +83,10 @@ int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* ma
  * before load_param.  Returns 0, or -1 if a registration was refused.
  */
 int ncnnhip_register_int8_layers(ncnn_net_t net);
+/* The same route for MultiHeadAttention with block-quantised weights (quantize_term 4xx / 6xx / 8xx,
+ * src/layer/multiheadattention.cpp:561-912).  Registered separately: a net whose attention layers are not
+ * block-quantised must keep the reference's own layer. */
+int ncnnhip_register_attention_layer(ncnn_net_t net);
 
 /* Device-resident ends of an inference (Option::use_hip_compute on): a blob uploaded once with ncnnhip_net_upload feeds any
  * number of extractors without another copy; ncnnhip_extractor_extract_hipmat enqueues the layers and returns the result

@@ -55,6 +55,8 @@ int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream);
 int ncnnhip_memcpy_d2h(void* host, const void* dev, size_t bytes, void* stream);
 int ncnnhip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 int ncnnhip_memset(void* dev, int byte, size_t bytes, void* stream);
+/* rows x row_bytes between two pitched device buffers (appending to a key/value cache whose rows grow) */
+int ncnnhip_copy2d(void* dst_dev, size_t dst_pitch, const void* src_dev, size_t src_pitch, size_t row_bytes, size_t rows, void* stream);
 int ncnnhip_event_create(void** event);
 int ncnnhip_event_destroy(void* event);
 int ncnnhip_event_record(void* event, void* stream);
@@ -283,6 +285,16 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
                                         const uint8_t* packed_w_dev, const float* packed_descale_dev, const float* c_dev,
                                         int broadcast_type_c, float alpha, float beta, float* out_dev, size_t out_stride,
                                         void* stream);
+
+/* ------------------------------------------------------------------ attention
+ * The core of MultiHeadAttention::forward_weight_block_quantize (src/layer/multiheadattention.cpp:776-866):
+ * per head, scores = q k^T (+ mask), softmax over the keys, times v.  q (already scaled) and out are
+ * [seq][num_heads*head_dim]; kt / vt are [num_heads*head_dim][dst_seqlen] with row stride kv_stride, the layout of
+ * the layer's cache blobs; mask is additive, [src][dst] (mask_heads 1) or [num_heads][src][dst], or NULL.
+ * head_dim + dst_seqlen <= 4096. */
+int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
+                          int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev,
+                          void* stream);
 
 #pragma GCC visibility pop
 

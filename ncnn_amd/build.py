@@ -9,7 +9,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 LIBNCNNHIP = os.path.join(LIBDIR, "libncnnhip.so")
 
-HIP_SOURCES = ["runtime.hip", "quantize.hip", "gemm_int8.hip", "gemm_int8_pipelined.hip", "conv_int8.hip", "conv_nhwc.hip", "conv_nhwc_pipelined.hip", "nhwc_ops.hip", "blockquant.hip"]
+HIP_SOURCES = ["runtime.hip", "quantize.hip", "gemm_int8.hip", "gemm_int8_pipelined.hip", "conv_int8.hip", "conv_nhwc.hip", "conv_nhwc_pipelined.hip", "nhwc_ops.hip", "attention.hip", "blockquant.hip"]
 
 # -ffp-contract=off: the reference arithmetic is separate mul and add, never FMA.
 # packed-fp32 ops are switched off for this pool's gfx950 parts.
@@ -48,7 +48,7 @@ def build_kernels(jobs=8):
 
 HOST_SOURCES = ["ncnn/allocator.cpp", "ncnn/mat.cpp", "ncnn/option.cpp", "ncnn/datareader.cpp", "ncnn/paramdict.cpp", "ncnn/modelbin.cpp", "ncnn/hipmat.cpp",
                 "ncnn/layer.cpp", "ncnn/net.cpp", "layers/glue_layers.cpp", "layers/hip_support.cpp", "layers/convolution_hip.cpp",
-                "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "c_api.cpp"]
+                "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "layers/multiheadattention_hip.cpp", "c_api.cpp"]
 LIBNCNN_AMD = os.path.join(LIBDIR, "libncnn_amd.so")
 
 # strict IEEE on the host too: the load-time weight quantiser and the scale folding must round

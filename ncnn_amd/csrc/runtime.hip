@@ -89,6 +89,14 @@ int ncnnhip_stream_synchronize(void* stream)
     return NCNNHIP_OK;
 }
 
+int ncnnhip_copy2d(void* dst_dev, size_t dst_pitch, const void* src_dev, size_t src_pitch, size_t row_bytes, size_t rows, void* stream)
+{
+    NCNNHIP_REQUIRE(dst_dev && src_dev && dst_pitch >= row_bytes && src_pitch >= row_bytes, "ncnnhip_copy2d: bad argument");
+    if (row_bytes == 0 || rows == 0) return NCNNHIP_OK;
+    NCNNHIP_CHECK(hipMemcpy2DAsync(dst_dev, dst_pitch, src_dev, src_pitch, row_bytes, rows, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_stream_begin_capture(void* stream)
 {
     NCNNHIP_REQUIRE(stream, "ncnnhip_stream_begin_capture: the default stream cannot be captured");

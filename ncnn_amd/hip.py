@@ -51,6 +51,8 @@ _SIGNATURES = {
     "ncnnhip_stream_destroy": [C.c_void_p],
     "ncnnhip_stream_synchronize": [C.c_void_p],
     "ncnnhip_device_synchronize": [],
+    "ncnnhip_copy2d": [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p],
+    "ncnnhip_attention_f32": [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_stream_begin_capture": [C.c_void_p],
     "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
     "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
@@ -370,6 +372,18 @@ class Runtime:
         out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.int8)
         check(lib().ncnnhip_maxpool_nhwc_int8(C.byref(d), src.ptr, out.ptr, self.stream))
         return self.from_channels_last(out, n, c, oh, ow)
+
+    def attention(self, q, kt, vt, num_heads, mask=None):
+        """q [src][embed] (scaled), kt / vt [embed][dst], mask [src][dst] or [heads][src][dst] -> [src][embed]."""
+        q, kt, vt = [np.ascontiguousarray(a, np.float32) for a in (q, kt, vt)]
+        src, embed = q.shape
+        dst = kt.shape[1]
+        dq, dk, dv = self.up(q), self.up(kt), self.up(vt)
+        dm = None if mask is None else self.up(np.ascontiguousarray(mask, np.float32))
+        mask_heads = 0 if mask is None else (1 if mask.ndim == 2 else mask.shape[0])
+        out = DeviceBuffer.empty((src, embed), np.float32)
+        check(lib().ncnnhip_attention_f32(dq.ptr, dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads, src, dst, out.ptr, self.stream))
+        return out.to_numpy(self.stream)
 
     def softmax(self, x):
         x = np.ascontiguousarray(x, np.float32)

@@ -41,7 +41,7 @@ def lib():
             "ncnn_net_get_input_name": (C.c_char_p, [vp, ci]), "ncnn_net_get_output_name": (C.c_char_p, [vp, ci]),
             "ncnn_extractor_create": (vp, [vp]), "ncnn_extractor_destroy": (None, [vp]), "ncnn_extractor_set_option": (None, [vp, vp]),
             "ncnn_extractor_input": (ci, [vp, C.c_char_p, vp]), "ncnn_extractor_extract": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
-            "ncnnhip_register_int8_layers": (ci, [vp]), "ncnnhip_extractor_attach_stream": (vp, [vp]), "ncnnhip_extractor_detach_stream": (None, [vp]),
+            "ncnnhip_register_int8_layers": (ci, [vp]), "ncnnhip_register_attention_layer": (ci, [vp]), "ncnnhip_extractor_attach_stream": (vp, [vp]), "ncnnhip_extractor_detach_stream": (None, [vp]),
             "ncnnhip_net_upload": (ci, [vp, vp, C.POINTER(vp)]), "ncnnhip_hipmat_destroy": (None, [vp]), "ncnnhip_hipmat_download": (ci, [vp, C.POINTER(vp)]),
             "ncnnhip_extractor_input_hipmat": (ci, [vp, C.c_char_p, vp]), "ncnnhip_extractor_extract_hipmat": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
             "ncnnhip_extractor_synchronize": (ci, [vp]),
@@ -252,6 +252,9 @@ class Net:
                 self.h_ = None
         except Exception:
             pass
+
+    def register_attention_layer(self):
+        return lib().ncnnhip_register_attention_layer(self.h_)
 
     def register_int8_layers(self):
         return lib().ncnnhip_register_int8_layers(self.h_)

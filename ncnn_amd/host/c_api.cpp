@@ -301,6 +301,11 @@ int ncnnhip_register_int8_layers(ncnn_net_t net)
     return ret ? -1 : 0;
 }
 
+int ncnnhip_register_attention_layer(ncnn_net_t net)
+{
+    return N(net)->register_custom_layer("MultiHeadAttention", ncnn_amd::MultiHeadAttention_hip_creator, ncnn_amd::hip_layer_destroyer, net) ? -1 : 0;
+}
+
 void* ncnnhip_extractor_attach_stream(ncnn_extractor_t ex)
 {
     ncnn_amd::HipBlobAllocator* a = new ncnn_amd::HipBlobAllocator;

@@ -121,6 +121,29 @@ private:
     int b_ready_int8; // constant B sits on the device quantised and transposed
 };
 
+// MultiHeadAttention with block-quantised weights (src/layer/multiheadattention.{h,cpp})
+class MultiHeadAttention_hip : public ncnn::Layer
+{
+public:
+    MultiHeadAttention_hip();
+    virtual ~MultiHeadAttention_hip();
+    virtual int load_param(const ncnn::ParamDict& pd);
+    virtual int load_model(const ncnn::ModelBin& mb);
+    virtual int create_pipeline(const ncnn::Option& opt);
+    virtual int destroy_pipeline(const ncnn::Option& opt);
+    virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+
+public:
+    int embed_dim, num_heads, weight_data_size, kdim, vdim, attn_mask, kv_cache, quantize_term, weight_block_quantize;
+    float scale;
+    // index 0..3 = the q, k, v and out projections
+    ncnn::Mat weight_data[4], bias_data[4], weight_data_quantize_scales[4], weight_data_input_scales[4];
+
+private:
+    void* dev[4][4]; // per projection: packed weights, block scales, input scales (or 0), bias
+};
+
+ncnn::Layer* MultiHeadAttention_hip_creator(void* userdata);
 ncnn::Layer* Convolution_hip_creator(void* userdata);
 ncnn::Layer* ConvolutionDepthWise_hip_creator(void* userdata);
 ncnn::Layer* InnerProduct_hip_creator(void* userdata);

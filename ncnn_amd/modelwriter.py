@@ -69,6 +69,30 @@ def gemm_param(name, bottoms, top, M=0, N=0, K=0, alpha=1.0, beta=1.0, transA=0,
                broadcast_type_C, output_N1M, output_transpose, quantize_term))
 
 
+def mha_param(name, bottoms, tops, embed_dim, num_heads, qdim, kdim=None, vdim=None, attn_mask=0, kv_cache=0, quantize_term=801, scale=None):
+    """MultiHeadAttention (src/layer/multiheadattention.cpp:64-76): 2 = weight_data_size = embed_dim * qdim."""
+    s = "%-24s %-24s %d %d %s %s 0=%d 1=%d 2=%d 3=%d 4=%d 5=%d" % ("MultiHeadAttention", name, len(bottoms), len(tops), " ".join(bottoms), " ".join(tops),
+                                                                 embed_dim, num_heads, embed_dim * qdim, kdim or embed_dim, vdim or embed_dim, attn_mask)
+    if scale is not None:
+        s += " 6=%s" % fmt(scale)
+    return s + " 7=%d 18=%d" % (kv_cache, quantize_term)
+
+
+def mha_blockquant_weights(weights):
+    """weights: 4 x (packed uint8 [rows][bytes], scales [rows][nblk], input scales [K] or None, bias [rows]) for q, k, v, out, in the order
+    MultiHeadAttention::load_model reads them (src/layer/multiheadattention.cpp:137-184): weight+bias pairs, then the block scales,
+    then the input scales."""
+    out = b""
+    for packed, scales, ins, bias in weights:
+        out += weight_blob(np.ascontiguousarray(packed).view(np.int8)) + raw_f32(bias)
+    for packed, scales, ins, bias in weights:
+        out += raw_f32(scales)
+    for packed, scales, ins, bias in weights:
+        if ins is not None:
+            out += raw_f32(ins)
+    return out
+
+
 def assemble_param(lines):
     """lines: layer lines in order; counts layers and distinct blobs for the header."""
     blobs = set()

@@ -22,6 +22,8 @@
  *   inner product int8  src/layer/innerproduct.cpp:168-273
  *   gemm int8           src/layer/gemm.cpp:495-567, 745-966
  *   gemm block quant    src/layer/gemm.cpp:318-483
+ *   attention with block-quantised weights  src/layer/multiheadattention.cpp:541-912 (which blob is
+ *                       q / k / v / mask / cache: :914-1028)
  *   load-time weight quantisation  convolution.cpp:89-107, convolutiondepthwise.cpp:118-140,
  *                       innerproduct.cpp:62-79
  *
@@ -31,6 +33,9 @@
  * packing inverse that ncnn's tests/test_gemm_block_quant.cpp:11-25,80-129 defines; structural
  * identities (1x1 conv == gemm rows, depthwise == group conv with group=C, zero weight scale
  * => act(bias)).
+ * the attention layer against a float64 evaluation of softmax(q k^T * scale + mask) v on the
+ * dequantised weights, against torch.nn.functional.multi_head_attention_forward, and through the
+ * cache identity (a pass over n tokens == n passes of one token that feed their cache back).
  * Parity unpinned: activation types 4 (sigmoid) and 5 (mish) depend on the host libm and are
  * not part of any benchmark configuration; the out-of-range/NaN branch of float2int8 follows
  * what x86 cvttss2si produces (INT_MIN -> -127) and is pinned only by that statement.
@@ -590,4 +595,160 @@ ORACLE_API void oracle_set_num_threads(int n)
 #else
     (void)n;
 #endif
+}
+
+
+/* ------------------------------------------------------------------ attention, block-quantised weights
+ * MultiHeadAttention::forward_weight_block_quantize (src/layer/multiheadattention.cpp:561-912).
+ * Inputs as the layer sees them: q [src_seqlen][qdim], k [cur_seqlen][kdim], v [cur_seqlen][vdim] fp32;
+ * mask [src][dst] (mask_heads 1) or [num_heads][src][dst]; cached_k / cached_v [embed_dim][past_seqlen].
+ * self_attention != 0: k and v are computed from their inputs and appended to the cache (dst = past + cur);
+ * self_attention == 0 with a cache: k and v ARE the cache (dst = past), their inputs are not read.
+ * Weight matrices in the .bin layout of the block-quantised Gemm; w[0..3] = q, k, v, out.
+ * out [src][qdim]; k_out / v_out (optional) [embed_dim][dst], the layout the layer hands back as its cache. */
+typedef struct
+{
+    const uint8_t* packed;   /* [rows][ceil(K*bits/8)] */
+    const float* scales;     /* [rows][ceil(K/block)] */
+    const float* in_scales;  /* [K] or NULL */
+    const float* bias;       /* [rows] */
+} oracle_mha_weight;
+
+typedef struct
+{
+    int embed_dim, num_heads, qdim, kdim, vdim;
+    int src_seqlen, cur_seqlen, past_seqlen;
+    int self_attention;
+    int mask_heads; /* 0: none */
+    float scale;
+    int bits, block;
+} oracle_mha_desc;
+
+/* one projection, result transposed: dst[j][col0 + i] = bias[j] + sum_k x[i][k] * w[j][k]  (times post) */
+static void mha_affine(const float* x, int rows, int K, const oracle_mha_weight* w, int out_rows, int bits, int block, float post, int use_post,
+                       float* dst, int dst_stride, int col0)
+{
+    const int packed = (int)(((size_t)K * bits + 7) / 8);
+    const int nblk = (K + block - 1) / block;
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int i = 0; i < rows; i++)
+    {
+        for (int j = 0; j < out_rows; j++)
+        {
+            const float* ptr = x + (size_t)i * K;
+            const uint8_t* kptr = w->packed + (size_t)j * packed;
+            const float* sr = w->scales + (size_t)j * nblk;
+            float sum = w->bias[j];
+            for (int k0 = 0; k0 < K; k0 += block)
+            {
+                const int kend = k0 + block < K ? k0 + block : K;
+                const float descale = 1.f / sr[k0 / block];
+                for (int k = k0; k < kend; k++)
+                {
+                    const int q = oracle_blockquant_unpack(kptr, k, bits, packed);
+                    float v = ptr[k];
+                    if (w->in_scales) v = v * w->in_scales[k];
+                    const float wv = (float)q * descale;
+                    const float prod = v * wv;
+                    sum = sum + prod;
+                }
+            }
+            dst[(size_t)j * dst_stride + col0 + i] = use_post ? sum * post : sum;
+        }
+    }
+}
+
+ORACLE_API int oracle_mha_blockquant(const oracle_mha_desc* d, const float* q, const float* k, const float* v, const float* mask, const float* cached_k,
+                                     const float* cached_v, const oracle_mha_weight* w, float* out, float* k_out, float* v_out)
+{
+    const int E = d->embed_dim, H = d->num_heads, src = d->src_seqlen, cur = d->cur_seqlen, past = d->past_seqlen;
+    if (E <= 0 || H <= 0 || E % H != 0) return -1;
+    const int hd = E / H;
+    const int dst = past > 0 ? (d->self_attention ? past + cur : past) : cur;
+    float* qa = (float*)malloc((size_t)E * src * sizeof(float));   /* [E][src] */
+    float* ka = (float*)malloc((size_t)E * dst * sizeof(float));   /* [E][dst] */
+    float* va = (float*)malloc((size_t)E * dst * sizeof(float));
+    float* att = (float*)malloc((size_t)H * src * dst * sizeof(float));
+    float* ctx = (float*)malloc((size_t)src * E * sizeof(float));  /* [src][E]: the out projection reads rows */
+    if (!qa || !ka || !va || !att || !ctx)
+    {
+        free(qa); free(ka); free(va); free(att); free(ctx);
+        return -100;
+    }
+    mha_affine(q, src, d->qdim, &w[0], E, d->bits, d->block, d->scale, 1, qa, src, 0);
+    if (past > 0 && !d->self_attention)
+    {
+        memcpy(ka, cached_k, (size_t)E * dst * sizeof(float));
+        memcpy(va, cached_v, (size_t)E * dst * sizeof(float));
+    }
+    else
+    {
+        for (int e = 0; e < E && past > 0; e++)
+        {
+            memcpy(ka + (size_t)e * dst, cached_k + (size_t)e * past, (size_t)past * sizeof(float));
+            memcpy(va + (size_t)e * dst, cached_v + (size_t)e * past, (size_t)past * sizeof(float));
+        }
+        mha_affine(k, cur, d->kdim, &w[1], E, d->bits, d->block, 0.f, 0, ka, dst, past);
+        mha_affine(v, cur, d->vdim, &w[2], E, d->bits, d->block, 0.f, 0, va, dst, past);
+    }
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int h = 0; h < H; h++)
+    {
+        for (int i = 0; i < src; i++)
+        {
+            float* row = att + ((size_t)h * src + i) * dst;
+            for (int j = 0; j < dst; j++)
+            {
+                float sum = 0.f;
+                for (int l = 0; l < hd; l++)
+                {
+                    const float prod = qa[(size_t)(h * hd + l) * src + i] * ka[(size_t)(h * hd + l) * dst + j];
+                    sum = sum + prod;
+                }
+                row[j] = sum;
+            }
+            if (d->mask_heads)
+            {
+                const float* m = mask + ((size_t)(d->mask_heads > 1 ? h : 0) * src + i) * dst;
+                for (int j = 0; j < dst; j++) row[j] = row[j] + m[j];
+            }
+            float mx = -3.402823466e+38f;
+            for (int j = 0; j < dst; j++) mx = row[j] > mx ? row[j] : mx;
+            float total = 0.f;
+            for (int j = 0; j < dst; j++)
+            {
+                row[j] = expf(row[j] - mx);
+                total = total + row[j];
+            }
+            for (int j = 0; j < dst; j++) row[j] = row[j] / total;
+            for (int l = 0; l < hd; l++)
+            {
+                const float* vr = va + (size_t)(h * hd + l) * dst;
+                float sum = 0.f;
+                for (int j = 0; j < dst; j++)
+                {
+                    const float prod = row[j] * vr[j];
+                    sum = sum + prod;
+                }
+                ctx[(size_t)i * E + h * hd + l] = sum;
+            }
+        }
+    }
+    /* out[i][j] = bias[j] + sum_k ctx[i][k] * w_out[j][k] */
+    {
+        float* tmp = (float*)malloc((size_t)d->qdim * src * sizeof(float));
+        if (!tmp)
+        {
+            free(qa); free(ka); free(va); free(att); free(ctx);
+            return -100;
+        }
+        mha_affine(ctx, src, E, &w[3], d->qdim, d->bits, d->block, 0.f, 0, tmp, src, 0);
+        for (int i = 0; i < src; i++)
+            for (int j = 0; j < d->qdim; j++) out[(size_t)i * d->qdim + j] = tmp[(size_t)j * src + i];
+        free(tmp);
+    }
+    if (k_out) memcpy(k_out, ka, (size_t)E * dst * sizeof(float));
+    if (v_out) memcpy(v_out, va, (size_t)E * dst * sizeof(float));
+    free(qa); free(ka); free(va); free(att); free(ctx);
+    return 0;
 }

@@ -235,3 +235,38 @@ def gemm_blockquant(a, b_packed, scales, bits, block, in_scales=None, c=None, br
                                  _p(in_scales), _p(c), int(broadcast_type_c if c is not None else -1), C.c_float(alpha),
                                  C.c_float(beta), _p(out), C.c_size_t(n))
     return out
+
+
+class MhaWeight(C.Structure):
+    _fields_ = [("packed", C.c_void_p), ("scales", C.c_void_p), ("in_scales", C.c_void_p), ("bias", C.c_void_p)]
+
+
+class MhaDesc(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("embed_dim", "num_heads", "qdim", "kdim", "vdim", "src_seqlen", "cur_seqlen", "past_seqlen", "self_attention",
+                                       "mask_heads")] + [("scale", C.c_float), ("bits", C.c_int), ("block", C.c_int)]
+
+
+def mha_blockquant(q, k, v, weights, embed_dim, num_heads, scale, bits, block, mask=None, cached_k=None, cached_v=None, self_attention=True):
+    """MultiHeadAttention with block-quantised weights.  q [src][qdim], k [cur][kdim], v [cur][vdim];
+    weights = 4 x (packed uint8 [rows][..], scales [rows][nblk], in_scales [K] or None, bias [rows]) for q, k, v, out;
+    mask [src][dst] or [heads][src][dst]; cached_k / cached_v [embed_dim][past].  Returns (out, k_cache, v_cache)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    src, qdim = q.shape
+    cur = k.shape[0]
+    past = 0 if cached_k is None else cached_k.shape[1]
+    dst = (past + cur if self_attention else past) if past > 0 else cur
+    keep, ws = [], (MhaWeight * 4)()
+    for i, (packed, scales, in_scales, bias) in enumerate(weights):
+        arrs = [np.ascontiguousarray(packed, np.uint8), _f32(scales), _f32(in_scales), _f32(bias)]
+        keep.append(arrs)
+        ws[i] = MhaWeight(*[None if a is None else a.ctypes.data for a in arrs])
+    mask, cached_k, cached_v = _f32(mask), _f32(cached_k), _f32(cached_v)
+    mask_heads = 0 if mask is None else (1 if mask.ndim == 2 else mask.shape[0])
+    d = MhaDesc(embed_dim, num_heads, qdim, k.shape[1], v.shape[1], src, cur, past, int(bool(self_attention)), mask_heads, float(scale), bits, block)
+    out = np.empty((src, qdim), np.float32)
+    ko = np.empty((embed_dim, dst), np.float32)
+    vo = np.empty((embed_dim, dst), np.float32)
+    ret = lib().oracle_mha_blockquant(C.byref(d), _p(q), _p(k), _p(v), _p(mask), _p(cached_k), _p(cached_v), ws, _p(out), _p(ko), _p(vo))
+    if ret != 0:
+        raise RuntimeError("oracle_mha_blockquant returned %d" % ret)
+    return out, ko, vo

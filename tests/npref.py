@@ -163,3 +163,43 @@ def blockquant_gemm_f64(a, packed, scales, bits, block, in_scales=None, c=None, 
         val = val + cv * float(np.float32(beta))
         floor = floor + np.abs(cv * float(np.float32(beta)))
     return val * float(np.float32(alpha)), floor * abs(float(np.float32(alpha)))
+
+
+def blockquant_dequantise(packed, scales, k, bits, block):
+    """The fp32 weight values q * (1/scale) the block-quantised layers multiply with, [n][k]."""
+    q = blockquant_unpack_all(packed, k, bits)
+    descale = (F(1) / np.asarray(scales, np.float32)).astype(np.float32)
+    return (q.astype(np.float32) * np.repeat(descale, block, axis=1)[:, :k]).astype(np.float32)
+
+
+def mha_f64(q, k, v, weights, embed_dim, num_heads, scale, bits, block, mask=None, cached_k=None, cached_v=None, self_attention=True):
+    """float64 softmax(q k^T * scale + mask) v with dequantised weights; the textbook formulation, batch-free.
+    weights: 4 x (packed, scales, in_scales or None, bias).  Returns (out [src][qdim], k [embed][dst], v [embed][dst])."""
+    def proj(x, w):
+        packed, scales, ins, bias = w
+        x = np.asarray(x, np.float64)
+        wd = blockquant_dequantise(packed, scales, x.shape[1], bits, block).astype(np.float64)
+        if ins is not None:
+            x = x * np.asarray(ins, np.float64)[None, :]
+        return x @ wd.T + np.asarray(bias, np.float64)[None, :]
+
+    qa = proj(q, weights[0]) * float(np.float32(scale))
+    past = 0 if cached_k is None else cached_k.shape[1]
+    if past > 0 and not self_attention:
+        ka, va = np.asarray(cached_k, np.float64).T, np.asarray(cached_v, np.float64).T
+    else:
+        ka, va = proj(k, weights[1]), proj(v, weights[2])
+        if past > 0:
+            ka = np.concatenate([np.asarray(cached_k, np.float64).T, ka])
+            va = np.concatenate([np.asarray(cached_v, np.float64).T, va])
+    hd = embed_dim // num_heads
+    ctx = np.empty((qa.shape[0], embed_dim))
+    for h in range(num_heads):
+        sl = slice(h * hd, (h + 1) * hd)
+        s = qa[:, sl] @ ka[:, sl].T
+        if mask is not None:
+            s = s + np.asarray(mask if mask.ndim == 2 else mask[h], np.float64)
+        s = np.exp(s - s.max(axis=1, keepdims=True))
+        s = s / s.sum(axis=1, keepdims=True)
+        ctx[:, sl] = s @ va[:, sl]
+    return proj(ctx, weights[3]), ka.T, va.T

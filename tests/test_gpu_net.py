@@ -3,6 +3,7 @@ create_extractor, input, extract -- against the oracle-based executor on the sam
 import numpy as np
 import pytest
 
+import cases
 import refnet
 from ncnn_amd import host, modelwriter as mw, zoo
 from oracle import oracle
@@ -135,6 +136,58 @@ def test_gemm_layer_block_quant(bits, block, insc):
     got = _single(lines, blob, {"a": a}, "out")
     val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins)
     assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
+
+
+@pytest.mark.parametrize("spec", cases.MHA_CASES, ids=[str(c[0]) for c in cases.MHA_CASES])
+def test_multiheadattention_layer_block_quant(spec):
+    """MultiHeadAttention with block-quantised weights through load_param / load_model / forward, against the oracle:
+    every arrangement of inputs the layer knows (self / cross attention, shared or per-head mask, cache in and out)."""
+    case = cases.mha_case(*spec)
+    seed, e, heads, qdim, kdim, vdim, src, cur, bits, block, insc, past, self_att, mask = spec
+    term = bits * 100 + int(insc) * 10 + {32: 0, 64: 1, 128: 2}[block]
+    feeds, lines, bottoms = {"q": case["q"]}, ["Input in_q 0 1 q 0=%d 1=%d" % (qdim, src)], ["q"]
+    if not self_att or case["k"] is not case["q"]:
+        feeds["k"] = case["k"]
+        lines.append("Input in_k 0 1 k 0=%d 1=%d" % (kdim, cur))
+        bottoms.append("k")
+        if case["v"] is not case["k"]:
+            feeds["v"] = case["v"]
+            lines.append("Input in_v 0 1 v 0=%d 1=%d" % (vdim, cur))
+            bottoms.append("v")
+    self_layout = len(bottoms) == 1  # the layer itself tells self from cross attention by the number of q/k/v blobs
+    if case["mask"] is not None:
+        feeds["m"] = case["mask"]
+        lines.append("Input in_m 0 1 m")
+        bottoms.append("m")
+    tops = ["out"]
+    if past:
+        feeds["ck"], feeds["cv"] = case["cached_k"], case["cached_v"]
+        lines += ["Input in_ck 0 1 ck", "Input in_cv 0 1 cv"]
+        bottoms += ["ck", "cv"]
+        tops += ["ko", "vo"]
+    lines.append(mw.mha_param("mha", bottoms, tops, e, heads, qdim, kdim, vdim, attn_mask=int(case["mask"] is not None), kv_cache=int(bool(past)),
+                              quantize_term=term))
+    net = host.Net()
+    assert net.register_attention_layer() == 0
+    assert net.load_param_mem(mw.assemble_param(lines)) == 0
+    assert net.load_model_mem(mw.mha_blockquant_weights(case["weights"])) == 0
+    ex = net.create_extractor()
+    for name, value in feeds.items():
+        ex.input(name, value)
+    got = ex.extract("out")
+    want, kw, vw = oracle.mha_blockquant(**dict(case, self_attention=self_layout))
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    if past:
+        assert np.abs(ex.extract("ko") - kw).max() <= 1e-5 * max(1.0, np.abs(kw).max())
+        assert np.abs(ex.extract("vo") - vw).max() <= 1e-5 * max(1.0, np.abs(vw).max())
+
+
+def test_multiheadattention_layer_rejects_other_weight_formats():
+    net = host.Net()
+    assert net.register_attention_layer() == 0
+    lines = ["Input in_q 0 1 q 0=64 1=4", mw.mha_param("mha", ["q"], ["out"], 64, 4, 64, quantize_term=0)]
+    assert net.load_param_mem(mw.assemble_param(lines)) != 0  # fp32 weights: no silent fallback, the load fails
 
 
 def test_innerproduct_layer_2d_rows_and_fp32_weights_quantised_at_load():

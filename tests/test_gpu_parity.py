@@ -311,3 +311,32 @@ def test_blockquant_exact_on_power_of_two_data(rt):
     a = rng.integers(-8, 9, (m, k)).astype(F)
     got = rt.gemm_blockquant(a, q.view(np.uint8), scales, 8, 64)
     assert np.array_equal(got, ((a.astype(np.int64) @ q.astype(np.int64).T) * 0.25).astype(F))
+
+
+# ---- attention core (src/layer/multiheadattention.cpp:776-866) ----------------------------------------------------------
+
+@pytest.mark.parametrize("heads,hd,src,dst,mask", [(4, 16, 9, 9, None), (3, 24, 7, 130, "2d"), (8, 64, 5, 300, "3d"), (2, 32, 1, 1, None), (1, 8, 70, 3, "2d")])
+def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
+    rng = np.random.default_rng(heads * 100 + dst)
+    e = heads * hd
+    q = (rng.normal(0, 1, (src, e)) / np.sqrt(hd)).astype(F)
+    kt = rng.normal(0, 1, (e, dst)).astype(F)
+    vt = rng.normal(0, 1, (e, dst)).astype(F)
+    m = None
+    if mask:
+        shape = (src, dst) if mask == "2d" else (heads, src, dst)
+        m = rng.normal(0, 1, shape).astype(F)
+        drop = rng.random(shape) < 0.3
+        drop[..., 0] = False
+        m[drop] = F(-1e30)
+    got = rt.attention(q, kt, vt, heads, m)
+    want = np.empty((src, e))
+    for h in range(heads):
+        sl = slice(h * hd, (h + 1) * hd)
+        s = q[:, sl].astype(np.float64) @ kt[sl].astype(np.float64)
+        if m is not None:
+            s = s + (m if m.ndim == 2 else m[h]).astype(np.float64)
+        s = np.exp(s - s.max(axis=1, keepdims=True))
+        want[:, sl] = (s / s.sum(axis=1, keepdims=True)) @ vt[sl].astype(np.float64).T
+    # fp32 sums over head_dim and dst terms of O(1) values, device expf
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())

@@ -9,6 +9,7 @@ import itertools
 import numpy as np
 import pytest
 
+import cases
 import npref
 from oracle import oracle
 
@@ -368,3 +369,52 @@ def test_float_pipe_formulation_of_float2int8_equals_the_oracle():
         got = np.where(np.abs(v) < F(2147483648.0), r, F(-127))
     want = oracle.float2int8(v).astype(F)
     assert np.array_equal(got, want)
+
+
+# ---- attention with block-quantised weights (src/layer/multiheadattention.cpp:561-912) ---------------------------------
+
+def _mha_tolerance(case):
+    """|error| allowed per output: fp32 sequential sums over <= max(K, dst) terms of O(1) values."""
+    return 2e-4
+
+
+@pytest.mark.parametrize("spec", cases.MHA_CASES, ids=[str(c[0]) for c in cases.MHA_CASES])
+def test_mha_blockquant_matches_float64_attention(spec):
+    case = cases.mha_case(*spec)
+    out, ko, vo = oracle.mha_blockquant(**case)
+    want, kw, vw = npref.mha_f64(**case)
+    assert out.shape == want.shape and ko.shape == kw.shape
+    assert np.abs(out - want).max() <= _mha_tolerance(case) * max(1.0, np.abs(want).max())
+    assert np.abs(ko - kw).max() <= 1e-4 * max(1.0, np.abs(kw).max())
+    assert np.abs(vo - vw).max() <= 1e-4 * max(1.0, np.abs(vw).max())
+
+
+def test_mha_blockquant_matches_torch_multi_head_attention():
+    """The layer follows torch.nn.MultiheadAttention (multiheadattention.cpp:234): with the dequantised weights as
+    its projection matrices torch's own routine must give the same numbers."""
+    torch = pytest.importorskip("torch")
+    case = cases.mha_case(21, 64, 4, 64, 48, 40, 6, 8, 8, 32, False, 0, True, "2d")
+    out, _, _ = oracle.mha_blockquant(**case)
+    wq, wk, wv, wo = [npref.blockquant_dequantise(w[0], w[1], k, 8, 32) for w, k in zip(case["weights"], (64, 48, 40, 64))]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32))
+    bias = np.concatenate([case["weights"][i][3] for i in range(3)])
+    got, _ = torch.nn.functional.multi_head_attention_forward(
+        t(case["q"])[:, None], t(case["k"])[:, None], t(case["v"])[:, None], 64, 4, None, t(bias), None, None, False, 0.0, t(wo), t(case["weights"][3][3]),
+        training=False, need_weights=False, attn_mask=t(case["mask"]), use_separate_proj_weight=True, q_proj_weight=t(wq), k_proj_weight=t(wk),
+        v_proj_weight=t(wv))
+    assert np.abs(got[:, 0].numpy() - out).max() <= 2e-5 * max(1.0, np.abs(out).max())
+
+
+def test_mha_blockquant_cache_identity():
+    """Causal self-attention over n tokens == n one-token calls that hand their keys / values back as the cache;
+    masked-out keys contribute exact zeros, so the two evaluations agree bit for bit."""
+    n, e = 6, 64
+    case = cases.mha_case(31, e, 4, e, e, e, n, n, 8, 64, False, 0, True, None)
+    causal = np.where(np.arange(n)[None, :] <= np.arange(n)[:, None], 0.0, -1e30).astype(F)
+    full, kfull, vfull = oracle.mha_blockquant(**dict(case, mask=causal))
+    ck = cv = None
+    for i in range(n):
+        x = case["q"][i:i + 1]
+        step, ck, cv = oracle.mha_blockquant(**dict(case, q=x, k=x, v=x, cached_k=ck, cached_v=cv))
+        assert np.array_equal(step[0], full[i]), i
+    assert np.array_equal(ck, kfull) and np.array_equal(cv, vfull)
