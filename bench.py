@@ -221,6 +221,66 @@ def bench_blockquant(args, n, k, m):
     }
 
 
+def bench_mha(args, embed, heads, src, past):
+    """Self-attention layer with 8-bit block-quantised weights (blocks of 64) on device-resident operands: the launches of
+    MultiHeadAttention_hip::forward without its host copies.  src new tokens are appended to a cache of `past` tokens."""
+    import ncnn_amd
+    from ncnn_amd.hip import check, lib as load
+    from oracle import oracle
+    lib = load()
+    rt = ncnn_amd.Runtime(0)
+    st = rt.stream
+    rng = np.random.default_rng(0)
+    dst = past + src
+    ws = []
+    for _ in range(4):
+        w = rng.normal(0, 1.0 / np.sqrt(embed), (embed, embed)).astype(np.float32)
+        packed, scales = oracle.blockquant_pack(w, 8, 64)
+        ws.append((rt.up(packed), rt.up(scales), rt.up(rng.uniform(-0.1, 0.1, embed).astype(np.float32)), packed.nbytes + scales.nbytes))
+    d_x = rt.up(rng.normal(0, 1, (src, embed)).astype(np.float32))
+    d_kt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
+    d_vt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
+    d_qa, d_aff, d_ctx, d_out = [ncnn_amd.DeviceBuffer.empty((src, embed), np.float32) for _ in range(4)]
+    scale = float(1.0 / np.sqrt(embed // heads))
+    wsb = C.c_size_t()
+    check(lib.ncnnhip_attention_workspace_bytes(heads, embed // heads, src, dst, C.byref(wsb)))
+    d_ws = ncnn_amd.DeviceBuffer.empty((max(wsb.value, 4),), np.uint8)
+
+    def step():
+        check(lib.ncnnhip_gemm_blockquant(d_x.ptr, embed, src, embed, embed, ws[0][0].ptr, 8, 64, ws[0][1].ptr, None, ws[0][2].ptr, 4, scale, 1.0, d_qa.ptr, embed, st))
+        for t, cache in ((1, d_kt), (2, d_vt)):
+            check(lib.ncnnhip_gemm_blockquant(d_x.ptr, embed, src, embed, embed, ws[t][0].ptr, 8, 64, ws[t][1].ptr, None, ws[t][2].ptr, 4, 1.0, 1.0, d_aff.ptr, embed, st))
+            check(lib.ncnnhip_transpose_f32(d_aff.ptr, embed, src, embed, C.c_void_p(cache.ptr.value + past * 4), dst, st))
+        check(lib.ncnnhip_attention_f32(d_qa.ptr, d_kt.ptr, d_vt.ptr, dst, None, 0, heads, embed // heads, src, dst, d_ctx.ptr, d_ws.ptr, wsb.value, st))
+        check(lib.ncnnhip_gemm_blockquant(d_ctx.ptr, embed, src, embed, embed, ws[3][0].ptr, 8, 64, ws[3][1].ptr, None, ws[3][2].ptr, 4, 1.0, 1.0, d_out.ptr, embed, st))
+
+    for _ in range(args.warmup):
+        step()
+    rt.sync()
+    evs = _events(lib, check, 2)
+    t0 = time.perf_counter()
+    check(lib.ncnnhip_event_record(evs[0], st))
+    for _ in range(args.steps):
+        step()
+    check(lib.ncnnhip_event_record(evs[1], st))
+    check(lib.ncnnhip_device_synchronize())
+    wall = time.perf_counter() - t0
+    k_ms = _elapsed(lib, check, evs[0], evs[1]) / args.steps
+    # bytes that must move: the four weight matrices with their scales, the keys and values of the cache, activations in and out
+    algo = sum(w[3] for w in ws) + 2 * embed * dst * 4 + 2 * src * embed * 4
+    ops = 2.0 * src * embed * embed * 4 + 4.0 * src * dst * embed
+    ms_per_step = wall * 1e3 / args.steps
+    achieved = algo / (k_ms * 1e-3) / 1e9
+    return {
+        "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "self-attention layer, embed %d, %d heads, %d new tokens on a cache of %d, 8-bit block-quantised weights (blocks of 64)"
+                               % (embed, heads, src, past), "launches_per_step": 7, "device_ms_per_step": k_ms, "gflop": ops / 1e9},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "whole layer (3 projections, 2 cache appends, attention core, output projection)", "bytes_per_launch": algo},
+    }
+
+
 def cpu_baseline_conv(c, h, w, cout, k, pad, budget_s=10.0):
     """Scalar oracle (ncnn's naive Convolution::forward_int8 restated, OpenMP over output channels) on whole layers."""
     from oracle import oracle
@@ -512,6 +572,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
                     help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
+                         "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
     ap.add_argument("--graph", type=int, default=0,
                     help="net workloads: 0 = one Extractor per pass, layer by layer on a stream (faster on this ROCm: a replayed graph costs more per kernel node "
@@ -530,6 +591,10 @@ def main():
     elif args.workload.startswith("blockquant:"):
         n, k, m = (int(v) for v in args.workload.split(":")[1].split("x"))
         line = bench_blockquant(args, n, k, m)
+    elif args.workload.startswith("mha:"):
+        dims, src, past = args.workload.split(":")[1:]
+        embed, heads = [int(v) for v in dims.split("x")]
+        line = bench_mha(args, embed, heads, int(src), int(past))
     elif args.workload.startswith("conv:"):
         line = bench_conv(args, args.workload[5:])
     elif args.workload.startswith("net:"):

@@ -291,10 +291,13 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
  * per head, scores = q k^T (+ mask), softmax over the keys, times v.  q (already scaled) and out are
  * [seq][num_heads*head_dim]; kt / vt are [num_heads*head_dim][dst_seqlen] with row stride kv_stride, the layout of
  * the layer's cache blobs; mask is additive, [src][dst] (mask_heads 1) or [num_heads][src][dst], or NULL.
- * head_dim + dst_seqlen <= 4096. */
+ * Head dimensions 32/64/96/128 run on the fp32 matrix cores with any dst_seqlen; others need head_dim + dst_seqlen <= 4096.
+ * With few queries and many keys (decoding against a cache) the keys are split over workgroups if the caller passes
+ * the scratch ncnnhip_attention_workspace_bytes asks for (may be 0 / NULL: then one workgroup per head and 32 queries). */
+int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqlen, int dst_seqlen, size_t* workspace_bytes);
 int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
                           int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev,
-                          void* stream);
+                          void* workspace_dev, size_t workspace_bytes, void* stream);
 
 #pragma GCC visibility pop
 

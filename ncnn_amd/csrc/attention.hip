@@ -114,22 +114,274 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float* __restr
     }
 }
 
+// ---- the same on the fp32 matrix cores, for head dimensions 32 / 64 / 96 / 128 ------------------------------------
+// One workgroup = 32 query rows of one head; its 4 wavefronts take key tiles (32 keys) in turn and each keeps a
+// running softmax (maximum m, sum l, unnormalised output) for its share; the shares are merged at the end.
+// Everything is computed transposed, so that both MFMA operands come straight from where they lie:
+//   S^T = K Q^T : A = k[channel][key] read coalesced along the keys, B = q values held in registers.  The result has
+//                 keys down the registers and the 32 queries across the lanes: a query's softmax is per-lane arithmetic
+//                 plus one exchange with lane^32.
+//   O^T = V P^T : B = exp(S^T - m) is used from the accumulator registers as they are: MFMA step kk of half hh is given
+//                 key 8*(kk/4) + 4*hh + kk%4, the key that register kk of that lane holds; A = v[channel][key] with the
+//                 same key order, four 16-byte loads per lane and 32 channels.
+// Scores and products are fp32 throughout; the order of the additions (and the running rescale by exp(m_old - m_new))
+// differs from the reference's two-pass softmax: compared with an fp32 tolerance.
+typedef float v16f_at __attribute__((ext_vector_type(16)));
+typedef float v4f_at __attribute__((ext_vector_type(4)));
+
+template<int HD>
+__global__ __launch_bounds__(256) void attention_f32_mfma_kernel(const float* __restrict__ q, const float* __restrict__ kt, const float* __restrict__ vt,
+                                                                 const float* __restrict__ mask, int mask_heads, int embed_dim, int src, int dst,
+                                                                 size_t kv_stride, float* __restrict__ out, int v_vec_ok, int keys_per_split,
+                                                                 float* __restrict__ partial)
+{
+    // keys_per_split > 0: blockIdx.z takes keys [z*keys_per_split, ...) and leaves (m, l, unnormalised o) in `partial`
+    // for attention_merge_kernel; 0: the workgroup sees every key and writes the result
+    constexpr int CB = HD / 32;
+    constexpr int LD = 33;
+    __shared__ float o_s[HD * LD];
+    __shared__ float m_s[4][32], l_s[4][32];
+    const int h = blockIdx.y, i0 = blockIdx.x * 32;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hh = lane >> 5;
+    const int qi = i0 + l32 < src ? i0 + l32 : src - 1; // lanes past the last query repeat it; nothing of theirs is stored
+
+    float qreg[HD / 2];
+#pragma unroll
+    for (int kk = 0; kk < HD / 2; kk++) qreg[kk] = q[(size_t)qi * embed_dim + h * HD + 2 * kk + hh];
+
+    v16f_at o[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[cb][r] = 0.f;
+    float m = -FLT_MAX, l = 0.f;
+
+    const float* kh = kt + (size_t)h * HD * kv_stride;
+    const float* vh = vt + (size_t)h * HD * kv_stride;
+    const float* mrow = mask ? mask + ((size_t)(mask_heads > 1 ? h : 0) * src + qi) * dst : nullptr;
+
+    const int key_begin = keys_per_split > 0 ? (int)blockIdx.z * keys_per_split : 0;
+    const int key_end = keys_per_split > 0 && key_begin + keys_per_split < dst ? key_begin + keys_per_split : dst; // a multiple of 32, or dst
+    for (int j0 = key_begin + wave * 32; j0 < key_end; j0 += 128)
+    {
+        const bool full = j0 + 32 <= dst;
+        const int kj = j0 + l32 < dst ? j0 + l32 : dst - 1;
+        v16f_at s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < HD / 2; kk++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kh[(size_t)(2 * kk + hh) * kv_stride + kj], qreg[kk], s, 0, 0, 0);
+        // register r of this lane: key j0 + 8*(r/4) + 4*hh + r%4 for query l32
+        float mx = -FLT_MAX;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int key = j0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+            if (mrow && key < dst) s[r] = add_rn(s[r], mrow[key]);
+            if (!full && key >= dst) s[r] = -INFINITY;
+            mx = fmaxf(mx, s[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx);
+        const float corr = expf(m - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            s[r] = expf(s[r] - m_new);
+            psum += s[r];
+        }
+        psum += __shfl_xor(psum, 32);
+        l = l * corr + psum;
+        m = m_new;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+        {
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[cb][r] *= corr;
+            const float* vr = vh + (size_t)(cb * 32 + l32) * kv_stride;
+            float vv[16];
+            if (full && v_vec_ok)
+            {
+#pragma unroll
+                for (int a = 0; a < 4; a++)
+                {
+                    const v4f_at t4 = *reinterpret_cast<const v4f_at*>(vr + j0 + 8 * a + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) vv[4 * a + e] = t4[e];
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int kk = 0; kk < 16; kk++)
+                {
+                    const int key = j0 + 8 * (kk >> 2) + 4 * hh + (kk & 3);
+                    vv[kk] = vr[key < dst ? key : dst - 1]; // its probability is 0
+                }
+            }
+#pragma unroll
+            for (int kk = 0; kk < 16; kk++) o[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[kk], s[kk], o[cb], 0, 0, 0);
+        }
+    }
+
+    // ---- merge the four shares: common maximum, then each wavefront adds its rescaled part in turn
+    if (hh == 0)
+    {
+        m_s[wave][l32] = m;
+        l_s[wave][l32] = l;
+    }
+    __syncthreads();
+    const float mall = fmaxf(fmaxf(m_s[0][l32], m_s[1][l32]), fmaxf(m_s[2][l32], m_s[3][l32]));
+    const float f = expf(m - mall); // a wavefront that saw no key has m = -FLT_MAX, l = 0, o = 0
+    for (int w = 0; w < 4; w++)
+    {
+        if (wave == w)
+        {
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                {
+                    const int ch = cb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                    const float v = o[cb][r] * f;
+                    o_s[ch * LD + l32] = w == 0 ? v : o_s[ch * LD + l32] + v;
+                }
+        }
+        __syncthreads();
+    }
+    if (keys_per_split > 0)
+    {
+        // [query block][head][split] records of 32 maxima, 32 sums, 32 x HD outputs (query-major; only real queries are written)
+        float* rec = partial + (((size_t)blockIdx.x * gridDim.y + h) * gridDim.z + blockIdx.z) * (size_t)(64 + HD * 32);
+        const int nq = src - i0 < 32 ? src - i0 : 32;
+        if (tid < 32)
+        {
+            const float ma = fmaxf(fmaxf(m_s[0][tid], m_s[1][tid]), fmaxf(m_s[2][tid], m_s[3][tid]));
+            float lt = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) lt += l_s[w][tid] * expf(m_s[w][tid] - ma);
+            rec[tid] = ma;
+            rec[32 + tid] = lt;
+        }
+        for (int idx = tid; idx < nq * HD; idx += 256) rec[64 + idx] = o_s[(idx % HD) * LD + idx / HD];
+        return;
+    }
+    for (int idx = tid; idx < 32 * HD; idx += 256)
+    {
+        const int qq = idx / HD, ch = idx - qq * HD;
+        if (i0 + qq < src)
+        {
+            float lt = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) lt += l_s[w][qq] * expf(m_s[w][qq] - fmaxf(fmaxf(m_s[0][qq], m_s[1][qq]), fmaxf(m_s[2][qq], m_s[3][qq])));
+            out[(size_t)(i0 + qq) * embed_dim + h * HD + ch] = div_rn(o_s[ch * LD + qq], lt);
+        }
+    }
+}
+
+// merges the records of the key splits: one workgroup per (query block, head)
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ partial, int splits, int head_dim, int embed_dim, int src,
+                                                              float* __restrict__ out)
+{
+    const int h = blockIdx.y, i0 = blockIdx.x * 32;
+    const size_t rec_size = (size_t)(64 + head_dim * 32);
+    const float* rec0 = partial + ((size_t)blockIdx.x * gridDim.y + h) * splits * rec_size;
+    const int nq = src - i0 < 32 ? src - i0 : 32;
+    for (int idx = threadIdx.x; idx < nq * head_dim; idx += 256)
+    {
+        const int qq = idx / head_dim, ch = idx - qq * head_dim;
+        float ma = -FLT_MAX;
+        for (int z = 0; z < splits; z++) ma = fmaxf(ma, rec0[z * rec_size + qq]);
+        float lt = 0.f, ot = 0.f;
+        for (int z = 0; z < splits; z++)
+        {
+            const float f = expf(rec0[z * rec_size + qq] - ma);
+            lt += rec0[z * rec_size + 32 + qq] * f;
+            ot += rec0[z * rec_size + 64 + idx] * f;
+        }
+        out[(size_t)(i0 + qq) * embed_dim + h * head_dim + ch] = div_rn(ot, lt);
+    }
+}
+
+// how many ways to split the keys: enough workgroups for the chip, at least 128 keys (one tile per wavefront) each
+static int attention_key_splits(int num_heads, int src, int dst)
+{
+    const long long groups = (long long)((src + 31) / 32) * num_heads;
+    if (groups >= 256 || dst < 256) return 1;
+    long long want = (512 + groups - 1) / groups;
+    const long long most = dst / 128;
+    if (want > most) want = most;
+    if (want > 64) want = 64;
+    return want < 2 ? 1 : (int)want;
+}
+
 } // namespace ncnnhip
 
 using namespace ncnnhip;
 
 extern "C" {
 
+int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqlen, int dst_seqlen, size_t* workspace_bytes)
+{
+    NCNNHIP_REQUIRE(num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && dst_seqlen >= 1 && workspace_bytes, "ncnnhip_attention_workspace_bytes: bad argument");
+    *workspace_bytes = 0;
+    if (head_dim % 32 == 0 && head_dim <= 128)
+    {
+        const int splits = attention_key_splits(num_heads, src_seqlen, dst_seqlen);
+        if (splits > 1) *workspace_bytes = (size_t)((src_seqlen + 31) / 32) * num_heads * splits * (size_t)(64 + head_dim * 32) * sizeof(float);
+    }
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev, int mask_heads,
-                          int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* stream)
+                          int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes,
+                          void* stream)
 {
     NCNNHIP_REQUIRE(q_dev && kt_dev && vt_dev && out_dev, "ncnnhip_attention_f32: null pointer");
     NCNNHIP_REQUIRE(num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && dst_seqlen >= 1, "ncnnhip_attention_f32: bad shape");
     NCNNHIP_REQUIRE(num_heads <= 65535, "ncnnhip_attention_f32: more than 65535 heads");
     NCNNHIP_REQUIRE(kv_stride >= (size_t)dst_seqlen, "ncnnhip_attention_f32: key/value row stride below dst_seqlen");
     NCNNHIP_REQUIRE(!mask_dev || mask_heads == 1 || mask_heads == num_heads, "ncnnhip_attention_f32: the mask is shared (1) or one per head");
+    if (head_dim % 32 == 0 && head_dim <= 128)
+    {
+        // 16-byte loads of the values need the rows and the start aligned
+        const int v_vec_ok = (kv_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(vt_dev) & 15) == 0) ? 1 : 0;
+        // few queries (decoding): split the keys over workgroups when the caller brought the scratch for it
+        int splits = attention_key_splits(num_heads, src_seqlen, dst_seqlen);
+        size_t need = 0;
+        if (splits > 1) need = (size_t)((src_seqlen + 31) / 32) * num_heads * splits * (size_t)(64 + head_dim * 32) * sizeof(float);
+        if (splits > 1 && (!workspace_dev || workspace_bytes < need)) splits = 1;
+        int keys_per_split = 0;
+        if (splits > 1)
+        {
+            keys_per_split = ((dst_seqlen + splits - 1) / splits + 31) / 32 * 32;
+            splits = (dst_seqlen + keys_per_split - 1) / keys_per_split;
+        }
+        dim3 grid((unsigned)((src_seqlen + 31) / 32), (unsigned)num_heads, (unsigned)(splits > 1 ? splits : 1));
+        if (splits <= 1) keys_per_split = 0;
+        float* partial = (float*)workspace_dev;
+        const int e = num_heads * head_dim, mh = mask_dev ? mask_heads : 0;
+        hipStream_t st = as_stream(stream);
+#define LAUNCH_ATT(HD_) \
+    hipLaunchKernelGGL(attention_f32_mfma_kernel<HD_>, grid, dim3(256), 0, st, q_dev, kt_dev, vt_dev, mask_dev, mh, e, src_seqlen, dst_seqlen, kv_stride, out_dev, \
+                       v_vec_ok, keys_per_split, partial)
+        if (head_dim == 32)
+            LAUNCH_ATT(32);
+        else if (head_dim == 64)
+            LAUNCH_ATT(64);
+        else if (head_dim == 96)
+            LAUNCH_ATT(96);
+        else
+            LAUNCH_ATT(128);
+#undef LAUNCH_ATT
+        if (keys_per_split > 0)
+            hipLaunchKernelGGL(attention_merge_kernel, dim3(grid.x, grid.y), dim3(256), 0, st, partial, splits, head_dim, e, src_seqlen, out_dev);
+        return launch_status("attention_f32_mfma_kernel");
+    }
     const size_t lds = (size_t)ATT_TQ * ((size_t)head_dim + (size_t)dst_seqlen) * sizeof(float);
-    NCNNHIP_REQUIRE(lds <= 65536, "ncnnhip_attention_f32: head_dim + dst_seqlen = %d exceeds the 4096 this kernel keeps in LDS", head_dim + dst_seqlen);
+    NCNNHIP_REQUIRE(lds <= 65536, "ncnnhip_attention_f32: head_dim %d is not 32/64/96/128 and head_dim + dst_seqlen = %d exceeds the 4096 the general kernel keeps in LDS",
+                    head_dim, head_dim + dst_seqlen);
     dim3 grid((unsigned)((src_seqlen + ATT_TQ - 1) / ATT_TQ), (unsigned)num_heads);
     hipLaunchKernelGGL(attention_f32_kernel, grid, dim3(256), lds, as_stream(stream), q_dev, kt_dev, vt_dev, mask_dev, mask_dev ? mask_heads : 0, head_dim,
                        num_heads * head_dim, src_seqlen, dst_seqlen, kv_stride, out_dev);

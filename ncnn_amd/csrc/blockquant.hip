@@ -287,6 +287,103 @@ static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K,
     return launch_status("blockquant8_stream_kernel");
 }
 
+// ---- 8-bit weights, many activation rows: fp32 matrix cores -----------------------------------
+// From 32 rows up streaming the weights once per 4 rows is the wrong shape; this kernel tiles 64 activation rows by 64
+// weight rows per workgroup (4 wavefronts, 32x32 each) and multiplies on v_mfma_f32_32x32x2_f32.  The B operand is the
+// weight as the reference forms it, (float)q * (1/scale), so every product is the reference's fp32 product; only the
+// order of the fp32 additions differs.  K in tiles of 32 through two LDS buffers (row stride 33 floats: a column of 32
+// rows hits 32 banks); the next tile's global loads are issued before the current tile's MFMAs.
+typedef float v16f_bq __attribute__((ext_vector_type(16)));
+typedef float v4f_bq __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void blockquant8_f32_mfma_kernel(const float* __restrict__ a, size_t a_stride, int M, int N, int K,
+                                                                   const int8_t* __restrict__ b, int block_shift, int nblk, const float* __restrict__ scales,
+                                                                   const float* __restrict__ in_scales, const float* __restrict__ c, int bt, float alpha,
+                                                                   float beta, float* __restrict__ out, size_t out_stride)
+{
+    constexpr int LD = 33;
+    __shared__ float sa[2][64 * LD];
+    __shared__ float sb[2][64 * LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
+
+    // loader role: row tid/4 of the tile, 8 consecutive k starting at (tid%4)*8
+    const int lr = tid >> 2, lk = (tid & 3) * 8;
+    const int arow = row0 + lr < M ? row0 + lr : M - 1; // rows past the end repeat the last one; their results are not stored
+    const int brow = col0 + lr < N ? col0 + lr : N - 1;
+    const float* ap = a + (size_t)arow * a_stride + lk;
+    const int8_t* bp = b + (size_t)brow * K + lk;
+    const float* sp = scales + (size_t)brow * nblk;
+
+    v4f_bq a0, a1;
+    uint2 bq;
+    float descale;
+    auto fetch = [&](int k0) {
+        a0 = *reinterpret_cast<const v4f_bq*>(ap + k0);
+        a1 = *reinterpret_cast<const v4f_bq*>(ap + k0 + 4);
+        bq = *reinterpret_cast<const uint2*>(bp + k0);
+        descale = div_rn(1.f, sp[(k0 + lk) >> block_shift]);
+        if (in_scales)
+        {
+            const v4f_bq s0 = *reinterpret_cast<const v4f_bq*>(in_scales + k0 + lk), s1 = *reinterpret_cast<const v4f_bq*>(in_scales + k0 + lk + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+            {
+                a0[e] = mul_rn(a0[e], s0[e]);
+                a1[e] = mul_rn(a1[e], s1[e]);
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+        float* pa = &sa[buf][lr * LD + lk];
+        float* pb = &sb[buf][lr * LD + lk];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            pa[e] = a0[e];
+            pa[4 + e] = a1[e];
+            pb[e] = mul_rn((float)(int)(int8_t)(bq.x >> (8 * e)), descale);
+            pb[4 + e] = mul_rn((float)(int)(int8_t)(bq.y >> (8 * e)), descale);
+        }
+    };
+
+    v16f_bq acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+    const int ntiles = K / 32;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    const int l32 = lane & 31, lhi = lane >> 5;
+    for (int t = 0; t < ntiles; t++)
+    {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) fetch((t + 1) * 32);
+        const float* pa = &sa[buf][(wm * 32 + l32) * LD + lhi];
+        const float* pb = &sb[buf][(wn * 32 + l32) * LD + lhi];
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[2 * kk], pb[2 * kk], acc, 0, 0, 0);
+        if (t + 1 < ntiles) stage(buf ^ 1); // the other buffer: its readers finished before the barrier that ended tile t-1
+        __syncthreads();
+    }
+
+    // accumulator register r of lane l: activation row 8*(r/4) + 4*(l/32) + r%4, weight row l%32
+    const int j = col0 + wn * 32 + l32;
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+    {
+        const int i = row0 + wm * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        if (i < M && j < N)
+        {
+            float v = acc[r];
+            if (bt >= 0) v = add_rn(mul_rn(load_c(c, bt, i, j, N), beta), v);
+            out[(size_t)i * out_stride + j] = mul_rn(v, alpha);
+        }
+    }
+}
+
 // ---- any bits / block / alignment --------------------------------------------------------
 __device__ __forceinline__ int unpack_field(const uint8_t* row, int k, int bits, int packed_k_bytes)
 {
@@ -527,6 +624,15 @@ int ncnnhip_gemm_blockquant(const float* a_dev, size_t a_stride, int M, int N, i
     NCNNHIP_REQUIRE(a_stride >= (size_t)K && out_stride >= (size_t)N, "ncnnhip_gemm_blockquant: stride too small");
     const int nblk = (K + block - 1) / block;
     dim3 grid(ceil_div(N, 4));
+    if (bits == 8 && M >= 32 && K % 32 == 0 && a_stride % 4 == 0 && al16(a_dev) && al16(b_dev) && (!in_scales_dev || al16(in_scales_dev)))
+    {
+        const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
+        dim3 tiles(ceil_div(N, 64), ceil_div(M, 64));
+        NCNNHIP_REQUIRE(tiles.y <= 65535, "ncnnhip_gemm_blockquant: more than 65535*64 activation rows");
+        hipLaunchKernelGGL(blockquant8_f32_mfma_kernel, tiles, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev),
+                           shift, nblk, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride);
+        return launch_status("blockquant8_f32_mfma_kernel");
+    }
     if (bits == 8 && K % 16 == 0 && al16(b_dev))
     {
         return launch_blockquant8<float>(a_dev, a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev), block, scales_dev, in_scales_dev,

@@ -52,7 +52,9 @@ _SIGNATURES = {
     "ncnnhip_stream_synchronize": [C.c_void_p],
     "ncnnhip_device_synchronize": [],
     "ncnnhip_copy2d": [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p],
-    "ncnnhip_attention_f32": [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_attention_workspace_bytes": [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
+    "ncnnhip_attention_f32": [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t,
+                              C.c_void_p],
     "ncnnhip_stream_begin_capture": [C.c_void_p],
     "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
     "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
@@ -373,7 +375,7 @@ class Runtime:
         check(lib().ncnnhip_maxpool_nhwc_int8(C.byref(d), src.ptr, out.ptr, self.stream))
         return self.from_channels_last(out, n, c, oh, ow)
 
-    def attention(self, q, kt, vt, num_heads, mask=None):
+    def attention(self, q, kt, vt, num_heads, mask=None, use_workspace=True):
         """q [src][embed] (scaled), kt / vt [embed][dst], mask [src][dst] or [heads][src][dst] -> [src][embed]."""
         q, kt, vt = [np.ascontiguousarray(a, np.float32) for a in (q, kt, vt)]
         src, embed = q.shape
@@ -382,7 +384,11 @@ class Runtime:
         dm = None if mask is None else self.up(np.ascontiguousarray(mask, np.float32))
         mask_heads = 0 if mask is None else (1 if mask.ndim == 2 else mask.shape[0])
         out = DeviceBuffer.empty((src, embed), np.float32)
-        check(lib().ncnnhip_attention_f32(dq.ptr, dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads, src, dst, out.ptr, self.stream))
+        wsb = C.c_size_t()
+        check(lib().ncnnhip_attention_workspace_bytes(num_heads, embed // num_heads, src, dst, C.byref(wsb)))
+        ws = DeviceBuffer.empty((max(wsb.value, 4),), np.uint8) if use_workspace else None
+        check(lib().ncnnhip_attention_f32(dq.ptr, dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads, src, dst, out.ptr,
+                                          _ptr(ws), wsb.value if use_workspace else 0, self.stream))
         return out.to_numpy(self.stream)
 
     def softmax(self, x):

@@ -298,7 +298,12 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
         if (rc != 0) return to_ncnn_status(rc, "upload mask");
         d_mask = m;
     }
-    rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, st);
+    size_t att_ws_bytes = 0;
+    rc = ncnnhip_attention_workspace_bytes(num_heads, head_dim, src, dst, &att_ws_bytes);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
+    void* att_ws = att_ws_bytes ? leases.get(att_ws_bytes) : 0;
+    if (att_ws_bytes && !att_ws) return -100;
+    rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
     rc = ncnnhip_gemm_blockquant(d_ctx, E, src, qdim, embed_dim, (const uint8_t*)dev[3][0], bits, block, (const float*)dev[3][1], (const float*)dev[3][2],
                                  (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);

@@ -262,7 +262,10 @@ def _bq_check(got, a, packed, scales, bits, block, ins=None, c=None, bt=-1, alph
 
 @pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
     (8, 64, 1, 24, 256, -1, False), (8, 64, 4, 16, 200, 4, False), (4, 32, 3, 9, 100, 3, True), (6, 128, 2, 7, 300, 1, True),
-    (8, 32, 16, 8, 64, 0, False), (4, 64, 1, 5, 65, 2, False), (8, 128, 5, 33, 1024, 4, True), (8, 64, 3, 10, 4096 + 16, -1, False)])
+    (8, 32, 16, 8, 64, 0, False), (4, 64, 1, 5, 65, 2, False), (8, 128, 5, 33, 1024, 4, True), (8, 64, 3, 10, 4096 + 16, -1, False),
+    # 32 rows and more: the fp32 matrix-core kernel (ragged tiles in both directions, every C broadcast, input scales)
+    (8, 64, 32, 64, 64, -1, False), (8, 64, 70, 100, 256, 4, True), (8, 32, 129, 65, 96, 3, False), (8, 128, 64, 31, 1024, 1, True),
+    (8, 64, 200, 130, 2048, 0, False), (8, 64, 33, 8, 4096 + 32, 2, False)])
 def test_blockquant_small(rt, bits, block, m, n, k, bt, in_sc):
     _say("blockquant", bits, block, m, n, k, bt, in_sc)
     rng = np.random.default_rng(bits + block + m + n + k)
@@ -315,7 +318,9 @@ def test_blockquant_exact_on_power_of_two_data(rt):
 
 # ---- attention core (src/layer/multiheadattention.cpp:776-866) ----------------------------------------------------------
 
-@pytest.mark.parametrize("heads,hd,src,dst,mask", [(4, 16, 9, 9, None), (3, 24, 7, 130, "2d"), (8, 64, 5, 300, "3d"), (2, 32, 1, 1, None), (1, 8, 70, 3, "2d")])
+@pytest.mark.parametrize("heads,hd,src,dst,mask", [(4, 16, 9, 9, None), (3, 24, 7, 130, "2d"), (8, 64, 5, 300, "3d"), (2, 32, 1, 1, None), (1, 8, 70, 3, "2d"),
+                                                    # head dimensions of the matrix-core kernel: ragged query blocks and key tiles, one to many tiles per wavefront
+                                                    (2, 96, 40, 70, "2d"), (1, 128, 33, 257, None), (4, 64, 100, 129, "3d"), (2, 64, 64, 1024, None), (3, 32, 1, 515, "2d"), (16, 64, 1, 1500, None), (2, 128, 33, 4100, "3d")])
 def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
     rng = np.random.default_rng(heads * 100 + dst)
     e = heads * hd
@@ -330,6 +335,8 @@ def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
         drop[..., 0] = False
         m[drop] = F(-1e30)
     got = rt.attention(q, kt, vt, heads, m)
+    assert np.array_equal(got.shape, (src, e))
+    plain = rt.attention(q, kt, vt, heads, m, use_workspace=False)  # without the scratch the keys are not split over workgroups
     want = np.empty((src, e))
     for h in range(heads):
         sl = slice(h * hd, (h + 1) * hd)
@@ -340,3 +347,4 @@ def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
         want[:, sl] = (s / s.sum(axis=1, keepdims=True)) @ vt[sl].astype(np.float64).T
     # fp32 sums over head_dim and dst terms of O(1) values, device expf
     assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    assert np.abs(plain - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
