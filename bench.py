@@ -162,7 +162,7 @@ def bench_gemm(args, size):
     return line
 
 
-def bench_blockquant(args, n, k, m):
+def bench_blockquant(args, n, k, m, bits=8, block=64):
     """LLM-decode block-quant Gemm: weights int8 in blocks of 64 with one fp32 scale per block, streamed from a
     rotating set of weight copies larger than the 256 MB last-level cache so that the rate is an HBM rate."""
     import ncnn_amd
@@ -170,11 +170,15 @@ def bench_blockquant(args, n, k, m):
     from ncnn_amd import synth
     lib = load()
     rt = ncnn_amd.Runtime(0)
-    a, packed, scales = synth.blockquant8_operands(n + k + m, m, n, k)
+    a, packed, scales = synth.blockquant_operands(n + k + m, m, n, k, bits, block)
     wbytes = packed.nbytes + scales.nbytes
     copies = int(np.ceil(512e6 / wbytes)) + 1
     half = args.act == "fp16"
-    if half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
+    lowbit = bits != 8 or block != 64  # these stream the .bin layout as it is (no matrix-core repack)
+    if lowbit:
+        d_w = [rt.up(packed) for _ in range(copies)]
+        d_s = [rt.up(scales) for _ in range(copies)]
+    elif half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
         pw, pd = rt.blockquant_pack(packed, scales, 64)
         wbytes = n * k + scales.nbytes  # algorithmic bytes: the int8 weights and one fp32 scale per block
         d_w = [rt.up(pw) for _ in range(copies)]
@@ -188,7 +192,11 @@ def bench_blockquant(args, n, k, m):
 
     def launch(i):
         j = i % copies
-        if half:
+        if lowbit and half:
+            check(lib.ncnnhip_gemm_blockquant_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, d_out.ptr, n, st))
+        elif lowbit:
+            check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
+        elif half:
             check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, None, -1, 1.0, 1.0, d_out.ptr, n, st))
         else:
             check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, 8, 64, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
@@ -213,11 +221,11 @@ def bench_blockquant(args, n, k, m):
     return {
         "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, int8 weights in blocks of 64, fp32 block scales, %s activations" % (m, n, k, args.act),
+        "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, %d-bit weights in blocks of %d, fp32 block scales, %s activations" % (m, n, k, bits, block, args.act),
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if half else None,
-                     "kernel": "blockquant8_mfma_kernel" if half else "blockquant8_stream_kernel", "bytes_per_launch": algo},
+                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and not lowbit) else None,
+                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_mfma_kernel", "bytes_per_launch": algo},
     }
 
 
@@ -226,7 +234,7 @@ def bench_mha(args, embed, heads, src, past):
     MultiHeadAttention_hip::forward without its host copies.  src new tokens are appended to a cache of `past` tokens."""
     import ncnn_amd
     from ncnn_amd.hip import check, lib as load
-    from oracle import oracle
+    from ncnn_amd import synth
     lib = load()
     rt = ncnn_amd.Runtime(0)
     st = rt.stream
@@ -235,7 +243,7 @@ def bench_mha(args, embed, heads, src, past):
     ws = []
     for _ in range(4):
         w = rng.normal(0, 1.0 / np.sqrt(embed), (embed, embed)).astype(np.float32)
-        packed, scales = oracle.blockquant_pack(w, 8, 64)
+        packed, scales = synth.blockquant_weights(w, 8, 64)
         ws.append((rt.up(packed), rt.up(scales), rt.up(rng.uniform(-0.1, 0.1, embed).astype(np.float32)), packed.nbytes + scales.nbytes))
     d_x = rt.up(rng.normal(0, 1, (src, embed)).astype(np.float32))
     d_kt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
@@ -571,7 +579,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
-                    help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M> | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
+                    help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
     ap.add_argument("--graph", type=int, default=0,
@@ -589,8 +597,9 @@ def main():
     if args.workload.startswith("gemm"):
         line = bench_gemm(args, int(args.workload[4:] or 4096))
     elif args.workload.startswith("blockquant:"):
-        n, k, m = (int(v) for v in args.workload.split(":")[1].split("x"))
-        line = bench_blockquant(args, n, k, m)
+        parts = args.workload.split(":")
+        n, k, m = (int(v) for v in parts[1].split("x"))
+        line = bench_blockquant(args, n, k, m, int(parts[2]) if len(parts) > 2 else 8, int(parts[3]) if len(parts) > 3 else 64)
     elif args.workload.startswith("mha:"):
         dims, src, past = args.workload.split(":")[1:]
         embed, heads = [int(v) for v in dims.split("x")]

@@ -46,9 +46,42 @@ __device__ __forceinline__ float to_f32(__half v)
 //     cover HBM latency;
 //   * a chunk never straddles a quantisation block (block >= 32), so the 16 products of a chunk
 //     are summed first and the block's 1/scale is applied once per chunk.
-template<typename AT, int MT, int R, int U>
+// BITS = 4 / 6 / 8: a chunk is always 16 weights, i.e. 8 / 12 / 16 bytes of the LSB-first field stream
+// (src/layer/gemm.cpp:318-336); a field is pulled out of its dword pair with one funnel shift + one signed bit-field extract.
+template<int BITS>
+__device__ __forceinline__ v4i_bq load_chunk(const uint8_t* p)
+{
+    v4i_bq w = {0, 0, 0, 0};
+    if (BITS == 8)
+        w = *reinterpret_cast<const v4i_bq*>(p);
+    else if (BITS == 6)
+    {
+        const int* q = reinterpret_cast<const int*>(p);
+        w[0] = q[0];
+        w[1] = q[1];
+        w[2] = q[2];
+    }
+    else
+    {
+        const int2 t = *reinterpret_cast<const int2*>(p);
+        w[0] = t.x;
+        w[1] = t.y;
+    }
+    return w;
+}
+template<int BITS>
+__device__ __forceinline__ float chunk_field(const v4i_bq& w, int t)
+{
+    const int bit = t * BITS, d = bit >> 5, sh = bit & 31;
+    unsigned lo = (unsigned)w[d];
+    if (sh + BITS > 32) lo = __funnelshift_r(lo, (unsigned)w[d + 1], sh); // the field straddles two dwords (6-bit only)
+    const int v = sh + BITS > 32 ? (int)lo : (int)(lo >> sh);
+    return (float)((v << (32 - BITS)) >> (32 - BITS));
+}
+
+template<typename AT, int MT, int R, int U, int BITS>
 __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __restrict__ a, size_t a_stride, int m0, int M, int N, int K,
-                                                                  const int8_t* __restrict__ b, int block_shift, int nblk,
+                                                                  const uint8_t* __restrict__ b, int block_shift, int nblk,
                                                                   const float* __restrict__ scales, const float* __restrict__ in_scales,
                                                                   const float* __restrict__ c, int bt, float alpha, float beta,
                                                                   float* __restrict__ out, size_t out_stride)
@@ -60,6 +93,7 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
     const int wave = threadIdx.x >> 6;
     const int j0 = (blockIdx.x * 4 + wave) * R;
     const int mcount = M - m0 < MT ? M - m0 : MT;
+    const size_t row_bytes = (size_t)K * BITS / 8; // K % 16 == 0
 
     float acc[R][MT];
 #pragma unroll
@@ -82,7 +116,7 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
                 const int j = j0 + r;
                 const bool ok = ch < nch && j < N;
                 const size_t koff = (size_t)kt0 + ((size_t)ch << 4);
-                w[r][u] = ok ? *reinterpret_cast<const v4i_bq*>(b + (size_t)j * K + koff) : v4i_bq{0, 0, 0, 0};
+                w[r][u] = ok ? load_chunk<BITS>(b + (size_t)j * row_bytes + koff * BITS / 8) : v4i_bq{0, 0, 0, 0};
                 d[r][u] = ok ? scales[(size_t)j * nblk + (koff >> block_shift)] : 1.f;
             }
     };
@@ -116,7 +150,7 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
 #pragma unroll
                     for (int t = 0; t < 16; t++)
                     {
-                        const float q = (float)(int)(int8_t)(w[r][u][t >> 2] >> ((t & 3) * 8));
+                        const float q = chunk_field<BITS>(w[r][u], t);
 #pragma unroll
                         for (int m = 0; m < MT; m++) part[m] = fmaf(av[m][t], q, part[m]);
                     }
@@ -250,8 +284,8 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
         }
 }
 
-template<typename AT>
-static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K, const int8_t* b8, int block, const float* scales,
+template<typename AT, int BITS = 8>
+static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K, const uint8_t* b8, int block, const float* scales,
                               const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride,
                               hipStream_t stream)
 {
@@ -267,19 +301,19 @@ static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K,
         const int left = M - m0;
         if (left >= 4)
         {
-            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 4, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 4, R, U, BITS>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
                                in_scales, c, bt, alpha, beta, out, out_stride);
             m0 += 4;
         }
         else if (left >= 2)
         {
-            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 2, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 2, R, U, BITS>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
                                in_scales, c, bt, alpha, beta, out, out_stride);
             m0 += 2;
         }
         else
         {
-            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 1, R, U>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
+            hipLaunchKernelGGL((blockquant8_stream_kernel<AT, 1, R, U, BITS>), grid, dim3(256), 0, stream, a, a_stride, m0, M, N, K, b8, shift, nblk, scales,
                                in_scales, c, bt, alpha, beta, out, out_stride);
             m0 += 1;
         }
@@ -296,8 +330,9 @@ static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K,
 typedef float v16f_bq __attribute__((ext_vector_type(16)));
 typedef float v4f_bq __attribute__((ext_vector_type(4)));
 
+template<int BITS>
 __global__ __launch_bounds__(256) void blockquant8_f32_mfma_kernel(const float* __restrict__ a, size_t a_stride, int M, int N, int K,
-                                                                   const int8_t* __restrict__ b, int block_shift, int nblk, const float* __restrict__ scales,
+                                                                   const uint8_t* __restrict__ b, int block_shift, int nblk, const float* __restrict__ scales,
                                                                    const float* __restrict__ in_scales, const float* __restrict__ c, int bt, float alpha,
                                                                    float beta, float* __restrict__ out, size_t out_stride)
 {
@@ -313,16 +348,29 @@ __global__ __launch_bounds__(256) void blockquant8_f32_mfma_kernel(const float* 
     const int arow = row0 + lr < M ? row0 + lr : M - 1; // rows past the end repeat the last one; their results are not stored
     const int brow = col0 + lr < N ? col0 + lr : N - 1;
     const float* ap = a + (size_t)arow * a_stride + lk;
-    const int8_t* bp = b + (size_t)brow * K + lk;
+    // the loader's 8 weights are BITS bytes of the field stream (2-byte aligned for 6-bit: three halfword loads)
+    const uint8_t* bp = b + (size_t)brow * ((size_t)K * BITS / 8) + (size_t)lk * BITS / 8;
     const float* sp = scales + (size_t)brow * nblk;
 
     v4f_bq a0, a1;
-    uint2 bq;
+    unsigned long long bq;
     float descale;
     auto fetch = [&](int k0) {
         a0 = *reinterpret_cast<const v4f_bq*>(ap + k0);
         a1 = *reinterpret_cast<const v4f_bq*>(ap + k0 + 4);
-        bq = *reinterpret_cast<const uint2*>(bp + k0);
+        const uint8_t* wp = bp + (size_t)k0 * BITS / 8;
+        if (BITS == 8)
+        {
+            const uint2 t = *reinterpret_cast<const uint2*>(wp);
+            bq = (unsigned long long)t.x | ((unsigned long long)t.y << 32);
+        }
+        else if (BITS == 6)
+        {
+            const unsigned short* hp = reinterpret_cast<const unsigned short*>(wp);
+            bq = (unsigned long long)hp[0] | ((unsigned long long)hp[1] << 16) | ((unsigned long long)hp[2] << 32);
+        }
+        else
+            bq = *reinterpret_cast<const unsigned*>(wp);
         descale = div_rn(1.f, sp[(k0 + lk) >> block_shift]);
         if (in_scales)
         {
@@ -343,8 +391,8 @@ __global__ __launch_bounds__(256) void blockquant8_f32_mfma_kernel(const float* 
         {
             pa[e] = a0[e];
             pa[4 + e] = a1[e];
-            pb[e] = mul_rn((float)(int)(int8_t)(bq.x >> (8 * e)), descale);
-            pb[4 + e] = mul_rn((float)(int)(int8_t)(bq.y >> (8 * e)), descale);
+            pb[e] = mul_rn((float)(((int)(unsigned)(bq >> (BITS * e)) << (32 - BITS)) >> (32 - BITS)), descale);
+            pb[4 + e] = mul_rn((float)(((int)(unsigned)(bq >> (BITS * (4 + e))) << (32 - BITS)) >> (32 - BITS)), descale);
         }
     };
 
@@ -624,19 +672,34 @@ int ncnnhip_gemm_blockquant(const float* a_dev, size_t a_stride, int M, int N, i
     NCNNHIP_REQUIRE(a_stride >= (size_t)K && out_stride >= (size_t)N, "ncnnhip_gemm_blockquant: stride too small");
     const int nblk = (K + block - 1) / block;
     dim3 grid(ceil_div(N, 4));
-    if (bits == 8 && M >= 32 && K % 32 == 0 && a_stride % 4 == 0 && al16(a_dev) && al16(b_dev) && (!in_scales_dev || al16(in_scales_dev)))
+    if (M >= 32 && K % 32 == 0 && a_stride % 4 == 0 && al16(a_dev) && al16(b_dev) && (!in_scales_dev || al16(in_scales_dev)))
     {
         const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
         dim3 tiles(ceil_div(N, 64), ceil_div(M, 64));
         NCNNHIP_REQUIRE(tiles.y <= 65535, "ncnnhip_gemm_blockquant: more than 65535*64 activation rows");
-        hipLaunchKernelGGL(blockquant8_f32_mfma_kernel, tiles, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev),
-                           shift, nblk, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride);
+#define LAUNCH_BQ_MFMA(BITS_) \
+    hipLaunchKernelGGL(blockquant8_f32_mfma_kernel<BITS_>, tiles, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, b_dev, shift, nblk, scales_dev, \
+                       in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride)
+        if (bits == 8)
+            LAUNCH_BQ_MFMA(8);
+        else if (bits == 6)
+            LAUNCH_BQ_MFMA(6);
+        else
+            LAUNCH_BQ_MFMA(4);
+#undef LAUNCH_BQ_MFMA
         return launch_status("blockquant8_f32_mfma_kernel");
     }
-    if (bits == 8 && K % 16 == 0 && al16(b_dev))
+    if (K % 16 == 0 && al16(b_dev))
     {
-        return launch_blockquant8<float>(a_dev, a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev), block, scales_dev, in_scales_dev,
-                                         c_dev, bt, alpha, beta, out_dev, out_stride, as_stream(stream));
+        // streaming kernel: 16 weights (8 / 12 / 16 bytes) per lane and step
+        if (bits == 8)
+            return launch_blockquant8<float, 8>(a_dev, a_stride, M, N, K, b_dev, block, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride,
+                                                as_stream(stream));
+        if (bits == 6)
+            return launch_blockquant8<float, 6>(a_dev, a_stride, M, N, K, b_dev, block, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride,
+                                                as_stream(stream));
+        return launch_blockquant8<float, 4>(a_dev, a_stride, M, N, K, b_dev, block, scales_dev, in_scales_dev, c_dev, bt, alpha, beta, out_dev, out_stride,
+                                            as_stream(stream));
     }
     const int packed = (int)(((size_t)K * bits + 7) / 8);
     hipLaunchKernelGGL(blockquant_generic_kernel, grid, dim3(256), 0, as_stream(stream), a_dev, a_stride, M, N, K, b_dev, bits, block, packed,
@@ -715,10 +778,17 @@ int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, 
 {
     int ret = check_blockquant(a_dev, b_dev, scales_dev, out_dev, M, N, K, bits, block, 0, -1);
     if (ret) return ret;
-    NCNNHIP_REQUIRE(bits == 8 && K % 16 == 0 && al16(b_dev), "ncnnhip_gemm_blockquant_f16a: needs 8-bit weights, K %% 16 == 0, aligned rows");
+    NCNNHIP_REQUIRE(K % 16 == 0 && al16(b_dev), "ncnnhip_gemm_blockquant_f16a: needs K %% 16 == 0 and 16-byte aligned weights");
     NCNNHIP_REQUIRE(a_stride >= (size_t)K && out_stride >= (size_t)N, "ncnnhip_gemm_blockquant_f16a: stride too small");
-    return launch_blockquant8<__half>(reinterpret_cast<const __half*>(a_dev), a_stride, M, N, K, reinterpret_cast<const int8_t*>(b_dev), block,
-                                      scales_dev, (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride, as_stream(stream));
+    const __half* ah = reinterpret_cast<const __half*>(a_dev);
+    if (bits == 8)
+        return launch_blockquant8<__half, 8>(ah, a_stride, M, N, K, b_dev, block, scales_dev, (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride,
+                                             as_stream(stream));
+    if (bits == 6)
+        return launch_blockquant8<__half, 6>(ah, a_stride, M, N, K, b_dev, block, scales_dev, (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride,
+                                             as_stream(stream));
+    return launch_blockquant8<__half, 4>(ah, a_stride, M, N, K, b_dev, block, scales_dev, (const float*)0, (const float*)0, -1, 1.f, 1.f, out_dev, out_stride,
+                                         as_stream(stream));
 }
 
 } // extern "C"

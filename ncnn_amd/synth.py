@@ -42,3 +42,36 @@ def blockquant8_operands(seed, m, n, k, block=64, half_exact=True):
     q = np.clip(_round_half_away((wp * scales[:, :, None]).astype(F)), -127, 127).astype(np.int8)
     packed = q.reshape(n, nblk * block)[:, :k].copy().view(np.uint8)
     return a, packed, scales
+
+
+def blockquant_weights(w, bits, block):
+    """fp32 [n][k] -> (packed uint8 [n][ceil(k*bits/8)], scales fp32 [n][ceil(k/block)]) in the .bin layout of the
+    block-quantised layers: scale = qmax/absmax per block (1 for an all-zero block), q = clamp(round_half_away(w*scale)),
+    fields of `bits` bits, two's complement, LSB first along K (src/layer/gemm.cpp:318-336; the packer of
+    tests/test_gemm_block_quant.cpp:80-129)."""
+    w = np.asarray(w, F)
+    n, k = w.shape
+    qmax = (1 << (bits - 1)) - 1
+    nblk = (k + block - 1) // block
+    wp = np.pad(w, ((0, 0), (0, nblk * block - k))).reshape(n, nblk, block)
+    absmax = np.abs(wp).max(axis=2)
+    with np.errstate(divide="ignore"):
+        scales = np.where(absmax == 0, F(1), F(qmax) / absmax).astype(F)
+    q = np.clip(_round_half_away((wp * scales[:, :, None]).astype(F)), -qmax, qmax).astype(np.int64).reshape(n, nblk * block)[:, :k]
+    if bits == 8:
+        return q.astype(np.int8).view(np.uint8).copy(), scales
+    fields = (q & ((1 << bits) - 1)).astype(np.uint8)
+    stream = ((fields[:, :, None] >> np.arange(bits, dtype=np.uint8)) & 1).reshape(n, k * bits)
+    return np.packbits(stream, axis=1, bitorder="little"), scales
+
+
+def blockquant_operands(seed, m, n, k, bits=8, block=64, half_exact=True):
+    """Activations N(0,1) (fp16-representable by default) and N(0,0.02) weights block-quantised to `bits` bits."""
+    if bits == 8:
+        return blockquant8_operands(seed, m, n, k, block, half_exact)
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((m, k), dtype=F)
+    if half_exact:
+        a = a.astype(np.float16).astype(F)
+    packed, scales = blockquant_weights((rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F), bits, block)
+    return a, packed, scales

@@ -265,7 +265,10 @@ def _bq_check(got, a, packed, scales, bits, block, ins=None, c=None, bt=-1, alph
     (8, 32, 16, 8, 64, 0, False), (4, 64, 1, 5, 65, 2, False), (8, 128, 5, 33, 1024, 4, True), (8, 64, 3, 10, 4096 + 16, -1, False),
     # 32 rows and more: the fp32 matrix-core kernel (ragged tiles in both directions, every C broadcast, input scales)
     (8, 64, 32, 64, 64, -1, False), (8, 64, 70, 100, 256, 4, True), (8, 32, 129, 65, 96, 3, False), (8, 128, 64, 31, 1024, 1, True),
-    (8, 64, 200, 130, 2048, 0, False), (8, 64, 33, 8, 4096 + 32, 2, False)])
+    (8, 64, 200, 130, 2048, 0, False), (8, 64, 33, 8, 4096 + 32, 2, False),
+    # 4- and 6-bit fields with K % 16 == 0: the streaming kernel (8 / 12 bytes per 16 weights) and the matrix-core kernel
+    (4, 32, 1, 24, 256, -1, False), (4, 64, 4, 40, 1024, 4, True), (6, 64, 3, 17, 512, 1, False), (6, 128, 2, 33, 4096 + 16, -1, True),
+    (4, 128, 70, 100, 256, 3, True), (6, 32, 40, 65, 96, 0, False), (4, 32, 16, 8, 11008, -1, False), (6, 64, 129, 31, 1024, 4, False)])
 def test_blockquant_small(rt, bits, block, m, n, k, bt, in_sc):
     _say("blockquant", bits, block, m, n, k, bt, in_sc)
     rng = np.random.default_rng(bits + block + m + n + k)
@@ -290,6 +293,19 @@ def test_blockquant_decode_shapes_fp32_and_fp16_activations(rt, m, n, k):
     _bq_check(got32, a, packed, scales, 8, 64)
     got16 = rt.gemm_blockquant(a.astype(np.float16), packed, scales, 8, 64)
     assert np.array_equal(got16, got32)  # fp16-representable activations: both entry points see the same numbers
+
+
+@pytest.mark.parametrize("bits", [4, 6])
+def test_blockquant_low_bit_decode_shape_fp16_activations(rt, bits):
+    _say("blockquant decode", bits)
+    m, n, k = 4, 256, 4096
+    rng = np.random.default_rng(bits)
+    a = rng.standard_normal((m, k)).astype(np.float16).astype(F)  # fp16-representable: both entry points see the same numbers
+    packed, scales = oracle.blockquant_pack((rng.standard_normal((n, k)) * 0.02).astype(F), bits, 32)
+    got32 = rt.gemm_blockquant(a, packed, scales, bits, 32)
+    _bq_check(got32, a, packed, scales, bits, 32)
+    got16 = rt.gemm_blockquant(a.astype(np.float16), packed, scales, bits, 32)
+    assert np.array_equal(got16, got32)
 
 
 @pytest.mark.parametrize("m,n,k,block,bt", [(1, 512, 4096, 64, -1), (4, 256, 4096, 64, 4), (16, 256, 4096, 64, 3), (16, 250, 11008, 64, -1),

@@ -418,3 +418,15 @@ def test_mha_blockquant_cache_identity():
         step, ck, cv = oracle.mha_blockquant(**dict(case, q=x, k=x, v=x, cached_k=ck, cached_v=cv))
         assert np.array_equal(step[0], full[i]), i
     assert np.array_equal(ck, kfull) and np.array_equal(cv, vfull)
+
+
+@pytest.mark.parametrize("bits,block", [(4, 32), (6, 128), (8, 64), (4, 64), (6, 32)])
+def test_product_side_block_quantiser_equals_the_oracles(bits, block):
+    """ncnn_amd.synth.blockquant_weights (numpy; feeds the benchmark and the model writer) against the oracle's packer."""
+    from ncnn_amd import synth
+    rng = np.random.default_rng(bits * block)
+    w = (rng.standard_normal((13, 200)) * 0.02).astype(F)
+    w[3, :64] = 0
+    p1, s1 = synth.blockquant_weights(w, bits, block)
+    p2, s2 = oracle.blockquant_pack(w, bits, block)
+    assert np.array_equal(p1, p2) and np.array_equal(s1, s2)
