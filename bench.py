@@ -139,15 +139,6 @@ def bench_gemm(args, size):
     ms_per_step = wall * 1e3 / args.steps
     achieved = ops / (gemm_ms * 1e-3) / 1e12
 
-    # correctness spot check of the timed buffers against the oracle on a row sample
-    from oracle import oracle
-    rows = np.arange(0, m, max(1, m // 8))[:8]
-    aq_ref, sa_ref = oracle.gemm_quantize_rows(a[rows])
-    ref = oracle.gemm_int8(aq_ref, bq, sa_ref, sb, bias, 4)
-    got = d_out.to_numpy(st)[rows]
-    if not np.array_equal(got, ref):
-        raise SystemExit("bench: GPU output differs from the oracle on the sampled rows")
-
     line = {
         "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -158,6 +149,14 @@ def bench_gemm(args, size):
                      "traffic": measured_traffic("gemm%d" % size), "kernel": "gemm_int8", "ops_per_launch": ops},
     }
     if not args.no_cpu:
+        # the CPU leg: first the checker (a row sample of the timed output buffer against the oracle), then the baseline timing
+        from oracle import oracle
+        rows = np.arange(0, m, max(1, m // 8))[:8]
+        aq_ref, sa_ref = oracle.gemm_quantize_rows(a[rows])
+        ref = oracle.gemm_int8(aq_ref, bq, sa_ref, sb, bias, 4)
+        got = d_out.to_numpy(st)[rows]
+        if not np.array_equal(got, ref):
+            raise SystemExit("bench: GPU output differs from the oracle on the sampled rows")
         line["cpu_baseline"] = cpu_baseline_gemm(n, k, args.b_scale == "per_column")
     return line
 

@@ -73,6 +73,41 @@ def test_batch_equals_per_sample(resident):
         assert np.array_equal(got[i].reshape(-1), refnet.run(param, blob, xs[i])["fc"])
 
 
+@RESIDENT
+def test_extractors_on_concurrent_threads_agree(resident):
+    """forward is const and re-entrant (src/layer.h:95-101; one Extractor per thread is ncnn's threading model): four
+    threads, each with its own Extractors and inputs, get what a single-threaded run gets."""
+    import threading
+    g, param, blob, info = zoo.build("mobilenetv2", input_hw=64, n_calib=1)
+    net = _load(param, blob, resident)
+    rng = np.random.default_rng(5)
+    xs = [rng.uniform(0, 1, g.input_shape).astype(F) for _ in range(4)]
+
+    def run(x):
+        ex = net.create_extractor()
+        ex.input("data", x)
+        return ex.extract("fc")
+
+    want = [run(x) for x in xs]
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(6):
+                if not np.array_equal(run(xs[i]), want[i]):
+                    errors.append("thread %d: result differs" % i)
+                    return
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (i, e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_int8_inference_switched_off_is_an_error_not_a_fallback():
     g, param, blob, info = zoo.build("tiny")
     net = _load(param, blob)
