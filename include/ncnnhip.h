@@ -160,6 +160,22 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
                                  const float* scale_in_dev, const float* bias_dev, ncnnhip_activation act, float* out_dev,
                                  const ncnnhip_conv_fusion* fusion, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Convolution::forward_int8 (src/layer/convolution.cpp:383-508) for layers with at most 4 input channels (the 3-channel
+ * first layer of an image net), group 1, dilation_w 1, zero border value.  The input is quantised into an image of 4 bytes
+ * per pixel with a physical zero border (ncnnhip_quantize_stem; source: channels-last fp32 blob with pixel stride src_cp, or
+ * int8), and one 16-byte K chunk of the contraction is 4 neighbouring pixels x 4 channels, so a 7x7x3 kernel costs K = 256
+ * instead of 832.  Output, epilogue, fused tail (may be NULL) and workspace contract as in ncnnhip_conv_int8_nhwc[_fused]
+ * with channels-last output; scale_out_dev non-NULL selects the requantised int8 output. */
+int ncnnhip_conv_stem_supported(const ncnnhip_conv_desc* desc);
+int ncnnhip_conv_stem_sizes(const ncnnhip_conv_desc* desc, size_t* image_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes);
+int ncnnhip_conv_stem_pack_weights(const ncnnhip_conv_desc* desc, const int8_t* weight_host, int8_t* packed_host);
+int ncnnhip_quantize_stem(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, int src_cp, const float* scale_dev,
+                          int8_t* image_dev, void* stream);
+int ncnnhip_conv_int8_stem(const ncnnhip_conv_desc* desc, const int8_t* image_dev, const int8_t* packed_weight_dev,
+                           const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
+                           void* out_dev, const ncnnhip_conv_fusion* fusion, void* workspace_dev, size_t workspace_bytes,
+                           void* stream);
+
 /* ------------------------------------------------------------------ device-resident blobs (channels-last)
  * Between layers a 3-D blob stays in HBM as [batch][h*w][Cp] (Cp = ncnnhip_padded_channels(c), fp32 or int8, pad
  * channels zero); 1-D / 2-D blobs are dense.  ncnn's planar Mat layout (src/mat.h:341-381) exists only at the host
@@ -168,6 +184,11 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
 int ncnnhip_padded_channels(int c);
 int ncnnhip_chw_to_nhwc(const void* src_dev, int elemsize, int c, int hw, int batch, size_t cstep, size_t nstep, void* dst_dev, void* stream);
 int ncnnhip_nhwc_to_chw(const void* src_dev, int elemsize, int c, int hw, int batch, void* dst_dev, size_t cstep, size_t nstep, void* stream);
+/* An fp32 image of at most 4 channels may stay at 4 floats per pixel, [n][h*w][4] (a quarter of the padded blob): the
+ * narrow-input convolution quantises straight from it (ncnnhip_quantize_stem with src_cp = 4); ncnnhip_widen_nhwc4_f32 turns
+ * it into the ordinary [n][h*w][16] blob for anything else. */
+int ncnnhip_chw_to_nhwc4_f32(const float* src_dev, int c, int hw, int batch, size_t cstep, size_t nstep, float* dst_dev, void* stream);
+int ncnnhip_widen_nhwc4_f32(const float* src_dev, float* dst_dev, size_t pixels, void* stream);
 /* Quantize::forward (src/layer/quantize.cpp:48-111) on a channels-last fp32 blob of npix pixels: one scale or one per channel. */
 int ncnnhip_quantize_nhwc(const float* src_dev, int8_t* dst_dev, size_t npix, int c, const float* scales_dev, int nscales, void* stream);
 /* The executor's int8 -> fp32 value cast for layers without int8 storage support (src/net.cpp:3007-3012 does the same at extract). */

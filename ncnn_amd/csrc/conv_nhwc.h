@@ -9,7 +9,9 @@ namespace ncnnhip {
 
 struct NhwcGeom
 {
-    int H, W, Cp;
+    int H, W, Cp; // Cp: bytes from one pixel to the next
+    int tapK;     // bytes of K one tap contributes (a multiple of 16).  Cp for an ordinary blob; 16 with Cp = 4 for the
+                  // narrow-input image, where one "tap" is 4 neighbouring pixels x 4 channels and kw counts such groups
     int kw, kh, dw, dh, sw, sh;
     int pad_top, pad_left;
     int outw, outh;

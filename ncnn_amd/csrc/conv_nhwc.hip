@@ -383,6 +383,69 @@ static SplitPlan plan_launch(int cout, long long npix, int steps)
 
 using namespace ncnnhip;
 
+// ---- narrow-input ("stem") convolution: up to 4 input channels ------------------------------------------------------
+// A 3-channel image padded to 16 channels wastes 13/16 of every K step.  Instead the quantised input is kept as an image
+// of 4 bytes per pixel with a zero border, [n][Hb][Wp][4], and one 16-byte K chunk is 4 NEIGHBOURING pixels x 4 channels:
+// a kernel row of kw taps becomes G = ceil(kw/4) chunks (weights beyond kw are zero).  In the pipelined kernel's terms this
+// is a convolution over pixels 4 bytes apart (Cp = 4) whose "taps" are G groups 4 pixels apart (dilation 4) contributing
+// 16 bytes each (tapK = 16); the border is physical, so no gather ever leaves the image.  7x7x3: K 832 -> 256.
+namespace ncnnhip {
+
+struct StemShape
+{
+    int G, Hb, Wp, K, outw, outh;
+    Pads4 pads;
+};
+
+static bool stem_supported(const ncnnhip_conv_desc& d)
+{
+    return d.group == 1 && d.c >= 1 && d.c <= 4 && d.dilation_w == 1 && ((int)(signed char)d.pad_value & 0xff) == 0;
+}
+
+static int stem_shape(const ncnnhip_conv_desc& d, StemShape& s)
+{
+    int ret = ncnnhip_conv_out_shape(&d, &s.outw, &s.outh);
+    if (ret) return ret;
+    s.pads = resolve_pads_nhwc(d);
+    s.G = (d.kernel_w + 3) / 4;
+    const int need_h = (s.outh - 1) * d.stride_h + (d.kernel_h - 1) * d.dilation_h + 1;
+    const int need_w = (s.outw - 1) * d.stride_w + (s.G - 1) * 4 + 4;
+    s.Hb = std::max(s.pads.top + d.h, need_h);
+    s.Wp = std::max(s.pads.left + d.w, need_w);
+    s.K = (d.kernel_h * s.G * 16 + 63) / 64 * 64;
+    return NCNNHIP_OK;
+}
+
+// one thread per pixel of the bordered image: 4 bytes out
+template<typename T>
+__global__ __launch_bounds__(256) void quantize_stem_kernel(const T* __restrict__ src, int src_cp, int c, int h, int w, int top, int left, int Hb, int Wp,
+                                                            size_t total, const float* __restrict__ scale, uint32_t* __restrict__ image)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int xb = (int)(i % (size_t)Wp);
+    const size_t rest = i / (size_t)Wp;
+    const int yb = (int)(rest % (size_t)Hb);
+    const size_t img = rest / (size_t)Hb;
+    const int y = yb - top, x = xb - left;
+    uint32_t word = 0;
+    if ((unsigned)y < (unsigned)h && (unsigned)x < (unsigned)w)
+    {
+        const T* p = src + ((img * h + y) * (size_t)w + x) * src_cp;
+        const float sc = sizeof(T) == 4 ? scale[0] : 1.f;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+        {
+            int v = 0;
+            if (q < c) v = sizeof(T) == 4 ? float2int8(mul_rn((float)p[q], sc)) : (int)p[q];
+            word |= (uint32_t)(v & 255) << (8 * q);
+        }
+    }
+    image[i] = word;
+}
+
+} // namespace ncnnhip
+
 extern "C" {
 
 int ncnnhip_conv_nhwc_sizes(const ncnnhip_conv_desc* desc, size_t* nhwc_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes)
@@ -458,6 +521,7 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc
     g.H = d.h;
     g.W = d.w;
     g.Cp = padded_channels(d.c);
+    g.tapK = g.Cp;
     g.kw = d.kernel_w;
     g.kh = d.kernel_h;
     g.dw = d.dilation_w;
@@ -561,6 +625,117 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
     f.q8_scale = fusion->quantise_scale;
     return conv_int8_nhwc_impl(desc, nhwc_dev, packed_weight_dev, scale_in_dev, bias_dev, 0, act, out_dev, NCNNHIP_CHANNELS_LAST, 0, 0, f, workspace_dev,
                                workspace_bytes, stream);
+}
+
+int ncnnhip_conv_stem_supported(const ncnnhip_conv_desc* desc)
+{
+    return desc && stem_supported(*desc) ? 1 : 0;
+}
+
+int ncnnhip_conv_stem_sizes(const ncnnhip_conv_desc* desc, size_t* image_bytes, size_t* packed_weight_bytes, size_t* workspace_bytes)
+{
+    NCNNHIP_REQUIRE(desc && stem_supported(*desc), "ncnnhip_conv_stem_sizes: needs group 1, at most 4 input channels, dilation_w 1, zero border value");
+    StemShape s;
+    int ret = stem_shape(*desc, s);
+    if (ret) return ret;
+    if (image_bytes) *image_bytes = (size_t)desc->batch * s.Hb * s.Wp * 4;
+    if (packed_weight_bytes) *packed_weight_bytes = (size_t)desc->num_output * s.K;
+    if (workspace_bytes) *workspace_bytes = conv_nhwc_pipelined_workspace_words(desc->num_output, (long long)desc->batch * s.outw * s.outh, s.K / 64) * sizeof(int32_t);
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_conv_stem_pack_weights(const ncnnhip_conv_desc* desc, const int8_t* weight_host, int8_t* packed_host)
+{
+    NCNNHIP_REQUIRE(desc && weight_host && packed_host && stem_supported(*desc), "ncnnhip_conv_stem_pack_weights: bad argument");
+    StemShape s;
+    int ret = stem_shape(*desc, s);
+    if (ret) return ret;
+    const int c = desc->c, kw = desc->kernel_w, kh = desc->kernel_h;
+    for (int p = 0; p < desc->num_output; p++)
+    {
+        int8_t* row = packed_host + (size_t)p * s.K;
+        for (int k = 0; k < s.K; k++) row[k] = 0;
+        for (int q = 0; q < c; q++)
+            for (int ky = 0; ky < kh; ky++)
+                for (int kx = 0; kx < kw; kx++)
+                    row[(ky * s.G + kx / 4) * 16 + (kx % 4) * 4 + q] = weight_host[(((size_t)p * c + q) * kh + ky) * kw + kx];
+    }
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_quantize_stem(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, int src_cp, const float* scale_dev, int8_t* image_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && nhwc_dev && image_dev && stem_supported(*desc), "ncnnhip_quantize_stem: bad argument");
+    NCNNHIP_REQUIRE((elemsize == 4 && scale_dev) || elemsize == 1, "ncnnhip_quantize_stem: fp32 (with a scale) or int8 input");
+    NCNNHIP_REQUIRE(src_cp >= desc->c, "ncnnhip_quantize_stem: source pixel stride below the channel count");
+    StemShape s;
+    int ret = stem_shape(*desc, s);
+    if (ret) return ret;
+    const size_t total = (size_t)desc->batch * s.Hb * s.Wp;
+    dim3 grid((unsigned)ceil_div((long long)total, 256));
+    if (elemsize == 4)
+        hipLaunchKernelGGL(quantize_stem_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)nhwc_dev, src_cp, desc->c, desc->h, desc->w, s.pads.top,
+                           s.pads.left, s.Hb, s.Wp, total, scale_dev, (uint32_t*)image_dev);
+    else
+        hipLaunchKernelGGL(quantize_stem_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)nhwc_dev, src_cp, desc->c, desc->h, desc->w,
+                           s.pads.top, s.pads.left, s.Hb, s.Wp, total, (const float*)0, (uint32_t*)image_dev);
+    return launch_status("quantize_stem_kernel");
+}
+
+int ncnnhip_conv_int8_stem(const ncnnhip_conv_desc* desc, const int8_t* image_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
+                           const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, const ncnnhip_conv_fusion* fusion,
+                           void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && image_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_stem: null pointer");
+    NCNNHIP_REQUIRE(stem_supported(*desc), "ncnnhip_conv_int8_stem: needs group 1, at most 4 input channels, dilation_w 1, zero border value");
+    NCNNHIP_REQUIRE(!fusion || !scale_out_dev, "ncnnhip_conv_int8_stem: the fused tail belongs to the fp32 output");
+    NCNNHIP_REQUIRE(!fusion || !fusion->quantised_out_dev || fusion->quantise_scale != 0.f, "ncnnhip_conv_int8_stem: quantised copy without a scale");
+    const ncnnhip_conv_desc& d = *desc;
+    StemShape s;
+    int ret = stem_shape(d, s);
+    if (ret) return ret;
+    const long long plane = (long long)s.outw * s.outh, npix = plane * d.batch;
+    NCNNHIP_REQUIRE(npix < (1ll << 31) && (long long)s.Hb * s.Wp * 4 < (1ll << 31), "ncnnhip_conv_int8_stem: extent too large");
+    NhwcGeom g;
+    g.H = s.Hb;
+    g.W = s.Wp;
+    g.Cp = 4;
+    g.tapK = 16;
+    g.kw = s.G;
+    g.kh = d.kernel_h;
+    g.dw = 4;
+    g.dh = d.dilation_h;
+    g.sw = d.stride_w;
+    g.sh = d.stride_h;
+    g.pad_top = g.pad_left = 0; // the border is part of the image
+    g.outw = s.outw;
+    g.outh = s.outh;
+    g.npix = (int)npix;
+    g.ntaps = d.kernel_h * s.G;
+    g.K = s.K;
+    g.cout = d.num_output;
+    g.pad_word = 0;
+    ConvEpilogue epi;
+    epi.scale_in = scale_in_dev;
+    epi.bias = bias_dev;
+    epi.scale_out = scale_out_dev;
+    epi.act = act;
+    epi.out = out_dev;
+    epi.out_cstep = epi.out_nstep = 0;
+    epi.pix_per_img = (int)plane;
+    epi.batch = d.batch;
+    epi.out_channel0 = 0;
+    epi.num_output = d.num_output;
+    epi.acc_out = 0;
+    ConvFusion f = {0, 0, 0, 0.f};
+    if (fusion)
+    {
+        f.residual = fusion->residual_dev;
+        f.relu_after = fusion->relu_after;
+        f.q8_out = fusion->quantised_out_dev;
+        f.q8_scale = fusion->quantise_scale;
+    }
+    return launch_conv_nhwc_pipelined(g, packed_weight_dev, image_dev, epi, f, padded_channels(d.num_output), workspace_dev, workspace_bytes, as_stream(stream));
 }
 
 } // extern "C"

@@ -112,8 +112,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     int q0, ky, kx, tap;
     {
         const int k = step_begin * 64 + ld_chunk * 16;
-        tap = k / g.Cp;
-        q0 = k - tap * g.Cp;
+        tap = k / g.tapK;
+        q0 = k - tap * g.tapK;
         ky = tap / g.kw;
         kx = tap - ky * g.kw;
     }
@@ -135,9 +135,9 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         for (int i = 0; i < LB; i++)
             __builtin_amdgcn_global_load_lds((const AS1 void*)(b_ptr[i] + (size_t)s * 64), (AS3 void*)(stage + BM * 64 + i * 4096), 16, 0, 0);
         q0 += 64;
-        while (q0 >= g.Cp)
+        while (q0 >= g.tapK)
         {
-            q0 -= g.Cp;
+            q0 -= g.tapK;
             tap++;
             if (++kx == g.kw)
             {
@@ -538,6 +538,7 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     g.H = 1;
     g.W = M;
     g.Cp = (int)aq_stride; // one "pixel" per row of A, its channels the K bytes of that row
+    g.tapK = g.Cp;
     g.kw = g.kh = g.dw = g.dh = g.sw = g.sh = 1;
     g.pad_top = g.pad_left = 0;
     g.outw = M;
@@ -601,6 +602,7 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
     g.H = 1;
     g.W = rows;
     g.Cp = (int)x_stride;
+    g.tapK = g.Cp;
     g.kw = g.kh = g.dw = g.dh = g.sw = g.sh = 1;
     g.pad_top = g.pad_left = 0;
     g.outw = rows;

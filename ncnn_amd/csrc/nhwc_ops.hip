@@ -56,6 +56,33 @@ __global__ __launch_bounds__(256) void nhwc_to_chw_kernel(const T* __restrict__ 
         if (q0 + e < c) dp[(size_t)(q0 + e) * cstep] = v[e];
 }
 
+// ---- narrow fp32 blobs: an image of at most 4 channels kept at 4 floats per pixel (instead of 16) as it comes from the
+// host; the first convolution quantises straight from it, anything else widens it first
+__global__ __launch_bounds__(256) void chw_to_nhwc4_f32_kernel(const float* __restrict__ src, size_t cstep, size_t nstep, int c, int hw, float* __restrict__ dst)
+{
+    const int pix = blockIdx.x * 256 + threadIdx.x;
+    const int img = blockIdx.y;
+    if (pix >= hw) return;
+    const float* sp = src + (size_t)img * nstep + pix;
+    v4f v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        if (q < c) v[q] = sp[(size_t)q * cstep];
+    *reinterpret_cast<v4f*>(dst + ((size_t)img * hw + pix) * 4) = v;
+}
+
+__global__ __launch_bounds__(256) void widen_nhwc4_f32_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t pixels)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= pixels) return;
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f* dp = reinterpret_cast<v4f*>(dst + i * 16);
+    dp[0] = *reinterpret_cast<const v4f*>(src + i * 4);
+    dp[1] = zero;
+    dp[2] = zero;
+    dp[3] = zero;
+}
+
 // ---- Quantize on a channels-last blob: 16 channels of one pixel per thread (64 bytes in, 16 out)
 __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float* __restrict__ src, int8_t* __restrict__ dst, size_t chunks, int c, int cp,
                                                              const float* __restrict__ scales, int nscales)
@@ -534,6 +561,20 @@ int ncnnhip_chw_to_nhwc(const void* src_dev, int elemsize, int c, int hw, int ba
     else
         hipLaunchKernelGGL(chw_to_nhwc_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)src_dev, cstep, nstep, c, hw, cp, (int8_t*)dst_dev);
     return launch_status("chw_to_nhwc_kernel");
+}
+
+int ncnnhip_chw_to_nhwc4_f32(const float* src_dev, int c, int hw, int batch, size_t cstep, size_t nstep, float* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && c >= 1 && c <= 4 && hw > 0 && batch > 0 && batch <= 65535 && cstep >= (size_t)hw, "ncnnhip_chw_to_nhwc4_f32: bad argument");
+    hipLaunchKernelGGL(chw_to_nhwc4_f32_kernel, dim3(ceil_div(hw, 256), batch), dim3(256), 0, as_stream(stream), src_dev, cstep, nstep, c, hw, dst_dev);
+    return launch_status("chw_to_nhwc4_f32_kernel");
+}
+
+int ncnnhip_widen_nhwc4_f32(const float* src_dev, float* dst_dev, size_t pixels, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev && pixels > 0, "ncnnhip_widen_nhwc4_f32: bad argument");
+    hipLaunchKernelGGL(widen_nhwc4_f32_kernel, dim3((unsigned)ceil_div((long long)pixels, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, pixels);
+    return launch_status("widen_nhwc4_f32_kernel");
 }
 
 int ncnnhip_nhwc_to_chw(const void* src_dev, int elemsize, int c, int hw, int batch, void* dst_dev, size_t cstep, size_t nstep, void* stream)

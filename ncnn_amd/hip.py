@@ -96,6 +96,14 @@ _SIGNATURES = {
     "ncnnhip_relu": [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p],
     "ncnnhip_scale": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_void_p],
     "ncnnhip_eltwise": [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.POINTER(C.c_float), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_chw_to_nhwc4_f32": [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_widen_nhwc4_f32": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_conv_stem_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_stem_sizes": [C.POINTER(ConvDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "ncnnhip_conv_stem_pack_weights": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p],
+    "ncnnhip_quantize_stem": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_conv_int8_stem": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.POINTER(ConvFusion),
+                               C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_pooling_nhwc": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
     "ncnnhip_maxpool_nhwc_int8": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
     "ncnnhip_softmax": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
@@ -401,9 +409,10 @@ class Runtime:
 
     def conv_channels_last(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
                            pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), residual=None, relu_after=False,
-                           quantise_scale=None):
+                           quantise_scale=None, stem=False):
         """Convolution (group 1) or depthwise (group == c == num_output) entirely on channels-last device blobs:
-        upload+convert, quantise if fp32, kernel writing channels-last, convert back.  x is [n][c][h][w]."""
+        upload+convert, quantise if fp32, kernel writing channels-last, convert back.  x is [n][c][h][w].
+        stem=True: the narrow-input form (at most 4 input channels, 4-byte pixels with a physical border)."""
         x = np.ascontiguousarray(x)
         if x.ndim == 3:
             x = x[None]
@@ -418,7 +427,16 @@ class Runtime:
         scale_in = self.fold_input_scales(w_scales, in_scales, num_output)
         requant = term > 100
         src = self.to_channels_last(x)
-        if x.dtype != np.int8:
+        if stem:
+            if not lib().ncnnhip_conv_stem_supported(C.byref(d)):
+                raise ValueError("not a narrow-input convolution")
+            ib, wb, sb_ = C.c_size_t(), C.c_size_t(), C.c_size_t()
+            check(lib().ncnnhip_conv_stem_sizes(C.byref(d), C.byref(ib), C.byref(wb), C.byref(sb_)))
+            image = DeviceBuffer.empty((ib.value,), np.int8)
+            dscale = self.up(in_scales[:1])
+            check(lib().ncnnhip_quantize_stem(C.byref(d), src.ptr, x.dtype.itemsize, src.shape[2], dscale.ptr, image.ptr, self.stream))
+            src = image
+        elif x.dtype != np.int8:
             per_channel = np.repeat(in_scales, c // in_scales.size).astype(np.float32) if in_scales.size > 1 else in_scales
             src = self.quantize_channels_last(src, c, per_channel)
         scale_out = None
@@ -429,7 +447,20 @@ class Runtime:
         ocp = lib().ncnnhip_padded_channels(num_output)
         dout = DeviceBuffer.empty((n, oh * ow, ocp), np.int8 if requant else np.float32)
         wq = np.ascontiguousarray(weight, np.int8)
-        if group == 1:
+        if stem:
+            pk = np.empty(wb.value, np.int8)
+            check(lib().ncnnhip_conv_stem_pack_weights(C.byref(d), wq.ctypes.data, pk.ctypes.data))
+            dpk, dws = self.up(pk), DeviceBuffer.zeros(sb_.value, self.stream)
+            fused = residual is not None or relu_after or quantise_scale is not None
+            dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))
+            dq8 = None if quantise_scale is None else DeviceBuffer.empty((n, oh * ow, ocp), np.int8)
+            fu = ConvFusion(_ptr(dres), int(relu_after), _ptr(dq8), float(quantise_scale or 0.0))
+            check(lib().ncnnhip_conv_int8_stem(C.byref(d), src.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso), Activation.make(act, act_params), dout.ptr,
+                                               C.byref(fu) if fused else None, dws.ptr, sb_.value, self.stream))
+            if fused:
+                q8 = None if dq8 is None else self.from_channels_last(dq8, n, num_output, oh, ow)
+                return self.from_channels_last(dout, n, num_output, oh, ow), q8
+        elif group == 1:
             nb, wb, sb_ = C.c_size_t(), C.c_size_t(), C.c_size_t()
             check(lib().ncnnhip_conv_nhwc_sizes(C.byref(d), C.byref(nb), C.byref(wb), C.byref(sb_)))
             pk = np.empty(wb.value, np.int8)

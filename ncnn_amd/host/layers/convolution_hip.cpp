@@ -18,7 +18,7 @@ Convolution_hip::Convolution_hip(bool depthwise_type) : is_depthwise_type(depthw
     one_blob_only = true;
     support_inplace = false;
     support_batch = true; // Mat.n is folded into the pixel dimension of the implicit GEMM
-    d_weight = d_weight_packed = d_weight_dw = d_bias = d_scale_in = d_scale_out = d_scale_out_uniform = d_input_scales = 0;
+    d_weight = d_weight_packed = d_weight_stem = d_weight_dw = d_bias = d_scale_in = d_scale_out = d_scale_out_uniform = d_input_scales = 0;
     uniform_scale_out = 0.f;
     output_abs_bound = 0.0;
     input_scale_count = 0;
@@ -210,6 +210,20 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
         rc = ncnnhip_conv_pack_weights(&desc, (const int8_t*)weight_data.data, packed.data());
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_pack_weights");
         ret = upload_constant(packed.data(), packed_bytes, &d_weight_packed);
+        // a layer with at most 4 input channels (the first layer of an image net) also gets the narrow-input packing
+        desc.dilation_w = dilation_w;
+        desc.dilation_h = dilation_h;
+        desc.pad_value = pad_value;
+        if (ret == 0 && ncnnhip_conv_stem_supported(&desc))
+        {
+            size_t stem_bytes = 0;
+            rc = ncnnhip_conv_stem_sizes(&desc, 0, &stem_bytes, 0);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_stem_sizes");
+            std::vector<int8_t> stem(stem_bytes);
+            rc = ncnnhip_conv_stem_pack_weights(&desc, (const int8_t*)weight_data.data, stem.data());
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_stem_pack_weights");
+            ret = upload_constant(stem.data(), stem_bytes, &d_weight_stem);
+        }
     }
     else
         ret = upload_constant(weight_data.data, (size_t)weight_data_size, &d_weight);
@@ -244,7 +258,7 @@ int Convolution_hip::create_pipeline(const Option& /*opt*/)
 
 int Convolution_hip::destroy_pipeline(const Option& /*opt*/)
 {
-    void** all[] = {&d_weight, &d_weight_packed, &d_weight_dw, &d_bias, &d_scale_in, &d_scale_out, &d_scale_out_uniform, &d_input_scales};
+    void** all[] = {&d_weight, &d_weight_packed, &d_weight_stem, &d_weight_dw, &d_bias, &d_scale_in, &d_scale_out, &d_scale_out_uniform, &d_input_scales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
@@ -386,6 +400,11 @@ int Convolution_hip::forward_hip_fused(const HipMat& bottom, const HipMat* resid
     return forward_device(bottom, residual, relu, q8_scale, 0.f, top, cmd, opt);
 }
 
+bool Convolution_hip::hip_accepts_narrow_input() const
+{
+    return support_hip; // the narrow-input kernel quantises straight from it; any other form widens it itself
+}
+
 int Convolution_hip::hip_prepare_requantise(float scale)
 {
     // fp32-output layers only: the reference's own requantising epilogue (convolution.cpp:489-496) then runs with
@@ -416,9 +435,15 @@ int Convolution_hip::forward_hip_requantised(const HipMat& bottom, float scale, 
     return forward_device(bottom, 0, false, 0.f, scale, top, cmd, opt);
 }
 
-int Convolution_hip::forward_device(const HipMat& bottom, const HipMat* residual, bool relu, float q8_scale, float only_scale, HipMat& top, HipCommand& cmd,
+int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* residual, bool relu, float q8_scale, float only_scale, HipMat& top, HipCommand& cmd,
                                     const Option& opt) const
 {
+    HipMat bottom = bottom_in;
+    if (bottom.narrow() && !(group == 1 && d_weight_stem))
+    {
+        int wret = cmd.widen(bottom_in, bottom);
+        if (wret != 0) return wret;
+    }
     const bool fused = residual || relu || q8_scale != 0.f;
     if (fused && !hip_can_fuse_tail()) return -1;
     if (!opt.use_int8_inference)
@@ -465,6 +490,36 @@ int Convolution_hip::forward_device(const HipMat& bottom, const HipMat* residual
     {
         NCNN_LOGE("%s %s: the residual blob does not have the output's shape", type.c_str(), name.c_str());
         return -1;
+    }
+    if (group == 1 && d_weight_stem && ncnnhip_conv_stem_supported(&desc))
+    {
+        // narrow input: quantise into the bordered 4-byte-per-pixel image, 4 neighbouring pixels per K chunk
+        size_t image_bytes = 0, workspace_bytes = 0;
+        rc = ncnnhip_conv_stem_sizes(&desc, &image_bytes, 0, &workspace_bytes);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_stem_sizes");
+        void* image = scratch.get(image_bytes);
+        if (!image) return -100;
+        rc = ncnnhip_quantize_stem(&desc, bottom.data, (int)bottom.elemsize, bottom.cp, (const float*)d_input_scales, (int8_t*)image, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_quantize_stem");
+        void* ws = workspace_bytes ? cmd.zeroed_workspace(workspace_bytes) : 0;
+        if (workspace_bytes && !ws) return -100;
+        ncnnhip_conv_fusion fu;
+        fu.residual_dev = residual ? (const float*)residual->data : 0;
+        fu.relu_after = relu ? 1 : 0;
+        fu.quantised_out_dev = 0;
+        fu.quantise_scale = q8_scale;
+        if (q8_scale != 0.f)
+        {
+            top.q8.reset(new HipMat);
+            top.q8->create(outw, outh, num_output, 1u, bottom.n, &cmd);
+            if (top.q8->empty()) return -100;
+            top.q8_scale = q8_scale;
+            fu.quantised_out_dev = (int8_t*)top.q8->data;
+        }
+        rc = ncnnhip_conv_int8_stem(&desc, (const int8_t*)image, (const int8_t*)d_weight_stem, (const float*)d_scale_in, (const float*)d_bias,
+                                    requant ? scale_out_table : 0, make_activation(activation_type, activation_params), top.data, fused ? &fu : 0, ws,
+                                    workspace_bytes, st);
+        return to_ncnn_status(rc, "ncnnhip_conv_int8_stem");
     }
     const int8_t* xq = (const int8_t*)bottom.data;
     if (bottom.elemsize == 4u && bottom.q8 && !bottom.q8->empty() && bottom.q8_scale == bottom_blob_int8_scales[0] && bottom.q8->count() == bottom.count())

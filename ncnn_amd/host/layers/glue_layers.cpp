@@ -63,6 +63,10 @@ public:
         support_int8_storage = true; // int8 blobs pass through untouched
         support_hip = true;
     }
+    virtual bool hip_accepts_narrow_input() const
+    {
+        return true; // handles are passed on, the data is not touched
+    }
     virtual int forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand&, const Option&) const
     {
         for (size_t i = 0; i < top_blobs.size(); i++) top_blobs[i] = bottom_blobs[0]; // shared, refcounted

@@ -28,6 +28,7 @@ public:
     virtual int forward_hip_fused(const ncnn::HipMat& bottom_blob, const ncnn::HipMat* residual, bool relu, float q8_scale, ncnn::HipMat& top_blob,
                                   ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
     virtual int hip_prepare_requantise(float scale);
+    virtual bool hip_accepts_narrow_input() const;
     virtual int forward_hip_requantised(const ncnn::HipMat& bottom_blob, float scale, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd,
                                         const ncnn::Option& opt) const;
 
@@ -46,6 +47,7 @@ private:
     // device copies made at create_pipeline
     void* d_weight;        // group > 1: [num_output][c/group][kh][kw] as stored in the model
     void* d_weight_packed; // group == 1: [num_output][kh*kw][16*ceil(c/16)] for the channels-last kernel
+    void* d_weight_stem;   // group == 1 and at most 4 input channels: [num_output][kh][ceil(kw/4)][4 pixels][4 channels]
     void* d_bias;
     void* d_scale_in;      // one per output channel: 1/(in_scale*w_scale), 0 when w_scale is 0
     void* d_scale_out;     // one per output channel, only when requantising

@@ -116,6 +116,19 @@ void HipMat::create(int _w, int _h, int _c, size_t _elemsize, int _n, HipCommand
     allocate(command);
 }
 
+void HipMat::create_narrow(int _w, int _h, int _c, int _n, HipCommand* command)
+{
+    release();
+    dims = 3;
+    w = _w;
+    h = _h;
+    c = _c;
+    n = _n < 1 ? 1 : _n;
+    cp = 4;
+    elemsize = 4u;
+    allocate(command);
+}
+
 void HipMat::create_like(const HipMat& m, HipCommand* command)
 {
     if (m.dims == 1)
@@ -243,7 +256,9 @@ int HipCommand::upload(const Mat& src, HipMat& dst)
         NCNN_LOGE("HipCommand::upload: needs a pack-1 fp32 or int8 blob of 1 to 3 dimensions");
         return -1;
     }
-    if (src.dims == 3)
+    if (src.dims == 3 && src.elemsize == 4u && src.c <= 4)
+        dst.create_narrow(src.w, src.h, src.c, src.n, this); // an image: a quarter of the padded blob's bytes
+    else if (src.dims == 3)
         dst.create(src.w, src.h, src.c, src.elemsize, src.n, this);
     else if (src.dims == 1)
         dst.create(src.w, src.elemsize, src.n, this);
@@ -270,7 +285,10 @@ int HipCommand::upload_into(const Mat& src, HipMat& dst)
         void* staging = scratch.get(host_bytes(src));
         if (!staging) return -100;
         int rc = ncnnhip_memcpy_h2d(staging, src.data, host_bytes(src), stream);
-        if (rc == 0) rc = ncnnhip_chw_to_nhwc(staging, (int)src.elemsize, src.c, src.w * src.h, src.n, src.cstep, src.nstep, dst.data, stream);
+        if (rc == 0 && dst.narrow())
+            rc = ncnnhip_chw_to_nhwc4_f32((const float*)staging, src.c, src.w * src.h, src.n, src.cstep, src.nstep, (float*)dst.data, stream);
+        else if (rc == 0)
+            rc = ncnnhip_chw_to_nhwc(staging, (int)src.elemsize, src.c, src.w * src.h, src.n, src.cstep, src.nstep, dst.data, stream);
         // the copy out of pageable host memory must have left the caller's buffer before we return
         if (rc == 0) rc = ncnnhip_stream_synchronize(stream);
         return hip_status(rc, "upload");
@@ -283,9 +301,27 @@ int HipCommand::upload_into(const Mat& src, HipMat& dst)
     return hip_status(rc, "upload");
 }
 
-int HipCommand::download(const HipMat& src, Mat& dst, Allocator* allocator)
+int HipCommand::widen(const HipMat& src, HipMat& dst)
 {
-    if (src.empty()) return -1;
+    if (src.empty() || !src.narrow() || src.elemsize != 4u) return -1;
+    HipMat wide;
+    wide.create(src.w, src.h, src.c, 4u, src.n, this);
+    if (wide.empty()) return -100;
+    int rc = ncnnhip_widen_nhwc4_f32((const float*)src.data, (float*)wide.data, (size_t)src.n * src.h * src.w, stream);
+    if (rc != 0) return hip_status(rc, "ncnnhip_widen_nhwc4_f32");
+    dst = wide;
+    return 0;
+}
+
+int HipCommand::download(const HipMat& blob, Mat& dst, Allocator* allocator)
+{
+    if (blob.empty()) return -1;
+    HipMat src = blob;
+    if (src.narrow())
+    {
+        int ret = widen(blob, src);
+        if (ret != 0) return ret;
+    }
     if (src.dims == 3)
     {
         dst.create(src.w, src.h, src.c, src.elemsize, 1, src.n, allocator);

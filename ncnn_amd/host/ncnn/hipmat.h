@@ -35,6 +35,13 @@ public:
     void create(int w, int h, size_t elemsize, int n, HipCommand* cmd);
     void create(int w, int h, int c, size_t elemsize, int n, HipCommand* cmd);
     void create_like(const HipMat& m, HipCommand* cmd);
+    // fp32 image of at most 4 channels at 4 floats per pixel (cp = 4): how such an input arrives from the host.  Only
+    // layers that say so (Layer::hip_accepts_narrow_input) see it; the executor widens it for everyone else.
+    void create_narrow(int w, int h, int c, int n, HipCommand* cmd);
+    bool narrow() const
+    {
+        return dims == 3 && cp < 16;
+    }
     void release();
 
     bool empty() const
@@ -60,7 +67,7 @@ public:
     int* refcount; // host side
     HipCommand* cmd;
     int dims, w, h, c, n;
-    int cp; // channels as padded in memory (dims 3), else 0
+    int cp; // channels as padded in memory (dims 3), else 0.  16*ceil(c/16), or 4 for a narrow fp32 image (create_narrow)
     size_t elemsize;
     // An fp32 blob may travel with an int8 copy of itself, float2int8(value * q8_scale), written by the kernel
     // that produced it: the convolution that consumes the blob with that input scale then skips its Quantize pass.
@@ -94,6 +101,7 @@ public:
     // host Mat (planar, any batch) -> device blob and back; download synchronises the stream
     int upload(const Mat& src, HipMat& dst);
     int upload_into(const Mat& src, HipMat& dst); // dst exists and has src's shape: new values for the same buffer
+    int widen(const HipMat& src, HipMat& dst);    // narrow blob -> ordinary 16-channel-padded blob (enqueued, not waited for)
     int download(const HipMat& src, Mat& dst, Allocator* allocator);
     int synchronize();
 

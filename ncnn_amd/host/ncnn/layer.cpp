@@ -120,6 +120,10 @@ bool Layer::hip_quantise_transparent() const
 {
     return false;
 }
+bool Layer::hip_accepts_narrow_input() const
+{
+    return false;
+}
 
 // ---- built-in type table ------------------------------------------------------------------
 

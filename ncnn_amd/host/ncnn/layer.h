@@ -69,6 +69,8 @@ public:
     // forward_hip_requantised(bottom, scale) gives the int8 blob float2int8(forward(bottom) * scale).
     virtual int hip_prepare_requantise(float scale);
     virtual int forward_hip_requantised(const HipMat& bottom_blob, float scale, HipMat& top_blob, HipCommand& cmd, const Option& opt) const;
+    // takes a narrow fp32 image (HipMat::narrow) as it is; everyone else gets it widened to the ordinary layout first
+    virtual bool hip_accepts_narrow_input() const;
     // forward_hip of an int8 blob holding Quantize(x, s), s > 0, gives Quantize(forward_hip(x), s) (windowed max pooling)
     virtual bool hip_quantise_transparent() const;
 

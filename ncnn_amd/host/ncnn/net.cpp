@@ -328,7 +328,7 @@ int NetPrivate::try_fused_tail(int layer_index, ExecState& st, const Option& opt
         }
         ins[k] = st.dev[bi];
     }
-    if (ins[1].elemsize != 4u || ins[1].dims != 3) return 0; // the residual must be an fp32 blob: take the plain route
+    if (ins[1].elemsize != 4u || ins[1].dims != 3 || ins[1].narrow()) return 0; // the residual must be an ordinary fp32 blob: take the plain route
     for (int k = 0; k < 2; k++)
     {
         st.dev[(size_t)needed[k]].release();
@@ -404,6 +404,11 @@ int NetPrivate::run_layer_hip(const Layer* layer, ExecState& st, const Option& o
         {
             st.dev[bi].release();
             st.host[bi].release();
+        }
+        if (ins[i].narrow() && !layer->hip_accepts_narrow_input())
+        {
+            ret = cmd.widen(ins[i], ins[i]);
+            if (ret != 0) return ret;
         }
         const bool passes_quantised = ins[i].elemsize == 1u && ins[i].q8_scale > 0.f && layer->one_blob_only && layer->hip_quantise_transparent();
         if (ins[i].elemsize == 1u && !layer->support_int8_storage && !passes_quantised)

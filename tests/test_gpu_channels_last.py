@@ -221,3 +221,41 @@ def test_convolution_with_residual_relu_and_quantised_copy_in_the_epilogue(rt, c
                                        residual=res, relu_after=relu, quantise_scale=next_scale)
     assert np.array_equal(got, want)
     assert np.array_equal(got_q, want_q)
+
+
+# ---- narrow-input ("stem") convolution: 4-byte pixels with a physical border, 4 neighbouring pixels per K chunk ---------
+
+@pytest.mark.parametrize("c,h,w,outc,kernel,stride,pads,dil_h,term,act", [
+    (3, 32, 32, 64, (7, 7), (2, 2), (3, 3, 3, 3), 1, 2, 1),      # the ResNet stem, small
+    (3, 33, 29, 32, (3, 3), (2, 2), (1, 1, 1, 1), 1, 101, 3),    # MobileNetV2's first layer: requantised output, clip
+    (1, 17, 40, 20, (5, 3), (1, 1), (0, 4, 2, 0), 1, 1, 0),      # one channel, uneven pads, stride 1 (4-byte aligned gathers)
+    (4, 20, 21, 70, (1, 1), (1, 2), (0, 0, 0, 0), 1, 2, 2),      # 1x1, leaky
+    (2, 25, 25, 16, (9, 2), (3, 1), (-233, -233, -233, -233), 2, 2, 1),  # SAME pads, two groups of taps + a partial one, dilated rows
+    (3, 16, 16, 130, (4, 4), (4, 4), (0, 0, 0, 0), 1, 102, 0),   # patch embedding, more output channels than one tile
+])
+def test_stem_convolution_matches_oracle(rt, c, h, w, outc, kernel, stride, pads, dil_h, term, act):
+    x, wq, b, ws, ins, tops = cases.conv_case(c * 1000 + h + outc, c, h, w, outc, kernel, 1, term, True)
+    act_params = {0: (0.0, 0.0), 1: (0.0, 0.0), 2: (0.1, 0.0), 3: (0.0, 3.0)}[act]
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, (1, dil_h), stride, pads, 0.0, 1, term, act, act_params, stem=True)
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, dil_h), stride, pads, 0.0, 1, 1, term, act, act_params)
+    want = oracle.convolution_int8(d, x[0], wq, b, ws, ins[0], None if tops is None else tops[0])
+    assert got.dtype == want.dtype and np.array_equal(got[0], want)
+
+
+def test_stem_convolution_batch_int8_input_and_fused_tail(rt):
+    """Batch of 3, an int8 input blob (already quantised upstream), and the fused tail (residual, ReLU, quantised copy)."""
+    c, h, w, outc, kernel = 3, 18, 22, 48, (3, 3)
+    x, wq, b, ws, ins, tops = cases.conv_case(77, c, h, w, outc, kernel, 1, 2, True, False, batch=3)
+    rng = np.random.default_rng(78)
+    xq = oracle.quantize(x.reshape(3 * c, -1), ins[:1]).reshape(x.shape)
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 1, 1, 2, 1)
+    plain = rt.conv_channels_last(xq, wq, b, ws, ins, None, outc, kernel, pads=(1, 1, 1, 1), term=2, act=1, stem=True)
+    res = rng.normal(0, 1, plain.shape).astype(F)
+    got, q8 = rt.conv_channels_last(x, wq, b, ws, ins, None, outc, kernel, pads=(1, 1, 1, 1), term=2, act=1, residual=res, relu_after=True,
+                                    quantise_scale=21.5, stem=True)
+    for i in range(3):
+        want = oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None)
+        assert np.array_equal(plain[i], want)
+        fused = np.maximum((want + res[i]).astype(F), 0)
+        assert np.array_equal(got[i], fused)
+        assert np.array_equal(q8[i], oracle.quantize(fused.reshape(1, -1), F(21.5)).reshape(fused.shape))

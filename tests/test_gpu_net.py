@@ -108,6 +108,23 @@ def test_extractors_on_concurrent_threads_agree(resident):
     assert not errors, errors
 
 
+def test_narrow_input_image_reaches_layers_that_need_the_ordinary_layout():
+    """A 3-channel input stays at 4 floats per pixel on the device; layers other than the first convolution get it
+    widened, and extracting it gives back what went in."""
+    lines = ["Input in0 0 1 data 0=12 1=10 2=3", "Split sp 1 3 data d1 d2 d3", "Pooling pool 1 1 d1 p 0=0 1=2 2=2", "ReLU relu 1 1 d2 r",
+             "Pooling gap 1 1 d3 g 0=1 4=1"]
+    net = _load(mw.assemble_param(lines), b"", True)
+    x = np.random.default_rng(2).normal(0, 1, (2, 3, 10, 12)).astype(F)
+    for name, want in (("p", x.reshape(2, 3, 5, 2, 6, 2).max(axis=(3, 5))), ("r", np.maximum(x, 0)), ("data", x)):
+        ex = net.create_extractor()
+        ex.input("data", x)
+        assert np.array_equal(ex.extract(name), want), name
+    ex = net.create_extractor()
+    ex.input("data", x)
+    flat = x.reshape(2, 3, -1)
+    assert np.array_equal(ex.extract("g"), (np.cumsum(flat, axis=2, dtype=F)[..., -1] / F(120)).astype(F))
+
+
 def test_int8_inference_switched_off_is_an_error_not_a_fallback():
     g, param, blob, info = zoo.build("tiny")
     net = _load(param, blob)
