@@ -441,14 +441,11 @@ struct PipePlan
 static PipePlan plan_pipelined(int cout, long long npix, int steps)
 {
     PipePlan p;
-    // channel tile: the whole channel count in one tile when it fits (activations are then read once), else the
-    // width that pads least
-    if (cout <= 64)
-        p.bn = 64;
-    else if (cout <= 128)
-        p.bn = 128;
-    else
-        p.bn = (ceil_div(cout, 256) * 256 <= ceil_div(cout, 128) * 128) ? 256 : 128;
+    // channel tile: the width that pads the channel count least (padded channels cost matrix-core time and unbalance the
+    // wavefronts' epilogues: 144 channels in one 256-wide tile ran 34 us, in three 64-wide tiles 21), the wider on a tie
+    p.bn = 64;
+    for (int bn = 128; bn <= 256; bn *= 2)
+        if (ceil_div(cout, bn) * bn <= ceil_div(cout, p.bn) * p.bn) p.bn = bn;
     p.bm = 128;
     auto tiles = [&]() { return (long long)ceil_div(npix, p.bm) * ceil_div(cout, p.bn); };
     // measured over the ResNet-50 / MobileNetV2 layers: more, smaller workgroups win until there are a few
