@@ -71,16 +71,25 @@ __device__ __forceinline__ int float2int8(float v)
     return q;
 }
 
-// the same value as (float)float2int8(v), computed without leaving the float pipe: round half away from zero as
-// trunc + exact remainder test, clamp with max/min (a NaN comes out as -127 either way), and the x86 conversion quirk
-// of the reference (|v| >= 2^31 converts to INT_MIN, hence -127) as one compare-select
+// A float whose truncation toward zero is float2int8(v); every user converts it with (int), i.e. v_cvt_i32_f32.
+//   clamp first: round-half-away(clamp(v, -127, 127)) == clamp(round-half-away(v), -127, 127)
+//   round as trunc(c + copysign(0.5, c)) with the ADD rounded toward zero: a nearest-even add would turn
+//   0.49999997 + 0.5 into 1.0; rounded toward zero the sum never reaches the next integer unless c + 0.5 does exactly
+//   (integers below 2^24 are representable, so RTZ(c + 0.5) >= floor(c + 0.5)).  The rounding mode lives in the wave's
+//   MODE register (bits 1:0, 3 = toward zero): it is switched for that one add and back inside one asm statement.
+//   NaN and |v| >= 2^31 give -127 like the x86 conversion of the reference (INT_MIN, then clamped).
+// 5 VALU instructions (med3, bfi, add, cmp, cndmask) instead of 10 for trunc + remainder test + clamp.
 __device__ __forceinline__ float float2int8_as_float(float v)
 {
-    const float t = truncf(v);
-    const float d = v - t; // exact
-    float r = t + (fabsf(d) >= 0.5f ? copysignf(1.f, v) : 0.f);
-    r = fminf(fmaxf(r, -127.f), 127.f);
-    return fabsf(v) < 2147483648.f ? r : -127.f;
+    const float c = __builtin_amdgcn_fmed3f(v, -127.f, 127.f);
+    const float h = copysignf(0.5f, c);
+    float y;
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\t"
+                 "v_add_f32 %0, %1, %2\n\t"
+                 "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+                 : "=v"(y)
+                 : "v"(c), "v"(h));
+    return fabsf(v) < 2147483648.f ? y : -127.f;
 }
 
 __device__ __forceinline__ float apply_activation(float v, const ncnnhip_activation& a)

@@ -352,23 +352,32 @@ def test_vnni_cpu_baseline_equals_the_scalar_oracle(m, n, k, per_col):
 
 
 def test_float_pipe_formulation_of_float2int8_equals_the_oracle():
-    """The convolution epilogue rounds without leaving the float pipe (trunc + exact remainder test, max/min clamp,
-    one compare-select for |v| >= 2^31).  The same IEEE operations in numpy float32 must give float2int8's value on
-    ties, near-ties, the clamp edges, huge values, infinities and NaN, and on a dense random sample."""
+    """The device rounds without leaving the float pipe: clamp to [-127, 127], add copysign(0.5) with the add rounded
+    TOWARD ZERO, truncate; one compare-select for NaN and |v| >= 2^31.  The same operations evaluated here (the add
+    exactly in float64, then rounded toward zero to float32) must give float2int8's value on ties, near-ties, the clamp
+    edges, huge values, infinities and NaN, and on a dense random sample -- and the nearest-even add it replaces must
+    fail on 0.49999997, which is why the rounding mode matters."""
     rng = np.random.default_rng(7)
     ks = np.arange(-300, 301, dtype=np.float64)
     ties = np.concatenate([ks + 0.5, np.nextafter((ks + 0.5).astype(F), F(np.inf)), np.nextafter((ks + 0.5).astype(F), F(-np.inf))]).astype(F)
     special = np.array([0.0, -0.0, 0.49999997, -0.49999997, 126.5, -126.5, 127.49, -127.49, 127.5, -127.5, 200, -200, 2147483520.0, 2147483648.0,
                         -2147483648.0, 4e9, -4e9, 1e30, -1e30, np.inf, -np.inf, np.nan, 8388607.5, -8388607.5, 1e-40, -1e-40], F)
     v = np.concatenate([ties, special, rng.normal(0, 60, 200000).astype(F), rng.uniform(-130, 130, 200000).astype(F)])
-    with np.errstate(invalid="ignore"):
-        t = np.trunc(v)
-        d = (v - t).astype(F)
-        r = (t + np.where(np.abs(d) >= F(0.5), np.copysign(F(1), v), F(0))).astype(F)
-        r = np.fmin(np.fmax(r, F(-127)), F(127))          # device fmaxf/fminf: a NaN operand yields the other one
-        got = np.where(np.abs(v) < F(2147483648.0), r, F(-127))
+
+    def formulation(toward_zero):
+        with np.errstate(invalid="ignore"):
+            c = np.where(np.isnan(v), F(0), np.clip(v, F(-127), F(127))).astype(F)  # a NaN is overridden below
+            exact = c.astype(np.float64) + np.copysign(0.5, c.astype(np.float64))   # exact: both fit in 53 bits
+            y = exact.astype(F)                                                     # nearest even
+            if toward_zero:
+                y = np.where(np.abs(y.astype(np.float64)) > np.abs(exact), np.nextafter(y, F(0)), y).astype(F)
+            r = np.trunc(y)
+            return np.where(np.abs(v) < F(2147483648.0), r, F(-127))
+
     want = oracle.float2int8(v).astype(F)
-    assert np.array_equal(got, want)
+    assert np.array_equal(formulation(True), want)
+    wrong = formulation(False) != want
+    assert wrong.any() and wrong[np.flatnonzero(v == F(0.49999997))[0]]
 
 
 # ---- attention with block-quantised weights (src/layer/multiheadattention.cpp:561-912) ---------------------------------
