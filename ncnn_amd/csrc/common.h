@@ -92,6 +92,27 @@ __device__ __forceinline__ float float2int8_as_float(float v)
     return fabsf(v) < 2147483648.f ? y : -127.f;
 }
 
+// four at a time: one switch of the rounding mode and back for four adds
+__device__ __forceinline__ void float2int8_as_float_x4(float& v0, float& v1, float& v2, float& v3)
+{
+    const float c0 = __builtin_amdgcn_fmed3f(v0, -127.f, 127.f), c1 = __builtin_amdgcn_fmed3f(v1, -127.f, 127.f);
+    const float c2 = __builtin_amdgcn_fmed3f(v2, -127.f, 127.f), c3 = __builtin_amdgcn_fmed3f(v3, -127.f, 127.f);
+    const float h0 = copysignf(0.5f, c0), h1 = copysignf(0.5f, c1), h2 = copysignf(0.5f, c2), h3 = copysignf(0.5f, c3);
+    float y0, y1, y2, y3;
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\t"
+                 "v_add_f32 %0, %4, %8\n\t"
+                 "v_add_f32 %1, %5, %9\n\t"
+                 "v_add_f32 %2, %6, %10\n\t"
+                 "v_add_f32 %3, %7, %11\n\t"
+                 "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+                 : "=&v"(y0), "=&v"(y1), "=&v"(y2), "=&v"(y3)
+                 : "v"(c0), "v"(c1), "v"(c2), "v"(c3), "v"(h0), "v"(h1), "v"(h2), "v"(h3));
+    v0 = fabsf(v0) < 2147483648.f ? y0 : -127.f;
+    v1 = fabsf(v1) < 2147483648.f ? y1 : -127.f;
+    v2 = fabsf(v2) < 2147483648.f ? y2 : -127.f;
+    v3 = fabsf(v3) < 2147483648.f ? y3 : -127.f;
+}
+
 __device__ __forceinline__ float apply_activation(float v, const ncnnhip_activation& a)
 {
     switch (a.type)

@@ -341,6 +341,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
             for (int c = 0; c < TN; c++)
             {
                 if (col0 + wn * CW + c * 32 >= col_limit) continue; // a whole 32-channel block of tile padding (uniform per wavefront)
+                float fr[16];
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                 {
@@ -355,10 +356,19 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                     }
                     else if (ACT != 0)
                         f = apply_activation(f, epi.act);
-                    if (to_int8) f = float2int8_as_float(mul_rn(f, s_out[c]));
+                    fr[r] = to_int8 ? mul_rn(f, s_out[c]) : f;
+                }
+                if (to_int8)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; r += 4) float2int8_as_float_x4(fr[r], fr[r + 1], fr[r + 2], fr[r + 3]);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                {
                     // pad channels carry zero scales and bias: with no activation or ReLU they are zero already
-                    if (ACT != 0 && ACT != 1 && !real[c]) f = 0.f;
-                    tile[(8 * (r >> 2) + 4 * lhi + (r & 3)) * LD + c * 32 + l32] = f;
+                    if (ACT != 0 && ACT != 1 && !real[c]) fr[r] = 0.f;
+                    tile[(8 * (r >> 2) + 4 * lhi + (r & 3)) * LD + c * 32 + l32] = fr[r];
                 }
             }
             __syncthreads();
@@ -413,8 +423,10 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                         {
                             v4f q;
 #pragma unroll
-                            for (int e = 0; e < 4; e++) q[e] = float2int8_as_float(mul_rn(v[e], fusion.q8_scale));
-                            *reinterpret_cast<uint32_t*>(fusion.q8_out + o) = pack4(q);
+                            for (int e = 0; e < 4; e++) q[e] = mul_rn(v[e], fusion.q8_scale);
+                            float q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
+                            float2int8_as_float_x4(q0, q1, q2, q3);
+                            *reinterpret_cast<uint32_t*>(fusion.q8_out + o) = pack4(v4f{q0, q1, q2, q3});
                         }
                     }
                 }

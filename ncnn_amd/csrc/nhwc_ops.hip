@@ -522,9 +522,12 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
             float v = mul_rn((float)acc[o][e], s_in[e]);
             if (bias) v = add_rn(v, s_b[e]);
             v = apply_activation(v, act);
-            if (!g.out_f32) v = float2int8_as_float(mul_rn(v, s_out[e]));
-            f[e] = (int)q0 + e < g.c ? v : 0.f;
+            f[e] = g.out_f32 ? v : mul_rn(v, s_out[e]);
         }
+        if (!g.out_f32) float2int8_as_float_x4(f[0], f[1], f[2], f[3]);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if ((int)q0 + e >= g.c) f[e] = 0.f;
         if (g.out_f32)
             *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
         else
