@@ -39,7 +39,7 @@ __device__ __forceinline__ float to_f32(__half v)
 // ---- 8-bit weights, K % 16 == 0, 16-byte aligned rows ------------------------------------
 // Streaming kernel for up to MT activation rows at a time.
 //   * the activations (times the optional input scales) are staged once per workgroup in LDS as
-//     fp32, in K tiles of KT = 16384 / MT values;
+//     fp32, in K tiles of KT = 8192 / MT values;
 //   * every wavefront owns R consecutive weight rows; per row each lane fetches 16-byte chunks
 //     lane, lane+64, ... of the K tile, U chunks per batch, and all R*U 16-byte loads of a batch
 //     are issued before the first one is consumed, which is what keeps enough bytes in flight to
@@ -48,6 +48,15 @@ __device__ __forceinline__ float to_f32(__half v)
 //     are summed first and the block's 1/scale is applied once per chunk.
 // BITS = 4 / 6 / 8: a chunk is always 16 weights, i.e. 8 / 12 / 16 bytes of the LSB-first field stream
 // (src/layer/gemm.cpp:318-336); a field is pulled out of its dword pair with one funnel shift + one signed bit-field extract.
+#ifndef BQ_R
+#define BQ_R 2
+#endif
+#ifndef BQ_U
+#define BQ_U 2 // chunks per row and batch; with 32 KB of LDS this keeps three workgroups on a CU (measured over R 1..4, U 1..4, 16/32/64 KB)
+#endif
+#ifndef BQ_KT
+#define BQ_KT 8192
+#endif
 template<int BITS>
 __device__ __forceinline__ v4i_bq load_chunk(const uint8_t* p)
 {
@@ -86,7 +95,7 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
                                                                   const float* __restrict__ c, int bt, float alpha, float beta,
                                                                   float* __restrict__ out, size_t out_stride)
 {
-    constexpr int KT = 16384 / MT;
+    constexpr int KT = BQ_KT / MT; // activation tile in LDS: BQ_KT floats
     __shared__ __attribute__((aligned(16))) float lds_a[MT * KT];
 
     const int lane = threadIdx.x & 63;
@@ -112,12 +121,17 @@ __global__ __launch_bounds__(256) void blockquant8_stream_kernel(const AT* __res
 #pragma unroll
             for (int u = 0; u < U; u++)
             {
+                // unconditional loads from clamped addresses, zeros selected afterwards: a guarded load becomes a branch,
+                // and past a branch the compiler waits for every load in flight
                 const int ch = c0 + u * 64 + lane;
                 const int j = j0 + r;
                 const bool ok = ch < nch && j < N;
-                const size_t koff = (size_t)kt0 + ((size_t)ch << 4);
-                w[r][u] = ok ? load_chunk<BITS>(b + (size_t)j * row_bytes + koff * BITS / 8) : v4i_bq{0, 0, 0, 0};
-                d[r][u] = ok ? scales[(size_t)j * nblk + (koff >> block_shift)] : 1.f;
+                const size_t jc = (size_t)(j < N ? j : N - 1);
+                const size_t koff = (size_t)kt0 + ((size_t)(ch < nch ? ch : 0) << 4);
+                v4i_bq wv = load_chunk<BITS>(b + jc * row_bytes + koff * BITS / 8);
+                if (!ok) wv = v4i_bq{0, 0, 0, 0};
+                w[r][u] = wv;
+                d[r][u] = scales[jc * nblk + (koff >> block_shift)];
             }
     };
     auto compute_batch = [&](int kt0, int c0, const v4i_bq (&w)[R][U], const float (&d)[R][U]) {
@@ -291,10 +305,7 @@ static int launch_blockquant8(const AT* a, size_t a_stride, int M, int N, int K,
 {
     const int shift = block == 32 ? 5 : block == 64 ? 6 : 7;
     const int nblk = (K + block - 1) / block;
-#ifndef BQ_R
-#define BQ_R 2
-#endif
-    constexpr int R = BQ_R, U = 4;
+    constexpr int R = BQ_R, U = BQ_U;
     dim3 grid(ceil_div(N, 4 * R));
     for (int m0 = 0; m0 < M;)
     {
@@ -489,7 +500,7 @@ __global__ __launch_bounds__(256) void blockquant_generic_kernel(const float* __
 // columns = activation rows.  Integer-valued q times an fp16 activation is exact in fp32, so the
 // only roundings are the fp32 accumulation and the one multiply by 1/scale per K block.
 #ifndef BQ_MFMA_U
-#define BQ_MFMA_U 2
+#define BQ_MFMA_U 1 // NS x U = 4 x 1: ~100 VGPRs, four wavefronts per SIMD (measured best of 2..8 x 1..4; see the load_batch comment)
 #endif
 #ifndef BQ_MFMA_NS
 #define BQ_MFMA_NS 4
@@ -536,11 +547,10 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
     const int kb_begin = wave * per_wave;
     const int kb_end = kb_begin + per_wave < kblocks ? kb_begin + per_wave : kblocks;
     const int nkb = kb_end > kb_begin ? kb_end - kb_begin : 0;
-    auto block_of = [&](int i) { return kb_begin + i; }; // i-th block this wave processes
+    auto block_of = [&](int i) { return kb_begin + i; }; // i-th block this wave processes (callers pass i < nkb, else block 0)
 
     const v4i_bq* wt = wpk + ((size_t)tile * kblocks) * 64 + lane;
     const __half* arow = a + (size_t)(m < M ? m : 0) * a_stride + kg * 16;
-    const bool a_live = m < M;
 
     // Requests are issued in the order their data is consumed (loads return in order): the tile's
     // descales, then per batch the activations (L2) followed by the weights (the HBM stream).  NS
@@ -551,22 +561,36 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
     {
         v4i_bq w[U], a0[U], a1[U];
     };
+    // Every load is unconditional (a guarded load becomes a branch, and after a branch the compiler waits for ALL loads in
+    // flight, which empties the ring every step): a batch beyond the range re-reads the wave's first block and is cancelled
+    // by a zero descale; a lane whose 16-half chunk lies beyond K (only when K % 64 != 0) reads chunk 0 and selects zeros;
+    // lanes of activation rows >= M read row 0 and their results are never stored.
     auto load_batch = [&](int kb0, Batch& bt_) {
 #pragma unroll
         for (int u = 0; u < U; u++)
         {
             const bool live = kb0 + u < nkb;
-            const int kb = block_of(live ? kb0 + u : 0);
-            const bool aok = live && a_live && kb * 64 + kg * 16 < K; // K % 16 == 0: a 16-half chunk is all in or all out
-            bt_.a0[u] = aok ? *reinterpret_cast<const v4i_bq*>(arow + (size_t)kb * 64) : v4i_bq{0, 0, 0, 0};
-            bt_.a1[u] = aok ? *reinterpret_cast<const v4i_bq*>(arow + (size_t)kb * 64 + 8) : v4i_bq{0, 0, 0, 0};
+            const int kb = live ? block_of(kb0 + u) : 0;
+            const bool aok = kb * 64 + kg * 16 < K; // K % 16 == 0: a 16-half chunk is all in or all out
+            const __half* ap = arow + (aok ? (size_t)kb * 64 : (size_t)0) - (aok ? 0 : kg * 16);
+            bt_.a0[u] = *reinterpret_cast<const v4i_bq*>(ap);
+            bt_.a1[u] = *reinterpret_cast<const v4i_bq*>(ap + 8);
+            if (K & 63)
+            {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                {
+                    bt_.a0[u][e] = aok ? bt_.a0[u][e] : 0;
+                    bt_.a1[u][e] = aok ? bt_.a1[u][e] : 0;
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; u++)
         {
             const bool live = kb0 + u < nkb;
-            const int kb = block_of(live ? kb0 + u : 0);
-            bt_.w[u] = live ? wt[(size_t)kb * 64] : v4i_bq{(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+            const int kb = live ? block_of(kb0 + u) : 0;
+            bt_.w[u] = wt[(size_t)kb * 64];
         }
     };
     v4f acc = {0.f, 0.f, 0.f, 0.f};
@@ -575,7 +599,7 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
         for (int u = 0; u < U; u++)
         {
             const bool live = kb0 + u < nkb;
-            const int kb = block_of(live ? kb0 + u : 0);
+            const int kb = live ? block_of(kb0 + u) : 0;
             const v8h wa = bytes_to_halves(bt_.w[u][0], bt_.w[u][1]);
             const v8h wb = bytes_to_halves(bt_.w[u][2], bt_.w[u][3]);
             union
@@ -588,7 +612,8 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
             v4f t = {0.f, 0.f, 0.f, 0.f};
             t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, t, 0, 0, 0);
             t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
-            const float4 d = live ? lds_d[kb * 4 + kg] : make_float4(0.f, 0.f, 0.f, 0.f);
+            float4 d = lds_d[kb * 4 + kg];
+            if (!live) d = make_float4(0.f, 0.f, 0.f, 0.f); // a select, not a branch
             acc[0] = fmaf(t[0], d.x, acc[0]);
             acc[1] = fmaf(t[1], d.y, acc[1]);
             acc[2] = fmaf(t[2], d.z, acc[2]);
