@@ -505,6 +505,9 @@ __global__ __launch_bounds__(256) void blockquant_generic_kernel(const float* __
 #ifndef BQ_MFMA_NS
 #define BQ_MFMA_NS 4
 #endif
+#ifndef BQ_MFMA_NS_LDS
+#define BQ_MFMA_NS_LDS 4 // ring depth when the activations are staged in LDS (4..12 measured)
+#endif
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -528,7 +531,10 @@ __device__ __forceinline__ v8h bytes_to_halves(int lo, int hi)
     return t.h8;
 }
 
-template<int NS, int U>
+// LDSA: the (few) activation rows are staged once per workgroup in LDS, zero-filled to a multiple of 64, instead of
+// travelling with every batch in registers: a batch is then 4 VGPRs per block and the ring can be twice as deep at the same
+// occupancy.  Used while M rows of K halves fit in 16 KB (decoding: M = 1..4) and there are many tiles.
+template<int NS, int U, bool LDSA>
 __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
                                                                 const v4i_bq* __restrict__ wpk, const float4* __restrict__ dpk,
                                                                 const float* __restrict__ c, int bt, float alpha, float beta,
@@ -559,8 +565,10 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
     // bytes land.
     struct Batch
     {
-        v4i_bq w[U], a0[U], a1[U];
+        v4i_bq w[U], a0[LDSA ? 1 : U], a1[LDSA ? 1 : U];
     };
+    const int Kp = kblocks * 64;
+    const __half* lds_act = reinterpret_cast<const __half*>(lds_d + (size_t)kblocks * 4) + (size_t)(m < M ? m : 0) * Kp + kg * 16;
     // Every load is unconditional (a guarded load becomes a branch, and after a branch the compiler waits for ALL loads in
     // flight, which empties the ring every step): a batch beyond the range re-reads the wave's first block and is cancelled
     // by a zero descale; a lane whose 16-half chunk lies beyond K (only when K % 64 != 0) reads chunk 0 and selects zeros;
@@ -571,17 +579,18 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
         {
             const bool live = kb0 + u < nkb;
             const int kb = live ? block_of(kb0 + u) : 0;
+            if (LDSA) continue; // activations wait in LDS
             const bool aok = kb * 64 + kg * 16 < K; // K % 16 == 0: a 16-half chunk is all in or all out
             const __half* ap = arow + (aok ? (size_t)kb * 64 : (size_t)0) - (aok ? 0 : kg * 16);
-            bt_.a0[u] = *reinterpret_cast<const v4i_bq*>(ap);
-            bt_.a1[u] = *reinterpret_cast<const v4i_bq*>(ap + 8);
+            bt_.a0[LDSA ? 0 : u] = *reinterpret_cast<const v4i_bq*>(ap);
+            bt_.a1[LDSA ? 0 : u] = *reinterpret_cast<const v4i_bq*>(ap + 8);
             if (K & 63)
             {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                 {
-                    bt_.a0[u][e] = aok ? bt_.a0[u][e] : 0;
-                    bt_.a1[u][e] = aok ? bt_.a1[u][e] : 0;
+                    bt_.a0[LDSA ? 0 : u][e] = aok ? bt_.a0[LDSA ? 0 : u][e] : 0;
+                    bt_.a1[LDSA ? 0 : u][e] = aok ? bt_.a1[LDSA ? 0 : u][e] : 0;
                 }
             }
         }
@@ -607,8 +616,16 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
                 v4i_bq i;
                 v8h h;
             } xa, xb;
-            xa.i = bt_.a0[u];
-            xb.i = bt_.a1[u];
+            if (LDSA)
+            {
+                xa.i = *reinterpret_cast<const v4i_bq*>(lds_act + (size_t)kb * 64);
+                xb.i = *reinterpret_cast<const v4i_bq*>(lds_act + (size_t)kb * 64 + 8);
+            }
+            else
+            {
+                xa.i = bt_.a0[LDSA ? 0 : u];
+                xb.i = bt_.a1[LDSA ? 0 : u];
+            }
             v4f t = {0.f, 0.f, 0.f, 0.f};
             t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, t, 0, 0, 0);
             t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
@@ -634,6 +651,17 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
     for (int i = 0; i < 4; i++)
         if (threadIdx.x + i * 256 < nd) lds_d[threadIdx.x + i * 256] = dreg[i];
     for (int i = threadIdx.x + 1024; i < nd; i += 256) lds_d[i] = dt[i]; // K beyond 16384
+    if (LDSA)
+    {
+        // M rows of Kp halves, 16 bytes per thread and step; beyond K zeros (K % 16 == 0: a vector is all in or all out)
+        v4i_bq* la = reinterpret_cast<v4i_bq*>(lds_d + (size_t)kblocks * 4);
+        const int vec_per_row = Kp / 8;
+        for (int i = threadIdx.x; i < M * vec_per_row; i += 256)
+        {
+            const int row = i / vec_per_row, v = i - row * vec_per_row;
+            la[i] = v * 8 < K ? *reinterpret_cast<const v4i_bq*>(a + (size_t)row * a_stride + v * 8) : v4i_bq{0, 0, 0, 0};
+        }
+    }
     __syncthreads();
     for (int kb0 = 0; kb0 < nkb; kb0 += NS * U)
     {
@@ -791,9 +819,15 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
         const float* cc = c_dev;
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
-        hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS, BQ_MFMA_U>), dim3(tiles), dim3(256), (size_t)kblocks * 64, as_stream(stream), ah + (size_t)m0 * a_stride, a_stride, mc, N, K,
-                           kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev), reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha,
-                           beta, out_dev + (size_t)m0 * out_stride, out_stride);
+        const size_t act_bytes = (size_t)mc * kblocks * 64 * sizeof(__half);
+        if (act_bytes <= 16384 && tiles >= 512) // measured: pays from about 8192 weight rows, not for long rows (K = 11008) or few tiles
+            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS_LDS, 1, true>), dim3(tiles), dim3(256), (size_t)kblocks * 64 + act_bytes, as_stream(stream),
+                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),
+                               reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride);
+        else
+            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS, BQ_MFMA_U, false>), dim3(tiles), dim3(256), (size_t)kblocks * 64, as_stream(stream),
+                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),
+                               reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride);
     }
     return launch_status("blockquant8_mfma_kernel");
 }
