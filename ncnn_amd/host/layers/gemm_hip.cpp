@@ -100,6 +100,10 @@ int Gemm_hip::load_param(const ParamDict& pd)
     }
     // one bottom blob is enough when two of the three operands are constants
     if (constantA + constantB + constantC == 2) one_blob_only = true;
+    // blobs stay in HBM for the form a network layer has: A is the only input, B (and C, if any) are constants, nothing
+    // is transposed on the way in or out.  Every other form takes host Mats as before.
+    support_hip = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottoms.size() == 1
+                  && (quantize_term != 0);
     return 0;
 }
 
@@ -200,6 +204,8 @@ int Gemm_hip::create_pipeline(const Option&)
             if (ret == 0) b_ready_int8 = 1;
         }
     }
+    // the device-resident form needs B ready on the device (int8 rows or block-quantised fields)
+    support_hip = support_hip && ret == 0 && (weight_block_quantize || b_ready_int8);
     if (ret != 0) destroy_pipeline(Option());
     return ret;
 }
@@ -228,6 +234,68 @@ int Gemm_hip::forward(const std::vector<Mat>& bottom_blobs, std::vector<Mat>& to
 {
     if (weight_block_quantize) return forward_block_quantize(bottom_blobs, top_blobs, opt);
     return forward_int8(bottom_blobs, top_blobs, opt);
+}
+
+int Gemm_hip::forward_hip(const HipMat& bottom_blob, HipMat& top_blob, HipCommand& cmd, const Option& opt) const
+{
+    std::vector<HipMat> ins(1, bottom_blob), outs(1);
+    int ret = forward_hip(ins, outs, cmd, opt);
+    top_blob = outs[0];
+    return ret;
+}
+
+int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option&) const
+{
+    if (bottom_blobs.size() != 1 || top_blobs.empty() || !d_B) return -1;
+    const HipMat& A = bottom_blobs[0];
+    if (A.elemsize != 4u || (A.dims != 1 && A.dims != 2))
+    {
+        NCNN_LOGE("Gemm %s: the device-resident form takes a 1-D or 2-D fp32 blob", name.c_str());
+        return -1;
+    }
+    // a batch of 2-D blobs is n*h rows; a 1-D blob is one row per sample
+    const int M = A.dims == 2 ? A.n * A.h : A.n, K = A.w, N = constantN;
+    if (K != constantK)
+    {
+        NCNN_LOGE("Gemm %s: K mismatch (%d vs constant %d)", name.c_str(), K, constantK);
+        return -1;
+    }
+    const float* d_c = constantC && !C_data.empty() && constant_broadcast_type_C >= 0 ? (const float*)d_C : 0;
+    const int bt = d_c ? constant_broadcast_type_C : -1;
+    if (A.n > 1 && (bt == 1 || bt == 2 || bt == 3))
+    {
+        NCNN_LOGE("Gemm %s: a per-row C does not extend to a batch", name.c_str());
+        return -1;
+    }
+    HipMat& top = top_blobs[0];
+    if (A.dims == 2)
+        top.create(N, A.h, 4u, A.n, &cmd);
+    else
+        top.create(N, 4u, A.n, &cmd);
+    if (top.empty()) return -100;
+    void* st = cmd.stream;
+    int rc = 0;
+    if (weight_block_quantize)
+    {
+        rc = ncnnhip_gemm_blockquant((const float*)A.data, (size_t)K, M, N, K, (const uint8_t*)d_B, term_bits(quantize_term), term_block(quantize_term),
+                                     (const float*)d_B_block_scales, (const float*)d_B_input_scales, d_c, bt, alpha, beta, (float*)top.data, (size_t)N, st);
+        return to_ncnn_status(rc, "ncnnhip_gemm_blockquant");
+    }
+    if (!b_ready_int8)
+    {
+        NCNN_LOGE("Gemm %s: constant B is not int8 on the device", name.c_str());
+        return -1;
+    }
+    ScopedScratch scratch(&cmd);
+    const size_t aq_stride = alignSize((size_t)K, 16);
+    void* q = scratch.get((size_t)M * aq_stride);
+    void* sa = scratch.get((size_t)M * 4);
+    if (!q || !sa) return -100;
+    rc = ncnnhip_gemm_quantize_rows((const float*)A.data, (size_t)K, M, K, (int8_t*)q, aq_stride, (float*)sa, st);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_quantize_rows");
+    rc = ncnnhip_gemm_int8((const int8_t*)q, aq_stride, (const int8_t*)d_B, (size_t)K, M, N, K, (const float*)sa, (const float*)d_B_scale, 1, d_c, bt, alpha, beta, 0,
+                           (float*)top.data, (size_t)N, 0, st);
+    return to_ncnn_status(rc, "ncnnhip_gemm_int8");
 }
 
 // rows / row stride of a matrix held in a Mat: 2-D (h rows of w) or 3-D with h == 1 (c rows, cstep apart)

@@ -101,6 +101,10 @@ public:
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
+    // device-resident form for the shape a network layer has: one dynamic A (rows of K floats), constant B, constant or no C
+    virtual int forward_hip(const std::vector<ncnn::HipMat>& bottom_blobs, std::vector<ncnn::HipMat>& top_blobs, ncnn::HipCommand& cmd,
+                            const ncnn::Option& opt) const;
+    virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
 
 public:
     float alpha, beta;

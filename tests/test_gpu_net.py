@@ -136,15 +136,16 @@ def test_int8_inference_switched_off_is_an_error_not_a_fallback():
 
 
 # ----------------------------------------------------------------------------- single layers through the boundary
-def _single(param_lines, blob, feeds, out):
-    net = _load(mw.assemble_param(param_lines), blob)
+def _single(param_lines, blob, feeds, out, resident=False):
+    net = _load(mw.assemble_param(param_lines), blob, resident)
     ex = net.create_extractor()
     for k, v in feeds.items():
         ex.input(k, v)
     return ex.extract(out)
 
 
-def test_gemm_layer_int8_constant_b_with_bias():
+@RESIDENT
+def test_gemm_layer_int8_constant_b_with_bias(resident):
     rng = np.random.default_rng(4)
     m, n, k = 37, 50, 96
     a = rng.standard_normal((m, k), dtype=F)
@@ -154,7 +155,7 @@ def test_gemm_layer_int8_constant_b_with_bias():
     lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m),
              mw.gemm_param("g", ["a"], "out", M=0, N=n, K=k, constantB=1, constantC=1, broadcast_type_C=4, quantize_term=2)]
     blob = mw.weight_blob(bq) + mw.weight_blob(c) + mw.raw_f32(sb)
-    got = _single(lines, blob, {"a": a}, "out")
+    got = _single(lines, blob, {"a": a}, "out", resident)
     aq, sa = oracle.gemm_quantize_rows(a)
     assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, [sb], c, 4))
 
@@ -173,8 +174,9 @@ def test_gemm_layer_int8_two_dynamic_operands_transposed_output():
     assert np.array_equal(got, want)
 
 
+@RESIDENT
 @pytest.mark.parametrize("bits,block,insc", [(8, 64, 0), (4, 32, 1), (6, 128, 0)])
-def test_gemm_layer_block_quant(bits, block, insc):
+def test_gemm_layer_block_quant(bits, block, insc, resident):
     import npref
     rng = np.random.default_rng(bits)
     m, n, k = 4, 24, 200
@@ -185,7 +187,7 @@ def test_gemm_layer_block_quant(bits, block, insc):
     term = bits * 100 + insc * 10 + {32: 0, 64: 1, 128: 2}[block]
     lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m), mw.gemm_param("g", ["a"], "out", N=n, K=k, constantB=1, quantize_term=term)]
     blob = mw.weight_blob(packed.view(np.int8)) + mw.raw_f32(scales) + (mw.raw_f32(ins) if insc else b"")
-    got = _single(lines, blob, {"a": a}, "out")
+    got = _single(lines, blob, {"a": a}, "out", resident)
     val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins)
     assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
 
