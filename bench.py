@@ -544,16 +544,24 @@ def bench_net(args, which, batch):
         ex.input_resident("data", xin)
         return ex, ex.extract_resident(out_name)
 
+    # --streams N keeps the last N Extractors alive, so N passes are in flight on N of the net's streams (each live
+    # Extractor borrows its own command); 1 = one pass after the other on one stream
+    ring = [None] * max(1, args.streams)
     ex = None
-    for _ in range(args.warmup):
+    for i in range(args.warmup):
         ex, out = step()
-    if ex is not None:
-        ex.synchronize()
+        ring[i % len(ring)] = ex
+    for e in ring:
+        if e is not None:
+            e.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
         ex, out = step()
+        ring[i % len(ring)] = ex
     enqueue = time.perf_counter() - t0  # the host is done describing the work; the GPU may still be running it
-    ex.synchronize()
+    for e in ring:
+        if e is not None:
+            e.synchronize()
     wall = time.perf_counter() - t0
     logits = (graph.output() if graph is not None else out).to_numpy()
     if not np.isfinite(logits).all():
@@ -566,7 +574,8 @@ def bench_net(args, which, batch):
         "config": {"workload": "%s-shaped int8 model (%d layers, %d quantised), whole forward pass through Net/Extractor with device-resident blobs, batch %d"
                                % (which, len(g.layers), len(rows), batch),
                    "images_per_s": batch / (ms_per_step * 1e-3), "host_enqueue_ms_per_step": enqueue * 1e3 / args.steps,
-                   "submission": "recorded pass replayed as one graph launch" if graph is not None else "layer by layer through an Extractor"},
+                   "submission": "recorded pass replayed as one graph launch" if graph is not None else "layer by layer through an Extractor",
+                   "passes_in_flight": len(ring)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": None, "kernel": "whole pass (conv_nhwc_kernel dominates)", "ops_per_launch": ops},
     }
@@ -581,6 +590,7 @@ def main():
                     help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
+    ap.add_argument("--streams", type=int, default=1, help="net workloads: forward passes kept in flight, each on its own stream of the net")
     ap.add_argument("--graph", type=int, default=0,
                     help="net workloads: 0 = one Extractor per pass, layer by layer on a stream (faster on this ROCm: a replayed graph costs more per kernel node "
                          "on the GPU than a stream launch does); 1 = replay the recorded pass (HipGraph), which takes the host out of the loop")
