@@ -421,7 +421,18 @@ def bench_layers(args, which, batch):
                 plan["d_x"] = rt.up(rng.uniform(-1, 1, (batch, h * w, cp(c))).astype(np.float32))
                 plan["d_s"] = rt.up(np.array([100.0], np.float32))
             taps = r["k"] * r["k"]
-            if r["group"] == 1:
+            if r["group"] == 1 and lib.ncnnhip_conv_stem_supported(C.byref(desc)):
+                # at most 4 input channels: the narrow-input form the layer takes inside a net (fp32 image at 4 floats per pixel,
+                # quantised into the bordered 4-byte-per-pixel image, 4 neighbouring pixels per K chunk)
+                ib, wb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
+                check(lib.ncnnhip_conv_stem_sizes(C.byref(desc), C.byref(ib), C.byref(wb), C.byref(sb)))
+                wq = rng.integers(-127, 128, cout * c * taps).astype(np.int8)
+                pk = np.empty(wb.value, np.int8)
+                check(lib.ncnnhip_conv_stem_pack_weights(C.byref(desc), wq.ctypes.data, pk.ctypes.data))
+                plan.update(kind="stem", d_pk=rt.up(pk), d_ws=ncnn_amd.DeviceBuffer.zeros(sb.value, st), ws_bytes=sb.value,
+                            d_img=ncnn_amd.DeviceBuffer.zeros(ib.value, st), d_x=rt.up(rng.uniform(-1, 1, (batch, h * w, 4)).astype(np.float32)),
+                            d_s=rt.up(np.array([100.0], np.float32)))
+            elif r["group"] == 1:
                 nb, wb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
                 check(lib.ncnnhip_conv_nhwc_sizes(C.byref(desc), C.byref(nb), C.byref(wb), C.byref(sb)))
                 wq = rng.integers(-127, 128, cout * c * taps).astype(np.int8)
@@ -445,6 +456,13 @@ def bench_layers(args, which, batch):
                 check(lib.ncnnhip_quantize(p["d_x"].ptr, p["k"], 0, p["d_xq"].ptr, p["k"], 0, batch, p["k"], 1, p["d_s"].ptr, 1, st))
             check(lib.ncnnhip_innerproduct_int8_ws(p["d_xq"].ptr, p["k"], batch, p["k"], p["n"], p["d_w"].ptr, p["d_si"].ptr, p["d_b"].ptr,
                                                    Activation.make(0), p["d_out"].ptr, p["n"], p["d_ws"].ptr, p["ws_bytes"], st))
+            return
+        so = p["d_so"].ptr if p["d_so"] else None
+        if p["kind"] == "stem":
+            if prepass:
+                check(lib.ncnnhip_quantize_stem(C.byref(p["desc"]), p["d_x"].ptr, 4, 4, p["d_s"].ptr, p["d_img"].ptr, st))
+            check(lib.ncnnhip_conv_int8_stem(C.byref(p["desc"]), p["d_img"].ptr, p["d_pk"].ptr, p["d_si"].ptr, p["d_b"].ptr, so, p["act"], p["d_out"].ptr, None,
+                                             p["d_ws"].ptr, p["ws_bytes"], st))
             return
         if prepass and not r["int8_in"]:
             check(lib.ncnnhip_quantize_nhwc(p["d_x"].ptr, p["d_xq"].ptr, p["npix"], r["in_shape"][0], p["d_s"].ptr, 1, st))
