@@ -113,6 +113,58 @@ __device__ __forceinline__ void float2int8_as_float_x4(float& v0, float& v1, flo
     v3 = fabsf(v3) < 2147483648.f ? y3 : -127.f;
 }
 
+// Clip (activation type 3) for a value known not to be NaN.  The reference writes `if (v < lo) v = lo; if (v > hi)
+// v = hi;` (src/layer/fused_activation.h:25-33); for every v that is finite or infinite, and any lo and hi (a NaN bound
+// leaves v alone in both forms, lo > hi ends at hi in both), max-then-min gives the same value.
+__device__ __forceinline__ float clip_not_nan(float v, float lo, float hi)
+{
+    return fminf(fmaxf(v, lo), hi);
+}
+
+// float2int8_as_float_x4 for values the caller knows to lie inside (-2^31, 2^31): the out-of-range answer of -127
+// cannot occur, so the compare and select that produce it are left out.  [lo, hi] is the clamp, inside [-127, 127]:
+// a narrower one folds a preceding clip into it (see clip_folds_into_requantise).
+__device__ __forceinline__ void float2int8_as_float_bounded_x4(float& v0, float& v1, float& v2, float& v3, float lo = -127.f, float hi = 127.f)
+{
+    const float c0 = __builtin_amdgcn_fmed3f(v0, lo, hi), c1 = __builtin_amdgcn_fmed3f(v1, lo, hi);
+    const float c2 = __builtin_amdgcn_fmed3f(v2, lo, hi), c3 = __builtin_amdgcn_fmed3f(v3, lo, hi);
+    const float h0 = copysignf(0.5f, c0), h1 = copysignf(0.5f, c1), h2 = copysignf(0.5f, c2), h3 = copysignf(0.5f, c3);
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\t"
+                 "v_add_f32 %0, %4, %8\n\t"
+                 "v_add_f32 %1, %5, %9\n\t"
+                 "v_add_f32 %2, %6, %10\n\t"
+                 "v_add_f32 %3, %7, %11\n\t"
+                 "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+                 : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+                 : "v"(c0), "v"(c1), "v"(c2), "v"(c3), "v"(h0), "v"(h1), "v"(h2), "v"(h3));
+}
+
+// the same with one clamp per value (four different channels)
+__device__ __forceinline__ void float2int8_as_float_bounded_lanes_x4(float& v0, float& v1, float& v2, float& v3, const float (&lo)[4], const float (&hi)[4])
+{
+    const float c0 = __builtin_amdgcn_fmed3f(v0, lo[0], hi[0]), c1 = __builtin_amdgcn_fmed3f(v1, lo[1], hi[1]);
+    const float c2 = __builtin_amdgcn_fmed3f(v2, lo[2], hi[2]), c3 = __builtin_amdgcn_fmed3f(v3, lo[3], hi[3]);
+    const float h0 = copysignf(0.5f, c0), h1 = copysignf(0.5f, c1), h2 = copysignf(0.5f, c2), h3 = copysignf(0.5f, c3);
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\t"
+                 "v_add_f32 %0, %4, %8\n\t"
+                 "v_add_f32 %1, %5, %9\n\t"
+                 "v_add_f32 %2, %6, %10\n\t"
+                 "v_add_f32 %3, %7, %11\n\t"
+                 "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+                 : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+                 : "v"(c0), "v"(c1), "v"(c2), "v"(c3), "v"(h0), "v"(h1), "v"(h2), "v"(h3));
+}
+
+// Clip, then multiply by the output scale, then clamp to [-127, 127] (what a clipping layer that requantises does per
+// value: src/layer/fused_activation.h:25-33, then float2int8 of v * scale_out) equals multiply first and clamp once to
+//   [ clamp(p0 * s), clamp(p1 * s) ]
+// when p0 <= p1, s >= 0 and everything is finite: x -> RN(x * s) never decreases, so it commutes with min and max,
+// and two nested clamps are one clamp to the clamped bounds.  Saves the max and the min per value.
+__device__ __forceinline__ bool clip_folds_into_requantise(float p0, float p1, float s)
+{
+    return p0 <= p1 && s >= 0.f && s < INFINITY;
+}
+
 __device__ __forceinline__ float apply_activation(float v, const ncnnhip_activation& a)
 {
     switch (a.type)

@@ -42,7 +42,7 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
 
 template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
+                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int dense, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
 {
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
@@ -63,10 +63,12 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         const int T = gridDim.x, xcd = b & 7, idx = b >> 3, rem = T & 7;
         b = xcd * (T >> 3) + (xcd < rem ? xcd : rem) + idx;
     }
-    const int tn = b % tiles_n;
-    const int rest = b / tiles_n;
-    const int tm = rest % tiles_m;
-    const int split = rest / tiles_m;
+    // b / tiles_n by multiplication: magic_n = 2^32/tiles_n + 1 is exact while b * tiles_n < 2^32 (checked at launch),
+    // and stays on the scalar unit, where a division would be some twenty vector instructions per wavefront
+    const int rest = tiles_n == 1 ? b : (int)__umulhi((unsigned)b, magic_n);
+    const int tn = b - rest * tiles_n;
+    const int split = SPLITK ? rest / tiles_m : 0;
+    const int tm = rest - split * tiles_m;
     const int row0 = tm * BM, col0 = tn * BN;
 
     const int total_steps = g.K / 64;
@@ -90,11 +92,16 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         const int n = row0 + i * 64 + ld_row;
         const bool ok = n < g.npix;
         const int nn = ok ? n : 0;
-        const int plane = g.outw * g.outh;
-        const int img = nn / plane;
-        const int rem = nn - img * plane;
-        const int oy = rem / g.outw;
-        const int ox = rem - oy * g.outw;
+        // dense: the launch presents a 1x1 stride-1 unpadded layer as one row of npix pixels, output pixel = input pixel
+        int img = 0, oy = 0, ox = nn;
+        if (!dense)
+        {
+            const int plane = g.outw * g.outh;
+            img = nn / plane;
+            const int rem = nn - img * plane;
+            oy = rem / g.outw;
+            ox = rem - oy * g.outw;
+        }
         // a pixel beyond the end gets coordinates that fail every bounds test
         a_iy0[i] = ok ? oy * g.sh - g.pad_top : -0x40000000;
         a_ix0[i] = ox * g.sw - g.pad_left;
@@ -112,10 +119,20 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     int q0, ky, kx, tap;
     {
         const int k = step_begin * 64 + ld_chunk * 16;
-        tap = k / g.tapK;
+        if (dense)
+        {
+            // one tap; K beyond it is the round-up to 64, less than one tap's worth
+            tap = k >= g.tapK ? 1 : 0;
+            ky = tap;
+            kx = 0;
+        }
+        else
+        {
+            tap = k / g.tapK;
+            ky = tap / g.kw;
+            kx = tap - ky * g.kw;
+        }
         q0 = k - tap * g.tapK;
-        ky = tap / g.kw;
-        kx = tap - ky * g.kw;
     }
 
     // issues the loads of the next stage in sequence (s = 0, 1, 2, ... relative to step_begin)
@@ -280,7 +297,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         else
         {
             s_in[c] = real[c] ? epi.scale_in[ch] : 0.f;
-            bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : 0.f;
+            // no bias: -0, the one value whose addition changes nothing (x + -0 = x for every x, -0 included)
+            bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : -0.f;
             s_out[c] = (real[c] && to_int8) ? epi.scale_out[ch] : 0.f;
         }
     }
@@ -334,6 +352,13 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     // the activation type is uniform: branch on it once, outside the unrolled loops
     auto finish = [&](auto act_tag) {
         constexpr int ACT = decltype(act_tag)::value;
+        float q_lo[TN], q_hi[TN]; // ACT 103 to int8: the clip's bounds in the output scale, inside [-127, 127]
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+        {
+            q_lo[c] = __builtin_amdgcn_fmed3f(mul_rn(epi.act.p0, s_out[c]), -127.f, 127.f);
+            q_hi[c] = __builtin_amdgcn_fmed3f(mul_rn(epi.act.p1, s_out[c]), -127.f, 127.f);
+        }
 #pragma unroll
         for (int a = 0; a < TM; a++)
         {
@@ -345,14 +370,17 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                 {
-                    float f = mul_rn((float)acc[a][c][r], s_in[c]);
-                    if (epi.bias) f = add_rn(f, bias[c]);
+                    float f = add_rn(mul_rn((float)acc[a][c][r], s_in[c]), bias[c]);
                     if (ACT == 1)
                         f = fmaxf(f, 0.f);
                     else if (ACT == 3)
                     {
                         if (f < epi.act.p0) f = epi.act.p0;
                         if (f > epi.act.p1) f = epi.act.p1;
+                    }
+                    else if (ACT == 103)
+                    {
+                        if (!to_int8) f = clip_not_nan(f, epi.act.p0, epi.act.p1); // (to int8: folded into the clamp below)
                     }
                     else if (ACT != 0)
                         f = apply_activation(f, epi.act);
@@ -361,13 +389,21 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 if (to_int8)
                 {
 #pragma unroll
-                    for (int r = 0; r < 16; r += 4) float2int8_as_float_x4(fr[r], fr[r + 1], fr[r + 2], fr[r + 3]);
+                    for (int r = 0; r < 16; r += 4)
+                    {
+                        if (ACT == 103)
+                            float2int8_as_float_bounded_x4(fr[r], fr[r + 1], fr[r + 2], fr[r + 3], q_lo[c], q_hi[c]);
+                        else
+                            float2int8_as_float_x4(fr[r], fr[r + 1], fr[r + 2], fr[r + 3]);
+                    }
                 }
+                // Pad channels carry zero scales and no bias: with no activation or ReLU they are zero already, and
+                // behind the bounded clip a pad's (finite) value times its zero output scale rounds to zero too.
+                const bool clear_pads = ACT != 0 && ACT != 1 && !(ACT == 103 && to_int8);
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                 {
-                    // pad channels carry zero scales and bias: with no activation or ReLU they are zero already
-                    if (ACT != 0 && ACT != 1 && !real[c]) fr[r] = 0.f;
+                    if (clear_pads && !real[c]) fr[r] = 0.f;
                     tile[(8 * (r >> 2) + 4 * lhi + (r & 3)) * LD + c * 32 + l32] = fr[r];
                 }
             }
@@ -440,7 +476,21 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     else if (epi.act.type == 1)
         finish(std::integral_constant<int, 1>{});
     else if (epi.act.type == 3)
-        finish(std::integral_constant<int, 3>{});
+    {
+        // Tame tables: every accumulator comes out of scale and bias finite (|acc| <= 2^31, so 2^90 and 2^120 leave
+        // room), so the clip is max-then-min; the clipped value times the output scale stays below 2^31, so float2int8
+        // needs no out-of-range branch; and the clip folds into the requantising clamp.
+        const float clip_abs = fmaxf(fabsf(epi.act.p0), fabsf(epi.act.p1));
+        bool tame = fabsf(epi.act.p0) < INFINITY && fabsf(epi.act.p1) < INFINITY;
+#pragma unroll
+        for (int c = 0; c < TN; c++)
+            tame = tame && fabsf(s_in[c]) < 0x1p90f && fabsf(bias[c]) < 0x1p120f && mul_rn(clip_abs, fabsf(s_out[c])) < 2147483648.f
+                   && clip_folds_into_requantise(epi.act.p0, epi.act.p1, s_out[c]);
+        if (__all(tame))
+            finish(std::integral_constant<int, 103>{});
+        else
+            finish(std::integral_constant<int, 3>{});
+    }
     else
         finish(std::integral_constant<int, -1>{});
 }
@@ -490,12 +540,27 @@ size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps)
     return SPLIT_COUNTER_BYTES / sizeof(int32_t) + (size_t)p.splits * p.tiles_m * p.tiles_n * p.bm * p.bn;
 }
 
-int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
+// multiplier that turns b / tiles_n into a high multiply, exact for b * tiles_n < 2^32 (tiles_n == 1 is special-cased)
+static inline unsigned tile_magic(int tiles_n)
+{
+    return tiles_n > 1 ? (unsigned)((1ull << 32) / (unsigned)tiles_n + 1) : 0u;
+}
+
+int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
                                void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
+    NhwcGeom g = g_in;
+    // A 1x1, stride-1, unpadded layer reads input pixel n for output pixel n, whatever the image shape: present it as
+    // one row of npix pixels, and the kernel skips the pixel -> (image, y, x) divisions.
+    const int dense = g.kw == 1 && g.kh == 1 && g.sw == 1 && g.sh == 1 && g.pad_top == 0 && g.pad_left == 0 && g.outw == g.W && g.outh == g.H && g.tapK == g.Cp;
+    if (dense)
+    {
+        g.H = g.outh = 1;
+        g.W = g.outw = g.npix;
+    }
     const PipePlan p = plan_pipelined(g.cout, g.npix, g.K / 64);
     const long long blocks = (long long)p.tiles_m * p.tiles_n * p.splits;
-    NCNNHIP_REQUIRE(blocks < (1ll << 31), "convolution: too many tiles");
+    NCNNHIP_REQUIRE(blocks < (1ll << 31) && blocks * p.tiles_n < (1ll << 32), "convolution: too many tiles");
     int32_t* partial = 0;
     unsigned* counters = 0;
     if (p.splits > 1)
@@ -512,10 +577,10 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
     {                                                                                                                                           \
         if (p.splits > 1)                                                                                                                       \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.splits, p.steps_per_split, partial, counters);                                                                                     \
+                               p.splits, p.steps_per_split, tile_magic(p.tiles_n), dense, partial, counters);                                                                                     \
         else                                                                                                                                    \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.splits, p.steps_per_split, partial, counters);                                                                                     \
+                               p.splits, p.steps_per_split, tile_magic(p.tiles_n), dense, partial, counters);                                                                                     \
     } while (0)
     // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
     if (p.bm == 128 && p.bn == 256)
@@ -575,11 +640,11 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     p.splits = 1;
     p.steps_per_split = K / 64;
     const long long blocks = (long long)p.tiles_m * p.tiles_n;
-    NCNNHIP_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    NCNNHIP_REQUIRE(blocks < (1ll << 31) && blocks * p.tiles_n < (1ll << 32), "gemm: too many tiles");
     dim3 grid((unsigned)blocks), block(256);
 #define LAUNCH_GEMM(BM_, BN_)                                                                                                                        \
     hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
-                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, (int32_t*)0, (unsigned*)0)
+                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, tile_magic(p.tiles_n), 1, (int32_t*)0, (unsigned*)0)
     if (p.bm == 128 && p.bn == 256)
         LAUNCH_GEMM(128, 256);
     else if (p.bm == 128 && p.bn == 128)
@@ -631,6 +696,7 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
         counters = (unsigned*)workspace;
         partial = (int32_t*)((char*)workspace + SPLIT_COUNTER_BYTES);
     }
+    NCNNHIP_REQUIRE((long long)p.tiles_m * p.tiles_n * p.splits * p.tiles_n < (1ll << 32), "innerproduct: too many tiles");
     dim3 grid((unsigned)((long long)p.tiles_m * p.tiles_n * p.splits)), block(256);
     // rows are few: only the 64-pixel tiles occur
 #define LAUNCH_FC(BN_)                                                                                                                                   \
@@ -638,10 +704,10 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
     {                                                                                                                                                    \
         if (p.splits > 1)                                                                                                                                \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, true, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,     \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, partial, counters);                       \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), 1, partial, counters);                       \
         else                                                                                                                                             \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, false, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,    \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, partial, counters);                       \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), 1, partial, counters);                       \
     } while (0)
     if (p.bm != 64)
     {

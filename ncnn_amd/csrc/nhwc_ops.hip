@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
     {
         const unsigned qc = q0 < (unsigned)g.c ? q0 : (unsigned)g.c - 4;
         const v4f a = *reinterpret_cast<const v4f*>(scale_in + qc);
-        const v4f b = bias ? *reinterpret_cast<const v4f*>(bias + qc) : v4f{0.f, 0.f, 0.f, 0.f};
+        const v4f b = bias ? *reinterpret_cast<const v4f*>(bias + qc) : v4f{-0.f, -0.f, -0.f, -0.f}; // x + -0 = x for every x
         const v4f c = g.out_f32 ? v4f{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const v4f*>(scale_out + qc);
 #pragma unroll
         for (int e = 0; e < 4; e++)
@@ -505,35 +505,65 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
         {
             const int qc = (int)q0 + e < g.c ? (int)q0 + e : g.c - 1;
             s_in[e] = scale_in[qc];
-            s_b[e] = bias ? bias[qc] : 0.f;
+            s_b[e] = bias ? bias[qc] : -0.f;
             s_out[e] = g.out_f32 ? 0.f : scale_out[qc];
         }
     }
+    // A clip whose operand cannot be NaN (finite tables: an int32 times a finite scale plus a finite bias is finite or
+    // infinite) is max-then-min, two instructions for the reference's two compare-and-selects, with the same result.
+    // If the clipped value times the output scale also stays below 2^31, float2int8 needs no out-of-range branch.
+    // And with finite values the clip folds into the requantising clamp (clip_folds_into_requantise).
+    const float clip_abs = fmaxf(fabsf(act.p0), fabsf(act.p1));
+    bool finite_tables = fabsf(act.p0) < INFINITY && fabsf(act.p1) < INFINITY;
+    float q_lo[4], q_hi[4];
 #pragma unroll
-    for (int o = 0; o < OUTS; o++)
+    for (int e = 0; e < 4; e++)
     {
-        const unsigned ox = ox0 + o;
-        if (ox >= (unsigned)g.outw) continue;
-        const size_t off = ((size_t)blockIdx.y * g.outw + ox) * g.cp + q0;
-        float f[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-        {
-            float v = mul_rn((float)acc[o][e], s_in[e]);
-            if (bias) v = add_rn(v, s_b[e]);
-            v = apply_activation(v, act);
-            f[e] = g.out_f32 ? v : mul_rn(v, s_out[e]);
-        }
-        if (!g.out_f32) float2int8_as_float_x4(f[0], f[1], f[2], f[3]);
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-            if ((int)q0 + e >= g.c) f[e] = 0.f;
-        if (g.out_f32)
-            *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
-        else
-            *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
-                (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
+        finite_tables = finite_tables && fabsf(s_in[e]) < 0x1p90f && fabsf(s_b[e]) < 0x1p120f && mul_rn(clip_abs, fabsf(s_out[e])) < 2147483648.f
+                        && clip_folds_into_requantise(act.p0, act.p1, s_out[e]);
+        q_lo[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p0, s_out[e]), -127.f, 127.f);
+        q_hi[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p1, s_out[e]), -127.f, 127.f);
     }
+    auto emit = [&](auto clip_tag) {
+        constexpr bool FAST_CLIP = decltype(clip_tag)::value;
+#pragma unroll
+        for (int o = 0; o < OUTS; o++)
+        {
+            const unsigned ox = ox0 + o;
+            if (ox >= (unsigned)g.outw) continue;
+            const size_t off = ((size_t)blockIdx.y * g.outw + ox) * g.cp + q0;
+            float f[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+            {
+                float v = add_rn(mul_rn((float)acc[o][e], s_in[e]), s_b[e]);
+                if (!FAST_CLIP)
+                    v = apply_activation(v, act);
+                else if (g.out_f32)
+                    v = clip_not_nan(v, act.p0, act.p1); // (to int8: folded into the clamp below)
+                f[e] = g.out_f32 ? v : mul_rn(v, s_out[e]);
+            }
+            if (!g.out_f32)
+            {
+                if (FAST_CLIP)
+                    float2int8_as_float_bounded_lanes_x4(f[0], f[1], f[2], f[3], q_lo, q_hi);
+                else
+                    float2int8_as_float_x4(f[0], f[1], f[2], f[3]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if ((int)q0 + e >= g.c) f[e] = 0.f;
+            if (g.out_f32)
+                *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
+            else
+                *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
+                    (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
+        }
+    };
+    if (act.type == 3 && __all(finite_tables))
+        emit(std::true_type{});
+    else
+        emit(std::false_type{});
 }
 
 static inline int padded16(int c)

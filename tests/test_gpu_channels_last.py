@@ -74,6 +74,31 @@ def test_convolution_channels_last_bit_exact(rt, shape, term, act, act_params, i
     assert got.dtype == want.dtype and np.array_equal(got[0], want)
 
 
+@pytest.mark.parametrize("act_params", [(-0.37, 0.41), (0.013, 0.02), (0.3, -0.2), (-1e30, 1e30), (float("-inf"), 0.5)])
+@pytest.mark.parametrize("term,bias,flip", [(102, True, False), (101, False, False), (102, True, True), (2, False, False)])
+def test_clip_is_the_reference_clip_whatever_its_bounds(rt, act_params, term, bias, flip):
+    """The kernels fold a clip into the requantising clamp when that is provably the same (bounds in order, finite
+    tables, output scales not negative) and take the literal compare-and-select path otherwise: both bounds active,
+    bounds that are no integers in the output scale, reversed bounds, huge and infinite bounds, negative output scales
+    (flip), no bias, fp32 output."""
+    _say("clip variants", act_params, term, bias, flip)
+    for group, c, outc, kernel, pads in [(1, 24, 40, (1, 1), (0, 0, 0, 0)), (1, 16, 16, (3, 3), (1, 1, 1, 1)), (48, 48, 48, (3, 3), (1, 1, 1, 1))]:
+        x, wq, b, ws, ins, tops = cases.conv_case(7 + term, c, 12, 11, outc, kernel, group, term, bias, term > 100, by_group=group > 1, batch=2)
+        if group > 1 and term in (2, 102):
+            ws = np.full(c, ws[0], F)
+        if tops is not None and flip:
+            tops = tops.copy()
+            tops[:] = -tops
+        d = oracle.make_desc((c, 12, 11), outc, kernel, (1, 1), (1, 1), pads, 0.0, 1 if bias else 0, group, term, 3, act_params)
+        got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, (1, 1), (1, 1), pads, 0.0, group, term, 3, act_params)
+        for i in range(2):
+            if group > 1:
+                want = oracle.convolutiondepthwise_int8(d, x[i], wq, b, ws, ins, tops)
+            else:
+                want = oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None if tops is None else tops[0])
+            assert got.dtype == want.dtype and np.array_equal(got[i], want), (group, kernel)
+
+
 def test_convolution_channels_last_batch_and_pad_value(rt):
     x, wq, b, ws, ins, tops = cases.conv_case(21, 20, 10, 9, 24, (3, 3), 1, 101, True, False, batch=3)
     d = oracle.make_desc((20, 10, 9), 24, (3, 3), pads=(1, 1, 1, 1), pad_value=-2.2, bias_term=1, int8_scale_term=101, activation_type=1)
