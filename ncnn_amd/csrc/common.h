@@ -139,6 +139,53 @@ __device__ __forceinline__ void float2int8_as_float_bounded_x4(float& v0, float&
                  : "v"(c0), "v"(c1), "v"(c2), "v"(c3), "v"(h0), "v"(h1), "v"(h2), "v"(h3));
 }
 
+// Four already-quantised values (integers in [-127, 127] held as floats) -> four bytes, first value lowest: each
+// conversion writes its low byte straight into its place in the word (sub-dword destination select), four
+// instructions instead of four conversions plus the masks, shifts and ors.  A vector instruction that reads a
+// register right after a sub-dword write to it needs one wait state on this chip, and the compiler does not look
+// inside asm: hence the s_nop after each write (the last one covers whatever the compiler schedules next).
+__device__ __forceinline__ uint32_t pack4_quantised(float a, float b, float c, float d)
+{
+    uint32_t r;
+    asm volatile("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %3 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %4 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0"
+                 : "=&v"(r)
+                 : "v"(a), "v"(b), "v"(c), "v"(d));
+    return r;
+}
+
+// Sixteen values -> four words; the four words advance together, so no write is read by the next instruction and
+// only the end needs its wait state.
+__device__ __forceinline__ void pack16_quantised(const float (&v)[16], uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3)
+{
+    asm volatile("v_cvt_i32_f32_sdwa %0, %4 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %1, %8 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %2, %12 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %3, %16 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %5 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %1, %9 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %2, %13 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %3, %17 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %6 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %1, %10 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %2, %14 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %3, %18 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %0, %7 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %1, %11 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %2, %15 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_i32_f32_sdwa %3, %19 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0"
+                 : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+                 : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(v[8]), "v"(v[9]), "v"(v[10]),
+                   "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));
+}
+
 // the same with one clamp per value (four different channels)
 __device__ __forceinline__ void float2int8_as_float_bounded_lanes_x4(float& v0, float& v1, float& v2, float& v3, const float (&lo)[4], const float (&hi)[4])
 {

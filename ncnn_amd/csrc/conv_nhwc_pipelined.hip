@@ -37,7 +37,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // four already-quantised values (integers in [-127,127] held as floats) -> four bytes
 __device__ __forceinline__ uint32_t pack4(const v4f& v)
 {
-    return (uint32_t)((int)v[0] & 0xff) | ((uint32_t)((int)v[1] & 0xff) << 8) | ((uint32_t)((int)v[2] & 0xff) << 16) | ((uint32_t)((int)v[3] & 0xff) << 24);
+    return pack4_quantised(v[0], v[1], v[2], v[3]);
 }
 
 template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
@@ -422,9 +422,16 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                     const int ch16 = col0 + wn * CW + 16 * j;
                     if (p < 32 && pix < g.npix && ch16 < col_limit)
                     {
-                        v4i pk;
+                        float q[16];
 #pragma unroll
-                        for (int w4 = 0; w4 < 4; w4++) pk[w4] = (int)pack4(*reinterpret_cast<const v4f*>(tile + p * LD + 16 * j + 4 * w4));
+                        for (int w4 = 0; w4 < 4; w4++)
+                        {
+                            const v4f t = *reinterpret_cast<const v4f*>(tile + p * LD + 16 * j + 4 * w4);
+                            q[4 * w4] = t[0], q[4 * w4 + 1] = t[1], q[4 * w4 + 2] = t[2], q[4 * w4 + 3] = t[3];
+                        }
+                        uint32_t p0, p1, p2, p3;
+                        pack16_quantised(q, p0, p1, p2, p3);
+                        const v4i pk = {(int)p0, (int)p1, (int)p2, (int)p3};
                         *reinterpret_cast<v4i*>(static_cast<int8_t*>(epi.out) + (size_t)pix * out_cp + ch16) = pk;
                     }
                 }

@@ -556,8 +556,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
             if (g.out_f32)
                 *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
             else
-                *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) =
-                    (uint32_t)((int)f[0] & 0xff) | ((uint32_t)((int)f[1] & 0xff) << 8) | ((uint32_t)((int)f[2] & 0xff) << 16) | ((uint32_t)((int)f[3] & 0xff) << 24);
+                *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) = pack4_quantised(f[0], f[1], f[2], f[3]);
         }
     };
     if (act.type == 3 && __all(finite_tables))
