@@ -105,7 +105,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         // a pixel beyond the end gets coordinates that fail every bounds test
         a_iy0[i] = ok ? oy * g.sh - g.pad_top : -0x40000000;
         a_ix0[i] = ox * g.sw - g.pad_left;
-        a_base[i] = x + (size_t)img * g.H * g.W * g.Cp;
+        // dense: the pixel's own address, so that a stage's source is one 64-bit add away
+        a_base[i] = dense ? x + (size_t)nn * g.Cp : x + (size_t)img * g.H * g.W * g.Cp;
     }
     const int8_t* b_ptr[LB];
 #pragma unroll
@@ -138,28 +139,49 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     // issues the loads of the next stage in sequence (s = 0, 1, 2, ... relative to step_begin)
     auto issue = [&](int s) {
         int8_t* stage = smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
-        const int dy = ky * g.dh, dx = kx * g.dw;
-        const bool tap_ok = tap < g.ntaps;
-#pragma unroll
-        for (int i = 0; i < LA; i++)
+        if (dense)
         {
-            const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
-            const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
-            const int8_t* src = in ? a_base[i] + ((size_t)iy * g.W + ix) * g.Cp + q0 : zero;
-            __builtin_amdgcn_global_load_lds((const AS1 void*)src, (AS3 void*)(stage + i * 4096), 16, 0, 0);
+            // one tap, no border: the row's pixel exists or it does not (a_iy0 is 0 or hugely negative)
+#pragma unroll
+            for (int i = 0; i < LA; i++)
+            {
+                const bool in = tap == 0 && a_iy0[i] == 0;
+                const int8_t* src = in ? a_base[i] + q0 : zero;
+                __builtin_amdgcn_global_load_lds((const AS1 void*)src, (AS3 void*)(stage + i * 4096), 16, 0, 0);
+            }
+        }
+        else
+        {
+            const int dy = ky * g.dh, dx = kx * g.dw;
+            const bool tap_ok = tap < g.ntaps;
+#pragma unroll
+            for (int i = 0; i < LA; i++)
+            {
+                const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+                const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                const int8_t* src = in ? a_base[i] + ((size_t)iy * g.W + ix) * g.Cp + q0 : zero;
+                __builtin_amdgcn_global_load_lds((const AS1 void*)src, (AS3 void*)(stage + i * 4096), 16, 0, 0);
+            }
         }
 #pragma unroll
         for (int i = 0; i < LB; i++)
             __builtin_amdgcn_global_load_lds((const AS1 void*)(b_ptr[i] + (size_t)s * 64), (AS3 void*)(stage + BM * 64 + i * 4096), 16, 0, 0);
         q0 += 64;
-        while (q0 >= g.tapK)
+        if (dense)
         {
-            q0 -= g.tapK;
-            tap++;
-            if (++kx == g.kw)
+            if (q0 >= g.tapK) tap = 1; // past the only tap: the rest of K is the round-up, zero-filled
+        }
+        else
+        {
+            while (q0 >= g.tapK)
             {
-                kx = 0;
-                ky++;
+                q0 -= g.tapK;
+                tap++;
+                if (++kx == g.kw)
+                {
+                    kx = 0;
+                    ky++;
+                }
             }
         }
     };
