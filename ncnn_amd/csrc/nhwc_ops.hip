@@ -416,26 +416,30 @@ __global__ __launch_bounds__(256) void dwconv_nhwc_kernel(const int8_t* __restri
 // Consecutive lanes are consecutive channel quads of a pixel: every load and store of a wavefront is a contiguous
 // run.  The kernel is bound by VALU issue (index arithmetic + ~20 single-rounded fp32 instructions of requantising
 // epilogue per output), so everything per-thread is amortised over as many outputs as the registers allow.
-template<int STRIDE>
+template<int STRIDE, int ROWS>
 __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __restrict__ x, const uint32_t* __restrict__ wrow /* [3][cp] */, DwNhwcGeom g,
                                                               const float* __restrict__ scale_in, const float* __restrict__ bias,
                                                               const float* __restrict__ scale_out, ncnnhip_activation act, void* __restrict__ out,
-                                                              unsigned quads, unsigned quads_magic, unsigned xgroups)
+                                                              unsigned quads, unsigned quads_magic, unsigned xgroups, unsigned rowgroups, unsigned rowgroups_magic)
 {
     constexpr int OUTS = STRIDE == 1 ? 2 : 1;
-    constexpr int PIX = STRIDE == 1 ? 4 : 3; // input pixels per kernel row
-    // blockIdx.y = output row (sample * outh + oy); within the row a thread is (x group, channel quad), quads fastest.
-    // xg = r / quads by multiplication with ceil(2^32 / quads), exact here because r * quads < 2^32
+    constexpr int PIX = STRIDE == 1 ? 4 : 3;          // input pixels per kernel row
+    constexpr int IN_ROWS = (ROWS - 1) * STRIDE + 3;  // input rows under ROWS output rows
+    // blockIdx.y = (sample, group of ROWS output rows); within the rows a thread is (x group, channel quad), quads
+    // fastest.  Each input row is loaded and transposed once and serves every output row of the group it lies under.
+    // xg = r / quads by multiplication with ceil(2^32 / quads), exact here because r * quads < 2^32; the sample index
+    // likewise (blockIdx.y * rowgroups < 2^32), on the scalar unit.
     const unsigned r = blockIdx.x * 256 + threadIdx.x;
     if (r >= xgroups * quads) return;
     unsigned xg = __umulhi(r, quads_magic);
     if (xg * quads > r) xg--;
     const unsigned q0 = (r - xg * quads) * 4;
     const unsigned ox0 = xg * OUTS;
-    const unsigned oy = blockIdx.y % (unsigned)g.outh;
-    const unsigned img = blockIdx.y / (unsigned)g.outh;
+    unsigned img = rowgroups == 1 ? blockIdx.y : __umulhi(blockIdx.y, rowgroups_magic);
+    if (img * rowgroups > blockIdx.y) img--;
+    const unsigned oy0 = (blockIdx.y - img * rowgroups) * ROWS;
     const int8_t* base = x + (size_t)img * g.h * g.w * g.cp + q0;
-    const int y0 = (int)oy * STRIDE - g.pad_top, x0 = (int)ox0 * STRIDE - g.pad_left;
+    const int y0 = (int)oy0 * STRIDE - g.pad_top, x0 = (int)ox0 * STRIDE - g.pad_left;
     const uint32_t padw = (uint32_t)(g.pad_byte & 0xff) * 0x01010101u;
 
     // column offsets (clamped into the image so that every load is unconditional) and their validity
@@ -449,15 +453,27 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
         xoff[p] = (unsigned)(xin[p] ? xx : 0) * (unsigned)g.cp;
     }
 
-    int acc[OUTS][4];
-#pragma unroll
-    for (int o = 0; o < OUTS; o++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) acc[o][e] = 0;
+    // weights: 4 channels x (w0,w1,w2,0) per kernel row; shifted one byte up, (0,w0,w1,w2), for the second output pixel
+    v4i wv[3], wv1[3];
 #pragma unroll
     for (int ky = 0; ky < 3; ky++)
     {
-        const int y = y0 + ky;
+        wv[ky] = *reinterpret_cast<const v4i*>(wrow + (size_t)ky * g.cp + q0);
+#pragma unroll
+        for (int c = 0; c < 4; c++) wv1[ky][c] = (int)((uint32_t)wv[ky][c] << 8);
+    }
+
+    int acc[ROWS][OUTS][4];
+#pragma unroll
+    for (int ro = 0; ro < ROWS; ro++)
+#pragma unroll
+        for (int o = 0; o < OUTS; o++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[ro][o][e] = 0;
+#pragma unroll
+    for (int iy = 0; iy < IN_ROWS; iy++)
+    {
+        const int y = y0 + iy;
         const bool yin = (unsigned)y < (unsigned)g.h;
         const unsigned rowoff = (unsigned)(yin ? y : 0) * (unsigned)g.w * (unsigned)g.cp; // one sample < 2^31 bytes
         uint32_t d[4];
@@ -468,17 +484,22 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
             d[p] = (yin && xin[p]) ? v : padw;
         }
         if (PIX == 3) d[3] = 0;
-        const v4i wv = *reinterpret_cast<const v4i*>(wrow + (size_t)ky * g.cp + q0); // 4 channels x (w0,w1,w2,0)
         // 4x4 byte transpose: t[c] = (pixel0.c, pixel1.c, pixel2.c, pixel3.c)
         const uint32_t p01l = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), p01h = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
         const uint32_t p23l = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), p23h = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
         const uint32_t t[4] = {__builtin_amdgcn_perm(p23l, p01l, 0x05040100u), __builtin_amdgcn_perm(p23l, p01l, 0x07060302u),
                                __builtin_amdgcn_perm(p23h, p01h, 0x05040100u), __builtin_amdgcn_perm(p23h, p01h, 0x07060302u)};
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int ro = 0; ro < ROWS; ro++)
         {
-            acc[0][c] = __builtin_amdgcn_sdot4((int)t[c], wv[c], acc[0][c], false);
-            if (OUTS == 2) acc[1][c] = __builtin_amdgcn_sdot4((int)t[c], (int)((uint32_t)wv[c] << 8), acc[1][c], false);
+            const int ky = iy - ro * STRIDE; // this input row is kernel row ky of output row ro (compile time)
+            if (ky < 0 || ky > 2) continue;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+            {
+                acc[ro][0][c] = __builtin_amdgcn_sdot4((int)t[c], wv[ky][c], acc[ro][0][c], false);
+                if (OUTS == 2) acc[ro][1][c] = __builtin_amdgcn_sdot4((int)t[c], wv1[ky][c], acc[ro][1][c], false);
+            }
         }
     }
 
@@ -527,16 +548,18 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
     auto emit = [&](auto clip_tag) {
         constexpr bool FAST_CLIP = decltype(clip_tag)::value;
 #pragma unroll
+        for (int ro = 0; ro < ROWS; ro++)
+#pragma unroll
         for (int o = 0; o < OUTS; o++)
         {
-            const unsigned ox = ox0 + o;
-            if (ox >= (unsigned)g.outw) continue;
-            const size_t off = ((size_t)blockIdx.y * g.outw + ox) * g.cp + q0;
+            const unsigned ox = ox0 + o, oy = oy0 + ro;
+            if (ox >= (unsigned)g.outw || oy >= (unsigned)g.outh) continue;
+            const size_t off = (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q0;
             float f[4];
 #pragma unroll
             for (int e = 0; e < 4; e++)
             {
-                float v = add_rn(mul_rn((float)acc[o][e], s_in[e]), s_b[e]);
+                float v = add_rn(mul_rn((float)acc[ro][o][e], s_in[e]), s_b[e]);
                 if (!FAST_CLIP)
                     v = apply_activation(v, act);
                 else if (g.out_f32)
@@ -815,15 +838,25 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
         const uint32_t* wrow = reinterpret_cast<const uint32_t*>(packed_weight_dev + (size_t)9 * g.cp);
         const unsigned quads = (unsigned)g.cp / 4;
         const unsigned xgroups = (unsigned)ceil_div(outw, d.stride_w == 1 ? 2 : 1);
-        const size_t rows = (size_t)d.batch * outh, row_threads = (size_t)xgroups * quads;
+        const size_t row_threads = (size_t)xgroups * quads;
         const unsigned quads_magic = (unsigned)(((1ull << 32) + quads - 1) / quads);
-        dim3 grid3(ceil_div((long long)row_threads, 256), (unsigned)rows);
-        if (d.stride_w == 1)
-            hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<1>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, quads, quads_magic, xgroups);
+        // two output rows per thread share their input rows; a single row when that leaves too few threads for the chip
+        const int rows_per_thread = (size_t)d.batch * ceil_div(outh, 2) * row_threads >= 256 * 256 * 2 ? 2 : 1;
+        const unsigned rowgroups = (unsigned)ceil_div(outh, rows_per_thread);
+        const unsigned rowgroups_magic = rowgroups > 1 ? (unsigned)((1ull << 32) / rowgroups + 1) : 0u;
+        dim3 grid3(ceil_div((long long)row_threads, 256), (unsigned)((size_t)d.batch * rowgroups));
+#define LAUNCH_DW(S_, R_)                                                                                                                                   \
+    hipLaunchKernelGGL((dwconv3x3_nhwc_kernel<S_, R_>), grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act, \
+                       out_nhwc_dev, quads, quads_magic, xgroups, rowgroups, rowgroups_magic)
+        if (d.stride_w == 1 && rows_per_thread == 2)
+            LAUNCH_DW(1, 2);
+        else if (d.stride_w == 1)
+            LAUNCH_DW(1, 1);
+        else if (rows_per_thread == 2)
+            LAUNCH_DW(2, 2);
         else
-            hipLaunchKernelGGL(dwconv3x3_nhwc_kernel<2>, grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act,
-                               out_nhwc_dev, quads, quads_magic, xgroups);
+            LAUNCH_DW(2, 1);
+#undef LAUNCH_DW
         return launch_status("dwconv3x3_nhwc_kernel");
     }
     const size_t total = (size_t)d.batch * outh * outw * (g.cp / 16);
