@@ -840,22 +840,34 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
         const unsigned xgroups = (unsigned)ceil_div(outw, d.stride_w == 1 ? 2 : 1);
         const size_t row_threads = (size_t)xgroups * quads;
         const unsigned quads_magic = (unsigned)(((1ull << 32) + quads - 1) / quads);
-        // two output rows per thread share their input rows; a single row when that leaves too few threads for the chip
-        const int rows_per_thread = (size_t)d.batch * ceil_div(outh, 2) * row_threads >= 256 * 256 * 2 ? 2 : 1;
+        // up to four output rows per thread share their input rows; fewer when that leaves too few threads for the chip
+        int rows_per_thread = 1;
+        for (int rp = 2; rp <= 4; rp *= 2)
+            if ((size_t)d.batch * ceil_div(outh, rp) * row_threads >= 256 * 256 * 2) rows_per_thread = rp;
         const unsigned rowgroups = (unsigned)ceil_div(outh, rows_per_thread);
         const unsigned rowgroups_magic = rowgroups > 1 ? (unsigned)((1ull << 32) / rowgroups + 1) : 0u;
         dim3 grid3(ceil_div((long long)row_threads, 256), (unsigned)((size_t)d.batch * rowgroups));
 #define LAUNCH_DW(S_, R_)                                                                                                                                   \
     hipLaunchKernelGGL((dwconv3x3_nhwc_kernel<S_, R_>), grid3, dim3(256), 0, as_stream(stream), nhwc_dev, wrow, g, scale_in_dev, bias_dev, scale_out_dev, act, \
                        out_nhwc_dev, quads, quads_magic, xgroups, rowgroups, rowgroups_magic)
-        if (d.stride_w == 1 && rows_per_thread == 2)
-            LAUNCH_DW(1, 2);
-        else if (d.stride_w == 1)
-            LAUNCH_DW(1, 1);
-        else if (rows_per_thread == 2)
-            LAUNCH_DW(2, 2);
+        if (d.stride_w == 1)
+        {
+            if (rows_per_thread == 4)
+                LAUNCH_DW(1, 4);
+            else if (rows_per_thread == 2)
+                LAUNCH_DW(1, 2);
+            else
+                LAUNCH_DW(1, 1);
+        }
         else
-            LAUNCH_DW(2, 1);
+        {
+            if (rows_per_thread == 4)
+                LAUNCH_DW(2, 4);
+            else if (rows_per_thread == 2)
+                LAUNCH_DW(2, 2);
+            else
+                LAUNCH_DW(2, 1);
+        }
 #undef LAUNCH_DW
         return launch_status("dwconv3x3_nhwc_kernel");
     }
