@@ -380,6 +380,37 @@ def test_float_pipe_formulation_of_float2int8_equals_the_oracle():
     assert wrong.any() and wrong[np.flatnonzero(v == F(0.49999997))[0]]
 
 
+def test_clip_folded_into_the_requantising_clamp_equals_clip_then_requantise():
+    """The device replaces  float2int8(clip(f, p0, p1) * s)  by  float2int8 of  clamp(f * s, lo, hi)  with
+    lo = clamp(p0 * s, -127, 127), hi = clamp(p1 * s, -127, 127)  when p0 <= p1, s >= 0 and everything is finite (the
+    multiplication is monotone, so it commutes with min and max; nested clamps are one clamp).  Both sides evaluated in
+    float32 here, the left one by the oracle's float2int8: equal on values at and around the clip bounds, around the
+    images of the bounds, on ties, and on a dense sample, for scales that make the bounds' images integers, half
+    integers, tiny, beyond 127, and zero -- and NOT equal once the scale is negative or the clipped value times the
+    scale can reach 2^31 (where float2int8 answers -127), which is why the device tests both before folding."""
+    rng = np.random.default_rng(11)
+    differs_for_negative_scale = differs_for_huge_bounds = False
+    for p0, p1 in [(0.0, 6.0), (-0.37, 0.41), (0.013, 0.02), (-1e30, 1e30), (-3.0, -1.0), (2.5, 2.5)]:
+        for s in [21.166666, 127.0 / 6.0, 0.25, 1e-3, 300.0, 0.0, 63.5 / 0.41, -21.0]:
+            p0f, p1f, sf = F(p0), F(p1), F(s)
+            around = [np.nextafter(b, d) for b in (p0f, p1f) for d in (F(-np.inf), F(np.inf))] + [p0f, p1f]
+            ties = ((np.arange(-140, 141) + 0.5) / s).astype(F) if s != 0 else np.zeros(1, F)
+            f = np.concatenate([np.array(around, F), ties, np.nextafter(ties, F(np.inf)), np.nextafter(ties, F(-np.inf)),
+                                rng.normal(0, 3, 20000).astype(F), rng.uniform(-8, 8, 20000).astype(F), np.array([0.0, -0.0, 1e20, -1e20], F)])
+            with np.errstate(over="ignore"):
+                want = oracle.float2int8((np.minimum(np.maximum(f, p0f), p1f) * sf).astype(F))
+                lo = np.clip(F(p0f * sf), F(-127), F(127))
+                hi = np.clip(F(p1f * sf), F(-127), F(127))
+                got = oracle.float2int8(np.clip((f * sf).astype(F), min(lo, hi), max(lo, hi)).astype(F))
+            if s >= 0 and max(abs(p0), abs(p1)) * s < 2.0 ** 31:
+                assert np.array_equal(got, want), (p0, p1, s)
+            elif s < 0:
+                differs_for_negative_scale |= not np.array_equal(got, want)
+            else:
+                differs_for_huge_bounds |= not np.array_equal(got, want)
+    assert differs_for_negative_scale and differs_for_huge_bounds
+
+
 # ---- attention with block-quantised weights (src/layer/multiheadattention.cpp:561-912) ---------------------------------
 
 def _mha_tolerance(case):
