@@ -416,32 +416,49 @@ static int stem_shape(const ncnnhip_conv_desc& d, StemShape& s)
     return NCNNHIP_OK;
 }
 
-// one thread per pixel of the bordered image: 4 bytes out
+// one thread per pixel of the bordered image: 4 bytes out.  blockIdx.y = row of the bordered image, blockIdx.z = sample.
 template<typename T>
 __global__ __launch_bounds__(256) void quantize_stem_kernel(const T* __restrict__ src, int src_cp, int c, int h, int w, int top, int left, int Hb, int Wp,
-                                                            size_t total, const float* __restrict__ scale, uint32_t* __restrict__ image)
+                                                            const float* __restrict__ scale, uint32_t* __restrict__ image)
 {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const int xb = (int)(i % (size_t)Wp);
-    const size_t rest = i / (size_t)Wp;
-    const int yb = (int)(rest % (size_t)Hb);
-    const size_t img = rest / (size_t)Hb;
+    const int xb = blockIdx.x * 256 + threadIdx.x;
+    if (xb >= Wp) return;
+    const int yb = blockIdx.y;
+    const size_t img = blockIdx.z;
     const int y = yb - top, x = xb - left;
     uint32_t word = 0;
     if ((unsigned)y < (unsigned)h && (unsigned)x < (unsigned)w)
     {
         const T* p = src + ((img * h + y) * (size_t)w + x) * src_cp;
-        const float sc = sizeof(T) == 4 ? scale[0] : 1.f;
-#pragma unroll
-        for (int q = 0; q < 4; q++)
+        if (sizeof(T) == 4)
         {
-            int v = 0;
-            if (q < c) v = sizeof(T) == 4 ? float2int8(mul_rn((float)p[q], sc)) : (int)p[q];
-            word |= (uint32_t)(v & 255) << (8 * q);
+            const float sc = scale[0];
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            if (src_cp == 4)
+            {
+                // the narrow image: one aligned 16-byte load per pixel (its unused channels are zero)
+                const v4f t = *reinterpret_cast<const v4f*>(p);
+                v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
+            }
+            else
+            {
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if (q < c) v[q] = (float)p[q];
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[q] = q < c ? mul_rn(v[q], sc) : 0.f;
+            float2int8_as_float_x4(v[0], v[1], v[2], v[3]);
+            word = pack4_quantised(v[0], v[1], v[2], v[3]);
+        }
+        else
+        {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (q < c) word |= (uint32_t)((int)p[q] & 255) << (8 * q);
         }
     }
-    image[i] = word;
+    image[(img * Hb + yb) * (size_t)Wp + xb] = word;
 }
 
 } // namespace ncnnhip
@@ -671,14 +688,15 @@ int ncnnhip_quantize_stem(const ncnnhip_conv_desc* desc, const void* nhwc_dev, i
     StemShape s;
     int ret = stem_shape(*desc, s);
     if (ret) return ret;
-    const size_t total = (size_t)desc->batch * s.Hb * s.Wp;
-    dim3 grid((unsigned)ceil_div((long long)total, 256));
+    NCNNHIP_REQUIRE(s.Hb <= 65535 && desc->batch <= 65535, "ncnnhip_quantize_stem: extent too large");
+    NCNNHIP_REQUIRE(elemsize != 4 || src_cp != 4 || (reinterpret_cast<uintptr_t>(nhwc_dev) & 15) == 0, "ncnnhip_quantize_stem: a 4-float-per-pixel image must be 16-byte aligned");
+    dim3 grid((unsigned)ceil_div(s.Wp, 256), (unsigned)s.Hb, (unsigned)desc->batch);
     if (elemsize == 4)
         hipLaunchKernelGGL(quantize_stem_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)nhwc_dev, src_cp, desc->c, desc->h, desc->w, s.pads.top,
-                           s.pads.left, s.Hb, s.Wp, total, scale_dev, (uint32_t*)image_dev);
+                           s.pads.left, s.Hb, s.Wp, scale_dev, (uint32_t*)image_dev);
     else
         hipLaunchKernelGGL(quantize_stem_kernel<int8_t>, grid, dim3(256), 0, as_stream(stream), (const int8_t*)nhwc_dev, src_cp, desc->c, desc->h, desc->w,
-                           s.pads.top, s.pads.left, s.Hb, s.Wp, total, (const float*)0, (uint32_t*)image_dev);
+                           s.pads.top, s.pads.left, s.Hb, s.Wp, (const float*)0, (uint32_t*)image_dev);
     return launch_status("quantize_stem_kernel");
 }
 
