@@ -40,6 +40,20 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
     return pack4_quantised(v[0], v[1], v[2], v[3]);
 }
 
+// n / d for 0 <= n < 2^20 and d >= 1: both are exact as floats and the float quotient (reciprocal good to an ulp or
+// two, one multiply) is within 2^20 * 2^-21 = one half of the true one, so its truncation is off by at most one, which
+// the remainder shows.  Seven instructions where the compiler's general 32-bit division takes about twenty-five.
+__device__ __forceinline__ int small_div(int n, int d)
+{
+    int q = (int)((float)n * __builtin_amdgcn_rcpf((float)d));
+    const int r = n - q * d;
+    if (r < 0)
+        q--;
+    else if (r >= d)
+        q++;
+    return q;
+}
+
 template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
                                                                    ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int dense, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
@@ -97,10 +111,20 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         if (!dense)
         {
             const int plane = g.outw * g.outh;
-            img = nn / plane;
-            const int rem = nn - img * plane;
-            oy = rem / g.outw;
-            ox = rem - oy * g.outw;
+            if (g.npix < (1 << 20))
+            {
+                img = small_div(nn, plane);
+                const int rem = nn - img * plane;
+                oy = small_div(rem, g.outw);
+                ox = rem - oy * g.outw;
+            }
+            else
+            {
+                img = nn / plane;
+                const int rem = nn - img * plane;
+                oy = rem / g.outw;
+                ox = rem - oy * g.outw;
+            }
         }
         // a pixel beyond the end gets coordinates that fail every bounds test
         a_iy0[i] = ok ? oy * g.sh - g.pad_top : -0x40000000;
@@ -129,8 +153,16 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
         else
         {
-            tap = k / g.tapK;
-            ky = tap / g.kw;
+            if (g.K < (1 << 20)) // k < K
+            {
+                tap = small_div(k, g.tapK);
+                ky = small_div(tap, g.kw);
+            }
+            else
+            {
+                tap = k / g.tapK;
+                ky = tap / g.kw;
+            }
             kx = tap - ky * g.kw;
         }
         q0 = k - tap * g.tapK;

@@ -411,6 +411,23 @@ def test_clip_folded_into_the_requantising_clamp_equals_clip_then_requantise():
     assert differs_for_negative_scale and differs_for_huge_bounds
 
 
+def test_float_quotient_is_within_one_of_the_integer_quotient_below_2_to_20():
+    """The convolution kernel splits a pixel index into (sample, row, column) with a float reciprocal instead of an
+    integer division when the index is below 2^20: trunc(float(n) * rcp(float(d))) is then off by at most one, which
+    the remainder corrects.  Checked here for reciprocals up to two ulps off in either direction (the hardware's is
+    good to one), over random and extreme operands."""
+    rng = np.random.default_rng(3)
+    n = np.concatenate([rng.integers(0, 1 << 20, 400000), np.array([0, 1, (1 << 20) - 1, (1 << 20) - 2, 1 << 19])]).astype(np.int64)
+    d = np.concatenate([rng.integers(1, 1 << 20, 200000), rng.integers(1, 300, 200000), np.array([1, 1, 2, 3, (1 << 20) - 1])]).astype(np.int64)
+    rcp = (F(1) / d.astype(F)).astype(F)
+    for ulps in (-2, -1, 0, 1, 2):
+        r = rcp.copy()
+        for _ in range(abs(ulps)):
+            r = np.nextafter(r, F(np.inf) if ulps > 0 else F(0))
+        q = np.trunc(n.astype(F) * r).astype(np.int64)
+        assert np.abs(q - n // d).max() <= 1, ulps
+
+
 # ---- attention with block-quantised weights (src/layer/multiheadattention.cpp:561-912) ---------------------------------
 
 def _mha_tolerance(case):
