@@ -58,6 +58,11 @@ size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps);
 int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
                                void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// The 1x1 small-K int8-output kernel (conv_pointwise.hip): does this problem fit it, and its launch.  The pipelined
+// launch asks first.
+bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
+int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream);
+
 // D[M][N] = A[M][K] * B[N][K]^T through the pipelined kernel; handled = false when the shape does not fit it
 // (K % 64, N % 4, strides, alignment) and the caller should take another kernel.
 int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmTail& tail,

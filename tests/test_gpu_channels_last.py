@@ -99,6 +99,28 @@ def test_clip_is_the_reference_clip_whatever_its_bounds(rt, act_params, term, bi
             assert got.dtype == want.dtype and np.array_equal(got[i], want), (group, kernel)
 
 
+@pytest.mark.parametrize("c,outc,act,act_params,flip", [
+    (16, 24, 3, (0.0, 6.0), False),     # clip folded into the clamp; second 16-channel block half padding
+    (40, 8, 0, (0.0, 0.0), False),      # 48 bytes per pixel: the last lane row reads bytes the zero weights cancel
+    (64, 100, 1, (0.0, 0.0), False),    # the full K, ReLU, channel count not a multiple of 16
+    (24, 32, 3, (-0.2, 0.3), True),     # negative output scales: the literal clip
+    (8, 16, 2, (0.1, 0.0), False),      # leaky ReLU: the general activation path
+])
+def test_pointwise_small_k_kernel_matches_oracle(rt, c, outc, act, act_params, flip):
+    """1x1 layers with at most 64 input channels, int8 output and 2^17 pixels or more take a kernel of their own
+    (MFMA fed weights-first, no LDS, lane-row transposes before the store): ragged pixel count, batch 2."""
+    _say("pointwise small-K", c, outc, act, act_params, flip)
+    h = w = 257
+    x, wq, b, ws, ins, tops = cases.conv_case(c + outc, c, h, w, outc, (1, 1), 1, 102, True, True, batch=2)
+    if flip:
+        tops = -tops
+    d = oracle.make_desc((c, h, w), outc, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), 0.0, 1, 1, 102, act, act_params)
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), 0.0, 1, 102, act, act_params)
+    for i in range(2):
+        want = oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], tops[0])
+        assert got.dtype == want.dtype and np.array_equal(got[i], want)
+
+
 def test_convolution_channels_last_batch_and_pad_value(rt):
     x, wq, b, ws, ins, tops = cases.conv_case(21, 20, 10, 9, 24, (3, 3), 1, 101, True, False, batch=3)
     d = oracle.make_desc((20, 10, 9), 24, (3, 3), pads=(1, 1, 1, 1), pad_value=-2.2, bias_term=1, int8_scale_term=101, activation_type=1)
