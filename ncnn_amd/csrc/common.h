@@ -161,7 +161,7 @@ __device__ __forceinline__ uint32_t pack4_quantised(float a, float b, float c, f
 }
 
 // Sixteen values -> four words; the four words advance together, so no write is read by the next instruction and
-// only the end needs its wait state.
+// only the end needs wait states: two, which also covers a lane-row swap (v_permlane*_swap) as the next reader.
 __device__ __forceinline__ void pack16_quantised(const float (&v)[16], uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3)
 {
     asm volatile("v_cvt_i32_f32_sdwa %0, %4 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
@@ -180,7 +180,7 @@ __device__ __forceinline__ void pack16_quantised(const float (&v)[16], uint32_t&
                  "v_cvt_i32_f32_sdwa %1, %11 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
                  "v_cvt_i32_f32_sdwa %2, %15 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
                  "v_cvt_i32_f32_sdwa %3, %19 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
-                 "s_nop 0"
+                 "s_nop 1"
                  : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
                  : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(v[8]), "v"(v[9]), "v"(v[10]),
                    "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));

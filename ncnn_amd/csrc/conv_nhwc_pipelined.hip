@@ -54,10 +54,15 @@ __device__ __forceinline__ int small_div(int n, int d)
     return q;
 }
 
-template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM>
+// MODE: how a lane finds its source bytes.  0: any geometry; 1: dense (1x1, stride 1, unpadded: one row of npix pixels,
+// also Gemm and InnerProduct); 2: taps of 16 or 32 bytes (the narrow-input image), a whole number of taps per K step.
+// A template parameter because the choice sits inside the K loop: as run-time branches there it cost the 3x3 layers
+// of ResNet-50's last stages 2-4 us each (15.4 against 11.4 us for 256 -> 256 on 14 x 14, batch 16).
+template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM, int MODE>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int dense, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
+                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
 {
+    constexpr bool dense = MODE == 1;
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
     static_assert(STAGES >= 2 && STAGES <= 7 && (STAGES - 2) * (LA + LB) < 64, "the vmcnt field counts to 63");
@@ -198,13 +203,22 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 #pragma unroll
         for (int i = 0; i < LB; i++)
             __builtin_amdgcn_global_load_lds((const AS1 void*)(b_ptr[i] + (size_t)s * 64), (AS3 void*)(stage + BM * 64 + i * 4096), 16, 0, 0);
-        q0 += 64;
-        if (dense)
+        // the lane's K position moves on by 64 bytes
+        if (MODE == 1)
         {
+            q0 += 64;
             if (q0 >= g.tapK) tap = 1; // past the only tap: the rest of K is the round-up, zero-filled
+        }
+        else if (MODE == 2)
+        {
+            // a whole number of taps per step; the offset inside the tap stays
+            tap += g.tapK == 16 ? 4 : 2;
+            ky = small_div(tap, g.kw);
+            kx = tap - ky * g.kw;
         }
         else
         {
+            q0 += 64;
             while (q0 >= g.tapK)
             {
                 q0 -= g.tapK;
@@ -634,15 +648,25 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
     }
     dim3 grid((unsigned)blocks), block(256);
     const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
+    // addressing mode (the kernel's MODE); the K-split kernels exist for modes 0 and 1 only (a narrow-input layer has
+    // too few K steps to be split)
+    const int mode = dense ? 1 : ((g.tapK == 16 || g.tapK == 32) && p.splits == 1) ? 2 : 0;
+#define LAUNCH_PIPE_MODE(BM_, BN_, ST_, SPLIT_, MODE_)                                                                                                          \
+    hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, SPLIT_, false, MODE_>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, \
+                       p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters)
 #define LAUNCH_PIPE(BM_, BN_, ST_)                                                                                                              \
     do                                                                                                                                          \
     {                                                                                                                                           \
-        if (p.splits > 1)                                                                                                                       \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, true, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.splits, p.steps_per_split, tile_magic(p.tiles_n), dense, partial, counters);                                                                                     \
+        if (p.splits > 1 && mode == 1)                                                                                                          \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, true, 1);                                                                                           \
+        else if (p.splits > 1)                                                                                                                  \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, true, 0);                                                                                           \
+        else if (mode == 1)                                                                                                                     \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 1);                                                                                          \
+        else if (mode == 2)                                                                                                                     \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 2);                                                                                          \
         else                                                                                                                                    \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, false, false>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                               p.splits, p.steps_per_split, tile_magic(p.tiles_n), dense, partial, counters);                                                                                     \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 0);                                                                                          \
     } while (0)
     // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
     if (p.bm == 128 && p.bn == 256)
@@ -658,6 +682,7 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
     else
         LAUNCH_PIPE(64, 64, 3);
 #undef LAUNCH_PIPE
+#undef LAUNCH_PIPE_MODE
     return launch_status("conv_nhwc_pipelined_kernel");
 }
 
@@ -705,8 +730,8 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     NCNNHIP_REQUIRE(blocks < (1ll << 31) && blocks * p.tiles_n < (1ll << 32), "gemm: too many tiles");
     dim3 grid((unsigned)blocks), block(256);
 #define LAUNCH_GEMM(BM_, BN_)                                                                                                                        \
-    hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
-                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, tile_magic(p.tiles_n), 1, (int32_t*)0, (unsigned*)0)
+    hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true, 1>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
+                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, tile_magic(p.tiles_n), (int32_t*)0, (unsigned*)0)
     if (p.bm == 128 && p.bn == 256)
         LAUNCH_GEMM(128, 256);
     else if (p.bm == 128 && p.bn == 128)
@@ -765,11 +790,11 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
     do                                                                                                                                                   \
     {                                                                                                                                                    \
         if (p.splits > 1)                                                                                                                                \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, true, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,     \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), 1, partial, counters);                       \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, true, false, 1>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,     \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters);                       \
         else                                                                                                                                             \
-            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, false, false>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,    \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), 1, partial, counters);                       \
+            hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, false, false, 1>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,    \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters);                       \
     } while (0)
     if (p.bm != 64)
     {
