@@ -173,6 +173,24 @@ def _pool_ref(x, kind, k, s, pt, pl, oh, ow, include_pad):
     return out
 
 
+@pytest.mark.parametrize("c,h,w,stride,pads,term,act", [
+    (64, 113, 112, 1, (1, 1, 1, 1), 101, 3),    # four output rows per thread, 113 rows: the last group has one
+    (128, 45, 64, 1, (1, 1, 1, 1), 101, 1),     # two output rows per thread, odd row count
+    (128, 91, 128, 2, (1, 1, 1, 1), 101, 3),    # stride 2, four rows per thread, 46 rows
+    (96, 50, 128, 2, (0, 1, 0, 1), 1, 0),       # stride 2, two rows per thread, fp32 output
+])
+def test_depthwise_several_output_rows_per_thread(rt, c, h, w, stride, pads, term, act):
+    """The 3x3 depthwise kernel gives a thread 1, 2 or 4 output rows depending on how many threads that leaves; the
+    small shapes above all take one row, these (batch 8) take two and four, with row counts that do not divide."""
+    _say("depthwise rows per thread", c, h, w, stride, term, act)
+    x, wq, b, ws, ins, tops = cases.conv_case(c + h, c, h, w, c, (3, 3), c, term, True, term > 100, by_group=True, batch=8)
+    d = oracle.make_desc((c, h, w), c, (3, 3), (1, 1), (stride, stride), pads, 0.0, 1, c, term, act, (0.0, 6.0))
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, c, (3, 3), (1, 1), (stride, stride), pads, 0.0, c, term, act, (0.0, 6.0))
+    for i in (0, 3, 7):
+        want = oracle.convolutiondepthwise_int8(d, x[i], wq, b, ws, ins, tops)
+        assert got.dtype == want.dtype and np.array_equal(got[i], want)
+
+
 @pytest.mark.parametrize("kind,k,s,pt,pl,include_pad", [(0, (3, 3), (2, 2), 0, 0, 0), (0, (3, 3), (2, 2), 1, 1, 0), (0, (2, 3), (1, 2), 0, 1, 0),
                                                          (1, (3, 3), (2, 2), 1, 1, 0), (1, (3, 3), (1, 1), 1, 1, 1), (1, (2, 2), (2, 2), 0, 0, 0)])
 def test_pooling_matches_scalar_restatement(rt, kind, k, s, pt, pl, include_pad):
