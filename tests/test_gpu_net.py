@@ -299,6 +299,29 @@ def test_benchmark_network_batch1_matches_oracle_executor(which, hw):
     assert np.array_equal(got[1].reshape(-1), ex1.extract(last_fc).reshape(-1))
 
 
+@pytest.mark.parametrize("which,batch", [("mobilenetv2", 32), ("resnet50", 16)])
+def test_benchmark_batch_equals_the_per_sample_passes(which, batch):
+    """At the benchmark's batch sizes the kernels take other variants than at batch 1 (several output rows per
+    depthwise thread, the pointwise small-K kernel, other tiles and K splits).  Batch 1 is pinned on the oracle
+    executor above; here the folded batch must reproduce, bit for bit, the logits and a requantised blob deep in the
+    net of single-sample passes (samples 0, a middle one, the last)."""
+    _say("building", which)
+    g, param, blob, info = zoo.build(which, input_hw=224, n_calib=1)
+    net = _load(param, blob, True)
+    xs = np.random.default_rng(21).uniform(0, 1, (batch,) + tuple(g.input_shape)).astype(F)
+    last_fc = "fc1000" if which == "resnet50" else "fc"
+    probe = "res2b_branch2b" if which == "resnet50" else "block2_dw"
+    for name in (last_fc, probe):
+        ex = net.create_extractor()
+        ex.input("data", xs)
+        got = np.asarray(ex.extract(name))
+        assert got.shape[0] == batch
+        for i in (0, batch // 2 - 1, batch - 1):
+            ex1 = net.create_extractor()
+            ex1.input("data", xs[i])
+            assert np.array_equal(got[i].reshape(-1), np.asarray(ex1.extract(name)).reshape(-1)), (name, i)
+
+
 @pytest.mark.parametrize("which,batch", [("tiny", 1), ("tiny", 3), ("mobilenetv2", 1), ("resnet50", 2)])
 def test_recorded_pass_replays_like_the_eager_pass(which, batch):
     """A pass recorded into a graph and replayed: every replay, with new input values and with eager work and
