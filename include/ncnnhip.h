@@ -230,6 +230,10 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
  * Quantize(maxpool(x), s), because rounding and clamping are monotonic (for |x*s| < 2^31; the caller knows a bound).  Lets a requantising convolution feed the
  * quantising consumers of its pooled output without an fp32 blob in between. */
 int ncnnhip_maxpool_nhwc_int8(const ncnnhip_pool_desc* desc, const int8_t* src_dev, int8_t* dst_dev, void* stream);
+/* Global pooling (src/layer/pooling.cpp:60-103) followed by the consumer's Quantize (src/layer/quantize.cpp:29-60, one
+ * scale for the tensor): dst[n][c] = float2int8(pool(x) * scale), dense int8.  Lets the pooled vector reach an int8
+ * InnerProduct without an fp32 blob and a Quantize launch in between. */
+int ncnnhip_global_pooling_nhwc_quantised(const ncnnhip_pool_desc* desc, const float* src_dev, float scale, int8_t* dst_dev, void* stream);
 /* Softmax::forward_inplace (src/layer/softmax.cpp) over a dense vector of `count` values per sample. */
 int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream);
 

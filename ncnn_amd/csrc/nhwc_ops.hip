@@ -269,7 +269,9 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(const int8_t* __re
 }
 
 // global pooling: [n][hw][cp] -> dense [n][c]; one thread per (sample, channel) walks the pixels in index order
-__global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type)
+// (q8 != 0: the quantised value float2int8(result * q8_scale) is stored instead, for a consumer that would quantise it so)
+__global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, int c, int hw, int cp, int type,
+                                                                int8_t* __restrict__ q8, float q8_scale)
 {
     const int q = blockIdx.x * 64 + threadIdx.x; // one wavefront per workgroup: the few channels spread over as many CUs as possible
     const int img = blockIdx.y;
@@ -288,7 +290,10 @@ __global__ __launch_bounds__(64) void global_pooling_nhwc_kernel(const float* __
     }
     for (; i < hw; i++) r = type == 0 ? fmaxf(r, p[(size_t)i * cp]) : add_rn(r, p[(size_t)i * cp]);
     if (type != 0) r = div_rn(r, (float)hw);
-    dst[(size_t)img * c + q] = r;
+    if (q8)
+        q8[(size_t)img * c + q] = (int8_t)float2int8(mul_rn(r, q8_scale));
+    else
+        dst[(size_t)img * c + q] = r;
 }
 
 // ---- Softmax over a dense vector (src/layer/softmax.cpp), one workgroup per sample
@@ -712,7 +717,8 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
     if (d.global_pooling)
     {
         NCNNHIP_REQUIRE(d.batch <= 65535, "ncnnhip_pooling_nhwc: batch above 65535");
-        hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 64), d.batch), dim3(64), 0, as_stream(stream), src_dev, dst_dev, d.c, d.w * d.h, cp, d.pooling_type);
+        hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 64), d.batch), dim3(64), 0, as_stream(stream), src_dev, dst_dev, d.c, d.w * d.h, cp, d.pooling_type,
+                           (int8_t*)0, 0.f);
         return launch_status("global_pooling_nhwc_kernel");
     }
     NCNNHIP_REQUIRE(d.kernel_w > 0 && d.kernel_h > 0 && d.stride_w > 0 && d.stride_h > 0 && d.outw > 0 && d.outh > 0, "ncnnhip_pooling_nhwc: bad window");
@@ -762,6 +768,17 @@ int ncnnhip_maxpool_nhwc_int8(const ncnnhip_pool_desc* desc, const int8_t* src_d
     const size_t total = (size_t)d.batch * d.outh * d.outw * (g.cp / 16);
     hipLaunchKernelGGL(maxpool_nhwc_s8_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
     return launch_status("maxpool_nhwc_s8_kernel");
+}
+
+int ncnnhip_global_pooling_nhwc_quantised(const ncnnhip_pool_desc* desc, const float* src_dev, float scale, int8_t* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && src_dev && dst_dev, "ncnnhip_global_pooling_nhwc_quantised: null pointer");
+    const ncnnhip_pool_desc& d = *desc;
+    NCNNHIP_REQUIRE(d.w > 0 && d.h > 0 && d.c > 0 && d.batch > 0 && d.batch <= 65535 && (d.pooling_type == 0 || d.pooling_type == 1),
+                    "ncnnhip_global_pooling_nhwc_quantised: bad shape or pooling type");
+    hipLaunchKernelGGL(global_pooling_nhwc_kernel, dim3(ceil_div(d.c, 64), d.batch), dim3(64), 0, as_stream(stream), src_dev, (float*)0, d.c, d.w * d.h, padded16(d.c),
+                       d.pooling_type, dst_dev, scale);
+    return launch_status("global_pooling_nhwc_kernel");
 }
 
 int ncnnhip_softmax(const float* src_dev, float* dst_dev, int count, int batch, void* stream)

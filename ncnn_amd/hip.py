@@ -106,6 +106,7 @@ _SIGNATURES = {
                                C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_pooling_nhwc": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
     "ncnnhip_maxpool_nhwc_int8": [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_global_pooling_nhwc_quantised": [C.POINTER(PoolDesc), C.c_void_p, C.c_float, C.c_void_p, C.c_void_p],
     "ncnnhip_softmax": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "ncnnhip_innerproduct_int8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation,
                                   C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -382,6 +383,16 @@ class Runtime:
         out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.int8)
         check(lib().ncnnhip_maxpool_nhwc_int8(C.byref(d), src.ptr, out.ptr, self.stream))
         return self.from_channels_last(out, n, c, oh, ow)
+
+    def global_pooling_quantised(self, x, pooling_type, scale):
+        """x [n][c][h][w] fp32 -> [n][c] int8 = float2int8(global pool * scale)."""
+        x = np.ascontiguousarray(x, np.float32)
+        n, c, h, w = x.shape
+        src = self.to_channels_last(x)
+        d = PoolDesc(w, h, c, n, pooling_type, 0, 0, 1, 1, 0, 0, 1, 1, 1, 0)
+        out = DeviceBuffer.empty((n, c), np.int8)
+        check(lib().ncnnhip_global_pooling_nhwc_quantised(C.byref(d), src.ptr, float(scale), out.ptr, self.stream))
+        return out.to_numpy(self.stream)
 
     def attention(self, q, kt, vt, num_heads, mask=None, use_workspace=True):
         """q [src][embed] (scaled), kt / vt [embed][dst], mask [src][dst] or [heads][src][dst] -> [src][embed]."""

@@ -213,6 +213,34 @@ public:
         return support_hip && pooling_type == 0 && !global_pooling;
     }
 
+    // Global pooling can hand its consumers the quantised vector directly: float2int8(pool(x) * scale), the value
+    // their own Quantize would compute from the fp32 result.
+    virtual int hip_prepare_requantise(float scale)
+    {
+        return (support_hip && global_pooling && scale > 0.f) ? 0 : -1;
+    }
+    virtual int forward_hip_requantised(const HipMat& bottom, float scale, HipMat& top, HipCommand& cmd, const Option&) const
+    {
+        if (!global_pooling || bottom.dims != 3 || bottom.elemsize != 4u)
+        {
+            NCNN_LOGE("Pooling: the quantised form needs global pooling of a 3-D fp32 blob");
+            return -1;
+        }
+        ncnnhip_pool_desc d;
+        memset(&d, 0, sizeof(d));
+        d.w = bottom.w;
+        d.h = bottom.h;
+        d.c = bottom.c;
+        d.batch = bottom.n;
+        d.pooling_type = pooling_type;
+        d.global_pooling = 1;
+        top.create(bottom.c, 1u, bottom.n, &cmd);
+        if (top.empty()) return -100;
+        top.q8_scale = scale;
+        return dev_status(ncnnhip_global_pooling_nhwc_quantised(&d, (const float*)bottom.data, scale, (int8_t*)top.data, cmd.stream),
+                          "ncnnhip_global_pooling_nhwc_quantised");
+    }
+
     virtual int forward_hip(const HipMat& bottom, HipMat& top, HipCommand& cmd, const Option&) const
     {
         // an int8 blob only arrives here when the executor routed quantised values through this layer

@@ -75,6 +75,7 @@ public:
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
     virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
+    virtual float hip_input_quantise_scale() const;
 
 public:
     int num_output, bias_term, weight_data_size, int8_scale_term, activation_type;

@@ -223,6 +223,13 @@ int InnerProduct_hip::forward_hip(const HipMat& bottom, HipMat& top, HipCommand&
     return to_ncnn_status(rc, "ncnnhip_innerproduct_int8_ws");
 }
 
+// The layer quantises an fp32 bottom with this one scale (Quantize with a single scale, as InnerProduct::forward_int8
+// does, src/layer/innerproduct.cpp:231-247): a producer that can emit float2int8(value * scale) itself may do so.
+float InnerProduct_hip::hip_input_quantise_scale() const
+{
+    return (support_hip && d_weight && bottom_blob_int8_scales.w > 0) ? bottom_blob_int8_scales[0] : 0.f;
+}
+
 Layer* InnerProduct_hip_creator(void*)
 {
     return new InnerProduct_hip;

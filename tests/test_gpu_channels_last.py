@@ -234,6 +234,22 @@ def test_global_pooling(rt, kind):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("kind", [0, 1])
+def test_global_pooling_quantised_is_quantize_of_the_pooled_vector(rt, kind):
+    """Global pooling that hands an int8 InnerProduct its input: float2int8(pool(x) * scale), the pooled value computed
+    as the fp32 entry point computes it (sequential sum, one division), quantised as Quantize would (the oracle)."""
+    rng = np.random.default_rng(10 + kind)
+    x = rng.normal(0, 1, (3, 70, 7, 7)).astype(F)
+    x[0, 0] = 1e9       # beyond the clamp
+    x[1, 3] = -0.0131   # a small negative mean
+    scale = F(37.3)
+    flat = x.reshape(3, 70, 49)
+    pooled = flat.max(axis=2) if kind == 0 else (np.cumsum(flat, axis=2, dtype=F)[..., -1] / F(49)).astype(F)
+    want = oracle.quantize(pooled.reshape(1, -1), np.array([scale], F)).reshape(3, 70)
+    got = rt.global_pooling_quantised(x, kind, scale)
+    assert got.dtype == np.int8 and np.array_equal(got, want)
+
+
 def test_relu_and_leaky_relu(rt):
     rng = np.random.default_rng(3)
     x = rng.normal(0, 1, 4096).astype(F)
