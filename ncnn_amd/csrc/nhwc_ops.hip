@@ -232,22 +232,32 @@ __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restri
 // Max pooling of an int8 blob, 16 channels of one output pixel per thread.  Quantize (round, clamp to [-127,127]) is
 // monotonic for a positive scale, so the maximum of the quantised values is the quantised maximum; a window without
 // any pixel gives -127, which is what -FLT_MAX quantises to.
-__global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, PoolGeom g, size_t total)
+// The 16 bytes are compared as eight pairs of 16-bit lanes: the even bytes of a dword moved into the high byte of
+// each half (v << 8, low bytes cleared), the odd bytes kept where they are (low bytes cleared); a signed 16-bit
+// maximum (v_pk_max_i16) of two such values whose low bytes are zero orders them like the signed bytes on top.
+// blockIdx.y = output row, blockIdx.z = sample: no division except the channel-group split of the column index.
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_i16(uint32_t a, uint32_t b)
 {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const int groups = g.cp / 16;
-    const int q16 = (int)(i % (size_t)groups);
-    size_t rest = i / (size_t)groups;
-    const int ox = (int)(rest % (size_t)g.outw);
-    rest /= (size_t)g.outw;
-    const int oy = (int)(rest % (size_t)g.outh);
-    const int img = (int)(rest / (size_t)g.outh);
+    const v2s x = __builtin_bit_cast(v2s, a), y = __builtin_bit_cast(v2s, b);
+    const v2s m = {x[0] > y[0] ? x[0] : y[0], x[1] > y[1] ? x[1] : y[1]};
+    return __builtin_bit_cast(uint32_t, m);
+}
+
+__global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, PoolGeom g, unsigned groups, unsigned groups_magic)
+{
+    const unsigned r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= (unsigned)g.outw * groups) return;
+    unsigned ox = groups == 1 ? r : __umulhi(r, groups_magic); // r / groups; exact: r * groups < 2^32 (checked at launch)
+    if (ox * groups > r) ox--;
+    const unsigned q16 = r - ox * groups;
+    const int oy = blockIdx.y, img = blockIdx.z;
     const int8_t* base = src + (size_t)img * g.h * g.w * g.cp + q16 * 16;
-    const int y0 = oy * g.sh - g.pad_top, x0 = ox * g.sw - g.pad_left;
-    int r[16];
+    const int y0 = oy * g.sh - g.pad_top, x0 = (int)ox * g.sw - g.pad_left;
+    const uint32_t lowest = 0x81008100u; // -127 in the high byte of both halves
+    uint32_t even[4], odd[4];
 #pragma unroll
-    for (int e = 0; e < 16; e++) r[e] = -127;
+    for (int d = 0; d < 4; d++) even[d] = odd[d] = lowest;
     for (int ky = 0; ky < g.kh; ky++)
         for (int kx = 0; kx < g.kw; kx++)
         {
@@ -255,16 +265,17 @@ __global__ __launch_bounds__(256) void maxpool_nhwc_s8_kernel(const int8_t* __re
             const bool in = (unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w;
             const v4i v = *reinterpret_cast<const v4i*>(base + (in ? ((size_t)y * g.w + x) * g.cp : (size_t)0)); // unconditional: loads overlap
 #pragma unroll
-            for (int e = 0; e < 16; e++)
+            for (int d = 0; d < 4; d++)
             {
-                const int b = (int)(int8_t)((unsigned)v[e >> 2] >> (8 * (e & 3)));
-                r[e] = in ? (b > r[e] ? b : r[e]) : r[e];
+                // a tap outside the image contributes -127, which changes no maximum
+                const uint32_t w = in ? (uint32_t)v[d] : 0x81818181u;
+                even[d] = pk_max_i16(even[d], (w << 8) & 0xff00ff00u);
+                odd[d] = pk_max_i16(odd[d], w & 0xff00ff00u);
             }
         }
     v4i o;
 #pragma unroll
-    for (int d = 0; d < 4; d++)
-        o[d] = (int)((unsigned)(r[4 * d] & 255) | ((unsigned)(r[4 * d + 1] & 255) << 8) | ((unsigned)(r[4 * d + 2] & 255) << 16) | ((unsigned)r[4 * d + 3] << 24));
+    for (int d = 0; d < 4; d++) o[d] = (int)(((even[d] >> 8) & 0x00ff00ffu) | odd[d]);
     *reinterpret_cast<v4i*>(dst + (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q16 * 16) = o;
 }
 
@@ -765,8 +776,11 @@ int ncnnhip_maxpool_nhwc_int8(const ncnnhip_pool_desc* desc, const int8_t* src_d
     g.pad_left = d.pad_left;
     g.type = 0;
     g.count_include_pad = 0;
-    const size_t total = (size_t)d.batch * d.outh * d.outw * (g.cp / 16);
-    hipLaunchKernelGGL(maxpool_nhwc_s8_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
+    const unsigned groups = (unsigned)g.cp / 16;
+    NCNNHIP_REQUIRE(d.batch <= 65535 && d.outh <= 65535 && (unsigned long long)d.outw * groups * groups < (1ull << 32), "ncnnhip_maxpool_nhwc_int8: extent too large");
+    const unsigned groups_magic = groups > 1 ? (unsigned)(((1ull << 32) + groups - 1) / groups) : 0u;
+    hipLaunchKernelGGL(maxpool_nhwc_s8_kernel, dim3(ceil_div((long long)d.outw * groups, 256), (unsigned)d.outh, (unsigned)d.batch), dim3(256), 0, as_stream(stream),
+                       src_dev, dst_dev, g, groups, groups_magic);
     return launch_status("maxpool_nhwc_s8_kernel");
 }
 
