@@ -247,6 +247,26 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     const unsigned rd_b = (unsigned)(BM * 64 + (wn * (BN / 2) + l32) * 64);
     const unsigned ch0 = (unsigned)(((0 + lhi) ^ sw) * 16), ch1 = (unsigned)(((2 + lhi) ^ sw) * 16);
 
+    // The epilogue's per-channel tables are requested now, before the first stage, so that they arrive during the K
+    // loop instead of costing a memory latency after it (a layer with a handful of K steps is little more than the
+    // sum of its latencies).  Only the raw loads happen here, from clamped indices and always-valid pointers: a select
+    // or a branch on the values would make the wavefront wait for them on the spot.
+    float raw_s_in[BN / 64], raw_bias[BN / 64], raw_s_out[BN / 64];
+    if (!GEMM)
+    {
+        const float* bias_src = epi.bias ? epi.bias : epi.scale_in;
+        const float* s_out_src = epi.scale_out ? epi.scale_out : epi.scale_in;
+#pragma unroll
+        for (int c = 0; c < BN / 64; c++)
+        {
+            int ch = col0 + wn * (BN / 2) + c * 32 + l32;
+            if (ch >= g.cout) ch = g.cout - 1;
+            raw_s_in[c] = epi.scale_in[ch];
+            raw_bias[c] = bias_src[ch];
+            raw_s_out[c] = s_out_src[ch];
+        }
+    }
+
 #pragma unroll
     for (int s = 0; s < STAGES - 1; s++)
         if (s < nk) issue(s);
@@ -364,10 +384,10 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
         else
         {
-            s_in[c] = real[c] ? epi.scale_in[ch] : 0.f;
+            s_in[c] = real[c] ? raw_s_in[c] : 0.f;
             // no bias: -0, the one value whose addition changes nothing (x + -0 = x for every x, -0 included)
-            bias[c] = (real[c] && epi.bias) ? epi.bias[ch] : -0.f;
-            s_out[c] = (real[c] && to_int8) ? epi.scale_out[ch] : 0.f;
+            bias[c] = (real[c] && epi.bias) ? raw_bias[c] : -0.f;
+            s_out[c] = (real[c] && to_int8) ? raw_s_out[c] : 0.f;
         }
     }
     if (GEMM)
