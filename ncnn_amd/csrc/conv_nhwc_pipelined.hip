@@ -450,6 +450,24 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 #pragma unroll
         for (int a = 0; a < TM; a++)
         {
+            // The residual this lane will add in the read-out below is requested now, so that it arrives while the
+            // accumulators are being converted (clamped addresses, nothing selected: see the tables above).
+            v4f resv[G / 2];
+            const bool with_residual = !to_int8 && fusion.residual != 0;
+            if (with_residual)
+            {
+#pragma unroll
+                for (int it = 0; it < G / 2; it++)
+                {
+                    const int idx = it * 64 + lane;
+                    const int p = idx / G, j = idx - p * G;
+                    int pix = row0 + wm * (BM / 2) + a * 32 + p;
+                    int ch4 = col0 + wn * CW + 4 * j;
+                    if (pix >= g.npix) pix = g.npix - 1;
+                    if (ch4 >= col_limit) ch4 = col_limit - 4;
+                    resv[it] = *reinterpret_cast<const v4f*>(fusion.residual + (size_t)pix * out_cp + ch4);
+                }
+            }
 #pragma unroll
             for (int c = 0; c < TN; c++)
             {
@@ -538,11 +556,10 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 {
                     const size_t o = (size_t)pix * out_cp + ch4;
                     {
-                        if (fusion.residual)
+                        if (with_residual)
                         {
-                            const v4f res = *reinterpret_cast<const v4f*>(fusion.residual + o);
 #pragma unroll
-                            for (int e = 0; e < 4; e++) v[e] = add_rn(v[e], res[e]);
+                            for (int e = 0; e < 4; e++) v[e] = add_rn(v[e], resv[it][e]);
                         }
                         if (fusion.relu_after)
                         {
