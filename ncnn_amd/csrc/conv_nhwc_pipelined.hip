@@ -631,10 +631,11 @@ static PipePlan plan_pipelined(int cout, long long npix, int steps)
     p.tiles_n = ceil_div(cout, p.bn);
     p.splits = 1;
     const long long t = tiles();
-    if (t < 128 && t <= SPLIT_MAX_TILES && steps >= 16)
+    if (t < 256 && t <= SPLIT_MAX_TILES && steps >= 16)
     {
-        // too few tiles to occupy the chip: split K until there is about one workgroup per CU, at least 8 steps each
-        // (measured best over the ResNet-50 / MobileNetV2 layers at batch 1 and 16)
+        // fewer tiles than CUs: split K until there is about one workgroup per CU (two splits from 128 tiles up), at
+        // least 8 steps each (measured best over the ResNet-50 / MobileNetV2 layers at batch 1 and 16; with the limit at
+        // 128 tiles the 196-tile 3x3 layers of ResNet-50's fourth stage at batch 16 ran unsplit on 196 of the 256 CUs)
         const int want = (int)((256 + t - 1) / t);
         const int max_splits = steps / 8;
         p.splits = want < max_splits ? want : max_splits;
