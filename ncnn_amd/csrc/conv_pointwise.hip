@@ -196,7 +196,7 @@ bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvF
     const bool plain = !fusion.residual && !fusion.relu_after && !fusion.q8_out && !epi.acc_out;
     const uintptr_t tables = reinterpret_cast<uintptr_t>(epi.scale_in) | reinterpret_cast<uintptr_t>(epi.bias) | reinterpret_cast<uintptr_t>(epi.scale_out);
     const bool aligned = ((tables | reinterpret_cast<uintptr_t>(epi.out)) & 15) == 0; // 16-byte table loads and stores
-    return dense && plain && aligned && epi.scale_out && g.Cp <= 64 && g.Cp % 16 == 0 && g.K == 64 && g.cout % 4 == 0 && out_cp % 16 == 0 && g.npix >= (1 << 17); // below that the general kernel's finer split of the work is as fast or faster
+    return dense && plain && aligned && epi.scale_out && g.Cp <= 64 && g.Cp % 16 == 0 && g.K == 64 && g.cout % 4 == 0 && out_cp % 16 == 0 && g.npix >= (1 << 16); // below that the general kernel's finer split of the work is as fast or faster
 }
 
 int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream)
@@ -204,10 +204,10 @@ int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x,
     NCNNHIP_REQUIRE(((reinterpret_cast<uintptr_t>(wpk) | reinterpret_cast<uintptr_t>(x)) & 15) == 0, "convolution: operands must be 16-byte aligned");
     const int channel_blocks = out_cp / 16;
     const int pixel_blocks = ceil_div(g.npix, 64);
-    // long runs amortise the wavefront's weights and tables; short ones fill the chip: aim at two rounds of the 4096+
-    // wavefronts the chip holds
+    // long runs amortise the wavefront's weights and tables; short ones fill the chip: at least 4096 wavefronts, about
+    // what the chip holds at once (measured best against 2048, 3072, 6144 and 8192 on MobileNetV2's layers at batch 32)
     int blocks_per_wave = 16;
-    while (blocks_per_wave > 2 && (long long)ceil_div(pixel_blocks, blocks_per_wave) * channel_blocks < 8192) blocks_per_wave /= 2;
+    while (blocks_per_wave > 2 && (long long)ceil_div(pixel_blocks, blocks_per_wave) * channel_blocks < 4096) blocks_per_wave /= 2;
     const long long waves = (long long)ceil_div(pixel_blocks, blocks_per_wave) * channel_blocks;
     NCNNHIP_REQUIRE(waves * channel_blocks < (1ll << 32), "convolution: too many tiles");
     const unsigned cb_magic = channel_blocks > 1 ? (unsigned)((1ull << 32) / (unsigned)channel_blocks + 1) : 0u;

@@ -107,7 +107,7 @@ def test_clip_is_the_reference_clip_whatever_its_bounds(rt, act_params, term, bi
     (8, 16, 2, (0.1, 0.0), False),      # leaky ReLU: the general activation path
 ])
 def test_pointwise_small_k_kernel_matches_oracle(rt, c, outc, act, act_params, flip):
-    """1x1 layers with at most 64 input channels, int8 output and 2^17 pixels or more take a kernel of their own
+    """1x1 layers with at most 64 input channels, int8 output and 2^16 pixels or more take a kernel of their own
     (MFMA fed weights-first, no LDS, lane-row transposes before the store): ragged pixel count, batch 2."""
     _say("pointwise small-K", c, outc, act, act_params, flip)
     h = w = 257
