@@ -67,14 +67,19 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     const int ld_row = wave * 16 + (lane >> 2);                 // + i*64
     const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);        // swizzled source chunk
     const int8_t* ga = A + ((size_t)tile_m * PT + ld_row) * lda + ld_chunk * 16;
-    const int8_t* gb = B + ((size_t)tile_n * PT + ld_row) * ldb + ld_chunk * 16;
-    const size_t a_step = 64 * lda, b_step = 64 * ldb;
+    // B rows are permuted on their way into LDS: LDS row wn*128 + j*32 + l holds B row wn*128 + 4*l + j, so that the four
+    // accumulator blocks j of a lane are four consecutive output columns and the epilogue stores 16 bytes per lane.
+    // LDS row of this lane in quarter i = i*64 + wave*16 + (lane >> 2): wn = i >> 1, j = (i & 1)*2 + (wave >> 1),
+    // l = (wave & 1)*16 + (lane >> 2).
+    const int ld_row_b = 4 * ((wave & 1) * 16 + (lane >> 2)) + (wave >> 1); // + (i >> 1)*128 + (i & 1)*2
+    const int8_t* gb = B + ((size_t)tile_n * PT + ld_row_b) * ldb + ld_chunk * 16;
+    const size_t a_step = 64 * lda;
 
     // quarter i of the loads of step t: 16 A rows and 16 B rows per wave
     auto issue_quarter = [&](int t, int i) {
         int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024 + i * 4096;
         __builtin_amdgcn_global_load_lds((const AS1 void*)(ga + (size_t)t * PK + i * a_step), (AS3 void*)sa, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const AS1 void*)(gb + (size_t)t * PK + i * b_step), (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const AS1 void*)(gb + (size_t)t * PK + (size_t)((i >> 1) * 128 + (i & 1) * 2) * ldb), (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
     };
     auto issue_stage = [&](int t) {
 #pragma unroll
@@ -204,36 +209,49 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     for (; t < nk; t++) k_step(t, std::false_type{});
 
     // ---- fused epilogue: dequantise, bias, scale, store fp32
-    const int row_base = tile_m * PT + wm * 128 + 4 * lhi;
-    const int col_base = tile_n * PT + wn * 128 + l32;
+    const int col_base = tile_n * PT + wn * 128 + 4 * l32; // accumulator block j of this lane is column col_base + j
     float colscale[4], colc[4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
     {
-        const int col = col_base + j * 32;
+        const int col = col_base + j;
         colscale[j] = PER_COL ? div_rn(1.f, b_scales[col]) : 0.f;
         colc[j] = BT == 4 ? mul_rn(cvec[col], beta) : 0.f;
     }
-    const float sb0 = b_scales[0];
+    // one descale per row of the tile, computed once by thread `row` and handed round through LDS (the stages are free
+    // once every wavefront has left the K loop)
+    float* rowscale_lds = reinterpret_cast<float*>(smem);
+    {
+        const float sa = a_scales[tile_m * PT + threadIdx.x];
+        const float rs = PER_COL ? div_rn(1.f, sa) : div_rn(1.f, mul_rn(sa, b_scales[0]));
+        __builtin_amdgcn_s_barrier();
+        rowscale_lds[threadIdx.x] = rs;
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++)
     {
 #pragma unroll
         for (int r = 0; r < 16; r++)
         {
-            const int row = row_base + i * 32 + 8 * (r >> 2) + (r & 3);
-            const float sa = a_scales[row];
-            const float rowscale = PER_COL ? div_rn(1.f, sa) : div_rn(1.f, mul_rn(sa, sb0));
-            float* orow = out + (size_t)row * ldo + col_base;
+            const int row_in_tile = wm * 128 + 4 * lhi + i * 32 + 8 * (r >> 2) + (r & 3);
+            const float rowscale = rowscale_lds[row_in_tile];
+            float* orow = out + (size_t)(tile_m * PT + row_in_tile) * ldo + col_base;
+            float f4[4];
 #pragma unroll
             for (int j = 0; j < 4; j++)
             {
                 float f = mul_rn((float)acc[i][j][r], rowscale);
                 if (PER_COL) f = mul_rn(f, colscale[j]);
                 if (BT == 4) f = add_rn(f, colc[j]);
-                f = mul_rn(f, alpha);
-                orow[j * 32] = f;
+                f4[j] = mul_rn(f, alpha);
             }
+#ifdef GEMM_NT_STORE
+            typedef float v4f_store __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store((v4f_store){f4[0], f4[1], f4[2], f4[3]}, reinterpret_cast<v4f_store*>(orow));
+#else
+            *reinterpret_cast<float4*>(orow) = make_float4(f4[0], f4[1], f4[2], f4[3]);
+#endif
         }
     }
 }
@@ -249,6 +267,7 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
     *handled = false;
     if (M % PT || N % PT || K % PK || aq_stride % 16 || bq_stride % 16 || !al16(aq) || !al16(bq)) return NCNNHIP_OK;
     if (epi.transpose || epi.acc_out || !(epi.bt == -1 || epi.bt == 4)) return NCNNHIP_OK;
+    if (epi.out_stride % 4 || !al16(epi.out)) return NCNNHIP_OK; // the epilogue stores 16 bytes per lane
     const int tm = M / PT, tn = N / PT, nk = K / PK;
     if ((long long)tm * tn > 0x7fffffff) return NCNNHIP_OK;
     *handled = true;

@@ -119,8 +119,16 @@ def gemm_quantize_rows(a):
     return float2int8(a * s[:, None]), s
 
 
-def gemm_int8(aq, bq, a_scales, b_scales, c=None, bt=-1, alpha=1.0, beta=1.0, transpose=False):
-    acc = aq.astype(np.int64) @ bq.astype(np.int64).T
+def gemm_acc_exact(aq, bq):
+    """int8 x int8 accumulators through a float64 BLAS matmul: every partial sum is an integer below 127*127*K < 2^53,
+    so no rounding happens whatever the summation order (fast enough for the 4096-cube benchmark size)."""
+    assert aq.shape[1] * 127 * 127 < 2 ** 53
+    return (aq.astype(np.float64) @ bq.astype(np.float64).T).astype(np.int64)
+
+
+def gemm_int8(aq, bq, a_scales, b_scales, c=None, bt=-1, alpha=1.0, beta=1.0, transpose=False, acc=None):
+    if acc is None:
+        acc = aq.astype(np.int64) @ bq.astype(np.int64).T
     m, n = acc.shape
     a_scales = np.asarray(a_scales, np.float32)
     b_scales = np.asarray(b_scales, np.float32).reshape(-1)

@@ -41,7 +41,7 @@ def test_quantize_matches_oracle(rt):
 
 
 # ----------------------------------------------------------------------------- gemm
-@pytest.mark.parametrize("m,k", [(5, 77), (9, 4096), (16, 4100), (33, 513)])
+@pytest.mark.parametrize("m,k", [(5, 77), (9, 4096), (16, 4100), (33, 513), (8200, 4096)])  # the last one is above 128 MB: non-temporal loads
 def test_gemm_quantize_rows(rt, m, k):
     _say("gemm_quantize_rows", m, k)
     a = np.random.default_rng(m * k).standard_normal((m, k), dtype=F)
@@ -116,6 +116,27 @@ def test_gemm_int8_1024_cube_against_numpy_int_matmul(rt):
     want, wacc = npref.gemm_int8(aq, bq, sa, sb, bias, 4)
     assert np.array_equal(gacc, wacc)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 64), (4096, 2048, 192), (2304, 3840, 320), (4096, 4096, 4096)])
+@pytest.mark.parametrize("bt,per_col", [(4, True), (-1, False)])
+def test_gemm_int8_256x256_kernel_sizes(rt, m, n, k, bt, per_col):
+    """From 128 tiles of 256 x 256 up (K % 64 == 0) the Gemm runs on the 256x256 ring kernel: one, three and five K steps
+    (shorter than, equal to and longer than the ring's prologue), a tile count that is not a multiple of 8 with a ragged last
+    row group, and the benchmark's own 4096 cube.  Every output element is compared; the accumulators come from a float64
+    matmul, which is exact here, and the 2048 x 4096 x 64 case is also checked against the scalar oracle."""
+    _say("gemm_int8 256x256", m, n, k, bt, per_col)
+    a, bq, sb, bias = cases.gemm_case(m + 3 * n + 7 * k, m, n, k, per_col)
+    c = bias.reshape(1, n) if bt == 4 else None
+    aq, sa = rt.gemm_quantize_rows(a)
+    oq, os_ = oracle.gemm_quantize_rows(a)
+    assert np.array_equal(aq, oq) and np.array_equal(sa, os_)
+    acc = npref.gemm_acc_exact(aq, bq)
+    want, _ = npref.gemm_int8(aq, bq, sa, sb, c, bt, acc=acc)
+    got = rt.gemm_int8(aq, bq, sa, sb, c, bt)
+    assert np.array_equal(got, want)
+    if k == 64 and not per_col:
+        assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, sb, c, bt))
 
 
 # ----------------------------------------------------------------------------- convolution
