@@ -277,6 +277,21 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
                       int broadcast_type_c, float alpha, float beta, int output_transpose, float* out_dev,
                       size_t out_stride, int32_t* acc_out_dev, void* stream);
 
+/* The same Gemm on operands in the 256x256 kernel's own layout, for the form a network layer has (dynamic A, constant B;
+ * gemm.cpp:745-966 with constantB=1, transB=1): element (r, k) of a tiled operand lies at
+ * ((r / 256 * (K / 64) + k / 64) * 256 + r % 256) * 64 + k % 64 (the B operand with its rows interleaved inside a tile, which
+ * ncnnhip_gemm_int8_tile_operand does), rows * K bytes, rows % 256 == 0, K % 64 == 0.  One K step of a tile is then 16 KB
+ * of consecutive memory instead of 256 pieces of 64 bytes.  B is tiled once where the weights are uploaded
+ * (create_pipeline), A is written tiled by the quantiser.  Results are those of ncnnhip_gemm_int8 bit for bit.
+ * operand: 0 = A, 1 = B.  C: none or per column (broadcast_type_c 4). */
+int ncnnhip_gemm_int8_tile_operand(const int8_t* src_dev, size_t src_stride, int rows, int K, int operand, int8_t* dst_dev,
+                                   void* stream);
+int ncnnhip_gemm_quantize_rows_tiled(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_tiled_dev,
+                                     float* scales_dev, void* stream);
+int ncnnhip_gemm_int8_tiled(const int8_t* aq_tiled_dev, const int8_t* bq_tiled_dev, int M, int N, int K,
+                            const float* a_scales_dev, const float* b_scales_dev, int n_b_scales, const float* c_dev,
+                            int broadcast_type_c, float alpha, float beta, float* out_dev, size_t out_stride, void* stream);
+
 /* ------------------------------------------------------------------ block-quantised Gemm
  * Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483): a fp32 [M][K];
  * b packed [N][ceil(K*bits/8)] LSB-first `bits`-wide signed fields (bits 4/6/8);

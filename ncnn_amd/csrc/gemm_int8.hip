@@ -83,6 +83,9 @@ static DenseOperand make_dense(const int8_t* base, size_t stride, int rows, int 
 int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K,
                                const GemmEpilogue& epi, hipStream_t stream, bool* handled);
 
+int launch_gemm_int8_tiled(const int8_t* aq_tiled, const int8_t* bq_tiled, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream);
+int launch_gemm_tile_operand(const int8_t* src, size_t stride, int rows, int K, int operand_b, int8_t* dst, hipStream_t stream);
+
 } // namespace ncnnhip
 
 using namespace ncnnhip;
@@ -214,6 +217,44 @@ int ncnnhip_innerproduct_int8_ws(const int8_t* x_dev, size_t x_stride, int rows,
         if (handled) return ret;
     }
     return ncnnhip_innerproduct_int8(x_dev, x_stride, rows, num_input, num_output, weight_dev, scale_in_dev, bias_dev, act, out_dev, out_stride, 0, stream);
+}
+
+int ncnnhip_gemm_int8_tile_operand(const int8_t* src_dev, size_t src_stride, int rows, int K, int operand, int8_t* dst_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(src_dev && dst_dev, "ncnnhip_gemm_int8_tile_operand: null pointer");
+    NCNNHIP_REQUIRE(rows >= 256 && rows % 256 == 0 && K >= 64 && K % 64 == 0, "ncnnhip_gemm_int8_tile_operand: %d rows of %d (multiples of 256 and 64 only)", rows, K);
+    NCNNHIP_REQUIRE(operand == 0 || operand == 1, "ncnnhip_gemm_int8_tile_operand: operand %d (0 = A, 1 = B)", operand);
+    NCNNHIP_REQUIRE(src_stride >= (size_t)K && src_stride % 16 == 0 && aligned16(src_dev) && aligned16(dst_dev),
+                    "ncnnhip_gemm_int8_tile_operand: rows must be 16-byte aligned");
+    return launch_gemm_tile_operand(src_dev, src_stride, rows, K, operand, dst_dev, as_stream(stream));
+}
+
+int ncnnhip_gemm_int8_tiled(const int8_t* aq_tiled_dev, const int8_t* bq_tiled_dev, int M, int N, int K, const float* a_scales_dev,
+                            const float* b_scales_dev, int n_b_scales, const float* c_dev, int broadcast_type_c, float alpha, float beta,
+                            float* out_dev, size_t out_stride, void* stream)
+{
+    NCNNHIP_REQUIRE(aq_tiled_dev && bq_tiled_dev && a_scales_dev && b_scales_dev && out_dev, "ncnnhip_gemm_int8_tiled: null pointer");
+    NCNNHIP_REQUIRE(M >= 256 && N >= 256 && K >= 64 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0,
+                    "ncnnhip_gemm_int8_tiled: shape %d %d %d (M, N multiples of 256, K of 64)", M, N, K);
+    NCNNHIP_REQUIRE(n_b_scales == 1 || n_b_scales == N, "ncnnhip_gemm_int8_tiled: %d B scales for N=%d", n_b_scales, N);
+    const int bt = c_dev ? broadcast_type_c : -1;
+    NCNNHIP_REQUIRE(bt == -1 || bt == 4, "ncnnhip_gemm_int8_tiled: C broadcast %d (none or per column only)", bt);
+    NCNNHIP_REQUIRE(out_stride >= (size_t)N && out_stride % 4 == 0 && aligned16(out_dev), "ncnnhip_gemm_int8_tiled: output rows must be 16-byte aligned");
+    NCNNHIP_REQUIRE(aligned16(aq_tiled_dev) && aligned16(bq_tiled_dev), "ncnnhip_gemm_int8_tiled: operands must be 16-byte aligned");
+    GemmEpilogue epi;
+    epi.a_scales = a_scales_dev;
+    epi.b_scales = b_scales_dev;
+    epi.per_col = n_b_scales != 1;
+    epi.c = c_dev;
+    epi.bt = bt;
+    epi.alpha = alpha;
+    epi.beta = beta;
+    epi.transpose = 0;
+    epi.out = out_dev;
+    epi.out_stride = out_stride;
+    epi.N = N;
+    epi.acc_out = 0;
+    return launch_gemm_int8_tiled(aq_tiled_dev, bq_tiled_dev, M, N, K, epi, as_stream(stream));
 }
 
 } // extern "C"

@@ -13,6 +13,13 @@
 // each lane fetches.  With it, any 16 consecutive rows read at one K offset hit 16 different
 // 16-byte bank groups.
 //
+// TILED operands: element (r, k) of an operand lies at ((r / 256 * (K / 64) + k / 64) * 256 + r % 256) * 64 + k % 64, i.e.
+// the 256 x 64-byte panel of one tile and one K step is 16 KB of consecutive memory, and every direct-to-LDS load of a
+// wavefront fetches one whole KB (eight full 128-byte lines).  From row-major operands the same load touches 16 half
+// lines, each line being fetched again one K step later: twice the L2-to-L1 traffic and twice the tag look-ups, which is
+// what bounds the row-major kernel (without any fills its K loop runs 25 % faster).  The B operand is tiled with its rows
+// already in the column-interleaved order described at the loads below.
+//
 // Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to XCDs)
 // works on a compact block of output tiles and re-uses its A/B panels out of its own L2.
 #include <type_traits>
@@ -35,7 +42,7 @@ constexpr int STAGE_BYTES = 2 * OPERAND_BYTES; // 32 KB
 #define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
 
 
-template<bool PER_COL, int BT>
+template<bool PER_COL, int BT, bool TILED>
 __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __restrict__ A, size_t lda, const int8_t* __restrict__ B,
                                                                  size_t ldb, int nk, int tiles_m, int tiles_n,
                                                                  const float* __restrict__ a_scales, const float* __restrict__ b_scales,
@@ -66,20 +73,22 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     // load i of wave w fills LDS rows (i*4 + w)*16 .. +16 of the operand stage
     const int ld_row = wave * 16 + (lane >> 2);                 // + i*64
     const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);        // swizzled source chunk
-    const int8_t* ga = A + ((size_t)tile_m * PT + ld_row) * lda + ld_chunk * 16;
+    const int8_t* ga = TILED ? A + ((size_t)tile_m * nk * PT + ld_row) * PK + ld_chunk * 16 : A + ((size_t)tile_m * PT + ld_row) * lda + ld_chunk * 16;
     // B rows are permuted on their way into LDS: LDS row wn*128 + j*32 + l holds B row wn*128 + 4*l + j, so that the four
     // accumulator blocks j of a lane are four consecutive output columns and the epilogue stores 16 bytes per lane.
     // LDS row of this lane in quarter i = i*64 + wave*16 + (lane >> 2): wn = i >> 1, j = (i & 1)*2 + (wave >> 1),
     // l = (wave & 1)*16 + (lane >> 2).
     const int ld_row_b = 4 * ((wave & 1) * 16 + (lane >> 2)) + (wave >> 1); // + (i >> 1)*128 + (i & 1)*2
-    const int8_t* gb = B + ((size_t)tile_n * PT + ld_row_b) * ldb + ld_chunk * 16;
+    const int8_t* gb = TILED ? B + ((size_t)tile_n * nk * PT + ld_row) * PK + ld_chunk * 16 : B + ((size_t)tile_n * PT + ld_row_b) * ldb + ld_chunk * 16;
     const size_t a_step = 64 * lda;
 
     // quarter i of the loads of step t: 16 A rows and 16 B rows per wave
     auto issue_quarter = [&](int t, int i) {
         int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024 + i * 4096;
-        __builtin_amdgcn_global_load_lds((const AS1 void*)(ga + (size_t)t * PK + i * a_step), (AS3 void*)sa, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const AS1 void*)(gb + (size_t)t * PK + (size_t)((i >> 1) * 128 + (i & 1) * 2) * ldb), (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
+        const int8_t* pa = TILED ? ga + (size_t)t * OPERAND_BYTES + i * 4096 : ga + (size_t)t * PK + i * a_step;
+        const int8_t* pb = TILED ? gb + (size_t)t * OPERAND_BYTES + i * 4096 : gb + (size_t)t * PK + (size_t)((i >> 1) * 128 + (i & 1) * 2) * ldb;
+        __builtin_amdgcn_global_load_lds((const AS1 void*)pa, (AS3 void*)sa, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const AS1 void*)pb, (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
     };
     auto issue_stage = [&](int t) {
 #pragma unroll
@@ -261,20 +270,15 @@ static inline bool al16(const void* p)
     return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
 
-int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K,
-                               const GemmEpilogue& epi, hipStream_t stream, bool* handled)
+template<bool TILED>
+static int launch_256x256(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmEpilogue& epi,
+                          hipStream_t stream)
 {
-    *handled = false;
-    if (M % PT || N % PT || K % PK || aq_stride % 16 || bq_stride % 16 || !al16(aq) || !al16(bq)) return NCNNHIP_OK;
-    if (epi.transpose || epi.acc_out || !(epi.bt == -1 || epi.bt == 4)) return NCNNHIP_OK;
-    if (epi.out_stride % 4 || !al16(epi.out)) return NCNNHIP_OK; // the epilogue stores 16 bytes per lane
     const int tm = M / PT, tn = N / PT, nk = K / PK;
-    if ((long long)tm * tn > 0x7fffffff) return NCNNHIP_OK;
-    *handled = true;
     dim3 grid(tm * tn), block(256);
 #define LAUNCH(PC, BTV)                                                                                                                    \
-    hipLaunchKernelGGL((gemm_int8_256x256_kernel<PC, BTV>), grid, block, 0, stream, aq, aq_stride, bq, bq_stride, nk, tm, tn, epi.a_scales, \
-                       epi.b_scales, epi.c, epi.alpha, epi.beta, epi.out, epi.out_stride)
+    hipLaunchKernelGGL((gemm_int8_256x256_kernel<PC, BTV, TILED>), grid, block, 0, stream, aq, aq_stride, bq, bq_stride, nk, tm, tn,        \
+                       epi.a_scales, epi.b_scales, epi.c, epi.alpha, epi.beta, epi.out, epi.out_stride)
     if (epi.per_col)
     {
         if (epi.bt == 4)
@@ -291,6 +295,50 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
     }
 #undef LAUNCH
     return launch_status("gemm_int8_256x256_kernel");
+}
+
+int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K,
+                               const GemmEpilogue& epi, hipStream_t stream, bool* handled)
+{
+    *handled = false;
+    if (M % PT || N % PT || K % PK || aq_stride % 16 || bq_stride % 16 || !al16(aq) || !al16(bq)) return NCNNHIP_OK;
+    if (epi.transpose || epi.acc_out || !(epi.bt == -1 || epi.bt == 4)) return NCNNHIP_OK;
+    if (epi.out_stride % 4 || !al16(epi.out)) return NCNNHIP_OK; // the epilogue stores 16 bytes per lane
+    if ((long long)(M / PT) * (N / PT) > 0x7fffffff) return NCNNHIP_OK;
+    *handled = true;
+    return launch_256x256<false>(aq, aq_stride, bq, bq_stride, M, N, K, epi, stream);
+}
+
+// operands in the tiled layout; the caller has checked shapes and alignment
+int launch_gemm_int8_tiled(const int8_t* aq_tiled, const int8_t* bq_tiled, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream)
+{
+    return launch_256x256<true>(aq_tiled, 0, bq_tiled, 0, M, N, K, epi, stream);
+}
+
+// row-major [rows][K] -> tiled; operand_b: position p of a 256-row tile holds row (p >> 7)*128 + 4*(p & 31) + ((p >> 5) & 3),
+// the order in which the kernel wants the rows of B in LDS.  One 16-byte chunk per thread.
+__global__ __launch_bounds__(256) void gemm_tile_operand_kernel(const int8_t* __restrict__ src, size_t stride, int nk, size_t chunks, int operand_b,
+                                                                 int8_t* __restrict__ dst)
+{
+    const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= chunks) return;
+    const int c = (int)(g & 3);
+    const int p = (int)((g >> 2) & 255);
+    const size_t panel = g >> 10; // tile * nk + t
+    const size_t tile = panel / nk;
+    const int t = (int)(panel - tile * nk);
+    const int r = operand_b ? (p >> 7) * 128 + 4 * (p & 31) + ((p >> 5) & 3) : p;
+    const v4i v = *reinterpret_cast<const v4i*>(src + (tile * PT + r) * stride + (size_t)t * PK + c * 16);
+    *reinterpret_cast<v4i*>(dst + g * 16) = v;
+}
+
+int launch_gemm_tile_operand(const int8_t* src, size_t stride, int rows, int K, int operand_b, int8_t* dst, hipStream_t stream)
+{
+    const size_t chunks = (size_t)rows * K / 16;
+    const size_t blocks = (chunks + 255) / 256;
+    if (blocks > 0x7fffffffull) return NCNNHIP_ERROR;
+    hipLaunchKernelGGL(gemm_tile_operand_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, stride, K / PK, chunks, operand_b, dst);
+    return launch_status("gemm_tile_operand_kernel");
 }
 
 } // namespace ncnnhip

@@ -99,12 +99,14 @@ __global__ __launch_bounds__(256) void quantize_rows_dynamic_kernel(const float*
 // the cache by the next pass over the same buffer and lose 1 us this way).
 template<int NV, bool NT>
 __global__ __launch_bounds__(256) void quantize_rows_dynamic_reg_kernel(const float* __restrict__ a, size_t as, int cols,
-                                                                         int8_t* __restrict__ aq, size_t aqs, float* __restrict__ scales)
+                                                                         int8_t* __restrict__ aq, size_t aqs, float* __restrict__ scales, int tiled)
 {
     __shared__ float red[4];
     const int r = blockIdx.x;
     const float4* ar = reinterpret_cast<const float4*>(a + (size_t)r * as);
-    uint32_t* qr = reinterpret_cast<uint32_t*>(aq + (size_t)r * aqs);
+    // tiled: the 256x256 Gemm kernel's operand layout, [r / 256][k / 64][r % 256][k % 64]; word i of the row (bytes 4i .. 4i+3)
+    // is word i % 16 of K step i / 16
+    uint32_t* qr = tiled ? reinterpret_cast<uint32_t*>(aq + ((size_t)(r >> 8) * (cols >> 6) * 256 + (r & 255)) * 64) : reinterpret_cast<uint32_t*>(aq + (size_t)r * aqs);
     const int n4 = cols >> 2; // cols % 4 == 0 here
     float4 v[NV];
     float m = 0.f;
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(256) void quantize_rows_dynamic_reg_kernel(const fl
     {
         const int i = threadIdx.x + j * 256;
         if (i < n4)
-            qr[i] = pack4((int)float2int8_as_float(mul_rn(v[j].x, s)), (int)float2int8_as_float(mul_rn(v[j].y, s)),
+            qr[tiled ? (size_t)(i >> 4) * 4096 + (i & 15) : (size_t)i] = pack4((int)float2int8_as_float(mul_rn(v[j].x, s)), (int)float2int8_as_float(mul_rn(v[j].y, s)),
                           (int)float2int8_as_float(mul_rn(v[j].z, s)), (int)float2int8_as_float(mul_rn(v[j].w, s)));
     }
 }
@@ -206,14 +208,11 @@ int ncnnhip_quantize(const float* x_dev, size_t x_stride, size_t x_nstep, int8_t
     return launch_status("quantize_kernel");
 }
 
-int ncnnhip_gemm_quantize_rows(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_dev, size_t aq_stride,
-                               float* scales_dev, void* stream)
+static int quantize_rows_impl(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_dev, size_t aq_stride, float* scales_dev,
+                              int tiled, void* stream)
 {
-    NCNNHIP_REQUIRE(a_dev && aq_dev && scales_dev, "ncnnhip_gemm_quantize_rows: null pointer");
-    NCNNHIP_REQUIRE(rows >= 0 && cols >= 0, "ncnnhip_gemm_quantize_rows: bad extent");
-    NCNNHIP_REQUIRE(a_stride >= (size_t)cols && aq_stride >= (size_t)cols, "ncnnhip_gemm_quantize_rows: stride below cols");
-    if (rows == 0) return NCNNHIP_OK;
     const bool vec = aligned(a_dev, 16) && aligned(aq_dev, 4) && a_stride % 4 == 0 && aq_stride % 4 == 0;
+    NCNNHIP_REQUIRE(!tiled || (vec && cols <= 8192), "ncnnhip_gemm_quantize_rows_tiled: needs 16-byte aligned rows of at most 8192 values");
     if (vec && cols % 4 == 0 && cols <= 8192)
     {
         const int nv = ceil_div(cols, 1024);
@@ -223,10 +222,10 @@ int ncnnhip_gemm_quantize_rows(const float* a_dev, size_t a_stride, int rows, in
     {                                                                                                                                            \
         if (nt)                                                                                                                                  \
             hipLaunchKernelGGL((quantize_rows_dynamic_reg_kernel<NV_, true>), dim3(rows), dim3(256), 0, as_stream(stream), a_dev, a_stride, cols, \
-                               aq_dev, aq_stride, scales_dev);                                                                                   \
+                               aq_dev, aq_stride, scales_dev, tiled);                                                                            \
         else                                                                                                                                     \
             hipLaunchKernelGGL((quantize_rows_dynamic_reg_kernel<NV_, false>), dim3(rows), dim3(256), 0, as_stream(stream), a_dev, a_stride,     \
-                               cols, aq_dev, aq_stride, scales_dev);                                                                             \
+                               cols, aq_dev, aq_stride, scales_dev, tiled);                                                                      \
     } while (0)
         if (nv <= 1)
             LAUNCH_REG(1);
@@ -243,6 +242,25 @@ int ncnnhip_gemm_quantize_rows(const float* a_dev, size_t a_stride, int rows, in
     else
         hipLaunchKernelGGL(quantize_rows_dynamic_kernel<false>, dim3(rows), dim3(256), 0, as_stream(stream), a_dev, a_stride, cols, aq_dev, aq_stride, scales_dev);
     return launch_status("quantize_rows_dynamic_kernel");
+}
+
+int ncnnhip_gemm_quantize_rows(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_dev, size_t aq_stride,
+                               float* scales_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(a_dev && aq_dev && scales_dev, "ncnnhip_gemm_quantize_rows: null pointer");
+    NCNNHIP_REQUIRE(rows >= 0 && cols >= 0, "ncnnhip_gemm_quantize_rows: bad extent");
+    NCNNHIP_REQUIRE(a_stride >= (size_t)cols && aq_stride >= (size_t)cols, "ncnnhip_gemm_quantize_rows: stride below cols");
+    if (rows == 0) return NCNNHIP_OK;
+    return quantize_rows_impl(a_dev, a_stride, rows, cols, aq_dev, aq_stride, scales_dev, 0, stream);
+}
+
+int ncnnhip_gemm_quantize_rows_tiled(const float* a_dev, size_t a_stride, int rows, int cols, int8_t* aq_tiled_dev, float* scales_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(a_dev && aq_tiled_dev && scales_dev, "ncnnhip_gemm_quantize_rows_tiled: null pointer");
+    NCNNHIP_REQUIRE(rows >= 256 && rows % 256 == 0 && cols >= 64 && cols % 64 == 0,
+                    "ncnnhip_gemm_quantize_rows_tiled: %d rows of %d (multiples of 256 and 64 only)", rows, cols);
+    NCNNHIP_REQUIRE(a_stride >= (size_t)cols, "ncnnhip_gemm_quantize_rows_tiled: stride below cols");
+    return quantize_rows_impl(a_dev, a_stride, rows, cols, aq_tiled_dev, (size_t)cols, scales_dev, 1, stream);
 }
 
 int ncnnhip_gemm_quantize_tensor(const float* b_dev, size_t b_stride, int rows, int cols, int8_t* bq_dev, size_t bq_stride,

@@ -119,6 +119,10 @@ _SIGNATURES = {
     "ncnnhip_transpose_s8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_int8": [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
                           C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_int8_tile_operand": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_quantize_rows_tiled": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_gemm_int8_tiled": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_blockquant": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_blockquant_packed_size": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
@@ -562,6 +566,34 @@ class Runtime:
                                       oshape[1], _ptr(dacc), self.stream))
         out = dout.to_numpy(self.stream)
         return (out, dacc.to_numpy(self.stream)) if want_acc else out
+
+    def gemm_tile_operand(self, q, operand):
+        """Row-major int8 [rows][K] -> the 256x256 Gemm kernel's tiled layout (operand 0 = A, 1 = B), as a flat array."""
+        q = np.ascontiguousarray(q, np.int8)
+        rows, k = q.shape
+        dq = self.up(q)
+        dt = DeviceBuffer.empty((rows * k,), np.int8)
+        check(lib().ncnnhip_gemm_int8_tile_operand(dq.ptr, k, rows, k, operand, dt.ptr, self.stream))
+        return dt.to_numpy(self.stream)
+
+    def gemm_quantize_rows_tiled(self, a):
+        a = np.ascontiguousarray(a, np.float32)
+        m, k = a.shape
+        da = self.up(a)
+        dq = DeviceBuffer.empty((m * k,), np.int8)
+        ds = DeviceBuffer.empty((m,), np.float32)
+        check(lib().ncnnhip_gemm_quantize_rows_tiled(da.ptr, k, m, k, dq.ptr, ds.ptr, self.stream))
+        return dq.to_numpy(self.stream), ds.to_numpy(self.stream)
+
+    def gemm_int8_tiled(self, aq_tiled, bq_tiled, m, n, k, a_scales, b_scales, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0):
+        b_scales = np.ascontiguousarray(np.atleast_1d(b_scales), np.float32)
+        daq, dbq = self.up(np.ascontiguousarray(aq_tiled, np.int8)), self.up(np.ascontiguousarray(bq_tiled, np.int8))
+        dsa, dsb = self.up(np.asarray(a_scales, np.float32)), self.up(b_scales)
+        dc = self.up(None if c is None else np.asarray(c, np.float32))
+        dout = DeviceBuffer.empty((m, n), np.float32)
+        check(lib().ncnnhip_gemm_int8_tiled(daq.ptr, dbq.ptr, m, n, k, dsa.ptr, dsb.ptr, b_scales.size, _ptr(dc),
+                                            broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
+        return dout.to_numpy(self.stream)
 
     def transpose(self, a):
         a = np.ascontiguousarray(a)

@@ -137,6 +137,35 @@ def test_gemm_int8_256x256_kernel_sizes(rt, m, n, k, bt, per_col):
     assert np.array_equal(got, want)
     if k == 64 and not per_col:
         assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, sb, c, bt))
+    # the same Gemm on operands in the kernel's tiled layout: the quantiser writes A tiled, B is tiled once
+    atq, ats = rt.gemm_quantize_rows_tiled(a)
+    assert np.array_equal(ats, sa)
+    assert np.array_equal(atq, _tiled(aq, False))
+    btq = rt.gemm_tile_operand(bq, 1)
+    assert np.array_equal(btq, _tiled(bq, True))
+    assert np.array_equal(rt.gemm_tile_operand(aq, 0), atq)
+    assert np.array_equal(rt.gemm_int8_tiled(atq, btq, m, n, k, sa, sb, c, bt), want)
+
+
+def _tiled(q, operand_b):
+    """numpy statement of the tiled operand layout: [r / 256][k / 64][r % 256][k % 64]; for B, position p of a tile holds row
+    (p >> 7) * 128 + 4 * (p & 31) + ((p >> 5) & 3)."""
+    rows, k = q.shape
+    t = q.reshape(rows // 256, 256, k // 64, 64)
+    if operand_b:
+        p = np.arange(256)
+        t = t[:, (p >> 7) * 128 + 4 * (p & 31) + ((p >> 5) & 3)]
+    return np.ascontiguousarray(t.transpose(0, 2, 1, 3)).reshape(-1)
+
+
+def test_gemm_int8_tiled_rejects_what_it_cannot_run(rt):
+    from ncnn_amd.hip import NcnnHipError
+    q = np.zeros((256, 64), np.int8)
+    for bad in (lambda: rt.gemm_tile_operand(np.zeros((255, 64), np.int8), 0), lambda: rt.gemm_tile_operand(np.zeros((256, 48), np.int8), 1),
+                lambda: rt.gemm_quantize_rows_tiled(np.zeros((256, 100), F)),
+                lambda: rt.gemm_int8_tiled(q.reshape(-1), q.reshape(-1), 256, 256, 64, np.ones(256, F), [1.0], np.zeros(256, F), 1)):
+        with pytest.raises(NcnnHipError):
+            bad()
 
 
 # ----------------------------------------------------------------------------- convolution
