@@ -90,6 +90,19 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
         __builtin_amdgcn_global_load_lds((const AS1 void*)pa, (AS3 void*)sa, 16, 0, 0);
         __builtin_amdgcn_global_load_lds((const AS1 void*)pb, (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
     };
+    auto issue_one = [&](int t, int i, int which) {
+        int8_t* sa = smem + (t & (STAGES - 1)) * STAGE_BYTES + wave * 1024 + i * 4096;
+        if (which == 0)
+        {
+            const int8_t* pa = TILED ? ga + (size_t)t * OPERAND_BYTES + i * 4096 : ga + (size_t)t * PK + i * a_step;
+            __builtin_amdgcn_global_load_lds((const AS1 void*)pa, (AS3 void*)sa, 16, 0, 0);
+        }
+        else
+        {
+            const int8_t* pb = TILED ? gb + (size_t)t * OPERAND_BYTES + i * 4096 : gb + (size_t)t * PK + (size_t)((i >> 1) * 128 + (i & 1) * 2) * ldb;
+            __builtin_amdgcn_global_load_lds((const AS1 void*)pb, (AS3 void*)(sa + OPERAND_BYTES), 16, 0, 0);
+        }
+    };
     auto issue_stage = [&](int t) {
 #pragma unroll
         for (int i = 0; i < 4; i++) issue_quarter(t, i);
@@ -115,12 +128,8 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     if (1 < nk) issue_stage(1);
     if (2 < nk) issue_stage(2);
 
-    // Fragment registers are double-buffered: while the 16 MFMAs of one K half-step run, the
-    // 8 LDS reads of the next half-step are already in flight.  The workgroup barrier sits
-    // between the two half-steps of a stage.
-    // The LDS reads and their waits are written as asm so that the wait before a group of MFMAs
-    // only covers the fragment set that group uses (lgkmcnt(8)) and leaves the 8 reads of the next
-    // set in flight.
+    // Fragment registers are double-buffered (F0 = first 32 bytes of a K step, F1 = second).  The LDS reads and their
+    // waits are written as asm so that a wait only covers the reads the next MFMAs need and leaves the others in flight.
     v4i fa0[4], fb0[4], fa1[4], fb1[4];
     const unsigned lds_base = (unsigned)(uintptr_t)(AS3 int8_t*)smem;
     auto frag_addr_a = [&](int t, int ks) { return lds_base + (unsigned)((t & (STAGES - 1)) * STAGE_BYTES) + (ks ? rd_a1 : rd_a0); };
@@ -162,24 +171,41 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     if (3 < nk) issue_stage(3);
     read_frags(0, 0, fa0, fb0);
 
-    // One K step.  Schedule (F0/F1 = the two fragment register sets):
-    //   reads(t, second half) -> F1 | wait F0 | 16 MFMA(F0) | wait loads of step t+1, barrier |
-    //   4 x { 4 MFMA(F1), one quarter of the global->LDS loads of step t+4, 2 reads of (t+1, first half) -> F0 }
-    // so the matrix pipe always has a full MFMA group queued behind the barrier, and every LDS or
-    // global access is issued at least 16 MFMAs before its data is needed.
-    // STEADY means steps t+1 .. t+4 all exist (branch-free body).
-    auto k_step = [&](int t, auto steady) {
+    // One K step, one memory instruction after each MFMA.  A wavefront issues in order and an MFMA occupies the matrix pipe
+    // for 32 cycles, so whatever stands between two MFMAs must issue within those 32 cycles or the pipe idles: the 8 reads of
+    // the second fragment set follow the first 8 MFMAs of the step one by one, and after the barrier the 8 reads of the next
+    // step's first set alternate with the 8 global->LDS loads of step t+4.  LDS reads return in order, so the wait before a row
+    // of MFMAs only covers the reads that row needs (counted in reads still allowed in flight).
+#define WAIT_LGKM(n, ...) asm volatile("s_waitcnt lgkmcnt(" #n ")" : __VA_ARGS__)
+    auto mma1 = [&](int i, int j, const v4i (&fa)[4], const v4i (&fb)[4]) {
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    auto k_step_fine = [&](int t, auto steady) {
         constexpr bool STEADY = decltype(steady)::value;
-        read_frags(t, 1, fa1, fb1);
-        WAIT_FRAGS(8, fa0, fb0);
-        PIN;
-        mma_row(0, fa0, fb0);
-        mma_row(1, fa0, fb0);
-        mma_row(2, fa0, fb0);
-        mma_row(3, fa0, fb0);
-        PIN;
         const bool more = STEADY || t + 1 < nk;
         const bool refill = STEADY || t + 4 < nk;
+        const unsigned qa = frag_addr_a(t, 1), qb = frag_addr_b(t, 1);
+        // first set: issued in the order fa0[0], fb0[0..3], fa0[1..3]
+        WAIT_LGKM(3, "+v"(fa0[0]), "+v"(fb0[0]), "+v"(fb0[1]), "+v"(fb0[2]), "+v"(fb0[3]));
+        PIN;
+        mma1(0, 0, fa0, fb0); PIN; LDS_READ(fa1[0], qa, 0); PIN;
+        mma1(0, 1, fa0, fb0); PIN; LDS_READ(fb1[0], qb, 0); PIN;
+        mma1(0, 2, fa0, fb0); PIN; LDS_READ(fb1[1], qb, 2048); PIN;
+        mma1(0, 3, fa0, fb0); PIN; LDS_READ(fb1[2], qb, 4096); PIN;
+        WAIT_LGKM(6, "+v"(fa0[1]));
+        PIN;
+        mma1(1, 0, fa0, fb0); PIN; LDS_READ(fb1[3], qb, 6144); PIN;
+        mma1(1, 1, fa0, fb0); PIN; LDS_READ(fa1[1], qa, 2048); PIN;
+        mma1(1, 2, fa0, fb0); PIN; LDS_READ(fa1[2], qa, 4096); PIN;
+        mma1(1, 3, fa0, fb0); PIN; LDS_READ(fa1[3], qa, 6144); PIN;
+        WAIT_LGKM(9, "+v"(fa0[2]));
+        PIN;
+        mma_row(2, fa0, fb0);
+        PIN;
+        WAIT_LGKM(8, "+v"(fa0[3]));
+        PIN;
+        mma_row(3, fa0, fb0);
+        PIN;
         if (more)
         {
             if (STEADY)
@@ -187,35 +213,30 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
             else
                 wait_step(t + 1);
         }
-        WAIT_FRAGS(0, fa1, fb1);      // this wave's reads of step t have landed
-        if (more) __builtin_amdgcn_s_barrier(); // step t+1 visible to all waves; nobody reads step t any more
+        WAIT_FRAGS(0, fa1, fb1);
+        if (more) __builtin_amdgcn_s_barrier();
         PIN;
         const unsigned pa = frag_addr_a(t + 1, 0), pb = frag_addr_b(t + 1, 0);
-        mma_row(0, fa1, fb1);
-        PIN;
-        if (refill) issue_quarter(t + 4, 0);
-        if (more) { LDS_READ(fa0[0], pa, 0); LDS_READ(fb0[0], pb, 0); }
-        PIN;
-        mma_row(1, fa1, fb1);
-        PIN;
-        if (refill) issue_quarter(t + 4, 1);
-        if (more) { LDS_READ(fb0[1], pb, 2048); LDS_READ(fb0[2], pb, 4096); }
-        PIN;
-        mma_row(2, fa1, fb1);
-        PIN;
-        if (refill) issue_quarter(t + 4, 2);
-        if (more) { LDS_READ(fb0[3], pb, 6144); LDS_READ(fa0[1], pa, 2048); }
-        PIN;
-        mma_row(3, fa1, fb1);
-        PIN;
-        if (refill) issue_quarter(t + 4, 3);
-        if (more) { LDS_READ(fa0[2], pa, 4096); LDS_READ(fa0[3], pa, 6144); }
-        PIN;
+        mma1(0, 0, fa1, fb1); PIN; if (more) LDS_READ(fa0[0], pa, 0); PIN;
+        mma1(0, 1, fa1, fb1); PIN; if (refill) issue_one(t + 4, 0, 0); PIN;
+        mma1(0, 2, fa1, fb1); PIN; if (more) LDS_READ(fb0[0], pb, 0); PIN;
+        mma1(0, 3, fa1, fb1); PIN; if (refill) issue_one(t + 4, 0, 1); PIN;
+        mma1(1, 0, fa1, fb1); PIN; if (more) LDS_READ(fb0[1], pb, 2048); PIN;
+        mma1(1, 1, fa1, fb1); PIN; if (refill) issue_one(t + 4, 1, 0); PIN;
+        mma1(1, 2, fa1, fb1); PIN; if (more) LDS_READ(fb0[2], pb, 4096); PIN;
+        mma1(1, 3, fa1, fb1); PIN; if (refill) issue_one(t + 4, 1, 1); PIN;
+        mma1(2, 0, fa1, fb1); PIN; if (more) LDS_READ(fb0[3], pb, 6144); PIN;
+        mma1(2, 1, fa1, fb1); PIN; if (refill) issue_one(t + 4, 2, 0); PIN;
+        mma1(2, 2, fa1, fb1); PIN; if (more) LDS_READ(fa0[1], pa, 2048); PIN;
+        mma1(2, 3, fa1, fb1); PIN; if (refill) issue_one(t + 4, 2, 1); PIN;
+        mma1(3, 0, fa1, fb1); PIN; if (more) LDS_READ(fa0[2], pa, 4096); PIN;
+        mma1(3, 1, fa1, fb1); PIN; if (refill) issue_one(t + 4, 3, 0); PIN;
+        mma1(3, 2, fa1, fb1); PIN; if (more) LDS_READ(fa0[3], pa, 6144); PIN;
+        mma1(3, 3, fa1, fb1); PIN; if (refill) issue_one(t + 4, 3, 1); PIN;
     };
-
     int t = 0;
-    for (; t + 4 < nk; t++) k_step(t, std::true_type{});
-    for (; t < nk; t++) k_step(t, std::false_type{});
+    for (; t + 4 < nk; t++) k_step_fine(t, std::true_type{});
+    for (; t < nk; t++) k_step_fine(t, std::false_type{});
 
     // ---- fused epilogue: dequantise, bias, scale, store fp32
     const int col_base = tile_n * PT + wn * 128 + 4 * l32; // accumulator block j of this lane is column col_base + j

@@ -35,7 +35,7 @@ Gemm_hip::Gemm_hip()
     support_inplace = false;
     weight_block_quantize = 0;
     B_data_int8_scale = 1.f;
-    d_A = d_B = d_C = d_A_scales = d_B_scale = d_B_block_scales = d_B_input_scales = 0;
+    d_A = d_B = d_B_tiled = d_C = d_A_scales = d_B_scale = d_B_block_scales = d_B_input_scales = 0;
     b_ready_int8 = 0;
 }
 
@@ -202,6 +202,14 @@ int Gemm_hip::create_pipeline(const Option&)
                 }
             }
             if (ret == 0) b_ready_int8 = 1;
+            if (ret == 0 && constantN % 256 == 0 && constantK % 64 == 0 && constantK <= 8192)
+            {
+                // second copy of B, laid out once for the 256x256 kernel (used from 128 output tiles up)
+                int rc = ncnnhip_malloc(&d_B_tiled, (size_t)constantN * constantK);
+                if (rc == 0) rc = ncnnhip_gemm_int8_tile_operand((const int8_t*)d_B, (size_t)constantK, constantN, constantK, 1, (int8_t*)d_B_tiled, 0);
+                if (rc == 0) rc = ncnnhip_stream_synchronize(0);
+                if (rc != 0) ret = to_ncnn_status(rc, "tile constant B");
+            }
         }
     }
     // the device-resident form needs B ready on the device (int8 rows or block-quantised fields)
@@ -212,7 +220,7 @@ int Gemm_hip::create_pipeline(const Option&)
 
 int Gemm_hip::destroy_pipeline(const Option&)
 {
-    void** all[] = {&d_A, &d_B, &d_C, &d_A_scales, &d_B_scale, &d_B_block_scales, &d_B_input_scales};
+    void** all[] = {&d_A, &d_B, &d_B_tiled, &d_C, &d_A_scales, &d_B_scale, &d_B_block_scales, &d_B_input_scales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
@@ -291,6 +299,15 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
     void* q = scratch.get((size_t)M * aq_stride);
     void* sa = scratch.get((size_t)M * 4);
     if (!q || !sa) return -100;
+    if (d_B_tiled && M % 256 == 0 && (long long)M * N >= 256ll * 256 * 128 && (bt == -1 || bt == 4))
+    {
+        // both operands in the 256x256 kernel's tiled layout: the quantiser writes A that way (aq_stride == K here)
+        rc = ncnnhip_gemm_quantize_rows_tiled((const float*)A.data, (size_t)K, M, K, (int8_t*)q, (float*)sa, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_quantize_rows_tiled");
+        rc = ncnnhip_gemm_int8_tiled((const int8_t*)q, (const int8_t*)d_B_tiled, M, N, K, (const float*)sa, (const float*)d_B_scale, 1, d_c, bt, alpha, beta,
+                                     (float*)top.data, (size_t)N, st);
+        return to_ncnn_status(rc, "ncnnhip_gemm_int8_tiled");
+    }
     rc = ncnnhip_gemm_quantize_rows((const float*)A.data, (size_t)K, M, K, (int8_t*)q, aq_stride, (float*)sa, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_quantize_rows");
     rc = ncnnhip_gemm_int8((const int8_t*)q, aq_stride, (const int8_t*)d_B, (size_t)K, M, N, K, (const float*)sa, (const float*)d_B_scale, 1, d_c, bt, alpha, beta, 0,

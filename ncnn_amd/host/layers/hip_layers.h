@@ -120,6 +120,7 @@ private:
     int forward_block_quantize(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
     void* d_A;        // constant A as loaded (fp32 or int8), row-major as stored
     void* d_B;        // constant B: int8 [N][K] for the int8 path (already K-contiguous), packed bytes for block quant
+    void* d_B_tiled;  // the same int8 B in the 256x256 Gemm kernel's tiled operand layout (N % 256 == 0, K % 64 == 0), else null
     void* d_C;
     void* d_A_scales; // [M] when A is constant int8
     void* d_B_scale;  // [1]

@@ -160,6 +160,27 @@ def test_gemm_layer_int8_constant_b_with_bias(resident):
     assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, [sb], c, 4))
 
 
+def test_gemm_layer_int8_constant_b_large_enough_for_the_tiled_operands():
+    """From 128 output tiles of 256 x 256 the device-resident Gemm layer quantises A straight into the 256x256 kernel's tiled
+    layout and multiplies it with the copy of B that create_pipeline tiled; the answer is the oracle's, bit for bit."""
+    import npref
+    rng = np.random.default_rng(5)
+    m, n, k = 2048, 4096, 128
+    a = rng.standard_normal((m, k), dtype=F)
+    bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sb = F(41.25)
+    c = rng.standard_normal((1, n), dtype=F)
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m),
+             mw.gemm_param("g", ["a"], "out", M=0, N=n, K=k, constantB=1, constantC=1, broadcast_type_C=4, quantize_term=2)]
+    blob = mw.weight_blob(bq) + mw.weight_blob(c) + mw.raw_f32(sb)
+    got = _single(lines, blob, {"a": a}, "out", True)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    want, _ = npref.gemm_int8(aq, bq, sa, [sb], c, 4, acc=npref.gemm_acc_exact(aq, bq))
+    assert np.array_equal(got, want)
+    rows = np.arange(0, m, 97)
+    assert np.array_equal(got[rows], oracle.gemm_int8(aq[rows], bq, sa[rows], [sb], c, 4))
+
+
 def test_gemm_layer_int8_two_dynamic_operands_transposed_output():
     rng = np.random.default_rng(5)
     m, n, k = 20, 33, 64
