@@ -132,8 +132,12 @@ __global__ __launch_bounds__(256) void quantize_rows_dynamic_reg_kernel(const fl
     {
         const int i = threadIdx.x + j * 256;
         if (i < n4)
-            qr[tiled ? (size_t)(i >> 4) * 4096 + (i & 15) : (size_t)i] = pack4((int)float2int8_as_float(mul_rn(v[j].x, s)), (int)float2int8_as_float(mul_rn(v[j].y, s)),
-                          (int)float2int8_as_float(mul_rn(v[j].z, s)), (int)float2int8_as_float(mul_rn(v[j].w, s)));
+        {
+            const uint32_t q4 = pack4((int)float2int8_as_float(mul_rn(v[j].x, s)), (int)float2int8_as_float(mul_rn(v[j].y, s)),
+                                      (int)float2int8_as_float(mul_rn(v[j].z, s)), (int)float2int8_as_float(mul_rn(v[j].w, s)));
+            uint32_t* dst = qr + (tiled ? (size_t)(i >> 4) * 4096 + (i & 15) : (size_t)i);
+            *dst = q4;
+        }
     }
 }
 
