@@ -186,7 +186,8 @@ int ncnnhip_event_create(void** event)
 {
     NCNNHIP_REQUIRE(event, "null out pointer");
     hipEvent_t e;
-    NCNNHIP_CHECK(hipEventCreate(&e));
+    // timing events only: no system-scope cache flush when the event is recorded (it would sit between the kernels being timed)
+    NCNNHIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableSystemFence));
     *event = e;
     return NCNNHIP_OK;
 }
