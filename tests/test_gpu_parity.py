@@ -147,6 +147,20 @@ def test_gemm_int8_256x256_kernel_sizes(rt, m, n, k, bt, per_col):
     assert np.array_equal(rt.gemm_int8_tiled(atq, btq, m, n, k, sa, sb, c, bt), want)
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 256, 8192), (512, 256, 64), (256, 768, 1088)])
+def test_gemm_int8_tiled_entry_few_tiles(rt, m, n, k):
+    """The tiled entry points take any whole number of tiles: one tile with the longest rows the tiled quantiser accepts
+    (8192, eight 16-byte loads per thread), two tiles with a single K step, three tiles with 17 steps."""
+    _say("gemm_int8 tiled, few tiles", m, n, k)
+    a, bq, sb, bias = cases.gemm_case(5 * m + n + k, m, n, k, True)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    atq, ats = rt.gemm_quantize_rows_tiled(a)
+    assert np.array_equal(ats, sa) and np.array_equal(atq, _tiled(aq, False))
+    want = oracle.gemm_int8(aq, bq, sa, sb, bias.reshape(1, n), 4, 0.75, 1.5)
+    got = rt.gemm_int8_tiled(atq, rt.gemm_tile_operand(bq, 1), m, n, k, sa, sb, bias.reshape(1, n), 4, 0.75, 1.5)
+    assert np.array_equal(got, want)
+
+
 def _tiled(q, operand_b):
     """numpy statement of the tiled operand layout: [r / 256][k / 64][r % 256][k % 64]; for B, position p of a tile holds row
     (p >> 7) * 128 + 4 * (p & 31) + ((p >> 5) & 3)."""
