@@ -57,7 +57,7 @@ def cpu_baseline_gemm(n, k, per_col, budget_s=12.0):
         a = rng.standard_normal((rows, k), dtype=np.float32)
         cpubaseline.gemm(a, packed, n, sb, bias)  # warm-up (threads, page faults)
         times, t_start = [], time.perf_counter()
-        while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 1000):
+        while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 10000):
             t0 = time.perf_counter()
             cpubaseline.gemm(a, packed, n, sb, bias)
             times.append(time.perf_counter() - t0)
