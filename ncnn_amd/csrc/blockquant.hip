@@ -535,7 +535,7 @@ __device__ __forceinline__ v8h bytes_to_halves(int lo, int hi)
 
 // LDSA: the (few) activation rows are staged once per workgroup in LDS, zero-filled to a multiple of 64, instead of
 // travelling with every batch in registers: a batch is then 4 VGPRs per block and the ring can be twice as deep at the same
-// occupancy.  Used while M rows of K halves fit in 16 KB (decoding: M = 1..4) and there are many tiles.
+// occupancy.  Used while M rows of K halves fit in 32 KB (decoding: M = 1..4 at K = 4096) and there are many tiles.
 template<int NS, int U, bool LDSA>
 __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
                                                                 const v4i_bq* __restrict__ wpk, const float4* __restrict__ dpk,
@@ -822,7 +822,7 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
         const size_t act_bytes = (size_t)mc * kblocks * 64 * sizeof(__half);
-        if (act_bytes <= 16384 && tiles >= 512) // measured: pays from about 8192 weight rows, not for long rows (K = 11008) or few tiles
+        if (act_bytes <= 32768 && tiles >= 512) // measured: pays from about 8192 weight rows (up to four rows of 4096), not for long rows (K = 11008) or few tiles
             hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS_LDS, 1, true>), dim3(tiles), dim3(256), (size_t)kblocks * 64 + act_bytes, as_stream(stream),
                                ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),
                                reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride);
