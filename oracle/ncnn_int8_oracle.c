@@ -36,9 +36,14 @@
  * the attention layer against a float64 evaluation of softmax(q k^T * scale + mask) v on the
  * dequantised weights, against torch.nn.functional.multi_head_attention_forward, and through the
  * cache identity (a pass over n tokens == n passes of one token that feed their cache back).
- * Parity unpinned: activation types 4 (sigmoid) and 5 (mish) depend on the host libm and are
- * not part of any benchmark configuration; the out-of-range/NaN branch of float2int8 follows
- * what x86 cvttss2si produces (INT_MIN -> -127) and is pinned only by that statement.
+ * Activation types 4 (sigmoid) and 5 (mish) call expf / logf / tanhf of the host libm, so they are pinned to a
+ * tolerance instead of a bit pattern: against the float64 closed forms 1/(1+exp(-v)) (4 ulp) and
+ * v*tanh(log1p(exp(v))) (1e-6*|v|), with exact known answers at 0, at the +-88.376 clamp and where tanh saturates.
+ * The out-of-range / NaN branch of float2int8 follows what x86 cvttss2si produces ("integer indefinite", INT_MIN,
+ * which then saturates to -127); the pin executes that conversion on the x86 host and compares.
+ * Parity unpinned: nothing in this file.  (The per-column-B Gemm epilogue of the standalone Gemm configuration is a
+ * generalisation ncnn cannot express -- one B scale only, src/layer/gemm.h:69 -- so the reference fixes no value for
+ * it: "parity unpinned by the reference"; oracle_gemm_int8 evaluates ((float)acc * (1/sA_i)) * (1/sB_j) for it.)
  */
 #include <math.h>
 #include <stddef.h>

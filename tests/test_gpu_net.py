@@ -325,18 +325,22 @@ def test_benchmark_batch_equals_the_per_sample_passes(which, batch):
     """At the benchmark's batch sizes the kernels take other variants than at batch 1 (several output rows per
     depthwise thread, the pointwise small-K kernel, other tiles and K splits).  Batch 1 is pinned on the oracle
     executor above; here the folded batch must reproduce, bit for bit, the logits and a requantised blob deep in the
-    net of single-sample passes (samples 0, a middle one, the last)."""
+    net of single-sample passes (samples 0, a middle one, the last), and ONE sample of the batch (the last) is also run
+    through the oracle executor: its logits and the deep int8 blob must equal the folded batch's bit for bit."""
     _say("building", which)
     g, param, blob, info = zoo.build(which, input_hw=224, n_calib=1)
     net = _load(param, blob, True)
     xs = np.random.default_rng(21).uniform(0, 1, (batch,) + tuple(g.input_shape)).astype(F)
     last_fc = "fc1000" if which == "resnet50" else "fc"
     probe = "res2b_branch2b" if which == "resnet50" else "block2_dw"
+    _say("oracle forward of the last sample", which)
+    ref = refnet.run(param, blob, xs[batch - 1], want=last_fc)
     for name in (last_fc, probe):
         ex = net.create_extractor()
         ex.input("data", xs)
         got = np.asarray(ex.extract(name))
         assert got.shape[0] == batch
+        assert np.array_equal(got[batch - 1].reshape(-1), np.asarray(ref[name], F).reshape(-1)), (name, "oracle")
         for i in (0, batch // 2 - 1, batch - 1):
             ex1 = net.create_extractor()
             ex1.input("data", xs[i])

@@ -39,6 +39,21 @@ def test_float2int8_matches_float64_rounding_on_grid():
     assert got.min() >= -127 and got.max() <= 127
 
 
+def test_float2int8_out_of_range_is_what_the_x86_conversion_gives():
+    """`static_cast<int>(round(v))` (src/layer/convolution.cpp:375-381) is undefined in C++ for NaN and |v| >= 2^31; the
+    reference's x86 builds get cvttss2si's "integer indefinite" 0x80000000, which the clamp turns into -127.  numpy's
+    float32 -> int32 cast executes that very instruction on an x86 host, so the pin is the hardware's own answer."""
+    import platform
+    if platform.machine() not in ("x86_64", "AMD64"):
+        pytest.skip("pins the x86 conversion")
+    v = np.array([np.nan, np.inf, -np.inf, 3e9, -3e9, 2147483648.0, -2147483904.0, 1e30, -1e30], F)
+    with np.errstate(invalid="ignore"):
+        as_int = np.round(v).astype(np.int32)
+    assert np.all(as_int == np.iinfo(np.int32).min)
+    want = np.clip(as_int, -127, 127).astype(np.int8)
+    assert np.array_equal(oracle.quantize(v[None, :], [1.0])[0], want)
+
+
 def test_activation_closed_forms():
     assert oracle.activation(-1.0, 1) == 0.0 and oracle.activation(2.0, 1) == 2.0
     assert oracle.activation(-2.0, 2, (0.25,)) == -0.5
@@ -54,6 +69,40 @@ def test_activation_closed_forms():
         want = npref.activation(v, t, p)
         got = np.array([oracle.activation(float(z), t, p) for z in v], F)
         assert np.array_equal(got, want), t
+
+
+def test_sigmoid_and_mish_against_float64_closed_forms():
+    """Activation types 4 and 5 (src/layer/fused_activation.h:34-45) call the host's expf / logf / tanhf, so the pin is a
+    tolerance, not a bit pattern: sigmoid against 1 / (1 + exp(-v)) in float64 to 4 units in the last place of a value
+    in (0, 1] (plus 2e-44 where the result is denormal); mish against v * tanh(log1p(exp(v))) in float64 to 1e-6 * |v| (the fp32 formula rounds exp(v) + 1, which
+    costs up to 6e-8 in the logarithm whatever its size, and the product scales that by |v|).  Known answers and the
+    clamp of the sigmoid's argument at +-88.376 are checked exactly.  A dropped term, a flipped sign or the clamp on the
+    wrong side fails these."""
+    sig = lambda z: oracle.activation(float(z), 4)
+    mish = lambda z: oracle.activation(float(z), 5)
+    assert sig(0.0) == 0.5 and mish(0.0) == 0.0
+    assert sig(100.0) == sig(88.3762626647949) and sig(-100.0) == sig(-88.3762626647949)
+    assert sig(100.0) == 1.0 and 0.0 < sig(-100.0) < 1e-37
+    assert abs(mish(1.0) - 0.8650983882673103) < 2e-7      # v * tanh(ln(1 + e)), 16 digits from the closed form
+    assert abs(mish(-1.0) + 0.30340146137410895) < 2e-7
+    assert mish(50.0) == 50.0 and mish(1000.0) == 1000.0    # tanh saturates; exp overflows to inf, log(inf) = inf, tanh = 1
+    assert abs(mish(-20.0) + 20.0 * np.exp(-20.0)) < 20 * 1.3e-7
+    rng = np.random.default_rng(45)
+    v = np.concatenate([rng.uniform(-12, 12, 4000), rng.uniform(-90, 90, 1000), rng.uniform(-0.01, 0.01, 200)]).astype(F)
+    v64 = v.astype(np.float64)
+    s_got = np.array([sig(z) for z in v], np.float64)
+    s_want = 1.0 / (1.0 + np.exp(-np.clip(v64, -88.3762626647949, 88.3762626647949)))
+    assert np.all(np.abs(s_got - s_want) <= 4 * np.spacing(s_want.astype(F)).astype(np.float64) + 2e-44)  # (+ a few denormal steps at the clamp)
+    assert np.all((s_got > 0) & (s_got <= 1))
+    # sigmoid(-v) = 1 - sigmoid(v)
+    s_neg = np.array([sig(-z) for z in v], np.float64)
+    assert np.all(np.abs(s_got + s_neg - 1.0) <= 3e-7)
+    m_got = np.array([mish(z) for z in v], np.float64)
+    with np.errstate(over="ignore"):
+        m_want = v64 * np.tanh(np.where(v64 > 40, v64, np.log1p(np.exp(np.minimum(v64, 40)))))
+    assert np.all(np.abs(m_got - m_want) <= 1e-6 * np.abs(v64) + 1e-12), np.abs(m_got - m_want).max()
+    # mish has one minimum, -0.308841 near v = -1.1924
+    assert m_got.min() > -0.30885 and abs(min(mish(z) for z in np.arange(-1.3, -1.1, 0.001)) + 0.308841) < 1e-5
 
 
 # ----------------------------------------------------------------------------- quantize
