@@ -252,6 +252,17 @@ int ncnnhip_innerproduct_int8_ws(const int8_t* x_dev, size_t x_stride, int rows,
                                  ncnnhip_activation act, float* out_dev, size_t out_stride, void* workspace_dev,
                                  size_t workspace_bytes, void* stream);
 
+/* The same again for callers that cannot allocate device memory or pass a workspace (code under stream capture, serving
+ * loops and harnesses that forbid hipMalloc).  No counterpart in the reference.  The K-split scratch is an array of
+ * 4 MiB + 4 KiB that the library itself holds on every device it runs on (its address is looked up at ncnnhip_init, or at
+ * the first call on a device); the call allocates and frees nothing.  Shapes whose split needs more scratch than that are
+ * refused with -1 and a message naming ncnnhip_innerproduct_int8_ws.  All calls on one device share the one array: calls
+ * that overlap on a device (two streams, two threads) race; calls in stream order on one stream do not.  Results are
+ * those of ncnnhip_innerproduct_int8_ws bit for bit. */
+int ncnnhip_innerproduct_int8_noalloc(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output,
+                                      const int8_t* weight_dev, const float* scale_in_dev, const float* bias_dev,
+                                      ncnnhip_activation act, float* out_dev, size_t out_stride, void* stream);
+
 /* ------------------------------------------------------------------ Gemm int8
  * Dynamic per-row quantisation of A (src/layer/gemm.cpp:791-823): scales[i] = 127/absmax_i (1 for a
  * zero row), aq = float2int8(a*scale). */

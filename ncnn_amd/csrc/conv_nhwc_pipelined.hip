@@ -19,6 +19,7 @@
 // dumps its accumulator registers to scratch (register-major, fully coalesced) and bumps the tile's counter; the
 // last one adds the others' dumps to its own registers (integer addition: exact in any order), resets the counter
 // and runs the normal epilogue.  Nobody waits for anybody, so the grid may be larger than the chip.
+#include <mutex>
 #include <type_traits>
 
 #include "conv_nhwc.h"
@@ -849,4 +850,85 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
     return launch_status("conv_nhwc_pipelined_kernel<fc>");
 }
 
+// ---- InnerProduct through the K-split kernel on a scratch buffer the library holds itself, for callers that cannot
+// allocate (under stream capture, in a serving loop that must not touch the allocator).  The array below is the
+// workspace launch_fc_via_conv_pipelined otherwise gets from its caller; every device the library runs on holds its own
+// copy of it, at its own address, until the process ends.
+constexpr size_t STATIC_SCRATCH_PARTIAL_BYTES = 4u << 20;
+constexpr size_t STATIC_SCRATCH_BYTES = SPLIT_COUNTER_BYTES + STATIC_SCRATCH_PARTIAL_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+static void* g_scratch_ptr[STATIC_SCRATCH_MAX_DEVICES]; // device address of `scratch` on each device, 0 = not looked up yet
+static std::mutex g_scratch_mutex;
+
+// The array's name is only a handle on the host; its address on the CURRENT device comes from the runtime, once per device.
+int static_scratch_for_current_device(void** ptr)
+{
+    int dev = 0;
+    NCNNHIP_CHECK(hipGetDevice(&dev));
+    NCNNHIP_REQUIRE(dev >= 0 && dev < STATIC_SCRATCH_MAX_DEVICES, "device %d beyond the %d the static scratch table covers", dev, STATIC_SCRATCH_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev])
+    {
+        void* p = 0;
+        NCNNHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        NCNNHIP_REQUIRE(p, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return NCNNHIP_OK;
+}
+
+// one workgroup: the arrival counters at the head of the scratch start every call at zero, whatever the last call left
+__global__ __launch_bounds__(256) void clear_split_counters_kernel(unsigned* __restrict__ counters)
+{
+    for (int i = threadIdx.x; i < SPLIT_MAX_TILES; i += 256) counters[i] = 0u;
+}
+
 } // namespace ncnnhip
+
+using namespace ncnnhip;
+
+extern "C" int ncnnhip_innerproduct_int8_noalloc(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output, const int8_t* weight_dev,
+                                                 const float* scale_in_dev, const float* bias_dev, ncnnhip_activation act, float* out_dev, size_t out_stride,
+                                                 void* stream)
+{
+    NCNNHIP_REQUIRE(x_dev && weight_dev && scale_in_dev && out_dev, "ncnnhip_innerproduct_int8_noalloc: null pointer");
+    NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1, "ncnnhip_innerproduct_int8_noalloc: bad shape");
+    NCNNHIP_REQUIRE(x_stride >= (size_t)num_input && out_stride >= (size_t)num_output, "ncnnhip_innerproduct_int8_noalloc: stride too small");
+    void* ptr = 0;
+    int ret = static_scratch_for_current_device(&ptr);
+    if (ret != NCNNHIP_OK) return ret;
+    if (rows >= 8 && num_input % 64 == 0)
+    {
+        const size_t need = conv_nhwc_pipelined_workspace_words(num_output, rows, num_input / 64) * sizeof(int32_t);
+        NCNNHIP_REQUIRE(need <= STATIC_SCRATCH_BYTES,
+                        "ncnnhip_innerproduct_int8_noalloc: %d x %d -> %d needs %zu bytes of scratch, the library holds %zu; use ncnnhip_innerproduct_int8_ws",
+                        rows, num_input, num_output, need, (size_t)STATIC_SCRATCH_BYTES);
+        ConvEpilogue epi;
+        epi.scale_in = scale_in_dev;
+        epi.bias = bias_dev;
+        epi.scale_out = 0;
+        epi.act = act;
+        epi.out = out_dev;
+        epi.out_cstep = epi.out_nstep = 0;
+        epi.pix_per_img = rows;
+        epi.batch = 1;
+        epi.out_channel0 = 0;
+        epi.num_output = num_output;
+        epi.acc_out = 0;
+        if (need)
+        {
+            hipLaunchKernelGGL(clear_split_counters_kernel, dim3(1), dim3(256), 0, as_stream(stream), (unsigned*)ptr);
+            ret = launch_status("clear_split_counters_kernel");
+            if (ret != NCNNHIP_OK) return ret;
+        }
+        bool handled = false;
+        ret = launch_fc_via_conv_pipelined(x_dev, x_stride, rows, num_input, num_output, weight_dev, epi, out_stride, ptr, STATIC_SCRATCH_BYTES,
+                                           as_stream(stream), &handled);
+        if (handled) return ret;
+    }
+    // shapes the matrix-core kernel does not take run on the kernel that needs no scratch at all
+    return ncnnhip_innerproduct_int8(x_dev, x_stride, rows, num_input, num_output, weight_dev, scale_in_dev, bias_dev, act, out_dev, out_stride, 0, stream);
+}

@@ -3,6 +3,7 @@
 #include <string.h>
 
 #include "common.h"
+#include "conv_nhwc.h"
 
 namespace ncnnhip {
 
@@ -45,7 +46,9 @@ int ncnnhip_init(int device)
     NCNNHIP_CHECK(hipGetDeviceProperties(&prop, device));
     NCNNHIP_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, "kernels are built for gfx950 only, device is %s",
                     prop.gcnArchName);
-    return NCNNHIP_OK;
+    // this device's address of the library-held scratch (ncnnhip_innerproduct_int8_noalloc), looked up once per device
+    void* scratch_ptr = 0;
+    return static_scratch_for_current_device(&scratch_ptr);
 }
 
 const char* ncnnhip_last_error(void)

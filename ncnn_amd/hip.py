@@ -113,6 +113,8 @@ _SIGNATURES = {
     "ncnnhip_innerproduct_workspace_bytes": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
     "ncnnhip_innerproduct_int8_ws": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_size_t,
                                      C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_innerproduct_int8_noalloc": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p,
+                                          C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_quantize_tensor": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_transpose_f32": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
