@@ -246,8 +246,87 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and not lowbit) else None,
-                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_mfma_kernel", "bytes_per_launch": algo},
+                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_upfront_kernel", "bytes_per_launch": algo},
     }
+
+
+def measure_peak_mfma_i8(lib, check, rt, random_operands, iters=20000, reps=5):
+    """int8 matrix-core rate with nothing else going on: (POP/s, shader MHz, operations per clock per compute unit)."""
+    import ncnn_amd
+    scratch = ncnn_amd.DeviceBuffer.empty((8,), np.int64)
+    scratch.fill_bytes(0, rt.stream)
+    name = C.create_string_buffer(128)
+    cus = C.c_int()
+    check(lib.ncnnhip_device_info(name, 128, C.byref(cus), None))
+    check(lib.ncnnhip_peak_mfma_i8(iters, int(random_operands), scratch.ptr, rt.stream))  # warm-up (clocks ramp)
+    rt.sync()
+    ev = _events(lib, check, 2)
+    best = None
+    for _ in range(reps):
+        check(lib.ncnnhip_event_record(ev[0], rt.stream))
+        check(lib.ncnnhip_peak_mfma_i8(iters, int(random_operands), scratch.ptr, rt.stream))
+        check(lib.ncnnhip_event_record(ev[1], rt.stream))
+        check(lib.ncnnhip_event_synchronize(ev[1]))
+        ms = _elapsed(lib, check, ev[0], ev[1])
+        clocks = scratch.to_numpy(rt.stream)
+        ops = cus.value * 4.0 * iters * 8 * 65536
+        r = (ops / (ms * 1e-3) / 1e12, float(clocks[0]) / max(float(clocks[1]), 1.0) * 100.0, 4.0 * iters * 8 * 65536 / max(float(clocks[0]), 1.0))
+        if best is None or r[0] > best[0]:
+            best = r
+    return {"tops": best[0], "shader_mhz": best[1], "ops_per_clk_per_cu": best[2], "compute_units": cus.value,
+            "operands": "random" if random_operands else "zeros", "instruction": "v_mfma_i32_32x32x32_i8", "mfma_per_wavefront": iters * 8}
+
+
+def measure_peak_hbm_read(lib, check, rt, nbytes, loads_per_lane=16, launches=200):
+    """GB/s of a kernel that only reads `nbytes`, back-to-back launches over rotating copies larger than the last-level cache."""
+    import ncnn_amd
+    nbytes = max(4096, nbytes // 16 * 16)
+    copies = int(np.ceil(600e6 / nbytes)) + 1
+    bufs = []
+    for _ in range(copies):
+        b = ncnn_amd.DeviceBuffer(nbytes)
+        b.fill_bytes(1, rt.stream)
+        bufs.append(b)
+    sink = ncnn_amd.DeviceBuffer.zeros(64, rt.stream)
+    for i in range(20):
+        check(lib.ncnnhip_peak_hbm_read(bufs[i % copies].ptr, nbytes, loads_per_lane, sink.ptr, rt.stream))
+    rt.sync()
+    ev = _events(lib, check, 2)
+    check(lib.ncnnhip_event_record(ev[0], rt.stream))
+    for i in range(launches):
+        check(lib.ncnnhip_peak_hbm_read(bufs[i % copies].ptr, nbytes, loads_per_lane, sink.ptr, rt.stream))
+    check(lib.ncnnhip_event_record(ev[1], rt.stream))
+    check(lib.ncnnhip_event_synchronize(ev[1]))
+    us = _elapsed(lib, check, ev[0], ev[1]) * 1e3 / launches
+    return {"gbs": nbytes / us / 1e3, "us_per_launch": us, "bytes": nbytes, "loads_per_lane": loads_per_lane, "copies_rotated": copies}
+
+
+def bench_peak(args, what, arg):
+    """The chip's own ceilings, measured: `peak:mfma_i8[:zeros|random]` and `peak:hbm_read:<bytes>[:<loads per lane>]`."""
+    import ncnn_amd
+    from ncnn_amd.hip import check, lib as load
+    lib = load()
+    rt = ncnn_amd.Runtime(0)
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic"}
+    if what == "mfma_i8":
+        kinds = [arg == "random"] if arg in ("zeros", "random") else [False, True]
+        res = [measure_peak_mfma_i8(lib, check, rt, k, iters=max(1000, args.steps * 400)) for k in kinds]
+        top = res[-1]
+        return dict(base, metric="int8 TOPS", value=top["tops"], unit="TOPS", ms_per_step=None, dtype="int8",
+                    config={"workload": "register-only spin of v_mfma_i32_32x32x32_i8 on every SIMD: the matrix pipe's sustained rate", "runs": res},
+                    roofline={"bound": "mfma", "achieved": top["tops"], "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": top["tops"] / INT8_MFMA_PEAK_TOPS,
+                              "traffic": None, "kernel": "peak_mfma_i8_kernel"})
+    if what == "hbm_read":
+        parts = arg.split(":") if arg else []
+        nbytes = int(float(parts[0])) if parts else 256 << 20
+        lpl = int(parts[1]) if len(parts) > 1 else 16
+        r = measure_peak_hbm_read(lib, check, rt, nbytes, lpl, launches=max(50, args.steps * 4))
+        return dict(base, metric="HBM GB/s", value=r["gbs"], unit="GB/s", ms_per_step=r["us_per_launch"] * 1e-3, dtype="u8",
+                    config={"workload": "read-only kernel over %d bytes, %d 16-byte loads in flight per lane, weight-stream rotation as in the block-quant workload"
+                                        % (r["bytes"], lpl), "run": r},
+                    roofline={"bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": r["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                              "kernel": "peak_hbm_read_kernel", "bytes_per_launch": r["bytes"]})
+    raise SystemExit("unknown peak workload " + what)
 
 
 def bench_mha(args, embed, heads, src, past):
@@ -629,7 +708,8 @@ def main():
     ap.add_argument("--workload", default="gemm4096",
                     help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
-                         "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI)")
+                         "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI) | "
+                         "peak:mfma_i8[:zeros|random] | peak:hbm_read:<bytes>[:<loads per lane>] (the chip's measured ceilings)")
     ap.add_argument("--streams", type=int, default=1, help="net workloads: forward passes kept in flight, each on its own stream of the net")
     ap.add_argument("--graph", type=int, default=0,
                     help="net workloads: 0 = one Extractor per pass, layer by layer on a stream (faster on this ROCm: a replayed graph costs more per kernel node "
@@ -658,6 +738,9 @@ def main():
     elif args.workload.startswith("net:"):
         _, which, batch = args.workload.split(":")
         line = bench_net(args, which, int(batch))
+    elif args.workload.startswith("peak:"):
+        parts = args.workload.split(":", 2)
+        line = bench_peak(args, parts[1], parts[2] if len(parts) > 2 else "")
     elif args.workload.startswith("layers:"):
         _, which, batch = args.workload.split(":")
         line = bench_layers(args, which, int(batch))

@@ -350,6 +350,17 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
                           int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev,
                           void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------ measured ceilings (benchmark support)
+ * No counterpart in the reference.  What this chip sustains, to set beside the published peaks in a roofline line:
+ * ncnnhip_peak_mfma_i8 spins v_mfma_i32_32x32x32_i8 from registers on every SIMD (one workgroup of four wavefronts per
+ * compute unit, eight independent accumulator chains, `iters` rounds of 8 instructions = iters * 8 * 65536 operations per
+ * wavefront) on all-zero or pseudo-random operands; scratch_dev (>= 64 bytes) receives two int64: the shader cycles and
+ * the 100 MHz wall ticks workgroup 0 spent in the loop.  ncnnhip_peak_hbm_read reads `bytes` (a multiple of 16) once with
+ * 16-byte non-temporal loads, `loads_per_lane` (4, 8, 16, 32) of them in flight per lane, and writes nothing; time it with
+ * events over buffers larger than the last-level cache to get the read bandwidth a kernel of that size can reach. */
+int ncnnhip_peak_mfma_i8(int iters, int random_operands, void* scratch_dev, void* stream);
+int ncnnhip_peak_hbm_read(const void* src_dev, size_t bytes, int loads_per_lane, void* scratch_dev, void* stream);
+
 #pragma GCC visibility pop
 
 #ifdef __cplusplus

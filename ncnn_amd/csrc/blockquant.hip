@@ -695,6 +695,263 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
     }
 }
 
+// ---- the same contraction with every weight byte of a wavefront requested before the first one is used ----
+// A bandwidth kernel on this chip is paced by the bytes it has in flight: 8 TB/s times a microsecond of memory latency is
+// 8 MB, 32 KB per compute unit, and a matrix of 4096 rows is only 64 KB per compute unit in all.  So a workgroup still owns
+// one tile of 16 weight rows, but its K blocks are dealt to as many wavefronts as it takes for each to hold ALL its blocks
+// in registers (NB of them, 4 VGPRs each): a wavefront issues its whole share of the weight stream in one go, then
+// multiplies block after block as the bytes arrive, and what is left to do when the last byte lands is one block.
+// Requests go out in the order their data is needed (loads return in order; the compiler's scheduler, left alone, issues
+// them in reverse, hence the scheduling barriers).  Activations and descales are parked in a piece of LDS that belongs to
+// the wavefront alone, so no workgroup barrier stands between the loads and the arithmetic (a barrier would first wait
+// for every load in flight).
+//   ACT_LDS (decoding, up to MT <= 4 activation rows): the rows' K range of this wavefront goes through that LDS piece
+//   once, ahead of the weights.
+//   otherwise (up to 16 rows): each block's 16 rows x 64 halves ride in registers (8 VGPRs per block), requested right
+//   behind the block's weights with a COALESCED lane mapping (8 lanes = one row's 128 bytes; in the matrix core's own
+//   operand mapping a 16-lane group touches 16 rows, 16 cache lines for 256 bytes, and the loads took four times the
+//   weight stream's share of the L1 pipe), and are turned into the operand mapping through 2.25 KB of LDS per wavefront
+//   when the block is multiplied.
+template<int NB, int MAXW, int MT, bool ACT_LDS>
+__global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
+                                                                        const v4i_bq* __restrict__ wpk, const float4* __restrict__ dpk,
+                                                                        const float* __restrict__ c, int bt, float alpha, float beta,
+                                                                        float* __restrict__ out, size_t out_stride)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_up[];
+    constexpr int ACT_PITCH = NB * 128 + 128;                               // ACT_LDS: bytes from one staged activation row to the next (off the bank stride)
+    constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;               // ACT_LDS: 16-byte activation loads per lane
+    constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;  // rows the staging stores touch (>= MT: every lane stores, no branch)
+    constexpr int TR_PITCH = 144;                                           // !ACT_LDS: one row of a block (128 bytes) + 16: 16 rows land on 16 different bank groups
+    constexpr int WAVE_BYTES = 1024 + (ACT_LDS ? AROWS * ACT_PITCH : 16 * TR_PITCH); // 64 float4 of descales (NB * 4 used), then the activations
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int tile = blockIdx.x;
+    const int m = lane & 15;
+    const int kg = lane >> 4;
+
+    // K blocks of this wavefront: NB each, the last one what is left (possibly none: it then re-reads block 0 and adds zeros)
+    const int kb_begin = wave * NB;
+    int nkb = kblocks - kb_begin;
+    nkb = nkb > NB ? NB : nkb;
+    nkb = nkb < 0 ? 0 : nkb;
+    const int kb_base = nkb > 0 ? kb_begin : 0;
+
+    unsigned char* mine = lds_up + wave * WAVE_BYTES;
+    float4* my_d = reinterpret_cast<float4*>(mine);
+    unsigned char* my_a = mine + 1024;
+
+    // (1) ACT_LDS: the activations of the wavefront's K range.  Every load is unconditional, from a clamped address, and
+    // masked afterwards (a guarded load becomes a branch, and the compiler waits for every load in flight past a branch).
+    v4i_bq areg[AV];
+    if (ACT_LDS)
+    {
+#pragma unroll
+        for (int q = 0; q < AV; q++)
+        {
+            const int idx = q * 64 + lane;
+            const int r = idx / (NB * 8), v = idx - r * (NB * 8);
+            const int k = kb_base * 64 + v * 8;
+            const bool ok = v < nkb * 8 && k < K; // K % 16 == 0: a vector of 8 halves is all in or all out
+            const int rr = r < M ? r : 0;
+            areg[q] = *reinterpret_cast<const v4i_bq*>(a + (size_t)rr * a_stride + (ok ? k : 0));
+        }
+    }
+    // (2) descales of the wavefront's blocks: float4 number j of them is (block j / 4, row group j % 4)
+    const float4* dt = dpk + ((size_t)tile * kblocks + kb_base) * 4;
+    __builtin_amdgcn_sched_barrier(0);
+    const float4 dreg = dt[lane < nkb * 4 ? lane : 0];
+    __builtin_amdgcn_sched_barrier(0);
+    // (3) the weights, all of them; !ACT_LDS: each block's activations right behind its weights.  Lane l fetches 16 bytes of
+    // rows l/8 and l/8 + 8, piece l%8 of the block's 128 bytes per row; a chunk beyond K is read from the start of the row
+    // (it meets packed weights that are zero there), rows from M up repeat row 0 (their results are never stored).
+    const v4i_bq* wt = wpk + ((size_t)tile * kblocks + kb_base) * 64 + lane;
+    v4i_bq w[NB];
+    v4i_bq a0[ACT_LDS ? 1 : NB], a1[ACT_LDS ? 1 : NB];
+    const int tr_row = lane >> 3, tr_piece = lane & 7;
+    const __half* arow0 = a + (size_t)(tr_row < M ? tr_row : 0) * a_stride;
+    const __half* arow1 = a + (size_t)(tr_row + 8 < M ? tr_row + 8 : 0) * a_stride;
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        w[i] = __builtin_nontemporal_load(wt + (size_t)(i < nkb ? i : 0) * 64);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!ACT_LDS)
+        {
+            const int k = (kb_base + (i < nkb ? i : 0)) * 64 + tr_piece * 8;
+            const int kk = k < K ? k : 0;
+            a0[ACT_LDS ? 0 : i] = *reinterpret_cast<const v4i_bq*>(arow0 + kk);
+            a1[ACT_LDS ? 0 : i] = *reinterpret_cast<const v4i_bq*>(arow1 + kk);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // (4) park activations and descales in the wavefront's own LDS (same wavefront writes and reads: program order holds)
+    if (ACT_LDS)
+    {
+#pragma unroll
+        for (int q = 0; q < AV; q++)
+        {
+            const int idx = q * 64 + lane;
+            const int r = idx / (NB * 8), v = idx - r * (NB * 8);
+            const int k = kb_base * 64 + v * 8;
+            const bool ok = v < nkb * 8 && k < K;
+            v4i_bq t = areg[q];
+#pragma unroll
+            for (int e = 0; e < 4; e++) t[e] = ok ? t[e] : 0;
+            *reinterpret_cast<v4i_bq*>(my_a + r * ACT_PITCH + v * 16) = t; // unconditional: a guarded store would pull its load into the branch
+        }
+    }
+    my_d[lane] = lane < nkb * 4 ? dreg : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    // (5) block after block, as the weights arrive
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    const unsigned char* act_rd = ACT_LDS ? my_a + (m < M && m < MT ? m : 0) * ACT_PITCH + kg * 32 : my_a + m * TR_PITCH + kg * 32;
+    unsigned char* tr_wr = my_a + tr_row * TR_PITCH + tr_piece * 16;
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        const v8h wa = bytes_to_halves(w[i][0], w[i][1]);
+        const v8h wb = bytes_to_halves(w[i][2], w[i][3]);
+        union
+        {
+            v4i_bq i4;
+            v8h h;
+        } xa, xb;
+        if (ACT_LDS)
+        {
+            xa.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128);
+            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128 + 16);
+        }
+        else
+        {
+            // the block's 16 rows x 128 bytes from the fetch mapping into the operand mapping (the wavefront's LDS operations
+            // execute in order, so the next block's stores cannot overtake these reads)
+            *reinterpret_cast<v4i_bq*>(tr_wr) = a0[ACT_LDS ? 0 : i];
+            *reinterpret_cast<v4i_bq*>(tr_wr + 8 * TR_PITCH) = a1[ACT_LDS ? 0 : i];
+            xa.i4 = *reinterpret_cast<const v4i_bq*>(act_rd);
+            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + 16);
+        }
+        v4f t = {0.f, 0.f, 0.f, 0.f};
+        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, t, 0, 0, 0);
+        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
+        const float4 d = my_d[i * 4 + kg]; // zero for a block beyond the wavefront's range
+        acc[0] = fmaf(t[0], d.x, acc[0]);
+        acc[1] = fmaf(t[1], d.y, acc[1]);
+        acc[2] = fmaf(t[2], d.z, acc[2]);
+        acc[3] = fmaf(t[3], d.w, acc[3]);
+    }
+
+    // (6) combine the wavefronts' K ranges in wavefront order; accumulator r of lane l is (weight row (l/16)*4 + r, activation row l%16)
+    // (the exchange buffer lies over the wavefronts' own pieces, which everybody has finished with after the first barrier)
+    float4* red = reinterpret_cast<float4*>(lds_up);
+    __syncthreads();
+    red[wave * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    if (wave == 0 && m < M)
+    {
+        float4 f = red[lane];
+        for (int w2 = 1; w2 < nwaves; w2++)
+        {
+            const float4 o = red[w2 * 64 + lane];
+            f.x = add_rn(f.x, o.x);
+            f.y = add_rn(f.y, o.y);
+            f.z = add_rn(f.z, o.z);
+            f.w = add_rn(f.w, o.w);
+        }
+        const float fr[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int j = tile * 16 + kg * 4 + r;
+            if (j < N)
+            {
+                float v = fr[r];
+                if (bt >= 0) v = add_rn(mul_rn(load_c(c, bt, m, j, N), beta), v);
+                out[(size_t)m * out_stride + j] = mul_rn(v, alpha); // (a non-temporal store measured 1-3 % slower)
+            }
+        }
+    }
+}
+
+// One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
+template<int NB, int MAXW, int MT, bool ACT_LDS>
+static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, int K, int kblocks, const v4i_bq* wpk, const float4* dpk, const float* c, int bt,
+                              float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+{
+    constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;
+    constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;
+    constexpr int WAVE_BYTES = 1024 + (ACT_LDS ? AROWS * (NB * 128 + 128) : 16 * 144);
+    const int nwaves = (kblocks + NB - 1) / NB;
+    const size_t lds = (size_t)nwaves * WAVE_BYTES; // >= 1 KB per wavefront, which the final exchange reuses
+    if (lds > 160 * 1024)
+    {
+        *handled = false;
+        return NCNNHIP_OK;
+    }
+    auto kernel = blockquant8_upfront_kernel<NB, MAXW, MT, ACT_LDS>;
+    if (lds > 65536)
+    {
+        // more than the 64 KB a kernel gets by default: raise this kernel's limit once (the chip has 160 KB per compute unit)
+        static bool raised = false;
+        if (!raised)
+        {
+            NCNNHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, c, bt, alpha, beta, out, out_stride);
+    return launch_status("blockquant8_upfront_kernel");
+}
+
+// handled = false: the shape is left to the ring kernel (K beyond 16384, or more than 4 rows with K beyond 8192)
+static int launch_blockquant8_upfront(const __half* a, size_t a_stride, int M, int N, int K, const v4i_bq* wpk, const float4* dpk, const float* c, int bt,
+                                      float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+{
+    const int kblocks = (K + 63) / 64;
+    *handled = true;
+#define UPFRONT(NB_, MAXW_, MT_, LDS_) \
+    return launch_upfront_one<NB_, MAXW_, MT_, LDS_>(a, a_stride, M, N, K, kblocks, wpk, dpk, c, bt, alpha, beta, out, out_stride, stream, handled)
+    if (M <= 4)
+    {
+        // decoding: 16 blocks per wavefront while 4, 8 or 16 wavefronts cover K; 12 where that wastes fewer requests (K = 11008: 15 wavefronts)
+        if (kblocks <= 64)
+        {
+            if (M == 1) UPFRONT(16, 4, 1, true);
+            if (M == 2) UPFRONT(16, 4, 2, true);
+            UPFRONT(16, 4, 4, true);
+        }
+        if (kblocks <= 128)
+        {
+            if (M == 1) UPFRONT(16, 8, 1, true);
+            if (M == 2) UPFRONT(16, 8, 2, true);
+            UPFRONT(16, 8, 4, true);
+        }
+        if (kblocks <= 192)
+        {
+            if (M == 1) UPFRONT(12, 16, 1, true);
+            if (M == 2) UPFRONT(12, 16, 2, true);
+            UPFRONT(12, 16, 4, true);
+        }
+        if (kblocks <= 256)
+        {
+            if (M == 1) UPFRONT(16, 16, 1, true);
+            if (M == 2) UPFRONT(16, 16, 2, true);
+            UPFRONT(16, 16, 4, true);
+        }
+    }
+    else
+    {
+        // 12 VGPRs per block: 16 blocks per wavefront fit while a SIMD holds at most two wavefronts of the workgroup
+        if (kblocks <= 64) UPFRONT(16, 4, 1, false);
+        if (kblocks <= 128) UPFRONT(16, 8, 1, false);
+    }
+#undef UPFRONT
+    *handled = false;
+    return NCNNHIP_OK;
+}
+
 static int check_blockquant(const void* a, const void* b, const void* scales, const void* out, int M, int N, int K, int bits, int block,
                             const void* c, int bt)
 {
@@ -822,6 +1079,12 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
         const size_t act_bytes = (size_t)mc * kblocks * 64 * sizeof(__half);
+        bool handled = false;
+        int ret = launch_blockquant8_upfront(ah + (size_t)m0 * a_stride, a_stride, mc, N, K, reinterpret_cast<const v4i_bq*>(packed_w_dev),
+                                             reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride,
+                                             as_stream(stream), &handled);
+        if (ret != NCNNHIP_OK) return ret;
+        if (handled) continue;
         if (act_bytes <= 32768 && tiles >= 512) // measured: pays from about 8192 weight rows (up to four rows of 4096), not for long rows (K = 11008) or few tiles
             hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS_LDS, 1, true>), dim3(tiles), dim3(256), (size_t)kblocks * 64 + act_bytes, as_stream(stream),
                                ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),

@@ -438,7 +438,12 @@ def test_blockquant_low_bit_decode_shape_fp16_activations(rt, bits):
 @pytest.mark.parametrize("m,n,k,block,bt", [(1, 512, 4096, 64, -1), (4, 256, 4096, 64, 4), (16, 256, 4096, 64, 3), (16, 250, 11008, 64, -1),
                                             (3, 37, 208, 64, 1), (1, 16, 64, 64, 0), (20, 64, 1024, 128, 2), (7, 100, 4096 + 48, 128, -1),
                                             # more than 512 tiles of 16 rows: workgroups stay and walk the tiles (ragged last tile, odd K blocks)
-                                            (1, 11008, 4096, 64, -1), (4, 8200 + 8, 4096, 64, -1), (4, 8200 + 5, 1024 + 64, 64, 4), (16, 9000, 512, 128, 3), (2, 16400, 192, 64, 1)])
+                                            (1, 11008, 4096, 64, -1), (4, 8200 + 8, 4096, 64, -1), (4, 8200 + 5, 1024 + 64, 64, 4), (16, 9000, 512, 128, 3), (2, 16400, 192, 64, 1),
+                                            # every wavefront count of the kernel that requests a wavefront's whole share at once (8, 15 and 16 wavefronts of 16 / 12 /
+                                            # 16 K blocks, a last wavefront with a single block and with none), rows through LDS (up to 4) and in registers (5 to 16),
+                                            # and K beyond its reach (the ring kernel takes over)
+                                            (2, 48, 8192, 64, -1), (1, 33, 12288, 64, 4), (3, 40, 11008 + 16, 64, 1), (4, 32, 16384, 128, -1), (1, 32, 16384 + 64, 64, -1),
+                                            (9, 40, 8192, 64, 1), (5, 24, 4096 + 64, 64, -1), (12, 40, 12288, 64, -1), (16, 4096, 4096, 64, 4), (2, 20, 1024 + 16, 64, 3)])
 def test_blockquant_packed_matrix_core_path(rt, m, n, k, block, bt):
     _say("blockquant packed", m, n, k, block, bt)
     a, packed, scales = cases.blockquant_case(m + n + k + block, m, n, k, 8, block)
