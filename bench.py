@@ -62,9 +62,20 @@ def cpu_baseline_gemm(n, k, per_col, budget_s=12.0):
             cpubaseline.gemm(a, packed, n, sb, bias)
             times.append(time.perf_counter() - t0)
         dt = float(np.mean(times))
-        return {"value": 2.0 * rows * n * k / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
-                "sample": "%d of %d rows of the same Gemm (N=%d, K=%d): per-row quantise + AVX512-VNNI int8 GEMM + dequantise/bias, OpenMP, mean of %d runs "
-                          "(%.1f s in all)" % (rows, n, n, k, len(times), sum(times))}
+        # the same on one thread, on an eighth of the rows
+        cpubaseline.set_num_threads(1)
+        a1 = a[: max(16, rows // 8)]
+        cpubaseline.gemm(a1, packed, n, sb, bias)
+        t1 = []
+        while len(t1) < 2 or (sum(t1) < budget_s / 4 and len(t1) < 1000):
+            t0 = time.perf_counter()
+            cpubaseline.gemm(a1, packed, n, sb, bias)
+            t1.append(time.perf_counter() - t0)
+        cpubaseline.set_num_threads(threads)
+        return dict({"value": 2.0 * rows * n * k / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+                     "value_1_thread": 2.0 * a1.shape[0] * n * k / min(t1) / 1e12,
+                     "sample": "%d of %d rows of the same Gemm (N=%d, K=%d): per-row quantise + AVX512-VNNI int8 GEMM + dequantise/bias, OpenMP, mean of %d runs "
+                               "(%.1f s in all); one thread: %d rows, best of %d" % (rows, n, n, k, len(times), sum(times), a1.shape[0], len(t1))}, **host_cpu_info())
     threads = min(oracle.num_threads(), 16)
     oracle.set_num_threads(threads)
     rng = np.random.default_rng(0)
@@ -82,6 +93,53 @@ def cpu_baseline_gemm(n, k, per_col, budget_s=12.0):
     tops = 2.0 * rows * n * k / dt / 1e12
     return {"value": tops, "unit": "TOPS", "cores": threads, "kind": "port",
             "sample": "%d of %d rows of the same Gemm (N=%d, K=%d), scalar OpenMP oracle, %.1f s" % (rows, n, n, k, dt)}
+
+
+def host_cpu_info():
+    """CPU model, logical CPUs and the ISA flags that matter for an int8 path, from /proc/cpuinfo."""
+    model, flags, n = "unknown", set(), 0
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name") and model == "unknown":
+                    model = ln.split(":", 1)[1].strip()
+                elif ln.startswith("flags") and not flags:
+                    flags = set(ln.split(":", 1)[1].split())
+                elif ln.startswith("processor"):
+                    n += 1
+    except OSError:
+        pass
+    keep = [f for f in ("sse4_2", "avx2", "fma", "avx512f", "avx512bw", "avx512_vnni", "avx_vnni", "amx_int8") if f in flags]
+    return {"cpu_model": model, "logical_cpus": n or (os.cpu_count() or 1), "isa_flags": keep}
+
+
+def cpu_baseline_blockquant(n, k, m, bits, block, budget_s=12.0):
+    """The reference's only block-quant implementation is the naive fp32 loop (src/layer/gemm.cpp:425-483), OpenMP over the M
+    activation rows only: restated in the oracle, timed here on a bounded number of weight rows with min(M, threads) threads
+    (one thread at M = 1, as the reference runs it), and again with every thread over the weight rows for comparison."""
+    from oracle import oracle
+    from ncnn_amd import synth
+    info = host_cpu_info()
+    all_threads = min(oracle.num_threads(), 16)
+    rows = min(n, 2048)
+    a, packed, scales = synth.blockquant_operands(7, m, rows, k, bits, block)
+    res = {}
+    for label, threads in (("reference_threads", max(1, min(m, all_threads))), ("all_threads", all_threads)):
+        oracle.set_num_threads(threads)
+        oracle.gemm_blockquant(a, packed, scales, bits, block)
+        times, t_start = [], time.perf_counter()
+        while len(times) < 2 or (time.perf_counter() - t_start < budget_s / 2 and len(times) < 1000):
+            t0 = time.perf_counter()
+            oracle.gemm_blockquant(a, packed, scales, bits, block)
+            times.append(time.perf_counter() - t0)
+        nbytes = packed.nbytes + scales.nbytes + a.nbytes + m * rows * 4
+        res[label] = (nbytes / min(times) / 1e9, threads, len(times), sum(times))
+    oracle.set_num_threads(all_threads)
+    v, threads, reps, total = res["reference_threads"]
+    return dict({"value": v, "unit": "GB/s", "cores": threads, "kind": "port", "value_all_threads": res["all_threads"][0], "cores_all_threads": res["all_threads"][1],
+                 "sample": "%d of %d weight rows of the same Gemm (K=%d, M=%d), naive fp32 block-quant loop as in the reference (OpenMP over M only: %d thread%s), "
+                           "best of %d runs (%.1f s); all_threads = the same loop with the weight rows spread over %d threads"
+                           % (rows, n, k, m, threads, "" if threads == 1 else "s", reps, total, res["all_threads"][1])}, **info)
 
 
 def measured_traffic(key):
@@ -165,11 +223,19 @@ def bench_gemm(args, size):
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "standalone int8 Gemm M=N=K=%d: per-row quantise A (fp32->int8) + int8 MFMA Gemm + fused dequantise/bias to fp32" % size,
-                   "b_scale": args.b_scale, "operand_layout": "tiled" if tiled else "row-major",
+                   "b_scale": args.b_scale,
+                   "parity": ("per-column B scales are a generalisation ncnn's Gemm cannot express: parity unpinned by the reference (own formula, "
+                              "((float)acc*(1/sA_i))*(1/sB_j)); --b-scale per_tensor is the reference's form" if args.b_scale == "per_column"
+                              else "the reference's per-tensor B scale: bit-exact against the oracle"), "operand_layout": "tiled" if tiled else "row-major",
                    "kernel_ms": {"gemm_int8": gemm_ms, "quantize_rows": quant_ms}},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": measured_traffic("gemm%d" % size), "kernel": "gemm_int8", "ops_per_launch": ops},
     }
+    # what the matrix pipe of THIS chip sustains on operands like these (register-only spin, random bytes), beside the published peak
+    mp = measure_peak_mfma_i8(lib, check, rt, True, iters=8000, reps=3)
+    line["roofline"].update(measured_peak=mp["tops"], frac_of_measured=achieved / mp["tops"],
+                            measured_peak_how="v_mfma_i32_32x32x32_i8 from registers on all %d SIMDs, pseudo-random operands: %.0f MHz, %.0f ops/clk/CU"
+                                              % (mp["compute_units"] * 4, mp["shader_mhz"], mp["ops_per_clk_per_cu"]))
     if not args.no_cpu:
         # the CPU leg: first the checker (a row sample of the timed output buffer against the oracle), then the baseline timing
         from oracle import oracle
@@ -239,15 +305,23 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     algo = wbytes + abytes + m * n * 4
     achieved = algo / (k_ms * 1e-3) / 1e9
     ms_per_step = wall * 1e3 / args.steps
-    return {
+    del d_w, d_s
+    floor = measure_peak_hbm_read(lib, check, rt, int(algo), 8, launches=200)  # a kernel that only READS as many bytes, same launch pattern
+    line = {
         "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, %d-bit weights in blocks of %d, fp32 block scales, %s activations" % (m, n, k, bits, block, args.act),
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and not lowbit) else None,
-                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_upfront_kernel", "bytes_per_launch": algo},
+                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_upfront_kernel", "bytes_per_launch": algo,
+                     "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
+                     "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"
+                                          % floor["us_per_launch"]},
     }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_blockquant(n, k, m, bits, block)
+    return line
 
 
 def measure_peak_mfma_i8(lib, check, rt, random_operands, iters=20000, reps=5):
@@ -630,7 +704,7 @@ def bench_layers(args, which, batch):
                                % (which, len(plans), batch),
                    "images_per_s": batch / (ms_per_step * 1e-3), "slowest_layer": [worst[0], worst[8]]},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": None, "kernel": "conv_nhwc_kernel (all layers of the pass)", "ops_per_launch": ops},
+                     "traffic": None, "kernel": "conv_nhwc_pipelined_kernel and the depthwise / pointwise / InnerProduct kernels (all layers of the pass)", "ops_per_launch": ops},
     }
 
 
@@ -696,7 +770,7 @@ def bench_net(args, which, batch):
                    "submission": "recorded pass replayed as one graph launch" if graph is not None else "layer by layer through an Extractor",
                    "passes_in_flight": len(ring)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": None, "kernel": "whole pass (conv_nhwc_kernel dominates)", "ops_per_launch": ops},
+                     "traffic": None, "kernel": "whole pass (conv_nhwc_pipelined_kernel dominates)", "ops_per_launch": ops},
     }
 
 

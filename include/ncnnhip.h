@@ -224,6 +224,12 @@ typedef struct ncnnhip_pool_desc
     int outw, outh;
     int global_pooling;
     int avgpool_count_include_pad;
+    /* Average pooling with avgpool_count_include_pad == 0 divides by the number of taps inside this rectangle of IMAGE
+     * coordinates, [count_x0, count_x1) x [count_y0, count_y1); taps inside it but outside the image add zero and still
+     * count.  The reference excludes taps by the layer's own pad parameters (and the tail pad only in pad_mode 0,
+     * src/layer/pooling.cpp:255-305), so with SAME padding (pad_mode 2 / 3, pad parameters 0) the rectangle is the whole
+     * bordered image.  count_x1 <= count_x0 or count_y1 <= count_y0 (e.g. all zero) means the image itself. */
+    int count_x0, count_x1, count_y0, count_y1;
 } ncnnhip_pool_desc;
 int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, float* dst_dev, void* stream);
 /* Windowed max pooling (src/layer/pooling.cpp:105-222) of an int8 blob that holds Quantize(x, s), s > 0: the result is

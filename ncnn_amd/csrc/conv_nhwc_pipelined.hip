@@ -565,7 +565,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                         if (fusion.relu_after)
                         {
 #pragma unroll
-                            for (int e = 0; e < 4; e++) v[e] = fmaxf(v[e], 0.f);
+                            for (int e = 0; e < 4; e++) v[e] = v[e] < 0.f ? 0.f : v[e]; // the ReLU LAYER's statement (src/layer/relu.cpp:36-37): a NaN stays, unlike fmaxf
                         }
                         *reinterpret_cast<v4f*>(static_cast<float*>(epi.out) + o) = v;
                         if (fusion.q8_out)

@@ -276,12 +276,7 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
                 if (BT == 4) f = add_rn(f, colc[j]);
                 f4[j] = mul_rn(f, alpha);
             }
-#ifdef GEMM_NT_STORE
-            typedef float v4f_store __attribute__((ext_vector_type(4)));
-            __builtin_nontemporal_store((v4f_store){f4[0], f4[1], f4[2], f4[3]}, reinterpret_cast<v4f_store*>(orow));
-#else
-            *reinterpret_cast<float4*>(orow) = make_float4(f4[0], f4[1], f4[2], f4[3]);
-#endif
+            *reinterpret_cast<float4*>(orow) = make_float4(f4[0], f4[1], f4[2], f4[3]); // (non-temporal stores: neutral at 4096 cubed, 3 % slower at 8192 cubed)
         }
     }
 }

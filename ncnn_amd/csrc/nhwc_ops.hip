@@ -172,6 +172,7 @@ struct PoolGeom
     int kw, kh, sw, sh, pad_top, pad_left;
     int type;              // 0 max, 1 average
     int count_include_pad; // average only
+    int cx0, cx1, cy0, cy1; // average without count_include_pad: taps inside this rectangle (image coordinates) make up the divisor
 };
 
 __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restrict__ src, float* __restrict__ dst, PoolGeom g, size_t total)
@@ -209,17 +210,17 @@ __global__ __launch_bounds__(256) void pooling_nhwc_kernel(const float* __restri
             for (int kx = 0; kx < g.kw; kx++)
             {
                 const int y = y0 + ky, x = x0 + kx;
-                if ((unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w)
+                const bool in = (unsigned)y < (unsigned)g.h && (unsigned)x < (unsigned)g.w;
+                // which taps take part: all of them with count_include_pad, else those inside the counted rectangle (the
+                // reference skips the others even where they lie on the image); a tap off the image is the border's zero
+                const bool counted = g.count_include_pad || (x >= g.cx0 && x < g.cx1 && y >= g.cy0 && y < g.cy1);
+                if (counted)
                 {
-                    const v4f v = *reinterpret_cast<const v4f*>(base + ((size_t)y * g.w + x) * g.cp);
+                    v4f v = {0.f, 0.f, 0.f, 0.f};
+                    if (in) v = *reinterpret_cast<const v4f*>(base + ((size_t)y * g.w + x) * g.cp);
 #pragma unroll
                     for (int e = 0; e < 4; e++) r[e] = add_rn(r[e], v[e]);
                     area++;
-                }
-                else if (g.count_include_pad)
-                {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) r[e] = add_rn(r[e], 0.f);
                 }
             }
         const float div = g.count_include_pad ? (float)(g.kw * g.kh) : (float)area;
@@ -749,6 +750,11 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
     g.pad_left = d.pad_left;
     g.type = d.pooling_type;
     g.count_include_pad = d.avgpool_count_include_pad;
+    const bool own_rect = d.count_x1 > d.count_x0 && d.count_y1 > d.count_y0;
+    g.cx0 = own_rect ? d.count_x0 : 0;
+    g.cx1 = own_rect ? d.count_x1 : d.w;
+    g.cy0 = own_rect ? d.count_y0 : 0;
+    g.cy1 = own_rect ? d.count_y1 : d.h;
     const size_t total = (size_t)d.batch * d.outh * d.outw * (cp / 4);
     hipLaunchKernelGGL(pooling_nhwc_kernel, dim3(ceil_div((long long)total, 256)), dim3(256), 0, as_stream(stream), src_dev, dst_dev, g, total);
     return launch_status("pooling_nhwc_kernel");

@@ -37,7 +37,7 @@ class ConvFusion(C.Structure):
 
 class PoolDesc(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("w", "h", "c", "batch", "pooling_type", "kernel_w", "kernel_h", "stride_w", "stride_h", "pad_top", "pad_left",
-                                       "outw", "outh", "global_pooling", "avgpool_count_include_pad")]
+                                       "outw", "outh", "global_pooling", "avgpool_count_include_pad", "count_x0", "count_x1", "count_y0", "count_y1")]
 
 
 def library_path():
@@ -365,8 +365,9 @@ class Runtime:
         check(lib().ncnnhip_eltwise(ptrs, len(bufs), int(op_type), co, 0 if coeffs is None else len(coeffs), out.ptr, xs[0].size, self.stream))
         return out.to_numpy(self.stream)
 
-    def pooling(self, x, pooling_type, kernel, stride, pad_top_left, out_hw, global_pooling=False, count_include_pad=0):
-        """x [n][c][h][w] fp32; the border is given resolved (head pads and output extent)."""
+    def pooling(self, x, pooling_type, kernel, stride, pad_top_left, out_hw, global_pooling=False, count_include_pad=0, count_rect=(0, 0, 0, 0)):
+        """x [n][c][h][w] fp32; the border is given resolved (head pads and output extent); count_rect = (x0, x1, y0, y1) in image
+        coordinates is the region whose taps make up an average's divisor without count_include_pad (all zero: the image)."""
         x = np.ascontiguousarray(x, np.float32)
         n, c, h, w = x.shape
         src = self.to_channels_last(x)
@@ -376,7 +377,8 @@ class Runtime:
             check(lib().ncnnhip_pooling_nhwc(C.byref(d), src.ptr, out.ptr, self.stream))
             return out.to_numpy(self.stream)
         oh, ow = out_hw
-        d = PoolDesc(w, h, c, n, pooling_type, kernel[0], kernel[1], stride[0], stride[1], pad_top_left[0], pad_top_left[1], ow, oh, 0, int(count_include_pad))
+        d = PoolDesc(w, h, c, n, pooling_type, kernel[0], kernel[1], stride[0], stride[1], pad_top_left[0], pad_top_left[1], ow, oh, 0, int(count_include_pad),
+                     *count_rect)
         out = DeviceBuffer.empty((n, oh * ow, src.shape[2]), np.float32)
         check(lib().ncnnhip_pooling_nhwc(C.byref(d), src.ptr, out.ptr, self.stream))
         return self.from_channels_last(out, n, c, oh, ow)

@@ -234,7 +234,11 @@ int ncnnhip_hipmat_download(const ncnn_hipmat_t m, ncnn_mat_t* out)
 {
     const HipMat* hm = (const HipMat*)m;
     Mat host;
-    int ret = (hm && hm->cmd) ? hm->cmd->download(*hm, host, 0) : -1;
+    // The command the blob came from may be gone (the blob keeps only its buffers alive), and whoever produced the values
+    // may have enqueued them on any stream: wait for the device, then copy on this thread's own command.
+    static thread_local HipCommand download_cmd;
+    int ret = -1;
+    if (hm && !hm->empty() && download_cmd.ensure_ready() == 0 && ncnnhip_device_synchronize() == 0) ret = download_cmd.download(*hm, host, 0);
     *out = (ncnn_mat_t) new Mat(host);
     return ret;
 }

@@ -208,6 +208,27 @@ public:
         outh = (h + pt + pb - kernel_h) / stride_h + 1;
     }
 
+    // The rectangle (image coordinates) whose taps make up the divisor of an average without count_include_pad.  The
+    // reference tests taps against the layer's own pad parameters in the bordered image -- rows [pad_top, hb - pad_bottom -
+    // htailpad), tail pad only in pad_mode 0 (src/layer/pooling.cpp:255-305) -- so in pad_mode 2 / 3 the SAME border counts.
+    void count_rect(int w, int h, int& x0, int& x1, int& y0, int& y1) const
+    {
+        int pt, pl, outw, outh;
+        resolve(w, h, pt, pl, outw, outh);
+        int wb = w + pad_left + pad_right, hb = h + pad_top + pad_bottom; // bordered extent without the tail pad of mode 0
+        if (pad_mode == 2 || pad_mode == 3)
+        {
+            const int wpad = kernel_w + (w - 1) / stride_w * stride_w - w;
+            const int hpad = kernel_h + (h - 1) / stride_h * stride_h - h;
+            wb = w + ((wpad > 0 || hpad > 0) ? wpad : 0);
+            hb = h + ((wpad > 0 || hpad > 0) ? hpad : 0);
+        }
+        x0 = pad_left - pl;
+        x1 = wb - pad_right - pl;
+        y0 = pad_top - pt;
+        y1 = hb - pad_bottom - pt;
+    }
+
     virtual bool hip_quantise_transparent() const
     {
         return support_hip && pooling_type == 0 && !global_pooling;
@@ -270,6 +291,7 @@ public:
         d.stride_w = stride_w;
         d.stride_h = stride_h;
         resolve(bottom.w, bottom.h, d.pad_top, d.pad_left, d.outw, d.outh);
+        count_rect(bottom.w, bottom.h, d.count_x0, d.count_x1, d.count_y0, d.count_y1);
         top.create(d.outw, d.outh, bottom.c, quantised ? (size_t)1u : (size_t)4u, bottom.n, &cmd);
         if (top.empty()) return -100;
         if (quantised)
@@ -318,9 +340,8 @@ public:
         top.create(outw, outh, channels, 4u, opt.blob_allocator);
         if (top.empty()) return -100;
 
-        // average with count_include_pad=0 counts only taps inside the image plus, in modes 2/3,
-        // nothing else; the reference additionally counts the literal pads of modes 0/1 as
-        // outside.  Either way "inside" is the original image rectangle.
+        int cx0, cx1, cy0, cy1;
+        count_rect(w, h, cx0, cx1, cy0, cy1);
         #pragma omp parallel for num_threads(opt.num_threads)
         for (int q = 0; q < channels; q++)
         {
@@ -352,14 +373,14 @@ public:
                         for (int ky = 0; ky < kernel_h; ky++)
                         {
                             const int y = y0 + ky;
-                            if (y < 0) continue;
-                            if (y >= h) break;
+                            if (y < cy0) continue;
+                            if (y >= cy1) break;
                             for (int kx = 0; kx < kernel_w; kx++)
                             {
                                 const int x = x0 + kx;
-                                if (x < 0) continue;
-                                if (x >= w) break;
-                                s += in[y * w + x];
+                                if (x < cx0) continue;
+                                if (x >= cx1) break;
+                                s += (y >= 0 && y < h && x >= 0 && x < w) ? in[y * w + x] : 0.f; // a counted border tap is the border's zero
                                 area++;
                             }
                         }

@@ -13,9 +13,9 @@ static int hip_status(int rc, const char* where)
 
 // ---- HipMat -----------------------------------------------------------------------------------
 
-HipMat::HipMat() : data(0), refcount(0), cmd(0), dims(0), w(0), h(0), c(0), n(0), cp(0), elemsize(0), q8_scale(0.f) {}
+HipMat::HipMat() : data(0), refcount(0), dims(0), w(0), h(0), c(0), n(0), cp(0), elemsize(0), q8_scale(0.f) {}
 
-HipMat::HipMat(const HipMat& m) : data(m.data), refcount(m.refcount), cmd(m.cmd), dims(m.dims), w(m.w), h(m.h), c(m.c), n(m.n), cp(m.cp), elemsize(m.elemsize), q8(m.q8), q8_scale(m.q8_scale)
+HipMat::HipMat(const HipMat& m) : data(m.data), refcount(m.refcount), pool(m.pool), dims(m.dims), w(m.w), h(m.h), c(m.c), n(m.n), cp(m.cp), elemsize(m.elemsize), q8(m.q8), q8_scale(m.q8_scale)
 {
     if (refcount) __sync_fetch_and_add(refcount, 1);
 }
@@ -32,7 +32,7 @@ HipMat& HipMat::operator=(const HipMat& m)
     release();
     data = m.data;
     refcount = m.refcount;
-    cmd = m.cmd;
+    pool = m.pool;
     dims = m.dims;
     w = m.w;
     h = m.h;
@@ -49,12 +49,12 @@ void HipMat::release()
 {
     if (refcount && __sync_fetch_and_add(refcount, -1) == 1)
     {
-        if (cmd && data) cmd->free(data);
+        if (pool && data) pool->give_back(data);
         delete refcount;
     }
     data = 0;
     refcount = 0;
-    cmd = 0;
+    pool.reset();
     dims = w = h = c = n = cp = 0;
     elemsize = 0;
     q8.reset();
@@ -73,7 +73,7 @@ void HipMat::allocate(HipCommand* command)
         return;
     }
     data = p;
-    cmd = command;
+    pool = command->pool;
     refcount = new int(1);
 }
 
@@ -141,12 +141,84 @@ void HipMat::create_like(const HipMat& m, HipCommand* command)
 
 // ---- HipCommand ---------------------------------------------------------------------------------
 
-HipCommand::HipCommand() : stream(0), ready(false), zero_ws(0), zero_ws_bytes(0) {}
+// ---- HipPool ------------------------------------------------------------------------------------
+
+HipPool::HipPool(bool defer) : defer_reuse(defer) {}
+
+HipPool::~HipPool()
+{
+    // the last owner: the command (which synchronised its stream when it went) and every blob are gone
+    for (size_t i = 0; i < slots.size(); i++) ncnnhip_free(slots[i].ptr);
+}
+
+void* HipPool::take(size_t bytes, int state)
+{
+    if (bytes == 0) bytes = 4;
+    std::lock_guard<std::mutex> g(lock);
+    for (int pass = 0; pass < 2; pass++)
+    {
+        // smallest idle buffer that fits without wasting more than half of it
+        int best = -1;
+        bool retired_fits = false;
+        for (size_t i = 0; i < slots.size(); i++)
+        {
+            const bool fits = slots[i].bytes >= bytes && slots[i].bytes <= 2 * bytes + 0x10000;
+            if (slots[i].state == 0 && fits && (best < 0 || slots[i].bytes < slots[(size_t)best].bytes)) best = (int)i;
+            if (slots[i].state == 3 && fits) retired_fits = true;
+        }
+        if (best >= 0)
+        {
+            slots[(size_t)best].state = state;
+            return slots[(size_t)best].ptr;
+        }
+        if (pass == 1 || !retired_fits) break;
+        // a returned buffer would do, but a kernel on some other stream may still read it: wait for the device once,
+        // after which every returned buffer is free to go out again
+        if (ncnnhip_device_synchronize() != 0) break;
+        for (size_t i = 0; i < slots.size(); i++)
+            if (slots[i].state == 3) slots[i].state = 0;
+    }
+    Slot s;
+    s.bytes = (bytes + 0xffff) & ~(size_t)0xffff;
+    s.state = state;
+    s.ptr = 0;
+    if (ncnnhip_malloc(&s.ptr, s.bytes) != 0 || !s.ptr) return 0;
+    slots.push_back(s);
+    return s.ptr;
+}
+
+void HipPool::give_back(void* ptr)
+{
+    std::lock_guard<std::mutex> g(lock);
+    for (size_t i = 0; i < slots.size(); i++)
+        if (slots[i].ptr == ptr)
+        {
+            slots[i].state = defer_reuse ? 3 : 0;
+            return;
+        }
+}
+
+void HipPool::give_back_all_borrowed()
+{
+    std::lock_guard<std::mutex> g(lock);
+    for (size_t i = 0; i < slots.size(); i++)
+        if (slots[i].state == 2) slots[i].state = 0; // scratch is only ever used on the command's own stream
+}
+
+size_t HipPool::pooled_bytes() const
+{
+    std::lock_guard<std::mutex> g(lock);
+    size_t s = 0;
+    for (size_t i = 0; i < slots.size(); i++) s += slots[i].bytes;
+    return s;
+}
+
+HipCommand::HipCommand(bool blobs_cross_streams) : stream(0), ready(false), pool(new HipPool(blobs_cross_streams)), zero_ws(0), zero_ws_bytes(0) {}
 
 HipCommand::~HipCommand()
 {
+    // whatever was enqueued on this stream has finished before the stream goes; the buffers go with the pool's last owner
     if (ready) ncnnhip_stream_synchronize(stream);
-    for (size_t i = 0; i < pool.size(); i++) ncnnhip_free(pool[i].ptr);
     if (zero_ws) ncnnhip_free(zero_ws);
     if (stream) ncnnhip_stream_destroy(stream);
 }
@@ -183,58 +255,29 @@ int HipCommand::ensure_ready()
     return 0;
 }
 
-void* HipCommand::take(size_t bytes, int state)
-{
-    if (bytes == 0) bytes = 4;
-    // smallest idle buffer that fits without wasting more than half of it
-    int best = -1;
-    for (size_t i = 0; i < pool.size(); i++)
-        if (pool[i].state == 0 && pool[i].bytes >= bytes && pool[i].bytes <= 2 * bytes + 0x10000 && (best < 0 || pool[i].bytes < pool[(size_t)best].bytes)) best = (int)i;
-    if (best >= 0)
-    {
-        pool[(size_t)best].state = state;
-        return pool[(size_t)best].ptr;
-    }
-    Slot s;
-    s.bytes = (bytes + 0xffff) & ~(size_t)0xffff;
-    s.state = state;
-    s.ptr = 0;
-    if (ncnnhip_malloc(&s.ptr, s.bytes) != 0 || !s.ptr) return 0;
-    pool.push_back(s);
-    return s.ptr;
-}
-
 void* HipCommand::alloc(size_t bytes)
 {
-    return take(bytes, 1);
+    return pool->take(bytes, 1);
 }
 
 void HipCommand::free(void* ptr)
 {
-    for (size_t i = 0; i < pool.size(); i++)
-        if (pool[i].ptr == ptr)
-        {
-            pool[i].state = 0;
-            return;
-        }
+    pool->give_back(ptr);
 }
 
 void* HipCommand::borrow(size_t bytes)
 {
-    return take(bytes, 2);
+    return pool->take(bytes, 2);
 }
 
 void HipCommand::give_back_all()
 {
-    for (size_t i = 0; i < pool.size(); i++)
-        if (pool[i].state == 2) pool[i].state = 0;
+    pool->give_back_all_borrowed();
 }
 
 size_t HipCommand::pooled_bytes() const
 {
-    size_t s = 0;
-    for (size_t i = 0; i < pool.size(); i++) s += pool[i].bytes;
-    return s;
+    return pool->pooled_bytes();
 }
 
 int HipCommand::synchronize()
@@ -316,6 +359,8 @@ int HipCommand::widen(const HipMat& src, HipMat& dst)
 int HipCommand::download(const HipMat& blob, Mat& dst, Allocator* allocator)
 {
     if (blob.empty()) return -1;
+    int ready_ret = ensure_ready();
+    if (ready_ret != 0) return ready_ret;
     HipMat src = blob;
     if (src.narrow())
     {

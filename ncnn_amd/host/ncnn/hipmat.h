@@ -4,15 +4,19 @@
 // HipMat is a refcounted handle to a blob in HBM:
 //   dims 3: channels-last [n][h*w][cp], cp = 16*ceil(c/16), pad channels zero  (fp32 or int8)
 //   dims 1: dense [n][w]            dims 2: dense [n][h][w]
-// HipCommand owns the stream every kernel of one Extractor runs on and a pool of device buffers.  All work of an
-// Extractor is stream-ordered, so a buffer that goes back to the pool can be handed out again at once: whatever
-// still reads it was enqueued earlier on the same stream.
+// HipCommand owns the stream every kernel of one Extractor runs on and shares a pool of device buffers (HipPool) with the
+// blobs cut from it: the pool lives until the command AND every such blob are gone, so a blob may outlive its command, its
+// Extractor and its Net.  All work of an Extractor is stream-ordered, so a buffer that goes back to the pool can be handed
+// out again at once: whatever still reads it was enqueued earlier on the same stream.  A pool whose blobs are read on
+// OTHER streams (the net's upload command) defers reuse instead: a returned buffer is handed out again only after a
+// device-wide synchronisation.
 #ifndef NCNN_HIPMAT_H
 #define NCNN_HIPMAT_H
 
 #include <stddef.h>
 
 #include <memory>
+#include <mutex>
 #include <vector>
 
 #include "mat.h"
@@ -21,6 +25,32 @@
 namespace ncnn {
 
 class HipCommand;
+
+// Device buffers of one command, shared (std::shared_ptr) with every blob allocated from it; the last owner frees them.
+// Safe to use from several threads.
+class NCNN_EXPORT HipPool
+{
+public:
+    explicit HipPool(bool defer_reuse);
+    ~HipPool();
+    void* take(size_t bytes, int state); // state 1 blob, 2 borrowed scratch; 0 when the device cannot serve the request
+    void give_back(void* ptr);
+    void give_back_all_borrowed();
+    size_t pooled_bytes() const;
+
+private:
+    HipPool(const HipPool&);
+    HipPool& operator=(const HipPool&);
+    struct Slot
+    {
+        void* ptr;
+        size_t bytes;
+        int state; // 0 idle, 1 blob, 2 borrowed scratch, 3 returned but possibly still read on another stream
+    };
+    mutable std::mutex lock;
+    std::vector<Slot> slots;
+    bool defer_reuse;
+};
 
 class NCNN_EXPORT HipMat
 {
@@ -65,7 +95,7 @@ public:
 
     void* data;
     int* refcount; // host side
-    HipCommand* cmd;
+    std::shared_ptr<HipPool> pool; // where data goes back to; keeps the buffers alive after the command is gone
     int dims, w, h, c, n;
     int cp; // channels as padded in memory (dims 3), else 0.  16*ceil(c/16), or 4 for a narrow fp32 image (create_narrow)
     size_t elemsize;
@@ -83,7 +113,8 @@ private:
 class NCNN_EXPORT HipCommand
 {
 public:
-    HipCommand();
+    // blobs_cross_streams: blobs of this command are consumed on other commands' streams (see HipPool)
+    explicit HipCommand(bool blobs_cross_streams = false);
     ~HipCommand();
     int ensure_ready(); // selects the device and creates the stream on first use
     void* stream;
@@ -110,15 +141,9 @@ public:
 private:
     HipCommand(const HipCommand&);
     HipCommand& operator=(const HipCommand&);
-    struct Slot
-    {
-        void* ptr;
-        size_t bytes;
-        int state; // 0 idle, 1 blob, 2 borrowed scratch
-    };
-    void* take(size_t bytes, int state);
+    friend class HipMat;
     bool ready;
-    std::vector<Slot> pool;
+    std::shared_ptr<HipPool> pool;
     void* zero_ws;
     size_t zero_ws_bytes;
 };

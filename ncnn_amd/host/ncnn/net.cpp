@@ -113,6 +113,7 @@ public:
     mutable std::mutex cmd_lock;
     mutable std::vector<std::shared_ptr<HipCommand> > idle_cmds;
     mutable std::shared_ptr<HipCommand> io_cmd; // carries blobs uploaded through Net::upload
+    mutable std::mutex io_lock;                 // one upload at a time on it (a command's stream and scratch serve one caller)
 
     std::shared_ptr<HipCommand> acquire_command() const
     {
@@ -291,6 +292,28 @@ void NetPrivate::build_fusion_plan()
 // Runs layer_index (a sum, or the ReLU after it) as the epilogue of the convolution in its plan, if nothing on the
 // way has been computed yet and the intermediate blobs may be skipped (light mode).  done = false: not applicable,
 // the caller runs the layers one by one.
+// A layer's featmask (param id 31) switches features off for that layer alone, at create_pipeline and at forward time:
+// NetPrivate::forward_layer with get_masked_option, src/net.cpp:100-121,163.  Bit 3 masks the int8 packing / storage /
+// arithmetic switches (not use_int8_inference, which the reference never masks); bit 4 masks the GPU path, which here is
+// use_hip_compute as well: such a layer sees host Mats.
+static Option masked_option(const Option& opt, int featmask)
+{
+    Option o = opt;
+    o.use_fp16_arithmetic = o.use_fp16_arithmetic && !(featmask & (1 << 0));
+    o.use_fp16_packed = o.use_fp16_packed && !(featmask & (1 << 1));
+    o.use_fp16_storage = o.use_fp16_storage && !(featmask & (1 << 1));
+    o.use_bf16_storage = o.use_bf16_storage && !(featmask & (1 << 2));
+    o.use_int8_packed = o.use_int8_packed && !(featmask & (1 << 3));
+    o.use_int8_storage = o.use_int8_storage && !(featmask & (1 << 3));
+    o.use_int8_arithmetic = o.use_int8_arithmetic && !(featmask & (1 << 3));
+    o.use_vulkan_compute = o.use_vulkan_compute && !(featmask & (1 << 4));
+    o.use_hip_compute = o.use_hip_compute && !(featmask & (1 << 4));
+    o.use_sgemm_convolution = o.use_sgemm_convolution && !(featmask & (1 << 5));
+    o.use_winograd_convolution = o.use_winograd_convolution && !(featmask & (1 << 6));
+    if (featmask & (1 << 7)) o.num_threads = 1;
+    return o;
+}
+
 int NetPrivate::try_fused_tail(int layer_index, ExecState& st, const Option& opt, bool& done) const
 {
     done = false;
@@ -301,6 +324,7 @@ int NetPrivate::try_fused_tail(int layer_index, ExecState& st, const Option& opt
     const Layer* sum = layers[(size_t)tp.eltwise];
     const Layer* last = layers[(size_t)layer_index];
     if (st.has(conv->tops[0]) || st.has(sum->tops[0])) return 0; // an intermediate exists already (fed or extracted)
+    if (conv->featmask || sum->featmask || last->featmask) return 0; // a masked layer runs on its own, under its own options
 
     const int needed[2] = {conv->bottoms[0], tp.residual};
     for (int k = 0; k < 2; k++)
@@ -376,6 +400,12 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
                 return -1;
             }
         }
+    }
+    if (layer->featmask)
+    {
+        const Option lopt = masked_option(opt, layer->featmask);
+        if (lopt.use_hip_compute && layer->support_hip) return run_layer_hip(layer, st, lopt);
+        return run_layer(layer, st, lopt);
     }
     if (opt.use_hip_compute && layer->support_hip) return run_layer_hip(layer, st, opt);
     return run_layer(layer, st, opt);
@@ -484,6 +514,8 @@ int NetPrivate::run_layer(const Layer* layer, ExecState& st, const Option& opt) 
         const size_t bi = (size_t)layer->bottoms[i];
         if (blob_mats[bi].dims == 0 && !st.dev[bi].empty())
         {
+            // (a blob fed with Extractor::input(name, HipMat) may be the first thing this Extractor does on the device)
+            if (!st.cmd) st.cmd = acquire_command();
             int ret = st.cmd->download(st.dev[bi], blob_mats[bi], opt.blob_allocator);
             if (ret != 0) return ret;
         }
@@ -892,10 +924,7 @@ int Net::load_model(const DataReader& dr)
             status = -1;
             break;
         }
-        Option layer_opt = opt;
-        if (layer->featmask & (1 << 3)) layer_opt.use_int8_inference = false;
-        if (layer->featmask & (1 << 7)) layer_opt.num_threads = 1;
-        ret = layer->create_pipeline(layer_opt);
+        ret = layer->create_pipeline(layer->featmask ? masked_option(opt, layer->featmask) : opt);
         if (ret != 0)
         {
             NCNN_LOGE("layer create_pipeline %d %s failed", (int)i, layer->name.c_str());
@@ -967,8 +996,9 @@ int Net::upload(const Mat& src, HipMat& dst) const
 {
     {
         std::lock_guard<std::mutex> g(d->cmd_lock);
-        if (!d->io_cmd) d->io_cmd.reset(new HipCommand);
+        if (!d->io_cmd) d->io_cmd.reset(new HipCommand(true)); // its blobs are read on the Extractors' streams
     }
+    std::lock_guard<std::mutex> g(d->io_lock);
     return d->io_cmd->upload(src, dst);
 }
 
@@ -1170,7 +1200,10 @@ int Extractor::extract(int blob_index, Mat& feat, int type)
         d->st.wanted = -1;
     }
     if (ret == 0 && d->st.host[bi].dims == 0 && !d->st.dev[bi].empty())
+    {
+        if (!d->st.cmd) d->st.cmd = d->net->d->acquire_command(); // the blob was fed as a HipMat and nothing ran yet
         ret = d->st.cmd->download(d->st.dev[bi], d->st.host[bi], d->opt.blob_allocator); // waits for the stream
+    }
     feat = d->st.host[bi];
     if (ret == 0 && type == 0 && feat.elemsize == 1u && !feat.empty())
     {

@@ -18,7 +18,21 @@
 #include <stdlib.h>
 #include <string.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #define ORACLE_API __attribute__((visibility("default")))
+
+/* OpenMP width of the calls that follow (the benchmark reports one thread and all threads) */
+ORACLE_API void cpu_vnni_set_num_threads(int n)
+{
+#ifdef _OPENMP
+    omp_set_num_threads(n > 0 ? n : 1);
+#else
+    (void)n;
+#endif
+}
 
 ORACLE_API int cpu_vnni_available(void)
 {

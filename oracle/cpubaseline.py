@@ -26,6 +26,8 @@ def lib():
         build()
         _lib = C.CDLL(_LIB_PATH)
         _lib.cpu_vnni_available.restype = C.c_int
+        _lib.cpu_vnni_set_num_threads.restype = None
+        _lib.cpu_vnni_set_num_threads.argtypes = [C.c_int]
         _lib.cpu_vnni_packed_bytes.restype = C.c_size_t
         _lib.cpu_vnni_packed_bytes.argtypes = [C.c_int, C.c_int]
         _lib.cpu_vnni_pack_b.restype = None
@@ -38,6 +40,10 @@ def lib():
 
 def available():
     return bool(lib().cpu_vnni_available())
+
+
+def set_num_threads(n):
+    lib().cpu_vnni_set_num_threads(int(n))
 
 
 def pack_b(bq):

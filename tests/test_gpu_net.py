@@ -125,6 +125,162 @@ def test_narrow_input_image_reaches_layers_that_need_the_ordinary_layout():
     assert np.array_equal(ex.extract("g"), (np.cumsum(flat, axis=2, dtype=F)[..., -1] / F(120)).astype(F))
 
 
+def _avgpool_reference(x, k, s, pads, pad_mode, include_pad):
+    """Pooling::forward for average pooling as the reference computes it (src/layer/pooling.cpp:150-330 with make_padding,
+    :347-414): build the bordered image, then per window skip taps by the LAYER'S pad parameters (tail pad only in pad_mode
+    0), so a SAME border (pad_mode 2 / 3, pad parameters 0) is summed as zeros and counted."""
+    c, h, w = x.shape
+    pl, pr, pt, pb = pads
+    wtailpad = htailpad = 0
+    if pad_mode == 0:
+        wtail, htail = (w + pl + pr - k[0]) % s[0], (h + pt + pb - k[1]) % s[1]
+        wtailpad = s[0] - wtail if wtail else 0
+        htailpad = s[1] - htail if htail else 0
+        border = (pt, pb + htailpad, pl, pr + wtailpad)
+    elif pad_mode == 1:
+        border = (pt, pb, pl, pr)
+    else:
+        wpad = k[0] + (w - 1) // s[0] * s[0] - w
+        hpad = k[1] + (h - 1) // s[1] * s[1] - h
+        border = (0, 0, 0, 0)
+        if wpad > 0 or hpad > 0:
+            border = (hpad // 2, hpad - hpad // 2, wpad // 2, wpad - wpad // 2) if pad_mode == 2 else (hpad - hpad // 2, hpad // 2, wpad - wpad // 2, wpad // 2)
+    xb = np.zeros((c, h + border[0] + border[1], w + border[2] + border[3]), F)
+    xb[:, border[0]:border[0] + h, border[2]:border[2] + w] = x
+    hb, wb = xb.shape[1:]
+    oh, ow = (hb - k[1]) // s[1] + 1, (wb - k[0]) // s[0] + 1
+    out = np.zeros((c, oh, ow), F)
+    for q in range(c):
+        for i in range(oh):
+            for j in range(ow):
+                acc, area = F(0), 0
+                for ki in range(k[1]):
+                    sy = i * s[1] + ki
+                    if not include_pad and (sy < pt or sy >= hb - pb - htailpad):
+                        continue
+                    for kj in range(k[0]):
+                        sx = j * s[0] + kj
+                        if not include_pad and (sx < pl or sx >= wb - pr - wtailpad):
+                            continue
+                        acc = F(acc + xb[q, sy, sx])
+                        area += 1
+                out[q, i, j] = F(acc / F(k[0] * k[1] if include_pad else area))
+    return out
+
+
+@RESIDENT
+@pytest.mark.parametrize("w,h,k,s,pads,pad_mode,include_pad", [
+    (5, 5, (3, 3), (2, 2), (0, 0, 0, 0), 2, 0),      # SAME_UPPER: the border's zeros count (area 3 per row at the edge, not 2)
+    (5, 7, (3, 3), (2, 2), (0, 0, 0, 0), 3, 0),      # SAME_LOWER
+    (8, 6, (3, 2), (2, 1), (0, 0, 0, 0), 2, 0),
+    (6, 6, (3, 3), (2, 2), (1, 0, 1, 0), 2, 0),      # SAME with non-zero pad parameters: they exclude taps of the SAME border
+    (7, 6, (3, 3), (2, 2), (1, 1, 1, 1), 0, 0),      # full padding with a tail pad: neither pads nor tail count
+    (7, 6, (3, 3), (2, 2), (1, 1, 1, 1), 1, 0),
+    (7, 6, (3, 3), (2, 2), (1, 1, 1, 1), 0, 1),
+    (5, 5, (3, 3), (2, 2), (0, 0, 0, 0), 2, 1),
+])
+def test_average_pooling_divisor_follows_the_reference_in_every_pad_mode(resident, w, h, k, s, pads, pad_mode, include_pad):
+    c = 5
+    x = np.random.default_rng(w * 10 + h + pad_mode).normal(0, 1, (c, h, w)).astype(F)
+    lines = ["Input in0 0 1 data 0=%d 1=%d 2=%d" % (w, h, c),
+             "Pooling pool 1 1 data out 0=1 1=%d 11=%d 2=%d 12=%d 3=%d 14=%d 13=%d 15=%d 5=%d 6=%d"
+             % (k[0], k[1], s[0], s[1], pads[0], pads[1], pads[2], pads[3], pad_mode, include_pad)]
+    got = _single(lines, b"", {"data": x}, "out", resident)
+    want = _avgpool_reference(x, k, s, pads, pad_mode, include_pad)
+    assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def test_resident_input_into_a_net_that_runs_on_host_blobs():
+    """A blob fed as a HipMat when nothing of the Extractor has touched the device yet: a net with use_hip_compute off
+    downloads it for its first layer, and extracting the fed blob itself gives back what went in."""
+    g, param, blob, info = zoo.build("tiny")
+    x = np.random.default_rng(3).uniform(0, 1, g.input_shape).astype(F)
+    ref = refnet.run(param, blob, x)
+    net = _load(param, blob, False)
+    xin = net.upload(x)
+    ex = net.create_extractor()
+    assert ex.input_resident("data", xin) == 0
+    assert np.array_equal(ex.extract("data"), x)
+    ex = net.create_extractor()
+    assert ex.input_resident("data", xin) == 0
+    assert np.array_equal(ex.extract("fc"), ref["fc"])
+
+
+def test_resident_blob_outlives_its_extractor_and_its_net():
+    """A HipMat shares the buffer pool it was cut from: it stays valid after the Extractor, the command and the Net that
+    produced it are gone."""
+    import gc
+    g, param, blob, info = zoo.build("tiny", seed=2)
+    x = np.random.default_rng(4).uniform(0, 1, g.input_shape).astype(F)
+    ref = refnet.run(param, blob, x)
+    net = _load(param, blob, True)
+    ex = net.create_extractor()
+    ex.input("data", x)
+    out = ex.extract_resident("fc")
+    ex.synchronize()
+    out.net = None
+    del ex, net
+    gc.collect()
+    assert np.array_equal(out.to_numpy().reshape(-1), ref["fc"].reshape(-1))
+
+
+def test_uploads_from_several_threads_and_reassigned_inputs():
+    """Net::upload from four threads at once, each reassigning its input blob in a loop and extracting resident results
+    without waiting in between: a buffer that returns to the upload pool is not refilled while a pass still reads it."""
+    import threading
+    g, param, blob, info = zoo.build("tiny", seed=7)
+    net = _load(param, blob, True)
+    rng = np.random.default_rng(8)
+    xs = [rng.uniform(0, 1, g.input_shape).astype(F) for _ in range(6)]
+    want = [refnet.run(param, blob, x)["fc"].reshape(-1) for x in xs]
+    errors = []
+
+    def worker(t):
+        try:
+            outs = []
+            for i in range(12):
+                xin = net.upload(xs[(t + i) % 6])  # the previous blob of this name goes back to the pool here
+                ex = net.create_extractor()
+                ex.input_resident("data", xin)
+                outs.append(((t + i) % 6, ex, ex.extract_resident("fc")))
+            for j, ex, o in outs:
+                ex.synchronize()
+                if not np.array_equal(o.to_numpy().reshape(-1), want[j]):
+                    errors.append("thread %d: wrong result for input %d" % (t, j))
+                    return
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (t, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
+@RESIDENT
+def test_featmask_switches_a_single_layer_to_host_blobs_and_one_thread(resident):
+    """Param id 31 (featmask) applies at create_pipeline AND at forward time (src/net.cpp:100-121,163): bit 4 takes the
+    layer off the device-resident path, bit 7 gives it one thread, bit 3 leaves use_int8_inference alone.  Results do not
+    change."""
+    g, param, blob, info = zoo.build("tiny", seed=9)
+    x = np.random.default_rng(9).uniform(0, 1, g.input_shape).astype(F)
+    ref = refnet.run(param, blob, x)
+    lines = param.split("\n")
+    masked, n = [], 0
+    for ln in lines:
+        if ln.startswith("Convolution ") and n < 2:
+            ln = ln + " 31=%d" % (16 + 128 + 8 if n == 0 else 8)
+            n += 1
+        masked.append(ln)
+    assert n == 2
+    net = _load("\n".join(masked), blob, resident)
+    ex = net.create_extractor()
+    ex.input("data", x)
+    assert np.array_equal(ex.extract("fc"), ref["fc"])
+
+
 def test_int8_inference_switched_off_is_an_error_not_a_fallback():
     g, param, blob, info = zoo.build("tiny")
     net = _load(param, blob)
