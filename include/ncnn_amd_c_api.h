@@ -16,7 +16,18 @@ extern "C" {
 
 #pragma GCC visibility push(default)
 
-typedef struct __ncnn_allocator_t* ncnn_allocator_t; /* always NULL here: the library's own host allocator */
+/* allocator api, src/c_api.h:21-34: a host allocator as a table of function pointers (the C++ object calls through the table,
+ * so an entry may be replaced); NULL wherever an allocator is asked for means the library's own */
+typedef struct __ncnn_allocator_t* ncnn_allocator_t;
+struct __ncnn_allocator_t
+{
+    void* pthis;
+    void* (*fast_malloc)(ncnn_allocator_t allocator, size_t size);
+    void (*fast_free)(ncnn_allocator_t allocator, void* ptr);
+};
+ncnn_allocator_t ncnn_allocator_create_pool_allocator(void);
+ncnn_allocator_t ncnn_allocator_create_unlocked_pool_allocator(void);
+void ncnn_allocator_destroy(ncnn_allocator_t allocator);
 typedef struct __ncnn_option_t* ncnn_option_t;
 typedef struct __ncnn_mat_t* ncnn_mat_t;
 typedef struct __ncnn_net_t* ncnn_net_t;
@@ -26,6 +37,8 @@ typedef struct __ncnn_extractor_t* ncnn_extractor_t;
 ncnn_option_t ncnn_option_create(void);
 void ncnn_option_destroy(ncnn_option_t opt);
 void ncnn_option_set_num_threads(ncnn_option_t opt, int num_threads);
+void ncnn_option_set_blob_allocator(ncnn_option_t opt, ncnn_allocator_t allocator);      /* src/c_api.h:64 */
+void ncnn_option_set_workspace_allocator(ncnn_option_t opt, ncnn_allocator_t allocator); /* src/c_api.h:65 */
 void ncnn_option_set_lightmode(ncnn_option_t opt, int enable); /* Option::lightmode */
 void ncnn_option_set_use_int8_inference(ncnn_option_t opt, int enable); /* Option::use_int8_inference */
 int ncnn_option_get_use_int8_inference(const ncnn_option_t opt);
@@ -39,8 +52,9 @@ int ncnn_option_get_use_hip_compute(const ncnn_option_t opt);
 ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
 ncnn_mat_t ncnn_mat_create_external_2d_elem(int w, int h, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
 ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
-/* owning, batched 3-D blob (Mat::create(w,h,c,elemsize,elempack,n)); fill it through ncnn_mat_get_batch_data */
-ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, size_t elemsize, int n);
+/* owning, batched 3-D blobs (src/c_api.h:117,131: fp32, or any element size); fill them through ncnn_mat_get_batch_data */
+ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_3d_elem_batch(int w, int h, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator);
 void ncnn_mat_destroy(ncnn_mat_t mat);
 int ncnn_mat_get_dims(const ncnn_mat_t mat);
 int ncnn_mat_get_w(const ncnn_mat_t mat);
@@ -75,6 +89,91 @@ void ncnn_extractor_destroy(ncnn_extractor_t ex);
 void ncnn_extractor_set_option(ncnn_extractor_t ex, const ncnn_option_t opt);
 int ncnn_extractor_input(ncnn_extractor_t ex, const char* name, const ncnn_mat_t mat);
 int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* mat);
+
+/* paramdict api, src/c_api.h:200-213: what a layer written in C reads its parameters from */
+typedef struct __ncnn_paramdict_t* ncnn_paramdict_t;
+ncnn_paramdict_t ncnn_paramdict_create(void);
+void ncnn_paramdict_destroy(ncnn_paramdict_t pd);
+int ncnn_paramdict_get_type(const ncnn_paramdict_t pd, int id);
+int ncnn_paramdict_get_int(const ncnn_paramdict_t pd, int id, int def);
+float ncnn_paramdict_get_float(const ncnn_paramdict_t pd, int id, float def);
+ncnn_mat_t ncnn_paramdict_get_array(const ncnn_paramdict_t pd, int id, const ncnn_mat_t def); /* caller destroys the result */
+void ncnn_paramdict_set_int(ncnn_paramdict_t pd, int id, int i);
+void ncnn_paramdict_set_float(ncnn_paramdict_t pd, int id, float f);
+void ncnn_paramdict_set_array(ncnn_paramdict_t pd, int id, const ncnn_mat_t v);
+
+/* modelbin api, src/c_api.h:238-251: what a layer written in C reads its weights from (results are the caller's to destroy) */
+typedef struct __ncnn_modelbin_t* ncnn_modelbin_t;
+struct __ncnn_modelbin_t
+{
+    void* pthis;
+    ncnn_mat_t (*load_1d)(const ncnn_modelbin_t mb, int w, int type);
+    ncnn_mat_t (*load_2d)(const ncnn_modelbin_t mb, int w, int h, int type);
+    ncnn_mat_t (*load_3d)(const ncnn_modelbin_t mb, int w, int h, int c, int type);
+};
+ncnn_modelbin_t ncnn_modelbin_create_from_mat_array(const ncnn_mat_t* weights, int n);
+void ncnn_modelbin_destroy(ncnn_modelbin_t mb);
+
+/* layer api, src/c_api.h:254-320: a layer as a table of function pointers.  ncnn_layer_create gives a layer whose table
+ * holds the base class's behaviour, for a C program to overwrite entry by entry; ncnn_layer_create_by_type / _by_typeindex
+ * wrap one of the library's built-in layers (NULL for a type it has no host implementation of -- the four int8 types among
+ * them); ncnnhip_layer_create_by_type (no counterpart in the reference) wraps the MI355X implementation of "Convolution",
+ * "ConvolutionDepthWise", "InnerProduct", "Gemm" or "MultiHeadAttention", for registration through
+ * ncnn_net_register_custom_layer_by_type below. */
+typedef struct __ncnn_layer_t* ncnn_layer_t;
+struct __ncnn_layer_t
+{
+    void* pthis;
+    int (*load_param)(ncnn_layer_t layer, const ncnn_paramdict_t pd);
+    int (*load_model)(ncnn_layer_t layer, const ncnn_modelbin_t mb);
+    int (*create_pipeline)(ncnn_layer_t layer, const ncnn_option_t opt);
+    int (*destroy_pipeline)(ncnn_layer_t layer, const ncnn_option_t opt);
+    int (*forward_1)(const ncnn_layer_t layer, const ncnn_mat_t bottom_blob, ncnn_mat_t* top_blob, const ncnn_option_t opt);
+    int (*forward_n)(const ncnn_layer_t layer, const ncnn_mat_t* bottom_blobs, int n, ncnn_mat_t* top_blobs, int n2, const ncnn_option_t opt);
+    int (*forward_inplace_1)(const ncnn_layer_t layer, ncnn_mat_t bottom_top_blob, const ncnn_option_t opt);
+    int (*forward_inplace_n)(const ncnn_layer_t layer, ncnn_mat_t* bottom_top_blobs, int n, const ncnn_option_t opt);
+};
+ncnn_layer_t ncnn_layer_create(void);
+ncnn_layer_t ncnn_layer_create_by_typeindex(int typeindex);
+ncnn_layer_t ncnn_layer_create_by_type(const char* type);
+int ncnn_layer_type_to_index(const char* type);
+ncnn_layer_t ncnnhip_layer_create_by_type(const char* type);
+void ncnn_layer_destroy(ncnn_layer_t layer);
+const char* ncnn_layer_get_name(const ncnn_layer_t layer);
+int ncnn_layer_get_typeindex(const ncnn_layer_t layer);
+const char* ncnn_layer_get_type(const ncnn_layer_t layer);
+int ncnn_layer_get_one_blob_only(const ncnn_layer_t layer);
+int ncnn_layer_get_support_inplace(const ncnn_layer_t layer);
+int ncnn_layer_get_support_vulkan(const ncnn_layer_t layer);
+int ncnn_layer_get_support_packing(const ncnn_layer_t layer);
+int ncnn_layer_get_support_bf16_storage(const ncnn_layer_t layer);
+int ncnn_layer_get_support_fp16_storage(const ncnn_layer_t layer);
+int ncnn_layer_get_support_vulkan_packing(const ncnn_layer_t layer);
+int ncnn_layer_get_support_any_packing(const ncnn_layer_t layer);
+int ncnn_layer_get_support_vulkan_any_packing(const ncnn_layer_t layer);
+void ncnn_layer_set_one_blob_only(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_inplace(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_vulkan(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_packing(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_bf16_storage(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_fp16_storage(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_vulkan_packing(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_any_packing(ncnn_layer_t layer, int enable);
+void ncnn_layer_set_support_vulkan_any_packing(ncnn_layer_t layer, int enable);
+int ncnn_layer_get_bottom_count(const ncnn_layer_t layer);
+int ncnn_layer_get_bottom(const ncnn_layer_t layer, int i);
+int ncnn_layer_get_top_count(const ncnn_layer_t layer);
+int ncnn_layer_get_top(const ncnn_layer_t layer, int i);
+void ncnn_blob_get_bottom_shape(const ncnn_layer_t layer, int i, int* dims, int* w, int* h, int* c);
+void ncnn_blob_get_top_shape(const ncnn_layer_t layer, int i, int* dims, int* w, int* h, int* c);
+
+/* layer factory functions and their registration on a net, src/c_api.h:322-352.  Registering under a built-in type name
+ * replaces the built-in layer (src/net.cpp:1214-1237).  Call before ncnn_net_load_param; the factories live until
+ * ncnn_net_destroy. */
+typedef ncnn_layer_t (*ncnn_layer_creator_t)(void* userdata);
+typedef void (*ncnn_layer_destroyer_t)(ncnn_layer_t layer, void* userdata);
+void ncnn_net_register_custom_layer_by_type(ncnn_net_t net, const char* type, ncnn_layer_creator_t creator, ncnn_layer_destroyer_t destroyer, void* userdata);
+void ncnn_net_register_custom_layer_by_typeindex(ncnn_net_t net, int typeindex, ncnn_layer_creator_t creator, ncnn_layer_destroyer_t destroyer, void* userdata);
 
 /*
  * Installs the MI355X implementations of Convolution, ConvolutionDepthWise, InnerProduct and

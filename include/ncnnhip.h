@@ -50,6 +50,10 @@ int ncnnhip_stream_end_capture(void* stream, void** graph_exec);
 int ncnnhip_graph_launch(void* graph_exec, void* stream);
 int ncnnhip_graph_destroy(void* graph_exec);
 int ncnnhip_malloc(void** dev, size_t bytes);
+/* Fault injection for out-of-memory tests (the reference forces the condition with an allocator that returns NULL,
+ * tests/testutil.cpp:2111-2156): the next `calls` ncnnhip_malloc calls succeed, every one after them returns -100 until the
+ * limit is lifted with a negative value.  No counterpart in the reference; not for production use. */
+int ncnnhip_debug_fail_malloc_after(int calls);
 int ncnnhip_free(void* dev);
 int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream);
 int ncnnhip_memcpy_d2h(void* host, const void* dev, size_t bytes, void* stream);

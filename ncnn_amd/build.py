@@ -48,8 +48,9 @@ def build_kernels(jobs=8):
 
 HOST_SOURCES = ["ncnn/allocator.cpp", "ncnn/mat.cpp", "ncnn/option.cpp", "ncnn/datareader.cpp", "ncnn/paramdict.cpp", "ncnn/modelbin.cpp", "ncnn/hipmat.cpp",
                 "ncnn/layer.cpp", "ncnn/net.cpp", "layers/glue_layers.cpp", "layers/hip_support.cpp", "layers/convolution_hip.cpp",
-                "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "layers/multiheadattention_hip.cpp", "c_api.cpp"]
+                "layers/innerproduct_hip.cpp", "layers/gemm_hip.cpp", "layers/multiheadattention_hip.cpp", "c_api.cpp", "c_api_layer.cpp"]
 LIBNCNN_AMD = os.path.join(LIBDIR, "libncnn_amd.so")
+LIBNCNN_AMD_ASAN = os.path.join(LIBDIR, "libncnn_amd_asan.so")
 
 # strict IEEE on the host too: the load-time weight quantiser and the scale folding must round
 # exactly like the reference's scalar code
@@ -57,14 +58,20 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fopenmp", "-fno-fast-math", "-ffp-
               "-Wno-unused-parameter"]
 
 
-def build_host():
+def build_host(sanitize=False):
     """libncnn_amd.so: the ncnn-API mirror (Mat, ParamDict, ModelBin, Net, Extractor), the four HIP layers and the C API.
-    It links against libncnnhip.so, which carries the kernels."""
+    It links against libncnnhip.so, which carries the kernels.
+    sanitize=True builds libncnn_amd_asan.so beside it with AddressSanitizer and UBSan on the host code (there is no GPU
+    code in this library).  Run the CPU tests on it with
+      LD_PRELOAD=$(gcc -print-file-name=libasan.so) ASAN_OPTIONS=detect_leaks=0 NCNN_AMD_HOST_LIB=<that file> python -m pytest tests -m "not gpu"
+    """
     hostdir = os.path.join(PKG, "host")
     srcs = [os.path.join(hostdir, s) for s in HOST_SOURCES]
-    _run(["g++"] + HOST_FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", hostdir, "-shared", "-o", LIBNCNN_AMD] + srcs
+    out = LIBNCNN_AMD_ASAN if sanitize else LIBNCNN_AMD
+    flags = HOST_FLAGS + (["-g", "-fsanitize=address,undefined", "-fno-omit-frame-pointer"] if sanitize else [])
+    _run(["g++"] + flags + ["-I", os.path.join(ROOT, "include"), "-I", hostdir, "-shared", "-o", out] + srcs
          + ["-L", LIBDIR, "-lncnnhip", "-Wl,-rpath,$ORIGIN"])
-    return LIBNCNN_AMD
+    return out
 
 
 def build_all():
@@ -73,6 +80,9 @@ def build_all():
 
 
 if __name__ == "__main__":
+    if "--asan-host" in sys.argv:
+        print("built", build_host(sanitize=True))
+        sys.exit(0)
     build_all()
     print("built", LIBNCNNHIP)
     sys.exit(0)

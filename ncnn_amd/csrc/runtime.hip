@@ -1,5 +1,7 @@
 // Device plumbing behind the C ABI: buffers, streams, events, error text.
 #include <stdarg.h>
+
+#include <atomic>
 #include <string.h>
 
 #include "common.h"
@@ -142,11 +144,30 @@ int ncnnhip_device_synchronize(void)
     return NCNNHIP_OK;
 }
 
+// fault injection for out-of-memory tests: the number of ncnnhip_malloc calls that still succeed, negative = no limit
+static std::atomic<long> g_mallocs_left(-1);
+
+int ncnnhip_debug_fail_malloc_after(int calls)
+{
+    g_mallocs_left.store(calls < 0 ? -1 : calls);
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_malloc(void** dev, size_t bytes)
 {
     NCNNHIP_REQUIRE(dev, "null out pointer");
     *dev = 0;
     if (bytes == 0) bytes = 4;
+    if (g_mallocs_left.load() >= 0)
+    {
+        // (tests only) the injected limit is spent: report what hipMalloc reports when the device is full
+        if (g_mallocs_left.fetch_sub(1) <= 0)
+        {
+            g_mallocs_left.store(0);
+            set_error("ncnnhip_malloc: out of memory (injected by ncnnhip_debug_fail_malloc_after)");
+            return NCNNHIP_OOM;
+        }
+    }
     NCNNHIP_CHECK(hipMalloc(dev, bytes));
     return NCNNHIP_OK;
 }

@@ -10,8 +10,50 @@ import tempfile
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_PKG, "lib", "libncnn_amd.so")
+# NCNN_AMD_HOST_LIB: another build of the same library (the sanitizer build of build.py --asan-host)
+_LIB = os.environ.get("NCNN_AMD_HOST_LIB") or os.path.join(_PKG, "lib", "libncnn_amd.so")
 _lib = None
+
+
+# ---- struct __ncnn_layer_t / __ncnn_modelbin_t of include/ncnn_amd_c_api.h: tables of function pointers -----------------------
+class LayerTable(C.Structure):
+    pass
+
+
+class ModelBinTable(C.Structure):
+    pass
+
+
+class AllocatorTable(C.Structure):
+    pass
+
+
+AllocatorTable._fields_ = [("pthis", C.c_void_p), ("fast_malloc", C.CFUNCTYPE(C.c_void_p, C.POINTER(AllocatorTable), C.c_size_t)),
+                           ("fast_free", C.CFUNCTYPE(None, C.POINTER(AllocatorTable), C.c_void_p))]
+
+
+_LT, _MT = C.POINTER(LayerTable), C.POINTER(ModelBinTable)
+LayerTable._fields_ = [
+    ("pthis", C.c_void_p),
+    ("load_param", C.CFUNCTYPE(C.c_int, _LT, C.c_void_p)),
+    ("load_model", C.CFUNCTYPE(C.c_int, _LT, _MT)),
+    ("create_pipeline", C.CFUNCTYPE(C.c_int, _LT, C.c_void_p)),
+    ("destroy_pipeline", C.CFUNCTYPE(C.c_int, _LT, C.c_void_p)),
+    ("forward_1", C.CFUNCTYPE(C.c_int, _LT, C.c_void_p, C.POINTER(C.c_void_p), C.c_void_p)),
+    ("forward_n", C.CFUNCTYPE(C.c_int, _LT, C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_void_p), C.c_int, C.c_void_p)),
+    ("forward_inplace_1", C.CFUNCTYPE(C.c_int, _LT, C.c_void_p, C.c_void_p)),
+    ("forward_inplace_n", C.CFUNCTYPE(C.c_int, _LT, C.POINTER(C.c_void_p), C.c_int, C.c_void_p)),
+]
+ModelBinTable._fields_ = [
+    ("pthis", C.c_void_p),
+    ("load_1d", C.CFUNCTYPE(C.c_void_p, _MT, C.c_int, C.c_int)),
+    ("load_2d", C.CFUNCTYPE(C.c_void_p, _MT, C.c_int, C.c_int, C.c_int)),
+    ("load_3d", C.CFUNCTYPE(C.c_void_p, _MT, C.c_int, C.c_int, C.c_int, C.c_int)),
+]
+LAYER_CREATOR = C.CFUNCTYPE(C.c_void_p, C.c_void_p)  # (a ctypes callback cannot return a structure pointer: the address)
+LAYER_DESTROYER = C.CFUNCTYPE(None, _LT, C.c_void_p)
+LAYER_FLAGS = ("one_blob_only", "support_inplace", "support_vulkan", "support_packing", "support_bf16_storage", "support_fp16_storage",
+               "support_vulkan_packing", "support_any_packing", "support_vulkan_any_packing")
 
 
 def lib():
@@ -24,12 +66,16 @@ def lib():
         L = C.CDLL(_LIB)
         vp, ci, cs = C.c_void_p, C.c_int, C.c_size_t
         sig = {
+            "ncnn_allocator_create_pool_allocator": (C.POINTER(AllocatorTable), []), "ncnn_allocator_create_unlocked_pool_allocator": (C.POINTER(AllocatorTable), []),
+            "ncnn_allocator_destroy": (None, [C.POINTER(AllocatorTable)]), "ncnn_option_set_blob_allocator": (None, [vp, C.POINTER(AllocatorTable)]),
+            "ncnn_option_set_workspace_allocator": (None, [vp, C.POINTER(AllocatorTable)]),
             "ncnn_option_create": (vp, []), "ncnn_option_destroy": (None, [vp]), "ncnn_option_set_num_threads": (None, [vp, ci]),
             "ncnn_option_set_lightmode": (None, [vp, ci]), "ncnn_option_set_use_int8_inference": (None, [vp, ci]),
             "ncnn_option_get_use_int8_inference": (ci, [vp]),
             "ncnn_option_set_use_hip_compute": (None, [vp, ci]), "ncnn_option_get_use_hip_compute": (ci, [vp]),
             "ncnn_mat_create_external_1d_elem": (vp, [ci, vp, cs, ci, vp]), "ncnn_mat_create_external_2d_elem": (vp, [ci, ci, vp, cs, ci, vp]),
-            "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, cs, ci]),
+            "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, ci, vp]),
+            "ncnn_mat_create_3d_elem_batch": (vp, [ci, ci, ci, cs, ci, ci, vp]),
             "ncnn_mat_destroy": (None, [vp]), "ncnn_mat_get_dims": (ci, [vp]), "ncnn_mat_get_w": (ci, [vp]), "ncnn_mat_get_h": (ci, [vp]),
             "ncnn_mat_get_d": (ci, [vp]), "ncnn_mat_get_c": (ci, [vp]), "ncnn_mat_get_n": (ci, [vp]), "ncnn_mat_get_elemsize": (cs, [vp]),
             "ncnn_mat_get_elempack": (ci, [vp]), "ncnn_mat_get_cstep": (cs, [vp]), "ncnn_mat_get_nstep": (cs, [vp]),
@@ -51,9 +97,29 @@ def lib():
             "ncnn_net_get_layer_count": (ci, [vp]), "ncnn_net_get_layer_type": (C.c_char_p, [vp, ci]), "ncnn_net_get_layer_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_layer_flags": (ci, [vp, ci]), "ncnn_net_get_blob_count": (ci, [vp]), "ncnn_net_get_blob_name": (C.c_char_p, [vp, ci]),
             "ncnn_net_get_blob_producer": (ci, [vp, ci]), "ncnn_net_get_blob_consumer": (ci, [vp, ci]),
+            # the layer half of the C API: parameter dictionaries, model readers, layers as function-pointer tables
+            "ncnn_paramdict_create": (vp, []), "ncnn_paramdict_destroy": (None, [vp]), "ncnn_paramdict_get_type": (ci, [vp, ci]),
+            "ncnn_paramdict_get_int": (ci, [vp, ci, ci]), "ncnn_paramdict_get_float": (C.c_float, [vp, ci, C.c_float]),
+            "ncnn_paramdict_get_array": (vp, [vp, ci, vp]), "ncnn_paramdict_set_int": (None, [vp, ci, ci]),
+            "ncnn_paramdict_set_float": (None, [vp, ci, C.c_float]), "ncnn_paramdict_set_array": (None, [vp, ci, vp]),
+            "ncnn_modelbin_create_from_mat_array": (C.POINTER(ModelBinTable), [C.POINTER(vp), ci]), "ncnn_modelbin_destroy": (None, [C.POINTER(ModelBinTable)]),
+            "ncnn_layer_create": (C.POINTER(LayerTable), []), "ncnn_layer_create_by_typeindex": (C.POINTER(LayerTable), [ci]),
+            "ncnn_layer_create_by_type": (C.POINTER(LayerTable), [C.c_char_p]), "ncnn_layer_type_to_index": (ci, [C.c_char_p]),
+            "ncnnhip_layer_create_by_type": (C.POINTER(LayerTable), [C.c_char_p]), "ncnn_layer_destroy": (None, [C.POINTER(LayerTable)]),
+            "ncnn_layer_get_name": (C.c_char_p, [C.POINTER(LayerTable)]), "ncnn_layer_get_typeindex": (ci, [C.POINTER(LayerTable)]),
+            "ncnn_layer_get_type": (C.c_char_p, [C.POINTER(LayerTable)]),
+            "ncnn_layer_get_bottom_count": (ci, [C.POINTER(LayerTable)]), "ncnn_layer_get_bottom": (ci, [C.POINTER(LayerTable), ci]),
+            "ncnn_layer_get_top_count": (ci, [C.POINTER(LayerTable)]), "ncnn_layer_get_top": (ci, [C.POINTER(LayerTable), ci]),
+            "ncnn_blob_get_bottom_shape": (None, [C.POINTER(LayerTable), ci] + [C.POINTER(ci)] * 4),
+            "ncnn_blob_get_top_shape": (None, [C.POINTER(LayerTable), ci] + [C.POINTER(ci)] * 4),
+            "ncnn_net_register_custom_layer_by_type": (None, [vp, C.c_char_p, LAYER_CREATOR, LAYER_DESTROYER, vp]),
+            "ncnn_net_register_custom_layer_by_typeindex": (None, [vp, ci, LAYER_CREATOR, LAYER_DESTROYER, vp]),
             "ncnn_paramdict_probe": (ci, [C.c_char_p, ci, C.POINTER(C.c_uint), C.POINTER(C.c_uint), ci]),
             "ncnn_modelbin_probe": (ci, [C.c_char_p, ci, ci, vp, C.POINTER(cs)]),
         }
+        for flag in LAYER_FLAGS:
+            sig["ncnn_layer_get_" + flag] = (ci, [C.POINTER(LayerTable)])
+            sig["ncnn_layer_set_" + flag] = (None, [C.POINTER(LayerTable), ci])
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
             fn.restype = res
@@ -122,7 +188,7 @@ class Mat:
 
     @classmethod
     def batch3d(cls, w, h, c, elemsize, n):
-        return cls(lib().ncnn_mat_create_3d_batch(w, h, c, elemsize, n))
+        return cls(lib().ncnn_mat_create_3d_elem_batch(w, h, c, elemsize, 1, n, None))
 
     @classmethod
     def from_numpy(cls, a):
@@ -252,6 +318,14 @@ class Net:
                 self.h_ = None
         except Exception:
             pass
+
+    def register_custom_layer(self, type_name, creator, destroyer):
+        """ncnn_net_register_custom_layer_by_type with Python callables: creator() -> ncnn_layer_t (a POINTER(LayerTable)),
+        destroyer(layer).  The C thunks are kept alive with the net."""
+        c = LAYER_CREATOR(lambda userdata: C.cast(creator(), C.c_void_p).value)
+        d = LAYER_DESTROYER(lambda layer, userdata: destroyer(layer))
+        self._custom = getattr(self, "_custom", []) + [(c, d)]
+        lib().ncnn_net_register_custom_layer_by_type(self.h_, type_name.encode(), c, d, None)
 
     def register_attention_layer(self):
         return lib().ncnnhip_register_attention_layer(self.h_)

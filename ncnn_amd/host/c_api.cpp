@@ -1,5 +1,6 @@
 #include "ncnn_amd_c_api.h"
 
+#include <stdlib.h>
 #include <string.h>
 
 #include "layers/hip_layers.h"
@@ -10,6 +11,10 @@
 #include "ncnn/paramdict.h"
 
 using namespace ncnn;
+
+namespace ncnn_amd {
+void release_custom_layer_factories(const ncnn::Net* net); // c_api_layer.cpp
+}
 
 static Option* O(ncnn_option_t p)
 {
@@ -28,7 +33,89 @@ static Extractor* E(ncnn_extractor_t p)
     return (Extractor*)p;
 }
 
+// ---- allocators as tables of function pointers (src/c_api.cpp:55-150): the C++ object calls through the table, so a C
+// program may replace an entry (that is how an out-of-memory test makes fastMalloc return NULL)
+static Allocator* A(ncnn_allocator_t a)
+{
+    return a ? (Allocator*)a->pthis : 0;
+}
+class PoolAllocator_c_api : public PoolAllocator
+{
+public:
+    explicit PoolAllocator_c_api(ncnn_allocator_t a) : allocator(a) {}
+    virtual void* fastMalloc(size_t size)
+    {
+        return allocator->fast_malloc(allocator, size);
+    }
+    virtual void fastFree(void* ptr)
+    {
+        allocator->fast_free(allocator, ptr);
+    }
+    ncnn_allocator_t allocator;
+};
+class UnlockedPoolAllocator_c_api : public UnlockedPoolAllocator
+{
+public:
+    explicit UnlockedPoolAllocator_c_api(ncnn_allocator_t a) : allocator(a) {}
+    virtual void* fastMalloc(size_t size)
+    {
+        return allocator->fast_malloc(allocator, size);
+    }
+    virtual void fastFree(void* ptr)
+    {
+        allocator->fast_free(allocator, ptr);
+    }
+    ncnn_allocator_t allocator;
+};
+static void* pool_fast_malloc(ncnn_allocator_t a, size_t size)
+{
+    return ((PoolAllocator*)a->pthis)->PoolAllocator::fastMalloc(size);
+}
+static void pool_fast_free(ncnn_allocator_t a, void* ptr)
+{
+    ((PoolAllocator*)a->pthis)->PoolAllocator::fastFree(ptr);
+}
+static void* unlocked_pool_fast_malloc(ncnn_allocator_t a, size_t size)
+{
+    return ((UnlockedPoolAllocator*)a->pthis)->UnlockedPoolAllocator::fastMalloc(size);
+}
+static void unlocked_pool_fast_free(ncnn_allocator_t a, void* ptr)
+{
+    ((UnlockedPoolAllocator*)a->pthis)->UnlockedPoolAllocator::fastFree(ptr);
+}
+
 extern "C" {
+
+ncnn_allocator_t ncnn_allocator_create_pool_allocator(void)
+{
+    ncnn_allocator_t a = (ncnn_allocator_t)malloc(sizeof(struct __ncnn_allocator_t));
+    a->pthis = (void*)static_cast<Allocator*>(new PoolAllocator_c_api(a));
+    a->fast_malloc = pool_fast_malloc;
+    a->fast_free = pool_fast_free;
+    return a;
+}
+ncnn_allocator_t ncnn_allocator_create_unlocked_pool_allocator(void)
+{
+    ncnn_allocator_t a = (ncnn_allocator_t)malloc(sizeof(struct __ncnn_allocator_t));
+    a->pthis = (void*)static_cast<Allocator*>(new UnlockedPoolAllocator_c_api(a));
+    a->fast_malloc = unlocked_pool_fast_malloc;
+    a->fast_free = unlocked_pool_fast_free;
+    return a;
+}
+void ncnn_allocator_destroy(ncnn_allocator_t allocator)
+{
+    if (!allocator) return;
+    delete (Allocator*)allocator->pthis;
+    free(allocator);
+}
+void ncnn_option_set_blob_allocator(ncnn_option_t opt, ncnn_allocator_t allocator)
+{
+    O(opt)->blob_allocator = A(allocator);
+}
+void ncnn_option_set_workspace_allocator(ncnn_option_t opt, ncnn_allocator_t allocator)
+{
+    O(opt)->workspace_allocator = A(allocator);
+}
 
 ncnn_option_t ncnn_option_create(void)
 {
@@ -81,10 +168,16 @@ ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, siz
     m->elempack = elempack;
     return (ncnn_mat_t)m;
 }
-ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, size_t elemsize, int n)
+ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, int n, ncnn_allocator_t allocator)
 {
     Mat* m = new Mat;
-    m->create(w, h, c, elemsize, 1, n, (Allocator*)0);
+    m->create(w, h, c, (size_t)4u, 1, n, A(allocator));
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_3d_elem_batch(int w, int h, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator)
+{
+    Mat* m = new Mat;
+    m->create(w, h, c, elemsize, elempack, n, A(allocator));
     return (ncnn_mat_t)m;
 }
 void ncnn_mat_destroy(ncnn_mat_t mat)
@@ -147,6 +240,7 @@ ncnn_net_t ncnn_net_create(void)
 void ncnn_net_destroy(ncnn_net_t net)
 {
     delete N(net);
+    ncnn_amd::release_custom_layer_factories(N(net)); // after the layers they made are gone
 }
 ncnn_option_t ncnn_net_get_option(ncnn_net_t net)
 {

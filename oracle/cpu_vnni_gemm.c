@@ -111,7 +111,7 @@ __attribute__((target("avx512f,avx512bw,avx512vnni"))) ORACLE_API int cpu_vnni_g
     int failed = 0;
 #pragma omp parallel
     {
-        uint8_t* au = (uint8_t*)aligned_alloc(64, 4 * k4 * 4 + 64);
+        uint8_t* au = (uint8_t*)aligned_alloc(64, ((size_t)4 * k4 * 4 + 127) & ~(size_t)63);
         int32_t acc[4 * 64];
         float sa[4];
         if (!au)
