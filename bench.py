@@ -375,8 +375,52 @@ def measure_peak_hbm_read(lib, check, rt, nbytes, loads_per_lane=16, launches=20
     return {"gbs": nbytes / us / 1e3, "us_per_launch": us, "bytes": nbytes, "loads_per_lane": loads_per_lane, "copies_rotated": copies}
 
 
+def measure_peak_launch(lib, check, rt, nodes, reps):
+    """us per dependent one-wavefront launch: `nodes` launches enqueued on a stream, and the same captured once into a
+    graph and replayed; events around `reps` repetitions of each, plus the host's time to enqueue them."""
+    import ncnn_amd
+    counter = ncnn_amd.DeviceBuffer.empty((16,), np.int32)
+    counter.fill_bytes(0, rt.stream)
+    ev = _events(lib, check, 2)
+    out = {"nodes": nodes, "reps": reps}
+    for r in range(3):
+        check(lib.ncnnhip_peak_launch_chain(nodes, counter.ptr, rt.stream))
+    rt.sync()
+    t0 = time.perf_counter()
+    check(lib.ncnnhip_event_record(ev[0], rt.stream))
+    for r in range(reps):
+        check(lib.ncnnhip_peak_launch_chain(nodes, counter.ptr, rt.stream))
+    check(lib.ncnnhip_event_record(ev[1], rt.stream))
+    host = time.perf_counter() - t0
+    check(lib.ncnnhip_event_synchronize(ev[1]))
+    out["stream_us_per_launch"] = _elapsed(lib, check, ev[0], ev[1]) * 1e3 / (nodes * reps)
+    out["stream_host_enqueue_us_per_launch"] = host * 1e6 / (nodes * reps)
+    exe = C.c_void_p()
+    check(lib.ncnnhip_stream_begin_capture(rt.stream))
+    check(lib.ncnnhip_peak_launch_chain(nodes, counter.ptr, rt.stream))
+    check(lib.ncnnhip_stream_end_capture(rt.stream, C.byref(exe)))
+    for r in range(3):
+        check(lib.ncnnhip_graph_launch(exe, rt.stream))
+    rt.sync()
+    t0 = time.perf_counter()
+    check(lib.ncnnhip_event_record(ev[0], rt.stream))
+    for r in range(reps):
+        check(lib.ncnnhip_graph_launch(exe, rt.stream))
+    check(lib.ncnnhip_event_record(ev[1], rt.stream))
+    host = time.perf_counter() - t0
+    check(lib.ncnnhip_event_synchronize(ev[1]))
+    out["graph_us_per_node"] = _elapsed(lib, check, ev[0], ev[1]) * 1e3 / (nodes * reps)
+    out["graph_host_enqueue_us_per_node"] = host * 1e6 / (nodes * reps)
+    check(lib.ncnnhip_graph_destroy(exe))
+    total = int(counter.to_numpy(rt.stream)[0])
+    if total != nodes * (2 * reps + 6):
+        raise SystemExit("bench.py: the launch chain counted %d, expected %d" % (total, nodes * (2 * reps + 6)))
+    return out
+
+
 def bench_peak(args, what, arg):
-    """The chip's own ceilings, measured: `peak:mfma_i8[:zeros|random]` and `peak:hbm_read:<bytes>[:<loads per lane>]`."""
+    """The chip's own ceilings, measured: `peak:mfma_i8[:zeros|random]`, `peak:hbm_read:<bytes>[:<loads per lane>]` and
+    `peak:launch[:<nodes>]` (what one dependent kernel launch costs, on a stream and as a node of a replayed graph)."""
     import ncnn_amd
     from ncnn_amd.hip import check, lib as load
     lib = load()
@@ -400,6 +444,13 @@ def bench_peak(args, what, arg):
                                         % (r["bytes"], lpl), "run": r},
                     roofline={"bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": r["gbs"] / HBM_PEAK_GBS, "traffic": None,
                               "kernel": "peak_hbm_read_kernel", "bytes_per_launch": r["bytes"]})
+    if what == "launch":
+        r = measure_peak_launch(lib, check, rt, int(arg) if arg else 57, reps=max(20, args.steps))
+        best = min(r["stream_us_per_launch"], r["graph_us_per_node"])
+        return dict(base, metric="us per dependent launch", value=best, unit="us", ms_per_step=best * r["nodes"] * 1e-3, dtype="none", higher_is_better=False,
+                    config={"workload": "chain of %d one-wavefront kernels, each reading what the one before wrote: stream launches against one replayed graph"
+                                        % r["nodes"], "run": r},
+                    roofline={"bound": "launch", "achieved": best, "peak": None, "unit": "us", "frac": None, "traffic": None, "kernel": "peak_launch_chain_kernel"})
     raise SystemExit("unknown peak workload " + what)
 
 
@@ -463,25 +514,84 @@ def bench_mha(args, embed, heads, src, past):
     }
 
 
-def cpu_baseline_conv(c, h, w, cout, k, pad, budget_s=10.0):
-    """Scalar oracle (ncnn's naive Convolution::forward_int8 restated, OpenMP over output channels) on whole layers."""
-    from oracle import oracle
-    threads = min(oracle.num_threads(), 16)
-    oracle.set_num_threads(threads)
+def _timed(fn, budget_s, min_reps=3, max_reps=100000):
+    fn()  # warm-up: threads, page faults, buffers that later calls write again
+    times, t_start = [], time.perf_counter()
+    while len(times) < min_reps or (time.perf_counter() - t_start < budget_s and len(times) < max_reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return times
+
+
+def cpu_baseline_conv(c, h, w, cout, k, pad, batch=1, budget_s=10.0):
+    """The same layer on this host's cores the way the reference's x86 path computes it (oracle/cpu_vnni_conv.c: quantise,
+    im2col, AVX512-VNNI, vector epilogue; bit-exact against the scalar oracle), on all threads and on one; the scalar
+    OpenMP oracle when the host has no AVX512-VNNI."""
+    from oracle import cpubaseline as cb, oracle
     rng = np.random.default_rng(0)
-    x = rng.uniform(-1, 1, (c, h, w)).astype(np.float32)
     wq = rng.integers(-127, 128, (cout, c, k, k)).astype(np.int8)
     ws = rng.uniform(50, 100, cout).astype(np.float32)
     b = rng.uniform(-0.1, 0.1, cout).astype(np.float32)
-    d = oracle.make_desc((c, h, w), cout, (k, k), (1, 1), (1, 1), (pad,) * 4, 0.0, 1, 1, 1, 1, (0.0, 0.0))
-    reps, t0 = 0, time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t0 < budget_s and reps < 200):
-        oracle.convolution_int8(d, x, wq, b, ws, np.float32(127.0), None)
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
     oh, ow = h + 2 * pad - k + 1, w + 2 * pad - k + 1
-    return {"value": 2.0 * cout * oh * ow * c * k * k / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
-            "sample": "%d whole forward passes of the same layer (quantise + convolution + epilogue), scalar OpenMP oracle, %.2f ms each" % (reps, dt * 1e3)}
+    ops = 2.0 * batch * cout * oh * ow * c * k * k
+    if cb.available():
+        threads = min(os.cpu_count() or 1, 16)
+        x = rng.uniform(-1, 1, (batch, h, w, c)).astype(np.float32)
+        d = cb.ConvDesc(w, h, c, batch, cout, k, k, 1, 1, 1, 1, pad, pad, pad, pad, 0.0)
+        packed, scale_in = cb.pack_conv_weights(wq), cb.fold_scales(ws, np.float32(127.0))  # load-time work, outside the timed region
+        res = {}
+        for label, th in (("all", threads), ("one", 1)):
+            cb.set_num_threads(th)
+            keep = [None]
+
+            def once():
+                keep[0] = cb.conv_nhwc(d, x, 127.0, packed, scale_in, b, None, 1, (0.0, 0.0), out=keep[0])
+            res[label] = _timed(once, budget_s if label == "all" else budget_s / 3)
+        cb.set_num_threads(threads)
+        dt = float(np.mean(res["all"]))
+        return dict({"value": ops / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port", "value_1_thread": ops / min(res["one"]) / 1e12,
+                     "sample": "%d whole forward passes of the same layer, batch %d (quantise + im2col + AVX512-VNNI int8 GEMM + dequantise/bias/ReLU, OpenMP), "
+                               "mean %.3f ms each; one thread: best of %d, %.3f ms" % (len(res["all"]), batch, dt * 1e3, len(res["one"]), min(res["one"]) * 1e3)},
+                    **host_cpu_info())
+    threads = min(oracle.num_threads(), 16)
+    oracle.set_num_threads(threads)
+    x = rng.uniform(-1, 1, (c, h, w)).astype(np.float32)
+    d = oracle.make_desc((c, h, w), cout, (k, k), (1, 1), (1, 1), (pad,) * 4, 0.0, 1, 1, 1, 1, (0.0, 0.0))
+    times = _timed(lambda: oracle.convolution_int8(d, x, wq, b, ws, np.float32(127.0), None), budget_s, max_reps=200)
+    dt = float(np.mean(times))
+    return dict({"value": ops / batch / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+                 "sample": "%d whole forward passes of the same layer at batch 1 (quantise + convolution + epilogue), scalar OpenMP oracle, %.2f ms each"
+                           % (len(times), dt * 1e3)}, **host_cpu_info())
+
+
+def cpu_baseline_net(param, blob, input_shape, batch, ops, budget_s=12.0):
+    """The same model on this host's cores: the whole-model pass of oracle/cpunet.py (VNNI convolution, depthwise and
+    inner-product layers plus the glue loops, bit-exact against the scalar oracle's executor), on a bounded batch, on all
+    threads and on one.  None when the host has no AVX512-VNNI (the scalar executor would take minutes per image)."""
+    from oracle import cpubaseline as cb, cpunet
+    if not cb.available():
+        return None
+    threads = min(os.cpu_count() or 1, 16)
+    nb = min(batch, 4)
+    x = np.random.default_rng(0).uniform(0, 1, (nb,) + tuple(input_shape)).astype(np.float32)
+    model = cpunet.load(param, blob)  # load-time work, outside the timed region
+    res = {}
+    for label, th, xs in (("all", threads, x), ("one", 1, x[:1])):
+        cb.set_num_threads(th)
+        keep = [None]
+
+        def once():
+            keep[0] = cpunet.run(model, xs, keep=keep[0])
+        res[label] = _timed(once, budget_s if label == "all" else budget_s / 2, min_reps=2)
+    cb.set_num_threads(threads)
+    dt = float(np.mean(res["all"]))
+    per_image = ops / batch
+    return dict({"value": per_image * nb / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port", "images_per_s": nb / dt,
+                 "value_1_thread": per_image / min(res["one"]) / 1e12, "images_per_s_1_thread": 1.0 / min(res["one"]),
+                 "sample": "%d whole forward passes of the same model at batch %d (of the workload's %d), every layer on the CPU: mean %.2f ms per pass; "
+                           "one thread, batch 1: best of %d, %.2f ms" % (len(res["all"]), nb, batch, dt * 1e3, len(res["one"]), min(res["one"]) * 1e3)},
+                **host_cpu_info())
 
 
 def bench_conv(args, spec):
@@ -550,8 +660,8 @@ def bench_conv(args, spec):
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": measured_traffic("conv:" + spec), "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
     }
-    if not args.no_cpu and batch == 1:
-        line["cpu_baseline"] = cpu_baseline_conv(c, h, w, cout, k, pad)
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_conv(c, h, w, cout, k, pad, batch)
     return line
 
 
@@ -738,40 +848,67 @@ def bench_net(args, which, batch):
         return ex, ex.extract_resident(out_name)
 
     # --streams N keeps the last N Extractors alive, so N passes are in flight on N of the net's streams (each live
-    # Extractor borrows its own command); 1 = one pass after the other on one stream
-    ring = [None] * max(1, args.streams)
-    ex = None
-    for i in range(args.warmup):
-        ex, out = step()
-        ring[i % len(ring)] = ex
-    for e in ring:
-        if e is not None:
-            e.synchronize()
+    # Extractor borrows its own command); 1 = one pass after the other on one stream.  --threads T: T host threads, each
+    # with such a ring of its own, enqueue their share of the steps side by side (the C calls release the interpreter
+    # lock): one thread cannot describe a batch-1 pass as fast as the GPU runs it.
+    threads = max(1, args.threads) if graph is None else 1
+    rings = [[None] * max(1, args.streams) for _ in range(threads)]
+    outs = [None] * threads
+
+    def run(t, count):
+        ring = rings[t]
+        for i in range(count):
+            ex, out = step()
+            ring[i % len(ring)] = ex
+            outs[t] = out
+
+    def run_all(total):
+        share = [total // threads + (1 if t < total % threads else 0) for t in range(threads)]
+        if threads == 1:
+            run(0, share[0])
+            return
+        import threading
+        ts = [threading.Thread(target=run, args=(t, share[t])) for t in range(threads)]
+        for th in ts:
+            th.start()
+        for th in ts:
+            th.join()
+
+    def drain():
+        for ring in rings:
+            for e in ring:
+                if e is not None:
+                    e.synchronize()
+
+    run_all(max(args.warmup, threads))
+    drain()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        ex, out = step()
-        ring[i % len(ring)] = ex
+    run_all(args.steps)
     enqueue = time.perf_counter() - t0  # the host is done describing the work; the GPU may still be running it
-    for e in ring:
-        if e is not None:
-            e.synchronize()
+    drain()
     wall = time.perf_counter() - t0
+    out = outs[0]
     logits = (graph.output() if graph is not None else out).to_numpy()
     if not np.isfinite(logits).all():
         raise SystemExit("bench.py: non-finite logits")
     ms_per_step = wall * 1e3 / args.steps
     achieved = ops / (ms_per_step * 1e-3) / 1e12
-    return {
+    line = {
         "metric": "int8 TOPS", "value": achieved, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "%s-shaped int8 model (%d layers, %d quantised), whole forward pass through Net/Extractor with device-resident blobs, batch %d"
                                % (which, len(g.layers), len(rows), batch),
                    "images_per_s": batch / (ms_per_step * 1e-3), "host_enqueue_ms_per_step": enqueue * 1e3 / args.steps,
                    "submission": "recorded pass replayed as one graph launch" if graph is not None else "layer by layer through an Extractor",
-                   "passes_in_flight": len(ring)},
+                   "passes_in_flight": threads * len(rings[0]), "host_threads": threads},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": None, "kernel": "whole pass (conv_nhwc_pipelined_kernel dominates)", "ops_per_launch": ops},
     }
+    if not args.no_cpu:
+        cpu = cpu_baseline_net(param, blob, g.input_shape, batch, ops)
+        if cpu is not None:
+            line["cpu_baseline"] = cpu
+    return line
 
 
 def main():
@@ -783,8 +920,9 @@ def main():
                     help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI) | "
-                         "peak:mfma_i8[:zeros|random] | peak:hbm_read:<bytes>[:<loads per lane>] (the chip's measured ceilings)")
+                         "peak:mfma_i8[:zeros|random] | peak:hbm_read:<bytes>[:<loads per lane>] | peak:launch[:<nodes>] (the chip's measured ceilings)")
     ap.add_argument("--streams", type=int, default=1, help="net workloads: forward passes kept in flight, each on its own stream of the net")
+    ap.add_argument("--threads", type=int, default=1, help="net workloads: host threads that enqueue passes side by side, each on streams of its own")
     ap.add_argument("--graph", type=int, default=0,
                     help="net workloads: 0 = one Extractor per pass, layer by layer on a stream (faster on this ROCm: a replayed graph costs more per kernel node "
                          "on the GPU than a stream launch does); 1 = replay the recorded pass (HipGraph), which takes the host out of the loop")

@@ -367,7 +367,11 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
  * wavefront) on all-zero or pseudo-random operands; scratch_dev (>= 64 bytes) receives two int64: the shader cycles and
  * the 100 MHz wall ticks workgroup 0 spent in the loop.  ncnnhip_peak_hbm_read reads `bytes` (a multiple of 16) once with
  * 16-byte non-temporal loads, `loads_per_lane` (4, 8, 16, 32) of them in flight per lane, and writes nothing; time it with
- * events over buffers larger than the last-level cache to get the read bandwidth a kernel of that size can reach. */
+ * events over buffers larger than the last-level cache to get the read bandwidth a kernel of that size can reach.
+ * ncnnhip_peak_launch_chain enqueues `launches` one-wavefront kernels, each adding 1 to the int at scratch_dev (so each
+ * depends on the one before, as the layers of a net do): timed with events, or captured into a graph and replayed, it
+ * gives what one dependent launch costs on this chip whatever the kernel does. */
+int ncnnhip_peak_launch_chain(int launches, void* scratch_dev, void* stream);
 int ncnnhip_peak_mfma_i8(int iters, int random_operands, void* scratch_dev, void* stream);
 int ncnnhip_peak_hbm_read(const void* src_dev, size_t bytes, int loads_per_lane, void* scratch_dev, void* stream);
 

@@ -70,6 +70,12 @@ __global__ __launch_bounds__(256) void peak_hbm_read_kernel(const v4i_pk* __rest
     if (s == 0x12345679) sink[0] = s; // practically never; keeps the loads alive without a store per lane
 }
 
+// one wavefront; each launch reads what the launch before it wrote, as the layers of a net do
+__global__ void __launch_bounds__(64) peak_launch_chain_kernel(int* counter)
+{
+    if (threadIdx.x == 0) counter[0] = counter[0] + 1;
+}
+
 } // namespace ncnnhip
 
 using namespace ncnnhip;
@@ -112,6 +118,13 @@ int ncnnhip_peak_hbm_read(const void* src_dev, size_t bytes, int loads_per_lane,
     }
 #undef LAUNCH_READ
     return launch_status("peak_hbm_read_kernel");
+}
+
+int ncnnhip_peak_launch_chain(int launches, void* scratch_dev, void* stream)
+{
+    NCNNHIP_REQUIRE(launches >= 1 && scratch_dev, "ncnnhip_peak_launch_chain: bad argument");
+    for (int i = 0; i < launches; i++) hipLaunchKernelGGL(peak_launch_chain_kernel, dim3(1), dim3(64), 0, as_stream(stream), static_cast<int*>(scratch_dev));
+    return launch_status("peak_launch_chain_kernel");
 }
 
 } // extern "C"

@@ -132,6 +132,7 @@ _SIGNATURES = {
     "ncnnhip_blockquant_pack": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_blockquant_packed_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                             C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_peak_launch_chain": [C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_mfma_i8": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_hbm_read": [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_blockquant_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,

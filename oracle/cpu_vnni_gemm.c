@@ -37,7 +37,7 @@ ORACLE_API void cpu_vnni_set_num_threads(int n)
 ORACLE_API int cpu_vnni_available(void)
 {
     __builtin_cpu_init();
-    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") && __builtin_cpu_supports("avx512vnni");
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") && __builtin_cpu_supports("avx512vl") && __builtin_cpu_supports("avx512vnni");
 }
 
 /* packed size in bytes for B[N][K]: K rounded up to 4, N rounded up to 64, plus N int32 column sums */
@@ -80,7 +80,7 @@ __attribute__((target("avx512f,avx512bw,avx512vnni"))) static void rows4_block(c
         const __m512i b1 = _mm512_loadu_si512((const void*)(bp + 64));
         const __m512i b2 = _mm512_loadu_si512((const void*)(bp + 128));
         const __m512i b3 = _mm512_loadu_si512((const void*)(bp + 192));
-        for (int r = 0; r < rows; r++)
+        for (int r = 0; r < 4; r++) /* all four rows, whatever `rows` is: constant trip counts keep the accumulators in registers */
         {
             int32_t a4;
             memcpy(&a4, au + (size_t)r * au_stride + kk * 4, 4);
@@ -91,7 +91,8 @@ __attribute__((target("avx512f,avx512bw,avx512vnni"))) static void rows4_block(c
             c[r][3] = _mm512_dpbusd_epi32(c[r][3], av, b3);
         }
     }
-    for (int r = 0; r < rows; r++)
+    (void)rows;
+    for (int r = 0; r < 4; r++)
         for (int v = 0; v < 4; v++) _mm512_storeu_si512((void*)(acc + r * 64 + v * 16), c[r][v]);
 }
 
@@ -119,6 +120,8 @@ __attribute__((target("avx512f,avx512bw,avx512vnni"))) ORACLE_API int cpu_vnni_g
 #pragma omp atomic write
             failed = 1;
         }
+        else
+            memset(au, 128, (size_t)4 * k4 * 4); /* the micro-kernel multiplies all four rows, also when fewer are asked for */
 #pragma omp for schedule(dynamic, 4)
         for (int i0 = 0; i0 < M; i0 += 4)
         {

@@ -108,6 +108,14 @@ def make_desc(x_shape, num_output, kernel, dilation=(1, 1), stride=(1, 1), pads=
     return d
 
 
+def resolve_padding(desc):
+    """Explicit (top, bottom, left, right) borders of a layer description (-233 / -234 resolved as the reference does)."""
+    out = (C.c_int * 4)()
+    lib().oracle_resolve_padding(desc.w, desc.h, desc.kernel_w, desc.kernel_h, desc.dilation_w, desc.dilation_h, desc.stride_w, desc.stride_h,
+                                 desc.pad_left, desc.pad_right, desc.pad_top, desc.pad_bottom, out)
+    return tuple(out)
+
+
 def conv_out_shape(desc):
     ow, oh = C.c_int(), C.c_int()
     lib().oracle_conv_out_shape(C.byref(desc), C.byref(ow), C.byref(oh))

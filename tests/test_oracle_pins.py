@@ -400,6 +400,114 @@ def test_vnni_cpu_baseline_equals_the_scalar_oracle(m, n, k, per_col):
     assert np.array_equal(got, want)
 
 
+def _cpu_conv_desc(cb, d, n):
+    top, bottom, left, right = oracle.resolve_padding(d)
+    return cb.ConvDesc(d.w, d.h, d.c, n, d.num_output, d.kernel_w, d.kernel_h, d.dilation_w, d.dilation_h, d.stride_w, d.stride_h,
+                       left, right, top, bottom, d.pad_value)
+
+
+_EDGE_VALUES = np.array([0.49999997, -0.49999997, 0.5, -0.5, 1.5, -2.5, 126.5, -126.5, 127.49, 300.0, -300.0, 3e9, -3e9, np.inf, -np.inf, np.nan], F)
+
+
+@pytest.mark.parametrize("c,h,w,outc,kernel,dilation,stride,pads,pad_value,term,act,int8_in", [
+    (16, 9, 11, 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 1, 1, False),
+    (3, 20, 20, 20, (7, 7), (1, 1), (2, 2), (3, 3, 3, 3), 0.0, 2, 0, False),        # K = 147: a tail of 3 bytes; 20 channels: a tail of 4 lanes
+    (64, 8, 8, 64, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), 0.0, 101, 1, True),        # rows are the pixels themselves
+    (24, 7, 7, 130, (1, 1), (1, 1), (2, 2), (0, 0, 0, 0), 0.0, 102, 3, True),
+    (8, 10, 9, 17, (3, 2), (2, 1), (1, 2), (-233, -233, -233, -233), 3.0, 1, 2, False),   # SAME_UPPER, a border value, dilation
+    (8, 6, 6, 16, (3, 3), (1, 1), (1, 1), (-234, -234, -234, -234), 0.0, 101, 4, True),
+    (12, 5, 5, 10, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 1, 5, False),
+    (12, 5, 5, 10, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 101, 6, False),
+])
+def test_vnni_convolution_baseline_equals_the_scalar_oracle(c, h, w, outc, kernel, dilation, stride, pads, pad_value, term, act, int8_in):
+    """The im2col + VNNI convolution timed beside the GPU is the oracle's function: fp32 and int8 outputs bit for bit, over
+    batches, every activation type, borders, strides, dilation, channel and K tails, a zero weight scale, and inputs that
+    quantise through float2int8's edge cases."""
+    from oracle import cpubaseline as cb
+    if not cb.available():
+        pytest.skip("host CPU has no AVX512-VNNI")
+    n = 3
+    rng = np.random.default_rng(c * h + outc)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(F)
+    in_scale = F(127.0)
+    x.reshape(-1)[: _EDGE_VALUES.size] = _EDGE_VALUES / in_scale if not int8_in else 0
+    if int8_in:
+        x = rng.integers(-127, 128, (n, c, h, w)).astype(np.int8)
+    wq = rng.integers(-127, 128, (outc, c, kernel[1], kernel[0])).astype(np.int8)
+    ws = rng.uniform(50, 200, outc).astype(F)
+    ws[1] = 0
+    bias = rng.uniform(-1, 1, outc).astype(F)
+    bias[2] = np.nan if act == 1 else bias[2]
+    top = np.array([F(20.0)], F) if term > 100 else None
+    ap = (0.1, 0.0) if act == 2 else (-0.5, 2.0) if act == 3 else (0.2, 0.5) if act == 6 else (0.0, 0.0)
+    d = oracle.make_desc((c, h, w), outc, kernel, dilation, stride, pads, pad_value, 1, 1, term, act, ap)
+    want = np.stack([oracle.convolution_int8(d, x[i], wq, bias, ws, in_scale, None if top is None else top[0]) for i in range(n)])
+    got = cb.conv_nhwc(_cpu_conv_desc(cb, d, n), np.ascontiguousarray(x.transpose(0, 2, 3, 1)), in_scale, cb.pack_conv_weights(wq),
+                       cb.fold_scales(ws, in_scale), bias, top, act, ap)
+    assert np.array_equal(got.transpose(0, 3, 1, 2), want, equal_nan=True)
+
+
+@pytest.mark.parametrize("c,h,w,kernel,stride,pads,term,act,int8_in", [
+    (32, 9, 9, (3, 3), (1, 1), (1, 1, 1, 1), 1, 3, False),
+    (20, 8, 10, (3, 3), (2, 2), (-233, -233, -233, -233), 101, 1, True),
+    (7, 6, 6, (5, 5), (1, 1), (2, 2, 2, 2), 102, 0, False),
+    (48, 7, 7, (3, 3), (1, 1), (1, 1, 1, 1), 2, 2, True),
+])
+def test_depthwise_baseline_equals_the_scalar_oracle(c, h, w, kernel, stride, pads, term, act, int8_in):
+    from oracle import cpubaseline as cb
+    if not cb.available():
+        pytest.skip("host CPU has no AVX512-VNNI")
+    n = 2
+    rng = np.random.default_rng(c + h)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(F)
+    x.reshape(-1)[: _EDGE_VALUES.size] = _EDGE_VALUES / F(100.0)
+    if int8_in:
+        x = rng.integers(-127, 128, (n, c, h, w)).astype(np.int8)
+    wq = rng.integers(-127, 128, (c, 1, kernel[1], kernel[0])).astype(np.int8)
+    per_group = term in (1, 101)
+    ws = rng.uniform(50, 200, c).astype(F) if per_group else np.full(c, F(77.0), F)
+    if per_group:
+        ws[1] = 0
+    ins = np.full(c, F(100.0), F)
+    tops = np.full(c, F(15.0), F) if term > 100 else None
+    bias = rng.uniform(-1, 1, c).astype(F)
+    ap = (0.1, 0.0) if act == 2 else (0.0, 6.0)
+    d = oracle.make_desc((c, h, w), c, kernel, (1, 1), stride, pads, 0.0, 1, c, term, act, ap)
+    want = np.stack([oracle.convolutiondepthwise_int8(d, x[i], wq, bias, ws, ins, tops) for i in range(n)])
+    taps = np.ascontiguousarray(wq.reshape(c, -1).T)
+    got = cb.dwconv_nhwc(_cpu_conv_desc(cb, d, n), np.ascontiguousarray(x.transpose(0, 2, 3, 1)), ins, taps, cb.fold_scales(ws, ins), bias, tops, act, ap)
+    assert np.array_equal(got.transpose(0, 3, 1, 2), want, equal_nan=True)
+
+
+@pytest.mark.parametrize("which,kw", [("tiny", {}), ("mobilenetv2", dict(input_hw=64, n_calib=1)), ("resnet50", dict(input_hw=64, n_calib=1))])
+def test_cpu_baseline_model_pass_equals_the_oracle_executor(which, kw):
+    """The whole-model CPU pass timed beside the GPU (VNNI layers + the glue loops, channels-last) gives the blobs of the
+    scalar oracle's executor bit for bit, for a batch, and again when it writes into the arrays of the pass before."""
+    from ncnn_amd import zoo
+    from oracle import cpubaseline as cb, cpunet
+    import refnet
+    if not cb.available():
+        pytest.skip("host CPU has no AVX512-VNNI")
+    g, param, blob, info = zoo.build(which, **kw)
+    x = np.random.default_rng(4).uniform(0, 1, (2,) + tuple(g.input_shape)).astype(F)
+    model = cpunet.load(param, blob)
+    first = cpunet.run(model, x)
+    again = cpunet.run(model, x[::-1].copy(), keep=first)
+    again = cpunet.run(model, x, keep=again)
+    layers = refnet.parse_param(param)
+    overwritten = {L["bottoms"][0] for L in layers if L["type"] == "ReLU"}  # in-place layers leave their result in the bottom blob
+    for i in range(2):
+        ref = refnet.run(param, blob, x[i])
+        checked = 0
+        for name, v in ref.items():
+            if name in overwritten or name not in again:
+                continue
+            want = v if v.ndim != 3 else v.transpose(1, 2, 0)
+            assert np.array_equal(again[name][i].reshape(want.shape), want), name
+            checked += 1
+        assert checked >= 8
+
+
 def test_float_pipe_formulation_of_float2int8_equals_the_oracle():
     """The device rounds without leaving the float pipe: clamp to [-127, 127], add copysign(0.5) with the add rounded
     TOWARD ZERO, truncate; one compare-select for NaN and |v| >= 2^31.  The same operations evaluated here (the add
