@@ -632,31 +632,48 @@ def bench_conv(args, spec):
     def conv():
         check(lib.ncnnhip_conv_int8_nhwc(C.byref(desc), d_xq.ptr, d_pk.ptr, d_si.ptr, d_b.ptr, None, act, d_out.ptr, 1, 0, 0, d_ws.ptr, sb.value, st))
 
-    for _ in range(args.warmup):
+    def two_launches():
         quantise()
         conv()
+
+    def one_launch():  # the Quantize pass inside the convolution's loader
+        check(lib.ncnnhip_conv_int8_nhwc_from_float(C.byref(desc), d_x.ptr, 4, d_s.ptr, d_pk.ptr, d_si.ptr, d_b.ptr, None, act, d_out.ptr, None, st))
+
+    fused_quantise = bool(lib.ncnnhip_conv_from_float_supported(C.byref(desc)))
+    step = one_launch if fused_quantise else two_launches
+    kernel = one_launch if fused_quantise else conv
+
+    def wall_ms(fn):
+        check(lib.ncnnhip_device_synchronize())
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        check(lib.ncnnhip_device_synchronize())
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    for _ in range(args.warmup):
+        two_launches()
+        step()
     rt.sync()
     ev = _events(lib, check, 2)
     check(lib.ncnnhip_event_record(ev[0], st))
     for _ in range(args.steps):
-        conv()
+        kernel()
     check(lib.ncnnhip_event_record(ev[1], st))
     check(lib.ncnnhip_event_synchronize(ev[1]))
     kernel_ms = _elapsed(lib, check, ev[0], ev[1]) / args.steps
-    check(lib.ncnnhip_device_synchronize())
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        quantise()
-        conv()
-    check(lib.ncnnhip_device_synchronize())
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = wall_ms(step)
+    two_launch_ms = wall_ms(two_launches)
     ops = 2.0 * batch * cout * h * w * c * k * k
     achieved = ops / (kernel_ms * 1e-3) / 1e12
     line = {
         "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "Convolution %dx%d %d->%d on %dx%d, batch %d, fp32 in -> quantise -> int8 implicit GEMM -> fp32 out with ReLU; "
-                               "back-to-back launches, channels-last resident blobs" % (k, k, c, cout, h, w, batch), "kernel_us": kernel_ms * 1e3},
+                               "back-to-back launches, channels-last resident blobs" % (k, k, c, cout, h, w, batch), "kernel_us": kernel_ms * 1e3,
+                   "launches_per_step": 1 if fused_quantise else 2,
+                   "submission": "one launch, the Quantize pass inside the convolution's loader" if fused_quantise else "Quantize kernel, then the convolution kernel",
+                   "quantize_then_convolution_us": two_launch_ms * 1e3},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": measured_traffic("conv:" + spec), "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
     }

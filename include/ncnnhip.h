@@ -164,6 +164,19 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
                                  const float* scale_in_dev, const float* bias_dev, ncnnhip_activation act, float* out_dev,
                                  const ncnnhip_conv_fusion* fusion, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* The same convolution in ONE launch for an input blob that is still fp32 (elemsize 4) or fp16 (2), channels-last: the
+ * layer's own Quantize pass (Quantize::forward, src/layer/quantize.cpp:48-111 as Convolution::forward_int8 calls it at
+ * src/layer/convolution.cpp:392-405: q = float2int8(x * in_scale[0])) runs inside the kernel's loader, so the int8 copy of
+ * the blob is never written.  Group 1, zero border value, channels-last output (fp32, or int8 when scale_out_dev is
+ * given); fusion (may be NULL) as in ncnnhip_conv_int8_nhwc_fused.  Layers whose K the plan would split over workgroups,
+ * or whose tile (64 pixels and up to 128 channels, all of K) exceeds 96 KiB of LDS, are refused: ask ncnnhip_conv_from_float_supported first and
+ * keep the separate ncnnhip_quantize_nhwc + ncnnhip_conv_int8_nhwc for those.  Needs no workspace. */
+int ncnnhip_conv_from_float_supported(const ncnnhip_conv_desc* desc);
+int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, const float* in_scale_dev,
+                                      const int8_t* packed_weight_dev, const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev,
+                                      ncnnhip_activation act, void* out_nhwc_dev, const ncnnhip_conv_fusion* fusion, void* stream);
+
+
 /* Convolution::forward_int8 (src/layer/convolution.cpp:383-508) for layers with at most 4 input channels (the 3-channel
  * first layer of an image net), group 1, dilation_w 1, zero border value.  The input is quantised into an image of 4 bytes
  * per pixel with a physical zero border (ncnnhip_quantize_stem; source: channels-last fp32 blob with pixel stride src_cp, or

@@ -60,6 +60,10 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
 
 // The 1x1 small-K int8-output kernel (conv_pointwise.hip): does this problem fit it, and its launch.  The pipelined
 // launch asks first.
+// One launch for a layer whose input is still fp32 (x_elemsize 4) or fp16 (2): quantised with x_scale[0] inside the kernel.
+bool conv_nhwc_staged_supported(const NhwcGeom& g);
+int launch_conv_nhwc_staged(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
+                            const ConvFusion& fusion, int out_cp, hipStream_t stream);
 bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
 int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream);
 

@@ -516,24 +516,9 @@ int ncnnhip_to_nhwc_int8(const ncnnhip_conv_desc* desc, const void* x_dev, int x
     return launch_status("to_nhwc_int8_kernel");
 }
 
-static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev, const int8_t* packed_weight_dev, const float* scale_in_dev,
-                               const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
-                               size_t out_cstep, size_t out_nstep, const ConvFusion& fusion, void* workspace_dev, size_t workspace_bytes, void* stream)
+static NhwcGeom nhwc_geometry(const ncnnhip_conv_desc& d, int outw, int outh, long long npix)
 {
-    NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_nhwc: null pointer");
-    NCNNHIP_REQUIRE(desc->group == 1, "ncnnhip_conv_int8_nhwc: group must be 1");
-    int outw, outh;
-    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
-    if (ret) return ret;
-    const ncnnhip_conv_desc& d = *desc;
-    const long long plane = (long long)outw * outh, npix = plane * d.batch;
-    NCNNHIP_REQUIRE(out_layout == NCNNHIP_PLANAR || out_layout == NCNNHIP_CHANNELS_LAST, "ncnnhip_conv_int8_nhwc: unknown output layout %d", out_layout);
-    const bool clast = out_layout == NCNNHIP_CHANNELS_LAST;
-    const int out_cp = padded_channels(desc->num_output);
-    NCNNHIP_REQUIRE(npix < (1ll << 31) && (clast || out_cstep >= (size_t)plane), "ncnnhip_conv_int8_nhwc: bad output extent");
-    NCNNHIP_REQUIRE((long long)d.h * d.w * padded_channels(d.c) < (1ll << 31), "ncnnhip_conv_int8_nhwc: one input sample exceeds 2 GiB");
     const Pads4 pads = resolve_pads_nhwc(d);
-
     NhwcGeom g;
     g.H = d.h;
     g.W = d.w;
@@ -555,6 +540,29 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc
     g.cout = d.num_output;
     const int pb = (int)(signed char)d.pad_value & 0xff;
     g.pad_word = (int)((uint32_t)pb * 0x01010101u);
+    return g;
+}
+
+// x_elemsize 1: nhwc_dev is the quantised blob.  4 / 2: it is the fp32 / fp16 blob, quantised with x_scale_dev[0] inside the
+// one launch (channels-last output and a layer ncnnhip_conv_from_float_supported accepts).
+static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int x_elemsize, const float* x_scale_dev, const int8_t* packed_weight_dev,
+                               const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_dev, int out_layout,
+                               size_t out_cstep, size_t out_nstep, const ConvFusion& fusion, void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(desc && nhwc_dev && packed_weight_dev && scale_in_dev && out_dev, "ncnnhip_conv_int8_nhwc: null pointer");
+    NCNNHIP_REQUIRE(desc->group == 1, "ncnnhip_conv_int8_nhwc: group must be 1");
+    int outw, outh;
+    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
+    if (ret) return ret;
+    const ncnnhip_conv_desc& d = *desc;
+    const long long plane = (long long)outw * outh, npix = plane * d.batch;
+    NCNNHIP_REQUIRE(out_layout == NCNNHIP_PLANAR || out_layout == NCNNHIP_CHANNELS_LAST, "ncnnhip_conv_int8_nhwc: unknown output layout %d", out_layout);
+    const bool clast = out_layout == NCNNHIP_CHANNELS_LAST;
+    const int out_cp = padded_channels(desc->num_output);
+    NCNNHIP_REQUIRE(npix < (1ll << 31) && (clast || out_cstep >= (size_t)plane), "ncnnhip_conv_int8_nhwc: bad output extent");
+    NCNNHIP_REQUIRE((long long)d.h * d.w * padded_channels(d.c) < (1ll << 31), "ncnnhip_conv_int8_nhwc: one input sample exceeds 2 GiB");
+    const NhwcGeom g = nhwc_geometry(d, outw, outh, npix);
+    const int pb = g.pad_word & 0xff;
 
     ConvEpilogue epi;
     epi.scale_in = scale_in_dev;
@@ -571,8 +579,14 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc
     epi.acc_out = 0;
 
     hipStream_t st = as_stream(stream);
+    if (x_elemsize != 1)
+    {
+        NCNNHIP_REQUIRE(clast && x_scale_dev, "ncnnhip_conv_int8_nhwc_from_float: needs channels-last output and the input scale");
+        return launch_conv_nhwc_staged(g, packed_weight_dev, nhwc_dev, x_elemsize, x_scale_dev, epi, fusion, out_cp, st);
+    }
+    const int8_t* xq = static_cast<const int8_t*>(nhwc_dev);
     // zero border and channels-last output: the pipelined kernel
-    if (clast && pb == 0) return launch_conv_nhwc_pipelined(g, packed_weight_dev, nhwc_dev, epi, fusion, out_cp, workspace_dev, workspace_bytes, st);
+    if (clast && pb == 0) return launch_conv_nhwc_pipelined(g, packed_weight_dev, xq, epi, fusion, out_cp, workspace_dev, workspace_bytes, st);
     NCNNHIP_REQUIRE(!fusion.residual && !fusion.relu_after && !fusion.q8_out, "ncnnhip_conv_int8_nhwc_fused: needs channels-last output and a zero border value");
     const SplitPlan p = plan_launch(d.num_output, npix, g.K / 64);
     dim3 grid(ceil_div(npix, p.bn), ceil_div(d.num_output, p.bm), p.splits);
@@ -590,13 +604,13 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const int8_t* nhwc
     do                                                                                                                                               \
     {                                                                                                                                                \
         if (p.splits > 1 && clast)                                                                                                                   \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, true>), grid, dim3(256), 0, st, packed_weight_dev, xq, g, epi, p.steps_per_split, partial, out_cp); \
         else if (p.splits > 1)                                                                                                                       \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, true, false>), grid, dim3(256), 0, st, packed_weight_dev, xq, g, epi, p.steps_per_split, partial, out_cp); \
         else if (clast)                                                                                                                              \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, true>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, true>), grid, dim3(256), 0, st, packed_weight_dev, xq, g, epi, p.steps_per_split, partial, out_cp); \
         else                                                                                                                                         \
-            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, false>), grid, dim3(256), 0, st, packed_weight_dev, nhwc_dev, g, epi, p.steps_per_split, partial, out_cp); \
+            hipLaunchKernelGGL((conv_nhwc_kernel<BM_, BN_, false, false>), grid, dim3(256), 0, st, packed_weight_dev, xq, g, epi, p.steps_per_split, partial, out_cp); \
     } while (0)
     if (p.bm == 128 && p.bn == 128)
         LAUNCH_NHWC(128, 128);
@@ -619,7 +633,7 @@ int ncnnhip_conv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_dev
                            size_t out_cstep, size_t out_nstep, void* workspace_dev, size_t workspace_bytes, void* stream)
 {
     const ConvFusion none = {0, 0, 0, 0.f};
-    return conv_int8_nhwc_impl(desc, nhwc_dev, packed_weight_dev, scale_in_dev, bias_dev, scale_out_dev, act, out_dev, out_layout, out_cstep, out_nstep, none,
+    return conv_int8_nhwc_impl(desc, nhwc_dev, 1, 0, packed_weight_dev, scale_in_dev, bias_dev, scale_out_dev, act, out_dev, out_layout, out_cstep, out_nstep, none,
                                workspace_dev, workspace_bytes, stream);
 }
 
@@ -640,8 +654,39 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
     f.relu_after = fusion->relu_after;
     f.q8_out = fusion->quantised_out_dev;
     f.q8_scale = fusion->quantise_scale;
-    return conv_int8_nhwc_impl(desc, nhwc_dev, packed_weight_dev, scale_in_dev, bias_dev, 0, act, out_dev, NCNNHIP_CHANNELS_LAST, 0, 0, f, workspace_dev,
+    return conv_int8_nhwc_impl(desc, nhwc_dev, 1, 0, packed_weight_dev, scale_in_dev, bias_dev, 0, act, out_dev, NCNNHIP_CHANNELS_LAST, 0, 0, f, workspace_dev,
                                workspace_bytes, stream);
+}
+
+int ncnnhip_conv_from_float_supported(const ncnnhip_conv_desc* desc)
+{
+    if (!desc || desc->group != 1 || (int)(signed char)desc->pad_value != 0) return 0;
+    int outw = 0, outh = 0;
+    if (ncnnhip_conv_out_shape(desc, &outw, &outh) != 0) return 0;
+    const long long npix = (long long)outw * outh * desc->batch;
+    if (npix >= (1ll << 31) || (long long)desc->h * desc->w * padded_channels(desc->c) >= (1ll << 31)) return 0;
+    return conv_nhwc_staged_supported(nhwc_geometry(*desc, outw, outh, npix)) ? 1 : 0;
+}
+
+int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, const float* in_scale_dev,
+                                      const int8_t* packed_weight_dev, const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev,
+                                      ncnnhip_activation act, void* out_dev, const ncnnhip_conv_fusion* fusion, void* stream)
+{
+    NCNNHIP_REQUIRE(elemsize == 4 || elemsize == 2, "ncnnhip_conv_int8_nhwc_from_float: activations are fp32 (4) or fp16 (2), not %d bytes", elemsize);
+    NCNNHIP_REQUIRE(ncnnhip_conv_from_float_supported(desc), "ncnnhip_conv_int8_nhwc_from_float: this layer needs its separate Quantize pass");
+    NCNNHIP_REQUIRE((reinterpret_cast<uintptr_t>(nhwc_dev) & 15) == 0, "ncnnhip_conv_int8_nhwc_from_float: the blob must be 16-byte aligned");
+    ConvFusion f = {0, 0, 0, 0.f};
+    if (fusion)
+    {
+        NCNNHIP_REQUIRE(!scale_out_dev, "ncnnhip_conv_int8_nhwc_from_float: the fused tail belongs to the fp32 output");
+        NCNNHIP_REQUIRE(!fusion->quantised_out_dev || fusion->quantise_scale != 0.f, "ncnnhip_conv_int8_nhwc_from_float: quantised copy without a scale");
+        f.residual = fusion->residual_dev;
+        f.relu_after = fusion->relu_after;
+        f.q8_out = fusion->quantised_out_dev;
+        f.q8_scale = fusion->quantise_scale;
+    }
+    return conv_int8_nhwc_impl(desc, nhwc_dev, elemsize, in_scale_dev, packed_weight_dev, scale_in_dev, bias_dev, scale_out_dev, act, out_dev, NCNNHIP_CHANNELS_LAST,
+                               0, 0, f, 0, 0, stream);
 }
 
 int ncnnhip_conv_stem_supported(const ncnnhip_conv_desc* desc)

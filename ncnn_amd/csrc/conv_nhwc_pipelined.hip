@@ -19,6 +19,7 @@
 // dumps its accumulator registers to scratch (register-major, fully coalesced) and bumps the tile's counter; the
 // last one adds the others' dumps to its own registers (integer addition: exact in any order), resets the counter
 // and runs the normal epilogue.  Nobody waits for anybody, so the grid may be larger than the chip.
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 
@@ -59,17 +60,29 @@ __device__ __forceinline__ int small_div(int n, int d)
 // also Gemm and InnerProduct); 2: taps of 16 or 32 bytes (the narrow-input image), a whole number of taps per K step.
 // A template parameter because the choice sits inside the K loop: as run-time branches there it cost the 3x3 layers
 // of ResNet-50's last stages 2-4 us each (15.4 against 11.4 us for 256 -> 256 on 14 x 14, batch 16).
-template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM, int MODE>
+//
+// AIN: bytes per activation value.  1: the blob is int8 and goes global -> LDS directly, as described above.  4 (fp32)
+// or 2 (fp16): the layer's Quantize pass happens here (Quantize::forward, src/layer/quantize.cpp:48-111, one scale):
+// before the K loop the workgroup gathers its BM pixels x K im2col tile through registers, float2int8(value * scale)
+// each value, and writes the bytes into a tile-sized LDS region (dynamic shared memory, BM * K bytes) in the layout a
+// stage would have.  The weights of the tile (BN * K bytes) are requested in full before that and land in a region of
+// their own while the loader works, so the K loop touches LDS only: no waits on memory, no barriers.  x points at the
+// fp32 / fp16 blob, same channels-last geometry counted in values.
+template<int BM, int BN, int STAGES, bool SPLITK, bool GEMM, int MODE, int AIN = 1>
 __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* __restrict__ wpk, const int8_t* __restrict__ x, NhwcGeom g, ConvEpilogue epi,
-                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int32_t* __restrict__ partial, unsigned* __restrict__ counters)
+                                                                   ConvFusion fusion, GemmTail gemm, int out_cp, int col_limit, int tiles_m, int tiles_n, int splits, int steps_per_split, unsigned magic_n, int32_t* __restrict__ partial, unsigned* __restrict__ counters,
+                                                                   const float* __restrict__ a_scale, int a_cache_bytes)
 {
     constexpr bool dense = MODE == 1;
+    constexpr bool STAGED = AIN != 1;
+    static_assert(!STAGED || (!SPLITK && !GEMM && MODE != 2), "the quantising loader exists for whole-K convolution tiles");
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
-    constexpr int LA = BM / 64, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
+    constexpr int LAR = BM / 64;              // 64-row groups of the activation tile
+    constexpr int LA = STAGED ? 0 : LAR, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
     static_assert(STAGES >= 2 && STAGES <= 7 && (STAGES - 2) * (LA + LB) < 64, "the vmcnt field counts to 63");
     constexpr int STAGE_BYTES = (BM + BN) * 64;
     constexpr int EPILOGUE_BYTES = 4 * 32 * (BN / 2 + 4) * 4; // per wavefront 32 pixels x (BN/2 + 4) floats
-    constexpr int SMEM_BYTES = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
+    constexpr int SMEM_BYTES = (!STAGED && STAGES * STAGE_BYTES > EPILOGUE_BYTES) ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
     __shared__ __attribute__((aligned(1024))) int8_t smem[SMEM_BYTES];
 
     const int lane = threadIdx.x & 63;
@@ -104,10 +117,11 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
     const int8_t* zero = g_zero_line;
 
-    const int8_t* a_base[LA];
-    int a_iy0[LA], a_ix0[LA];
+    const int8_t* a_base[LAR];
+    int a_iy0[LAR], a_ix0[LAR];
+    int a_img0[LAR]; // first pixel of the row's image, counted in input pixels over the whole batch (the quantising loader's cache)
 #pragma unroll
-    for (int i = 0; i < LA; i++)
+    for (int i = 0; i < LAR; i++)
     {
         const int n = row0 + i * 64 + ld_row;
         const bool ok = n < g.npix;
@@ -136,7 +150,8 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         a_iy0[i] = ok ? oy * g.sh - g.pad_top : -0x40000000;
         a_ix0[i] = ox * g.sw - g.pad_left;
         // dense: the pixel's own address, so that a stage's source is one 64-bit add away
-        a_base[i] = dense ? x + (size_t)nn * g.Cp : x + (size_t)img * g.H * g.W * g.Cp;
+        a_base[i] = dense ? x + (size_t)nn * g.Cp * AIN : x + (size_t)img * g.H * g.W * g.Cp * AIN;
+        a_img0[i] = img * g.H * g.W;
     }
     const int8_t* b_ptr[LB];
 #pragma unroll
@@ -173,10 +188,14 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
         q0 = k - tap * g.tapK;
     }
+    const int first_q0 = q0, first_tap = tap, first_ky = ky, first_kx = kx; // where the quantising loader starts (issue() moves the others on)
 
     // issues the loads of the next stage in sequence (s = 0, 1, 2, ... relative to step_begin)
+    extern __shared__ __attribute__((aligned(1024))) int8_t a_tile[]; // quantising loader: [K/64][BM][64] activations, then [K/64][BN][64] weights, then the input cache
     auto issue = [&](int s) {
-        int8_t* stage = smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
+        // quantising loader: every step has its own place (written once); the address below is that place minus the
+        // activation part a ring stage would start with
+        int8_t* stage = STAGED ? a_tile + total_steps * (BM * 64) + s * (BN * 64) - BM * 64 + wave * 1024 : smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
         if (dense)
         {
             // one tap, no border: the row's pixel exists or it does not (a_iy0 is 0 or hugely negative)
@@ -268,26 +287,320 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         }
     }
 
+    if constexpr (STAGED)
+        for (int s = 0; s < nk; s++) issue(s); // all the tile's weights at once (at most 48 loads per lane: the launch checks K)
+    else
+    {
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; s++)
-        if (s < nk) issue(s);
+        for (int s = 0; s < STAGES - 1; s++)
+            if (s < nk) issue(s);
+    }
+
+    // ---- the quantising loader: the whole activation tile, fp32 / fp16 -> int8, while the first weight stages arrive
+    unsigned a_tile_lds = 0;
+    if constexpr (STAGED)
+    {
+        a_tile_lds = (unsigned)(uintptr_t)(AS3 int8_t*)a_tile;
+        const float sc = a_scale[0];
+        int pq0 = first_q0, ptap = first_tap, pky = first_ky, pkx = first_kx;
+        // The taps of neighbouring output pixels overlap: a 3x3 layer reads every input value nine times.  The input
+        // pixels a tile touches form one contiguous run of the blob (counted over the whole batch, first tap of the
+        // first row to last tap of the last row); when that run fits the cache region behind the tile, it is fetched
+        // and quantised ONCE, fully coalesced and all loads in flight together, and the im2col tile is then gathered
+        // from LDS.  Otherwise (and for 1x1 stride-1 layers, which read nothing twice) the tile is gathered from global
+        // memory directly, three K steps at a time.
+        bool cached = false;
+        // (barriers in here wait for LDS traffic only: the weight stages requested above stay in flight)
+        auto lds_barrier = [] {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        };
+        if (!dense && a_cache_bytes > 0)
+        {
+            // first and last input pixel of the tile: a wavefront reduction, then the four wavefronts' results through LDS
+            __shared__ int run[4][2];
+            int first = 0x7fffffff, last = -0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < LAR; i++)
+                if (a_iy0[i] > -0x40000000) // the row is a real output pixel
+                {
+                    const int f = a_img0[i] + a_iy0[i] * g.W + a_ix0[i];
+                    const int l = f + (g.kh - 1) * g.dh * g.W + (g.kw - 1) * g.dw;
+                    first = f < first ? f : first;
+                    last = l > last ? l : last;
+                }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1)
+            {
+                const int of = __shfl_xor(first, d), ol = __shfl_xor(last, d);
+                first = of < first ? of : first;
+                last = ol > last ? ol : last;
+            }
+            if (lane == 0)
+            {
+                run[wave][0] = first;
+                run[wave][1] = last;
+            }
+            lds_barrier();
+#pragma unroll
+            for (int w2 = 0; w2 < 4; w2++)
+            {
+                first = run[w2][0] < first ? run[w2][0] : first;
+                last = run[w2][1] > last ? run[w2][1] : last;
+            }
+            // taps outside the image are never looked up, so the run may be cut to the blob
+            const int in_pixels = epi.batch * g.H * g.W;
+            const int lo = __builtin_amdgcn_readfirstlane(first > 0 ? first : 0);
+            const int hi = __builtin_amdgcn_readfirstlane(last < in_pixels - 1 ? last : in_pixels - 1);
+            const int count = hi - lo + 1;
+            if (count > 0 && (long long)count * g.Cp <= (long long)a_cache_bytes)
+            {
+                cached = true;
+                int8_t* cache = a_tile + total_steps * ((BM + BN) * 64);
+                // 4 values per lane and load: a wavefront instruction reads 1 KiB (fp32) or 512 B (fp16) of consecutive addresses
+                const int nquad = count * (g.Cp >> 2);
+                const int8_t* src0 = x + (size_t)lo * g.Cp * AIN;
+                constexpr int INFL = 12; // loads in flight per lane
+                for (int q0v = 0; q0v < nquad; q0v += 256 * INFL)
+                {
+                    v4f val[INFL];
+#pragma unroll
+                    for (int j = 0; j < INFL; j++)
+                    {
+                        int qi = q0v + j * 256 + (int)threadIdx.x;
+                        if (qi >= nquad) qi = nquad - 1; // a valid address; the value is not stored
+                        if constexpr (AIN == 4)
+                            val[j] = *reinterpret_cast<const v4f*>(src0 + (size_t)qi * 16);
+                        else
+                        {
+                            typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                            const v2u pair = *reinterpret_cast<const v2u*>(src0 + (size_t)qi * 8);
+                            val[j][0] = (float)__builtin_bit_cast(_Float16, (unsigned short)(pair[0] & 0xffffu));
+                            val[j][1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(pair[0] >> 16));
+                            val[j][2] = (float)__builtin_bit_cast(_Float16, (unsigned short)(pair[1] & 0xffffu));
+                            val[j][3] = (float)__builtin_bit_cast(_Float16, (unsigned short)(pair[1] >> 16));
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < INFL; j++)
+                    {
+                        const int qi = q0v + j * 256 + (int)threadIdx.x;
+                        float v0 = mul_rn(val[j][0], sc), v1 = mul_rn(val[j][1], sc), v2 = mul_rn(val[j][2], sc), v3 = mul_rn(val[j][3], sc);
+                        float2int8_as_float_x4(v0, v1, v2, v3);
+                        const uint32_t word = pack4_quantised(v0, v1, v2, v3);
+                        if (qi < nquad) *reinterpret_cast<uint32_t*>(cache + (size_t)qi * 4) = word;
+                    }
+                }
+                lds_barrier();
+                // the gather, LDS -> LDS: four K steps' reads in flight, then their writes
+                constexpr int GATHER = 12;
+                // the lane's first tap of its row, as a byte offset into the cache (may point outside: only looked up when the tap is inside the image)
+                int row_byte0[LAR];
+#pragma unroll
+                for (int i = 0; i < LAR; i++) row_byte0[i] = (a_img0[i] + a_iy0[i] * g.W + a_ix0[i] - lo) * g.Cp;
+                int8_t* const tile_lane = a_tile + wave * 1024 + lane * 16;
+                if ((g.tapK & 63) == 0)
+                {
+                    // a K step lies inside one tap, the same for every lane: its position is wavefront-uniform arithmetic
+                    const int chunk_byte = ld_chunk * 16;
+                    int stap = 0, sq0 = 0, sky = 0, skx = 0; // (the tile starts at K = 0: this loader is never split over workgroups)
+                    for (int s0 = 0; s0 < nk; s0 += GATHER)
+                    {
+                        v4i piece[GATHER][LAR];
+#pragma unroll
+                        for (int u = 0; u < GATHER; u++)
+                        {
+                            const bool tap_ok = s0 + u < nk && stap < g.ntaps;
+                            const int dy = sky * g.dh, dx = skx * g.dw;
+                            const int step_byte = (dy * g.W + dx) * g.Cp + sq0 + chunk_byte;
+#pragma unroll
+                            for (int i = 0; i < LAR; i++)
+                            {
+                                const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+                                const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                                const v4i got = *reinterpret_cast<const v4i*>(cache + (in ? row_byte0[i] + step_byte : 0));
+                                piece[u][i] = in ? got : v4i{0, 0, 0, 0}; // the border is zero bytes whatever the scale
+                            }
+                            sq0 += 64;
+                            if (sq0 >= g.tapK)
+                            {
+                                sq0 = 0;
+                                stap++;
+                                if (++skx == g.kw)
+                                {
+                                    skx = 0;
+                                    sky++;
+                                }
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < GATHER; u++)
+                            if (s0 + u < nk)
+                            {
+#pragma unroll
+                                for (int i = 0; i < LAR; i++) *reinterpret_cast<v4i*>(tile_lane + (s0 + u) * (BM * 64) + i * 4096) = piece[u][i];
+                            }
+                    }
+                }
+                else
+                    for (int s0 = 0; s0 < nk; s0 += GATHER)
+                    {
+                        v4i piece[GATHER][LAR];
+#pragma unroll
+                        for (int u = 0; u < GATHER; u++)
+                        {
+                            const bool tap_ok = s0 + u < nk && ptap < g.ntaps;
+                            const int dy = pky * g.dh, dx = pkx * g.dw;
+#pragma unroll
+                            for (int i = 0; i < LAR; i++)
+                            {
+                                const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+                                const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                                const v4i got = *reinterpret_cast<const v4i*>(cache + (in ? row_byte0[i] + (dy * g.W + dx) * g.Cp + pq0 : 0));
+                                piece[u][i] = in ? got : v4i{0, 0, 0, 0};
+                            }
+                            pq0 += 64;
+                            while (pq0 >= g.tapK)
+                            {
+                                pq0 -= g.tapK;
+                                ptap++;
+                                if (++pkx == g.kw)
+                                {
+                                    pkx = 0;
+                                    pky++;
+                                }
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < GATHER; u++)
+                            if (s0 + u < nk)
+                            {
+#pragma unroll
+                                for (int i = 0; i < LAR; i++) *reinterpret_cast<v4i*>(tile_lane + (s0 + u) * (BM * 64) + i * 4096) = piece[u][i];
+                            }
+                    }
+            }
+        }
+        constexpr int GRP = AIN == 4 ? 3 : 6; // K steps whose loads are in flight together (48 registers of raw values)
+        constexpr int NLD = AIN == 4 ? 4 : 2; // 16-byte loads per 16 values
+        for (int s0 = cached ? nk : 0; s0 < nk; s0 += GRP)
+        {
+            v4i raw[GRP][LAR][NLD];
+            unsigned inside = 0; // bit u * LAR + i: the values are real (not border, not beyond K, not beyond the last pixel)
+#pragma unroll
+            for (int u = 0; u < GRP; u++)
+            {
+                const bool tap_ok = s0 + u < nk && (dense ? ptap == 0 : ptap < g.ntaps);
+                const int dy = pky * g.dh, dx = pkx * g.dw;
+#pragma unroll
+                for (int i = 0; i < LAR; i++)
+                {
+                    bool in;
+                    size_t off;
+                    if (dense)
+                    {
+                        in = tap_ok && a_iy0[i] == 0;
+                        off = (size_t)pq0;
+                    }
+                    else
+                    {
+                        const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+                        in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                        off = ((size_t)iy * g.W + ix) * g.Cp + pq0;
+                    }
+                    const int8_t* src = in ? a_base[i] + off * AIN : zero;
+                    inside |= in ? 1u << (u * LAR + i) : 0u;
+#pragma unroll
+                    for (int j = 0; j < NLD; j++) raw[u][i][j] = *reinterpret_cast<const v4i*>(src + 16 * j);
+                }
+                pq0 += 64;
+                if (dense)
+                {
+                    if (pq0 >= g.tapK) ptap = 1;
+                }
+                else
+                    while (pq0 >= g.tapK)
+                    {
+                        pq0 -= g.tapK;
+                        ptap++;
+                        if (++pkx == g.kw)
+                        {
+                            pkx = 0;
+                            pky++;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < GRP; u++)
+            {
+                if (s0 + u < nk)
+                {
+#pragma unroll
+                    for (int i = 0; i < LAR; i++)
+                    {
+                        float v[16];
+                        if constexpr (AIN == 4)
+                        {
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+#pragma unroll
+                                for (int e = 0; e < 4; e++) v[j * 4 + e] = mul_rn(__int_as_float(raw[u][i][j][e]), sc);
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int j = 0; j < 2; j++)
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                {
+                                    const unsigned pair = (unsigned)raw[u][i][j][e]; // two halves, the first in the low 16 bits
+                                    v[j * 8 + e * 2] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair & 0xffffu)), sc);
+                                    v[j * 8 + e * 2 + 1] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair >> 16)), sc);
+                                }
+                        }
+#pragma unroll
+                        for (int e = 0; e < 16; e += 4) float2int8_as_float_x4(v[e], v[e + 1], v[e + 2], v[e + 3]);
+                        v4i w;
+                        uint32_t r0, r1, r2, r3;
+                        pack16_quantised(v, r0, r1, r2, r3);
+                        // the border is zero bytes whatever the scale (the reference pads after it quantises)
+                        const bool real = (inside >> (u * LAR + i)) & 1u;
+                        w[0] = real ? (int)r0 : 0;
+                        w[1] = real ? (int)r1 : 0;
+                        w[2] = real ? (int)r2 : 0;
+                        w[3] = real ? (int)r3 : 0;
+                        const unsigned dst = a_tile_lds + (unsigned)((s0 + u) * (BM * 64) + i * 4096 + wave * 1024 + lane * 16);
+                        asm volatile("ds_write_b128 %0, %1" ::"v"(dst), "v"(w) : "memory");
+                    }
+                }
+            }
+        }
+        // every wavefront's bytes, and the weights it asked for, are in place before anybody multiplies
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    }
 
     for (int t = 0; t < nk; t++)
     {
-        // this wavefront's loads of step t have landed (later stages may stay in flight) ...
-        const int ahead = nk - 1 - t < STAGES - 2 ? nk - 1 - t : STAGES - 2;
-        switch (ahead)
+        if constexpr (!STAGED)
         {
-        case 0: WAIT_VMCNT(0); break;
-        case 1: WAIT_VMCNT(1 * (LA + LB)); break;
-        case 2: WAIT_VMCNT(2 * (LA + LB)); break;
-        case 3: WAIT_VMCNT(3 * (LA + LB)); break;
-        case 4: WAIT_VMCNT(4 * (LA + LB)); break;
-        default: WAIT_VMCNT(5 * (LA + LB)); break; // STAGES <= 7
+            // this wavefront's loads of step t have landed (later stages may stay in flight) ...
+            const int ahead = nk - 1 - t < STAGES - 2 ? nk - 1 - t : STAGES - 2;
+            switch (ahead)
+            {
+            case 0: WAIT_VMCNT(0); break;
+            case 1: WAIT_VMCNT(1 * (LA + LB)); break;
+            case 2: WAIT_VMCNT(2 * (LA + LB)); break;
+            case 3: WAIT_VMCNT(3 * (LA + LB)); break;
+            case 4: WAIT_VMCNT(4 * (LA + LB)); break;
+            default: WAIT_VMCNT(5 * (LA + LB)); break; // STAGES <= 7
+            }
+            // ... and everybody's: the barrier also says nobody still reads the stage refilled next
+            __builtin_amdgcn_s_barrier();
         }
-        // ... and everybody's: the barrier also says nobody still reads the stage refilled next
-        __builtin_amdgcn_s_barrier();
-        const unsigned st = lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
+        // (quantising loader: step t's weights at their own place, see issue())
+        const unsigned st = STAGED ? a_tile_lds + (unsigned)(total_steps * (BM * 64) + t * (BN * 64) - BM * 64) : lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
         // fragment reads of both K halves go out first; the address arithmetic and the global loads of the stage
         // refilled next are issued while they are in flight
         v4i fa[2][TM], fb[2][TN];
@@ -296,11 +609,12 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         {
             const unsigned chunk = ks ? ch1 : ch0;
 #pragma unroll
-            for (int a = 0; a < TM; a++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[ks][a]) : "v"(st + rd_a + chunk + (unsigned)(a * 32 * 64)));
+            for (int a = 0; a < TM; a++)
+                asm volatile("ds_read_b128 %0, %1" : "=v"(fa[ks][a]) : "v"((STAGED ? a_tile_lds + (unsigned)(t * (BM * 64)) : st) + rd_a + chunk + (unsigned)(a * 32 * 64)));
 #pragma unroll
             for (int c = 0; c < TN; c++) asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks][c]) : "v"(st + rd_b + chunk + (unsigned)(c * 32 * 64)));
         }
-        if (t + STAGES - 1 < nk) issue(t + STAGES - 1);
+        if (!STAGED && t + STAGES - 1 < nk) issue(t + STAGES - 1);
         // the reads are asm, so the wait is too; passing each fragment through an (empty) volatile asm after it
         // keeps the MFMAs, which consume those values, below the wait
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -692,7 +1006,7 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
     const int mode = dense ? 1 : ((g.tapK == 16 || g.tapK == 32) && p.splits == 1) ? 2 : 0;
 #define LAUNCH_PIPE_MODE(BM_, BN_, ST_, SPLIT_, MODE_)                                                                                                          \
     hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, SPLIT_, false, MODE_>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, \
-                       p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters)
+                       p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters, (const float*)0, 0)
 #define LAUNCH_PIPE(BM_, BN_, ST_)                                                                                                              \
     do                                                                                                                                          \
     {                                                                                                                                           \
@@ -723,6 +1037,91 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
 #undef LAUNCH_PIPE
 #undef LAUNCH_PIPE_MODE
     return launch_status("conv_nhwc_pipelined_kernel");
+}
+
+// ---- one launch for a layer whose input is still fp32 / fp16: the kernel's quantising loader (AIN = 4 / 2)
+static const size_t STAGED_TILE_LIMIT = 96u << 10; // bytes of LDS for the tile's operands: (64 pixels + BN channels) x K
+static const size_t STAGED_LDS_LIMIT = 124u << 10; // operands + input cache (the epilogue staging takes up to 34 KiB more)
+
+static bool staged_plan(const NhwcGeom& g_in, NhwcGeom& g, PipePlan& p, int& mode)
+{
+    g = g_in;
+    const int dense = g.kw == 1 && g.kh == 1 && g.sw == 1 && g.sh == 1 && g.pad_top == 0 && g.pad_left == 0 && g.outw == g.W && g.outh == g.H && g.tapK == g.Cp;
+    if (dense)
+    {
+        g.H = g.outh = 1;
+        g.W = g.outw = g.npix;
+    }
+    p = plan_pipelined(g.cout, g.npix, g.K / 64);
+    mode = dense ? 1 : 0;
+    // whole-K tiles of 64 pixels only: a layer the plan would split over workgroups keeps its separate Quantize pass
+    return p.splits == 1 && p.bm == 64 && p.bn <= 128 && (size_t)g.K * (64 + p.bn) <= STAGED_TILE_LIMIT && g.K / 64 * (p.bn / 64) <= 48 && g.pad_word == 0 &&
+           g.tapK == g.Cp &&
+           (long long)p.tiles_m * p.tiles_n * p.tiles_n < (1ll << 32);
+}
+
+bool conv_nhwc_staged_supported(const NhwcGeom& g_in)
+{
+    NhwcGeom g;
+    PipePlan p;
+    int mode;
+    return staged_plan(g_in, g, p, mode);
+}
+
+int launch_conv_nhwc_staged(const NhwcGeom& g_in, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
+                            const ConvFusion& fusion, int out_cp, hipStream_t stream)
+{
+    NhwcGeom g;
+    PipePlan p;
+    int mode;
+    NCNNHIP_REQUIRE(x_elemsize == 4 || x_elemsize == 2, "convolution: activations of %d bytes per value", x_elemsize);
+    NCNNHIP_REQUIRE(staged_plan(g_in, g, p, mode), "convolution: this layer does not fit the one-launch form (ask ncnnhip_conv_from_float_supported first)");
+    const size_t tile_bytes = (size_t)g.K * (64 + p.bn);
+    // Behind the tile, a cache for the run of input pixels a tile touches (quantised once instead of once per tap): 64
+    // consecutive output pixels span at most (63 / outw + 2) output rows, one more image-to-image gap of at most
+    // (H + pad) rows, and the kernel's own extent.  An estimate only: the kernel measures each tile's run and gathers
+    // from global memory when it does not fit.
+    size_t cache_bytes = 0;
+    if (mode == 0 && (long long)epi.batch * g.H * g.W < (1ll << 30))
+    {
+        const long long rows = (63 / g.outw + 2) * (long long)g.sh + (long long)(g.kh - 1) * g.dh + g.H - (long long)(g.outh - 1) * g.sh + 2;
+        const long long pixels = rows * g.W + (long long)(g.kw - 1) * g.dw + 64ll * g.sw;
+        const size_t room = STAGED_LDS_LIMIT - tile_bytes;
+        cache_bytes = (size_t)std::min<long long>(pixels * g.Cp, (long long)room) & ~(size_t)15;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+    const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
+    const int8_t* xb = static_cast<const int8_t*>(x);
+#define LAUNCH_STAGED(BN_, MODE_, AIN_)                                                                                                                      \
+    do                                                                                                                                                       \
+    {                                                                                                                                                        \
+        auto kernel = conv_nhwc_pipelined_kernel<64, BN_, 3, false, false, MODE_, AIN_>;                                                                     \
+        static std::once_flag once;                                                                                                                          \
+        static hipError_t attr = hipSuccess;                                                                                                                 \
+        std::call_once(once, [&]() { attr = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)STAGED_LDS_LIMIT); });  \
+        NCNNHIP_CHECK(attr);                                                                                                                                 \
+        hipLaunchKernelGGL(kernel, grid, block, tile_bytes + cache_bytes, stream, wpk, xb, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
+                           1, p.steps_per_split, tile_magic(p.tiles_n), (int32_t*)0, (unsigned*)0, x_scale, (int)cache_bytes);                              \
+    } while (0)
+#define LAUNCH_STAGED_IN(BN_, MODE_)        \
+    do                                      \
+    {                                       \
+        if (x_elemsize == 4)                \
+            LAUNCH_STAGED(BN_, MODE_, 4);   \
+        else                                \
+            LAUNCH_STAGED(BN_, MODE_, 2);   \
+    } while (0)
+    if (p.bn == 128 && mode == 1)
+        LAUNCH_STAGED_IN(128, 1);
+    else if (p.bn == 128)
+        LAUNCH_STAGED_IN(128, 0);
+    else if (mode == 1)
+        LAUNCH_STAGED_IN(64, 1);
+    else
+        LAUNCH_STAGED_IN(64, 0);
+#undef LAUNCH_STAGED_IN
+#undef LAUNCH_STAGED
+    return launch_status("conv_nhwc_pipelined_kernel (quantising loader)");
 }
 
 int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmTail& tail,
@@ -770,7 +1169,7 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
     dim3 grid((unsigned)blocks), block(256);
 #define LAUNCH_GEMM(BM_, BN_)                                                                                                                        \
     hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, 3, false, true, 1>), grid, block, 0, stream, bq, aq, g, epi, no_fusion, tail, (int)out_stride, N, \
-                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, tile_magic(p.tiles_n), (int32_t*)0, (unsigned*)0)
+                       p.tiles_m, p.tiles_n, 1, p.steps_per_split, tile_magic(p.tiles_n), (int32_t*)0, (unsigned*)0, (const float*)0, 0)
     if (p.bm == 128 && p.bn == 256)
         LAUNCH_GEMM(128, 256);
     else if (p.bm == 128 && p.bn == 128)
@@ -830,10 +1229,10 @@ int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int
     {                                                                                                                                                    \
         if (p.splits > 1)                                                                                                                                \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, true, false, 1>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,     \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters);                       \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters, (const float*)0, 0);   \
         else                                                                                                                                             \
             hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<64, BN_, 3, false, false, 1>), grid, block, 0, stream, weight, x, g, epi, no_fusion, no_gemm,    \
-                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters);                       \
+                               (int)out_stride, num_output, p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters, (const float*)0, 0);   \
     } while (0)
     if (p.bm != 64)
     {

@@ -83,6 +83,9 @@ _SIGNATURES = {
     "ncnnhip_conv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_int,
                                C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_conv_fusion_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_from_float_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_int8_nhwc_from_float": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p,
+                                          C.POINTER(ConvFusion), C.c_void_p],
     "ncnnhip_conv_int8_nhwc_fused": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.POINTER(ConvFusion), C.c_void_p,
                                      C.c_size_t, C.c_void_p],
     "ncnnhip_conv_resolved_pads": [C.POINTER(ConvDesc), C.POINTER(C.c_int), C.POINTER(C.c_int)],
@@ -432,10 +435,11 @@ class Runtime:
 
     def conv_channels_last(self, x, weight, bias, w_scales, in_scales, top_scales, num_output, kernel, dilation=(1, 1), stride=(1, 1),
                            pads=(0, 0, 0, 0), pad_value=0.0, group=1, term=1, act=0, act_params=(0.0, 0.0), residual=None, relu_after=False,
-                           quantise_scale=None, stem=False):
+                           quantise_scale=None, stem=False, from_float=None):
         """Convolution (group 1) or depthwise (group == c == num_output) entirely on channels-last device blobs:
         upload+convert, quantise if fp32, kernel writing channels-last, convert back.  x is [n][c][h][w].
-        stem=True: the narrow-input form (at most 4 input channels, 4-byte pixels with a physical border)."""
+        stem=True: the narrow-input form (at most 4 input channels, 4-byte pixels with a physical border).
+        from_float=np.float32 / np.float16: one launch, the fp32 / fp16 blob quantised inside the kernel."""
         x = np.ascontiguousarray(x)
         if x.ndim == 3:
             x = x[None]
@@ -449,6 +453,40 @@ class Runtime:
         in_scales = np.atleast_1d(np.asarray(in_scales, np.float32))
         scale_in = self.fold_input_scales(w_scales, in_scales, num_output)
         requant = term > 100
+        if from_float is not None:
+            if not lib().ncnnhip_conv_from_float_supported(C.byref(d)):
+                raise ValueError("this layer keeps its separate Quantize pass")
+            if np.dtype(from_float) == np.float32:
+                src = self.to_channels_last(x.astype(np.float32))
+            else:  # fp16: the layout change on the host (the device converter moves 1- and 4-byte values)
+                cp = lib().ncnnhip_padded_channels(c)
+                xh = np.zeros((n, h * w, cp), np.float16)
+                xh[:, :, :c] = x.astype(np.float16).reshape(n, c, h * w).transpose(0, 2, 1)
+                src = self.up(xh)
+            dsi, db = self.up(scale_in), self.up(None if bias is None else np.asarray(bias, np.float32))
+            dso = None
+            if requant:
+                ts = np.atleast_1d(np.asarray(top_scales, np.float32))
+                dso = self.up(np.repeat(ts, num_output // ts.size).astype(np.float32))
+            pk_bytes = C.c_size_t()
+            check(lib().ncnnhip_conv_nhwc_sizes(C.byref(d), None, C.byref(pk_bytes), None))
+            pk = np.empty(pk_bytes.value, np.int8)
+            check(lib().ncnnhip_conv_pack_weights(C.byref(d), np.ascontiguousarray(weight, np.int8).ctypes.data, pk.ctypes.data))
+            dpk, dscale = self.up(pk), self.up(in_scales[:1])
+            ocp = lib().ncnnhip_padded_channels(num_output)
+            dout = DeviceBuffer.empty((n, oh * ow, ocp), np.int8 if requant else np.float32)
+            fused = residual is not None or relu_after or quantise_scale is not None
+            dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))
+            dq8 = None if quantise_scale is None else DeviceBuffer.empty((n, oh * ow, ocp), np.int8)
+            fu = ConvFusion(_ptr(dres), int(relu_after), _ptr(dq8), float(quantise_scale or 0.0))
+            check(lib().ncnnhip_conv_int8_nhwc_from_float(C.byref(d), src.ptr, np.dtype(from_float).itemsize, dscale.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso),
+                                                          Activation.make(act, act_params), dout.ptr, C.byref(fu) if fused else None, self.stream))
+            raw = dout.to_numpy(self.stream)
+            assert not raw[:, :, num_output:].any(), "pad channels of a channels-last blob must be zero"
+            if fused:
+                q8 = None if dq8 is None else self.from_channels_last(dq8, n, num_output, oh, ow)
+                return self.from_channels_last(dout, n, num_output, oh, ow), q8
+            return self.from_channels_last(dout, n, num_output, oh, ow)
         src = self.to_channels_last(x)
         if stem:
             if not lib().ncnnhip_conv_stem_supported(C.byref(d)):

@@ -524,6 +524,27 @@ int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* resid
     const int8_t* xq = (const int8_t*)bottom.data;
     if (bottom.elemsize == 4u && bottom.q8 && !bottom.q8->empty() && bottom.q8_scale == bottom_blob_int8_scales[0] && bottom.q8->count() == bottom.count())
         xq = (const int8_t*)bottom.q8->data; // the producer's epilogue already quantised this blob with our scale
+    else if (bottom.elemsize == 4u && group == 1 && ncnnhip_conv_from_float_supported(&desc))
+    {
+        // one launch: the kernel's loader quantises the fp32 blob on its way into LDS
+        ncnnhip_conv_fusion fu;
+        fu.residual_dev = residual ? (const float*)residual->data : 0;
+        fu.relu_after = relu ? 1 : 0;
+        fu.quantised_out_dev = 0;
+        fu.quantise_scale = q8_scale;
+        if (q8_scale != 0.f)
+        {
+            top.q8.reset(new HipMat);
+            top.q8->create(outw, outh, num_output, 1u, bottom.n, &cmd);
+            if (top.q8->empty()) return -100;
+            top.q8_scale = q8_scale;
+            fu.quantised_out_dev = (int8_t*)top.q8->data;
+        }
+        rc = ncnnhip_conv_int8_nhwc_from_float(&desc, bottom.data, 4, (const float*)d_input_scales, (const int8_t*)d_weight_packed, (const float*)d_scale_in,
+                                               (const float*)d_bias, requant ? scale_out_table : 0, make_activation(activation_type, activation_params), top.data,
+                                               fused ? &fu : 0, st);
+        return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc_from_float");
+    }
     else if (bottom.elemsize == 4u)
     {
         void* q = scratch.get(bottom.count());

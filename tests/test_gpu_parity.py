@@ -316,6 +316,63 @@ def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pad
         assert got.min() >= 0
 
 
+@pytest.mark.parametrize("name,c,h,w,outc,kernel,stride,pads,term,act,batch", [
+    ("single-layer config 3x3 64->64 @56", 64, 56, 56, 64, (3, 3), (1, 1), (1, 1, 1, 1), 1, 1, 1),
+    ("same, batch 3, requantised output", 64, 20, 20, 64, (3, 3), (1, 1), (1, 1, 1, 1), 101, 3, 3),
+    ("1x1 256->128 @28 (rows are the pixels themselves)", 256, 28, 28, 128, (1, 1), (1, 1), (0, 0, 0, 0), 2, 0, 2),
+    ("1x1/2 96->100 @28 (channel tails on both sides)", 96, 28, 28, 100, (1, 1), (2, 2), (0, 0, 0, 0), 1, 2, 1),
+    ("3x3/2 20->48 @33 SAME_UPPER (20 channels in 32)", 20, 33, 33, 48, (3, 3), (2, 2), (-233, -233, -233, -233), 1, 1, 2),
+    ("5x3 dilated 16->64 @40x30", 16, 30, 40, 64, (5, 3), (1, 1), (4, 4, 2, 2), 1, 0, 1),
+])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+def test_convolution_one_launch_from_float_blob(rt, name, c, h, w, outc, kernel, stride, pads, term, act, batch, dtype):
+    """The layer's Quantize pass inside the convolution kernel (fp32 and fp16 blobs): every output bit for bit the oracle's
+    quantise-then-convolve, including inputs that meet float2int8's ties and the out-of-range rule."""
+    _say("conv from float", name, np.dtype(dtype).name)
+    dil = (2, 2) if "dilated" in name else (1, 1)
+    x, wq, b, ws, ins, tops = cases.conv_case(len(name) + batch, c, h, w, outc, kernel, 1, term, True, False, batch=batch)
+    x = x.astype(dtype).astype(F)  # the values the device will see
+    edge = np.array([0.5, -0.5, 1.5, -2.5, 126.5, -126.5, 127.49, 300.0, -300.0, 0.49999997, -0.49999997], F) / ins[0]
+    x.reshape(-1)[: edge.size] = edge.astype(dtype).astype(F)
+    if dtype == np.float32:
+        x.reshape(-1)[edge.size: edge.size + 4] = [np.inf, -np.inf, np.nan, 3e38]
+    ap = (0.1, 0.0) if act == 2 else (0.0, 6.0)
+    d = oracle.make_desc((c, h, w), outc, kernel, dil, stride, pads, 0.0, 1, 1, term, act, ap)
+    want = np.stack([oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None if tops is None else tops[0]) for i in range(batch)])
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, dil, stride, pads, 0.0, 1, term, act, ap, from_float=dtype)
+    assert np.array_equal(got, want, equal_nan=True)
+
+
+def test_convolution_one_launch_from_float_blob_with_the_fused_tail(rt):
+    c, hw, outc = 64, 14, 64
+    x, wq, b, ws, ins, tops = cases.conv_case(5, c, hw, hw, outc, (3, 3), 1, 1, True, False, batch=2)
+    rng = np.random.default_rng(6)
+    res = rng.uniform(-1, 1, (2, outc, hw, hw)).astype(F)
+    d = oracle.make_desc((c, hw, hw), outc, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 1, 1, 1, 0, (0.0, 0.0))
+    conv = np.stack([oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None) for i in range(2)])
+    want = np.maximum(conv + res, 0).astype(F)
+    q_scale = F(9.5)
+    want_q = oracle.quantize(want.reshape(2 * outc, -1), [q_scale]).reshape(want.shape)
+    got, got_q = rt.conv_channels_last(x, wq, b, ws, ins, None, outc, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 0.0, 1, 1, 0, (0.0, 0.0),
+                                       residual=res, relu_after=True, quantise_scale=q_scale, from_float=np.float32)
+    assert np.array_equal(got, want) and np.array_equal(got_q, want_q)
+
+
+def test_convolution_from_float_refuses_what_needs_its_own_quantize_pass(rt):
+    import ctypes as C
+    import ncnn_amd
+    from ncnn_amd.hip import ConvDesc, lib
+    # K split over workgroups (512 -> 512 3x3 on 7x7), a non-zero border value, a tile beyond the LDS budget
+    split = ConvDesc(7, 7, 512, 1, 512, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 1)
+    border = ConvDesc(56, 56, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 3.0, 1)
+    deep = ConvDesc(56, 56, 2048, 1, 64, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0.0, 1)
+    ok = ConvDesc(56, 56, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 1)
+    assert [lib().ncnnhip_conv_from_float_supported(C.byref(d)) for d in (split, border, deep, ok)] == [0, 0, 0, 1]
+    x, wq, b, ws, ins, tops = cases.conv_case(1, 512, 7, 7, 512, (3, 3), 1, 1, True, False)
+    with pytest.raises(ValueError):
+        rt.conv_channels_last(x, wq, b, ws, ins, None, 512, (3, 3), pads=(1, 1, 1, 1), from_float=np.float32)
+
+
 def test_convolution_batch_equals_per_sample_loop(rt):
     # ncnn runs a batch as a per-sample loop (src/net.cpp:654-700); the folded launch must match it
     x, wq, b, ws, ins, tops = cases.conv_case(77, 16, 14, 14, 40, (3, 3), 1, 101, True, False, batch=3)
