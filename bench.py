@@ -637,9 +637,13 @@ def bench_conv(args, spec):
         conv()
 
     def one_launch():  # the Quantize pass inside the convolution's loader
-        check(lib.ncnnhip_conv_int8_nhwc_from_float(C.byref(desc), d_x.ptr, 4, d_s.ptr, d_pk.ptr, d_si.ptr, d_b.ptr, None, act, d_out.ptr, None, st))
+        check(lib.ncnnhip_conv_int8_nhwc_from_float(C.byref(desc), d_x.ptr, 4, d_s.ptr, d_pk.ptr, d_si.ptr, d_b.ptr, None, act, d_out.ptr, None, d_fws.ptr, fws.value, st))
 
     fused_quantise = bool(lib.ncnnhip_conv_from_float_supported(C.byref(desc)))
+    fws = C.c_size_t(0)
+    if fused_quantise:
+        check(lib.ncnnhip_conv_from_float_workspace_bytes(C.byref(desc), C.byref(fws)))
+    d_fws = ncnn_amd.DeviceBuffer.zeros(fws.value, st)
     step = one_launch if fused_quantise else two_launches
     kernel = one_launch if fused_quantise else conv
 

@@ -168,13 +168,18 @@ int ncnnhip_conv_int8_nhwc_fused(const ncnnhip_conv_desc* desc, const int8_t* nh
  * layer's own Quantize pass (Quantize::forward, src/layer/quantize.cpp:48-111 as Convolution::forward_int8 calls it at
  * src/layer/convolution.cpp:392-405: q = float2int8(x * in_scale[0])) runs inside the kernel's loader, so the int8 copy of
  * the blob is never written.  Group 1, zero border value, channels-last output (fp32, or int8 when scale_out_dev is
- * given); fusion (may be NULL) as in ncnnhip_conv_int8_nhwc_fused.  Layers whose K the plan would split over workgroups,
- * or whose tile (64 pixels and up to 128 channels, all of K) exceeds 96 KiB of LDS, are refused: ask ncnnhip_conv_from_float_supported first and
- * keep the separate ncnnhip_quantize_nhwc + ncnnhip_conv_int8_nhwc for those.  Needs no workspace. */
+ * given); fusion (may be NULL) as in ncnnhip_conv_int8_nhwc_fused.  A workgroup holds its share of both operands in LDS
+ * (64 pixels and up to 128 channels times its K steps, at most 96 KiB); layers beyond that are refused: ask
+ * ncnnhip_conv_from_float_supported first and keep the separate ncnnhip_quantize_nhwc + ncnnhip_conv_int8_nhwc for those.
+ * Layers with few output tiles split K over workgroups and need a workspace of ncnnhip_conv_from_float_workspace_bytes
+ * (0 for the others), under the contract of ncnnhip_conv_int8_nhwc's workspace: zero-filled once by the caller, left
+ * zero by every launch, used by one launch at a time. */
 int ncnnhip_conv_from_float_supported(const ncnnhip_conv_desc* desc);
+int ncnnhip_conv_from_float_workspace_bytes(const ncnnhip_conv_desc* desc, size_t* workspace_bytes);
 int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, const float* in_scale_dev,
                                       const int8_t* packed_weight_dev, const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev,
-                                      ncnnhip_activation act, void* out_nhwc_dev, const ncnnhip_conv_fusion* fusion, void* stream);
+                                      ncnnhip_activation act, void* out_nhwc_dev, const ncnnhip_conv_fusion* fusion, void* workspace_dev,
+                                      size_t workspace_bytes, void* stream);
 
 
 /* Convolution::forward_int8 (src/layer/convolution.cpp:383-508) for layers with at most 4 input channels (the 3-channel

@@ -61,9 +61,12 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g, const int8_t* wpk, const int8_
 // The 1x1 small-K int8-output kernel (conv_pointwise.hip): does this problem fit it, and its launch.  The pipelined
 // launch asks first.
 // One launch for a layer whose input is still fp32 (x_elemsize 4) or fp16 (2): quantised with x_scale[0] inside the kernel.
+// Layers with few tiles split K over workgroups and need the workspace of conv_nhwc_staged_workspace_bytes (same contract
+// as the other channels-last convolutions: zero when handed over, left zero).
 bool conv_nhwc_staged_supported(const NhwcGeom& g);
+size_t conv_nhwc_staged_workspace_bytes(const NhwcGeom& g);
 int launch_conv_nhwc_staged(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
-                            const ConvFusion& fusion, int out_cp, hipStream_t stream);
+                            const ConvFusion& fusion, int out_cp, void* workspace, size_t workspace_bytes, hipStream_t stream);
 bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
 int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream);
 

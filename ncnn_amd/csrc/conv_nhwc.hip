@@ -582,7 +582,7 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const void* nhwc_d
     if (x_elemsize != 1)
     {
         NCNNHIP_REQUIRE(clast && x_scale_dev, "ncnnhip_conv_int8_nhwc_from_float: needs channels-last output and the input scale");
-        return launch_conv_nhwc_staged(g, packed_weight_dev, nhwc_dev, x_elemsize, x_scale_dev, epi, fusion, out_cp, st);
+        return launch_conv_nhwc_staged(g, packed_weight_dev, nhwc_dev, x_elemsize, x_scale_dev, epi, fusion, out_cp, workspace_dev, workspace_bytes, st);
     }
     const int8_t* xq = static_cast<const int8_t*>(nhwc_dev);
     // zero border and channels-last output: the pipelined kernel
@@ -668,9 +668,22 @@ int ncnnhip_conv_from_float_supported(const ncnnhip_conv_desc* desc)
     return conv_nhwc_staged_supported(nhwc_geometry(*desc, outw, outh, npix)) ? 1 : 0;
 }
 
+int ncnnhip_conv_from_float_workspace_bytes(const ncnnhip_conv_desc* desc, size_t* workspace_bytes)
+{
+    NCNNHIP_REQUIRE(workspace_bytes, "ncnnhip_conv_from_float_workspace_bytes: null pointer");
+    *workspace_bytes = 0;
+    NCNNHIP_REQUIRE(ncnnhip_conv_from_float_supported(desc), "ncnnhip_conv_from_float_workspace_bytes: this layer needs its separate Quantize pass");
+    int outw = 0, outh = 0;
+    int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
+    if (ret) return ret;
+    *workspace_bytes = conv_nhwc_staged_workspace_bytes(nhwc_geometry(*desc, outw, outh, (long long)outw * outh * desc->batch));
+    return NCNNHIP_OK;
+}
+
 int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void* nhwc_dev, int elemsize, const float* in_scale_dev,
                                       const int8_t* packed_weight_dev, const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev,
-                                      ncnnhip_activation act, void* out_dev, const ncnnhip_conv_fusion* fusion, void* stream)
+                                      ncnnhip_activation act, void* out_dev, const ncnnhip_conv_fusion* fusion, void* workspace_dev, size_t workspace_bytes,
+                                      void* stream)
 {
     NCNNHIP_REQUIRE(elemsize == 4 || elemsize == 2, "ncnnhip_conv_int8_nhwc_from_float: activations are fp32 (4) or fp16 (2), not %d bytes", elemsize);
     NCNNHIP_REQUIRE(ncnnhip_conv_from_float_supported(desc), "ncnnhip_conv_int8_nhwc_from_float: this layer needs its separate Quantize pass");
@@ -686,7 +699,7 @@ int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void*
         f.q8_scale = fusion->quantise_scale;
     }
     return conv_int8_nhwc_impl(desc, nhwc_dev, elemsize, in_scale_dev, packed_weight_dev, scale_in_dev, bias_dev, scale_out_dev, act, out_dev, NCNNHIP_CHANNELS_LAST,
-                               0, 0, f, 0, 0, stream);
+                               0, 0, f, workspace_dev, workspace_bytes, stream);
 }
 
 int ncnnhip_conv_stem_supported(const ncnnhip_conv_desc* desc)

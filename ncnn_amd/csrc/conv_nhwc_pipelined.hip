@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 {
     constexpr bool dense = MODE == 1;
     constexpr bool STAGED = AIN != 1;
-    static_assert(!STAGED || (!SPLITK && !GEMM && MODE != 2), "the quantising loader exists for whole-K convolution tiles");
+    static_assert(!STAGED || (!GEMM && MODE != 2), "the quantising loader exists for convolutions on ordinary blobs");
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LAR = BM / 64;              // 64-row groups of the activation tile
     constexpr int LA = STAGED ? 0 : LAR, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     int step_end = SPLITK ? step_begin + steps_per_split : total_steps;
     if (step_end > total_steps) step_end = total_steps;
     const int nk = step_end - step_begin;
+    const int tile_steps = SPLITK ? steps_per_split : total_steps; // K steps the quantising loader's LDS regions are sized for
     if (!SPLITK && nk <= 0) return; // (a split workgroup always has steps, and must reach the tile counter in any case)
 
     // ---- sources of this lane's loads.  Load i of a wavefront fills LDS rows i*64 + wave*16 .. +16 of the operand;
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
     auto issue = [&](int s) {
         // quantising loader: every step has its own place (written once); the address below is that place minus the
         // activation part a ring stage would start with
-        int8_t* stage = STAGED ? a_tile + total_steps * (BM * 64) + s * (BN * 64) - BM * 64 + wave * 1024 : smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
+        int8_t* stage = STAGED ? a_tile + tile_steps * (BM * 64) + s * (BN * 64) - BM * 64 + wave * 1024 : smem + (s % STAGES) * STAGE_BYTES + wave * 1024;
         if (dense)
         {
             // one tap, no border: the row's pixel exists or it does not (a_iy0 is 0 or hugely negative)
@@ -321,12 +322,24 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
             // first and last input pixel of the tile: a wavefront reduction, then the four wavefronts' results through LDS
             __shared__ int run[4][2];
             int first = 0x7fffffff, last = -0x7fffffff;
+            // taps this workgroup's K steps cover (all of them unless K is split); a tap's offset from the first one grows
+            // with its index (the launch checks dh * W > (kw - 1) * dw), so the first and the last tap bound the run
+            int tap_lo = 0, tap_hi = g.ntaps - 1;
+            if (SPLITK)
+            {
+                tap_lo = (step_begin * 64) / g.tapK;
+                const int t_hi = (step_end * 64 - 1) / g.tapK;
+                tap_hi = t_hi < tap_hi ? t_hi : tap_hi;
+                if (tap_lo > tap_hi) tap_lo = tap_hi; // a range that lies in the round-up of K: nothing is looked up
+            }
+            const int off_lo = (tap_lo / g.kw) * g.dh * g.W + (tap_lo % g.kw) * g.dw;
+            const int off_hi = (tap_hi / g.kw) * g.dh * g.W + (tap_hi % g.kw) * g.dw;
 #pragma unroll
             for (int i = 0; i < LAR; i++)
                 if (a_iy0[i] > -0x40000000) // the row is a real output pixel
                 {
-                    const int f = a_img0[i] + a_iy0[i] * g.W + a_ix0[i];
-                    const int l = f + (g.kh - 1) * g.dh * g.W + (g.kw - 1) * g.dw;
+                    const int f0 = a_img0[i] + a_iy0[i] * g.W + a_ix0[i];
+                    const int f = f0 + off_lo, l = f0 + off_hi;
                     first = f < first ? f : first;
                     last = l > last ? l : last;
                 }
@@ -357,7 +370,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
             if (count > 0 && (long long)count * g.Cp <= (long long)a_cache_bytes)
             {
                 cached = true;
-                int8_t* cache = a_tile + total_steps * ((BM + BN) * 64);
+                int8_t* cache = a_tile + tile_steps * ((BM + BN) * 64);
                 // 4 values per lane and load: a wavefront instruction reads 1 KiB (fp32) or 512 B (fp16) of consecutive addresses
                 const int nquad = count * (g.Cp >> 2);
                 const int8_t* src0 = x + (size_t)lo * g.Cp * AIN;
@@ -404,7 +417,11 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 {
                     // a K step lies inside one tap, the same for every lane: its position is wavefront-uniform arithmetic
                     const int chunk_byte = ld_chunk * 16;
-                    int stap = 0, sq0 = 0, sky = 0, skx = 0; // (the tile starts at K = 0: this loader is never split over workgroups)
+                    // position of the workgroup's first K step
+                    int stap = (step_begin * 64) / g.tapK;
+                    int sq0 = step_begin * 64 - stap * g.tapK;
+                    int sky = stap / g.kw;
+                    int skx = stap - sky * g.kw;
                     for (int s0 = 0; s0 < nk; s0 += GATHER)
                     {
                         v4i piece[GATHER][LAR];
@@ -600,7 +617,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
             __builtin_amdgcn_s_barrier();
         }
         // (quantising loader: step t's weights at their own place, see issue())
-        const unsigned st = STAGED ? a_tile_lds + (unsigned)(total_steps * (BM * 64) + t * (BN * 64) - BM * 64) : lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
+        const unsigned st = STAGED ? a_tile_lds + (unsigned)(tile_steps * (BM * 64) + t * (BN * 64) - BM * 64) : lds_base + (unsigned)((t % STAGES) * STAGE_BYTES);
         // fragment reads of both K halves go out first; the address arithmetic and the global loads of the stage
         // refilled next are issued while they are in flight
         v4i fa[2][TM], fb[2][TN];
@@ -1052,12 +1069,18 @@ static bool staged_plan(const NhwcGeom& g_in, NhwcGeom& g, PipePlan& p, int& mod
         g.H = g.outh = 1;
         g.W = g.outw = g.npix;
     }
-    p = plan_pipelined(g.cout, g.npix, g.K / 64);
+    const int steps = g.K / 64;
+    p = plan_pipelined(g.cout, g.npix, steps);
     mode = dense ? 1 : 0;
-    // whole-K tiles of 64 pixels only: a layer the plan would split over workgroups keeps its separate Quantize pass
-    return p.splits == 1 && p.bm == 64 && p.bn <= 128 && (size_t)g.K * (64 + p.bn) <= STAGED_TILE_LIMIT && g.K / 64 * (p.bn / 64) <= 48 && g.pad_word == 0 &&
-           g.tapK == g.Cp &&
-           (long long)p.tiles_m * p.tiles_n * p.tiles_n < (1ll << 32);
+    // (K is split over workgroups exactly where the plan splits it for an int8 blob.  Splitting shorter K loops as well
+    // -- three steps per workgroup for a 3x3 64 -> 64 layer on 56x56, 147 workgroups instead of 49 -- was measured: the
+    // hand-off through memory costs more than the shorter loader saves, 10.7 us against 8.6.)
+    const int wg_steps = p.splits > 1 ? p.steps_per_split : steps;
+    // 64-pixel tiles; the workgroup's share of both operands in LDS; at most 48 weight loads in flight per lane (the
+    // counter holds 63); zero border; tap offsets that grow with the tap index (the cached run is bounded by the first and last tap)
+    return p.bm == 64 && p.bn <= 128 && (size_t)wg_steps * 64 * (64 + p.bn) <= STAGED_TILE_LIMIT && wg_steps * (p.bn / 64) <= 48 && g.pad_word == 0 &&
+           g.tapK == g.Cp && (dense || (long long)g.dh * g.W > (long long)(g.kw - 1) * g.dw) &&
+           (long long)p.tiles_m * p.tiles_n * p.splits * p.tiles_n < (1ll << 32);
 }
 
 bool conv_nhwc_staged_supported(const NhwcGeom& g_in)
@@ -1068,16 +1091,35 @@ bool conv_nhwc_staged_supported(const NhwcGeom& g_in)
     return staged_plan(g_in, g, p, mode);
 }
 
+size_t conv_nhwc_staged_workspace_bytes(const NhwcGeom& g_in)
+{
+    NhwcGeom g;
+    PipePlan p;
+    int mode;
+    if (!staged_plan(g_in, g, p, mode) || p.splits <= 1) return 0;
+    return SPLIT_COUNTER_BYTES + (size_t)p.splits * p.tiles_m * p.tiles_n * p.bm * p.bn * sizeof(int32_t);
+}
+
 int launch_conv_nhwc_staged(const NhwcGeom& g_in, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
-                            const ConvFusion& fusion, int out_cp, hipStream_t stream)
+                            const ConvFusion& fusion, int out_cp, void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
     NhwcGeom g;
     PipePlan p;
     int mode;
     NCNNHIP_REQUIRE(x_elemsize == 4 || x_elemsize == 2, "convolution: activations of %d bytes per value", x_elemsize);
     NCNNHIP_REQUIRE(staged_plan(g_in, g, p, mode), "convolution: this layer does not fit the one-launch form (ask ncnnhip_conv_from_float_supported first)");
-    const size_t tile_bytes = (size_t)g.K * (64 + p.bn);
-    // Behind the tile, a cache for the run of input pixels a tile touches (quantised once instead of once per tap): 64
+    const int wg_steps = p.splits > 1 ? p.steps_per_split : g.K / 64;
+    const size_t tile_bytes = (size_t)wg_steps * 64 * (64 + p.bn);
+    int32_t* partial = 0;
+    unsigned* counters = 0;
+    if (p.splits > 1)
+    {
+        const size_t need = SPLIT_COUNTER_BYTES + (size_t)p.splits * p.tiles_m * p.tiles_n * p.bm * p.bn * sizeof(int32_t);
+        NCNNHIP_REQUIRE(workspace && workspace_bytes >= need, "convolution: workspace of %zu bytes required", need);
+        counters = (unsigned*)workspace; // zero on entry (the caller cleared the workspace once), zero again on exit
+        partial = (int32_t*)((char*)workspace + SPLIT_COUNTER_BYTES);
+    }
+    // Behind the operands, a cache for the run of input pixels a tile touches (quantised once instead of once per tap): 64
     // consecutive output pixels span at most (63 / outw + 2) output rows, one more image-to-image gap of at most
     // (H + pad) rows, and the kernel's own extent.  An estimate only: the kernel measures each tile's run and gathers
     // from global memory when it does not fit.
@@ -1089,27 +1131,31 @@ int launch_conv_nhwc_staged(const NhwcGeom& g_in, const int8_t* wpk, const void*
         const size_t room = STAGED_LDS_LIMIT - tile_bytes;
         cache_bytes = (size_t)std::min<long long>(pixels * g.Cp, (long long)room) & ~(size_t)15;
     }
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits)), block(256);
     const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
     const int8_t* xb = static_cast<const int8_t*>(x);
-#define LAUNCH_STAGED(BN_, MODE_, AIN_)                                                                                                                      \
+#define LAUNCH_STAGED(BN_, SPLIT_, MODE_, AIN_)                                                                                                              \
     do                                                                                                                                                       \
     {                                                                                                                                                        \
-        auto kernel = conv_nhwc_pipelined_kernel<64, BN_, 3, false, false, MODE_, AIN_>;                                                                     \
+        auto kernel = conv_nhwc_pipelined_kernel<64, BN_, 3, SPLIT_, false, MODE_, AIN_>;                                                                    \
         static std::once_flag once;                                                                                                                          \
         static hipError_t attr = hipSuccess;                                                                                                                 \
         std::call_once(once, [&]() { attr = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)STAGED_LDS_LIMIT); });  \
         NCNNHIP_CHECK(attr);                                                                                                                                 \
         hipLaunchKernelGGL(kernel, grid, block, tile_bytes + cache_bytes, stream, wpk, xb, g, epi, fusion, no_gemm, out_cp, out_cp, p.tiles_m, p.tiles_n, \
-                           1, p.steps_per_split, tile_magic(p.tiles_n), (int32_t*)0, (unsigned*)0, x_scale, (int)cache_bytes);                              \
+                           p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters, x_scale, (int)cache_bytes);                               \
     } while (0)
-#define LAUNCH_STAGED_IN(BN_, MODE_)        \
-    do                                      \
-    {                                       \
-        if (x_elemsize == 4)                \
-            LAUNCH_STAGED(BN_, MODE_, 4);   \
-        else                                \
-            LAUNCH_STAGED(BN_, MODE_, 2);   \
+#define LAUNCH_STAGED_IN(BN_, MODE_)                 \
+    do                                               \
+    {                                                \
+        if (x_elemsize == 4 && p.splits > 1)         \
+            LAUNCH_STAGED(BN_, true, MODE_, 4);      \
+        else if (x_elemsize == 4)                    \
+            LAUNCH_STAGED(BN_, false, MODE_, 4);     \
+        else if (p.splits > 1)                       \
+            LAUNCH_STAGED(BN_, true, MODE_, 2);      \
+        else                                         \
+            LAUNCH_STAGED(BN_, false, MODE_, 2);     \
     } while (0)
     if (p.bn == 128 && mode == 1)
         LAUNCH_STAGED_IN(128, 1);

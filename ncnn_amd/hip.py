@@ -84,8 +84,9 @@ _SIGNATURES = {
                                C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_conv_fusion_supported": [C.POINTER(ConvDesc)],
     "ncnnhip_conv_from_float_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_from_float_workspace_bytes": [C.POINTER(ConvDesc), C.POINTER(C.c_size_t)],
     "ncnnhip_conv_int8_nhwc_from_float": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p,
-                                          C.POINTER(ConvFusion), C.c_void_p],
+                                          C.POINTER(ConvFusion), C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_conv_int8_nhwc_fused": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.POINTER(ConvFusion), C.c_void_p,
                                      C.c_size_t, C.c_void_p],
     "ncnnhip_conv_resolved_pads": [C.POINTER(ConvDesc), C.POINTER(C.c_int), C.POINTER(C.c_int)],
@@ -479,8 +480,12 @@ class Runtime:
             dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))
             dq8 = None if quantise_scale is None else DeviceBuffer.empty((n, oh * ow, ocp), np.int8)
             fu = ConvFusion(_ptr(dres), int(relu_after), _ptr(dq8), float(quantise_scale or 0.0))
-            check(lib().ncnnhip_conv_int8_nhwc_from_float(C.byref(d), src.ptr, np.dtype(from_float).itemsize, dscale.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso),
-                                                          Activation.make(act, act_params), dout.ptr, C.byref(fu) if fused else None, self.stream))
+            wsb = C.c_size_t()
+            check(lib().ncnnhip_conv_from_float_workspace_bytes(C.byref(d), C.byref(wsb)))
+            dws = DeviceBuffer.zeros(wsb.value, self.stream)
+            for _ in range(2):  # twice: the second launch finds the workspace as the first one left it
+                check(lib().ncnnhip_conv_int8_nhwc_from_float(C.byref(d), src.ptr, np.dtype(from_float).itemsize, dscale.ptr, dpk.ptr, dsi.ptr, _ptr(db), _ptr(dso),
+                                                              Activation.make(act, act_params), dout.ptr, C.byref(fu) if fused else None, dws.ptr, wsb.value, self.stream))
             raw = dout.to_numpy(self.stream)
             assert not raw[:, :, num_output:].any(), "pad channels of a channels-last blob must be zero"
             if fused:

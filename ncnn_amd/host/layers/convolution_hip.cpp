@@ -435,6 +435,19 @@ int Convolution_hip::forward_hip_requantised(const HipMat& bottom, float scale, 
     return forward_device(bottom, 0, false, 0.f, scale, top, cmd, opt);
 }
 
+// The one-launch form is taken where it measured faster than Quantize + convolution: every layer it accepts whose K
+// stays in one workgroup, and of those that split K over workgroups (few output tiles, long K) only the 1x1 stride-1
+// ones -- a 3x3 layer split nine ways quantises the same input pixels in nine workgroups (512 -> 512 on 7x7: 15.6 us
+// against 14.6 in two launches; 1024 -> 256 1x1 on 14x14: 10.1 against 10.9).
+static bool one_launch_from_float_pays(const ncnnhip_conv_desc& desc)
+{
+    if (!ncnnhip_conv_from_float_supported(&desc)) return false;
+    size_t workspace_bytes = 0;
+    if (ncnnhip_conv_from_float_workspace_bytes(&desc, &workspace_bytes) != 0) return false;
+    const bool pointwise = desc.kernel_w == 1 && desc.kernel_h == 1 && desc.stride_w == 1 && desc.stride_h == 1;
+    return workspace_bytes == 0 || pointwise;
+}
+
 int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* residual, bool relu, float q8_scale, float only_scale, HipMat& top, HipCommand& cmd,
                                     const Option& opt) const
 {
@@ -524,7 +537,7 @@ int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* resid
     const int8_t* xq = (const int8_t*)bottom.data;
     if (bottom.elemsize == 4u && bottom.q8 && !bottom.q8->empty() && bottom.q8_scale == bottom_blob_int8_scales[0] && bottom.q8->count() == bottom.count())
         xq = (const int8_t*)bottom.q8->data; // the producer's epilogue already quantised this blob with our scale
-    else if (bottom.elemsize == 4u && group == 1 && ncnnhip_conv_from_float_supported(&desc))
+    else if (bottom.elemsize == 4u && group == 1 && one_launch_from_float_pays(desc))
     {
         // one launch: the kernel's loader quantises the fp32 blob on its way into LDS
         ncnnhip_conv_fusion fu;
@@ -540,9 +553,14 @@ int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* resid
             top.q8_scale = q8_scale;
             fu.quantised_out_dev = (int8_t*)top.q8->data;
         }
+        size_t workspace_bytes = 0;
+        rc = ncnnhip_conv_from_float_workspace_bytes(&desc, &workspace_bytes);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_from_float_workspace_bytes");
+        void* ws = workspace_bytes ? cmd.zeroed_workspace(workspace_bytes) : 0;
+        if (workspace_bytes && !ws) return -100;
         rc = ncnnhip_conv_int8_nhwc_from_float(&desc, bottom.data, 4, (const float*)d_input_scales, (const int8_t*)d_weight_packed, (const float*)d_scale_in,
                                                (const float*)d_bias, requant ? scale_out_table : 0, make_activation(activation_type, activation_params), top.data,
-                                               fused ? &fu : 0, st);
+                                               fused ? &fu : 0, ws, workspace_bytes, st);
         return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc_from_float");
     }
     else if (bottom.elemsize == 4u)

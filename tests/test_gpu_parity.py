@@ -323,6 +323,9 @@ def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pad
     ("1x1/2 96->100 @28 (channel tails on both sides)", 96, 28, 28, 100, (1, 1), (2, 2), (0, 0, 0, 0), 1, 2, 1),
     ("3x3/2 20->48 @33 SAME_UPPER (20 channels in 32)", 20, 33, 33, 48, (3, 3), (2, 2), (-233, -233, -233, -233), 1, 1, 2),
     ("5x3 dilated 16->64 @40x30", 16, 30, 40, 64, (5, 3), (1, 1), (4, 4, 2, 2), 1, 0, 1),
+    ("3x3 512->512 @7 (K split over 9 workgroups per tile)", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 1, 1, 1),
+    ("3x3 64->96 @12 requantised, batch 2 (K split three ways, a partly filled last tile)", 64, 12, 12, 96, (3, 3), (1, 1), (1, 1, 1, 1), 101, 1, 2),
+    ("1x1 512->64 @9 (rows are the pixels, K split)", 512, 9, 9, 64, (1, 1), (1, 1), (0, 0, 0, 0), 1, 0, 1),
 ])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
 def test_convolution_one_launch_from_float_blob(rt, name, c, h, w, outc, kernel, stride, pads, term, act, batch, dtype):
@@ -362,15 +365,19 @@ def test_convolution_from_float_refuses_what_needs_its_own_quantize_pass(rt):
     import ctypes as C
     import ncnn_amd
     from ncnn_amd.hip import ConvDesc, lib
-    # K split over workgroups (512 -> 512 3x3 on 7x7), a non-zero border value, a tile beyond the LDS budget
-    split = ConvDesc(7, 7, 512, 1, 512, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 1)
+    # a non-zero border value, a workgroup's share of the operands beyond the LDS budget, a grouped layer
     border = ConvDesc(56, 56, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 3.0, 1)
-    deep = ConvDesc(56, 56, 2048, 1, 64, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0.0, 1)
+    deep = ConvDesc(112, 112, 2048, 1, 64, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0.0, 1)
+    grouped = ConvDesc(56, 56, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 2)
     ok = ConvDesc(56, 56, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 1)
-    assert [lib().ncnnhip_conv_from_float_supported(C.byref(d)) for d in (split, border, deep, ok)] == [0, 0, 0, 1]
-    x, wq, b, ws, ins, tops = cases.conv_case(1, 512, 7, 7, 512, (3, 3), 1, 1, True, False)
+    split = ConvDesc(7, 7, 512, 1, 512, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0.0, 1)
+    assert [lib().ncnnhip_conv_from_float_supported(C.byref(d)) for d in (border, deep, grouped, ok, split)] == [0, 0, 0, 1, 1]
+    need = C.c_size_t()
+    assert lib().ncnnhip_conv_from_float_workspace_bytes(C.byref(split), C.byref(need)) == 0 and need.value > 0
+    assert lib().ncnnhip_conv_from_float_workspace_bytes(C.byref(border), C.byref(need)) != 0
+    x, wq, b, ws, ins, tops = cases.conv_case(1, 64, 56, 56, 64, (3, 3), 1, 1, True, False)
     with pytest.raises(ValueError):
-        rt.conv_channels_last(x, wq, b, ws, ins, None, 512, (3, 3), pads=(1, 1, 1, 1), from_float=np.float32)
+        rt.conv_channels_last(x, wq, b, ws, ins, None, 64, (3, 3), pads=(1, 1, 1, 1), pad_value=3.0, from_float=np.float32)
 
 
 def test_convolution_batch_equals_per_sample_loop(rt):
