@@ -165,7 +165,9 @@ static int base_forward_inplace_n(const ncnn_layer_t layer, ncnn_mat_t* bottom_t
 {
     std::vector<Mat> blobs((size_t)n);
     for (int i = 0; i < n; i++) blobs[(size_t)i] = *(Mat*)bottom_top_blobs[i];
-    return L(layer)->Layer::forward_inplace(blobs, *(const Option*)opt);
+    int ret = L(layer)->Layer::forward_inplace(blobs, *(const Option*)opt);
+    for (int i = 0; i < n; i++) *(Mat*)bottom_top_blobs[i] = blobs[(size_t)i];
+    return ret;
 }
 
 // table entries of a layer that exists in C++ (ncnn_layer_create_by_type, ncnnhip_layer_create_by_type): its virtuals
@@ -217,6 +219,11 @@ static ncnn_layer_t wrap_real_layer(Layer* layer)
 {
     if (!layer) return 0;
     ncnn_layer_t h = (ncnn_layer_t)malloc(sizeof(struct __ncnn_layer_t));
+    if (!h)
+    {
+        delete layer;
+        return 0;
+    }
     h->pthis = (void*)layer;
     h->load_param = real_load_param;
     h->load_model = real_load_model;
@@ -321,6 +328,7 @@ void ncnn_paramdict_set_array(ncnn_paramdict_t pd, int id, const ncnn_mat_t v)
 ncnn_modelbin_t ncnn_modelbin_create_from_mat_array(const ncnn_mat_t* weights, int n)
 {
     ncnn_modelbin_t mb = (ncnn_modelbin_t)malloc(sizeof(struct __ncnn_modelbin_t));
+    if (!mb) return 0;
     mb->pthis = (void*)static_cast<ModelBin*>(new OwnedMatArrayModelBin(weights, n));
     mb->load_1d = modelbin_load_1d;
     mb->load_2d = modelbin_load_2d;
@@ -338,6 +346,7 @@ void ncnn_modelbin_destroy(ncnn_modelbin_t mb)
 ncnn_layer_t ncnn_layer_create(void)
 {
     ncnn_layer_t layer = (ncnn_layer_t)malloc(sizeof(struct __ncnn_layer_t));
+    if (!layer) return 0;
     layer->pthis = (void*)(new Layer_c_api(layer));
     layer->load_param = base_load_param;
     layer->load_model = base_load_model;
@@ -365,6 +374,7 @@ ncnn_layer_t ncnnhip_layer_create_by_type(const char* type)
 {
     using namespace ncnn_amd;
     Layer* layer = 0;
+    if (!type) return 0;
     if (strcmp(type, "Convolution") == 0) layer = Convolution_hip_creator(0);
     else if (strcmp(type, "ConvolutionDepthWise") == 0) layer = ConvolutionDepthWise_hip_creator(0);
     else if (strcmp(type, "InnerProduct") == 0) layer = InnerProduct_hip_creator(0);

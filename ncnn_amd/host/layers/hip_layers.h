@@ -140,6 +140,8 @@ public:
     virtual int create_pipeline(const ncnn::Option& opt);
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+    // the same on blobs that already lie in HBM (2-D blobs are dense there; a per-head mask arrives channels-last)
+    virtual int forward_hip(const std::vector<ncnn::HipMat>& bottom_blobs, std::vector<ncnn::HipMat>& top_blobs, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
 
 public:
     int embed_dim, num_heads, weight_data_size, kdim, vdim, attn_mask, kv_cache, quantize_term, weight_block_quantize;

@@ -44,6 +44,7 @@ MultiHeadAttention_hip::MultiHeadAttention_hip()
 {
     one_blob_only = false;
     support_inplace = false;
+    support_hip = true;
     weight_block_quantize = 0;
     memset(dev, 0, sizeof(dev));
 }
@@ -316,6 +317,155 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     }
     if (rc == 0) rc = ncnnhip_stream_synchronize(st);
     if (rc != 0) return to_ncnn_status(rc, "download");
+    if (kv_cache)
+    {
+        top_blobs[1] = k_out;
+        top_blobs[2] = v_out;
+    }
+    return 0;
+}
+
+// dense 2-D fp32 device blob of one sample
+static bool dense_2d_dev(const HipMat& m)
+{
+    return m.dims == 2 && m.elemsize == 4u && m.n == 1;
+}
+
+int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& /*opt*/) const
+{
+    if (!dev[0][0])
+    {
+        NCNN_LOGE("MultiHeadAttention %s: forward before create_pipeline", name.c_str());
+        return -1;
+    }
+    const int extra = (attn_mask ? 1 : 0) + (kv_cache ? 2 : 0);
+    const int n_qkv = (int)bottom_blobs.size() - extra;
+    if (n_qkv < 1 || n_qkv > 3 || (int)top_blobs.size() < (kv_cache ? 3 : 1))
+    {
+        NCNN_LOGE("MultiHeadAttention %s: %d bottom blobs do not fit attn_mask=%d kv_cache=%d", name.c_str(), (int)bottom_blobs.size(), attn_mask, kv_cache);
+        return -1;
+    }
+    const int k_i = n_qkv >= 2 ? 1 : 0, v_i = n_qkv == 3 ? 2 : k_i;
+    const HipMat& q_blob = bottom_blobs[0];
+    const HipMat& k_blob = bottom_blobs[(size_t)k_i];
+    const HipMat& v_blob = bottom_blobs[(size_t)v_i];
+    const HipMat mask_blob = attn_mask ? bottom_blobs[(size_t)n_qkv] : HipMat();
+    const HipMat cached_k = kv_cache ? bottom_blobs[(size_t)(n_qkv + (attn_mask ? 1 : 0))] : HipMat();
+    const HipMat cached_v = kv_cache ? bottom_blobs[(size_t)(n_qkv + (attn_mask ? 1 : 0) + 1)] : HipMat();
+    const bool self_attention = k_i == 0;
+
+    const int qdim = weight_data_size / embed_dim;
+    const int bits = att_bits(quantize_term), block = att_block(quantize_term);
+    const int head_dim = embed_dim / num_heads;
+    if (!dense_2d_dev(q_blob) || !dense_2d_dev(k_blob) || !dense_2d_dev(v_blob) || q_blob.w != qdim || k_blob.w != kdim || v_blob.w != vdim || k_blob.h != v_blob.h)
+    {
+        NCNN_LOGE("MultiHeadAttention %s: q/k/v must be 2-D fp32 blobs of widths %d/%d/%d", name.c_str(), qdim, kdim, vdim);
+        return -1;
+    }
+    const int src = q_blob.h, cur = k_blob.h;
+    const int past = (kv_cache && !cached_k.empty()) ? cached_k.w : 0;
+    const int dst = past > 0 ? (self_attention ? past + cur : past) : cur;
+    const bool reuse_cache = past > 0 && !self_attention; // keys and values are the cache as it is
+    if (past > 0 && (!dense_2d_dev(cached_k) || !dense_2d_dev(cached_v) || cached_k.h != embed_dim || cached_v.h != embed_dim || cached_v.w != past))
+    {
+        NCNN_LOGE("MultiHeadAttention %s: the cache blobs must be [%d][past] fp32", name.c_str(), embed_dim);
+        return -1;
+    }
+    ScopedScratch scratch(&cmd);
+    void* st = cmd.stream;
+    const size_t E = (size_t)embed_dim;
+    int rc = 0;
+
+    int mask_heads = 0;
+    const float* d_mask = 0;
+    if (attn_mask)
+    {
+        const bool ok2 = mask_blob.dims == 2 && mask_blob.w == dst && mask_blob.h == src;
+        const bool ok3 = mask_blob.dims == 3 && mask_blob.w == dst && mask_blob.h == src && mask_blob.c == num_heads;
+        if ((!ok2 && !ok3) || mask_blob.elemsize != 4u || mask_blob.n != 1)
+        {
+            NCNN_LOGE("MultiHeadAttention %s: the mask must be [%d][%d] or [%d][%d][%d] fp32", name.c_str(), src, dst, num_heads, src, dst);
+            return -1;
+        }
+        mask_heads = ok3 ? num_heads : 1;
+        d_mask = (const float*)mask_blob.data;
+        if (ok3)
+        {
+            // a 3-D blob lies channels-last in HBM; the attention kernel reads one [src][dst] plane per head
+            const size_t plane = (size_t)src * dst;
+            float* planar = (float*)scratch.get(plane * num_heads * 4);
+            if (!planar) return -100;
+            rc = ncnnhip_nhwc_to_chw(mask_blob.data, 4, num_heads, (int)plane, 1, planar, plane, plane * num_heads, st);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_nhwc_to_chw");
+            d_mask = planar;
+        }
+    }
+
+    HipMat& top = top_blobs[0];
+    top.create(qdim, src, 4u, 1, &cmd);
+    if (top.empty()) return -100;
+    HipMat k_out, v_out;
+    float* d_kt = 0;
+    float* d_vt = 0;
+    if (reuse_cache)
+    {
+        k_out = cached_k;
+        v_out = cached_v;
+        d_kt = (float*)cached_k.data;
+        d_vt = (float*)cached_v.data;
+    }
+    else if (kv_cache)
+    {
+        k_out.create(dst, embed_dim, 4u, 1, &cmd);
+        v_out.create(dst, embed_dim, 4u, 1, &cmd);
+        if (k_out.empty() || v_out.empty()) return -100;
+        d_kt = (float*)k_out.data;
+        d_vt = (float*)v_out.data;
+    }
+    else
+    {
+        d_kt = (float*)scratch.get(E * dst * 4);
+        d_vt = (float*)scratch.get(E * dst * 4);
+        if (!d_kt || !d_vt) return -100;
+    }
+    float* d_qa = (float*)scratch.get((size_t)src * E * 4);
+    float* d_ctx = (float*)scratch.get((size_t)src * E * 4);
+    if (!d_qa || !d_ctx) return -100;
+
+    rc = ncnnhip_gemm_blockquant((const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, (const uint8_t*)dev[0][0], bits, block, (const float*)dev[0][1],
+                                 (const float*)dev[0][2], (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
+    if (rc != 0) return to_ncnn_status(rc, "q projection");
+    if (!reuse_cache)
+    {
+        if (past > 0)
+        {
+            rc = ncnnhip_copy2d(d_kt, (size_t)dst * 4, cached_k.data, (size_t)past * 4, (size_t)past * 4, E, st);
+            if (rc == 0) rc = ncnnhip_copy2d(d_vt, (size_t)dst * 4, cached_v.data, (size_t)past * 4, (size_t)past * 4, E, st);
+            if (rc != 0) return to_ncnn_status(rc, "cache into keys/values");
+        }
+        const HipMat* in[2] = {&k_blob, &v_blob};
+        float* outT[2] = {d_kt, d_vt};
+        const int in_dim[2] = {kdim, vdim};
+        for (int t = 0; t < 2; t++)
+        {
+            float* d_aff = (float*)scratch.get((size_t)cur * E * 4);
+            if (!d_aff) return -100;
+            rc = ncnnhip_gemm_blockquant((const float*)in[t]->data, (size_t)in_dim[t], cur, embed_dim, in_dim[t], (const uint8_t*)dev[1 + t][0], bits, block,
+                                         (const float*)dev[1 + t][1], (const float*)dev[1 + t][2], (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
+            if (rc == 0) rc = ncnnhip_transpose_f32(d_aff, E, cur, embed_dim, outT[t] + past, (size_t)dst, st);
+            if (rc != 0) return to_ncnn_status(rc, "k/v projection");
+        }
+    }
+    size_t att_ws_bytes = 0;
+    rc = ncnnhip_attention_workspace_bytes(num_heads, head_dim, src, dst, &att_ws_bytes);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
+    void* att_ws = att_ws_bytes ? scratch.get(att_ws_bytes) : 0;
+    if (att_ws_bytes && !att_ws) return -100;
+    rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
+    rc = ncnnhip_gemm_blockquant(d_ctx, E, src, qdim, embed_dim, (const uint8_t*)dev[3][0], bits, block, (const float*)dev[3][1], (const float*)dev[3][2],
+                                 (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);
+    if (rc != 0) return to_ncnn_status(rc, "out projection");
     if (kv_cache)
     {
         top_blobs[1] = k_out;

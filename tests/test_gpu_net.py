@@ -369,10 +369,12 @@ def test_gemm_layer_block_quant(bits, block, insc, resident):
     assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
 
 
+@RESIDENT
 @pytest.mark.parametrize("spec", cases.MHA_CASES, ids=[str(c[0]) for c in cases.MHA_CASES])
-def test_multiheadattention_layer_block_quant(spec):
+def test_multiheadattention_layer_block_quant(spec, resident):
     """MultiHeadAttention with block-quantised weights through load_param / load_model / forward, against the oracle:
-    every arrangement of inputs the layer knows (self / cross attention, shared or per-head mask, cache in and out)."""
+    every arrangement of inputs the layer knows (self / cross attention, shared or per-head mask, cache in and out), on
+    host blobs and with every blob (the caches and the per-head mask included) resident in HBM."""
     case = cases.mha_case(*spec)
     seed, e, heads, qdim, kdim, vdim, src, cur, bits, block, insc, past, self_att, mask = spec
     term = bits * 100 + int(insc) * 10 + {32: 0, 64: 1, 128: 2}[block]
@@ -400,6 +402,7 @@ def test_multiheadattention_layer_block_quant(spec):
                               quantize_term=term))
     net = host.Net()
     assert net.register_attention_layer() == 0
+    net.set_use_hip_compute(resident)
     assert net.load_param_mem(mw.assemble_param(lines)) == 0
     assert net.load_model_mem(mw.mha_blockquant_weights(case["weights"])) == 0
     ex = net.create_extractor()
