@@ -199,6 +199,13 @@ int ncnnhip_hipmat_download(const ncnn_hipmat_t m, ncnn_mat_t* out);
 int ncnnhip_extractor_input_hipmat(ncnn_extractor_t ex, const char* name, const ncnn_hipmat_t m);
 int ncnnhip_extractor_extract_hipmat(ncnn_extractor_t ex, const char* name, ncnn_hipmat_t* out);
 int ncnnhip_extractor_synchronize(ncnn_extractor_t ex);
+/* Per-layer timing, the run-time form of the reference's NCNN_BENCHMARK build switch (src/net.cpp:145-180, printed by
+ * benchmark(), src/benchmark.cpp): while enabled, every layer the extractor runs is recorded (device layers between two
+ * events on its stream, host layers by the wall clock).  ncnnhip_extractor_layer_timing waits for the stream and writes one
+ * line per record, in execution order: "<layer index>\t<type>\t<name>\t<device|host>\t<milliseconds>\n"; `needed`
+ * (may be NULL) receives the size of the whole text with its terminator, text (may be NULL) at most `capacity` bytes. */
+void ncnnhip_extractor_set_layer_timing(ncnn_extractor_t ex, int enable);
+int ncnnhip_extractor_layer_timing(ncnn_extractor_t ex, char* text, size_t capacity, size_t* needed);
 
 /* A forward pass recorded once and replayed with one launch (the reference's GPU path records a VkCompute command buffer
  * and submits it, src/command.h:22-67).  record runs the pass from blob `input_name` (= input, resident) to `output_name`

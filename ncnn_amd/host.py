@@ -91,6 +91,7 @@ def lib():
             "ncnnhip_net_upload": (ci, [vp, vp, C.POINTER(vp)]), "ncnnhip_hipmat_destroy": (None, [vp]), "ncnnhip_hipmat_download": (ci, [vp, C.POINTER(vp)]),
             "ncnnhip_extractor_input_hipmat": (ci, [vp, C.c_char_p, vp]), "ncnnhip_extractor_extract_hipmat": (ci, [vp, C.c_char_p, C.POINTER(vp)]),
             "ncnnhip_extractor_synchronize": (ci, [vp]),
+            "ncnnhip_extractor_set_layer_timing": (None, [vp, ci]), "ncnnhip_extractor_layer_timing": (ci, [vp, C.c_char_p, cs, C.POINTER(cs)]),
             "ncnnhip_graph_record": (ci, [vp, C.c_char_p, vp, C.c_char_p, C.POINTER(vp)]), "ncnnhip_graph_update_input": (ci, [vp, vp]),
             "ncnnhip_graph_replay": (ci, [vp]), "ncnnhip_graph_synchronize": (ci, [vp]), "ncnnhip_graph_output": (ci, [vp, C.POINTER(vp)]),
             "ncnnhip_graph_release": (None, [vp]),
@@ -427,6 +428,22 @@ class Extractor:
 
     def synchronize(self):
         return lib().ncnnhip_extractor_synchronize(self.h_)
+
+    def set_layer_timing(self, enable=True):
+        lib().ncnnhip_extractor_set_layer_timing(self.h_, int(enable))
+
+    def layer_timing(self):
+        """[(layer index, type, name, 'device' | 'host', milliseconds)] of the layers run since timing was switched on."""
+        need = C.c_size_t()
+        if lib().ncnnhip_extractor_layer_timing(self.h_, None, 0, C.byref(need)) != 0:
+            raise RuntimeError("layer_timing failed")
+        buf = C.create_string_buffer(need.value)
+        lib().ncnnhip_extractor_layer_timing(self.h_, buf, need.value, None)
+        rows = []
+        for ln in buf.value.decode().splitlines():
+            i, t, n, where, ms = ln.split("\t")
+            rows.append((int(i), t, n, where, float(ms)))
+        return rows
 
     def extract(self, name):
         out = C.c_void_p()

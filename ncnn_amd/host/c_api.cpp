@@ -3,6 +3,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <string>
+#include <string.h>
+
 #include "layers/hip_layers.h"
 #include "layers/hip_support.h"
 #include "ncnn/datareader.h"
@@ -346,6 +349,31 @@ int ncnnhip_extractor_extract_hipmat(ncnn_extractor_t ex, const char* name, ncnn
     int ret = E(ex)->extract(name, *m);
     *out = (ncnn_hipmat_t)m;
     return ret;
+}
+void ncnnhip_extractor_set_layer_timing(ncnn_extractor_t ex, int enable)
+{
+    E(ex)->set_layer_timing(enable != 0);
+}
+int ncnnhip_extractor_layer_timing(ncnn_extractor_t ex, char* text, size_t capacity, size_t* needed)
+{
+    std::vector<Extractor::LayerTime> t;
+    int ret = E(ex)->layer_timing(t);
+    if (ret != 0) return ret;
+    std::string out;
+    char line[512];
+    for (size_t i = 0; i < t.size(); i++)
+    {
+        snprintf(line, sizeof(line), "%d\t%s\t%s\t%s\t%.6f\n", t[i].layer_index, t[i].type.c_str(), t[i].name.c_str(), t[i].on_device ? "device" : "host", t[i].ms);
+        out += line;
+    }
+    if (needed) *needed = out.size() + 1;
+    if (text && capacity)
+    {
+        const size_t n = out.size() < capacity - 1 ? out.size() : capacity - 1;
+        memcpy(text, out.data(), n);
+        text[n] = 0;
+    }
+    return 0;
 }
 int ncnnhip_extractor_synchronize(ncnn_extractor_t ex)
 {

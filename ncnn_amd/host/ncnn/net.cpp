@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include <map>
+#include <chrono>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -27,13 +28,54 @@ struct CustomEntry
 static const int CUSTOM_BIT = 1 << 8; // type indexes of non-built-in custom layers carry this bit
 
 // what one Extractor holds while it runs: every blob as a host Mat, a device HipMat, or both
+// One entry per layer that ran, when the Extractor was asked to time its layers (the role of the reference's
+// NCNN_BENCHMARK switch, src/net.cpp:145-180): a device layer is bracketed by two events on the command's stream, a host
+// layer by the wall clock.
+struct LayerTimingSlot
+{
+    int layer_index;
+    void* start;    // events of a device layer (0 for a host layer)
+    void* stop;
+    double host_ms; // wall clock of a host layer
+};
+
 struct ExecState
 {
     std::vector<Mat> host;
     std::vector<HipMat> dev;
     std::shared_ptr<HipCommand> cmd; // created on the first layer that runs device-resident
     int wanted;                      // the blob an extract call asked for (-1: none): it is produced as the model defines it
-    ExecState() : wanted(-1) {}
+    bool time_layers;
+    std::vector<LayerTimingSlot> timing;
+    ExecState() : wanted(-1), time_layers(false) {}
+    // a copy shares the blobs and the command but starts its own timing record (the events belong to one state)
+    ExecState(const ExecState& r) : host(r.host), dev(r.dev), cmd(r.cmd), wanted(r.wanted), time_layers(r.time_layers) {}
+    ExecState& operator=(const ExecState& r)
+    {
+        if (this != &r)
+        {
+            host = r.host;
+            dev = r.dev;
+            cmd = r.cmd;
+            wanted = r.wanted;
+            time_layers = r.time_layers;
+            drop_timing();
+        }
+        return *this;
+    }
+    ~ExecState()
+    {
+        drop_timing();
+    }
+    void drop_timing()
+    {
+        for (size_t i = 0; i < timing.size(); i++)
+        {
+            if (timing[i].start) ncnnhip_event_destroy(timing[i].start);
+            if (timing[i].stop) ncnnhip_event_destroy(timing[i].stop);
+        }
+        timing.clear();
+    }
 
     bool has(int blob) const
     {
@@ -375,8 +417,19 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
     if (layer->bottoms.empty() && layer->type == "Input") return 0; // inputs are fed, not computed
 
     {
+        // (a tail folded into its producer's epilogue is timed as that one launch, under the layer that asked for it)
+        LayerTimingSlot slot = {layer_index, 0, 0, 0.0};
+        const bool timed = st.time_layers && st.cmd && ncnnhip_event_create(&slot.start) == 0 && ncnnhip_event_create(&slot.stop) == 0 &&
+                           ncnnhip_event_record(slot.start, st.cmd->stream) == 0;
         bool done = false;
         int ret = try_fused_tail(layer_index, st, opt, done);
+        if (timed && done && ret == 0 && ncnnhip_event_record(slot.stop, st.cmd->stream) == 0)
+            st.timing.push_back(slot);
+        else
+        {
+            if (slot.start) ncnnhip_event_destroy(slot.start);
+            if (slot.stop) ncnnhip_event_destroy(slot.stop);
+        }
         if (ret != 0 || done) return ret;
     }
 
@@ -401,14 +454,34 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
             }
         }
     }
-    if (layer->featmask)
+    const Option lopt = layer->featmask ? masked_option(opt, layer->featmask) : opt;
+    const bool on_device = lopt.use_hip_compute && layer->support_hip;
+    if (!st.time_layers) return on_device ? run_layer_hip(layer, st, lopt) : run_layer(layer, st, lopt);
+
+    LayerTimingSlot slot = {layer_index, 0, 0, 0.0};
+    int ret;
+    if (on_device)
     {
-        const Option lopt = masked_option(opt, layer->featmask);
-        if (lopt.use_hip_compute && layer->support_hip) return run_layer_hip(layer, st, lopt);
-        return run_layer(layer, st, lopt);
+        if (!st.cmd) st.cmd = acquire_command();
+        ret = st.cmd->ensure_ready();
+        if (ret != 0) return ret;
+        if (ncnnhip_event_create(&slot.start) != 0 || ncnnhip_event_create(&slot.stop) != 0 || ncnnhip_event_record(slot.start, st.cmd->stream) != 0)
+        {
+            if (slot.start) ncnnhip_event_destroy(slot.start);
+            if (slot.stop) ncnnhip_event_destroy(slot.stop);
+            return -1;
+        }
+        ret = run_layer_hip(layer, st, lopt);
+        ncnnhip_event_record(slot.stop, st.cmd->stream);
     }
-    if (opt.use_hip_compute && layer->support_hip) return run_layer_hip(layer, st, opt);
-    return run_layer(layer, st, opt);
+    else
+    {
+        const std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+        ret = run_layer(layer, st, lopt);
+        slot.host_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    }
+    st.timing.push_back(slot); // (copied as plain pointers: the state owns the events from here on)
+    return ret;
 }
 
 // A layer with forward_hip: inputs are made device-resident (uploaded once if they only exist on the host), the
@@ -1171,6 +1244,41 @@ int Extractor::extract(int blob_index, HipMat& feat)
 int Extractor::synchronize()
 {
     return d->st.cmd ? d->st.cmd->synchronize() : 0;
+}
+
+void Extractor::set_layer_timing(bool enable)
+{
+    d->st.time_layers = enable;
+    if (!enable) d->st.drop_timing();
+}
+
+int Extractor::layer_timing(std::vector<LayerTime>& out)
+{
+    out.clear();
+    if (d->st.cmd)
+    {
+        int ret = d->st.cmd->synchronize();
+        if (ret != 0) return ret;
+    }
+    const std::vector<Layer*>& layers = d->net->d->layers;
+    for (size_t i = 0; i < d->st.timing.size(); i++)
+    {
+        const LayerTimingSlot& s = d->st.timing[i];
+        LayerTime t;
+        t.layer_index = s.layer_index;
+        t.name = layers[(size_t)s.layer_index]->name;
+        t.type = layers[(size_t)s.layer_index]->type;
+        t.on_device = s.start != 0;
+        t.ms = s.host_ms;
+        if (s.start)
+        {
+            float ms = 0.f;
+            if (ncnnhip_event_elapsed_ms(s.start, s.stop, &ms) != 0) return -1;
+            t.ms = ms;
+        }
+        out.push_back(t);
+    }
+    return 0;
 }
 
 int Extractor::extract(const char* blob_name, Mat& feat, int type)

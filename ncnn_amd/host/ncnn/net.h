@@ -5,6 +5,7 @@
 
 #include <stdio.h>
 
+#include <string>
 #include <vector>
 
 #include "blob.h"
@@ -97,6 +98,20 @@ public:
     int extract(const char* blob_name, HipMat& feat);
     int extract(int blob_index, HipMat& feat);
     int synchronize();
+
+    // Per-layer timing (what the reference prints under its NCNN_BENCHMARK build switch, src/net.cpp:145-180, a run-time
+    // switch here): while enabled every layer this Extractor runs is recorded, device layers between two events on the
+    // Extractor's stream, host layers by the wall clock.  layer_timing() waits for the stream and returns the records in
+    // execution order; a layer folded into its producer's epilogue appears as that one launch.
+    struct LayerTime
+    {
+        int layer_index;
+        std::string name, type;
+        bool on_device;
+        double ms;
+    };
+    void set_layer_timing(bool enable);
+    int layer_timing(std::vector<LayerTime>& out);
 
 protected:
     friend Extractor Net::create_extractor() const;

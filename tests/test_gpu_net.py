@@ -417,6 +417,31 @@ def test_multiheadattention_layer_block_quant(spec, resident):
         assert np.abs(ex.extract("vo") - vw).max() <= 1e-5 * max(1.0, np.abs(vw).max())
 
 
+@RESIDENT
+def test_per_layer_timing_lists_every_layer_that_ran(resident):
+    """The executor's per-layer timing (the reference's NCNN_BENCHMARK output): one record per layer run, in execution order,
+    device layers timed by events, host layers by the wall clock; results are unchanged and nothing is recorded when off."""
+    g, param, blob, info = zoo.build("tiny", seed=11)
+    net = _load(param, blob, resident)
+    x = np.random.default_rng(12).uniform(0, 1, g.input_shape).astype(F)
+    want = refnet.run(param, blob, x)["fc"]
+    ex = net.create_extractor()
+    ex.set_layer_timing(True)
+    ex.input("data", x)
+    assert np.array_equal(ex.extract("fc").reshape(-1), want.reshape(-1))
+    rows = ex.layer_timing()
+    names = [r[2] for r in rows]
+    assert "c1" in names and "fc" in names and names.index("c1") < names.index("fc")
+    assert all(r[4] >= 0.0 and r[4] < 1000.0 for r in rows)
+    where = {r[2]: r[3] for r in rows}
+    assert where["fc"] == ("device" if resident else "host")
+    assert sum(r[4] for r in rows) > 0.0
+    ex2 = net.create_extractor()
+    ex2.input("data", x)
+    ex2.extract("fc")
+    assert ex2.layer_timing() == []
+
+
 def test_multiheadattention_layer_rejects_other_weight_formats():
     net = host.Net()
     assert net.register_attention_layer() == 0
