@@ -261,14 +261,9 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     wbytes = packed.nbytes + scales.nbytes
     copies = int(np.ceil(512e6 / wbytes)) + 1
     half = args.act == "fp16"
-    lowbit = bits != 8 or block != 64  # these stream the .bin layout as it is (no matrix-core repack)
-    if lowbit:
-        d_w = [rt.up(packed) for _ in range(copies)]
-        d_s = [rt.up(scales) for _ in range(copies)]
-    elif half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
-        pw, pd = rt.blockquant_pack(packed, scales, 64)
-        wbytes = n * k + scales.nbytes  # algorithmic bytes: the int8 weights and one fp32 scale per block
-        d_w = [rt.up(pw) for _ in range(copies)]
+    if half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
+        pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+        d_w = [rt.up(pw) for _ in range(copies)]  # algorithmic bytes stay those of the .bin: the fields and one fp32 scale per block
         d_s = [rt.up(pd) for _ in range(copies)]
     else:
         d_w = [rt.up(packed) for _ in range(copies)]
@@ -279,14 +274,10 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
 
     def launch(i):
         j = i % copies
-        if lowbit and half:
-            check(lib.ncnnhip_gemm_blockquant_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, d_out.ptr, n, st))
-        elif lowbit:
-            check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
-        elif half:
-            check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, None, -1, 1.0, 1.0, d_out.ptr, n, st))
+        if half:
+            check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, -1, 1.0, 1.0, d_out.ptr, n, st))
         else:
-            check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, 8, 64, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
+            check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
 
     for i in range(args.warmup):
         launch(i)
@@ -313,8 +304,9 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
         "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, %d-bit weights in blocks of %d, fp32 block scales, %s activations" % (m, n, k, bits, block, args.act),
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and not lowbit) else None,
-                     "kernel": "blockquant8_stream_kernel" if (lowbit or not half) else "blockquant8_upfront_kernel", "bytes_per_launch": algo,
+                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and bits == 8 and block == 64) else None,
+                     "kernel": "blockquant8_upfront_kernel" if half else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
+                     "bytes_per_launch": algo,
                      "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
                      "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"
                                           % floor["us_per_launch"]},

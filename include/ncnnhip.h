@@ -348,22 +348,28 @@ int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, 
                                  int bits, int block, const float* scales_dev, float* out_dev, size_t out_stride,
                                  void* stream);
 
-/* Packed form of the 8-bit block-quantised weights, made once at create_pipeline (the repacking
- * of constant weights into matrix-core tiles).  ncnn keeps B_data [N][K] and B_data_quantize_scales
- * [N][ceil(K/block)] as loaded (src/layer/gemm.cpp:182-221); here they become
- *   weights  [ceil(N/16)][ceil(K/64)][64][16] bytes, byte = q + 128, lane l = row l%16, K (l/16)*16..+15
- *   descales [ceil(N/16)][ceil(K/64)][16] fp32 = 1.f/scale (the reference's per-block division).
- * block must be 64 or 128.  Both functions run on the host. */
-int ncnnhip_blockquant_packed_size(int N, int K, int block, size_t* weight_bytes, size_t* descale_bytes);
+/* Packed form of the block-quantised weights, made once at create_pipeline (the repacking of
+ * constant weights into matrix-core tiles).  ncnn keeps B_data [N][ceil(K*bits/8)] and
+ * B_data_quantize_scales [N][ceil(K/block)] as loaded (src/layer/gemm.cpp:182-221); here they become
+ * tiles of 16 weight rows by 64 K, [ceil(N/16)][ceil(K/64)], each holding what the 64 lanes of a
+ * wavefront load for it, every field stored as q + 2^(bits-1):
+ *   8-bit fields in blocks of 64 or 128:  [64 lanes][16 bytes], lane l = row l%16, K (l/16)*16..+15;
+ *     descales [tile][step][16 rows] fp32 = 1.f/scale (the reference's per-block division);
+ *   every other combination (bits 4/6/8, block 32/64/128; K <= 16384):  lane l = row l%16 and the
+ *     eight K (l/16)*8..+7 of each 32-wide half of the step; 8-bit 16 bytes per lane, 4-bit 8 bytes
+ *     (a dword per half, fields 2p and 2p+1 in nibbles p and p+4), 6-bit [64 lanes][8 bytes] then
+ *     [64 lanes][4 bytes]; descales as above, for blocks of 32 [tile][step][2 halves][16 rows].
+ * Both functions run on the host. */
+int ncnnhip_blockquant_packed_size(int N, int K, int bits, int block, size_t* weight_bytes, size_t* descale_bytes);
 int ncnnhip_blockquant_pack(const uint8_t* b_host, const float* scales_host, int N, int K, int bits, int block,
                             uint8_t* packed_w_host, float* packed_descale_host);
 /* Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483) on the packed weights with fp16
- * activations a [M][K] (K % 16 == 0), any M; out fp32 [M][N].  Same C / alpha / beta meaning as
- * ncnnhip_gemm_blockquant. */
+ * activations a [M][K] (K % 16 == 0), any M; out fp32 [M][N].  bits / block as given to the packer.
+ * Same C / alpha / beta meaning as ncnnhip_gemm_blockquant. */
 int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K,
-                                        const uint8_t* packed_w_dev, const float* packed_descale_dev, const float* c_dev,
-                                        int broadcast_type_c, float alpha, float beta, float* out_dev, size_t out_stride,
-                                        void* stream);
+                                        const uint8_t* packed_w_dev, const float* packed_descale_dev, int bits, int block,
+                                        const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
+                                        size_t out_stride, void* stream);
 
 /* ------------------------------------------------------------------ attention
  * The core of MultiHeadAttention::forward_weight_block_quantize (src/layer/multiheadattention.cpp:776-866):

@@ -5,6 +5,7 @@
 // order of the fp32 additions differs from the reference's single sequential sum, which is why
 // this output is compared with a relative tolerance and not bit-for-bit.
 #include <hip/hip_fp16.h>
+#include <string.h>
 
 #include "common.h"
 
@@ -533,6 +534,54 @@ __device__ __forceinline__ v8h bytes_to_halves(int lo, int hi)
     return t.h8;
 }
 
+// 8 nibbles u = q + 8; nibbles p and p + 4 of the dword are the two halves of pair p, so one mask serves both.
+__device__ __forceinline__ v8h nibbles_to_halves(unsigned w)
+{
+    union
+    {
+        unsigned i[4];
+        v2h h2[4];
+        v8h h8;
+    } t;
+#pragma unroll
+    for (int p = 0; p < 4; p++) t.i[p] = ((w >> (4 * p)) & 0x000F000Fu) | 0x64006400u; // halves 1024 + u
+    const v2h off = {(_Float16)1032.f, (_Float16)1032.f};
+#pragma unroll
+    for (int e = 0; e < 4; e++) t.h2[e] = t.h2[e] - off;
+    return t.h8;
+}
+
+// 16 six-bit fields u = q + 32 in three dwords.  A dword carries two whole pairs (the low-half field at bit 0 or 6,
+// the high-half field 16 bits above) and, in bits 12-15 / 28-31, a third of a pair: pairs 6 and 7 have their low four
+// bits in dword 0 / dword 1 and their high two bits side by side in dword 2.
+__device__ __forceinline__ void sixbit_to_halves(unsigned d0, unsigned d1, unsigned d2, v8h& wa, v8h& wb)
+{
+    union
+    {
+        unsigned i[4];
+        v2h h2[4];
+        v8h h8;
+    } a, b;
+    const unsigned magic = 0x64006400u;
+    a.i[0] = (d0 & 0x003F003Fu) | magic;
+    a.i[1] = ((d0 >> 6) & 0x003F003Fu) | magic;
+    a.i[2] = (d1 & 0x003F003Fu) | magic;
+    a.i[3] = ((d1 >> 6) & 0x003F003Fu) | magic;
+    b.i[0] = (d2 & 0x003F003Fu) | magic;
+    b.i[1] = ((d2 >> 6) & 0x003F003Fu) | magic;
+    b.i[2] = ((d0 >> 12) & 0x000F000Fu) | (((d2 >> 8) & 0x00300030u) | magic);
+    b.i[3] = ((d1 >> 12) & 0x000F000Fu) | (((d2 >> 10) & 0x00300030u) | magic);
+    const v2h off = {(_Float16)1056.f, (_Float16)1056.f};
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+    {
+        a.h2[e] = a.h2[e] - off;
+        b.h2[e] = b.h2[e] - off;
+    }
+    wa = a.h8;
+    wb = b.h8;
+}
+
 // LDSA: the (few) activation rows are staged once per workgroup in LDS, zero-filled to a multiple of 64, instead of
 // travelling with every batch in registers: a batch is then 4 VGPRs per block and the ring can be twice as deep at the same
 // occupancy.  Used while M rows of K halves fit in 32 KB (decoding: M = 1..4 at K = 4096) and there are many tiles.
@@ -712,18 +761,28 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
 //   operand mapping a 16-lane group touches 16 rows, 16 cache lines for 256 bytes, and the loads took four times the
 //   weight stream's share of the L1 pipe), and are turned into the operand mapping through 2.25 KB of LDS per wavefront
 //   when the block is multiplied.
-template<int NB, int MAXW, int MT, bool ACT_LDS>
+// BITS / HALVES: the packed layouts of ncnnhip_blockquant_pack.  HALVES = false is the 8-bit layout for quantisation
+// blocks of 64 or 128 (a lane's 16 weights are 16 consecutive K, one descale per 64).  HALVES = true serves 4- and 6-bit
+// fields and blocks of 32: the first matrix-core instruction of a 64-wide step covers K 0..31 and the second K 32..63
+// (a lane holds K (l/16)*8..+7 of either half), each with a descale of its own (`split` = 1: blocks of 32; 0: the same
+// descale twice).  A lane's share of a step is 2 * BITS bytes: one 16-byte load, one 8-byte load, or 8 + 4 bytes.
+typedef int v2i_bq __attribute__((ext_vector_type(2)));
+
+template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS>
 __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
-                                                                        const v4i_bq* __restrict__ wpk, const float4* __restrict__ dpk,
+                                                                        const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
                                                                         const float* __restrict__ c, int bt, float alpha, float beta,
                                                                         float* __restrict__ out, size_t out_stride)
 {
+    static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_up[];
     constexpr int ACT_PITCH = NB * 128 + 128;                               // ACT_LDS: bytes from one staged activation row to the next (off the bank stride)
     constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;               // ACT_LDS: 16-byte activation loads per lane
     constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;  // rows the staging stores touch (>= MT: every lane stores, no branch)
     constexpr int TR_PITCH = 144;                                           // !ACT_LDS: one row of a block (128 bytes) + 16: 16 rows land on 16 different bank groups
-    constexpr int WAVE_BYTES = 1024 + (ACT_LDS ? AROWS * ACT_PITCH : 16 * TR_PITCH); // 64 float4 of descales (NB * 4 used), then the activations
+    const int D_BYTES = HALVES ? 1024 << split : 1024;                      // 64 (128 with blocks of 32) float4 of descales: NB * 4 (* 2) used
+    const int WAVE_BYTES = D_BYTES + (ACT_LDS ? AROWS * ACT_PITCH : 16 * TR_PITCH); // descales, then the activations
+    constexpr int STEP_BYTES = 128 * BITS;                                  // one tile's weights for a 64-wide K step
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nwaves = blockDim.x >> 6;
@@ -740,7 +799,7 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
 
     unsigned char* mine = lds_up + wave * WAVE_BYTES;
     float4* my_d = reinterpret_cast<float4*>(mine);
-    unsigned char* my_a = mine + 1024;
+    unsigned char* my_a = mine + D_BYTES;
 
     // (1) ACT_LDS: the activations of the wavefront's K range.  Every load is unconditional, from a clamped address, and
     // masked afterwards (a guarded load becomes a branch, and the compiler waits for every load in flight past a branch).
@@ -758,16 +817,22 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
             areg[q] = *reinterpret_cast<const v4i_bq*>(a + (size_t)rr * a_stride + (ok ? k : 0));
         }
     }
-    // (2) descales of the wavefront's blocks: float4 number j of them is (block j / 4, row group j % 4)
-    const float4* dt = dpk + ((size_t)tile * kblocks + kb_base) * 4;
+    // (2) descales of the wavefront's blocks: float4 number j of them is (block j / 4, row group j % 4); with blocks of 32,
+    // (step j / 8, half (j / 4) % 2, row group j % 4)
+    const int dper = HALVES ? 4 << split : 4; // float4 per step
+    const float4* dt = dpk + ((size_t)tile * kblocks + kb_base) * dper;
     __builtin_amdgcn_sched_barrier(0);
-    const float4 dreg = dt[lane < nkb * 4 ? lane : 0];
+    const float4 dreg = dt[lane < nkb * dper ? lane : 0];
+    float4 dreg2 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (HALVES) dreg2 = dt[lane + 64 < nkb * dper ? lane + 64 : 0];
     __builtin_amdgcn_sched_barrier(0);
     // (3) the weights, all of them; !ACT_LDS: each block's activations right behind its weights.  Lane l fetches 16 bytes of
     // rows l/8 and l/8 + 8, piece l%8 of the block's 128 bytes per row; a chunk beyond K is read from the start of the row
     // (it meets packed weights that are zero there), rows from M up repeat row 0 (their results are never stored).
-    const v4i_bq* wt = wpk + ((size_t)tile * kblocks + kb_base) * 64 + lane;
-    v4i_bq w[NB];
+    const unsigned char* wt = wpk + ((size_t)tile * kblocks + kb_base) * STEP_BYTES;
+    v4i_bq w[BITS == 8 ? NB : 1]; // 8-bit: 16 bytes per lane and step
+    v2i_bq w2[BITS != 8 ? NB : 1]; // 4-bit: all 8 bytes; 6-bit: the first two of three dwords
+    int w1[BITS == 6 ? NB : 1];    // 6-bit: the third dword (the step's 64 x 8 bytes first, then its 64 x 4 bytes)
     v4i_bq a0[ACT_LDS ? 1 : NB], a1[ACT_LDS ? 1 : NB];
     const int tr_row = lane >> 3, tr_piece = lane & 7;
     const __half* arow0 = a + (size_t)(tr_row < M ? tr_row : 0) * a_stride;
@@ -775,7 +840,12 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
 #pragma unroll
     for (int i = 0; i < NB; i++)
     {
-        w[i] = __builtin_nontemporal_load(wt + (size_t)(i < nkb ? i : 0) * 64);
+        const unsigned char* ws = wt + (size_t)(i < nkb ? i : 0) * STEP_BYTES;
+        if (BITS == 8)
+            w[BITS == 8 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const v4i_bq*>(ws) + lane);
+        else
+            w2[BITS != 8 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const v2i_bq*>(ws) + lane);
+        if (BITS == 6) w1[BITS == 6 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const int*>(ws + 512) + lane);
         __builtin_amdgcn_sched_barrier(0);
         if (!ACT_LDS)
         {
@@ -803,17 +873,31 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
             *reinterpret_cast<v4i_bq*>(my_a + r * ACT_PITCH + v * 16) = t; // unconditional: a guarded store would pull its load into the branch
         }
     }
-    my_d[lane] = lane < nkb * 4 ? dreg : make_float4(0.f, 0.f, 0.f, 0.f);
+    my_d[lane] = lane < nkb * dper ? dreg : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (HALVES && split) my_d[lane + 64] = lane + 64 < nkb * dper ? dreg2 : make_float4(0.f, 0.f, 0.f, 0.f);
 
     // (5) block after block, as the weights arrive
     v4f acc = {0.f, 0.f, 0.f, 0.f};
-    const unsigned char* act_rd = ACT_LDS ? my_a + (m < M && m < MT ? m : 0) * ACT_PITCH + kg * 32 : my_a + m * TR_PITCH + kg * 32;
+    constexpr int A_LANE = HALVES ? 16 : 32; // bytes from one K group's operand to the next inside a staged row
+    constexpr int A_SECOND = HALVES ? 64 : 16; // and from the first instruction's operand to the second's
+    const unsigned char* act_rd = ACT_LDS ? my_a + (m < M && m < MT ? m : 0) * ACT_PITCH + kg * A_LANE : my_a + m * TR_PITCH + kg * A_LANE;
     unsigned char* tr_wr = my_a + tr_row * TR_PITCH + tr_piece * 16;
 #pragma unroll
     for (int i = 0; i < NB; i++)
     {
-        const v8h wa = bytes_to_halves(w[i][0], w[i][1]);
-        const v8h wb = bytes_to_halves(w[i][2], w[i][3]);
+        v8h wa, wb;
+        if (BITS == 8)
+        {
+            wa = bytes_to_halves(w[BITS == 8 ? i : 0][0], w[BITS == 8 ? i : 0][1]);
+            wb = bytes_to_halves(w[BITS == 8 ? i : 0][2], w[BITS == 8 ? i : 0][3]);
+        }
+        else if (BITS == 4)
+        {
+            wa = nibbles_to_halves((unsigned)w2[BITS != 8 ? i : 0][0]);
+            wb = nibbles_to_halves((unsigned)w2[BITS != 8 ? i : 0][1]);
+        }
+        else
+            sixbit_to_halves((unsigned)w2[BITS != 8 ? i : 0][0], (unsigned)w2[BITS != 8 ? i : 0][1], (unsigned)w1[BITS == 6 ? i : 0], wa, wb);
         union
         {
             v4i_bq i4;
@@ -822,7 +906,7 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
         if (ACT_LDS)
         {
             xa.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128);
-            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128 + 16);
+            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128 + A_SECOND);
         }
         else
         {
@@ -831,16 +915,31 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
             *reinterpret_cast<v4i_bq*>(tr_wr) = a0[ACT_LDS ? 0 : i];
             *reinterpret_cast<v4i_bq*>(tr_wr + 8 * TR_PITCH) = a1[ACT_LDS ? 0 : i];
             xa.i4 = *reinterpret_cast<const v4i_bq*>(act_rd);
-            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + 16);
+            xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + A_SECOND);
         }
-        v4f t = {0.f, 0.f, 0.f, 0.f};
-        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, t, 0, 0, 0);
-        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
-        const float4 d = my_d[i * 4 + kg]; // zero for a block beyond the wavefront's range
-        acc[0] = fmaf(t[0], d.x, acc[0]);
-        acc[1] = fmaf(t[1], d.y, acc[1]);
-        acc[2] = fmaf(t[2], d.z, acc[2]);
-        acc[3] = fmaf(t[3], d.w, acc[3]);
+        const v4f zero = {0.f, 0.f, 0.f, 0.f};
+        if (HALVES)
+        {
+            // the two halves of the step apart: a block of 32 ends between them
+            const v4f t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, zero, 0, 0, 0);
+            const v4f t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, zero, 0, 0, 0);
+            const float4 da = my_d[i * dper + kg]; // zero for a step beyond the wavefront's range
+            const float4 db = my_d[i * dper + (split << 2) + kg];
+            acc[0] = fmaf(t1[0], db.x, fmaf(t0[0], da.x, acc[0]));
+            acc[1] = fmaf(t1[1], db.y, fmaf(t0[1], da.y, acc[1]));
+            acc[2] = fmaf(t1[2], db.z, fmaf(t0[2], da.z, acc[2]));
+            acc[3] = fmaf(t1[3], db.w, fmaf(t0[3], da.w, acc[3]));
+        }
+        else
+        {
+            v4f t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, zero, 0, 0, 0);
+            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
+            const float4 d = my_d[i * 4 + kg]; // zero for a block beyond the wavefront's range
+            acc[0] = fmaf(t[0], d.x, acc[0]);
+            acc[1] = fmaf(t[1], d.y, acc[1]);
+            acc[2] = fmaf(t[2], d.z, acc[2]);
+            acc[3] = fmaf(t[3], d.w, acc[3]);
+        }
     }
 
     // (6) combine the wavefronts' K ranges in wavefront order; accumulator r of lane l is (weight row (l/16)*4 + r, activation row l%16)
@@ -876,13 +975,13 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
 }
 
 // One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
-template<int NB, int MAXW, int MT, bool ACT_LDS>
-static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, int K, int kblocks, const v4i_bq* wpk, const float4* dpk, const float* c, int bt,
-                              float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS>
+static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
+                              const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
 {
     constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;
     constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;
-    constexpr int WAVE_BYTES = 1024 + (ACT_LDS ? AROWS * (NB * 128 + 128) : 16 * 144);
+    const int WAVE_BYTES = (HALVES ? 1024 << split : 1024) + (ACT_LDS ? AROWS * (NB * 128 + 128) : 16 * 144);
     const int nwaves = (kblocks + NB - 1) / NB;
     const size_t lds = (size_t)nwaves * WAVE_BYTES; // >= 1 KB per wavefront, which the final exchange reuses
     if (lds > 160 * 1024)
@@ -890,7 +989,7 @@ static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, in
         *handled = false;
         return NCNNHIP_OK;
     }
-    auto kernel = blockquant8_upfront_kernel<NB, MAXW, MT, ACT_LDS>;
+    auto kernel = blockquant8_upfront_kernel<BITS, HALVES, NB, MAXW, MT, ACT_LDS>;
     if (lds > 65536)
     {
         // more than the 64 KB a kernel gets by default: raise this kernel's limit once (the chip has 160 KB per compute unit)
@@ -901,51 +1000,58 @@ static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, in
             raised = true;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, c, bt, alpha, beta, out, out_stride);
+    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, c, bt, alpha, beta, out,
+                       out_stride);
     return launch_status("blockquant8_upfront_kernel");
 }
 
-// handled = false: the shape is left to the ring kernel (K beyond 16384, or more than 4 rows with K beyond 8192)
-static int launch_blockquant8_upfront(const __half* a, size_t a_stride, int M, int N, int K, const v4i_bq* wpk, const float4* dpk, const float* c, int bt,
-                                      float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+// handled = false: the shape is left to the caller (K beyond 16384, or more than 4 rows with K beyond 8192)
+template<int BITS, bool HALVES>
+static int launch_blockquant8_upfront(const __half* a, size_t a_stride, int M, int N, int K, const unsigned char* wpk, const float4* dpk, int split,
+                                      const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
 {
     const int kblocks = (K + 63) / 64;
     *handled = true;
 #define UPFRONT(NB_, MAXW_, MT_, LDS_) \
-    return launch_upfront_one<NB_, MAXW_, MT_, LDS_>(a, a_stride, M, N, K, kblocks, wpk, dpk, c, bt, alpha, beta, out, out_stride, stream, handled)
+    return launch_upfront_one<BITS, HALVES, NB_, MAXW_, MT_, LDS_>(a, a_stride, M, N, K, kblocks, wpk, dpk, split, c, bt, alpha, beta, out, out_stride, stream, \
+                                                                    handled)
     if (M <= 4)
     {
-        // decoding: 16 blocks per wavefront while 4, 8 or 16 wavefronts cover K; 12 where that wastes fewer requests (K = 11008: 15 wavefronts)
+        // decoding: 8 steps per wavefront while 8 or 16 wavefronts cover K (K up to 8192; measured against 16 steps on half
+        // as many wavefronts: the same at 4096 x 4096, 3-6 % faster from 11008 rows up), then 12 and 16 steps on 16 wavefronts
+        // (K = 11008: 15 wavefronts of 12).  Two rows run as four in the halves layout (fewer kernels to build; the
+        // staging reads row 0 again for the missing ones).
         if (kblocks <= 64)
         {
-            if (M == 1) UPFRONT(16, 4, 1, true);
-            if (M == 2) UPFRONT(16, 4, 2, true);
-            UPFRONT(16, 4, 4, true);
+            if (M == 1) UPFRONT(8, 8, 1, true);
+            if constexpr (!HALVES) { if (M == 2) UPFRONT(8, 8, 2, true); }
+            UPFRONT(8, 8, 4, true);
         }
         if (kblocks <= 128)
         {
-            if (M == 1) UPFRONT(16, 8, 1, true);
-            if (M == 2) UPFRONT(16, 8, 2, true);
-            UPFRONT(16, 8, 4, true);
+            if (M == 1) UPFRONT(8, 16, 1, true);
+            if constexpr (!HALVES) { if (M == 2) UPFRONT(8, 16, 2, true); }
+            UPFRONT(8, 16, 4, true);
         }
         if (kblocks <= 192)
         {
             if (M == 1) UPFRONT(12, 16, 1, true);
-            if (M == 2) UPFRONT(12, 16, 2, true);
+            if constexpr (!HALVES) { if (M == 2) UPFRONT(12, 16, 2, true); }
             UPFRONT(12, 16, 4, true);
         }
         if (kblocks <= 256)
         {
             if (M == 1) UPFRONT(16, 16, 1, true);
-            if (M == 2) UPFRONT(16, 16, 2, true);
+            if constexpr (!HALVES) { if (M == 2) UPFRONT(16, 16, 2, true); }
             UPFRONT(16, 16, 4, true);
         }
     }
     else
     {
-        // 12 VGPRs per block: 16 blocks per wavefront fit while a SIMD holds at most two wavefronts of the workgroup
-        if (kblocks <= 64) UPFRONT(16, 4, 1, false);
-        if (kblocks <= 128) UPFRONT(16, 8, 1, false);
+        // up to 12 VGPRs per step (weights and the 16 rows' activations): 8 steps per wavefront, up to 16 wavefronts
+        // (7.7 -> 6.7 us at 4096 x 4096 against 16 steps on 4 wavefronts)
+        if (kblocks <= 64) UPFRONT(8, 8, 1, false);
+        if (kblocks <= 128) UPFRONT(8, 16, 1, false);
     }
 #undef UPFRONT
     *handled = false;
@@ -1019,13 +1125,33 @@ int ncnnhip_gemm_blockquant(const float* a_dev, size_t a_stride, int M, int N, i
     return launch_status("blockquant_generic_kernel");
 }
 
-int ncnnhip_blockquant_packed_size(int N, int K, int block, size_t* weight_bytes, size_t* descale_bytes)
+// the halves layout (see blockquant8_upfront_kernel): everything but 8-bit fields in blocks of 64 or 128
+static inline bool halves_layout(int bits, int block)
+{
+    return bits != 8 || block == 32;
+}
+
+// field k of a row of the .bin's LSB-first stream (src/layer/gemm.cpp:318-336), sign-extended
+static inline int host_field(const uint8_t* row, size_t row_bytes, int k, int bits)
+{
+    const size_t bit = (size_t)k * bits, byte = bit >> 3;
+    unsigned v = row[byte];
+    if (byte + 1 < row_bytes) v |= (unsigned)row[byte + 1] << 8;
+    const int field = (int)((v >> (bit & 7)) & ((1u << bits) - 1u));
+    const int sign = 1 << (bits - 1);
+    return (field ^ sign) - sign;
+}
+
+int ncnnhip_blockquant_packed_size(int N, int K, int bits, int block, size_t* weight_bytes, size_t* descale_bytes)
 {
     NCNNHIP_REQUIRE(N >= 1 && K >= 1, "ncnnhip_blockquant_packed_size: bad shape");
-    NCNNHIP_REQUIRE(block == 64 || block == 128, "ncnnhip_blockquant_packed_size: packed layout needs block 64 or 128, got %d", block);
+    NCNNHIP_REQUIRE(bits == 4 || bits == 6 || bits == 8, "ncnnhip_blockquant_packed_size: weight bits %d", bits);
+    NCNNHIP_REQUIRE(block == 32 || block == 64 || block == 128, "ncnnhip_blockquant_packed_size: block size %d", block);
+    NCNNHIP_REQUIRE(!halves_layout(bits, block) || K <= 16384, "ncnnhip_blockquant_packed_size: %d-bit fields in blocks of %d are packed for K up to 16384, got %d",
+                    bits, block, K);
     const size_t tiles = (size_t)(N + 15) / 16, kblocks = (size_t)(K + 63) / 64;
-    if (weight_bytes) *weight_bytes = tiles * kblocks * 1024;
-    if (descale_bytes) *descale_bytes = tiles * kblocks * 16 * sizeof(float);
+    if (weight_bytes) *weight_bytes = tiles * kblocks * 128 * bits;
+    if (descale_bytes) *descale_bytes = tiles * kblocks * 16 * sizeof(float) * (block == 32 ? 2 : 1);
     return NCNNHIP_OK;
 }
 
@@ -1033,66 +1159,137 @@ int ncnnhip_blockquant_pack(const uint8_t* b_host, const float* scales_host, int
                             float* packed_descale_host)
 {
     NCNNHIP_REQUIRE(b_host && scales_host && packed_w_host && packed_descale_host, "ncnnhip_blockquant_pack: null pointer");
-    NCNNHIP_REQUIRE(bits == 8, "ncnnhip_blockquant_pack: only 8-bit weights have a packed layout");
-    NCNNHIP_REQUIRE(block == 64 || block == 128, "ncnnhip_blockquant_pack: block %d", block);
+    int ret = ncnnhip_blockquant_packed_size(N, K, bits, block, 0, 0);
+    if (ret) return ret;
     const int tiles = (N + 15) / 16, kblocks = (K + 63) / 64, nblk = (K + block - 1) / block;
+    const size_t row_bytes = ((size_t)K * bits + 7) / 8;
+    const bool halves = halves_layout(bits, block);
+    const int bias = 1 << (bits - 1);
+    const int dper = block == 32 ? 2 : 1; // descale groups per 64-wide step
     for (int t = 0; t < tiles; t++)
         for (int kb = 0; kb < kblocks; kb++)
         {
-            uint8_t* wt = packed_w_host + ((size_t)t * kblocks + kb) * 1024;
-            float* dt = packed_descale_host + ((size_t)t * kblocks + kb) * 16;
+            uint8_t* wt = packed_w_host + ((size_t)t * kblocks + kb) * 128 * bits;
+            float* dt = packed_descale_host + ((size_t)t * kblocks + kb) * 16 * dper;
             for (int l = 0; l < 64; l++)
+            {
+                unsigned u[16]; // the lane's 16 fields, offset to be non-negative
                 for (int e = 0; e < 16; e++)
                 {
-                    const int j = t * 16 + (l & 15), k = kb * 64 + (l >> 4) * 16 + e;
-                    const int q = (j < N && k < K) ? (int)(int8_t)b_host[(size_t)j * K + k] : 0;
-                    wt[l * 16 + e] = (uint8_t)(q + 128);
+                    const int j = t * 16 + (l & 15);
+                    const int k = halves ? kb * 64 + (e >> 3) * 32 + (l >> 4) * 8 + (e & 7) : kb * 64 + (l >> 4) * 16 + e;
+                    const int q = (j < N && k < K) ? host_field(b_host + (size_t)j * row_bytes, row_bytes, k, bits) : 0;
+                    u[e] = (unsigned)(q + bias);
                 }
-            for (int r = 0; r < 16; r++)
-            {
-                const int j = t * 16 + r;
-                // same single rounded division the reference performs per block (gemm.cpp:465)
-                volatile float sc = j < N ? scales_host[(size_t)j * nblk + (size_t)kb * 64 / block] : 1.f;
-                dt[r] = j < N ? 1.f / sc : 0.f;
+                if (bits == 8)
+                    for (int e = 0; e < 16; e++) wt[l * 16 + e] = (uint8_t)u[e];
+                else if (bits == 4)
+                {
+                    unsigned d[2] = {0, 0};
+                    for (int e = 0; e < 16; e++) d[e >> 3] |= u[e] << (4 * ((e & 7) >> 1) + 16 * (e & 1)); // pair p = fields 2p, 2p+1: nibbles p and p + 4
+                    memcpy(wt + l * 8, d, 8);
+                }
+                else
+                {
+                    // pair P = fields 2P (low half) and 2P+1 (high half); dword P/2 holds pair P at bit 0 (P even) or 6 (P odd) for P < 6,
+                    // pairs 6 and 7 lie in the dwords' top nibbles: low four bits in dword 0 / 1, high two bits in dword 2
+                    unsigned d[3] = {0, 0, 0};
+                    for (int P = 0; P < 6; P++) d[P >> 1] |= (u[2 * P] | (u[2 * P + 1] << 16)) << (6 * (P & 1));
+                    for (int P = 6; P < 8; P++)
+                    {
+                        d[P - 6] |= ((u[2 * P] & 15u) | ((u[2 * P + 1] & 15u) << 16)) << 12;
+                        d[2] |= ((u[2 * P] >> 4) | ((u[2 * P + 1] >> 4) << 16)) << (12 + 2 * (P - 6));
+                    }
+                    memcpy(wt + l * 8, d, 8);
+                    memcpy(wt + 512 + l * 4, d + 2, 4);
+                }
             }
+            for (int h = 0; h < dper; h++)
+                for (int r = 0; r < 16; r++)
+                {
+                    const int j = t * 16 + r;
+                    const int blk = (kb * 64 + h * 32) / block;
+                    const bool live = j < N && blk < nblk;
+                    // same single rounded division the reference performs per block (gemm.cpp:465)
+                    volatile float sc = live ? scales_host[(size_t)j * nblk + blk] : 1.f;
+                    dt[h * 16 + r] = live ? 1.f / sc : 0.f;
+                }
         }
     return NCNNHIP_OK;
 }
 
 int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
-                                        const float* packed_descale_dev, const float* c_dev, int broadcast_type_c, float alpha, float beta,
-                                        float* out_dev, size_t out_stride, void* stream)
+                                        const float* packed_descale_dev, int bits, int block, const float* c_dev, int broadcast_type_c, float alpha,
+                                        float beta, float* out_dev, size_t out_stride, void* stream)
 {
     NCNNHIP_REQUIRE(a_dev && packed_w_dev && packed_descale_dev && out_dev, "ncnnhip_gemm_blockquant_packed_f16a: null pointer");
     NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1 && K % 16 == 0, "ncnnhip_gemm_blockquant_packed_f16a: bad shape %d %d %d (K must be a multiple of 16)", M, N, K);
+    NCNNHIP_REQUIRE(bits == 4 || bits == 6 || bits == 8, "ncnnhip_gemm_blockquant_packed_f16a: weight bits %d", bits);
+    NCNNHIP_REQUIRE(block == 32 || block == 64 || block == 128, "ncnnhip_gemm_blockquant_packed_f16a: block size %d", block);
     NCNNHIP_REQUIRE(a_stride >= (size_t)K && a_stride % 8 == 0 && al16(a_dev), "ncnnhip_gemm_blockquant_packed_f16a: activation rows must be 16-byte aligned");
     NCNNHIP_REQUIRE(out_stride >= (size_t)N, "ncnnhip_gemm_blockquant_packed_f16a: output stride too small");
     const int bt = c_dev ? broadcast_type_c : -1;
     NCNNHIP_REQUIRE(bt >= -1 && bt <= 4, "ncnnhip_gemm_blockquant_packed_f16a: C broadcast %d", bt);
     NCNNHIP_REQUIRE((size_t)(K + 63) / 64 * 64 <= 60 * 1024, "ncnnhip_gemm_blockquant_packed_f16a: K %d too large for the descale stage", K);
+    const bool halves = halves_layout(bits, block);
+    NCNNHIP_REQUIRE(!halves || K <= 16384, "ncnnhip_gemm_blockquant_packed_f16a: %d-bit fields in blocks of %d need K <= 16384, got %d", bits, block, K);
     const int tiles = (N + 15) / 16, kblocks = (K + 63) / 64;
     const __half* ah = reinterpret_cast<const __half*>(a_dev);
+    const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
+    const int split = block == 32 ? 1 : 0;
+    hipStream_t st = as_stream(stream);
+    // one pass over the weights for rows m0 .. m0 + mc - 1
+    auto upfront = [&](int m0, int mc, bool* handled) -> int {
+        const float* cc = c_dev;
+        if (cc && (bt == 1 || bt == 2)) cc += m0;
+        if (cc && bt == 3) cc += (size_t)m0 * N;
+        const __half* ap = ah + (size_t)m0 * a_stride;
+        float* op = out_dev + (size_t)m0 * out_stride;
+        if (!halves) return launch_blockquant8_upfront<8, false>(ap, a_stride, mc, N, K, packed_w_dev, dpk, 0, cc, bt, alpha, beta, op, out_stride, st, handled);
+        if (bits == 8) return launch_blockquant8_upfront<8, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
+        if (bits == 6) return launch_blockquant8_upfront<6, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
+        return launch_blockquant8_upfront<4, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
+    };
     for (int m0 = 0; m0 < M; m0 += 16)
     {
         const int mc = M - m0 < 16 ? M - m0 : 16;
+        bool handled = false;
+        int ret = upfront(m0, mc, &handled);
+        if (ret != NCNNHIP_OK) return ret;
+        if (handled) continue;
+        if (halves)
+        {
+            // long rows with more than four activation rows: four at a time, or one at a time where four rows of K and the
+            // descales of blocks of 32 do not fit in LDS together (K beyond 12288)
+            for (int m1 = m0; m1 < m0 + mc;)
+            {
+                const int left = m0 + mc - m1;
+                ret = upfront(m1, left < 4 ? left : 4, &handled);
+                if (ret != NCNNHIP_OK) return ret;
+                if (handled)
+                {
+                    m1 += 4;
+                    continue;
+                }
+                ret = upfront(m1, 1, &handled);
+                if (ret != NCNNHIP_OK) return ret;
+                NCNNHIP_REQUIRE(handled, "ncnnhip_gemm_blockquant_packed_f16a: no kernel for M %d K %d", M, K);
+                m1 += 1;
+            }
+            continue;
+        }
         const float* cc = c_dev;
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
         const size_t act_bytes = (size_t)mc * kblocks * 64 * sizeof(__half);
-        bool handled = false;
-        int ret = launch_blockquant8_upfront(ah + (size_t)m0 * a_stride, a_stride, mc, N, K, reinterpret_cast<const v4i_bq*>(packed_w_dev),
-                                             reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride,
-                                             as_stream(stream), &handled);
-        if (ret != NCNNHIP_OK) return ret;
-        if (handled) continue;
         if (act_bytes <= 32768 && tiles >= 512) // measured: pays from about 8192 weight rows (up to four rows of 4096), not for long rows (K = 11008) or few tiles
-            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS_LDS, 1, true>), dim3(tiles), dim3(256), (size_t)kblocks * 64 + act_bytes, as_stream(stream),
-                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),
-                               reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride);
+            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS_LDS, 1, true>), dim3(tiles), dim3(256), (size_t)kblocks * 64 + act_bytes, st,
+                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev), dpk, cc, bt, alpha, beta,
+                               out_dev + (size_t)m0 * out_stride, out_stride);
         else
-            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS, BQ_MFMA_U, false>), dim3(tiles), dim3(256), (size_t)kblocks * 64, as_stream(stream),
-                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev),
-                               reinterpret_cast<const float4*>(packed_descale_dev), cc, bt, alpha, beta, out_dev + (size_t)m0 * out_stride, out_stride);
+            hipLaunchKernelGGL((blockquant8_mfma_kernel<BQ_MFMA_NS, BQ_MFMA_U, false>), dim3(tiles), dim3(256), (size_t)kblocks * 64, st,
+                               ah + (size_t)m0 * a_stride, a_stride, mc, N, K, kblocks, reinterpret_cast<const v4i_bq*>(packed_w_dev), dpk, cc, bt, alpha, beta,
+                               out_dev + (size_t)m0 * out_stride, out_stride);
     }
     return launch_status("blockquant8_mfma_kernel");
 }

@@ -132,10 +132,10 @@ _SIGNATURES = {
                                 C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_blockquant": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
-    "ncnnhip_blockquant_packed_size": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "ncnnhip_blockquant_packed_size": [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "ncnnhip_blockquant_pack": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
-    "ncnnhip_gemm_blockquant_packed_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
-                                            C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_blockquant_packed_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                            C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_peak_launch_chain": [C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_mfma_i8": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_hbm_read": [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p],
@@ -673,24 +673,25 @@ class Runtime:
                                                 broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
         return dout.to_numpy(self.stream)
 
-    def blockquant_pack(self, b_packed, scales, block):
-        """Host-side repack of 8-bit block-quantised weights into the matrix-core tile layout."""
+    def blockquant_pack(self, b_packed, scales, block, bits=8, k=None):
+        """Host-side repack of block-quantised weights (the .bin's field stream, [N][ceil(K*bits/8)] bytes) into matrix-core tiles."""
         b_packed = np.ascontiguousarray(b_packed, np.uint8)
         scales = np.ascontiguousarray(scales, np.float32)
-        n, k = b_packed.shape
+        n = b_packed.shape[0]
+        k = b_packed.shape[1] * 8 // bits if k is None else k
         wb, db = C.c_size_t(), C.c_size_t()
-        check(lib().ncnnhip_blockquant_packed_size(n, k, block, C.byref(wb), C.byref(db)))
+        check(lib().ncnnhip_blockquant_packed_size(n, k, bits, block, C.byref(wb), C.byref(db)))
         pw = np.empty(wb.value, np.uint8)
         pd = np.empty(db.value // 4, np.float32)
-        check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, 8, block, pw.ctypes.data, pd.ctypes.data))
+        check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, bits, block, pw.ctypes.data, pd.ctypes.data))
         return pw, pd
 
-    def gemm_blockquant_packed(self, a_half, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0):
+    def gemm_blockquant_packed(self, a_half, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64):
         a_half = np.ascontiguousarray(a_half, np.float16)
         m, k = a_half.shape
         da, dw_, dd = self.up(a_half), self.up(pw), self.up(pd)
         dc = self.up(None if c is None else np.asarray(c, np.float32))
         dout = DeviceBuffer.empty((m, n), np.float32)
-        check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, _ptr(dc), broadcast_type_c if c is not None else -1,
-                                                        alpha, beta, dout.ptr, n, self.stream))
+        check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dc),
+                                                        broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
         return dout.to_numpy(self.stream)

@@ -516,8 +516,33 @@ def test_blockquant_packed_matrix_core_path(rt, m, n, k, block, bt):
          4: rng.normal(size=(1, n))}[bt]
     c = None if c is None else c.astype(F)
     pw, pd = rt.blockquant_pack(packed, scales, block)
-    got = rt.gemm_blockquant_packed(a.astype(np.float16), pw, pd, n, c, bt, 0.75, 1.5)
+    got = rt.gemm_blockquant_packed(a.astype(np.float16), pw, pd, n, c, bt, 0.75, 1.5, bits=8, block=block)
     _bq_check(got, a, packed, scales, 8, block, None, c, bt, 0.75, 1.5)
+
+
+@pytest.mark.parametrize("bits,block,m,n,k,bt", [
+    # every field width and block size of the layout whose steps are split in two halves, at one, few (through LDS) and up to 16 (registers) activation rows
+    (4, 64, 1, 512, 4096, -1), (4, 32, 1, 256, 4096, 4), (4, 128, 1, 256, 4096, -1), (6, 64, 1, 512, 4096, -1), (6, 32, 1, 256, 4096, 0), (6, 128, 1, 100, 4096, -1),
+    (8, 32, 1, 512, 4096, -1), (4, 64, 2, 48, 4096, 1), (6, 32, 3, 40, 4096, 2), (8, 32, 4, 256, 4096, 4), (4, 32, 4, 250, 4096, 3), (6, 64, 4, 64, 4096, -1),
+    (4, 64, 16, 256, 4096, 3), (4, 32, 16, 250, 4096, -1), (6, 64, 16, 128, 4096, 4), (6, 32, 9, 40, 4096, 1), (8, 32, 16, 256, 4096, -1), (4, 128, 5, 24, 4096 + 64, -1),
+    # 8, 15 and 16 wavefronts; a last wavefront with one step and with none; K that ends inside a step and inside a block
+    (4, 64, 1, 40, 8192, -1), (6, 64, 2, 33, 12288, 4), (4, 32, 3, 40, 11008 + 16, 1), (8, 32, 4, 32, 16384, -1), (6, 128, 1, 32, 16384, -1), (4, 64, 1, 250, 11008, -1),
+    (4, 64, 3, 37, 208, 1), (6, 32, 1, 16, 64, 0), (8, 32, 2, 20, 1024 + 16, 3), (4, 128, 7, 100, 4096 + 48, -1), (6, 64, 12, 40, 8192, -1), (4, 32, 16, 64, 96, 2),
+    # more than 16 rows (one pass per 16), and more than 4 rows with K beyond 8192 (four at a time)
+    (4, 64, 20, 64, 1024, 2), (6, 32, 33, 40, 512, 3), (4, 64, 9, 40, 12288, 1), (6, 64, 16, 24, 16384, 3), (8, 32, 7, 40, 11008, 4),
+    # many tiles
+    (4, 64, 1, 11008, 4096, -1), (6, 64, 4, 8200 + 5, 1024 + 64, 4), (4, 32, 16, 9000, 512, 3)])
+def test_blockquant_packed_low_bit_widths_and_blocks_of_32(rt, bits, block, m, n, k, bt):
+    _say("blockquant packed", bits, block, m, n, k, bt)
+    from ncnn_amd import synth
+    a, packed, scales = synth.blockquant_operands(bits + block + m + n + k, m, n, k, bits, block)  # activations are fp16-representable
+    rng = np.random.default_rng(bt + 51)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+    got = rt.gemm_blockquant_packed(a.astype(np.float16), pw, pd, n, c, bt, 0.75, 1.5, bits=bits, block=block)
+    _bq_check(got, a, packed, scales, bits, block, None, c, bt, 0.75, 1.5)
 
 
 def test_blockquant_exact_on_power_of_two_data(rt):

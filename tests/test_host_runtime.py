@@ -178,3 +178,80 @@ def test_load_model_fails_loudly_without_a_gpu():
         modelwriter.conv_weights(rng.integers(-127, 128, 36).astype(np.int8), None, np.full(6, 50, F), 10.0, None),
     ])
     assert net.load_model_mem(binimg) != 0  # create_pipeline needs the device
+
+
+# ---- packed block-quant layouts: what the kernel's lanes load, undone in numpy -------------------------------------------
+
+def _unpack_tiles(pw, n, k, bits, block):
+    """Inverse of ncnnhip_blockquant_pack's weight layout, written from the layout's description in include/ncnnhip.h:
+    int [tiles*16][steps*64], fields back to signed values."""
+    tiles, steps = (n + 15) // 16, (k + 63) // 64
+    halves = bits != 8 or block == 32
+    chunk = np.asarray(pw, np.uint8).reshape(tiles, steps, 128 * bits)
+    u = np.zeros((tiles, steps, 64, 16), np.int64)  # [lane][field]
+    if bits == 8:
+        u[:] = chunk.reshape(tiles, steps, 64, 16)
+    elif bits == 4:
+        d = chunk.reshape(tiles, steps, 64, 8).copy().view(np.uint32).astype(np.int64)  # [lane][2 dwords]
+        for e in range(16):
+            u[..., e] = (d[..., e >> 3] >> (4 * ((e & 7) >> 1) + 16 * (e & 1))) & 15
+    else:
+        d01 = chunk[..., :512].reshape(tiles, steps, 64, 8).copy().view(np.uint32).astype(np.int64)
+        d2 = chunk[..., 512:].reshape(tiles, steps, 64, 4).copy().view(np.uint32).astype(np.int64)[..., 0]
+        d = [d01[..., 0], d01[..., 1], d2]
+        for pair in range(8):
+            for hi in range(2):
+                if pair < 6:
+                    v = (d[pair >> 1] >> (6 * (pair & 1) + 16 * hi)) & 63
+                else:
+                    v = ((d[pair - 6] >> (12 + 16 * hi)) & 15) | (((d[2] >> (12 + 2 * (pair - 6) + 16 * hi)) & 3) << 4)
+                u[..., 2 * pair + hi] = v
+    q = np.zeros((tiles * 16, steps * 64), np.int64)
+    for l in range(64):
+        for e in range(16):
+            kk = (e >> 3) * 32 + (l >> 4) * 8 + (e & 7) if halves else (l >> 4) * 16 + e
+            q[(l & 15)::16, kk::64] = u[:, :, l, e]
+    return q - (1 << (bits - 1))
+
+
+@pytest.mark.parametrize("bits", [4, 6, 8])
+@pytest.mark.parametrize("block", [32, 64, 128])
+@pytest.mark.parametrize("n,k", [(16, 64), (37, 208), (5, 4096 + 48), (33, 96)])
+def test_blockquant_pack_layouts_hold_every_field_and_descale(bits, block, n, k):
+    from ncnn_amd import synth
+    import npref
+    rng = np.random.default_rng(bits * 1000 + block + n + k)
+    packed, scales = synth.blockquant_weights(rng.standard_normal((n, k)).astype(np.float32), bits, block)
+    lib = hip.lib()
+    wb, db = C.c_size_t(), C.c_size_t()
+    assert lib.ncnnhip_blockquant_packed_size(n, k, bits, block, C.byref(wb), C.byref(db)) == 0
+    tiles, steps, nblk = (n + 15) // 16, (k + 63) // 64, (k + block - 1) // block
+    per_step = 2 if block == 32 else 1
+    assert wb.value == tiles * steps * 128 * bits and db.value == tiles * steps * 16 * 4 * per_step
+    pw = np.full(wb.value, 0xA5, np.uint8)
+    pd = np.full(db.value // 4, np.nan, np.float32)
+    assert lib.ncnnhip_blockquant_pack(packed.ctypes.data, scales.ctypes.data, n, k, bits, block, pw.ctypes.data, pd.ctypes.data) == 0
+    q = _unpack_tiles(pw, n, k, bits, block)
+    want = np.zeros_like(q)
+    want[:n, :k] = npref.blockquant_unpack_all(packed, k, bits)  # padding rows / K hold zeros
+    assert np.array_equal(q, want)
+    d = pd.reshape(tiles, steps, per_step, 16)
+    with np.errstate(divide="ignore"):
+        inv = (np.float32(1) / scales).astype(np.float32)
+    for t in range(tiles):
+        for s in range(steps):
+            for h in range(per_step):
+                blk = (s * 64 + h * 32) // block
+                for r in range(16):
+                    j = t * 16 + r
+                    want_d = inv[j, blk] if (j < n and blk < nblk) else np.float32(0)
+                    assert d[t, s, h, r] == want_d, (t, s, h, r)
+
+
+def test_blockquant_pack_refuses_what_has_no_kernel():
+    lib = hip.lib()
+    wb, db = C.c_size_t(), C.c_size_t()
+    assert lib.ncnnhip_blockquant_packed_size(16, 16384 + 64, 4, 64, C.byref(wb), C.byref(db)) != 0  # the halves layout stops at K = 16384
+    assert lib.ncnnhip_blockquant_packed_size(16, 16384 + 64, 8, 64, C.byref(wb), C.byref(db)) == 0
+    assert lib.ncnnhip_blockquant_packed_size(16, 64, 5, 64, C.byref(wb), C.byref(db)) != 0
+    assert lib.ncnnhip_blockquant_packed_size(16, 64, 8, 48, C.byref(wb), C.byref(db)) != 0
