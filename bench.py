@@ -261,7 +261,8 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     wbytes = packed.nbytes + scales.nbytes
     copies = int(np.ceil(512e6 / wbytes)) + 1
     half = args.act == "fp16"
-    if half:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
+    packed_form = half or (args.act == "fp32" and m < 32 and lib.ncnnhip_gemm_blockquant_packed_supported(k))
+    if packed_form:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
         pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
         d_w = [rt.up(pw) for _ in range(copies)]  # algorithmic bytes stay those of the .bin: the fields and one fp32 scale per block
         d_s = [rt.up(pd) for _ in range(copies)]
@@ -276,6 +277,8 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
         j = i % copies
         if half:
             check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, -1, 1.0, 1.0, d_out.ptr, n, st))
+        elif packed_form:
+            check(lib.ncnnhip_gemm_blockquant_packed(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
         else:
             check(lib.ncnnhip_gemm_blockquant(d_a.ptr, k, m, n, k, d_w[j].ptr, bits, block, d_s[j].ptr, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
 
@@ -305,7 +308,7 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and bits == 8 and block == 64) else None,
-                     "kernel": "blockquant8_upfront_kernel" if half else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
+                     "kernel": "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
                      "bytes_per_launch": algo,
                      "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
                      "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"
@@ -941,7 +944,9 @@ def main():
                          "on the GPU than a stream launch does); 1 = replay the recorded pass (HipGraph), which takes the host out of the loop")
     ap.add_argument("--b-scale", dest="b_scale", default="per_column", choices=["per_column", "per_tensor"],
                     help="per_column is the benchmark configuration; per_tensor is what ncnn's Gemm layer can express")
-    ap.add_argument("--act", default="fp16", choices=["fp16", "fp32"], help="activation type of the block-quant workload")
+    ap.add_argument("--act", default="fp16", choices=["fp16", "fp32", "fp32-bin"],
+                    help="activation type of the block-quant workload; fp32 = the layer's contract on packed weights where they have a kernel, "
+                         "fp32-bin = always the kernel that streams the .bin layout")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layer-table", default=None, help="layers workloads: write the per-layer timing table to this file")
     ap.add_argument("--calib-copy", action="store_true", help="issue one D2D copy of M*K*4 bytes first (calibrates HBM byte counters)")

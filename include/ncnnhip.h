@@ -371,6 +371,17 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
                                         const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
                                         size_t out_stride, void* stream);
 
+/* The layer's own contract on the packed weights: fp32 activations a [M][K] (16-byte aligned rows, K % 16 == 0,
+ * K <= 16384: ncnnhip_gemm_blockquant_packed_supported says whether a K qualifies), optional in_scales [K], any M (rows
+ * go four at a time, fewer where K is long).  Each activation (times its input scale) is split exactly into three bf16
+ * numbers, so every product is the reference's q * a and the result differs from ncnnhip_gemm_blockquant's only by the
+ * order of the fp32 additions.  From 32 rows up ncnnhip_gemm_blockquant (fp32 matrix cores, one pass) is the faster call. */
+int ncnnhip_gemm_blockquant_packed_supported(int K);
+int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
+                                   const float* packed_descale_dev, int bits, int block, const float* in_scales_dev,
+                                   const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
+                                   size_t out_stride, void* stream);
+
 /* ------------------------------------------------------------------ attention
  * The core of MultiHeadAttention::forward_weight_block_quantize (src/layer/multiheadattention.cpp:776-866):
  * per head, scores = q k^T (+ mask), softmax over the keys, times v.  q (already scaled) and out are

@@ -766,22 +766,114 @@ __global__ __launch_bounds__(256) void blockquant8_mfma_kernel(const __half* __r
 // fields and blocks of 32: the first matrix-core instruction of a 64-wide step covers K 0..31 and the second K 32..63
 // (a lane holds K (l/16)*8..+7 of either half), each with a descale of its own (`split` = 1: blocks of 32; 0: the same
 // descale twice).  A lane's share of a step is 2 * BITS bytes: one 16-byte load, one 8-byte load, or 8 + 4 bytes.
+// AIN = 4: fp32 activations (times the optional input scales, INSC), the layer's own contract.  The matrix cores take no fp32
+// operand of this shape, so a value is split into three bf16 numbers hi + mid + lo that add up to it EXACTLY (each takes the
+// next 8 significant bits, by truncation, so every remainder is exact), when it is staged in LDS: three planes, which
+// enter the matrix cores as three COLUMNS per activation row (up to 5 rows in the 16 columns), the weights converted to
+// bf16 (integers up to 128 are exact there).  Every
+// product is then the exact q * a of the reference and only the order of the fp32 additions differs, as with fp16
+// activations.  (A remainder below 2^-126 is a denormal and may be dropped by the matrix core: |a| < 2^-110 or so.)
 typedef int v2i_bq __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS>
-__global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
+__device__ __forceinline__ void split_bf16x3(float v, unsigned& hi, unsigned& mid, unsigned& lo) // each in the upper half of its dword
+{
+    const unsigned b = __float_as_uint(v);
+    hi = b & 0xFFFF0000u;
+    const bool finite = (b & 0x7F800000u) != 0x7F800000u; // infinities and NaNs travel in hi alone
+    const float r1 = finite ? v - __uint_as_float(hi) : 0.f;
+    mid = __float_as_uint(r1) & 0xFFFF0000u;
+    const float r2 = r1 - __uint_as_float(mid);
+    lo = __float_as_uint(r2) & 0xFFFF0000u; // at most 8 significant bits are left
+}
+
+__device__ __forceinline__ unsigned bf16_pair(float even, float odd) // both exactly representable: truncation loses nothing
+{
+    return (__float_as_uint(even) >> 16) | (__float_as_uint(odd) & 0xFFFF0000u);
+}
+
+// the 8 fields that bytes_to_halves / nibbles_to_halves / sixbit_to_halves turn into halves, as bf16
+__device__ __forceinline__ v8bf bytes_to_bf16(unsigned lo, unsigned hi)
+{
+    union
+    {
+        unsigned i[4];
+        v8bf h;
+    } t;
+    const unsigned slo = lo ^ 0x80808080u, shi = hi ^ 0x80808080u; // q + 128 -> q as a signed byte
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+    {
+        t.i[p] = bf16_pair((float)(signed char)(slo >> (16 * p)), (float)(signed char)(slo >> (16 * p + 8)));
+        t.i[2 + p] = bf16_pair((float)(signed char)(shi >> (16 * p)), (float)(signed char)(shi >> (16 * p + 8)));
+    }
+    return t.h;
+}
+__device__ __forceinline__ v8bf nibbles_to_bf16(unsigned w)
+{
+    union
+    {
+        unsigned i[4];
+        v8bf h;
+    } t;
+    const unsigned x = w ^ 0x88888888u; // q + 8 -> q as a two's complement nibble: one signed bit-field extract each
+#pragma unroll
+    for (int p = 0; p < 4; p++) t.i[p] = bf16_pair((float)((int)(x << (28 - 4 * p)) >> 28), (float)((int)(x << (12 - 4 * p)) >> 28));
+    return t.h;
+}
+__device__ __forceinline__ void sixbit_to_bf16(unsigned d0, unsigned d1, unsigned d2, v8bf& wa, v8bf& wb)
+{
+    union
+    {
+        unsigned i[4];
+        v8bf h;
+    } a, b;
+    // q + 32 -> q in two's complement: flip bit 5 of every field (for pairs 6 and 7 that bit sits in dword 2's top nibbles)
+    const unsigned d[3] = {d0 ^ 0x08200820u, d1 ^ 0x08200820u, d2 ^ 0xA820A820u};
+#pragma unroll
+    for (int P = 0; P < 8; P++)
+    {
+        float f[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+        {
+            int q;
+            if (P < 6)
+                q = (int)(d[P >> 1] << (26 - 6 * (P & 1) - 16 * h)) >> 26; // a signed bit-field extract
+            else
+            {
+                const unsigned u = ((d[P - 6] >> (12 + 16 * h)) & 15u) | (((d[2] >> (12 + 2 * (P - 6) + 16 * h)) & 3u) << 4);
+                q = (int)(u << 26) >> 26;
+            }
+            f[h] = (float)q;
+        }
+        (P < 4 ? a.i[P & 3] : b.i[P & 3]) = bf16_pair(f[0], f[1]);
+    }
+    wa = a.h;
+    wb = b.h;
+}
+
+template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN = 2, bool INSC = false>
+__global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const void* __restrict__ a_, size_t a_stride, int M, int N, int K, int kblocks,
                                                                         const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
-                                                                        const float* __restrict__ c, int bt, float alpha, float beta,
-                                                                        float* __restrict__ out, size_t out_stride)
+                                                                        const float* __restrict__ in_scales, const float* __restrict__ c, int bt, float alpha,
+                                                                        float beta, float* __restrict__ out, size_t out_stride)
 {
     static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
+    static_assert(AIN == 2 || (AIN == 4 && ACT_LDS), "fp32 activations are staged in LDS");
+    static_assert(AIN == 4 || !INSC, "input scales come with fp32 activations");
+    constexpr bool F32 = AIN == 4;
+    const __half* a = static_cast<const __half*>(a_);
+    const float* af = static_cast<const float*>(a_);
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_up[];
     constexpr int ACT_PITCH = NB * 128 + 128;                               // ACT_LDS: bytes from one staged activation row to the next (off the bank stride)
-    constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;               // ACT_LDS: 16-byte activation loads per lane
-    constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;  // rows the staging stores touch (>= MT: every lane stores, no branch)
+    constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;               // ACT_LDS: vectors of 8 activations per lane
+    // rows the staging stores touch (>= MT: every lane stores, no branch); fp32: exactly MT, spare lanes store into row 0's padding
+    constexpr int AROWS = ACT_LDS ? (F32 ? MT : (AV * 64 + NB * 8 - 1) / (NB * 8)) : 0;
+    constexpr int PLANE_BYTES = AROWS * ACT_PITCH;                          // fp32: the hi, mid and lo planes follow one another
     constexpr int TR_PITCH = 144;                                           // !ACT_LDS: one row of a block (128 bytes) + 16: 16 rows land on 16 different bank groups
     const int D_BYTES = HALVES ? 1024 << split : 1024;                      // 64 (128 with blocks of 32) float4 of descales: NB * 4 (* 2) used
-    const int WAVE_BYTES = D_BYTES + (ACT_LDS ? AROWS * ACT_PITCH : 16 * TR_PITCH); // descales, then the activations
+    const int WAVE_BYTES = D_BYTES + (ACT_LDS ? (F32 ? 3 : 1) * PLANE_BYTES : 16 * TR_PITCH); // descales, then the activations
     constexpr int STEP_BYTES = 128 * BITS;                                  // one tile's weights for a 64-wide K step
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -804,6 +896,8 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
     // (1) ACT_LDS: the activations of the wavefront's K range.  Every load is unconditional, from a clamped address, and
     // masked afterwards (a guarded load becomes a branch, and the compiler waits for every load in flight past a branch).
     v4i_bq areg[AV];
+    v4i_bq areg2[F32 ? AV : 1];                // fp32: the vector's second 16 bytes
+    v4i_bq sreg[INSC ? AV : 1], sreg2[INSC ? AV : 1]; // its input scales
     if (ACT_LDS)
     {
 #pragma unroll
@@ -812,9 +906,21 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
             const int idx = q * 64 + lane;
             const int r = idx / (NB * 8), v = idx - r * (NB * 8);
             const int k = kb_base * 64 + v * 8;
-            const bool ok = v < nkb * 8 && k < K; // K % 16 == 0: a vector of 8 halves is all in or all out
+            const bool ok = v < nkb * 8 && k < K; // K % 16 == 0: a vector of 8 activations is all in or all out
             const int rr = r < M ? r : 0;
-            areg[q] = *reinterpret_cast<const v4i_bq*>(a + (size_t)rr * a_stride + (ok ? k : 0));
+            if (F32)
+            {
+                const float* p = af + (size_t)rr * a_stride + (ok ? k : 0);
+                areg[q] = *reinterpret_cast<const v4i_bq*>(p);
+                areg2[F32 ? q : 0] = *reinterpret_cast<const v4i_bq*>(p + 4);
+                if (INSC)
+                {
+                    sreg[INSC ? q : 0] = *reinterpret_cast<const v4i_bq*>(in_scales + (ok ? k : 0));
+                    sreg2[INSC ? q : 0] = *reinterpret_cast<const v4i_bq*>(in_scales + (ok ? k : 0) + 4);
+                }
+            }
+            else
+                areg[q] = *reinterpret_cast<const v4i_bq*>(a + (size_t)rr * a_stride + (ok ? k : 0));
         }
     }
     // (2) descales of the wavefront's blocks: float4 number j of them is (block j / 4, row group j % 4); with blocks of 32,
@@ -867,6 +973,32 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
             const int r = idx / (NB * 8), v = idx - r * (NB * 8);
             const int k = kb_base * 64 + v * 8;
             const bool ok = v < nkb * 8 && k < K;
+            if (F32)
+            {
+                // 8 floats -> 8 bf16 in each of the three planes; lanes beyond the rows' vectors store into the padding behind row 0
+                const bool spare = idx >= MT * NB * 8;
+                unsigned char* dst = my_a + (spare ? NB * 128 : r * ACT_PITCH + v * 16);
+                v4i_bq pl[3];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                {
+                    unsigned h[2][3];
+#pragma unroll
+                    for (int o = 0; o < 2; o++)
+                    {
+                        const int j = 2 * e + o; // element of the vector
+                        float x = __int_as_float(j < 4 ? areg[q][j & 3] : areg2[F32 ? q : 0][j & 3]);
+                        if (INSC) x = mul_rn(x, __int_as_float(j < 4 ? sreg[INSC ? q : 0][j & 3] : sreg2[INSC ? q : 0][j & 3]));
+                        x = ok ? x : 0.f;
+                        split_bf16x3(x, h[o][0], h[o][1], h[o][2]);
+                    }
+#pragma unroll
+                    for (int pnum = 0; pnum < 3; pnum++) pl[pnum][e] = (int)((h[0][pnum] >> 16) | h[1][pnum]);
+                }
+#pragma unroll
+                for (int pnum = 0; pnum < 3; pnum++) *reinterpret_cast<v4i_bq*>(dst + pnum * PLANE_BYTES) = pl[pnum];
+                continue;
+            }
             v4i_bq t = areg[q];
 #pragma unroll
             for (int e = 0; e < 4; e++) t[e] = ok ? t[e] : 0;
@@ -881,10 +1013,66 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
     constexpr int A_LANE = HALVES ? 16 : 32; // bytes from one K group's operand to the next inside a staged row
     constexpr int A_SECOND = HALVES ? 64 : 16; // and from the first instruction's operand to the second's
     const unsigned char* act_rd = ACT_LDS ? my_a + (m < M && m < MT ? m : 0) * ACT_PITCH + kg * A_LANE : my_a + m * TR_PITCH + kg * A_LANE;
+    if (F32)
+    {
+        static_assert(!F32 || MT <= 5, "three columns per row, 16 columns");
+        const int prow = m / 3, ppl = m - prow * 3;
+        const bool used = prow < M && prow < MT;
+        act_rd = my_a + (used ? ppl * PLANE_BYTES + prow * ACT_PITCH : 0) + kg * A_LANE;
+    }
     unsigned char* tr_wr = my_a + tr_row * TR_PITCH + tr_piece * 16;
 #pragma unroll
     for (int i = 0; i < NB; i++)
     {
+        if (F32)
+        {
+            v8bf fa, fb;
+            if (BITS == 8)
+            {
+                fa = bytes_to_bf16((unsigned)w[BITS == 8 ? i : 0][0], (unsigned)w[BITS == 8 ? i : 0][1]);
+                fb = bytes_to_bf16((unsigned)w[BITS == 8 ? i : 0][2], (unsigned)w[BITS == 8 ? i : 0][3]);
+            }
+            else if (BITS == 4)
+            {
+                fa = nibbles_to_bf16((unsigned)w2[BITS != 8 ? i : 0][0]);
+                fb = nibbles_to_bf16((unsigned)w2[BITS != 8 ? i : 0][1]);
+            }
+            else
+                sixbit_to_bf16((unsigned)w2[BITS != 8 ? i : 0][0], (unsigned)w2[BITS != 8 ? i : 0][1], (unsigned)w1[BITS == 6 ? i : 0], fa, fb);
+            // column l%16 of the matrix-core product is (row, plane) = ((l%16) / 3, (l%16) % 3): the three partial products of a row
+            // come out of the same two instructions, side by side, and are added at the very end
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            union
+            {
+                v4i_bq i4;
+                v8bf h;
+            } ya, yb;
+            ya.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128);
+            yb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + i * 128 + A_SECOND);
+            v4f t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, ya.h, zero, 0, 0, 0), t1 = zero;
+            if (HALVES)
+                t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb, yb.h, zero, 0, 0, 0);
+            else
+                t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb, yb.h, t0, 0, 0, 0);
+            if (HALVES)
+            {
+                const float4 da = my_d[i * dper + kg];
+                const float4 db = my_d[i * dper + (split << 2) + kg];
+                acc[0] = fmaf(t1[0], db.x, fmaf(t0[0], da.x, acc[0]));
+                acc[1] = fmaf(t1[1], db.y, fmaf(t0[1], da.y, acc[1]));
+                acc[2] = fmaf(t1[2], db.z, fmaf(t0[2], da.z, acc[2]));
+                acc[3] = fmaf(t1[3], db.w, fmaf(t0[3], da.w, acc[3]));
+            }
+            else
+            {
+                const float4 d = my_d[i * 4 + kg];
+                acc[0] = fmaf(t0[0], d.x, acc[0]);
+                acc[1] = fmaf(t0[1], d.y, acc[1]);
+                acc[2] = fmaf(t0[2], d.z, acc[2]);
+                acc[3] = fmaf(t0[3], d.w, acc[3]);
+            }
+            continue;
+        }
         v8h wa, wb;
         if (BITS == 8)
         {
@@ -950,14 +1138,36 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
     __syncthreads();
     if (wave == 0 && m < M)
     {
-        float4 f = red[lane];
+        // fp32 activations: lane (l/16, row) adds the row's three columns, each summed over the wavefronts first
+        const int src = F32 ? (lane & 48) + m * 3 : lane;
+        float4 f = red[src];
         for (int w2 = 1; w2 < nwaves; w2++)
         {
-            const float4 o = red[w2 * 64 + lane];
+            const float4 o = red[w2 * 64 + src];
             f.x = add_rn(f.x, o.x);
             f.y = add_rn(f.y, o.y);
             f.z = add_rn(f.z, o.z);
             f.w = add_rn(f.w, o.w);
+        }
+        if (F32)
+        {
+#pragma unroll
+            for (int pnum = 1; pnum < 3; pnum++)
+            {
+                float4 g = red[src + pnum];
+                for (int w2 = 1; w2 < nwaves; w2++)
+                {
+                    const float4 o = red[w2 * 64 + src + pnum];
+                    g.x = add_rn(g.x, o.x);
+                    g.y = add_rn(g.y, o.y);
+                    g.z = add_rn(g.z, o.z);
+                    g.w = add_rn(g.w, o.w);
+                }
+                f.x = add_rn(f.x, g.x);
+                f.y = add_rn(f.y, g.y);
+                f.z = add_rn(f.z, g.z);
+                f.w = add_rn(f.w, g.w);
+            }
         }
         const float fr[4] = {f.x, f.y, f.z, f.w};
 #pragma unroll
@@ -975,13 +1185,14 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const __
 }
 
 // One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
-template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS>
-static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
-                              const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN, bool INSC>
+static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
+                              const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream,
+                              bool* handled)
 {
     constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;
-    constexpr int AROWS = ACT_LDS ? (AV * 64 + NB * 8 - 1) / (NB * 8) : 0;
-    const int WAVE_BYTES = (HALVES ? 1024 << split : 1024) + (ACT_LDS ? AROWS * (NB * 128 + 128) : 16 * 144);
+    constexpr int AROWS = ACT_LDS ? (AIN == 4 ? MT : (AV * 64 + NB * 8 - 1) / (NB * 8)) : 0;
+    const int WAVE_BYTES = (HALVES ? 1024 << split : 1024) + (ACT_LDS ? (AIN == 4 ? 3 : 1) * AROWS * (NB * 128 + 128) : 16 * 144);
     const int nwaves = (kblocks + NB - 1) / NB;
     const size_t lds = (size_t)nwaves * WAVE_BYTES; // >= 1 KB per wavefront, which the final exchange reuses
     if (lds > 160 * 1024)
@@ -989,7 +1200,7 @@ static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, in
         *handled = false;
         return NCNNHIP_OK;
     }
-    auto kernel = blockquant8_upfront_kernel<BITS, HALVES, NB, MAXW, MT, ACT_LDS>;
+    auto kernel = blockquant8_upfront_kernel<BITS, HALVES, NB, MAXW, MT, ACT_LDS, AIN, INSC>;
     if (lds > 65536)
     {
         // more than the 64 KB a kernel gets by default: raise this kernel's limit once (the chip has 160 KB per compute unit)
@@ -1000,53 +1211,64 @@ static int launch_upfront_one(const __half* a, size_t a_stride, int M, int N, in
             raised = true;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, c, bt, alpha, beta, out,
-                       out_stride);
+    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta,
+                       out, out_stride);
     return launch_status("blockquant8_upfront_kernel");
 }
 
-// handled = false: the shape is left to the caller (K beyond 16384, or more than 4 rows with K beyond 8192)
-template<int BITS, bool HALVES>
-static int launch_blockquant8_upfront(const __half* a, size_t a_stride, int M, int N, int K, const unsigned char* wpk, const float4* dpk, int split,
-                                      const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream, bool* handled)
+// handled = false: the shape is left to the caller (K beyond 16384; fp16: more than 4 rows with K beyond 8192; fp32: more than 4 rows,
+// or rows whose three planes do not fit in LDS together: the caller then passes fewer rows)
+template<int BITS, bool HALVES, int AIN, bool INSC>
+static int launch_blockquant8_upfront(const void* a, size_t a_stride, int M, int N, int K, const unsigned char* wpk, const float4* dpk, int split,
+                                      const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride,
+                                      hipStream_t stream, bool* handled)
 {
     const int kblocks = (K + 63) / 64;
     *handled = true;
 #define UPFRONT(NB_, MAXW_, MT_, LDS_) \
-    return launch_upfront_one<BITS, HALVES, NB_, MAXW_, MT_, LDS_>(a, a_stride, M, N, K, kblocks, wpk, dpk, split, c, bt, alpha, beta, out, out_stride, stream, \
-                                                                    handled)
+    return launch_upfront_one<BITS, HALVES, NB_, MAXW_, MT_, LDS_, AIN, INSC>(a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta, out, \
+                                                                              out_stride, stream, handled)
     if (M <= 4)
     {
         // decoding: 8 steps per wavefront while 8 or 16 wavefronts cover K (K up to 8192; measured against 16 steps on half
         // as many wavefronts: the same at 4096 x 4096, 3-6 % faster from 11008 rows up), then 12 and 16 steps on 16 wavefronts
-        // (K = 11008: 15 wavefronts of 12).  Two rows run as four in the halves layout (fewer kernels to build; the
-        // staging reads row 0 again for the missing ones).
+        // (K = 11008: 15 wavefronts of 12).  Two rows run as four in the halves layout with fp16 activations (fewer kernels
+        // to build; the staging reads row 0 again for the missing ones); with fp32 activations two rows have a kernel of their
+        // own, because LDS holds three planes per row.
+        constexpr bool TWO = !HALVES || AIN == 4;
+        constexpr bool F32 = AIN == 4; // its three planes per row: four rows fit up to K = 4096, two up to 8192, one beyond (no kernels built for the rest)
         if (kblocks <= 64)
         {
             if (M == 1) UPFRONT(8, 8, 1, true);
-            if constexpr (!HALVES) { if (M == 2) UPFRONT(8, 8, 2, true); }
+            if constexpr (TWO) { if (M == 2) UPFRONT(8, 8, 2, true); }
             UPFRONT(8, 8, 4, true);
         }
         if (kblocks <= 128)
         {
             if (M == 1) UPFRONT(8, 16, 1, true);
-            if constexpr (!HALVES) { if (M == 2) UPFRONT(8, 16, 2, true); }
-            UPFRONT(8, 16, 4, true);
+            if constexpr (TWO) { if (M == 2) UPFRONT(8, 16, 2, true); }
+            if constexpr (!F32) UPFRONT(8, 16, 4, true);
         }
-        if (kblocks <= 192)
+        else if (kblocks <= 192)
         {
             if (M == 1) UPFRONT(12, 16, 1, true);
-            if constexpr (!HALVES) { if (M == 2) UPFRONT(12, 16, 2, true); }
-            UPFRONT(12, 16, 4, true);
+            if constexpr (!F32)
+            {
+                if constexpr (TWO) { if (M == 2) UPFRONT(12, 16, 2, true); }
+                UPFRONT(12, 16, 4, true);
+            }
         }
-        if (kblocks <= 256)
+        else if (kblocks <= 256)
         {
             if (M == 1) UPFRONT(16, 16, 1, true);
-            if constexpr (!HALVES) { if (M == 2) UPFRONT(16, 16, 2, true); }
-            UPFRONT(16, 16, 4, true);
+            if constexpr (!F32)
+            {
+                if constexpr (TWO) { if (M == 2) UPFRONT(16, 16, 2, true); }
+                UPFRONT(16, 16, 4, true);
+            }
         }
     }
-    else
+    else if constexpr (AIN == 2)
     {
         // up to 12 VGPRs per step (weights and the 16 rows' activations): 8 steps per wavefront, up to 16 wavefronts
         // (7.7 -> 6.7 us at 4096 x 4096 against 16 steps on 4 wavefronts)
@@ -1218,23 +1440,24 @@ int ncnnhip_blockquant_pack(const uint8_t* b_host, const float* scales_host, int
     return NCNNHIP_OK;
 }
 
-int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
-                                        const float* packed_descale_dev, int bits, int block, const float* c_dev, int broadcast_type_c, float alpha,
-                                        float beta, float* out_dev, size_t out_stride, void* stream)
+// shared body of the two packed entry points; ain = 2 (fp16 activations) or 4 (fp32)
+static int gemm_blockquant_packed(const char* who, const void* a_dev, int ain, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
+                                  const float* packed_descale_dev, int bits, int block, const float* in_scales_dev, const float* c_dev, int broadcast_type_c,
+                                  float alpha, float beta, float* out_dev, size_t out_stride, void* stream)
 {
-    NCNNHIP_REQUIRE(a_dev && packed_w_dev && packed_descale_dev && out_dev, "ncnnhip_gemm_blockquant_packed_f16a: null pointer");
-    NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1 && K % 16 == 0, "ncnnhip_gemm_blockquant_packed_f16a: bad shape %d %d %d (K must be a multiple of 16)", M, N, K);
-    NCNNHIP_REQUIRE(bits == 4 || bits == 6 || bits == 8, "ncnnhip_gemm_blockquant_packed_f16a: weight bits %d", bits);
-    NCNNHIP_REQUIRE(block == 32 || block == 64 || block == 128, "ncnnhip_gemm_blockquant_packed_f16a: block size %d", block);
-    NCNNHIP_REQUIRE(a_stride >= (size_t)K && a_stride % 8 == 0 && al16(a_dev), "ncnnhip_gemm_blockquant_packed_f16a: activation rows must be 16-byte aligned");
-    NCNNHIP_REQUIRE(out_stride >= (size_t)N, "ncnnhip_gemm_blockquant_packed_f16a: output stride too small");
+    NCNNHIP_REQUIRE(a_dev && packed_w_dev && packed_descale_dev && out_dev, "%s: null pointer", who);
+    NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1 && K % 16 == 0, "%s: bad shape %d %d %d (K must be a multiple of 16)", who, M, N, K);
+    NCNNHIP_REQUIRE(bits == 4 || bits == 6 || bits == 8, "%s: weight bits %d", who, bits);
+    NCNNHIP_REQUIRE(block == 32 || block == 64 || block == 128, "%s: block size %d", who, block);
+    NCNNHIP_REQUIRE(a_stride >= (size_t)K && a_stride % (16 / ain) == 0 && al16(a_dev), "%s: activation rows must be 16-byte aligned", who);
+    NCNNHIP_REQUIRE(!in_scales_dev || al16(in_scales_dev), "%s: input scales must be 16-byte aligned", who);
+    NCNNHIP_REQUIRE(out_stride >= (size_t)N, "%s: output stride too small", who);
     const int bt = c_dev ? broadcast_type_c : -1;
-    NCNNHIP_REQUIRE(bt >= -1 && bt <= 4, "ncnnhip_gemm_blockquant_packed_f16a: C broadcast %d", bt);
-    NCNNHIP_REQUIRE((size_t)(K + 63) / 64 * 64 <= 60 * 1024, "ncnnhip_gemm_blockquant_packed_f16a: K %d too large for the descale stage", K);
+    NCNNHIP_REQUIRE(bt >= -1 && bt <= 4, "%s: C broadcast %d", who, bt);
+    NCNNHIP_REQUIRE((size_t)(K + 63) / 64 * 64 <= 60 * 1024, "%s: K %d too large for the descale stage", who, K);
     const bool halves = halves_layout(bits, block);
-    NCNNHIP_REQUIRE(!halves || K <= 16384, "ncnnhip_gemm_blockquant_packed_f16a: %d-bit fields in blocks of %d need K <= 16384, got %d", bits, block, K);
+    NCNNHIP_REQUIRE(!(halves || ain == 4) || K <= 16384, "%s: K %d beyond 16384 has a kernel only for 8-bit fields in blocks of 64 or 128 with fp16 activations", who, K);
     const int tiles = (N + 15) / 16, kblocks = (K + 63) / 64;
-    const __half* ah = reinterpret_cast<const __half*>(a_dev);
     const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
     const int split = block == 32 ? 1 : 0;
     hipStream_t st = as_stream(stream);
@@ -1243,41 +1466,55 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
         const float* cc = c_dev;
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
-        const __half* ap = ah + (size_t)m0 * a_stride;
+        const void* ap = static_cast<const char*>(a_dev) + (size_t)m0 * a_stride * ain;
         float* op = out_dev + (size_t)m0 * out_stride;
-        if (!halves) return launch_blockquant8_upfront<8, false>(ap, a_stride, mc, N, K, packed_w_dev, dpk, 0, cc, bt, alpha, beta, op, out_stride, st, handled);
-        if (bits == 8) return launch_blockquant8_upfront<8, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
-        if (bits == 6) return launch_blockquant8_upfront<6, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
-        return launch_blockquant8_upfront<4, true>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, cc, bt, alpha, beta, op, out_stride, st, handled);
+#define UP(BITS_, HALVES_, AIN_, INSC_) \
+    return launch_blockquant8_upfront<BITS_, HALVES_, AIN_, INSC_>(ap, a_stride, mc, N, K, packed_w_dev, dpk, split, in_scales_dev, cc, bt, alpha, beta, op, out_stride, \
+                                                                   st, handled)
+#define UP_BITS(AIN_, INSC_)                 \
+    if (!halves) UP(8, false, AIN_, INSC_);  \
+    if (bits == 8) UP(8, true, AIN_, INSC_); \
+    if (bits == 6) UP(6, true, AIN_, INSC_); \
+    UP(4, true, AIN_, INSC_)
+        if (ain == 2)
+        {
+            UP_BITS(2, false);
+        }
+        if (in_scales_dev)
+        {
+            UP_BITS(4, true);
+        }
+        UP_BITS(4, false);
+#undef UP_BITS
+#undef UP
     };
-    for (int m0 = 0; m0 < M; m0 += 16)
+    const int pass = ain == 4 ? 4 : 16; // rows per pass at most
+    for (int m0 = 0; m0 < M; m0 += pass)
     {
-        const int mc = M - m0 < 16 ? M - m0 : 16;
+        const int mc = M - m0 < pass ? M - m0 : pass;
         bool handled = false;
         int ret = upfront(m0, mc, &handled);
         if (ret != NCNNHIP_OK) return ret;
         if (handled) continue;
-        if (halves)
+        if (halves || ain == 4)
         {
-            // long rows with more than four activation rows: four at a time, or one at a time where four rows of K and the
-            // descales of blocks of 32 do not fit in LDS together (K beyond 12288)
+            // rows that do not fit in LDS together (long K; fp32: three planes per row): four, two, one at a time
             for (int m1 = m0; m1 < m0 + mc;)
             {
-                const int left = m0 + mc - m1;
-                ret = upfront(m1, left < 4 ? left : 4, &handled);
-                if (ret != NCNNHIP_OK) return ret;
-                if (handled)
+                int rows = m0 + mc - m1 < 4 ? m0 + mc - m1 : 4;
+                for (;;)
                 {
-                    m1 += 4;
-                    continue;
+                    ret = upfront(m1, rows, &handled);
+                    if (ret != NCNNHIP_OK) return ret;
+                    if (handled || rows == 1) break;
+                    rows = rows > 2 ? 2 : 1;
                 }
-                ret = upfront(m1, 1, &handled);
-                if (ret != NCNNHIP_OK) return ret;
-                NCNNHIP_REQUIRE(handled, "ncnnhip_gemm_blockquant_packed_f16a: no kernel for M %d K %d", M, K);
-                m1 += 1;
+                NCNNHIP_REQUIRE(handled, "%s: no kernel for M %d K %d", who, M, K);
+                m1 += rows;
             }
             continue;
         }
+        const __half* ah = static_cast<const __half*>(a_dev);
         const float* cc = c_dev;
         if (cc && (bt == 1 || bt == 2)) cc += m0;
         if (cc && bt == 3) cc += (size_t)m0 * N;
@@ -1292,6 +1529,27 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
                                out_dev + (size_t)m0 * out_stride, out_stride);
     }
     return launch_status("blockquant8_mfma_kernel");
+}
+
+int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
+                                        const float* packed_descale_dev, int bits, int block, const float* c_dev, int broadcast_type_c, float alpha,
+                                        float beta, float* out_dev, size_t out_stride, void* stream)
+{
+    return gemm_blockquant_packed("ncnnhip_gemm_blockquant_packed_f16a", a_dev, 2, a_stride, M, N, K, packed_w_dev, packed_descale_dev, bits, block, 0, c_dev,
+                                  broadcast_type_c, alpha, beta, out_dev, out_stride, stream);
+}
+
+int ncnnhip_gemm_blockquant_packed_supported(int K)
+{
+    return K >= 1 && K % 16 == 0 && K <= 16384;
+}
+
+int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev, const float* packed_descale_dev,
+                                   int bits, int block, const float* in_scales_dev, const float* c_dev, int broadcast_type_c, float alpha, float beta,
+                                   float* out_dev, size_t out_stride, void* stream)
+{
+    return gemm_blockquant_packed("ncnnhip_gemm_blockquant_packed", a_dev, 4, a_stride, M, N, K, packed_w_dev, packed_descale_dev, bits, block, in_scales_dev,
+                                  c_dev, broadcast_type_c, alpha, beta, out_dev, out_stride, stream);
 }
 
 int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* b_dev, int bits,

@@ -136,6 +136,9 @@ _SIGNATURES = {
     "ncnnhip_blockquant_pack": [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_blockquant_packed_f16a": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                             C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_blockquant_packed_supported": [C.c_int],
+    "ncnnhip_gemm_blockquant_packed": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                       C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_peak_launch_chain": [C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_mfma_i8": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_hbm_read": [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p],
@@ -686,12 +689,20 @@ class Runtime:
         check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, bits, block, pw.ctypes.data, pd.ctypes.data))
         return pw, pd
 
-    def gemm_blockquant_packed(self, a_half, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64):
-        a_half = np.ascontiguousarray(a_half, np.float16)
-        m, k = a_half.shape
-        da, dw_, dd = self.up(a_half), self.up(pw), self.up(pd)
+    def gemm_blockquant_packed(self, a, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64, in_scales=None):
+        """a fp16: the fp16-activation entry point; a fp32 (optionally with in_scales): the layer's contract, activations split into three bf16."""
+        half = a.dtype == np.float16
+        a = np.ascontiguousarray(a, np.float16 if half else np.float32)
+        m, k = a.shape
+        da, dw_, dd = self.up(a), self.up(pw), self.up(pd)
         dc = self.up(None if c is None else np.asarray(c, np.float32))
         dout = DeviceBuffer.empty((m, n), np.float32)
-        check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dc),
-                                                        broadcast_type_c if c is not None else -1, alpha, beta, dout.ptr, n, self.stream))
+        bt = broadcast_type_c if c is not None else -1
+        if half:
+            assert in_scales is None
+            check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dc), bt, alpha, beta, dout.ptr, n, self.stream))
+        else:
+            dis = self.up(None if in_scales is None else np.asarray(in_scales, np.float32))
+            check(lib().ncnnhip_gemm_blockquant_packed(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dis), _ptr(dc), bt, alpha, beta, dout.ptr, n,
+                                                       self.stream))
         return dout.to_numpy(self.stream)

@@ -35,7 +35,7 @@ Gemm_hip::Gemm_hip()
     support_inplace = false;
     weight_block_quantize = 0;
     B_data_int8_scale = 1.f;
-    d_A = d_B = d_B_tiled = d_C = d_A_scales = d_B_scale = d_B_block_scales = d_B_input_scales = 0;
+    d_A = d_B = d_B_tiled = d_C = d_A_scales = d_B_scale = d_B_block_scales = d_B_input_scales = d_B_packed = d_B_packed_descales = 0;
     b_ready_int8 = 0;
 }
 
@@ -176,6 +176,10 @@ int Gemm_hip::create_pipeline(const Option&)
         ret = upload_constant(B_data.data, (size_t)B_data.w * B_data.h, &d_B);
         if (ret == 0) ret = upload_constant(B_data_quantize_scales.data, B_data_quantize_scales.total() * 4, &d_B_block_scales);
         if (ret == 0 && !B_data_input_scales.empty()) ret = upload_constant(B_data_input_scales.data, (size_t)constantK * 4, &d_B_input_scales);
+        // second form of B for few activation rows (decoding): matrix-core tiles
+        if (ret == 0)
+            ret = upload_blockquant_packed(B_data.data, (const float*)B_data_quantize_scales.data, constantN, constantK, term_bits(quantize_term),
+                                           term_block(quantize_term), &d_B_packed, &d_B_packed_descales);
     }
     else if (ret == 0 && constantB == 1)
     {
@@ -220,7 +224,7 @@ int Gemm_hip::create_pipeline(const Option&)
 
 int Gemm_hip::destroy_pipeline(const Option&)
 {
-    void** all[] = {&d_A, &d_B, &d_B_tiled, &d_C, &d_A_scales, &d_B_scale, &d_B_block_scales, &d_B_input_scales};
+    void** all[] = {&d_A, &d_B, &d_B_tiled, &d_C, &d_A_scales, &d_B_scale, &d_B_block_scales, &d_B_input_scales, &d_B_packed, &d_B_packed_descales};
     for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++)
     {
         if (*all[i]) ncnnhip_free(*all[i]);
@@ -285,8 +289,8 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
     int rc = 0;
     if (weight_block_quantize)
     {
-        rc = ncnnhip_gemm_blockquant((const float*)A.data, (size_t)K, M, N, K, (const uint8_t*)d_B, term_bits(quantize_term), term_block(quantize_term),
-                                     (const float*)d_B_block_scales, (const float*)d_B_input_scales, d_c, bt, alpha, beta, (float*)top.data, (size_t)N, st);
+        rc = blockquant_gemm_device((const float*)A.data, (size_t)K, M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
+                                    d_B_input_scales, d_B_packed, d_B_packed_descales, d_c, bt, alpha, beta, (float*)top.data, (size_t)N, st);
         return to_ncnn_status(rc, "ncnnhip_gemm_blockquant");
     }
     if (!b_ready_int8)
@@ -575,9 +579,8 @@ int Gemm_hip::forward_block_quantize(const std::vector<Mat>& bottom_blobs, std::
             d_c = (const float*)p;
         }
     }
-    rc = ncnnhip_gemm_blockquant((const float*)d_a, mat_row_stride(A), M, N, K, (const uint8_t*)d_B, term_bits(quantize_term), term_block(quantize_term),
-                                 (const float*)d_B_block_scales, (const float*)d_B_input_scales, d_c, d_c ? bt : -1, alpha, beta, (float*)d_out,
-                                 (size_t)N, st);
+    rc = blockquant_gemm_device((const float*)d_a, mat_row_stride(A), M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
+                                d_B_input_scales, d_B_packed, d_B_packed_descales, d_c, d_c ? bt : -1, alpha, beta, (float*)d_out, (size_t)N, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_blockquant");
     rc = ncnnhip_memcpy_d2h(top.data, d_out, (size_t)M * N * 4, st);
     if (rc == 0) rc = ncnnhip_stream_synchronize(st);

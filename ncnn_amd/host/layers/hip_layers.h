@@ -126,6 +126,8 @@ private:
     void* d_B_scale;  // [1]
     void* d_B_block_scales;
     void* d_B_input_scales;
+    void* d_B_packed;          // block-quantised B as matrix-core tiles + its descales (null when K has no kernel for them)
+    void* d_B_packed_descales;
     int b_ready_int8; // constant B sits on the device quantised and transposed
 };
 
@@ -150,7 +152,7 @@ public:
     ncnn::Mat weight_data[4], bias_data[4], weight_data_quantize_scales[4], weight_data_input_scales[4];
 
 private:
-    void* dev[4][4]; // per projection: packed weights, block scales, input scales (or 0), bias
+    void* dev[4][6]; // per projection: weight fields, block scales, input scales (or 0), bias, matrix-core tiles and their descales (or 0)
 };
 
 ncnn::Layer* MultiHeadAttention_hip_creator(void* userdata);

@@ -2,6 +2,9 @@
 
 #include "../ncnn/platform.h"
 
+#include <stdint.h>
+#include <vector>
+
 namespace ncnn_amd {
 
 HipBlobAllocator::HipBlobAllocator()
@@ -43,6 +46,42 @@ int upload_constant(const void* host, size_t bytes, void** dev)
     rc = ncnnhip_memcpy_h2d(*dev, host, bytes, 0);
     if (rc == 0) rc = ncnnhip_stream_synchronize(0);
     return to_ncnn_status(rc, "upload_constant");
+}
+
+int upload_blockquant_packed(const void* fields_host, const float* scales_host, int n, int k, int bits, int block, void** d_packed, void** d_descales)
+{
+    *d_packed = 0;
+    *d_descales = 0;
+    if (!ncnnhip_gemm_blockquant_packed_supported(k)) return 0;
+    size_t wb = 0, db = 0;
+    if (ncnnhip_blockquant_packed_size(n, k, bits, block, &wb, &db) != 0) return 0;
+    std::vector<uint8_t> pw(wb);
+    std::vector<float> pd(db / sizeof(float));
+    int rc = ncnnhip_blockquant_pack((const uint8_t*)fields_host, scales_host, n, k, bits, block, pw.data(), pd.data());
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_blockquant_pack");
+    int ret = upload_constant(pw.data(), wb, d_packed);
+    if (ret == 0) ret = upload_constant(pd.data(), db, d_descales);
+    if (ret != 0)
+    {
+        if (*d_packed) ncnnhip_free(*d_packed);
+        if (*d_descales) ncnnhip_free(*d_descales);
+        *d_packed = 0;
+        *d_descales = 0;
+    }
+    return ret;
+}
+
+int blockquant_gemm_device(const float* a_dev, size_t a_stride, int M, int N, int K, const void* d_fields, int bits, int block, const void* d_scales,
+                           const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt, float alpha, float beta,
+                           float* out_dev, size_t out_stride, void* stream)
+{
+    // few rows: the packed tiles (one pass over the weights per four rows at most); from 32 rows up the fp32 matrix-core kernel of the
+    // .bin layout does all rows in one pass
+    if (d_packed && d_descales && M < 32 && a_stride % 4 == 0 && ((uintptr_t)a_dev & 15) == 0 && (!d_in_scales || ((uintptr_t)d_in_scales & 15) == 0))
+        return ncnnhip_gemm_blockquant_packed(a_dev, a_stride, M, N, K, (const uint8_t*)d_packed, (const float*)d_descales, bits, block,
+                                              (const float*)d_in_scales, c_dev, bt, alpha, beta, out_dev, out_stride, stream);
+    return ncnnhip_gemm_blockquant(a_dev, a_stride, M, N, K, (const uint8_t*)d_fields, bits, block, (const float*)d_scales, (const float*)d_in_scales, c_dev, bt,
+                                   alpha, beta, out_dev, out_stride, stream);
 }
 
 } // namespace ncnn_amd

@@ -64,6 +64,16 @@ int to_ncnn_status(int rc, const char* where);
 // constant table -> device (create_pipeline); *dev is freed with ncnnhip_free at destroy_pipeline
 int upload_constant(const void* host, size_t bytes, void** dev);
 
+// Block-quantised weights (fields [n][ceil(k*bits/8)] and scales [n][ceil(k/block)] as the .bin holds them) repacked into
+// matrix-core tiles and uploaded; both pointers stay null (and 0 is returned) when K has no kernel for that form.
+int upload_blockquant_packed(const void* fields_host, const float* scales_host, int n, int k, int bits, int block, void** d_packed, void** d_descales);
+
+// Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483) on device operands: the packed tiles for fewer than 32
+// activation rows when they exist and the rows are 16-byte aligned, else the .bin layout.  Returns an ncnnhip status.
+int blockquant_gemm_device(const float* a_dev, size_t a_stride, int M, int N, int K, const void* d_fields, int bits, int block, const void* d_scales,
+                           const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt, float alpha, float beta,
+                           float* out_dev, size_t out_stride, void* stream);
+
 // payload bytes of a Mat as it lies in memory (whole batch, including plane padding)
 static inline size_t mat_bytes(const ncnn::Mat& m)
 {

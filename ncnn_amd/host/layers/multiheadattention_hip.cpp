@@ -123,6 +123,13 @@ int MultiHeadAttention_hip::create_pipeline(const Option&)
         if (ret == 0) ret = upload_constant(weight_data_quantize_scales[i].data, (size_t)weight_data_quantize_scales[i].w * weight_data_quantize_scales[i].h * 4, &dev[i][1]);
         if (ret == 0 && !weight_data_input_scales[i].empty()) ret = upload_constant(weight_data_input_scales[i].data, (size_t)weight_data_input_scales[i].w * 4, &dev[i][2]);
         if (ret == 0) ret = upload_constant(bias_data[i].data, (size_t)bias_data[i].w * 4, &dev[i][3]);
+        // second form of the weights for few rows (decoding): matrix-core tiles
+        if (ret == 0)
+        {
+            const int in_dim[4] = {weight_data_size / embed_dim, kdim, vdim, embed_dim};
+            ret = upload_blockquant_packed(weight_data[i].data, (const float*)weight_data_quantize_scales[i].data, weight_data[i].h, in_dim[i],
+                                           att_bits(quantize_term), att_block(quantize_term), &dev[i][4], &dev[i][5]);
+        }
     }
     if (ret != 0) destroy_pipeline(Option());
     return ret;
@@ -131,7 +138,7 @@ int MultiHeadAttention_hip::create_pipeline(const Option&)
 int MultiHeadAttention_hip::destroy_pipeline(const Option&)
 {
     for (int i = 0; i < 4; i++)
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < 6; j++)
         {
             if (dev[i][j]) ncnnhip_free(dev[i][j]);
             dev[i][j] = 0;
@@ -235,8 +242,8 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
 
     int rc = ncnnhip_memcpy_h2d(d_q, q_blob.data, (size_t)src * qdim * 4, st);
     if (rc == 0)
-        rc = ncnnhip_gemm_blockquant(d_q, (size_t)qdim, src, embed_dim, qdim, (const uint8_t*)dev[0][0], bits, block, (const float*)dev[0][1], (const float*)dev[0][2],
-                                     (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
+        rc = blockquant_gemm_device(d_q, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
+                                    (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
 
     if (reuse_cache)
@@ -281,8 +288,8 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
             }
             float* d_aff = (float*)leases.get((size_t)cur * E * 4);
             if (!d_aff) return -100;
-            rc = ncnnhip_gemm_blockquant(d_in, (size_t)in_dim[t], cur, embed_dim, in_dim[t], (const uint8_t*)dev[1 + t][0], bits, block, (const float*)dev[1 + t][1],
-                                         (const float*)dev[1 + t][2], (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
+            rc = blockquant_gemm_device(d_in, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
+                                    (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
             if (rc == 0) rc = ncnnhip_transpose_f32(d_aff, E, cur, embed_dim, outT[t] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v projection");
         }
@@ -306,8 +313,8 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     if (att_ws_bytes && !att_ws) return -100;
     rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
-    rc = ncnnhip_gemm_blockquant(d_ctx, E, src, qdim, embed_dim, (const uint8_t*)dev[3][0], bits, block, (const float*)dev[3][1], (const float*)dev[3][2],
-                                 (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);
+    rc = blockquant_gemm_device(d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
+                                    (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);
     if (rc != 0) return to_ncnn_status(rc, "out projection");
     rc = ncnnhip_memcpy_d2h(top.data, d_out, (size_t)src * qdim * 4, st);
     if (rc == 0 && kv_cache && !reuse_cache)
@@ -432,8 +439,8 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     float* d_ctx = (float*)scratch.get((size_t)src * E * 4);
     if (!d_qa || !d_ctx) return -100;
 
-    rc = ncnnhip_gemm_blockquant((const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, (const uint8_t*)dev[0][0], bits, block, (const float*)dev[0][1],
-                                 (const float*)dev[0][2], (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
+    rc = blockquant_gemm_device((const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
+                                    (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
     if (!reuse_cache)
     {
@@ -450,8 +457,8 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         {
             float* d_aff = (float*)scratch.get((size_t)cur * E * 4);
             if (!d_aff) return -100;
-            rc = ncnnhip_gemm_blockquant((const float*)in[t]->data, (size_t)in_dim[t], cur, embed_dim, in_dim[t], (const uint8_t*)dev[1 + t][0], bits, block,
-                                         (const float*)dev[1 + t][1], (const float*)dev[1 + t][2], (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
+            rc = blockquant_gemm_device((const float*)in[t]->data, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
+                                    (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
             if (rc == 0) rc = ncnnhip_transpose_f32(d_aff, E, cur, embed_dim, outT[t] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v projection");
         }
@@ -463,8 +470,8 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     if (att_ws_bytes && !att_ws) return -100;
     rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
-    rc = ncnnhip_gemm_blockquant(d_ctx, E, src, qdim, embed_dim, (const uint8_t*)dev[3][0], bits, block, (const float*)dev[3][1], (const float*)dev[3][2],
-                                 (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);
+    rc = blockquant_gemm_device(d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
+                                    (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);
     if (rc != 0) return to_ncnn_status(rc, "out projection");
     if (kv_cache)
     {

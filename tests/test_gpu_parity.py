@@ -545,6 +545,57 @@ def test_blockquant_packed_low_bit_widths_and_blocks_of_32(rt, bits, block, m, n
     _bq_check(got, a, packed, scales, bits, block, None, c, bt, 0.75, 1.5)
 
 
+@pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
+    # fp32 activations on the packed weights (three bf16 planes): one, two and four rows per pass, more rows in several passes
+    (8, 64, 1, 512, 4096, -1, False), (8, 64, 2, 100, 4096, 4, True), (8, 64, 4, 256, 4096, 3, False), (8, 128, 3, 40, 4096, 1, True), (8, 64, 16, 64, 4096, 3, False),
+    (4, 64, 1, 256, 4096, -1, False), (4, 32, 4, 250, 4096, 4, True), (6, 64, 1, 128, 4096, -1, True), (6, 32, 3, 40, 4096, 2, False), (8, 32, 4, 64, 4096, -1, False),
+    (4, 128, 7, 40, 2048 + 48, 0, True),
+    # K up to 8192: two rows per pass; beyond: one; K that ends inside a step; a last wavefront without work
+    (8, 64, 4, 48, 8192, -1, False), (4, 64, 3, 33, 8192, 1, True), (8, 64, 2, 40, 11008, -1, False), (4, 32, 1, 40, 11008 + 16, 4, False), (6, 64, 4, 32, 12288, 3, True),
+    (8, 64, 1, 32, 16384, -1, False), (6, 128, 2, 20, 16384, 1, False), (8, 64, 3, 37, 208, 1, True), (4, 64, 1, 16, 64, 0, False), (8, 32, 2, 20, 1024 + 16, 3, False),
+    # many tiles
+    (8, 64, 1, 11008, 4096, -1, False), (4, 64, 4, 8200 + 5, 1024 + 64, 4, True)])
+def test_blockquant_packed_fp32_activations(rt, bits, block, m, n, k, bt, in_sc):
+    _say("blockquant packed fp32", bits, block, m, n, k, bt, in_sc)
+    from ncnn_amd import synth
+    a, packed, scales = synth.blockquant_operands(bits + block + m + n + k + 1, m, n, k, bits, block, half_exact=False)  # full fp32 mantissas
+    a[0, : min(k, 8)] = [3.0e-30, -1.5e30, 1.0, -1.0, 1.0 + 2.0 ** -23, 2.0 ** -100, 0.0, -7.25e12][: min(k, 8)]  # the far ends of the exponent range
+    rng = np.random.default_rng(bt + 52)
+    ins = rng.uniform(0.5, 1.5, k).astype(F) if in_sc else None
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+    got = rt.gemm_blockquant_packed(a, pw, pd, n, c, bt, 0.75, 1.5, bits=bits, block=block, in_scales=ins)
+    _bq_check(got, a, packed, scales, bits, block, ins, c, bt, 0.75, 1.5)
+
+
+@pytest.mark.parametrize("bits,block", [(8, 64), (8, 32), (6, 64), (4, 128)])
+def test_blockquant_packed_fp32_split_keeps_all_24_bits(rt, bits, block):
+    """One non-zero activation per row, power-of-two scales: an output is a single product x * q * 2^-2, known to float64
+    exactly, and the three partial products of the bf16 split add up with at most two roundings.  A split that lost its
+    lowest plane would be off by up to 2^-16, one that lost the middle plane by 2^-8; the sum's tolerance of the other
+    tests (1e-5 of sum |a w|) would not notice the former."""
+    k, n, m = 256, 48, 4
+    rng = np.random.default_rng(bits * 10 + block)
+    qmax = (1 << (bits - 1)) - 1
+    q = rng.integers(-qmax, qmax + 1, (n, k))
+    w = (q * 0.25).astype(F)  # quantises back to q with scale 4 when a block holds +-qmax; force that
+    w[:, ::block] = qmax * 0.25
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    assert np.all(scales == F(4.0))
+    qq = npref.blockquant_unpack_all(packed, k, bits)
+    a = np.zeros((m, k), F)
+    pos = [5, 64 + 40, 128 + 17, 255]
+    vals = [F(1.0) + F(2.0 ** -23), F(-3.1415927e-20), F(16777215.0 * 2.0 ** 40), F(0.7071068)]
+    for i in range(m):
+        a[i, pos[i]] = vals[i]
+    pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+    got = rt.gemm_blockquant_packed(a, pw, pd, n, bits=bits, block=block).astype(np.float64)
+    want = np.stack([float(vals[i]) * qq[:, pos[i]].astype(np.float64) * 0.25 for i in range(m)])
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -22), float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-300)))
+
+
 def test_blockquant_exact_on_power_of_two_data(rt):
     k, n, m = 128, 6, 2
     rng = np.random.default_rng(3)
