@@ -307,7 +307,8 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
         "config": {"workload": "block-quant Gemm M=%d N=%d K=%d, %d-bit weights in blocks of %d, fp32 block scales, %s activations" % (m, n, k, bits, block, args.act),
                    "weight_copies_rotated": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": measured_traffic("blockquant:%dx%dx%d" % (n, k, m)) if (half and bits == 8 and block == 64) else None,
+                     "traffic": measured_traffic("blockquant:%dx%dx%d%s%s" % (n, k, m, "" if (bits, block) == (8, 64) else ":%d:%d" % (bits, block),
+                                                                              "" if half else ":" + args.act)) if packed_form else None,
                      "kernel": "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
                      "bytes_per_launch": algo,
                      "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
