@@ -7,6 +7,8 @@
 #include <hip/hip_fp16.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace ncnnhip {
@@ -1184,6 +1186,181 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const vo
     }
 }
 
+// The 5-to-16-row form for many weight rows: one workgroup takes TWO neighbouring tiles of 16 weight rows and multiplies both
+// with the same activation registers.  A tile's 64 KB of weights at K = 4096 come with 128 KB of activations through the same
+// L1; sharing them between two tiles takes that from 192 to 128 KB per tile (fp16 activations, K up to 4096).
+template<int BITS, bool HALVES, int NB, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void blockquant8_rows16_pair_kernel(const __half* __restrict__ a, size_t a_stride, int M, int N, int K, int kblocks,
+                                                                            int ntiles, const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk,
+                                                                            int split, const float* __restrict__ c, int bt, float alpha, float beta,
+                                                                            float* __restrict__ out, size_t out_stride)
+{
+    static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_up[];
+    constexpr int TR_PITCH = 144; // one row of a step (128 bytes) + 16: 16 rows land on 16 different bank groups
+    const int D_BYTES = HALVES ? 1024 << split : 1024;
+    const int WAVE_BYTES = 2 * D_BYTES + 16 * TR_PITCH; // both tiles' descales, then the transpose buffer
+    constexpr int STEP_BYTES = 128 * BITS;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int tile0 = blockIdx.x * 2;
+    const int m = lane & 15;
+    const int kg = lane >> 4;
+
+    const int kb_begin = wave * NB;
+    int nkb = kblocks - kb_begin;
+    nkb = nkb > NB ? NB : nkb;
+    nkb = nkb < 0 ? 0 : nkb;
+    const int kb_base = nkb > 0 ? kb_begin : 0;
+
+    unsigned char* mine = lds_up + wave * WAVE_BYTES;
+    unsigned char* my_a = mine + 2 * D_BYTES;
+
+    // an odd tile count: the last workgroup's second tile reads the first one's operands again and stores nothing
+    const int dper = HALVES ? 4 << split : 4;
+    float4 dreg[2], dreg2[2];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+    {
+        const int tl = tile0 + tt < ntiles ? tile0 + tt : tile0;
+        const float4* dt = dpk + ((size_t)tl * kblocks + kb_base) * dper;
+        dreg[tt] = dt[lane < nkb * dper ? lane : 0];
+        dreg2[tt] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (HALVES) dreg2[tt] = dt[lane + 64 < nkb * dper ? lane + 64 : 0];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    v4i_bq w[BITS == 8 ? 2 * NB : 1];
+    v2i_bq w2[BITS != 8 ? 2 * NB : 1];
+    int w1[BITS == 6 ? 2 * NB : 1];
+    v4i_bq a0[NB], a1[NB];
+    const int tr_row = lane >> 3, tr_piece = lane & 7;
+    const __half* arow0 = a + (size_t)(tr_row < M ? tr_row : 0) * a_stride;
+    const __half* arow1 = a + (size_t)(tr_row + 8 < M ? tr_row + 8 : 0) * a_stride;
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+        {
+            const int tl = tile0 + tt < ntiles ? tile0 + tt : tile0;
+            const unsigned char* ws = wpk + ((size_t)tl * kblocks + kb_base + (i < nkb ? i : 0)) * STEP_BYTES;
+            if (BITS == 8)
+                w[BITS == 8 ? 2 * i + tt : 0] = __builtin_nontemporal_load(reinterpret_cast<const v4i_bq*>(ws) + lane);
+            else
+                w2[BITS != 8 ? 2 * i + tt : 0] = __builtin_nontemporal_load(reinterpret_cast<const v2i_bq*>(ws) + lane);
+            if (BITS == 6) w1[BITS == 6 ? 2 * i + tt : 0] = __builtin_nontemporal_load(reinterpret_cast<const int*>(ws + 512) + lane);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int k = (kb_base + (i < nkb ? i : 0)) * 64 + tr_piece * 8;
+        const int kk = k < K ? k : 0;
+        a0[i] = *reinterpret_cast<const v4i_bq*>(arow0 + kk);
+        a1[i] = *reinterpret_cast<const v4i_bq*>(arow1 + kk);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+    {
+        float4* my_d = reinterpret_cast<float4*>(mine + tt * D_BYTES);
+        my_d[lane] = lane < nkb * dper ? dreg[tt] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (HALVES && split) my_d[lane + 64] = lane + 64 < nkb * dper ? dreg2[tt] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    v4f acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    constexpr int A_LANE = HALVES ? 16 : 32;
+    constexpr int A_SECOND = HALVES ? 64 : 16;
+    const unsigned char* act_rd = my_a + m * TR_PITCH + kg * A_LANE;
+    unsigned char* tr_wr = my_a + tr_row * TR_PITCH + tr_piece * 16;
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        union
+        {
+            v4i_bq i4;
+            v8h h;
+        } xa, xb;
+        *reinterpret_cast<v4i_bq*>(tr_wr) = a0[i];
+        *reinterpret_cast<v4i_bq*>(tr_wr + 8 * TR_PITCH) = a1[i];
+        xa.i4 = *reinterpret_cast<const v4i_bq*>(act_rd);
+        xb.i4 = *reinterpret_cast<const v4i_bq*>(act_rd + A_SECOND);
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+        {
+            v8h wa, wb;
+            if (BITS == 8)
+            {
+                wa = bytes_to_halves(w[BITS == 8 ? 2 * i + tt : 0][0], w[BITS == 8 ? 2 * i + tt : 0][1]);
+                wb = bytes_to_halves(w[BITS == 8 ? 2 * i + tt : 0][2], w[BITS == 8 ? 2 * i + tt : 0][3]);
+            }
+            else if (BITS == 4)
+            {
+                wa = nibbles_to_halves((unsigned)w2[BITS != 8 ? 2 * i + tt : 0][0]);
+                wb = nibbles_to_halves((unsigned)w2[BITS != 8 ? 2 * i + tt : 0][1]);
+            }
+            else
+                sixbit_to_halves((unsigned)w2[BITS != 8 ? 2 * i + tt : 0][0], (unsigned)w2[BITS != 8 ? 2 * i + tt : 0][1], (unsigned)w1[BITS == 6 ? 2 * i + tt : 0], wa, wb);
+            const float4* my_d = reinterpret_cast<const float4*>(mine + tt * D_BYTES);
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            if (HALVES)
+            {
+                const v4f t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, zero, 0, 0, 0);
+                const v4f t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, zero, 0, 0, 0);
+                const float4 da = my_d[i * dper + kg];
+                const float4 db = my_d[i * dper + (split << 2) + kg];
+                acc[tt][0] = fmaf(t1[0], db.x, fmaf(t0[0], da.x, acc[tt][0]));
+                acc[tt][1] = fmaf(t1[1], db.y, fmaf(t0[1], da.y, acc[tt][1]));
+                acc[tt][2] = fmaf(t1[2], db.z, fmaf(t0[2], da.z, acc[tt][2]));
+                acc[tt][3] = fmaf(t1[3], db.w, fmaf(t0[3], da.w, acc[tt][3]));
+            }
+            else
+            {
+                v4f t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, xa.h, zero, 0, 0, 0);
+                t = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, xb.h, t, 0, 0, 0);
+                const float4 d = my_d[i * 4 + kg];
+                acc[tt][0] = fmaf(t[0], d.x, acc[tt][0]);
+                acc[tt][1] = fmaf(t[1], d.y, acc[tt][1]);
+                acc[tt][2] = fmaf(t[2], d.z, acc[tt][2]);
+                acc[tt][3] = fmaf(t[3], d.w, acc[tt][3]);
+            }
+        }
+    }
+
+    // combine the wavefronts' K ranges in wavefront order: wavefront 0 finishes the first tile, wavefront 1 the second
+    float4* red = reinterpret_cast<float4*>(lds_up);
+    __syncthreads();
+    red[wave * 64 + lane] = make_float4(acc[0][0], acc[0][1], acc[0][2], acc[0][3]);
+    red[(nwaves + wave) * 64 + lane] = make_float4(acc[1][0], acc[1][1], acc[1][2], acc[1][3]);
+    __syncthreads();
+    // (a single wavefront, K up to 512, finishes both)
+    for (int tt = wave; tt < 2 && m < M; tt += nwaves)
+    {
+        const float4* mr = red + tt * nwaves * 64;
+        float4 f = mr[lane];
+        for (int w2i = 1; w2i < nwaves; w2i++)
+        {
+            const float4 o = mr[w2i * 64 + lane];
+            f.x = add_rn(f.x, o.x);
+            f.y = add_rn(f.y, o.y);
+            f.z = add_rn(f.z, o.z);
+            f.w = add_rn(f.w, o.w);
+        }
+        const float fr[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int j = (tile0 + tt) * 16 + kg * 4 + r;
+            if (j < N)
+            {
+                float v = fr[r];
+                if (bt >= 0) v = add_rn(mul_rn(load_c(c, bt, m, j, N), beta), v);
+                out[(size_t)m * out_stride + j] = mul_rn(v, alpha);
+            }
+        }
+    }
+}
+
 // One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
 template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN, bool INSC>
 static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
@@ -1203,12 +1380,15 @@ static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int 
     auto kernel = blockquant8_upfront_kernel<BITS, HALVES, NB, MAXW, MT, ACT_LDS, AIN, INSC>;
     if (lds > 65536)
     {
-        // more than the 64 KB a kernel gets by default: raise this kernel's limit once (the chip has 160 KB per compute unit)
-        static bool raised = false;
-        if (!raised)
+        // more than the 64 KB a kernel gets by default: raise this kernel's limit once per device (the chip has 160 KB per compute
+        // unit).  The flags only ever go from 0 to 1 and the call may be repeated, so a race between two first callers is harmless.
+        static std::atomic<unsigned char> raised[64];
+        int device = 0;
+        NCNNHIP_CHECK(hipGetDevice(&device));
+        if (device < 0 || device >= 64 || !raised[device].load(std::memory_order_acquire))
         {
             NCNNHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            raised = true;
+            if (device >= 0 && device < 64) raised[device].store(1, std::memory_order_release);
         }
     }
     hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta,
@@ -1272,6 +1452,19 @@ static int launch_blockquant8_upfront(const void* a, size_t a_stride, int M, int
     {
         // up to 12 VGPRs per step (weights and the 16 rows' activations): 8 steps per wavefront, up to 16 wavefronts
         // (7.7 -> 6.7 us at 4096 x 4096 against 16 steps on 4 wavefronts)
+        const int ntiles = (N + 15) / 16;
+#ifndef BQ_PAIR_MIN_TILES
+#define BQ_PAIR_MIN_TILES 1024
+#endif
+        if (kblocks <= 64 && ntiles >= BQ_PAIR_MIN_TILES)
+        {
+            // many weight rows: two tiles per workgroup share the activation registers
+            const int nwaves = (kblocks + 7) / 8;
+            const size_t lds = (size_t)nwaves * (2 * (HALVES ? 1024 << split : 1024) + 16 * 144);
+            hipLaunchKernelGGL((blockquant8_rows16_pair_kernel<BITS, HALVES, 8, 8>), dim3((ntiles + 1) / 2), dim3(nwaves * 64), lds, stream,
+                               static_cast<const __half*>(a), a_stride, M, N, K, kblocks, ntiles, wpk, dpk, split, c, bt, alpha, beta, out, out_stride);
+            return launch_status("blockquant8_rows16_pair_kernel");
+        }
         if (kblocks <= 64) UPFRONT(8, 8, 1, false);
         if (kblocks <= 128) UPFRONT(8, 16, 1, false);
     }

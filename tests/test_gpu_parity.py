@@ -507,7 +507,9 @@ def test_blockquant_low_bit_decode_shape_fp16_activations(rt, bits):
                                             # 16 K blocks, a last wavefront with a single block and with none), rows through LDS (up to 4) and in registers (5 to 16),
                                             # and K beyond its reach (the ring kernel takes over)
                                             (2, 48, 8192, 64, -1), (1, 33, 12288, 64, 4), (3, 40, 11008 + 16, 64, 1), (4, 32, 16384, 128, -1), (1, 32, 16384 + 64, 64, -1),
-                                            (9, 40, 8192, 64, 1), (5, 24, 4096 + 64, 64, -1), (12, 40, 12288, 64, -1), (16, 4096, 4096, 64, 4), (2, 20, 1024 + 16, 64, 3)])
+                                            (9, 40, 8192, 64, 1), (5, 24, 4096 + 64, 64, -1), (12, 40, 12288, 64, -1), (16, 4096, 4096, 64, 4), (2, 20, 1024 + 16, 64, 3),
+                                            # from 1024 tiles up, 5 to 16 rows take two tiles per workgroup: an odd tile count with a ragged last tile, an even one, K inside a step
+                                            (16, 16384 + 11, 512, 64, 3), (9, 16384 + 32, 1024 + 48, 128, 4), (5, 16400, 4096, 64, -1)])
 def test_blockquant_packed_matrix_core_path(rt, m, n, k, block, bt):
     _say("blockquant packed", m, n, k, block, bt)
     a, packed, scales = cases.blockquant_case(m + n + k + block, m, n, k, 8, block)
@@ -530,8 +532,9 @@ def test_blockquant_packed_matrix_core_path(rt, m, n, k, block, bt):
     (4, 64, 3, 37, 208, 1), (6, 32, 1, 16, 64, 0), (8, 32, 2, 20, 1024 + 16, 3), (4, 128, 7, 100, 4096 + 48, -1), (6, 64, 12, 40, 8192, -1), (4, 32, 16, 64, 96, 2),
     # more than 16 rows (one pass per 16), and more than 4 rows with K beyond 8192 (four at a time)
     (4, 64, 20, 64, 1024, 2), (6, 32, 33, 40, 512, 3), (4, 64, 9, 40, 12288, 1), (6, 64, 16, 24, 16384, 3), (8, 32, 7, 40, 11008, 4),
-    # many tiles
-    (4, 64, 1, 11008, 4096, -1), (6, 64, 4, 8200 + 5, 1024 + 64, 4), (4, 32, 16, 9000, 512, 3)])
+    # many tiles; from 1024 up two tiles per workgroup at 5 to 16 rows
+    (4, 64, 1, 11008, 4096, -1), (6, 64, 4, 8200 + 5, 1024 + 64, 4), (4, 32, 16, 9000, 512, 3), (4, 64, 16, 16384 + 11, 512, -1), (6, 32, 7, 16400, 256 + 16, 3),
+    (8, 32, 12, 16384 + 40, 1024, 4)])
 def test_blockquant_packed_low_bit_widths_and_blocks_of_32(rt, bits, block, m, n, k, bt):
     _say("blockquant packed", bits, block, m, n, k, bt)
     from ncnn_amd import synth
