@@ -465,7 +465,8 @@ def bench_mha(args, embed, heads, src, past):
     for _ in range(4):
         w = rng.normal(0, 1.0 / np.sqrt(embed), (embed, embed)).astype(np.float32)
         packed, scales = synth.blockquant_weights(w, 8, 64)
-        ws.append((rt.up(packed), rt.up(scales), rt.up(rng.uniform(-0.1, 0.1, embed).astype(np.float32)), packed.nbytes + scales.nbytes))
+        pw, pd = rt.blockquant_pack(packed, scales, 64)  # the second form create_pipeline uploads: matrix-core tiles
+        ws.append((rt.up(packed), rt.up(scales), rt.up(rng.uniform(-0.1, 0.1, embed).astype(np.float32)), packed.nbytes + scales.nbytes, rt.up(pw), rt.up(pd)))
     d_x = rt.up(rng.normal(0, 1, (src, embed)).astype(np.float32))
     d_kt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
     d_vt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
@@ -475,13 +476,31 @@ def bench_mha(args, embed, heads, src, past):
     check(lib.ncnnhip_attention_workspace_bytes(heads, embed // heads, src, dst, C.byref(wsb)))
     d_ws = ncnn_amd.DeviceBuffer.empty((max(wsb.value, 4),), np.uint8)
 
+    # the projections as the layer dispatches them (blockquant_gemm_device): fewer than 32 rows on the packed tiles four rows per pass,
+    # 32 and more through the tiled bf16 kernel with its workspace; `--act fp32-bin` keeps the kernels of the .bin layout
+    packed_ok = args.act != "fp32-bin" and lib.ncnnhip_gemm_blockquant_packed_supported(embed)
+    rows_ws = None
+    if packed_ok and src >= 32:
+        rb = C.c_size_t()
+        check(lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(src, embed, C.byref(rb)))
+        rows_ws = (ncnn_amd.DeviceBuffer.empty((rb.value,), np.uint8), rb.value)
+
+    def project(x, w, alpha, out):
+        if rows_ws is not None:
+            check(lib.ncnnhip_gemm_blockquant_packed_rows(x.ptr, embed, src, embed, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed,
+                                                          rows_ws[0].ptr, rows_ws[1], st))
+        elif packed_ok:
+            check(lib.ncnnhip_gemm_blockquant_packed(x.ptr, embed, src, embed, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed, st))
+        else:
+            check(lib.ncnnhip_gemm_blockquant(x.ptr, embed, src, embed, embed, w[0].ptr, 8, 64, w[1].ptr, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed, st))
+
     def step():
-        check(lib.ncnnhip_gemm_blockquant(d_x.ptr, embed, src, embed, embed, ws[0][0].ptr, 8, 64, ws[0][1].ptr, None, ws[0][2].ptr, 4, scale, 1.0, d_qa.ptr, embed, st))
+        project(d_x, ws[0], scale, d_qa)
         for t, cache in ((1, d_kt), (2, d_vt)):
-            check(lib.ncnnhip_gemm_blockquant(d_x.ptr, embed, src, embed, embed, ws[t][0].ptr, 8, 64, ws[t][1].ptr, None, ws[t][2].ptr, 4, 1.0, 1.0, d_aff.ptr, embed, st))
+            project(d_x, ws[t], 1.0, d_aff)
             check(lib.ncnnhip_transpose_f32(d_aff.ptr, embed, src, embed, C.c_void_p(cache.ptr.value + past * 4), dst, st))
         check(lib.ncnnhip_attention_f32(d_qa.ptr, d_kt.ptr, d_vt.ptr, dst, None, 0, heads, embed // heads, src, dst, d_ctx.ptr, d_ws.ptr, wsb.value, st))
-        check(lib.ncnnhip_gemm_blockquant(d_ctx.ptr, embed, src, embed, embed, ws[3][0].ptr, 8, 64, ws[3][1].ptr, None, ws[3][2].ptr, 4, 1.0, 1.0, d_out.ptr, embed, st))
+        project(d_ctx, ws[3], 1.0, d_out)
 
     for _ in range(args.warmup):
         step()
@@ -504,7 +523,7 @@ def bench_mha(args, embed, heads, src, past):
         "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "self-attention layer, embed %d, %d heads, %d new tokens on a cache of %d, 8-bit block-quantised weights (blocks of 64)"
-                               % (embed, heads, src, past), "launches_per_step": 7, "device_ms_per_step": k_ms, "gflop": ops / 1e9},
+                               % (embed, heads, src, past), "launches_per_step": 11 if rows_ws is not None else 7, "projections": "tiled bf16x3 kernel" if rows_ws is not None else ("packed tiles" if packed_ok else ".bin layout"), "device_ms_per_step": k_ms, "gflop": ops / 1e9},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "whole layer (3 projections, 2 cache appends, attention core, output projection)", "bytes_per_launch": algo},
     }

@@ -382,6 +382,16 @@ int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, i
                                    const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
                                    size_t out_stride, void* stream);
 
+/* The same contract for many activation rows (prefill, attention projections): the three-way split is made once into
+ * the workspace (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: 6 bytes per activation, rows and K rounded up to 64),
+ * then a tiled Gemm runs on the bf16 matrix cores, 128 weight rows x 64 activation rows per workgroup.  K % 16 == 0; the
+ * workspace is scratch (overwritten by every call). */
+int ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(int M, int K, size_t* bytes);
+int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
+                                        const float* packed_descale_dev, int bits, int block, const float* in_scales_dev,
+                                        const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
+                                        size_t out_stride, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ attention
  * The core of MultiHeadAttention::forward_weight_block_quantize (src/layer/multiheadattention.cpp:776-866):
  * per head, scores = q k^T (+ mask), softmax over the keys, times v.  q (already scaled) and out are

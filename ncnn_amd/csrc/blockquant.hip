@@ -1361,6 +1361,297 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_rows16_pair_kernel(cons
     }
 }
 
+// ---- many activation rows (prefill, attention projections) on the packed weights, fp32 activations ------------------------
+// The same exact three-way bf16 split, made ONCE by a pass of its own into a workspace (three planes [rows][K], rows and K
+// padded with zeros to multiples of 64), then a tiled Gemm on v_mfma_f32_16x16x32_bf16: three bf16 instructions do the work
+// of one fp32 product exactly, at 16 times the fp32 matrix-core rate per instruction.  A workgroup (4 wavefronts) owns 128
+// weight rows x 64 activation rows; a wavefront 32 weight rows (two packed tiles, straight from HBM into the operand layout
+// they were packed in, converted to bf16 in registers) x all 64 activation rows, whose planes the workgroup stages per
+// 64-wide K step in LDS (two buffers, 144-byte row pitch: 16 rows fall on 16 different bank groups).  Per step and
+// (tile, 16-row group) the six instructions (3 planes x 2 halves of the step) add into a fresh accumulator that is then
+// scaled by the step's 1/scale, like the few-row kernels do.
+__global__ __launch_bounds__(256) void blockquant_split_activations_kernel(const float* __restrict__ a, size_t a_stride, int M, int K,
+                                                                            const float* __restrict__ in_scales, unsigned short* __restrict__ planes, int Mp,
+                                                                            int Kp)
+{
+    const int vec_per_row = Kp >> 3;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)Mp * vec_per_row) return;
+    const int row = (int)(idx / vec_per_row), k = (int)(idx - (size_t)row * vec_per_row) << 3;
+    unsigned pl[3][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    if (row < M && k < K) // K % 16 == 0: a vector of 8 is all in or all out
+    {
+        const float* p = a + (size_t)row * a_stride + k;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            unsigned h[2][3];
+#pragma unroll
+            for (int o = 0; o < 2; o++)
+            {
+                float x = p[2 * e + o];
+                if (in_scales) x = mul_rn(x, in_scales[k + 2 * e + o]);
+                split_bf16x3(x, h[o][0], h[o][1], h[o][2]);
+            }
+#pragma unroll
+            for (int pn = 0; pn < 3; pn++) pl[pn][e] = (h[0][pn] >> 16) | h[1][pn];
+        }
+    }
+#pragma unroll
+    for (int pn = 0; pn < 3; pn++)
+        *reinterpret_cast<uint4*>(planes + ((size_t)pn * Mp + row) * Kp + k) = make_uint4(pl[pn][0], pl[pn][1], pl[pn][2], pl[pn][3]);
+}
+
+#define BQ_AS1 __attribute__((address_space(1)))
+#define BQ_AS3 __attribute__((address_space(3)))
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
+#define BQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | ((((n) >> 4) & 3) << 14))
+
+// Everything a K step needs goes from global memory straight into LDS (no registers in between), into a ring of STAGES
+// stages of which STAGES - 1 are in flight while one is multiplied: one wait + one barrier per step, and a step's memory
+// latency is spread over the arithmetic of the steps before it.  A direct load writes the wavefront's 64 x 16 bytes in lane
+// order, so the layout is made on the SOURCE side: the 16-byte chunk c of activation row r lands at chunk position
+// c ^ ((r / 2) % 8) of its 128-byte row, which makes the operand reads (16 rows x one chunk) conflict-free without padding.
+// A stage: 3 planes x 64 rows x 128 bytes, then the workgroup's 8 weight tiles (1 KB apiece reserved) and their descales
+// (128 bytes apiece).  Every wavefront issues exactly ten loads per stage (6 of activations, its 2 tiles, their 2 descale
+// rows; beyond the last step it loads the last step again into a stage nobody reads any more), which is what the wait counts.
+template<int BITS, bool HALVES, int STAGES, int RW>
+__global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsigned short* __restrict__ planes, int Mp, int Kp, int M, int N, int kblocks,
+                                                                      int ntiles, const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
+                                                                      const float* __restrict__ c, int bt, float alpha, float beta, float* __restrict__ out,
+                                                                      size_t out_stride)
+{
+    static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
+    constexpr int LOADS = 6 + 2 * RW; // per wavefront and stage
+    static_assert(STAGES >= 2 && (STAGES - 2) * LOADS < 64, "the vmcnt field counts to 63");
+    static_assert(RW == 2 || RW == 4, "two or four tiles of 16 weight rows per wavefront");
+    constexpr int PLANE = 64 * 128;
+    constexpr int ACT_BYTES = 3 * PLANE;
+    constexpr int W_OFF = ACT_BYTES, D_OFF = ACT_BYTES + 4 * RW * 1024;
+    constexpr int STAGE_BYTES = D_OFF + 4 * RW * 128;
+    constexpr int STEP_BYTES = 128 * BITS;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds_rows[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m = lane & 15, kg = lane >> 4;
+    const int row0 = blockIdx.y * 64;
+    const int dper = HALVES ? 4 << split : 4;
+
+    // the wavefront's RW tiles (a tile beyond the last reads the last one again and stores nothing)
+    const unsigned char* wsrc[RW];
+    const float4* dsrc[RW];
+#pragma unroll
+    for (int rw = 0; rw < RW; rw++)
+    {
+        const int t = (blockIdx.x * 4 + wave) * RW + rw;
+        const int tl = t < ntiles ? t : ntiles - 1;
+        wsrc[rw] = wpk + (size_t)tl * kblocks * STEP_BYTES + lane * 16;
+        dsrc[rw] = dpk + (size_t)tl * kblocks * dper + lane;
+    }
+    // activation loads: load i of wavefront w fills rows (i % 2) * 32 + w * 8 .. +8 of plane i / 2; lane l brings row + l / 8,
+    // the chunk that belongs at position l % 8
+    const unsigned short* asrc[6];
+#pragma unroll
+    for (int i = 0; i < 6; i++)
+    {
+        const int r = (i & 1) * 32 + wave * 8 + (lane >> 3);
+        const int ch = (lane & 7) ^ ((r >> 1) & 7);
+        asrc[i] = planes + ((size_t)(i >> 1) * Mp + row0 + r) * Kp + ch * 8;
+    }
+    auto issue = [&](int step, int slot) {
+        unsigned char* st = lds_rows + slot * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 6; i++)
+            __builtin_amdgcn_global_load_lds((const BQ_AS1 void*)(asrc[i] + (size_t)step * 64),
+                                             (BQ_AS3 void*)(st + (i >> 1) * PLANE + ((i & 1) * 32 + wave * 8) * 128), 16, 0, 0);
+#pragma unroll
+        for (int rw = 0; rw < RW; rw++)
+        {
+            if (lane < STEP_BYTES / 16)
+                __builtin_amdgcn_global_load_lds((const BQ_AS1 void*)(wsrc[rw] + (size_t)step * STEP_BYTES), (BQ_AS3 void*)(st + W_OFF + (wave * RW + rw) * 1024), 16, 0,
+                                                 0);
+        }
+#pragma unroll
+        for (int rw = 0; rw < RW; rw++)
+        {
+            if (lane < dper)
+                __builtin_amdgcn_global_load_lds((const BQ_AS1 void*)(dsrc[rw] + (size_t)step * dper), (BQ_AS3 void*)(st + D_OFF + (wave * RW + rw) * 128), 16, 0, 0);
+        }
+    };
+
+    v4f acc[RW][4];
+#pragma unroll
+    for (int rw = 0; rw < RW; rw++)
+#pragma unroll
+        for (int cw = 0; cw < 4; cw++) acc[rw][cw] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // operand reads: row cw * 16 + m, chunk positions of the lane's two K groups (the swizzle does not depend on cw)
+    const int sw = (m >> 1) & 7;
+    const int rd_a = m * 128 + (((HALVES ? kg : 2 * kg) ^ sw) << 4);
+    const int rd_b = m * 128 + (((HALVES ? 4 + kg : 2 * kg + 1) ^ sw) << 4);
+    const int last = kblocks - 1;
+    const unsigned lds_base = (unsigned)(uintptr_t)(BQ_AS3 unsigned char*)lds_rows;
+
+#pragma unroll
+    for (int j = 0; j < STAGES - 1; j++) issue(j < last ? j : last, j);
+    int slot = 0, fill = STAGES - 1; // the stage multiplied in this step, and the one its loads refill (the one step - 1 used)
+    for (int step = 0; step < kblocks; step++)
+    {
+        BQ_WAIT_VMCNT((STAGES - 2) * LOADS); // this wavefront's loads of stage `step` have landed; STAGES - 2 newer stages may still be on their way
+        __builtin_amdgcn_s_barrier();     // and everybody else's; everybody has also left stage step - 1, which the next loads overwrite
+        asm volatile("" ::: "memory");
+        {
+            const int ahead = step + STAGES - 1;
+            issue(ahead < last ? ahead : last, fill);
+        }
+        // LDS is read with hand-written instructions and waits: the compiler treats a direct-to-LDS load as a store to all of LDS
+        // and would drain every load in flight (vmcnt(0)) in front of each read it emits itself.  A wait names the registers it
+        // covers as in/out operands, so nothing can use them ahead of it.
+        const unsigned st = lds_base + (unsigned)(slot * STAGE_BYTES);
+        fill = slot;
+        slot = slot + 1 == STAGES ? 0 : slot + 1;
+        v4i_bq wq[RW], dq0[RW], dq1[RW];
+        v2i_bq wlo[RW]; // 4- and 6-bit: the lane's first 8 bytes
+        int whi[RW];    // 6-bit: its third dword
+#pragma unroll
+        for (int rw = 0; rw < RW; rw++)
+        {
+            wq[rw] = v4i_bq{0, 0, 0, 0};
+            wlo[rw] = v2i_bq{0, 0};
+            whi[rw] = 0;
+        }
+        {
+            const unsigned wl = st + W_OFF + (unsigned)(wave * RW * 1024) + (unsigned)(lane * (BITS == 8 ? 16 : 8));
+            const unsigned wl3 = st + W_OFF + (unsigned)(wave * RW * 1024) + 512u + (unsigned)(lane * 4);
+            const unsigned dl = st + D_OFF + (unsigned)(wave * RW * 128) + (unsigned)(kg * 16);
+            const unsigned dl2 = dl + (unsigned)(split << 6);
+#pragma unroll
+            for (int rw = 0; rw < RW; rw++)
+            {
+                // every result register is written by its read and first touched after the wait below
+                if (BITS == 8)
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wq[rw]) : "v"(wl), "n"(rw * 1024));
+                else
+                    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(wlo[rw]) : "v"(wl), "n"(rw * 1024));
+                if (BITS == 6) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(whi[rw]) : "v"(wl3), "n"(rw * 1024));
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dq0[rw]) : "v"(dl), "n"(rw * 128));
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dq1[rw]) : "v"(dl2), "n"(rw * 128));
+            }
+#pragma unroll
+            for (int rw = 0; rw < RW; rw += 2) // (the first wait already covers every read; the later ones only tie their registers to it)
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(wq[rw]), "+v"(wq[rw + 1]), "+v"(wlo[rw]), "+v"(wlo[rw + 1]), "+v"(whi[rw]), "+v"(whi[rw + 1]), "+v"(dq0[rw]), "+v"(dq0[rw + 1]),
+                               "+v"(dq1[rw]), "+v"(dq1[rw + 1]));
+        }
+        v8bf fa[RW], fb[RW];
+#pragma unroll
+        for (int rw = 0; rw < RW; rw++)
+        {
+            if (BITS == 8)
+            {
+                fa[rw] = bytes_to_bf16((unsigned)wq[rw][0], (unsigned)wq[rw][1]);
+                fb[rw] = bytes_to_bf16((unsigned)wq[rw][2], (unsigned)wq[rw][3]);
+            }
+            else if (BITS == 4)
+            {
+                fa[rw] = nibbles_to_bf16((unsigned)wlo[rw][0]);
+                fb[rw] = nibbles_to_bf16((unsigned)wlo[rw][1]);
+            }
+            else
+                sixbit_to_bf16((unsigned)wlo[rw][0], (unsigned)wlo[rw][1], (unsigned)whi[rw], fa[rw], fb[rw]);
+        }
+        // the six operand fragments of a 16-row group (3 planes x 2 halves of the step); the next group's are requested before this one is multiplied
+        union Act
+        {
+            v4i_bq i4;
+            v8bf h;
+        };
+        Act ya[2][3], yb[2][3];
+        const unsigned ra = st + (unsigned)rd_a, rb = st + (unsigned)rd_b;
+        auto read_group = [&](int set, int cw) {
+            const unsigned pa = ra + (unsigned)(cw * 2048), pb = rb + (unsigned)(cw * 2048);
+            asm volatile("ds_read_b128 %0, %1" : "=v"(ya[set][0].i4) : "v"(pa));
+            asm volatile("ds_read_b128 %0, %1" : "=v"(yb[set][0].i4) : "v"(pb));
+            asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(ya[set][1].i4) : "v"(pa));
+            asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(yb[set][1].i4) : "v"(pb));
+            asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(ya[set][2].i4) : "v"(pa));
+            asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(yb[set][2].i4) : "v"(pb));
+        };
+        read_group(0, 0);
+#pragma unroll
+        for (int cw = 0; cw < 4; cw++)
+        {
+            const int set = cw & 1;
+            if (cw + 1 < 4)
+            {
+                read_group(set ^ 1, cw + 1);
+                asm volatile("s_waitcnt lgkmcnt(6)"
+                             : "+v"(ya[set][0].i4), "+v"(yb[set][0].i4), "+v"(ya[set][1].i4), "+v"(yb[set][1].i4), "+v"(ya[set][2].i4), "+v"(yb[set][2].i4));
+            }
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(ya[set][0].i4), "+v"(yb[set][0].i4), "+v"(ya[set][1].i4), "+v"(yb[set][1].i4), "+v"(ya[set][2].i4), "+v"(yb[set][2].i4));
+            // the tiles' chains alternate, so that no instruction waits for the one right before it
+            v4f t0[RW], t1[RW];
+#pragma unroll
+            for (int rw = 0; rw < RW; rw++) t0[rw] = t1[rw] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int pn = 0; pn < 3; pn++)
+            {
+#pragma unroll
+                for (int rw = 0; rw < RW; rw++) t0[rw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[rw], ya[set][pn].h, t0[rw], 0, 0, 0);
+#pragma unroll
+                for (int rw = 0; rw < RW; rw++)
+                {
+                    if (HALVES)
+                        t1[rw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[rw], yb[set][pn].h, t1[rw], 0, 0, 0);
+                    else
+                        t0[rw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[rw], yb[set][pn].h, t0[rw], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int rw = 0; rw < RW; rw++)
+            {
+                const float da[4] = {__int_as_float(dq0[rw][0]), __int_as_float(dq0[rw][1]), __int_as_float(dq0[rw][2]), __int_as_float(dq0[rw][3])};
+                const float db[4] = {__int_as_float(dq1[rw][0]), __int_as_float(dq1[rw][1]), __int_as_float(dq1[rw][2]), __int_as_float(dq1[rw][3])};
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                {
+                    if (HALVES)
+                        acc[rw][cw][r] = fmaf(t1[rw][r], db[r], fmaf(t0[rw][r], da[r], acc[rw][cw][r]));
+                    else
+                        acc[rw][cw][r] = fmaf(t0[rw][r], da[r], acc[rw][cw][r]);
+                }
+            }
+        }
+    }
+    BQ_WAIT_VMCNT(0); // the surplus loads of the last steps must not outlive the workgroup's LDS
+
+    // accumulator r of lane l: weight row (l/16)*4 + r of the tile, activation row l%16 of the 16-row group
+#pragma unroll
+    for (int rw = 0; rw < RW; rw++)
+    {
+        const int t = (blockIdx.x * 4 + wave) * RW + rw;
+#pragma unroll
+        for (int cw = 0; cw < 4; cw++)
+        {
+            const int i = row0 + cw * 16 + m;
+            if (i >= M) continue;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                const int j = t * 16 + kg * 4 + r;
+                if (j < N)
+                {
+                    float v = acc[rw][cw][r];
+                    if (bt >= 0) v = add_rn(mul_rn(load_c(c, bt, i, j, N), beta), v);
+                    out[(size_t)i * out_stride + j] = mul_rn(v, alpha);
+                }
+            }
+        }
+    }
+}
+
 // One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
 template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN, bool INSC>
 static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
@@ -1730,6 +2021,73 @@ int ncnnhip_gemm_blockquant_packed_f16a(const uint16_t* a_dev, size_t a_stride, 
 {
     return gemm_blockquant_packed("ncnnhip_gemm_blockquant_packed_f16a", a_dev, 2, a_stride, M, N, K, packed_w_dev, packed_descale_dev, bits, block, 0, c_dev,
                                   broadcast_type_c, alpha, beta, out_dev, out_stride, stream);
+}
+
+int ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(int M, int K, size_t* bytes)
+{
+    NCNNHIP_REQUIRE(bytes && M >= 1 && K >= 1, "ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: bad arguments");
+    const size_t Mp = ((size_t)M + 63) / 64 * 64, Kp = ((size_t)K + 63) / 64 * 64;
+    *bytes = 3 * Mp * Kp * sizeof(unsigned short);
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev, const float* packed_descale_dev,
+                                        int bits, int block, const float* in_scales_dev, const float* c_dev, int broadcast_type_c, float alpha, float beta,
+                                        float* out_dev, size_t out_stride, void* workspace_dev, size_t workspace_bytes, void* stream)
+{
+    const char* who = "ncnnhip_gemm_blockquant_packed_rows";
+    NCNNHIP_REQUIRE(a_dev && packed_w_dev && packed_descale_dev && out_dev && workspace_dev, "%s: null pointer", who);
+    NCNNHIP_REQUIRE(M >= 1 && N >= 1 && K >= 1 && K % 16 == 0, "%s: bad shape %d %d %d (K must be a multiple of 16)", who, M, N, K);
+    NCNNHIP_REQUIRE(bits == 4 || bits == 6 || bits == 8, "%s: weight bits %d", who, bits);
+    NCNNHIP_REQUIRE(block == 32 || block == 64 || block == 128, "%s: block size %d", who, block);
+    NCNNHIP_REQUIRE(a_stride >= (size_t)K && out_stride >= (size_t)N, "%s: stride too small", who);
+    const int bt = c_dev ? broadcast_type_c : -1;
+    NCNNHIP_REQUIRE(bt >= -1 && bt <= 4, "%s: C broadcast %d", who, bt);
+    const bool halves = halves_layout(bits, block);
+    NCNNHIP_REQUIRE(!halves || K <= 16384, "%s: %d-bit fields in blocks of %d are packed for K up to 16384, got %d", who, bits, block, K);
+    size_t need = 0;
+    ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(M, K, &need);
+    NCNNHIP_REQUIRE(workspace_bytes >= need && al16(workspace_dev), "%s: the workspace must hold %zu bytes, 16-byte aligned (got %zu)", who, need, workspace_bytes);
+    const int Mp = (M + 63) / 64 * 64, Kp = (K + 63) / 64 * 64, kblocks = Kp / 64, ntiles = (N + 15) / 16;
+    NCNNHIP_REQUIRE(Mp / 64 <= 65535, "%s: more than 65535*64 activation rows", who);
+    hipStream_t st = as_stream(stream);
+    unsigned short* planes = static_cast<unsigned short*>(workspace_dev);
+    const size_t vectors = (size_t)Mp * (Kp / 8);
+    hipLaunchKernelGGL(blockquant_split_activations_kernel, dim3((unsigned)((vectors + 255) / 256)), dim3(256), 0, st, a_dev, a_stride, M, K, in_scales_dev, planes, Mp,
+                       Kp);
+    const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
+    const int split = block == 32 ? 1 : 0;
+    // Two tiles per wavefront and two stages: 66 KB of LDS, so two workgroups share a compute unit and one's loads, waits and
+    // vector work overlap the other's matrix-core instructions.  Measured at 1024 x 4096 x 4096 / 2048 x 11008 x 4096: 135 / 616 us;
+    // four tiles per wavefront with three stages (one workgroup per unit, half the LDS reads per instruction) 145 / 714 us; two
+    // tiles with four stages (one workgroup per unit) 172 / 795 us.
+    constexpr int ROWS_STAGES = 2, ROWS_RW = 2;
+    const dim3 grid((ntiles + 4 * ROWS_RW - 1) / (4 * ROWS_RW), Mp / 64);
+    const size_t lds = (size_t)ROWS_STAGES * (3 * 64 * 128 + 4 * ROWS_RW * 1024 + 4 * ROWS_RW * 128);
+#define ROWS(BITS_, HALVES_)                                                                                                                                       \
+    do                                                                                                                                                             \
+    {                                                                                                                                                              \
+        auto kernel = blockquant_rows_bf16x3_kernel<BITS_, HALVES_, ROWS_STAGES, ROWS_RW>;                                                                         \
+        static std::atomic<unsigned char> raised[64];                                                                                                              \
+        int device = 0;                                                                                                                                            \
+        NCNNHIP_CHECK(hipGetDevice(&device));                                                                                                                      \
+        if (device < 0 || device >= 64 || !raised[device].load(std::memory_order_acquire))                                                                         \
+        {                                                                                                                                                          \
+            NCNNHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                     \
+            if (device >= 0 && device < 64) raised[device].store(1, std::memory_order_release);                                                                    \
+        }                                                                                                                                                          \
+        hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, planes, Mp, Kp, M, N, kblocks, ntiles, packed_w_dev, dpk, split, c_dev, bt, alpha, beta, out_dev, out_stride); \
+    } while (0)
+    if (!halves)
+        ROWS(8, false);
+    else if (bits == 8)
+        ROWS(8, true);
+    else if (bits == 6)
+        ROWS(6, true);
+    else
+        ROWS(4, true);
+#undef ROWS
+    return launch_status("blockquant_rows_bf16x3_kernel");
 }
 
 int ncnnhip_gemm_blockquant_packed_supported(int K)

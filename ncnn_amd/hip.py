@@ -139,6 +139,9 @@ _SIGNATURES = {
     "ncnnhip_gemm_blockquant_packed_supported": [C.c_int],
     "ncnnhip_gemm_blockquant_packed": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_blockquant_packed_rows_workspace_bytes": [C.c_int, C.c_int, C.POINTER(C.c_size_t)],
+    "ncnnhip_gemm_blockquant_packed_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                            C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_peak_launch_chain": [C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_mfma_i8": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
     "ncnnhip_peak_hbm_read": [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p],
@@ -689,8 +692,9 @@ class Runtime:
         check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, bits, block, pw.ctypes.data, pd.ctypes.data))
         return pw, pd
 
-    def gemm_blockquant_packed(self, a, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64, in_scales=None):
-        """a fp16: the fp16-activation entry point; a fp32 (optionally with in_scales): the layer's contract, activations split into three bf16."""
+    def gemm_blockquant_packed(self, a, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64, in_scales=None, rows_kernel=False):
+        """a fp16: the fp16-activation entry point; a fp32 (optionally with in_scales): the layer's contract, activations split into three bf16
+        (rows_kernel: the tiled form for many rows, with its workspace)."""
         half = a.dtype == np.float16
         a = np.ascontiguousarray(a, np.float16 if half else np.float32)
         m, k = a.shape
@@ -701,6 +705,13 @@ class Runtime:
         if half:
             assert in_scales is None
             check(lib().ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dc), bt, alpha, beta, dout.ptr, n, self.stream))
+        elif rows_kernel:
+            dis = self.up(None if in_scales is None else np.asarray(in_scales, np.float32))
+            wsb = C.c_size_t()
+            check(lib().ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(m, k, C.byref(wsb)))
+            ws = DeviceBuffer.empty((wsb.value,), np.uint8)
+            check(lib().ncnnhip_gemm_blockquant_packed_rows(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dis), _ptr(dc), bt, alpha, beta, dout.ptr, n,
+                                                            ws.ptr, wsb.value, self.stream))
         else:
             dis = self.up(None if in_scales is None else np.asarray(in_scales, np.float32))
             check(lib().ncnnhip_gemm_blockquant_packed(da.ptr, k, m, n, k, dw_.ptr, dd.ptr, bits, block, _ptr(dis), _ptr(dc), bt, alpha, beta, dout.ptr, n,

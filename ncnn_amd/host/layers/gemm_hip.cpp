@@ -289,7 +289,8 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
     int rc = 0;
     if (weight_block_quantize)
     {
-        rc = blockquant_gemm_device((const float*)A.data, (size_t)K, M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
+        ScopedScratch bq_scratch(&cmd);
+        rc = blockquant_gemm_with_scratch(bq_scratch, (const float*)A.data, (size_t)K, M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
                                     d_B_input_scales, d_B_packed, d_B_packed_descales, d_c, bt, alpha, beta, (float*)top.data, (size_t)N, st);
         return to_ncnn_status(rc, "ncnnhip_gemm_blockquant");
     }
@@ -579,7 +580,7 @@ int Gemm_hip::forward_block_quantize(const std::vector<Mat>& bottom_blobs, std::
             d_c = (const float*)p;
         }
     }
-    rc = blockquant_gemm_device((const float*)d_a, mat_row_stride(A), M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
+    rc = blockquant_gemm_with_scratch(leases, (const float*)d_a, mat_row_stride(A), M, N, K, d_B, term_bits(quantize_term), term_block(quantize_term), d_B_block_scales,
                                 d_B_input_scales, d_B_packed, d_B_packed_descales, d_c, d_c ? bt : -1, alpha, beta, (float*)d_out, (size_t)N, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_blockquant");
     rc = ncnnhip_memcpy_d2h(top.data, d_out, (size_t)M * N * 4, st);

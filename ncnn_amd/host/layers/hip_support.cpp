@@ -52,7 +52,9 @@ int upload_blockquant_packed(const void* fields_host, const float* scales_host, 
 {
     *d_packed = 0;
     *d_descales = 0;
-    if (!ncnnhip_gemm_blockquant_packed_supported(k)) return 0;
+    if (k % 16 != 0) return 0;
+    const bool halves = bits != 8 || block == 32; // those layouts stop at K = 16384; 8-bit fields in blocks of 64 / 128 serve the tiled kernel beyond it
+    if (halves && k > 16384) return 0;
     size_t wb = 0, db = 0;
     if (ncnnhip_blockquant_packed_size(n, k, bits, block, &wb, &db) != 0) return 0;
     std::vector<uint8_t> pw(wb);
@@ -71,13 +73,26 @@ int upload_blockquant_packed(const void* fields_host, const float* scales_host, 
     return ret;
 }
 
+size_t blockquant_gemm_workspace_bytes(int M, int K, const void* d_packed)
+{
+    if (!d_packed || M < 32 || K % 16 != 0) return 0;
+    size_t bytes = 0;
+    if (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(M, K, &bytes) != 0) return 0;
+    return bytes;
+}
+
 int blockquant_gemm_device(const float* a_dev, size_t a_stride, int M, int N, int K, const void* d_fields, int bits, int block, const void* d_scales,
                            const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt, float alpha, float beta,
-                           float* out_dev, size_t out_stride, void* stream)
+                           float* out_dev, size_t out_stride, void* workspace, size_t workspace_bytes, void* stream)
 {
-    // few rows: the packed tiles (one pass over the weights per four rows at most); from 32 rows up the fp32 matrix-core kernel of the
-    // .bin layout does all rows in one pass
-    if (d_packed && d_descales && M < 32 && a_stride % 4 == 0 && ((uintptr_t)a_dev & 15) == 0 && (!d_in_scales || ((uintptr_t)d_in_scales & 15) == 0))
+    // 32 rows and more: the tiled kernel on the bf16 matrix cores, when the caller brought its workspace
+    const size_t need = blockquant_gemm_workspace_bytes(M, K, d_packed);
+    if (need && d_descales && workspace && workspace_bytes >= need)
+        return ncnnhip_gemm_blockquant_packed_rows(a_dev, a_stride, M, N, K, (const uint8_t*)d_packed, (const float*)d_descales, bits, block,
+                                                   (const float*)d_in_scales, c_dev, bt, alpha, beta, out_dev, out_stride, workspace, workspace_bytes, stream);
+    // few rows: the packed tiles, one pass over the weights per four rows at most
+    if (d_packed && d_descales && M < 32 && ncnnhip_gemm_blockquant_packed_supported(K) && a_stride % 4 == 0 && ((uintptr_t)a_dev & 15) == 0
+        && (!d_in_scales || ((uintptr_t)d_in_scales & 15) == 0))
         return ncnnhip_gemm_blockquant_packed(a_dev, a_stride, M, N, K, (const uint8_t*)d_packed, (const float*)d_descales, bits, block,
                                               (const float*)d_in_scales, c_dev, bt, alpha, beta, out_dev, out_stride, stream);
     return ncnnhip_gemm_blockquant(a_dev, a_stride, M, N, K, (const uint8_t*)d_fields, bits, block, (const float*)d_scales, (const float*)d_in_scales, c_dev, bt,

@@ -68,11 +68,28 @@ int upload_constant(const void* host, size_t bytes, void** dev);
 // matrix-core tiles and uploaded; both pointers stay null (and 0 is returned) when K has no kernel for that form.
 int upload_blockquant_packed(const void* fields_host, const float* scales_host, int n, int k, int bits, int block, void** d_packed, void** d_descales);
 
-// Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483) on device operands: the packed tiles for fewer than 32
-// activation rows when they exist and the rows are 16-byte aligned, else the .bin layout.  Returns an ncnnhip status.
+// Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:338-483) on device operands: for fewer than 32 activation rows the
+// packed tiles when they exist and the rows are 16-byte aligned; from 32 rows up the tiled bf16 kernel on the packed tiles
+// when the caller passes the scratch blockquant_gemm_workspace_bytes asks for (0: not applicable); else the .bin layout.
+// Returns an ncnnhip status.
+size_t blockquant_gemm_workspace_bytes(int M, int K, const void* d_packed);
 int blockquant_gemm_device(const float* a_dev, size_t a_stride, int M, int N, int K, const void* d_fields, int bits, int block, const void* d_scales,
                            const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt, float alpha, float beta,
-                           float* out_dev, size_t out_stride, void* stream);
+                           float* out_dev, size_t out_stride, void* workspace, size_t workspace_bytes, void* stream);
+
+// blockquant_gemm_device with the scratch its many-row form wants, borrowed from the call's own allocator (leases / scratch: both
+// hand the buffer back when the call's scope ends, after everything was enqueued on the one stream)
+template<typename Alloc>
+static inline int blockquant_gemm_with_scratch(Alloc& alloc, const float* a_dev, size_t a_stride, int M, int N, int K, const void* d_fields, int bits, int block,
+                                        const void* d_scales, const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt,
+                                        float alpha, float beta, float* out_dev, size_t out_stride, void* stream)
+{
+    const size_t bytes = blockquant_gemm_workspace_bytes(M, K, d_packed);
+    void* ws = bytes ? alloc.get(bytes) : 0; // no room: the call falls back to the kernels that need none
+    return blockquant_gemm_device(a_dev, a_stride, M, N, K, d_fields, bits, block, d_scales, d_in_scales, d_packed, d_descales, c_dev, bt, alpha, beta, out_dev,
+                                  out_stride, ws, ws ? bytes : 0, stream);
+}
+
 
 // payload bytes of a Mat as it lies in memory (whole batch, including plane padding)
 static inline size_t mat_bytes(const ncnn::Mat& m)

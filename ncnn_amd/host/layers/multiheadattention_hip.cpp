@@ -242,7 +242,7 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
 
     int rc = ncnnhip_memcpy_h2d(d_q, q_blob.data, (size_t)src * qdim * 4, st);
     if (rc == 0)
-        rc = blockquant_gemm_device(d_q, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
+        rc = blockquant_gemm_with_scratch(leases, d_q, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
                                     (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
 
@@ -288,7 +288,7 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
             }
             float* d_aff = (float*)leases.get((size_t)cur * E * 4);
             if (!d_aff) return -100;
-            rc = blockquant_gemm_device(d_in, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
+            rc = blockquant_gemm_with_scratch(leases, d_in, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
                                     (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
             if (rc == 0) rc = ncnnhip_transpose_f32(d_aff, E, cur, embed_dim, outT[t] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v projection");
@@ -313,7 +313,7 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     if (att_ws_bytes && !att_ws) return -100;
     rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
-    rc = blockquant_gemm_device(d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
+    rc = blockquant_gemm_with_scratch(leases, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);
     if (rc != 0) return to_ncnn_status(rc, "out projection");
     rc = ncnnhip_memcpy_d2h(top.data, d_out, (size_t)src * qdim * 4, st);
@@ -439,7 +439,7 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     float* d_ctx = (float*)scratch.get((size_t)src * E * 4);
     if (!d_qa || !d_ctx) return -100;
 
-    rc = blockquant_gemm_device((const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
+    rc = blockquant_gemm_with_scratch(scratch, (const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
                                     (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
     if (!reuse_cache)
@@ -457,7 +457,7 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         {
             float* d_aff = (float*)scratch.get((size_t)cur * E * 4);
             if (!d_aff) return -100;
-            rc = blockquant_gemm_device((const float*)in[t]->data, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
+            rc = blockquant_gemm_with_scratch(scratch, (const float*)in[t]->data, (size_t)in_dim[t], cur, embed_dim, in_dim[t], dev[1 + t][0], bits, block, dev[1 + t][1], dev[1 + t][2], dev[1 + t][4], dev[1 + t][5],
                                     (const float*)dev[1 + t][3], 4, 1.f, 1.f, d_aff, E, st);
             if (rc == 0) rc = ncnnhip_transpose_f32(d_aff, E, cur, embed_dim, outT[t] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v projection");
@@ -470,7 +470,7 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     if (att_ws_bytes && !att_ws) return -100;
     rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
-    rc = blockquant_gemm_device(d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
+    rc = blockquant_gemm_with_scratch(scratch, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);
     if (rc != 0) return to_ncnn_status(rc, "out projection");
     if (kv_cache)

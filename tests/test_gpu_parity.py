@@ -573,6 +573,25 @@ def test_blockquant_packed_fp32_activations(rt, bits, block, m, n, k, bt, in_sc)
     _bq_check(got, a, packed, scales, bits, block, ins, c, bt, 0.75, 1.5)
 
 
+@pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
+    # the tiled form for many rows: ragged in rows (64), weight rows (128 per workgroup, 16 per tile) and K (64); every layout; C broadcasts; input scales
+    (8, 64, 64, 128, 64, -1, False), (8, 64, 70, 100, 256, 4, True), (8, 32, 129, 65, 96, 3, False), (8, 128, 64, 31, 1024, 1, True), (8, 64, 200, 130, 2048, 0, False),
+    (8, 64, 33, 8, 4096 + 32, 2, False), (4, 128, 70, 100, 256, 3, True), (6, 32, 40, 65, 96, 0, False), (6, 64, 129, 31, 1024, 4, False), (4, 64, 1, 300, 208, -1, False),
+    (4, 32, 300, 260, 1024 + 16, 4, True), (8, 64, 1500, 1024, 1024, 4, False)])
+def test_blockquant_packed_rows_kernel(rt, bits, block, m, n, k, bt, in_sc):
+    _say("blockquant packed rows", bits, block, m, n, k, bt, in_sc)
+    from ncnn_amd import synth
+    a, packed, scales = synth.blockquant_operands(bits + block + m + n + k + 2, m, n, k, bits, block, half_exact=False)
+    rng = np.random.default_rng(bt + 53)
+    ins = rng.uniform(0.5, 1.5, k).astype(F) if in_sc else None
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)),
+         4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+    got = rt.gemm_blockquant_packed(a, pw, pd, n, c, bt, 0.75, 1.5, bits=bits, block=block, in_scales=ins, rows_kernel=True)
+    _bq_check(got, a, packed, scales, bits, block, ins, c, bt, 0.75, 1.5)
+
+
 @pytest.mark.parametrize("bits,block", [(8, 64), (8, 32), (6, 64), (4, 128)])
 def test_blockquant_packed_fp32_split_keeps_all_24_bits(rt, bits, block):
     """One non-zero activation per row, power-of-two scales: an output is a single product x * q * 2^-2, known to float64
@@ -594,9 +613,10 @@ def test_blockquant_packed_fp32_split_keeps_all_24_bits(rt, bits, block):
     for i in range(m):
         a[i, pos[i]] = vals[i]
     pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
-    got = rt.gemm_blockquant_packed(a, pw, pd, n, bits=bits, block=block).astype(np.float64)
     want = np.stack([float(vals[i]) * qq[:, pos[i]].astype(np.float64) * 0.25 for i in range(m)])
-    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -22), float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-300)))
+    for rows_kernel in (False, True):  # the few-row kernel (split while staging in LDS) and the tiled one (split by a pass of its own)
+        got = rt.gemm_blockquant_packed(a, pw, pd, n, bits=bits, block=block, rows_kernel=rows_kernel).astype(np.float64)
+        assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -22), (rows_kernel, float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-300))))
 
 
 def test_blockquant_exact_on_power_of_two_data(rt):
