@@ -261,7 +261,10 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     wbytes = packed.nbytes + scales.nbytes
     copies = int(np.ceil(512e6 / wbytes)) + 1
     half = args.act == "fp16"
-    packed_form = half or (args.act == "fp32" and m < 32 and lib.ncnnhip_gemm_blockquant_packed_supported(k))
+    packed_form = half or (args.act == "fp32" and k % 16 == 0 and (m >= 32 or lib.ncnnhip_gemm_blockquant_packed_supported(k)))
+    # fp32 activations as the layers dispatch them: up to 4 rows (and 5 to 31 rows of a long K) the few-row kernel, else the kernels that
+    # split the activations in a pass of their own into a workspace
+    rows_entry = packed_form and not half and m >= 5
     if packed_form:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
         pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
         d_w = [rt.up(pw) for _ in range(copies)]  # algorithmic bytes stay those of the .bin: the fields and one fp32 scale per block
@@ -272,11 +275,18 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     d_a = rt.up(a.astype(np.float16) if half else a)
     d_out = ncnn_amd.DeviceBuffer.empty((m, n), np.float32)
     st = rt.stream
+    rows_ws_bytes = C.c_size_t(0)
+    if rows_entry:
+        check(lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(m, k, C.byref(rows_ws_bytes)))
+        d_rows_ws = ncnn_amd.DeviceBuffer.empty((rows_ws_bytes.value,), np.uint8)
 
     def launch(i):
         j = i % copies
         if half:
             check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, -1, 1.0, 1.0, d_out.ptr, n, st))
+        elif rows_entry:
+            check(lib.ncnnhip_gemm_blockquant_packed_rows(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, None, -1, 1.0, 1.0, d_out.ptr, n,
+                                                          d_rows_ws.ptr, rows_ws_bytes.value, st))
         elif packed_form:
             check(lib.ncnnhip_gemm_blockquant_packed(d_a.ptr, k, m, n, k, d_w[j].ptr, d_s[j].ptr, bits, block, None, None, -1, 1.0, 1.0, d_out.ptr, n, st))
         else:
@@ -309,7 +319,7 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic("blockquant:%dx%dx%d%s%s" % (n, k, m, "" if (bits, block) == (8, 64) else ":%d:%d" % (bits, block),
                                                                               "" if half else ":" + args.act)) if packed_form else None,
-                     "kernel": "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
+                     "kernel": ("blockquant_rows16_bf16x3_kernel" if (m <= 48 or (m <= 96 and n >= 128 * 16 - 15)) else "blockquant_rows_bf16x3_kernel") if rows_entry else "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
                      "bytes_per_launch": algo,
                      "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
                      "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"

@@ -382,10 +382,12 @@ int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, i
                                    const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
                                    size_t out_stride, void* stream);
 
-/* The same contract for many activation rows (prefill, attention projections): the three-way split is made once into
- * the workspace (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: 6 bytes per activation, rows and K rounded up to 64),
- * then a tiled Gemm runs on the bf16 matrix cores, 128 weight rows x 64 activation rows per workgroup.  K % 16 == 0; the
- * workspace is scratch (overwritten by every call). */
+/* The same contract from five activation rows up, with a workspace: the three-way split is made once, by a pass of its own,
+ * into the workspace (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: 6 bytes per activation, rows and K rounded up to 64).
+ * Up to 48 rows (96 over 2048 weight rows and more) the weights are then streamed once per 16 rows in the few-row kernel's
+ * shape, the activations pre-arranged as the lanes load them; beyond, a tiled Gemm runs on the bf16 matrix cores, 128 weight
+ * rows x 64 activation rows per workgroup (prefill, attention projections).  K % 16 == 0; the workspace is scratch
+ * (overwritten by every call). */
 int ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(int M, int K, size_t* bytes);
 int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,
                                         const float* packed_descale_dev, int bits, int block, const float* in_scales_dev,

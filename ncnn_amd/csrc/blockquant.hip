@@ -1652,6 +1652,214 @@ __global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsig
     }
 }
 
+// ---- 5 to 16 activation rows in fp32, K up to 4096: weight-streaming shape, exact split made by a pass of its own ----
+// Between the four rows per pass of the few-row kernel (LDS cannot hold more rows' planes) and the tiled kernel (too few
+// workgroups to stream the weights at this row count): the few-row kernel's shape -- one workgroup per tile of 16 weight
+// rows, 8 wavefronts of 8 K steps, every weight byte requested up front -- with the activations' three bf16 planes
+// written beforehand, by blockquant_split_operands_kernel, in the very order the lanes load them: for K step s the six
+// operand fragments (plane p, half h of the step) are 64 x 16 bytes each, lane l = activation row l % 16, K group l / 16.
+// They come from L2 in a window of three steps kept three ahead of the arithmetic (24 VGPRs per step).
+template<bool HALVES>
+__global__ __launch_bounds__(256) void blockquant_split_operands_kernel(const float* __restrict__ a, size_t a_stride, int M, int K, int kblocks,
+                                                                         const float* __restrict__ in_scales, uint4* __restrict__ frags)
+{
+    // one thread = one lane's 8 activations of one (step, half): fragments [step][plane * 2 + half][lane]
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= kblocks * 128) return;
+    const int lane = idx & 63, h = (idx >> 6) & 1, step = idx >> 7;
+    const int row = lane & 15, kg = lane >> 4;
+    const int k = step * 64 + (HALVES ? h * 32 + kg * 8 : kg * 16 + h * 8);
+    unsigned pl[3][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    if (row < M && k < K) // K % 16 == 0: the 8 values are all in or all out
+    {
+        const float* p = a + (size_t)row * a_stride + k;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+        {
+            unsigned hh[2][3];
+#pragma unroll
+            for (int o = 0; o < 2; o++)
+            {
+                float x = p[2 * e + o];
+                if (in_scales) x = mul_rn(x, in_scales[k + 2 * e + o]);
+                split_bf16x3(x, hh[o][0], hh[o][1], hh[o][2]);
+            }
+#pragma unroll
+            for (int pn = 0; pn < 3; pn++) pl[pn][e] = (hh[0][pn] >> 16) | hh[1][pn];
+        }
+    }
+#pragma unroll
+    for (int pn = 0; pn < 3; pn++) frags[((size_t)step * 6 + pn * 2 + h) * 64 + lane] = make_uint4(pl[pn][0], pl[pn][1], pl[pn][2], pl[pn][3]);
+}
+
+template<int BITS, bool HALVES>
+__global__ __launch_bounds__(512) void blockquant_rows16_bf16x3_kernel(const uint4* __restrict__ frags, int M, int N, int kblocks,
+                                                                        const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
+                                                                        const float* __restrict__ c, int bt, float alpha, float beta, float* __restrict__ out,
+                                                                        size_t out_stride)
+{
+    static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
+    constexpr int NB = 8, WIN = 3;
+    constexpr int STEP_BYTES = 128 * BITS;
+    __shared__ float4 red[8 * 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int tile = blockIdx.x;
+    const int m = lane & 15, kg = lane >> 4;
+    const int dper = HALVES ? 4 << split : 4;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    // K beyond 8 wavefronts x 8 steps (4096) goes round by round: round r of wavefront w is steps (r * wavefronts + w) * 8 .. + 8
+    // (a round's requests go out when the round before it is done: its registers are the same)
+    const int rounds = (kblocks + nwaves * NB - 1) / (nwaves * NB);
+    for (int round = 0; round < rounds; round++)
+    {
+    const int kb_begin = (round * nwaves + wave) * NB;
+    int nkb = kblocks - kb_begin;
+    nkb = nkb > NB ? NB : nkb;
+    nkb = nkb < 0 ? 0 : nkb;
+    const int kb_base = nkb > 0 ? kb_begin : 0;
+
+    const unsigned char* wt = wpk + ((size_t)tile * kblocks + kb_base) * STEP_BYTES;
+    const float4* dt = dpk + ((size_t)tile * kblocks + kb_base) * dper;
+    const uint4* ft = frags + (size_t)kb_base * 6 * 64 + lane;
+    v4i_bq w[BITS == 8 ? NB : 1];
+    v2i_bq w2[BITS != 8 ? NB : 1];
+    int w1[BITS == 6 ? NB : 1];
+    float4 d0[NB], d1[HALVES ? NB : 1];
+    uint4 fr[WIN][6];
+    auto load_w = [&](int i) {
+        const unsigned char* ws = wt + (size_t)(i < nkb ? i : 0) * STEP_BYTES;
+        if (BITS == 8)
+            w[BITS == 8 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const v4i_bq*>(ws) + lane);
+        else
+            w2[BITS != 8 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const v2i_bq*>(ws) + lane);
+        if (BITS == 6) w1[BITS == 6 ? i : 0] = __builtin_nontemporal_load(reinterpret_cast<const int*>(ws + 512) + lane);
+    };
+#define R16_LOAD_FRAGS(slot_, i_)                                                          \
+    do                                                                                     \
+    {                                                                                      \
+        const uint4* f_ = ft + (size_t)((i_) < nkb ? (i_) : 0) * 6 * 64;                   \
+        _Pragma("unroll") for (int q = 0; q < 6; q++) fr[slot_][q] = f_[q * 64];           \
+    } while (0)
+    // requests in the order their data is needed: the first steps' weights and operands interleaved, then the rest of the weights,
+    // then the descales (a step beyond the wavefront's range reads step 0 again and meets a zero descale)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < WIN; i++)
+    {
+        load_w(i);
+        __builtin_amdgcn_sched_barrier(0);
+        R16_LOAD_FRAGS(i, i);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = WIN; i < NB; i++)
+    {
+        load_w(i);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 a0 = dt[(size_t)(i < nkb ? i : 0) * dper + kg];
+        d0[i] = i < nkb ? a0 : z;
+        if (HALVES)
+        {
+            const float4 a1 = dt[(size_t)(i < nkb ? i : 0) * dper + (split << 2) + kg];
+            d1[HALVES ? i : 0] = i < nkb ? a1 : z;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        const int slot = i % WIN;
+        v8bf fa, fb;
+        if (BITS == 8)
+        {
+            fa = bytes_to_bf16((unsigned)w[BITS == 8 ? i : 0][0], (unsigned)w[BITS == 8 ? i : 0][1]);
+            fb = bytes_to_bf16((unsigned)w[BITS == 8 ? i : 0][2], (unsigned)w[BITS == 8 ? i : 0][3]);
+        }
+        else if (BITS == 4)
+        {
+            fa = nibbles_to_bf16((unsigned)w2[BITS != 8 ? i : 0][0]);
+            fb = nibbles_to_bf16((unsigned)w2[BITS != 8 ? i : 0][1]);
+        }
+        else
+            sixbit_to_bf16((unsigned)w2[BITS != 8 ? i : 0][0], (unsigned)w2[BITS != 8 ? i : 0][1], (unsigned)w1[BITS == 6 ? i : 0], fa, fb);
+        union
+        {
+            uint4 u;
+            v8bf h;
+        } y[6];
+#pragma unroll
+        for (int q = 0; q < 6; q++) y[q].u = fr[slot][q];
+        v4f t0 = {0.f, 0.f, 0.f, 0.f}, t1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int pn = 0; pn < 3; pn++)
+        {
+            t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, y[pn * 2].h, t0, 0, 0, 0);
+            if (HALVES)
+                t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb, y[pn * 2 + 1].h, t1, 0, 0, 0);
+            else
+                t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb, y[pn * 2 + 1].h, t0, 0, 0, 0);
+        }
+        if (i + WIN < NB)
+        {
+            R16_LOAD_FRAGS(slot, i + WIN);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const float4 da = d0[i];
+        if (HALVES)
+        {
+            const float4 db = d1[HALVES ? i : 0];
+            acc[0] = fmaf(t1[0], db.x, fmaf(t0[0], da.x, acc[0]));
+            acc[1] = fmaf(t1[1], db.y, fmaf(t0[1], da.y, acc[1]));
+            acc[2] = fmaf(t1[2], db.z, fmaf(t0[2], da.z, acc[2]));
+            acc[3] = fmaf(t1[3], db.w, fmaf(t0[3], da.w, acc[3]));
+        }
+        else
+        {
+            acc[0] = fmaf(t0[0], da.x, acc[0]);
+            acc[1] = fmaf(t0[1], da.y, acc[1]);
+            acc[2] = fmaf(t0[2], da.z, acc[2]);
+            acc[3] = fmaf(t0[3], da.w, acc[3]);
+        }
+    }
+#undef R16_LOAD_FRAGS
+    } // rounds
+
+    red[wave * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    if (wave == 0 && m < M)
+    {
+        float4 f = red[lane];
+        for (int w2i = 1; w2i < nwaves; w2i++)
+        {
+            const float4 o = red[w2i * 64 + lane];
+            f.x = add_rn(f.x, o.x);
+            f.y = add_rn(f.y, o.y);
+            f.z = add_rn(f.z, o.z);
+            f.w = add_rn(f.w, o.w);
+        }
+        const float frr[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int j = tile * 16 + kg * 4 + r;
+            if (j < N)
+            {
+                float v = frr[r];
+                if (bt >= 0) v = add_rn(mul_rn(load_c(c, bt, m, j, N), beta), v);
+                out[(size_t)m * out_stride + j] = mul_rn(v, alpha);
+            }
+        }
+    }
+}
+
 // One pass of up to 16 activation rows; nwaves = ceil(kblocks / NB) wavefronts per workgroup.
 template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN, bool INSC>
 static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
@@ -2051,12 +2259,47 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     const int Mp = (M + 63) / 64 * 64, Kp = (K + 63) / 64 * 64, kblocks = Kp / 64, ntiles = (N + 15) / 16;
     NCNNHIP_REQUIRE(Mp / 64 <= 65535, "%s: more than 65535*64 activation rows", who);
     hipStream_t st = as_stream(stream);
+    const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
+    const int split = block == 32 ? 1 : 0;
+    if (M <= 48 || (M <= 96 && ntiles >= 128))
+    {
+        // fewer rows than the tiled kernel can spread over the chip (its 64-row tiles take 75 us at 4096 x 4096 whatever the row
+        // count, a pass here 11-12; at 1024 x 1024 the tiled kernel wins from 64 rows): 16 rows per pass in the weight-streaming shape
+        // (the fragments of a pass take kblocks * 6 KB of the workspace, less than the planes it was sized for)
+        uint4* frags = static_cast<uint4*>(workspace_dev);
+        const int nwaves = kblocks >= 64 ? 8 : (kblocks + 7) / 8; // K beyond 4096: rounds of 8 x 8 steps
+        for (int m0 = 0; m0 < M; m0 += 16)
+        {
+            const int mc = M - m0 < 16 ? M - m0 : 16;
+            const float* cc = c_dev;
+            if (cc && (bt == 1 || bt == 2)) cc += m0;
+            if (cc && bt == 3) cc += (size_t)m0 * N;
+            const float* ap = a_dev + (size_t)m0 * a_stride;
+            float* op = out_dev + (size_t)m0 * out_stride;
+            const dim3 sgrid((kblocks * 128 + 255) / 256);
+            if (halves)
+                hipLaunchKernelGGL(blockquant_split_operands_kernel<true>, sgrid, dim3(256), 0, st, ap, a_stride, mc, K, kblocks, in_scales_dev, frags);
+            else
+                hipLaunchKernelGGL(blockquant_split_operands_kernel<false>, sgrid, dim3(256), 0, st, ap, a_stride, mc, K, kblocks, in_scales_dev, frags);
+#define ROWS16(BITS_, HALVES_)                                                                                                                       \
+    hipLaunchKernelGGL((blockquant_rows16_bf16x3_kernel<BITS_, HALVES_>), dim3(ntiles), dim3(nwaves * 64), 0, st, frags, mc, N, kblocks, packed_w_dev, dpk, split, cc, \
+                       bt, alpha, beta, op, out_stride)
+            if (!halves)
+                ROWS16(8, false);
+            else if (bits == 8)
+                ROWS16(8, true);
+            else if (bits == 6)
+                ROWS16(6, true);
+            else
+                ROWS16(4, true);
+#undef ROWS16
+        }
+        return launch_status("blockquant_rows16_bf16x3_kernel");
+    }
     unsigned short* planes = static_cast<unsigned short*>(workspace_dev);
     const size_t vectors = (size_t)Mp * (Kp / 8);
     hipLaunchKernelGGL(blockquant_split_activations_kernel, dim3((unsigned)((vectors + 255) / 256)), dim3(256), 0, st, a_dev, a_stride, M, K, in_scales_dev, planes, Mp,
                        Kp);
-    const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
-    const int split = block == 32 ? 1 : 0;
     // Two tiles per wavefront and two stages: 66 KB of LDS, so two workgroups share a compute unit and one's loads, waits and
     // vector work overlap the other's matrix-core instructions.  Measured at 1024 x 4096 x 4096 / 2048 x 11008 x 4096: 135 / 616 us;
     // four tiles per wavefront with three stages (one workgroup per unit, half the LDS reads per instruction) 145 / 714 us; two

@@ -75,7 +75,9 @@ int upload_blockquant_packed(const void* fields_host, const float* scales_host, 
 
 size_t blockquant_gemm_workspace_bytes(int M, int K, const void* d_packed)
 {
-    if (!d_packed || M < 32 || K % 16 != 0) return 0;
+    // 5 rows and more: the kernels that split the activations in a pass of their own (up to 48-96 rows the weight-streaming one on
+    // pre-split operands, 16 rows per pass; beyond, the tiled one)
+    if (!d_packed || K % 16 != 0 || M < 5) return 0;
     size_t bytes = 0;
     if (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(M, K, &bytes) != 0) return 0;
     return bytes;
@@ -85,7 +87,7 @@ int blockquant_gemm_device(const float* a_dev, size_t a_stride, int M, int N, in
                            const void* d_in_scales, const void* d_packed, const void* d_descales, const float* c_dev, int bt, float alpha, float beta,
                            float* out_dev, size_t out_stride, void* workspace, size_t workspace_bytes, void* stream)
 {
-    // 32 rows and more: the tiled kernel on the bf16 matrix cores, when the caller brought its workspace
+    // five rows and more: the kernels that split the activations in a pass of their own, when the caller brought the workspace for it
     const size_t need = blockquant_gemm_workspace_bytes(M, K, d_packed);
     if (need && d_descales && workspace && workspace_bytes >= need)
         return ncnnhip_gemm_blockquant_packed_rows(a_dev, a_stride, M, N, K, (const uint8_t*)d_packed, (const float*)d_descales, bits, block,

@@ -577,7 +577,13 @@ def test_blockquant_packed_fp32_activations(rt, bits, block, m, n, k, bt, in_sc)
     # the tiled form for many rows: ragged in rows (64), weight rows (128 per workgroup, 16 per tile) and K (64); every layout; C broadcasts; input scales
     (8, 64, 64, 128, 64, -1, False), (8, 64, 70, 100, 256, 4, True), (8, 32, 129, 65, 96, 3, False), (8, 128, 64, 31, 1024, 1, True), (8, 64, 200, 130, 2048, 0, False),
     (8, 64, 33, 8, 4096 + 32, 2, False), (4, 128, 70, 100, 256, 3, True), (6, 32, 40, 65, 96, 0, False), (6, 64, 129, 31, 1024, 4, False), (4, 64, 1, 300, 208, -1, False),
-    (4, 32, 300, 260, 1024 + 16, 4, True), (8, 64, 1500, 1024, 1024, 4, False)])
+    (4, 32, 300, 260, 1024 + 16, 4, True), (8, 64, 1500, 1024, 1024, 4, False),
+    # up to 48 rows (96 over many weight rows): the weight-streaming form on pre-split operand fragments, 16 rows per pass (one and two passes, ragged rows,
+    # 1 to 8 wavefronts, a last wavefront with fewer steps, K that ends inside a step)
+    (8, 64, 5, 100, 256, -1, False), (8, 64, 16, 256, 4096, 3, False), (4, 32, 9, 40, 1024 + 16, 1, True), (6, 64, 31, 33, 512, 4, False), (8, 32, 17, 20, 96, 2, False),
+    (8, 128, 12, 24, 4096, -1, True), (4, 64, 16, 4100, 2048 + 48, 4, False), (6, 128, 8, 16, 64, 0, False), (8, 64, 20, 40, 3072 + 64, 3, True), (8, 64, 16, 24, 4096 + 64, -1, False),
+    # K beyond 4096: rounds of 8 wavefronts x 8 steps (a last round with idle wavefronts, with a ragged wavefront)
+    (4, 64, 9, 40, 11008, 1, False), (8, 64, 20, 33, 8192 + 16, 4, True), (6, 64, 5, 20, 12288, -1, False), (8, 128, 16, 250, 11008, 3, False)])
 def test_blockquant_packed_rows_kernel(rt, bits, block, m, n, k, bt, in_sc):
     _say("blockquant packed rows", bits, block, m, n, k, bt, in_sc)
     from ncnn_amd import synth
