@@ -255,3 +255,39 @@ def test_blockquant_pack_refuses_what_has_no_kernel():
     assert lib.ncnnhip_blockquant_packed_size(16, 16384 + 64, 8, 64, C.byref(wb), C.byref(db)) == 0
     assert lib.ncnnhip_blockquant_packed_size(16, 64, 5, 64, C.byref(wb), C.byref(db)) != 0
     assert lib.ncnnhip_blockquant_packed_size(16, 64, 8, 48, C.byref(wb), C.byref(db)) != 0
+
+
+def test_packed_blockquant_entry_points_refuse_bad_arguments_before_touching_the_device():
+    """Argument checks come first, so they can be exercised without a GPU: every call below must return an error code
+    (never crash, never report success)."""
+    lib = hip.lib()
+    fake = C.c_void_p(0x1000)  # never dereferenced: the calls stop at their checks
+    wsb = C.c_size_t()
+    assert lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(70, 4096 + 16, C.byref(wsb)) == 0
+    assert wsb.value == 3 * 128 * (4096 + 64) * 2  # rows and K rounded up to 64, three bf16 planes
+    assert lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(0, 64, C.byref(wsb)) != 0
+    rows = lib.ncnnhip_gemm_blockquant_packed_rows
+    few = lib.ncnnhip_gemm_blockquant_packed
+    half = lib.ncnnhip_gemm_blockquant_packed_f16a
+    ok_rows = dict(a=fake, stride=64, m=8, n=16, k=64, w=fake, d=fake, bits=8, block=64, ins=None, c=None, bt=-1, out=fake, ostride=16, ws=fake, wsb=1 << 20)
+
+    def call_rows(**kw):
+        p = dict(ok_rows, **kw)
+        return rows(p["a"], p["stride"], p["m"], p["n"], p["k"], p["w"], p["d"], p["bits"], p["block"], p["ins"], p["c"], p["bt"], 1.0, 1.0, p["out"], p["ostride"],
+                    p["ws"], p["wsb"], None)
+
+    assert call_rows(a=None) != 0 and call_rows(w=None) != 0 and call_rows(out=None) != 0 and call_rows(ws=None) != 0
+    assert call_rows(k=72) != 0            # K % 16
+    assert call_rows(bits=5) != 0 and call_rows(block=48) != 0
+    assert call_rows(stride=32) != 0 and call_rows(ostride=8) != 0
+    assert call_rows(wsb=1024) != 0        # workspace too small
+    assert call_rows(c=fake, bt=7) != 0
+    assert call_rows(bits=4, k=16384 + 64) != 0  # the halves layout stops at K = 16384
+    assert few(fake, 64, 1, 16, 72, fake, fake, 8, 64, None, None, -1, 1.0, 1.0, fake, 16, None) != 0
+    assert few(fake, 64, 1, 16, 64, fake, fake, 8, 64, C.c_void_p(0x1004), None, -1, 1.0, 1.0, fake, 16, None) != 0  # input scales not 16-byte aligned
+    assert few(C.c_void_p(0x1004), 64, 1, 16, 64, fake, fake, 8, 64, None, None, -1, 1.0, 1.0, fake, 16, None) != 0
+    assert few(fake, 64, 1, 16, 16384 + 64, fake, fake, 8, 64, None, None, -1, 1.0, 1.0, fake, 16, None) != 0       # fp32 rows: K <= 16384
+    assert half(fake, 60, 1, 16, 64, fake, fake, 8, 64, None, -1, 1.0, 1.0, fake, 16, None) != 0                    # row stride below K
+    assert lib.ncnnhip_gemm_blockquant_packed_supported(4096) == 1 and lib.ncnnhip_gemm_blockquant_packed_supported(4100) == 0
+    assert lib.ncnnhip_gemm_blockquant_packed_supported(16384 + 16) == 0
+    assert b"ncnnhip_gemm_blockquant_packed" in lib.ncnnhip_last_error()
