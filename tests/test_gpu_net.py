@@ -534,6 +534,39 @@ def test_benchmark_batch_equals_the_per_sample_passes(which, batch):
             assert np.array_equal(got[i].reshape(-1), np.asarray(ex1.extract(name)).reshape(-1)), (name, i)
 
 
+@pytest.mark.parametrize("m", [3, 16, 70])
+def test_recorded_block_quant_gemm_replays_like_the_eager_pass(m):
+    """A block-quantised Gemm layer inside a recorded pass, at row counts that take its three forms (the few-row kernel; the split pass
+    + the weight-streaming kernel; the split pass + the tiled kernel, each with scratch borrowed from the command the graph owns):
+    replays with new inputs equal the eager Extractor bit for bit."""
+    n, k, bits, block = 48, 256, 8, 64
+    rng = np.random.default_rng(m)
+    w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    lines = ["Input data 0 1 data 0=%d 1=%d" % (k, m), mw.gemm_param("g", ["data"], "out", N=n, K=k, constantB=1, quantize_term=bits * 100 + 1)]
+    blob = mw.weight_blob(packed.view(np.int8)) + mw.raw_f32(scales)
+    net = _load(mw.assemble_param(lines), blob, True)
+
+    def eager(x):
+        ex = net.create_extractor()
+        ex.input("data", x)
+        return np.asarray(ex.extract("out"))
+
+    x0 = rng.standard_normal((m, k), dtype=F)
+    graph = net.record("data", net.upload(x0), "out")
+    graph.launch()
+    graph.synchronize()
+    assert np.array_equal(graph.output().to_numpy().reshape(m, n), eager(x0))
+    for i in range(3):
+        x = rng.standard_normal((m, k), dtype=F)
+        want = eager(x)
+        graph.update_input(x)
+        graph.launch()
+        graph.launch()
+        graph.synchronize()
+        assert np.array_equal(graph.output().to_numpy().reshape(m, n), want), i
+
+
 @pytest.mark.parametrize("which,batch", [("tiny", 1), ("tiny", 3), ("mobilenetv2", 1), ("resnet50", 2)])
 def test_recorded_pass_replays_like_the_eager_pass(which, batch):
     """A pass recorded into a graph and replayed: every replay, with new input values and with eager work and
