@@ -1402,6 +1402,9 @@ __global__ __launch_bounds__(256) void blockquant_split_activations_kernel(const
         *reinterpret_cast<uint4*>(planes + ((size_t)pn * Mp + row) * Kp + k) = make_uint4(pl[pn][0], pl[pn][1], pl[pn][2], pl[pn][3]);
 }
 
+#ifndef BQ_ROWS_RW1_BELOW
+#define BQ_ROWS_RW1_BELOW 256
+#endif
 #define BQ_AS1 __attribute__((address_space(1)))
 #define BQ_AS3 __attribute__((address_space(3)))
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
@@ -1424,7 +1427,7 @@ __global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsig
     static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
     constexpr int LOADS = 6 + 2 * RW; // per wavefront and stage
     static_assert(STAGES >= 2 && (STAGES - 2) * LOADS < 64, "the vmcnt field counts to 63");
-    static_assert(RW == 2 || RW == 4, "two or four tiles of 16 weight rows per wavefront");
+    static_assert(RW == 1 || RW == 2 || RW == 4, "one, two or four tiles of 16 weight rows per wavefront");
     constexpr int PLANE = 64 * 128;
     constexpr int ACT_BYTES = 3 * PLANE;
     constexpr int W_OFF = ACT_BYTES, D_OFF = ACT_BYTES + 4 * RW * 1024;
@@ -1538,10 +1541,8 @@ __global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsig
                 asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dq1[rw]) : "v"(dl2), "n"(rw * 128));
             }
 #pragma unroll
-            for (int rw = 0; rw < RW; rw += 2) // (the first wait already covers every read; the later ones only tie their registers to it)
-                asm volatile("s_waitcnt lgkmcnt(0)"
-                             : "+v"(wq[rw]), "+v"(wq[rw + 1]), "+v"(wlo[rw]), "+v"(wlo[rw + 1]), "+v"(whi[rw]), "+v"(whi[rw + 1]), "+v"(dq0[rw]), "+v"(dq0[rw + 1]),
-                               "+v"(dq1[rw]), "+v"(dq1[rw + 1]));
+            for (int rw = 0; rw < RW; rw++) // (the first wait already covers every read; the later ones only tie their registers to it)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wq[rw]), "+v"(wlo[rw]), "+v"(whi[rw]), "+v"(dq0[rw]), "+v"(dq1[rw]));
         }
         v8bf fa[RW], fb[RW];
 #pragma unroll
@@ -2303,14 +2304,17 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     // Two tiles per wavefront and two stages: 66 KB of LDS, so two workgroups share a compute unit and one's loads, waits and
     // vector work overlap the other's matrix-core instructions.  Measured at 1024 x 4096 x 4096 / 2048 x 11008 x 4096: 135 / 616 us;
     // four tiles per wavefront with three stages (one workgroup per unit, half the LDS reads per instruction) 145 / 714 us; two
-    // tiles with four stages (one workgroup per unit) 172 / 795 us.
-    constexpr int ROWS_STAGES = 2, ROWS_RW = 2;
-    const dim3 grid((ntiles + 4 * ROWS_RW - 1) / (4 * ROWS_RW), Mp / 64);
-    const size_t lds = (size_t)ROWS_STAGES * (3 * 64 * 128 + 4 * ROWS_RW * 1024 + 4 * ROWS_RW * 128);
-#define ROWS(BITS_, HALVES_)                                                                                                                                       \
+    // tiles with four stages (one workgroup per unit) 172 / 795 us.  While that leaves fewer workgroups than the chip has compute
+    // units, one tile per wavefront (64 weight rows per workgroup) doubles them: 128 x 4096 x 4096 77 -> 58 us, 256 rows 82 -> 63,
+    // 512 x 1024 x 1024 28.6 -> 22.3.
+    const int rw_tiles = ((ntiles + 7) / 8) * (Mp / 64) < BQ_ROWS_RW1_BELOW ? 1 : 2;
+    // (a ring of four stages where a workgroup has its compute unit to itself measured the same as two: 57.6 against 57.8 us at 128 x 4096 x 4096)
+    const dim3 grid((ntiles + 4 * rw_tiles - 1) / (4 * rw_tiles), Mp / 64);
+#define ROWS_RW(BITS_, HALVES_, RW_, STAGES_)                                                                                                                      \
     do                                                                                                                                                             \
     {                                                                                                                                                              \
-        auto kernel = blockquant_rows_bf16x3_kernel<BITS_, HALVES_, ROWS_STAGES, ROWS_RW>;                                                                         \
+        auto kernel = blockquant_rows_bf16x3_kernel<BITS_, HALVES_, STAGES_, RW_>;                                                                                 \
+        const size_t lds = (size_t)(STAGES_) * (3 * 64 * 128 + 4 * (RW_) * 1024 + 4 * (RW_) * 128);                                                                  \
         static std::atomic<unsigned char> raised[64];                                                                                                              \
         int device = 0;                                                                                                                                            \
         NCNNHIP_CHECK(hipGetDevice(&device));                                                                                                                      \
@@ -2321,6 +2325,14 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
         }                                                                                                                                                          \
         hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, planes, Mp, Kp, M, N, kblocks, ntiles, packed_w_dev, dpk, split, c_dev, bt, alpha, beta, out_dev, out_stride); \
     } while (0)
+#define ROWS(BITS_, HALVES_)            \
+    do                                  \
+    {                                   \
+        if (rw_tiles == 1)                 \
+            ROWS_RW(BITS_, HALVES_, 1, 2); \
+        else                               \
+            ROWS_RW(BITS_, HALVES_, 2, 2); \
+    } while (0)
     if (!halves)
         ROWS(8, false);
     else if (bits == 8)
@@ -2330,6 +2342,7 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     else
         ROWS(4, true);
 #undef ROWS
+#undef ROWS_RW
     return launch_status("blockquant_rows_bf16x3_kernel");
 }
 
