@@ -18,6 +18,11 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-cont
                "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option"]
 
 
+# per-file additions.  blockquant.hip: matrix-core results that go straight into vector arithmetic (the per-block descale) stay in
+# VGPRs instead of AGPRs, which saves a register read per value (tiled kernel 135 -> 125 us at 1024 x 4096 x 4096).
+HIPCC_FILE_FLAGS = {"blockquant.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _run(cmd):
     print("+ " + " ".join(cmd), flush=True)
     subprocess.check_call(cmd)
@@ -32,7 +37,7 @@ def build_kernels(jobs=8):
     for src in HIP_SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = ["hipcc"] + HIPCC_FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = ["hipcc"] + HIPCC_FLAGS + HIPCC_FILE_FLAGS.get(src, []) + ["-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
         print("+ " + " ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd)))
         if len(procs) >= jobs:
