@@ -6,6 +6,8 @@ required to be bit-exact too (stricter than the 1e-5 relative the task allows). 
 Gemm accumulates in a different order than the reference's sequential sum and is held to
 |gpu - ref| <= 1e-5 * sum_k |a_k * w_k|.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -623,6 +625,52 @@ def test_blockquant_packed_fp32_split_keeps_all_24_bits(rt, bits, block):
     for rows_kernel in (False, True):  # the few-row kernel (split while staging in LDS) and the tiled one (split by a pass of its own)
         got = rt.gemm_blockquant_packed(a, pw, pd, n, bits=bits, block=block, rows_kernel=rows_kernel).astype(np.float64)
         assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -22), (rows_kernel, float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-300))))
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("m,act", [(1, "fp16"), (16, "fp16"), (1, "fp32"), (4, "fp32"), (16, "fp32"), (64, "fp32"), (200, "fp32")])
+def test_blockquant_full_size_properties(rt, n, k, m, act):
+    """The decode configuration at its full sizes, through size-independent properties (no oracle pass over 45 M weights per case):
+    doubling the activations doubles every output exactly (a power of two commutes with the split, the products and the sums);
+    permuting the activation rows permutes the output rows bit for bit (a row's result does not depend on its neighbours or on its
+    position modulo the kernel's row grouping... only on which kernel runs, which the row count fixes); and 48 sampled weight rows agree
+    with the float64 value within the usual 1e-5 of sum |a w|."""
+    _say("blockquant full size", n, k, m, act)
+    import ncnn_amd
+    from ncnn_amd import hip, synth
+    a, packed, scales = synth.blockquant_operands(n + k + m, m, n, k, 8, 64, half_exact=(act == "fp16"))
+    pw, pd = rt.blockquant_pack(packed, scales, 64)
+    dw_, dd = rt.up(pw), rt.up(pd)
+
+    def run(x):
+        x = x.astype(np.float16) if act == "fp16" else x
+        # the weights stay on the device between the calls; only the activations change
+        m_, k_ = x.shape
+        da = rt.up(np.ascontiguousarray(x))
+        dout = ncnn_amd.DeviceBuffer.empty((m_, n), np.float32)
+        lib = hip.lib()
+        if act == "fp16":
+            hip.check(lib.ncnnhip_gemm_blockquant_packed_f16a(da.ptr, k_, m_, n, k_, dw_.ptr, dd.ptr, 8, 64, None, -1, 1.0, 1.0, dout.ptr, n, rt.stream))
+        elif m_ >= 5:
+            wsb = C.c_size_t()
+            hip.check(lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(m_, k_, C.byref(wsb)))
+            ws = ncnn_amd.DeviceBuffer.empty((wsb.value,), np.uint8)
+            hip.check(lib.ncnnhip_gemm_blockquant_packed_rows(da.ptr, k_, m_, n, k_, dw_.ptr, dd.ptr, 8, 64, None, None, -1, 1.0, 1.0, dout.ptr, n, ws.ptr, wsb.value,
+                                                              rt.stream))
+        else:
+            hip.check(lib.ncnnhip_gemm_blockquant_packed(da.ptr, k_, m_, n, k_, dw_.ptr, dd.ptr, 8, 64, None, None, -1, 1.0, 1.0, dout.ptr, n, rt.stream))
+        return dout.to_numpy(rt.stream)
+
+    out = run(a)
+    assert np.array_equal(run(a * F(2)), out * F(2))
+    if m > 1:
+        perm = np.random.default_rng(m).permutation(m)
+        if m > 16:  # 16-row groups share a pass / a tile: keep rows inside their group of 16 so that the same lanes' sums are compared
+            perm = np.concatenate([g0 + np.random.default_rng(g0).permutation(min(16, m - g0)) for g0 in range(0, m, 16)])
+        assert np.array_equal(run(a[perm]), out[perm])
+    cols = np.random.default_rng(n).choice(n, 48, replace=False)
+    val, floor = npref.blockquant_gemm_f64(a, packed[cols], scales[cols], 8, 64)
+    assert np.all(np.abs(out[:, cols] - val) <= 1e-5 * floor + 1e-30)
 
 
 def test_blockquant_exact_on_power_of_two_data(rt):
