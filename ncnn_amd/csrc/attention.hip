@@ -126,8 +126,74 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float* __restr
 //                 same key order, four 16-byte loads per lane and 32 channels.
 // Scores and products are fp32 throughout; the order of the additions (and the running rescale by exp(m_old - m_new))
 // differs from the reference's two-pass softmax: compared with an fp32 tolerance.
+// e^x for x <= 0 in three instructions: the hardware's 2^y (1 ulp) on y = x * log2(e).  Rounding y moves the result by at most
+// |y| * 2^-24 of itself, so a term of relative size e^x carries an error below 2^-24 * |x| e^x <= 2.2e-8 of the row's largest
+// term; -inf and differences beyond the exponent range give 0.  (The library's expf spends 14 instructions on range
+// reduction and range checks; with 16 probabilities per lane and tile that was the largest part of the vector work.)
+__device__ __forceinline__ float exp_of_nonpositive(float x)
+{
+    return __builtin_amdgcn_exp2f(mul_rn(x, 1.44269504088896341f));
+}
+
 typedef float v16f_at __attribute__((ext_vector_type(16)));
 typedef float v4f_at __attribute__((ext_vector_type(4)));
+
+// Nothing moves across it: the empty asm holds memory accesses in place for the passes that work on the IR, the scheduling
+// barrier holds every instruction in place for the machine scheduler.
+#define ATT_PHASE_BOUNDARY()                \
+    do                                      \
+    {                                       \
+        asm volatile("" ::: "memory");      \
+        __builtin_amdgcn_sched_barrier(0);  \
+    } while (0)
+
+// the 16 values of one channel that a lane feeds to the products of O^T: keys j0 + 8*(kk/4) + 4*hh + kk%4
+__device__ __forceinline__ void load_value_block(float (&vv)[16], const float* __restrict__ vr, int j0, int hh, int dst, bool vec)
+{
+    if (vec)
+    {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+        {
+            const v4f_at t4 = *reinterpret_cast<const v4f_at*>(vr + j0 + 8 * a + 4 * hh);
+#pragma unroll
+            for (int e = 0; e < 4; e++) vv[4 * a + e] = t4[e];
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++)
+        {
+            const int key = j0 + 8 * (kk >> 2) + 4 * hh + (kk & 3);
+            vv[kk] = vr[key < dst ? key : dst - 1]; // past the end: its probability is 0
+        }
+    }
+}
+
+// One tile's step of the running softmax of a query (lanes l and l^32 hold the two halves of its 32 scores): scores
+// become exp(score - new maximum), the running sum and maximum are brought up to date, and the factor that rescales what
+// was accumulated under the old maximum is returned.
+__device__ __forceinline__ float running_softmax_step(v16f_at& s, float& m, float& l)
+{
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx);
+    const float corr = exp_of_nonpositive(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+    {
+        s[r] = exp_of_nonpositive(s[r] - m_new);
+        psum += s[r];
+    }
+    psum += __shfl_xor(psum, 32);
+    l = l * corr + psum;
+    m = m_new;
+    return corr;
+}
 
 template<int HD>
 __global__ __launch_bounds__(256) void attention_f32_mfma_kernel(const float* __restrict__ q, const float* __restrict__ kt, const float* __restrict__ vt,
@@ -162,67 +228,112 @@ __global__ __launch_bounds__(256) void attention_f32_mfma_kernel(const float* __
 
     const int key_begin = keys_per_split > 0 ? (int)blockIdx.z * keys_per_split : 0;
     const int key_end = keys_per_split > 0 && key_begin + keys_per_split < dst ? key_begin + keys_per_split : dst; // a multiple of 32, or dst
-    for (int j0 = key_begin + wave * 32; j0 < key_end; j0 += 128)
+    // Key loads: channel pair kk starts at a wave-uniform address (scalar registers), the lane adds one 32-bit offset that
+    // is the same for every kk (the host checks that kv_stride + dst fits) - 64-bit per-lane addresses for 32 rows would
+    // cost 64 registers and with them the second wavefront per SIMD.
+    //
+    // The loop is pipelined by hand over the wavefront's tiles of 32 keys.  Iteration t:
+    //   (1) request the values of tile t (and its mask values), (2) add the mask / drop keys past the end in the scores of
+    //   tile t, which the previous iteration left in s_cur, (3) the products of S^T for tile t+1 (its keys were requested
+    //   one iteration ago) together with the softmax arithmetic of tile t: one block of code, the vector instructions
+    //   issue while the matrix pipe works on the chain of products, (4) request the keys of tile t+2, (5) the products
+    //   of O^T for tile t.
+    // The phase boundaries keep the compiler from sinking loads back to their first use (left to itself it keeps one to
+    // eight loads in flight and a wavefront stands on each latency in turn).
+    constexpr int VB = CB <= 2 ? CB : 1; // value blocks requested ahead: all of them while the registers last, else one at a time
+    const int j_first = key_begin + wave * 32;
+    float kreg[HD / 2];
+    v16f_at s_cur;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s_cur[r] = 0.f;
+    if (j_first < key_end)
+    {
+        {
+            const unsigned koff = (unsigned)hh * (unsigned)kv_stride + (unsigned)(j_first + l32 < dst ? j_first + l32 : dst - 1);
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++) kreg[kk] = (kh + (size_t)(2 * kk) * kv_stride)[koff];
+        }
+        ATT_PHASE_BOUNDARY();
+#pragma unroll
+        for (int kk = 0; kk < HD / 2; kk++) s_cur = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[kk], qreg[kk], s_cur, 0, 0, 0);
+        asm volatile("" : "+v"(s_cur)); // the products are pure arithmetic and would be sunk past the boundary to their first use: this pins them before it
+        ATT_PHASE_BOUNDARY();
+        {
+            // past the last tile of this wavefront the loads repeat a key and are never used
+            const int jn = j_first + 128 < key_end ? j_first + 128 : j_first;
+            const unsigned koff = (unsigned)hh * (unsigned)kv_stride + (unsigned)(jn + l32 < dst ? jn + l32 : dst - 1);
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++) kreg[kk] = (kh + (size_t)(2 * kk) * kv_stride)[koff];
+        }
+    }
+    for (int j0 = j_first; j0 < key_end; j0 += 128)
     {
         const bool full = j0 + 32 <= dst;
-        const int kj = j0 + l32 < dst ? j0 + l32 : dst - 1;
-        v16f_at s;
+        float vv[VB][16];
+        if constexpr (CB <= 2)
+        {
 #pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < HD / 2; kk++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kh[(size_t)(2 * kk + hh) * kv_stride + kj], qreg[kk], s, 0, 0, 0);
+            for (int cb = 0; cb < CB; cb++) load_value_block(vv[cb], vh + (size_t)(cb * 32 + l32) * kv_stride, j0, hh, dst, full && v_vec_ok);
+        }
         // register r of this lane: key j0 + 8*(r/4) + 4*hh + r%4 for query l32
-        float mx = -FLT_MAX;
-#pragma unroll
-        for (int r = 0; r < 16; r++)
+        if (mrow)
         {
-            const int key = j0 + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (mrow && key < dst) s[r] = add_rn(s[r], mrow[key]);
-            if (!full && key >= dst) s[r] = -INFINITY;
-            mx = fmaxf(mx, s[r]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx);
-        const float corr = expf(m - m_new);
-        float psum = 0.f;
+            // all 16 mask values requested before the first is used; a key past the end repeats the last one and is dropped below
+            float mv[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-            s[r] = expf(s[r] - m_new);
-            psum += s[r];
+            for (int r = 0; r < 16; r++)
+            {
+                const int key = j0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                mv[r] = mrow[key < dst ? key : dst - 1];
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) s_cur[r] = add_rn(s_cur[r], mv[r]);
         }
-        psum += __shfl_xor(psum, 32);
-        l = l * corr + psum;
-        m = m_new;
+        if (!full)
+        {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (j0 + 8 * (r >> 2) + 4 * hh + (r & 3) >= dst) s_cur[r] = -INFINITY;
+        }
+        ATT_PHASE_BOUNDARY();
+        v16f_at s_next;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s_next[r] = 0.f;
+        float corr;
+        if (j0 + 128 < key_end)
+        {
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++) s_next = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[kk], qreg[kk], s_next, 0, 0, 0);
+            corr = running_softmax_step(s_cur, m, l);
+            // issue order within the block: one product, then three of the vector instructions, while these last
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            }
+        }
+        else
+            corr = running_softmax_step(s_cur, m, l);
+        asm volatile("" : "+v"(s_next), "+v"(s_cur));
+        ATT_PHASE_BOUNDARY();
+        {
+            const int jn = j0 + 256 < key_end ? j0 + 256 : j0;
+            const unsigned koff = (unsigned)hh * (unsigned)kv_stride + (unsigned)(jn + l32 < dst ? jn + l32 : dst - 1);
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++) kreg[kk] = (kh + (size_t)(2 * kk) * kv_stride)[koff];
+        }
+        ATT_PHASE_BOUNDARY();
 #pragma unroll
         for (int cb = 0; cb < CB; cb++)
         {
 #pragma unroll
             for (int r = 0; r < 16; r++) o[cb][r] *= corr;
-            const float* vr = vh + (size_t)(cb * 32 + l32) * kv_stride;
-            float vv[16];
-            if (full && v_vec_ok)
-            {
+            if constexpr (CB > 2) load_value_block(vv[0], vh + (size_t)(cb * 32 + l32) * kv_stride, j0, hh, dst, full && v_vec_ok);
 #pragma unroll
-                for (int a = 0; a < 4; a++)
-                {
-                    const v4f_at t4 = *reinterpret_cast<const v4f_at*>(vr + j0 + 8 * a + 4 * hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) vv[4 * a + e] = t4[e];
-                }
-            }
-            else
-            {
-#pragma unroll
-                for (int kk = 0; kk < 16; kk++)
-                {
-                    const int key = j0 + 8 * (kk >> 2) + 4 * hh + (kk & 3);
-                    vv[kk] = vr[key < dst ? key : dst - 1]; // its probability is 0
-                }
-            }
-#pragma unroll
-            for (int kk = 0; kk < 16; kk++) o[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[kk], s[kk], o[cb], 0, 0, 0);
+            for (int kk = 0; kk < 16; kk++) o[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[CB <= 2 ? cb : 0][kk], s_cur[kk], o[cb], 0, 0, 0);
         }
+        s_cur = s_next;
     }
 
     // ---- merge the four shares: common maximum, then each wavefront adds its rescaled part in turn
@@ -304,7 +415,10 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     }
 }
 
-// how many ways to split the keys: enough workgroups for the chip, at least 128 keys (one tile per wavefront) each
+// how many ways to split the keys: enough workgroups for the chip, at least 128 keys (one tile per wavefront) each.
+// (With 256 workgroups or more a split does not pay even where the last round over the chip is mostly empty - 47 query
+// blocks x 16 heads at head dimension 64 run in 1.47 rounds of 512: split in two, the kernel took 145 us against 136 and
+// the merge another 13.)
 static int attention_key_splits(int num_heads, int src, int dst)
 {
     const long long groups = (long long)((src + 31) / 32) * num_heads;
@@ -342,6 +456,7 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
     NCNNHIP_REQUIRE(num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && dst_seqlen >= 1, "ncnnhip_attention_f32: bad shape");
     NCNNHIP_REQUIRE(num_heads <= 65535, "ncnnhip_attention_f32: more than 65535 heads");
     NCNNHIP_REQUIRE(kv_stride >= (size_t)dst_seqlen, "ncnnhip_attention_f32: key/value row stride below dst_seqlen");
+    NCNNHIP_REQUIRE(kv_stride + (size_t)dst_seqlen < ((size_t)1 << 30), "ncnnhip_attention_f32: key/value row stride beyond the 32-bit byte offsets of the kernel");
     NCNNHIP_REQUIRE(!mask_dev || mask_heads == 1 || mask_heads == num_heads, "ncnnhip_attention_f32: the mask is shared (1) or one per head");
     if (head_dim % 32 == 0 && head_dim <= 128)
     {
