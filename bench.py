@@ -471,16 +471,22 @@ def bench_mha(args, embed, heads, src, past):
     st = rt.stream
     rng = np.random.default_rng(0)
     dst = past + src
-    ws = []
+    ws, host = [], []
     for _ in range(4):
         w = rng.normal(0, 1.0 / np.sqrt(embed), (embed, embed)).astype(np.float32)
         packed, scales = synth.blockquant_weights(w, 8, 64)
+        bias = rng.uniform(-0.1, 0.1, embed).astype(np.float32)
+        host.append((packed, scales, bias))
         pw, pd = rt.blockquant_pack(packed, scales, 64)  # the second form create_pipeline uploads: matrix-core tiles
-        ws.append((rt.up(packed), rt.up(scales), rt.up(rng.uniform(-0.1, 0.1, embed).astype(np.float32)), packed.nbytes + scales.nbytes, rt.up(pw), rt.up(pd)))
+        ws.append((rt.up(packed), rt.up(scales), rt.up(bias), packed.nbytes + scales.nbytes, rt.up(pw), rt.up(pd)))
+    packed, scales, bias = [np.concatenate([h[i] for h in host[:3]]) for i in range(3)]
+    pw, pd = rt.blockquant_pack(packed, scales, 64)
+    w_qkv = (rt.up(packed), rt.up(scales), rt.up(bias), packed.nbytes + scales.nbytes, rt.up(pw), rt.up(pd))
     d_x = rt.up(rng.normal(0, 1, (src, embed)).astype(np.float32))
     d_kt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
     d_vt = rt.up(rng.normal(0, 1, (embed, dst)).astype(np.float32))
-    d_qa, d_aff, d_ctx, d_out = [ncnn_amd.DeviceBuffer.empty((src, embed), np.float32) for _ in range(4)]
+    d_ctx, d_out = [ncnn_amd.DeviceBuffer.empty((src, embed), np.float32) for _ in range(2)]
+    d_qkv = ncnn_amd.DeviceBuffer.empty((src, 3 * embed), np.float32)
     scale = float(1.0 / np.sqrt(embed // heads))
     wsb = C.c_size_t()
     check(lib.ncnnhip_attention_workspace_bytes(heads, embed // heads, src, dst, C.byref(wsb)))
@@ -495,22 +501,24 @@ def bench_mha(args, embed, heads, src, past):
         check(lib.ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(src, embed, C.byref(rb)))
         rows_ws = (ncnn_amd.DeviceBuffer.empty((rb.value,), np.uint8), rb.value)
 
-    def project(x, w, alpha, out):
+    def project(x, w, n, out, out_stride):
         if rows_ws is not None:
-            check(lib.ncnnhip_gemm_blockquant_packed_rows(x.ptr, embed, src, embed, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed,
+            check(lib.ncnnhip_gemm_blockquant_packed_rows(x.ptr, embed, src, n, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, 1.0, 1.0, out.ptr, out_stride,
                                                           rows_ws[0].ptr, rows_ws[1], st))
         elif packed_ok:
-            check(lib.ncnnhip_gemm_blockquant_packed(x.ptr, embed, src, embed, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed, st))
+            check(lib.ncnnhip_gemm_blockquant_packed(x.ptr, embed, src, n, embed, w[4].ptr, w[5].ptr, 8, 64, None, w[2].ptr, 4, 1.0, 1.0, out.ptr, out_stride, st))
         else:
-            check(lib.ncnnhip_gemm_blockquant(x.ptr, embed, src, embed, embed, w[0].ptr, 8, 64, w[1].ptr, None, w[2].ptr, 4, alpha, 1.0, out.ptr, embed, st))
+            check(lib.ncnnhip_gemm_blockquant(x.ptr, embed, src, n, embed, w[0].ptr, 8, 64, w[1].ptr, None, w[2].ptr, 4, 1.0, 1.0, out.ptr, out_stride, st))
 
     def step():
-        project(d_x, ws[0], scale, d_qa)
+        # self-attention: q, k and v out of one Gemm over the three weight matrices as one (what create_pipeline keeps for this case),
+        # k and v transposed out of its rows into the cache columns, the query's scale applied where the attention kernel reads it
+        project(d_x, w_qkv, 3 * embed, d_qkv, 3 * embed)
         for t, cache in ((1, d_kt), (2, d_vt)):
-            project(d_x, ws[t], 1.0, d_aff)
-            check(lib.ncnnhip_transpose_f32(d_aff.ptr, embed, src, embed, C.c_void_p(cache.ptr.value + past * 4), dst, st))
-        check(lib.ncnnhip_attention_f32(d_qa.ptr, d_kt.ptr, d_vt.ptr, dst, None, 0, heads, embed // heads, src, dst, d_ctx.ptr, d_ws.ptr, wsb.value, st))
-        project(d_ctx, ws[3], 1.0, d_out)
+            check(lib.ncnnhip_transpose_f32(C.c_void_p(d_qkv.ptr.value + t * embed * 4), 3 * embed, src, embed, C.c_void_p(cache.ptr.value + past * 4), dst, st))
+        check(lib.ncnnhip_attention_f32_strided(d_qkv.ptr, 3 * embed, scale, d_kt.ptr, d_vt.ptr, dst, None, 0, heads, embed // heads, src, dst, d_ctx.ptr, d_ws.ptr,
+                                                wsb.value, st))
+        project(d_ctx, ws[3], embed, d_out, embed)
 
     for _ in range(args.warmup):
         step()
@@ -533,9 +541,9 @@ def bench_mha(args, embed, heads, src, past):
         "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "self-attention layer, embed %d, %d heads, %d new tokens on a cache of %d, 8-bit block-quantised weights (blocks of 64)"
-                               % (embed, heads, src, past), "launches_per_step": 11 if rows_ws is not None else 7, "projections": "tiled bf16x3 kernel" if rows_ws is not None else ("packed tiles" if packed_ok else ".bin layout"), "device_ms_per_step": k_ms, "gflop": ops / 1e9},
+                               % (embed, heads, src, past), "launches_per_step": (7 if rows_ws is not None else 5) + (1 if wsb.value else 0), "projections": "tiled bf16x3 kernel" if rows_ws is not None else ("packed tiles" if packed_ok else ".bin layout"), "device_ms_per_step": k_ms, "gflop": ops / 1e9},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "whole layer (3 projections, 2 cache appends, attention core, output projection)", "bytes_per_launch": algo},
+                     "kernel": "whole layer (q/k/v projection, 2 cache appends, attention core, output projection)", "bytes_per_launch": algo},
     }
 
 

@@ -406,6 +406,12 @@ int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqle
 int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
                           int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev,
                           void* workspace_dev, size_t workspace_bytes, void* stream);
+/* The same with the queries taken as they come out of one Gemm that makes q, k and v together: row stride q_stride
+ * (>= num_heads*head_dim) and every query value multiplied by q_scale on load - the (sum + bias) * scale of
+ * src/layer/multiheadattention.cpp:618-634 with the same roundings, made where the query is read. */
+int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_scale, const float* kt_dev, const float* vt_dev,
+                                  size_t kv_stride, const float* mask_dev, int mask_heads, int num_heads, int head_dim, int src_seqlen,
+                                  int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ measured ceilings (benchmark support)
  * No counterpart in the reference.  What this chip sustains, to set beside the published peaks in a roofline line:

@@ -33,7 +33,7 @@ __device__ __forceinline__ float wave_sum(float v)
 
 __global__ __launch_bounds__(256) void attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ kt, const float* __restrict__ vt,
                                                             const float* __restrict__ mask, int mask_heads, int head_dim, int embed_dim, int src, int dst,
-                                                            size_t kv_stride, float* __restrict__ out)
+                                                            size_t kv_stride, float* __restrict__ out, size_t q_stride, float q_scale)
 {
     extern __shared__ float smem[];
     float* qs = smem;                     // [ATT_TQ][head_dim]
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float* __restr
     for (int e = tid; e < ATT_TQ * head_dim; e += 256)
     {
         const int t = e / head_dim, l = e - t * head_dim;
-        qs[e] = t < rows ? q[(size_t)(i0 + t) * embed_dim + h * head_dim + l] : 0.f;
+        qs[e] = t < rows ? mul_rn(q[(size_t)(i0 + t) * q_stride + h * head_dim + l], q_scale) : 0.f;
     }
     __syncthreads();
 
@@ -199,7 +199,7 @@ template<int HD>
 __global__ __launch_bounds__(256) void attention_f32_mfma_kernel(const float* __restrict__ q, const float* __restrict__ kt, const float* __restrict__ vt,
                                                                  const float* __restrict__ mask, int mask_heads, int embed_dim, int src, int dst,
                                                                  size_t kv_stride, float* __restrict__ out, int v_vec_ok, int keys_per_split,
-                                                                 float* __restrict__ partial)
+                                                                 float* __restrict__ partial, size_t q_stride, float q_scale)
 {
     // keys_per_split > 0: blockIdx.z takes keys [z*keys_per_split, ...) and leaves (m, l, unnormalised o) in `partial`
     // for attention_merge_kernel; 0: the workgroup sees every key and writes the result
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void attention_f32_mfma_kernel(const float* __
 
     float qreg[HD / 2];
 #pragma unroll
-    for (int kk = 0; kk < HD / 2; kk++) qreg[kk] = q[(size_t)qi * embed_dim + h * HD + 2 * kk + hh];
+    for (int kk = 0; kk < HD / 2; kk++) qreg[kk] = mul_rn(q[(size_t)qi * q_stride + h * HD + 2 * kk + hh], q_scale);
 
     v16f_at o[CB];
 #pragma unroll
@@ -452,9 +452,18 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
                           int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes,
                           void* stream)
 {
+    return ncnnhip_attention_f32_strided(q_dev, (size_t)num_heads * (size_t)(head_dim > 0 ? head_dim : 0), 1.f, kt_dev, vt_dev, kv_stride, mask_dev, mask_heads, num_heads,
+                                         head_dim, src_seqlen, dst_seqlen, out_dev, workspace_dev, workspace_bytes, stream);
+}
+
+int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_scale, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
+                                  int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev,
+                                  size_t workspace_bytes, void* stream)
+{
     NCNNHIP_REQUIRE(q_dev && kt_dev && vt_dev && out_dev, "ncnnhip_attention_f32: null pointer");
     NCNNHIP_REQUIRE(num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && dst_seqlen >= 1, "ncnnhip_attention_f32: bad shape");
     NCNNHIP_REQUIRE(num_heads <= 65535, "ncnnhip_attention_f32: more than 65535 heads");
+    NCNNHIP_REQUIRE(q_stride >= (size_t)num_heads * (size_t)head_dim, "ncnnhip_attention_f32: query row stride below embed_dim");
     NCNNHIP_REQUIRE(kv_stride >= (size_t)dst_seqlen, "ncnnhip_attention_f32: key/value row stride below dst_seqlen");
     NCNNHIP_REQUIRE(kv_stride + (size_t)dst_seqlen < ((size_t)1 << 30), "ncnnhip_attention_f32: key/value row stride beyond the 32-bit byte offsets of the kernel");
     NCNNHIP_REQUIRE(!mask_dev || mask_heads == 1 || mask_heads == num_heads, "ncnnhip_attention_f32: the mask is shared (1) or one per head");
@@ -480,7 +489,7 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
         hipStream_t st = as_stream(stream);
 #define LAUNCH_ATT(HD_) \
     hipLaunchKernelGGL(attention_f32_mfma_kernel<HD_>, grid, dim3(256), 0, st, q_dev, kt_dev, vt_dev, mask_dev, mh, e, src_seqlen, dst_seqlen, kv_stride, out_dev, \
-                       v_vec_ok, keys_per_split, partial)
+                       v_vec_ok, keys_per_split, partial, q_stride, q_scale)
         if (head_dim == 32)
             LAUNCH_ATT(32);
         else if (head_dim == 64)
@@ -499,7 +508,7 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
                     head_dim, head_dim + dst_seqlen);
     dim3 grid((unsigned)((src_seqlen + ATT_TQ - 1) / ATT_TQ), (unsigned)num_heads);
     hipLaunchKernelGGL(attention_f32_kernel, grid, dim3(256), lds, as_stream(stream), q_dev, kt_dev, vt_dev, mask_dev, mask_dev ? mask_heads : 0, head_dim,
-                       num_heads * head_dim, src_seqlen, dst_seqlen, kv_stride, out_dev);
+                       num_heads * head_dim, src_seqlen, dst_seqlen, kv_stride, out_dev, q_stride, q_scale);
     return launch_status("attention_f32_kernel");
 }
 

@@ -55,6 +55,8 @@ _SIGNATURES = {
     "ncnnhip_attention_workspace_bytes": [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
     "ncnnhip_attention_f32": [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t,
                               C.c_void_p],
+    "ncnnhip_attention_f32_strided": [C.c_void_p, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                      C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_stream_begin_capture": [C.c_void_p],
     "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
     "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
@@ -416,11 +418,14 @@ class Runtime:
         check(lib().ncnnhip_global_pooling_nhwc_quantised(C.byref(d), src.ptr, float(scale), out.ptr, self.stream))
         return out.to_numpy(self.stream)
 
-    def attention(self, q, kt, vt, num_heads, mask=None, use_workspace=True):
-        """q [src][embed] (scaled), kt / vt [embed][dst], mask [src][dst] or [heads][src][dst] -> [src][embed]."""
+    def attention(self, q, kt, vt, num_heads, mask=None, use_workspace=True, q_scale=None):
+        """q [src][embed] (scaled), kt / vt [embed][dst], mask [src][dst] or [heads][src][dst] -> [src][embed].
+
+        With q_scale, q may be wider than embed (its first embed columns are the queries, the row stride is its width) and
+        every query value is multiplied by q_scale on load."""
         q, kt, vt = [np.ascontiguousarray(a, np.float32) for a in (q, kt, vt)]
-        src, embed = q.shape
-        dst = kt.shape[1]
+        src, q_stride = q.shape
+        embed, dst = kt.shape
         dq, dk, dv = self.up(q), self.up(kt), self.up(vt)
         dm = None if mask is None else self.up(np.ascontiguousarray(mask, np.float32))
         mask_heads = 0 if mask is None else (1 if mask.ndim == 2 else mask.shape[0])
@@ -428,8 +433,13 @@ class Runtime:
         wsb = C.c_size_t()
         check(lib().ncnnhip_attention_workspace_bytes(num_heads, embed // num_heads, src, dst, C.byref(wsb)))
         ws = DeviceBuffer.empty((max(wsb.value, 4),), np.uint8) if use_workspace else None
-        check(lib().ncnnhip_attention_f32(dq.ptr, dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads, src, dst, out.ptr,
-                                          _ptr(ws), wsb.value if use_workspace else 0, self.stream))
+        if q_scale is None:
+            assert q_stride == embed
+            check(lib().ncnnhip_attention_f32(dq.ptr, dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads, src, dst, out.ptr,
+                                              _ptr(ws), wsb.value if use_workspace else 0, self.stream))
+        else:
+            check(lib().ncnnhip_attention_f32_strided(dq.ptr, q_stride, float(q_scale), dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads,
+                                                      src, dst, out.ptr, _ptr(ws), wsb.value if use_workspace else 0, self.stream))
         return out.to_numpy(self.stream)
 
     def softmax(self, x):

@@ -153,6 +153,7 @@ public:
 
 private:
     void* dev[4][6]; // per projection: weight fields, block scales, input scales (or 0), bias, matrix-core tiles and their descales (or 0)
+    void* dev_qkv[6]; // the same six for the q, k and v matrices as one (self-attention with equal input widths and no input scales), or all 0
 };
 
 ncnn::Layer* MultiHeadAttention_hip_creator(void* userdata);

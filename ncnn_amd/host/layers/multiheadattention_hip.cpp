@@ -7,6 +7,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <vector>
+
 #include "hip_layers.h"
 #include "hip_support.h"
 
@@ -47,6 +49,7 @@ MultiHeadAttention_hip::MultiHeadAttention_hip()
     support_hip = true;
     weight_block_quantize = 0;
     memset(dev, 0, sizeof(dev));
+    memset(dev_qkv, 0, sizeof(dev_qkv));
 }
 
 MultiHeadAttention_hip::~MultiHeadAttention_hip()
@@ -131,6 +134,33 @@ int MultiHeadAttention_hip::create_pipeline(const Option&)
                                            att_bits(quantize_term), att_block(quantize_term), &dev[i][4], &dev[i][5]);
         }
     }
+    // Self-attention reads one blob three times: with equal input widths and no per-projection input scales the three
+    // weight matrices are also kept as one of 3 * embed_dim rows (q rows, k rows, v rows), so that q, k and v come out of
+    // one Gemm.  The query's scale is applied where the attention kernel reads it.
+    const int qdim = embed_dim > 0 ? weight_data_size / embed_dim : 0;
+    if (ret == 0 && qdim == kdim && qdim == vdim && !att_has_input_scale(quantize_term))
+    {
+        const size_t wbytes = (size_t)weight_data[0].w * weight_data[0].h, sfloats = (size_t)weight_data_quantize_scales[0].w * weight_data_quantize_scales[0].h;
+        bool same = true;
+        for (int i = 1; i < 3; i++)
+            same = same && (size_t)weight_data[i].w * weight_data[i].h == wbytes && (size_t)weight_data_quantize_scales[i].w * weight_data_quantize_scales[i].h == sfloats && weight_data[i].h == embed_dim;
+        if (same && weight_data[0].h == embed_dim)
+        {
+            std::vector<unsigned char> fields(3 * wbytes);
+            std::vector<float> scales(3 * sfloats), bias(3 * (size_t)embed_dim);
+            for (int i = 0; i < 3; i++)
+            {
+                memcpy(fields.data() + i * wbytes, weight_data[i].data, wbytes);
+                memcpy(scales.data() + i * sfloats, weight_data_quantize_scales[i].data, sfloats * 4);
+                memcpy(bias.data() + (size_t)i * embed_dim, bias_data[i].data, (size_t)embed_dim * 4);
+            }
+            ret = upload_constant(fields.data(), fields.size(), &dev_qkv[0]);
+            if (ret == 0) ret = upload_constant(scales.data(), scales.size() * 4, &dev_qkv[1]);
+            if (ret == 0) ret = upload_constant(bias.data(), bias.size() * 4, &dev_qkv[3]);
+            if (ret == 0)
+                ret = upload_blockquant_packed(fields.data(), scales.data(), 3 * embed_dim, qdim, att_bits(quantize_term), att_block(quantize_term), &dev_qkv[4], &dev_qkv[5]);
+        }
+    }
     if (ret != 0) destroy_pipeline(Option());
     return ret;
 }
@@ -143,6 +173,11 @@ int MultiHeadAttention_hip::destroy_pipeline(const Option&)
             if (dev[i][j]) ncnnhip_free(dev[i][j]);
             dev[i][j] = 0;
         }
+    for (int j = 0; j < 6; j++)
+    {
+        if (dev_qkv[j]) ncnnhip_free(dev_qkv[j]);
+        dev_qkv[j] = 0;
+    }
     return 0;
 }
 
@@ -232,8 +267,10 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     void* st = ctx->stream;
     const size_t E = (size_t)embed_dim;
 
+    const bool fused_qkv = dev_qkv[0] && self_attention; // one blob in, q / k / v out of one Gemm
+    const size_t q_stride = fused_qkv ? 3 * E : E;
     float* d_q = (float*)leases.get((size_t)src * qdim * 4);
-    float* d_qa = (float*)leases.get((size_t)src * E * 4);
+    float* d_qa = (float*)leases.get((size_t)src * q_stride * 4);
     float* d_kt = (float*)leases.get(E * dst * 4);
     float* d_vt = (float*)leases.get(E * dst * 4);
     float* d_ctx = (float*)leases.get((size_t)src * E * 4);
@@ -241,7 +278,10 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     if (!d_q || !d_qa || !d_kt || !d_vt || !d_ctx || !d_out) return -100;
 
     int rc = ncnnhip_memcpy_h2d(d_q, q_blob.data, (size_t)src * qdim * 4, st);
-    if (rc == 0)
+    if (rc == 0 && fused_qkv)
+        rc = blockquant_gemm_with_scratch(leases, d_q, (size_t)qdim, src, 3 * embed_dim, qdim, dev_qkv[0], bits, block, dev_qkv[1], dev_qkv[2], dev_qkv[4], dev_qkv[5],
+                                    (const float*)dev_qkv[3], 4, 1.f, 1.f, d_qa, q_stride, st);
+    else if (rc == 0)
         rc = blockquant_gemm_with_scratch(leases, d_q, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
                                     (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
@@ -270,7 +310,12 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
         float* d_kv_in = 0;
-        for (int t = 0; t < 2; t++)
+        for (int t = 0; t < 2 && fused_qkv; t++)
+        {
+            rc = ncnnhip_transpose_f32(d_qa + (1 + t) * E, q_stride, cur, embed_dim, outT[t] + past, (size_t)dst, st);
+            if (rc != 0) return to_ncnn_status(rc, "k/v columns");
+        }
+        for (int t = 0; t < 2 && !fused_qkv; t++)
         {
             const float* d_in = d_q;
             if (!(in[t]->data == q_blob.data && in_dim[t] == qdim))
@@ -311,7 +356,8 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
     void* att_ws = att_ws_bytes ? leases.get(att_ws_bytes) : 0;
     if (att_ws_bytes && !att_ws) return -100;
-    rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
+    rc = ncnnhip_attention_f32_strided(d_qa, q_stride, fused_qkv ? scale : 1.f, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws,
+                                       att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
     rc = blockquant_gemm_with_scratch(leases, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);
@@ -435,11 +481,17 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         d_vt = (float*)scratch.get(E * dst * 4);
         if (!d_kt || !d_vt) return -100;
     }
-    float* d_qa = (float*)scratch.get((size_t)src * E * 4);
+    const bool fused_qkv = dev_qkv[0] && self_attention; // one blob in, q / k / v out of one Gemm
+    const size_t q_stride = fused_qkv ? 3 * E : E;
+    float* d_qa = (float*)scratch.get((size_t)src * q_stride * 4);
     float* d_ctx = (float*)scratch.get((size_t)src * E * 4);
     if (!d_qa || !d_ctx) return -100;
 
-    rc = blockquant_gemm_with_scratch(scratch, (const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
+    if (fused_qkv)
+        rc = blockquant_gemm_with_scratch(scratch, (const float*)q_blob.data, (size_t)qdim, src, 3 * embed_dim, qdim, dev_qkv[0], bits, block, dev_qkv[1], dev_qkv[2], dev_qkv[4],
+                                    dev_qkv[5], (const float*)dev_qkv[3], 4, 1.f, 1.f, d_qa, q_stride, st);
+    else
+        rc = blockquant_gemm_with_scratch(scratch, (const float*)q_blob.data, (size_t)qdim, src, embed_dim, qdim, dev[0][0], bits, block, dev[0][1], dev[0][2], dev[0][4], dev[0][5],
                                     (const float*)dev[0][3], 4, scale, 1.f, d_qa, E, st);
     if (rc != 0) return to_ncnn_status(rc, "q projection");
     if (!reuse_cache)
@@ -453,7 +505,12 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         const HipMat* in[2] = {&k_blob, &v_blob};
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
-        for (int t = 0; t < 2; t++)
+        for (int t = 0; t < 2 && fused_qkv; t++)
+        {
+            rc = ncnnhip_transpose_f32(d_qa + (1 + t) * E, q_stride, cur, embed_dim, outT[t] + past, (size_t)dst, st);
+            if (rc != 0) return to_ncnn_status(rc, "k/v columns");
+        }
+        for (int t = 0; t < 2 && !fused_qkv; t++)
         {
             float* d_aff = (float*)scratch.get((size_t)cur * E * 4);
             if (!d_aff) return -100;
@@ -468,7 +525,8 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
     void* att_ws = att_ws_bytes ? scratch.get(att_ws_bytes) : 0;
     if (att_ws_bytes && !att_ws) return -100;
-    rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
+    rc = ncnnhip_attention_f32_strided(d_qa, q_stride, fused_qkv ? scale : 1.f, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws,
+                                       att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
     rc = blockquant_gemm_with_scratch(scratch, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);

@@ -717,3 +717,18 @@ def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
     # fp32 sums over head_dim and dst terms of O(1) values, device expf
     assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
     assert np.abs(plain - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("heads,hd,src,dst", [(4, 64, 37, 200), (2, 32, 1, 300), (3, 24, 5, 40)])
+def test_attention_reads_strided_queries_and_scales_them_on_load(rt, heads, hd, src, dst):
+    """Queries taken out of a wider row (q, k and v made by one Gemm) and multiplied by the layer's scale where they are read:
+    bit for bit what the plain entry gives on the scaled queries (src/layer/multiheadattention.cpp:634 rounds the same product)."""
+    rng = np.random.default_rng(heads + dst)
+    e = heads * hd
+    wide = rng.normal(0, 1, (src, 3 * e)).astype(F)
+    kt = rng.normal(0, 1, (e, dst)).astype(F)
+    vt = rng.normal(0, 1, (e, dst)).astype(F)
+    scale = F(1.0 / np.sqrt(hd))
+    want = rt.attention(wide[:, :e] * scale, kt, vt, heads)
+    got = rt.attention(wide, kt, vt, heads, q_scale=scale)
+    assert np.array_equal(got, want)
