@@ -305,6 +305,11 @@ int ncnnhip_transpose_f32(const float* src_dev, size_t src_stride, int rows, int
                           void* stream);
 int ncnnhip_transpose_s8(const int8_t* src_dev, size_t src_stride, int rows, int cols, int8_t* dst_dev, size_t dst_stride,
                          void* stream);
+/* Two fp32 transposes of one shape and one pair of strides in a single launch: the new key and value rows of
+ * MultiHeadAttention written as columns past.. of the [embed_dim][time] blobs (src/layer/multiheadattention.cpp:662-692,
+ * 716-746 write k_affine / v_affine column by column). */
+int ncnnhip_transpose_pair_f32(const float* src_a_dev, const float* src_b_dev, size_t src_stride, int rows, int cols,
+                               float* dst_a_dev, float* dst_b_dev, size_t dst_stride, void* stream);
 
 /* gemm_transB_int8 (src/layer/gemm.cpp:495-567): out = alpha*((float)acc / (sA_i*sB) + beta*C).
  * aq [M][K], bq [N][K] (K contiguous).  n_b_scales == 1 is ncnn's per-tensor B scale;

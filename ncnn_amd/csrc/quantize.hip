@@ -184,6 +184,30 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ sr
     }
 }
 
+// two transposes of the same shape and strides in one launch (the key and the value columns of an attention layer's cache)
+__global__ __launch_bounds__(256) void transpose_pair_kernel(const float* __restrict__ src_a, const float* __restrict__ src_b, size_t ss, int rows, int cols,
+                                                             float* __restrict__ dst_a, float* __restrict__ dst_b, size_t ds)
+{
+    __shared__ float tile[32][33];
+    const float* __restrict__ src = blockIdx.z ? src_b : src_a;
+    float* __restrict__ dst = blockIdx.z ? dst_b : dst_a;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+#pragma unroll
+    for (int k = 0; k < 32; k += 8)
+    {
+        const int r = r0 + ty + k, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + k][tx] = src[(size_t)r * ss + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 32; k += 8)
+    {
+        const int c = c0 + ty + k, r = r0 + tx; // dst[c][r]
+        if (r < rows && c < cols) dst[(size_t)c * ds + r] = tile[tx][ty + k];
+    }
+}
+
 static inline bool aligned(const void* p, size_t a)
 {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
@@ -288,6 +312,16 @@ int ncnnhip_transpose_f32(const float* src_dev, size_t src_stride, int rows, int
     NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_transpose_f32: too many rows");
     hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, as_stream(stream), src_dev, src_stride, rows, cols, dst_dev, dst_stride);
     return launch_status("transpose_kernel<float>");
+}
+
+int ncnnhip_transpose_pair_f32(const float* src_a_dev, const float* src_b_dev, size_t src_stride, int rows, int cols, float* dst_a_dev, float* dst_b_dev,
+                               size_t dst_stride, void* stream)
+{
+    NCNNHIP_REQUIRE(src_a_dev && src_b_dev && dst_a_dev && dst_b_dev && rows >= 1 && cols >= 1, "ncnnhip_transpose_pair_f32: bad argument");
+    dim3 grid(ceil_div(cols, 32), ceil_div(rows, 32), 2);
+    NCNNHIP_REQUIRE(grid.y <= 65535, "ncnnhip_transpose_pair_f32: too many rows");
+    hipLaunchKernelGGL(transpose_pair_kernel, grid, dim3(256), 0, as_stream(stream), src_a_dev, src_b_dev, src_stride, rows, cols, dst_a_dev, dst_b_dev, dst_stride);
+    return launch_status("transpose_pair_kernel");
 }
 
 int ncnnhip_transpose_s8(const int8_t* src_dev, size_t src_stride, int rows, int cols, int8_t* dst_dev, size_t dst_stride, void* stream)

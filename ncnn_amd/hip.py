@@ -125,6 +125,7 @@ _SIGNATURES = {
     "ncnnhip_gemm_quantize_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_quantize_tensor": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
     "ncnnhip_transpose_f32": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_transpose_pair_f32": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_transpose_s8": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_gemm_int8": [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
                           C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
@@ -670,6 +671,18 @@ class Runtime:
         fn = lib().ncnnhip_transpose_f32 if a.dtype == np.float32 else lib().ncnnhip_transpose_s8
         check(fn(da.ptr, c_, r, c_, dt.ptr, r, self.stream))
         return dt.to_numpy(self.stream)
+
+    def transpose_pair_into(self, wide, col_a, col_b, cols, dst_a, dst_b, past):
+        """Columns [col_a, col_a+cols) and [col_b, col_b+cols) of the fp32 matrix `wide`, transposed, written as columns past.. of dst_a / dst_b
+        ([cols][time], returned as new arrays)."""
+        wide = np.ascontiguousarray(wide, np.float32)
+        rows, stride = wide.shape
+        dst_a, dst_b = [np.ascontiguousarray(d, np.float32) for d in (dst_a, dst_b)]
+        time = dst_a.shape[1]
+        dw, da, db = self.up(wide), self.up(dst_a), self.up(dst_b)
+        check(lib().ncnnhip_transpose_pair_f32(C.c_void_p(dw.ptr.value + col_a * 4), C.c_void_p(dw.ptr.value + col_b * 4), stride, rows, cols,
+                                               C.c_void_p(da.ptr.value + past * 4), C.c_void_p(db.ptr.value + past * 4), time, self.stream))
+        return da.to_numpy(self.stream), db.to_numpy(self.stream)
 
     # -- block-quantised Gemm -----------------------------------------------------------------
     def gemm_blockquant(self, a, b_packed, scales, bits, block, in_scales=None, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0):

@@ -310,9 +310,9 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
         float* d_kv_in = 0;
-        for (int t = 0; t < 2 && fused_qkv; t++)
+        if (fused_qkv)
         {
-            rc = ncnnhip_transpose_f32(d_qa + (1 + t) * E, q_stride, cur, embed_dim, outT[t] + past, (size_t)dst, st);
+            rc = ncnnhip_transpose_pair_f32(d_qa + E, d_qa + 2 * E, q_stride, cur, embed_dim, outT[0] + past, outT[1] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v columns");
         }
         for (int t = 0; t < 2 && !fused_qkv; t++)
@@ -505,9 +505,9 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         const HipMat* in[2] = {&k_blob, &v_blob};
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
-        for (int t = 0; t < 2 && fused_qkv; t++)
+        if (fused_qkv)
         {
-            rc = ncnnhip_transpose_f32(d_qa + (1 + t) * E, q_stride, cur, embed_dim, outT[t] + past, (size_t)dst, st);
+            rc = ncnnhip_transpose_pair_f32(d_qa + E, d_qa + 2 * E, q_stride, cur, embed_dim, outT[0] + past, outT[1] + past, (size_t)dst, st);
             if (rc != 0) return to_ncnn_status(rc, "k/v columns");
         }
         for (int t = 0; t < 2 && !fused_qkv; t++)

@@ -732,3 +732,16 @@ def test_attention_reads_strided_queries_and_scales_them_on_load(rt, heads, hd, 
     want = rt.attention(wide[:, :e] * scale, kt, vt, heads)
     got = rt.attention(wide, kt, vt, heads, q_scale=scale)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("rows,cols,past", [(1, 64, 13), (37, 96, 0), (70, 33, 5)])
+def test_transpose_pair_appends_key_and_value_columns(rt, rows, cols, past):
+    rng = np.random.default_rng(rows + cols)
+    wide = rng.normal(0, 1, (rows, 3 * cols)).astype(F)
+    ka = rng.normal(0, 1, (cols, past + rows)).astype(F)
+    va = rng.normal(0, 1, (cols, past + rows)).astype(F)
+    got_k, got_v = rt.transpose_pair_into(wide, cols, 2 * cols, cols, ka, va, past)
+    want_k, want_v = ka.copy(), va.copy()
+    want_k[:, past:] = wide[:, cols:2 * cols].T
+    want_v[:, past:] = wide[:, 2 * cols:].T
+    assert np.array_equal(got_k, want_k) and np.array_equal(got_v, want_v)
