@@ -406,7 +406,9 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
  * the layer's cache blobs; mask is additive, [src][dst] (mask_heads 1) or [num_heads][src][dst], or NULL.
  * Head dimensions 32/64/96/128 run on the fp32 matrix cores with any dst_seqlen; others need head_dim + dst_seqlen <= 4096.
  * With few queries and many keys (decoding against a cache) the keys are split over workgroups if the caller passes
- * the scratch ncnnhip_attention_workspace_bytes asks for (may be 0 / NULL: then one workgroup per head and 32 queries). */
+ * the scratch ncnnhip_attention_workspace_bytes asks for (may be 0 / NULL: then one workgroup per head and 32 queries);
+ * one to four queries on 256 to 32768 keys then run on a streaming kernel of their own (64 keys per workgroup, any
+ * head_dim up to 256) followed by a merge. */
 int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqlen, int dst_seqlen, size_t* workspace_bytes);
 int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
                           int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev,

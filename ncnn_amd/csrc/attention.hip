@@ -415,6 +415,222 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     }
 }
 
+// ---- one to four queries on a long key sequence (a decoding step against a cache) ------------------------------------
+// With so few queries the work is reading the keys and values once, and the matrix-core kernel above, built around 32
+// queries per workgroup, spends its time in a chain of latencies.  Here one workgroup streams 64 keys of one head:
+//   scores : thread = (key, quarter of the channels); k[channel][key] is read coalesced along the keys, the four partial
+//            dot products of a key are added through LDS;
+//   softmax: wavefront t takes query t (maximum, exp, sum over the 64 keys by shuffles);
+//   p v    : thread = (channel, quarter of the keys); v[channel][key] is read as 16-byte pieces along the keys, four lanes
+//            add their parts by shuffles.
+// It leaves (maximum, sum, unnormalised output) per query for attention_fewq_merge_kernel.  fp32 throughout; the order of
+// the additions differs from the reference's: fp32 tolerance.
+static constexpr int FEWQ_KEYS = 64;
+static constexpr int FEWQ_MAX_HEAD_DIM = 256;
+
+// 16 consecutive values of one channel from key j on: 16-byte pieces where the rows allow, else one by one (a key past the
+// end repeats the last one; its probability is 0)
+__device__ __forceinline__ void load_fewq_values(float (&vv)[16], const float* __restrict__ vr, int j, int dst, bool vec)
+{
+    if (vec)
+    {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+        {
+            const v4f_at t4 = *reinterpret_cast<const v4f_at*>(vr + j + 4 * a);
+#pragma unroll
+            for (int e = 0; e < 4; e++) vv[4 * a + e] = t4[e];
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int e = 0; e < 16; e++) vv[e] = vr[j + e < dst ? j + e : dst - 1];
+    }
+}
+
+__global__ __launch_bounds__(256) void attention_fewq_split_kernel(const float* __restrict__ q, size_t q_stride, float q_scale, const float* __restrict__ kt,
+                                                                   const float* __restrict__ vt, size_t kv_stride, const float* __restrict__ mask, int mask_heads,
+                                                                   int head_dim, int src, int dst, int v_vec_ok, float* __restrict__ partial)
+{
+    __shared__ float qs[ATT_TQ * FEWQ_MAX_HEAD_DIM];
+    __shared__ float red[4][ATT_TQ][FEWQ_KEYS];
+    __shared__ float sc[ATT_TQ][FEWQ_KEYS];
+    const int split = blockIdx.x, h = blockIdx.y, i0 = blockIdx.z * ATT_TQ;
+    const int rows = src - i0 < ATT_TQ ? src - i0 : ATT_TQ;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j0 = split * FEWQ_KEYS;
+
+    // every load that does not depend on the scores is requested before the first wait: the first 16 channels of this
+    // wavefront's keys, this thread's values of the first 64 channels, the queries
+    const int per = (head_dim + 3) >> 2, c0 = wave * per, c1 = c0 + per < head_dim ? c0 + per : head_dim;
+    const int key = j0 + lane < dst ? j0 + lane : dst - 1; // past the end: repeated, dropped below
+    const float* kp = kt + ((size_t)h * head_dim + c0) * kv_stride + key;
+    float kfirst[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) kfirst[i] = c0 + i < c1 ? kp[(size_t)i * kv_stride] : 0.f;
+    const int kq = tid & 3;
+    const bool vec = v_vec_ok && j0 + FEWQ_KEYS <= dst;
+    float vfirst[16];
+    load_fewq_values(vfirst, vt + ((size_t)h * head_dim + ((tid >> 2) < head_dim ? (tid >> 2) : 0)) * kv_stride, j0 + 16 * kq, dst, vec);
+    for (int e = tid; e < ATT_TQ * head_dim; e += 256)
+    {
+        const int t = e / head_dim, l = e - t * head_dim;
+        qs[e] = t < rows ? mul_rn(q[(size_t)(i0 + t) * q_stride + h * head_dim + l], q_scale) : 0.f;
+    }
+    __syncthreads();
+
+    // ---- scores: wavefront g takes the g-th quarter of the channels, lane = key
+    {
+        float acc[ATT_TQ];
+#pragma unroll
+        for (int t = 0; t < ATT_TQ; t++) acc[t] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            if (c0 + i < c1)
+            {
+#pragma unroll
+                for (int t = 0; t < ATT_TQ; t++) acc[t] = add_rn(acc[t], mul_rn(qs[t * head_dim + c0 + i], kfirst[i]));
+            }
+        kp += (size_t)16 * kv_stride;
+#pragma unroll 8
+        for (int c = c0 + 16; c < c1; c++)
+        {
+            const float kv = *kp;
+            kp += kv_stride;
+#pragma unroll
+            for (int t = 0; t < ATT_TQ; t++) acc[t] = add_rn(acc[t], mul_rn(qs[t * head_dim + c], kv));
+        }
+#pragma unroll
+        for (int t = 0; t < ATT_TQ; t++) red[wave][t][lane] = acc[t];
+    }
+    __syncthreads();
+
+    // ---- softmax over this workgroup's keys: wavefront t = query t
+    float m_t = -FLT_MAX, l_t = 0.f;
+    {
+        const int t = wave;
+        float s = add_rn(add_rn(red[0][t][lane], red[1][t][lane]), add_rn(red[2][t][lane], red[3][t][lane]));
+        const bool live = j0 + lane < dst && t < rows;
+        if (live && mask) s = add_rn(s, mask[((size_t)(mask_heads > 1 ? h : 0) * src + i0 + t) * dst + j0 + lane]);
+        if (!live) s = -INFINITY;
+        m_t = fmaxf(wave_max(s), -FLT_MAX); // a query that is not there (or all keys at -inf): every probability 0
+        const float pr = exp_of_nonpositive(s - m_t);
+        l_t = wave_sum(pr);
+        sc[t][lane] = pr;
+    }
+    __syncthreads();
+
+    // ---- p v: thread = (channel tid/4, keys 16*(tid%4)..+15), four lanes share a channel
+    float* rec = partial + (((size_t)blockIdx.z * gridDim.y + h) * gridDim.x + split) * (size_t)(2 * ATT_TQ + ATT_TQ * head_dim);
+    for (int ch = tid >> 2; ch < ((head_dim + 63) & ~63); ch += 64)
+    {
+        float acc[ATT_TQ];
+#pragma unroll
+        for (int t = 0; t < ATT_TQ; t++) acc[t] = 0.f;
+        if (ch < head_dim)
+        {
+            float vv[16];
+            if (ch < 64)
+            {
+#pragma unroll
+                for (int e = 0; e < 16; e++) vv[e] = vfirst[e];
+            }
+            else
+                load_fewq_values(vv, vt + ((size_t)h * head_dim + ch) * kv_stride, j0 + 16 * kq, dst, vec);
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+#pragma unroll
+                for (int t = 0; t < ATT_TQ; t++) acc[t] = add_rn(acc[t], mul_rn(sc[t][16 * kq + e], vv[e]));
+        }
+#pragma unroll
+        for (int t = 0; t < ATT_TQ; t++)
+        {
+            acc[t] = add_rn(acc[t], __shfl_xor(acc[t], 1));
+            acc[t] = add_rn(acc[t], __shfl_xor(acc[t], 2));
+        }
+        if (kq == 0 && ch < head_dim)
+#pragma unroll
+            for (int t = 0; t < ATT_TQ; t++) rec[2 * ATT_TQ + t * head_dim + ch] = acc[t];
+    }
+    if (lane == 0)
+    {
+        rec[wave] = m_t;
+        rec[ATT_TQ + wave] = l_t;
+    }
+}
+
+// merges the records of attention_fewq_split_kernel: one workgroup per (head, group of four queries).  The maxima and
+// sums of all splits are fetched side by side into LDS (wavefront t = query t) and turned into one factor per split;
+// then four groups of 64 threads each add every fourth split's outputs, eight loads in flight, and the groups' parts
+// are added through LDS - a thread that walks the splits one load after the other takes 14 us for 24 of them.
+static constexpr int FEWQ_MAX_SPLITS = 512;
+
+__global__ __launch_bounds__(256) void attention_fewq_merge_kernel(const float* __restrict__ partial, int splits, int head_dim, int embed_dim, int src,
+                                                                   float* __restrict__ out)
+{
+    __shared__ float fac[ATT_TQ][FEWQ_MAX_SPLITS];
+    __shared__ float l_all[ATT_TQ];
+    __shared__ float part[4][64];
+    const int h = blockIdx.x, i0 = blockIdx.y * ATT_TQ;
+    const int rows = src - i0 < ATT_TQ ? src - i0 : ATT_TQ;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const size_t rec_size = (size_t)(2 * ATT_TQ + ATT_TQ * head_dim);
+    const float* rec0 = partial + ((size_t)blockIdx.y * gridDim.x + h) * splits * rec_size;
+    {
+        const int t = wave;
+        float ma = -FLT_MAX;
+        for (int z = lane; z < splits; z += 64)
+        {
+            const float mz = rec0[z * rec_size + t];
+            fac[t][z] = mz;
+            ma = fmaxf(ma, mz);
+        }
+        ma = wave_max(ma);
+        float lt = 0.f;
+        for (int z = lane; z < splits; z += 64) // each lane reads back what it wrote
+        {
+            const float f = exp_of_nonpositive(fac[t][z] - ma);
+            fac[t][z] = f;
+            lt += rec0[z * rec_size + ATT_TQ + t] * f;
+        }
+        lt = wave_sum(lt);
+        if (lane == 0) l_all[t] = lt;
+    }
+    __syncthreads();
+    for (int base = 0; base < rows * head_dim; base += 64)
+    {
+        const int idx = base + lane;
+        float ot = 0.f;
+        if (idx < rows * head_dim)
+        {
+            const int t = idx / head_dim;
+            const float* op = rec0 + 2 * ATT_TQ + idx;
+#pragma unroll 8
+            for (int z = wave; z < splits; z += 4) ot += op[z * rec_size] * fac[t][z];
+        }
+        part[wave][lane] = ot;
+        __syncthreads();
+        if (wave == 0 && idx < rows * head_dim)
+        {
+            const int t = idx / head_dim;
+            const float sum = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+            out[(size_t)(i0 + t) * embed_dim + h * head_dim + (idx - t * head_dim)] = div_rn(sum, l_all[t]);
+        }
+        __syncthreads();
+    }
+}
+
+// the few-query kernels take over where they apply: up to four queries, a key sequence long enough to be worth splitting
+static bool attention_fewq_applies(int head_dim, int src, int dst)
+{
+    return src <= ATT_TQ && dst >= 256 && dst <= FEWQ_KEYS * FEWQ_MAX_SPLITS && head_dim <= FEWQ_MAX_HEAD_DIM;
+}
+static size_t attention_fewq_workspace_bytes(int num_heads, int head_dim, int src, int dst)
+{
+    return (size_t)((src + ATT_TQ - 1) / ATT_TQ) * num_heads * ((dst + FEWQ_KEYS - 1) / FEWQ_KEYS) * (size_t)(2 * ATT_TQ + ATT_TQ * head_dim) * sizeof(float);
+}
+
 // how many ways to split the keys: enough workgroups for the chip, at least 128 keys (one tile per wavefront) each.
 // (With 256 workgroups or more a split does not pay even where the last round over the chip is mostly empty - 47 query
 // blocks x 16 heads at head dimension 64 run in 1.47 rounds of 512: split in two, the kernel took 145 us against 136 and
@@ -445,6 +661,11 @@ int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqle
         const int splits = attention_key_splits(num_heads, src_seqlen, dst_seqlen);
         if (splits > 1) *workspace_bytes = (size_t)((src_seqlen + 31) / 32) * num_heads * splits * (size_t)(64 + head_dim * 32) * sizeof(float);
     }
+    if (attention_fewq_applies(head_dim, src_seqlen, dst_seqlen))
+    {
+        const size_t need = attention_fewq_workspace_bytes(num_heads, head_dim, src_seqlen, dst_seqlen);
+        if (need > *workspace_bytes) *workspace_bytes = need;
+    }
     return NCNNHIP_OK;
 }
 
@@ -467,6 +688,18 @@ int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_s
     NCNNHIP_REQUIRE(kv_stride >= (size_t)dst_seqlen, "ncnnhip_attention_f32: key/value row stride below dst_seqlen");
     NCNNHIP_REQUIRE(kv_stride + (size_t)dst_seqlen < ((size_t)1 << 30), "ncnnhip_attention_f32: key/value row stride beyond the 32-bit byte offsets of the kernel");
     NCNNHIP_REQUIRE(!mask_dev || mask_heads == 1 || mask_heads == num_heads, "ncnnhip_attention_f32: the mask is shared (1) or one per head");
+    if (attention_fewq_applies(head_dim, src_seqlen, dst_seqlen) && workspace_dev
+        && workspace_bytes >= attention_fewq_workspace_bytes(num_heads, head_dim, src_seqlen, dst_seqlen))
+    {
+        const int v_vec_ok = (kv_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(vt_dev) & 15) == 0) ? 1 : 0;
+        const int splits = (dst_seqlen + FEWQ_KEYS - 1) / FEWQ_KEYS, qgroups = (src_seqlen + ATT_TQ - 1) / ATT_TQ;
+        hipStream_t st = as_stream(stream);
+        hipLaunchKernelGGL(attention_fewq_split_kernel, dim3((unsigned)splits, (unsigned)num_heads, (unsigned)qgroups), dim3(256), 0, st, q_dev, q_stride, q_scale, kt_dev,
+                           vt_dev, kv_stride, mask_dev, mask_dev ? mask_heads : 0, head_dim, src_seqlen, dst_seqlen, v_vec_ok, (float*)workspace_dev);
+        hipLaunchKernelGGL(attention_fewq_merge_kernel, dim3((unsigned)num_heads, (unsigned)qgroups), dim3(256), 0, st, (const float*)workspace_dev, splits, head_dim,
+                           num_heads * head_dim, src_seqlen, out_dev);
+        return launch_status("attention_fewq_split_kernel");
+    }
     if (head_dim % 32 == 0 && head_dim <= 128)
     {
         // 16-byte loads of the values need the rows and the start aligned

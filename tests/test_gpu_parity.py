@@ -688,8 +688,11 @@ def test_blockquant_exact_on_power_of_two_data(rt):
 @pytest.mark.parametrize("heads,hd,src,dst,mask", [(4, 16, 9, 9, None), (3, 24, 7, 130, "2d"), (8, 64, 5, 300, "3d"), (2, 32, 1, 1, None), (1, 8, 70, 3, "2d"),
                                                     # head dimensions of the matrix-core kernel: ragged query blocks and key tiles, one to many tiles per wavefront
                                                     (2, 96, 40, 70, "2d"), (1, 128, 33, 257, None), (4, 64, 100, 129, "3d"), (2, 64, 64, 1024, None), (3, 32, 1, 515, "2d"), (16, 64, 1, 1500, None), (2, 128, 33, 4100, "3d"),
-                                                    # many workgroups whose last round over the chip would be mostly empty: the keys are split in two
-                                                    (16, 64, 1500, 1500, None), (16, 32, 1920, 300, "2d")])
+                                                    # many workgroups (two and a half per compute unit)
+                                                    (16, 64, 1500, 1500, None), (16, 32, 1920, 300, "2d"),
+                                                    # one to four queries on 256 keys and more: the streaming kernels (64 keys per workgroup + merge), head
+                                                    # dimensions of any size, partial last chunks, rows that are / are not 16-byte aligned
+                                                    (4, 40, 3, 700, "3d"), (2, 200, 4, 260, None), (5, 64, 2, 1024, "2d"), (1, 256, 4, 301, None), (3, 7, 1, 257, "2d")])
 def test_attention_core_matches_float64(rt, heads, hd, src, dst, mask):
     rng = np.random.default_rng(heads * 100 + dst)
     e = heads * hd
