@@ -94,4 +94,6 @@ MHA_CASES = [
     (5, 64, 2, 48, 56, 56, 3, 4, 8, 32, True, 10, False, "2d"),    # cross attention on cached keys / values
     (6, 64, 4, 64, 64, 64, 40, 40, 8, 64, False, 0, True, None),   # 32 rows and more: the projections take the tiled kernel with its workspace
     (7, 128, 8, 128, 128, 128, 33, 33, 4, 32, True, 0, True, "2d"),
+    (8, 64, 2, 64, 64, 64, 1, 1, 8, 64, False, 300, True, None),   # decode steps on a long cache: the few-query attention kernels
+    (9, 96, 4, 96, 96, 96, 3, 3, 8, 32, False, 401, True, "2d"),
 ]
