@@ -512,12 +512,10 @@ def bench_mha(args, embed, heads, src, past):
 
     def step():
         # self-attention: q, k and v out of one Gemm over the three weight matrices as one (what create_pipeline keeps for this case),
-        # k and v transposed out of its rows into the cache columns, the query's scale applied where the attention kernel reads it
+        # its k and v columns appended to the cache and the query's scale applied by the attention call
         project(d_x, w_qkv, 3 * embed, d_qkv, 3 * embed)
-        check(lib.ncnnhip_transpose_pair_f32(C.c_void_p(d_qkv.ptr.value + embed * 4), C.c_void_p(d_qkv.ptr.value + 2 * embed * 4), 3 * embed, src, embed,
-                                             C.c_void_p(d_kt.ptr.value + past * 4), C.c_void_p(d_vt.ptr.value + past * 4), dst, st))
-        check(lib.ncnnhip_attention_f32_strided(d_qkv.ptr, 3 * embed, scale, d_kt.ptr, d_vt.ptr, dst, None, 0, heads, embed // heads, src, dst, d_ctx.ptr, d_ws.ptr,
-                                                wsb.value, st))
+        check(lib.ncnnhip_attention_f32_append(d_qkv.ptr, 3 * embed, scale, d_kt.ptr, d_vt.ptr, dst, past, None, 0, heads, embed // heads, src, d_ctx.ptr, d_ws.ptr,
+                                               wsb.value, st))
         project(d_ctx, ws[3], embed, d_out, embed)
 
     for _ in range(args.warmup):
@@ -541,7 +539,7 @@ def bench_mha(args, embed, heads, src, past):
         "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "self-attention layer, embed %d, %d heads, %d new tokens on a cache of %d, 8-bit block-quantised weights (blocks of 64)"
-                               % (embed, heads, src, past), "launches_per_step": (6 if rows_ws is not None else 4) + (1 if wsb.value else 0), "projections": "tiled bf16x3 kernel" if rows_ws is not None else ("packed tiles" if packed_ok else ".bin layout"), "device_ms_per_step": k_ms, "gflop": ops / 1e9},
+                               % (embed, heads, src, past), "launches_per_step": (6 if rows_ws is not None else 3) + (1 if wsb.value else 0), "projections": "tiled bf16x3 kernel" if rows_ws is not None else ("packed tiles" if packed_ok else ".bin layout"), "device_ms_per_step": k_ms, "gflop": ops / 1e9},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "whole layer (q/k/v projection, cache append, attention core, output projection)", "bytes_per_launch": algo},
     }

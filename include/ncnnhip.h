@@ -419,6 +419,16 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
 int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_scale, const float* kt_dev, const float* vt_dev,
                                   size_t kv_stride, const float* mask_dev, int mask_heads, int num_heads, int head_dim, int src_seqlen,
                                   int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
+/* Self-attention on rows that hold q, k and v side by side ([src_seqlen][>= 3*embed_dim]: q at column 0, k at embed_dim, v at
+ * 2*embed_dim): the new keys and values are first written as columns past_seqlen.. of kt / vt (rows of kv_stride >=
+ * past_seqlen + src_seqlen; columns 0..past_seqlen-1 hold the cache), then the attention runs over all past_seqlen +
+ * src_seqlen keys - what src/layer/multiheadattention.cpp:640-746 does by writing k_affine / v_affine behind the cached
+ * columns.  One to four queries on 256 keys and more write the columns inside the attention kernel (no launch of their
+ * own); other shapes run ncnnhip_transpose_pair_f32 first.  Workspace as for ncnnhip_attention_f32 with dst_seqlen =
+ * past_seqlen + src_seqlen. */
+int ncnnhip_attention_f32_append(const float* qkv_dev, size_t qkv_stride, float q_scale, float* kt_dev, float* vt_dev, size_t kv_stride,
+                                 int past_seqlen, const float* mask_dev, int mask_heads, int num_heads, int head_dim, int src_seqlen,
+                                 float* out_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ measured ceilings (benchmark support)
  * No counterpart in the reference.  What this chip sustains, to set beside the published peaks in a roofline line:

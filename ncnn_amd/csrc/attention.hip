@@ -11,6 +11,7 @@
 //   p v    : a wavefront takes channels w, w+4, ...; lanes stride over time reading v[channel][k] coalesced, then a
 //            shuffle reduction (so the sum over k is a tree, not the reference's sequence: fp32 tolerance)
 #include <float.h>
+#include <limits.h>
 
 #include "common.h"
 
@@ -449,9 +450,13 @@ __device__ __forceinline__ void load_fewq_values(float (&vv)[16], const float* _
     }
 }
 
-__global__ __launch_bounds__(256) void attention_fewq_split_kernel(const float* __restrict__ q, size_t q_stride, float q_scale, const float* __restrict__ kt,
-                                                                   const float* __restrict__ vt, size_t kv_stride, const float* __restrict__ mask, int mask_heads,
-                                                                   int head_dim, int src, int dst, int v_vec_ok, float* __restrict__ partial)
+// new_k / new_v (or null): the keys and values of the last dst - past positions, rows of new_stride floats ([position][embed]).
+// The workgroup whose 64 keys reach past `past` first copies its share of them into kt / vt (appending to the cache is then
+// no launch of its own) and reads them back like the rest after a barrier; nobody else reads those columns.
+__global__ __launch_bounds__(256) void attention_fewq_split_kernel(const float* __restrict__ q, size_t q_stride, float q_scale, float* kt, float* vt, size_t kv_stride,
+                                                                   const float* __restrict__ mask, int mask_heads, int head_dim, int src, int dst, int v_vec_ok,
+                                                                   float* __restrict__ partial, const float* __restrict__ new_k, const float* __restrict__ new_v,
+                                                                   size_t new_stride, int past)
 {
     __shared__ float qs[ATT_TQ * FEWQ_MAX_HEAD_DIM];
     __shared__ float red[4][ATT_TQ][FEWQ_KEYS];
@@ -461,6 +466,20 @@ __global__ __launch_bounds__(256) void attention_fewq_split_kernel(const float* 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j0 = split * FEWQ_KEYS;
 
+    if (new_k && j0 + FEWQ_KEYS > past) // uniform
+    {
+        const int kb = j0 > past ? j0 : past, ke = j0 + FEWQ_KEYS < dst ? j0 + FEWQ_KEYS : dst;
+        for (int e = tid; e < (ke - kb) * head_dim; e += 256)
+        {
+            const int pos = e / head_dim, c = e - pos * head_dim;
+            const size_t from = (size_t)(kb + pos - past) * new_stride + (size_t)h * head_dim + c;
+            const size_t to = ((size_t)h * head_dim + c) * kv_stride + kb + pos;
+            kt[to] = new_k[from];
+            vt[to] = new_v[from];
+        }
+        __threadfence_block();
+        __syncthreads();
+    }
     // every load that does not depend on the scores is requested before the first wait: the first 16 channels of this
     // wavefront's keys, this thread's values of the first 64 channels, the queries
     const int per = (head_dim + 3) >> 2, c0 = wave * per, c1 = c0 + per < head_dim ? c0 + per : head_dim;
@@ -669,6 +688,11 @@ int ncnnhip_attention_workspace_bytes(int num_heads, int head_dim, int src_seqle
     return NCNNHIP_OK;
 }
 
+// append_k / append_v (or null): new rows to be written into columns past.. of kt / vt before they are read
+static int attention_dispatch(const float* q_dev, size_t q_stride, float q_scale, float* kt_dev, float* vt_dev, size_t kv_stride, const float* mask_dev, int mask_heads,
+                              int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes, void* stream,
+                              const float* append_k, const float* append_v, size_t append_stride, int past);
+
 int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev, int mask_heads,
                           int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes,
                           void* stream)
@@ -680,6 +704,28 @@ int ncnnhip_attention_f32(const float* q_dev, const float* kt_dev, const float* 
 int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_scale, const float* kt_dev, const float* vt_dev, size_t kv_stride, const float* mask_dev,
                                   int mask_heads, int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev,
                                   size_t workspace_bytes, void* stream)
+{
+    return attention_dispatch(q_dev, q_stride, q_scale, const_cast<float*>(kt_dev), const_cast<float*>(vt_dev), kv_stride, mask_dev, mask_heads, num_heads, head_dim,
+                              src_seqlen, dst_seqlen, out_dev, workspace_dev, workspace_bytes, stream, nullptr, nullptr, 0, 0);
+}
+
+int ncnnhip_attention_f32_append(const float* qkv_dev, size_t qkv_stride, float q_scale, float* kt_dev, float* vt_dev, size_t kv_stride, int past_seqlen,
+                                 const float* mask_dev, int mask_heads, int num_heads, int head_dim, int src_seqlen, float* out_dev, void* workspace_dev,
+                                 size_t workspace_bytes, void* stream)
+{
+    NCNNHIP_REQUIRE(qkv_dev && num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && past_seqlen >= 0, "ncnnhip_attention_f32_append: bad argument");
+    const size_t e = (size_t)num_heads * (size_t)head_dim;
+    NCNNHIP_REQUIRE(qkv_stride >= 3 * e, "ncnnhip_attention_f32_append: rows of q, k and v need a stride of at least 3 * embed_dim");
+    NCNNHIP_REQUIRE(past_seqlen <= INT_MAX - src_seqlen, "ncnnhip_attention_f32_append: sequence too long");
+    return attention_dispatch(qkv_dev, qkv_stride, q_scale, kt_dev, vt_dev, kv_stride, mask_dev, mask_heads, num_heads, head_dim, src_seqlen, past_seqlen + src_seqlen,
+                              out_dev, workspace_dev, workspace_bytes, stream, qkv_dev + e, qkv_dev + 2 * e, qkv_stride, past_seqlen);
+}
+
+} // extern "C"
+
+static int attention_dispatch(const float* q_dev, size_t q_stride, float q_scale, float* kt_dev, float* vt_dev, size_t kv_stride, const float* mask_dev, int mask_heads,
+                              int num_heads, int head_dim, int src_seqlen, int dst_seqlen, float* out_dev, void* workspace_dev, size_t workspace_bytes, void* stream,
+                              const float* append_k, const float* append_v, size_t append_stride, int past)
 {
     NCNNHIP_REQUIRE(q_dev && kt_dev && vt_dev && out_dev, "ncnnhip_attention_f32: null pointer");
     NCNNHIP_REQUIRE(num_heads >= 1 && head_dim >= 1 && src_seqlen >= 1 && dst_seqlen >= 1, "ncnnhip_attention_f32: bad shape");
@@ -695,10 +741,17 @@ int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_s
         const int splits = (dst_seqlen + FEWQ_KEYS - 1) / FEWQ_KEYS, qgroups = (src_seqlen + ATT_TQ - 1) / ATT_TQ;
         hipStream_t st = as_stream(stream);
         hipLaunchKernelGGL(attention_fewq_split_kernel, dim3((unsigned)splits, (unsigned)num_heads, (unsigned)qgroups), dim3(256), 0, st, q_dev, q_stride, q_scale, kt_dev,
-                           vt_dev, kv_stride, mask_dev, mask_dev ? mask_heads : 0, head_dim, src_seqlen, dst_seqlen, v_vec_ok, (float*)workspace_dev);
+                           vt_dev, kv_stride, mask_dev, mask_dev ? mask_heads : 0, head_dim, src_seqlen, dst_seqlen, v_vec_ok, (float*)workspace_dev, append_k, append_v,
+                           append_stride, past);
         hipLaunchKernelGGL(attention_fewq_merge_kernel, dim3((unsigned)num_heads, (unsigned)qgroups), dim3(256), 0, st, (const float*)workspace_dev, splits, head_dim,
                            num_heads * head_dim, src_seqlen, out_dev);
         return launch_status("attention_fewq_split_kernel");
+    }
+    if (append_k)
+    {
+        // the other kernels read a finished cache: the new columns are written by a launch of their own
+        const int rc = ncnnhip_transpose_pair_f32(append_k, append_v, append_stride, dst_seqlen - past, num_heads * head_dim, kt_dev + past, vt_dev + past, kv_stride, stream);
+        if (rc != NCNNHIP_OK) return rc;
     }
     if (head_dim % 32 == 0 && head_dim <= 128)
     {
@@ -744,5 +797,3 @@ int ncnnhip_attention_f32_strided(const float* q_dev, size_t q_stride, float q_s
                        num_heads * head_dim, src_seqlen, dst_seqlen, kv_stride, out_dev, q_stride, q_scale);
     return launch_status("attention_f32_kernel");
 }
-
-} // extern "C"

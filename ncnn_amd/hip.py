@@ -57,6 +57,8 @@ _SIGNATURES = {
                               C.c_void_p],
     "ncnnhip_attention_f32_strided": [C.c_void_p, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                       C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_attention_f32_append": [C.c_void_p, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                     C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_stream_begin_capture": [C.c_void_p],
     "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
     "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
@@ -442,6 +444,23 @@ class Runtime:
             check(lib().ncnnhip_attention_f32_strided(dq.ptr, q_stride, float(q_scale), dk.ptr, dv.ptr, dst, _ptr(dm), mask_heads, num_heads, embed // num_heads,
                                                       src, dst, out.ptr, _ptr(ws), wsb.value if use_workspace else 0, self.stream))
         return out.to_numpy(self.stream)
+
+    def attention_append(self, qkv, kt, vt, num_heads, past, q_scale, mask=None):
+        """qkv [src][>= 3*embed]; kt / vt [embed][past + src] with the cache in their first `past` columns.  Returns (out, kt, vt) after the call."""
+        qkv, kt, vt = [np.ascontiguousarray(a, np.float32) for a in (qkv, kt, vt)]
+        src, stride = qkv.shape
+        embed, dst = kt.shape
+        assert dst == past + src
+        dq, dk, dv = self.up(qkv), self.up(kt), self.up(vt)
+        dm = None if mask is None else self.up(np.ascontiguousarray(mask, np.float32))
+        mask_heads = 0 if mask is None else (1 if mask.ndim == 2 else mask.shape[0])
+        out = DeviceBuffer.empty((src, embed), np.float32)
+        wsb = C.c_size_t()
+        check(lib().ncnnhip_attention_workspace_bytes(num_heads, embed // num_heads, src, dst, C.byref(wsb)))
+        ws = DeviceBuffer.empty((max(wsb.value, 4),), np.uint8)
+        check(lib().ncnnhip_attention_f32_append(dq.ptr, stride, float(q_scale), dk.ptr, dv.ptr, dst, past, _ptr(dm), mask_heads, num_heads, embed // num_heads, src,
+                                                 out.ptr, ws.ptr, wsb.value, self.stream))
+        return out.to_numpy(self.stream), dk.to_numpy(self.stream), dv.to_numpy(self.stream)
 
     def softmax(self, x):
         x = np.ascontiguousarray(x, np.float32)

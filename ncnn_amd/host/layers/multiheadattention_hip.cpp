@@ -310,11 +310,6 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
         float* d_kv_in = 0;
-        if (fused_qkv)
-        {
-            rc = ncnnhip_transpose_pair_f32(d_qa + E, d_qa + 2 * E, q_stride, cur, embed_dim, outT[0] + past, outT[1] + past, (size_t)dst, st);
-            if (rc != 0) return to_ncnn_status(rc, "k/v columns");
-        }
         for (int t = 0; t < 2 && !fused_qkv; t++)
         {
             const float* d_in = d_q;
@@ -356,8 +351,10 @@ int MultiHeadAttention_hip::forward(const std::vector<Mat>& bottom_blobs, std::v
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
     void* att_ws = att_ws_bytes ? leases.get(att_ws_bytes) : 0;
     if (att_ws_bytes && !att_ws) return -100;
-    rc = ncnnhip_attention_f32_strided(d_qa, q_stride, fused_qkv ? scale : 1.f, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws,
-                                       att_ws_bytes, st);
+    if (fused_qkv) // the new key and value columns are written behind the cache by the same call
+        rc = ncnnhip_attention_f32_append(d_qa, q_stride, scale, d_kt, d_vt, (size_t)dst, past, d_mask, mask_heads, num_heads, head_dim, src, d_ctx, att_ws, att_ws_bytes, st);
+    else
+        rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
     rc = blockquant_gemm_with_scratch(leases, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, d_out, (size_t)qdim, st);
@@ -505,11 +502,6 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
         const HipMat* in[2] = {&k_blob, &v_blob};
         float* outT[2] = {d_kt, d_vt};
         const int in_dim[2] = {kdim, vdim};
-        if (fused_qkv)
-        {
-            rc = ncnnhip_transpose_pair_f32(d_qa + E, d_qa + 2 * E, q_stride, cur, embed_dim, outT[0] + past, outT[1] + past, (size_t)dst, st);
-            if (rc != 0) return to_ncnn_status(rc, "k/v columns");
-        }
         for (int t = 0; t < 2 && !fused_qkv; t++)
         {
             float* d_aff = (float*)scratch.get((size_t)cur * E * 4);
@@ -525,8 +517,10 @@ int MultiHeadAttention_hip::forward_hip(const std::vector<HipMat>& bottom_blobs,
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_workspace_bytes");
     void* att_ws = att_ws_bytes ? scratch.get(att_ws_bytes) : 0;
     if (att_ws_bytes && !att_ws) return -100;
-    rc = ncnnhip_attention_f32_strided(d_qa, q_stride, fused_qkv ? scale : 1.f, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws,
-                                       att_ws_bytes, st);
+    if (fused_qkv) // the new key and value columns are written behind the cache by the same call
+        rc = ncnnhip_attention_f32_append(d_qa, q_stride, scale, d_kt, d_vt, (size_t)dst, past, d_mask, mask_heads, num_heads, head_dim, src, d_ctx, att_ws, att_ws_bytes, st);
+    else
+        rc = ncnnhip_attention_f32(d_qa, d_kt, d_vt, (size_t)dst, d_mask, mask_heads, num_heads, head_dim, src, dst, d_ctx, att_ws, att_ws_bytes, st);
     if (rc != 0) return to_ncnn_status(rc, "ncnnhip_attention_f32");
     rc = blockquant_gemm_with_scratch(scratch, d_ctx, E, src, qdim, embed_dim, dev[3][0], bits, block, dev[3][1], dev[3][2], dev[3][4], dev[3][5],
                                     (const float*)dev[3][3], 4, 1.f, 1.f, (float*)top.data, (size_t)qdim, st);

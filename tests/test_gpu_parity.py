@@ -748,3 +748,25 @@ def test_transpose_pair_appends_key_and_value_columns(rt, rows, cols, past):
     want_k[:, past:] = wide[:, cols:2 * cols].T
     want_v[:, past:] = wide[:, 2 * cols:].T
     assert np.array_equal(got_k, want_k) and np.array_equal(got_v, want_v)
+
+
+@pytest.mark.parametrize("heads,hd,src,past,mask", [(4, 64, 1, 299, None), (2, 40, 3, 318, "2d"), (3, 32, 4, 255, None), (2, 64, 2, 62, "3d"), (2, 64, 40, 100, None), (3, 24, 1, 7, None)])
+def test_attention_appends_the_new_keys_and_values_itself(rt, heads, hd, src, past, mask):
+    """q, k and v side by side in one row per token: the call writes the new key / value columns behind the cache and attends over
+    all of them - bit for bit what the separate append and the strided call give, and the cache columns stay as they were."""
+    rng = np.random.default_rng(heads * 1000 + past)
+    e, dst = heads * hd, past + src
+    qkv = rng.normal(0, 1, (src, 3 * e + 5)).astype(F)
+    kt = rng.normal(0, 1, (e, dst)).astype(F)
+    vt = rng.normal(0, 1, (e, dst)).astype(F)
+    m = None
+    if mask:
+        m = rng.normal(0, 1, (src, dst) if mask == "2d" else (heads, src, dst)).astype(F)
+    scale = F(1.0 / np.sqrt(hd))
+    want_kt, want_vt = kt.copy(), vt.copy()
+    want_kt[:, past:] = qkv[:, e:2 * e].T
+    want_vt[:, past:] = qkv[:, 2 * e:3 * e].T
+    want = rt.attention(qkv, want_kt, want_vt, heads, m, q_scale=scale)
+    got, got_kt, got_vt = rt.attention_append(qkv, kt, vt, heads, past, scale, m)
+    assert np.array_equal(got_kt, want_kt) and np.array_equal(got_vt, want_vt)
+    assert np.array_equal(got, want)
