@@ -583,7 +583,7 @@ __global__ __launch_bounds__(256) void attention_fewq_split_kernel(const float* 
 // sums of all splits are fetched side by side into LDS (wavefront t = query t) and turned into one factor per split;
 // then four groups of 64 threads each add every fourth split's outputs, eight loads in flight, and the groups' parts
 // are added through LDS - a thread that walks the splits one load after the other takes 14 us for 24 of them.
-static constexpr int FEWQ_MAX_SPLITS = 512;
+static constexpr int FEWQ_MAX_SPLITS = 512; // 8 per lane of a wavefront in the merge
 
 __global__ __launch_bounds__(256) void attention_fewq_merge_kernel(const float* __restrict__ partial, int splits, int head_dim, int embed_dim, int src,
                                                                    float* __restrict__ out)
@@ -596,22 +596,35 @@ __global__ __launch_bounds__(256) void attention_fewq_merge_kernel(const float* 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t rec_size = (size_t)(2 * ATT_TQ + ATT_TQ * head_dim);
     const float* rec0 = partial + ((size_t)blockIdx.y * gridDim.x + h) * splits * rec_size;
+    // Everything the first 64 outputs need is requested before the first wait (one trip to memory instead of three): this
+    // lane's maxima and sums of chunks lane, lane + 64, ... and, for output `lane`, the parts of this group's first 8 chunks.
+    float ofirst[8], mz[8], lz[8];
+    {
+        const float* op = rec0 + 2 * ATT_TQ + lane;
+#pragma unroll
+        for (int k = 0; k < 8; k++) ofirst[k] = lane < rows * head_dim && wave + 4 * k < splits ? op[(size_t)(wave + 4 * k) * rec_size] : 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+        {
+            const int z = lane + 64 * k; // FEWQ_MAX_SPLITS = 8 * 64
+            mz[k] = z < splits ? rec0[z * rec_size + wave] : -FLT_MAX;
+            lz[k] = z < splits ? rec0[z * rec_size + ATT_TQ + wave] : 0.f;
+        }
+    }
     {
         const int t = wave;
         float ma = -FLT_MAX;
-        for (int z = lane; z < splits; z += 64)
-        {
-            const float mz = rec0[z * rec_size + t];
-            fac[t][z] = mz;
-            ma = fmaxf(ma, mz);
-        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) ma = fmaxf(ma, mz[k]);
         ma = wave_max(ma);
         float lt = 0.f;
-        for (int z = lane; z < splits; z += 64) // each lane reads back what it wrote
+#pragma unroll
+        for (int k = 0; k < 8; k++)
         {
-            const float f = exp_of_nonpositive(fac[t][z] - ma);
-            fac[t][z] = f;
-            lt += rec0[z * rec_size + ATT_TQ + t] * f;
+            const int z = lane + 64 * k;
+            const float f = exp_of_nonpositive(mz[k] - ma);
+            if (z < splits) fac[t][z] = f;
+            lt += lz[k] * f;
         }
         lt = wave_sum(lt);
         if (lane == 0) l_all[t] = lt;
@@ -625,8 +638,16 @@ __global__ __launch_bounds__(256) void attention_fewq_merge_kernel(const float* 
         {
             const int t = idx / head_dim;
             const float* op = rec0 + 2 * ATT_TQ + idx;
+            int z = wave;
+            if (base == 0)
+            {
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    if (wave + 4 * k < splits) ot += ofirst[k] * fac[t][wave + 4 * k];
+                z = wave + 32;
+            }
 #pragma unroll 8
-            for (int z = wave; z < splits; z += 4) ot += op[z * rec_size] * fac[t][z];
+            for (; z < splits; z += 4) ot += op[z * rec_size] * fac[t][z];
         }
         part[wave][lane] = ot;
         __syncthreads();
