@@ -227,26 +227,6 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
                              const float* scale_in_dev, const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act,
                              void* out_nhwc_dev, void* stream);
 
-/* A depthwise convolution and the 1x1, stride-1, unpadded convolution that consumes it, in one launch
- * (ConvolutionDepthWise::forward_int8, src/layer/convolutiondepthwise.cpp:505-559, with its requantising epilogue, then
- * Convolution::forward_int8, src/layer/convolution.cpp:383-508): the int8 blob between the two layers stays in LDS, byte for
- * byte what the depthwise layer would have written.  dw_desc describes the depthwise layer (group == c == num_output, any
- * kernel, stride, dilation and padding); dw_packed_weight_dev is ncnnhip_dwconv_pack_weights' output; dw_scale_out_dev is
- * required (the intermediate is int8).  num_output, pointwise_rows_dev (ncnnhip_dwconv_pointwise_pack_weights: one row of the
- * 1x1 weights per output channel, rows of the input's padded channels rounded up to 64 bytes, zero-filled), scale_in / bias /
- * scale_out / act and the optional fused tail describe the 1x1 convolution as in ncnnhip_conv_int8_nhwc[_fused]:
- * channels-last int8 output when scale_out_dev is given, else channels-last fp32 (+ tail).  One workgroup computes 16 pixels
- * x 64 output channels and recomputes the depthwise tile per channel group: meant for small feature maps, where a pass is
- * bound by its launches. */
-int ncnnhip_dwconv_pointwise_supported(const ncnnhip_conv_desc* dw_desc, int num_output);
-int ncnnhip_dwconv_pointwise_packed_bytes(int channels, int num_output, size_t* bytes);
-int ncnnhip_dwconv_pointwise_pack_weights(int channels, int num_output, const int8_t* weight_host, int8_t* packed_host);
-int ncnnhip_dwconv_pointwise_int8(const ncnnhip_conv_desc* dw_desc, const int8_t* nhwc_dev, const int8_t* dw_packed_weight_dev,
-                                  const float* dw_scale_in_dev, const float* dw_bias_dev, const float* dw_scale_out_dev,
-                                  ncnnhip_activation dw_act, int num_output, const int8_t* pointwise_rows_dev, const float* scale_in_dev,
-                                  const float* bias_dev, const float* scale_out_dev, ncnnhip_activation act, void* out_nhwc_dev,
-                                  const ncnnhip_conv_fusion* fusion, void* stream);
-
 /* ------------------------------------------------------------------ fp32 layers between the int8 layers
  * ReLU::forward_inplace (src/layer/relu.cpp): x < 0 ? x*slope : x; int8 blobs clamp at zero.  Flat over `count` elements. */
 int ncnnhip_relu(const void* src_dev, void* dst_dev, int elemsize, size_t count, float slope, void* stream);

@@ -101,11 +101,6 @@ _SIGNATURES = {
     "ncnnhip_int8_to_f32": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_dwconv_packed_bytes": [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)],
     "ncnnhip_dwconv_pack_weights": [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p],
-    "ncnnhip_dwconv_pointwise_supported": [C.POINTER(ConvDesc), C.c_int],
-    "ncnnhip_dwconv_pointwise_packed_bytes": [C.c_int, C.c_int, C.POINTER(C.c_size_t)],
-    "ncnnhip_dwconv_pointwise_pack_weights": [C.c_int, C.c_int, C.c_void_p, C.c_void_p],
-    "ncnnhip_dwconv_pointwise_int8": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_int, C.c_void_p, C.c_void_p,
-                                      C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.POINTER(ConvFusion), C.c_void_p],
     "ncnnhip_dwconv_int8_nhwc": [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p, C.c_void_p],
     "ncnnhip_relu": [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p],
     "ncnnhip_scale": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_void_p],
@@ -594,54 +589,6 @@ class Runtime:
         raw = dout.to_numpy(self.stream)
         assert not raw[:, :, num_output:].any(), "pad channels of a channels-last blob must be zero"
         return self.from_channels_last(dout, n, num_output, oh, ow)
-
-    def dwconv_pointwise(self, xq, dw_weight, dw_bias, dw_w_scales, dw_in_scale, mid_scale, kernel, stride, pads, dw_act, dw_act_params,
-                         pw_weight, pw_bias, pw_w_scales, pw_top_scales, pw_act=0, pw_act_params=(0.0, 0.0), dilation=(1, 1), pad_value=0.0,
-                         residual=None, relu_after=False, quantise_scale=None):
-        """Depthwise convolution (int8 in, requantised with mid_scale) and the 1x1 convolution on its output in one launch.
-        xq int8 [n][c][h][w]; pw_top_scales None: fp32 output (returns (out, int8 copy or None) when a tail is asked for)."""
-        xq = np.ascontiguousarray(xq, np.int8)
-        n, c, h, w = xq.shape
-        cout = pw_weight.shape[0]
-        d = ConvDesc(w, h, c, n, c, kernel[0], kernel[1], dilation[0], dilation[1], stride[0], stride[1], pads[0], pads[1], pads[2], pads[3], float(pad_value), c)
-        if not lib().ncnnhip_dwconv_pointwise_supported(C.byref(d), cout):
-            raise ValueError("shape not supported by the fused depthwise + pointwise kernel")
-        ow, oh = C.c_int(), C.c_int()
-        check(lib().ncnnhip_conv_out_shape(C.byref(d), C.byref(ow), C.byref(oh)))
-        ow, oh = ow.value, oh.value
-        src = self.to_channels_last(xq)
-        nbytes = C.c_size_t()
-        check(lib().ncnnhip_dwconv_packed_bytes(c, kernel[0], kernel[1], C.byref(nbytes)))
-        dwpk = np.empty(nbytes.value, np.int8)
-        check(lib().ncnnhip_dwconv_pack_weights(c, kernel[0], kernel[1], np.ascontiguousarray(dw_weight, np.int8).ctypes.data, dwpk.ctypes.data))
-        check(lib().ncnnhip_dwconv_pointwise_packed_bytes(c, cout, C.byref(nbytes)))
-        rows = np.empty(nbytes.value, np.int8)
-        check(lib().ncnnhip_dwconv_pointwise_pack_weights(c, cout, np.ascontiguousarray(pw_weight, np.int8).ctypes.data, rows.ctypes.data))
-        dsi = self.up(self.fold_input_scales(dw_w_scales, [dw_in_scale], c))
-        ddb = self.up(None if dw_bias is None else np.asarray(dw_bias, np.float32))
-        dso = self.up(np.full(c, mid_scale, np.float32))
-        psi = self.up(self.fold_input_scales(pw_w_scales, [mid_scale], cout))
-        pdb = self.up(None if pw_bias is None else np.asarray(pw_bias, np.float32))
-        pso = None
-        if pw_top_scales is not None:
-            ts = np.atleast_1d(np.asarray(pw_top_scales, np.float32))
-            pso = self.up(np.repeat(ts, cout // ts.size).astype(np.float32))
-        ocp = lib().ncnnhip_padded_channels(cout)
-        dout = DeviceBuffer.empty((n, oh * ow, ocp), np.int8 if pso is not None else np.float32)
-        fused = residual is not None or relu_after or quantise_scale is not None
-        dres = None if residual is None else self.to_channels_last(np.asarray(residual, np.float32))
-        dq8 = None if quantise_scale is None else DeviceBuffer.empty((n, oh * ow, ocp), np.int8)
-        fu = ConvFusion(_ptr(dres), int(relu_after), _ptr(dq8), float(quantise_scale or 0.0))
-        ddw, drows = self.up(dwpk), self.up(rows)
-        check(lib().ncnnhip_dwconv_pointwise_int8(C.byref(d), src.ptr, ddw.ptr, dsi.ptr, _ptr(ddb), dso.ptr, Activation.make(dw_act, dw_act_params), cout, drows.ptr,
-                                                  psi.ptr, _ptr(pdb), _ptr(pso), Activation.make(pw_act, pw_act_params), dout.ptr, C.byref(fu) if fused else None,
-                                                  self.stream))
-        raw = dout.to_numpy(self.stream)
-        assert not raw[:, :, cout:].any(), "pad channels of a channels-last blob must be zero"
-        out = self.from_channels_last(dout, n, cout, oh, ow)
-        if fused:
-            return out, (None if dq8 is None else self.from_channels_last(dq8, n, cout, oh, ow))
-        return out
 
     # -- InnerProduct -------------------------------------------------------------------------
     def innerproduct_layer(self, x, weight, bias, w_scales, in_scale, act=0, act_params=(0.0, 0.0), want_acc=False):

@@ -770,48 +770,3 @@ def test_attention_appends_the_new_keys_and_values_itself(rt, heads, hd, src, pa
     got, got_kt, got_vt = rt.attention_append(qkv, kt, vt, heads, past, scale, m)
     assert np.array_equal(got_kt, want_kt) and np.array_equal(got_vt, want_vt)
     assert np.array_equal(got, want)
-
-
-# ---- depthwise + the 1x1 convolution behind it in one launch ------------------------------------------------------------------
-
-@pytest.mark.parametrize("n,c,h,w,stride,cout,dw_act,tail", [
-    (1, 96, 14, 14, 1, 24, 3, "int8"), (1, 576, 14, 14, 1, 96, 3, "residual"), (1, 144, 28, 28, 2, 32, 3, "int8"), (2, 40, 9, 7, 2, 20, 1, "fp32"),
-    (1, 960, 7, 7, 1, 320, 3, "q8"), (3, 16, 5, 5, 1, 70, 0, "relu")])
-def test_depthwise_and_pointwise_in_one_launch_equal_the_two_layers(rt, n, c, h, w, stride, cout, dw_act, tail):
-    """The fused kernel against the depthwise layer followed by the 1x1 convolution, each through its own entry: every byte of
-    the int8 output, every bit of the fp32 output and of its int8 copy (the layers themselves are pinned on the oracle)."""
-    rng = np.random.default_rng(c * 7 + cout)
-    xq = rng.integers(-127, 128, (n, c, h, w)).astype(np.int8)
-    dw_w = rng.integers(-127, 128, (c, 9)).astype(np.int8)
-    dw_b = rng.uniform(-1, 1, c).astype(F)
-    dw_ws = rng.uniform(20, 60, c).astype(F)
-    in_scale, mid_scale = F(31.5), F(17.25)
-    pw_w = rng.integers(-127, 128, (cout, c)).astype(np.int8)
-    pw_b = rng.uniform(-1, 1, cout).astype(F)
-    pw_ws = rng.uniform(50, 100, cout).astype(F)
-    act_params = (0.0, 6.0) if dw_act == 3 else (0.0, 0.0)
-    pads = (1, 1, 1, 1)
-    mid = rt.conv_channels_last(xq, dw_w, dw_b, dw_ws, [in_scale], [mid_scale], c, (3, 3), stride=(stride, stride), pads=pads, group=c, term=101, act=dw_act,
-                                act_params=act_params)
-    assert mid.dtype == np.int8
-    kw = dict(residual=None, relu_after=False, quantise_scale=None)
-    top = None
-    if tail == "int8":
-        top = [F(9.5)]
-    elif tail == "residual":
-        oh, ow = mid.shape[2], mid.shape[3]
-        kw = dict(residual=rng.normal(0, 1, (n, cout, oh, ow)).astype(F), relu_after=False, quantise_scale=F(12.5))
-    elif tail == "q8":
-        kw = dict(residual=None, relu_after=False, quantise_scale=F(7.75))
-    elif tail == "relu":
-        kw = dict(residual=None, relu_after=True, quantise_scale=None)
-    want = rt.conv_channels_last(mid, pw_w.reshape(cout, c, 1, 1), pw_b, pw_ws, [mid_scale], top, cout, (1, 1), term=101 if top else 1, **kw)
-    got = rt.dwconv_pointwise(xq, dw_w, dw_b, dw_ws, in_scale, mid_scale, (3, 3), (stride, stride), pads, dw_act, act_params, pw_w, pw_b, pw_ws, top, **kw)
-    if isinstance(want, tuple):
-        assert np.array_equal(got[0].view(np.uint32), want[0].view(np.uint32))
-        assert (got[1] is None) == (want[1] is None)
-        if want[1] is not None:
-            assert np.array_equal(got[1], want[1])
-    else:
-        assert got.dtype == want.dtype
-        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
