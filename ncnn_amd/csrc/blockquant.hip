@@ -1370,36 +1370,58 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_rows16_pair_kernel(cons
 // 64-wide K step in LDS (two buffers, 144-byte row pitch: 16 rows fall on 16 different bank groups).  Per step and
 // (tile, 16-row group) the six instructions (3 planes x 2 halves of the step) add into a fresh accumulator that is then
 // scaled by the step's 1/scale, like the few-row kernels do.
+// SPLIT_VECS vectors of 8 activations per thread, all of them requested before the first is split: with one vector per thread
+// the pass ran at 2 TB/s (20 us for 1024 x 4096), short of bytes in flight; with four 11 us; eight measured slower again.
+static constexpr int SPLIT_VECS = 4;
 __global__ __launch_bounds__(256) void blockquant_split_activations_kernel(const float* __restrict__ a, size_t a_stride, int M, int K,
                                                                             const float* __restrict__ in_scales, unsigned short* __restrict__ planes, int Mp,
                                                                             int Kp)
 {
     const int vec_per_row = Kp >> 3;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (size_t)Mp * vec_per_row) return;
-    const int row = (int)(idx / vec_per_row), k = (int)(idx - (size_t)row * vec_per_row) << 3;
-    unsigned pl[3][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
-    if (row < M && k < K) // K % 16 == 0: a vector of 8 is all in or all out
+    const size_t total = (size_t)Mp * vec_per_row;
+    const size_t first = (size_t)blockIdx.x * (256 * SPLIT_VECS) + threadIdx.x;
+    float x[SPLIT_VECS][8];
+    int row[SPLIT_VECS], k[SPLIT_VECS];
+#pragma unroll
+    for (int u = 0; u < SPLIT_VECS; u++)
     {
-        const float* p = a + (size_t)row * a_stride + k;
+        const size_t idx = first + (size_t)u * 256;
+        const size_t ii = idx < total ? idx : 0;
+        row[u] = (int)(ii / vec_per_row);
+        k[u] = (int)(ii - (size_t)row[u] * vec_per_row) << 3;
+        const bool inside = idx < total && row[u] < M && k[u] < K; // K % 16 == 0: a vector of 8 is all in or all out
+        const float* p = a + (inside ? (size_t)row[u] * a_stride + k[u] : (size_t)0);
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[u][j] = p[j]; // a valid address either way (K >= 16)
+        if (!inside)
+        {
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[u][j] = 0.f;
+        }
+        else if (in_scales)
+        {
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[u][j] = mul_rn(x[u][j], in_scales[k[u] + j]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < SPLIT_VECS; u++)
+    {
+        if (first + (size_t)u * 256 >= total) break;
+        unsigned pl[3][4];
 #pragma unroll
         for (int e = 0; e < 4; e++)
         {
             unsigned h[2][3];
 #pragma unroll
-            for (int o = 0; o < 2; o++)
-            {
-                float x = p[2 * e + o];
-                if (in_scales) x = mul_rn(x, in_scales[k + 2 * e + o]);
-                split_bf16x3(x, h[o][0], h[o][1], h[o][2]);
-            }
+            for (int o = 0; o < 2; o++) split_bf16x3(x[u][2 * e + o], h[o][0], h[o][1], h[o][2]);
 #pragma unroll
             for (int pn = 0; pn < 3; pn++) pl[pn][e] = (h[0][pn] >> 16) | h[1][pn];
         }
-    }
 #pragma unroll
-    for (int pn = 0; pn < 3; pn++)
-        *reinterpret_cast<uint4*>(planes + ((size_t)pn * Mp + row) * Kp + k) = make_uint4(pl[pn][0], pl[pn][1], pl[pn][2], pl[pn][3]);
+        for (int pn = 0; pn < 3; pn++)
+            *reinterpret_cast<uint4*>(planes + ((size_t)pn * Mp + row[u]) * Kp + k[u]) = make_uint4(pl[pn][0], pl[pn][1], pl[pn][2], pl[pn][3]);
+    }
 }
 
 #ifndef BQ_ROWS_RW1_BELOW
@@ -2299,7 +2321,7 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     }
     unsigned short* planes = static_cast<unsigned short*>(workspace_dev);
     const size_t vectors = (size_t)Mp * (Kp / 8);
-    hipLaunchKernelGGL(blockquant_split_activations_kernel, dim3((unsigned)((vectors + 255) / 256)), dim3(256), 0, st, a_dev, a_stride, M, K, in_scales_dev, planes, Mp,
+    hipLaunchKernelGGL(blockquant_split_activations_kernel, dim3((unsigned)((vectors + 256 * SPLIT_VECS - 1) / (256 * SPLIT_VECS))), dim3(256), 0, st, a_dev, a_stride, M, K, in_scales_dev, planes, Mp,
                        Kp);
     // Two tiles per wavefront and two stages: 66 KB of LDS, so two workgroups share a compute unit and one's loads, waits and
     // vector work overlap the other's matrix-core instructions.  Measured at 1024 x 4096 x 4096 / 2048 x 11008 x 4096: 135 / 616 us;
