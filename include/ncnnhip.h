@@ -389,9 +389,10 @@ int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, i
 
 /* The same contract from five activation rows up, with a workspace: the three-way split is made once, by a pass of its own,
  * into the workspace (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: 6 bytes per activation, rows and K rounded up to 64).
- * Up to 48 rows (96 over 2048 weight rows and more) the weights are then streamed once per 16 rows in the few-row kernel's
- * shape, the activations pre-arranged as the lanes load them; beyond, a tiled Gemm runs on the bf16 matrix cores, 128 weight
- * rows x 64 activation rows per workgroup (prefill, attention projections).  K % 16 == 0; the workspace is scratch
+ * Up to 128 rows, while streaming the weights once per 16 rows is cheaper than a tiled pass (small weight matrices, or few
+ * rows), the weights are streamed once per 16 rows in the few-row kernel's shape, all passes in one launch, the activations
+ * pre-arranged as the lanes load them; otherwise a tiled Gemm runs on the bf16 matrix cores, 128 weight rows x 64 activation
+ * rows per workgroup (prefill, attention projections).  K % 16 == 0; the workspace is scratch
  * (overwritten by every call). */
 int ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(int M, int K, size_t* bytes);
 int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* packed_w_dev,

@@ -1683,9 +1683,13 @@ __global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsig
 // operand fragments (plane p, half h of the step) are 64 x 16 bytes each, lane l = activation row l % 16, K group l / 16.
 // They come from L2 in a window of three steps kept three ahead of the arithmetic (24 VGPRs per step).
 template<bool HALVES>
-__global__ __launch_bounds__(256) void blockquant_split_operands_kernel(const float* __restrict__ a, size_t a_stride, int M, int K, int kblocks,
+__global__ __launch_bounds__(256) void blockquant_split_operands_kernel(const float* __restrict__ a, size_t a_stride, int M_total, int K, int kblocks,
                                                                          const float* __restrict__ in_scales, uint4* __restrict__ frags)
 {
+    // blockIdx.y = pass: rows 16 * pass .. + 15, fragments of their own (kblocks * 384 vectors per pass)
+    a += (size_t)blockIdx.y * 16 * a_stride;
+    frags += (size_t)blockIdx.y * kblocks * 384;
+    const int M = M_total - 16 * (int)blockIdx.y < 16 ? M_total - 16 * (int)blockIdx.y : 16;
     // one thread = one lane's 8 activations of one (step, half): fragments [step][plane * 2 + half][lane]
     const int idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= kblocks * 128) return;
@@ -1716,12 +1720,19 @@ __global__ __launch_bounds__(256) void blockquant_split_operands_kernel(const fl
 }
 
 template<int BITS, bool HALVES>
-__global__ __launch_bounds__(512) void blockquant_rows16_bf16x3_kernel(const uint4* __restrict__ frags, int M, int N, int kblocks,
+__global__ __launch_bounds__(512) void blockquant_rows16_bf16x3_kernel(const uint4* __restrict__ frags, int M_total, int N, int kblocks,
                                                                         const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
                                                                         const float* __restrict__ c, int bt, float alpha, float beta, float* __restrict__ out,
                                                                         size_t out_stride)
 {
     static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
+    // blockIdx.y = pass: activation rows 16 * pass .. + 15 (all passes in one launch: the weights of a tile are streamed once per
+    // pass, from L2 after the first)
+    const int M = M_total - 16 * (int)blockIdx.y < 16 ? M_total - 16 * (int)blockIdx.y : 16;
+    frags += (size_t)blockIdx.y * kblocks * 384;
+    if (c && (bt == 1 || bt == 2)) c += 16 * blockIdx.y;
+    if (c && bt == 3) c += (size_t)16 * blockIdx.y * N;
+    out += (size_t)16 * blockIdx.y * out_stride;
     constexpr int NB = 8, WIN = 3;
     constexpr int STEP_BYTES = 128 * BITS;
     __shared__ float4 red[8 * 64];
@@ -2284,39 +2295,37 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     hipStream_t st = as_stream(stream);
     const float4* dpk = reinterpret_cast<const float4*>(packed_descale_dev);
     const int split = block == 32 ? 1 : 0;
-    if (M <= 48 || (M <= 96 && ntiles >= 128))
+    // Which form: the 16-row passes (all in one launch, spread over the chip; every pass streams the weights again, from L2
+    // after the first) cost about 5 us + passes x weight bytes at 2 TB/s; the tiled kernel's 64-row tiles about 6 us + K / 85
+    // whatever the row count up to 64 (18-20 us at K = 1024, 54-58 at K = 4096).  Measured on 16..96 rows: 3072 x 1024
+    // 6.9..12.5 us against 18..20 tiled, 4096 x 4096 11.7..52.7 against 55..58, 11008 x 4096 26.8 / 49 / 72 / 90 at
+    // 16 / 32 / 48 / 64 rows against 57..59.
+    const double weight_mb = (double)N * (double)K * bits / 8.0 / 1.0e6;
+    const int passes16 = (M + 15) / 16;
+    if (M <= 128 && 5.0 + passes16 * weight_mb / 2.0 <= 6.0 + K / 85.0)
     {
-        // fewer rows than the tiled kernel can spread over the chip (its 64-row tiles take 75 us at 4096 x 4096 whatever the row
-        // count, a pass here 11-12; at 1024 x 1024 the tiled kernel wins from 64 rows): 16 rows per pass in the weight-streaming shape
-        // (the fragments of a pass take kblocks * 6 KB of the workspace, less than the planes it was sized for)
+        // fewer rows than the tiled kernel can spread over the chip: 16 rows per pass in the weight-streaming shape
+        // (the fragments of a pass take kblocks * 6 KB of the workspace: all passes together no more than the planes it was sized for)
         uint4* frags = static_cast<uint4*>(workspace_dev);
         const int nwaves = kblocks >= 64 ? 8 : (kblocks + 7) / 8; // K beyond 4096: rounds of 8 x 8 steps
-        for (int m0 = 0; m0 < M; m0 += 16)
-        {
-            const int mc = M - m0 < 16 ? M - m0 : 16;
-            const float* cc = c_dev;
-            if (cc && (bt == 1 || bt == 2)) cc += m0;
-            if (cc && bt == 3) cc += (size_t)m0 * N;
-            const float* ap = a_dev + (size_t)m0 * a_stride;
-            float* op = out_dev + (size_t)m0 * out_stride;
-            const dim3 sgrid((kblocks * 128 + 255) / 256);
-            if (halves)
-                hipLaunchKernelGGL(blockquant_split_operands_kernel<true>, sgrid, dim3(256), 0, st, ap, a_stride, mc, K, kblocks, in_scales_dev, frags);
-            else
-                hipLaunchKernelGGL(blockquant_split_operands_kernel<false>, sgrid, dim3(256), 0, st, ap, a_stride, mc, K, kblocks, in_scales_dev, frags);
-#define ROWS16(BITS_, HALVES_)                                                                                                                       \
-    hipLaunchKernelGGL((blockquant_rows16_bf16x3_kernel<BITS_, HALVES_>), dim3(ntiles), dim3(nwaves * 64), 0, st, frags, mc, N, kblocks, packed_w_dev, dpk, split, cc, \
-                       bt, alpha, beta, op, out_stride)
-            if (!halves)
-                ROWS16(8, false);
-            else if (bits == 8)
-                ROWS16(8, true);
-            else if (bits == 6)
-                ROWS16(6, true);
-            else
-                ROWS16(4, true);
+        const unsigned passes = (unsigned)((M + 15) / 16);
+        const dim3 sgrid((kblocks * 128 + 255) / 256, passes);
+        if (halves)
+            hipLaunchKernelGGL(blockquant_split_operands_kernel<true>, sgrid, dim3(256), 0, st, a_dev, a_stride, M, K, kblocks, in_scales_dev, frags);
+        else
+            hipLaunchKernelGGL(blockquant_split_operands_kernel<false>, sgrid, dim3(256), 0, st, a_dev, a_stride, M, K, kblocks, in_scales_dev, frags);
+#define ROWS16(BITS_, HALVES_)                                                                                                                                 \
+    hipLaunchKernelGGL((blockquant_rows16_bf16x3_kernel<BITS_, HALVES_>), dim3(ntiles, passes), dim3(nwaves * 64), 0, st, frags, M, N, kblocks, packed_w_dev, dpk, split, \
+                       c_dev, bt, alpha, beta, out_dev, out_stride)
+        if (!halves)
+            ROWS16(8, false);
+        else if (bits == 8)
+            ROWS16(8, true);
+        else if (bits == 6)
+            ROWS16(6, true);
+        else
+            ROWS16(4, true);
 #undef ROWS16
-        }
         return launch_status("blockquant_rows16_bf16x3_kernel");
     }
     unsigned short* planes = static_cast<unsigned short*>(workspace_dev);
