@@ -319,7 +319,7 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic("blockquant:%dx%dx%d%s%s" % (n, k, m, "" if (bits, block) == (8, 64) else ":%d:%d" % (bits, block),
                                                                               "" if half else ":" + args.act)) if packed_form else None,
-                     "kernel": ("blockquant_rows16_bf16x3_kernel" if (m <= 48 or (m <= 96 and n >= 128 * 16 - 15)) else "blockquant_rows_bf16x3_kernel") if rows_entry else "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
+                     "kernel": ("blockquant_rows16_bf16x3_kernel" if (m <= 128 and 5.0 + ((m + 15) // 16) * (n * k * bits / 8.0 / 1.0e6) / 2.0 <= 6.0 + k / 85.0) else "blockquant_rows_bf16x3_kernel") if rows_entry else "blockquant8_upfront_kernel" if packed_form else ("blockquant8_f32_mfma_kernel" if m >= 32 else "blockquant8_stream_kernel"),
                      "bytes_per_launch": algo,
                      "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
                      "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"

@@ -75,8 +75,8 @@ int upload_blockquant_packed(const void* fields_host, const float* scales_host, 
 
 size_t blockquant_gemm_workspace_bytes(int M, int K, const void* d_packed)
 {
-    // 5 rows and more: the kernels that split the activations in a pass of their own (up to 48-96 rows the weight-streaming one on
-    // pre-split operands, 16 rows per pass; beyond, the tiled one)
+    // 5 rows and more: the kernels that split the activations in a pass of their own (the weight-streaming one on pre-split
+    // operands, 16 rows per pass, while that is cheaper than a tiled pass; else the tiled one: the entry point picks)
     if (!d_packed || K % 16 != 0 || M < 5) return 0;
     size_t bytes = 0;
     if (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(M, K, &bytes) != 0) return 0;
