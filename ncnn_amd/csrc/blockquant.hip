@@ -1424,9 +1424,6 @@ __global__ __launch_bounds__(256) void blockquant_split_activations_kernel(const
     }
 }
 
-#ifndef BQ_ROWS_RW1_BELOW
-#define BQ_ROWS_RW1_BELOW 256
-#endif
 #define BQ_AS1 __attribute__((address_space(1)))
 #define BQ_AS3 __attribute__((address_space(3)))
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
@@ -1449,7 +1446,7 @@ __global__ __launch_bounds__(256) void blockquant_rows_bf16x3_kernel(const unsig
     static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
     constexpr int LOADS = 6 + 2 * RW; // per wavefront and stage
     static_assert(STAGES >= 2 && (STAGES - 2) * LOADS < 64, "the vmcnt field counts to 63");
-    static_assert(RW == 1 || RW == 2 || RW == 4, "one, two or four tiles of 16 weight rows per wavefront");
+    static_assert(RW >= 1 && RW <= 4, "one to four tiles of 16 weight rows per wavefront");
     constexpr int PLANE = 64 * 128;
     constexpr int ACT_BYTES = 3 * PLANE;
     constexpr int W_OFF = ACT_BYTES, D_OFF = ACT_BYTES + 4 * RW * 1024;
@@ -2338,7 +2335,35 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     // tiles with four stages (one workgroup per unit) 172 / 795 us.  While that leaves fewer workgroups than the chip has compute
     // units, one tile per wavefront (64 weight rows per workgroup) doubles them: 128 x 4096 x 4096 77 -> 58 us, 256 rows 82 -> 63,
     // 512 x 1024 x 1024 28.6 -> 22.3.
-    const int rw_tiles = ((ntiles + 7) / 8) * (Mp / 64) < BQ_ROWS_RW1_BELOW ? 1 : 2;
+    // One, two or three tiles per wavefront (64, 128 or 192 weight rows per workgroup).  The chip holds 512 workgroups at once:
+    // where some choice fits in one round, the one with the most workgroups; else the fewest rounds weighted by a
+    // workgroup's cost (0.68 : 1 : 1.4, measured).  1500 x 3072 x 1024 is 576 workgroups with two tiles - a second round
+    // for 64 of them - and 384 with three: 63.6 -> 55.9 us; 1100 x 4096 x 4096 189 -> 173; 2048 x 11008 x 4096 672 -> 650.
+    int rw_tiles = 2;
+    {
+        const long long row_tiles = Mp / 64;
+        const double cost[4] = {0.0, 0.68, 1.0, 1.4};
+        int fits = 0;
+        double best = 0.0;
+        for (int rw = 1; rw <= 3; rw++)
+        {
+            const long long groups = (long long)((ntiles + 4 * rw - 1) / (4 * rw)) * row_tiles;
+            if (groups <= 512)
+            {
+                if (!fits) rw_tiles = rw; // the smallest such rw has the most workgroups
+                fits = 1;
+            }
+            else if (!fits)
+            {
+                const double t = (double)((groups + 511) / 512) * cost[rw];
+                if (best == 0.0 || t < best)
+                {
+                    best = t;
+                    rw_tiles = rw;
+                }
+            }
+        }
+    }
     // (a ring of four stages where a workgroup has its compute unit to itself measured the same as two: 57.6 against 57.8 us at 128 x 4096 x 4096)
     const dim3 grid((ntiles + 4 * rw_tiles - 1) / (4 * rw_tiles), Mp / 64);
 #define ROWS_RW(BITS_, HALVES_, RW_, STAGES_)                                                                                                                      \
@@ -2361,6 +2386,8 @@ int ncnnhip_gemm_blockquant_packed_rows(const float* a_dev, size_t a_stride, int
     {                                   \
         if (rw_tiles == 1)                 \
             ROWS_RW(BITS_, HALVES_, 1, 2); \
+        else if (rw_tiles == 3)            \
+            ROWS_RW(BITS_, HALVES_, 3, 2); \
         else                               \
             ROWS_RW(BITS_, HALVES_, 2, 2); \
     } while (0)
