@@ -14,13 +14,15 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(DenseOperand a, DenseOpe
 // skinny case (up to a few dozen activation rows): one wavefront per output channel streams the weight row with
 // 16-byte loads, multiplies it against up to 8 activation rows at a time held in registers (v_dot4_i32_i8) and
 // reduces with cross-lane adds; no matrix cores involved.  The layer is bound by reading the weights once.
+// ROW_FIRST: the epilogue takes (activation row, output column, acc), as Gemm's does; else (output channel, row, acc)
+template<typename Epilogue, bool ROW_FIRST>
 __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__ x, size_t xs, int rows, int K,
-                                                       const int8_t* __restrict__ wgt, int num_output, FcEpilogue epi, int vec)
+                                                       const int8_t* __restrict__ wgt, size_t ws, int num_output, Epilogue epi, int vec)
 {
     const int lane = threadIdx.x & 63;
     const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (p >= num_output) return;
-    const int8_t* wr = wgt + (size_t)p * K;
+    const int8_t* wr = wgt + (size_t)p * ws;
     for (int r0 = 0; r0 < rows; r0 += 8)
     {
         const int nr = rows - r0 < 8 ? rows - r0 : 8;
@@ -59,11 +61,20 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__
             int v = acc[r];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-            if (lane == 0 && r < nr) epi(p, r0 + r, v);
+            if (lane == 0 && r < nr)
+            {
+                if (ROW_FIRST)
+                    epi(r0 + r, p, v);
+                else
+                    epi(p, r0 + r, v);
+            }
         }
     }
 }
 
+#ifndef GEMM_GEMV_MAX_ROWS
+#define GEMM_GEMV_MAX_ROWS 4
+#endif
 static inline bool aligned16(const void* p)
 {
     return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
@@ -119,6 +130,18 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
     epi.N = N;
     epi.acc_out = acc_out_dev;
 
+    // up to four rows of A (a decoding step through a Gemm layer): the work is reading B once, which the skinny kernel does with
+    // one wavefront per row of B.  Quantise + Gemm, one / four rows: 4096 x 4096 19.6 / 20.3 -> 9.2 / 12.3 us, 11008 x 4096
+    // 21.9 / 22.0 -> 16.9 / 23.3, 1024 x 1024 9.5 / 9.5 -> 7.0 / 8.1; from 16 rows the tiled kernels are faster.  (Eight
+    // pieces of the weight row requested at once per lane instead of one were measured: no better at 4096 x 4096, worse on
+    // the other two.)
+    if (M <= GEMM_GEMV_MAX_ROWS && N >= 64)
+    {
+        const int vec = (aligned16(aq_dev) && aligned16(bq_dev) && aq_stride % 16 == 0 && bq_stride % 16 == 0) ? 1 : 0;
+        hipLaunchKernelGGL((fc_gemv_kernel<GemmEpilogue, true>), dim3(ceil_div(N, 4)), dim3(256), 0, as_stream(stream), aq_dev, aq_stride, M, K, bq_dev, bq_stride, N, epi,
+                           vec);
+        return launch_status("fc_gemv_kernel");
+    }
     // big aligned problems: the 256x256 kernel (it needs a few hundred tiles to fill the chip)
     bool handled = false;
     int ret = NCNNHIP_OK;
@@ -170,8 +193,8 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
     if (rows <= 64)
     {
         const int vec = aligned16(x_dev) && aligned16(weight_dev) && x_stride % 16 == 0 && num_input % 16 == 0;
-        hipLaunchKernelGGL(fc_gemv_kernel, dim3(ceil_div(num_output, 4)), dim3(256), 0, as_stream(stream), x_dev, x_stride, rows,
-                           num_input, weight_dev, num_output, epi, vec);
+        hipLaunchKernelGGL((fc_gemv_kernel<FcEpilogue, false>), dim3(ceil_div(num_output, 4)), dim3(256), 0, as_stream(stream), x_dev, x_stride, rows,
+                           num_input, weight_dev, (size_t)num_input, num_output, epi, vec);
         return launch_status("fc_gemv_kernel");
     }
 

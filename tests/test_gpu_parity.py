@@ -68,7 +68,9 @@ def test_transposes(rt):
     assert np.array_equal(rt.transpose(q), q.T)
 
 
-GEMM_SHAPES = [(13, 17, 96), (1, 1, 1), (128, 128, 64), (130, 257, 100), (64, 300, 77), (256, 512, 1024), (300, 200, 4100)]
+GEMM_SHAPES = [(13, 17, 96), (1, 1, 1), (128, 128, 64), (130, 257, 100), (64, 300, 77), (256, 512, 1024), (300, 200, 4100),
+               # one to four rows of A on 64 columns and more: one wavefront per row of B (aligned rows, ragged K, K below a vector)
+               (1, 4096, 4096), (4, 1000, 2048), (3, 64, 100), (2, 333, 8)]
 
 
 @pytest.mark.parametrize("shape", GEMM_SHAPES)
