@@ -72,8 +72,63 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__
     }
 }
 
+// Up to 16 rows of A on the matrix cores: a workgroup owns 16 rows of B, its four wavefronts every fourth 64-wide K step each
+// (v_mfma_i32_16x16x64_i8: the rows of B as one operand, the rows of A as the other, so a lane ends up with four consecutive
+// columns of one output row); eight steps of B and A are requested before the first product; the four partial tiles are
+// added through LDS.  B is read once; A (at most 16 x K bytes) comes from the cache.
+typedef int v4i_sk __attribute__((ext_vector_type(4)));
+template<typename Epilogue>
+__global__ __launch_bounds__(256) void gemm_skinny_int8_kernel(const int8_t* __restrict__ a, size_t as, int M_total, const int8_t* __restrict__ b, size_t bs, int N, int K,
+                                                                Epilogue epi)
+{
+    __shared__ int red[4][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, q = lane >> 4;
+    const int tile = blockIdx.x;
+    const int row0 = blockIdx.y * 16; // blockIdx.y: which 16 rows of A (every group of 16 reads B again, from the cache after the first)
+    const int M = M_total - row0 < 16 ? M_total - row0 : 16;
+    a += (size_t)row0 * as;
+    const int brow = tile * 16 + c16 < N ? tile * 16 + c16 : N - 1; // rows past the end repeat the last one; nothing of theirs is stored
+    const int arow = c16 < M ? c16 : M - 1;
+    const int8_t* bp = b + (size_t)brow * bs + q * 16;
+    const int8_t* ap = a + (size_t)arow * as + q * 16;
+    const int ksteps = K >> 6;
+    v4i_sk acc = {0, 0, 0, 0};
+    for (int k0 = wave; k0 < ksteps; k0 += 32) // this wavefront's steps k0, k0 + 4, ..., eight at a time
+    {
+        v4i_sk wv[8], xv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+        {
+            const int ks = k0 + 4 * u;
+            const int kk = ks < ksteps ? ks : k0; // past the end: a step that is there, its product dropped below
+            wv[u] = *reinterpret_cast<const v4i_sk*>(bp + (size_t)kk * 64);
+            xv[u] = *reinterpret_cast<const v4i_sk*>(ap + (size_t)kk * 64);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (k0 + 4 * u < ksteps) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u], xv[u], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) red[wave][lane][r] = acc[r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+    {
+        const int v = (red[0][lane][r] + red[1][lane][r]) + (red[2][lane][r] + red[3][lane][r]);
+        const int j = tile * 16 + 4 * q + r;
+        if (c16 < M && j < N) epi(row0 + c16, j, v);
+    }
+}
+
 #ifndef GEMM_GEMV_MAX_ROWS
 #define GEMM_GEMV_MAX_ROWS 4
+#endif
+#ifndef GEMM_SKINNY_MIN_ROWS
+#define GEMM_SKINNY_MIN_ROWS 0
+#endif
+#ifndef GEMM_SKINNY_MAX_ROWS
+#define GEMM_SKINNY_MAX_ROWS 48
 #endif
 static inline bool aligned16(const void* p)
 {
@@ -130,11 +185,22 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
     epi.N = N;
     epi.acc_out = acc_out_dev;
 
-    // up to four rows of A (a decoding step through a Gemm layer): the work is reading B once, which the skinny kernel does with
-    // one wavefront per row of B.  Quantise + Gemm, one / four rows: 4096 x 4096 19.6 / 20.3 -> 9.2 / 12.3 us, 11008 x 4096
-    // 21.9 / 22.0 -> 16.9 / 23.3, 1024 x 1024 9.5 / 9.5 -> 7.0 / 8.1; from 16 rows the tiled kernels are faster.  (Eight
-    // pieces of the weight row requested at once per lane instead of one were measured: no better at 4096 x 4096, worse on
-    // the other two.)
+    // up to four rows of A whose shape the matrix-core form above does not take (K % 64, unaligned rows): one wavefront per row
+    // of B with v_dot4.  Quantise + Gemm, one / four rows: 4096 x 4096 19.6 / 20.3 -> 9.2 / 12.3 us, 11008 x 4096
+    // 21.9 / 22.0 -> 16.9 / 23.3, 1024 x 1024 9.5 / 9.5 -> 7.0 / 8.1.  (Eight pieces of the weight row requested at once per
+    // lane instead of one were measured: no better at 4096 x 4096, worse on the other two.)
+    // up to 16 rows of A, or up to 48 while reading B once per 16 rows (about 3 us + groups x bytes of B at 4 TB/s, from the cache
+    // after the first) stays below what the tiled kernels take for so few rows (about 4 us + K / 300): quantise + Gemm for
+    // 16 / 32 / 48 rows 4096 x 4096 20.6 / 21.2 / 21.4 -> 10.1 / 13.6 / 17.3 us, 11008 x 4096 22.1 -> 17.6 at 16 rows (beyond:
+    // tiled), 1024 x 1024 9.9 / 10.2 / 10.3 -> 7.2 / 7.5 / 7.3; one row 19.6 -> 8.7 / 21.9 -> 13.7 / 9.5 -> 7.5
+    const int groups16 = (M + 15) / 16;
+    const bool skinny_pays = M <= 16 || 3.0 + groups16 * ((double)N * (double)K / 4.0e6) <= 4.0 + K / 300.0;
+    if (skinny_pays && M > GEMM_SKINNY_MIN_ROWS && M <= GEMM_SKINNY_MAX_ROWS && N >= 64 && K % 64 == 0 && aligned16(aq_dev) && aligned16(bq_dev) && aq_stride % 16 == 0 && bq_stride % 16 == 0)
+    {
+        hipLaunchKernelGGL((gemm_skinny_int8_kernel<GemmEpilogue>), dim3(ceil_div(N, 16), ceil_div(M, 16)), dim3(256), 0, as_stream(stream), aq_dev, aq_stride, M, bq_dev, bq_stride, N, K,
+                           epi);
+        return launch_status("gemm_skinny_int8_kernel");
+    }
     if (M <= GEMM_GEMV_MAX_ROWS && N >= 64)
     {
         const int vec = (aligned16(aq_dev) && aligned16(bq_dev) && aq_stride % 16 == 0 && bq_stride % 16 == 0) ? 1 : 0;

@@ -70,7 +70,9 @@ def test_transposes(rt):
 
 GEMM_SHAPES = [(13, 17, 96), (1, 1, 1), (128, 128, 64), (130, 257, 100), (64, 300, 77), (256, 512, 1024), (300, 200, 4100),
                # one to four rows of A on 64 columns and more: one wavefront per row of B (aligned rows, ragged K, K below a vector)
-               (1, 4096, 4096), (4, 1000, 2048), (3, 64, 100), (2, 333, 8)]
+               (1, 4096, 4096), (4, 1000, 2048), (3, 64, 100), (2, 333, 8),
+               # up to 48 rows on the matrix cores, 16 rows of A per group: ragged last group, ragged last tile of B, one K step
+               (16, 256, 64), (17, 1000, 1024), (48, 70, 2048), (33, 4096, 128)]
 
 
 @pytest.mark.parametrize("shape", GEMM_SHAPES)
