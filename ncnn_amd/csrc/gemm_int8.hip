@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const int8_t* __restrict__
 // columns of one output row); eight steps of B and A are requested before the first product; the four partial tiles are
 // added through LDS.  B is read once; A (at most 16 x K bytes) comes from the cache.
 typedef int v4i_sk __attribute__((ext_vector_type(4)));
-template<typename Epilogue>
+template<typename Epilogue, bool ROW_FIRST>
 __global__ __launch_bounds__(256) void gemm_skinny_int8_kernel(const int8_t* __restrict__ a, size_t as, int M_total, const int8_t* __restrict__ b, size_t bs, int N, int K,
                                                                 Epilogue epi)
 {
@@ -117,9 +117,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_int8_kernel(const int8_t* __r
     {
         const int v = (red[0][lane][r] + red[1][lane][r]) + (red[2][lane][r] + red[3][lane][r]);
         const int j = tile * 16 + 4 * q + r;
-        if (c16 < M && j < N) epi(row0 + c16, j, v);
+        if (c16 < M && j < N)
+        {
+            if (ROW_FIRST)
+                epi(row0 + c16, j, v); // Gemm's epilogue: (row of A, column)
+            else
+                epi(j, row0 + c16, v); // InnerProduct's: (output channel, row)
+        }
     }
 }
+
+// InnerProduct on 2 to 48 rows (a batch through the classifier of a net): the same kernel with InnerProduct's epilogue, under the
+// same estimate as Gemm's.  false: the shape is not one it takes.
+static bool launch_fc_skinny(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output, const int8_t* weight_dev, const FcEpilogue& epi,
+                             hipStream_t stream);
 
 #ifndef GEMM_GEMV_MAX_ROWS
 #define GEMM_GEMV_MAX_ROWS 4
@@ -151,6 +162,18 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
 
 int launch_gemm_int8_tiled(const int8_t* aq_tiled, const int8_t* bq_tiled, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream);
 int launch_gemm_tile_operand(const int8_t* src, size_t stride, int rows, int K, int operand_b, int8_t* dst, hipStream_t stream);
+
+static bool launch_fc_skinny(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output, const int8_t* weight_dev, const FcEpilogue& epi,
+                             hipStream_t stream)
+{
+    if (rows < 2 || rows > GEMM_SKINNY_MAX_ROWS || num_output < 64 || num_input % 64 != 0) return false;
+    if (!aligned16(x_dev) || !aligned16(weight_dev) || x_stride % 16 != 0) return false;
+    const int groups16 = (rows + 15) / 16;
+    if (rows > 16 && 3.0 + groups16 * ((double)num_output * (double)num_input / 4.0e6) > 4.0 + num_input / 300.0) return false;
+    hipLaunchKernelGGL((gemm_skinny_int8_kernel<FcEpilogue, false>), dim3(ceil_div(num_output, 16), groups16), dim3(256), 0, stream, x_dev, x_stride, rows, weight_dev,
+                       (size_t)num_input, num_output, num_input, epi);
+    return true;
+}
 
 } // namespace ncnnhip
 
@@ -197,7 +220,7 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
     const bool skinny_pays = M <= 16 || 3.0 + groups16 * ((double)N * (double)K / 4.0e6) <= 4.0 + K / 300.0;
     if (skinny_pays && M > GEMM_SKINNY_MIN_ROWS && M <= GEMM_SKINNY_MAX_ROWS && N >= 64 && K % 64 == 0 && aligned16(aq_dev) && aligned16(bq_dev) && aq_stride % 16 == 0 && bq_stride % 16 == 0)
     {
-        hipLaunchKernelGGL((gemm_skinny_int8_kernel<GemmEpilogue>), dim3(ceil_div(N, 16), ceil_div(M, 16)), dim3(256), 0, as_stream(stream), aq_dev, aq_stride, M, bq_dev, bq_stride, N, K,
+        hipLaunchKernelGGL((gemm_skinny_int8_kernel<GemmEpilogue, true>), dim3(ceil_div(N, 16), ceil_div(M, 16)), dim3(256), 0, as_stream(stream), aq_dev, aq_stride, M, bq_dev, bq_stride, N, K,
                            epi);
         return launch_status("gemm_skinny_int8_kernel");
     }
@@ -256,6 +279,7 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
     epi.num_output = num_output;
     epi.acc_out = acc_out_dev;
 
+    if (launch_fc_skinny(x_dev, x_stride, rows, num_input, num_output, weight_dev, epi, as_stream(stream))) return launch_status("gemm_skinny_int8_kernel<fc>");
     if (rows <= 64)
     {
         const int vec = aligned16(x_dev) && aligned16(weight_dev) && x_stride % 16 == 0 && num_input % 16 == 0;
@@ -286,6 +310,17 @@ int ncnnhip_innerproduct_int8_ws(const int8_t* x_dev, size_t x_stride, int rows,
     NCNNHIP_REQUIRE(x_dev && weight_dev && scale_in_dev && out_dev, "ncnnhip_innerproduct_int8_ws: null pointer");
     NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1, "ncnnhip_innerproduct_int8_ws: bad shape");
     NCNNHIP_REQUIRE(x_stride >= (size_t)num_input && out_stride >= (size_t)num_output, "ncnnhip_innerproduct_int8_ws: stride too small");
+    {
+        FcEpilogue fe;
+        fe.scale_in = scale_in_dev;
+        fe.bias = bias_dev;
+        fe.act = act;
+        fe.out = out_dev;
+        fe.out_stride = out_stride;
+        fe.num_output = num_output;
+        fe.acc_out = 0;
+        if (launch_fc_skinny(x_dev, x_stride, rows, num_input, num_output, weight_dev, fe, as_stream(stream))) return launch_status("gemm_skinny_int8_kernel<fc>");
+    }
     if (rows >= 8)
     {
         ConvEpilogue epi;
