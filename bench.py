@@ -152,13 +152,13 @@ def measured_traffic(key):
         return None
 
 
-def bench_gemm(args, size):
+def bench_gemm(args, size, shape=None):
     import ncnn_amd
     from ncnn_amd.hip import check, lib as load
     from ncnn_amd import synth
     lib = load()
     rt = ncnn_amd.Runtime(0)
-    m = n = k = size
+    m, n, k = shape if shape else (size, size, size)
     a, bq, sb, bias = synth.gemm_operands(size, m, n, k, per_col=args.b_scale == "per_column")
     d_a, d_bq, d_sb, d_bias = rt.up(a), rt.up(bq), rt.up(sb), rt.up(bias)
     d_aq = ncnn_amd.DeviceBuffer.empty((m, k), np.int8)
@@ -222,7 +222,7 @@ def bench_gemm(args, size):
         "metric": "int8 TOPS", "value": ops / (ms_per_step * 1e-3) / 1e12, "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "standalone int8 Gemm M=N=K=%d: per-row quantise A (fp32->int8) + int8 MFMA Gemm + fused dequantise/bias to fp32" % size,
+        "config": {"workload": ("standalone int8 Gemm M=N=K=%d" % size if not shape else "standalone int8 Gemm M=%d N=%d K=%d" % (m, n, k)) + ": per-row quantise A (fp32->int8) + int8 MFMA Gemm + fused dequantise/bias to fp32",
                    "b_scale": args.b_scale,
                    "parity": ("per-column B scales are a generalisation ncnn's Gemm cannot express: parity unpinned by the reference (own formula, "
                               "((float)acc*(1/sA_i))*(1/sB_j)); --b-scale per_tensor is the reference's form" if args.b_scale == "per_column"
@@ -231,6 +231,15 @@ def bench_gemm(args, size):
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
                      "traffic": measured_traffic("gemm%d" % size), "kernel": "gemm_int8", "ops_per_launch": ops},
     }
+    if m <= 48:
+        # a few rows of A: the work is reading B once, so the line is priced against the memory system
+        algo = n * k + m * k + m * n * 4
+        gbs = algo / (gemm_ms * 1e-3) / 1e9
+        line["roofline"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                            "kernel": "gemm_int8 (few rows: gemm_skinny_int8_kernel where the shape allows)", "bytes_per_launch": algo}
+        if not args.no_cpu:
+            line["cpu_baseline"] = cpu_baseline_gemm(n, k, args.b_scale == "per_column")
+        return line
     # what the matrix pipe of THIS chip sustains on operands like these (register-only spin, random bytes), beside the published peak
     mp = measure_peak_mfma_i8(lib, check, rt, True, iters=8000, reps=3)
     line["roofline"].update(measured_peak=mp["tops"], frac_of_measured=achieved / mp["tops"],
@@ -969,7 +978,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm4096",
-                    help="gemm<size> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
+                    help="gemm<size> | gemm:<M>x<N>x<K> | conv:<cin>x<h>x<w>:<cout>:k<k>[:b<batch>] | blockquant:<N>x<K>x<M>[:<bits>[:<block>]] | net:<resnet50|mobilenetv2>:<batch> (whole model through Net/Extractor) | "
                          "mha:<embed>x<heads>:<new tokens>:<cached tokens> | "
                          "layers:<resnet50|mobilenetv2>:<batch> (each quantised layer alone through the C ABI) | "
                          "peak:mfma_i8[:zeros|random] | peak:hbm_read:<bytes>[:<loads per lane>] | peak:launch[:<nodes>] (the chip's measured ceilings)")
@@ -989,7 +998,9 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU only (--gpus 1); multi-GPU figures are not produced")
-    if args.workload.startswith("gemm"):
+    if args.workload.startswith("gemm:"):
+        line = bench_gemm(args, 0, tuple(int(v) for v in args.workload[5:].split("x")))
+    elif args.workload.startswith("gemm"):
         line = bench_gemm(args, int(args.workload[4:] or 4096))
     elif args.workload.startswith("blockquant:"):
         parts = args.workload.split(":")
