@@ -236,7 +236,8 @@ def bench_gemm(args, size, shape=None):
         algo = n * k + m * k + m * n * 4
         gbs = algo / (gemm_ms * 1e-3) / 1e9
         line["roofline"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
-                            "kernel": "gemm_int8 (few rows: gemm_skinny_int8_kernel where the shape allows)", "bytes_per_launch": algo}
+                            "kernel": "gemm_int8 (few rows: gemm_skinny_int8_kernel where the shape allows)", "bytes_per_launch": algo,
+                            "note": "B is the same buffer in every step and may be served by the memory-side cache: an upper bound on what a pass over cold weights reaches"}
         if not args.no_cpu:
             line["cpu_baseline"] = cpu_baseline_gemm(n, k, args.b_scale == "per_column")
         return line
