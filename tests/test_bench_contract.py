@@ -37,7 +37,7 @@ def test_cpu_baseline_objects_name_the_cpu_and_both_thread_counts():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("workload", ["gemm1024", "conv:64x56x56:64:k3", "blockquant:4096x4096x1", "net:mobilenetv2:1", "peak:launch:8"])
+@pytest.mark.parametrize("workload", ["gemm1024", "gemm:16x1024x512", "conv:64x56x56:64:k3", "blockquant:4096x4096x1", "mha:256x4:1:300", "net:mobilenetv2:1", "peak:launch:8"])
 def test_bench_prints_one_json_line_with_the_agreed_keys(workload):
     p = _bench("--workload", workload, "--steps", "3", "--warmup", "1", "--no-cpu")
     assert p.returncode == 0, p.stderr[-2000:]
