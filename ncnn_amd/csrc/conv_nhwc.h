@@ -68,6 +68,10 @@ size_t conv_nhwc_staged_workspace_bytes(const NhwcGeom& g);
 int launch_conv_nhwc_staged(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
                             const ConvFusion& fusion, int out_cp, void* workspace, size_t workspace_bytes, hipStream_t stream);
 bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
+// The weights-resident kernel for layers with many output pixels (conv_resident.hip): does this problem fit it, and its
+// launch.  The pipelined launch asks first.
+bool conv_resident_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
+int launch_conv_resident(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp, hipStream_t stream);
 int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream);
 
 // D[M][N] = A[M][K] * B[N][K]^T through the pipelined kernel; handled = false when the shape does not fit it
