@@ -50,11 +50,19 @@ int ncnnhip_stream_end_capture(void* stream, void** graph_exec);
 int ncnnhip_graph_launch(void* graph_exec, void* stream);
 int ncnnhip_graph_destroy(void* graph_exec);
 int ncnnhip_malloc(void** dev, size_t bytes);
-/* Fault injection for out-of-memory tests (the reference forces the condition with an allocator that returns NULL,
- * tests/testutil.cpp:2111-2156): the next `calls` ncnnhip_malloc calls succeed, every one after them returns -100 until the
- * limit is lifted with a negative value.  No counterpart in the reference; not for production use. */
-int ncnnhip_debug_fail_malloc_after(int calls);
 int ncnnhip_free(void* dev);
+/* The device allocator behind ncnnhip_malloc / ncnnhip_free, and so behind every device buffer the host library cuts its
+ * blobs and workspaces from: the role ncnn::VkAllocator plays for the reference's GPU path (src/allocator.h:267-300,
+ * Option::blob_vkallocator, src/option.h:48).  A caller that already runs a device pool installs its own pair; malloc_fn returns 0 and a
+ * device pointer, or anything else to refuse (ncnnhip_malloc then reports -100, as the reference's layers do when an
+ * allocator returns NULL: tests/testutil.cpp:2111-2156 forces that condition the same way).  Passing two null functions
+ * restores hipMalloc / hipFree, which ncnnhip_default_device_malloc / _free expose for allocators that wrap them.  Install
+ * before the first buffer is allocated or make free_fn accept pointers of the previous allocator. */
+typedef int (*ncnnhip_device_malloc_fn)(void** dev, size_t bytes, void* user);
+typedef int (*ncnnhip_device_free_fn)(void* dev, void* user);
+int ncnnhip_set_device_allocator(ncnnhip_device_malloc_fn malloc_fn, ncnnhip_device_free_fn free_fn, void* user);
+int ncnnhip_default_device_malloc(void** dev, size_t bytes);
+int ncnnhip_default_device_free(void* dev);
 int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream);
 int ncnnhip_memcpy_d2h(void* host, const void* dev, size_t bytes, void* stream);
 int ncnnhip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);

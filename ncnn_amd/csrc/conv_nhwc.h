@@ -85,6 +85,9 @@ int launch_gemm_via_conv_pipelined(const int8_t* aq, size_t aq_stride, const int
 int launch_fc_via_conv_pipelined(const int8_t* x, size_t x_stride, int rows, int K, int num_output, const int8_t* weight, const ConvEpilogue& epi,
                                  size_t out_stride, void* workspace, size_t workspace_bytes, hipStream_t stream, bool* handled);
 
+// InnerProduct shapes the few-row kernel (gemm_int8.hip) serves without any workspace, given aligned operands
+bool fc_skinny_takes(int rows, int num_input, int num_output);
+
 // Device address, on the current device, of the scratch array the library holds for ncnnhip_innerproduct_int8_noalloc
 // (looked up once per device; ncnnhip_init calls it so that the first real call finds it ready).
 int static_scratch_for_current_device(void** ptr);

@@ -1346,6 +1346,10 @@ extern "C" int ncnnhip_innerproduct_int8_noalloc(const int8_t* x_dev, size_t x_s
     void* ptr = 0;
     int ret = static_scratch_for_current_device(&ptr);
     if (ret != NCNNHIP_OK) return ret;
+    // few rows: the kernel that needs no scratch (and so no ordering between calls that share it)
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(weight_dev)) & 15) == 0 && x_stride % 16 == 0;
+    if (aligned && fc_skinny_takes(rows, num_input, num_output))
+        return ncnnhip_innerproduct_int8(x_dev, x_stride, rows, num_input, num_output, weight_dev, scale_in_dev, bias_dev, act, out_dev, out_stride, 0, stream);
     if (rows >= 8 && num_input % 64 == 0)
     {
         const size_t need = conv_nhwc_pipelined_workspace_words(num_output, rows, num_input / 64) * sizeof(int32_t);

@@ -163,13 +163,20 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
 int launch_gemm_int8_tiled(const int8_t* aq_tiled, const int8_t* bq_tiled, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream);
 int launch_gemm_tile_operand(const int8_t* src, size_t stride, int rows, int K, int operand_b, int8_t* dst, hipStream_t stream);
 
+// the shapes the few-row kernel takes for InnerProduct (operands aligned): no workspace, no hand-off between workgroups
+bool fc_skinny_takes(int rows, int num_input, int num_output)
+{
+    if (rows < 2 || rows > GEMM_SKINNY_MAX_ROWS || num_output < 64 || num_input % 64 != 0) return false;
+    const int groups16 = (rows + 15) / 16;
+    return !(rows > 16 && 3.0 + groups16 * ((double)num_output * (double)num_input / 4.0e6) > 4.0 + num_input / 300.0);
+}
+
 static bool launch_fc_skinny(const int8_t* x_dev, size_t x_stride, int rows, int num_input, int num_output, const int8_t* weight_dev, const FcEpilogue& epi,
                              hipStream_t stream)
 {
-    if (rows < 2 || rows > GEMM_SKINNY_MAX_ROWS || num_output < 64 || num_input % 64 != 0) return false;
+    if (!fc_skinny_takes(rows, num_input, num_output)) return false;
     if (!aligned16(x_dev) || !aligned16(weight_dev) || x_stride % 16 != 0) return false;
     const int groups16 = (rows + 15) / 16;
-    if (rows > 16 && 3.0 + groups16 * ((double)num_output * (double)num_input / 4.0e6) > 4.0 + num_input / 300.0) return false;
     hipLaunchKernelGGL((gemm_skinny_int8_kernel<FcEpilogue, false>), dim3(ceil_div(num_output, 16), groups16), dim3(256), 0, stream, x_dev, x_stride, rows, weight_dev,
                        (size_t)num_input, num_output, num_input, epi);
     return true;
@@ -299,7 +306,10 @@ int ncnnhip_innerproduct_int8(const int8_t* x_dev, size_t x_stride, int rows, in
 int ncnnhip_innerproduct_workspace_bytes(int rows, int num_input, int num_output, size_t* workspace_bytes)
 {
     NCNNHIP_REQUIRE(rows >= 1 && num_input >= 1 && num_output >= 1 && workspace_bytes, "ncnnhip_innerproduct_workspace_bytes: bad argument");
-    *workspace_bytes = (rows >= 8 && num_input % 64 == 0) ? conv_nhwc_pipelined_workspace_words(num_output, rows, num_input / 64) * sizeof(int32_t) : 0;
+    // (the few-row kernel needs none; the tiled kernel splits K over workgroups when its tiles are few)
+    *workspace_bytes = (rows >= 8 && num_input % 64 == 0 && !fc_skinny_takes(rows, num_input, num_output))
+                           ? conv_nhwc_pipelined_workspace_words(num_output, rows, num_input / 64) * sizeof(int32_t)
+                           : 0;
     return NCNNHIP_OK;
 }
 

@@ -2,6 +2,7 @@
 #include <stdarg.h>
 
 #include <atomic>
+#include <mutex>
 #include <string.h>
 
 #include "common.h"
@@ -144,13 +145,49 @@ int ncnnhip_device_synchronize(void)
     return NCNNHIP_OK;
 }
 
-// fault injection for out-of-memory tests: the number of ncnnhip_malloc calls that still succeed, negative = no limit
-static std::atomic<long> g_mallocs_left(-1);
-
-int ncnnhip_debug_fail_malloc_after(int calls)
+// The device allocator every buffer of the library comes from: hipMalloc / hipFree unless the caller has installed a
+// table of its own (a pool it already runs, an arena per request, an allocator that refuses: the out-of-memory tests).
+static int default_device_malloc(void** dev, size_t bytes, void*)
 {
-    g_mallocs_left.store(calls < 0 ? -1 : calls);
+    hipError_t e = hipMalloc(dev, bytes);
+    if (e != hipSuccess) return map_hip_error(e, "hipMalloc");
     return NCNNHIP_OK;
+}
+static int default_device_free(void* dev, void*)
+{
+    hipError_t e = hipFree(dev);
+    if (e != hipSuccess) return map_hip_error(e, "hipFree");
+    return NCNNHIP_OK;
+}
+struct DeviceAllocator
+{
+    ncnnhip_device_malloc_fn malloc_fn;
+    ncnnhip_device_free_fn free_fn;
+    void* user;
+};
+static std::mutex g_allocator_mutex;
+static DeviceAllocator g_allocator = {default_device_malloc, default_device_free, 0};
+
+int ncnnhip_set_device_allocator(ncnnhip_device_malloc_fn malloc_fn, ncnnhip_device_free_fn free_fn, void* user)
+{
+    NCNNHIP_REQUIRE((malloc_fn != 0) == (free_fn != 0), "ncnnhip_set_device_allocator: give both functions, or neither to restore hipMalloc / hipFree");
+    std::lock_guard<std::mutex> lock(g_allocator_mutex);
+    if (malloc_fn)
+        g_allocator = {malloc_fn, free_fn, user};
+    else
+        g_allocator = {default_device_malloc, default_device_free, 0};
+    return NCNNHIP_OK;
+}
+
+int ncnnhip_default_device_malloc(void** dev, size_t bytes)
+{
+    NCNNHIP_REQUIRE(dev, "null out pointer");
+    return default_device_malloc(dev, bytes, 0);
+}
+
+int ncnnhip_default_device_free(void* dev)
+{
+    return dev ? default_device_free(dev, 0) : NCNNHIP_OK;
 }
 
 int ncnnhip_malloc(void** dev, size_t bytes)
@@ -158,24 +195,30 @@ int ncnnhip_malloc(void** dev, size_t bytes)
     NCNNHIP_REQUIRE(dev, "null out pointer");
     *dev = 0;
     if (bytes == 0) bytes = 4;
-    if (g_mallocs_left.load() >= 0)
+    DeviceAllocator a;
     {
-        // (tests only) the injected limit is spent: report what hipMalloc reports when the device is full
-        if (g_mallocs_left.fetch_sub(1) <= 0)
-        {
-            g_mallocs_left.store(0);
-            set_error("ncnnhip_malloc: out of memory (injected by ncnnhip_debug_fail_malloc_after)");
-            return NCNNHIP_OOM;
-        }
+        std::lock_guard<std::mutex> lock(g_allocator_mutex);
+        a = g_allocator;
     }
-    NCNNHIP_CHECK(hipMalloc(dev, bytes));
+    const int ret = a.malloc_fn(dev, bytes, a.user);
+    if (ret != NCNNHIP_OK || !*dev)
+    {
+        *dev = 0;
+        if (ret == NCNNHIP_OK || a.malloc_fn != default_device_malloc) set_error("ncnnhip_malloc: the device allocator refused %zu bytes", bytes);
+        return NCNNHIP_OOM;
+    }
     return NCNNHIP_OK;
 }
 
 int ncnnhip_free(void* dev)
 {
-    if (dev) NCNNHIP_CHECK(hipFree(dev));
-    return NCNNHIP_OK;
+    if (!dev) return NCNNHIP_OK;
+    DeviceAllocator a;
+    {
+        std::lock_guard<std::mutex> lock(g_allocator_mutex);
+        a = g_allocator;
+    }
+    return a.free_fn(dev, a.user);
 }
 
 int ncnnhip_memcpy_h2d(void* dev, const void* host, size_t bytes, void* stream)

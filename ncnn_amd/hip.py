@@ -63,7 +63,9 @@ _SIGNATURES = {
     "ncnnhip_stream_end_capture": [C.c_void_p, C.POINTER(C.c_void_p)],
     "ncnnhip_graph_launch": [C.c_void_p, C.c_void_p],
     "ncnnhip_graph_destroy": [C.c_void_p],
-    "ncnnhip_debug_fail_malloc_after": [C.c_int],
+    "ncnnhip_set_device_allocator": [C.c_void_p, C.c_void_p, C.c_void_p],
+    "ncnnhip_default_device_malloc": [c_void_pp, C.c_size_t],
+    "ncnnhip_default_device_free": [C.c_void_p],
     "ncnnhip_malloc": [c_void_pp, C.c_size_t],
     "ncnnhip_free": [C.c_void_p],
     "ncnnhip_memcpy_h2d": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],

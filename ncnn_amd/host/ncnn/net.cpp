@@ -472,13 +472,21 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
             return -1;
         }
         ret = run_layer_hip(layer, st, lopt);
-        ncnnhip_event_record(slot.stop, st.cmd->stream);
+        // a record is kept only when the layer ran and its stop event was recorded: a half-recorded pair could not be
+        // read back and would cost the records around it
+        if (ret != 0 || ncnnhip_event_record(slot.stop, st.cmd->stream) != 0)
+        {
+            ncnnhip_event_destroy(slot.start);
+            ncnnhip_event_destroy(slot.stop);
+            return ret != 0 ? ret : -1;
+        }
     }
     else
     {
         const std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
         ret = run_layer(layer, st, lopt);
         slot.host_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        if (ret != 0) return ret;
     }
     st.timing.push_back(slot); // (copied as plain pointers: the state owns the events from here on)
     return ret;
@@ -1272,9 +1280,10 @@ int Extractor::layer_timing(std::vector<LayerTime>& out)
         t.ms = s.host_ms;
         if (s.start)
         {
+            // a pair that cannot be read (recorded while the stream was being captured into a graph) is reported as
+            // -1 ms; the other records stay valid
             float ms = 0.f;
-            if (ncnnhip_event_elapsed_ms(s.start, s.stop, &ms) != 0) return -1;
-            t.ms = ms;
+            t.ms = ncnnhip_event_elapsed_ms(s.start, s.stop, &ms) == 0 ? ms : -1.0;
         }
         out.push_back(t);
     }

@@ -1,8 +1,8 @@
 """Out-of-memory behaviour at the boundary (the reference's tests/test_convolution_oom.cpp and tests/test_gemm_oom.cpp
 through tests/testutil.cpp:2111-2340): an allocator that returns NULL at its N-th call, for every N up to the number of
 calls a clean pass makes, must make the pass return -100 -- no crash, nothing left behind that spoils the next pass.
-On the host the NULL comes from a replaced entry of the allocator's function-pointer table; on the device from the
-fault-injection switch of ncnnhip_malloc."""
+On the host the NULL comes from a replaced entry of the allocator's function-pointer table; on the device from a device
+allocator installed with ncnnhip_set_device_allocator that refuses from its N-th call on."""
 import ctypes as C
 
 import numpy as np
@@ -13,6 +13,8 @@ from ncnn_amd import hip, host, zoo
 
 pytestmark = pytest.mark.gpu
 F = np.float32
+MALLOC_FN = C.CFUNCTYPE(C.c_int, C.POINTER(C.c_void_p), C.c_size_t, C.c_void_p)
+FREE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p)
 
 
 class FailingAllocator:
@@ -104,13 +106,32 @@ def test_device_allocation_failing_gives_minus_100(resident):
         ex.input("data", x)
         return _extract_code(ex, "fc")
 
+    # a device allocator that wraps the default one and refuses from the n-th call on (the reference's test allocator
+    # returns NULL the same way: tests/testutil.cpp:2111-2156)
+    left = [0]
+
+    @MALLOC_FN
+    def counting_malloc(dev, nbytes, user):
+        if left[0] <= 0:
+            return -100
+        left[0] -= 1
+        return K.ncnnhip_default_device_malloc(dev, nbytes)
+
+    @FREE_FN
+    def plain_free(dev, user):
+        return K.ncnnhip_default_device_free(dev)
+
+    def restore():
+        hip.check(K.ncnnhip_set_device_allocator(None, None, None))
+
     try:
         failures = 0
         for n in range(0, 200):
             print("device allocation limit", n, flush=True)
-            hip.check(K.ncnnhip_debug_fail_malloc_after(n))
+            left[0] = n
+            hip.check(K.ncnnhip_set_device_allocator(C.cast(counting_malloc, C.c_void_p), C.cast(plain_free, C.c_void_p), None))
             ret, got = one_pass()
-            hip.check(K.ncnnhip_debug_fail_malloc_after(-1))
+            restore()
             if ret == 0:
                 assert np.array_equal(got, want)
                 break
@@ -120,6 +141,6 @@ def test_device_allocation_failing_gives_minus_100(resident):
             pytest.fail("a pass still ran out of device memory with 200 allocations allowed")
         assert failures >= 1, "the first pass of a net allocates device buffers: a limit of 0 must fail"
     finally:
-        hip.check(K.ncnnhip_debug_fail_malloc_after(-1))
+        restore()
     ret, got = one_pass()
     assert ret == 0 and np.array_equal(got, want)

@@ -632,7 +632,7 @@ def test_blockquant_packed_fp32_split_keeps_all_24_bits(rt, bits, block):
 
 
 @pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008)])
-@pytest.mark.parametrize("m,act", [(1, "fp16"), (16, "fp16"), (1, "fp32"), (4, "fp32"), (16, "fp32"), (64, "fp32"), (200, "fp32")])
+@pytest.mark.parametrize("m,act", [(1, "fp16"), (4, "fp16"), (16, "fp16"), (1, "fp32"), (4, "fp32"), (16, "fp32"), (64, "fp32"), (200, "fp32")])
 def test_blockquant_full_size_properties(rt, n, k, m, act):
     """The decode configuration at its full sizes, through size-independent properties (no oracle pass over 45 M weights per case):
     doubling the activations doubles every output exactly (a power of two commutes with the split, the products and the sums);

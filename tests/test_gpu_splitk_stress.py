@@ -72,7 +72,7 @@ def test_k_split_convolution_200_launches_on_two_streams(rt):
 
 
 def test_k_split_innerproduct_200_launches_on_two_streams(rt):
-    rows, k, n = 16, 2048, 1000
+    rows, k, n = 64, 2048, 1000  # beyond the few-row kernel's 48 rows: 16 tiles of 64 x 64, K split over workgroups
     rng = np.random.default_rng(5)
     xq = rng.integers(-127, 128, (rows, k)).astype(np.int8)
     wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
@@ -83,7 +83,7 @@ def test_k_split_innerproduct_200_launches_on_two_streams(rt):
 
     wsb = C.c_size_t()
     check(lib().ncnnhip_innerproduct_workspace_bytes(rows, k, n, C.byref(wsb)))
-    assert wsb.value > 0, "this shape is meant to take the K-split path"
+    assert wsb.value > 0, "this shape is meant to take the K-split path (the few-row kernel, which hands nothing over, reports no workspace)"
     dx, dw, dsi, db = rt.up(xq), rt.up(wq), rt.up(rt.fold_input_scales(ws, [in_scale], n)), rt.up(b)
     rt.sync()
     out_bytes = rows * n * 4

@@ -301,6 +301,44 @@ def test_gemm_int8_matches_numpy(bt, alpha, beta, transpose, per_col):
     assert np.array_equal(gacc, wacc) and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("bt", [-1, 0, 1, 4])
+@pytest.mark.parametrize("per_col", [False, True])
+@pytest.mark.parametrize("scale_span", [(50.0, 500.0), (1e-3, 1e3)])
+def test_gemm_int8_dequantisation_is_the_closed_form_to_a_few_ulp(bt, per_col, scale_span):
+    """What the mathematics fixes for the Gemm epilogue, independent of any restatement of its formula: the result is
+    alpha * (acc / (sA_i * sB_j) + beta * c) evaluated in float64, and the fp32 statements of the reference
+    (src/layer/gemm.cpp:509-555: one division for the descale, one multiply by it, the C term, the multiply by alpha; with
+    one B scale per column two divisions and two multiplies) round at most five times on the way, so every output lies
+    within 4 ulp of the float64 value's magnitude (measured on the larger of the result and its two addends: the sum may
+    cancel).  A transposed operand, a scale applied to the wrong axis, a dropped beta or alpha miss this by orders of
+    magnitude on scales that span six decades."""
+    rng = np.random.default_rng(7 + bt + 10 * per_col)
+    m, n, k = 13, 17, 96
+    a = rng.normal(0, 1, (m, k)).astype(F) * np.exp(rng.uniform(np.log(scale_span[0]), np.log(scale_span[1]), (m, 1))).astype(F)
+    aq, sa = oracle.gemm_quantize_rows(a)
+    bq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sb = np.exp(rng.uniform(np.log(scale_span[0]), np.log(scale_span[1]), n if per_col else 1)).astype(F)
+    c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 4: rng.normal(size=(1, n))}[bt]
+    c = None if c is None else c.astype(F)
+    alpha, beta = 1.7, 0.3
+    got = oracle.gemm_int8(aq, bq, sa, sb, c, bt, alpha, beta, False).astype(np.float64)
+    acc = aq.astype(np.int64) @ bq.astype(np.int64).T
+    scale = sa.astype(np.float64)[:, None] * (sb.astype(np.float64)[None, :] if per_col else float(sb[0]))
+    deq = acc / scale
+    cterm = np.zeros((m, n))
+    if bt == 0:
+        cterm[:] = float(c[0])
+    elif bt == 1:
+        cterm[:] = c.astype(np.float64)[:, None]
+    elif bt == 4:
+        cterm[:] = c.astype(np.float64).reshape(1, n)
+    want = float(F(alpha)) * (deq + float(F(beta)) * cterm)
+    magnitude = float(F(alpha)) * np.maximum(np.abs(deq), np.abs(float(F(beta)) * cterm))
+    ulp = np.maximum(magnitude, 1e-300) * 2.0 ** -23
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= 4 * ulp), float(np.max(np.abs(got - want) / ulp))
+
+
 def test_gemm_operands_are_not_transposed():
     # asymmetric one-hot probes: acc[i][j] must be sum_k A[i][k]*B[j][k]
     aq = np.zeros((2, 4), np.int8)

@@ -44,9 +44,10 @@ def test_noalloc_innerproduct_equals_the_workspace_form_on_calls_in_a_row():
     import ncnn_amd
     from ncnn_amd import hip
     rt = ncnn_amd.Runtime(0)
-    # K-split shapes first (FC 2048 -> 1000 at batch 16 is the ResNet-50 head), each smaller than the one before, then a
-    # shape without a split and one the gemv kernel takes; all share the one scratch
-    shapes = [(16, 2048, 1000), (16, 1280, 1000), (8, 1024, 256), (64, 512, 128), (300, 256, 64), (3, 100, 10)]
+    # K-split shapes first (FC 2048 -> 1000 is the ResNet-50 head, at a batch beyond the few-row kernel's 48 rows), each
+    # smaller than the one before, then shapes without a split: the few-row kernel's, a tiled one, the gemv kernel's; all
+    # share the one scratch
+    shapes = [(64, 2048, 1000), (56, 1280, 1000), (50, 1024, 256), (16, 2048, 1000), (64, 512, 128), (300, 256, 64), (3, 100, 10)]
     used_scratch = 0
     for i, (rows, k, n) in enumerate(shapes):
         print("noalloc innerproduct", rows, k, n, flush=True)
@@ -58,7 +59,7 @@ def test_noalloc_innerproduct_equals_the_workspace_form_on_calls_in_a_row():
         assert np.array_equal(got, ref), "no-alloc form differs from the oracle at %s" % ((rows, k, n),)
     assert used_scratch >= 3, "the shapes were meant to exercise the K split"
     # the same large shape again after the small ones: whatever they left in the scratch must not matter
-    xq, wq, w_scales, in_scale, bias = _case(7, 16, 2048, 1000)
+    xq, wq, w_scales, in_scale, bias = _case(7, 64, 2048, 1000)
     got, want, _ = _both_forms(rt, hip, xq, wq, w_scales, in_scale, bias, act=0)
     assert np.array_equal(got, want)
 
