@@ -340,6 +340,80 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     return line
 
 
+def bench_blockquant_multi(args, ns, k, m, bits=8, block=64):
+    """Sibling block-quant Gemms of a decoder layer (gate + up, q + k + v) on the same activation rows: all matrices in ONE launch
+    (ncnnhip_gemm_blockquant_packed_multi), against one launch per matrix, weights rotated over more copies than the last-level
+    cache holds.  One step = every matrix of the group once."""
+    import ncnn_amd
+    from ncnn_amd.hip import check, lib as load
+    from ncnn_amd import synth
+    lib = load()
+    rt = ncnn_amd.Runtime(0)
+    half = args.act == "fp16"
+    if not half and args.act != "fp32":
+        raise SystemExit("blockquant-multi runs on the packed weights: --act fp16 or fp32")
+    a = None
+    packs, wbytes = [], 0
+    for i, n in enumerate(ns):
+        ai, packed, scales = synth.blockquant_operands(n + k + m + i, m, n, k, bits, block)
+        a = ai if a is None else a
+        wbytes += packed.nbytes + scales.nbytes
+        packs.append(rt.blockquant_pack(packed, scales, block, bits=bits, k=k))
+    copies = int(np.ceil(512e6 / wbytes)) + 1
+    dev = [[(rt.up(pw), rt.up(pd), n, None, -1, 1.0, 1.0) for (pw, pd), n in zip(packs, ns)] for _ in range(copies)]
+    d_a = rt.up(a.astype(np.float16) if half else a)
+    douts = [ncnn_amd.DeviceBuffer.empty((m, n), np.float32) for n in ns]
+    multi_args = [rt.blockquant_multi_args(mats, douts) for mats in dev]
+    st = rt.stream
+    esize = 2 if half else 4
+
+    def launch_multi(i):
+        nn, ws, ds, cs, bts, als, bes, outs, strides = multi_args[i % copies]
+        check(lib.ncnnhip_gemm_blockquant_packed_multi(d_a.ptr, esize, k, m, k, len(ns), nn, ws, ds, bits, block, None, cs, bts, als, bes, outs, strides, st))
+
+    def launch_singles(i):
+        for (dw, dd, n, _, _, _, _), do in zip(dev[i % copies], douts):
+            if half:
+                check(lib.ncnnhip_gemm_blockquant_packed_f16a(d_a.ptr, k, m, n, k, dw.ptr, dd.ptr, bits, block, None, -1, 1.0, 1.0, do.ptr, n, st))
+            else:
+                check(lib.ncnnhip_gemm_blockquant_packed(d_a.ptr, k, m, n, k, dw.ptr, dd.ptr, bits, block, None, None, -1, 1.0, 1.0, do.ptr, n, st))
+
+    def timed(fn):
+        for i in range(args.warmup):
+            fn(i)
+        rt.sync()
+        evs = _events(lib, check, 2)
+        t0 = time.perf_counter()
+        check(lib.ncnnhip_event_record(evs[0], st))
+        for i in range(args.steps):
+            fn(i)
+        check(lib.ncnnhip_event_record(evs[1], st))
+        check(lib.ncnnhip_device_synchronize())
+        return _elapsed(lib, check, evs[0], evs[1]) / args.steps, (time.perf_counter() - t0) * 1e3 / args.steps
+
+    singles_ms, _ = timed(launch_singles)
+    k_ms, ms_per_step = timed(launch_multi)
+    algo = wbytes + m * k * esize + sum(m * n * 4 for n in ns)
+    achieved = algo / (k_ms * 1e-3) / 1e9
+    del dev, multi_args
+    floor = measure_peak_hbm_read(lib, check, rt, int(algo), 8, launches=200)
+    line = {
+        "metric": "HBM GB/s", "value": algo / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "block-quant Gemms %s x K=%d on the same M=%d activation rows in one launch, %d-bit weights in blocks of %d, fp32 block scales, %s activations"
+                               % ("+".join(str(n) for n in ns), k, m, bits, block, args.act),
+                   "weight_copies_rotated": copies, "one_launch_per_matrix_us": singles_ms * 1e3, "one_launch_us": k_ms * 1e3},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "blockquant8_upfront_kernel (several matrices per launch)", "bytes_per_launch": algo,
+                     "measured_peak": floor["gbs"], "frac_of_measured": achieved / floor["gbs"],
+                     "measured_peak_how": "read-only kernel over the same number of bytes, back-to-back launches over rotating copies: %.2f us per launch"
+                                          % floor["us_per_launch"]},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_blockquant(sum(ns), k, m, bits, block)
+    return line
+
+
 def measure_peak_mfma_i8(lib, check, rt, random_operands, iters=20000, reps=5):
     """int8 matrix-core rate with nothing else going on: (POP/s, shader MHz, operations per clock per compute unit)."""
     import ncnn_amd
@@ -1003,6 +1077,11 @@ def main():
         line = bench_gemm(args, 0, tuple(int(v) for v in args.workload[5:].split("x")))
     elif args.workload.startswith("gemm"):
         line = bench_gemm(args, int(args.workload[4:] or 4096))
+    elif args.workload.startswith("blockquant-multi:"):
+        parts = args.workload.split(":")
+        nspec, k, m = parts[1].split("x")
+        line = bench_blockquant_multi(args, [int(v) for v in nspec.split("+")], int(k), int(m), int(parts[2]) if len(parts) > 2 else 8,
+                                      int(parts[3]) if len(parts) > 3 else 64)
     elif args.workload.startswith("blockquant:"):
         parts = args.workload.split(":")
         n, k, m = (int(v) for v in parts[1].split("x"))

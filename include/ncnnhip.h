@@ -395,6 +395,20 @@ int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, i
                                    const float* c_dev, int broadcast_type_c, float alpha, float beta, float* out_dev,
                                    size_t out_stride, void* stream);
 
+/* Several packed weight matrices on the SAME activation rows in one launch: the gate and up projections of a decoder layer, the
+ * q / k / v projections of an attention layer -- in the reference one Gemm / MultiHeadAttention projection after the other
+ * (src/layer/gemm.cpp:425-483 per matrix); the results are those of `count` calls of ncnnhip_gemm_blockquant_packed(_f16a), bit
+ * for bit.  a_elemsize 2: fp16 activations (up to 16 rows in one pass); 4: fp32 (up to 4 rows, with optional in_scales [K]).
+ * All matrices share K, bits and block; N, the packed weights and descales, C (c_dev or its entries may be null), its broadcast
+ * type, alpha, beta (null: 1) and the outputs are per matrix, count <= 8.  A decode-sized launch is paced by its ramp and tail,
+ * not by bandwidth: one launch over 2 x 45.8 MB reaches what two launches of 45.8 MB cannot.  Shapes the one-pass kernel does
+ * not take run matrix by matrix. */
+int ncnnhip_gemm_blockquant_packed_multi(const void* a_dev, int a_elemsize, size_t a_stride, int M, int K, int count, const int* N,
+                                         const uint8_t* const* packed_w_dev, const float* const* packed_descale_dev, int bits,
+                                         int block, const float* in_scales_dev, const float* const* c_dev, const int* broadcast_type_c,
+                                         const float* alpha, const float* beta, float* const* out_dev, const size_t* out_stride,
+                                         void* stream);
+
 /* The same contract from five activation rows up, with a workspace: the three-way split is made once, by a pass of its own,
  * into the workspace (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes: 6 bytes per activation, rows and K rounded up to 64).
  * Up to 128 rows, while streaming the weights once per 16 rows is cheaper than a tiled pass (small weight matrices, or few

@@ -855,12 +855,50 @@ __device__ __forceinline__ void sixbit_to_bf16(unsigned d0, unsigned d1, unsigne
     wb = b.h;
 }
 
-template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN = 2, bool INSC = false>
-__global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const void* __restrict__ a_, size_t a_stride, int M, int N, int K, int kblocks,
-                                                                        const unsigned char* __restrict__ wpk, const float4* __restrict__ dpk, int split,
-                                                                        const float* __restrict__ in_scales, const float* __restrict__ c, int bt, float alpha,
-                                                                        float beta, float* __restrict__ out, size_t out_stride)
+// Several weight matrices that share the activation rows, K and the field format in ONE launch (the gate and up projections of a
+// decoder layer, q / k / v of an attention layer): the tiles of matrix i follow those of matrix i - 1 in the grid, and a workgroup
+// finds its matrix by comparing its index with the running tile counts.  A launch of 17.8 or 45.8 MB is paced by its ramp and its
+// tail, not by bandwidth; two or three of them in one launch are one ramp and one tail.  count == 0: the kernel's own arguments
+// describe the one matrix.
+constexpr int BQ_MULTI_MAX = 8;
+struct BqMulti
 {
+    int count;
+    int tile_end[BQ_MULTI_MAX]; // first tile (of the whole launch) that no longer belongs to matrix i
+    int N[BQ_MULTI_MAX];
+    int bt[BQ_MULTI_MAX];
+    float alpha[BQ_MULTI_MAX], beta[BQ_MULTI_MAX];
+    const unsigned char* wpk[BQ_MULTI_MAX];
+    const float4* dpk[BQ_MULTI_MAX];
+    const float* c[BQ_MULTI_MAX];
+    float* out[BQ_MULTI_MAX];
+    size_t out_stride[BQ_MULTI_MAX];
+};
+
+template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN = 2, bool INSC = false>
+__global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const void* __restrict__ a_, size_t a_stride, int M, int N_, int K, int kblocks,
+                                                                        const unsigned char* __restrict__ wpk_, const float4* __restrict__ dpk_, int split,
+                                                                        const float* __restrict__ in_scales, const float* __restrict__ c_, int bt_, float alpha_,
+                                                                        float beta_, float* __restrict__ out_, size_t out_stride_, BqMulti multi)
+{
+    // which matrix, which of its tiles (all wavefront-uniform: scalar loads from the argument block)
+    int tile = blockIdx.x;
+    int N = N_, bt = bt_;
+    float alpha = alpha_, beta = beta_;
+    const unsigned char* wpk = wpk_;
+    const float4* dpk = dpk_;
+    const float* c = c_;
+    float* out = out_;
+    size_t out_stride = out_stride_;
+    if (multi.count)
+    {
+        int mi = 0;
+#pragma unroll
+        for (int i = 0; i < BQ_MULTI_MAX - 1; i++) mi += (i + 1 < multi.count && tile >= multi.tile_end[i]) ? 1 : 0;
+        tile -= mi ? multi.tile_end[mi - 1] : 0;
+        N = multi.N[mi], bt = multi.bt[mi], alpha = multi.alpha[mi], beta = multi.beta[mi];
+        wpk = multi.wpk[mi], dpk = multi.dpk[mi], c = multi.c[mi], out = multi.out[mi], out_stride = multi.out_stride[mi];
+    }
     static_assert(HALVES || BITS == 8, "4- and 6-bit fields come in the halves layout");
     static_assert(AIN == 2 || (AIN == 4 && ACT_LDS), "fp32 activations are staged in LDS");
     static_assert(AIN == 4 || !INSC, "input scales come with fp32 activations");
@@ -880,7 +918,6 @@ __global__ __launch_bounds__(MAXW * 64) void blockquant8_upfront_kernel(const vo
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nwaves = blockDim.x >> 6;
-    const int tile = blockIdx.x;
     const int m = lane & 15;
     const int kg = lane >> 4;
 
@@ -1895,7 +1932,7 @@ __global__ __launch_bounds__(512) void blockquant_rows16_bf16x3_kernel(const uin
 template<int BITS, bool HALVES, int NB, int MAXW, int MT, bool ACT_LDS, int AIN, bool INSC>
 static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int K, int kblocks, const unsigned char* wpk, const float4* dpk, int split,
                               const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride, hipStream_t stream,
-                              bool* handled)
+                              bool* handled, const BqMulti* multi)
 {
     constexpr int AV = ACT_LDS ? (MT * NB * 8 + 63) / 64 : 1;
     constexpr int AROWS = ACT_LDS ? (AIN == 4 ? MT : (AV * 64 + NB * 8 - 1) / (NB * 8)) : 0;
@@ -1921,8 +1958,11 @@ static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int 
             if (device >= 0 && device < 64) raised[device].store(1, std::memory_order_release);
         }
     }
-    hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta,
-                       out, out_stride);
+    BqMulti one;
+    one.count = 0;
+    const int grid = multi ? multi->tile_end[multi->count - 1] : (N + 15) / 16;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(nwaves * 64), lds, stream, a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta,
+                       out, out_stride, multi ? *multi : one);
     return launch_status("blockquant8_upfront_kernel");
 }
 
@@ -1931,13 +1971,13 @@ static int launch_upfront_one(const void* a, size_t a_stride, int M, int N, int 
 template<int BITS, bool HALVES, int AIN, bool INSC>
 static int launch_blockquant8_upfront(const void* a, size_t a_stride, int M, int N, int K, const unsigned char* wpk, const float4* dpk, int split,
                                       const float* in_scales, const float* c, int bt, float alpha, float beta, float* out, size_t out_stride,
-                                      hipStream_t stream, bool* handled)
+                                      hipStream_t stream, bool* handled, const BqMulti* multi = 0)
 {
     const int kblocks = (K + 63) / 64;
     *handled = true;
 #define UPFRONT(NB_, MAXW_, MT_, LDS_) \
     return launch_upfront_one<BITS, HALVES, NB_, MAXW_, MT_, LDS_, AIN, INSC>(a, a_stride, M, N, K, kblocks, wpk, dpk, split, in_scales, c, bt, alpha, beta, out, \
-                                                                              out_stride, stream, handled)
+                                                                              out_stride, stream, handled, multi)
     if (M <= 4)
     {
         // decoding: 8 steps per wavefront while 8 or 16 wavefronts cover K (K up to 8192; measured against 16 steps on half
@@ -1986,7 +2026,7 @@ static int launch_blockquant8_upfront(const void* a, size_t a_stride, int M, int
 #ifndef BQ_PAIR_MIN_TILES
 #define BQ_PAIR_MIN_TILES 1024
 #endif
-        if (kblocks <= 64 && ntiles >= BQ_PAIR_MIN_TILES)
+        if (kblocks <= 64 && ntiles >= BQ_PAIR_MIN_TILES && !multi)
         {
             // many weight rows: two tiles per workgroup share the activation registers
             const int nwaves = (kblocks + 7) / 8;
@@ -2415,6 +2455,91 @@ int ncnnhip_gemm_blockquant_packed(const float* a_dev, size_t a_stride, int M, i
 {
     return gemm_blockquant_packed("ncnnhip_gemm_blockquant_packed", a_dev, 4, a_stride, M, N, K, packed_w_dev, packed_descale_dev, bits, block, in_scales_dev,
                                   c_dev, broadcast_type_c, alpha, beta, out_dev, out_stride, stream);
+}
+
+// Several matrices on the same activation rows in one launch (see BqMulti).  Shapes the one-pass kernel does not take (more
+// than 16 rows of fp16 or 4 of fp32 activations, long K) run matrix by matrix through the single-matrix entries.
+int ncnnhip_gemm_blockquant_packed_multi(const void* a_dev, int a_elemsize, size_t a_stride, int M, int K, int count, const int* N,
+                                         const uint8_t* const* packed_w_dev, const float* const* packed_descale_dev, int bits, int block,
+                                         const float* in_scales_dev, const float* const* c_dev, const int* broadcast_type_c, const float* alpha,
+                                         const float* beta, float* const* out_dev, const size_t* out_stride, void* stream)
+{
+    const char* who = "ncnnhip_gemm_blockquant_packed_multi";
+    NCNNHIP_REQUIRE(a_dev && N && packed_w_dev && packed_descale_dev && out_dev && out_stride, "%s: null pointer", who);
+    NCNNHIP_REQUIRE(count >= 1 && count <= BQ_MULTI_MAX, "%s: %d matrices (1 to %d)", who, count, BQ_MULTI_MAX);
+    NCNNHIP_REQUIRE(a_elemsize == 2 || a_elemsize == 4, "%s: activations of %d bytes", who, a_elemsize);
+    NCNNHIP_REQUIRE(a_elemsize == 4 || !in_scales_dev, "%s: input scales come with fp32 activations", who);
+    auto single = [&](int i) -> int {
+        const float* ci = c_dev ? c_dev[i] : 0;
+        return gemm_blockquant_packed(who, a_dev, a_elemsize, a_stride, M, N[i], K, packed_w_dev[i], packed_descale_dev[i], bits, block, in_scales_dev, ci,
+                                      broadcast_type_c ? broadcast_type_c[i] : -1, alpha ? alpha[i] : 1.f, beta ? beta[i] : 1.f, out_dev[i], out_stride[i], stream);
+    };
+    const bool halves = halves_layout(bits, block);
+    bool one_pass = count > 1 && M >= 1 && K >= 1 && K % 16 == 0 && K <= 16384 && M <= (a_elemsize == 2 ? 16 : 4) && (bits == 4 || bits == 6 || bits == 8) &&
+                    (block == 32 || block == 64 || block == 128) && a_stride >= (size_t)K && a_stride % (16 / a_elemsize) == 0 && al16(a_dev) &&
+                    (!in_scales_dev || al16(in_scales_dev));
+    BqMulti mm;
+    mm.count = count;
+    long long tiles = 0;
+    for (int i = 0; i < count && one_pass; i++)
+    {
+        const int bt = (c_dev && c_dev[i]) ? (broadcast_type_c ? broadcast_type_c[i] : -1) : -1;
+        one_pass = packed_w_dev[i] && packed_descale_dev[i] && out_dev[i] && N[i] >= 1 && out_stride[i] >= (size_t)N[i] && bt >= -1 && bt <= 4;
+        tiles += (N[i] + 15) / 16;
+        one_pass = one_pass && tiles < (1ll << 31);
+        mm.tile_end[i] = (int)tiles;
+        mm.N[i] = N[i];
+        mm.bt[i] = bt;
+        mm.alpha[i] = alpha ? alpha[i] : 1.f;
+        mm.beta[i] = beta ? beta[i] : 1.f;
+        mm.wpk[i] = packed_w_dev[i];
+        mm.dpk[i] = reinterpret_cast<const float4*>(packed_descale_dev[i]);
+        mm.c[i] = bt >= 0 ? c_dev[i] : 0;
+        mm.out[i] = out_dev[i];
+        mm.out_stride[i] = out_stride[i];
+    }
+    for (int i = count; i < BQ_MULTI_MAX; i++)
+    {
+        mm.tile_end[i] = (int)tiles, mm.N[i] = 0, mm.bt[i] = -1, mm.alpha[i] = mm.beta[i] = 1.f;
+        mm.wpk[i] = 0, mm.dpk[i] = 0, mm.c[i] = 0, mm.out[i] = 0, mm.out_stride[i] = 0;
+    }
+    if (one_pass)
+    {
+        const int split = block == 32 ? 1 : 0;
+        hipStream_t st = as_stream(stream);
+        bool handled = false;
+        int ret = NCNNHIP_OK;
+        auto up = [&]() -> int {
+#define UPM(BITS_, HALVES_, AIN_, INSC_)                                                                                                                        \
+    return launch_blockquant8_upfront<BITS_, HALVES_, AIN_, INSC_>(a_dev, a_stride, M, N[0], K, mm.wpk[0], mm.dpk[0], split, in_scales_dev, mm.c[0], mm.bt[0], \
+                                                                   mm.alpha[0], mm.beta[0], mm.out[0], mm.out_stride[0], st, &handled, &mm)
+#define UPM_BITS(AIN_, INSC_)                 \
+    if (!halves) UPM(8, false, AIN_, INSC_);  \
+    if (bits == 8) UPM(8, true, AIN_, INSC_); \
+    if (bits == 6) UPM(6, true, AIN_, INSC_); \
+    UPM(4, true, AIN_, INSC_)
+            if (a_elemsize == 2)
+            {
+                UPM_BITS(2, false);
+            }
+            if (in_scales_dev)
+            {
+                UPM_BITS(4, true);
+            }
+            UPM_BITS(4, false);
+#undef UPM_BITS
+#undef UPM
+        };
+        ret = up();
+        if (ret != NCNNHIP_OK) return ret;
+        if (handled) return NCNNHIP_OK;
+    }
+    for (int i = 0; i < count; i++)
+    {
+        const int ret = single(i);
+        if (ret != NCNNHIP_OK) return ret;
+    }
+    return NCNNHIP_OK;
 }
 
 int ncnnhip_gemm_blockquant_f16a(const uint16_t* a_dev, size_t a_stride, int M, int N, int K, const uint8_t* b_dev, int bits,

@@ -146,6 +146,8 @@ _SIGNATURES = {
     "ncnnhip_gemm_blockquant_packed_supported": [C.c_int],
     "ncnnhip_gemm_blockquant_packed": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p],
+    "ncnnhip_gemm_blockquant_packed_multi": [C.c_void_p, C.c_int, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p],
     "ncnnhip_gemm_blockquant_packed_rows_workspace_bytes": [C.c_int, C.c_int, C.POINTER(C.c_size_t)],
     "ncnnhip_gemm_blockquant_packed_rows": [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                             C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
@@ -735,6 +737,30 @@ class Runtime:
         pd = np.empty(db.value // 4, np.float32)
         check(lib().ncnnhip_blockquant_pack(b_packed.ctypes.data, scales.ctypes.data, n, k, bits, block, pw.ctypes.data, pd.ctypes.data))
         return pw, pd
+
+    def blockquant_multi_args(self, mats, douts):
+        """ctypes argument arrays of ncnnhip_gemm_blockquant_packed_multi for device-resident matrices:
+        mats = [(dev packed weights, dev descales, n, dev c or None, broadcast type, alpha, beta)], douts = output buffers."""
+        k = len(mats)
+        PtrArr, IntArr, FloatArr, SizeArr = C.c_void_p * k, C.c_int * k, C.c_float * k, C.c_size_t * k
+        return (IntArr(*[m[2] for m in mats]), PtrArr(*[m[0].ptr.value for m in mats]), PtrArr(*[m[1].ptr.value for m in mats]),
+                PtrArr(*[(m[3].ptr.value if m[3] is not None else None) for m in mats]), IntArr(*[(m[4] if m[3] is not None else -1) for m in mats]),
+                FloatArr(*[m[5] for m in mats]), FloatArr(*[m[6] for m in mats]), PtrArr(*[d.ptr.value for d in douts]), SizeArr(*[m[2] for m in mats]))
+
+    def gemm_blockquant_packed_multi(self, a, mats, bits=8, block=64, in_scales=None):
+        """Several packed matrices on the same activation rows in one launch.  mats = [(pw, pd, n, c or None, broadcast type, alpha, beta)];
+        a fp16 or fp32.  Returns the list of outputs."""
+        half = a.dtype == np.float16
+        a = np.ascontiguousarray(a, np.float16 if half else np.float32)
+        m, k = a.shape
+        da = self.up(a)
+        dis = self.up(None if in_scales is None else np.asarray(in_scales, np.float32))
+        dev = [(self.up(pw), self.up(pd), n, self.up(None if c is None else np.asarray(c, np.float32)), bt, alpha, beta) for pw, pd, n, c, bt, alpha, beta in mats]
+        douts = [DeviceBuffer.empty((m, mt[2]), np.float32) for mt in mats]
+        ns, ws, ds, cs, bts, als, bes, outs, strides = self.blockquant_multi_args(dev, douts)
+        check(lib().ncnnhip_gemm_blockquant_packed_multi(da.ptr, 2 if half else 4, k, m, k, len(mats), ns, ws, ds, bits, block, _ptr(dis), cs, bts, als, bes, outs, strides,
+                                                         self.stream))
+        return [d.to_numpy(self.stream) for d in douts]
 
     def gemm_blockquant_packed(self, a, pw, pd, n, c=None, broadcast_type_c=-1, alpha=1.0, beta=1.0, bits=8, block=64, in_scales=None, rows_kernel=False):
         """a fp16: the fp16-activation entry point; a fp32 (optionally with in_scales): the layer's contract, activations split into three bf16

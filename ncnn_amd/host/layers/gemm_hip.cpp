@@ -320,6 +320,69 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
     return to_ncnn_status(rc, "ncnnhip_gemm_int8");
 }
 
+// Layers with equal keys may share a launch: block-quantised constant B in the packed form, the plain network form
+// (one dynamic A, no transposes, fp32 out), no per-layer input scales (the shared launch has one activation operand),
+// and the same K and field format.  0: this layer runs on its own.
+unsigned long long Gemm_hip::hip_sibling_key() const
+{
+    if (!weight_block_quantize || !d_B_packed || !d_B_packed_descales || d_B_input_scales) return 0;
+    if (constantA != 0 || constantB != 1 || transA != 0 || output_transpose != 0 || output_N1M != 0) return 0;
+    if (constantC && !C_data.empty() && constant_broadcast_type_C >= 0 && constant_broadcast_type_C != 0 && constant_broadcast_type_C != 4) return 0; // per-row C: not with a batch
+    if (!ncnnhip_gemm_blockquant_packed_supported(constantK)) return 0;
+    return 1ull | ((unsigned long long)constantK << 1) | ((unsigned long long)term_bits(quantize_term) << 33) | ((unsigned long long)term_block(quantize_term) << 41);
+}
+
+// Every member's forward_hip on the one bottom, in one launch of ncnnhip_gemm_blockquant_packed_multi: bit for bit what
+// the members give one by one (the same kernel; a workgroup only finds its matrix differently).  Up to four activation
+// rows (the one-pass form of fp32 activations) and eight members; anything else: done = false, the layers run on their own.
+int Gemm_hip::forward_hip_siblings(const std::vector<const Layer*>& group, const HipMat& A, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option&,
+                                   bool& done) const
+{
+    done = false;
+    if (group.size() < 2 || group.size() > 8 || top_blobs.size() != group.size()) return 0;
+    if (A.elemsize != 4u || (A.dims != 1 && A.dims != 2)) return 0;
+    const int M = A.dims == 2 ? A.n * A.h : A.n, K = A.w;
+    if (M > 4 || K != constantK) return 0;
+    const unsigned long long key = hip_sibling_key();
+    if (!key) return 0;
+    int n[8], bt[8];
+    const uint8_t* w[8];
+    const float* d[8];
+    const float* c[8];
+    float al[8], be[8];
+    float* out[8];
+    size_t stride[8];
+    for (size_t i = 0; i < group.size(); i++)
+    {
+        const Gemm_hip* g = static_cast<const Gemm_hip*>(group[i]); // equal keys: the executor only groups layers of this class
+        if (g->hip_sibling_key() != key) return 0;
+        n[i] = g->constantN;
+        w[i] = (const uint8_t*)g->d_B_packed;
+        d[i] = (const float*)g->d_B_packed_descales;
+        const bool has_c = g->constantC && !g->C_data.empty() && g->constant_broadcast_type_C >= 0;
+        c[i] = has_c ? (const float*)g->d_C : 0;
+        bt[i] = has_c ? g->constant_broadcast_type_C : -1;
+        al[i] = g->alpha;
+        be[i] = g->beta;
+    }
+    for (size_t i = 0; i < group.size(); i++)
+    {
+        HipMat& top = top_blobs[i];
+        if (A.dims == 2)
+            top.create(n[i], A.h, 4u, A.n, &cmd);
+        else
+            top.create(n[i], 4u, A.n, &cmd);
+        if (top.empty()) return -100;
+        out[i] = (float*)top.data;
+        stride[i] = (size_t)n[i];
+    }
+    const int rc = ncnnhip_gemm_blockquant_packed_multi(A.data, 4, (size_t)K, M, K, (int)group.size(), n, w, d, term_bits(quantize_term), term_block(quantize_term), 0, c,
+                                                        bt, al, be, out, stride, cmd.stream);
+    if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_blockquant_packed_multi");
+    done = true;
+    return 0;
+}
+
 // rows / row stride of a matrix held in a Mat: 2-D (h rows of w) or 3-D with h == 1 (c rows, cstep apart)
 static int mat_rows(const Mat& m)
 {

@@ -106,6 +106,10 @@ public:
     virtual int forward_hip(const std::vector<ncnn::HipMat>& bottom_blobs, std::vector<ncnn::HipMat>& top_blobs, ncnn::HipCommand& cmd,
                             const ncnn::Option& opt) const;
     virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
+    // block-quantised Gemms on the same activation rows (gate + up of a decoder layer behind one Split) as one launch
+    virtual unsigned long long hip_sibling_key() const;
+    virtual int forward_hip_siblings(const std::vector<const ncnn::Layer*>& group, const ncnn::HipMat& bottom_blob, std::vector<ncnn::HipMat>& top_blobs,
+                                     ncnn::HipCommand& cmd, const ncnn::Option& opt, bool& done) const;
 
 public:
     float alpha, beta;

@@ -104,6 +104,15 @@ bool Layer::hip_can_fuse_tail() const
 {
     return false;
 }
+unsigned long long Layer::hip_sibling_key() const
+{
+    return 0;
+}
+int Layer::forward_hip_siblings(const std::vector<const Layer*>&, const HipMat&, std::vector<HipMat>&, HipCommand&, const Option&, bool& done) const
+{
+    done = false;
+    return 0;
+}
 int Layer::forward_hip_fused(const HipMat&, const HipMat*, bool, float, HipMat&, HipCommand&, const Option&) const
 {
     return -1;

@@ -69,6 +69,13 @@ public:
     // forward_hip_requantised(bottom, scale) gives the int8 blob float2int8(forward(bottom) * scale).
     virtual int hip_prepare_requantise(float scale);
     virtual int forward_hip_requantised(const HipMat& bottom_blob, float scale, HipMat& top_blob, HipCommand& cmd, const Option& opt) const;
+    // Sibling layers that read the same blob (through a Split) and can run as ONE launch: a layer that can take part
+    // describes itself with a key (layers with equal non-zero keys may share a launch); forward_hip_siblings is called on
+    // the first layer of such a group with the whole group (itself included, all of its own class) and the one bottom,
+    // and fills one top per layer, each identical to what that layer's forward_hip gives on its own.
+    virtual unsigned long long hip_sibling_key() const;
+    virtual int forward_hip_siblings(const std::vector<const Layer*>& group, const HipMat& bottom_blob, std::vector<HipMat>& top_blobs, HipCommand& cmd,
+                                     const Option& opt, bool& done) const;
     // takes a narrow fp32 image (HipMat::narrow) as it is; everyone else gets it widened to the ordinary layout first
     virtual bool hip_accepts_narrow_input() const;
     // forward_hip of an int8 blob holding Quantize(x, s), s > 0, gives Quantize(forward_hip(x), s) (windowed max pooling)

@@ -1,5 +1,7 @@
 #include "net.h"
 
+#include <algorithm>
+
 #include <stdint.h>
 #include <string.h>
 
@@ -186,6 +188,10 @@ public:
         bool relu;
     };
     std::vector<TailPlan> tail_plan;
+    // sibling_group[L]: the layers (L among them, in layer order) that read outputs of one Split, have equal sibling keys and
+    // may therefore run as one launch; empty: none
+    std::vector<std::vector<int> > sibling_group;
+    int try_siblings(int layer_index, ExecState& st, const Option& opt, bool& done) const;
     std::vector<float> quantise_scale;
     // requant_scale[b] != 0: blob b is produced as int8, float2int8(value * scale), by its layer (a convolution
     // that agreed in hip_prepare_requantise): every consumer, through Split and windowed max pooling, quantises with
@@ -329,6 +335,80 @@ void NetPrivate::build_fusion_plan()
             tail_plan[(size_t)ri] = tp;
         }
     }
+    // layers behind one Split that can share a launch (block-quantised Gemms on the same activation rows)
+    sibling_group.assign(layers.size(), std::vector<int>());
+    for (size_t li = 0; li < layers.size(); li++)
+    {
+        const Layer* sp = layers[li];
+        if (sp->type != "Split" || sp->tops.size() < 2) continue;
+        std::vector<int> members;
+        unsigned long long key = 0;
+        for (size_t t = 0; t < sp->tops.size(); t++)
+        {
+            const int ci = blobs[(size_t)sp->tops[t]].consumer;
+            if (ci < 0) continue;
+            const Layer* c = layers[(size_t)ci];
+            if (!c->support_hip || c->featmask || c->bottoms.size() != 1 || c->tops.size() != 1) continue;
+            const unsigned long long k = c->hip_sibling_key();
+            if (!k) continue;
+            if (members.empty()) key = k;
+            if (k == key) members.push_back(ci);
+        }
+        if (members.size() < 2) continue;
+        std::sort(members.begin(), members.end());
+        for (size_t m = 0; m < members.size(); m++) sibling_group[(size_t)members[m]] = members;
+    }
+}
+
+// Runs layer_index together with its siblings that have not run yet, as one launch, when their (shared) input is there.
+// done = false: not applicable, the caller runs the layer on its own.
+int NetPrivate::try_siblings(int layer_index, ExecState& st, const Option& opt, bool& done) const
+{
+    done = false;
+    if (!opt.use_hip_compute || sibling_group.size() != layers.size()) return 0;
+    const std::vector<int>& group = sibling_group[(size_t)layer_index];
+    if (group.size() < 2) return 0;
+    // the members whose output is still missing and whose input exists (all outputs of one Split: the same blob)
+    std::vector<const Layer*> run;
+    for (size_t m = 0; m < group.size(); m++)
+    {
+        const Layer* l = layers[(size_t)group[m]];
+        if (!st.has(l->tops[0]) && st.has(l->bottoms[0])) run.push_back(l);
+    }
+    if (run.size() < 2) return 0;
+    const Layer* self = layers[(size_t)layer_index];
+    if (std::find(run.begin(), run.end(), self) == run.end()) return 0;
+    if (!st.cmd) st.cmd = acquire_command();
+    HipCommand& cmd = *st.cmd;
+    int ret = cmd.ensure_ready();
+    if (ret != 0) return ret;
+    const size_t b0 = (size_t)run[0]->bottoms[0];
+    if (st.dev[b0].empty())
+    {
+        ret = cmd.upload(st.host[b0], st.dev[b0]);
+        if (ret != 0) return ret;
+    }
+    const HipMat bottom = st.dev[b0];
+    // the members' inputs must be the very same device blob (a Split hands one blob to all its outputs)
+    for (size_t m = 1; m < run.size(); m++)
+    {
+        const size_t bi = (size_t)run[m]->bottoms[0];
+        if (st.dev[bi].empty() || st.dev[bi].data != bottom.data) return 0;
+    }
+    std::vector<HipMat> tops(run.size());
+    ret = run[0]->forward_hip_siblings(run, bottom, tops, cmd, opt, done);
+    if (ret != 0 || !done) return ret;
+    for (size_t m = 0; m < run.size(); m++)
+    {
+        st.dev[(size_t)run[m]->tops[0]] = tops[m];
+        st.host[(size_t)run[m]->tops[0]].release();
+        if (opt.lightmode)
+        {
+            st.dev[(size_t)run[m]->bottoms[0]].release();
+            st.host[(size_t)run[m]->bottoms[0]].release();
+        }
+    }
+    return 0;
 }
 
 // Runs layer_index (a sum, or the ReLU after it) as the epilogue of the convolution in its plan, if nothing on the
@@ -456,6 +536,13 @@ int NetPrivate::forward_layer(int layer_index, ExecState& st, const Option& opt)
     }
     const Option lopt = layer->featmask ? masked_option(opt, layer->featmask) : opt;
     const bool on_device = lopt.use_hip_compute && layer->support_hip;
+    if (on_device && !st.time_layers)
+    {
+        // siblings behind one Split that can share a launch (timed runs keep one record per layer and take the plain route)
+        bool together = false;
+        int ret = try_siblings(layer_index, st, lopt, together);
+        if (ret != 0 || together) return ret;
+    }
     if (!st.time_layers) return on_device ? run_layer_hip(layer, st, lopt) : run_layer(layer, st, lopt);
 
     LayerTimingSlot slot = {layer_index, 0, 0, 0.0};
@@ -1060,6 +1147,7 @@ void Net::clear()
     d->input_nm.clear();
     d->output_nm.clear();
     d->tail_plan.clear();
+    d->sibling_group.clear();
     d->quantise_scale.clear();
     d->requant_scale.clear();
     d->quantised_zone.clear();

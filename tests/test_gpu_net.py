@@ -372,6 +372,45 @@ def test_gemm_layer_block_quant(bits, block, insc, m, n, k, resident):
     assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
 
 
+@pytest.mark.parametrize("m", [1, 4, 9])
+def test_sibling_block_quant_gemms_behind_a_split_share_one_launch(m):
+    """The gate / up pair of a decoder layer: block-quantised Gemm layers that read the outputs of one Split run as ONE launch
+    on device-resident blobs (up to four activation rows), and every output is bit for bit what the layer gives in a net of
+    its own; a sibling with per-layer input scales, and every sibling at nine rows, keeps its own launch.  The reference runs
+    the layers one after the other (src/net.cpp:625-700 for the executor, src/layer/gemm.cpp:425-483 for each)."""
+    import npref
+    rng = np.random.default_rng(m)
+    k, bits, block = 512, 8, 64
+    a = rng.standard_normal((m, k), dtype=F)
+    specs = [("gate", 176, False, False), ("up", 100, True, False), ("third", 48, False, True)]  # name, N, constant C per column, input scales
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m), "Split sp 1 3 a a_g a_u a_t"]
+    blob, parts = b"", {}
+    for name, n, with_c, insc in specs:
+        w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+        packed, scales = oracle.blockquant_pack(w, bits, block)
+        c = rng.standard_normal((1, n), dtype=F) if with_c else None
+        ins = (0.75 + (np.arange(k) % 5) * 0.15).astype(F) if insc else None
+        term = bits * 100 + (10 if insc else 0) + 1
+        kw = dict(N=n, K=k, constantB=1, quantize_term=term, alpha=0.5 if with_c else 1.0)
+        if with_c:
+            kw.update(constantC=1, broadcast_type_C=4)
+        line = mw.gemm_param(name, ["a_" + name[0]], name + "_out", **kw)
+        piece = mw.weight_blob(packed.view(np.int8)) + (mw.weight_blob(c) if with_c else b"") + mw.raw_f32(scales) + (mw.raw_f32(ins) if insc else b"")
+        lines.append(line)
+        blob += piece
+        parts[name] = (line.replace("a_" + name[0], "a"), piece, packed, scales, c, ins, kw.get("alpha", 1.0))
+    net = _load(mw.assemble_param(lines), blob, True)
+    ex = net.create_extractor()
+    ex.input("a", a)
+    got = {name: ex.extract(name + "_out") for name, _, _, _ in specs}
+    for name, n, with_c, insc in specs:
+        line, piece, packed, scales, c, ins, alpha = parts[name]
+        alone = _single(["Input in0 0 1 a 0=%d 1=%d" % (k, m), line], piece, {"a": a}, name + "_out", True)
+        assert np.array_equal(got[name], alone), name
+        val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins, c, 4 if with_c else -1, alpha, 1.0)
+        assert np.all(np.abs(got[name] - val) <= 1e-5 * floor + 1e-30), name
+
+
 @RESIDENT
 @pytest.mark.parametrize("spec", cases.MHA_CASES, ids=[str(c[0]) for c in cases.MHA_CASES])
 def test_multiheadattention_layer_block_quant(spec, resident):

@@ -579,6 +579,42 @@ def test_blockquant_packed_fp32_activations(rt, bits, block, m, n, k, bt, in_sc)
     _bq_check(got, a, packed, scales, bits, block, ins, c, bt, 0.75, 1.5)
 
 
+@pytest.mark.parametrize("act,bits,block,m,k,ns,in_sc", [
+    # the decode shapes' siblings: gate + up, q + k + v; fp16 and fp32 activations; every layout; ragged N; one matrix; eight
+    ("fp16", 8, 64, 1, 4096, (176, 160), False), ("fp16", 8, 64, 16, 1024, (64, 100, 37), False), ("fp16", 4, 32, 4, 2048 + 16, (48, 16, 250), False),
+    ("fp16", 6, 128, 7, 512, (33,), False), ("fp32", 8, 64, 1, 4096, (176, 160), False), ("fp32", 8, 64, 4, 4096, (40, 256, 100), True),
+    ("fp32", 4, 64, 2, 1024, (16,) * 8, True), ("fp32", 6, 32, 3, 256, (300, 20), False),
+    # shapes the one-pass kernel does not take: matrix by matrix behind the same call
+    ("fp16", 8, 64, 20, 1024, (64, 48), False), ("fp32", 8, 64, 4, 8192, (32, 48), False)])
+def test_blockquant_packed_multi_equals_the_single_calls_and_the_oracle(rt, act, bits, block, m, k, ns, in_sc):
+    """Several weight matrices on the same activation rows in one launch: each output is bit for bit what the single-matrix entry
+    gives (same kernel, same order of additions; the workgroup only finds its matrix differently), and within the usual bound of the
+    oracle's Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:425-483) per matrix -- with a different C, alpha and beta each."""
+    _say("blockquant multi", act, bits, block, m, k, ns, in_sc)
+    from ncnn_amd import synth
+    rng = np.random.default_rng(len(ns) + m + k)
+    a = None
+    mats, refs = [], []
+    for i, n in enumerate(ns):
+        ai, packed, scales = synth.blockquant_operands(bits + block + m + n + k + i, m, n, k, bits, block, half_exact=(act == "fp16"))
+        a = ai if a is None else a
+        bt = (-1, 4, 0, 3, 1, 2)[i % 6]
+        c = {-1: None, 0: rng.normal(size=1), 1: rng.normal(size=m), 2: rng.normal(size=(m, 1)), 3: rng.normal(size=(m, n)), 4: rng.normal(size=(1, n))}[bt]
+        c = None if c is None else c.astype(F)
+        alpha, beta = float(F(0.5 + 0.25 * i)), float(F(1.5 - 0.125 * i))
+        pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
+        mats.append((pw, pd, n, c, bt, alpha, beta))
+        refs.append((packed, scales, c, bt, alpha, beta))
+    ins = rng.uniform(0.5, 1.5, k).astype(F) if in_sc else None
+    x = a.astype(np.float16) if act == "fp16" else a
+    got = rt.gemm_blockquant_packed_multi(x, mats, bits=bits, block=block, in_scales=ins)
+    for i, (pw, pd, n, c, bt, alpha, beta) in enumerate(mats):
+        single = rt.gemm_blockquant_packed(x, pw, pd, n, c, bt, alpha, beta, bits=bits, block=block, in_scales=ins)
+        assert np.array_equal(got[i], single), "matrix %d differs from the single-matrix call" % i
+        packed, scales = refs[i][0], refs[i][1]
+        _bq_check(got[i], a, packed, scales, bits, block, ins, c, bt, alpha, beta)
+
+
 @pytest.mark.parametrize("bits,block,m,n,k,bt,in_sc", [
     # the tiled form for many rows: ragged in rows (64), weight rows (128 per workgroup, 16 per tile) and K (64); every layout; C broadcasts; input scales
     (8, 64, 64, 128, 64, -1, False), (8, 64, 70, 100, 256, 4, True), (8, 32, 129, 65, 96, 3, False), (8, 128, 64, 31, 1024, 1, True), (8, 64, 200, 130, 2048, 0, False),
