@@ -80,9 +80,31 @@ def build_host(sanitize=False):
     return out
 
 
+LIBPLUGIN = os.path.join(LIBDIR, "libncnnhip_plugin.so")
+
+
+def build_plugin(c_api_include=None):
+    """libncnnhip_plugin.so from plugin/ncnnhip_plugin.c: the four int8 layers written against ncnn's public C API only.
+    Without arguments it is compiled against this repository's copy of that API and linked to libncnn_amd.so (what the tests
+    load); with c_api_include = the directories that hold an ncnn build's c_api.h, platform.h and ncnn_export.h it is compiled
+    against those and left to resolve the ncnn_* symbols from the libncnn the host program links."""
+    src = os.path.join(ROOT, "plugin", "ncnnhip_plugin.c")
+    cmd = ["gcc", "-std=c99", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", "-fno-fast-math", "-ffp-contract=off", "-Wall", "-Wextra",
+           "-I", os.path.join(ROOT, "include")]
+    if c_api_include:
+        cmd += [x for d in c_api_include for x in ("-I", d)]
+        cmd += [src, "-o", LIBPLUGIN, "-L", LIBDIR, "-lncnnhip", "-lm", "-lpthread", "-Wl,-rpath,$ORIGIN"]
+    else:
+        cmd += ["-DNCNNHIP_PLUGIN_AGAINST_NCNN_AMD", src, "-o", LIBPLUGIN, "-L", LIBDIR, "-lncnn_amd", "-lncnnhip", "-lm", "-lpthread",
+                "-Wl,-rpath,$ORIGIN"]
+    _run(cmd)
+    return LIBPLUGIN
+
+
 def build_all():
     build_kernels()
     build_host()
+    build_plugin()
 
 
 if __name__ == "__main__":

@@ -76,6 +76,8 @@ def lib():
             "ncnn_mat_create_external_1d_elem": (vp, [ci, vp, cs, ci, vp]), "ncnn_mat_create_external_2d_elem": (vp, [ci, ci, vp, cs, ci, vp]),
             "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, ci, vp]),
             "ncnn_mat_create_3d_elem_batch": (vp, [ci, ci, ci, cs, ci, ci, vp]),
+            "ncnn_mat_create": (vp, []), "ncnn_mat_create_1d_elem": (vp, [ci, cs, ci, vp]), "ncnn_mat_create_2d_elem": (vp, [ci, ci, cs, ci, vp]),
+            "ncnn_mat_create_3d_elem": (vp, [ci, ci, ci, cs, ci, vp]),
             "ncnn_mat_destroy": (None, [vp]), "ncnn_mat_get_dims": (ci, [vp]), "ncnn_mat_get_w": (ci, [vp]), "ncnn_mat_get_h": (ci, [vp]),
             "ncnn_mat_get_d": (ci, [vp]), "ncnn_mat_get_c": (ci, [vp]), "ncnn_mat_get_n": (ci, [vp]), "ncnn_mat_get_elemsize": (cs, [vp]),
             "ncnn_mat_get_elempack": (ci, [vp]), "ncnn_mat_get_cstep": (cs, [vp]), "ncnn_mat_get_nstep": (cs, [vp]),

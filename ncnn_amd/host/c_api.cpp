@@ -171,6 +171,28 @@ ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, siz
     m->elempack = elempack;
     return (ncnn_mat_t)m;
 }
+ncnn_mat_t ncnn_mat_create(void)
+{
+    return (ncnn_mat_t)(new Mat);
+}
+ncnn_mat_t ncnn_mat_create_1d_elem(int w, size_t elemsize, int elempack, ncnn_allocator_t allocator)
+{
+    Mat* m = new Mat;
+    m->create(w, elemsize, elempack, A(allocator));
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_2d_elem(int w, int h, size_t elemsize, int elempack, ncnn_allocator_t allocator)
+{
+    Mat* m = new Mat;
+    m->create(w, h, elemsize, elempack, A(allocator));
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_3d_elem(int w, int h, int c, size_t elemsize, int elempack, ncnn_allocator_t allocator)
+{
+    Mat* m = new Mat;
+    m->create(w, h, c, elemsize, elempack, A(allocator));
+    return (ncnn_mat_t)m;
+}
 ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, int n, ncnn_allocator_t allocator)
 {
     Mat* m = new Mat;

@@ -62,7 +62,12 @@ private:
 class Layer_c_api : public Layer
 {
 public:
-    explicit Layer_c_api(ncnn_layer_t _layer) : Layer(), layer(_layer) {}
+    explicit Layer_c_api(ncnn_layer_t _layer) : Layer(), layer(_layer)
+    {
+        // the reference's executor hands a layer an int8 blob as it is (convert_layout, src/net.cpp:344-600, has no int8 cast):
+        // a layer behind the table sees here what it would see there
+        support_int8_storage = true;
+    }
 
     virtual int load_param(const ParamDict& pd)
     {
