@@ -101,7 +101,7 @@ typedef struct plugin_state
     int b_ready_int8;
 } plugin_state;
 
-/* ncnn_layer_create() owns the table and its pthis (src/c_api.cpp:1234-1252), so a layer's own state lives beside it, found
+/* ncnn_layer_create() owns the table and its pthis (src/c_api.cpp:1352-1365), so a layer's own state lives beside it, found
  * by the table's address */
 static plugin_state* g_states = 0;
 static pthread_mutex_t g_states_lock = PTHREAD_MUTEX_INITIALIZER;
@@ -1292,7 +1292,7 @@ static void destroyer(ncnn_layer_t layer, void* userdata)
     (void)userdata;
     if (s)
     {
-        /* Net::clear calls destroy_pipeline before the destroyer (src/net.cpp:1378-1410); a layer dropped before that still
+        /* Net::clear calls destroy_pipeline before the destroyer (src/net.cpp:2419-2460); a layer dropped before that still
          * holds its device memory, so the call is repeated here (it is idempotent) */
         if (s->kind == KIND_GEMM)
             gemm_destroy_pipeline(layer, 0);
