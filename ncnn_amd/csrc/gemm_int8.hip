@@ -161,6 +161,8 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
                                const GemmEpilogue& epi, hipStream_t stream, bool* handled);
 
 int launch_gemm_int8_tiled(const int8_t* aq_tiled, const int8_t* bq_tiled, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream);
+int launch_gemm_int8_ring128(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmEpilogue& epi,
+                             hipStream_t stream, bool* handled);
 int launch_gemm_tile_operand(const int8_t* src, size_t stride, int rows, int K, int operand_b, int8_t* dst, hipStream_t stream);
 
 // the shapes the few-row kernel takes for InnerProduct (operands aligned): no workspace, no hand-off between workgroups
@@ -244,6 +246,13 @@ int ncnnhip_gemm_int8(const int8_t* aq_dev, size_t aq_stride, const int8_t* bq_d
     if ((long long)M * N >= 256ll * 256 * 128)
     {
         ret = launch_gemm_int8_pipelined(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, epi, as_stream(stream), &handled);
+        if (handled) return ret;
+    }
+    // too few 256x256 tiles for that: the same ring on 128x128 tiles, from 48 of them up (below, the 64-row tiles of the convolution
+    // kernel spread the work over more CUs)
+    if ((long long)(M / 128) * (N / 128) >= 48)
+    {
+        ret = launch_gemm_int8_ring128(aq_dev, aq_stride, bq_dev, bq_stride, M, N, K, epi, as_stream(stream), &handled);
         if (handled) return ret;
     }
     // anything else with K % 64 == 0: the convolution's pipelined kernel run as a 1x1 convolution over the rows of A

@@ -22,6 +22,7 @@
 //
 // Workgroup ids are remapped so that each of the 8 XCDs (ids are dealt round-robin to XCDs)
 // works on a compact block of output tiles and re-uses its A/B panels out of its own L2.
+#include <cstdlib>
 #include <type_traits>
 
 #include "epilogues.h"
@@ -281,6 +282,216 @@ __global__ __launch_bounds__(256) void gemm_int8_256x256_kernel(const int8_t* __
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// The same ring with a 128x128 output tile, for problems that have too few 256x256 tiles to fill 256 CUs (1024 cubed is
+// 16 of them, 2048 cubed 64).  Four wavefronts own 64x64 quadrants (2x2 blocks, 64 accumulators per lane); a stage is 128 A
+// rows and 128 B rows of 64 bytes (16 KB), S stages deep.  A wavefront issues 4 direct-to-LDS loads, 8 LDS reads and 8 MFMA
+// per K step; the loads of step t + S and the reads of step t + 1 are dealt out between the MFMAs of step t as above.  Per
+// output the tile reads twice the operand bytes of the 256x256 tile, which is what it costs to have four times the tiles.
+constexpr int QT = 128;
+constexpr int Q_OPERAND = QT * PK;     // 8 KB
+constexpr int Q_STAGE = 2 * Q_OPERAND; // 16 KB
+
+template<bool PER_COL, int BT, int S>
+__global__ __launch_bounds__(256) void gemm_int8_128x128_kernel(const int8_t* __restrict__ A, size_t lda, const int8_t* __restrict__ B, size_t ldb, int nk,
+                                                                 int tiles_m, int tiles_n, const float* __restrict__ a_scales,
+                                                                 const float* __restrict__ b_scales, const float* __restrict__ cvec, float alpha, float beta,
+                                                                 float* __restrict__ out, size_t ldo)
+{
+    static_assert(S == 4 || S == 8, "the ring is indexed with a mask");
+    __shared__ __attribute__((aligned(1024))) int8_t smem[S * Q_STAGE];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    // XCD-aware tile choice, as in the 256x256 kernel
+    int b = blockIdx.x;
+    const int T = tiles_m * tiles_n;
+    if ((T & 7) == 0) b = (b & 7) * (T >> 3) + (b >> 3);
+    constexpr int GM = 4;
+    const int per_group = GM * tiles_n;
+    const int group = b / per_group;
+    const int first_m = group * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int in_group = b - group * per_group;
+    const int tile_m = first_m + in_group % gsz;
+    const int tile_n = in_group / gsz;
+
+    // load i (0, 1) of wave w fills LDS rows i*64 + w*16 .. +16 of an operand stage; chunks swizzled as in the 256x256 kernel
+    const int ld_row = wave * 16 + (lane >> 2);
+    const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int8_t* ga = A + ((size_t)tile_m * QT + ld_row) * lda + ld_chunk * 16;
+    // LDS row wn*64 + j*32 + l holds B row wn*64 + 2*l + j: the two accumulator blocks j of a lane are two consecutive output
+    // columns (8-byte stores).  LDS row of this lane in half i = i*64 + wave*16 + (lane >> 2): wn = i, j = wave >> 1,
+    // l = (wave & 1)*16 + (lane >> 2).
+    const int ld_row_b = 2 * ((wave & 1) * 16 + (lane >> 2)) + (wave >> 1);
+    const int8_t* gb = B + ((size_t)tile_n * QT + ld_row_b) * ldb + ld_chunk * 16;
+    const size_t a_half = 64 * lda, b_half = 64 * ldb;
+
+    auto issue_one = [&](int t, int i, int which) {
+        int8_t* sa = smem + (t & (S - 1)) * Q_STAGE + wave * 1024 + i * 4096;
+        if (which == 0)
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(ga + (size_t)t * PK + i * a_half), (AS3 void*)sa, 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(gb + (size_t)t * PK + i * b_half), (AS3 void*)(sa + Q_OPERAND), 16, 0, 0);
+    };
+    auto issue_stage = [&](int t) {
+        issue_one(t, 0, 0);
+        issue_one(t, 0, 1);
+        issue_one(t, 1, 0);
+        issue_one(t, 1, 1);
+    };
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // what the epilogue needs from memory is requested now, so that it has arrived long before the K loop ends
+    const int col_base = tile_n * QT + wn * 64 + 2 * l32; // accumulator block j of this lane is column col_base + j
+    // (as asm: these loads must stand before the direct-to-LDS loads, whose waits count instructions; EARLY_ARRIVED below ties
+    // the values to a point behind the K loop, where every load of the wavefront has returned)
+    float early_sa, early_sb[2] = {0.f, 0.f}, early_c[2] = {0.f, 0.f};
+#define EARLY_LOAD(dst, ptr) asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory")
+    EARLY_LOAD(early_sa, a_scales + tile_m * QT + (threadIdx.x & (QT - 1)));
+    EARLY_LOAD(early_sb[0], b_scales + (PER_COL ? col_base : 0));
+    if (PER_COL) EARLY_LOAD(early_sb[1], b_scales + col_base + 1);
+    if (BT == 4)
+    {
+        EARLY_LOAD(early_c[0], cvec + col_base);
+        EARLY_LOAD(early_c[1], cvec + col_base + 1);
+    }
+#undef EARLY_LOAD
+#define EARLY_ARRIVED asm volatile("s_waitcnt vmcnt(0)" : "+v"(early_sa), "+v"(early_sb[0]), "+v"(early_sb[1]), "+v"(early_c[0]), "+v"(early_c[1]))
+    PIN;
+
+    const int sw = (l32 >> 2) & 3;
+    const int rd_a0 = (wm * 64 + l32) * PK + ((0 + lhi) ^ sw) * 16;
+    const int rd_a1 = (wm * 64 + l32) * PK + ((2 + lhi) ^ sw) * 16;
+    const int rd_b0 = Q_OPERAND + (wn * 64 + l32) * PK + ((0 + lhi) ^ sw) * 16;
+    const int rd_b1 = Q_OPERAND + (wn * 64 + l32) * PK + ((2 + lhi) ^ sw) * 16;
+    const unsigned lds_base = (unsigned)(uintptr_t)(AS3 int8_t*)smem;
+    auto frag_addr_a = [&](int t, int ks) { return lds_base + (unsigned)((t & (S - 1)) * Q_STAGE) + (ks ? rd_a1 : rd_a0); };
+    auto frag_addr_b = [&](int t, int ks) { return lds_base + (unsigned)((t & (S - 1)) * Q_STAGE) + (ks ? rd_b1 : rd_b0); };
+
+    // at most `newer` stages (4 loads each) may stay in flight
+    auto wait_stages = [&](int newer) {
+        switch (newer)
+        {
+        case 0: WAIT_VMCNT(0); break;
+        case 1: WAIT_VMCNT(4); break;
+        case 2: WAIT_VMCNT(8); break;
+        case 3: WAIT_VMCNT(12); break;
+        case 4: WAIT_VMCNT(16); break;
+        case 5: WAIT_VMCNT(20); break;
+        default: WAIT_VMCNT(24); break;
+        }
+    };
+
+    // ---- prologue: the whole ring in flight
+#pragma unroll
+    for (int t0 = 0; t0 < S; t0++)
+        if (t0 < nk) issue_stage(t0);
+    {
+        const int newer = nk - 1 < S - 1 ? nk - 1 : S - 1;
+        if (newer == S - 1)
+            WAIT_VMCNT((S - 1) * 4);
+        else
+            wait_stages(newer);
+    }
+    __builtin_amdgcn_s_barrier();
+
+    v4i fa0[2], fb0[2], fa1[2], fb1[2];
+    {
+        const unsigned pa = frag_addr_a(0, 0), pb = frag_addr_b(0, 0);
+        LDS_READ(fa0[0], pa, 0);
+        LDS_READ(fb0[0], pb, 0);
+        LDS_READ(fb0[1], pb, 2048);
+        LDS_READ(fa0[1], pa, 2048);
+    }
+    auto mma1 = [&](int i, int j, const v4i (&fa)[2], const v4i (&fb)[2]) {
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    auto k_step = [&](int t, auto steady) {
+        constexpr bool STEADY = decltype(steady)::value;
+        const bool more = STEADY || t + 1 < nk;
+        const bool refill = STEADY || t + S < nk;
+        const unsigned qa = frag_addr_a(t, 1), qb = frag_addr_b(t, 1);
+        // first set: requested in the order fa0[0], fb0[0], fb0[1], fa0[1]
+        WAIT_LGKM(1, "+v"(fa0[0]), "+v"(fb0[0]), "+v"(fb0[1]));
+        PIN;
+        mma1(0, 0, fa0, fb0); PIN; LDS_READ(fa1[0], qa, 0); PIN;
+        mma1(0, 1, fa0, fb0); PIN; LDS_READ(fb1[0], qb, 0); PIN;
+        WAIT_LGKM(2, "+v"(fa0[1]));
+        PIN;
+        mma1(1, 0, fa0, fb0); PIN; LDS_READ(fb1[1], qb, 2048); PIN;
+        mma1(1, 1, fa0, fb0); PIN; LDS_READ(fa1[1], qa, 2048); PIN;
+        if (more)
+        {
+            // the loads of step t + 1; stages t + 2 .. t + S - 1 may stay in flight
+            if (STEADY)
+                WAIT_VMCNT((S - 2) * 4);
+            else
+                wait_stages(nk - 2 - t < S - 2 ? nk - 2 - t : S - 2);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0]), "+v"(fb1[1]));
+        if (more) __builtin_amdgcn_s_barrier();
+        PIN;
+        const unsigned pa = frag_addr_a(t + 1, 0), pb = frag_addr_b(t + 1, 0);
+        mma1(0, 0, fa1, fb1); PIN; if (more) LDS_READ(fa0[0], pa, 0); PIN; if (refill) issue_one(t + S, 0, 0); PIN;
+        mma1(0, 1, fa1, fb1); PIN; if (more) LDS_READ(fb0[0], pb, 0); PIN; if (refill) issue_one(t + S, 0, 1); PIN;
+        mma1(1, 0, fa1, fb1); PIN; if (more) LDS_READ(fb0[1], pb, 2048); PIN; if (refill) issue_one(t + S, 1, 0); PIN;
+        mma1(1, 1, fa1, fb1); PIN; if (more) LDS_READ(fa0[1], pa, 2048); PIN; if (refill) issue_one(t + S, 1, 1); PIN;
+    };
+    int t = 0;
+    for (; t + S < nk; t++) k_step(t, std::true_type{});
+    for (; t < nk; t++) k_step(t, std::false_type{});
+
+    // ---- fused epilogue: dequantise, bias, scale, store fp32
+    EARLY_ARRIVED;
+#undef EARLY_ARRIVED
+    float colscale[2], colc[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+    {
+        colscale[j] = PER_COL ? div_rn(1.f, early_sb[j]) : 0.f;
+        colc[j] = BT == 4 ? mul_rn(early_c[j], beta) : 0.f;
+    }
+    float* rowscale_lds = reinterpret_cast<float*>(smem);
+    {
+        const float rs = PER_COL ? div_rn(1.f, early_sa) : div_rn(1.f, mul_rn(early_sa, early_sb[0]));
+        __builtin_amdgcn_s_barrier(); // every wavefront has left the K loop: the stages are free
+        if (threadIdx.x < QT) rowscale_lds[threadIdx.x] = rs;
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+    {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int row_in_tile = wm * 64 + 4 * lhi + i * 32 + 8 * (r >> 2) + (r & 3);
+            const float rowscale = rowscale_lds[row_in_tile];
+            float* orow = out + (size_t)(tile_m * QT + row_in_tile) * ldo + col_base;
+            float f2[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                float f = mul_rn((float)acc[i][j][r], rowscale);
+                if (PER_COL) f = mul_rn(f, colscale[j]);
+                if (BT == 4) f = add_rn(f, colc[j]);
+                f2[j] = mul_rn(f, alpha);
+            }
+            *reinterpret_cast<float2*>(orow) = make_float2(f2[0], f2[1]);
+        }
+    }
+}
+
 static inline bool al16(const void* p)
 {
     return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
@@ -323,6 +534,288 @@ int launch_gemm_int8_pipelined(const int8_t* aq, size_t aq_stride, const int8_t*
     if ((long long)(M / PT) * (N / PT) > 0x7fffffff) return NCNNHIP_OK;
     *handled = true;
     return launch_256x256<false>(aq, aq_stride, bq, bq_stride, M, N, K, epi, stream);
+}
+
+// The 128x128 tile with K steps of 128 bytes (K % 128 == 0).  A direct-to-LDS load of a wavefront then fetches 8 whole 128-byte
+// lines instead of 16 half lines: the fills of this tile are bound by the lines a CU can have in flight (about 32 KB of 64-byte
+// pieces), not by bytes, and whole lines double what that buys.  A stage is 128 A rows and 128 B rows of 128 bytes (32 KB), four
+// stages; row r keeps its eight 16-byte chunks at positions c ^ ((r >> 1) & 7), which spreads any 16 consecutive rows read at one
+// K offset over the 16 bank groups.  Per K step a wavefront issues 8 loads, 16 LDS reads and 16 MFMA; the step's four quarters
+// alternate between two fragment sets, the barrier stands before the last quarter (all reads of the stage are done by then), and
+// the loads of step t + 4 and the first reads of step t + 1 go between the last quarter's MFMAs.  Global addresses are a uniform
+// base (SGPRs, advanced per step) plus a per-lane 32-bit offset, so the loop spends no vector instructions on them.
+constexpr int RK = 128;
+constexpr int R_OPERAND = QT * RK;     // 16 KB
+constexpr int R_STAGE = 2 * R_OPERAND; // 32 KB
+constexpr int R_STAGES = 4;
+
+template<bool PER_COL, int BT>
+__global__ __launch_bounds__(256) void gemm_int8_128x128_k128_kernel(const int8_t* __restrict__ A, size_t lda, const int8_t* __restrict__ B, size_t ldb,
+                                                                      int nk, int tiles_m, int tiles_n, const float* __restrict__ a_scales,
+                                                                      const float* __restrict__ b_scales, const float* __restrict__ cvec, float alpha,
+                                                                      float beta, float* __restrict__ out, size_t ldo)
+{
+    constexpr int S = R_STAGES;
+    __shared__ __attribute__((aligned(1024))) int8_t smem[S * R_STAGE];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    int b = blockIdx.x;
+    const int T = tiles_m * tiles_n;
+    if ((T & 7) == 0) b = (b & 7) * (T >> 3) + (b >> 3);
+    constexpr int GM = 4;
+    const int per_group = GM * tiles_n;
+    const int group = b / per_group;
+    const int first_m = group * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int in_group = b - group * per_group;
+    const int tile_m = first_m + in_group % gsz;
+    const int tile_n = in_group / gsz;
+
+    // load i (0..3) of wave w fills LDS rows (i*4 + w)*8 .. +8 of an operand stage: lane l writes row + (l >> 3), chunk position l & 7,
+    // and fetches the chunk that belongs there: (l & 7) ^ ((row >> 1) & 7) with row >> 1 = 4*(i*4 + w) + (l >> 4)
+    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    const int8_t* ua = A + (size_t)tile_m * QT * lda; // uniform
+    const int8_t* ub = B + (size_t)tile_n * QT * ldb;
+    unsigned off_a[4], off_b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+    {
+        const int row_a = (i * 4 + wave) * 8 + (lane >> 3);
+        // LDS row wn*64 + j*32 + l holds B row wn*64 + 2*l + j (two consecutive output columns per lane): here wn = i >> 1, j = i & 1,
+        // l = wave*8 + (lane >> 3)
+        const int row_b = (i >> 1) * 64 + 2 * (wave * 8 + (lane >> 3)) + (i & 1);
+        off_a[i] = (unsigned)(row_a * lda + ld_chunk * 16);
+        off_b[i] = (unsigned)(row_b * ldb + ld_chunk * 16);
+    }
+    auto issue_one = [&](int t, int i, int which) {
+        int8_t* sa = smem + (t & (S - 1)) * R_STAGE + (i * 4 + wave) * 1024;
+        if (which == 0)
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(ua + (size_t)t * RK + off_a[i]), (AS3 void*)sa, 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((const AS1 void*)(ub + (size_t)t * RK + off_b[i]), (AS3 void*)(sa + R_OPERAND), 16, 0, 0);
+    };
+    auto issue_stage = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+        {
+            issue_one(t, i, 0);
+            issue_one(t, i, 1);
+        }
+    };
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // what the epilogue needs from memory is requested now, so that it has arrived long before the K loop ends
+    const int col_base = tile_n * QT + wn * 64 + 2 * l32; // accumulator block j of this lane is column col_base + j
+    // (as asm: these loads must stand before the direct-to-LDS loads, whose waits count instructions; EARLY_ARRIVED below ties
+    // the values to a point behind the K loop, where every load of the wavefront has returned)
+    float early_sa, early_sb[2] = {0.f, 0.f}, early_c[2] = {0.f, 0.f};
+#define EARLY_LOAD(dst, ptr) asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory")
+    EARLY_LOAD(early_sa, a_scales + tile_m * QT + (threadIdx.x & (QT - 1)));
+    EARLY_LOAD(early_sb[0], b_scales + (PER_COL ? col_base : 0));
+    if (PER_COL) EARLY_LOAD(early_sb[1], b_scales + col_base + 1);
+    if (BT == 4)
+    {
+        EARLY_LOAD(early_c[0], cvec + col_base);
+        EARLY_LOAD(early_c[1], cvec + col_base + 1);
+    }
+#undef EARLY_LOAD
+#define EARLY_ARRIVED asm volatile("s_waitcnt vmcnt(0)" : "+v"(early_sa), "+v"(early_sb[0]), "+v"(early_sb[1]), "+v"(early_c[0]), "+v"(early_c[1]))
+    PIN;
+
+    // fragment of quarter q (32 bytes of K): chunk 2q + lhi of row l32 (+32 for the second block), swizzled
+    const int sw = (l32 >> 1) & 7;
+    int rd_a[4], rd_b[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+    {
+        rd_a[q] = (wm * 64 + l32) * RK + ((2 * q + lhi) ^ sw) * 16;
+        rd_b[q] = R_OPERAND + (wn * 64 + l32) * RK + ((2 * q + lhi) ^ sw) * 16;
+    }
+    const unsigned lds_base = (unsigned)(uintptr_t)(AS3 int8_t*)smem;
+
+    auto wait_stages = [&](int newer) { // at most `newer` stages (8 loads each) may stay in flight
+        switch (newer)
+        {
+        case 0: WAIT_VMCNT(0); break;
+        case 1: WAIT_VMCNT(8); break;
+        case 2: WAIT_VMCNT(16); break;
+        default: WAIT_VMCNT(24); break;
+        }
+    };
+
+    // ---- prologue: the whole ring in flight
+#pragma unroll
+    for (int t0 = 0; t0 < S; t0++)
+        if (t0 < nk) issue_stage(t0);
+    wait_stages(nk - 1 < S - 1 ? nk - 1 : S - 1);
+    __builtin_amdgcn_s_barrier();
+
+    v4i fa0[2], fb0[2], fa1[2], fb1[2];
+    // requests one quarter's fragments in the order a[0], b[0], b[1], a[1]
+#define REQUEST_QUARTER(fa, fb, stage_base, q)                  \
+    do                                                          \
+    {                                                           \
+        const unsigned pa_ = (stage_base) + (unsigned)rd_a[q];  \
+        const unsigned pb_ = (stage_base) + (unsigned)rd_b[q];  \
+        LDS_READ(fa[0], pa_, 0);                                \
+        LDS_READ(fb[0], pb_, 0);                                \
+        LDS_READ(fb[1], pb_, 4096);                             \
+        LDS_READ(fa[1], pa_, 4096);                             \
+    } while (0)
+    REQUEST_QUARTER(fa0, fb0, lds_base, 0);
+
+    auto mma1 = [&](int i, int j, const v4i (&fa)[2], const v4i (&fb)[2]) {
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    // one quarter's four MFMAs with the next quarter's four reads between them (LDS answers in order: the wait before a product
+    // counts the reads that may still be out)
+#define QUARTER(fa, fb, na, nb, stage_base, nq)                                          \
+    do                                                                                   \
+    {                                                                                    \
+        const unsigned pa_ = (stage_base) + (unsigned)rd_a[nq];                          \
+        const unsigned pb_ = (stage_base) + (unsigned)rd_b[nq];                          \
+        WAIT_LGKM(1, "+v"(fa[0]), "+v"(fb[0]), "+v"(fb[1]));                             \
+        PIN;                                                                             \
+        mma1(0, 0, fa, fb); PIN; LDS_READ(na[0], pa_, 0); PIN;                           \
+        mma1(0, 1, fa, fb); PIN; LDS_READ(nb[0], pb_, 0); PIN;                           \
+        WAIT_LGKM(2, "+v"(fa[1]));                                                       \
+        PIN;                                                                             \
+        mma1(1, 0, fa, fb); PIN; LDS_READ(nb[1], pb_, 4096); PIN;                        \
+        mma1(1, 1, fa, fb); PIN; LDS_READ(na[1], pa_, 4096); PIN;                        \
+    } while (0)
+    auto k_step = [&](int t, auto steady) {
+        constexpr bool STEADY = decltype(steady)::value;
+        const bool more = STEADY || t + 1 < nk;
+        const bool refill = STEADY || t + S < nk;
+        const unsigned cur = lds_base + (unsigned)((t & (S - 1)) * R_STAGE);
+        const unsigned nxt = lds_base + (unsigned)(((t + 1) & (S - 1)) * R_STAGE);
+        QUARTER(fa0, fb0, fa1, fb1, cur, 1);
+        QUARTER(fa1, fb1, fa0, fb0, cur, 2);
+        QUARTER(fa0, fb0, fa1, fb1, cur, 3);
+        if (more)
+        {
+            // the loads of step t + 1; stages t + 2 .. t + S - 1 may stay in flight
+            if (STEADY)
+                WAIT_VMCNT((S - 2) * 8);
+            else
+                wait_stages(nk - 2 - t < S - 2 ? nk - 2 - t : S - 2);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0]), "+v"(fb1[1]));
+        if (more) __builtin_amdgcn_s_barrier(); // every wavefront has read the last of stage t and seen its own loads of stage t + 1
+        PIN;
+        const unsigned pa = nxt + (unsigned)rd_a[0], pb = nxt + (unsigned)rd_b[0];
+        mma1(0, 0, fa1, fb1); PIN; if (more) LDS_READ(fa0[0], pa, 0); PIN; if (refill) { issue_one(t + S, 0, 0); issue_one(t + S, 0, 1); } PIN;
+        mma1(0, 1, fa1, fb1); PIN; if (more) LDS_READ(fb0[0], pb, 0); PIN; if (refill) { issue_one(t + S, 1, 0); issue_one(t + S, 1, 1); } PIN;
+        mma1(1, 0, fa1, fb1); PIN; if (more) LDS_READ(fb0[1], pb, 4096); PIN; if (refill) { issue_one(t + S, 2, 0); issue_one(t + S, 2, 1); } PIN;
+        mma1(1, 1, fa1, fb1); PIN; if (more) LDS_READ(fa0[1], pa, 4096); PIN; if (refill) { issue_one(t + S, 3, 0); issue_one(t + S, 3, 1); } PIN;
+    };
+    int t = 0;
+    for (; t + S < nk; t++) k_step(t, std::true_type{});
+    for (; t < nk; t++) k_step(t, std::false_type{});
+#undef QUARTER
+#undef REQUEST_QUARTER
+
+    // ---- fused epilogue: dequantise, bias, scale, store fp32
+    EARLY_ARRIVED;
+#undef EARLY_ARRIVED
+    float colscale[2], colc[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+    {
+        colscale[j] = PER_COL ? div_rn(1.f, early_sb[j]) : 0.f;
+        colc[j] = BT == 4 ? mul_rn(early_c[j], beta) : 0.f;
+    }
+    float* rowscale_lds = reinterpret_cast<float*>(smem);
+    {
+        const float rs = PER_COL ? div_rn(1.f, early_sa) : div_rn(1.f, mul_rn(early_sa, early_sb[0]));
+        __builtin_amdgcn_s_barrier(); // every wavefront has left the K loop: the stages are free
+        if (threadIdx.x < QT) rowscale_lds[threadIdx.x] = rs;
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+    {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int row_in_tile = wm * 64 + 4 * lhi + i * 32 + 8 * (r >> 2) + (r & 3);
+            const float rowscale = rowscale_lds[row_in_tile];
+            float* orow = out + (size_t)(tile_m * QT + row_in_tile) * ldo + col_base;
+            float f2[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                float f = mul_rn((float)acc[i][j][r], rowscale);
+                if (PER_COL) f = mul_rn(f, colscale[j]);
+                if (BT == 4) f = add_rn(f, colc[j]);
+                f2[j] = mul_rn(f, alpha);
+            }
+            *reinterpret_cast<float2*>(orow) = make_float2(f2[0], f2[1]);
+        }
+    }
+}
+
+template<int KSTEP>
+static int launch_128x128(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmEpilogue& epi, hipStream_t stream)
+{
+    const int tm = M / QT, tn = N / QT, nk = K / KSTEP;
+    dim3 grid(tm * tn), block(256);
+#define LAUNCH(PC, BTV)                                                                                                                              \
+    do                                                                                                                                               \
+    {                                                                                                                                                \
+        if (KSTEP == 128)                                                                                                                            \
+            hipLaunchKernelGGL((gemm_int8_128x128_k128_kernel<PC, BTV>), grid, block, 0, stream, aq, aq_stride, bq, bq_stride, nk, tm, tn,           \
+                               epi.a_scales, epi.b_scales, epi.c, epi.alpha, epi.beta, epi.out, epi.out_stride);                                     \
+        else                                                                                                                                         \
+            hipLaunchKernelGGL((gemm_int8_128x128_kernel<PC, BTV, 4>), grid, block, 0, stream, aq, aq_stride, bq, bq_stride, nk, tm, tn,             \
+                               epi.a_scales, epi.b_scales, epi.c, epi.alpha, epi.beta, epi.out, epi.out_stride);                                     \
+    } while (0)
+    if (epi.per_col)
+    {
+        if (epi.bt == 4)
+            LAUNCH(true, 4);
+        else
+            LAUNCH(true, -1);
+    }
+    else
+    {
+        if (epi.bt == 4)
+            LAUNCH(false, 4);
+        else
+            LAUNCH(false, -1);
+    }
+#undef LAUNCH
+    return launch_status("gemm_int8_128x128_kernel");
+}
+
+// Problems between the few-row kernels and the 256x256 kernel: M and N multiples of 128 (the caller decides from how many tiles up).
+// K % 128 == 0 takes the form with 128-byte K steps, other K % 64 == 0 the form with 64-byte steps.
+// NCNNHIP_GEMM_RING128 (read at every call): 0 switches both off, 64 forces the 64-byte form.
+int launch_gemm_int8_ring128(const int8_t* aq, size_t aq_stride, const int8_t* bq, size_t bq_stride, int M, int N, int K, const GemmEpilogue& epi,
+                             hipStream_t stream, bool* handled)
+{
+    *handled = false;
+    if (M % QT || N % QT || K % PK || aq_stride % 16 || bq_stride % 16 || !al16(aq) || !al16(bq)) return NCNNHIP_OK;
+    if (epi.transpose || epi.acc_out || !(epi.bt == -1 || epi.bt == 4)) return NCNNHIP_OK;
+    if (epi.out_stride % 2 || (reinterpret_cast<uintptr_t>(epi.out) & 7)) return NCNNHIP_OK; // the epilogue stores 8 bytes per lane
+    if ((unsigned long long)QT * aq_stride + 256 > 0xffffffffull || (unsigned long long)QT * bq_stride + 256 > 0xffffffffull) return NCNNHIP_OK; // 32-bit lane offsets
+    const char* e = getenv("NCNNHIP_GEMM_RING128");
+    const int mode = e ? atoi(e) : 128;
+    if (mode == 0) return NCNNHIP_OK;
+    *handled = true;
+    if (K % RK == 0 && mode != 64) return launch_128x128<128>(aq, aq_stride, bq, bq_stride, M, N, K, epi, stream);
+    return launch_128x128<64>(aq, aq_stride, bq, bq_stride, M, N, K, epi, stream);
 }
 
 // operands in the tiled layout; the caller has checked shapes and alignment

@@ -8,6 +8,8 @@ Gemm accumulates in a different order than the reference's sequential sum and is
 """
 import ctypes as C
 
+import os
+
 import numpy as np
 import pytest
 
@@ -151,6 +153,39 @@ def test_gemm_int8_256x256_kernel_sizes(rt, m, n, k, bt, per_col):
     assert np.array_equal(btq, _tiled(bq, True))
     assert np.array_equal(rt.gemm_tile_operand(aq, 0), atq)
     assert np.array_equal(rt.gemm_int8_tiled(atq, btq, m, n, k, sa, sb, c, bt), want)
+
+
+@pytest.mark.parametrize("depth", [64, 128])
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 64), (1024, 1024, 128), (1024, 1024, 192), (896, 1024, 384), (896, 1024, 448), (1152, 768, 512), (1024, 1024, 576),
+                                   (1024, 1024, 640), (1024, 1024, 1024), (1280, 1408, 1280), (2048, 2048, 2048)])
+@pytest.mark.parametrize("bt,per_col", [(4, True), (-1, False)])
+def test_gemm_int8_128x128_kernel_sizes(rt, m, n, k, bt, per_col, depth):
+    """Between 48 tiles of 128 x 128 and 128 tiles of 256 x 256 the Gemm runs on the 128x128 ring kernels: K steps of 128 bytes
+    where K allows, of 64 bytes otherwise or when NCNNHIP_GEMM_RING128=64 (read at every call) forces them.  K steps fewer than,
+    equal to and more than the ring's four stages in either form, tile counts that are not a multiple of 8 with a ragged last row
+    group, the 1024 and 2048 cubes of the benchmark's grid.  Every output element
+    against the epilogue op by op on exact accumulators; the 1024 x 1024 x 64 case also against the scalar oracle; and the same
+    call with the kernel switched off (the 64-row tiles of the convolution kernel) gives the same bits."""
+    _say("gemm_int8 128x128", m, n, k, bt, per_col, depth)
+    a, bq, sb, bias = cases.gemm_case(m + 3 * n + 7 * k, m, n, k, per_col)
+    c = bias.reshape(1, n) if bt == 4 else None
+    aq, sa = oracle.gemm_quantize_rows(a)
+    want, _ = npref.gemm_int8(aq, bq, sa, sb, c, bt, acc=npref.gemm_acc_exact(aq, bq))
+    saved = os.environ.get("NCNNHIP_GEMM_RING128")
+    try:
+        os.environ["NCNNHIP_GEMM_RING128"] = str(depth)
+        got = rt.gemm_int8(aq, bq, sa, sb, c, bt)
+        os.environ["NCNNHIP_GEMM_RING128"] = "0"
+        other = rt.gemm_int8(aq, bq, sa, sb, c, bt) if depth == 128 else got
+    finally:
+        if saved is None:
+            os.environ.pop("NCNNHIP_GEMM_RING128", None)
+        else:
+            os.environ["NCNNHIP_GEMM_RING128"] = saved
+    assert np.array_equal(got, want)
+    assert np.array_equal(other, want)
+    if k == 64 and not per_col:
+        assert np.array_equal(got, oracle.gemm_int8(aq, bq, sa, sb, c, bt))
 
 
 def test_gemm_int8_8192_cube(rt):
