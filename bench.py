@@ -272,9 +272,9 @@ def bench_blockquant(args, n, k, m, bits=8, block=64):
     copies = int(np.ceil(512e6 / wbytes)) + 1
     half = args.act == "fp16"
     packed_form = half or (args.act == "fp32" and k % 16 == 0 and (m >= 32 or lib.ncnnhip_gemm_blockquant_packed_supported(k)))
-    # fp32 activations as the layers dispatch them: up to 4 rows (and 5 to 31 rows of a long K) the few-row kernel, else the kernels that
+    # fp32 activations as the layers dispatch them: up to 4 rows (2 where K is beyond 4096) the few-row kernel, else the kernels that
     # split the activations in a pass of their own into a workspace
-    rows_entry = packed_form and not half and m >= 5
+    rows_entry = packed_form and not half and (m >= 5 or (m >= 3 and k > 4096))
     if packed_form:  # constant weights are repacked once into matrix-core tiles, as create_pipeline does
         pw, pd = rt.blockquant_pack(packed, scales, block, bits=bits, k=k)
         d_w = [rt.up(pw) for _ in range(copies)]  # algorithmic bytes stay those of the .bin: the fields and one fp32 scale per block

@@ -76,8 +76,10 @@ int upload_blockquant_packed(const void* fields_host, const float* scales_host, 
 size_t blockquant_gemm_workspace_bytes(int M, int K, const void* d_packed)
 {
     // 5 rows and more: the kernels that split the activations in a pass of their own (the weight-streaming one on pre-split
-    // operands, 16 rows per pass, while that is cheaper than a tiled pass; else the tiled one: the entry point picks)
-    if (!d_packed || K % 16 != 0 || M < 5) return 0;
+    // operands, 16 rows per pass, while that is cheaper than a tiled pass; else the tiled one: the entry point picks).
+    // 3 and 4 rows of a K beyond 4096 too: the few-row kernel holds three planes per row in LDS and takes such rows one at
+    // a time, a pass over the weights each (4096 x 11008, 4 rows: 48 us against 26 us this way).
+    if (!d_packed || K % 16 != 0 || M < 3 || (M < 5 && K <= 4096)) return 0;
     size_t bytes = 0;
     if (ncnnhip_gemm_blockquant_packed_rows_workspace_bytes(M, K, &bytes) != 0) return 0;
     return bytes;

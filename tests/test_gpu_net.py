@@ -356,7 +356,9 @@ def test_gemm_layer_int8_two_dynamic_operands_transposed_output():
     (8, 64, 0, 4, 24, 200), (4, 32, 1, 4, 24, 200), (6, 128, 0, 4, 24, 200),  # K % 16 != 0: the .bin layout as it is
     # K % 16 == 0: create_pipeline also uploads matrix-core tiles; few rows take them four per pass, 32 rows and more the tiled bf16 kernel
     (8, 64, 0, 1, 40, 256), (8, 64, 1, 4, 33, 256), (4, 32, 1, 3, 24, 512), (6, 128, 0, 16, 40, 1024), (8, 32, 0, 20, 24, 256),
-    (8, 64, 0, 40, 100, 256), (4, 64, 1, 70, 33, 512), (6, 32, 0, 129, 40, 96), (8, 128, 1, 33, 130, 1024)])
+    (8, 64, 0, 40, 100, 256), (4, 64, 1, 70, 33, 512), (6, 32, 0, 129, 40, 96), (8, 128, 1, 33, 130, 1024),
+    # K beyond 4096: three and four rows take the pre-split kernels (the few-row kernel would stream the weights once per row), two rows do not
+    (8, 64, 0, 4, 24, 4352), (4, 32, 1, 3, 40, 8192), (8, 64, 1, 2, 24, 4352)])
 def test_gemm_layer_block_quant(bits, block, insc, m, n, k, resident):
     import npref
     rng = np.random.default_rng(bits + m + k)
