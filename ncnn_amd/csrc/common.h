@@ -186,6 +186,64 @@ __device__ __forceinline__ void pack16_quantised(const float (&v)[16], uint32_t&
                    "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));
 }
 
+// Values already clamped into [0, 127] (a clamp whose lower bound is not negative: ReLU, ReLU6 and their like folded into the
+// requantising clamp): rounding half away from zero is floor(c + 0.5) there, which v_cvt_rpi_i32_f32 computes exactly -- no
+// intermediate sum is rounded (0.49999997 gives 0; compared on the device with floor((double)c + 0.5) for every float within
+// 64 ulp of an integer or a half below 8 and a sweep of [0.125, 128)).  One instruction per value instead of three (sign-copied
+// half, add rounded toward zero, truncating conversion), and no switch of the rounding mode.  Same wait states as above.
+__device__ __forceinline__ uint32_t pack4_nonneg(float a, float b, float c, float d)
+{
+    uint32_t r;
+    asm volatile("v_cvt_rpi_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %3 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %4 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 0"
+                 : "=&v"(r)
+                 : "v"(a), "v"(b), "v"(c), "v"(d));
+    return r;
+}
+__device__ __forceinline__ void pack8_nonneg(const float (&v)[8], uint32_t& r0, uint32_t& r1)
+{
+    asm volatile("v_cvt_rpi_i32_f32_sdwa %0, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 1"
+                 : "=&v"(r0), "=&v"(r1)
+                 : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]));
+}
+__device__ __forceinline__ void pack16_nonneg(const float (&v)[16], uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3)
+{
+    asm volatile("v_cvt_rpi_i32_f32_sdwa %0, %4 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %8 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %2, %12 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %3, %16 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %5 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %9 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %2, %13 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %3, %17 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %6 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %10 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %2, %14 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %3, %18 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %0, %7 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %1, %11 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %2, %15 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "v_cvt_rpi_i32_f32_sdwa %3, %19 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+                 "s_nop 1"
+                 : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+                 : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(v[8]), "v"(v[9]), "v"(v[10]),
+                   "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));
+}
+
 // the same with one clamp per value (four different channels)
 __device__ __forceinline__ void float2int8_as_float_bounded_lanes_x4(float& v0, float& v1, float& v2, float& v3, const float (&lo)[4], const float (&hi)[4])
 {

@@ -26,7 +26,8 @@ namespace ncnnhip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// ACT: 0 none, 1 ReLU, 3 clip as written, 103 clip folded into the clamp (tame tables), -1 anything else.
+// ACT: 0 none, 1 ReLU, 3 clip as written, 103 clip folded into the clamp (tame tables), 203 the same with no negative clamp
+// bound (rounding by one conversion, pack16_nonneg), -1 anything else.
 // acc[pg][r]: pixel group pg, channel r of the lane's four; returns one packed word per pixel group.
 template<int ACT>
 __device__ __forceinline__ void pointwise_requantise(const v4i (&acc)[4], const float (&s_in)[4], const float (&bias)[4], const float (&s_out)[4],
@@ -51,12 +52,20 @@ __device__ __forceinline__ void pointwise_requantise(const v4i (&acc)[4], const 
                 v = apply_activation(v, act);
             f[4 * pg + r] = mul_rn(v, s_out[r]);
         }
-        if (ACT == 103)
+        if (ACT == 203)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; r++) f[4 * pg + r] = __builtin_amdgcn_fmed3f(f[4 * pg + r], q_lo[r], q_hi[r]);
+        }
+        else if (ACT == 103)
             float2int8_as_float_bounded_lanes_x4(f[4 * pg], f[4 * pg + 1], f[4 * pg + 2], f[4 * pg + 3], q_lo, q_hi);
         else
             float2int8_as_float_x4(f[4 * pg], f[4 * pg + 1], f[4 * pg + 2], f[4 * pg + 3]);
     }
-    pack16_quantised(f, word[0], word[1], word[2], word[3]);
+    if (ACT == 203)
+        pack16_nonneg(f, word[0], word[1], word[2], word[3]);
+    else
+        pack16_quantised(f, word[0], word[1], word[2], word[3]);
 }
 
 // grid: one wavefront per (run of `blocks_per_wave` 64-pixel blocks, 16-channel block), channel block fastest so that
@@ -149,7 +158,8 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
         }
         tame = __all(tame);
     }
-    const int mode = act.type == 0 ? 0 : act.type == 1 ? 1 : act.type == 3 ? (tame ? 103 : 3) : -1;
+    const bool nonneg = tame && __all(q_lo[0] >= 0.f && q_lo[1] >= 0.f && q_lo[2] >= 0.f && q_lo[3] >= 0.f);
+    const int mode = act.type == 0 ? 0 : act.type == 1 ? 1 : act.type == 3 ? (nonneg ? 203 : tame ? 103 : 3) : -1;
 
     const unsigned store_off = (unsigned)(q * 16 + c16) * (unsigned)out_cp + (unsigned)cb * 16; // within a 64-pixel block
     for (int pb0 = pb_begin; pb0 < pb_end; pb0 += 2)
@@ -165,7 +175,9 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
             for (int pg = 0; pg < 4; pg++) acc[pg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw, fx[j][pg], v4i{0, 0, 0, 0}, 0, 0, 0);
 
             uint32_t word[4];
-            if (mode == 103)
+            if (mode == 203)
+                pointwise_requantise<203>(acc, s_in, bias, s_out, q_lo, q_hi, act, word);
+            else if (mode == 103)
                 pointwise_requantise<103>(acc, s_in, bias, s_out, q_lo, q_hi, act, word);
             else if (mode == 1)
                 pointwise_requantise<1>(acc, s_in, bias, s_out, q_lo, q_hi, act, word);

@@ -317,7 +317,7 @@ __global__ __launch_bounds__(256, 2) void conv_resident_kernel(const int8_t* __r
     // ---- everything this wavefront asked for has landed.  Tables into LDS: input scale, bias, output scale and the
     // requantising clamp [lo, hi] that also holds a ReLU or a clip when that is provably the same value (see below)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    bool tame = true;
+    bool tame = true, nonneg = true;
     if (tid < BN)
     {
         const bool real = col0 + tid < P.cout;
@@ -343,6 +343,7 @@ __global__ __launch_bounds__(256, 2) void conv_resident_kernel(const int8_t* __r
             if (epi.act.type == 1) lo = 0.f;
         }
         tame = ok;
+        nonneg = lo >= 0.f; // a clamp without a negative bound: the rounding is one conversion (pack8_nonneg / pack4_nonneg)
         float* tab = reinterpret_cast<float*>(lds + P.lds_tab);
         tab[tid] = si;
         tab[BN + tid] = bi;
@@ -350,7 +351,11 @@ __global__ __launch_bounds__(256, 2) void conv_resident_kernel(const int8_t* __r
         tab[3 * BN + tid] = lo;
         tab[4 * BN + tid] = hi;
     }
-    tame = __syncthreads_and(tame) != 0; // (also: everybody's share of the operands and the tables are in LDS)
+    {
+        const int failed = __syncthreads_or((tame ? 0 : 1) | (nonneg ? 0 : 2)); // (also: everybody's share of the operands and the tables are in LDS)
+        tame = !(failed & 1);
+        nonneg = tame && !(failed & 2);
+    }
 
     // ---- fragment addresses that do not depend on the tile
     unsigned w_base[TN];
@@ -584,7 +589,14 @@ __global__ __launch_bounds__(256, 2) void conv_resident_kernel(const int8_t* __r
                             const float f = mul_rn(add_rn(mul_rn((float)acc[a][c][4 * g + e], cur.si[e]), cur.bi[e]), cur.so[e]);
                             v[a * 4 + e] = __builtin_amdgcn_fmed3f(f, cur.lo[e], cur.hi[e]);
                         }
-                    if constexpr (TM == 2)
+                    if (nonneg)
+                    {
+                        if constexpr (TM == 2)
+                            pack8_nonneg(v, word[0][idx], word[1][idx]);
+                        else
+                            word[0][idx] = pack4_nonneg(v[0], v[1], v[2], v[3]);
+                    }
+                    else if constexpr (TM == 2)
                         round_pack_2x4(v, word[0][idx], word[1][idx]);
                     else
                         round_pack_1x4(v, word[0][idx]);

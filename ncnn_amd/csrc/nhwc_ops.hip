@@ -562,8 +562,10 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
         q_lo[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p0, s_out[e]), -127.f, 127.f);
         q_hi[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p1, s_out[e]), -127.f, 127.f);
     }
+    // no negative clamp bound (ReLU6 and its like): the rounding is one conversion (pack4_nonneg)
     auto emit = [&](auto clip_tag) {
-        constexpr bool FAST_CLIP = decltype(clip_tag)::value;
+        constexpr bool FAST_CLIP = decltype(clip_tag)::value > 0;
+        constexpr bool NONNEG = decltype(clip_tag)::value > 1;
 #pragma unroll
         for (int ro = 0; ro < ROWS; ro++)
 #pragma unroll
@@ -585,7 +587,12 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
             }
             if (!g.out_f32)
             {
-                if (FAST_CLIP)
+                if (NONNEG)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) f[e] = __builtin_amdgcn_fmed3f(f[e], q_lo[e], q_hi[e]);
+                }
+                else if (FAST_CLIP)
                     float2int8_as_float_bounded_lanes_x4(f[0], f[1], f[2], f[3], q_lo, q_hi);
                 else
                     float2int8_as_float_x4(f[0], f[1], f[2], f[3]);
@@ -595,14 +602,21 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
                 if ((int)q0 + e >= g.c) f[e] = 0.f;
             if (g.out_f32)
                 *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
+            else if (NONNEG)
+                *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) = pack4_nonneg(f[0], f[1], f[2], f[3]);
             else
                 *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) = pack4_quantised(f[0], f[1], f[2], f[3]);
         }
     };
     if (act.type == 3 && __all(finite_tables))
-        emit(std::true_type{});
+    {
+        if (!g.out_f32 && __all(q_lo[0] >= 0.f && q_lo[1] >= 0.f && q_lo[2] >= 0.f && q_lo[3] >= 0.f))
+            emit(std::integral_constant<int, 2>{});
+        else
+            emit(std::integral_constant<int, 1>{});
+    }
     else
-        emit(std::false_type{});
+        emit(std::integral_constant<int, 0>{});
 }
 
 static inline int padded16(int c)
