@@ -875,14 +875,19 @@ static int resident_choose(const NhwcGeom& g, const ConvEpilogue& epi, const Con
 }
 
 // Which layers take this kernel: kernels with taps (a 1x1 layer reads nothing twice and is bound by HBM or by its epilogue
-// either way: measured no faster here) from 1536 output pixels up (measured on the 3x3 layers of a ResNet-50 at batch 1 to
-// 128: from there on as fast or faster than the pipelined kernel, 5 to 25 % on the 56 x 56 to 14 x 14 maps).
+// either way: measured no faster here) from 40000 output pixels up.  Launched alone, the kernel is as fast or faster than the
+// pipelined kernel from 1536 pixels up (the 3x3 layers of a ResNet-50 at batch 16 to 128: 56 x 56 maps 8 to 25 % faster,
+// 28 x 28 4 to 7 %, 14 x 14 15 % at batch 16 and 2 to 4 % slower beyond).  Inside a whole pass, where launches follow one
+// another without a gap, the long-lived workgroups of the smaller layers hold their CUs' LDS until the last tile is done and
+// the next launch starts later than behind the pipelined kernel's short ones: with every 3x3 layer on this kernel a ResNet-50
+// pass is 2 % slower at batch 32 and 1 % at batch 128 (equal at batch 16); from 40000 pixels up (the 56 x 56 maps from batch
+// 16, the 28 x 28 maps from batch 64) the passes are as fast as without it and those layers are the ones that gain most alone.
 // Environment, read at every launch: NCNNHIP_RESIDENT_OFF (any value) switches the kernel off, NCNNHIP_RESIDENT_MIN sets
 // the pixel threshold, NCNNHIP_RESIDENT_CFG forces one tile configuration (0..7): for measurements and tests.
 bool conv_resident_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp)
 {
     if (getenv("NCNNHIP_RESIDENT_OFF")) return false;
-    long long min_pixels = 1536;
+    long long min_pixels = 40000;
     if (const char* e = getenv("NCNNHIP_RESIDENT_MIN")) min_pixels = atoll(e);
     if (g.npix < min_pixels || g.ntaps < 2) return false;
     ResidentPlan P;

@@ -1,7 +1,7 @@
 """The weights-resident convolution kernel (kernels with taps on layers with many output pixels: the batched nets)
 against the oracle.
 
-The kernel is chosen by the layer's shape (taps, 1536 output pixels and more); the environment variables
+The kernel is chosen by the layer's shape (taps, 40000 output pixels and more); the environment variables
 NCNNHIP_RESIDENT_MIN (pixel threshold) and NCNNHIP_RESIDENT_CFG (tile configuration 0..7) are read at every launch, so
 the small cases here lower the threshold and walk every tile configuration, and the large ones run as a net would.
 Semantics: Convolution::forward_int8 (src/layer/convolution.cpp:383-508) per sample, batch as src/net.cpp:654-700."""
@@ -122,7 +122,10 @@ def test_fused_tail_residual_relu_quantised_copy(rt, resident_env, c, h, w, outc
     (5, 64, 57, 57, 96, (3, 3), (2, 2), (0, 0, 0, 0), 2, 0),       # stride 2 without padding, fp32 out
     (3, 64, 40, 40, 48, (3, 3), (1, 1), (1, 1, 1, 1), 102, 3),     # clip
 ])
-def test_benchmark_layer_shapes_as_a_net_runs_them(rt, batch, c, h, w, outc, kernel, stride, pads, term, act):
-    """No environment overrides: the shapes are large enough for the shape rule to pick the kernel by itself."""
+def test_benchmark_layer_shapes_as_a_net_runs_them(rt, resident_env, batch, c, h, w, outc, kernel, stride, pads, term, act):
+    """The first shape is large enough for the shape rule to pick the kernel by itself (no environment override); the others run
+    with the threshold lowered to 1536 pixels, the tile configuration still chosen by the kernel's own cost estimate."""
     _say("resident at size", batch, c, h, w, outc, kernel)
+    if batch * h * w < 40000 * stride[0] * stride[1]:
+        resident_env(min_pixels=1536)
     _check(rt, 11, batch, c, h, w, outc, kernel, (1, 1), stride, pads, term, act, (0.0, 6.0))
