@@ -143,7 +143,7 @@ void HipMat::create_like(const HipMat& m, HipCommand* command)
 
 // ---- HipPool ------------------------------------------------------------------------------------
 
-HipPool::HipPool(bool defer) : defer_reuse(defer) {}
+HipPool::HipPool(bool defer) : returns(0), defer_reuse(defer) {}
 
 HipPool::~HipPool()
 {
@@ -154,35 +154,46 @@ HipPool::~HipPool()
 void* HipPool::take(size_t bytes, int state)
 {
     if (bytes == 0) bytes = 4;
-    std::lock_guard<std::mutex> g(lock);
-    for (int pass = 0; pass < 2; pass++)
     {
-        // smallest idle buffer that fits without wasting more than half of it
-        int best = -1;
-        bool retired_fits = false;
-        for (size_t i = 0; i < slots.size(); i++)
+        std::unique_lock<std::mutex> g(lock);
+        for (int pass = 0; pass < 2; pass++)
         {
-            const bool fits = slots[i].bytes >= bytes && slots[i].bytes <= 2 * bytes + 0x10000;
-            if (slots[i].state == 0 && fits && (best < 0 || slots[i].bytes < slots[(size_t)best].bytes)) best = (int)i;
-            if (slots[i].state == 3 && fits) retired_fits = true;
+            // smallest idle buffer that fits without wasting more than half of it
+            int best = -1;
+            bool retired_fits = false;
+            for (size_t i = 0; i < slots.size(); i++)
+            {
+                const bool fits = slots[i].bytes >= bytes && slots[i].bytes <= 2 * bytes + 0x10000;
+                if (slots[i].state == 0 && fits && (best < 0 || slots[i].bytes < slots[(size_t)best].bytes)) best = (int)i;
+                if (slots[i].state == 3 && fits) retired_fits = true;
+            }
+            if (best >= 0)
+            {
+                slots[(size_t)best].state = state;
+                return slots[(size_t)best].ptr;
+            }
+            if (pass == 1 || !retired_fits) break;
+            // A returned buffer would do, but a kernel on some other stream may still read it: wait for the device once,
+            // after which every buffer that had come back BEFORE the wait began is free to go out again.  The wait runs
+            // without the lock (other threads keep taking and returning buffers meanwhile; what they return during the wait
+            // stays retired), and fails under another thread's stream capture: a new allocation then serves the request.
+            const unsigned long long seen = returns;
+            g.unlock();
+            const bool waited = ncnnhip_device_synchronize() == 0;
+            g.lock();
+            if (!waited) break;
+            for (size_t i = 0; i < slots.size(); i++)
+                if (slots[i].state == 3 && slots[i].retired <= seen) slots[i].state = 0;
         }
-        if (best >= 0)
-        {
-            slots[(size_t)best].state = state;
-            return slots[(size_t)best].ptr;
-        }
-        if (pass == 1 || !retired_fits) break;
-        // a returned buffer would do, but a kernel on some other stream may still read it: wait for the device once,
-        // after which every returned buffer is free to go out again
-        if (ncnnhip_device_synchronize() != 0) break;
-        for (size_t i = 0; i < slots.size(); i++)
-            if (slots[i].state == 3) slots[i].state = 0;
     }
+    // nothing idle fits: a new buffer, allocated without the lock
     Slot s;
     s.bytes = (bytes + 0xffff) & ~(size_t)0xffff;
     s.state = state;
     s.ptr = 0;
+    s.retired = 0;
     if (ncnnhip_malloc(&s.ptr, s.bytes) != 0 || !s.ptr) return 0;
+    std::lock_guard<std::mutex> g(lock);
     slots.push_back(s);
     return s.ptr;
 }
@@ -194,6 +205,7 @@ void HipPool::give_back(void* ptr)
         if (slots[i].ptr == ptr)
         {
             slots[i].state = defer_reuse ? 3 : 0;
+            slots[i].retired = ++returns;
             return;
         }
 }

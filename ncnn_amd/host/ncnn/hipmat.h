@@ -46,7 +46,9 @@ private:
         void* ptr;
         size_t bytes;
         int state; // 0 idle, 1 blob, 2 borrowed scratch, 3 returned but possibly still read on another stream
+        unsigned long long retired; // state 3: the pool's return count when the buffer came back
     };
+    unsigned long long returns; // buffers given back so far (orders the state-3 slots against a device-wide wait)
     mutable std::mutex lock;
     std::vector<Slot> slots;
     bool defer_reuse;
