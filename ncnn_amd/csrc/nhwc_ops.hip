@@ -482,12 +482,6 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
 
     int acc[ROWS][OUTS][4];
 #pragma unroll
-    for (int ro = 0; ro < ROWS; ro++)
-#pragma unroll
-        for (int o = 0; o < OUTS; o++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[ro][o][e] = 0;
-#pragma unroll
     for (int iy = 0; iy < IN_ROWS; iy++)
     {
         const int y = y0 + iy;
@@ -514,26 +508,30 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
 #pragma unroll
             for (int c = 0; c < 4; c++)
             {
-                acc[ro][0][c] = __builtin_amdgcn_sdot4((int)t[c], wv[ky][c], acc[ro][0][c], false);
-                if (OUTS == 2) acc[ro][1][c] = __builtin_amdgcn_sdot4((int)t[c], wv1[ky][c], acc[ro][1][c], false);
+                // kernel row 0 is an output row's first contribution: it starts from a literal zero (no register to clear)
+                acc[ro][0][c] = __builtin_amdgcn_sdot4((int)t[c], wv[ky][c], ky == 0 ? 0 : acc[ro][0][c], false);
+                if (OUTS == 2) acc[ro][1][c] = __builtin_amdgcn_sdot4((int)t[c], wv1[ky][c], ky == 0 ? 0 : acc[ro][1][c], false);
             }
         }
     }
 
     // per-channel tables: one vector load each when the channel count is a multiple of 4 (uniform), else clamped scalars
+    // Pad channels (from g.c up) get scale 0, bias -0 and output scale 0: whatever the activation, a finite value times a
+    // zero output scale is a zero byte, so the int8 epilogues need no select per value (the fp32 one keeps its own).
     float s_in[4], s_b[4], s_out[4];
     if ((g.c & 3) == 0)
     {
-        const unsigned qc = q0 < (unsigned)g.c ? q0 : (unsigned)g.c - 4;
+        const bool real = q0 < (unsigned)g.c; // a quad is real or it is not
+        const unsigned qc = real ? q0 : (unsigned)g.c - 4;
         const v4f a = *reinterpret_cast<const v4f*>(scale_in + qc);
         const v4f b = bias ? *reinterpret_cast<const v4f*>(bias + qc) : v4f{-0.f, -0.f, -0.f, -0.f}; // x + -0 = x for every x
         const v4f c = g.out_f32 ? v4f{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const v4f*>(scale_out + qc);
 #pragma unroll
         for (int e = 0; e < 4; e++)
         {
-            s_in[e] = a[e];
-            s_b[e] = b[e];
-            s_out[e] = c[e];
+            s_in[e] = real ? a[e] : 0.f;
+            s_b[e] = real ? b[e] : -0.f;
+            s_out[e] = real ? c[e] : 0.f;
         }
     }
     else
@@ -541,10 +539,11 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
 #pragma unroll
         for (int e = 0; e < 4; e++)
         {
-            const int qc = (int)q0 + e < g.c ? (int)q0 + e : g.c - 1;
-            s_in[e] = scale_in[qc];
-            s_b[e] = bias ? bias[qc] : -0.f;
-            s_out[e] = g.out_f32 ? 0.f : scale_out[qc];
+            const bool real = (int)q0 + e < g.c;
+            const int qc = real ? (int)q0 + e : g.c - 1;
+            s_in[e] = real ? scale_in[qc] : 0.f;
+            s_b[e] = (real && bias) ? bias[qc] : -0.f;
+            s_out[e] = (real && !g.out_f32) ? scale_out[qc] : 0.f;
         }
     }
     // A clip whose operand cannot be NaN (finite tables: an int32 times a finite scale plus a finite bias is finite or
@@ -562,6 +561,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
         q_lo[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p0, s_out[e]), -127.f, 127.f);
         q_hi[e] = __builtin_amdgcn_fmed3f(mul_rn(act.p1, s_out[e]), -127.f, 127.f);
     }
+    const size_t off00 = (((size_t)img * g.outh + oy0) * g.outw + ox0) * g.cp + q0; // output (row 0, pixel 0) of this thread
     // no negative clamp bound (ReLU6 and its like): the rounding is one conversion (pack4_nonneg)
     auto emit = [&](auto clip_tag) {
         constexpr bool FAST_CLIP = decltype(clip_tag)::value > 0;
@@ -573,7 +573,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
         {
             const unsigned ox = ox0 + o, oy = oy0 + ro;
             if (ox >= (unsigned)g.outw || oy >= (unsigned)g.outh) continue;
-            const size_t off = (((size_t)img * g.outh + oy) * g.outw + ox) * g.cp + q0;
+            const size_t off = off00 + (size_t)(unsigned)((ro * g.outw + o) * g.cp); // (uniform: a scalar product, one 64-bit add)
             float f[4];
 #pragma unroll
             for (int e = 0; e < 4; e++)
@@ -597,11 +597,13 @@ __global__ __launch_bounds__(256) void dwconv3x3_nhwc_kernel(const int8_t* __res
                 else
                     float2int8_as_float_x4(f[0], f[1], f[2], f[3]);
             }
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if ((int)q0 + e >= g.c) f[e] = 0.f;
             if (g.out_f32)
+            {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if ((int)q0 + e >= g.c) f[e] = 0.f;
                 *reinterpret_cast<v4f*>(static_cast<float*>(out) + off) = v4f{f[0], f[1], f[2], f[3]};
+            }
             else if (NONNEG)
                 *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(out) + off) = pack4_nonneg(f[0], f[1], f[2], f[3]);
             else
