@@ -21,7 +21,8 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-cont
 # per-file additions.  blockquant.hip: matrix-core results that go straight into vector arithmetic (the per-block descale) stay in
 # VGPRs instead of AGPRs, which saves a register read per value (tiled kernel 135 -> 125 us at 1024 x 4096 x 4096).
 # attention.hip: the same for the scores and the context on their way into the softmax arithmetic (attention core of 1500 tokens 183 -> 155 us).
-HIPCC_FILE_FLAGS = {"blockquant.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+HIPCC_FILE_FLAGS = {"blockquant.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+                    "conv_pointwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "conv_resident.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _run(cmd):

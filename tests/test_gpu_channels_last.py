@@ -99,18 +99,22 @@ def test_clip_is_the_reference_clip_whatever_its_bounds(rt, act_params, term, bi
             assert got.dtype == want.dtype and np.array_equal(got[i], want), (group, kernel)
 
 
-@pytest.mark.parametrize("c,outc,act,act_params,flip", [
-    (16, 24, 3, (0.0, 6.0), False),     # clip folded into the clamp; second 16-channel block half padding
-    (40, 8, 0, (0.0, 0.0), False),      # 48 bytes per pixel: the last lane row reads bytes the zero weights cancel
-    (64, 100, 1, (0.0, 0.0), False),    # the full K, ReLU, channel count not a multiple of 16
-    (24, 32, 3, (-0.2, 0.3), True),     # negative output scales: the literal clip
-    (8, 16, 2, (0.1, 0.0), False),      # leaky ReLU: the general activation path
+@pytest.mark.parametrize("c,outc,act,act_params,flip,hw", [
+    (16, 24, 3, (0.0, 6.0), False, 257),     # clip folded into the clamp; second 16-channel block half padding
+    (40, 8, 0, (0.0, 0.0), False, 257),      # 48 bytes per pixel: the last lane row reads bytes the zero weights cancel
+    (64, 100, 1, (0.0, 0.0), False, 257),    # the full K, ReLU, channel count not a multiple of 16
+    (24, 32, 3, (-0.2, 0.3), True, 257),     # negative output scales: the literal clip
+    (8, 16, 2, (0.1, 0.0), False, 257),      # leaky ReLU: the general activation path
+    (16, 96, 3, (0.0, 6.0), False, 365),     # MobileNetV2's first expansion: six channel blocks, three per wavefront pair
+    (32, 144, 3, (0.5, 4.0), False, 257),    # a clip with a positive lower bound; nine channel blocks over two wavefronts
+    (24, 40, 3, (-1.0, 2.0), False, 257),    # a clip with a negative lower bound: folded, rounded the general way
 ])
-def test_pointwise_small_k_kernel_matches_oracle(rt, c, outc, act, act_params, flip):
+def test_pointwise_small_k_kernel_matches_oracle(rt, c, outc, act, act_params, flip, hw):
     """1x1 layers with at most 64 input channels, int8 output and 2^16 pixels or more take a kernel of their own
-    (MFMA fed weights-first, no LDS, lane-row transposes before the store): ragged pixel count, batch 2."""
-    _say("pointwise small-K", c, outc, act, act_params, flip)
-    h = w = 257
+    (MFMA fed weights-first, tables in LDS, lane-row transposes before the store; a workgroup owns whole pixel rows of the
+    output): ragged pixel count, batch 2."""
+    _say("pointwise small-K", c, outc, act, act_params, flip, hw)
+    h = w = hw
     x, wq, b, ws, ins, tops = cases.conv_case(c + outc, c, h, w, outc, (1, 1), 1, 102, True, True, batch=2)
     if flip:
         tops = -tops
