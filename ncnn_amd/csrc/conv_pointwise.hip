@@ -201,9 +201,8 @@ int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x,
     const int channel_blocks = out_cp / 16;
     const int pixel_blocks = ceil_div(g.npix, 64);
     // pixel blocks per workgroup: two, each with two wavefronts that take the even and the odd channel blocks (measured on
-    // MobileNetV2's expand layers at batch 32 against one block with four wavefronts and four blocks with one each:
-    // 16 -> 96 on 112 x 112 19.8 / 22.7 / 31.3 us, 24 -> 144 on 56 x 56 10.6 / 11.5 / 10.8); a layer too small for that many
-    // workgroups keeps one block per workgroup
+    // MobileNetV2's 16 -> 96 expansion on 112 x 112 at batch 32: 19.8 us, against 23.1 for one block with four wavefronts and
+    // 31 for four blocks with one wavefront each); a layer too small for that many workgroups keeps one block per workgroup
     const int G = pixel_blocks >= 1024 ? 2 : 1;
     const size_t lds = (size_t)5 * out_cp * sizeof(float);
     NCNNHIP_REQUIRE(lds <= 60 * 1024, "convolution: %d output channels are too many for the pointwise kernel's tables", g.cout);
