@@ -189,6 +189,15 @@ int ncnnhip_conv_int8_nhwc_from_float(const ncnnhip_conv_desc* desc, const void*
                                       ncnnhip_activation act, void* out_nhwc_dev, const ncnnhip_conv_fusion* fusion, void* workspace_dev,
                                       size_t workspace_bytes, void* stream);
 
+/* Which kernel a channels-last layer gets: 1 when ncnnhip_conv_int8_nhwc / _fused (elemsize 1) or
+ * ncnnhip_conv_int8_nhwc_from_float (elemsize 4 or 2) would run this layer on the small-tile kernel -- two-dimensional
+ * tiles of 32 output pixels x 64 channels whose input patch is quantised into LDS, for layers with too few output pixels
+ * to fill the chip with 64-pixel tiles; it needs no workspace -- and 0 otherwise.  The same arithmetic either way
+ * (Convolution::forward_int8, src/layer/convolution.cpp:383-508); the answer depends on the shape and on the environment
+ * variable NCNNHIP_PATCH (0: never, 1: whenever the layer fits).  No counterpart in the reference: a query for tests
+ * and for callers that size workspaces. */
+int ncnnhip_conv_small_tile_selected(const ncnnhip_conv_desc* desc, int elemsize);
+
 
 /* Convolution::forward_int8 (src/layer/convolution.cpp:383-508) for layers with at most 4 input channels (the 3-channel
  * first layer of an image net), group 1, dilation_w 1, zero border value.  The input is quantised into an image of 4 bytes

@@ -67,6 +67,13 @@ bool conv_nhwc_staged_supported(const NhwcGeom& g);
 size_t conv_nhwc_staged_workspace_bytes(const NhwcGeom& g);
 int launch_conv_nhwc_staged(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi,
                             const ConvFusion& fusion, int out_cp, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// The small-tile kernel (conv_patch.hip: 2-D tiles of 32 output pixels, the input patch quantised into LDS, no
+// workspace) for layers with few output pixels; x_elemsize 1 (int8 blob), 4 or 2 (fp32 / fp16 blob + x_scale).
+// conv_patch_pays: the layer fits AND is of the kind that measured faster there than on the pipelined kernel.
+bool conv_patch_supported(const NhwcGeom& g, int batch);
+bool conv_patch_pays(const NhwcGeom& g, int batch, int x_elemsize);
+int launch_conv_patch(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi, const ConvFusion& fusion,
+                      int out_cp, hipStream_t stream);
 bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
 // The weights-resident kernel for layers with many output pixels (conv_resident.hip): does this problem fit it, and its
 // launch.  The pipelined launch asks first.

@@ -579,6 +579,8 @@ static int conv_int8_nhwc_impl(const ncnnhip_conv_desc* desc, const void* nhwc_d
     epi.acc_out = 0;
 
     hipStream_t st = as_stream(stream);
+    if (clast && pb == 0 && conv_patch_pays(g, d.batch, x_elemsize))
+        return launch_conv_patch(g, packed_weight_dev, nhwc_dev, x_elemsize, x_scale_dev, epi, fusion, out_cp, st);
     if (x_elemsize != 1)
     {
         NCNNHIP_REQUIRE(clast && x_scale_dev, "ncnnhip_conv_int8_nhwc_from_float: needs channels-last output and the input scale");
@@ -665,7 +667,18 @@ int ncnnhip_conv_from_float_supported(const ncnnhip_conv_desc* desc)
     if (ncnnhip_conv_out_shape(desc, &outw, &outh) != 0) return 0;
     const long long npix = (long long)outw * outh * desc->batch;
     if (npix >= (1ll << 31) || (long long)desc->h * desc->w * padded_channels(desc->c) >= (1ll << 31)) return 0;
-    return conv_nhwc_staged_supported(nhwc_geometry(*desc, outw, outh, npix)) ? 1 : 0;
+    const NhwcGeom g = nhwc_geometry(*desc, outw, outh, npix);
+    return (conv_patch_pays(g, desc->batch, 4) || conv_nhwc_staged_supported(g)) ? 1 : 0;
+}
+
+int ncnnhip_conv_small_tile_selected(const ncnnhip_conv_desc* desc, int elemsize)
+{
+    if (!desc || desc->group != 1 || (int)(signed char)desc->pad_value != 0 || (elemsize != 1 && elemsize != 2 && elemsize != 4)) return 0;
+    int outw = 0, outh = 0;
+    if (ncnnhip_conv_out_shape(desc, &outw, &outh) != 0) return 0;
+    const long long npix = (long long)outw * outh * desc->batch;
+    if (npix >= (1ll << 31) || (long long)desc->h * desc->w * padded_channels(desc->c) >= (1ll << 31)) return 0;
+    return conv_patch_pays(nhwc_geometry(*desc, outw, outh, npix), desc->batch, elemsize) ? 1 : 0;
 }
 
 int ncnnhip_conv_from_float_workspace_bytes(const ncnnhip_conv_desc* desc, size_t* workspace_bytes)
@@ -676,7 +689,8 @@ int ncnnhip_conv_from_float_workspace_bytes(const ncnnhip_conv_desc* desc, size_
     int outw = 0, outh = 0;
     int ret = ncnnhip_conv_out_shape(desc, &outw, &outh);
     if (ret) return ret;
-    *workspace_bytes = conv_nhwc_staged_workspace_bytes(nhwc_geometry(*desc, outw, outh, (long long)outw * outh * desc->batch));
+    const NhwcGeom g = nhwc_geometry(*desc, outw, outh, (long long)outw * outh * desc->batch);
+    if (!conv_patch_pays(g, desc->batch, 4)) *workspace_bytes = conv_nhwc_staged_workspace_bytes(g); // (the small-tile kernel needs none)
     return NCNNHIP_OK;
 }
 

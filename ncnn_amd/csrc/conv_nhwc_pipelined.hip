@@ -42,20 +42,6 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
     return pack4_quantised(v[0], v[1], v[2], v[3]);
 }
 
-// n / d for 0 <= n < 2^20 and d >= 1: both are exact as floats and the float quotient (reciprocal good to an ulp or
-// two, one multiply) is within 2^20 * 2^-21 = one half of the true one, so its truncation is off by at most one, which
-// the remainder shows.  Seven instructions where the compiler's general 32-bit division takes about twenty-five.
-__device__ __forceinline__ int small_div(int n, int d)
-{
-    int q = (int)((float)n * __builtin_amdgcn_rcpf((float)d));
-    const int r = n - q * d;
-    if (r < 0)
-        q--;
-    else if (r >= d)
-        q++;
-    return q;
-}
-
 // MODE: how a lane finds its source bytes.  0: any geometry; 1: dense (1x1, stride 1, unpadded: one row of npix pixels,
 // also Gemm and InnerProduct); 2: taps of 16 or 32 bytes (the narrow-input image), a whole number of taps per K step.
 // A template parameter because the choice sits inside the K loop: as run-time branches there it cost the 3x3 layers

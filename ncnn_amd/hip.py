@@ -90,6 +90,7 @@ _SIGNATURES = {
                                C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p],
     "ncnnhip_conv_fusion_supported": [C.POINTER(ConvDesc)],
     "ncnnhip_conv_from_float_supported": [C.POINTER(ConvDesc)],
+    "ncnnhip_conv_small_tile_selected": [C.POINTER(ConvDesc), C.c_int],
     "ncnnhip_conv_from_float_workspace_bytes": [C.POINTER(ConvDesc), C.POINTER(C.c_size_t)],
     "ncnnhip_conv_int8_nhwc_from_float": [C.POINTER(ConvDesc), C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, Activation, C.c_void_p,
                                           C.POINTER(ConvFusion), C.c_void_p, C.c_size_t, C.c_void_p],
