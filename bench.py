@@ -761,6 +761,7 @@ def bench_conv(args, spec):
     d_fws = ncnn_amd.DeviceBuffer.zeros(fws.value, st)
     step = one_launch if fused_quantise else two_launches
     kernel = one_launch if fused_quantise else conv
+    small_tile = bool(lib.ncnnhip_conv_small_tile_selected(C.byref(desc), 4 if fused_quantise else 1))
 
     def wall_ms(fn):
         check(lib.ncnnhip_device_synchronize())
@@ -794,7 +795,7 @@ def bench_conv(args, spec):
                    "submission": "one launch, the Quantize pass inside the convolution's loader" if fused_quantise else "Quantize kernel, then the convolution kernel",
                    "quantize_then_convolution_us": two_launch_ms * 1e3},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOPS", "frac": achieved / INT8_MFMA_PEAK_TOPS,
-                     "traffic": measured_traffic("conv:" + spec), "kernel": "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
+                     "traffic": measured_traffic("conv:" + spec), "kernel": "conv_patch_kernel" if small_tile else "conv_nhwc_pipelined_kernel", "ops_per_launch": ops},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_conv(c, h, w, cout, k, pad, batch)
