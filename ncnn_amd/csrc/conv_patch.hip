@@ -54,14 +54,31 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const int8_t* __restric
     const int l32 = lane & 31, lhi = lane >> 5;
     const int twl = pl.twl, tw_mask = (1 << twl) - 1;
 
-    int img = blockIdx.z, tn = 0;
-    if (pl.tiles_n > 1)
+    // Workgroup ids are dealt round-robin to the 8 XCDs; they are remapped so that an XCD works on consecutive tiles
+    // (channel tiles of one pixel tile, then the tiles of one row of tiles, then the rows): neighbours share their
+    // patches' borders in that XCD's L2.
+    int b = blockIdx.x;
     {
-        img = (int)blockIdx.z / pl.tiles_n;
-        tn = (int)blockIdx.z - img * pl.tiles_n;
+        const int T = gridDim.x, xcd = b & 7, idx = b >> 3, rem = T & 7;
+        b = xcd * (T >> 3) + (xcd < rem ? xcd : rem) + idx;
+    }
+    b = __builtin_amdgcn_readfirstlane(b);
+    int tn = 0, txi, tyi, img;
+    {
+        int t = b;
+        if (pl.tiles_n > 1)
+        {
+            const int q = t / pl.tiles_n;
+            tn = t - q * pl.tiles_n;
+            t = q;
+        }
+        const int row = t / pl.tiles_x;
+        txi = t - row * pl.tiles_x;
+        img = row / pl.tiles_y;
+        tyi = row - img * pl.tiles_y;
     }
     const int col0 = tn * 64;
-    const int oy0 = (int)blockIdx.y * (32 >> twl), ox0 = (int)blockIdx.x << twl;
+    const int oy0 = tyi * (32 >> twl), ox0 = txi << twl;
     const int iy0 = oy0 * g.sh - g.pad_top, ix0 = ox0 * g.sw - g.pad_left;
 
     // ---- 1. this lane's weights: channel row col0 + wn*32 + l32, K bytes (2i + wk)*32 + lhi*16 .. +16 for its i-th step
@@ -360,7 +377,7 @@ static bool patch_plan(const NhwcGeom& g, int batch, PatchPlan& pl)
     pl.tiles_y = ceil_div(g.outh, 32 >> pl.twl);
     pl.tiles_n = ceil_div(g.cout, 64);
     pl.batch = batch;
-    return pl.tiles_y <= 65535 && (long long)batch * pl.tiles_n <= 65535;
+    return (long long)pl.tiles_x * pl.tiles_y * pl.tiles_n * batch < (1ll << 31);
 }
 
 bool conv_patch_supported(const NhwcGeom& g, int batch)
@@ -394,7 +411,7 @@ int launch_conv_patch(const NhwcGeom& g, const int8_t* wpk, const void* x, int x
     NCNNHIP_REQUIRE(patch_plan(g, epi.batch, pl), "convolution: this layer does not fit the small-tile kernel");
     NCNNHIP_REQUIRE(epi.batch >= 1 && (long long)epi.batch * g.outw * g.outh == (long long)g.npix, "convolution: pixel count and batch disagree");
     const size_t patch_bytes = (size_t)pl.pr * pl.pc * g.Cp;
-    dim3 grid((unsigned)pl.tiles_x, (unsigned)pl.tiles_y, (unsigned)(pl.batch * pl.tiles_n)), block(256);
+    dim3 grid((unsigned)((long long)pl.tiles_x * pl.tiles_y * pl.tiles_n * pl.batch)), block(256);
     const int8_t* xb = static_cast<const int8_t*>(x);
     const int per_wave = (pl.nsteps + 1) / 2;
 #define LAUNCH_PATCH(AIN_, MAXS_)                                                                                                                            \
