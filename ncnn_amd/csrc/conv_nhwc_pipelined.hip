@@ -44,6 +44,9 @@ __device__ __forceinline__ uint32_t pack4(const v4f& v)
 
 // MODE: how a lane finds its source bytes.  0: any geometry; 1: dense (1x1, stride 1, unpadded: one row of npix pixels,
 // also Gemm and InnerProduct); 2: taps of 16 or 32 bytes (the narrow-input image), a whole number of taps per K step.
+// 3: any geometry whose taps are whole 64-byte steps (tapK % 64 == 0): a K step then lies inside ONE tap, the same for every
+// lane, so the walk over taps is wavefront-uniform scalar arithmetic, and a lane's bounds test and address are computed
+// once per tap instead of once per step (a tap of 256 channels is four steps: the other three are a load and an add).
 // A template parameter because the choice sits inside the K loop: as run-time branches there it cost the 3x3 layers
 // of ResNet-50's last stages 2-4 us each (15.4 against 11.4 us for 256 -> 256 on 14 x 14, batch 16).
 //
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
 {
     constexpr bool dense = MODE == 1;
     constexpr bool STAGED = AIN != 1;
-    static_assert(!STAGED || (!GEMM && MODE != 2), "the quantising loader exists for convolutions on ordinary blobs");
+    static_assert(!STAGED || (!GEMM && MODE != 2 && MODE != 3), "the quantising loader exists for convolutions on ordinary blobs");
     constexpr int TM = BM / 64, TN = BN / 64; // 32x32 blocks per wavefront along pixels / channels
     constexpr int LAR = BM / 64;              // 64-row groups of the activation tile
     constexpr int LA = STAGED ? 0 : LAR, LB = BN / 64; // direct-to-LDS loads per wavefront per stage
@@ -176,6 +179,26 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         q0 = k - tap * g.tapK;
     }
     const int first_q0 = q0, first_tap = tap, first_ky = ky, first_kx = kx; // where the quantising loader starts (issue() moves the others on)
+    // MODE 3: the wavefront's position in K (the same in every lane) and, per lane, where the current tap's bytes of its
+    // row are (or the line of zeros) and how far the next step moves on (64 bytes, or nothing on the line of zeros)
+    int u_q0 = 0, u_tap = 0, u_ky = 0, u_kx = 0;
+    bool u_new_tap = true;
+    const int8_t* m3_src[LAR];
+    int m3_step[LAR];
+    if (MODE == 3)
+    {
+        const int k = step_begin * 64;
+        u_tap = k / g.tapK;
+        u_q0 = k - u_tap * g.tapK;
+        u_ky = u_tap / g.kw;
+        u_kx = u_tap - u_ky * g.kw;
+#pragma unroll
+        for (int i = 0; i < LAR; i++)
+        {
+            m3_src[i] = zero;
+            m3_step[i] = 0;
+        }
+    }
 
     // issues the loads of the next stage in sequence (s = 0, 1, 2, ... relative to step_begin)
     extern __shared__ __attribute__((aligned(1024))) int8_t a_tile[]; // quantising loader: [K/64][BM][64] activations, then [K/64][BN][64] weights, then the input cache
@@ -192,6 +215,28 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
                 const bool in = tap == 0 && a_iy0[i] == 0;
                 const int8_t* src = in ? a_base[i] + q0 : zero;
                 __builtin_amdgcn_global_load_lds((const AS1 void*)src, (AS3 void*)(stage + i * 4096), 16, 0, 0);
+            }
+        }
+        else if (MODE == 3)
+        {
+            if (u_new_tap) // (uniform)
+            {
+                const int dy = u_ky * g.dh, dx = u_kx * g.dw;
+                const bool tap_ok = u_tap < g.ntaps;
+#pragma unroll
+                for (int i = 0; i < LA; i++)
+                {
+                    const int iy = a_iy0[i] + dy, ix = a_ix0[i] + dx;
+                    const bool in = tap_ok && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                    m3_src[i] = in ? a_base[i] + ((size_t)iy * g.W + ix) * g.Cp + u_q0 + ld_chunk * 16 : zero;
+                    m3_step[i] = in ? 64 : 0;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < LA; i++)
+            {
+                __builtin_amdgcn_global_load_lds((const AS1 void*)m3_src[i], (AS3 void*)(stage + i * 4096), 16, 0, 0);
+                m3_src[i] += m3_step[i];
             }
         }
         else
@@ -215,6 +260,21 @@ __global__ __launch_bounds__(256) void conv_nhwc_pipelined_kernel(const int8_t* 
         {
             q0 += 64;
             if (q0 >= g.tapK) tap = 1; // past the only tap: the rest of K is the round-up, zero-filled
+        }
+        else if (MODE == 3)
+        {
+            u_q0 += 64;
+            u_new_tap = u_q0 >= g.tapK;
+            if (u_new_tap)
+            {
+                u_q0 = 0;
+                u_tap++;
+                if (++u_kx == g.kw)
+                {
+                    u_kx = 0;
+                    u_ky++;
+                }
+            }
         }
         else if (MODE == 2)
         {
@@ -1005,9 +1065,12 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
     }
     dim3 grid((unsigned)blocks), block(256);
     const GemmTail no_gemm = {0, 0, 0, 0, -1, 1.f, 1.f};
-    // addressing mode (the kernel's MODE); the K-split kernels exist for modes 0 and 1 only (a narrow-input layer has
+    // addressing mode (the kernel's MODE); the K-split kernels exist for modes 0, 1 and 3 only (a narrow-input layer has
     // too few K steps to be split)
-    const int mode = dense ? 1 : ((g.tapK == 16 || g.tapK == 32) && p.splits == 1) ? 2 : 0;
+    const int mode = dense ? 1 : ((g.tapK == 16 || g.tapK == 32) && p.splits == 1) ? 2 : (g.tapK % 64 == 0 && g.tapK == g.Cp) ? 3 : 0;
+#ifndef PIPE_RING
+#define PIPE_RING 3
+#endif
 #define LAUNCH_PIPE_MODE(BM_, BN_, ST_, SPLIT_, MODE_)                                                                                                          \
     hipLaunchKernelGGL((conv_nhwc_pipelined_kernel<BM_, BN_, ST_, SPLIT_, false, MODE_>), grid, block, 0, stream, wpk, x, g, epi, fusion, no_gemm, out_cp, out_cp, \
                        p.tiles_m, p.tiles_n, p.splits, p.steps_per_split, tile_magic(p.tiles_n), partial, counters, (const float*)0, 0)
@@ -1016,28 +1079,32 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
     {                                                                                                                                           \
         if (p.splits > 1 && mode == 1)                                                                                                          \
             LAUNCH_PIPE_MODE(BM_, BN_, ST_, true, 1);                                                                                           \
+        else if (p.splits > 1 && mode == 3)                                                                                                     \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, true, 3);                                                                                           \
         else if (p.splits > 1)                                                                                                                  \
             LAUNCH_PIPE_MODE(BM_, BN_, ST_, true, 0);                                                                                           \
         else if (mode == 1)                                                                                                                     \
             LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 1);                                                                                          \
         else if (mode == 2)                                                                                                                     \
             LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 2);                                                                                          \
+        else if (mode == 3)                                                                                                                     \
+            LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 3);                                                                                          \
         else                                                                                                                                    \
             LAUNCH_PIPE_MODE(BM_, BN_, ST_, false, 0);                                                                                          \
     } while (0)
     // three stages everywhere: deeper rings (4 to 6 stages) measured slower on every ResNet-50 / MobileNetV2 layer
     if (p.bm == 128 && p.bn == 256)
-        LAUNCH_PIPE(128, 256, 3);
+        LAUNCH_PIPE(128, 256, PIPE_RING);
     else if (p.bm == 128 && p.bn == 128)
-        LAUNCH_PIPE(128, 128, 3);
+        LAUNCH_PIPE(128, 128, PIPE_RING);
     else if (p.bm == 128)
-        LAUNCH_PIPE(128, 64, 3);
+        LAUNCH_PIPE(128, 64, PIPE_RING);
     else if (p.bn == 256)
-        LAUNCH_PIPE(64, 256, 3);
+        LAUNCH_PIPE(64, 256, PIPE_RING);
     else if (p.bn == 128)
-        LAUNCH_PIPE(64, 128, 3);
+        LAUNCH_PIPE(64, 128, PIPE_RING);
     else
-        LAUNCH_PIPE(64, 64, 3);
+        LAUNCH_PIPE(64, 64, PIPE_RING);
 #undef LAUNCH_PIPE
 #undef LAUNCH_PIPE_MODE
     return launch_status("conv_nhwc_pipelined_kernel");
