@@ -9,7 +9,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 LIBNCNNHIP = os.path.join(LIBDIR, "libncnnhip.so")
 
-HIP_SOURCES = ["runtime.hip", "quantize.hip", "gemm_int8.hip", "gemm_int8_pipelined.hip", "conv_int8.hip", "conv_nhwc.hip", "conv_nhwc_pipelined.hip", "conv_pointwise.hip", "conv_resident.hip", "conv_patch.hip", "nhwc_ops.hip", "attention.hip", "blockquant.hip", "peaks.hip"]
+HIP_SOURCES = ["runtime.hip", "quantize.hip", "gemm_int8.hip", "gemm_int8_pipelined.hip", "conv_int8.hip", "conv_nhwc.hip", "conv_nhwc_pipelined.hip", "conv_nhwc_pipelined_split.hip", "conv_nhwc_pipelined_staged.hip", "conv_pointwise.hip", "conv_resident.hip", "conv_patch.hip", "nhwc_ops.hip", "attention.hip", "blockquant.hip", "peaks.hip"]
 
 # -ffp-contract=off: the reference arithmetic is separate mul and add, never FMA.
 # packed-fp32 ops are switched off for this pool's gfx950 parts.
