@@ -75,6 +75,7 @@ bool conv_patch_pays(const NhwcGeom& g, int batch, int x_elemsize);
 int launch_conv_patch(const NhwcGeom& g, const int8_t* wpk, const void* x, int x_elemsize, const float* x_scale, const ConvEpilogue& epi, const ConvFusion& fusion,
                       int out_cp, hipStream_t stream);
 bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);
+bool conv_pointwise_stem_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp); // the narrow-input first layer on the same kernel
 // The weights-resident kernel for layers with many output pixels (conv_resident.hip): does this problem fit it, and its
 // launch.  The pipelined launch asks first.
 bool conv_resident_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp);

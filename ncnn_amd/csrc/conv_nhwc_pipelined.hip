@@ -49,7 +49,7 @@ size_t conv_nhwc_pipelined_workspace_words(int cout, long long npix, int steps)
 int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp,
                                void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
-    if (conv_pointwise_fits(g_in, epi, fusion, out_cp)) return launch_conv_pointwise(g_in, wpk, x, epi, out_cp, stream);
+    if (conv_pointwise_fits(g_in, epi, fusion, out_cp) || conv_pointwise_stem_fits(g_in, epi, fusion, out_cp)) return launch_conv_pointwise(g_in, wpk, x, epi, out_cp, stream);
     if (conv_resident_fits(g_in, epi, fusion, out_cp)) return launch_conv_resident(g_in, wpk, x, epi, fusion, out_cp, stream);
     NhwcGeom g = g_in;
     // A 1x1, stride-1, unpadded layer reads input pixel n for output pixel n, whatever the image shape: present it as

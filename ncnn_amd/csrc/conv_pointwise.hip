@@ -16,6 +16,11 @@
 //   * the four packed words of a lane (same channels, four pixel groups) and those of the lanes 16, 32 and 48 away
 //     (same pixels, the other channels) are a 4x4 matrix across lane rows and registers: four lane-row swaps transpose
 //     it, after which every lane holds 16 consecutive output bytes of one pixel: one 16-byte store.
+// The same kernel serves the narrow-input first layer of a net (STEM: at most 4 input channels, the quantised image of 4
+// bytes per pixel with its physical zero border, kernels of up to 4 x 4 taps at any stride): there a 16-byte operand
+// chunk is 4 neighbouring pixels of one kernel row, and a lane finds its chunk by its output pixel's position in the
+// bordered image.  Everything after the MFMAs is shared.  (KSTEPS > 1 -- longer K -- compiles and is bit-exact, but
+// measured slower than the pipelined kernel and is not launched.)
 // About 9 vector instructions per output value at 4+ wavefronts per SIMD.  Activations: none, ReLU, clip (literal or,
 // when the tables allow it, folded into the requantising clamp: clip_folds_into_requantise in common.h), others.
 #include "common.h"
@@ -76,19 +81,25 @@ __device__ __forceinline__ void pointwise_requantise(const v4i (&acc)[4], const 
 // The channel tables (input scale, bias, output scale, clamp bounds) are worked out once per workgroup into LDS, with the
 // decision whether the clip folds into the clamp; a wavefront keeps its pixel block's four operands in registers for all
 // its channel blocks and fetches the next channel block's weights while it requantises this one.
-__global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* __restrict__ wpk /* [cout][64] */, const int8_t* __restrict__ x, int cp_in, int npix,
-                                                                   int cout, int out_cp, const float* __restrict__ scale_in, const float* __restrict__ bias_tab,
+// KSTEPS: 64-byte K steps (MFMAs per result); STEM: the narrow-input geometry (g is the bordered image then: pixels 4 bytes
+// apart, kw counts groups of 4 pixels, no padding left to apply).  G = 4 (one wavefront per pixel block, every channel block)
+// exists for layers of one or two channel blocks.
+template<int KSTEPS, bool STEM>
+__global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* __restrict__ wpk /* [cout][KSTEPS * 64] */, const int8_t* __restrict__ x, NhwcGeom g,
+                                                                   int out_cp, const float* __restrict__ scale_in, const float* __restrict__ bias_tab,
                                                                    const float* __restrict__ scale_out, ncnnhip_activation act, int8_t* __restrict__ out,
                                                                    int channel_blocks, int G)
 {
     extern __shared__ __attribute__((aligned(16))) float pw_tab[]; // [5][out_cp]: input scale, bias, output scale, clamp low, clamp high
+    typedef int v4i_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+    const int cp_in = g.Cp, npix = g.npix, cout = g.cout;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c16 = lane & 15, q = lane >> 4;
     const int pixel_blocks = (npix + 63) >> 6;
-    const int pb = (int)blockIdx.x * G + (G == 2 ? (wave & 1) : 0);
-    const int cb_first = G == 2 ? (wave >> 1) : wave;
-    const int cb_step = 4 / G;
+    const int pb = (int)blockIdx.x * G + (G == 4 ? wave : G == 2 ? (wave & 1) : 0);
+    const int cb_first = G == 4 ? 0 : G == 2 ? (wave >> 1) : wave;
+    const int cb_step = G == 4 ? 1 : 4 / G;
     const bool live = pb < pixel_blocks; // (uniform per wavefront; a dead wavefront still helps with the tables and the barrier)
 
     // ---- this wavefront's pixels: lane = pixel pb*64 + pg*16 + c16, bytes q*16 .. +16.  Nothing is selected after the load: a
@@ -96,23 +107,71 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
     // zero there (the packed rows are zero-filled from cp_in up); a lane whose pixel lies beyond the end reads the last pixel,
     // and its results are never stored.
     const unsigned koff = q * 16 < cp_in ? q * 16 : 0;
-    v4i fx[4];
+    v4i fx[4][KSTEPS];
     {
         const int pbl = live ? pb : pixel_blocks - 1;
-#pragma unroll
-        for (int pg = 0; pg < 4; pg++)
+        if constexpr (STEM)
         {
-            int p = pbl * 64 + pg * 16 + c16;
-            if (p >= npix) p = npix - 1;
-            fx[pg] = *reinterpret_cast<const v4i*>(x + (size_t)p * cp_in + koff);
+            // chunk c = 4 * step + q of K is kernel row c / kw, pixel group c % kw: (row * dh * W + group * 4) pixels from the
+            // output pixel's corner; chunks beyond the kernel meet zero weights and read the first chunk again
+            int chunk_off[KSTEPS];
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++)
+            {
+                int c = 4 * st + q;
+                if (c >= g.ntaps) c = 0;
+                const int ky = small_div(c, g.kw);
+                chunk_off[st] = (ky * g.dh * g.W + (c - ky * g.kw) * 4) * 4;
+            }
+            // the block's first pixel by (uniform) division, the lane's own by walking on from there
+            const int plane = g.outw * g.outh;
+            const int p0 = pbl * 64;
+            const int img0 = p0 / plane, rem0 = p0 - img0 * plane;
+            const int oy0 = rem0 / g.outw, ox0 = rem0 - oy0 * g.outw;
+#pragma unroll
+            for (int pg = 0; pg < 4; pg++)
+            {
+                int step = pg * 16 + c16;
+                if (p0 + step >= npix) step = npix - 1 - p0; // a pixel beyond the end reads the last one; never stored
+                int img = img0, oy = oy0, ox = ox0 + step;
+                while (ox >= g.outw)
+                {
+                    ox -= g.outw;
+                    if (++oy == g.outh)
+                    {
+                        oy = 0;
+                        img++;
+                    }
+                }
+                const int8_t* corner = x + ((size_t)(img * g.H + oy * g.sh) * g.W + ox * g.sw) * 4;
+#pragma unroll
+                for (int st = 0; st < KSTEPS; st++) fx[pg][st] = *reinterpret_cast<const v4i_dword_aligned*>(corner + chunk_off[st]);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int pg = 0; pg < 4; pg++)
+            {
+                int p = pbl * 64 + pg * 16 + c16;
+                if (p >= npix) p = npix - 1;
+                fx[pg][0] = *reinterpret_cast<const v4i*>(x + (size_t)p * cp_in + koff);
+            }
         }
     }
+    struct Weights
+    {
+        v4i w[KSTEPS];
+    };
     auto load_weights = [&](int cb) {
         int ch = cb * 16 + c16;
         if (ch >= cout) ch = cout - 1; // rows beyond cout give values that the zero tables turn into zero bytes
-        return *reinterpret_cast<const v4i*>(wpk + (size_t)ch * 64 + q * 16);
+        Weights r;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; st++) r.w[st] = *reinterpret_cast<const v4i*>(wpk + (size_t)ch * (KSTEPS * 64) + st * 64 + q * 16);
+        return r;
     };
-    v4i fw = load_weights(cb_first < channel_blocks ? cb_first : 0);
+    Weights fw = load_weights(cb_first < channel_blocks ? cb_first : 0);
 
     // ---- tables of every channel, once per workgroup.  Channels from cout up (the blob's padding) get scale 0 and bias -0:
     // their bytes come out 0.  A clip folds into the requantising clamp when every table allows it (finite tables, products
@@ -149,7 +208,7 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
     int8_t* orow = out + (size_t)p_store * out_cp;
     for (int cb = cb_first; cb < channel_blocks; cb += cb_step)
     {
-        const v4i w_now = fw;
+        const Weights w_now = fw;
         if (cb + cb_step < channel_blocks) fw = load_weights(cb + cb_step); // in flight while this block is requantised
         const float* t = pw_tab + cb * 16 + 4 * q;
         const v4f vsi = *reinterpret_cast<const v4f*>(t), vbi = *reinterpret_cast<const v4f*>(t + out_cp), vso = *reinterpret_cast<const v4f*>(t + 2 * out_cp);
@@ -158,7 +217,12 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
         const float q_lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, q_hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
         v4i acc[4];
 #pragma unroll
-        for (int pg = 0; pg < 4; pg++) acc[pg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w_now, fx[pg], v4i{0, 0, 0, 0}, 0, 0, 0);
+        for (int pg = 0; pg < 4; pg++)
+        {
+            acc[pg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w_now.w[0], fx[pg][0], v4i{0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+            for (int st = 1; st < KSTEPS; st++) acc[pg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w_now.w[st], fx[pg][st], acc[pg], 0, 0, 0);
+        }
 
         uint32_t word[4];
         if (mode == 203)
@@ -195,18 +259,44 @@ bool conv_pointwise_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvF
     return dense && plain && aligned && epi.scale_out && g.Cp <= 64 && g.Cp % 16 == 0 && g.K == 64 && g.cout % 4 == 0 && out_cp % 16 == 0 && g.npix >= (1 << 16); // below that the general kernel's finer split of the work is as fast or faster (measured again with this kernel's present form on MobileNetV2's 28 x 28 to 7 x 7 layers at batch 32: 5.7-6.1 us there against 6.9-10 here)
 }
 
+// The narrow-input first layer (ncnnhip_conv_int8_stem presents it as pixels 4 bytes apart whose taps are groups of 4
+// pixels, with the border inside the image): int8 output, no fused tail, as many pixels as the 1x1 layers need before this
+// kernel is the faster one, and a K of ONE step (kernels of up to 4 rows of up to 4 taps: MobileNetV2's 3x3 first layer at
+// batch 32 17.4 -> 10.3 us).  With four steps (ResNet-50's 7x7: 14 chunks) it measured SLOWER than the pipelined kernel,
+// 18.9 against 16.1 us at batch 16 and 187 against 132 at batch 128: sixteen 16-byte gathers per lane from windows that
+// overlap their neighbours' by half, fetched again by the wavefront that takes the other channel blocks.
+bool conv_pointwise_stem_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp)
+{
+    const bool stem = g.Cp == 4 && g.tapK == 16 && g.dw == 4 && g.pad_top == 0 && g.pad_left == 0 && g.pad_word == 0 && g.ntaps == g.kw * g.kh;
+    const bool plain = !fusion.residual && !fusion.relu_after && !fusion.q8_out && !epi.acc_out;
+    const uintptr_t tables = reinterpret_cast<uintptr_t>(epi.scale_in) | reinterpret_cast<uintptr_t>(epi.bias) | reinterpret_cast<uintptr_t>(epi.scale_out);
+    const bool aligned = ((tables | reinterpret_cast<uintptr_t>(epi.out)) & 15) == 0;
+    return stem && plain && aligned && epi.scale_out && g.ntaps <= 4 && g.K == 64 && g.cout % 4 == 0 && out_cp % 16 == 0 &&
+           g.npix >= (1 << 16) && (long long)g.npix + 64 < (1ll << 31);
+}
+
 int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x, const ConvEpilogue& epi, int out_cp, hipStream_t stream)
 {
     NCNNHIP_REQUIRE(((reinterpret_cast<uintptr_t>(wpk) | reinterpret_cast<uintptr_t>(x)) & 15) == 0, "convolution: operands must be 16-byte aligned");
     const int channel_blocks = out_cp / 16;
     const int pixel_blocks = ceil_div(g.npix, 64);
+    const size_t tab_bytes = (size_t)5 * out_cp * sizeof(float);
+    NCNNHIP_REQUIRE(tab_bytes <= 60 * 1024, "convolution: %d output channels are too many for the pointwise kernel's tables", g.cout);
+    if (g.Cp == 4 && g.tapK == 16)
+    {
+        // one wavefront per pixel block walks one or two channel blocks; more are dealt to wavefront pairs as below
+        const int Gs = channel_blocks <= 2 ? 4 : 2;
+        const dim3 grid((unsigned)ceil_div(pixel_blocks, Gs));
+        NCNNHIP_REQUIRE(g.K == 64 && g.ntaps <= 4, "convolution: %d bytes of K in the narrow-input form of the pointwise kernel", g.K);
+        hipLaunchKernelGGL((conv_pointwise_int8_kernel<1, true>), grid, dim3(256), tab_bytes, stream, wpk, x, g, out_cp, epi.scale_in, epi.bias, epi.scale_out,
+                           epi.act, static_cast<int8_t*>(epi.out), channel_blocks, Gs);
+        return launch_status("conv_pointwise_int8_kernel (narrow input)");
+    }
     // pixel blocks per workgroup: two, each with two wavefronts that take the even and the odd channel blocks (measured on
     // MobileNetV2's 16 -> 96 expansion on 112 x 112 at batch 32: 19.8 us, against 23.1 for one block with four wavefronts and
     // 31 for four blocks with one wavefront each); a layer too small for that many workgroups keeps one block per workgroup
     const int G = pixel_blocks >= 1024 ? 2 : 1;
-    const size_t lds = (size_t)5 * out_cp * sizeof(float);
-    NCNNHIP_REQUIRE(lds <= 60 * 1024, "convolution: %d output channels are too many for the pointwise kernel's tables", g.cout);
-    hipLaunchKernelGGL(conv_pointwise_int8_kernel, dim3((unsigned)ceil_div(pixel_blocks, G)), dim3(256), lds, stream, wpk, x, g.Cp, g.npix, g.cout, out_cp, epi.scale_in,
+    hipLaunchKernelGGL((conv_pointwise_int8_kernel<1, false>), dim3((unsigned)ceil_div(pixel_blocks, G)), dim3(256), tab_bytes, stream, wpk, x, g, out_cp, epi.scale_in,
                        epi.bias, epi.scale_out, epi.act, static_cast<int8_t*>(epi.out), channel_blocks, G);
     return launch_status("conv_pointwise_int8_kernel");
 }

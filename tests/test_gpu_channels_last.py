@@ -327,6 +327,30 @@ def test_stem_convolution_matches_oracle(rt, c, h, w, outc, kernel, stride, pads
     assert got.dtype == want.dtype and np.array_equal(got[0], want)
 
 
+@pytest.mark.parametrize("batch,c,h,w,outc,kernel,stride,pads,term,act,act_params,flip", [
+    (1, 3, 514, 514, 32, (3, 3), (2, 2), (1, 1, 1, 1), 101, 3, (0.0, 6.0), False),     # MobileNetV2's first layer: one K step, two channel blocks
+    (1, 3, 520, 518, 64, (7, 7), (2, 2), (3, 3, 3, 3), 102, 1, (0.0, 0.0), False),     # ResNet-50's at the same size: 14 chunks, stays on the pipelined kernel
+    (3, 3, 300, 302, 24, (3, 3), (2, 2), (-233, -233, -233, -233), 101, 0, (0.0, 0.0), False),  # pixel blocks that cross rows and images; 24 channels in 32
+    (2, 4, 186, 190, 40, (3, 3), (1, 1), (1, 1, 1, 1), 102, 3, (-1.0, 2.0), False),    # stride 1: chunks on 4-byte boundaries; a negative clip bound
+    (1, 1, 260, 259, 16, (4, 4), (1, 1), (0, 0, 0, 0), 101, 1, (0.0, 0.0), True),      # all four rows of a step in use; negative output scales
+    (2, 3, 372, 370, 100, (4, 4), (2, 2), (1, 1, 1, 1), 102, 2, (0.1, 0.0), False),    # seven channel blocks, the last partly padding
+])
+def test_stem_convolution_on_the_pointwise_kernel(rt, batch, c, h, w, outc, kernel, stride, pads, term, act, act_params, flip):
+    """A first layer of up to 4 x 4 taps with 65536 output pixels and more and an int8 output runs on the pointwise kernel's
+    narrow-input form (operands straight from the bordered image): bit for bit the oracle's, as is the 7 x 7 layer of the
+    same size beside it."""
+    _say("stem on the pointwise kernel", batch, c, h, w, outc, kernel, stride, term, act)
+    x, wq, b, ws, ins, tops = cases.conv_case(c * 100 + outc + kernel[0], c, h, w, outc, kernel, 1, term, True, False, batch=batch)
+    if flip:
+        tops = -tops
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, 1), stride, pads, 0.0, 1, 1, term, act, act_params)
+    got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, (1, 1), stride, pads, 0.0, 1, term, act, act_params, stem=True)
+    assert got.shape[2] * got.shape[3] * batch >= 65536
+    for i in range(batch):
+        want = oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], tops[0])
+        assert got.dtype == want.dtype and np.array_equal(got[i], want), "sample %d" % i
+
+
 def test_stem_convolution_batch_int8_input_and_fused_tail(rt):
     """Batch of 3, an int8 input blob (already quantised upstream), and the fused tail (residual, ReLU, quantised copy)."""
     c, h, w, outc, kernel = 3, 18, 22, 48, (3, 3)
