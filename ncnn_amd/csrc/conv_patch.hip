@@ -4,14 +4,15 @@
 // One workgroup (4 wavefronts) owns a two-dimensional tile of 32 output pixels (32x1, 16x2, 8x4, ... whichever covers
 // the output plane with the fewest tiles) and 64 output channels.  A 2-D tile keeps the halo small: 8x4 outputs of a
 // 3x3 layer read 10x6 input pixels, where 32 consecutive outputs of a 56-wide image read a run of 146.
-//   1. Every lane requests its share of the weights straight into registers (a lane's B operand of
-//      v_mfma_i32_32x32x32_i8 is 16 consecutive K bytes of one channel row: no staging, nothing shared).
-//   2. The input patch -- patch rows x patch columns x Cp channels -- is fetched once, quantised on the way when the
-//      blob is still fp32 / fp16 (Quantize::forward, src/layer/quantize.cpp:48-111, one scale), and written to LDS as
-//      [row][column][Cp] int8 with ZEROS wherever the patch leaves the image: the convolution's border
-//      (src/layer/convolution.cpp:383-508 pads after it quantises, with zero bytes).
-//   3. The K loop touches LDS only and has no bounds tests: the A operand of output pixel (ty, tx) and tap (ky, kx) is
-//      16 bytes at ((ty*sh + ky*dh) * patch columns + tx*sw + kx*dw) * Cp + channel -- a per-lane base plus a
+//   1. The input patch -- patch rows x patch columns x Cp channels -- is requested first, 16 bytes per lane and load (it is
+//      what the workgroup waits for: load, quantise, LDS, barrier), then every lane requests its share of the weights
+//      straight into registers (a lane's B operand of v_mfma_i32_32x32x32_i8 is 16 consecutive K bytes of one channel
+//      row: no staging, nothing shared).
+//   2. The patch is quantised on the way when the blob is still fp32 / fp16 (Quantize::forward,
+//      src/layer/quantize.cpp:48-111, one scale) and written to LDS as [row][column][Cp] int8 with ZEROS wherever it
+//      leaves the image: the convolution's border (src/layer/convolution.cpp:383-508 pads after it quantises, with zero bytes).
+//   3. The K loop touches LDS and registers only and has no bounds tests (its LDS reads all go out before the first
+//      product): the A operand of output pixel (ty, tx) and tap (ky, kx) is 16 bytes at ((ty*sh + ky*dh) * patch columns + tx*sw + kx*dw) * Cp + channel -- a per-lane base plus a
 //      wavefront-uniform offset.  The four wavefronts are 2 channel halves x 2 K halves (even / odd 32-byte steps).
 //   4. The two K halves exchange half of their accumulators through LDS (integer addition: exact in any order), so each
 //      wavefront finishes 16 pixels x 32 channels; results go through LDS once more so that global memory sees whole
@@ -81,7 +82,79 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const int8_t* __restric
     const int oy0 = tyi * (32 >> twl), ox0 = txi << twl;
     const int iy0 = oy0 * g.sh - g.pad_top, ix0 = ox0 * g.sw - g.pad_left;
 
-    // ---- 1. this lane's weights: channel row col0 + wn*32 + l32, K bytes (2i + wk)*32 + lhi*16 .. +16 for its i-th step
+    // ---- 1. the input patch, 16 bytes of the blob per lane and load: the first round of requests goes out before anything
+    // else (the patch is what the workgroup waits for first: load, quantise, LDS, barrier); the weights follow
+    constexpr int VPI = 16 / AIN;          // values per load
+    constexpr int INFL = 8;                // loads in flight per lane
+    const int ipp = g.Cp / VPI;            // loads per pixel
+    const int rowitems = pl.pc * ipp;      // per patch row
+    const int nitems = pl.pr * rowitems;
+    const int8_t* img_base = x + (size_t)img * g.H * g.W * g.Cp * AIN;
+    auto patch_request = [&](int base, v4i (&raw)[INFL], unsigned& inside) {
+        inside = 0;
+#pragma unroll
+        for (int j = 0; j < INFL; j++)
+        {
+            if (base + j * 256 >= nitems) break; // (uniform) nobody has a j-th item
+            int qi = base + j * 256 + (int)threadIdx.x;
+            if (qi >= nitems) qi = nitems - 1;
+            const int row = small_div(qi, rowitems);
+            const int rem = qi - row * rowitems;
+            const int col = small_div(rem, ipp);
+            const int c = rem - col * ipp;
+            const int iy = iy0 + row, ix = ix0 + col;
+            const bool in = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+            const size_t off = in ? ((size_t)(iy * g.W + ix) * g.Cp + c * VPI) * AIN : 0;
+            raw[j] = *reinterpret_cast<const v4i*>(img_base + off);
+            inside |= in ? 1u << j : 0u;
+        }
+    };
+    auto patch_store = [&](int base, const v4i (&raw)[INFL], unsigned inside, float sc) {
+#pragma unroll
+        for (int j = 0; j < INFL; j++)
+        {
+            if (base + j * 256 >= nitems) break;
+            const int qi = base + j * 256 + (int)threadIdx.x;
+            const bool in = (inside >> j) & 1u;
+            if constexpr (AIN == 1)
+            {
+                const v4i w = in ? raw[j] : v4i{0, 0, 0, 0};
+                if (qi < nitems) *reinterpret_cast<v4i*>(patch + (size_t)qi * 16) = w;
+            }
+            else if constexpr (AIN == 4)
+            {
+                float v0 = mul_rn(__int_as_float(raw[j][0]), sc), v1 = mul_rn(__int_as_float(raw[j][1]), sc);
+                float v2 = mul_rn(__int_as_float(raw[j][2]), sc), v3 = mul_rn(__int_as_float(raw[j][3]), sc);
+                float2int8_as_float_x4(v0, v1, v2, v3);
+                const uint32_t word = pack4_quantised(v0, v1, v2, v3);
+                if (qi < nitems) *reinterpret_cast<uint32_t*>(patch + (size_t)qi * 4) = in ? word : 0u;
+            }
+            else
+            {
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                {
+                    const unsigned pair = (unsigned)raw[j][e]; // two halves, the first in the low 16 bits
+                    v[2 * e] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair & 0xffffu)), sc);
+                    v[2 * e + 1] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair >> 16)), sc);
+                }
+                float2int8_as_float_x4(v[0], v[1], v[2], v[3]);
+                float2int8_as_float_x4(v[4], v[5], v[6], v[7]);
+                typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                v2u w = {pack4_quantised(v[0], v[1], v[2], v[3]), pack4_quantised(v[4], v[5], v[6], v[7])};
+                if (!in) w = v2u{0u, 0u};
+                if (qi < nitems) *reinterpret_cast<v2u*>(patch + (size_t)qi * 8) = w;
+            }
+        }
+    };
+    v4i raw0[INFL];
+    unsigned inside0;
+    patch_request(0, raw0, inside0);
+    float sc = 0.f;
+    if constexpr (AIN != 1) sc = a_scale[0];
+
+    // ---- 2. this lane's weights: channel row col0 + wn*32 + l32, K bytes (2i + wk)*32 + lhi*16 .. +16 for its i-th step
     const int ch = col0 + wn * 32 + l32;
     const int chc = ch < g.cout ? ch : g.cout - 1; // a valid row; its products land in columns nobody stores
     const int my_steps = (pl.nsteps - wk + 1) >> 1;
@@ -98,74 +171,14 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const int8_t* __restric
     const float raw_bias = (epi.bias ? epi.bias : epi.scale_in)[chc];
     const float raw_s_out = (epi.scale_out ? epi.scale_out : epi.scale_in)[chc];
 
-    // ---- 2. the input patch -> LDS, 16 bytes of the blob per lane and load
+    // ---- the patch -> LDS (quantised on the way when the blob is fp32 / fp16); further rounds for a patch of more than 2048 loads
+    patch_store(0, raw0, inside0, sc);
+    for (int base = 256 * INFL; base < nitems; base += 256 * INFL)
     {
-        constexpr int VPI = 16 / AIN;          // values per load
-        const int ipp = g.Cp / VPI;            // loads per pixel
-        const int rowitems = pl.pc * ipp;      // per patch row
-        const int nitems = pl.pr * rowitems;
-        float sc = 0.f;
-        if constexpr (AIN != 1) sc = a_scale[0];
-        const int8_t* img_base = x + (size_t)img * g.H * g.W * g.Cp * AIN;
-        constexpr int INFL = 8; // loads in flight per lane
-        for (int base = 0; base < nitems; base += 256 * INFL)
-        {
-            v4i raw[INFL];
-            unsigned inside = 0;
-#pragma unroll
-            for (int j = 0; j < INFL; j++)
-            {
-                if (base + j * 256 >= nitems) break; // (uniform) nobody has a j-th item
-                int qi = base + j * 256 + (int)threadIdx.x;
-                if (qi >= nitems) qi = nitems - 1;
-                const int row = small_div(qi, rowitems);
-                const int rem = qi - row * rowitems;
-                const int col = small_div(rem, ipp);
-                const int c = rem - col * ipp;
-                const int iy = iy0 + row, ix = ix0 + col;
-                const bool in = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
-                const size_t off = in ? ((size_t)(iy * g.W + ix) * g.Cp + c * VPI) * AIN : 0;
-                raw[j] = *reinterpret_cast<const v4i*>(img_base + off);
-                inside |= in ? 1u << j : 0u;
-            }
-#pragma unroll
-            for (int j = 0; j < INFL; j++)
-            {
-                if (base + j * 256 >= nitems) break;
-                const int qi = base + j * 256 + (int)threadIdx.x;
-                const bool in = (inside >> j) & 1u;
-                if constexpr (AIN == 1)
-                {
-                    const v4i w = in ? raw[j] : v4i{0, 0, 0, 0};
-                    if (qi < nitems) *reinterpret_cast<v4i*>(patch + (size_t)qi * 16) = w;
-                }
-                else if constexpr (AIN == 4)
-                {
-                    float v0 = mul_rn(__int_as_float(raw[j][0]), sc), v1 = mul_rn(__int_as_float(raw[j][1]), sc);
-                    float v2 = mul_rn(__int_as_float(raw[j][2]), sc), v3 = mul_rn(__int_as_float(raw[j][3]), sc);
-                    float2int8_as_float_x4(v0, v1, v2, v3);
-                    const uint32_t word = pack4_quantised(v0, v1, v2, v3);
-                    if (qi < nitems) *reinterpret_cast<uint32_t*>(patch + (size_t)qi * 4) = in ? word : 0u;
-                }
-                else
-                {
-                    float v[8];
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                    {
-                        const unsigned pair = (unsigned)raw[j][e]; // two halves, the first in the low 16 bits
-                        v[2 * e] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair & 0xffffu)), sc);
-                        v[2 * e + 1] = mul_rn((float)__builtin_bit_cast(_Float16, (unsigned short)(pair >> 16)), sc);
-                    }
-                    float2int8_as_float_x4(v[0], v[1], v[2], v[3]);
-                    float2int8_as_float_x4(v[4], v[5], v[6], v[7]);
-                    typedef unsigned v2u __attribute__((ext_vector_type(2)));
-                    v2u w = {pack4_quantised(v[0], v[1], v[2], v[3]), pack4_quantised(v[4], v[5], v[6], v[7])};
-                    if (!in) w = v2u{0u, 0u};
-                    if (qi < nitems) *reinterpret_cast<v2u*>(patch + (size_t)qi * 8) = w;
-                }
-            }
-        }
+        v4i raw[INFL];
+        unsigned inside;
+        patch_request(base, raw, inside);
+        patch_store(base, raw, inside, sc);
     }
     __syncthreads();
 
@@ -187,24 +200,27 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const int8_t* __restric
                 ky++;
             }
         }
+        // every A operand is requested before the first product (a step beyond this wavefront's share reads the first one again)
+        v4i fa[MAXS];
 #pragma unroll
         for (int i = 0; i < MAXS; i++)
-            if (i < my_steps)
+        {
+            const int off = i < my_steps ? ((ky * g.dh) * pl.pc + kx * g.dw) * g.Cp + q : 0;
+            fa[i] = *reinterpret_cast<const v4i*>(a_lane + off);
+            q += 64;
+            while (q >= g.tapK)
             {
-                const int off = ((ky * g.dh) * pl.pc + kx * g.dw) * g.Cp + q;
-                const v4i fa = *reinterpret_cast<const v4i*>(a_lane + off);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, bw[i], acc, 0, 0, 0);
-                q += 64;
-                while (q >= g.tapK)
+                q -= g.tapK;
+                if (++kx == g.kw)
                 {
-                    q -= g.tapK;
-                    if (++kx == g.kw)
-                    {
-                        kx = 0;
-                        ky++;
-                    }
+                    kx = 0;
+                    ky++;
                 }
             }
+        }
+#pragma unroll
+        for (int i = 0; i < MAXS; i++)
+            if (i < my_steps) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], bw[i], acc, 0, 0, 0);
     }
 
     // ---- 4. epilogue
