@@ -100,10 +100,11 @@ int Gemm_hip::load_param(const ParamDict& pd)
     }
     // one bottom blob is enough when two of the three operands are constants
     if (constantA + constantB + constantC == 2) one_blob_only = true;
-    // blobs stay in HBM for the form a network layer has: A is the only input, B (and C, if any) are constants, nothing
-    // is transposed on the way in or out.  Every other form takes host Mats as before.
-    support_hip = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottoms.size() == 1
-                  && (quantize_term != 0);
+    // Blobs stay in HBM for every int8 form whose output is a 2-D blob: constant or dynamic A, B and C, transposed inputs,
+    // transposed output (Gemm::forward_int8, src/layer/gemm.cpp:745-966, runs them all in place as well).  output_N1M (a 3-D
+    // output) and a block-quantised B with a second bottom blob take host Mats.
+    support_hip = quantize_term != 0 && output_N1M == 0 && !bottoms.empty()
+                  && (!term_is_block_quant(quantize_term) || (constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && bottoms.size() == 1));
     return 0;
 }
 
@@ -216,8 +217,9 @@ int Gemm_hip::create_pipeline(const Option&)
             }
         }
     }
-    // the device-resident form needs B ready on the device (int8 rows or block-quantised fields)
-    support_hip = support_hip && ret == 0 && (weight_block_quantize || b_ready_int8);
+    // the device-resident forms need a constant B ready on the device (int8 rows, block-quantised fields, or the fp32 table
+    // the forward pass quantises as the reference does, src/layer/gemm.cpp:826-860)
+    support_hip = support_hip && ret == 0 && (weight_block_quantize || b_ready_int8 || constantB == 0 || (d_B && B_data.elemsize == 4u));
     if (ret != 0) destroy_pipeline(Option());
     return ret;
 }
@@ -256,9 +258,52 @@ int Gemm_hip::forward_hip(const HipMat& bottom_blob, HipMat& top_blob, HipComman
     return ret;
 }
 
-int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option&) const
+// One operand of the general form as it lies in HBM.  A 1-D or 2-D blob is the matrix itself, [rows][cols] with `stride`
+// elements from row to row; a 3-D blob of height 1 -- c rows of w values to the reference (src/layer/gemm.cpp:769-785 reads
+// A0.channel(j)[i]) -- is channels-last here, i.e. the TRANSPOSE of that matrix, [w][cp].
+struct DeviceOperand
 {
-    if (bottom_blobs.size() != 1 || top_blobs.empty() || !d_B) return -1;
+    const char* data; // sample 0
+    size_t sample_bytes;
+    int rows, cols;   // of the matrix the reference sees
+    size_t stride;    // of the stored matrix, in elements
+    bool stored_transposed;
+    int n;
+};
+
+static bool device_operand(const HipMat& m, DeviceOperand& v)
+{
+    if (m.empty() || m.elemsize != 4u) return false;
+    v.data = (const char*)m.data;
+    v.n = m.n;
+    if (m.dims == 1 || m.dims == 2)
+    {
+        v.rows = m.dims == 2 ? m.h : 1;
+        v.cols = m.w;
+        v.stride = (size_t)m.w;
+        v.stored_transposed = false;
+        v.sample_bytes = (size_t)v.rows * v.cols * 4;
+        return true;
+    }
+    if (m.dims == 3 && m.h == 1 && !m.narrow())
+    {
+        v.rows = m.c;
+        v.cols = m.w;
+        v.stride = (size_t)m.cp;
+        v.stored_transposed = true;
+        v.sample_bytes = (size_t)m.w * m.cp * 4;
+        return true;
+    }
+    return false;
+}
+
+int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& opt) const
+{
+    if (bottom_blobs.empty() || top_blobs.empty()) return -1;
+    const bool network_form = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && bottom_blobs.size() == 1
+                              && (weight_block_quantize || b_ready_int8) && (bottom_blobs[0].dims == 1 || bottom_blobs[0].dims == 2);
+    if (!network_form) return forward_hip_general(bottom_blobs, top_blobs[0], cmd, opt);
+    if (!d_B) return -1;
     const HipMat& A = bottom_blobs[0];
     if (A.elemsize != 4u || (A.dims != 1 && A.dims != 2))
     {
@@ -318,6 +363,261 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
     rc = ncnnhip_gemm_int8((const int8_t*)q, aq_stride, (const int8_t*)d_B, (size_t)K, M, N, K, (const float*)sa, (const float*)d_B_scale, 1, d_c, bt, alpha, beta, 0,
                            (float*)top.data, (size_t)N, 0, st);
     return to_ncnn_status(rc, "ncnnhip_gemm_int8");
+}
+
+// Every other int8 form on blobs that lie in HBM, one sample at a time (the reference runs a batch as a per-sample loop,
+// src/net.cpp:654-700): the steps of Gemm::forward_int8 (src/layer/gemm.cpp:745-966) in its order -- A to row-major,
+// one scale per row of A, one scale for the whole of B, B to K-contiguous rows, C by its shape, the product written plain
+// or transposed -- each as the device kernel the host-Mat path uses too.
+int Gemm_hip::forward_hip_general(const std::vector<HipMat>& bottom_blobs, HipMat& top, HipCommand& cmd, const Option&) const
+{
+    if (weight_block_quantize)
+    {
+        NCNN_LOGE("Gemm %s: a block-quantised B takes one 1-D or 2-D bottom blob on the device", name.c_str());
+        return -1;
+    }
+    // which bottom blob is what (src/layer/gemm.cpp:747-748, 889-902)
+    const HipMat* a_blob = constantA ? 0 : &bottom_blobs[0];
+    const HipMat* b_blob = constantB ? 0 : (constantA ? &bottom_blobs[0] : (bottom_blobs.size() > 1 ? &bottom_blobs[1] : 0));
+    const HipMat* c_blob = 0;
+    if (!constantC)
+    {
+        if (constantA && constantB && bottom_blobs.size() == 1)
+            c_blob = &bottom_blobs[0];
+        else if ((constantA || constantB) && bottom_blobs.size() == 2)
+            c_blob = &bottom_blobs[1];
+        else if (bottom_blobs.size() == 3)
+            c_blob = &bottom_blobs[2];
+    }
+    if ((!constantA && !a_blob) || (!constantB && !b_blob))
+    {
+        NCNN_LOGE("Gemm %s: %d bottom blobs do not cover its dynamic operands", name.c_str(), (int)bottom_blobs.size());
+        return -1;
+    }
+
+    DeviceOperand a, b;
+    int samples = 1;
+    if (a_blob)
+    {
+        if (!device_operand(*a_blob, a))
+        {
+            NCNN_LOGE("Gemm %s: A must be an fp32 blob of 1 or 2 dimensions, or of 3 with height 1", name.c_str());
+            return -1;
+        }
+        samples = a.n;
+    }
+    else
+    {
+        if (!d_A || (A_data.elemsize != 4u && A_data.elemsize != 1u)) return -1;
+        a.data = (const char*)d_A;
+        a.rows = A_data.dims == 3 ? A_data.c : A_data.h;
+        a.cols = A_data.w;
+        a.stride = A_data.dims == 3 ? A_data.cstep : (size_t)A_data.w;
+        a.stored_transposed = false;
+        a.sample_bytes = 0;
+        a.n = 1;
+        if (A_data.elemsize == 1u && !d_A_scales)
+        {
+            NCNN_LOGE("Gemm %s: int8 A without A_data_int8_scales", name.c_str());
+            return -1;
+        }
+    }
+    const bool a_int8 = !a_blob && A_data.elemsize == 1u;
+    const int M = transA ? a.cols : a.rows, K = transA ? a.rows : a.cols;
+
+    int N = 0;
+    if (b_ready_int8)
+    {
+        N = constantN;
+        if (constantK != K)
+        {
+            NCNN_LOGE("Gemm %s: K mismatch (%d vs constant %d)", name.c_str(), K, constantK);
+            return -1;
+        }
+        b.n = 1;
+    }
+    else
+    {
+        if (b_blob)
+        {
+            if (!device_operand(*b_blob, b))
+            {
+                NCNN_LOGE("Gemm %s: B must be an fp32 blob of 1 or 2 dimensions, or of 3 with height 1", name.c_str());
+                return -1;
+            }
+        }
+        else
+        {
+            if (!d_B || B_data.elemsize != 4u)
+            {
+                NCNN_LOGE("Gemm %s: B must be an fp32 blob or a constant int8 table", name.c_str());
+                return -1;
+            }
+            b.data = (const char*)d_B;
+            b.rows = B_data.dims == 3 ? B_data.c : B_data.h;
+            b.cols = B_data.w;
+            b.stride = B_data.dims == 3 ? B_data.cstep : (size_t)B_data.w;
+            b.stored_transposed = false;
+            b.sample_bytes = 0;
+            b.n = 1;
+        }
+        N = transB ? b.rows : b.cols;
+        if ((transB ? b.cols : b.rows) != K)
+        {
+            NCNN_LOGE("Gemm %s: A and B disagree on K", name.c_str());
+            return -1;
+        }
+        if (b_blob)
+        {
+            if (a_blob && b.n != samples)
+            {
+                NCNN_LOGE("Gemm %s: A and B disagree on the batch (%d vs %d)", name.c_str(), samples, b.n);
+                return -1;
+            }
+            samples = b.n;
+        }
+    }
+
+    // C: constant, or a blob classified by its shape (src/layer/gemm.cpp:904-943; a shape that matches nothing is read as a scalar)
+    const char* c_data = 0;
+    size_t c_sample_bytes = 0;
+    int bt = -1;
+    if (constantC)
+    {
+        if (!C_data.empty() && constant_broadcast_type_C >= 0 && d_C)
+        {
+            c_data = (const char*)d_C;
+            bt = constant_broadcast_type_C;
+        }
+    }
+    else if (c_blob && !c_blob->empty())
+    {
+        if (c_blob->elemsize != 4u || (a_blob || b_blob ? c_blob->n != samples : false))
+        {
+            NCNN_LOGE("Gemm %s: C must be an fp32 blob with the batch of the other operands", name.c_str());
+            return -1;
+        }
+        if (!a_blob && !b_blob) samples = c_blob->n;
+        bt = 0;
+        if (c_blob->dims == 1 && c_blob->w == 1) bt = 0;
+        if (c_blob->dims == 1 && c_blob->w == M) bt = 1;
+        if (c_blob->dims == 1 && c_blob->w == N) bt = 4;
+        if (c_blob->dims == 2 && c_blob->w == 1 && c_blob->h == M) bt = 2;
+        if (c_blob->dims == 2 && c_blob->w == N && c_blob->h == M) bt = 3;
+        if (c_blob->dims == 2 && c_blob->w == N && c_blob->h == 1) bt = 4;
+        c_data = (const char*)c_blob->data;
+        c_sample_bytes = c_blob->bytes() / (size_t)c_blob->n;
+    }
+
+    const int ow = output_transpose ? M : N, oh = output_transpose ? N : M;
+    top.create(ow, oh, 4u, samples, &cmd);
+    if (top.empty()) return -100;
+
+    ScopedScratch scratch(&cmd);
+    void* st = cmd.stream;
+    const size_t aq_stride = alignSize((size_t)K, 16);
+    // scratch of one sample, used again by the next (everything is ordered on the one stream)
+    void* a_rm = 0; // A as [M][K] row-major fp32, where the stored matrix is not that already
+    void* a_q = 0;
+    void* a_s = 0;
+    const bool a_needs_transpose = a_int8 ? transA != 0 : (a.stored_transposed != (transA != 0));
+    if (a_needs_transpose)
+    {
+        a_rm = scratch.get((size_t)M * K * (a_int8 ? 1 : 4));
+        if (!a_rm) return -100;
+    }
+    if (!a_int8)
+    {
+        a_q = scratch.get((size_t)M * aq_stride);
+        a_s = scratch.get((size_t)M * 4);
+        if (!a_q || !a_s) return -100;
+    }
+    void* b_q = 0;
+    void* b_t = 0;
+    void* b_s = 0;
+    // the stored matrix has b_srows rows of b_scols values; it is [N][K] already when (stored transposed) == (transB == 0)
+    const int b_srows = b_ready_int8 ? 0 : (b.stored_transposed ? b.cols : b.rows), b_scols = b_ready_int8 ? 0 : (b.stored_transposed ? b.rows : b.cols);
+    const bool b_needs_transpose = !b_ready_int8 && (b.stored_transposed == (transB != 0));
+    if (!b_ready_int8)
+    {
+        b_q = scratch.get((size_t)b_srows * b_scols);
+        b_s = scratch.get(4);
+        if (!b_q || !b_s) return -100;
+        if (b_needs_transpose)
+        {
+            b_t = scratch.get((size_t)N * K);
+            if (!b_t) return -100;
+        }
+    }
+
+    for (int s = 0; s < samples; s++)
+    {
+        int rc = 0;
+        // ---- A: [M][K] K-contiguous int8 + one scale per row
+        const char* a_src = a.data + (size_t)s * a.sample_bytes;
+        const int8_t* d_aq = 0;
+        const float* d_sa = 0;
+        size_t d_aq_stride = 0;
+        if (a_int8)
+        {
+            d_aq = (const int8_t*)a_src;
+            d_aq_stride = a.stride;
+            if (transA)
+            {
+                rc = ncnnhip_transpose_s8((const int8_t*)a_src, a.stride, a.rows, a.cols, (int8_t*)a_rm, (size_t)K, st);
+                if (rc != 0) return to_ncnn_status(rc, "transpose A");
+                d_aq = (const int8_t*)a_rm;
+                d_aq_stride = (size_t)K;
+            }
+            d_sa = (const float*)d_A_scales;
+        }
+        else
+        {
+            const float* rows_src = (const float*)a_src;
+            size_t rows_stride = a.stride;
+            if (a_needs_transpose)
+            {
+                // the stored matrix ([cols][rows] when it lies transposed) -> its transpose, dense
+                const int srows = a.stored_transposed ? a.cols : a.rows, scols = a.stored_transposed ? a.rows : a.cols;
+                rc = ncnnhip_transpose_f32((const float*)a_src, a.stride, srows, scols, (float*)a_rm, (size_t)srows, st);
+                if (rc != 0) return to_ncnn_status(rc, "transpose A");
+                rows_src = (const float*)a_rm;
+                rows_stride = (size_t)K;
+            }
+            rc = ncnnhip_gemm_quantize_rows(rows_src, rows_stride, M, K, (int8_t*)a_q, aq_stride, (float*)a_s, st);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_quantize_rows");
+            d_aq = (const int8_t*)a_q;
+            d_aq_stride = aq_stride;
+            d_sa = (const float*)a_s;
+        }
+
+        // ---- B: [N][K] K-contiguous int8 + one scale
+        const int8_t* d_bq = (const int8_t*)d_B;
+        const float* d_sb = (const float*)d_B_scale;
+        size_t d_bq_stride = (size_t)K;
+        if (!b_ready_int8)
+        {
+            const char* b_src = b.data + (size_t)s * b.sample_bytes;
+            rc = ncnnhip_gemm_quantize_tensor((const float*)b_src, b.stride, b_srows, b_scols, (int8_t*)b_q, (size_t)b_scols, (float*)b_s, st);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_quantize_tensor");
+            d_sb = (const float*)b_s;
+            d_bq = (const int8_t*)b_q;
+            d_bq_stride = (size_t)b_scols;
+            if (b_needs_transpose)
+            {
+                rc = ncnnhip_transpose_s8((const int8_t*)b_q, (size_t)b_scols, b_srows, b_scols, (int8_t*)b_t, (size_t)b_srows, st);
+                if (rc != 0) return to_ncnn_status(rc, "transpose B");
+                d_bq = (const int8_t*)b_t;
+                d_bq_stride = (size_t)b_srows;
+            }
+        }
+
+        const float* d_c = c_data ? (const float*)(c_data + (size_t)s * c_sample_bytes) : 0;
+        float* d_out = (float*)top.data + (size_t)s * ow * oh;
+        rc = ncnnhip_gemm_int8(d_aq, d_aq_stride, d_bq, d_bq_stride, M, N, K, d_sa, d_sb, 1, d_c, d_c ? bt : -1, alpha, beta, output_transpose, d_out, (size_t)ow, 0, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_int8");
+    }
+    return 0;
 }
 
 // Layers with equal keys may share a launch: block-quantised constant B in the packed form, the plain network form

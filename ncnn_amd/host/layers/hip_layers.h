@@ -102,7 +102,8 @@ public:
     virtual int destroy_pipeline(const ncnn::Option& opt);
     virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
-    // device-resident form for the shape a network layer has: one dynamic A (rows of K floats), constant B, constant or no C
+    // device-resident forms: the shape a network layer has (one dynamic A, constant B, constant or no C: rows of a batch
+    // folded into one product) and, sample by sample, every other int8 form with a 2-D output
     virtual int forward_hip(const std::vector<ncnn::HipMat>& bottom_blobs, std::vector<ncnn::HipMat>& top_blobs, ncnn::HipCommand& cmd,
                             const ncnn::Option& opt) const;
     virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
@@ -122,6 +123,7 @@ public:
 private:
     int forward_int8(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
     int forward_block_quantize(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
+    int forward_hip_general(const std::vector<ncnn::HipMat>& bottom_blobs, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;
     void* d_A;        // constant A as loaded (fp32 or int8), row-major as stored
     void* d_B;        // constant B: int8 [N][K] for the int8 path (already K-contiguous), packed bytes for block quant
     void* d_B_tiled;  // the same int8 B in the 256x256 Gemm kernel's tiled operand layout (N % 256 == 0, K % 64 == 0), else null

@@ -351,6 +351,94 @@ def test_gemm_layer_int8_two_dynamic_operands_transposed_output():
     assert np.array_equal(got, want)
 
 
+def _single_where(param_lines, blob, feeds, out, resident, layer="g"):
+    """extract(out) and where the named layer ran ('device' | 'host')."""
+    net = _load(mw.assemble_param(param_lines), blob, resident)
+    ex = net.create_extractor()
+    ex.set_layer_timing(True)
+    for k, v in feeds.items():
+        ex.input(k, v)
+    got = ex.extract(out)
+    where = {r[2]: r[3] for r in ex.layer_timing()}
+    return got, where[layer]
+
+
+GEMM_FORMS = ["two dynamic operands, B stored [K][N], transposed output", "constant int8 A, dynamic B, dynamic per-column C",
+              "transA, constant int8 B, constant per-row C", "3-D operands of height 1", "batch of three, two dynamic 3-D operands",
+              "constant fp32 A stored transposed, dynamic B stored [K][N]", "both operands constant, dynamic full C, transposed output",
+              "one row: 1-D A, dynamic B, scalar C"]
+
+
+@RESIDENT
+@pytest.mark.parametrize("form", range(len(GEMM_FORMS)), ids=GEMM_FORMS)
+def test_gemm_layer_int8_every_form_stays_on_the_device(form, resident):
+    """Gemm::forward_int8 (src/layer/gemm.cpp:745-966) beyond the network form: constant or dynamic A, B and C, transposed
+    inputs and output, 3-D operands (c rows of w values), a batch.  Bit for bit the oracle's on host Mats and on blobs that
+    stay in HBM -- where the layer must run as a device layer, not through host Mats."""
+    rng = np.random.default_rng(40 + form)
+    m, n, k = 24, 40, 96
+    a = rng.standard_normal((m, k), dtype=F)
+    b = (rng.standard_normal((n, k), dtype=F) * F(0.05)).astype(F)  # [N][K]
+    aq, sa = oracle.gemm_quantize_rows(a)
+    bq, sb = oracle.gemm_quantize_tensor(b)
+    in_a, in_b = "Input in0 0 1 a 0=%d 1=%d" % (k, m), "Input in1 0 1 b 0=%d 1=%d" % (k, n)
+    if form == 0:
+        lines = [in_a, "Input in1 0 1 b 0=%d 1=%d" % (n, k), mw.gemm_param("g", ["a", "b"], "out", transB=0, constantB=0, output_transpose=1, alpha=0.5)]
+        got, where = _single_where(lines, b"", {"a": a, "b": b.T.copy()}, "out", resident)
+        want = oracle.gemm_int8(aq, bq, sa, [sb], None, -1, 0.5, 1.0, True)
+    elif form == 1:
+        c = rng.standard_normal(n, dtype=F)
+        ca_scales = (F(127) / np.abs(a).max(axis=1)).astype(F)
+        caq = oracle.quantize(a, ca_scales)  # one scale per row, as a constant int8 A carries them
+        lines = [in_b, "Input in2 0 1 c 0=%d" % n, mw.gemm_param("g", ["b", "c"], "out", M=m, K=k, constantA=1, constantB=0, beta=0.25)]
+        got, where = _single_where(lines, mw.weight_blob(caq) + mw.raw_f32(ca_scales), {"b": b, "c": c}, "out", resident)
+        want = oracle.gemm_int8(caq, bq, ca_scales, [sb], c, 4, 1.0, 0.25)
+    elif form == 2:
+        c = rng.standard_normal((m, 1), dtype=F)
+        cbq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+        csb = F(51.0)
+        lines = ["Input in0 0 1 a 0=%d 1=%d" % (m, k), mw.gemm_param("g", ["a"], "out", N=n, K=k, M=m, transA=1, constantB=1, constantC=1, broadcast_type_C=2, beta=0.5)]
+        got, where = _single_where(lines, mw.weight_blob(cbq) + mw.weight_blob(c) + mw.raw_f32(csb), {"a": a.T.copy()}, "out", resident)
+        want = oracle.gemm_int8(aq, cbq, sa, [csb], c, 2, 1.0, 0.5)
+    elif form == 3:
+        lines = ["Input in0 0 1 a 0=%d 1=1 2=%d" % (k, m), "Input in1 0 1 b 0=%d 1=1 2=%d" % (k, n), mw.gemm_param("g", ["a", "b"], "out", constantB=0)]
+        got, where = _single_where(lines, b"", {"a": a.reshape(m, 1, k), "b": b.reshape(n, 1, k)}, "out", resident)
+        want = oracle.gemm_int8(aq, bq, sa, [sb], None, -1)
+    elif form == 4:
+        a3 = rng.standard_normal((3, m, k), dtype=F)
+        b3 = (rng.standard_normal((3, n, k), dtype=F) * F(0.05)).astype(F)
+        # (a batch is a 4-D array of 3-D blobs: the operands are 3-D blobs of height 1 here too)
+        lines = ["Input in0 0 1 a 0=%d 1=1 2=%d" % (k, m), "Input in1 0 1 b 0=%d 1=1 2=%d" % (k, n), mw.gemm_param("g", ["a", "b"], "out", constantB=0, alpha=2.0)]
+        got, where = _single_where(lines, b"", {"a": a3.reshape(3, m, 1, k), "b": b3.reshape(3, n, 1, k)}, "out", resident)
+        want = []
+        for i in range(3):
+            qa, s_a = oracle.gemm_quantize_rows(a3[i])
+            qb, s_b = oracle.gemm_quantize_tensor(b3[i])
+            want.append(oracle.gemm_int8(qa, qb, s_a, [s_b], None, -1, 2.0))
+        want = np.stack(want)
+    elif form == 5:
+        lines = ["Input in1 0 1 b 0=%d 1=%d" % (n, k), mw.gemm_param("g", ["b"], "out", M=m, K=k, transA=1, transB=0, constantA=1, constantB=0)]
+        blob = mw.weight_blob(a.T.copy()) + mw.raw_f32(np.ones(m, F))  # fp32 A: quantised row by row at forward time; the scale table is read and not used
+        got, where = _single_where(lines, blob, {"b": b.T.copy()}, "out", resident)
+        want = oracle.gemm_int8(aq, bq, sa, [sb], None, -1)
+    elif form == 6:
+        c = rng.standard_normal((m, n), dtype=F)
+        ca_scales = (F(127) / np.abs(a).max(axis=1)).astype(F)
+        caq = oracle.quantize(a, ca_scales)
+        cbq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+        csb = F(33.0)
+        lines = ["Input in0 0 1 c 0=%d 1=%d" % (n, m), mw.gemm_param("g", ["c"], "out", M=m, N=n, K=k, constantA=1, constantB=1, output_transpose=1)]
+        got, where = _single_where(lines, mw.weight_blob(caq) + mw.weight_blob(cbq) + mw.raw_f32(ca_scales) + mw.raw_f32(csb), {"c": c}, "out", resident)
+        want = oracle.gemm_int8(caq, cbq, ca_scales, [csb], c, 3, 1.0, 1.0, True)
+    else:
+        c = np.array([0.75], F)
+        lines = ["Input in0 0 1 a 0=%d" % k, in_b, "Input in2 0 1 c 0=1", mw.gemm_param("g", ["a", "b", "c"], "out", constantB=0)]
+        got, where = _single_where(lines, b"", {"a": a[0], "b": b, "c": c}, "out", resident)
+        want = oracle.gemm_int8(aq[:1], bq, sa[:1], [sb], c, 0)
+    assert np.array_equal(np.asarray(got).reshape(want.shape), want)
+    assert where == ("device" if resident else "host")
+
+
 @RESIDENT
 @pytest.mark.parametrize("bits,block,insc,m,n,k", [
     (8, 64, 0, 4, 24, 200), (4, 32, 1, 4, 24, 200), (6, 128, 0, 4, 24, 200),  # K % 16 != 0: the .bin layout as it is
