@@ -100,11 +100,12 @@ int Gemm_hip::load_param(const ParamDict& pd)
     }
     // one bottom blob is enough when two of the three operands are constants
     if (constantA + constantB + constantC == 2) one_blob_only = true;
-    // Blobs stay in HBM for every int8 form whose output is a 2-D blob: constant or dynamic A, B and C, transposed inputs,
-    // transposed output (Gemm::forward_int8, src/layer/gemm.cpp:745-966, runs them all in place as well).  output_N1M (a 3-D
-    // output) and a block-quantised B with a second bottom blob take host Mats.
-    support_hip = quantize_term != 0 && output_N1M == 0 && !bottoms.empty()
-                  && (!term_is_block_quant(quantize_term) || (constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && bottoms.size() == 1));
+    // Blobs stay in HBM for every int8 form: constant or dynamic A, B and C, transposed inputs, transposed and N x 1 x M
+    // output (Gemm::forward_int8, src/layer/gemm.cpp:745-966, runs them all in place as well).  A block-quantised B stays
+    // there in the network form only; with a second bottom blob or a 3-D output it takes host Mats.
+    support_hip = quantize_term != 0 && !bottoms.empty()
+                  && (!term_is_block_quant(quantize_term)
+                      || (constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottoms.size() == 1));
     return 0;
 }
 
@@ -300,7 +301,7 @@ static bool device_operand(const HipMat& m, DeviceOperand& v)
 int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& opt) const
 {
     if (bottom_blobs.empty() || top_blobs.empty()) return -1;
-    const bool network_form = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && bottom_blobs.size() == 1
+    const bool network_form = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottom_blobs.size() == 1
                               && (weight_block_quantize || b_ready_int8) && (bottom_blobs[0].dims == 1 || bottom_blobs[0].dims == 2);
     if (!network_form) return forward_hip_general(bottom_blobs, top_blobs[0], cmd, opt);
     if (!d_B) return -1;
@@ -509,12 +510,23 @@ int Gemm_hip::forward_hip_general(const std::vector<HipMat>& bottom_blobs, HipMa
         c_sample_bytes = c_blob->bytes() / (size_t)c_blob->n;
     }
 
+    // the output: oh rows of ow values, or (output_N1M, src/layer/gemm.cpp:945-959) a 3-D blob of oh channels, height 1 and
+    // width ow -- channels-last in HBM, so the rows are written to scratch and laid out (pad channels zero) by the converter
     const int ow = output_transpose ? M : N, oh = output_transpose ? N : M;
-    top.create(ow, oh, 4u, samples, &cmd);
+    if (output_N1M)
+        top.create(ow, 1, oh, 4u, samples, &cmd);
+    else
+        top.create(ow, oh, 4u, samples, &cmd);
     if (top.empty()) return -100;
 
     ScopedScratch scratch(&cmd);
     void* st = cmd.stream;
+    void* rows_out = 0;
+    if (output_N1M)
+    {
+        rows_out = scratch.get((size_t)ow * oh * 4);
+        if (!rows_out) return -100;
+    }
     const size_t aq_stride = alignSize((size_t)K, 16);
     // scratch of one sample, used again by the next (everything is ordered on the one stream)
     void* a_rm = 0; // A as [M][K] row-major fp32, where the stored matrix is not that already
@@ -613,9 +625,14 @@ int Gemm_hip::forward_hip_general(const std::vector<HipMat>& bottom_blobs, HipMa
         }
 
         const float* d_c = c_data ? (const float*)(c_data + (size_t)s * c_sample_bytes) : 0;
-        float* d_out = (float*)top.data + (size_t)s * ow * oh;
+        float* d_out = output_N1M ? (float*)rows_out : (float*)top.data + (size_t)s * ow * oh;
         rc = ncnnhip_gemm_int8(d_aq, d_aq_stride, d_bq, d_bq_stride, M, N, K, d_sa, d_sb, 1, d_c, d_c ? bt : -1, alpha, beta, output_transpose, d_out, (size_t)ow, 0, st);
         if (rc != 0) return to_ncnn_status(rc, "ncnnhip_gemm_int8");
+        if (output_N1M)
+        {
+            rc = ncnnhip_chw_to_nhwc(rows_out, 4, oh, ow, 1, (size_t)ow, (size_t)ow * oh, (float*)top.data + (size_t)s * ow * top.cp, st);
+            if (rc != 0) return to_ncnn_status(rc, "ncnnhip_chw_to_nhwc");
+        }
     }
     return 0;
 }

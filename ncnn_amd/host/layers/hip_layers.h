@@ -103,7 +103,7 @@ public:
     virtual int forward(const std::vector<ncnn::Mat>& bottom_blobs, std::vector<ncnn::Mat>& top_blobs, const ncnn::Option& opt) const;
     virtual int forward(const ncnn::Mat& bottom_blob, ncnn::Mat& top_blob, const ncnn::Option& opt) const;
     // device-resident forms: the shape a network layer has (one dynamic A, constant B, constant or no C: rows of a batch
-    // folded into one product) and, sample by sample, every other int8 form with a 2-D output
+    // folded into one product) and, sample by sample, every other int8 form
     virtual int forward_hip(const std::vector<ncnn::HipMat>& bottom_blobs, std::vector<ncnn::HipMat>& top_blobs, ncnn::HipCommand& cmd,
                             const ncnn::Option& opt) const;
     virtual int forward_hip(const ncnn::HipMat& bottom_blob, ncnn::HipMat& top_blob, ncnn::HipCommand& cmd, const ncnn::Option& opt) const;

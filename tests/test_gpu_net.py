@@ -366,7 +366,7 @@ def _single_where(param_lines, blob, feeds, out, resident, layer="g"):
 GEMM_FORMS = ["two dynamic operands, B stored [K][N], transposed output", "constant int8 A, dynamic B, dynamic per-column C",
               "transA, constant int8 B, constant per-row C", "3-D operands of height 1", "batch of three, two dynamic 3-D operands",
               "constant fp32 A stored transposed, dynamic B stored [K][N]", "both operands constant, dynamic full C, transposed output",
-              "one row: 1-D A, dynamic B, scalar C"]
+              "one row: 1-D A, dynamic B, scalar C", "N x 1 x M output, 20 channels in 32", "transposed N x 1 x M output"]
 
 
 @RESIDENT
@@ -430,11 +430,23 @@ def test_gemm_layer_int8_every_form_stays_on_the_device(form, resident):
         lines = ["Input in0 0 1 c 0=%d 1=%d" % (n, m), mw.gemm_param("g", ["c"], "out", M=m, N=n, K=k, constantA=1, constantB=1, output_transpose=1)]
         got, where = _single_where(lines, mw.weight_blob(caq) + mw.weight_blob(cbq) + mw.raw_f32(ca_scales) + mw.raw_f32(csb), {"c": c}, "out", resident)
         want = oracle.gemm_int8(caq, cbq, ca_scales, [csb], c, 3, 1.0, 1.0, True)
-    else:
+    elif form == 7:
         c = np.array([0.75], F)
         lines = ["Input in0 0 1 a 0=%d" % k, in_b, "Input in2 0 1 c 0=1", mw.gemm_param("g", ["a", "b", "c"], "out", constantB=0)]
         got, where = _single_where(lines, b"", {"a": a[0], "b": b, "c": c}, "out", resident)
         want = oracle.gemm_int8(aq[:1], bq, sa[:1], [sb], c, 0)
+    elif form == 8:
+        # output (w = N, h = 1, c = M) with M = 20 rows: a channels-last blob of 32 channels in HBM
+        lines = ["Input in0 0 1 a 0=%d 1=20" % k, in_b, mw.gemm_param("g", ["a", "b"], "out", constantB=0, output_N1M=1)]
+        got, where = _single_where(lines, b"", {"a": a[:20], "b": b}, "out", resident)
+        want = oracle.gemm_int8(aq[:20], bq, sa[:20], [sb], None, -1).reshape(20, 1, n)
+    else:
+        cbq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+        csb = F(47.0)
+        c = rng.standard_normal((1, n), dtype=F)
+        lines = [in_a, mw.gemm_param("g", ["a"], "out", N=n, K=k, constantB=1, constantC=1, broadcast_type_C=4, output_N1M=1, output_transpose=1)]
+        got, where = _single_where(lines, mw.weight_blob(cbq) + mw.weight_blob(c) + mw.raw_f32(csb), {"a": a}, "out", resident)
+        want = oracle.gemm_int8(aq, cbq, sa, [csb], c, 4, 1.0, 1.0, True).reshape(n, 1, m)
     assert np.array_equal(np.asarray(got).reshape(want.shape), want)
     assert where == ("device" if resident else "host")
 
