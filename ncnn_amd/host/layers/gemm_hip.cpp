@@ -101,11 +101,11 @@ int Gemm_hip::load_param(const ParamDict& pd)
     // one bottom blob is enough when two of the three operands are constants
     if (constantA + constantB + constantC == 2) one_blob_only = true;
     // Blobs stay in HBM for every int8 form: constant or dynamic A, B and C, transposed inputs, transposed and N x 1 x M
-    // output (Gemm::forward_int8, src/layer/gemm.cpp:745-966, runs them all in place as well).  A block-quantised B stays
-    // there in the network form only; with a second bottom blob or a 3-D output it takes host Mats.
+    // output (Gemm::forward_int8, src/layer/gemm.cpp:745-966, runs them all in place as well).  A block-quantised B
+    // (Gemm::forward_weight_block_quantize, src/layer/gemm.cpp:339-483: A is the first bottom blob, C a constant or the second)
+    // stays there too; the reference's function knows no transposes and no other output shape.
     support_hip = quantize_term != 0 && !bottoms.empty()
-                  && (!term_is_block_quant(quantize_term)
-                      || (constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottoms.size() == 1));
+                  && (!term_is_block_quant(quantize_term) || (constantA == 0 && constantB == 1 && bottoms.size() <= 2 && (bottoms.size() == 1 || constantC == 0)));
     return 0;
 }
 
@@ -301,8 +301,9 @@ static bool device_operand(const HipMat& m, DeviceOperand& v)
 int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<HipMat>& top_blobs, HipCommand& cmd, const Option& opt) const
 {
     if (bottom_blobs.empty() || top_blobs.empty()) return -1;
-    const bool network_form = constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottom_blobs.size() == 1
-                              && (weight_block_quantize || b_ready_int8) && (bottom_blobs[0].dims == 1 || bottom_blobs[0].dims == 2);
+    const bool network_form = weight_block_quantize
+                              || (constantA == 0 && constantB == 1 && transA == 0 && output_transpose == 0 && output_N1M == 0 && bottom_blobs.size() == 1
+                                  && b_ready_int8 && (bottom_blobs[0].dims == 1 || bottom_blobs[0].dims == 2));
     if (!network_form) return forward_hip_general(bottom_blobs, top_blobs[0], cmd, opt);
     if (!d_B) return -1;
     const HipMat& A = bottom_blobs[0];
@@ -319,7 +320,24 @@ int Gemm_hip::forward_hip(const std::vector<HipMat>& bottom_blobs, std::vector<H
         return -1;
     }
     const float* d_c = constantC && !C_data.empty() && constant_broadcast_type_C >= 0 ? (const float*)d_C : 0;
-    const int bt = d_c ? constant_broadcast_type_C : -1;
+    int bt = d_c ? constant_broadcast_type_C : -1;
+    if (!constantC && bottom_blobs.size() == 2 && !bottom_blobs[1].empty())
+    {
+        // a block-quantised B with C as its second bottom blob: the shape must be one the reference names (src/layer/gemm.cpp:378-421)
+        const HipMat& C = bottom_blobs[1];
+        if (C.dims == 1 && C.w == 1) bt = 0;
+        if (C.dims == 1 && C.w == M) bt = 1;
+        if (C.dims == 1 && C.w == N) bt = 4;
+        if (C.dims == 2 && C.w == 1 && C.h == M) bt = 2;
+        if (C.dims == 2 && C.w == N && C.h == M) bt = 3;
+        if (C.dims == 2 && C.w == N && C.h == 1) bt = 4;
+        if (bt < 0 || C.elemsize != 4u || C.n != 1 || A.n != 1)
+        {
+            NCNN_LOGE("Gemm %s: unsupported C", name.c_str());
+            return -1;
+        }
+        d_c = (const float*)C.data;
+    }
     if (A.n > 1 && (bt == 1 || bt == 2 || bt == 3))
     {
         NCNN_LOGE("Gemm %s: a per-row C does not extend to a batch", name.c_str());

@@ -474,6 +474,26 @@ def test_gemm_layer_block_quant(bits, block, insc, m, n, k, resident):
     assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
 
 
+@RESIDENT
+@pytest.mark.parametrize("m,n,k,c_shape,bt", [(4, 40, 256, (40,), 4), (20, 33, 512, (20, 33), 3), (3, 24, 200, (3, 1), 2), (1, 48, 256, (1,), 0)])
+def test_gemm_layer_block_quant_with_c_as_the_second_bottom_blob(m, n, k, c_shape, bt, resident):
+    """Gemm::forward_weight_block_quantize takes C from the second bottom blob when it is not a constant
+    (src/layer/gemm.cpp:372-421): per column, full, per row, scalar -- on host Mats and as a device layer."""
+    import npref
+    rng = np.random.default_rng(m + n + k)
+    a = rng.standard_normal((m, k), dtype=F)
+    w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+    c = rng.standard_normal(c_shape, dtype=F)
+    packed, scales = oracle.blockquant_pack(w, 8, 64)
+    c_in = "Input in1 0 1 c 0=%d" % c_shape[0] if len(c_shape) == 1 else "Input in1 0 1 c 0=%d 1=%d" % (c_shape[1], c_shape[0])
+    lines = ["Input in0 0 1 a 0=%d 1=%d" % (k, m), c_in, mw.gemm_param("g", ["a", "c"], "out", N=n, K=k, constantB=1, quantize_term=801, alpha=0.5, beta=2.0)]
+    blob = mw.weight_blob(packed.view(np.int8)) + mw.raw_f32(scales)
+    got, where = _single_where(lines, blob, {"a": a, "c": c}, "out", resident)
+    val, floor = npref.blockquant_gemm_f64(a, packed, scales, 8, 64, None, c, bt, 0.5, 2.0)
+    assert np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
+    assert where == ("device" if resident else "host")
+
+
 @pytest.mark.parametrize("m", [1, 4, 9])
 def test_sibling_block_quant_gemms_behind_a_split_share_one_launch(m):
     """The gate / up pair of a decoder layer: block-quantised Gemm layers that read the outputs of one Split run as ONE launch
