@@ -65,11 +65,9 @@ int Convolution_hip::load_param(const ParamDict& pd)
         return -1;
     }
     support_int8_storage = true;
-    // device-resident kernels exist for plain convolutions and for true depthwise ones; a grouped convolution in
-    // between takes host Mats (and still runs on the device, through the planar kernel)
-    const int taps = kernel_w * kernel_h;
-    const bool depthwise = group > 1 && group == num_output && taps > 0 && weight_data_size == num_output * taps;
-    support_hip = group == 1 || depthwise;
+    // channels-last kernels exist for plain convolutions and for true depthwise ones; a grouped convolution in between
+    // stays in HBM as well, through the planar kernel with a layout change on either side (forward_device)
+    support_hip = true;
     return 0;
 }
 
@@ -464,7 +462,7 @@ int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* resid
         NCNN_LOGE("%s %s: use_int8_inference is off and there is no fp32 path in this runtime", type.c_str(), name.c_str());
         return -1;
     }
-    if (!d_scale_in || (group == 1 ? !d_weight_packed : !d_weight_dw))
+    if (!d_scale_in || (group == 1 ? !d_weight_packed : (is_depthwise() ? !d_weight_dw : !d_weight)))
     {
         NCNN_LOGE("%s %s: forward before create_pipeline", type.c_str(), name.c_str());
         return -1;
@@ -604,6 +602,25 @@ int Convolution_hip::forward_device(const HipMat& bottom_in, const HipMat* resid
         rc = ncnnhip_conv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_packed, (const float*)d_scale_in, (const float*)d_bias, scale_out_table, act,
                                     top.data, NCNNHIP_CHANNELS_LAST, 0, 0, ws, workspace_bytes, st);
         return to_ncnn_status(rc, "ncnnhip_conv_int8_nhwc");
+    }
+    if (!is_depthwise())
+    {
+        // A grouped convolution that is not depthwise (ConvolutionDepthWise::forward_int8, src/layer/convolutiondepthwise.cpp:
+        // 515-636, group by group): the planar kernel of the host-Mat path, on planar copies made and undone in HBM.
+        const size_t hw = (size_t)bottom.w * bottom.h, ohw = (size_t)outw * outh;
+        const size_t x_cstep = alignSize(hw, 16), x_nstep = x_cstep * channels;
+        const size_t out_es = requant ? 1u : 4u;
+        const size_t o_cstep = alignSize(ohw * out_es, 16) / out_es, o_nstep = o_cstep * num_output;
+        void* x_planar = scratch.get(x_nstep * bottom.n);
+        void* o_planar = scratch.get(o_nstep * out_es * bottom.n);
+        if (!x_planar || !o_planar) return -100;
+        rc = ncnnhip_nhwc_to_chw(xq, 1, channels, (int)hw, bottom.n, x_planar, x_cstep, x_nstep, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_nhwc_to_chw");
+        rc = ncnnhip_conv_int8(&desc, (const int8_t*)x_planar, x_cstep, x_nstep, (const int8_t*)d_weight, (const float*)d_scale_in, (const float*)d_bias,
+                               scale_out_table, act, o_planar, o_cstep, o_nstep, 0, st);
+        if (rc != 0) return to_ncnn_status(rc, "ncnnhip_conv_int8");
+        rc = ncnnhip_chw_to_nhwc(o_planar, (int)out_es, num_output, (int)ohw, bottom.n, o_cstep, o_nstep, top.data, st);
+        return to_ncnn_status(rc, "ncnnhip_chw_to_nhwc");
     }
     rc = ncnnhip_dwconv_int8_nhwc(&desc, xq, (const int8_t*)d_weight_dw, (const float*)d_scale_in, (const float*)d_bias, scale_out_table, act, top.data, st);
     return to_ncnn_status(rc, "ncnnhip_dwconv_int8_nhwc");

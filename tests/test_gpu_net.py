@@ -363,6 +363,29 @@ def _single_where(param_lines, blob, feeds, out, resident, layer="g"):
     return got, where[layer]
 
 
+@RESIDENT
+@pytest.mark.parametrize("c,outc,group,h,w,stride,term,act", [(8, 4, 2, 12, 12, 2, 1, 1), (64, 64, 4, 14, 14, 1, 101, 3), (6, 12, 3, 9, 10, 1, 2, 0),
+                                                              (32, 48, 8, 10, 7, 1, 102, 1)])
+def test_grouped_convolution_layer_stays_on_the_device(c, outc, group, h, w, stride, term, act, resident):
+    """ConvolutionDepthWise with 1 < group < channels (src/layer/convolutiondepthwise.cpp:515-636: group by group) through
+    load_param / load_model / forward, batch of two: bit for bit the oracle's, on host Mats and as a device layer (the
+    planar kernel between two layout changes in HBM)."""
+    x, wq, b, ws, ins, tops = cases.conv_case(c + outc + group + term, c, h, w, outc, (3, 3), group, term, True, False, by_group=True, batch=2)
+    one_weight_scale = term in (2, 102)
+    if one_weight_scale:
+        ws[:] = ws[0]
+    ap = (0.0, 6.0) if act == 3 else ()
+    lines = ["Input in0 0 1 data 0=%d 1=%d 2=%d" % (w, h, c),
+             mw.conv_param("g", "data", "out", outc, 3, stride=stride, pad=1, weight_size=wq.size, term=term, act=act, act_params=ap, group=group)]
+    blob = mw.conv_weights(wq, b, ws[:1] if one_weight_scale else ws, ins[0], None if tops is None else tops[0])
+    got, where = _single_where(lines, blob, {"data": x}, "out", resident)
+    d = oracle.make_desc((c, h, w), outc, (3, 3), (1, 1), (stride, stride), (1, 1, 1, 1), 0.0, 1, group, term, act, (0.0, 6.0))
+    for i in range(2):
+        want = oracle.convolutiondepthwise_int8(d, x[i], wq, b, ws, ins, tops)
+        assert np.array_equal(got[i], want.astype(F)), "sample %d" % i  # (extract hands an int8 blob over as fp32 values, src/net.cpp:3007-3012)
+    assert where == ("device" if resident else "host")
+
+
 GEMM_FORMS = ["two dynamic operands, B stored [K][N], transposed output", "constant int8 A, dynamic B, dynamic per-column C",
               "transA, constant int8 B, constant per-row C", "3-D operands of height 1", "batch of three, two dynamic 3-D operands",
               "constant fp32 A stored transposed, dynamic B stored [K][N]", "both operands constant, dynamic full C, transposed output",
