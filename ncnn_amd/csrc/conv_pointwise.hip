@@ -15,7 +15,8 @@
 //     the current one is being requantised;
 //   * the four packed words of a lane (same channels, four pixel groups) and those of the lanes 16, 32 and 48 away
 //     (same pixels, the other channels) are a 4x4 matrix across lane rows and registers: four lane-row swaps transpose
-//     it, after which every lane holds 16 consecutive output bytes of one pixel: one 16-byte store.
+//     it, after which every lane holds 16 consecutive output bytes of one pixel: one 16-byte store -- to global memory where
+//     that is the whole pixel record, else to LDS, from where the workgroup's pixel blocks leave as whole lines.
 // The same kernel serves the narrow-input first layer of a net (STEM: at most 4 input channels, the quantised image of 4
 // bytes per pixel with its physical zero border, kernels of up to 4 x 4 taps at any stride): there a 16-byte operand
 // chunk is 4 neighbouring pixels of one kernel row, and a lane finds its chunk by its output pixel's position in the
@@ -88,9 +89,9 @@ template<int KSTEPS, bool STEM>
 __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* __restrict__ wpk /* [cout][KSTEPS * 64] */, const int8_t* __restrict__ x, NhwcGeom g,
                                                                    int out_cp, const float* __restrict__ scale_in, const float* __restrict__ bias_tab,
                                                                    const float* __restrict__ scale_out, ncnnhip_activation act, int8_t* __restrict__ out,
-                                                                   int channel_blocks, int G)
+                                                                   int channel_blocks, int G, int staged)
 {
-    extern __shared__ __attribute__((aligned(16))) float pw_tab[]; // [5][out_cp]: input scale, bias, output scale, clamp low, clamp high
+    extern __shared__ __attribute__((aligned(16))) float pw_tab[]; // [5][out_cp]: input scale, bias, output scale, clamp low, clamp high; then (staged) the G pixel blocks' results, [64][out_cp] bytes each
     typedef int v4i_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
     const int cp_in = g.Cp, npix = g.npix, cout = g.cout;
     const int lane = threadIdx.x & 63;
@@ -206,6 +207,10 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
 
     const int p_store = pb * 64 + q * 16 + c16;
     int8_t* orow = out + (size_t)p_store * out_cp;
+    // staged: the pixel block's results meet in LDS as they lie in the blob -- 64 consecutive pixel records are 64 * out_cp
+    // consecutive bytes -- and leave as whole lines (a lane's own 16 bytes are 1/6 of a 96-byte record: one partial line per lane)
+    int8_t* const stage_block = reinterpret_cast<int8_t*>(pw_tab + 5 * out_cp) + (size_t)(G == 4 ? wave : G == 2 ? (wave & 1) : 0) * 64 * out_cp;
+    int8_t* const srow = stage_block + (q * 16 + c16) * out_cp;
     for (int cb = cb_first; cb < channel_blocks; cb += cb_step)
     {
         const Weights w_now = fw;
@@ -246,7 +251,21 @@ __global__ __launch_bounds__(256) void conv_pointwise_int8_kernel(const int8_t* 
         auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
         auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
         const v4i pk = {(int)t01[0], (int)t01[1], (int)t23[0], (int)t23[1]};
-        if (p_store < npix) *reinterpret_cast<v4i*>(orow + cb * 16) = pk;
+        if (staged)
+            *reinterpret_cast<v4i*>(srow + cb * 16) = pk;
+        else if (p_store < npix)
+            *reinterpret_cast<v4i*>(orow + cb * 16) = pk;
+    }
+    if (staged)
+    {
+        // (wavefronts of pixel blocks beyond the end have left; the barrier counts those that remain)
+        __syncthreads();
+        const int waves_per_block = G == 4 ? 1 : 4 / G, my = G == 4 ? 0 : wave / G;
+        const int pixels_here = npix - pb * 64 < 64 ? npix - pb * 64 : 64;
+        const int nchunks = pixels_here * (out_cp >> 4);
+        int8_t* const gblock = out + (size_t)pb * 64 * out_cp;
+        for (int i = my * 64 + lane; i < nchunks; i += 64 * waves_per_block)
+            *reinterpret_cast<v4i*>(gblock + (size_t)i * 16) = *reinterpret_cast<const v4i*>(stage_block + (size_t)i * 16);
     }
 }
 
@@ -289,15 +308,20 @@ int launch_conv_pointwise(const NhwcGeom& g, const int8_t* wpk, const int8_t* x,
         const dim3 grid((unsigned)ceil_div(pixel_blocks, Gs));
         NCNNHIP_REQUIRE(g.K == 64 && g.ntaps <= 4, "convolution: %d bytes of K in the narrow-input form of the pointwise kernel", g.K);
         hipLaunchKernelGGL((conv_pointwise_int8_kernel<1, true>), grid, dim3(256), tab_bytes, stream, wpk, x, g, out_cp, epi.scale_in, epi.bias, epi.scale_out,
-                           epi.act, static_cast<int8_t*>(epi.out), channel_blocks, Gs);
+                           epi.act, static_cast<int8_t*>(epi.out), channel_blocks, Gs, 0);
         return launch_status("conv_pointwise_int8_kernel (narrow input)");
     }
     // pixel blocks per workgroup: two, each with two wavefronts that take the even and the odd channel blocks (measured on
     // MobileNetV2's 16 -> 96 expansion on 112 x 112 at batch 32: 19.8 us, against 23.1 for one block with four wavefronts and
     // 31 for four blocks with one wavefront each); a layer too small for that many workgroups keeps one block per workgroup
     const int G = pixel_blocks >= 1024 ? 2 : 1;
-    hipLaunchKernelGGL((conv_pointwise_int8_kernel<1, false>), dim3((unsigned)ceil_div(pixel_blocks, G)), dim3(256), tab_bytes, stream, wpk, x, g, out_cp, epi.scale_in,
-                       epi.bias, epi.scale_out, epi.act, static_cast<int8_t*>(epi.out), channel_blocks, G);
+    // results through LDS, leaving as whole lines, where a pixel record is several channel blocks long (MobileNetV2 at batch 32:
+    // 16 -> 96 on 112 x 112 21.8 -> 20.6 us, 24 -> 144 on 56 x 56 11.25 -> 10.5); a record of one block is a lane's own 16 bytes
+    // already (32 -> 16 on 112 x 112: 10.5 us direct, 12.3 staged)
+    const int staged = channel_blocks > 1 && tab_bytes + (size_t)G * 64 * out_cp <= 60 * 1024;
+    const size_t lds = tab_bytes + (staged ? (size_t)G * 64 * out_cp : 0);
+    hipLaunchKernelGGL((conv_pointwise_int8_kernel<1, false>), dim3((unsigned)ceil_div(pixel_blocks, G)), dim3(256), lds, stream, wpk, x, g, out_cp, epi.scale_in,
+                       epi.bias, epi.scale_out, epi.act, static_cast<int8_t*>(epi.out), channel_blocks, G, staged);
     return launch_status("conv_pointwise_int8_kernel");
 }
 
