@@ -411,7 +411,7 @@ static int stem_shape(const ncnnhip_conv_desc& d, StemShape& s)
     const int need_h = (s.outh - 1) * d.stride_h + (d.kernel_h - 1) * d.dilation_h + 1;
     const int need_w = (s.outw - 1) * d.stride_w + (s.G - 1) * 4 + 4;
     s.Hb = std::max(s.pads.top + d.h, need_h);
-    s.Wp = std::max(s.pads.left + d.w, need_w);
+    s.Wp = (std::max(s.pads.left + d.w, need_w) + 3) & ~3; // whole groups of four pixels: the quantiser stores 16 bytes per thread
     s.K = (d.kernel_h * s.G * 16 + 63) / 64 * 64;
     return NCNNHIP_OK;
 }
@@ -459,6 +459,42 @@ __global__ __launch_bounds__(256) void quantize_stem_kernel(const T* __restrict_
         }
     }
     image[(img * Hb + yb) * (size_t)Wp + xb] = word;
+}
+
+// The same from the narrow fp32 image (4 floats per pixel): four neighbouring pixels of the bordered image per thread,
+// up to four aligned 16-byte loads and one 16-byte store (Wp is a multiple of 4, the image 16-byte aligned).
+__global__ __launch_bounds__(256) void quantize_stem_narrow_kernel(const float* __restrict__ src, int c, int h, int w, int top, int left, int Hb, int Wp,
+                                                                   const float* __restrict__ scale, int8_t* __restrict__ image)
+{
+    const int xb0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (xb0 >= Wp) return;
+    const int yb = blockIdx.y;
+    const size_t img = blockIdx.z;
+    const int y = yb - top;
+    const bool row_in = (unsigned)y < (unsigned)h;
+    const float* row = src + ((img * h + (row_in ? y : 0)) * (size_t)w) * 4;
+    v4f t[4];
+    bool in[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+    {
+        const int x = xb0 + i - left;
+        in[i] = row_in && (unsigned)x < (unsigned)w;
+        t[i] = *reinterpret_cast<const v4f*>(row + (size_t)(in[i] ? x : 0) * 4); // unconditional: the four loads overlap
+    }
+    const float sc = scale[0];
+    v4i word;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+    {
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[q] = q < c ? mul_rn(t[i][q], sc) : 0.f;
+        float2int8_as_float_x4(v[0], v[1], v[2], v[3]);
+        const uint32_t pk = pack4_quantised(v[0], v[1], v[2], v[3]);
+        word[i] = in[i] ? (int)pk : 0;
+    }
+    *reinterpret_cast<v4i*>(image + ((img * Hb + yb) * (size_t)Wp + xb0) * 4) = word;
 }
 
 } // namespace ncnnhip
@@ -763,6 +799,12 @@ int ncnnhip_quantize_stem(const ncnnhip_conv_desc* desc, const void* nhwc_dev, i
     NCNNHIP_REQUIRE(s.Hb <= 65535 && desc->batch <= 65535, "ncnnhip_quantize_stem: extent too large");
     NCNNHIP_REQUIRE(elemsize != 4 || src_cp != 4 || (reinterpret_cast<uintptr_t>(nhwc_dev) & 15) == 0, "ncnnhip_quantize_stem: a 4-float-per-pixel image must be 16-byte aligned");
     dim3 grid((unsigned)ceil_div(s.Wp, 256), (unsigned)s.Hb, (unsigned)desc->batch);
+    if (elemsize == 4 && src_cp == 4 && (reinterpret_cast<uintptr_t>(image_dev) & 15) == 0)
+    {
+        hipLaunchKernelGGL(quantize_stem_narrow_kernel, dim3((unsigned)ceil_div(s.Wp / 4, 256), (unsigned)s.Hb, (unsigned)desc->batch), dim3(256), 0, as_stream(stream),
+                           (const float*)nhwc_dev, desc->c, desc->h, desc->w, s.pads.top, s.pads.left, s.Hb, s.Wp, scale_dev, image_dev);
+        return launch_status("quantize_stem_narrow_kernel");
+    }
     if (elemsize == 4)
         hipLaunchKernelGGL(quantize_stem_kernel<float>, grid, dim3(256), 0, as_stream(stream), (const float*)nhwc_dev, src_cp, desc->c, desc->h, desc->w, s.pads.top,
                            s.pads.left, s.Hb, s.Wp, scale_dev, (uint32_t*)image_dev);
