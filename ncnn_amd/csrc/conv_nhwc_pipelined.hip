@@ -60,7 +60,14 @@ int launch_conv_nhwc_pipelined(const NhwcGeom& g_in, const int8_t* wpk, const in
         g.H = g.outh = 1;
         g.W = g.outw = g.npix;
     }
-    const PipePlan p = plan_pipelined(g.cout, g.npix, g.K / 64);
+    PipePlan p = plan_pipelined(g.cout, g.npix, g.K / 64);
+    // the narrow-input first layer has four K steps at most: from a million output pixels up, 128-pixel tiles halve the number of
+    // workgroup prologues (ResNet-50's 7 x 7 first layer at batch 128: the pass 2.22 -> 2.20 ms; at batch 16, 0.2 M pixels, no gain)
+    if ((g.tapK == 16 || g.tapK == 32) && p.splits == 1 && p.bm == 64 && g.npix >= (1 << 20))
+    {
+        p.bm = 128;
+        p.tiles_m = ceil_div(g.npix, 128);
+    }
     const long long blocks = (long long)p.tiles_m * p.tiles_n * p.splits;
     NCNNHIP_REQUIRE(blocks < (1ll << 31) && blocks * p.tiles_n < (1ll << 32), "convolution: too many tiles");
     int32_t* partial = 0;
