@@ -351,6 +351,18 @@ def test_stem_convolution_on_the_pointwise_kernel(rt, batch, c, h, w, outc, kern
         assert got.dtype == want.dtype and np.array_equal(got[i], want), "sample %d" % i
 
 
+def test_stem_convolution_of_a_million_output_pixels(rt):
+    """From 2^20 output pixels up the narrow-input layer runs on 128-pixel tiles of the pipelined kernel (fp32 output here, so
+    the pointwise form does not take it): bit for bit the oracle's, batch of two, a last tile that is partly empty."""
+    c, h, w, outc, kernel = 3, 1450, 1454, 16, (3, 3)
+    x, wq, b, ws, ins, tops = cases.conv_case(123, c, h, w, outc, kernel, 1, 2, True, False, batch=2)
+    d = oracle.make_desc((c, h, w), outc, kernel, (1, 1), (2, 2), (1, 1, 1, 1), 0.0, 1, 1, 2, 1)
+    got = rt.conv_channels_last(x, wq, b, ws, ins, None, outc, kernel, (1, 1), (2, 2), (1, 1, 1, 1), 0.0, 1, 2, 1, (0.0, 0.0), stem=True)
+    assert got.shape[0] * got.shape[2] * got.shape[3] >= (1 << 20)
+    for i in range(2):
+        assert np.array_equal(got[i], oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None))
+
+
 def test_stem_convolution_batch_int8_input_and_fused_tail(rt):
     """Batch of 3, an int8 input blob (already quantised upstream), and the fused tail (residual, ReLU, quantised copy)."""
     c, h, w, outc, kernel = 3, 18, 22, 48, (3, 3)
