@@ -5,6 +5,8 @@
 
 namespace ncnnhip {
 
+constexpr int SPLIT_MIN_STEPS = 12;
+
 PipePlan plan_pipelined(int cout, long long npix, int steps)
 {
     PipePlan p;
@@ -24,13 +26,17 @@ PipePlan plan_pipelined(int cout, long long npix, int steps)
     p.tiles_n = ceil_div(cout, p.bn);
     p.splits = 1;
     const long long t = tiles();
-    if (t < 256 && t <= SPLIT_MAX_TILES && steps >= 16)
+    if (t < 256 && t <= SPLIT_MAX_TILES && steps >= 2 * SPLIT_MIN_STEPS)
     {
-        // fewer tiles than CUs: split K until there is about one workgroup per CU (two splits from 128 tiles up), at
-        // least 8 steps each (measured best over the ResNet-50 / MobileNetV2 layers at batch 1 and 16; with the limit at
-        // 128 tiles the 196-tile 3x3 layers of ResNet-50's fourth stage at batch 16 ran unsplit on 196 of the 256 CUs)
+        // fewer tiles than CUs: split K until there is about one workgroup per CU (two splits from 128 tiles up; with the
+        // limit at 128 tiles the 196-tile 3x3 layers of ResNet-50's fourth stage at batch 16 ran unsplit on 196 of the 256
+        // CUs), at least 12 steps each.  A split costs about 2 us (partial sums through memory, the last workgroup of a
+        // tile adds them up): with 8 steps each, the 16-step 1x1 layers 1024 -> 256 of ResNet-50 ran 8.6 us in two halves
+        // and 6.8 whole at batch 16, the 18-step 3x3 layers 128 -> 128 9.6 and 7.5 at batch 8; summed over a pass the
+        // kernels take 350 / 355 / 362 / 385 us at batch 1 with at least 8 / 12 / 16 / 24 steps, 404 / 389 / 395 / 414
+        // at batch 4, 459 / 449 / 446 / 466 at batch 8, 568 / 555 / 556 / 565 at batch 16 (MobileNetV2: no difference)
         const int want = (int)((256 + t - 1) / t);
-        const int max_splits = steps / 8;
+        const int max_splits = steps / SPLIT_MIN_STEPS;
         p.splits = want < max_splits ? want : max_splits;
         if (p.splits < 1) p.splits = 1;
     }

@@ -886,10 +886,11 @@ static int resident_choose(const NhwcGeom& g, const ConvEpilogue& epi, const Con
 // the pixel threshold, NCNNHIP_RESIDENT_CFG forces one tile configuration (0..7): for measurements and tests.
 bool conv_resident_fits(const NhwcGeom& g, const ConvEpilogue& epi, const ConvFusion& fusion, int out_cp)
 {
+    if (g.ntaps < 2) return false; // first: most layers of a network are 1x1 and need not look the environment up
     if (getenv("NCNNHIP_RESIDENT_OFF")) return false;
     long long min_pixels = 40000;
     if (const char* e = getenv("NCNNHIP_RESIDENT_MIN")) min_pixels = atoll(e);
-    if (g.npix < min_pixels || g.ntaps < 2) return false;
+    if (g.npix < min_pixels) return false;
     ResidentPlan P;
     size_t lds_bytes;
     return resident_choose(g, epi, fusion, out_cp, P, lds_bytes) >= 0;

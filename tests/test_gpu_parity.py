@@ -364,7 +364,7 @@ def test_convolution_network_shapes(rt, name, c, h, w, outc, kernel, stride, pad
     ("1x1/2 96->100 @28 (channel tails on both sides)", 96, 28, 28, 100, (1, 1), (2, 2), (0, 0, 0, 0), 1, 2, 1),
     ("3x3/2 20->48 @33 SAME_UPPER (20 channels in 32)", 20, 33, 33, 48, (3, 3), (2, 2), (-233, -233, -233, -233), 1, 1, 2),
     ("5x3 dilated 16->64 @40x30", 16, 30, 40, 64, (5, 3), (1, 1), (4, 4, 2, 2), 1, 0, 1),
-    ("3x3 512->512 @7 (K split over 9 workgroups per tile)", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 1, 1, 1),
+    ("3x3 512->512 @7 (K split over workgroups)", 512, 7, 7, 512, (3, 3), (1, 1), (1, 1, 1, 1), 1, 1, 1),
     ("3x3 64->96 @12 requantised, batch 2 (K split three ways, a partly filled last tile)", 64, 12, 12, 96, (3, 3), (1, 1), (1, 1, 1, 1), 101, 1, 2),
     ("1x1 512->64 @9 (rows are the pixels, K split)", 512, 9, 9, 64, (1, 1), (1, 1), (0, 0, 0, 0), 1, 0, 1),
 ])

@@ -47,7 +47,7 @@ def test_noalloc_innerproduct_equals_the_workspace_form_on_calls_in_a_row():
     # K-split shapes first (FC 2048 -> 1000 is the ResNet-50 head, at a batch beyond the few-row kernel's 48 rows), each
     # smaller than the one before, then shapes without a split: the few-row kernel's, a tiled one, the gemv kernel's; all
     # share the one scratch
-    shapes = [(64, 2048, 1000), (56, 1280, 1000), (50, 1024, 256), (16, 2048, 1000), (64, 512, 128), (300, 256, 64), (3, 100, 10)]
+    shapes = [(64, 2048, 1000), (56, 1536, 1000), (50, 3072, 256), (16, 2048, 1000), (64, 512, 128), (300, 256, 64), (3, 100, 10)]
     used_scratch = 0
     for i, (rows, k, n) in enumerate(shapes):
         print("noalloc innerproduct", rows, k, n, flush=True)
