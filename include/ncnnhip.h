@@ -108,7 +108,10 @@ typedef struct ncnnhip_conv_desc
     int group;                                    /* 1 for Convolution */
 } ncnnhip_conv_desc;
 
-/* Output extent after make_padding (src/layer/convolution.cpp:328-372, 412-413). */
+/* Output extent after make_padding (src/layer/convolution.cpp:328-372, 412-413).  NCNNHIP_ERROR for an empty output and
+ * for a SAME mode (-233 / -234) that resolves to a negative border (kernel extent below the stride in one dimension while
+ * the other needs a border): the reference's border copy (src/layer/padding.cpp:62-87) writes out of bounds there and has
+ * no defined result.  Every convolution entry point sizes its output through this call and refuses the same layers. */
 int ncnnhip_conv_out_shape(const ncnnhip_conv_desc* desc, int* outw, int* outh);
 /* Head pads make_padding resolves to (literal values, or the SAME_UPPER / SAME_LOWER split, :348-371). */
 int ncnnhip_conv_resolved_pads(const ncnnhip_conv_desc* desc, int* pad_top, int* pad_left);

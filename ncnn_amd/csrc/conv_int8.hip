@@ -142,6 +142,13 @@ int ncnnhip_conv_out_shape(const ncnnhip_conv_desc* desc, int* outw, int* outh)
     int ret = check_desc(desc, "ncnnhip_conv_out_shape");
     if (ret) return ret;
     const ResolvedPads p = resolve_pads(*desc);
+    // A SAME mode gives a negative border where the kernel's extent is below the stride in one dimension while the other
+    // dimension needs a border (3 x 1 at stride 3 on 37 x 20: bottom = -1).  The reference's border copy then writes every
+    // source row into a blob with fewer rows (src/layer/padding.cpp:62-87), out of bounds and with a result that depends on
+    // the order its threads run in: no result to reproduce, so the layer is refused.
+    NCNNHIP_REQUIRE(p.top >= 0 && p.bottom >= 0 && p.left >= 0 && p.right >= 0,
+                    "convolution: the padding mode resolves to a negative border (top %d bottom %d left %d right %d): kernel extent below the stride in one "
+                    "dimension, a border needed in the other; the reference's border copy runs out of bounds for such a layer", p.top, p.bottom, p.left, p.right);
     const int W = desc->w + p.left + p.right;
     const int H = desc->h + p.top + p.bottom;
     const int ow = (W - (desc->dilation_w * (desc->kernel_w - 1) + 1)) / desc->stride_w + 1;

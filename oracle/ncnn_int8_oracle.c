@@ -172,8 +172,14 @@ ORACLE_API void oracle_resolve_padding(int w, int h, int kernel_w, int kernel_h,
 }
 
 /* Builds the bordered int8 tensor (dense, channel stride = ph*pw). Border byte is the C cast
- * of the float pad value to signed char. Negative resolved pads are not produced by ncnn's
- * call sites for these layers. */
+ * of the float pad value to signed char.
+ * A SAME mode resolves to a NEGATIVE border in one dimension when the kernel's extent is below the
+ * stride there while the other dimension needs a border (e.g. a 3 x 1 kernel at stride 3 on 37 x 20:
+ * wpad 2, hpad -1, so bottom = -1).  The reference then makes a bordered blob smaller than the source
+ * and still copies every source row and column into it (src/layer/padding.cpp:62-87: the centre loop
+ * runs to top + src.h whatever dst.h is), i.e. it writes past the rows it allocated, and which values
+ * end up inside the blob depends on the order its threads write the channels in.  There is no result
+ * to restate: conv_core returns -1 for such a layer and never comes here with a negative border. */
 static int8_t* make_bordered(const int8_t* x, size_t cstep, int c, int h, int w, const int pads[4], float pad_value,
                              int* ph, int* pw)
 {
@@ -238,6 +244,7 @@ static int conv_core(const oracle_conv_desc* d, const int8_t* x_q, size_t x_cste
     int pads[4];
     oracle_resolve_padding(d->w, d->h, d->kernel_w, d->kernel_h, d->dilation_w, d->dilation_h, d->stride_w, d->stride_h,
                            d->pad_left, d->pad_right, d->pad_top, d->pad_bottom, pads);
+    if (pads[0] < 0 || pads[1] < 0 || pads[2] < 0 || pads[3] < 0) return -1; /* see make_bordered */
     int H, W;
     int8_t* xb = make_bordered(x_q, x_cstep, d->c, d->h, d->w, pads, d->pad_value, &H, &W);
     if (!xb) return -100;

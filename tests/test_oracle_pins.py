@@ -245,6 +245,41 @@ def test_invalid_group_is_rejected_with_minus_100():
         oracle.convolutiondepthwise_int8(d, x, wt, b, np.ones(4, F), np.ones(4, F), None)
 
 
+@pytest.mark.parametrize("mode", [-233, -234])
+@pytest.mark.parametrize("h,w,kernel,stride,resolved_upper", [
+    (20, 37, (3, 1), (3, 3), (0, -1, 1, 1)),   # hpad = 1 + 18 - 20 = -1, wpad = 3 + 36 - 37 = 2
+    (21, 37, (3, 1), (3, 3), (-1, -1, 1, 1)),  # hpad = -2: a negative border on both sides
+    (10, 12, (1, 3), (2, 2), (0, 1, 0, -1)),   # the same across: wpad = 1 + 10 - 12 = -1, hpad = 3 + 8 - 10 = 1
+])
+def test_same_padding_with_a_negative_border_is_refused_by_oracle_and_library(mode, h, w, kernel, stride, resolved_upper):
+    """src/layer/convolution.cpp:328-372 pads when wpad > 0 OR hpad > 0, with both values as they come: a kernel extent
+    below the stride in one dimension gives a negative border there, and src/layer/padding.cpp:62-87 then copies all
+    source rows into a smaller blob.  The reference has no defined result; the oracle returns -1, the library an error
+    from the one call every entry point sizes its output with.  SAME layers whose two values are both <= 0 get no
+    border at all and stay accepted."""
+    import ctypes as C
+    from ncnn_amd.hip import ConvDesc, lib
+    rng = np.random.default_rng(h + w)
+    d, x, wt, b, ws, ins, tops = _conv_case(rng, 8, h, w, 4, kernel, (1, 1), stride, (mode,) * 4, 1, 1, 0, (0, 0), False, True, False)
+    t, bo, l, r = oracle.resolve_padding(d)
+    if mode == -233:
+        assert (t, bo, l, r) == resolved_upper
+    assert min(t, bo, l, r) < 0 and max(t, bo, l, r) > 0
+    with pytest.raises(RuntimeError, match="-1"):
+        oracle.convolution_int8(d, x, wt, b, ws, ins[0], None)
+    cd = ConvDesc(w, h, 8, 1, 4, kernel[0], kernel[1], 1, 1, stride[0], stride[1], mode, mode, mode, mode, 0.0, 1)
+    ow, oh = C.c_int(), C.c_int()
+    assert lib().ncnnhip_conv_out_shape(C.byref(cd), C.byref(ow), C.byref(oh)) == -1
+    assert b"negative border" in lib().ncnnhip_last_error()
+    assert lib().ncnnhip_conv_from_float_supported(C.byref(cd)) == 0
+    # 1 x 1 at stride 2: both values are <= 0, no border is made, the layer runs
+    d1, x1, w1, b1, ws1, ins1, _ = _conv_case(rng, 8, h, w, 4, (1, 1), (1, 1), (2, 2), (mode,) * 4, 1, 1, 0, (0, 0), False, True, False)
+    assert oracle.resolve_padding(d1) == (0, 0, 0, 0)
+    assert oracle.convolution_int8(d1, x1, w1, b1, ws1, ins1[0], None).shape == (4, (h - 1) // 2 + 1, (w - 1) // 2 + 1)
+    cd1 = ConvDesc(w, h, 8, 1, 4, 1, 1, 1, 1, 2, 2, mode, mode, mode, mode, 0.0, 1)
+    assert lib().ncnnhip_conv_out_shape(C.byref(cd1), C.byref(ow), C.byref(oh)) == 0 and (oh.value, ow.value) == ((h - 1) // 2 + 1, (w - 1) // 2 + 1)
+
+
 # ----------------------------------------------------------------------------- inner product
 @pytest.mark.parametrize("rows,num_input,num_output,act,bias,int8_in", [
     (1, 64, 10, 0, False, False), (1, 2048, 100, 1, True, False), (5, 33, 7, 3, True, False), (3, 16, 4, 0, True, True)])
