@@ -233,6 +233,27 @@ class Mat:
 
 
 # ---- Net / Extractor -------------------------------------------------------------------------------
+class _Owned:
+    """C handles that have to be destroyed before the Net they belong to.  The wrapper object and its Net both hold
+    this record; whichever of the two is finalised first destroys the handles (when both die in one pass of the cyclic
+    garbage collector -- e.g. held by the traceback of a failed test -- Python runs their finalisers in any order, and
+    destroying an extractor after its net is a use after free)."""
+
+    def __init__(self, net, *pairs):
+        self.pairs = [(fn, h) for fn, h in pairs if h]
+        self.net_records = net._owned
+        self.net_records.add(self)
+
+    def close(self):
+        pairs, self.pairs = self.pairs, []
+        for fn, h in pairs:
+            try:
+                getattr(lib(), fn)(h)
+            except Exception:
+                pass
+        self.net_records.discard(self)
+
+
 class HipMat:
     """Handle to a device-resident blob (keep the Net alive for as long as this exists)."""
 
@@ -243,7 +264,7 @@ class HipMat:
     def __del__(self):
         try:
             if self.h_:
-                lib().ncnnhip_hipmat_destroy(self.h_)
+                lib().ncnnhip_hipmat_destroy(self.h_)  # (a device blob shares its buffer pool and may outlive its net)
                 self.h_ = None
         except Exception:
             pass
@@ -296,6 +317,7 @@ class HipGraph:
 class Net:
     def __init__(self):
         self.h_ = lib().ncnn_net_create()
+        self._owned = set()  # _Owned records of the extractors that live on this net
 
     def record(self, input_name, input_blob, output_name):
         """Runs the pass from the resident input blob to output_name once, then records it for replay."""
@@ -316,6 +338,8 @@ class Net:
 
     def __del__(self):
         try:
+            for rec in list(self._owned):  # the extractors first: they hand their command back to the net
+                rec.close()
             if self.h_:
                 lib().ncnn_net_destroy(self.h_)
                 self.h_ = None
@@ -393,17 +417,11 @@ class Extractor:
         self.h_ = lib().ncnn_extractor_create(net.h_)
         self.stream_handle = lib().ncnnhip_extractor_attach_stream(self.h_) if own_stream else None
         self._inputs = []
+        self._owned = _Owned(net, ("ncnn_extractor_destroy", self.h_), ("ncnnhip_extractor_detach_stream", self.stream_handle))
 
     def __del__(self):
-        try:
-            if self.h_:
-                lib().ncnn_extractor_destroy(self.h_)
-                self.h_ = None
-            if self.stream_handle:
-                lib().ncnnhip_extractor_detach_stream(self.stream_handle)
-                self.stream_handle = None
-        except Exception:
-            pass
+        self._owned.close()
+        self.h_ = self.stream_handle = None
 
     def set_lightmode(self, enable):
         opt = lib().ncnn_option_create()

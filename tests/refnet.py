@@ -73,7 +73,19 @@ def _pool(x, p):
     c, h, w = x.shape
     ph, pw = (s - (h - k) % s) % s, (s - (w - k) % s) % s
     oh, ow = (h + ph - k) // s + 1, (w + pw - k) // s + 1
-    assert kind == 0, "windowed average pooling is not used by the test nets"
+    if kind == 1:
+        # average without the border in the count (avgpool_count_include_pad = 0, src/layer/pooling.cpp:253-300): the taps of
+        # a window that lie inside the image are added in float32, rows first, and divided by their number
+        assert p.get(6, 0) == 0
+        xp = np.pad(x, ((0, 0), (0, ph), (0, pw)))
+        inside = np.pad(np.ones((h, w), bool), ((0, ph), (0, pw)))
+        acc, area = np.zeros((c, oh, ow), F), np.zeros((oh, ow), F)
+        for ky in range(k):
+            for kx in range(k):
+                sl = (slice(ky, ky + (oh - 1) * s + 1, s), slice(kx, kx + (ow - 1) * s + 1, s))
+                acc = (acc + xp[(slice(None),) + sl]).astype(F)  # border taps are zeros: adding them changes nothing
+                area += inside[sl]
+        return (acc / area).astype(F)
     xp = np.pad(x, ((0, 0), (0, ph), (0, pw)), constant_values=-np.finfo(F).max)
     win = np.stack([xp[:, ky: ky + (oh - 1) * s + 1: s, kx: kx + (ow - 1) * s + 1: s] for ky in range(k) for kx in range(k)])
     return win.max(axis=0).astype(F)

@@ -1,0 +1,130 @@
+"""Seeded random int8 networks through load_param -> load_model -> create_extractor -> extract, against the oracle-based
+executor on the same .param/.bin bytes, with blobs crossing the host per layer and with blobs resident in HBM.
+
+The topologies are drawn from the blocks the two benchmark networks are made of -- plain and strided convolutions,
+depthwise + pointwise pairs with and without a shortcut, bottlenecks with identity and projection shortcuts, max / average
+pooling, global pooling, InnerProduct, Softmax -- in random order, widths, map sizes and batch, so that the executor's
+fusion rules (Eltwise / ReLU / the next layer's Quantize inside a convolution's epilogue, sibling layers behind a Split,
+int8 blobs between requantising layers) meet combinations the two fixed networks do not contain.
+Every blob of every layer is compared bit for bit (Softmax to 1e-6); batch is the reference's per-sample loop
+(src/net.cpp:654-700)."""
+import os
+
+import numpy as np
+import pytest
+
+import refnet
+from ncnn_amd import host, zoo
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+COUNT = int(os.environ.get("NCNN_RANDOM_NETS", "40"))  # NCNN_RANDOM_NETS=<count> widens the walk
+
+
+def _pick(rng, options):
+    return options[int(rng.integers(len(options)))]
+
+
+def random_net(seed):
+    rng = np.random.default_rng(300 + seed)
+    cin = _pick(rng, [1, 3, 3, 4])
+    hw = int(rng.integers(14, 49))
+    g = zoo.Graph(seed, (cin, hw, hw))
+    relu6 = dict(act=3, act_params=(0.0, 6.0))
+    acts = [dict(act=0), dict(act=1), dict(act=1), relu6]
+    k = _pick(rng, [3, 3, 5, 7])
+    c = _pick(rng, [8, 16, 24, 32])
+    stride = _pick(rng, [1, 2])
+    x = g.conv("stem", "data", cin, c, k, stride=stride, pad=k // 2, **_pick(rng, acts))
+    size = (hw + 2 * (k // 2) - k) // stride + 1
+    for bi in range(int(rng.integers(2, 6))):
+        tag = "b%d" % bi
+        kind = _pick(rng, ["conv", "conv", "dwpw", "dwpw", "bottleneck", "bottleneck", "pool"])
+        if kind == "pool" and size >= 6:
+            pk = _pick(rng, [2, 3])
+            x = g.pool(tag + "_pool", x, _pick(rng, ["max", "avg"]), k=pk, stride=2)
+            size = -(-(size - pk) // 2) + 1
+        elif kind == "conv" or kind == "pool":
+            cout = _pick(rng, [8, 16, 20, 32, 48, 64])
+            ck = _pick(rng, [1, 3, 3])
+            cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
+            x = g.conv(tag + "_conv", x, c, cout, ck, stride=cs, pad=ck // 2, bias=rng.random() < 0.8, **_pick(rng, acts))
+            size = (size + 2 * (ck // 2) - ck) // cs + 1
+            c = cout
+        elif kind == "dwpw":
+            t = _pick(rng, [1, 2, 6])
+            cout = _pick(rng, [c, c, 16, 24, 40])
+            cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
+            residual = cs == 1 and cout == c
+            xa, xb = g.split(x) if residual else (x, None)
+            y = xa
+            hidden = c * t
+            if t != 1:
+                y = g.conv(tag + "_expand", y, c, hidden, 1, **relu6)
+            y = g.conv(tag + "_dw", y, hidden, hidden, 3, stride=cs, pad=1, group=hidden, **relu6)
+            y = g.conv(tag + "_project", y, hidden, cout, 1)
+            x = g.add(tag + "_add", xb, y) if residual else y
+            size = (size + 2 - 3) // cs + 1
+            c = cout
+        else:
+            mid = _pick(rng, [8, 16, 32])
+            cout = _pick(rng, [c, c, 32, 64, 96])
+            cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
+            xa, xb = g.split(x)
+            short = g.conv(tag + "_branch1", xb, c, cout, 1, stride=cs) if (cout != c or cs != 1 or rng.random() < 0.2) else xb
+            y = g.conv(tag + "_2a", xa, c, mid, 1, stride=cs, act=1)
+            y = g.conv(tag + "_2b", y, mid, mid, 3, pad=1, act=1)
+            y = g.conv(tag + "_2c", y, mid, cout, 1)
+            x = g.add(tag + "_sum", short, y)
+            if rng.random() < 0.8:
+                x = g.relu(tag + "_relu", x)
+            size = (size - 1) // cs + 1
+            c = cout
+    x = g.pool("gap", x, _pick(rng, ["avg", "avg", "max"]), global_pool=True)
+    n_out = _pick(rng, [5, 10, 37, 100])
+    x = g.fc("fc", x, c, n_out)
+    g.softmax("prob", x)
+    absmax = zoo.calibrate(g, 2)
+    param, blob, _ = zoo.to_int8_model(g, absmax)
+    return g, param, blob
+
+
+@pytest.mark.parametrize("resident", [False, True], ids=["host-blobs", "device-resident"])
+@pytest.mark.parametrize("seed", range(COUNT))
+def test_random_net_every_blob_matches(seed, resident):
+    g, param, blob = random_net(seed)
+    rng = np.random.default_rng(seed)
+    batch = _pick(rng, [1, 1, 2, 3])
+    xs = rng.uniform(0, 1, (batch,) + tuple(g.input_shape)).astype(F)
+    print("[case] random net", seed, "resident" if resident else "host", "batch", batch, "input", g.input_shape,
+          [L["name"] for L in g.layers if L["type"] not in ("Input", "Split")], flush=True)
+    refs = [refnet.run(param, blob, xs[i]) for i in range(batch)]
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(resident)
+    assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+    names = [t for L in g.layers if L["type"] not in ("Input", "Split", "Softmax") for t in L["tops"]]
+    # one extractor per blob: each pass may fuse what the blob asked for allows; then all of them from one extractor, in
+    # the network's order (in light mode a pass releases what it has consumed, the input included: asking one extractor for
+    # an earlier blob after a later one is an error here as in the reference)
+    for name in names:
+        ex = net.create_extractor()
+        ex.input("data", xs if batch > 1 else xs[0])
+        got = ex.extract(name)
+        for i in range(batch):
+            want = refs[i][name]
+            want = want.astype(F) if want.dtype == np.int8 else want
+            gi = got[i] if batch > 1 else got
+            assert gi.reshape(want.shape).shape == want.shape and np.array_equal(gi.reshape(want.shape), want), (name, i)
+    ex = net.create_extractor()
+    ex.input("data", xs if batch > 1 else xs[0])
+    for name in names:
+        got = ex.extract(name)
+        for i in range(batch):
+            want = refs[i][name]
+            want = want.astype(F) if want.dtype == np.int8 else want
+            gi = got[i] if batch > 1 else got
+            assert np.array_equal(gi.reshape(want.shape), want), ("one extractor", name, i)
+    prob = ex.extract("prob")
+    for i in range(batch):
+        assert np.allclose((prob[i] if batch > 1 else prob).reshape(-1), refs[i]["prob"].reshape(-1), rtol=1e-6, atol=1e-7)

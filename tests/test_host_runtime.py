@@ -152,6 +152,29 @@ def test_load_param_with_hip_layers_registered():
     assert blobs["c1"] == (1, 2) and blobs["c1a"] == (2, 3) and blobs["sum"] == (5, 6) and blobs["out"] == (6, -1)
 
 
+def test_python_wrappers_destroy_extractors_before_their_net_whatever_the_finaliser_order():
+    """Objects that die in one pass of the cyclic garbage collector (held, say, by the traceback of a failed test) are
+    finalised in any order; an extractor destroyed after its net would hand its command back to freed memory.  The net's
+    finaliser therefore destroys what lives on it first, and the extractor's own finaliser finds nothing left to do."""
+    import gc
+    net = host.Net()
+    net.register_int8_layers()
+    assert net.load_param_mem(PARAM) == 0
+    exs = [net.create_extractor(), net.create_extractor(own_stream=False)]
+    assert len(net._owned) == 2 and all(len(e._owned.pairs) >= 1 for e in exs)
+    host.Net.__del__(net)  # the net first, as the collector may do
+    assert net.h_ is None and not net._owned and all(e._owned.pairs == [] for e in exs)
+    for e in exs:
+        host.Extractor.__del__(e)  # nothing is destroyed twice
+    # and the ordinary order: an extractor that goes first takes its record off the net
+    net2 = host.Net()
+    ex = net2.create_extractor()
+    assert len(net2._owned) == 1
+    del ex
+    gc.collect()
+    assert not net2._owned
+
+
 def test_hot_layers_have_no_host_fallback():
     # without the HIP layers a net using Convolution cannot even be built
     net = host.Net()
