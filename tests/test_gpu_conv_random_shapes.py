@@ -86,11 +86,50 @@ def _float_edges(x, dtype, in_scale):
     return x
 
 
+def _draw_large(seed):
+    """A layer of 30 to 400 thousand output pixels (a batch of mid-sized maps): the kernels built for many pixels."""
+    rng = np.random.default_rng(50000 + seed)
+    depthwise = rng.random() < 0.2
+    batch = _pick(rng, [2, 4, 8, 16])
+    kernel, stride = _pick(rng, [((1, 1), (1, 1)), ((1, 1), (1, 1)), ((3, 3), (1, 1)), ((3, 3), (1, 1)), ((3, 3), (2, 2)), ((1, 1), (2, 2)), ((5, 5), (1, 1)),
+                                 ((3, 1), (1, 1))])
+    if depthwise:
+        c = outc = _pick(rng, [16, 32, 64, 96, 144])
+        if kernel[0] == 1:
+            kernel = (3, 3)
+    else:
+        c = _pick(rng, [8, 16, 32, 64, 64, 128])
+        outc = _pick(rng, [16, 24, 64, 64, 100, 128, 256])
+    pads = _pick(rng, [(kernel[0] // 2, kernel[0] // 2, kernel[1] // 2, kernel[1] // 2), (-233,) * 4, (0, 0, 0, 0)])
+    lo = 30000 * stride[0] * stride[1]
+    for _ in range(100):
+        h, w = int(rng.integers(24, 161)), int(rng.integers(24, 161))
+        if lo <= batch * h * w <= 400000 * stride[0] * stride[1]:
+            break
+    per_px = outc * (1 if depthwise else c) * kernel[0] * kernel[1]
+    while batch * h * w // (stride[0] * stride[1]) * per_px > 4e9 and h > 24:
+        h = h * 3 // 4
+    term = _pick(rng, [1, 2, 101, 102])
+    act, ap = _pick(rng, [(0, (0.0, 0.0)), (1, (0.0, 0.0)), (1, (0.0, 0.0)), (3, (0.0, 6.0)), (2, (0.1, 0.0))])
+    dtype = _pick(rng, [np.int8, np.int8, np.float32, np.float16])
+    tail = (not depthwise) and term < 100 and act == 0 and rng.random() < 0.6
+    return dict(depthwise=depthwise, batch=batch, c=c, h=h, w=w, outc=outc, kernel=kernel, dilation=(1, 1), stride=stride, pads=pads, term=term, act=act,
+                ap=ap, dtype=dtype, bias=rng.random() < 0.8, pad_value=0.0, tail=tail)
+
+
 # NCNN_RANDOM_LAYERS=<count> widens the walk (5000 layers take about a minute)
 @pytest.mark.parametrize("seed", range(int(os.environ.get("NCNN_RANDOM_LAYERS", "400"))))
 def test_random_layer_matches_oracle(rt, seed):
+    _check(rt, seed, _draw(seed))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("NCNN_RANDOM_LARGE_LAYERS", "32"))))
+def test_random_large_layer_matches_oracle(rt, seed):
+    _check(rt, seed, _draw_large(seed))
+
+
+def _check(rt, seed, p):
     from ncnn_amd.hip import ConvDesc, lib
-    p = _draw(seed)
     print("[case] random layer", seed, {k: (np.dtype(v).name if k == "dtype" else v) for k, v in p.items()}, flush=True)
     c, h, w, outc, batch, term = p["c"], p["h"], p["w"], p["outc"], p["batch"], p["term"]
     kernel, dilation, stride, pads, act, ap = p["kernel"], p["dilation"], p["stride"], p["pads"], p["act"], p["ap"]
