@@ -270,7 +270,8 @@ typedef struct ncnnhip_pool_desc
      * coordinates, [count_x0, count_x1) x [count_y0, count_y1); taps inside it but outside the image add zero and still
      * count.  The reference excludes taps by the layer's own pad parameters (and the tail pad only in pad_mode 0,
      * src/layer/pooling.cpp:255-305), so with SAME padding (pad_mode 2 / 3, pad parameters 0) the rectangle is the whole
-     * bordered image.  count_x1 <= count_x0 or count_y1 <= count_y0 (e.g. all zero) means the image itself. */
+     * bordered image.  All four zero means the image itself; any other rectangle is taken as given, an empty one too (pad
+     * parameters that leave no tap to count: the reference then divides 0 by 0 and so does this). */
     int count_x0, count_x1, count_y0, count_y1;
 } ncnnhip_pool_desc;
 int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, float* dst_dev, void* stream);

@@ -766,7 +766,9 @@ int ncnnhip_pooling_nhwc(const ncnnhip_pool_desc* desc, const float* src_dev, fl
     g.pad_left = d.pad_left;
     g.type = d.pooling_type;
     g.count_include_pad = d.avgpool_count_include_pad;
-    const bool own_rect = d.count_x1 > d.count_x0 && d.count_y1 > d.count_y0;
+    // all four zero: the image itself.  Any other rectangle is taken as it is, an empty one too (pad parameters that leave
+    // nothing to count: the reference then divides 0 by 0)
+    const bool own_rect = d.count_x0 != 0 || d.count_x1 != 0 || d.count_y0 != 0 || d.count_y1 != 0;
     g.cx0 = own_rect ? d.count_x0 : 0;
     g.cx1 = own_rect ? d.count_x1 : d.w;
     g.cy0 = own_rect ? d.count_y0 : 0;

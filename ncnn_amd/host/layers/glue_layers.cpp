@@ -208,6 +208,19 @@ public:
         outh = (h + pt + pb - kernel_h) / stride_h + 1;
     }
 
+    // A SAME mode gives a negative border where the window is below the stride in one dimension while the other dimension
+    // needs a border; the reference's border copy then writes every source row into a blob with fewer rows
+    // (src/layer/padding.cpp:62-87), out of bounds and with no defined result: such a layer is refused.
+    bool negative_same_border(int w, int h) const
+    {
+        if (pad_mode != 2 && pad_mode != 3) return false;
+        const int wpad = kernel_w + (w - 1) / stride_w * stride_w - w;
+        const int hpad = kernel_h + (h - 1) / stride_h * stride_h - h;
+        if (!((wpad > 0 || hpad > 0) && (wpad < 0 || hpad < 0))) return false;
+        NCNN_LOGE("Pooling: the padding mode resolves to a negative border (wpad %d hpad %d); the reference's border copy runs out of bounds for such a layer", wpad, hpad);
+        return true;
+    }
+
     // The rectangle (image coordinates) whose taps make up the divisor of an average without count_include_pad.  The
     // reference tests taps against the layer's own pad parameters in the bordered image -- rows [pad_top, hb - pad_bottom -
     // htailpad), tail pad only in pad_mode 0 (src/layer/pooling.cpp:255-305) -- so in pad_mode 2 / 3 the SAME border counts.
@@ -227,6 +240,13 @@ public:
         x1 = wb - pad_right - pl;
         y0 = pad_top - pt;
         y1 = hb - pad_bottom - pt;
+        if (x1 <= x0 || y1 <= y0)
+        {
+            // pad parameters that leave no tap to count (the reference divides 0 by 0): an empty rectangle that is not the
+            // all-zero one, which the kernel's interface reads as "the image itself"
+            x0 = y0 = 1;
+            x1 = y1 = 0;
+        }
     }
 
     virtual bool hip_quantise_transparent() const
@@ -290,6 +310,7 @@ public:
         d.kernel_h = kernel_h;
         d.stride_w = stride_w;
         d.stride_h = stride_h;
+        if (negative_same_border(bottom.w, bottom.h)) return -1;
         resolve(bottom.w, bottom.h, d.pad_top, d.pad_left, d.outw, d.outh);
         count_rect(bottom.w, bottom.h, d.count_x0, d.count_x1, d.count_y0, d.count_y1);
         top.create(d.outw, d.outh, bottom.c, quantised ? (size_t)1u : (size_t)4u, bottom.n, &cmd);
@@ -336,6 +357,7 @@ public:
         }
 
         int pt, pl, outw, outh;
+        if (negative_same_border(w, h)) return -1;
         resolve(w, h, pt, pl, outw, outh);
         top.create(outw, outh, channels, 4u, opt.blob_allocator);
         if (top.empty()) return -100;
