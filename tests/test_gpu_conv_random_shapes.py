@@ -150,6 +150,10 @@ def _check(rt, seed, p):
         x, wq, b, ws, ins, tops = cases.conv_case(seed, c, h, w, c, kernel, c, term, True, int8_in, by_group=True, batch=batch)
         if not by_group:
             ws = np.full(c, ws[0], F)
+        # a scale of its own for every channel, so that a table read with the wrong index shows
+        vary = np.random.default_rng(seed + 77)
+        ins = (ins * vary.uniform(0.6, 1.0, c)).astype(F)
+        tops = None if tops is None else (tops * vary.uniform(0.6, 1.4, c)).astype(F)
         if not int8_in:
             x = _float_edges(x, np.float32, ins[0])
         d = oracle.make_desc((c, h, w), c, kernel, dilation, stride, pads, 0.0, 1, c, term, act, ap)
@@ -182,3 +186,55 @@ def _check(rt, seed, p):
         return
     got = rt.conv_channels_last(x, wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, 0.0, 1, term, act, ap, from_float=from_float)
     assert got.dtype == want.dtype and np.array_equal(got, want, equal_nan=True)
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("NCNN_RANDOM_LAYERS", "400")) // 2))
+def test_random_planar_and_grouped_layer_matches_oracle(rt, seed):
+    """The entry point on planar [c][h][w] blobs (ncnn's own layout: the path of host Mats): dense, depthwise and grouped
+    layers (1 < group < channels, src/layer/convolutiondepthwise.cpp:515-636), with the int32 accumulators dumped beside the
+    result, and the dense ones again through the channels-last kernels behind a layout change."""
+    rng = np.random.default_rng(21000 + seed)
+    group = _pick(rng, [1, 1, 2, 3, 4, 8, 0, 0])  # 0: depthwise
+    if group == 0:
+        c = outc = group = _pick(rng, [3, 8, 16, 24, 40])
+    else:
+        c = group * int(rng.integers(1, 9))
+        outc = group * int(rng.integers(1, 13))
+    batch = _pick(rng, [1, 1, 2, 3])
+    kernel = _pick(rng, [(1, 1), (3, 3), (3, 3), (2, 2), (5, 3), (1, 3)])
+    dilation = _pick(rng, [(1, 1), (1, 1), (2, 1), (2, 2)])
+    stride = _pick(rng, [(1, 1), (1, 1), (2, 2), (1, 2)])
+    ext_w, ext_h = (kernel[0] - 1) * dilation[0] + 1, (kernel[1] - 1) * dilation[1] + 1
+    pads = _pick(rng, [(0, 0, 0, 0), tuple(int(v) for v in rng.integers(0, 3, 4)), (-233,) * 4, (-234,) * 4])
+    grow = 0 if pads[0] < 0 else pads[0] + pads[1]
+    w = int(rng.integers(max(1, ext_w - grow), 25))
+    grow = 0 if pads[0] < 0 else pads[2] + pads[3]
+    h = int(rng.integers(max(1, ext_h - grow), 25))
+    term = _pick(rng, [1, 2, 101, 102])
+    act, ap = _pick(rng, [(0, (0.0, 0.0)), (1, (0.0, 0.0)), (2, (0.1, 0.0)), (3, (0.0, 6.0)), (6, (0.2, 0.5))])
+    int8_in = bool(rng.integers(2))
+    pad_value = float(_pick(rng, [0.0, 0.0, -2.2, 3.7]))
+    print("[case] random planar layer", seed, dict(batch=batch, c=c, h=h, w=w, outc=outc, group=group, kernel=kernel, dilation=dilation, stride=stride, pads=pads,
+                                                 term=term, act=act, int8_in=int8_in, pad_value=pad_value), flush=True)
+    d = oracle.make_desc((c, h, w), outc, kernel, dilation, stride, pads, pad_value, 1, group, term, act, ap)
+    if min(oracle.resolve_padding(d)) < 0:
+        return  # (the refused SAME layers are walked by the first test of this file)
+    x, wq, b, ws, ins, tops = cases.conv_case(seed, c, h, w, outc, kernel, group, term, True, int8_in, by_group=group > 1, batch=batch)
+    if group > 1 and term in (2, 102):
+        ws[:] = ws[0]
+    if group > 1:
+        # a scale of its own for every group, so that a table read with the wrong index shows
+        ins = (ins * rng.uniform(0.6, 1.0, group)).astype(F)
+        tops = None if tops is None else (tops * rng.uniform(0.6, 1.4, group)).astype(F)
+        if int8_in:
+            x = np.clip(np.round(x.astype(F) * rng.uniform(0.5, 1.0)), -127, 127).astype(np.int8)
+    got, gacc = rt.conv_layer(x, wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, pad_value, group, term, act, ap, want_acc=True)
+    for i in range(batch):
+        if group > 1:
+            want, wacc = oracle.convolutiondepthwise_int8(d, x[i], wq, b, ws, ins, tops, want_acc=True)
+        else:
+            want, wacc = oracle.convolution_int8(d, x[i], wq, b, ws, ins[0], None if tops is None else tops[0], want_acc=True)
+        assert np.array_equal(gacc[i], wacc) and got.dtype == want.dtype and np.array_equal(got[i], want), "sample %d" % i
+    if group == 1:
+        again = rt.conv_layer(x, wq, b, ws, ins, tops, outc, kernel, dilation, stride, pads, pad_value, 1, term, act, ap)
+        assert np.array_equal(again, got)
