@@ -314,3 +314,42 @@ def test_packed_blockquant_entry_points_refuse_bad_arguments_before_touching_the
     assert lib.ncnnhip_gemm_blockquant_packed_supported(4096) == 1 and lib.ncnnhip_gemm_blockquant_packed_supported(4100) == 0
     assert lib.ncnnhip_gemm_blockquant_packed_supported(16384 + 16) == 0
     assert b"ncnnhip_gemm_blockquant_packed" in lib.ncnnhip_last_error()
+
+
+def test_every_entry_point_survives_null_arguments():
+    """Every exported function of the kernel library called with null pointers and zero sizes: an error code (or, for the
+    queries and the releases of nothing listed below, 0), never a crash.  The checks come before anything touches the device,
+    so this runs without a GPU; it runs in a child process so that a crash fails this test instead of ending the run."""
+    import subprocess
+    import sys
+    code = r'''
+import ctypes as C, sys
+sys.path.insert(0, %r)
+from ncnn_amd import hip
+lib = hip.lib()
+benign = {"ncnnhip_conv_from_float_supported", "ncnnhip_conv_fusion_supported", "ncnnhip_conv_small_tile_selected", "ncnnhip_conv_stem_supported",
+          "ncnnhip_gemm_blockquant_packed_supported", "ncnnhip_padded_channels",                      # queries: 0 = no
+          "ncnnhip_default_device_free", "ncnnhip_free", "ncnnhip_event_destroy", "ncnnhip_graph_destroy", "ncnnhip_stream_destroy",  # release of nothing
+          "ncnnhip_memcpy_d2d", "ncnnhip_memcpy_d2h", "ncnnhip_memcpy_h2d", "ncnnhip_memset",            # zero bytes
+          "ncnnhip_set_device_allocator"}                                                                # back to the default allocator
+bad = []
+for name in sorted(hip._SIGNATURES):
+    args = []
+    for t in hip._SIGNATURES[name]:
+        if t in (C.c_int, C.c_size_t):
+            args.append(0)
+        elif t is C.c_float:
+            args.append(0.0)
+        elif t is hip.Activation:
+            args.append(hip.Activation.make(0, (0.0, 0.0)))
+        else:
+            args.append(None)
+    print(name, flush=True)
+    r = getattr(lib, name)(*args)
+    if (r == 0) != (name in benign):
+        bad.append((name, r))
+print("BAD", bad)
+sys.exit(1 if bad else 0)
+''' % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, "last lines: %s %s" % (p.stdout.strip().splitlines()[-3:], p.stderr.strip().splitlines()[-3:])
