@@ -1460,15 +1460,26 @@ int HipGraph::record(const Net& net, const char* input_name, const HipMat& input
     std::shared_ptr<HipCommand> cmd = net.d->acquire_command();
     int ret = cmd->ensure_ready();
     if (ret != 0) return ret;
-    // a plain pass first: every pool buffer, workspace and lazily created table exists afterwards, so the recorded
-    // pass allocates nothing
+    // Plain passes first: every pool buffer, workspace and lazily created table exists afterwards, so the recorded pass
+    // allocates nothing.  One pass is not enough: it starts on an empty pool and gives every request a buffer of its own
+    // size, while the recorded pass starts with all of those idle and may hand an early request a buffer that a later,
+    // smaller one had made -- whose own request then finds only buffers the pool holds too wasteful for it and would
+    // allocate, which a stream under capture cannot.  So passes are repeated until one adds nothing to the pool; the
+    // recorded pass starts from the same state as that one (everything idle) and takes the same buffers.
+    size_t pooled = 0;
+    for (int pass = 0; pass < 8 && ret == 0; pass++)
     {
-        Extractor ex = net.create_extractor();
-        ex.d->st.cmd = cmd;
-        HipMat warm;
-        ret = ex.input(input_name, input);
-        if (ret == 0) ret = ex.extract(output_name, warm);
-        if (ret == 0) ret = cmd->synchronize();
+        {
+            Extractor ex = net.create_extractor();
+            ex.d->st.cmd = cmd;
+            HipMat warm;
+            ret = ex.input(input_name, input);
+            if (ret == 0) ret = ex.extract(output_name, warm);
+            if (ret == 0) ret = cmd->synchronize();
+        }
+        const size_t now = cmd->pooled_bytes();
+        if (pass > 0 && now == pooled) break;
+        pooled = now;
     }
     if (ret != 0) return ret;
     if (ncnnhip_stream_begin_capture(cmd->stream) != 0)

@@ -128,3 +128,33 @@ def test_random_net_every_blob_matches(seed, resident):
     prob = ex.extract("prob")
     for i in range(batch):
         assert np.allclose((prob[i] if batch > 1 else prob).reshape(-1), refs[i]["prob"].reshape(-1), rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("seed", range(COUNT))
+def test_random_net_recorded_pass_replays_like_the_oracle(seed):
+    """The same networks recorded into a graph once and replayed with new input values: every replay gives the oracle
+    executor's logits bit for bit (replays with eager passes and synchronisations in between)."""
+    g, param, blob = random_net(seed)
+    rng = np.random.default_rng(1000 + seed)
+    batch = _pick(rng, [1, 1, 2, 3])
+    shape = (batch,) + tuple(g.input_shape)
+    print("[case] random net, recorded", seed, "batch", batch, "input", g.input_shape, flush=True)
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(True)
+    assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+    x0 = rng.uniform(0, 1, shape).astype(F)
+    graph = net.record("data", net.upload(x0 if batch > 1 else x0[0]), "fc")
+    for i in range(3):
+        x = x0 if i == 0 else rng.uniform(0, 1, shape).astype(F)
+        want = np.stack([refnet.run(param, blob, x[j], want="fc")["fc"].reshape(-1) for j in range(batch)])
+        if i:
+            graph.update_input(x if batch > 1 else x[0])
+            ex = net.create_extractor()  # eager work on the same net between the replays
+            ex.input("data", x[0])
+            assert np.array_equal(np.asarray(ex.extract("fc")).reshape(-1), want[0])
+        graph.launch()
+        if i == 1:
+            graph.launch()  # back-to-back replays of the same values
+        graph.synchronize()
+        assert np.array_equal(graph.output().to_numpy().reshape(batch, -1), want), i
