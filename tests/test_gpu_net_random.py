@@ -158,3 +158,31 @@ def test_random_net_recorded_pass_replays_like_the_oracle(seed):
             graph.launch()  # back-to-back replays of the same values
         graph.synchronize()
         assert np.array_equal(graph.output().to_numpy().reshape(batch, -1), want), i
+
+
+@pytest.mark.parametrize("seed", range(COUNT))
+def test_random_net_through_the_plugin_matches_the_oracle(seed):
+    """The same networks with their Convolution / ConvolutionDepthWise / InnerProduct layers supplied by the plug-in, the C
+    shim written against nothing but the reference's c_api.h (function-pointer layer tables registered by type): every blob
+    bit for bit, from one extractor in the network's order."""
+    import ctypes as C
+    from ncnn_amd import build
+    host.lib()
+    if not os.path.exists(build.LIBPLUGIN):
+        raise RuntimeError("%s is missing: build it with python ncnn_amd/build.py" % build.LIBPLUGIN)
+    plugin = C.CDLL(build.LIBPLUGIN)
+    plugin.ncnnhip_plugin_register.restype = C.c_int
+    plugin.ncnnhip_plugin_register.argtypes = [C.c_void_p]
+    g, param, blob = random_net(seed)
+    x = np.random.default_rng(2000 + seed).uniform(0, 1, g.input_shape).astype(F)
+    print("[case] random net through the plug-in", seed, "input", g.input_shape, flush=True)
+    ref = refnet.run(param, blob, x)
+    net = host.Net()
+    assert plugin.ncnnhip_plugin_register(net.h_) == 0
+    assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+    ex = net.create_extractor()
+    ex.input("data", x)
+    for name in [t for L in g.layers if L["type"] not in ("Input", "Split", "Softmax") for t in L["tops"]]:
+        want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
+        got = ex.extract(name)
+        assert np.array_equal(np.asarray(got).reshape(want.shape), want), name
