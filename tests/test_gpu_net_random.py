@@ -25,15 +25,16 @@ def _pick(rng, options):
     return options[int(rng.integers(len(options)))]
 
 
-def random_net(seed):
-    rng = np.random.default_rng(300 + seed)
+def random_net(seed, wide=1):
+    """wide = 4: four times the channels on maps of 48 to 112 pixels (the kernels built for many pixels and channels)."""
+    rng = np.random.default_rng(300 + seed + 100000 * (wide - 1))
     cin = _pick(rng, [1, 3, 3, 4])
-    hw = int(rng.integers(14, 49))
+    hw = int(rng.integers(14, 49)) if wide == 1 else int(rng.integers(48, 113))
     g = zoo.Graph(seed, (cin, hw, hw))
     relu6 = dict(act=3, act_params=(0.0, 6.0))
     acts = [dict(act=0), dict(act=1), dict(act=1), relu6]
     k = _pick(rng, [3, 3, 5, 7])
-    c = _pick(rng, [8, 16, 24, 32])
+    c = _pick(rng, [8, 16, 24, 32]) * (2 if wide > 1 else 1)
     stride = _pick(rng, [1, 2])
     x = g.conv("stem", "data", cin, c, k, stride=stride, pad=k // 2, **_pick(rng, acts))
     size = (hw + 2 * (k // 2) - k) // stride + 1
@@ -45,7 +46,7 @@ def random_net(seed):
             x = g.pool(tag + "_pool", x, _pick(rng, ["max", "avg"]), k=pk, stride=2)
             size = -(-(size - pk) // 2) + 1
         elif kind == "conv" or kind == "pool":
-            cout = _pick(rng, [8, 16, 20, 32, 48, 64])
+            cout = _pick(rng, [8, 16, 20, 32, 48, 64]) * wide
             ck = _pick(rng, [1, 3, 3])
             cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
             x = g.conv(tag + "_conv", x, c, cout, ck, stride=cs, pad=ck // 2, bias=rng.random() < 0.8, **_pick(rng, acts))
@@ -53,7 +54,7 @@ def random_net(seed):
             c = cout
         elif kind == "dwpw":
             t = _pick(rng, [1, 2, 6])
-            cout = _pick(rng, [c, c, 16, 24, 40])
+            cout = _pick(rng, [c, c, 16 * wide, 24 * wide, 40 * wide])
             cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
             residual = cs == 1 and cout == c
             xa, xb = g.split(x) if residual else (x, None)
@@ -67,8 +68,8 @@ def random_net(seed):
             size = (size + 2 - 3) // cs + 1
             c = cout
         else:
-            mid = _pick(rng, [8, 16, 32])
-            cout = _pick(rng, [c, c, 32, 64, 96])
+            mid = _pick(rng, [8, 16, 32]) * wide
+            cout = _pick(rng, [c, c, 32 * wide, 64 * wide, 96 * wide])
             cs = 2 if (size >= 8 and rng.random() < 0.3) else 1
             xa, xb = g.split(x)
             short = g.conv(tag + "_branch1", xb, c, cout, 1, stride=cs) if (cout != c or cs != 1 or rng.random() < 0.2) else xb
@@ -84,7 +85,7 @@ def random_net(seed):
     n_out = _pick(rng, [5, 10, 37, 100])
     x = g.fc("fc", x, c, n_out)
     g.softmax("prob", x)
-    absmax = zoo.calibrate(g, 2)
+    absmax = zoo.calibrate(g, 2 if wide == 1 else 1)
     param, blob, _ = zoo.to_int8_model(g, absmax)
     return g, param, blob
 
@@ -186,3 +187,30 @@ def test_random_net_through_the_plugin_matches_the_oracle(seed):
         want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
         got = ex.extract(name)
         assert np.array_equal(np.asarray(got).reshape(want.shape), want), name
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("NCNN_RANDOM_WIDE_NETS", "10"))))
+def test_random_wide_net_at_a_batch_matches_the_oracle(seed):
+    """Networks of the same blocks with four times the channels on maps of 48 to 112 pixels, at batch 4 to 16, device
+    resident: the class scores and the deepest blobs of every sample bit for bit the oracle executor's."""
+    g, param, blob = random_net(seed, wide=4)
+    rng = np.random.default_rng(3000 + seed)
+    batch = _pick(rng, [4, 8, 16])
+    xs = rng.uniform(0, 1, (batch,) + tuple(g.input_shape)).astype(F)
+    names = [t for L in g.layers if L["type"] not in ("Input", "Split", "Softmax") for t in L["tops"]]
+    probes = names[-4:]
+    print("[case] random wide net", seed, "batch", batch, "input", g.input_shape, names, flush=True)
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(True)
+    assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+    got = {}
+    for name in probes:
+        ex = net.create_extractor()
+        ex.input("data", xs)
+        got[name] = np.asarray(ex.extract(name))
+    for i in (0, batch // 2, batch - 1):
+        ref = refnet.run(param, blob, xs[i])
+        for name in probes:
+            want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
+            assert np.array_equal(got[name][i].reshape(want.shape), want), (name, i)
