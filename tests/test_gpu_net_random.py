@@ -214,3 +214,47 @@ def test_random_wide_net_at_a_batch_matches_the_oracle(seed):
         for name in probes:
             want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
             assert np.array_equal(got[name][i].reshape(want.shape), want), (name, i)
+
+
+def test_random_nets_on_concurrent_threads():
+    """Six threads at once, each with a network of its own (its own Net, layers, weights, streams and pools) plus one
+    network they all share, pass after pass with new inputs: whatever the library keeps per process -- lazily built
+    tables, the device allocator, the zero line of the convolution kernels -- serves them all.  Every result bit for
+    bit the oracle executor's."""
+    import threading
+
+    def load(param, blob):
+        net = host.Net()
+        assert net.register_int8_layers() == 0
+        net.set_use_hip_compute(True)
+        assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+        return net
+
+    shared_g, shared_param, shared_blob = random_net(7000)
+    shared = load(shared_param, shared_blob)
+    errors = []
+
+    def worker(t):
+        try:
+            g, param, blob = random_net(7001 + t, wide=4 if t % 2 else 1)
+            net = load(param, blob)
+            rng = np.random.default_rng(t)
+            for it in range(6):
+                for gg, pp, bb, nn in ((g, param, blob, net), (shared_g, shared_param, shared_blob, shared)):
+                    x = rng.uniform(0, 1, gg.input_shape).astype(F)
+                    ex = nn.create_extractor()
+                    ex.input("data", x)
+                    got = np.asarray(ex.extract("fc")).reshape(-1)
+                    want = refnet.run(pp, bb, x, want="fc")["fc"].reshape(-1)
+                    if not np.array_equal(got, want):
+                        errors.append("thread %d pass %d: result differs" % (t, it))
+                        return
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (t, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(6)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
