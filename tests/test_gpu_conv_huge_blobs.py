@@ -35,3 +35,27 @@ def test_output_blobs_beyond_32_bit_offsets(rt, batch, c, hw, outc, kernel, grou
     for i in (0, 1, batch // 2, batch - 2, batch - 1):
         one = rt.conv_channels_last(xb[i:i + 1], *args)
         assert np.array_equal(got[i], one[0]), "sample %d" % i
+
+
+@pytest.mark.parametrize("which,out", [("resnet50", "fc1000"), ("mobilenetv2", "fc")])
+def test_benchmark_network_at_batch_1500(which, out):
+    """The whole networks at 224 x 224 and batch 1500, device resident: the fp32 shortcut blobs of ResNet-50's second stage
+    are 4.8e9 bytes each, MobileNetV2's widest int8 blob 1.8e9 elements.  Class scores of the first, middle and last
+    samples against single-sample passes, bit for bit."""
+    from ncnn_amd import host, zoo
+    batch = 1500
+    print("[case] huge net", which, batch, flush=True)
+    g, param, blob, info = zoo.build(which, input_hw=224, n_calib=1)
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(True)
+    assert net.load_param_mem(param) == 0 and net.load_model_mem(blob) == 0
+    base = np.random.default_rng(1).uniform(0, 1, (8,) + tuple(g.input_shape)).astype(F)
+    xs = np.concatenate([np.roll(base, i, axis=3) for i in range((batch + 7) // 8)])[:batch]
+    ex = net.create_extractor()
+    ex.input("data", xs)
+    got = np.asarray(ex.extract(out)).reshape(batch, -1)
+    for i in (0, 1, batch // 2, batch - 2, batch - 1):
+        one = net.create_extractor()
+        one.input("data", xs[i])
+        assert np.array_equal(got[i], np.asarray(one.extract(out)).reshape(-1)), "sample %d" % i
