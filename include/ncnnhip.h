@@ -248,7 +248,9 @@ int ncnnhip_dwconv_int8_nhwc(const ncnnhip_conv_desc* desc, const int8_t* nhwc_d
                              void* out_nhwc_dev, void* stream);
 
 /* ------------------------------------------------------------------ fp32 layers between the int8 layers
- * ReLU::forward_inplace (src/layer/relu.cpp): x < 0 ? x*slope : x; int8 blobs clamp at zero.  Flat over `count` elements. */
+ * ReLU::forward_inplace (src/layer/relu.cpp): x < 0 ? x*slope : x; int8 blobs clamp at zero.  Flat over `count` elements.
+ * fp32: count is a multiple of 4 and the blobs are 16-byte aligned, as device blobs are (channels padded to 16); anything
+ * else is NCNNHIP_ERROR.  The same holds for ncnnhip_eltwise. */
 int ncnnhip_relu(const void* src_dev, void* dst_dev, int elemsize, size_t count, float slope, void* stream);
 /* Dropout::forward_inplace (src/layer/dropout.cpp): x * scale. */
 int ncnnhip_scale(const float* src_dev, float* dst_dev, size_t count, float scale, void* stream);
