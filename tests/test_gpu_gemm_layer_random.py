@@ -3,8 +3,8 @@
 Gemm::forward_int8 (src/layer/gemm.cpp:745-966) takes A, B and C each as a constant of the model or as a bottom blob, A
 and B stored either way round, C in one of five broadcast shapes (named by a parameter when constant, found from its shape
 when it is a blob), the output plain, transposed and / or as an N x 1 x M blob.  The forms are drawn here instead of listed,
-with odd M, N, K; every one has to come out bit for bit the oracle's, on host Mats and on blobs that stay in HBM, and in the
-second mode the layer has to run as a device layer."""
+with odd M, N, K; every one has to come out bit for bit the oracle's, on host Mats, on blobs that stay in HBM (where the
+layer has to run as a device layer) and through the plug-in written against the reference's c_api.h."""
 import os
 
 import numpy as np
@@ -22,8 +22,28 @@ def _pick(rng, options):
     return options[int(rng.integers(len(options)))]
 
 
+def _plugin():
+    import ctypes as C
+    from ncnn_amd import build
+    host.lib()
+    if not os.path.exists(build.LIBPLUGIN):
+        raise RuntimeError("%s is missing: build it with python ncnn_amd/build.py" % build.LIBPLUGIN)
+    p = C.CDLL(build.LIBPLUGIN)
+    p.ncnnhip_plugin_register.restype = C.c_int
+    p.ncnnhip_plugin_register.argtypes = [C.c_void_p]
+    return p
+
+
 def _run(lines, blob, feeds, resident):
     net = host.Net()
+    if resident == "plugin":
+        # the layer as the C shim written against the reference's c_api.h supplies it (function-pointer table, host Mats)
+        assert _plugin().ncnnhip_plugin_register(net.h_) == 0
+        assert net.load_param_mem(mw.assemble_param(lines)) == 0 and net.load_model_mem(blob) == 0
+        ex = net.create_extractor()
+        for k, v in feeds.items():
+            ex.input(k, v)
+        return ex.extract("out"), "plugin"
     assert net.register_int8_layers() == 0
     net.set_use_hip_compute(resident)
     assert net.load_param_mem(mw.assemble_param(lines)) == 0 and net.load_model_mem(blob) == 0
@@ -36,7 +56,7 @@ def _run(lines, blob, feeds, resident):
     return got, where["g"]
 
 
-@pytest.mark.parametrize("resident", [False, True], ids=["host-blobs", "device-resident"])
+@pytest.mark.parametrize("resident", [False, True, "plugin"], ids=["host-blobs", "device-resident", "plug-in"])
 @pytest.mark.parametrize("seed", range(COUNT))
 def test_random_gemm_layer_form_matches_oracle(seed, resident):
     rng = np.random.default_rng(11000 + seed)
@@ -49,7 +69,7 @@ def test_random_gemm_layer_form_matches_oracle(seed, resident):
     bt = _pick(rng, [0, 1, 2, 3, 4]) if form_c != "none" else -1
     alpha, beta = _pick(rng, [1.0, 1.0, 0.5, 1.7, -1.0]), _pick(rng, [1.0, 1.0, 0.25, 2.0, -1.0])
     transpose, n1m = bool(rng.integers(2)), rng.random() < 0.25
-    print("[case] random gemm layer", seed, "resident" if resident else "host", (m, n, k), "A:", form_a, "B:", form_b, "C:", form_c, bt,
+    print("[case] random gemm layer", seed, resident if resident == "plugin" else "resident" if resident else "host", (m, n, k), "A:", form_a, "B:", form_b, "C:", form_c, bt,
           alpha, beta, "transposed" if transpose else "", "N1M" if n1m else "", flush=True)
 
     a = rng.standard_normal((m, k), dtype=F)
@@ -118,4 +138,4 @@ def test_random_gemm_layer_form_matches_oracle(seed, resident):
     if n1m:
         want = want.reshape(want.shape[0], 1, want.shape[1])
     assert np.asarray(got).size == want.size and np.array_equal(np.asarray(got).reshape(want.shape), want)
-    assert where == ("device" if resident else "host")
+    assert where == ("plugin" if resident == "plugin" else "device" if resident else "host")
