@@ -139,3 +139,49 @@ def test_random_gemm_layer_form_matches_oracle(seed, resident):
         want = want.reshape(want.shape[0], 1, want.shape[1])
     assert np.asarray(got).size == want.size and np.array_equal(np.asarray(got).reshape(want.shape), want)
     assert where == ("plugin" if resident == "plugin" else "device" if resident else "host")
+
+
+@pytest.mark.parametrize("resident", [False, True, "plugin"], ids=["host-blobs", "device-resident", "plug-in"])
+@pytest.mark.parametrize("seed", range(COUNT))
+def test_random_block_quantised_gemm_layer_matches_float64(seed, resident):
+    """Gemm::forward_weight_block_quantize (src/layer/gemm.cpp:339-483) as a layer: 4 / 6 / 8-bit weights in blocks of 32 / 64
+    / 128, with and without per-K input scales, C absent, a constant of the model or the second bottom blob in any of its
+    shapes, 1 to 140 activation rows, K in whole 16s (the matrix-core layouts) and not.  |got - value| <= 1e-5 * sum |a * w|
+    against float64."""
+    from tests import npref
+    rng = np.random.default_rng(15000 + seed)
+    bits, block, insc = _pick(rng, [8, 8, 4, 6]), _pick(rng, [32, 64, 64, 128]), bool(rng.integers(2))
+    m = int(_pick(rng, [1, 1, 2, 3, 4, 5, 9, 16, 20, 33, 70, 140]))
+    n = int(rng.integers(1, 200))
+    k = int(_pick(rng, [16 * int(rng.integers(1, 40)), 64 * int(rng.integers(1, 80)), int(rng.integers(1, 700)), 4096 + 64 * int(rng.integers(0, 70))]))
+    form_c = _pick(rng, ["none", "none", "constant", "blob"])
+    bt = _pick(rng, [0, 1, 2, 3, 4]) if form_c != "none" else -1
+    if m == n:
+        n += 1
+    alpha, beta = _pick(rng, [1.0, 0.5, -1.0]), _pick(rng, [1.0, 2.0, 0.25])
+    print("[case] random block-quantised gemm layer", seed, resident, bits, block, insc, (m, n, k), "C:", form_c, bt, alpha, beta, flush=True)
+    a = rng.standard_normal((m, k), dtype=F)
+    w = (rng.standard_normal((n, k), dtype=F) * F(0.02)).astype(F)
+    packed, scales = oracle.blockquant_pack(w, bits, block)
+    ins = rng.uniform(0.5, 1.5, k).astype(F) if insc else None
+    term = bits * 100 + int(insc) * 10 + {32: 0, 64: 1, 128: 2}[block]
+    lines, feeds, bottoms = ["Input in0 0 1 a 0=%d 1=%d" % (k, m)], {"a": a}, ["a"]
+    kw = dict(N=n, K=k, constantB=1, quantize_term=term, alpha=alpha, beta=beta)
+    blob = mw.weight_blob(packed.view(np.int8))
+    c = None
+    if form_c != "none":
+        c = {0: rng.standard_normal(1), 1: rng.standard_normal(m), 2: rng.standard_normal((m, 1)), 3: rng.standard_normal((m, n)),
+             4: rng.standard_normal((1, n))}[bt].astype(F)
+        if form_c == "constant":
+            blob += mw.weight_blob(c)
+            kw.update(constantC=1, broadcast_type_C=bt, M=m)
+        else:
+            lines.append("Input in1 0 1 c 0=%d" % c.size if c.ndim == 1 else "Input in1 0 1 c 0=%d 1=%d" % (c.shape[1], c.shape[0]))
+            feeds["c"] = c
+            bottoms.append("c")
+    blob += mw.raw_f32(scales) + (mw.raw_f32(ins) if insc else b"")
+    lines.append(mw.gemm_param("g", bottoms, "out", **kw))
+    got, where = _run(lines, blob, feeds, resident)
+    val, floor = npref.blockquant_gemm_f64(a, packed, scales, bits, block, ins, c, bt, alpha, beta)
+    assert got.shape == val.shape and np.all(np.abs(got - val) <= 1e-5 * floor + 1e-30)
+    assert where == ("plugin" if resident == "plugin" else "device" if resident else "host")
