@@ -58,6 +58,16 @@ int Convolution_hip::load_param(const ParamDict& pd)
         NCNN_LOGE("%s: dynamic weights are not part of the int8 path", type.c_str());
         return -1;
     }
+    // values a model file cannot mean (a damaged file): refused here, before any product of them is formed
+    const int lim = 32767;
+    if (num_output < 1 || num_output > (1 << 24) || kernel_w < 1 || kernel_h < 1 || kernel_w > lim || kernel_h > lim || dilation_w < 1 || dilation_h < 1 ||
+        dilation_w > lim || dilation_h > lim || stride_w < 1 || stride_h < 1 || stride_w > lim || stride_h > lim || weight_data_size < 1 ||
+        (long long)kernel_w * kernel_h > (1 << 24))
+    {
+        NCNN_LOGE("%s %s: parameters out of range (num_output %d, kernel %d x %d, dilation %d x %d, stride %d x %d, weight_data_size %d)", type.c_str(),
+                  name.c_str(), num_output, kernel_w, kernel_h, dilation_w, dilation_h, stride_w, stride_h, weight_data_size);
+        return -1;
+    }
     if (group < 1 || num_output % group != 0) return -100; // the reference rejects an invalid group this way
     if (!int8_scale_term)
     {

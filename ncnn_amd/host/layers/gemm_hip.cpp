@@ -64,6 +64,11 @@ int Gemm_hip::load_param(const ParamDict& pd)
     quantize_term = pd.get(18, 0);
     weight_block_quantize = term_is_block_quant(quantize_term);
 
+    if (constantM < 0 || constantN < 0 || constantK < 0 || constantM > (1 << 24) || constantN > (1 << 24) || constantK > (1 << 24))
+    {
+        NCNN_LOGE("Gemm %s: constant sizes out of range (M %d, N %d, K %d)", name.c_str(), constantM, constantN, constantK);
+        return -1;
+    }
     if (quantize_term == 0)
     {
         NCNN_LOGE("Gemm %s: no quantize_term; only the quantised paths run on this device runtime", name.c_str());

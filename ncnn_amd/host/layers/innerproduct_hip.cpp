@@ -27,6 +27,11 @@ int InnerProduct_hip::load_param(const ParamDict& pd)
     int8_scale_term = pd.get(8, 0);
     activation_type = pd.get(9, 0);
     activation_params = pd.get(10, Mat());
+    if (num_output < 1 || num_output > (1 << 24) || weight_data_size < 1 || weight_data_size % num_output != 0)
+    {
+        NCNN_LOGE("InnerProduct %s: parameters out of range (num_output %d, weight_data_size %d)", name.c_str(), num_output, weight_data_size);
+        return -1;
+    }
     if (!int8_scale_term)
     {
         NCNN_LOGE("InnerProduct %s: no int8_scale_term; only the quantised path runs on this device runtime", name.c_str());

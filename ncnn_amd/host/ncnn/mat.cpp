@@ -48,6 +48,7 @@ void Mat::create_any(int _dims, int _w, int _h, int _d, int _c, size_t _elemsize
 {
     if (same_as(_dims, _w, _h, _d, _c, _elemsize, _elempack, _n, _allocator)) return;
     release();
+    if (_w < 0 || _h < 0 || _d < 0 || _c < 0) return; // a negative extent (a damaged model file): the Mat stays empty, callers test empty()
     set_shape(_dims, _w, _h, _d, _c, _elemsize, _elempack, _n);
     allocate(_allocator);
 }

@@ -897,7 +897,9 @@ int Net::load_param(const DataReader& dr)
         return -1;
     }
     int layer_count = 0, blob_count = 0;
-    if (dr.scan("%d", &layer_count) != 1 || dr.scan("%d", &blob_count) != 1 || layer_count <= 0 || blob_count <= 0)
+    // (counts are bounded so that a damaged file gives an error instead of an allocation of gigabytes)
+    if (dr.scan("%d", &layer_count) != 1 || dr.scan("%d", &blob_count) != 1 || layer_count <= 0 || blob_count <= 0 || layer_count > (1 << 24) ||
+        blob_count > (1 << 24))
     {
         NCNN_LOGE("invalid layer_count or blob_count");
         return -1;
@@ -915,6 +917,12 @@ int Net::load_param(const DataReader& dr)
         if (dr.scan("%255s", type) != 1 || dr.scan("%255s", name) != 1 || dr.scan("%d", &nbottom) != 1 || dr.scan("%d", &ntop) != 1)
         {
             NCNN_LOGE("parse layer header failed at layer %d", li);
+            clear();
+            return -1;
+        }
+        if (nbottom < 0 || ntop < 0 || nbottom > blob_count || ntop > blob_count)
+        {
+            NCNN_LOGE("layer %d %s: %d bottom and %d top blobs in a net of %d blobs", li, name, nbottom, ntop, blob_count);
             clear();
             return -1;
         }

@@ -166,7 +166,7 @@ int ParamDict::load_param(const DataReader& dr)
         if (counted_array)
         {
             int len = 0;
-            if (dr.scan("%d", &len) != 1)
+            if (dr.scan("%d", &len) != 1 || len < 0 || len > (1 << 24))
             {
                 NCNN_LOGE("ParamDict read array length failed");
                 return -1;

@@ -353,3 +353,39 @@ sys.exit(1 if bad else 0)
 ''' % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0, "last lines: %s %s" % (p.stdout.strip().splitlines()[-3:], p.stderr.strip().splitlines()[-3:])
+
+
+@pytest.mark.parametrize("damage,what", [
+    (("Convolution              c1                       1 1 data c1", "Convolution              c1                       -1 1 data c1"), "a negative bottom count"),
+    (("Convolution              c1                       1 1 data c1", "Convolution              c1                       1 99999999 data c1"), "more top blobs than the net has"),
+    ((" 9=1", " 9=1 -23310=-5,1"), "a counted array of negative length"),
+    ((" 9=1", " 9=1 -23310=999999999,1"), "a counted array of absurd length"),
+    (("7767517\n3 3", "7767517\n2000000000 3"), "an absurd layer count"),
+    ((" 1=3 11=3 ", " 1=1133903872 11=3 "), "a kernel whose tap count overflows an int"),
+    ((" 0=16 1=3 ", " 0=-16 1=3 "), "a negative num_output"),
+])
+def test_load_param_refuses_damaged_counts_and_sizes(damage, what):
+    """Counts and sizes a model file cannot mean are answered with an error code, before anything is allocated or multiplied
+    with them (found by mutating .param texts: a negative blob count reached std::vector::resize, a negative array length
+    Mat::create)."""
+    text = ("7767517\n3 3\nInput                    data                     0 1 data 0=16 1=16 2=4\n"
+            "Convolution              c1                       1 1 data c1 0=16 1=3 11=3 2=1 3=1 4=1 5=1 6=576 8=101 9=1\n"
+            "ReLU                     r                        1 1 c1 out\n")
+    net = host.Net()
+    net.register_int8_layers()
+    assert net.load_param_mem(text) == 0
+    old, new = damage
+    assert old in text, what
+    net = host.Net()
+    net.register_int8_layers()
+    assert net.load_param_mem(text.replace(old, new, 1)) != 0, what
+
+
+def test_param_parser_survives_mutated_text():
+    """600 mutated .param texts (tests/paramfuzz.py) in a child process: return codes, never a crash."""
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    p = subprocess.run([sys.executable, os.path.join(here, "paramfuzz.py"), "11", "600"], capture_output=True, text=True, timeout=300,
+                       cwd=os.path.dirname(here), env=dict(os.environ, PYTHONPATH=os.path.dirname(here)))
+    assert p.returncode == 0 and "survived 600" in p.stdout, (p.returncode, p.stdout[-300:], p.stderr[-600:])
