@@ -389,3 +389,29 @@ def test_param_parser_survives_mutated_text():
     p = subprocess.run([sys.executable, os.path.join(here, "paramfuzz.py"), "11", "600"], capture_output=True, text=True, timeout=300,
                        cwd=os.path.dirname(here), env=dict(os.environ, PYTHONPATH=os.path.dirname(here)))
     assert p.returncode == 0 and "survived 600" in p.stdout, (p.returncode, p.stdout[-300:], p.stderr[-600:])
+
+
+def test_paramdict_text_parser_on_the_reference_tests_own_vectors():
+    """tests/golden/paramdict_vectors.json: the inputs and expected values that the reference's tests/test_paramdict.cpp holds
+    for the text parser (src/paramdict.cpp:263-489) -- types, ints, floats compared as float32 the way the reference test
+    compares them (f != 0.01f), arrays with a trailing comma, bare and quoted strings."""
+    import json
+    here = os.path.dirname(os.path.abspath(__file__))
+    data = json.load(open(os.path.join(here, "golden", "paramdict_vectors.json")))
+    checked = 0
+    for vec in data["vectors"]:
+        for e in vec["expect"]:
+            t, v, arr = host.paramdict_probe(vec["text"] + "\n", e["id"])
+            assert t == e["type"], (vec["text"], e)
+            if "int" in e:
+                assert np.array([v], np.uint32).view(np.int32)[0] == e["int"]
+            elif "float" in e:
+                assert v == bits(float(np.float32(e["float"])))
+            elif "ints" in e:
+                assert v == len(e["ints"]) and list(np.array(arr[:v], np.uint32).view(np.int32)) == e["ints"]
+            elif "floats" in e:
+                assert v == len(e["floats"]) and arr[:v] == [bits(float(np.float32(f))) for f in e["floats"]]
+            else:
+                assert v == len(e["string"]) and bytes(arr[:v]).decode() == e["string"]
+            checked += 1
+    assert checked == 14
