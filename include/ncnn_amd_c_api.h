@@ -245,6 +245,8 @@ int ncnn_net_get_blob_consumer(const ncnn_net_t net, int i);
  * type (0 unset, 2 int, 3 float, 5 int array, 6 float array, 7 string, -1 parse error); the raw
  * 32-bit payload (or the array length) goes to *value_bits, array elements to array_bits[0..cap). */
 int ncnn_paramdict_probe(const char* text, int id, unsigned int* value_bits, unsigned int* array_bits, int cap);
+/* the same for the binary form (ParamDict::load_param_bin, src/paramdict.cpp:491-637); mem ends with the end mark -233 */
+int ncnn_paramdict_probe_bin(const unsigned char* mem, int id, unsigned int* value_bits, unsigned int* array_bits, int cap);
 
 /* Reads one blob of `w` elements of load-type `type` (0 tagged / 1 raw fp32) from a .bin image and
  * copies it as fp32 or int8 to out; returns the element size (4 or 1), 0 on failure. *consumed =

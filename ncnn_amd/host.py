@@ -118,6 +118,7 @@ def lib():
             "ncnn_net_register_custom_layer_by_type": (None, [vp, C.c_char_p, LAYER_CREATOR, LAYER_DESTROYER, vp]),
             "ncnn_net_register_custom_layer_by_typeindex": (None, [vp, ci, LAYER_CREATOR, LAYER_DESTROYER, vp]),
             "ncnn_paramdict_probe": (ci, [C.c_char_p, ci, C.POINTER(C.c_uint), C.POINTER(C.c_uint), ci]),
+            "ncnn_paramdict_probe_bin": (ci, [C.c_char_p, ci, C.POINTER(C.c_uint), C.POINTER(C.c_uint), ci]),
             "ncnn_modelbin_probe": (ci, [C.c_char_p, ci, ci, vp, C.POINTER(cs)]),
         }
         for flag in LAYER_FLAGS:
@@ -136,6 +137,13 @@ def paramdict_probe(text, pid):
     v = C.c_uint(0)
     arr = (C.c_uint * 64)()
     t = lib().ncnn_paramdict_probe(text.encode(), pid, C.byref(v), arr, 64)
+    return t, v.value, list(arr)
+
+
+def paramdict_probe_bin(mem, pid):
+    v = C.c_uint(0)
+    arr = (C.c_uint * 64)()
+    t = lib().ncnn_paramdict_probe_bin(bytes(mem), pid, C.byref(v), arr, 64)
     return t, v.value, list(arr)
 
 

@@ -499,19 +499,36 @@ int ncnn_net_get_blob_consumer(const ncnn_net_t net, int i)
     return N(net)->blobs()[(size_t)i].consumer;
 }
 
+static int paramdict_probe_slot(const ParamDict& pd, int id, unsigned int* value_bits, unsigned int* array_bits, int cap);
+
+// the same for the binary form (ParamDict::load_param_bin): mem must hold the end mark -233
+int ncnn_paramdict_probe_bin(const unsigned char* mem, int id, unsigned int* value_bits, unsigned int* array_bits, int cap)
+{
+    const unsigned char* cursor = mem;
+    DataReaderFromMemory dr(cursor);
+    ParamDict pd;
+    if (pd.load_param_bin(dr) != 0) return -1;
+    return paramdict_probe_slot(pd, id, value_bits, array_bits, cap);
+}
+
 int ncnn_paramdict_probe(const char* text, int id, unsigned int* value_bits, unsigned int* array_bits, int cap)
 {
     const unsigned char* cursor = (const unsigned char*)text;
     DataReaderFromMemory dr(cursor);
     ParamDict pd;
     if (pd.load_param(dr) != 0) return -1;
+    return paramdict_probe_slot(pd, id, value_bits, array_bits, cap);
+}
+
+static int paramdict_probe_slot(const ParamDict& pd, int id, unsigned int* value_bits, unsigned int* array_bits, int cap)
+{
     const int t = pd.type(id);
-    if (t == 2 || t == 3)
+    if (t == 1 || t == 2 || t == 3)
     {
         const int raw = pd.get(id, 0); // the slot's 32 bits, whichever way it was written
         memcpy(value_bits, &raw, 4);
     }
-    else if (t == 5 || t == 6)
+    else if (t == 4 || t == 5 || t == 6)
     {
         Mat v = pd.get(id, Mat());
         *value_bits = (unsigned)v.w;

@@ -266,4 +266,81 @@ int ParamDict::load_param(const DataReader& dr)
     return 0;
 }
 
+// The binary form of a layer's parameters (src/paramdict.cpp:491-637): little-endian 32-bit words, `id value` pairs up to
+// the end mark -233.  An id <= -23300 announces an array (id = -id - 23300; a length word, then that many 32-bit values),
+// an id <= -23400 a string (id = -id - 23400; a length word of at most 255, then the bytes padded to whole words).  The
+// file does not say whether a value is an int or a float: a scalar gets type 1 and an array type 4, and the getters hand
+// out the stored bits either way.
+int ParamDict::load_param_bin(const DataReader& dr)
+{
+    clear();
+    int id = 0;
+    if (dr.read(&id, 4) != 4)
+    {
+        NCNN_LOGE("ParamDict read id failed");
+        return -1;
+    }
+    while (id != -233)
+    {
+        const bool is_string = id <= -23400, is_array = id <= -23300;
+        if (is_string)
+            id = -id - 23400;
+        else if (is_array)
+            id = -id - 23300;
+        if (id < 0 || id >= NCNN_MAX_PARAM_COUNT)
+        {
+            NCNN_LOGE("id < NCNN_MAX_PARAM_COUNT failed (id=%d, NCNN_MAX_PARAM_COUNT=%d)", id, NCNN_MAX_PARAM_COUNT);
+            return -1;
+        }
+        Slot& slot = slots[id];
+        if (is_string || is_array)
+        {
+            int len = 0;
+            if (dr.read(&len, 4) != 4 || len < 0 || len > (is_string ? 255 : (1 << 24)))
+            {
+                NCNN_LOGE("ParamDict read %s length failed (id=%d)", is_string ? "string" : "array", id);
+                return -1;
+            }
+            if (is_string)
+            {
+                char text[260];
+                const size_t padded = ((size_t)len + 3) / 4 * 4;
+                if (dr.read(text, padded) != padded)
+                {
+                    NCNN_LOGE("ParamDict read string failed");
+                    return -1;
+                }
+                text[padded] = 0;
+                slot.s = text; // up to the first zero byte, as the reference assigns it
+                slot.type = 7;
+            }
+            else
+            {
+                slot.v.create(len);
+                if (len > 0 && (slot.v.empty() || dr.read(slot.v.data, (size_t)len * 4) != (size_t)len * 4))
+                {
+                    NCNN_LOGE("ParamDict read array element failed");
+                    return -1;
+                }
+                slot.type = 4;
+            }
+        }
+        else
+        {
+            if (dr.read(&slot.f, 4) != 4)
+            {
+                NCNN_LOGE("ParamDict read value failed");
+                return -1;
+            }
+            slot.type = 1;
+        }
+        if (dr.read(&id, 4) != 4)
+        {
+            NCNN_LOGE("ParamDict read EOP failed");
+            return -1;
+        }
+    }
+    return 0;
+}
+
 } // namespace ncnn

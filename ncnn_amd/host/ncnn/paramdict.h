@@ -39,6 +39,7 @@ public:
     // exposed for the net loader and for tests
     void clear();
     int load_param(const DataReader& dr);
+    int load_param_bin(const DataReader& dr);
 
 private:
     struct Slot

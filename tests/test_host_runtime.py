@@ -415,3 +415,25 @@ def test_paramdict_text_parser_on_the_reference_tests_own_vectors():
                 assert v == len(e["string"]) and bytes(arr[:v]).decode() == e["string"]
             checked += 1
     assert checked == 14
+    # the binary form (ParamDict::load_param_bin, src/paramdict.cpp:491-637): the byte arrays of test_paramdict_3, _4, _5
+    for vec in data["binary_vectors"]:
+        mem = bytes.fromhex(vec["hex"])
+        for e in vec["expect"]:
+            t, v, arr = host.paramdict_probe_bin(mem, e["id"])
+            assert t == e["type"], e
+            if "int" in e:
+                assert np.array([v], np.uint32).view(np.int32)[0] == e["int"]
+            elif "float" in e:
+                assert v == bits(float(np.float32(e["float"])))
+            elif "ints" in e:
+                assert v == len(e["ints"]) and list(np.array(arr[:v], np.uint32).view(np.int32)) == e["ints"]
+            elif "floats" in e:
+                assert v == len(e["floats"]) and arr[:v] == [bits(float(np.float32(f))) for f in e["floats"]]
+            else:
+                assert v == len(e["string"]) and bytes(arr[:v]).decode() == e["string"]
+            checked += 1
+    assert checked == 25
+    # damaged binary forms are answered with -1: no end mark, an id out of range, a negative array length, a string too long
+    import struct
+    for bad in (struct.pack("<ii", 0, 5), struct.pack("<iii", 40, 1, -233), struct.pack("<iii", -23301, -4, -233), struct.pack("<iii", -23400, 300, -233)):
+        assert host.paramdict_probe_bin(bad + b"\0" * 8, 0)[0] == -1
