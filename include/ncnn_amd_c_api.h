@@ -47,6 +47,32 @@ int ncnn_option_get_use_int8_inference(const ncnn_option_t opt);
  * ncnn_extractor_create. */
 void ncnn_option_set_use_hip_compute(ncnn_option_t opt, int enable);
 int ncnn_option_get_use_hip_compute(const ncnn_option_t opt);
+/* the switches of src/c_api.h:61-99 that ncnn::Option has here; none of them changes what the int8 layers compute */
+int ncnn_option_get_num_threads(const ncnn_option_t opt);
+int ncnn_option_get_use_vulkan_compute(const ncnn_option_t opt);
+int ncnn_option_get_use_local_pool_allocator(const ncnn_option_t opt);
+int ncnn_option_get_use_winograd_convolution(const ncnn_option_t opt);
+int ncnn_option_get_use_sgemm_convolution(const ncnn_option_t opt);
+int ncnn_option_get_use_packing_layout(const ncnn_option_t opt);
+int ncnn_option_get_use_fp16_packed(const ncnn_option_t opt);
+int ncnn_option_get_use_fp16_storage(const ncnn_option_t opt);
+int ncnn_option_get_use_fp16_arithmetic(const ncnn_option_t opt);
+int ncnn_option_get_use_int8_packed(const ncnn_option_t opt);
+int ncnn_option_get_use_int8_storage(const ncnn_option_t opt);
+int ncnn_option_get_use_int8_arithmetic(const ncnn_option_t opt);
+int ncnn_option_get_use_bf16_storage(const ncnn_option_t opt);
+void ncnn_option_set_use_vulkan_compute(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_local_pool_allocator(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_winograd_convolution(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_sgemm_convolution(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_packing_layout(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_fp16_packed(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_fp16_storage(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_fp16_arithmetic(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_int8_packed(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_int8_storage(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_int8_arithmetic(ncnn_option_t opt, int enable);
+void ncnn_option_set_use_bf16_storage(ncnn_option_t opt, int enable);
 
 /* src/c_api.h:134-165; data is caller-owned memory laid out as ncnn::Mat lays it out */
 ncnn_mat_t ncnn_mat_create_external_1d_elem(int w, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
@@ -60,6 +86,30 @@ ncnn_mat_t ncnn_mat_create_3d_elem(int w, int h, int c, size_t elemsize, int ele
 /* owning, batched 3-D blobs (src/c_api.h:117,131: fp32, or any element size); fill them through ncnn_mat_get_batch_data */
 ncnn_mat_t ncnn_mat_create_3d_batch(int w, int h, int c, int n, ncnn_allocator_t allocator);
 ncnn_mat_t ncnn_mat_create_3d_elem_batch(int w, int h, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator);
+/* the remaining constructors of src/c_api.h:110-137 (fp32 unless an element size is given; "external" wraps caller memory) */
+ncnn_mat_t ncnn_mat_create_1d(int w, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_2d(int w, int h, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_3d(int w, int h, int c, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_4d(int w, int h, int d, int c, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_1d_batch(int w, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_2d_batch(int w, int h, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_4d_batch(int w, int h, int d, int c, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_1d(int w, void* data, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_2d(int w, int h, void* data, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_3d(int w, int h, int c, void* data, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_4d(int w, int h, int d, int c, void* data, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_4d_elem(int w, int h, int d, int c, size_t elemsize, int elempack, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_1d_elem_batch(int w, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_2d_elem_batch(int w, int h, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_4d_elem_batch(int w, int h, int d, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_create_external_4d_elem(int w, int h, int d, int c, void* data, size_t elemsize, int elempack, ncnn_allocator_t allocator);
+/* src/c_api.h:140-146,165: fill, deep copy (batch included), reshape (a new handle; shares the data where the layout allows) */
+void ncnn_mat_fill_float(ncnn_mat_t mat, float v);
+ncnn_mat_t ncnn_mat_clone(const ncnn_mat_t mat, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_reshape_1d(const ncnn_mat_t mat, int w, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_reshape_2d(const ncnn_mat_t mat, int w, int h, ncnn_allocator_t allocator);
+ncnn_mat_t ncnn_mat_reshape_3d(const ncnn_mat_t mat, int w, int h, int c, ncnn_allocator_t allocator);
+void* ncnn_mat_get_channel_data(const ncnn_mat_t mat, int c);
 void ncnn_mat_destroy(ncnn_mat_t mat);
 int ncnn_mat_get_dims(const ncnn_mat_t mat);
 int ncnn_mat_get_w(const ncnn_mat_t mat);
@@ -83,6 +133,10 @@ int ncnn_net_load_param(ncnn_net_t net, const char* path);
 int ncnn_net_load_model(ncnn_net_t net, const char* path);
 int ncnn_net_load_param_memory(ncnn_net_t net, const char* mem);
 size_t ncnn_net_load_model_memory(ncnn_net_t net, const unsigned char* mem);
+/* src/c_api.h:382,390-391 */
+void ncnn_net_clear(ncnn_net_t net);
+int ncnn_net_get_input_index(const ncnn_net_t net, int i);
+int ncnn_net_get_output_index(const ncnn_net_t net, int i);
 int ncnn_net_get_input_count(const ncnn_net_t net);
 int ncnn_net_get_output_count(const ncnn_net_t net);
 const char* ncnn_net_get_input_name(const ncnn_net_t net, int i);
@@ -94,6 +148,9 @@ void ncnn_extractor_destroy(ncnn_extractor_t ex);
 void ncnn_extractor_set_option(ncnn_extractor_t ex, const ncnn_option_t opt);
 int ncnn_extractor_input(ncnn_extractor_t ex, const char* name, const ncnn_mat_t mat);
 int ncnn_extractor_extract(ncnn_extractor_t ex, const char* name, ncnn_mat_t* mat);
+/* by blob index (src/c_api.h:405-406); the indices of a net's inputs and outputs come from ncnn_net_get_input_index / _output_index */
+int ncnn_extractor_input_index(ncnn_extractor_t ex, int index, const ncnn_mat_t mat);
+int ncnn_extractor_extract_index(ncnn_extractor_t ex, int index, ncnn_mat_t* mat);
 
 /* paramdict api, src/c_api.h:200-213: what a layer written in C reads its parameters from */
 typedef struct __ncnn_paramdict_t* ncnn_paramdict_t;

@@ -56,6 +56,10 @@ LAYER_FLAGS = ("one_blob_only", "support_inplace", "support_vulkan", "support_pa
                "support_vulkan_packing", "support_any_packing", "support_vulkan_any_packing")
 
 
+OPTION_SWITCHES = ("use_vulkan_compute", "use_local_pool_allocator", "use_winograd_convolution", "use_sgemm_convolution", "use_packing_layout", "use_fp16_packed",
+                   "use_fp16_storage", "use_fp16_arithmetic", "use_int8_packed", "use_int8_storage", "use_int8_arithmetic", "use_bf16_storage")
+
+
 def lib():
     global _lib
     if _lib is None:
@@ -72,12 +76,25 @@ def lib():
             "ncnn_option_create": (vp, []), "ncnn_option_destroy": (None, [vp]), "ncnn_option_set_num_threads": (None, [vp, ci]),
             "ncnn_option_set_lightmode": (None, [vp, ci]), "ncnn_option_set_use_int8_inference": (None, [vp, ci]),
             "ncnn_option_get_use_int8_inference": (ci, [vp]),
+            **{"ncnn_option_get_" + f: (ci, [vp]) for f in OPTION_SWITCHES}, **{"ncnn_option_set_" + f: (None, [vp, ci]) for f in OPTION_SWITCHES},
             "ncnn_option_set_use_hip_compute": (None, [vp, ci]), "ncnn_option_get_use_hip_compute": (ci, [vp]),
             "ncnn_mat_create_external_1d_elem": (vp, [ci, vp, cs, ci, vp]), "ncnn_mat_create_external_2d_elem": (vp, [ci, ci, vp, cs, ci, vp]),
             "ncnn_mat_create_external_3d_elem": (vp, [ci, ci, ci, vp, cs, ci, vp]), "ncnn_mat_create_3d_batch": (vp, [ci, ci, ci, ci, vp]),
             "ncnn_mat_create_3d_elem_batch": (vp, [ci, ci, ci, cs, ci, ci, vp]),
             "ncnn_mat_create": (vp, []), "ncnn_mat_create_1d_elem": (vp, [ci, cs, ci, vp]), "ncnn_mat_create_2d_elem": (vp, [ci, ci, cs, ci, vp]),
             "ncnn_mat_create_3d_elem": (vp, [ci, ci, ci, cs, ci, vp]),
+            "ncnn_mat_create_1d": (vp, [ci, vp]), "ncnn_mat_create_2d": (vp, [ci, ci, vp]), "ncnn_mat_create_3d": (vp, [ci, ci, ci, vp]),
+            "ncnn_mat_create_4d": (vp, [ci, ci, ci, ci, vp]), "ncnn_mat_create_1d_batch": (vp, [ci, ci, vp]), "ncnn_mat_create_2d_batch": (vp, [ci, ci, ci, vp]),
+            "ncnn_mat_create_4d_batch": (vp, [ci, ci, ci, ci, ci, vp]), "ncnn_mat_create_external_1d": (vp, [ci, vp, vp]),
+            "ncnn_mat_create_external_2d": (vp, [ci, ci, vp, vp]), "ncnn_mat_create_external_3d": (vp, [ci, ci, ci, vp, vp]),
+            "ncnn_mat_create_external_4d": (vp, [ci, ci, ci, ci, vp, vp]), "ncnn_mat_create_4d_elem": (vp, [ci, ci, ci, ci, cs, ci, vp]),
+            "ncnn_mat_create_1d_elem_batch": (vp, [ci, cs, ci, ci, vp]), "ncnn_mat_create_2d_elem_batch": (vp, [ci, ci, cs, ci, ci, vp]),
+            "ncnn_mat_create_4d_elem_batch": (vp, [ci, ci, ci, ci, cs, ci, ci, vp]), "ncnn_mat_create_external_4d_elem": (vp, [ci, ci, ci, ci, vp, cs, ci, vp]),
+            "ncnn_mat_fill_float": (None, [vp, C.c_float]), "ncnn_mat_clone": (vp, [vp, vp]), "ncnn_mat_reshape_1d": (vp, [vp, ci, vp]),
+            "ncnn_mat_reshape_2d": (vp, [vp, ci, ci, vp]), "ncnn_mat_reshape_3d": (vp, [vp, ci, ci, ci, vp]), "ncnn_mat_get_channel_data": (vp, [vp, ci]),
+            "ncnn_option_get_num_threads": (ci, [vp]), "ncnn_net_clear": (None, [vp]), "ncnn_net_get_input_index": (ci, [vp, ci]),
+            "ncnn_net_get_output_index": (ci, [vp, ci]), "ncnn_extractor_input_index": (ci, [vp, ci, vp]),
+            "ncnn_extractor_extract_index": (ci, [vp, ci, C.POINTER(vp)]),
             "ncnn_mat_destroy": (None, [vp]), "ncnn_mat_get_dims": (ci, [vp]), "ncnn_mat_get_w": (ci, [vp]), "ncnn_mat_get_h": (ci, [vp]),
             "ncnn_mat_get_d": (ci, [vp]), "ncnn_mat_get_c": (ci, [vp]), "ncnn_mat_get_n": (ci, [vp]), "ncnn_mat_get_elemsize": (cs, [vp]),
             "ncnn_mat_get_elempack": (ci, [vp]), "ncnn_mat_get_cstep": (cs, [vp]), "ncnn_mat_get_nstep": (cs, [vp]),

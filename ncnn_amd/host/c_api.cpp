@@ -171,6 +171,163 @@ ncnn_mat_t ncnn_mat_create_external_3d_elem(int w, int h, int c, void* data, siz
     m->elempack = elempack;
     return (ncnn_mat_t)m;
 }
+static ncnn_mat_t made(int dims, int w, int h, int d, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator)
+{
+    Mat* m = new Mat;
+    if (dims == 1)
+        m->create(w, elemsize, elempack, n, A(allocator));
+    else if (dims == 2)
+        m->create(w, h, elemsize, elempack, n, A(allocator));
+    else if (dims == 3)
+        m->create(w, h, c, elemsize, elempack, n, A(allocator));
+    else
+        m->create(w, h, d, c, elemsize, elempack, n, A(allocator));
+    return (ncnn_mat_t)m;
+}
+ncnn_mat_t ncnn_mat_create_1d(int w, ncnn_allocator_t allocator)
+{
+    return made(1, w, 1, 1, 1, 4u, 1, 1, allocator);
+}
+ncnn_mat_t ncnn_mat_create_2d(int w, int h, ncnn_allocator_t allocator)
+{
+    return made(2, w, h, 1, 1, 4u, 1, 1, allocator);
+}
+ncnn_mat_t ncnn_mat_create_3d(int w, int h, int c, ncnn_allocator_t allocator)
+{
+    return made(3, w, h, 1, c, 4u, 1, 1, allocator);
+}
+ncnn_mat_t ncnn_mat_create_4d(int w, int h, int d, int c, ncnn_allocator_t allocator)
+{
+    return made(4, w, h, d, c, 4u, 1, 1, allocator);
+}
+ncnn_mat_t ncnn_mat_create_1d_batch(int w, int n, ncnn_allocator_t allocator)
+{
+    return made(1, w, 1, 1, 1, 4u, 1, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_2d_batch(int w, int h, int n, ncnn_allocator_t allocator)
+{
+    return made(2, w, h, 1, 1, 4u, 1, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_4d_batch(int w, int h, int d, int c, int n, ncnn_allocator_t allocator)
+{
+    return made(4, w, h, d, c, 4u, 1, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_4d_elem(int w, int h, int d, int c, size_t elemsize, int elempack, ncnn_allocator_t allocator)
+{
+    return made(4, w, h, d, c, elemsize, elempack, 1, allocator);
+}
+ncnn_mat_t ncnn_mat_create_1d_elem_batch(int w, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator)
+{
+    return made(1, w, 1, 1, 1, elemsize, elempack, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_2d_elem_batch(int w, int h, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator)
+{
+    return made(2, w, h, 1, 1, elemsize, elempack, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_4d_elem_batch(int w, int h, int d, int c, size_t elemsize, int elempack, int n, ncnn_allocator_t allocator)
+{
+    return made(4, w, h, d, c, elemsize, elempack, n, allocator);
+}
+ncnn_mat_t ncnn_mat_create_external_1d(int w, void* data, ncnn_allocator_t)
+{
+    return (ncnn_mat_t)(new Mat(w, data, (size_t)4u));
+}
+ncnn_mat_t ncnn_mat_create_external_2d(int w, int h, void* data, ncnn_allocator_t)
+{
+    return (ncnn_mat_t)(new Mat(w, h, data, (size_t)4u));
+}
+ncnn_mat_t ncnn_mat_create_external_3d(int w, int h, int c, void* data, ncnn_allocator_t)
+{
+    return (ncnn_mat_t)(new Mat(w, h, c, data, (size_t)4u));
+}
+ncnn_mat_t ncnn_mat_create_external_4d(int w, int h, int d, int c, void* data, ncnn_allocator_t)
+{
+    return (ncnn_mat_t)(new Mat(w, h, d, c, data, (size_t)4u));
+}
+ncnn_mat_t ncnn_mat_create_external_4d_elem(int w, int h, int d, int c, void* data, size_t elemsize, int elempack, ncnn_allocator_t)
+{
+    Mat* m = new Mat(w, h, d, c, data, elemsize);
+    m->elempack = elempack;
+    return (ncnn_mat_t)m;
+}
+void ncnn_mat_fill_float(ncnn_mat_t mat, float v)
+{
+    M(mat)->fill(v);
+}
+ncnn_mat_t ncnn_mat_clone(const ncnn_mat_t mat, ncnn_allocator_t allocator)
+{
+    return (ncnn_mat_t)(new Mat(M(mat)->clone(A(allocator))));
+}
+ncnn_mat_t ncnn_mat_reshape_1d(const ncnn_mat_t mat, int w, ncnn_allocator_t allocator)
+{
+    return (ncnn_mat_t)(new Mat(M(mat)->reshape(w, A(allocator))));
+}
+ncnn_mat_t ncnn_mat_reshape_2d(const ncnn_mat_t mat, int w, int h, ncnn_allocator_t allocator)
+{
+    return (ncnn_mat_t)(new Mat(M(mat)->reshape(w, h, A(allocator))));
+}
+ncnn_mat_t ncnn_mat_reshape_3d(const ncnn_mat_t mat, int w, int h, int c, ncnn_allocator_t allocator)
+{
+    return (ncnn_mat_t)(new Mat(M(mat)->reshape(w, h, c, A(allocator))));
+}
+void* ncnn_mat_get_channel_data(const ncnn_mat_t mat, int c)
+{
+    return M(mat)->channel(c).data;
+}
+
+#define OPTION_SWITCH(field)                                              \
+    int ncnn_option_get_##field(const ncnn_option_t opt)                  \
+    {                                                                     \
+        return O(opt)->field;                                             \
+    }                                                                     \
+    void ncnn_option_set_##field(ncnn_option_t opt, int enable)           \
+    {                                                                     \
+        O(opt)->field = enable != 0;                                      \
+    }
+OPTION_SWITCH(use_vulkan_compute)
+OPTION_SWITCH(use_local_pool_allocator)
+OPTION_SWITCH(use_winograd_convolution)
+OPTION_SWITCH(use_sgemm_convolution)
+OPTION_SWITCH(use_packing_layout)
+OPTION_SWITCH(use_fp16_packed)
+OPTION_SWITCH(use_fp16_storage)
+OPTION_SWITCH(use_fp16_arithmetic)
+OPTION_SWITCH(use_int8_packed)
+OPTION_SWITCH(use_int8_storage)
+OPTION_SWITCH(use_int8_arithmetic)
+OPTION_SWITCH(use_bf16_storage)
+#undef OPTION_SWITCH
+int ncnn_option_get_num_threads(const ncnn_option_t opt)
+{
+    return O(opt)->num_threads;
+}
+
+void ncnn_net_clear(ncnn_net_t net)
+{
+    N(net)->clear();
+}
+int ncnn_net_get_input_index(const ncnn_net_t net, int i)
+{
+    const std::vector<int>& v = N(net)->input_indexes();
+    return (i >= 0 && (size_t)i < v.size()) ? v[(size_t)i] : -1;
+}
+int ncnn_net_get_output_index(const ncnn_net_t net, int i)
+{
+    const std::vector<int>& v = N(net)->output_indexes();
+    return (i >= 0 && (size_t)i < v.size()) ? v[(size_t)i] : -1;
+}
+int ncnn_extractor_input_index(ncnn_extractor_t ex, int index, const ncnn_mat_t mat)
+{
+    return E(ex)->input(index, *M(mat));
+}
+int ncnn_extractor_extract_index(ncnn_extractor_t ex, int index, ncnn_mat_t* mat)
+{
+    Mat out;
+    int ret = E(ex)->extract(index, out);
+    *mat = (ncnn_mat_t) new Mat(out);
+    return ret;
+}
+
 ncnn_mat_t ncnn_mat_create(void)
 {
     return (ncnn_mat_t)(new Mat);

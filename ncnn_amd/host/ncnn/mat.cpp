@@ -269,9 +269,42 @@ static Mat densify(const Mat& m, Allocator* allocator)
     return flat;
 }
 
+// A batched blob under a new shape (src/mat.cpp:113-250 hands these to its reshape_batch): every sample is reshaped by
+// itself and the samples stay nstep apart.  Dense planes on both sides share the storage; otherwise each sample is copied.
+Mat Mat::reshape_samples(int _dims, int _w, int _h, int _c, Allocator* _allocator) const
+{
+    const size_t plane = _dims == 3 ? (size_t)_w * _h : _dims == 2 ? (size_t)_w * _h : (size_t)_w;
+    const size_t padded = _dims == 3 ? alignSize(plane * elemsize, 16) / elemsize : plane;
+    if (planes_are_dense(*this) && padded == plane)
+    {
+        Mat m = *this; // n and nstep stay as they are
+        m.dims = _dims;
+        m.w = _w;
+        m.h = _dims >= 2 ? _h : 1;
+        m.d = 1;
+        m.c = _dims == 3 ? _c : 1;
+        m.cstep = plane;
+        return m;
+    }
+    Mat out;
+    out.create_any(_dims, _w, _dims >= 2 ? _h : 1, 1, _dims == 3 ? _c : 1, elemsize, elempack, n, _allocator);
+    if (out.empty()) return out;
+    for (int b = 0; b < n; b++)
+    {
+        const Mat sample = batch(b);
+        const Mat r = _dims == 3 ? sample.reshape(_w, _h, _c, _allocator) : _dims == 2 ? sample.reshape(_w, _h, _allocator) : sample.reshape(_w, _allocator);
+        if (r.empty()) return Mat();
+        unsigned char* to = (unsigned char*)out.data + out.nstep * b * elemsize;
+        for (int q = 0; q < out.c; q++)
+            memcpy(to + out.cstep * q * elemsize, (const unsigned char*)r.data + r.cstep * q * elemsize, plane * elemsize);
+    }
+    return out;
+}
+
 Mat Mat::reshape(int _w, Allocator* _allocator) const
 {
     if ((size_t)w * h * d * c != (size_t)_w) return Mat();
+    if (n > 1) return reshape_samples(1, _w, 1, 1, _allocator);
     if (!planes_are_dense(*this)) return densify(*this, _allocator);
     Mat m = *this;
     m.dims = 1;
@@ -285,6 +318,7 @@ Mat Mat::reshape(int _w, Allocator* _allocator) const
 Mat Mat::reshape(int _w, int _h, Allocator* _allocator) const
 {
     if ((size_t)w * h * d * c != (size_t)_w * _h) return Mat();
+    if (n > 1) return reshape_samples(2, _w, _h, 1, _allocator);
     if (!planes_are_dense(*this))
     {
         Mat flat = densify(*this, _allocator);
@@ -304,6 +338,7 @@ Mat Mat::reshape(int _w, int _h, Allocator* _allocator) const
 Mat Mat::reshape(int _w, int _h, int _c, Allocator* _allocator) const
 {
     if ((size_t)w * h * d * c != (size_t)_w * _h * _c) return Mat();
+    if (n > 1) return reshape_samples(3, _w, _h, _c, _allocator);
     const size_t plane = (size_t)_w * _h;
     const size_t padded = alignSize(plane * elemsize, 16) / elemsize;
     const bool src_dense = planes_are_dense(*this);
@@ -397,6 +432,8 @@ Mat Mat::batch(int b)
 {
     Mat m;
     m.set_shape(dims, w, h, d, c, elemsize, elempack, 1);
+    m.cstep = cstep; // a reshaped blob may hold dense planes where a created one pads them
+    m.nstep = cstep * c;
     m.data = (unsigned char*)data + nstep * b * elemsize;
     m.refcount = 0;
     m.allocator = allocator;

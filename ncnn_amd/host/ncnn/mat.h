@@ -153,6 +153,7 @@ private:
     void allocate(Allocator* allocator);
     bool same_as(int dims, int w, int h, int d, int c, size_t elemsize, int elempack, int n, Allocator* allocator) const;
     void create_any(int dims, int w, int h, int d, int c, size_t elemsize, int elempack, int n, Allocator* allocator);
+    Mat reshape_samples(int dims, int w, int h, int c, Allocator* allocator) const;
     void view(int dims, int w, int h, int d, int c, void* data, size_t elemsize, Allocator* allocator);
 };
 

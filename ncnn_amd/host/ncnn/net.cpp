@@ -998,8 +998,11 @@ int Net::load_param(const DataReader& dr)
 
         if (pd.load_param(dr) != 0)
         {
+            // a parameter line that cannot be read ends the load, as in the reference (src/net.cpp:1477-1484): going on would leave
+            // a layer whose load_param never ran
             NCNN_LOGE("ParamDict load_param %d %s failed", li, name);
-            continue;
+            clear();
+            return -1;
         }
 
         // id 30: shape hints, [dims, w, h, c] per top blob;  id 31: feature mask

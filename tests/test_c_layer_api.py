@@ -146,3 +146,87 @@ def test_hip_layers_registered_through_function_pointers(resident):
         ex.input("data", x)
         want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
         assert np.array_equal(ex.extract(name), want), name
+
+
+def test_mat_constructors_clone_and_reshape_as_the_references_c_api_test_uses_them():
+    """tests/test_c_api.cpp:407-480 (test_c_api_batch) step by step: a batch of 3-D blobs written through
+    ncnn_mat_get_batch_data, its deep copy, its reshape to vectors (the batch kept), a 2-D batch of 2-byte elements; then the
+    remaining constructors of src/c_api.h:110-137, ncnn_mat_fill_float and ncnn_mat_get_channel_data."""
+    import ctypes as C
+    L = host.lib()
+    W, H, Cc, B = 4, 3, 2, 3
+    a = L.ncnn_mat_create_3d_batch(W, H, Cc, B, None)
+    assert (L.ncnn_mat_get_dims(a), L.ncnn_mat_get_w(a), L.ncnn_mat_get_h(a), L.ncnn_mat_get_c(a), L.ncnn_mat_get_n(a)) == (3, W, H, Cc, B)
+    assert L.ncnn_mat_get_nstep(a) != 0
+
+    def floats(ptr, count):
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_float)), (count,))
+
+    cstep = L.ncnn_mat_get_cstep(a)
+    for bi in range(B):
+        data = floats(L.ncnn_mat_get_batch_data(a, bi), cstep * Cc)
+        for q in range(Cc):
+            data[q * cstep: q * cstep + W * H] = [bi * 100 + q * 10 + i for i in range(W * H)]
+    b = L.ncnn_mat_clone(a, None)
+    assert L.ncnn_mat_get_n(b) == B and L.ncnn_mat_get_data(b) != L.ncnn_mat_get_data(a)
+    c = L.ncnn_mat_reshape_1d(a, W * H * Cc, None)
+    assert (L.ncnn_mat_get_dims(c), L.ncnn_mat_get_w(c), L.ncnn_mat_get_n(c)) == (1, W * H * Cc, B)
+    bstep = L.ncnn_mat_get_cstep(b)
+    for bi in range(B):
+        bdata = floats(L.ncnn_mat_get_batch_data(b, bi), bstep * Cc)
+        cdata = floats(L.ncnn_mat_get_batch_data(c, bi), W * H * Cc)
+        for q in range(Cc):
+            want = np.array([bi * 100 + q * 10 + i for i in range(W * H)], np.float32)
+            assert np.array_equal(bdata[q * bstep: q * bstep + W * H], want) and np.array_equal(cdata[q * W * H: (q + 1) * W * H], want)
+    d = L.ncnn_mat_create_2d_elem_batch(5, 6, 2, 1, 2, None)
+    assert (L.ncnn_mat_get_dims(d), L.ncnn_mat_get_w(d), L.ncnn_mat_get_h(d), L.ncnn_mat_get_n(d), L.ncnn_mat_get_elemsize(d)) == (2, 5, 6, 2, 2)
+    for m in (a, b, c, d):
+        L.ncnn_mat_destroy(m)
+
+    shapes = {L.ncnn_mat_create_1d(7, None): (1, 7, 1, 1, 1, 1), L.ncnn_mat_create_2d(7, 5, None): (2, 7, 5, 1, 1, 1), L.ncnn_mat_create_3d(7, 5, 3, None): (3, 7, 5, 1, 3, 1),
+              L.ncnn_mat_create_4d(7, 5, 2, 3, None): (4, 7, 5, 2, 3, 1), L.ncnn_mat_create_1d_batch(7, 4, None): (1, 7, 1, 1, 1, 4),
+              L.ncnn_mat_create_2d_batch(7, 5, 4, None): (2, 7, 5, 1, 1, 4), L.ncnn_mat_create_4d_batch(7, 5, 2, 3, 4, None): (4, 7, 5, 2, 3, 4),
+              L.ncnn_mat_create_4d_elem(7, 5, 2, 3, 1, 1, None): (4, 7, 5, 2, 3, 1), L.ncnn_mat_create_1d_elem_batch(7, 1, 1, 2, None): (1, 7, 1, 1, 1, 2),
+              L.ncnn_mat_create_4d_elem_batch(7, 5, 2, 3, 4, 1, 2, None): (4, 7, 5, 2, 3, 2)}
+    for m, want in shapes.items():
+        assert (L.ncnn_mat_get_dims(m), L.ncnn_mat_get_w(m), L.ncnn_mat_get_h(m), L.ncnn_mat_get_d(m), L.ncnn_mat_get_c(m), L.ncnn_mat_get_n(m)) == want
+        L.ncnn_mat_destroy(m)
+    backing = np.arange(7 * 5 * 3, dtype=np.float32)
+    for m, dims in ((L.ncnn_mat_create_external_1d(105, backing.ctypes.data, None), 1), (L.ncnn_mat_create_external_2d(21, 5, backing.ctypes.data, None), 2),
+                    (L.ncnn_mat_create_external_4d(7, 5, 1, 3, backing.ctypes.data, None), 4), (L.ncnn_mat_create_external_4d_elem(7, 5, 1, 3, backing.ctypes.data, 4, 1, None), 4)):
+        assert L.ncnn_mat_get_dims(m) == dims and L.ncnn_mat_get_data(m) == backing.ctypes.data
+        L.ncnn_mat_destroy(m)
+    m = L.ncnn_mat_create_3d(4, 3, 2, None)
+    L.ncnn_mat_fill_float(m, 2.5)
+    step = L.ncnn_mat_get_cstep(m)
+    assert L.ncnn_mat_get_channel_data(m, 1) == L.ncnn_mat_get_data(m) + step * 4
+    assert np.all(floats(L.ncnn_mat_get_channel_data(m, 1), 12) == 2.5)
+    r = L.ncnn_mat_reshape_2d(m, 6, 4, None)
+    assert (L.ncnn_mat_get_dims(r), L.ncnn_mat_get_w(r), L.ncnn_mat_get_h(r)) == (2, 6, 4) and np.all(floats(L.ncnn_mat_get_data(r), 24) == 2.5)
+    r3 = L.ncnn_mat_reshape_3d(r, 2, 3, 4, None)
+    assert (L.ncnn_mat_get_dims(r3), L.ncnn_mat_get_c(r3)) == (3, 4)
+    for x in (m, r, r3):
+        L.ncnn_mat_destroy(x)
+
+
+def test_option_switches_net_indices_and_clear():
+    """src/c_api.h:61-99 (the Option switches this runtime holds: set, read back), :382-391 (ncnn_net_clear, the blob indices of
+    a net's inputs and outputs)."""
+    L = host.lib()
+    opt = L.ncnn_option_create()
+    for f in host.OPTION_SWITCHES:
+        for v in (1, 0, 1):
+            getattr(L, "ncnn_option_set_" + f)(opt, v)
+            assert getattr(L, "ncnn_option_get_" + f)(opt) == v, f
+    L.ncnn_option_set_num_threads(opt, 3)
+    assert L.ncnn_option_get_num_threads(opt) == 3
+    L.ncnn_option_destroy(opt)
+    net = host.Net()
+    text = "7767517\n3 3\nInput in0 0 1 data 0=4 1=4 2=2\nReLU r 1 1 data mid\nReLU r2 1 1 mid out\n"
+    assert net.load_param_mem(text) == 0
+    blobs = net.blobs()
+    assert L.ncnn_net_get_input_index(net.h_, 0) == list(blobs).index("data") and L.ncnn_net_get_output_index(net.h_, 0) == list(blobs).index("out")
+    assert L.ncnn_net_get_input_index(net.h_, 5) == -1
+    L.ncnn_net_clear(net.h_)
+    assert L.ncnn_net_get_layer_count(net.h_) == 0 and L.ncnn_net_get_input_count(net.h_) == 0
+    assert net.load_param_mem(text) == 0 and L.ncnn_net_get_layer_count(net.h_) == 3  # a cleared net loads again
