@@ -9,12 +9,17 @@
 #define NCNN_AMD_C_API_H
 
 #include <stddef.h>
+#include <stdio.h>
 
 #ifdef __cplusplus
 extern "C" {
 #endif
 
 #pragma GCC visibility push(default)
+
+/* src/c_api.h:18-19.  ncnn's version is 1.0.<date of the build>; this library gives the date its interface was taken from. */
+const char* ncnn_version(void);
+int ncnn_version_number(void);
 
 /* allocator api, src/c_api.h:21-34: a host allocator as a table of function pointers (the C++ object calls through the table,
  * so an entry may be replaced); NULL wherever an allocator is asked for means the library's own */
@@ -132,6 +137,11 @@ void ncnn_net_set_option(ncnn_net_t net, ncnn_option_t opt);
 int ncnn_net_load_param(ncnn_net_t net, const char* path);
 int ncnn_net_load_model(ncnn_net_t net, const char* path);
 int ncnn_net_load_param_memory(ncnn_net_t net, const char* mem);
+/* src/c_api.h:357,373: the binary form of the .param text that tools/ncnn2mem.cpp writes (layers by the reference's type
+ * numbers, blobs by number, no names: feed and extract with ncnn_extractor_input_index / _extract_index).  The memory form
+ * returns the bytes consumed, 0 when the load failed. */
+int ncnn_net_load_param_bin(ncnn_net_t net, const char* path);
+size_t ncnn_net_load_param_bin_memory(ncnn_net_t net, const unsigned char* mem);
 size_t ncnn_net_load_model_memory(ncnn_net_t net, const unsigned char* mem);
 /* src/c_api.h:382,390-391 */
 void ncnn_net_clear(ncnn_net_t net);
@@ -175,6 +185,26 @@ struct __ncnn_modelbin_t
 };
 ncnn_modelbin_t ncnn_modelbin_create_from_mat_array(const ncnn_mat_t* weights, int n);
 void ncnn_modelbin_destroy(ncnn_modelbin_t mb);
+
+/* datareader api, src/c_api.h:218-235: where .param text and .bin bytes come from, as a table a C program may fill in with
+ * functions of its own (pthis is then the program's to use).  ncnn_datareader_create gives a table that reads nothing. */
+typedef struct __ncnn_datareader_t* ncnn_datareader_t;
+struct __ncnn_datareader_t
+{
+    void* pthis;
+    int (*scan)(ncnn_datareader_t dr, const char* format, void* p);
+    size_t (*read)(ncnn_datareader_t dr, void* buf, size_t size);
+};
+ncnn_datareader_t ncnn_datareader_create(void);
+ncnn_datareader_t ncnn_datareader_create_from_stdio(FILE* fp);
+ncnn_datareader_t ncnn_datareader_create_from_memory(const unsigned char** mem); /* *mem is advanced as bytes are read */
+void ncnn_datareader_destroy(ncnn_datareader_t dr);
+/* src/c_api.h:248 */
+ncnn_modelbin_t ncnn_modelbin_create_from_datareader(const ncnn_datareader_t dr);
+/* src/c_api.h:377-380 */
+int ncnn_net_load_param_datareader(ncnn_net_t net, const ncnn_datareader_t dr);
+int ncnn_net_load_param_bin_datareader(ncnn_net_t net, const ncnn_datareader_t dr);
+int ncnn_net_load_model_datareader(ncnn_net_t net, const ncnn_datareader_t dr);
 
 /* layer api, src/c_api.h:254-320: a layer as a table of function pointers.  ncnn_layer_create gives a layer whose table
  * holds the base class's behaviour, for a C program to overwrite entry by entry; ncnn_layer_create_by_type / _by_typeindex

@@ -101,6 +101,12 @@ def lib():
             "ncnn_mat_get_data": (vp, [vp]), "ncnn_mat_get_batch_data": (vp, [vp, ci]),
             "ncnn_net_create": (vp, []), "ncnn_net_destroy": (None, [vp]), "ncnn_net_get_option": (vp, [vp]), "ncnn_net_set_option": (None, [vp, vp]),
             "ncnn_net_load_param": (ci, [vp, C.c_char_p]), "ncnn_net_load_model": (ci, [vp, C.c_char_p]),
+            "ncnn_net_load_param_bin": (ci, [vp, C.c_char_p]), "ncnn_net_load_param_bin_memory": (cs, [vp, C.c_char_p]),
+            "ncnn_version": (C.c_char_p, []), "ncnn_version_number": (ci, []),
+            "ncnn_datareader_create": (vp, []), "ncnn_datareader_create_from_memory": (vp, [C.POINTER(C.c_char_p)]),
+            "ncnn_datareader_create_from_stdio": (vp, [vp]), "ncnn_datareader_destroy": (None, [vp]),
+            "ncnn_modelbin_create_from_datareader": (vp, [vp]), "ncnn_net_load_param_datareader": (ci, [vp, vp]),
+            "ncnn_net_load_param_bin_datareader": (ci, [vp, vp]), "ncnn_net_load_model_datareader": (ci, [vp, vp]),
             "ncnn_net_load_param_memory": (ci, [vp, C.c_char_p]), "ncnn_net_load_model_memory": (cs, [vp, C.c_char_p]),
             "ncnn_net_get_input_count": (ci, [vp]), "ncnn_net_get_output_count": (ci, [vp]),
             "ncnn_net_get_input_name": (C.c_char_p, [vp, ci]), "ncnn_net_get_output_name": (C.c_char_p, [vp, ci]),
@@ -401,6 +407,13 @@ class Net:
     def load_param_mem(self, text):
         return lib().ncnn_net_load_param_memory(self.h_, text.encode())
 
+    def load_param_bin(self, path):
+        return lib().ncnn_net_load_param_bin(self.h_, path.encode())
+
+    def load_param_bin_mem(self, data):
+        """The binary .param form: 0 when all of `data` was read as a net, -1 otherwise."""
+        return 0 if lib().ncnn_net_load_param_bin_memory(self.h_, data) == len(data) else -1
+
     def load_model(self, path):
         return lib().ncnn_net_load_model(self.h_, path.encode())
 
@@ -457,6 +470,8 @@ class Extractor:
     def input(self, name, array):
         m = array if isinstance(array, Mat) else Mat.from_numpy(array)
         self._inputs.append(m)
+        if isinstance(name, int):  # a blob by number, the only way into a net loaded from the binary .param form in ncnn
+            return lib().ncnn_extractor_input_index(self.h_, name, m.h_)
         return lib().ncnn_extractor_input(self.h_, name.encode(), m.h_)
 
     def input_resident(self, name, hipmat):
@@ -492,7 +507,10 @@ class Extractor:
 
     def extract(self, name):
         out = C.c_void_p()
-        ret = lib().ncnn_extractor_extract(self.h_, name.encode(), C.byref(out))
+        if isinstance(name, int):
+            ret = lib().ncnn_extractor_extract_index(self.h_, name, C.byref(out))
+        else:
+            ret = lib().ncnn_extractor_extract(self.h_, name.encode(), C.byref(out))
         m = Mat(out.value)
         if ret != 0:
             raise RuntimeError("extract(%s) returned %d" % (name, ret))

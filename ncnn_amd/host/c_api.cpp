@@ -444,6 +444,22 @@ int ncnn_net_load_param_memory(ncnn_net_t net, const char* mem)
 {
     return N(net)->load_param_mem(mem);
 }
+const char* ncnn_version(void)
+{
+    return "1.0.20251101";
+}
+int ncnn_version_number(void)
+{
+    return 20251101;
+}
+int ncnn_net_load_param_bin(ncnn_net_t net, const char* path)
+{
+    return N(net)->load_param_bin(path);
+}
+size_t ncnn_net_load_param_bin_memory(ncnn_net_t net, const unsigned char* mem)
+{
+    return N(net)->load_param_bin_mem(mem);
+}
 size_t ncnn_net_load_model_memory(ncnn_net_t net, const unsigned char* mem)
 {
     return N(net)->load_model(mem);

@@ -10,6 +10,7 @@
 
 #include "layers/hip_layers.h"
 #include "ncnn/layer.h"
+#include "ncnn/datareader.h"
 #include "ncnn/modelbin.h"
 #include "ncnn/net.h"
 #include "ncnn/paramdict.h"
@@ -345,6 +346,111 @@ void ncnn_modelbin_destroy(ncnn_modelbin_t mb)
     if (!mb) return;
     delete (ModelBin*)mb->pthis;
     free(mb);
+}
+
+/* datareader api, src/c_api.cpp:845-1000.  The table's entries forward to the reader that pthis holds; a C program may
+ * replace them (a reader of its own over an asset, a decrypting one).  The loaders below read through the table, so the
+ * replaced entries are the ones that run. */
+namespace {
+class TableDataReader : public DataReader
+{
+public:
+    explicit TableDataReader(ncnn_datareader_t _table) : table(_table) {}
+    virtual int scan(const char* format, void* p) const
+    {
+        return table && table->scan ? table->scan(table, format, p) : 0;
+    }
+    virtual size_t read(void* buf, size_t size) const
+    {
+        return table && table->read ? table->read(table, buf, size) : 0;
+    }
+
+private:
+    ncnn_datareader_t table;
+};
+
+int held_reader_scan(ncnn_datareader_t dr, const char* format, void* p)
+{
+    return ((const DataReader*)dr->pthis)->scan(format, p);
+}
+size_t held_reader_read(ncnn_datareader_t dr, void* buf, size_t size)
+{
+    return ((const DataReader*)dr->pthis)->read(buf, size);
+}
+ncnn_datareader_t table_over(DataReader* held)
+{
+    ncnn_datareader_t dr = (ncnn_datareader_t)malloc(sizeof(struct __ncnn_datareader_t));
+    if (!dr)
+    {
+        delete held;
+        return 0;
+    }
+    dr->pthis = (void*)held;
+    dr->scan = held_reader_scan;
+    dr->read = held_reader_read;
+    return dr;
+}
+
+// a ModelBin that reads through a table for as long as it lives
+class TableModelBin : public ModelBin
+{
+public:
+    explicit TableModelBin(ncnn_datareader_t table) : through(table), reader(through) {}
+    virtual Mat load(int w, int type) const
+    {
+        return reader.load(w, type);
+    }
+
+private:
+    TableDataReader through;
+    ModelBinFromDataReader reader;
+};
+} // namespace
+
+ncnn_datareader_t ncnn_datareader_create(void)
+{
+    return table_over(new DataReader()); // reads nothing until the caller fills the table in
+}
+ncnn_datareader_t ncnn_datareader_create_from_stdio(FILE* fp)
+{
+    return table_over(new DataReaderFromStdio(fp));
+}
+ncnn_datareader_t ncnn_datareader_create_from_memory(const unsigned char** mem)
+{
+    if (!mem) return 0;
+    return table_over(new DataReaderFromMemory(*mem)); // *mem moves on as bytes are consumed
+}
+void ncnn_datareader_destroy(ncnn_datareader_t dr)
+{
+    if (!dr) return;
+    delete (DataReader*)dr->pthis;
+    free(dr);
+}
+ncnn_modelbin_t ncnn_modelbin_create_from_datareader(const ncnn_datareader_t dr)
+{
+    if (!dr) return 0;
+    ncnn_modelbin_t mb = (ncnn_modelbin_t)malloc(sizeof(struct __ncnn_modelbin_t));
+    if (!mb) return 0;
+    mb->pthis = (void*)static_cast<ModelBin*>(new TableModelBin(dr));
+    mb->load_1d = modelbin_load_1d;
+    mb->load_2d = modelbin_load_2d;
+    mb->load_3d = modelbin_load_3d;
+    return mb;
+}
+int ncnn_net_load_param_datareader(ncnn_net_t net, const ncnn_datareader_t dr)
+{
+    if (!net || !dr) return -1;
+    return ((Net*)net)->load_param(TableDataReader(dr));
+}
+int ncnn_net_load_param_bin_datareader(ncnn_net_t net, const ncnn_datareader_t dr)
+{
+    if (!net || !dr) return -1;
+    return ((Net*)net)->load_param_bin(TableDataReader(dr));
+}
+int ncnn_net_load_model_datareader(ncnn_net_t net, const ncnn_datareader_t dr)
+{
+    if (!net || !dr) return -1;
+    return ((Net*)net)->load_model(TableDataReader(dr));
 }
 
 /* layer api, src/c_api.cpp:1352-1600 */

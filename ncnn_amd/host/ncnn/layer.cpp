@@ -145,33 +145,50 @@ Layer* Flatten_layer_creator(void*);
 Layer* Softmax_layer_creator(void*);
 Layer* Dropout_layer_creator(void*);
 
+// The index of a type is its place in the reference's list of layers (the ncnn_add_layer calls of src/CMakeLists.txt:66-176,
+// numbered from 0 by cmake/ncnn_add_layer.cmake into layer_type_enum.h): a .param.bin file names its layers by these numbers.
 static const layer_registry_entry g_builtin[] = {
-    {"Input", Input_layer_creator},
-    {"Convolution", 0},
-    {"ConvolutionDepthWise", 0},
-    {"InnerProduct", 0},
-    {"Gemm", 0},
-    {"Split", Split_layer_creator},
-    {"ReLU", ReLU_layer_creator},
-    {"Pooling", Pooling_layer_creator},
-    {"Eltwise", Eltwise_layer_creator},
-    {"Flatten", Flatten_layer_creator},
-    {"Softmax", Softmax_layer_creator},
-    {"Dropout", Dropout_layer_creator},
+    {"Input", Input_layer_creator, 16},
+    {"Convolution", 0, 6},
+    {"ConvolutionDepthWise", 0, 42},
+    {"InnerProduct", 0, 15},
+    {"Gemm", 0, 74},
+    {"MultiHeadAttention", 0, 79},
+    {"Split", Split_layer_creator, 33},
+    {"ReLU", ReLU_layer_creator, 26},
+    {"Pooling", Pooling_layer_creator, 21},
+    {"Eltwise", Eltwise_layer_creator, 10},
+    {"Flatten", Flatten_layer_creator, 14},
+    {"Softmax", Softmax_layer_creator, 32},
+    {"Dropout", Dropout_layer_creator, 9},
 };
 static const int g_builtin_count = (int)(sizeof(g_builtin) / sizeof(g_builtin[0]));
+
+static const layer_registry_entry* builtin_of(int index)
+{
+    for (int i = 0; i < g_builtin_count; i++)
+        if (g_builtin[i].typeindex == index) return &g_builtin[i];
+    return 0;
+}
 
 int layer_to_index(const char* type)
 {
     for (int i = 0; i < g_builtin_count; i++)
-        if (strcmp(type, g_builtin[i].name) == 0) return i;
+        if (strcmp(type, g_builtin[i].name) == 0) return g_builtin[i].typeindex;
     return -1;
+}
+
+const char* layer_index_to_type(int index)
+{
+    const layer_registry_entry* e = builtin_of(index);
+    return e ? e->name : 0;
 }
 
 Layer* create_layer(int index)
 {
-    if (index < 0 || index >= g_builtin_count || !g_builtin[index].creator) return 0;
-    Layer* layer = g_builtin[index].creator(0);
+    const layer_registry_entry* e = builtin_of(index);
+    if (!e || !e->creator) return 0;
+    Layer* layer = e->creator(0);
     layer->typeindex = index;
     return layer;
 }

@@ -98,12 +98,14 @@ struct layer_registry_entry
 {
     const char* name;
     layer_creator_func creator; // NULL: the type is known but has no host implementation
+    int typeindex;              // the reference's number for the type
 };
 
 // built-in type table.  The four int8 hot-path types are listed (so that registering them
 // through Net::register_custom_layer takes the overwrite-builtin route) but deliberately have
 // no host implementation: without the HIP layers registered, loading a net that uses them fails.
 NCNN_EXPORT int layer_to_index(const char* type);
+NCNN_EXPORT const char* layer_index_to_type(int index); // NULL for a number no built-in type has
 NCNN_EXPORT Layer* create_layer(const char* type);
 NCNN_EXPORT Layer* create_layer(int index);
 NCNN_EXPORT Layer* create_layer_cpu(const char* type);

@@ -133,6 +133,73 @@ public:
         return layer;
     }
 
+    // shape hints (id 30: [dims, w, h, c] per top blob), feature mask (id 31), then the layer's own load_param
+    int configure_layer(Layer* layer, const ParamDict& pd)
+    {
+        const int nbottom = (int)layer->bottoms.size(), ntop = (int)layer->tops.size();
+        const Mat hints = pd.get(30, Mat());
+        if (!hints.empty())
+        {
+            const int* p = hints;
+            int pos = 0;
+            for (int j = 0; j < ntop && pos < hints.w; j++)
+            {
+                const int dims = p[pos];
+                if (pos + 4 > hints.w) break;
+                Blob& b = blobs[layer->tops[j]];
+                Mat s;
+                s.dims = dims;
+                s.w = p[pos + 1];
+                s.h = dims >= 2 ? p[pos + 2] : 1;
+                s.c = dims >= 3 ? p[pos + 3] : 1;
+                s.d = 1;
+                b.shape = s;
+                pos += 4;
+            }
+        }
+        layer->bottom_shapes.resize((size_t)nbottom);
+        for (int j = 0; j < nbottom; j++) layer->bottom_shapes[j] = blobs[layer->bottoms[j]].shape;
+        layer->top_shapes.resize((size_t)ntop);
+        for (int j = 0; j < ntop; j++) layer->top_shapes[j] = blobs[layer->tops[j]].shape;
+        layer->featmask = pd.get(31, 0);
+        return layer->load_param(pd);
+    }
+
+    // graph inputs are the tops of Input layers, outputs are blobs nobody consumes
+    void index_inputs_and_outputs()
+    {
+        for (size_t li = 0; li < layers.size(); li++)
+            if (layers[li]->type == "Input")
+                for (size_t j = 0; j < layers[li]->tops.size(); j++) input_idx.push_back(layers[li]->tops[j]);
+        for (size_t bi = 0; bi < blobs.size(); bi++)
+            if (blobs[bi].producer >= 0 && blobs[bi].consumer < 0) output_idx.push_back((int)bi);
+        for (size_t i = 0; i < input_idx.size(); i++) input_nm.push_back(blobs[input_idx[i]].name.c_str());
+        for (size_t i = 0; i < output_idx.size(); i++) output_nm.push_back(blobs[output_idx[i]].name.c_str());
+    }
+
+    // a layer by the number a .param.bin file holds: a built-in type (possibly replaced) or a registered custom slot
+    Layer* make_layer(int typeindex)
+    {
+        if (typeindex < 0) return 0;
+        if (typeindex & CUSTOM_BIT)
+        {
+            const size_t i = (size_t)(typeindex & ~CUSTOM_BIT);
+            if (i >= custom.size() || !custom[i].creator) return 0;
+            Layer* layer = custom[i].creator(custom[i].userdata);
+            if (layer)
+            {
+                layer->typeindex = typeindex;
+                layer->type = custom[i].name;
+            }
+            return layer;
+        }
+        const char* type = layer_index_to_type(typeindex);
+        if (!type) return 0;
+        Layer* layer = make_layer(type);
+        if (layer) layer->type = type;
+        return layer;
+    }
+
     void destroy_layer(Layer* layer)
     {
         const int ti = layer->typeindex;
@@ -1005,51 +1072,128 @@ int Net::load_param(const DataReader& dr)
             return -1;
         }
 
-        // id 30: shape hints, [dims, w, h, c] per top blob;  id 31: feature mask
-        const Mat hints = pd.get(30, Mat());
-        if (!hints.empty())
-        {
-            const int* p = hints;
-            int pos = 0;
-            for (int j = 0; j < ntop && pos < hints.w; j++)
-            {
-                const int dims = p[pos];
-                if (pos + 4 > hints.w) break;
-                Blob& b = d->blobs[layer->tops[j]];
-                Mat s;
-                s.dims = dims;
-                s.w = p[pos + 1];
-                s.h = dims >= 2 ? p[pos + 2] : 1;
-                s.c = dims >= 3 ? p[pos + 3] : 1;
-                s.d = 1;
-                b.shape = s;
-                pos += 4;
-            }
-        }
-        layer->bottom_shapes.resize((size_t)nbottom);
-        for (int j = 0; j < nbottom; j++) layer->bottom_shapes[j] = d->blobs[layer->bottoms[j]].shape;
-        layer->top_shapes.resize((size_t)ntop);
-        for (int j = 0; j < ntop; j++) layer->top_shapes[j] = d->blobs[layer->tops[j]].shape;
-        layer->featmask = pd.get(31, 0);
-
-        int ret = layer->load_param(pd);
-        if (ret != 0)
+        if (d->configure_layer(layer, pd) != 0)
         {
             NCNN_LOGE("layer load_param %d %s failed", li, name);
             clear();
             return -1;
         }
     }
-
-    // graph inputs are the tops of Input layers, outputs are blobs nobody consumes
-    for (int li = 0; li < layer_count; li++)
-        if (d->layers[li]->type == "Input")
-            for (size_t j = 0; j < d->layers[li]->tops.size(); j++) d->input_idx.push_back(d->layers[li]->tops[j]);
-    for (size_t bi = 0; bi < d->blobs.size(); bi++)
-        if (d->blobs[bi].producer >= 0 && d->blobs[bi].consumer < 0) d->output_idx.push_back((int)bi);
-    for (size_t i = 0; i < d->input_idx.size(); i++) d->input_nm.push_back(d->blobs[d->input_idx[i]].name.c_str());
-    for (size_t i = 0; i < d->output_idx.size(); i++) d->output_nm.push_back(d->blobs[d->output_idx[i]].name.c_str());
+    d->index_inputs_and_outputs();
     return 0;
+}
+
+// The binary form of the .param text (src/net.cpp:1667-2018; tools/ncnn2mem.cpp writes it): 32-bit little-endian words, no
+// names.  magic, layer count, blob count; per layer its type number, bottom count, top count, the blob numbers, and the
+// parameters as ParamDict::load_param_bin reads them.  Layers and blobs are then known by number (the .id.h file that
+// ncnn2mem writes beside it holds the numbers); a layer also gets the name of its type, which the executor reads.
+int Net::load_param_bin(const DataReader& dr)
+{
+    int head[3] = {0, 0, 0};
+    if (dr.read(head, sizeof(head)) != sizeof(head))
+    {
+        NCNN_LOGE("read magic and counts failed");
+        return -1;
+    }
+    if (head[0] != 7767517)
+    {
+        NCNN_LOGE("param is too old, please regenerate");
+        return -1;
+    }
+    const int layer_count = head[1], blob_count = head[2];
+    if (layer_count <= 0 || blob_count <= 0 || layer_count > (1 << 24) || blob_count > (1 << 24))
+    {
+        NCNN_LOGE("invalid layer_count or blob_count");
+        return -1;
+    }
+    d->layers.assign((size_t)layer_count, (Layer*)0);
+    d->blobs.assign((size_t)blob_count, Blob());
+    ParamDict pd;
+    for (int li = 0; li < layer_count; li++)
+    {
+        int lh[3] = {0, 0, 0}; // type number, bottom count, top count
+        if (dr.read(lh, sizeof(lh)) != sizeof(lh) || lh[1] < 0 || lh[2] < 0 || lh[1] > blob_count || lh[2] > blob_count)
+        {
+            NCNN_LOGE("read layer header failed at layer %d", li);
+            clear();
+            return -1;
+        }
+        Layer* layer = d->make_layer(lh[0]);
+        if (!layer)
+        {
+            NCNN_LOGE("layer %d not exists or registered", lh[0]);
+            clear();
+            return -1;
+        }
+        d->layers[li] = layer;
+        layer->bottoms.resize((size_t)lh[1]);
+        layer->tops.resize((size_t)lh[2]);
+        for (int j = 0; j < lh[1] + lh[2]; j++)
+        {
+            int bi = -1;
+            if (dr.read(&bi, 4) != 4 || bi < 0 || bi >= blob_count)
+            {
+                NCNN_LOGE("layer %d: blob number %d in a net of %d blobs", li, bi, blob_count);
+                clear();
+                return -1;
+            }
+            if (j < lh[1])
+            {
+                d->blobs[bi].consumer = li;
+                layer->bottoms[j] = bi;
+            }
+            else
+            {
+                d->blobs[bi].producer = li;
+                layer->tops[j - lh[1]] = bi;
+            }
+        }
+        if (pd.load_param_bin(dr) != 0)
+        {
+            NCNN_LOGE("ParamDict load_param_bin %d failed", li);
+            clear();
+            return -1;
+        }
+        if (d->configure_layer(layer, pd) != 0)
+        {
+            NCNN_LOGE("layer load_param %d failed", li);
+            clear();
+            return -1;
+        }
+    }
+    // the reference leaves layers and blobs of such a net without names; here each is named by its number in decimal, so that
+    // the entry points that take a name (the device-resident ones among them) reach it too
+    for (int li = 0; li < layer_count; li++) d->layers[li]->name = std::to_string(li);
+    for (int bi = 0; bi < blob_count; bi++) d->blobs[bi].name = std::to_string(bi);
+    d->index_inputs_and_outputs();
+    return 0;
+}
+
+int Net::load_param_bin(FILE* fp)
+{
+    DataReaderFromStdio dr(fp);
+    return load_param_bin(dr);
+}
+
+int Net::load_param_bin(const char* protopath)
+{
+    FILE* fp = fopen(protopath, "rb");
+    if (!fp)
+    {
+        NCNN_LOGE("fopen %s failed", protopath);
+        return -1;
+    }
+    int ret = load_param_bin(fp);
+    fclose(fp);
+    return ret;
+}
+
+size_t Net::load_param_bin_mem(const unsigned char* mem)
+{
+    const unsigned char* cursor = mem;
+    DataReaderFromMemory dr(cursor);
+    if (load_param_bin(dr) != 0) return 0;
+    return (size_t)(cursor - mem);
 }
 
 int Net::load_param(FILE* fp)

@@ -37,6 +37,11 @@ public:
     int load_param(FILE* fp);
     int load_param(const char* protopath);
     int load_param_mem(const char* mem);
+    // the binary form (32-bit words, layers and blobs by number)
+    int load_param_bin(const DataReader& dr);
+    int load_param_bin(FILE* fp);
+    int load_param_bin(const char* protopath);
+    size_t load_param_bin_mem(const unsigned char* mem); // bytes consumed, 0 on failure
 
     int load_model(const DataReader& dr);
     int load_model(FILE* fp);

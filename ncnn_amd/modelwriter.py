@@ -101,3 +101,51 @@ def assemble_param(lines):
         nb, nt = int(tok[2]), int(tok[3])
         blobs.update(tok[4: 4 + nb + nt])
     return "7767517\n%d %d\n%s\n" % (len(lines), len(blobs), "\n".join(lines))
+
+
+# The reference's number for a layer type: its place among the ncnn_add_layer calls of src/CMakeLists.txt:66-176 (the
+# generated layer_type_enum.h); a .param.bin file names its layers by these numbers.
+LAYER_TYPE_INDEX = {"Dropout": 9, "Eltwise": 10, "Flatten": 14, "InnerProduct": 15, "Input": 16, "Pooling": 21, "ReLU": 26, "Softmax": 32,
+                    "Split": 33, "Convolution": 6, "ConvolutionDepthWise": 42, "Gemm": 74, "MultiHeadAttention": 79}
+
+
+def _is_float_text(v):
+    return "." in v or "e" in v.lower()
+
+
+def assemble_param_bin(lines, custom_types=()):
+    """The same net as assemble_param(lines) in the binary form Net::load_param_bin reads (src/net.cpp:1667-2018), as
+    tools/ncnn2mem.cpp writes it: 32-bit little-endian words; magic, layer count, blob count; per layer the type number,
+    bottom count, top count, the blob numbers (in order of first appearance in the text), then per parameter its id and
+    value -- id as it is for a scalar (a value with '.' or 'e' in its text is a float, anything else an int), -23300 - id
+    and a length before an array, -23400 - id, a length and the bytes padded to words before a string -- and -233 to end
+    the layer.  custom_types: names of registered custom layers, numbered 256 + place."""
+    number, out = {}, []
+    for ln in lines:
+        tok = ln.split()
+        nb, nt = int(tok[2]), int(tok[3])
+        for b in tok[4: 4 + nb + nt]:
+            number.setdefault(b, len(number))
+    out.append(struct.pack("<3i", 7767517, len(lines), len(number)))
+    for ln in lines:
+        tok = ln.split()
+        nb, nt = int(tok[2]), int(tok[3])
+        ti = LAYER_TYPE_INDEX[tok[0]] if tok[0] in LAYER_TYPE_INDEX else 256 + list(custom_types).index(tok[0])
+        out.append(struct.pack("<3i", ti, nb, nt))
+        out.append(struct.pack("<%di" % (nb + nt), *[number[b] for b in tok[4: 4 + nb + nt]]))
+        for item in tok[4 + nb + nt:]:
+            key, value = item.split("=", 1)
+            pid = int(key)
+            if pid <= -23300:
+                vals = value.split(",")
+                count = int(vals[0])
+                out.append(struct.pack("<2i", pid, count))
+                for v in vals[1: 1 + count]:
+                    out.append(struct.pack("<f", float(v)) if _is_float_text(v) else struct.pack("<i", int(v)))
+            elif value[:1] == '"' or value[:1].isalpha():
+                text = value.strip('"').encode()
+                out.append(struct.pack("<2i", -23400 - pid, len(text)) + _pad4(text))
+            else:
+                out.append(struct.pack("<i", pid) + (struct.pack("<f", float(value)) if _is_float_text(value) else struct.pack("<i", int(value))))
+        out.append(struct.pack("<i", -233))
+    return b"".join(out), number

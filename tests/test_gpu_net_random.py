@@ -14,7 +14,7 @@ import numpy as np
 import pytest
 
 import refnet
-from ncnn_amd import host, zoo
+from ncnn_amd import host, modelwriter as mw, zoo
 
 pytestmark = pytest.mark.gpu
 F = np.float32
@@ -186,6 +186,29 @@ def test_random_net_through_the_plugin_matches_the_oracle(seed):
     for name in [t for L in g.layers if L["type"] not in ("Input", "Split", "Softmax") for t in L["tops"]]:
         want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
         got = ex.extract(name)
+        assert np.array_equal(np.asarray(got).reshape(want.shape), want), name
+
+
+@pytest.mark.parametrize("resident", [False, True], ids=["host-blobs", "device-resident"])
+@pytest.mark.parametrize("seed", range(COUNT))
+def test_random_net_from_the_binary_param_form_matches_the_oracle(seed, resident):
+    """The same networks loaded from the binary form of their .param text (Net::load_param_bin, src/net.cpp:1667-2018, the
+    file tools/ncnn2mem.cpp writes: layers by the reference's type numbers, blobs by number, no names), fed and read by blob
+    number: every blob bit for bit."""
+    g, param, blob = random_net(seed)
+    x = np.random.default_rng(2000 + seed).uniform(0, 1, g.input_shape).astype(F)
+    print("[case] random net from .param.bin", seed, "resident" if resident else "host", "input", g.input_shape, flush=True)
+    ref = refnet.run(param, blob, x)
+    data, number = mw.assemble_param_bin(param.splitlines()[2:])
+    net = host.Net()
+    assert net.register_int8_layers() == 0
+    net.set_use_hip_compute(resident)
+    assert net.load_param_bin_mem(data) == 0 and net.load_model_mem(blob) == 0
+    ex = net.create_extractor()
+    ex.input(number["data"], x)
+    for name in [t for L in g.layers if L["type"] not in ("Input", "Split", "Softmax") for t in L["tops"]]:
+        want = ref[name].astype(F) if ref[name].dtype == np.int8 else ref[name]
+        got = ex.extract(number[name])
         assert np.array_equal(np.asarray(got).reshape(want.shape), want), name
 
 

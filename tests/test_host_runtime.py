@@ -437,3 +437,120 @@ def test_paramdict_text_parser_on_the_reference_tests_own_vectors():
     import struct
     for bad in (struct.pack("<ii", 0, 5), struct.pack("<iii", 40, 1, -233), struct.pack("<iii", -23301, -4, -233), struct.pack("<iii", -23400, 300, -233)):
         assert host.paramdict_probe_bin(bad + b"\0" * 8, 0)[0] == -1
+
+
+_GLUE_NET = ["Input in0 0 1 data 0=8 1=6 2=3", "Split sp 1 2 data a b", "ReLU r 1 1 a ra 0=1.000000e-01", "Pooling p 1 1 b pb 0=0 1=2 2=2",
+             "Pooling p2 1 1 ra pa 0=1 1=2 2=2 -23330=4,3,4,3,3", "Eltwise e 2 1 pa pb out 0=1 -23301=2,5.000000e-01,2.000000e+00"]
+
+
+def test_net_from_the_binary_param_form_equals_the_net_from_the_text(tmp_path):
+    """Net::load_param_bin (src/net.cpp:1667-2018) on the binary form of a .param text as tools/ncnn2mem.cpp writes it:
+    the same layers, fed and read by blob number (and by the number in decimal, this library's addition); a file cut short
+    anywhere is refused."""
+    from ncnn_amd import modelwriter as mw
+    x = np.random.default_rng(0).normal(size=(3, 6, 8)).astype(np.float32)
+    text_net = host.Net()
+    assert text_net.load_param_mem(mw.assemble_param(_GLUE_NET)) == 0 and text_net.load_model_mem(b"") == 0
+    ex = text_net.create_extractor()
+    ex.input("data", x)
+    want = ex.extract("out")
+    data, number = mw.assemble_param_bin(_GLUE_NET)
+    net = host.Net()
+    assert net.load_param_bin_mem(data) == 0 and net.load_model_mem(b"") == 0
+    assert net.layer_types() == text_net.layer_types() and net.input_names() == [str(number["data"])]
+    ex = net.create_extractor()
+    ex.input(number["data"], x)
+    assert np.array_equal(ex.extract(number["out"]), want)
+    ex = net.create_extractor()
+    ex.input(str(number["data"]), x)
+    assert np.array_equal(ex.extract(str(number["out"])), want)
+    path = tmp_path / "net.param.bin"
+    path.write_bytes(data)
+    assert host.Net().load_param_bin(str(path)) == 0
+    for cut in range(0, len(data), 3):
+        path.write_bytes(data[:cut])
+        assert host.Net().load_param_bin(str(path)) == -1, cut
+    # a type number no layer has, a blob number beyond the count
+    words = np.frombuffer(data, np.int32).copy()
+    words[3] = 200
+    path.write_bytes(words.tobytes())
+    assert host.Net().load_param_bin(str(path)) == -1
+    words = np.frombuffer(data, np.int32).copy()
+    words[6] = 99
+    path.write_bytes(words.tobytes())
+    assert host.Net().load_param_bin(str(path)) == -1
+
+
+def test_layer_type_numbers_are_the_references():
+    """A .param.bin file names layer types by their place among the ncnn_add_layer calls of the reference's
+    src/CMakeLists.txt; the library's table and the writer's have to hold those numbers."""
+    from ncnn_amd import modelwriter as mw
+    L = host.lib()
+    for name, index in mw.LAYER_TYPE_INDEX.items():
+        assert L.ncnn_layer_type_to_index(name.encode()) == index, name
+    cmake = "/root/reference/src/CMakeLists.txt"
+    if not os.path.exists(cmake):
+        pytest.skip("the reference tree is not present on this machine")
+    import re
+    order = re.findall(r"^ncnn_add_layer\((\w+)", open(cmake).read(), re.M)
+    for name, index in mw.LAYER_TYPE_INDEX.items():
+        assert order.index(name) == index, name
+
+
+def test_datareader_tables_feed_the_loaders():
+    """The C API's datareader (src/c_api.h:218-235, 377-380): a table over bytes in memory, whose pointer moves on as the
+    loaders read; a table whose read entry a C program replaced is the one the loader calls."""
+    from ncnn_amd import modelwriter as mw
+    L = host.lib()
+    assert L.ncnn_version().startswith(b"1.0.") and L.ncnn_version_number() == int(L.ncnn_version()[4:])
+    x = np.random.default_rng(1).normal(size=(3, 6, 8)).astype(np.float32)
+    ref = host.Net()
+    assert ref.load_param_mem(mw.assemble_param(_GLUE_NET)) == 0 and ref.load_model_mem(b"") == 0
+    ex = ref.create_extractor()
+    ex.input("data", x)
+    want = ex.extract("out")
+
+    text = mw.assemble_param(_GLUE_NET).encode() + b"\0"
+    buf = C.create_string_buffer(text, len(text))
+    cursor = C.c_char_p(C.addressof(buf))
+    dr = L.ncnn_datareader_create_from_memory(C.byref(cursor))
+    net = host.Net()
+    assert L.ncnn_net_load_param_datareader(net.h_, dr) == 0
+    moved = C.cast(cursor, C.c_void_p).value - C.addressof(buf)
+    assert 0 < moved <= len(text)
+    L.ncnn_datareader_destroy(dr)
+    assert net.load_model_mem(b"") == 0
+    ex = net.create_extractor()
+    ex.input("data", x)
+    assert np.array_equal(ex.extract("out"), want)
+
+    # the binary form through a table whose read entry is the program's own
+    data, number = mw.assemble_param_bin(_GLUE_NET)
+    state = {"pos": 0, "calls": 0}
+    READ = C.CFUNCTYPE(C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t)
+
+    def read(_dr, out, size):
+        chunk = data[state["pos"]: state["pos"] + size]
+        C.memmove(out, chunk, len(chunk))
+        state["pos"] += len(chunk)
+        state["calls"] += 1
+        return len(chunk)
+
+    class Table(C.Structure):
+        _fields_ = [("pthis", C.c_void_p), ("scan", C.c_void_p), ("read", READ)]
+
+    dr = L.ncnn_datareader_create()
+    table = C.cast(dr, C.POINTER(Table)).contents
+    keep = READ(read)
+    table.read = keep
+    net = host.Net()
+    assert L.ncnn_net_load_param_bin_datareader(net.h_, dr) == 0 and state["pos"] == len(data) and state["calls"] > 0
+    L.ncnn_datareader_destroy(dr)
+    assert net.load_model_mem(b"") == 0
+    ex = net.create_extractor()
+    ex.input(number["data"], x)
+    assert np.array_equal(ex.extract(number["out"]), want)
+    # a table that reads nothing: the loaders fail instead of reading stale memory
+    dr = L.ncnn_datareader_create()
+    assert L.ncnn_net_load_param_datareader(host.Net().h_, dr) == -1 and L.ncnn_net_load_param_bin_datareader(host.Net().h_, dr) == -1
+    L.ncnn_datareader_destroy(dr)
