@@ -391,6 +391,16 @@ def test_param_parser_survives_mutated_text():
     assert p.returncode == 0 and "survived 600" in p.stdout, (p.returncode, p.stdout[-300:], p.stderr[-600:])
 
 
+def test_binary_param_loader_survives_mutated_files():
+    """600 mutated .param.bin files (tests/paramfuzz.py) in a child process: return codes, never a crash."""
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    p = subprocess.run([sys.executable, os.path.join(here, "paramfuzz.py"), "21", "600", "bin"], capture_output=True, text=True, timeout=300,
+                       cwd=os.path.dirname(here), env=dict(os.environ, PYTHONPATH=os.path.dirname(here)))
+    assert p.returncode == 0 and "survived 600" in p.stdout, (p.returncode, p.stdout[-300:], p.stderr[-600:])
+
+
 def test_paramdict_text_parser_on_the_reference_tests_own_vectors():
     """tests/golden/paramdict_vectors.json: the inputs and expected values that the reference's tests/test_paramdict.cpp holds
     for the text parser (src/paramdict.cpp:263-489) -- types, ints, floats compared as float32 the way the reference test
