@@ -189,20 +189,32 @@ def test_random_net_through_the_plugin_matches_the_oracle(seed):
         assert np.array_equal(np.asarray(got).reshape(want.shape), want), name
 
 
-@pytest.mark.parametrize("resident", [False, True], ids=["host-blobs", "device-resident"])
+@pytest.mark.parametrize("resident", [False, True, "plugin"], ids=["host-blobs", "device-resident", "plug-in"])
 @pytest.mark.parametrize("seed", range(COUNT))
 def test_random_net_from_the_binary_param_form_matches_the_oracle(seed, resident):
     """The same networks loaded from the binary form of their .param text (Net::load_param_bin, src/net.cpp:1667-2018, the
     file tools/ncnn2mem.cpp writes: layers by the reference's type numbers, blobs by number, no names), fed and read by blob
-    number: every blob bit for bit."""
+    number: every blob bit for bit.  Also with the layers supplied by the plug-in, which registers them by type name and is
+    found by type number here."""
     g, param, blob = random_net(seed)
     x = np.random.default_rng(2000 + seed).uniform(0, 1, g.input_shape).astype(F)
-    print("[case] random net from .param.bin", seed, "resident" if resident else "host", "input", g.input_shape, flush=True)
+    print("[case] random net from .param.bin", seed, resident if resident == "plugin" else "resident" if resident else "host", "input", g.input_shape, flush=True)
     ref = refnet.run(param, blob, x)
     data, number = mw.assemble_param_bin(param.splitlines()[2:])
     net = host.Net()
-    assert net.register_int8_layers() == 0
-    net.set_use_hip_compute(resident)
+    if resident == "plugin":
+        import ctypes as C
+        from ncnn_amd import build
+        host.lib()
+        if not os.path.exists(build.LIBPLUGIN):
+            raise RuntimeError("%s is missing: build it with python ncnn_amd/build.py" % build.LIBPLUGIN)
+        plugin = C.CDLL(build.LIBPLUGIN)
+        plugin.ncnnhip_plugin_register.restype = C.c_int
+        plugin.ncnnhip_plugin_register.argtypes = [C.c_void_p]
+        assert plugin.ncnnhip_plugin_register(net.h_) == 0
+    else:
+        assert net.register_int8_layers() == 0
+        net.set_use_hip_compute(resident)
     assert net.load_param_bin_mem(data) == 0 and net.load_model_mem(blob) == 0
     ex = net.create_extractor()
     ex.input(number["data"], x)
